@@ -1,0 +1,165 @@
+/*
+ * mesh_moe.h -- C ABI of libmesh_moe_hip.so: the top-2 Mixture-of-Experts
+ * forward path of Mesh TensorFlow (mesh_tensorflow/transformer/moe.py) as
+ * hand-written HIP kernels for gfx950 (MI355X).
+ *
+ * Conventions
+ *   - every pointer is a DEVICE pointer owned by the caller unless the
+ *     parameter name ends in _host; the library never allocates or frees;
+ *   - every call is asynchronous on the hipStream_t passed as `stream`
+ *     (a void* here so that C callers need no HIP headers; 0 = null stream);
+ *   - return value 0 = launched, negative = rejected before any launch
+ *     (MESH_MOE_E_*); mesh_moe_last_error() gives the reason for the calling
+ *     thread's last rejected call;
+ *   - all tensors are dense row-major with the shapes written in brackets.
+ *
+ * Each entry point names the part of the reference it replaces
+ * (file:line under the reference tree).  The reference itself has no FFI: it
+ * lowers the layer to ~100 TensorFlow ops through MeshImpl.slicewise
+ * (mesh_tensorflow/ops.py:1019-1030); these functions are what a MeshImpl's
+ * slice function binds instead.
+ */
+#ifndef MESH_MOE_H_
+#define MESH_MOE_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MESH_MOE_ABI_VERSION 1
+
+/* element types of activations / weights */
+#define MESH_MOE_F32 0
+#define MESH_MOE_BF16 1
+
+/* moe_second_policy_* (transformer/moe.py:1452-1467) */
+#define MESH_MOE_SECOND_ALL 0
+#define MESH_MOE_SECOND_NONE 1
+#define MESH_MOE_SECOND_THRESHOLD 2
+#define MESH_MOE_SECOND_RANDOM 3
+
+/* expert activation (mesh_tensorflow/ops.py:1818-1921) */
+#define MESH_MOE_ACT_LINEAR 0
+#define MESH_MOE_ACT_RELU 1
+#define MESH_MOE_ACT_GELU 2
+#define MESH_MOE_ACT_SIGMOID 3
+#define MESH_MOE_ACT_TANH 4
+#define MESH_MOE_ACT_SWISH 5
+
+/* error codes */
+#define MESH_MOE_E_ARG (-1)        /* bad argument (null, size, enum)        */
+#define MESH_MOE_E_UNSUPPORTED (-2) /* shape outside what the kernels handle */
+#define MESH_MOE_E_HIP (-3)        /* a HIP runtime call failed              */
+
+int mesh_moe_abi_version(void);
+const char* mesh_moe_last_error(void);
+
+/*
+ * Router projection: logits[b,t,e] = sum_m float(x[b,t,m]) * float(w[b,m,e])
+ * (+ bias[e] if bias != NULL), float32 accumulate.
+ * Replaces the `mtf.layers.dense(gate_inputs, experts_dim, use_bias=False)`
+ * einsum of _top_2_gating (transformer/moe.py:1384-1390; layers.py:129-208).
+ * batch > 1 is the inner level of the hierarchical layer, where every outer
+ * expert has its own router (outer_expert_dims, moe.py:743-753).
+ *   x [batch, tokens, M] dtype; w [batch, M, E] dtype; logits [batch,tokens,E]
+ * `bias` is a benchmark hook (skewed-routing stress); the reference has none.
+ */
+int mesh_moe_router_logits(const void* x, const void* w, const float* bias,
+                           float* logits, int batch, int64_t tokens, int M,
+                           int E, int dtype, void* stream);
+
+/* Bytes of scratch mesh_moe_top2_gating needs for (G, S, E). */
+size_t mesh_moe_gating_workspace_bytes(int G, int S, int E);
+
+/*
+ * Top-2 gating from router logits: softmax, first/second expert, gate
+ * normalisation, second-place policy, per-group capacity positions with
+ * overflow drop, and the load-balancing loss.
+ * Replaces _top_2_gating after the router projection
+ * (transformer/moe.py:1391-1496, :1508) -- softmax ops.py:5493-5541, top_1
+ * ops.py:4937-4940, cumsum ops.py:2761-2781 -- without building the dense
+ * [G,S,E,C] combine/dispatch tensors (moe.py:1499-1511): the per-token record
+ * below carries the same information.
+ *   logits      [G,S,E] float32
+ *   importance  [G,S] of importance_dtype, or NULL  (moe.py:1401-1411)
+ *   second_uniform [G,S] float32 U(0,1) samples, required for policy RANDOM
+ *   idx  [G,S,2] int32   expert of first / second choice
+ *   pos  [G,S,2] int32   position_in_expert_k (raw; >= C when dropped)
+ *   gate [G,S,2] float32 normalised gate_k * mask_k_flat (moe.py:1485,:1494)
+ *   kept [G,S,2] uint8   mask_k_flat
+ *   fill [G,E]   int32   occupied slots of each expert after both passes
+ *   loss [1]     float32 balancing loss before moe_loss_coef (moe.py:1420-1442)
+ * Limits: 2 <= E <= 512, S <= 16384, C >= 1.
+ */
+int mesh_moe_top2_gating(const float* logits, const void* importance,
+                         int importance_dtype, const float* second_uniform,
+                         int G, int S, int E, int C, int policy,
+                         double threshold, int use_second_place_loss,
+                         int num_microbatches, int32_t* idx, int32_t* pos,
+                         float* gate, uint8_t* kept, int32_t* fill,
+                         float* loss, void* workspace, size_t workspace_bytes,
+                         void* stream);
+
+/*
+ * Dispatch: expert_in[e,g,c,:] = x[g,s,:] for the token holding slot (e,g,c),
+ * zero rows for empty slots.  Replaces the one-hot dispatch einsum
+ * (transformer/moe.py:443-447; a slot whose activation-dtype gate is exactly
+ * zero is not dispatched, moe.py:1510-1511).
+ *   x [G,S,M] dtype; expert_in [E,G,C,M] dtype
+ *   slot_gate [E,G,C] float32 or NULL: the activation-dtype combine weight of
+ *   the token in each slot (0 for empty slots) = reduce_sum(combine_tensor)
+ *   over the group-size dim, which the hierarchical layer turns into the
+ *   importance of the inner level (moe.py:724-727).
+ */
+int mesh_moe_dispatch(const void* x, const int32_t* idx, const int32_t* pos,
+                      const float* gate, const uint8_t* kept,
+                      const int32_t* fill, void* expert_in, float* slot_gate,
+                      int G, int S, int E, int C, int M, int dtype,
+                      void* stream);
+
+/*
+ * Expert weights are consumed in a K-contiguous ("packed") layout:
+ *   packed[e][n][k] = (dtype) src[e][k][n]
+ * mesh_moe_pack_weights converts the reference's variable layout
+ * (`wi/kernel` [experts, d_model, expert_hidden], `wo/kernel`
+ * [experts, expert_hidden, d_model], transformer/moe.py:469-486,
+ * layers.py:239-251) and casts master dtype -> activation dtype, i.e. it is
+ * the copy_master_to_slices + cast of Variable.lower (ops.py:4039-4051,
+ * placement_mesh_impl.py:67-157) for this MeshImpl.
+ *   src [E,K,N] src_dtype; dst [E,N,K] dst_dtype
+ */
+int mesh_moe_pack_weights(const void* src, void* dst, int E, int K, int N,
+                          int src_dtype, int dst_dtype, void* stream);
+
+/*
+ * Expert feed-forward: h = act(expert_in . wi); y = h . wo, per expert,
+ * float32 accumulate, h and y stored in dtype.  Replaces dense_product "wi" +
+ * dense "wo" (transformer/moe.py:469-486; v2 :765-774).
+ *   expert_in [E,R,M] dtype (R = rows per expert = groups * capacity)
+ *   wi_packed [E,H,M] dtype; wo_packed [E,N,H] dtype  (see pack_weights)
+ *   h [E,R,H] dtype (caller-provided scratch); y [E,R,N] dtype
+ * bf16 with M and H multiples of 8 runs on the MFMA kernel; float32 and other
+ * shapes run on a plain FMA tile kernel.
+ */
+int mesh_moe_expert_ffn(const void* expert_in, const void* wi_packed,
+                        const void* wo_packed, void* h, void* y, int E, int R,
+                        int M, int H, int N, int activation, int dtype,
+                        void* stream);
+
+/*
+ * Combine: out[g,s,:] = w1 * y[idx1,g,pos1,:] + w2 * y[idx2,g,pos2,:] with
+ * w_k the activation-dtype-rounded gate_k; zero for tokens with no kept
+ * choice.  Replaces the combine einsum (transformer/moe.py:509-510).
+ *   y [E,G,C,N] dtype; out [G,S,N] dtype
+ */
+int mesh_moe_combine(const void* y, const int32_t* idx, const int32_t* pos,
+                     const float* gate, const uint8_t* kept, void* out, int G,
+                     int S, int E, int C, int N, int dtype, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif  /* MESH_MOE_H_ */

@@ -1,0 +1,120 @@
+// Shared helpers for the MoE HIP kernels (gfx950 only).
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#include "../../include/mesh_moe.h"
+
+namespace mesh_moe {
+
+// Per-thread error text returned by mesh_moe_last_error().
+void set_error(const char* fmt, ...);
+
+#define MOE_REQUIRE(cond, code, ...)      \
+  do {                                    \
+    if (!(cond)) {                        \
+      mesh_moe::set_error(__VA_ARGS__);   \
+      return (code);                      \
+    }                                     \
+  } while (0)
+
+#define MOE_CHECK_LAUNCH(what)                                         \
+  do {                                                                 \
+    hipError_t e__ = hipGetLastError();                                \
+    if (e__ != hipSuccess) {                                           \
+      mesh_moe::set_error("%s: %s", (what), hipGetErrorString(e__));   \
+      return MESH_MOE_E_HIP;                                           \
+    }                                                                  \
+  } while (0)
+
+// Raises a kernel's dynamic-LDS limit when `bytes` exceeds the default.
+#define MOE_ALLOW_LDS(kernel, bytes)                                        \
+  do {                                                                      \
+    if ((bytes) > 160 * 1024) {                                             \
+      mesh_moe::set_error("needs %zu bytes of LDS (limit 163840)",          \
+                          (size_t)(bytes));                                 \
+      return MESH_MOE_E_UNSUPPORTED;                                        \
+    }                                                                       \
+    if ((bytes) > 32 * 1024) {                                              \
+      hipError_t e__ = hipFuncSetAttribute(                                 \
+          (const void*)(kernel), hipFuncAttributeMaxDynamicSharedMemorySize,\
+          (int)(bytes));                                                    \
+      if (e__ != hipSuccess) {                                              \
+        mesh_moe::set_error("hipFuncSetAttribute: %s",                      \
+                            hipGetErrorString(e__));                        \
+        return MESH_MOE_E_HIP;                                              \
+      }                                                                     \
+    }                                                                       \
+  } while (0)
+
+static inline bool valid_dtype(int d) {
+  return d == MESH_MOE_F32 || d == MESH_MOE_BF16;
+}
+static inline size_t dtype_size(int d) { return d == MESH_MOE_BF16 ? 2 : 4; }
+
+// ---- bfloat16 as raw bits -------------------------------------------------
+typedef uint16_t bf16_t;
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t v) {
+  return __uint_as_float(((uint32_t)v) << 16);
+}
+
+// round-to-nearest-even, NaN kept quiet
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x0040u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+// value of `f` after a cast to the activation dtype and back
+template <typename T>
+__device__ __forceinline__ float round_to(float f);
+template <>
+__device__ __forceinline__ float round_to<float>(float f) { return f; }
+template <>
+__device__ __forceinline__ float round_to<bf16_t>(float f) {
+  return bf16_to_f32(f32_to_bf16(f));
+}
+
+template <typename T>
+__device__ __forceinline__ float load_f32(const T* p);
+template <>
+__device__ __forceinline__ float load_f32<float>(const float* p) { return *p; }
+template <>
+__device__ __forceinline__ float load_f32<bf16_t>(const bf16_t* p) {
+  return bf16_to_f32(*p);
+}
+
+template <typename T>
+__device__ __forceinline__ void store_f32(T* p, float v);
+template <>
+__device__ __forceinline__ void store_f32<float>(float* p, float v) { *p = v; }
+template <>
+__device__ __forceinline__ void store_f32<bf16_t>(bf16_t* p, float v) {
+  *p = f32_to_bf16(v);
+}
+
+__device__ __forceinline__ float apply_activation(float v, int act) {
+  switch (act) {
+    case MESH_MOE_ACT_RELU:
+      return v > 0.f ? v : 0.f;
+    case MESH_MOE_ACT_GELU: {
+      float c = 0.5f * (1.0f + tanhf(0.7978845608028654f *
+                                     (v + 0.044715f * v * v * v)));
+      return v * c;
+    }
+    case MESH_MOE_ACT_SIGMOID:
+      return 1.0f / (1.0f + expf(-v));
+    case MESH_MOE_ACT_TANH:
+      return tanhf(v);
+    case MESH_MOE_ACT_SWISH:
+      return v / (1.0f + expf(-v));
+    default:
+      return v;
+  }
+}
+
+}  // namespace mesh_moe

@@ -1,0 +1,299 @@
+// Expert feed-forward as a grouped GEMM for gfx950:
+//   h[e] = act(expert_in[e] . wi[e]),  y[e] = h[e] . wo[e]
+// Replaces layers.dense_product "wi" + layers.dense "wo" of
+// mesh_tensorflow/transformer/moe.py:469-486 (hierarchical layer: :765-774).
+//
+// Both GEMMs are "TN": A [R, K] and the packed weight B [N, K] are
+// K-contiguous, C [R, N] = A . B^T.  The bf16 kernel uses
+// v_mfma_f32_32x32x16_bf16 with LDS double buffering; float32 and odd shapes
+// use a plain FMA tile kernel.
+#include "common.h"
+
+namespace mesh_moe {
+
+typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
+typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+
+// ---------------------------------------------------------------------------
+// bf16 MFMA kernel.
+// Block tile BM x BN, K step BK, 4 wavefronts in a 2 x 2 grid, each owning a
+// (BM/2) x (BN/2) sub-tile made of 32 x 32 MFMA tiles.  LDS rows hold BK bf16
+// plus 8 bf16 of padding, which makes the 16-byte fragment reads of 16
+// consecutive rows hit disjoint banks.
+//
+// MFMA 32x32x16 operand layout (per lane l): A row l%32, k = 8*(l/32)..+7;
+// B column l%32, same k; accumulator register r holds row
+// 8*(r/4) + 4*(l/32) + r%4, column l%32.
+// ---------------------------------------------------------------------------
+template <int BM, int BN, int BK>
+struct GemmCfg {
+  static constexpr int THREADS = 256;
+  static constexpr int LDK = BK + 8;  // padded LDS row, in bf16
+  static constexpr int WTM = BM / 2, WTN = BN / 2;
+  static constexpr int TM = WTM / 32, TN = WTN / 32;
+  static constexpr int CPR = BK / 8;  // 16-byte chunks per tile row
+  static constexpr int A_CHUNKS = BM * CPR / THREADS;
+  static constexpr int B_CHUNKS = BN * CPR / THREADS;
+  static constexpr size_t LDS_BYTES = 2ull * (BM + BN) * LDK * sizeof(bf16_t);
+};
+
+template <int BM, int BN, int BK>
+__global__ __launch_bounds__(256) void grouped_gemm_bf16_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
+    bf16_t* __restrict__ Cout, int R, int N, int K, int tiles_m, int tiles_n,
+    int act) {
+  using Cfg = GemmCfg<BM, BN, BK>;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  bf16_t* As = reinterpret_cast<bf16_t*>(smem_raw);  // [2][BM][LDK]
+  bf16_t* Bs = As + 2 * BM * Cfg::LDK;               // [2][BN][LDK]
+
+  // tile decode: consecutive blocks walk the N tiles of one (expert, M tile)
+  // so that blocks resident together share the A panel and stream B once.
+  const int tiles_per_e = tiles_m * tiles_n;
+  const int e = blockIdx.x / tiles_per_e;
+  const int rem = blockIdx.x - e * tiles_per_e;
+  const int tn = rem / tiles_m;
+  const int tm = rem - tn * tiles_m;
+  const int row0 = tm * BM, col0 = tn * BN;
+  const bf16_t* Ae = A + (int64_t)e * R * K;
+  const bf16_t* Be = B + (int64_t)e * N * K;
+  bf16_t* Ce = Cout + (int64_t)e * R * N;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // global -> register staging (rows clamped; the K tail reads zeros)
+  uint4 areg[Cfg::A_CHUNKS], breg[Cfg::B_CHUNKS];
+  auto load_global = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < Cfg::A_CHUNKS; ++i) {
+      int c = tid + i * Cfg::THREADS;
+      int r = c / Cfg::CPR, kc = c % Cfg::CPR;
+      int gr = min(row0 + r, R - 1);
+      int gk = k0 + kc * 8;
+      areg[i] = gk < K ? *reinterpret_cast<const uint4*>(Ae + (int64_t)gr * K + gk)
+                       : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < Cfg::B_CHUNKS; ++i) {
+      int c = tid + i * Cfg::THREADS;
+      int r = c / Cfg::CPR, kc = c % Cfg::CPR;
+      int gr = min(col0 + r, N - 1);
+      int gk = k0 + kc * 8;
+      breg[i] = gk < K ? *reinterpret_cast<const uint4*>(Be + (int64_t)gr * K + gk)
+                       : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto store_lds = [&](int buf) {
+    bf16_t* as = As + buf * BM * Cfg::LDK;
+    bf16_t* bs = Bs + buf * BN * Cfg::LDK;
+#pragma unroll
+    for (int i = 0; i < Cfg::A_CHUNKS; ++i) {
+      int c = tid + i * Cfg::THREADS;
+      int r = c / Cfg::CPR, kc = c % Cfg::CPR;
+      *reinterpret_cast<uint4*>(as + r * Cfg::LDK + kc * 8) = areg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < Cfg::B_CHUNKS; ++i) {
+      int c = tid + i * Cfg::THREADS;
+      int r = c / Cfg::CPR, kc = c % Cfg::CPR;
+      *reinterpret_cast<uint4*>(bs + r * Cfg::LDK + kc * 8) = breg[i];
+    }
+  };
+
+  f32x16_t acc[Cfg::TM][Cfg::TN];
+#pragma unroll
+  for (int i = 0; i < Cfg::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < Cfg::TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const int nk = (K + BK - 1) / BK;
+  load_global(0);
+  store_lds(0);
+  __syncthreads();
+  const int frag_row = lane & 31;
+  const int frag_k = (lane >> 5) * 8;
+  for (int kt = 0; kt < nk; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < nk) load_global((kt + 1) * BK);
+    const bf16_t* as = As + buf * BM * Cfg::LDK + (wm * Cfg::WTM + frag_row) * Cfg::LDK + frag_k;
+    const bf16_t* bs = Bs + buf * BN * Cfg::LDK + (wn * Cfg::WTN + frag_row) * Cfg::LDK + frag_k;
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; ++kk) {
+      bf16x8_t af[Cfg::TM], bfr[Cfg::TN];
+#pragma unroll
+      for (int i = 0; i < Cfg::TM; ++i)
+        af[i] = *reinterpret_cast<const bf16x8_t*>(as + i * 32 * Cfg::LDK + kk * 16);
+#pragma unroll
+      for (int j = 0; j < Cfg::TN; ++j)
+        bfr[j] = *reinterpret_cast<const bf16x8_t*>(bs + j * 32 * Cfg::LDK + kk * 16);
+#pragma unroll
+      for (int i = 0; i < Cfg::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < Cfg::TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+    }
+    if (kt + 1 < nk) store_lds(buf ^ 1);
+    __syncthreads();
+  }
+
+  // epilogue: round to bf16, activation on the rounded value, store
+  const int col_l = lane & 31;
+  const int row_l = (lane >> 5) * 4;
+#pragma unroll
+  for (int i = 0; i < Cfg::TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < Cfg::TN; ++j) {
+      const int col = col0 + wn * Cfg::WTN + j * 32 + col_l;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const int row = row0 + wm * Cfg::WTM + i * 32 + 8 * (r / 4) + row_l + (r % 4);
+        if (row < R && col < N) {
+          float v = round_to<bf16_t>(acc[i][j][r]);
+          if (act != MESH_MOE_ACT_LINEAR) v = apply_activation(v, act);
+          Ce[(int64_t)row * N + col] = f32_to_bf16(v);
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Plain FMA tile kernel (float32, and bf16 shapes the MFMA kernel rejects):
+// 64 x 64 tile, 16-deep K step, each thread a 4 x 4 patch, float32 accumulate
+// in k order.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void grouped_gemm_simple_kernel(
+    const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ Cout,
+    int R, int N, int K, int tiles_m, int tiles_n, int act) {
+  __shared__ float As[16][64 + 4];
+  __shared__ float Bs[16][64 + 4];
+  const int tiles_per_e = tiles_m * tiles_n;
+  const int e = blockIdx.x / tiles_per_e;
+  const int rem = blockIdx.x - e * tiles_per_e;
+  const int tn = rem / tiles_m, tm = rem - tn * tiles_m;
+  const int row0 = tm * 64, col0 = tn * 64;
+  const T* Ae = A + (int64_t)e * R * K;
+  const T* Be = B + (int64_t)e * N * K;
+  T* Ce = Cout + (int64_t)e * R * N;
+  const int tid = threadIdx.x;
+  const int tx = tid & 15, ty = tid >> 4;
+  float acc[4][4];
+#pragma unroll
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[i][j] = 0.f;
+  for (int k0 = 0; k0 < K; k0 += 16) {
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      int c = tid + i * 256;
+      int r = c >> 4, k = c & 15;
+      int gr = row0 + r, gc = col0 + r, gk = k0 + k;
+      As[k][r] = (gr < R && gk < K) ? load_f32<T>(Ae + (int64_t)gr * K + gk) : 0.f;
+      Bs[k][r] = (gc < N && gk < K) ? load_f32<T>(Be + (int64_t)gc * K + gk) : 0.f;
+    }
+    __syncthreads();
+#pragma unroll
+    for (int k = 0; k < 16; ++k) {
+      float a[4], b[4];
+#pragma unroll
+      for (int i = 0; i < 4; ++i) a[i] = As[k][ty * 4 + i];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) b[j] = Bs[k][tx * 4 + j];
+#pragma unroll
+      for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[i][j] = fmaf(a[i], b[j], acc[i][j]);
+    }
+    __syncthreads();
+  }
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    int row = row0 + ty * 4 + i;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      int col = col0 + tx * 4 + j;
+      if (row < R && col < N) {
+        float v = round_to<T>(acc[i][j]);
+        if (act != MESH_MOE_ACT_LINEAR) v = apply_activation(v, act);
+        store_f32<T>(Ce + (int64_t)row * N + col, v);
+      }
+    }
+  }
+}
+
+template <int BM, int BN, int BK>
+static int launch_mfma(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
+                       int R, int N, int K, int act, hipStream_t st) {
+  using Cfg = GemmCfg<BM, BN, BK>;
+  const int tiles_m = (R + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  const int64_t blocks = (int64_t)tiles_m * tiles_n * E;
+  MOE_REQUIRE(blocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
+              "expert_ffn: too many tiles (%lld)", (long long)blocks);
+  auto k = grouped_gemm_bf16_kernel<BM, BN, BK>;
+  MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
+  k<<<(unsigned)blocks, 256, Cfg::LDS_BYTES, st>>>(A, B, C, R, N, K, tiles_m,
+                                                    tiles_n, act);
+  MOE_CHECK_LAUNCH("expert_ffn (mfma)");
+  return 0;
+}
+
+template <typename T>
+static int launch_simple(const T* A, const T* B, T* C, int E, int R, int N,
+                         int K, int act, hipStream_t st) {
+  const int tiles_m = (R + 63) / 64, tiles_n = (N + 63) / 64;
+  const int64_t blocks = (int64_t)tiles_m * tiles_n * E;
+  MOE_REQUIRE(blocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
+              "expert_ffn: too many tiles (%lld)", (long long)blocks);
+  grouped_gemm_simple_kernel<T><<<(unsigned)blocks, 256, 0, st>>>(
+      A, B, C, R, N, K, tiles_m, tiles_n, act);
+  MOE_CHECK_LAUNCH("expert_ffn (fma)");
+  return 0;
+}
+
+// C[e] = act(A[e] . B[e]^T) for every expert.
+static int grouped_gemm(const void* A, const void* B, void* C, int E, int R,
+                        int N, int K, int act, int dtype, hipStream_t st) {
+  if (dtype == MESH_MOE_F32)
+    return launch_simple<float>((const float*)A, (const float*)B, (float*)C, E,
+                                R, N, K, act, st);
+  const bool mfma_ok = (K % 8 == 0) && (((uintptr_t)A | (uintptr_t)B) % 16 == 0);
+  if (!mfma_ok)
+    return launch_simple<bf16_t>((const bf16_t*)A, (const bf16_t*)B,
+                                 (bf16_t*)C, E, R, N, K, act, st);
+  if (R >= 1024 && N >= 1024)
+    return launch_mfma<256, 256, 64>((const bf16_t*)A, (const bf16_t*)B,
+                                     (bf16_t*)C, E, R, N, K, act, st);
+  return launch_mfma<128, 128, 64>((const bf16_t*)A, (const bf16_t*)B,
+                                   (bf16_t*)C, E, R, N, K, act, st);
+}
+
+}  // namespace mesh_moe
+
+using namespace mesh_moe;
+
+extern "C" int mesh_moe_expert_ffn(const void* expert_in, const void* wi_packed,
+                                   const void* wo_packed, void* h, void* y,
+                                   int E, int R, int M, int H, int N,
+                                   int activation, int dtype, void* stream) {
+  MOE_REQUIRE(expert_in && wi_packed && wo_packed && h && y, MESH_MOE_E_ARG,
+              "expert_ffn: null pointer");
+  MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG, "expert_ffn: bad dtype %d",
+              dtype);
+  MOE_REQUIRE(E >= 1 && R >= 1 && M >= 1 && H >= 1 && N >= 1, MESH_MOE_E_ARG,
+              "expert_ffn: bad sizes E=%d R=%d M=%d H=%d N=%d", E, R, M, H, N);
+  MOE_REQUIRE(activation >= MESH_MOE_ACT_LINEAR &&
+                  activation <= MESH_MOE_ACT_SWISH,
+              MESH_MOE_E_ARG, "expert_ffn: unknown activation %d", activation);
+  hipStream_t st = (hipStream_t)stream;
+  int rc = grouped_gemm(expert_in, wi_packed, h, E, R, H, M, activation, dtype,
+                        st);
+  if (rc != 0) return rc;
+  return grouped_gemm(h, wo_packed, y, E, R, N, H, MESH_MOE_ACT_LINEAR, dtype,
+                      st);
+}

@@ -1,0 +1,461 @@
+// Router projection and top-2 gating (softmax, expert choice, capacity
+// positions, balancing loss) for gfx950.
+//
+// Follows _top_2_gating, mesh_tensorflow/transformer/moe.py:1384-1496, with the
+// float32 operation order of mtf.softmax (ops.py:5493-5541) and mtf.top_1
+// (ops.py:4937-4940).  The dense [G,S,E] masks and the S x S cumsum matmul
+// (ops.py:2761-2781) are replaced by a per-token record and integer counting.
+#include "common.h"
+
+namespace mesh_moe {
+
+// ---------------------------------------------------------------------------
+// Router logits: logits[b,t,e] = sum_m x[b,t,m] * w[b,m,e] (+ bias[e]).
+// One block = 64 tokens; thread (tok = tid % 64, eg = tid / 64) accumulates
+// experts eg*EPT .. eg*EPT+EPT-1 with EPT = ceil(E / 4) <= 32.  x and w are
+// staged through LDS as float32 in chunks of KC columns of M.
+// ---------------------------------------------------------------------------
+constexpr int RL_TOK = 64;
+constexpr int RL_KC = 64;
+constexpr int RL_MAX_EPT = 32;
+
+template <typename T>
+__global__ __launch_bounds__(256) void router_logits_kernel(
+    const T* __restrict__ x, const T* __restrict__ w,
+    const float* __restrict__ bias, float* __restrict__ logits,
+    int64_t tokens, int M, int E, int ept) {
+  extern __shared__ float smem[];
+  float* xs = smem;                       // [RL_TOK][RL_KC + 1]
+  float* ws = smem + RL_TOK * (RL_KC + 1);  // [RL_KC][E]
+  const int b = blockIdx.y;
+  const int64_t t0 = (int64_t)blockIdx.x * RL_TOK;
+  const int tid = threadIdx.x;
+  const int tok = tid & 63;
+  const int eg = tid >> 6;
+  const T* xb = x + ((int64_t)b * tokens) * M;
+  const T* wb = w + (int64_t)b * M * E;
+  float acc[RL_MAX_EPT];
+#pragma unroll
+  for (int j = 0; j < RL_MAX_EPT; ++j) acc[j] = 0.f;
+
+  for (int k0 = 0; k0 < M; k0 += RL_KC) {
+    // x tile: 64 tokens x KC, coalesced along M
+    for (int i = tid; i < RL_TOK * RL_KC; i += 256) {
+      int r = i / RL_KC, c = i % RL_KC;
+      int64_t t = t0 + r;
+      float v = 0.f;
+      if (t < tokens && k0 + c < M) v = load_f32<T>(xb + t * M + k0 + c);
+      xs[r * (RL_KC + 1) + c] = v;
+    }
+    for (int i = tid; i < RL_KC * E; i += 256) {
+      int r = i / E, c = i % E;
+      float v = 0.f;
+      if (k0 + r < M) v = load_f32<T>(wb + (int64_t)(k0 + r) * E + c);
+      ws[i] = v;
+    }
+    __syncthreads();
+    const int e0 = eg * ept;
+    for (int k = 0; k < RL_KC; ++k) {
+      float xv = xs[tok * (RL_KC + 1) + k];
+      const float* wr = ws + k * E + e0;
+#pragma unroll
+      for (int j = 0; j < RL_MAX_EPT; ++j) {
+        if (j < ept && e0 + j < E) acc[j] = fmaf(xv, wr[j], acc[j]);
+      }
+    }
+    __syncthreads();
+  }
+  int64_t t = t0 + tok;
+  if (t < tokens) {
+    float* out = logits + ((int64_t)b * tokens + t) * E;
+#pragma unroll
+    for (int j = 0; j < RL_MAX_EPT; ++j) {
+      int e = eg * ept + j;
+      if (j < ept && e < E) out[e] = bias ? acc[j] + bias[e] : acc[j];
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Gating step 1: per token softmax, top-2, gate normalisation, second-place
+// policy; per block column sums of the balancing-loss proxies.
+// Grid (blocks per group, G); one thread per token; the logits tile is staged
+// in LDS with row stride E+1 so that per-thread row walks are conflict-free.
+// ---------------------------------------------------------------------------
+struct GateParams {
+  int G, S, E, C;
+  int policy;
+  float threshold;      // float32(threshold)            (moe.py:1460)
+  float inv_threshold;  // float32(1 / max(thr, 1e-9))   (moe.py:1465)
+  int use_second_place_loss;
+  int num_microbatches;
+  int tt;    // tokens per block of step 1
+  int nblk;  // blocks per group of step 1
+};
+
+// bit 0 of the step-1 `kept` byte: the token competes for a slot (mask_k after
+// importance and policy); bit 1 (second choice only): mask_2 before the policy,
+// which is what the second-place loss counts (moe.py:1430).
+template <typename IT>
+__global__ __launch_bounds__(256) void gate_select_kernel(
+    const float* __restrict__ logits, const IT* __restrict__ importance,
+    const float* __restrict__ second_uniform, GateParams p,
+    int32_t* __restrict__ idx, int32_t* __restrict__ pos,
+    float* __restrict__ gate, uint8_t* __restrict__ kept,
+    float* __restrict__ part1, float* __restrict__ part2) {
+  extern __shared__ float smem[];
+  const int E = p.E, S = p.S;
+  const int ld = E + 1;
+  float* tile = smem;                                  // [tt][E+1]
+  float* isone = smem + (size_t)p.tt * ld;             // [tt]
+  const int g = blockIdx.y;
+  const int blk = blockIdx.x;
+  const int t0 = blk * p.tt;
+  const int ntok = min(p.tt, S - t0);
+  const int tid = threadIdx.x;
+  const float* src = logits + ((int64_t)g * S + t0) * E;
+  for (int i = tid; i < ntok * E; i += blockDim.x) {
+    int r = i / E, c = i - r * E;
+    tile[r * ld + c] = src[i];
+  }
+  __syncthreads();
+
+  float qscale = 0.f;
+  int i1 = 0;
+  bool sel1 = false;
+  if (tid < ntok) {
+    float* row = tile + tid * ld;
+    const int64_t t = (int64_t)g * S + t0 + tid;
+    float m = row[0];
+    for (int e = 1; e < E; ++e) m = fmaxf(m, row[e]);       // reduce_max
+    const float negm = -m;
+    float s = 0.f;
+    for (int e = 0; e < E; ++e) s += expf(row[e] + negm);   // exp, reduce_sum
+    const float neglse = -(logf(s) + m);                    // log + max
+    float g1 = -1.f;
+    for (int e = 0; e < E; ++e) {
+      float pe = expf(row[e] + neglse);                     // exp(log_softmax)
+      row[e] = pe;
+      if (pe > g1) { g1 = pe; i1 = e; }                     // first argmax
+    }
+    sel1 = true;
+    bool sel2 = true;
+    if (importance != nullptr) {
+      float imp = load_f32<IT>(importance + t);
+      sel1 = (imp == 1.0f);                                 // moe.py:1402-1404
+      sel2 = (imp > 0.0f);                                  // moe.py:1411
+    }
+    if (!sel1) g1 = g1 * 0.0f;
+    // gates_without_top_1 = raw_gates * (1 - mask_1); its first argmax.
+    float g2 = -1.f, qsum = 0.f;
+    int i2 = 0;
+    for (int e = 0; e < E; ++e) {
+      float keep = (sel1 && e == i1) ? 0.0f : 1.0f;         // 1 + (-mask_1)
+      float q = row[e] * keep;
+      qsum += q;
+      if (q > g2) { g2 = q; i2 = e; }
+    }
+    const float denom = (g1 + g2) + 1e-9f;                  // moe.py:1413
+    const float r = 1.0f / denom;                           // reciprocal
+    const float g1n = g1 * r, g2n = g2 * r;
+    const bool sel2_loss = sel2;
+    if (p.policy == MESH_MOE_SECOND_NONE) {
+      sel2 = false;
+    } else if (p.policy == MESH_MOE_SECOND_THRESHOLD) {
+      sel2 = sel2 && (g2n > p.threshold);
+    } else if (p.policy == MESH_MOE_SECOND_RANDOM) {
+      sel2 = sel2 && (second_uniform[t] < g2n * p.inv_threshold);
+    }
+    idx[t * 2 + 0] = i1;
+    idx[t * 2 + 1] = i2;
+    pos[t * 2 + 0] = 0;
+    pos[t * 2 + 1] = 0;
+    gate[t * 2 + 0] = g1n;
+    gate[t * 2 + 1] = g2n;
+    kept[t * 2 + 0] = sel1 ? 1 : 0;
+    kept[t * 2 + 1] = (sel2 ? 1 : 0) | (sel2_loss ? 2 : 0);
+    isone[tid] = sel1 ? 1.0f : 0.0f;
+    qscale = 1.0f / (qsum + 1e-9f);                         // moe.py:1433-1434
+  }
+  __syncthreads();
+  // density_1_proxy partial: sum over the block's tokens of p * (imp == 1)
+  for (int e = tid; e < E; e += blockDim.x) {
+    float s = 0.f;
+    for (int r = 0; r < ntok; ++r) s += tile[r * ld + e] * isone[r];
+    part1[((int64_t)g * p.nblk + blk) * E + e] = s;
+  }
+  if (p.use_second_place_loss) {
+    __syncthreads();
+    if (tid < ntok) {
+      float* row = tile + tid * ld;
+      for (int e = 0; e < E; ++e) {
+        float keep = (sel1 && e == i1) ? 0.0f : 1.0f;
+        row[e] = (row[e] * keep) * qscale;
+      }
+    }
+    __syncthreads();
+    for (int e = tid; e < E; e += blockDim.x) {
+      float s = 0.f;
+      for (int r = 0; r < ntok; ++r) s += tile[r * ld + e];
+      part2[((int64_t)g * p.nblk + blk) * E + e] = s;
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Gating step 2: capacity positions for one group per block (moe.py:1472-1496).
+// Thread (e = tid % EL, chunk = tid / EL) counts, over its chunk of the
+// group's tokens, those whose choice is expert e; an exclusive prefix over the
+// chunks gives each chunk's starting slot; a second walk assigns positions in
+// token order.  Second choices start after the kept first choices of the same
+// expert.  The token's expert ids live in LDS as int16 (-1 = not competing).
+// ---------------------------------------------------------------------------
+constexpr int CAP_THREADS = 1024;
+
+__global__ __launch_bounds__(CAP_THREADS) void gate_capacity_kernel(
+    GateParams p, const int32_t* __restrict__ idx, int32_t* __restrict__ pos,
+    float* __restrict__ gate, uint8_t* __restrict__ kept,
+    int32_t* __restrict__ fill, const float* __restrict__ part1,
+    const float* __restrict__ part2, float* __restrict__ gsum, int el) {
+  extern __shared__ int32_t smem_i[];
+  const int S = p.S, E = p.E, C = p.C;
+  int32_t* cnt = smem_i;                        // [nchunks][el] = CAP_THREADS
+  int32_t* tot = cnt + CAP_THREADS;             // [3][el]: total1,total2,loss2
+  float* prod = reinterpret_cast<float*>(tot + 3 * el);  // [2][el]
+  int16_t* c1 = reinterpret_cast<int16_t*>(prod + 2 * el);  // [S]
+  int16_t* c2 = c1 + S;                                      // [S]
+  int16_t* c2l = c2 + S;                                     // [S] (loss only)
+  const int g = blockIdx.x;
+  const int tid = threadIdx.x;
+  const int64_t base = (int64_t)g * S;
+  const bool loss2 = p.use_second_place_loss != 0;
+  for (int s = tid; s < S; s += CAP_THREADS) {
+    int64_t t = base + s;
+    int a = idx[t * 2], b = idx[t * 2 + 1];
+    uint8_t k1 = kept[t * 2], k2 = kept[t * 2 + 1];
+    c1[s] = (k1 & 1) ? (int16_t)a : (int16_t)-1;
+    c2[s] = (k2 & 1) ? (int16_t)b : (int16_t)-1;
+    if (loss2) c2l[s] = (k2 & 2) ? (int16_t)b : (int16_t)-1;
+  }
+  __syncthreads();
+  const int e = tid % el;
+  const int chunk = tid / el;
+  const int nchunks = CAP_THREADS / el;
+  const int clen = (S + nchunks - 1) / nchunks;
+  const int s_begin = min(S, chunk * clen);
+  const int s_end = min(S, s_begin + clen);
+
+  int count1 = 0;  // kept first choices of expert e (valid after round 0)
+  for (int round = 0; round < 2; ++round) {
+    const int16_t* ch = round == 0 ? c1 : c2;
+    int c = 0;
+    for (int s = s_begin; s < s_end; ++s) c += (ch[s] == e);
+    cnt[chunk * el + e] = c;
+    __syncthreads();
+    int before = 0, total = 0;
+    for (int k = 0; k < nchunks; ++k) {
+      int v = cnt[k * el + e];
+      total += v;
+      if (k < chunk) before += v;
+    }
+    int running = before + (round == 0 ? 0 : count1);
+    for (int s = s_begin; s < s_end; ++s) {
+      if (ch[s] == e) {
+        int64_t t = base + s;
+        const bool ok = running < C;
+        pos[t * 2 + round] = running;
+        kept[t * 2 + round] = ok ? 1 : 0;
+        if (!ok) gate[t * 2 + round] = gate[t * 2 + round] * 0.0f;
+        ++running;
+      }
+    }
+    if (chunk == 0 && e < E) tot[round * el + e] = total;
+    if (round == 0) count1 = min(total, C);
+    __syncthreads();
+  }
+  // tokens that did not compete: mask_k_flat = 0 -> gate_k * 0, kept = 0
+  for (int s = tid; s < S; s += CAP_THREADS) {
+    int64_t t = base + s;
+    if (c1[s] < 0) { kept[t * 2] = 0; gate[t * 2] = gate[t * 2] * 0.0f; }
+    if (c2[s] < 0) {
+      kept[t * 2 + 1] = 0;
+      gate[t * 2 + 1] = gate[t * 2 + 1] * 0.0f;
+    }
+  }
+  if (loss2) {
+    int c = 0;
+    for (int s = s_begin; s < s_end; ++s) c += (c2l[s] == e);
+    cnt[chunk * el + e] = c;
+    __syncthreads();
+    if (chunk == 0 && e < E) {
+      int total = 0;
+      for (int k = 0; k < nchunks; ++k) total += cnt[k * el + e];
+      tot[2 * el + e] = total;
+    }
+    __syncthreads();
+  }
+  // per-expert outputs and the group's share of the balancing loss
+  if (tid < E) {
+    const int t1 = tot[tid], t2 = tot[el + tid];
+    const int k1 = min(t1, C);
+    fill[(int64_t)g * E + tid] = k1 + min(t2, C - k1);
+    const float inv_s = (float)(1.0 / (double)S);
+    float proxy = 0.f;
+    for (int b = 0; b < p.nblk; ++b)
+      proxy += part1[((int64_t)g * p.nblk + b) * E + tid];
+    prod[tid] = (proxy * inv_s) * ((float)t1 * inv_s);       // moe.py:1420-1423
+    if (loss2) {
+      float proxy2 = 0.f;
+      for (int b = 0; b < p.nblk; ++b)
+        proxy2 += part2[((int64_t)g * p.nblk + b) * E + tid];
+      prod[el + tid] = (proxy2 * inv_s) * ((float)tot[2 * el + tid] * inv_s);
+    }
+  }
+  __syncthreads();
+  if (tid == 0) {
+    float s1 = 0.f, s2 = 0.f;
+    for (int k = 0; k < E; ++k) s1 += prod[k];
+    if (loss2)
+      for (int k = 0; k < E; ++k) s2 += prod[el + k];
+    gsum[g * 2] = s1;
+    gsum[g * 2 + 1] = s2;
+  }
+}
+
+__global__ void gate_loss_kernel(GateParams p, const float* __restrict__ gsum,
+                                 float* __restrict__ loss) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  float s1 = 0.f, s2 = 0.f;
+  for (int g = 0; g < p.G; ++g) { s1 += gsum[g * 2]; s2 += gsum[g * 2 + 1]; }
+  const float inv_ge = (float)(1.0 / ((double)p.G * (double)p.E));
+  const float ee = (float)((double)p.E * (double)p.E);
+  float l = (s1 * inv_ge) * ee;                              // moe.py:1423-1424
+  if (p.use_second_place_loss) l = l + ((s2 * inv_ge) * ee) * 0.5f;
+  if (p.num_microbatches > 1)
+    l = l * (float)(1.0 / (double)p.num_microbatches);       // moe.py:1439-1442
+  loss[0] = l;
+}
+
+static int gate_tokens_per_block(int E) {
+  if (E <= 128) return 256;
+  if (E <= 256) return 128;
+  return 64;
+}
+
+}  // namespace mesh_moe
+
+using namespace mesh_moe;
+
+extern "C" int mesh_moe_router_logits(const void* x, const void* w,
+                                      const float* bias, float* logits,
+                                      int batch, int64_t tokens, int M, int E,
+                                      int dtype, void* stream) {
+  MOE_REQUIRE(x && w && logits, MESH_MOE_E_ARG, "router_logits: null pointer");
+  MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG, "router_logits: bad dtype %d",
+              dtype);
+  MOE_REQUIRE(batch >= 1 && tokens >= 0 && M >= 1 && E >= 1, MESH_MOE_E_ARG,
+              "router_logits: bad sizes batch=%d tokens=%lld M=%d E=%d", batch,
+              (long long)tokens, M, E);
+  MOE_REQUIRE(E <= 4 * RL_MAX_EPT, MESH_MOE_E_UNSUPPORTED,
+              "router_logits: E=%d > %d", E, 4 * RL_MAX_EPT);
+  MOE_REQUIRE(batch <= 65535, MESH_MOE_E_UNSUPPORTED,
+              "router_logits: batch=%d > 65535", batch);
+  if (tokens == 0) return 0;
+  const int ept = (E + 3) / 4;
+  dim3 grid((unsigned)((tokens + RL_TOK - 1) / RL_TOK), (unsigned)batch);
+  size_t smem = sizeof(float) * (RL_TOK * (RL_KC + 1) + (size_t)RL_KC * E);
+  hipStream_t st = (hipStream_t)stream;
+  MOE_ALLOW_LDS(router_logits_kernel<float>, smem);
+  MOE_ALLOW_LDS(router_logits_kernel<bf16_t>, smem);
+  if (dtype == MESH_MOE_F32) {
+    router_logits_kernel<float><<<grid, 256, smem, st>>>(
+        (const float*)x, (const float*)w, bias, logits, tokens, M, E, ept);
+  } else {
+    router_logits_kernel<bf16_t><<<grid, 256, smem, st>>>(
+        (const bf16_t*)x, (const bf16_t*)w, bias, logits, tokens, M, E, ept);
+  }
+  MOE_CHECK_LAUNCH("router_logits");
+  return 0;
+}
+
+extern "C" size_t mesh_moe_gating_workspace_bytes(int G, int S, int E) {
+  if (G < 1 || S < 1 || E < 1) return 0;
+  const int tt = gate_tokens_per_block(E);
+  const size_t nblk = (size_t)(S + tt - 1) / tt;
+  return sizeof(float) * (2 * (size_t)G * nblk * E + 2 * (size_t)G) + 256;
+}
+
+extern "C" int mesh_moe_top2_gating(
+    const float* logits, const void* importance, int importance_dtype,
+    const float* second_uniform, int G, int S, int E, int C, int policy,
+    double threshold, int use_second_place_loss, int num_microbatches,
+    int32_t* idx, int32_t* pos, float* gate, uint8_t* kept, int32_t* fill,
+    float* loss, void* workspace, size_t workspace_bytes, void* stream) {
+  MOE_REQUIRE(logits && idx && pos && gate && kept && fill && loss && workspace,
+              MESH_MOE_E_ARG, "top2_gating: null pointer");
+  MOE_REQUIRE(G >= 1 && S >= 1 && C >= 1, MESH_MOE_E_ARG,
+              "top2_gating: bad sizes G=%d S=%d C=%d", G, S, C);
+  MOE_REQUIRE(E >= 2 && E <= 512, MESH_MOE_E_UNSUPPORTED,
+              "top2_gating: E=%d outside [2, 512]", E);
+  MOE_REQUIRE(S <= 16384, MESH_MOE_E_UNSUPPORTED,
+              "top2_gating: group size S=%d > 16384", S);
+  MOE_REQUIRE(G <= 65535, MESH_MOE_E_UNSUPPORTED, "top2_gating: G=%d > 65535",
+              G);
+  MOE_REQUIRE(policy >= MESH_MOE_SECOND_ALL && policy <= MESH_MOE_SECOND_RANDOM,
+              MESH_MOE_E_ARG, "top2_gating: unknown policy %d", policy);
+  MOE_REQUIRE(policy != MESH_MOE_SECOND_RANDOM || second_uniform,
+              MESH_MOE_E_ARG,
+              "top2_gating: policy RANDOM needs second_uniform samples");
+  MOE_REQUIRE(!importance || valid_dtype(importance_dtype), MESH_MOE_E_ARG,
+              "top2_gating: bad importance dtype %d", importance_dtype);
+  MOE_REQUIRE(workspace_bytes >= mesh_moe_gating_workspace_bytes(G, S, E),
+              MESH_MOE_E_ARG, "top2_gating: workspace too small (%zu < %zu)",
+              workspace_bytes, mesh_moe_gating_workspace_bytes(G, S, E));
+  GateParams p;
+  p.G = G; p.S = S; p.E = E; p.C = C;
+  p.policy = policy;
+  p.threshold = (float)threshold;
+  p.inv_threshold = (float)(1.0 / (threshold > 1e-9 ? threshold : 1e-9));
+  p.use_second_place_loss = use_second_place_loss ? 1 : 0;
+  p.num_microbatches = num_microbatches;
+  p.tt = gate_tokens_per_block(E);
+  p.nblk = (S + p.tt - 1) / p.tt;
+  hipStream_t st = (hipStream_t)stream;
+  uintptr_t wsp = ((uintptr_t)workspace + 255) & ~(uintptr_t)255;
+  float* part1 = (float*)wsp;
+  float* part2 = part1 + (size_t)G * p.nblk * E;
+  float* gsum = part2 + (size_t)G * p.nblk * E;
+
+  {
+    dim3 grid((unsigned)p.nblk, (unsigned)G);
+    size_t smem = sizeof(float) * ((size_t)p.tt * (E + 1) + p.tt);
+    if (importance && importance_dtype == MESH_MOE_BF16) {
+      auto k = gate_select_kernel<bf16_t>;
+      MOE_ALLOW_LDS(k, smem);
+      k<<<grid, p.tt, smem, st>>>(logits, (const bf16_t*)importance,
+                                  second_uniform, p, idx, pos, gate, kept,
+                                  part1, part2);
+    } else {
+      auto k = gate_select_kernel<float>;
+      MOE_ALLOW_LDS(k, smem);
+      k<<<grid, p.tt, smem, st>>>(logits, (const float*)importance,
+                                  second_uniform, p, idx, pos, gate, kept,
+                                  part1, part2);
+    }
+    MOE_CHECK_LAUNCH("gate_select");
+  }
+  {
+    int el = 2;
+    while (el < E) el *= 2;
+    size_t smem = sizeof(int32_t) * (CAP_THREADS + 3 * (size_t)el) +
+                  sizeof(float) * 2 * (size_t)el +
+                  sizeof(int16_t) * 3 * (size_t)S;
+    MOE_ALLOW_LDS(gate_capacity_kernel, smem);
+    gate_capacity_kernel<<<G, CAP_THREADS, smem, st>>>(
+        p, idx, pos, gate, kept, fill, part1, part2, gsum, el);
+    MOE_CHECK_LAUNCH("gate_capacity");
+  }
+  gate_loss_kernel<<<1, 64, 0, st>>>(p, gsum, loss);
+  MOE_CHECK_LAUNCH("gate_loss");
+  return 0;
+}

@@ -1,0 +1,259 @@
+"""ctypes binding of libmesh_moe_hip.so (declared in include/mesh_moe.h).
+
+The functions here take torch tensors that live on the GPU, check shapes and
+dtypes on the host (a kernel launched on mismatched shapes faults the device),
+and pass raw device pointers plus the current HIP stream through the C ABI.
+torch is used for device memory and streams only.
+
+There is no CPU fallback: if the shared library has not been built, loading
+raises, and so does every call.
+"""
+
+import ctypes
+import os
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(_HERE, "csrc", "libmesh_moe_hip.so")
+
+F32 = 0
+BF16 = 1
+POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
+ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
+               "tanh": 4, "swish": 5}
+ABI_VERSION = 1
+
+_vp = ctypes.c_void_p
+_SIGNATURES = {
+    "mesh_moe_abi_version": (ctypes.c_int, []),
+    "mesh_moe_last_error": (ctypes.c_char_p, []),
+    "mesh_moe_router_logits": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, _vp]),
+    "mesh_moe_gating_workspace_bytes": (ctypes.c_size_t, [
+        ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "mesh_moe_top2_gating": (ctypes.c_int, [
+        _vp, _vp, ctypes.c_int, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_double, ctypes.c_int,
+        ctypes.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_size_t,
+        _vp]),
+    "mesh_moe_dispatch": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
+    "mesh_moe_pack_weights": (ctypes.c_int, [
+        _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, _vp]),
+    "mesh_moe_expert_ffn": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
+    "mesh_moe_combine": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
+}
+EXPORTS = sorted(_SIGNATURES)
+
+_lib = None
+
+
+class MoeHipError(RuntimeError):
+  """A call into libmesh_moe_hip.so was rejected."""
+
+
+def load_library(path=None):
+  """Loads the shared library (once) and declares every entry point."""
+  global _lib
+  if _lib is not None and path is None:
+    return _lib
+  path = path or LIB_PATH
+  if not os.path.exists(path):
+    raise MoeHipError(
+        "%s not found: build it with `python -m mesh_amd.csrc.build` "
+        "(there is no CPU fallback)" % path)
+  lib = ctypes.CDLL(path)
+  for name, (restype, argtypes) in _SIGNATURES.items():
+    fn = getattr(lib, name)  # AttributeError if a symbol is missing
+    fn.restype = restype
+    fn.argtypes = argtypes
+  version = lib.mesh_moe_abi_version()
+  if version != ABI_VERSION:
+    raise MoeHipError("ABI version %d, expected %d" % (version, ABI_VERSION))
+  _lib = lib
+  return lib
+
+
+def _check(rc, what):
+  if rc != 0:
+    msg = load_library().mesh_moe_last_error().decode("utf-8", "replace")
+    raise MoeHipError("%s failed (%d): %s" % (what, rc, msg))
+
+
+def dtype_code(dtype):
+  if dtype == torch.float32:
+    return F32
+  if dtype == torch.bfloat16:
+    return BF16
+  raise MoeHipError("unsupported dtype %s (float32 and bfloat16 only)" % dtype)
+
+
+def _dev(t, name, dtype=None, shape=None):
+  if not isinstance(t, torch.Tensor) or not t.is_cuda:
+    raise MoeHipError("%s must be a GPU tensor" % name)
+  if not t.is_contiguous():
+    raise MoeHipError("%s must be contiguous" % name)
+  if dtype is not None and t.dtype != dtype:
+    raise MoeHipError("%s: dtype %s, expected %s" % (name, t.dtype, dtype))
+  if shape is not None and tuple(t.shape) != tuple(shape):
+    raise MoeHipError("%s: shape %s, expected %s"
+                      % (name, tuple(t.shape), tuple(shape)))
+  return t.data_ptr()
+
+
+def _stream():
+  return torch.cuda.current_stream().cuda_stream
+
+
+def router_logits(x, w, bias=None, out=None):
+  """x [B, T, M] or [T, M]; w [B, M, E] or [M, E] -> float32 logits [.., T, E]."""
+  lib = load_library()
+  squeeze = x.dim() == 2
+  if squeeze:
+    x, w = x.unsqueeze(0), w.unsqueeze(0)
+  b, t, m = x.shape
+  e = w.shape[-1]
+  code = dtype_code(x.dtype)
+  xp = _dev(x, "x")
+  wp = _dev(w, "w", x.dtype, (b, m, e))
+  if out is None:
+    out = torch.empty((b, t, e), dtype=torch.float32, device=x.device)
+  op = _dev(out, "logits", torch.float32, (b, t, e))
+  bp = None if bias is None else _dev(bias, "bias", torch.float32, (e,))
+  _check(lib.mesh_moe_router_logits(xp, wp, bp, op, b, t, m, e, code,
+                                    _stream()), "router_logits")
+  return out[0] if squeeze else out
+
+
+class Routing(object):
+  """Per-token routing record written by top2_gating."""
+
+  def __init__(self, idx, pos, gate, kept, fill, loss, capacity, num_experts):
+    self.idx, self.pos, self.gate, self.kept = idx, pos, gate, kept
+    self.fill, self.loss = fill, loss
+    self.capacity, self.num_experts = capacity, num_experts
+
+
+def top2_gating(logits, capacity, importance=None, policy="all",
+                threshold=0.2, use_second_place_loss=False,
+                num_microbatches=None, second_uniform=None):
+  """logits float32 [G, S, E] -> Routing (all tensors on the GPU)."""
+  lib = load_library()
+  if policy not in POLICIES:
+    raise ValueError("Unknown policy %s" % policy)
+  g, s, e = logits.shape
+  lp = _dev(logits, "logits", torch.float32)
+  dev = logits.device
+  ip, icode = None, F32
+  if importance is not None:
+    icode = dtype_code(importance.dtype)
+    ip = _dev(importance, "importance", None, (g, s))
+  up = None
+  if second_uniform is not None:
+    up = _dev(second_uniform, "second_uniform", torch.float32, (g, s))
+  idx = torch.empty((g, s, 2), dtype=torch.int32, device=dev)
+  pos = torch.empty((g, s, 2), dtype=torch.int32, device=dev)
+  gate = torch.empty((g, s, 2), dtype=torch.float32, device=dev)
+  kept = torch.empty((g, s, 2), dtype=torch.uint8, device=dev)
+  fill = torch.empty((g, e), dtype=torch.int32, device=dev)
+  loss = torch.empty((1,), dtype=torch.float32, device=dev)
+  ws_bytes = lib.mesh_moe_gating_workspace_bytes(g, s, e)
+  ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
+  _check(lib.mesh_moe_top2_gating(
+      lp, ip, icode, up, g, s, e, int(capacity), POLICIES[policy],
+      float(threshold), int(bool(use_second_place_loss)),
+      int(num_microbatches or 1), idx.data_ptr(), pos.data_ptr(),
+      gate.data_ptr(), kept.data_ptr(), fill.data_ptr(), loss.data_ptr(),
+      ws.data_ptr(), ws_bytes, _stream()), "top2_gating")
+  return Routing(idx, pos, gate, kept, fill, loss, int(capacity), e)
+
+
+def dispatch(x, r, want_slot_gate=False, out=None):
+  """x [G, S, M] -> expert_in [E, G, C, M] (and slot_gate [E, G, C])."""
+  lib = load_library()
+  g, s, m = x.shape
+  e, c = r.num_experts, r.capacity
+  code = dtype_code(x.dtype)
+  xp = _dev(x, "x")
+  if out is None:
+    out = torch.empty((e, g, c, m), dtype=x.dtype, device=x.device)
+  op = _dev(out, "expert_in", x.dtype, (e, g, c, m))
+  slot_gate = None
+  if want_slot_gate:
+    slot_gate = torch.empty((e, g, c), dtype=torch.float32, device=x.device)
+  _check(lib.mesh_moe_dispatch(
+      xp, _dev(r.idx, "idx", torch.int32, (g, s, 2)),
+      _dev(r.pos, "pos", torch.int32, (g, s, 2)),
+      _dev(r.gate, "gate", torch.float32, (g, s, 2)),
+      _dev(r.kept, "kept", torch.uint8, (g, s, 2)),
+      _dev(r.fill, "fill", torch.int32, (g, e)), op,
+      None if slot_gate is None else slot_gate.data_ptr(),
+      g, s, e, c, m, code, _stream()), "dispatch")
+  return (out, slot_gate) if want_slot_gate else out
+
+
+def pack_weights(w, dtype):
+  """w [E, K, N] (any supported dtype) -> packed [E, N, K] of `dtype`."""
+  lib = load_library()
+  e, k, n = w.shape
+  out = torch.empty((e, n, k), dtype=dtype, device=w.device)
+  _check(lib.mesh_moe_pack_weights(
+      _dev(w, "w"), out.data_ptr(), e, k, n, dtype_code(w.dtype),
+      dtype_code(dtype), _stream()), "pack_weights")
+  return out
+
+
+def expert_ffn(expert_in, wi_packed, wo_packed, activation="relu", h=None,
+               y=None):
+  """expert_in [E, R, M]; wi_packed [E, H, M]; wo_packed [E, N, H] -> y [E,R,N]."""
+  lib = load_library()
+  if activation not in ACTIVATIONS:
+    raise ValueError("unsupported expert activation %r" % (activation,))
+  e, rows, m = expert_in.shape
+  hdim = wi_packed.shape[1]
+  n = wo_packed.shape[1]
+  dt = expert_in.dtype
+  code = dtype_code(dt)
+  ip = _dev(expert_in, "expert_in")
+  wip = _dev(wi_packed, "wi_packed", dt, (e, hdim, m))
+  wop = _dev(wo_packed, "wo_packed", dt, (e, n, hdim))
+  if h is None:
+    h = torch.empty((e, rows, hdim), dtype=dt, device=expert_in.device)
+  if y is None:
+    y = torch.empty((e, rows, n), dtype=dt, device=expert_in.device)
+  hp = _dev(h, "h", dt, (e, rows, hdim))
+  yp = _dev(y, "y", dt, (e, rows, n))
+  _check(lib.mesh_moe_expert_ffn(ip, wip, wop, hp, yp, e, rows, m, hdim, n,
+                                 ACTIVATIONS[activation], code, _stream()),
+         "expert_ffn")
+  return y
+
+
+def combine(y, r, group_size, out=None):
+  """y [E, G, C, N] -> out [G, S, N]."""
+  lib = load_library()
+  e, g, c, n = y.shape
+  s = group_size
+  code = dtype_code(y.dtype)
+  yp = _dev(y, "y")
+  if (e, c) != (r.num_experts, r.capacity):
+    raise MoeHipError("combine: y is [E=%d, C=%d], routing has E=%d, C=%d"
+                      % (e, c, r.num_experts, r.capacity))
+  if out is None:
+    out = torch.empty((g, s, n), dtype=y.dtype, device=y.device)
+  op = _dev(out, "out", y.dtype, (g, s, n))
+  _check(lib.mesh_moe_combine(
+      yp, _dev(r.idx, "idx", torch.int32, (g, s, 2)),
+      _dev(r.pos, "pos", torch.int32, (g, s, 2)),
+      _dev(r.gate, "gate", torch.float32, (g, s, 2)),
+      _dev(r.kept, "kept", torch.uint8, (g, s, 2)), op, g, s, e, c, n, code,
+      _stream()), "combine")
+  return out

@@ -1,0 +1,598 @@
+"""CPU restatement of Mesh TensorFlow's top-2 Mixture-of-Experts forward path.
+
+TEST INFRASTRUCTURE ONLY -- never imported by the product package.
+
+Every function restates, in NumPy float32 arithmetic with one rounding per
+reference op, what the reference's single-device lowering computes.  The
+reference builds the layer from ~100 separately lowered primitives; each line
+below that performs arithmetic corresponds to one of those primitives, so the
+rounding points are the reference's.
+
+What pins each function (the reference holds no test or golden vector of its
+MoE file, and its TensorFlow dependency cannot run here):
+
+  split_into_groups, expert_capacity  brute force over the defining
+                                      constraints + the five config capacities
+  softmax                             float64 scipy softmax, row-sum invariant
+  top_1 / top-2 selection             stable argsort brute force, exact ties
+  capacity positions / drops          sequential integer loop
+                                      (routing_sequential) + a hand-worked case
+  combine / dispatch tensors          rebuilt from (idx, pos, gate, kept)
+  dispatch / combine einsums          gather/scatter form vs np.einsum
+  expert FFN                          float64 matmul
+  aux loss                            balanced-routing closed form (= 1.0)
+  v2                                  x=1 outer expert reduces to v1
+
+PARITY UNPINNED against TensorFlow itself (only running the reference could
+pin these): near-tie behaviour of argmax after TF's exp/log, the accumulation
+order of TF's bf16 einsum, and the "random" second-place policy's RNG stream.
+
+Citations are to files under the reference tree (mesh_tensorflow/...).
+"""
+
+import numpy as np
+
+F32 = np.float32
+
+
+# ----------------------------------------------------------------------------
+# dtype helpers
+# ----------------------------------------------------------------------------
+def round_bf16(a):
+  """float32 -> bfloat16 (round to nearest even) -> float32.
+
+  Stands in for tf.cast(x, tf.bfloat16) (ops.py:1945-1951).
+  """
+  shape = np.shape(a)
+  a = np.ascontiguousarray(a, dtype=F32).reshape(-1)
+  u = a.view(np.uint32)
+  nan = np.isnan(a)
+  rounded = (u + (np.uint32(0x7FFF) + ((u >> np.uint32(16)) & np.uint32(1))))
+  rounded = rounded & np.uint32(0xFFFF0000)
+  out = rounded.view(F32).copy()
+  if nan.any():
+    out[nan] = np.nan
+  return out.reshape(shape)
+
+
+def cast_act(a, act_dtype):
+  """tf.cast to the activation dtype ("float32" or "bfloat16")."""
+  if act_dtype == "bfloat16":
+    return round_bf16(a)
+  if act_dtype == "float32":
+    return np.asarray(a, dtype=F32)
+  raise ValueError("unsupported activation dtype %r" % (act_dtype,))
+
+
+# ----------------------------------------------------------------------------
+# host integer logic
+# ----------------------------------------------------------------------------
+def split_into_groups(n, max_group_size, mesh_dim_size):
+  """transformer/moe.py:1549-1582."""
+  if n % mesh_dim_size != 0:
+    raise ValueError(
+        "n=%d is not a multiple of mesh_dim_size=%d" % (n, mesh_dim_size))
+  num_groups = max(1, n // max_group_size)
+  while num_groups % mesh_dim_size != 0 or n % num_groups != 0:
+    num_groups += 1
+  return num_groups, n // num_groups
+
+
+def expert_capacity(group_size, capacity_factor, num_experts,
+                    min_expert_capacity):
+  """transformer/moe.py:368-371 (v2: :671-672, :686-689)."""
+  c = min(group_size, int((group_size * capacity_factor) / num_experts))
+  return max(c, min_expert_capacity)
+
+
+# ----------------------------------------------------------------------------
+# mtf primitives, restated
+# ----------------------------------------------------------------------------
+def seq_sum(x, axis=-1):
+  """Sequential float32 sum in index order (the order tf.reduce_sum uses is
+  Eigen's and is not specified; this is the order the HIP kernels use)."""
+  x = np.asarray(x, dtype=F32)
+  return np.add.accumulate(x, axis=axis, dtype=F32).take(-1, axis=axis)
+
+
+def softmax(x):
+  """mtf.softmax over the last axis: exp(x - logsumexp(x)).
+
+  ops.py:5539-5541 -> log_softmax :5523-5536 -> reduce_logsumexp :5493-5520.
+  Subtraction is add(x, negative(y)) (ops.py:5116-5132).
+  """
+  x = np.asarray(x, dtype=F32)
+  m = x.max(axis=-1, keepdims=True)                      # reduce_max
+  t = x + (-m)                                           # x -= max_logit
+  u = np.exp(t).astype(F32)                              # exp
+  s = seq_sum(u, axis=-1)[..., None]                     # reduce_sum
+  lse = np.log(s).astype(F32) + m                        # log(...) + max_logit
+  return np.exp(x + (-lse)).astype(F32)                  # exp(log_softmax)
+
+
+def top_1(x):
+  """mtf.top_1 over the last axis: (reduce_max, int32 first argmax).
+
+  ops.py:5018-5033 -> TopKOperation k=1 branch ops.py:4937-4940.
+  """
+  return x.max(axis=-1), np.argmax(x, axis=-1).astype(np.int32)
+
+
+def one_hot(idx, depth):
+  """tf.one_hot semantics: an out-of-range index gives an all-zero row
+  (ops.py:3830-3851)."""
+  idx = np.asarray(idx)
+  return (idx[..., None] == np.arange(depth, dtype=idx.dtype)).astype(F32)
+
+
+def cumsum_exclusive(x, dense=False):
+  """mtf.cumsum(x, group_size_dim, exclusive=True) for x of shape [..., S, E].
+
+  ops.py:2761-2781 implements it as an einsum with an S x S triangular 0/1
+  matrix.  With dense=True that matmul is performed literally (used for the CPU
+  baseline timing and on tiny cases); otherwise np.cumsum is used, which gives
+  identical values because every partial sum is an integer below 2**24.
+  """
+  x = np.asarray(x, dtype=F32)
+  s = x.shape[-2]
+  if dense:
+    r = np.arange(s, dtype=F32)
+    tri = (r[:, None] < r[None, :]).astype(F32)          # [s, s'] = s < s'
+    return np.einsum("...se,st->...te", x, tri).astype(F32)
+  return (np.cumsum(x, axis=-2, dtype=F32) - x).astype(F32)
+
+
+# ----------------------------------------------------------------------------
+# _top_2_gating  (transformer/moe.py:1312-1513)
+# ----------------------------------------------------------------------------
+def top_2_gating(logits, capacity, importance=None, policy="all",
+                 threshold=0.2, use_second_place_loss=False,
+                 num_microbatches=None, act_dtype="float32",
+                 second_uniform=None, dense=False):
+  """Everything in _top_2_gating after the router projection.
+
+  Args:
+    logits: float32 [G, S, E] router logits (output of the `dense` at
+      moe.py:1386-1390; leading dims may be flattened into G).
+    capacity: int, expert_capacity_dim.size.
+    importance: optional float [G, S].
+    policy, threshold: moe_second_policy_* / moe_second_threshold_*.
+    second_uniform: U(0,1) samples [G, S] for policy "random" (the reference
+      draws them with mtf.random_uniform, moe.py:1464).
+    dense: build the dense [G,S,E,C] tensors and use the S x S cumsum matmul.
+
+  Returns a dict with
+    combine, dispatch: [G,S,E,C] in the activation dtype (only if dense),
+    loss: float32 scalar cast to the activation dtype (moe.py:1508),
+    index_1/2 int32 [G,S], pos_1/2 int32 [G,S] (raw, meaningful where kept),
+    kept_1/2 bool [G,S] (mask_k_flat), gate_1/2 float32 [G,S] (after the
+    multiplication by mask_k_flat, before the activation-dtype cast),
+    fill int32 [G,E] occupied slots per expert.
+  """
+  logits = np.asarray(logits, dtype=F32)
+  g_, s_, e_ = logits.shape
+  cap_f = F32(float(capacity))
+
+  raw_gates = softmax(logits)                                    # :1391
+  gate_1, index_1 = top_1(raw_gates)                             # :1397
+  mask_1 = one_hot(index_1, e_)                                  # :1399
+  density_1_proxy = raw_gates                                    # :1400
+  if importance is not None:
+    importance = np.asarray(importance, dtype=F32)
+    is_one = (importance == F32(1.0)).astype(F32)                # :1402-1404
+    mask_1 = mask_1 * is_one[..., None]
+    gate_1 = gate_1 * is_one
+    density_1_proxy = density_1_proxy * is_one[..., None]
+  gates_without_top_1 = raw_gates * (F32(1.0) + (-mask_1))       # :1405
+  gate_2, index_2 = top_1(gates_without_top_1)                   # :1407
+  mask_2 = one_hot(index_2, e_)                                  # :1409
+  if importance is not None:
+    mask_2 = mask_2 * (importance > F32(0.0)).astype(F32)[..., None]  # :1411
+
+  denom = (gate_1 + gate_2) + F32(1e-9)                          # :1413
+  recip = (F32(1.0) / denom).astype(F32)                         # reciprocal
+  gate_1 = gate_1 * recip                                        # :1414
+  gate_2 = gate_2 * recip                                        # :1415
+
+  # balancing loss (:1420-1442); reduce_mean = reduce_sum * (out/in), the
+  # Python quotient becoming a float32 scalar (ops.py:4804-4808).
+  inv_s = F32(1.0 / s_)
+  density_1 = seq_sum(mask_1, axis=-2) * inv_s                   # [G,E]
+  density_1_proxy = seq_sum(density_1_proxy, axis=-2) * inv_s    # [G,E]
+  prod = density_1_proxy * density_1
+  loss = seq_sum(prod.reshape(-1)) * F32(1.0 / prod.size)
+  loss = loss * F32(float(e_ * e_))
+  if use_second_place_loss:                                      # :1426-1438
+    density_2 = seq_sum(mask_2, axis=-2) * inv_s
+    qsum = seq_sum(gates_without_top_1, axis=-1) + F32(1e-9)
+    normalized = gates_without_top_1 * (F32(1.0) / qsum).astype(F32)[..., None]
+    density_2_proxy = seq_sum(normalized, axis=-2) * inv_s
+    prod2 = density_2_proxy * density_2
+    loss_2 = seq_sum(prod2.reshape(-1)) * F32(1.0 / prod2.size)
+    loss_2 = loss_2 * F32(float(e_ * e_))
+    loss = loss + loss_2 * F32(0.5)
+  if num_microbatches and num_microbatches > 1:                  # :1439-1442
+    loss = loss * F32(1.0 / num_microbatches)
+
+  if policy == "all":                                            # :1452-1467
+    pass
+  elif policy == "none":
+    mask_2 = np.zeros_like(mask_2)
+  elif policy == "threshold":
+    mask_2 = mask_2 * (gate_2 > F32(threshold)).astype(F32)[..., None]
+  elif policy == "random":
+    if second_uniform is None:
+      raise ValueError("policy 'random' needs second_uniform samples")
+    u = np.asarray(second_uniform, dtype=F32)
+    lim = gate_2 * F32(1.0 / max(threshold, 1e-9))
+    mask_2 = mask_2 * (u < lim).astype(F32)[..., None]
+  else:
+    raise ValueError("Unknown policy %s" % policy)
+
+  # capacity assignment (:1472-1496)
+  position_in_expert_1 = cumsum_exclusive(mask_1, dense) * mask_1
+  mask_1 = mask_1 * (position_in_expert_1 < cap_f).astype(F32)
+  mask_1_count = seq_sum(mask_1, axis=-2)                        # [G,E]
+  mask_1_flat = seq_sum(mask_1, axis=-1)                         # [G,S]
+  position_in_expert_1 = seq_sum(position_in_expert_1, axis=-1)
+  gate_1 = gate_1 * mask_1_flat
+
+  position_in_expert_2 = (
+      cumsum_exclusive(mask_2, dense) + mask_1_count[:, None, :])
+  position_in_expert_2 = position_in_expert_2 * mask_2
+  mask_2 = mask_2 * (position_in_expert_2 < cap_f).astype(F32)
+  mask_2_flat = seq_sum(mask_2, axis=-1)
+  gate_2 = gate_2 * mask_2_flat
+  position_in_expert_2 = seq_sum(position_in_expert_2, axis=-1)
+
+  pos_1 = position_in_expert_1.astype(np.int32)                  # to_int32
+  pos_2 = position_in_expert_2.astype(np.int32)
+  out = dict(
+      index_1=index_1, index_2=index_2, pos_1=pos_1, pos_2=pos_2,
+      kept_1=mask_1_flat > 0, kept_2=mask_2_flat > 0,
+      gate_1=gate_1, gate_2=gate_2,
+      fill=(mask_1_count + seq_sum(mask_2, axis=-2)).astype(np.int32),
+      loss=cast_act(loss, act_dtype)[()])                        # :1508
+  if dense:
+    combine = (                                                  # :1499-1505
+        (gate_1 * mask_1_flat)[..., None, None]
+        * one_hot(index_1, e_)[..., None]
+        * one_hot(pos_1, capacity)[..., None, :]
+        + (gate_2 * mask_2_flat)[..., None, None]
+        * one_hot(index_2, e_)[..., None]
+        * one_hot(pos_2, capacity)[..., None, :])
+    combine = cast_act(combine, act_dtype)                       # :1507
+    out["combine"] = combine
+    out["dispatch"] = (combine != 0).astype(F32)                 # :1510-1511
+  return out
+
+
+def routing_sequential(index_1, index_2, sel_1, sel_2, num_experts, capacity):
+  """Integer brute force for moe.py:1472-1496, one token at a time.
+
+  sel_k[g, s] says whether token s enters the k-th choice competition (mask_k
+  before capacity).  Per group: first choices claim slots in token order; a
+  first choice whose running count has reached `capacity` is dropped; second
+  choices then claim slots starting from the kept first-choice count, and the
+  running second-choice counter advances for every selected second choice,
+  kept or not.
+
+  Returns pos_1, kept_1, pos_2, kept_2, fill ([G,E] occupied slots).
+  """
+  g_, s_ = index_1.shape
+  pos_1 = np.zeros((g_, s_), np.int32)
+  pos_2 = np.zeros((g_, s_), np.int32)
+  kept_1 = np.zeros((g_, s_), bool)
+  kept_2 = np.zeros((g_, s_), bool)
+  fill = np.zeros((g_, num_experts), np.int32)
+  for g in range(g_):
+    seen = [0] * num_experts
+    for s in range(s_):
+      if sel_1[g, s]:
+        e = int(index_1[g, s])
+        pos_1[g, s] = seen[e]
+        kept_1[g, s] = seen[e] < capacity
+        seen[e] += 1
+    count_1 = [min(c, capacity) for c in seen]
+    seen2 = [0] * num_experts
+    kept2_count = [0] * num_experts
+    for s in range(s_):
+      if sel_2[g, s]:
+        e = int(index_2[g, s])
+        p = seen2[e] + count_1[e]
+        pos_2[g, s] = p
+        kept_2[g, s] = p < capacity
+        kept2_count[e] += int(p < capacity)
+        seen2[e] += 1
+    for e in range(num_experts):
+      fill[g, e] = count_1[e] + kept2_count[e]
+  return pos_1, kept_1, pos_2, kept_2, fill
+
+
+# ----------------------------------------------------------------------------
+# index-form dispatch / combine (what the HIP kernels compute)
+# ----------------------------------------------------------------------------
+def combine_weights(r, act_dtype):
+  """The two per-token combine weights as the dense tensor holds them: gate_k
+  (already multiplied by mask_k_flat) cast to the activation dtype
+  (moe.py:1499-1507)."""
+  return cast_act(r["gate_1"], act_dtype), cast_act(r["gate_2"], act_dtype)
+
+
+def dispatch_gather(x, r, num_experts, capacity, act_dtype):
+  """expert_in[e, g, c, :] from the routing record; equals the dense einsum at
+  moe.py:443-447 because each slot receives at most one token.  A kept choice
+  whose activation-dtype gate is exactly zero is not dispatched
+  (moe.py:1510-1511)."""
+  g_, s_, m_ = x.shape
+  w1, w2 = combine_weights(r, act_dtype)
+  out = np.zeros((num_experts, g_, capacity, m_), F32)
+  for k, w in (("1", w1), ("2", w2)):
+    sel = r["kept_" + k] & (w != 0)
+    gi, si = np.nonzero(sel)
+    out[r["index_" + k][gi, si], gi, r["pos_" + k][gi, si]] = x[gi, si]
+  return out
+
+
+def combine_gather(y, r, act_dtype):
+  """out[g, s, :] = w1 * y[idx1, g, pos1] + w2 * y[idx2, g, pos2]
+  (moe.py:509-510 with at most two non-zero terms), float32 accumulate, one
+  rounding to the activation dtype."""
+  e_, g_, c_, n_ = y.shape
+  w1, w2 = combine_weights(r, act_dtype)
+  s_ = w1.shape[1]
+  out = np.zeros((g_, s_, n_), F32)
+  for k, w in (("1", w1), ("2", w2)):
+    sel = r["kept_" + k] & (w != 0)
+    gi, si = np.nonzero(sel)
+    out[gi, si] += (w[gi, si][:, None]
+                    * y[r["index_" + k][gi, si], gi, r["pos_" + k][gi, si]])
+  return cast_act(out, act_dtype)
+
+
+# ----------------------------------------------------------------------------
+# activations (ops.py:1818-1921)
+# ----------------------------------------------------------------------------
+def _gelu(x):
+  # ops.py:1862-1874: 0.5 * x * (1 + tanh(sqrt(2/pi) * (x + 0.044715 x^3)))
+  x = x.astype(F32)
+  cdf = F32(0.5) * (F32(1.0) + np.tanh(
+      F32(np.sqrt(2 / np.pi)) * (x + F32(0.044715) * x * x * x)).astype(F32))
+  return x * cdf
+
+
+ACTIVATIONS = {
+    "relu": lambda x: np.maximum(x, F32(0)),
+    "linear": lambda x: x,
+    None: lambda x: x,
+    "gelu": _gelu,
+    "sigmoid": lambda x: (F32(1) / (F32(1) + np.exp(-x))).astype(F32),
+    "tanh": lambda x: np.tanh(x).astype(F32),
+    "swish": lambda x: (x / (F32(1) + np.exp(-x))).astype(F32),
+}
+
+
+# ----------------------------------------------------------------------------
+# the layers
+# ----------------------------------------------------------------------------
+class HParams(object):
+  """Attribute bag (transformer/moe.py:1585-1596)."""
+
+  def __init__(self, **kwargs):
+    for k, v in kwargs.items():
+      setattr(self, k, v)
+
+
+def default_hparams(**overrides):
+  hp = dict(
+      moe_gating="top_2", moe_num_experts=16, moe_loss_coef=1e-2,
+      moe_hidden_size=4096, moe_group_size=1024, moe_min_expert_capacity=4,
+      moe_capacity_factor_train=1.25, moe_capacity_factor_eval=2.0,
+      moe_capacity_factor_second_level=1.0,
+      moe_use_second_place_loss=False,
+      moe_second_policy_train="random", moe_second_policy_eval="random",
+      moe_second_threshold_train=0.2, moe_second_threshold_eval=0.2,
+      moe_dropout_rate=0.0, moe_use_experts_attention=False)
+  hp.update(overrides)
+  return HParams(**hp)
+
+
+def router_logits(x, w):
+  """raw_gates = dense(to_float(inputs), experts_dim, use_bias=False)
+  (moe.py:1384-1390; layers.py:129-208, einsum in float32).  x [..., M] and
+  w [M, E] already hold activation-dtype-rounded values (ops.py:4046-4047,
+  layers.py:252)."""
+  return np.matmul(x.astype(F32), w.astype(F32)).astype(F32)
+
+
+def _policy(hp, train):
+  if train:
+    return hp.moe_second_policy_train, hp.moe_second_threshold_train
+  return hp.moe_second_policy_eval, hp.moe_second_threshold_eval
+
+
+def _scale_loss(loss, coef, act_dtype):
+  """`loss * hparams.moe_loss_coef` on an activation-dtype scalar
+  (moe.py:525; ScalarMultiplyOperation ops.py:2006-2023)."""
+  return cast_act(cast_act(loss, act_dtype) * cast_act(F32(coef), act_dtype),
+                  act_dtype)[()]
+
+
+def expert_ffn(expert_in, wi, wo, activation, act_dtype):
+  """h = act(expert_in . wi), y = h . wo per expert (moe.py:469-486).
+  expert_in [E, R, M], wi [E, M, H], wo [E, H, N]; float32 accumulate, results
+  rounded to the activation dtype."""
+  act = ACTIVATIONS[activation]
+  h = cast_act(np.matmul(expert_in, wi), act_dtype)
+  h = cast_act(act(h), act_dtype)
+  return cast_act(np.matmul(h, wo), act_dtype)
+
+
+def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
+                 nonpadding=None, activation="relu", num_microbatches=None,
+                 logit_bias=None, second_uniform=None, dense=True,
+                 mesh_dim_size=1):
+  """transformer_moe_layer_v1 forward (transformer/moe.py:191-525).
+
+  x: [batch..., length, M] float32 array holding activation-dtype values.
+  w_gate [M, E], wi [E, M, H], wo [E, H, N]: master (float32) weights; they are
+  cast to the activation dtype as Variable.lower does (ops.py:4046-4047).
+  logit_bias: optional [E] added to the router logits (benchmark-only hook for
+  the skewed-routing config; the reference router has no bias).
+  dense=True follows the reference dataflow literally (one-hot [G,S,E,C]
+  tensors, einsums); dense=False uses the index form.
+
+  Returns (output [batch..., length, N], loss scalar, aux dict).
+  """
+  if hp.moe_gating != "top_2":
+    raise ValueError("unknown hparams.moe_gating=%s" % hp.moe_gating)
+  x = cast_act(x, act_dtype)
+  lead = x.shape[:-1]
+  m_ = x.shape[-1]
+  n_tok = int(np.prod(lead))
+  e_ = hp.moe_num_experts
+  g_, s_ = split_into_groups(n_tok, hp.moe_group_size, mesh_dim_size)
+  cf = hp.moe_capacity_factor_train if train else hp.moe_capacity_factor_eval
+  c_ = expert_capacity(s_, cf, e_, hp.moe_min_expert_capacity)
+  xg = x.reshape(g_, s_, m_)                                     # :359-361
+  importance = None
+  if nonpadding is not None:                                     # :376-379
+    importance = cast_act(np.broadcast_to(nonpadding, lead), act_dtype)
+    importance = importance.reshape(g_, s_)
+  wg = cast_act(w_gate, act_dtype)
+  logits = router_logits(xg, wg)
+  if logit_bias is not None:
+    logits = logits + np.asarray(logit_bias, F32)
+  policy, threshold = _policy(hp, train)
+  r = top_2_gating(logits, c_, importance, policy, threshold,
+                   hp.moe_use_second_place_loss, num_microbatches, act_dtype,
+                   second_uniform, dense=dense)
+  wi_a = cast_act(wi, act_dtype)
+  wo_a = cast_act(wo, act_dtype)
+  if dense:
+    disp = r["dispatch"].reshape(g_, s_, e_ * c_)
+    expert_in = np.matmul(disp.transpose(0, 2, 1), xg)           # [G, EC, M]
+    expert_in = cast_act(expert_in, act_dtype).reshape(g_, e_, c_, m_)
+    expert_in = expert_in.transpose(1, 0, 2, 3)                  # [E,G,C,M]
+  else:
+    expert_in = dispatch_gather(xg, r, e_, c_, act_dtype)
+  y = expert_ffn(expert_in.reshape(e_, g_ * c_, m_), wi_a, wo_a, activation,
+                 act_dtype)
+  n_ = y.shape[-1]
+  y = y.reshape(e_, g_, c_, n_)
+  if dense:
+    comb = r["combine"].reshape(g_, s_, e_ * c_)
+    yg = y.transpose(1, 0, 2, 3).reshape(g_, e_ * c_, n_)
+    out = cast_act(np.matmul(comb, yg), act_dtype)               # :509-510
+  else:
+    out = combine_gather(y, r, act_dtype)
+  aux = dict(r, logits=logits, expert_in=expert_in, expert_out=y,
+             num_groups=g_, group_size=s_, capacity=c_)
+  return (out.reshape(lead + (n_,)),
+          _scale_loss(r["loss"], hp.moe_loss_coef, act_dtype), aux)
+
+
+def moe_layer_v2(x, w_outer, w_inner, wi, wo, hp, train, act_dtype="float32",
+                 nonpadding=None, num_microbatches=None, second_uniform=None,
+                 dense=True, mesh_dim_size=1):
+  """transformer_moe_layer_v2 forward (transformer/moe.py:528-801).
+
+  x: [a0?, b1, l, M]; w_outer [M, X]; w_inner [X, M, Y];
+  wi [Y, X, M, H]; wo [Y, X, H, N] (moe.py:702-712, :743-753, :765-774).
+  second_uniform: optional pair (outer [g1,s], inner [x,h0,t]).
+  Returns (output, loss, aux).
+  """
+  if hp.moe_gating != "top_2":
+    raise ValueError("unknown hparams.moe_gating=%s" % hp.moe_gating)
+  x = cast_act(x, act_dtype)
+  orig_shape = x.shape
+  if x.ndim == 3:                                                # :641-644
+    x = x[None]
+  a0, b1, l_, m_ = x.shape
+  x_e, y_e = hp.moe_num_experts
+  g1, s_ = split_into_groups(b1 * l_, hp.moe_group_size, mesh_dim_size)
+  cf = hp.moe_capacity_factor_train if train else hp.moe_capacity_factor_eval
+  c_ = expert_capacity(s_, cf, x_e, hp.moe_min_expert_capacity)
+  h0, t_ = split_into_groups(a0 * g1 * c_, hp.moe_group_size, mesh_dim_size)
+  d_ = expert_capacity(t_, hp.moe_capacity_factor_second_level, y_e,
+                       hp.moe_min_expert_capacity)
+  policy, threshold = _policy(hp, train)
+  u_outer, u_inner = second_uniform if second_uniform is not None else (None,
+                                                                        None)
+  xg = x.reshape(a0 * g1, s_, m_)                                # :695
+  importance = None
+  if nonpadding is not None:                                     # :638-640,:697
+    importance = cast_act(np.broadcast_to(nonpadding, (a0, b1, l_)), act_dtype)
+    importance = importance.reshape(a0 * g1, s_)
+
+  # ---- outer level (:702-727)
+  logits_x = router_logits(xg, cast_act(w_outer, act_dtype))
+  rx = top_2_gating(logits_x, c_, importance, policy, threshold,
+                    hp.moe_use_second_place_loss, num_microbatches, act_dtype,
+                    u_outer, dense=dense)
+  ag = a0 * g1
+  if dense:
+    disp = rx["dispatch"].reshape(ag, s_, x_e * c_)
+    ein = cast_act(np.matmul(disp.transpose(0, 2, 1), xg), act_dtype)
+    ein = ein.reshape(ag, x_e, c_, m_).transpose(1, 0, 2, 3)     # [x,ag,c,m]
+    imp_w = seq_sum(rx["combine"], axis=1)                       # [ag,x,c]
+    imp_w = cast_act(imp_w, act_dtype).transpose(1, 0, 2)        # [x,ag,c]
+  else:
+    ein = dispatch_gather(xg, rx, x_e, c_, act_dtype)
+    w1, w2 = combine_weights(rx, act_dtype)
+    imp_w = np.zeros((x_e, ag, c_), F32)
+    for k, w in (("1", w1), ("2", w2)):
+      gi, si = np.nonzero(rx["kept_" + k])
+      imp_w[rx["index_" + k][gi, si], gi, rx["pos_" + k][gi, si]] = w[gi, si]
+  imp2 = F32(0.5) * ((imp_w > F32(0.5)).astype(F32)
+                     + (imp_w > F32(0.0)).astype(F32))           # :725-727
+  imp2 = cast_act(imp2, act_dtype)
+
+  # ---- inner level (:737-759); a0 is the group-ish dim being re-split
+  inputs_y = ein.reshape(x_e, h0, t_, m_)
+  imp2 = imp2.reshape(x_e, h0, t_)
+  w_in = cast_act(w_inner, act_dtype)                            # [X, M, Y]
+  logits_y = np.matmul(inputs_y.reshape(x_e, h0 * t_, m_), w_in).astype(F32)
+  logits_y = logits_y.reshape(x_e * h0, t_, y_e)
+  ry = top_2_gating(logits_y, d_, imp2.reshape(x_e * h0, t_), policy,
+                    threshold, hp.moe_use_second_place_loss, num_microbatches,
+                    act_dtype, u_inner, dense=dense)
+  xin = inputs_y.reshape(x_e * h0, t_, m_)
+  if dense:
+    disp = ry["dispatch"].reshape(x_e * h0, t_, y_e * d_)
+    ein_y = cast_act(np.matmul(disp.transpose(0, 2, 1), xin), act_dtype)
+    ein_y = ein_y.reshape(x_e, h0, y_e, d_, m_).transpose(2, 0, 1, 3, 4)
+  else:
+    ein_y = dispatch_gather(xin, ry, y_e, d_, act_dtype)          # [y,xh,d,m]
+    ein_y = ein_y.reshape(y_e, x_e, h0, d_, m_)
+
+  # ---- experts (:765-774), weights [Y, X, ...]
+  wi_a = cast_act(wi, act_dtype)
+  wo_a = cast_act(wo, act_dtype)
+  h_dim = wi_a.shape[-1]
+  n_ = wo_a.shape[-1]
+  yy = expert_ffn(ein_y.reshape(y_e * x_e, h0 * d_, m_),
+                  wi_a.reshape(y_e * x_e, m_, h_dim),
+                  wo_a.reshape(y_e * x_e, h_dim, n_), "relu", act_dtype)
+  yy = yy.reshape(y_e, x_e * h0, d_, n_)
+
+  # ---- inner combine (:784), regroup (:788-791), outer combine (:794)
+  if dense:
+    comb = ry["combine"].reshape(x_e * h0, t_, y_e * d_)
+    yg = yy.transpose(1, 0, 2, 3).reshape(x_e * h0, y_e * d_, n_)
+    out_y = cast_act(np.matmul(comb, yg), act_dtype)
+  else:
+    out_y = combine_gather(yy, ry, act_dtype)
+  eo_x = out_y.reshape(x_e, ag, c_, n_)
+  if dense:
+    comb = rx["combine"].reshape(ag, s_, x_e * c_)
+    yg = eo_x.transpose(1, 0, 2, 3).reshape(ag, x_e * c_, n_)
+    out = cast_act(np.matmul(comb, yg), act_dtype)
+  else:
+    out = combine_gather(eo_x, rx, act_dtype)
+  out = out.reshape(orig_shape[:-1] + (n_,))
+  loss = cast_act(rx["loss"] + ry["loss"], act_dtype)            # :801
+  aux = dict(outer=rx, inner=ry, capacity_x=c_, capacity_y=d_,
+             groups_x=(g1, s_), groups_y=(h0, t_), importance_inner=imp2,
+             logits_outer=logits_x, logits_inner=logits_y)
+  return out, _scale_loss(loss, hp.moe_loss_coef, act_dtype), aux

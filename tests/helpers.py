@@ -1,0 +1,59 @@
+"""Shared input generators and comparison helpers for the tests."""
+
+import numpy as np
+import torch
+
+from oracle import moe_oracle as O
+
+ACT_TORCH = {"float32": torch.float32, "bfloat16": torch.bfloat16}
+
+
+def to_gpu(a, act_dtype="float32"):
+  """float32 NumPy array holding activation-dtype values -> GPU tensor."""
+  t = torch.from_numpy(np.ascontiguousarray(a, dtype=np.float32))
+  return t.to(ACT_TORCH[act_dtype]).cuda().contiguous()
+
+
+def to_np(t):
+  return t.detach().float().cpu().numpy()
+
+
+def random_logits(rng, g, s, e, scale=1.0, quantum=None):
+  x = rng.standard_normal((g, s, e)).astype(np.float32) * np.float32(scale)
+  if quantum:
+    x = (np.round(x / quantum) * quantum).astype(np.float32)
+  return x
+
+
+def min_relative_gap(p, k=3):
+  """Smallest relative gap between consecutive members of the top-k of each
+  softmax row: routing is only implementation-independent when this is well
+  above a few float32 ulps."""
+  top = -np.sort(-p, axis=-1)[..., :k]
+  gaps = (top[..., :-1] - top[..., 1:]) / np.maximum(top[..., :-1], 1e-30)
+  return float(gaps.min())
+
+
+def zipf_bias(rng, e, scale=3.0, s=1.2):
+  ranks = rng.permutation(e) + 1
+  return (scale * ranks.astype(np.float64) ** (-s)).astype(np.float32)
+
+
+def routing_to_np(r):
+  """mesh_amd.moe_hip.Routing -> dict shaped like the oracle's record."""
+  idx, pos = to_np(r.idx).astype(np.int32), to_np(r.pos).astype(np.int32)
+  gate, kept = to_np(r.gate), to_np(r.kept) != 0
+  return dict(index_1=idx[..., 0], index_2=idx[..., 1], pos_1=pos[..., 0],
+              pos_2=pos[..., 1], gate_1=gate[..., 0], gate_2=gate[..., 1],
+              kept_1=kept[..., 0], kept_2=kept[..., 1],
+              fill=to_np(r.fill).astype(np.int32), loss=to_np(r.loss)[0])
+
+
+def assert_routing_equal(got, want, gate_rtol=1e-5):
+  """Bit-exact expert indices, positions, kept masks and fill counts; gates to
+  float32 round-off."""
+  for k in ("index_1", "index_2", "kept_1", "kept_2", "pos_1", "pos_2", "fill"):
+    np.testing.assert_array_equal(got[k], want[k], err_msg=k)
+  for k in ("gate_1", "gate_2"):
+    np.testing.assert_allclose(got[k], want[k], rtol=gate_rtol, atol=1e-7,
+                               err_msg=k)

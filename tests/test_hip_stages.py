@@ -1,0 +1,200 @@
+"""GPU parity of each C-ABI entry point against the CPU oracle."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hip():
+  from mesh_amd import moe_hip
+  moe_hip.load_library()
+  return moe_hip
+
+
+# (G, S, E, C) -- the first three are the routing shapes of the benchmark
+# configurations 1-3; the rest are ragged / odd shapes and the wide-E paths.
+GATING_SHAPES = [
+    (2, 1024, 8, 160), (16, 1024, 32, 40), (16, 2048, 64, 32),
+    (3, 77, 5, 7), (1, 1, 2, 1), (2, 300, 128, 6), (2, 130, 200, 4),
+    (1, 257, 300, 3), (5, 64, 16, 64), (1, 4096, 64, 128),
+]
+
+
+@pytest.mark.parametrize("shape", GATING_SHAPES)
+def test_gating_random_logits(hip, shape):
+  g, s, e, c = shape
+  rng = np.random.default_rng(hash(shape) % (2 ** 31))
+  logits = H.random_logits(rng, g, s, e, scale=1.5)
+  if shape == (16, 2048, 64, 32):
+    logits = logits + H.zipf_bias(rng, e)
+  assert H.min_relative_gap(O.softmax(logits), min(3, e)) > 1e-5
+  want = O.top_2_gating(logits, c)
+  r = hip.top2_gating(torch.from_numpy(logits).cuda(), c)
+  got = H.routing_to_np(r)
+  H.assert_routing_equal(got, want)
+  np.testing.assert_allclose(got["loss"], want["loss"], rtol=2e-5)
+
+
+@pytest.mark.parametrize("shape", [(2, 256, 8, 40), (3, 500, 64, 9)])
+def test_gating_exact_ties(hip, shape):
+  """Logits on a coarse grid: many exact ties, where the lowest index must win
+  both times; unequal logits differ by >= 0.25 so nothing is a near-tie."""
+  g, s, e, c = shape
+  rng = np.random.default_rng(7)
+  logits = H.random_logits(rng, g, s, e, scale=0.6, quantum=0.25)
+  want = O.top_2_gating(logits, c)
+  got = H.routing_to_np(hip.top2_gating(torch.from_numpy(logits).cuda(), c))
+  H.assert_routing_equal(got, want)
+
+
+@pytest.mark.parametrize("imp_dtype", ["float32", "bfloat16"])
+def test_gating_importance(hip, imp_dtype):
+  g, s, e, c = 4, 320, 16, 24
+  rng = np.random.default_rng(11)
+  logits = H.random_logits(rng, g, s, e)
+  imp = rng.choice(np.array([0.0, 0.5, 1.0], np.float32), size=(g, s),
+                   p=[0.2, 0.3, 0.5])
+  assert H.min_relative_gap(O.softmax(logits)) > 1e-5
+  want = O.top_2_gating(logits, c, importance=imp, use_second_place_loss=True)
+  r = hip.top2_gating(torch.from_numpy(logits).cuda(), c,
+                      importance=H.to_gpu(imp, imp_dtype),
+                      use_second_place_loss=True)
+  got = H.routing_to_np(r)
+  H.assert_routing_equal(got, want)
+  np.testing.assert_allclose(got["loss"], want["loss"], rtol=2e-5)
+  # importance 0.5 rows go to their best expert as a second-priority choice
+  half = imp == 0.5
+  assert (got["index_1"][half] == got["index_2"][half]).all()
+  assert not got["kept_1"][half].any()
+  assert not got["kept_1"][imp == 0].any() and not got["kept_2"][imp == 0].any()
+
+
+@pytest.mark.parametrize("policy", ["none", "threshold", "random"])
+def test_gating_second_policy(hip, policy):
+  g, s, e, c = 3, 512, 8, 200
+  rng = np.random.default_rng(13)
+  logits = H.random_logits(rng, g, s, e)
+  u = rng.random((g, s)).astype(np.float32)
+  thr = 0.3
+  ref_all = O.top_2_gating(logits, 10 ** 6)  # uncapped: raw normalised gates
+  g2 = ref_all["gate_2"]
+  if policy == "threshold":
+    assert np.abs(g2 - np.float32(thr)).min() > 1e-6
+  if policy == "random":
+    assert np.abs(u - g2 * np.float32(1.0 / thr)).min() > 1e-6
+  want = O.top_2_gating(logits, c, policy=policy, threshold=thr,
+                        second_uniform=u, use_second_place_loss=True,
+                        num_microbatches=4)
+  r = hip.top2_gating(torch.from_numpy(logits).cuda(), c, policy=policy,
+                      threshold=thr, second_uniform=torch.from_numpy(u).cuda(),
+                      use_second_place_loss=True, num_microbatches=4)
+  got = H.routing_to_np(r)
+  H.assert_routing_equal(got, want)
+  np.testing.assert_allclose(got["loss"], want["loss"], rtol=2e-5)
+
+
+@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape", [(2, 1024, 512, 8), (3, 100, 72, 5),
+                                   (1, 640, 1024, 128)])
+def test_router_logits(hip, act_dtype, shape):
+  g, s, m, e = shape
+  rng = np.random.default_rng(17)
+  x = O.cast_act(rng.standard_normal((g * s, m)).astype(np.float32), act_dtype)
+  w = O.cast_act(rng.standard_normal((m, e)).astype(np.float32) / np.sqrt(m),
+                 act_dtype)
+  bias = rng.standard_normal(e).astype(np.float32)
+  want = (x.astype(np.float64) @ w.astype(np.float64))
+  got = H.to_np(hip.router_logits(H.to_gpu(x, act_dtype), H.to_gpu(w, act_dtype)))
+  np.testing.assert_allclose(got, want, rtol=1e-5, atol=2e-5)
+  got_b = H.to_np(hip.router_logits(H.to_gpu(x, act_dtype),
+                                    H.to_gpu(w, act_dtype),
+                                    bias=torch.from_numpy(bias).cuda()))
+  np.testing.assert_allclose(got_b, want + bias, rtol=1e-5, atol=2e-5)
+
+
+def test_router_logits_batched(hip):
+  b, t, m, e = 4, 150, 64, 16
+  rng = np.random.default_rng(19)
+  x = rng.standard_normal((b, t, m)).astype(np.float32)
+  w = rng.standard_normal((b, m, e)).astype(np.float32)
+  want = np.matmul(x.astype(np.float64), w.astype(np.float64))
+  got = H.to_np(hip.router_logits(H.to_gpu(x), H.to_gpu(w)))
+  np.testing.assert_allclose(got, want, rtol=1e-5, atol=2e-5)
+
+
+@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape", [(2, 256, 8, 40, 64), (3, 77, 5, 7, 36),
+                                   (4, 128, 16, 8, 1024)])
+def test_dispatch_combine(hip, act_dtype, shape):
+  g, s, e, c, m = shape
+  rng = np.random.default_rng(23)
+  logits = H.random_logits(rng, g, s, e)
+  x = O.cast_act(rng.standard_normal((g, s, m)).astype(np.float32), act_dtype)
+  want_r = O.top_2_gating(logits, c)
+  r = hip.top2_gating(torch.from_numpy(logits).cuda(), c)
+  H.assert_routing_equal(H.routing_to_np(r), want_r)
+  ein, slot_gate = hip.dispatch(H.to_gpu(x, act_dtype), r, want_slot_gate=True)
+  want_ein = O.dispatch_gather(x, want_r, e, c, act_dtype)
+  np.testing.assert_array_equal(H.to_np(ein), want_ein)
+  # slot weights: the dense combine tensor summed over the group-size dim
+  dense = O.top_2_gating(logits, c, act_dtype=act_dtype, dense=True)
+  want_sg = dense["combine"].sum(axis=1).transpose(1, 0, 2)       # [E,G,C]
+  np.testing.assert_allclose(H.to_np(slot_gate), want_sg, rtol=1e-5, atol=1e-7)
+  # the gather form equals the reference's dense einsum
+  dense_ein = np.einsum("gsm,gsec->egcm", x, dense["dispatch"])
+  np.testing.assert_array_equal(want_ein, dense_ein.astype(np.float32))
+  # combine
+  y = O.cast_act(rng.standard_normal((e, g, c, m)).astype(np.float32), act_dtype)
+  got_out = H.to_np(hip.combine(H.to_gpu(y, act_dtype), r, s))
+  gpu_r = H.routing_to_np(r)
+  want_out = O.combine_gather(y, gpu_r, act_dtype)
+  np.testing.assert_array_equal(got_out, want_out)
+  dense_out = O.cast_act(np.einsum("egcn,gsec->gsn", y, dense["combine"]),
+                         act_dtype)
+  tol = dict(rtol=2e-2, atol=1e-2) if act_dtype == "bfloat16" else dict(
+      rtol=1e-4, atol=1e-5)
+  np.testing.assert_allclose(got_out, dense_out, **tol)
+
+
+@pytest.mark.parametrize("act_dtype,activation", [
+    ("float32", "relu"), ("bfloat16", "relu"), ("bfloat16", "gelu"),
+    ("float32", "linear")])
+@pytest.mark.parametrize("shape", [(3, 320, 64, 128, 64), (2, 100, 72, 200, 40),
+                                   (2, 1100, 128, 1152, 1024),
+                                   (1, 40, 30, 50, 20)])
+def test_expert_ffn(hip, act_dtype, activation, shape):
+  e, rows, m, hdim, n = shape
+  rng = np.random.default_rng(29)
+  ein = O.cast_act(rng.standard_normal((e, rows, m)).astype(np.float32), act_dtype)
+  wi = rng.standard_normal((e, m, hdim)).astype(np.float32) / np.sqrt(m)
+  wo = rng.standard_normal((e, hdim, n)).astype(np.float32) / np.sqrt(hdim)
+  dt = H.ACT_TORCH[act_dtype]
+  wi_p = hip.pack_weights(torch.from_numpy(wi).cuda(), dt)
+  wo_p = hip.pack_weights(torch.from_numpy(wo).cuda(), dt)
+  np.testing.assert_array_equal(
+      H.to_np(wi_p), O.cast_act(wi, act_dtype).transpose(0, 2, 1))
+  got = H.to_np(hip.expert_ffn(H.to_gpu(ein, act_dtype), wi_p, wo_p, activation))
+  want = O.expert_ffn(ein, O.cast_act(wi, act_dtype), O.cast_act(wo, act_dtype),
+                      activation, act_dtype)
+  tol = dict(rtol=2e-2, atol=1e-2) if act_dtype == "bfloat16" else dict(
+      rtol=1e-4, atol=1e-5)
+  np.testing.assert_allclose(got, want, **tol)
+
+
+def test_rejects_bad_arguments(hip):
+  logits = torch.zeros((1, 8, 4), device="cuda")
+  with pytest.raises(ValueError):
+    hip.top2_gating(logits, 2, policy="sometimes")
+  with pytest.raises(hip.MoeHipError):
+    hip.top2_gating(logits, 2, policy="random")          # no samples given
+  with pytest.raises(hip.MoeHipError):
+    hip.top2_gating(torch.zeros((1, 8, 1), device="cuda"), 2)   # E < 2
+  with pytest.raises(hip.MoeHipError):
+    hip.router_logits(torch.zeros((4, 8), device="cuda"),
+                      torch.zeros((9, 2), device="cuda"))
