@@ -25,6 +25,26 @@ def random_logits(rng, g, s, e, scale=1.0, quantum=None):
   return x
 
 
+def safe_logits(rng, g, s, e, scale=1.0, bias=None, min_gap=1e-4):
+  """Random logits whose three largest entries per row differ by at least
+  `min_gap` (rows that do not are redrawn), so that the top-2 choice does not
+  depend on the last ulps of exp/log."""
+  x = random_logits(rng, g, s, e, scale)
+  if bias is not None:
+    x = x + bias
+  k = min(3, e)
+  for _ in range(100):
+    top = -np.sort(-x, axis=-1)[..., :k]
+    bad = ((top[..., :-1] - top[..., 1:]) < min_gap).any(axis=-1)
+    if not bad.any():
+      return x
+    fresh = random_logits(rng, 1, int(bad.sum()), e, scale)[0]
+    if bias is not None:
+      fresh = fresh + bias
+    x[bad] = fresh
+  raise AssertionError("could not separate the top-3 logits")
+
+
 def min_relative_gap(p, k=3):
   """Smallest relative gap between consecutive members of the top-k of each
   softmax row: routing is only implementation-independent when this is well

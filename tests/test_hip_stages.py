@@ -30,10 +30,9 @@ GATING_SHAPES = [
 def test_gating_random_logits(hip, shape):
   g, s, e, c = shape
   rng = np.random.default_rng(hash(shape) % (2 ** 31))
-  logits = H.random_logits(rng, g, s, e, scale=1.5)
-  if shape == (16, 2048, 64, 32):
-    logits = logits + H.zipf_bias(rng, e)
-  assert H.min_relative_gap(O.softmax(logits), min(3, e)) > 1e-5
+  bias = H.zipf_bias(rng, e) if shape == (16, 2048, 64, 32) else None
+  logits = H.safe_logits(rng, g, s, e, scale=1.5, bias=bias)
+  assert H.min_relative_gap(O.softmax(logits), min(3, e)) > 2e-5
   want = O.top_2_gating(logits, c)
   r = hip.top2_gating(torch.from_numpy(logits).cuda(), c)
   got = H.routing_to_np(r)
@@ -57,7 +56,7 @@ def test_gating_exact_ties(hip, shape):
 def test_gating_importance(hip, imp_dtype):
   g, s, e, c = 4, 320, 16, 24
   rng = np.random.default_rng(11)
-  logits = H.random_logits(rng, g, s, e)
+  logits = H.safe_logits(rng, g, s, e)
   imp = rng.choice(np.array([0.0, 0.5, 1.0], np.float32), size=(g, s),
                    p=[0.2, 0.3, 0.5])
   assert H.min_relative_gap(O.softmax(logits)) > 1e-5
@@ -79,7 +78,7 @@ def test_gating_importance(hip, imp_dtype):
 def test_gating_second_policy(hip, policy):
   g, s, e, c = 3, 512, 8, 200
   rng = np.random.default_rng(13)
-  logits = H.random_logits(rng, g, s, e)
+  logits = H.safe_logits(rng, g, s, e)
   u = rng.random((g, s)).astype(np.float32)
   thr = 0.3
   ref_all = O.top_2_gating(logits, 10 ** 6)  # uncapped: raw normalised gates
@@ -134,7 +133,7 @@ def test_router_logits_batched(hip):
 def test_dispatch_combine(hip, act_dtype, shape):
   g, s, e, c, m = shape
   rng = np.random.default_rng(23)
-  logits = H.random_logits(rng, g, s, e)
+  logits = H.safe_logits(rng, g, s, e)
   x = O.cast_act(rng.standard_normal((g, s, m)).astype(np.float32), act_dtype)
   want_r = O.top_2_gating(logits, c)
   r = hip.top2_gating(torch.from_numpy(logits).cuda(), c)
@@ -172,8 +171,8 @@ def test_expert_ffn(hip, act_dtype, activation, shape):
   e, rows, m, hdim, n = shape
   rng = np.random.default_rng(29)
   ein = O.cast_act(rng.standard_normal((e, rows, m)).astype(np.float32), act_dtype)
-  wi = rng.standard_normal((e, m, hdim)).astype(np.float32) / np.sqrt(m)
-  wo = rng.standard_normal((e, hdim, n)).astype(np.float32) / np.sqrt(hdim)
+  wi = (rng.standard_normal((e, m, hdim)) / np.sqrt(m)).astype(np.float32)
+  wo = (rng.standard_normal((e, hdim, n)) / np.sqrt(hdim)).astype(np.float32)
   dt = H.ACT_TORCH[act_dtype]
   wi_p = hip.pack_weights(torch.from_numpy(wi).cuda(), dt)
   wo_p = hip.pack_weights(torch.from_numpy(wo).cuda(), dt)
