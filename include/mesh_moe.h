@@ -84,7 +84,10 @@ size_t mesh_moe_gating_workspace_bytes(int G, int S, int E);
  * [G,S,E,C] combine/dispatch tensors (moe.py:1499-1511): the per-token record
  * below carries the same information.
  *   logits      [G,S,E] float32
- *   importance  [G,S] of importance_dtype, or NULL  (moe.py:1401-1411)
+ *   importance  [G,S] of importance_dtype, or NULL  (moe.py:1401-1411).
+ *               With importance_from_slot_gate != 0 the array holds the slot
+ *               weights w written by mesh_moe_dispatch and the importance is
+ *               0.5 * ((w > 0.5) + (w > 0))  (hierarchical layer, moe.py:725-727)
  *   second_uniform [G,S] float32 U(0,1) samples, required for policy RANDOM
  *   idx  [G,S,2] int32   expert of first / second choice
  *   pos  [G,S,2] int32   position_in_expert_k (raw; >= C when dropped)
@@ -95,8 +98,9 @@ size_t mesh_moe_gating_workspace_bytes(int G, int S, int E);
  * Limits: 2 <= E <= 512, S <= 16384, C >= 1.
  */
 int mesh_moe_top2_gating(const float* logits, const void* importance,
-                         int importance_dtype, const float* second_uniform,
-                         int G, int S, int E, int C, int policy,
+                         int importance_dtype, int importance_from_slot_gate,
+                         const float* second_uniform, int G, int S, int E,
+                         int C, int policy,
                          double threshold, int use_second_place_loss,
                          int num_microbatches, int32_t* idx, int32_t* pos,
                          float* gate, uint8_t* kept, int32_t* fill,

@@ -89,6 +89,7 @@ struct GateParams {
   float inv_threshold;  // float32(1 / max(thr, 1e-9))   (moe.py:1465)
   int use_second_place_loss;
   int num_microbatches;
+  int importance_from_slot_gate;  // importance = 0.5*((w>0.5)+(w>0))
   int tt;    // tokens per block of step 1
   int nblk;  // blocks per group of step 1
 };
@@ -142,6 +143,8 @@ __global__ __launch_bounds__(256) void gate_select_kernel(
     bool sel2 = true;
     if (importance != nullptr) {
       float imp = load_f32<IT>(importance + t);
+      if (p.importance_from_slot_gate)                      // moe.py:725-727
+        imp = 0.5f * ((imp > 0.5f ? 1.0f : 0.0f) + (imp > 0.0f ? 1.0f : 0.0f));
       sel1 = (imp == 1.0f);                                 // moe.py:1402-1404
       sel2 = (imp > 0.0f);                                  // moe.py:1411
     }
@@ -387,7 +390,8 @@ extern "C" size_t mesh_moe_gating_workspace_bytes(int G, int S, int E) {
 
 extern "C" int mesh_moe_top2_gating(
     const float* logits, const void* importance, int importance_dtype,
-    const float* second_uniform, int G, int S, int E, int C, int policy,
+    int importance_from_slot_gate, const float* second_uniform, int G, int S,
+    int E, int C, int policy,
     double threshold, int use_second_place_loss, int num_microbatches,
     int32_t* idx, int32_t* pos, float* gate, uint8_t* kept, int32_t* fill,
     float* loss, void* workspace, size_t workspace_bytes, void* stream) {
@@ -418,6 +422,7 @@ extern "C" int mesh_moe_top2_gating(
   p.inv_threshold = (float)(1.0 / (threshold > 1e-9 ? threshold : 1e-9));
   p.use_second_place_loss = use_second_place_loss ? 1 : 0;
   p.num_microbatches = num_microbatches;
+  p.importance_from_slot_gate = importance_from_slot_gate ? 1 : 0;
   p.tt = gate_tokens_per_block(E);
   p.nblk = (S + p.tt - 1) / p.tt;
   hipStream_t st = (hipStream_t)stream;

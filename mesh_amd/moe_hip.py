@@ -34,8 +34,8 @@ _SIGNATURES = {
     "mesh_moe_gating_workspace_bytes": (ctypes.c_size_t, [
         ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "mesh_moe_top2_gating": (ctypes.c_int, [
-        _vp, _vp, ctypes.c_int, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
-        ctypes.c_int, ctypes.c_int, ctypes.c_double, ctypes.c_int,
+        _vp, _vp, ctypes.c_int, ctypes.c_int, _vp, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_double, ctypes.c_int,
         ctypes.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_size_t,
         _vp]),
     "mesh_moe_dispatch": (ctypes.c_int, [
@@ -144,7 +144,8 @@ class Routing(object):
 
 def top2_gating(logits, capacity, importance=None, policy="all",
                 threshold=0.2, use_second_place_loss=False,
-                num_microbatches=None, second_uniform=None):
+                num_microbatches=None, second_uniform=None,
+                importance_from_slot_gate=False):
   """logits float32 [G, S, E] -> Routing (all tensors on the GPU)."""
   lib = load_library()
   if policy not in POLICIES:
@@ -168,7 +169,8 @@ def top2_gating(logits, capacity, importance=None, policy="all",
   ws_bytes = lib.mesh_moe_gating_workspace_bytes(g, s, e)
   ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
   _check(lib.mesh_moe_top2_gating(
-      lp, ip, icode, up, g, s, e, int(capacity), POLICIES[policy],
+      lp, ip, icode, int(bool(importance_from_slot_gate)), up, g, s, e,
+      int(capacity), POLICIES[policy],
       float(threshold), int(bool(use_second_place_loss)),
       int(num_microbatches or 1), idx.data_ptr(), pos.data_ptr(),
       gate.data_ptr(), kept.data_ptr(), fill.data_ptr(), loss.data_ptr(),

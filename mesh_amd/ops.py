@@ -1,0 +1,874 @@
+"""A small named-dimension graph language with the vocabulary of Mesh TensorFlow.
+
+Only what the Mixture-of-Experts layers need is here: Dimension / Shape /
+LayoutRules, Graph / Mesh / Tensor / Operation, variables with master and slice
+copies, reshape, import/export, a slicewise escape hatch, and the Lowering that
+runs a graph on a MeshImpl.  Names, argument order and error types follow
+mesh_tensorflow/ops.py so that code written against `mtf` reads the same
+(`import mesh_amd as mtf`); the implementation is new.
+
+Differences that matter:
+  * tensors are torch tensors, dtypes are torch dtypes;
+  * there is no deferred TensorFlow graph: `Lowering(graph, {mesh: impl})`
+    executes each Operation's `lower` once, on the current HIP stream, and
+    `Lowering.run(feeds)` executes the non-variable operations again (the
+    counterpart of session.run with a feed_dict).
+"""
+
+import collections
+import contextlib
+import re
+
+import numpy as np
+import torch
+
+float32 = torch.float32
+bfloat16 = torch.bfloat16
+int32 = torch.int32
+
+
+# ----------------------------------------------------------------------------
+# Dimension, Shape, layout  (mesh_tensorflow/ops.py:41-377)
+# ----------------------------------------------------------------------------
+Dimension = collections.namedtuple("Dimension", ["name", "size"])
+
+
+def convert_to_dimension(d):
+  """Dimension, (name, size) pair or None -> Dimension or None."""
+  if d is None:
+    return None
+  if isinstance(d, Dimension):
+    name, size = d.name, d.size
+  else:
+    name, size = d
+  if not isinstance(name, str) or not isinstance(size, int):
+    raise ValueError("could not convert %s to Dimension" % (d,))
+  return Dimension(name, size)
+
+
+class Shape(object):
+  """Ordered list of uniquely named Dimensions."""
+
+  def __init__(self, dims):
+    self._dims = [convert_to_dimension(d) for d in tuple(dims)]
+    names = [d.name for d in self._dims]
+    if len(set(names)) != len(names):
+      raise ValueError("Shape must not have repeated dimensions %s" % names)
+
+  @property
+  def dims(self):
+    return list(self._dims)
+
+  @property
+  def ndims(self):
+    return len(self._dims)
+
+  @property
+  def size(self):
+    return list_product(self.to_integer_list)
+
+  @property
+  def to_integer_list(self):
+    return [d.size for d in self._dims]
+
+  @property
+  def dimension_names(self):
+    return [d.name for d in self._dims]
+
+  @property
+  def to_string(self):
+    return "Shape[%s]" % ", ".join(
+        "%s=%d" % (d.name, d.size) for d in self._dims)
+
+  @property
+  def cumprod(self):
+    """cumprod[i] = product of the sizes of dims[i+1:] (plus a trailing 1)."""
+    out, acc = [], 1
+    for s in reversed(self.to_integer_list):
+      out.append(acc)
+      acc *= s
+    return list(reversed(out))
+
+  def __repr__(self):
+    return self.to_string
+
+  def __eq__(self, other):
+    return isinstance(other, Shape) and self._dims == other._dims
+
+  def __ne__(self, other):
+    return not self == other
+
+  def __hash__(self):
+    return hash(tuple(self._dims))
+
+  def __len__(self):
+    return len(self._dims)
+
+  def __iter__(self):
+    return iter(self._dims)
+
+  def __getitem__(self, key):
+    ret = self._dims[key]
+    return Shape(ret) if isinstance(key, slice) else ret
+
+  def __add__(self, other):
+    if isinstance(other, Shape):
+      other = other.dims
+    if isinstance(other, Dimension):
+      other = [other]
+    return Shape(self._dims + list(other))
+
+  def __sub__(self, other):
+    if other is None:
+      return self
+    if isinstance(other, Dimension):
+      other = [other]
+    if isinstance(other, Shape):
+      other = other.dims
+    return Shape([d for d in self._dims if d not in other])
+
+  def get_dim_by_name(self, name):
+    for d in self._dims:
+      if d.name == name:
+        return d
+    raise ValueError("Dimension %s not found in %s" % (name, self.to_string))
+
+  def rename_dimension(self, old_name, new_name):
+    if old_name not in self.dimension_names:
+      raise ValueError("Shape %s does not have dimension named %s"
+                       % (self, old_name))
+    return Shape([Dimension(new_name, d.size) if d.name == old_name else d
+                  for d in self._dims])
+
+  def resize_dimension(self, name, new_size):
+    if name not in self.dimension_names:
+      raise ValueError("Shape %s does not have dimension named %s"
+                       % (self, name))
+    return Shape([Dimension(name, new_size) if d.name == name else d
+                  for d in self._dims])
+
+
+def list_product(xs):
+  ret = 1
+  for x in xs:
+    ret *= x
+  return ret
+
+
+def _parse_pairs(s, sep):
+  """"a:b,c:d" (or with ';' / whitespace between pairs) -> [(a, b), (c, d)]."""
+  pairs = []
+  for item in re.split(r"[,;\s]+", s.strip()):
+    if not item:
+      continue
+    left, right = item.split(sep)
+    pairs.append((left.strip(), right.strip()))
+  return pairs
+
+
+def convert_to_shape(x):
+  """Shape, list of Dimensions, "name:size,..." string, or None -> Shape."""
+  if x is None:
+    return None
+  if isinstance(x, Shape):
+    return x
+  if isinstance(x, str):
+    x = [(n, int(s)) for n, s in _parse_pairs(x, ":")]
+  return Shape(x)
+
+
+class LayoutRules(object):
+  """Set of (tensor dimension name, mesh dimension name) pairs."""
+
+  def __init__(self, pairs):
+    self._pairs = set(tuple(p) for p in pairs)
+
+  def __repr__(self):
+    return "LayoutRules%s" % sorted(self._pairs)
+
+  def tensor_dimension_to_mesh_axis(self, tensor_dimension, mesh_shape):
+    axes = [i for i, md in enumerate(mesh_shape)
+            if (tensor_dimension.name, md.name) in self._pairs]
+    if len(axes) > 1:
+      raise ValueError(
+          "Tensor dimension maps to multiple mesh dimensions"
+          " tensor_dimension=%s mesh_shape=%s layout=%s"
+          % (tensor_dimension, mesh_shape, self._pairs))
+    return axes[0] if axes else None
+
+  def tensor_layout(self, tensor_shape, mesh_shape):
+    axes = [self.tensor_dimension_to_mesh_axis(d, mesh_shape)
+            for d in tensor_shape]
+    used = [a for a in axes if a is not None]
+    if len(used) != len(set(used)):
+      raise ValueError(
+          "Two Tensor Dimensions may not map to the same Mesh Dimension:"
+          " layout=%s tensor_shape=%s mesh_shape=%s"
+          % (self, tensor_shape, mesh_shape))
+    return TensorLayout(axes)
+
+
+class TensorLayout(object):
+  """For each tensor axis, the mesh axis it is split over (or None)."""
+
+  def __init__(self, tensor_axis_to_mesh_axis):
+    self._t2m = tuple(tensor_axis_to_mesh_axis)
+
+  @property
+  def tensor_axis_to_mesh_axis(self):
+    return self._t2m
+
+  @property
+  def is_fully_replicated(self):
+    return all(a is None for a in self._t2m)
+
+  def __repr__(self):
+    return "TensorLayout%s" % (self._t2m,)
+
+
+def convert_to_layout_rules(x):
+  """LayoutRules, "tensor_dim:mesh_dim,..." string, pairs or None."""
+  if isinstance(x, LayoutRules):
+    return x
+  if x is None:
+    return LayoutRules([])
+  if isinstance(x, str):
+    x = _parse_pairs(x, ":")
+  if isinstance(x, dict):
+    x = list(x.items())
+  return LayoutRules(x)
+
+
+def tensor_dim_to_mesh_dim_size(layout, mesh_shape, tensor_dim):
+  """How many ways `tensor_dim` is split under (layout, mesh_shape); 1 if it is
+  not split (mesh_tensorflow/ops.py:6455-6477)."""
+  layout_rules = convert_to_layout_rules(layout)
+  mesh_shape = convert_to_shape(mesh_shape)
+  if mesh_shape is None:
+    return 1
+  axis = layout_rules.tensor_dimension_to_mesh_axis(tensor_dim, mesh_shape)
+  return 1 if axis is None else mesh_shape.dims[axis].size
+
+
+# ----------------------------------------------------------------------------
+# variable scopes: names only (the reference leans on tf.variable_scope)
+# ----------------------------------------------------------------------------
+_SCOPE_STACK = []
+
+
+@contextlib.contextmanager
+def variable_scope(name):
+  """Prefixes the names of variables created inside with `name/`."""
+  _SCOPE_STACK.append(name)
+  try:
+    yield
+  finally:
+    _SCOPE_STACK.pop()
+
+
+def current_scope_name():
+  return "/".join(s for s in _SCOPE_STACK if s)
+
+
+# ----------------------------------------------------------------------------
+# Graph, Mesh, Tensor, Operation  (mesh_tensorflow/ops.py:380-674, :841-865,
+# :1423-1650)
+# ----------------------------------------------------------------------------
+class Graph(object):
+  """Container of Operations in creation order."""
+
+  def __init__(self):
+    self._operations = []
+    self._trainable_variables = []
+    self._all_variables = []
+    self._names = collections.Counter()
+
+  @property
+  def operations(self):
+    return self._operations
+
+  @property
+  def trainable_variables(self):
+    return self._trainable_variables
+
+  @property
+  def all_variables(self):
+    return self._all_variables
+
+  def unique_name(self, name):
+    n = self._names[name]
+    self._names[name] += 1
+    return name if n == 0 else "%s_%d" % (name, n)
+
+  def variable_by_name(self, name):
+    for v in self._all_variables:
+      if v.name == name:
+        return v
+    raise KeyError("no variable named %s (have %s)"
+                   % (name, [v.name for v in self._all_variables]))
+
+
+class Mesh(object):
+  """A placeholder; a Lowering assigns each Mesh a MeshImpl."""
+
+  def __init__(self, graph, name, variable_placer=None):
+    self._graph = graph
+    self._name = name
+    self._variable_placer = variable_placer
+
+  @property
+  def graph(self):
+    return self._graph
+
+  @property
+  def name(self):
+    return self._name
+
+
+class Tensor(object):
+  """An output of an Operation: named Shape + dtype."""
+
+  def __init__(self, operation, shape, dtype, name=None, index=0):
+    if not isinstance(shape, Shape):
+      raise ValueError("shape must be a Shape got %s" % (shape,))
+    self._operation = operation
+    self._shape = shape
+    self._dtype = dtype
+    self._mesh = operation.mesh
+    self._name = name if name is not None else "%s:%d" % (operation.name, index)
+
+  shape = property(lambda self: self._shape)
+  size = property(lambda self: self._shape.size)
+  mesh = property(lambda self: self._mesh)
+  graph = property(lambda self: self._mesh.graph)
+  operation = property(lambda self: self._operation)
+  dtype = property(lambda self: self._dtype)
+  name = property(lambda self: self._name)
+
+  @property
+  def to_string(self):
+    return "Tensor[%s, %s, %s]" % (self.name, self.shape.to_string, self.dtype)
+
+  def __repr__(self):
+    return self.to_string
+
+  def __add__(self, other):
+    return add(self, other)
+
+  def __radd__(self, other):
+    return add(self, other)
+
+  def __mul__(self, other):
+    return multiply(self, other)
+
+  def __rmul__(self, other):
+    return multiply(self, other)
+
+  def __truediv__(self, other):
+    if isinstance(other, Tensor):
+      raise NotImplementedError("Tensor / Tensor is not part of this subset")
+    return multiply(self, 1.0 / other)
+
+
+class Operation(object):
+  """A node of the graph: inputs -> outputs, with a `lower` method."""
+
+  def __init__(self, inputs, mesh=None, name=None):
+    if mesh is None:
+      if not inputs:
+        raise ValueError("mesh must be specified if no inputs")
+      mesh = inputs[0].mesh
+    self._inputs = list(inputs)
+    self._outputs = []
+    self._mesh = mesh
+    assert name is not None
+    scope = current_scope_name()
+    self._name = mesh.graph.unique_name(scope + "/" + name if scope else name)
+    mesh.graph.operations.append(self)
+
+  inputs = property(lambda self: self._inputs[:])
+  outputs = property(lambda self: self._outputs[:])
+  mesh = property(lambda self: self._mesh)
+  graph = property(lambda self: self._mesh.graph)
+  name = property(lambda self: self._name)
+
+  @property
+  def to_string(self):
+    return "%s[Inputs=(%s) Outputs=(%s)]" % (
+        type(self).__name__,
+        ", ".join(t.to_string for t in self._inputs),
+        ", ".join(t.to_string for t in self._outputs))
+
+  def lower(self, lowering):
+    raise NotImplementedError("Lower not implemented")
+
+
+# ----------------------------------------------------------------------------
+# MeshImpl  (mesh_tensorflow/ops.py:867-1340)
+# ----------------------------------------------------------------------------
+class MeshImpl(object):
+  """Implementation of a Mesh: mesh shape + layout rules (+ devices in
+  subclasses).  Subclasses provide slicewise, the LaidOutTensor /
+  LaidOutVariable types, import/export and the collectives."""
+
+  def __init__(self, shape, layout_rules):
+    self._shape = convert_to_shape(shape)
+    self._layout_rules = convert_to_layout_rules(layout_rules)
+
+  shape = property(lambda self: self._shape)
+  ndims = property(lambda self: len(self._shape))
+  layout_rules = property(lambda self: self._layout_rules)
+  size = property(lambda self: self._shape.size)
+
+  @property
+  def supports_control_dependencies(self):
+    return True
+
+  def tensor_dimension_to_mesh_axis(self, tensor_dimension):
+    return self.layout_rules.tensor_dimension_to_mesh_axis(
+        tensor_dimension, self.shape)
+
+  def tensor_layout(self, arg):
+    if isinstance(arg, Tensor):
+      arg = arg.shape
+    return self.layout_rules.tensor_layout(arg, self.shape)
+
+  def slice_shape(self, tensor_shape):
+    """Per-device slice shape; ValueError if a mesh dim does not divide."""
+    layout = self.tensor_layout(tensor_shape)
+    ret = []
+    for dim, axis in zip(tensor_shape, layout.tensor_axis_to_mesh_axis):
+      if axis is None:
+        ret.append(dim.size)
+      else:
+        n = self.shape[axis].size
+        if dim.size % n != 0:
+          raise ValueError(
+              "Tensor dimension size not divisible by mesh dimension size:"
+              " tensor_shape=%s tensor_layout=%s" % (tensor_shape, layout))
+        ret.append(dim.size // n)
+    return ret
+
+  def slice_begin(self, tensor_shape, pnum):
+    if self.size != 1:
+      raise NotImplementedError("only single-device meshes are implemented")
+    return [0] * tensor_shape.ndims
+
+  def slice_size(self, tensor_shape):
+    return list_product(self.slice_shape(tensor_shape))
+
+  def laid_out_size(self, tensor_shape):
+    return self.slice_size(tensor_shape) * self.size
+
+  # -- to be provided by subclasses
+  def slicewise(self, fn, *inputs):
+    raise NotImplementedError("Slicewise not implemented")
+
+  def einsum(self, equation, *slices):
+    raise NotImplementedError("einsum not implemented")
+
+  def allreduce(self, x, mesh_axes, reduction_fn_string):
+    raise NotImplementedError("Allreduce not implemented")
+
+  def allconcat(self, x, mesh_axis, concat_axis):
+    raise NotImplementedError("Allconcat not implemented")
+
+  def alltoall(self, x, mesh_axis, split_axis, concat_axis):
+    raise NotImplementedError("Alltoall not implemented")
+
+  def receive(self, x, mesh_axis, source_pcoord):
+    raise NotImplementedError("Receive not implemented")
+
+  def import_tf_tensor(self, x, tf_x):
+    raise NotImplementedError("Import not implemented")
+
+  def export_to_tf_tensor(self, x, laid_out_x):
+    raise NotImplementedError("Export not implemented")
+
+  def make_slices(self, tf_tensor, tensor_shape):
+    if self.size != 1:
+      raise NotImplementedError("only single-device meshes are implemented")
+    return [tf_tensor]
+
+  def combine_slices(self, slices, tensor_shape, device=None):
+    if self.size != 1:
+      raise NotImplementedError("only single-device meshes are implemented")
+    return slices[0]
+
+
+def convert_args_to_laid_out_tensors(xs):
+  """Calls to_laid_out_tensor() on the arguments that have it."""
+  return [x.to_laid_out_tensor() if hasattr(x, "to_laid_out_tensor") else x
+          for x in xs]
+
+
+# ----------------------------------------------------------------------------
+# Lowering  (mesh_tensorflow/ops.py:676-838)
+# ----------------------------------------------------------------------------
+class Lowering(object):
+  """Runs a Graph on MeshImpls.
+
+  Construction lowers (= executes) every Operation once, in graph order.
+  `run(feeds)` executes them again without re-creating variables.
+  """
+
+  def __init__(self, graph, mesh_to_impl, autostack=True, log_file=None,
+               initial_values=None):
+    del autostack, log_file  # accepted for signature compatibility
+    self.mesh_to_impl = mesh_to_impl
+    self.graph = graph
+    self._counters = []
+    self.tensors = {}      # {Tensor: LaidOutTensor}
+    self.operations = {}   # {Operation: lowered handle}
+    self.variables = {}    # {Variable: LaidOutVariable}
+    self.initial_values = dict(initial_values or {})
+    self._feeds = {}
+    for op in graph.operations:
+      op.lower(self)
+      for out in op.outputs:
+        self.add_counter("output/%s" % type(op).__name__,
+                         self.laid_out_size(out))
+        self.add_counter("output_unique/%s" % type(op).__name__, out.size)
+
+  def run(self, feeds=None):
+    """Executes the graph's non-variable operations again.  `feeds` maps
+    imported Tensors to new torch tensors of the same shape."""
+    self._feeds = dict(feeds or {})
+    try:
+      for op in self.graph.operations:
+        if not isinstance(op, Variable):
+          op.lower(self)
+    finally:
+      self._feeds = {}
+
+  def fed_value(self, tensor, default):
+    return self._feeds.get(tensor, default)
+
+  def mesh_impl(self, m):
+    if not isinstance(m, Mesh):
+      m = m.mesh
+    return self.mesh_to_impl[m]
+
+  def export_to_tf_tensor(self, x):
+    """Tensor -> torch tensor (the name is the reference's)."""
+    mesh_impl = self.mesh_impl(x)
+    return mesh_impl.export_to_tf_tensor(
+        x, self.tensors[x].to_laid_out_tensor())
+
+  export_to_torch = export_to_tf_tensor
+
+  def lowered_operation(self, op):
+    return self.operations[op]
+
+  def copy_masters_to_slices(self):
+    for v in self.variables.values():
+      v.copy_master_to_slices()
+
+  def copy_slices_to_masters(self):
+    for v in self.variables.values():
+      v.copy_slices_to_master()
+
+  def add_counter(self, key, value):
+    assert isinstance(value, int)
+    self._counters.append((key, value))
+
+  @property
+  def counters(self):
+    return self._counters
+
+  def laid_out_size(self, tensor):
+    return self.mesh_impl(tensor).laid_out_size(tensor.shape)
+
+  def set_tensor_lowering(self, tensor, laid_out_tensor):
+    self.verify_slice_shapes(tensor, laid_out_tensor)
+    self.tensors[tensor] = laid_out_tensor
+
+  def verify_slice_shapes(self, tensor, laid_out_tensor):
+    correct_shape = self.mesh_impl(tensor).slice_shape(tensor.shape)
+    actual_shape = list(laid_out_tensor.slice_shape)
+    if actual_shape != correct_shape:
+      raise ValueError(
+          "Wrong slice shape: correct_shape = %s actual shape = %s"
+          % (correct_shape, actual_shape))
+
+
+# ----------------------------------------------------------------------------
+# operations
+# ----------------------------------------------------------------------------
+class SlicewiseOperation(Operation):
+  """Applies a torch function to the slices (mesh_tensorflow/ops.py:1651-1723).
+  `tf_fn` maps input slices to one output slice or a tuple of them."""
+
+  def __init__(self, tf_fn, inputs, output_shapes, output_dtypes,
+               splittable_dims=None, grad_function=None, name=None):
+    super(SlicewiseOperation, self).__init__(inputs, name=name or "slicewise")
+    del splittable_dims, grad_function
+    self._tf_fn = tf_fn
+    self._outputs = [Tensor(self, convert_to_shape(s), d, index=i)
+                     for i, (s, d) in enumerate(zip(output_shapes,
+                                                    output_dtypes))]
+
+  def lower(self, lowering):
+    mesh_impl = lowering.mesh_impl(self)
+    values = mesh_impl.slicewise(
+        self._tf_fn, *[lowering.tensors[x] for x in self.inputs])
+    if len(self.outputs) == 1 and not isinstance(values, tuple):
+      values = (values,)
+    for out, v in zip(self.outputs, values):
+      lowering.set_tensor_lowering(out, v)
+
+
+def slicewise(tf_fn, xs, output_shape=None, output_dtype=None,
+              splittable_dims=None, grad_function=None, name=None):
+  """mtf.slicewise (mesh_tensorflow/ops.py:1726-1763)."""
+  multiple = isinstance(output_shape, list)
+  shapes = output_shape if multiple else [output_shape or xs[0].shape]
+  dtypes = output_dtype if multiple else [output_dtype or xs[0].dtype]
+  outs = SlicewiseOperation(tf_fn, xs, shapes, dtypes, splittable_dims,
+                            grad_function, name=name).outputs
+  return tuple(outs) if multiple else outs[0]
+
+
+def cwise(tf_fn, xs, output_dtype=None, grad_function=None, name=None):
+  return slicewise(tf_fn, xs, output_dtype=output_dtype,
+                   grad_function=grad_function, name=name or "cwise")
+
+
+def cast(x, dtype, name="cast"):
+  if dtype == x.dtype:
+    return x
+  return cwise(lambda t: t.to(dtype), [x], output_dtype=dtype, name=name)
+
+
+def to_float(x, name="to_float"):
+  return cast(x, float32, name=name)
+
+
+def to_bfloat16(x, name="to_bfloat16"):
+  return cast(x, bfloat16, name=name)
+
+
+def _scalar_in(dtype, value):
+  """A Python scalar as the reference's scalar ops see it: rounded to the
+  tensor's dtype first."""
+  return torch.tensor(value, dtype=dtype).item()
+
+
+def add(x1, x2, output_shape=None, name=None):
+  """Tensor + scalar, or Tensor + Tensor with broadcasting of x2's dims that
+  are a subsequence of x1's (all the MoE layers need)."""
+  del output_shape
+  if not isinstance(x2, Tensor):
+    c = _scalar_in(x1.dtype, x2)
+    return cwise(lambda t: t + c, [x1], name=name or "scalar_add")
+  if not isinstance(x1, Tensor):
+    return add(x2, x1)
+  big, small = (x1, x2) if x1.shape.ndims >= x2.shape.ndims else (x2, x1)
+  names = big.shape.dimension_names
+  if any(d not in big.shape.dims for d in small.shape.dims):
+    raise ValueError("cannot broadcast %s to %s" % (small.shape, big.shape))
+  view = [d.size if d in small.shape.dims else 1 for d in big.shape.dims]
+  order = [names.index(d.name) for d in small.shape.dims]
+  if order != sorted(order):
+    raise ValueError("dimension order differs: %s vs %s"
+                     % (small.shape, big.shape))
+
+  def fn(a, b):
+    return a + b.reshape(view).to(a.dtype)
+  return slicewise(fn, [big, small], output_shape=big.shape,
+                   output_dtype=big.dtype, name=name or "add")
+
+
+def multiply(x1, x2, output_shape=None, name=None):
+  """Tensor * Python scalar (ScalarMultiplyOperation,
+  mesh_tensorflow/ops.py:2006-2023)."""
+  del output_shape
+  if isinstance(x2, Tensor) and not isinstance(x1, Tensor):
+    x1, x2 = x2, x1
+  if isinstance(x2, Tensor):
+    raise NotImplementedError("Tensor * Tensor is not part of this subset")
+  c = _scalar_in(x1.dtype, x2)
+  return cwise(lambda t: t * c, [x1], name=name or "scalar_mul")
+
+
+class ReshapeOperation(Operation):
+  """Reshape to a Shape of equal size (mesh_tensorflow/ops.py:4477-4580); on a
+  single device this is a view."""
+
+  def __init__(self, x, new_shape, name=None):
+    super(ReshapeOperation, self).__init__([x], name=name or "reshape")
+    if x.shape.size != new_shape.size:
+      raise ValueError("Cannot reshape Tensor %s to shape %s - sizes differ."
+                       % (x, new_shape))
+    self._outputs = [Tensor(self, new_shape, x.dtype)]
+
+  def lower(self, lowering):
+    mesh_impl = lowering.mesh_impl(self)
+    new_shape = self.outputs[0].shape
+    if mesh_impl.size != 1:
+      raise NotImplementedError("reshape across a split mesh dimension")
+    sizes = new_shape.to_integer_list
+    lowering.set_tensor_lowering(
+        self.outputs[0],
+        mesh_impl.slicewise(lambda t: t.reshape(sizes),
+                            lowering.tensors[self.inputs[0]]))
+
+
+def reshape(x, new_shape, name="reshape"):
+  new_shape = convert_to_shape(new_shape)
+  if new_shape == x.shape:
+    return x
+  return ReshapeOperation(x, new_shape, name=name).outputs[0]
+
+
+def rename_dimension(x, old_name, new_name):
+  return reshape(x, x.shape.rename_dimension(old_name, new_name))
+
+
+class ImportOperation(Operation):
+  """Brings a torch tensor into the graph (mesh_tensorflow/ops.py:3854-3875)."""
+
+  def __init__(self, mesh, tf_tensor, shape, name=None):
+    super(ImportOperation, self).__init__([], mesh=mesh, name=name or "import")
+    tf_tensor = torch.as_tensor(tf_tensor)
+    if list(tf_tensor.shape) != shape.to_integer_list:
+      raise ValueError("Incompatible shape; have %s, want %s"
+                       % (list(tf_tensor.shape), shape))
+    self._outputs = [Tensor(self, shape, tf_tensor.dtype)]
+    self._tf_tensor = tf_tensor
+
+  def lower(self, lowering):
+    mesh_impl = lowering.mesh_impl(self)
+    value = lowering.fed_value(self.outputs[0], self._tf_tensor)
+    lowering.set_tensor_lowering(
+        self.outputs[0], mesh_impl.import_tf_tensor(self.outputs[0], value))
+
+
+def import_tf_tensor(mesh, tf_tensor, shape=None, name=None):
+  """Torch tensor (or array) -> Tensor.  The name is the reference's."""
+  tf_tensor = torch.as_tensor(tf_tensor)
+  if shape is None:
+    shape = Shape([Dimension("anon_%d" % i, int(s))
+                   for i, s in enumerate(tf_tensor.shape)])
+  return ImportOperation(mesh, tf_tensor, convert_to_shape(shape),
+                         name=name).outputs[0]
+
+
+import_tensor = import_tf_tensor
+
+
+class Constant(Operation):
+  """A tensor filled with one value (mesh_tensorflow/ops.py:4337-4355)."""
+
+  def __init__(self, mesh, value, shape, dtype, name=None):
+    super(Constant, self).__init__([], mesh, name=name or "constant")
+    self._outputs = [Tensor(self, shape, dtype)]
+    self._value = value
+
+  def lower(self, lowering):
+    mesh_impl = lowering.mesh_impl(self)
+    out = self.outputs[0]
+    sizes = mesh_impl.slice_shape(out.shape)
+    lowering.set_tensor_lowering(
+        out, mesh_impl.slicewise(
+            lambda: torch.full(sizes, self._value, dtype=out.dtype,
+                               device=mesh_impl.device)))
+
+
+def constant(mesh, value, shape=None, dtype=float32):
+  return Constant(mesh, value, convert_to_shape(shape or []), dtype).outputs[0]
+
+
+def zeros(mesh, shape, dtype=float32):
+  return constant(mesh, 0, shape=convert_to_shape(shape), dtype=dtype)
+
+
+class VariableDType(object):
+  """master / slice / activation dtypes of a variable
+  (mesh_tensorflow/ops.py:3961-4003)."""
+
+  def __init__(self, master_dtype=float32, slice_dtype=None,
+               activation_dtype=None):
+    self._master_dtype = master_dtype
+    self._slice_dtype = slice_dtype or master_dtype
+    self._activation_dtype = activation_dtype or master_dtype
+
+  master_dtype = property(lambda self: self._master_dtype)
+  slice_dtype = property(lambda self: self._slice_dtype)
+  activation_dtype = property(lambda self: self._activation_dtype)
+
+
+class Variable(Operation):
+  """A named parameter (mesh_tensorflow/ops.py:4006-4093).  Lowering creates a
+  LaidOutVariable; its output is the slice cast to the activation dtype,
+  produced lazily so that consumers with their own packed copy never pay for
+  the cast."""
+
+  def __init__(self, mesh, name, shape, dtype, initializer, trainable,
+               **kwargs):
+    del kwargs
+    super(Variable, self).__init__([], mesh, name=name)
+    if not isinstance(dtype, VariableDType):
+      raise ValueError("dtype must be a VariableDType got %s" % dtype)
+    self._dtype = dtype
+    self._trainable = trainable
+    self._initializer = initializer
+    self._outputs = [Tensor(self, shape, dtype.activation_dtype)]
+    self.graph.all_variables.append(self)
+    if trainable:
+      self.graph.trainable_variables.append(self)
+
+  def __repr__(self):
+    return "Variable(%s)" % self.value
+
+  value = property(lambda self: self.outputs[0])
+  shape = property(lambda self: self.value.shape)
+  dtype = property(lambda self: self._dtype)
+  master_dtype = property(lambda self: self._dtype.master_dtype)
+  slice_dtype = property(lambda self: self._dtype.slice_dtype)
+  activation_dtype = property(lambda self: self._dtype.activation_dtype)
+  trainable = property(lambda self: self._trainable)
+  initializer = property(lambda self: self._initializer)
+
+  def lower(self, lowering):
+    mesh_impl = lowering.mesh_impl(self)
+    initial = lowering.initial_values.get(self.name)
+    sv = mesh_impl.LaidOutVariable(self, mesh_impl, initial_value=initial)
+    lowering.variables[self] = sv
+    lowering.set_tensor_lowering(self.outputs[0], sv.activation_tensor())
+    key = "variables/trainable" if self._trainable else "variables/untrainable"
+    lowering.add_counter(key, self.outputs[0].size)
+
+
+def get_variable(mesh, name, shape, dtype=float32, master_dtype=None,
+                 slice_dtype=None, activation_dtype=None, initializer=None,
+                 trainable=True, **kwargs):
+  """Creates a variable named `<scope>/<name>`
+  (mesh_tensorflow/ops.py:4160-4208).  Unlike the reference there is no reuse:
+  asking for an existing name raises."""
+  if dtype is None:
+    dtype = VariableDType(master_dtype, slice_dtype, activation_dtype)
+  elif isinstance(dtype, VariableDType):
+    if master_dtype or slice_dtype or activation_dtype:
+      raise ValueError("dtype is a VariableDType; do not also pass its parts")
+  else:
+    dtype = VariableDType(master_dtype or dtype, slice_dtype or dtype,
+                          activation_dtype or dtype)
+  scope = current_scope_name()
+  full = scope + "/" + name if scope else name
+  if any(v.name == full for v in mesh.graph.all_variables):
+    raise ValueError("Variable %s already exists" % full)
+  return Variable(mesh, name, convert_to_shape(shape), dtype, initializer,
+                  trainable, **kwargs).outputs[0]
+
+
+def relu(x, name="relu"):
+  return cwise(torch.relu, [x], name=name)
+
+
+def to_numpy(t):
+  """Torch tensor -> float32/int NumPy array on the host."""
+  t = t.detach()
+  if t.dtype == torch.bfloat16:
+    t = t.float()
+  return np.asarray(t.cpu())

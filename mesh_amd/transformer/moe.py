@@ -1,0 +1,578 @@
+"""Top-2 gated Mixture-of-Experts layers on HipMeshImpl.
+
+Same entry points, argument order, defaults, dimension names, variable names
+and error types as mesh_tensorflow/transformer/moe.py (MoE1D :37-128, MoE2D
+:131-188, transformer_moe_layer_v1 :191-525, transformer_moe_layer_v2
+:528-801, _split_into_groups :1549-1582, HParams :1585-1596).  Where the
+reference expands the layer into ~100 graph primitives and dense one-hot
+[G,S,E,C] tensors, each layer here is ONE Operation whose slice function calls
+the HIP kernels: router -> top-2 gating -> dispatch -> expert FFN -> combine.
+
+Built: moe_gating="top_2" with every second-place policy, nonpadding /
+importance, the second-place loss, float32 and bfloat16.  Not built (they
+raise NotImplementedError): the other routers of the reference's file,
+expert dropout while training, moe_use_experts_attention, gated (list)
+activations, and a mesh with more than one device.
+"""
+
+import torch
+
+from mesh_amd import layers as mtf_layers
+from mesh_amd import moe_hip
+from mesh_amd import ops as mtf
+
+_OTHER_GATINGS = ("switch", "ntlb", "switch_max", "expert_selection")
+
+
+class HParams(object):
+  """Attribute bag standing in for tf.contrib.training.HParams."""
+
+  def __init__(self, **kwargs):
+    for k, v in kwargs.items():
+      setattr(self, k, v)
+
+  def add_hparam(self, k, v):
+    setattr(self, k, v)
+
+
+def set_default_moe_hparams(hparams):
+  """Adds the reference's default MoE hyperparameters (moe.py:1516-1546)."""
+  hparams.moe_num_experts = 16
+  hparams.moe_loss_coef = 1e-2
+  hparams.add_hparam("moe_gating", "top_2")
+  hparams.add_hparam("moe_capacity_factor_train", 1.25)
+  hparams.add_hparam("moe_capacity_factor_eval", 2.0)
+  hparams.add_hparam("moe_capacity_factor_second_level", 1.0)
+  hparams.add_hparam("moe_hidden_size", 4096)
+  hparams.add_hparam("moe_group_size", 1024)
+  hparams.add_hparam("moe_use_second_place_loss", 0)
+  hparams.add_hparam("moe_second_policy_train", "random")
+  hparams.add_hparam("moe_second_policy_eval", "random")
+  hparams.add_hparam("moe_second_threshold_train", 0.2)
+  hparams.add_hparam("moe_second_threshold_eval", 0.2)
+
+
+def _split_into_groups(n, max_group_size, mesh_dim_size):
+  """n = num_groups * group_size with group_size the largest value that is
+  <= max_group_size and leaves num_groups a multiple of mesh_dim_size."""
+  if n % mesh_dim_size != 0:
+    raise ValueError(
+        "n=%d is not a multiple of mesh_dim_size=%d" % (n, mesh_dim_size))
+  num_groups = max(1, n // max_group_size)
+  while num_groups % mesh_dim_size != 0 or n % num_groups != 0:
+    num_groups += 1
+  return num_groups, n // num_groups
+
+
+def _expert_capacity(group_size, capacity_factor, num_experts, min_capacity):
+  """Slots per expert per group (moe.py:368-371)."""
+  capacity = min(group_size, int((group_size * capacity_factor) / num_experts))
+  return max(capacity, min_capacity)
+
+
+def _activation_name(activation):
+  """mtf.relu / "relu" / None / "linear" -> name understood by the kernels."""
+  if isinstance(activation, (list, tuple)):
+    if len(activation) != 1:
+      raise NotImplementedError(
+          "products of several dense layers (gated activations) are not "
+          "implemented: %r" % (activation,))
+    activation = activation[0]
+  if activation is None or activation == "linear":
+    return "linear"
+  name = activation if isinstance(activation, str) else getattr(
+      activation, "__name__", None)
+  if name not in moe_hip.ACTIVATIONS:
+    raise NotImplementedError("expert activation %r is not implemented"
+                              % (activation,))
+  return name
+
+
+def _check_gating(hparams):
+  if hparams.moe_gating == "top_2":
+    return
+  if hparams.moe_gating in _OTHER_GATINGS:
+    raise NotImplementedError(
+        "moe_gating=%s is not implemented (top_2 only)" % hparams.moe_gating)
+  raise ValueError("unknown hparams.moe_gating=%s" % hparams.moe_gating)
+
+
+def _second_policy(hparams, train):
+  if train:
+    policy = hparams.moe_second_policy_train
+    threshold = hparams.moe_second_threshold_train
+  else:
+    policy = hparams.moe_second_policy_eval
+    threshold = hparams.moe_second_threshold_eval
+  if policy not in moe_hip.POLICIES:
+    raise ValueError("Unknown policy %s" % policy)
+  return policy, threshold
+
+
+class _GatingSpec(object):
+  """Static configuration of one _top_2_gating call (moe.py:1312-1513)."""
+
+  def __init__(self, hparams, train, num_microbatches):
+    self.policy, self.threshold = _second_policy(hparams, train)
+    self.use_second_place_loss = bool(hparams.moe_use_second_place_loss)
+    self.num_microbatches = num_microbatches
+
+  def run(self, logits, capacity, importance=None,
+          importance_from_slot_gate=False):
+    uniform = None
+    if self.policy == "random":
+      uniform = torch.rand(logits.shape[:2], dtype=torch.float32,
+                           device=logits.device)
+    return moe_hip.top2_gating(
+        logits, capacity, importance=importance, policy=self.policy,
+        threshold=self.threshold,
+        use_second_place_loss=self.use_second_place_loss,
+        num_microbatches=self.num_microbatches, second_uniform=uniform,
+        importance_from_slot_gate=importance_from_slot_gate)
+
+
+def _packed(lowering, kernel_tensor, dtype):
+  """K-contiguous copy of an expert kernel variable, cached on the variable."""
+  return lowering.variables[kernel_tensor.operation].packed(dtype)
+
+
+class MoEV1Operation(mtf.Operation):
+  """The whole of transformer_moe_layer_v1 after the reshape to groups:
+  inputs [outer_batch, groups, group, d_model] -> (outputs with d_model
+  replaced by output_dim, scalar balancing loss before moe_loss_coef)."""
+
+  def __init__(self, inputs, w_gate, wi, wo, importance, output_dim, capacity,
+               gating, activation, name="moe_v1"):
+    ins = [inputs, w_gate, wi, wo] + ([importance] if importance is not None
+                                      else [])
+    super(MoEV1Operation, self).__init__(ins, name=name)
+    self._has_importance = importance is not None
+    self._capacity = capacity
+    self._gating = gating
+    self._activation = activation
+    self._num_experts = wi.shape.dims[0].size
+    out_shape = mtf.Shape(inputs.shape.dims[:-1] + [output_dim])
+    self._outputs = [mtf.Tensor(self, out_shape, inputs.dtype, index=0),
+                     mtf.Tensor(self, mtf.Shape([]), inputs.dtype, index=1)]
+
+  def lower(self, lowering):
+    mesh_impl = lowering.mesh_impl(self)
+    x, w_gate, wi, wo = self.inputs[:4]
+    dt = x.dtype
+    wi_p = _packed(lowering, wi, dt)
+    wo_p = _packed(lowering, wo, dt)
+    o_, g_, s_, m_ = x.shape.to_integer_list
+    n_ = self.outputs[0].shape.dims[-1].size
+    e_, c_ = self._num_experts, self._capacity
+    groups = o_ * g_
+
+    def fn(x_s, wg_s, imp_s=None):
+      xg = x_s.reshape(groups, s_, m_)
+      logits = moe_hip.router_logits(xg.reshape(groups * s_, m_), wg_s)
+      if imp_s is not None:
+        imp_s = imp_s.reshape(groups, s_)
+      r = self._gating.run(logits.reshape(groups, s_, e_), c_, imp_s)
+      expert_in = moe_hip.dispatch(xg, r)
+      y = moe_hip.expert_ffn(expert_in.reshape(e_, groups * c_, m_), wi_p,
+                             wo_p, self._activation)
+      out = moe_hip.combine(y.reshape(e_, groups, c_, n_), r, s_)
+      return out.reshape(o_, g_, s_, n_), r.loss.to(dt).reshape(())
+
+    args = [lowering.tensors[x], lowering.tensors[w_gate]]
+    if self._has_importance:
+      args.append(lowering.tensors[self.inputs[4]])
+    out, loss = mesh_impl.slicewise(fn, *args)
+    lowering.set_tensor_lowering(self.outputs[0], out)
+    lowering.set_tensor_lowering(self.outputs[1], loss)
+
+
+def transformer_moe_layer_v1(
+    inputs, output_dim, hparams, train, variable_dtype,
+    layout=None, mesh_shape=None, nonpadding=None, activation=mtf.relu,
+    num_microbatches=None):
+  """Local mixture of experts: each position goes to 0-2 experts chosen by a
+  learned top-2 gate, with a fixed per-group capacity per expert.
+
+  Args:
+    inputs: a mtf.Tensor with shape [batch_dim(s), length_dim, input_dim]
+    output_dim: a mtf.Dimension (for Transformer, this is input_dim)
+    hparams: model hyperparameters (moe_num_experts, moe_hidden_size,
+      moe_group_size, moe_capacity_factor_train/eval, moe_min_expert_capacity,
+      moe_gating, moe_dropout_rate, moe_use_experts_attention, moe_loss_coef,
+      moe_use_second_place_loss, moe_second_policy_train/eval,
+      moe_second_threshold_train/eval)
+    train: a boolean
+    variable_dtype: a mtf.VariableDType
+    layout: optional - an input to mtf.convert_to_layout_rules
+    mesh_shape: optional - an input to mtf.convert_to_shape
+    nonpadding: an optional Tensor with shape [batch_dim(s), length_dim]
+      and the same dtype as inputs, consisting of ones(nonpadding)
+      and zeros(padding).
+    activation: a function, or the name of one.
+    num_microbatches: number of microbatches.
+
+  Returns:
+    outputs: a Tensor with shape [batch_dim(s), length_dim, output_dim]
+    loss: a mtf scalar
+
+  Raises:
+    ValueError: on unrecognized hparams.moe_gating
+  """
+  orig_inputs = inputs
+  hidden_dim = mtf.Dimension("expert_hidden", hparams.moe_hidden_size)
+  experts_dim = mtf.Dimension("experts", hparams.moe_num_experts)
+  batch_and_length_dims = orig_inputs.shape.dims[:-1]
+  input_dim = orig_inputs.shape.dims[-1]
+  if orig_inputs.shape.dims[0].name == "outer_batch":
+    outer_batch_dim, orig_batch_dim = orig_inputs.shape.dims[:2]
+  else:
+    outer_batch_dim = mtf.Dimension("outer_batch", 1)
+    orig_batch_dim = orig_inputs.shape.dims[0]
+
+  n = mtf.list_product(d.size for d in batch_and_length_dims)
+  n = n // outer_batch_dim.size
+  mesh_dim_size = mtf.tensor_dim_to_mesh_dim_size(layout, mesh_shape,
+                                                  orig_batch_dim)
+  num_groups, group_size = _split_into_groups(n, hparams.moe_group_size,
+                                              mesh_dim_size)
+  group_size_dim = mtf.Dimension("group", group_size)
+  num_groups_dim = mtf.Dimension(orig_batch_dim.name, num_groups)
+  moe_input_dims = [outer_batch_dim, num_groups_dim, group_size_dim, input_dim]
+  inputs = mtf.reshape(inputs, moe_input_dims)
+
+  capacity_factor = (hparams.moe_capacity_factor_train if train
+                     else hparams.moe_capacity_factor_eval)
+  expert_capacity = _expert_capacity(group_size_dim.size, capacity_factor,
+                                     experts_dim.size,
+                                     hparams.moe_min_expert_capacity)
+  experts_dim_unsplit = mtf.Dimension("expert_unsplit", experts_dim.size)
+  if nonpadding is not None:
+    nonpadding = mtf.zeros(
+        inputs.mesh, batch_and_length_dims, dtype=inputs.dtype) + nonpadding
+    nonpadding = mtf.reshape(nonpadding, moe_input_dims[:-1])
+
+  _check_gating(hparams)
+  if hparams.moe_dropout_rate != 0.0 and train:
+    raise NotImplementedError("expert dropout while training is not "
+                              "implemented (moe_dropout_rate must be 0)")
+  if hparams.moe_use_experts_attention:
+    raise NotImplementedError("moe_use_experts_attention is not implemented")
+  gating = _GatingSpec(hparams, train, num_microbatches)
+  act_name = _activation_name(activation)
+
+  # variables, named and shaped as the reference's dense layers create them
+  w_gate = mtf_layers.get_dense_kernel_weights(
+      inputs, [experts_dim_unsplit], [input_dim], [], None,
+      name="top_2_gating", variable_dtype=variable_dtype)
+  wi = mtf_layers.get_dense_kernel_weights(
+      inputs, [hidden_dim], [input_dim], [experts_dim], None, name="wi",
+      variable_dtype=variable_dtype)
+  wo = mtf_layers.get_dense_kernel_weights(
+      inputs, [output_dim], [hidden_dim], [experts_dim], None, name="wo",
+      variable_dtype=variable_dtype)
+
+  output, loss = MoEV1Operation(
+      inputs, w_gate, wi, wo, nonpadding, output_dim, expert_capacity, gating,
+      act_name).outputs
+  output = mtf.reshape(output, batch_and_length_dims + [output_dim])
+  return output, loss * hparams.moe_loss_coef
+
+
+class MoEV2Operation(mtf.Operation):
+  """The whole of transformer_moe_layer_v2 after the reshape to groups:
+  inputs [a0, g1, s, m] -> (outputs [a0, g1, s, n], loss_outer + loss_inner).
+
+  Level 1 routes tokens to expert groups x with capacity c; the occupied slots
+  of each x, taken in (a0, g, c) order, are regrouped into h0 groups of t and
+  routed again to experts y with capacity d, with importance 1.0 for slots
+  holding a first choice, 0.5 for a second choice and 0 for empty slots
+  (moe.py:692-801)."""
+
+  def __init__(self, inputs, w_outer, w_inner, wi, wo, importance, output_dim,
+               dims, gating, name="moe_v2"):
+    ins = [inputs, w_outer, w_inner, wi, wo] + (
+        [importance] if importance is not None else [])
+    super(MoEV2Operation, self).__init__(ins, name=name)
+    self._has_importance = importance is not None
+    self._dims = dims
+    self._gating = gating
+    out_shape = mtf.Shape(inputs.shape.dims[:-1] + [output_dim])
+    self._outputs = [mtf.Tensor(self, out_shape, inputs.dtype, index=0),
+                     mtf.Tensor(self, mtf.Shape([]), inputs.dtype, index=1)]
+
+  def lower(self, lowering):
+    mesh_impl = lowering.mesh_impl(self)
+    x, w_outer, w_inner, wi, wo = self.inputs[:5]
+    dt = x.dtype
+    wi_p = _packed(lowering, wi, dt)      # [y*x, hidden, m]
+    wo_p = _packed(lowering, wo, dt)      # [y*x, n, hidden]
+    a0, g1, s_, m_ = x.shape.to_integer_list
+    n_ = self.outputs[0].shape.dims[-1].size
+    x_e, y_e, c_, h0, t_, d_ = self._dims
+    ag = a0 * g1
+
+    def fn(x_s, wo_s, wi_s, imp_s=None):
+      xg = x_s.reshape(ag, s_, m_)
+      # outer level
+      logits_x = moe_hip.router_logits(xg.reshape(ag * s_, m_), wo_s)
+      if imp_s is not None:
+        imp_s = imp_s.reshape(ag, s_)
+      rx = self._gating.run(logits_x.reshape(ag, s_, x_e), c_, imp_s)
+      ein_x, slot_gate = moe_hip.dispatch(xg, rx, want_slot_gate=True)
+      # inner level: each outer expert's a0*g*c slots become h0 groups of t
+      inputs_y = ein_x.reshape(x_e, h0 * t_, m_)
+      logits_y = moe_hip.router_logits(inputs_y, wi_s)      # [x, h0*t, y]
+      ry = self._gating.run(logits_y.reshape(x_e * h0, t_, y_e), d_,
+                            slot_gate.reshape(x_e * h0, t_),
+                            importance_from_slot_gate=True)
+      ein_y = moe_hip.dispatch(inputs_y.reshape(x_e * h0, t_, m_), ry)
+      # experts: weights are [y, x, ...]; rows of (y, x) are its h0*d slots
+      yy = moe_hip.expert_ffn(ein_y.reshape(y_e * x_e, h0 * d_, m_), wi_p,
+                              wo_p, "relu")
+      out_y = moe_hip.combine(yy.reshape(y_e, x_e * h0, d_, n_), ry, t_)
+      out = moe_hip.combine(out_y.reshape(x_e, ag, c_, n_), rx, s_)
+      loss = (rx.loss.to(dt) + ry.loss.to(dt)).reshape(())
+      return out.reshape(a0, g1, s_, n_), loss
+
+    args = [lowering.tensors[x], lowering.tensors[w_outer],
+            lowering.tensors[w_inner]]
+    if self._has_importance:
+      args.append(lowering.tensors[self.inputs[5]])
+    out, loss = mesh_impl.slicewise(fn, *args)
+    lowering.set_tensor_lowering(self.outputs[0], out)
+    lowering.set_tensor_lowering(self.outputs[1], loss)
+
+
+def transformer_moe_layer_v2(
+    inputs, output_dim, hparams, train, variable_dtype,
+    layout=None, mesh_shape=None, nonpadding=None, num_microbatches=None):
+  """2-level mixture of experts: hparams.moe_num_experts = [x, y]; a position
+  goes to up to two expert groups and, inside each, to up to two experts
+  (one for its second-choice group).
+
+  Args:
+    inputs: a mtf.Tensor with shape [a, b, l, m] (or [b, l, m])
+    output_dim: a mtf.Dimension (for Transformer, this is input_dim)
+    hparams: model hyperparameters (those of transformer_moe_layer_v1 plus
+      moe_capacity_factor_second_level)
+    train: a boolean
+    variable_dtype: a mtf.VariableDType
+    layout: optional - an input to mtf.convert_to_layout_rules
+    mesh_shape: optional - an input to mtf.convert_to_shape
+    nonpadding: an optional mtf.Tensor with shape [a, b, l]
+      and the same dtype as inputs, consisting of ones(nonpadding)
+      and zeros(padding).
+    num_microbatches: number of microbatches.
+
+  Returns:
+    outputs: a Tensor with shape [a, b, l, n]
+    loss: a mtf scalar
+
+  Raises:
+    ValueError: on unrecognized hparams.moe_gating
+  """
+  if nonpadding is not None:
+    nonpadding = mtf.zeros(inputs.mesh, inputs.shape.dims[:-1],
+                           dtype=inputs.dtype) + nonpadding
+  insert_outer_batch_dim = (len(inputs.shape.dims) == 3)
+  if insert_outer_batch_dim:
+    inputs = mtf.reshape(
+        inputs, [mtf.Dimension("outer_batch", 1)] + inputs.shape.dims)
+
+  assert len(hparams.moe_num_experts) == 2
+  a0, b1, l, m = inputs.shape.dims
+  hidden_dim = mtf.Dimension("expert_hidden", hparams.moe_hidden_size)
+  x1 = mtf.Dimension("expert_x", hparams.moe_num_experts[0])
+  y0 = mtf.Dimension("expert_y", hparams.moe_num_experts[1])
+  x = mtf.Dimension("expert_x_unsplit", hparams.moe_num_experts[0])
+  y = mtf.Dimension("expert_y_unsplit", hparams.moe_num_experts[1])
+  n = output_dim
+
+  num_groups, group_size = _split_into_groups(
+      b1.size * l.size, hparams.moe_group_size,
+      mtf.tensor_dim_to_mesh_dim_size(layout, mesh_shape, b1))
+  g1 = mtf.Dimension(b1.name, num_groups)
+  s = mtf.Dimension("group_size_x", group_size)
+  capacity_factor = (hparams.moe_capacity_factor_train if train
+                     else hparams.moe_capacity_factor_eval)
+  c = mtf.Dimension("expert_capacity_x", _expert_capacity(
+      s.size, capacity_factor, x.size, hparams.moe_min_expert_capacity))
+
+  num_groups, group_size = _split_into_groups(
+      a0.size * g1.size * c.size, hparams.moe_group_size,
+      mtf.tensor_dim_to_mesh_dim_size(layout, mesh_shape, a0))
+  t = mtf.Dimension("group_size_y", group_size)
+  h0 = mtf.Dimension(a0.name, num_groups)
+  d = mtf.Dimension("expert_capacity_y", _expert_capacity(
+      t.size, hparams.moe_capacity_factor_second_level, y.size,
+      hparams.moe_min_expert_capacity))
+
+  inputs = mtf.reshape(inputs, [a0, g1, s, m])
+  if nonpadding is not None:
+    nonpadding = mtf.reshape(nonpadding, [a0, g1, s])
+
+  if hparams.moe_gating != "top_2":
+    raise ValueError("unknown hparams.moe_gating=%s" % hparams.moe_gating)
+  gating = _GatingSpec(hparams, train, num_microbatches)
+
+  w_outer = mtf_layers.get_dense_kernel_weights(
+      inputs, [x], [m], [], None, name="outer_gating",
+      variable_dtype=variable_dtype)
+  w_inner = mtf_layers.get_dense_kernel_weights(
+      inputs, [y], [m], [x1], None, name="inner_gating",
+      variable_dtype=variable_dtype)
+  wi = mtf_layers.get_dense_kernel_weights(
+      inputs, [hidden_dim], [m], [y0, x1], None, name="wi",
+      variable_dtype=variable_dtype)
+  wo = mtf_layers.get_dense_kernel_weights(
+      inputs, [n], [hidden_dim], [y0, x1], None, name="wo",
+      variable_dtype=variable_dtype)
+
+  output, loss = MoEV2Operation(
+      inputs, w_outer, w_inner, wi, wo, nonpadding, n,
+      (x.size, y.size, c.size, h0.size, t.size, d.size), gating).outputs
+  output = mtf.reshape(output, [a0, b1, l, n])
+  if insert_outer_batch_dim:
+    output = mtf.reshape(output, [b1, l, n])
+  return output, loss * hparams.moe_loss_coef
+
+
+class MoE1D(object):
+  """Mixture of Experts Layer (transformer layer adapter, moe.py:37-128)."""
+
+  def __init__(self,
+               num_experts=16,
+               loss_coef=1e-2,
+               hidden_size=4096,
+               group_size=1024,
+               capacity_factor_train=1.25,
+               capacity_factor_eval=2.0,
+               use_second_place_loss=False,
+               second_policy_train="random",
+               second_policy_eval="random",
+               second_threshold_train=0.2,
+               second_threshold_eval=0.2,
+               dropout_rate=0.0,
+               activation="relu",
+               moe_gating="top_2",
+               min_expert_capacity=4,
+               switch_policy_train="input_jitter",
+               switch_policy_eval="input_jitter",
+               switch_dropout=0.1,
+               switch_temperature=1.0,
+               switch_jitter=1e-2,
+               ntlb_top_k=4,
+               output_dim=None,
+               use_experts_attention=False,
+               z_loss=None):
+    self._hparams = HParams(
+        moe_gating=moe_gating,
+        moe_num_experts=num_experts,
+        moe_loss_coef=loss_coef,
+        moe_hidden_size=hidden_size,
+        moe_group_size=group_size,
+        moe_min_expert_capacity=min_expert_capacity,
+        moe_capacity_factor_train=capacity_factor_train,
+        moe_capacity_factor_eval=capacity_factor_eval,
+        moe_use_second_place_loss=use_second_place_loss,
+        moe_second_policy_train=second_policy_train,
+        moe_second_policy_eval=second_policy_eval,
+        moe_second_threshold_train=second_threshold_train,
+        moe_second_threshold_eval=second_threshold_eval,
+        moe_dropout_rate=dropout_rate,
+        moe_switch_policy_train=switch_policy_train,
+        moe_switch_policy_eval=switch_policy_eval,
+        moe_switch_dropout=switch_dropout,
+        moe_switch_temperature=switch_temperature,
+        moe_switch_jitter=switch_jitter,
+        moe_output_dim=output_dim,
+        moe_ntlb_top_k=ntlb_top_k,
+        moe_use_experts_attention=use_experts_attention,
+        moe_z_loss=z_loss)
+    self._activation = activation
+
+  def call(self, context, x, losses=None):
+    """Call the layer.  `context` supplies model.ensemble_dim, length_dim,
+    model.model_dim/layout/mesh_shape, train, variable_dtype, nonpadding,
+    num_microbatches and the `losses` list the balancing loss is appended to."""
+    del losses
+    if context.model.ensemble_dim:
+      raise NotImplementedError("MoE not yet implemented with ensembles")
+    has_length_dim = context.length_dim in x.shape.dims
+    if not has_length_dim:
+      x_shape = x.shape
+      shape_with_length = mtf.Shape(
+          x_shape.dims[:-1] + [mtf.Dimension("length", 1)] + x_shape.dims[-1:])
+      x = mtf.reshape(x, shape_with_length)
+    if self._hparams.moe_output_dim is not None:
+      output_dim = self._hparams.moe_output_dim
+    else:
+      output_dim = context.model.model_dim
+    y, loss = transformer_moe_layer_v1(
+        x, output_dim, self._hparams, context.train, context.variable_dtype,
+        layout=context.model.layout, mesh_shape=context.model.mesh_shape,
+        nonpadding=context.nonpadding, activation=self._activation,
+        num_microbatches=context.num_microbatches)
+    if context.losses is not None:
+      context.losses.append(loss)
+    if not has_length_dim:
+      y = mtf.reshape(y, x_shape)
+    return y
+
+
+class MoE2D(object):
+  """Hierarchical Mixture of Experts Layer (moe.py:131-188).  Unlike the
+  reference's constructor this one also sets moe_min_expert_capacity (= 4, the
+  MoE1D default), which transformer_moe_layer_v2 reads."""
+
+  def __init__(self,
+               expert_x=8,
+               expert_y=8,
+               loss_coef=1e-2,
+               hidden_size=4096,
+               group_size=1024,
+               capacity_factor_train=1.25,
+               capacity_factor_eval=2.0,
+               capacity_factor_second_level=1.0,
+               use_second_place_loss=False,
+               second_policy_train="random",
+               second_policy_eval="random",
+               second_threshold_train=0.2,
+               second_threshold_eval=0.2):
+    self._hparams = HParams(
+        moe_gating="top_2",
+        moe_num_experts=[expert_x, expert_y],
+        moe_loss_coef=loss_coef,
+        moe_hidden_size=hidden_size,
+        moe_group_size=group_size,
+        moe_min_expert_capacity=4,
+        moe_capacity_factor_train=capacity_factor_train,
+        moe_capacity_factor_eval=capacity_factor_eval,
+        moe_capacity_factor_second_level=capacity_factor_second_level,
+        moe_use_second_place_loss=use_second_place_loss,
+        moe_second_policy_train=second_policy_train,
+        moe_second_policy_eval=second_policy_eval,
+        moe_second_threshold_train=second_threshold_train,
+        moe_second_threshold_eval=second_threshold_eval)
+
+  def call(self, context, x, losses=None):
+    """Call the layer."""
+    del losses
+    if context.model.ensemble_dim:
+      raise NotImplementedError("MoE not yet implemented with ensembles")
+    has_length_dim = context.length_dim in x.shape.dims
+    if not has_length_dim:
+      x_shape = x.shape
+      shape_with_length = mtf.Shape(
+          x_shape.dims[:-1] + [mtf.Dimension("length", 1)] + x_shape.dims[-1:])
+      x = mtf.reshape(x, shape_with_length)
+    y, loss = transformer_moe_layer_v2(
+        x, context.model.model_dim, self._hparams, context.train,
+        context.variable_dtype, layout=context.model.layout,
+        mesh_shape=context.model.mesh_shape, nonpadding=context.nonpadding,
+        num_microbatches=context.num_microbatches)
+    if context.losses is not None:
+      context.losses.append(loss)
+    if not has_length_dim:
+      y = mtf.reshape(y, x_shape)
+    return y

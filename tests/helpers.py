@@ -77,3 +77,37 @@ def assert_routing_equal(got, want, gate_rtol=1e-5):
   for k in ("gate_1", "gate_2"):
     np.testing.assert_allclose(got[k], want[k], rtol=gate_rtol, atol=1e-7,
                                err_msg=k)
+
+
+def safe_tokens(rng, n_tok, m, w_gate, act_dtype, bias=None, min_gap=1e-3,
+                ones_column=False):
+  """x [n_tok, m] ~ N(0,1) in the activation dtype such that the router logits
+  x . w_gate (+ bias) have their three largest entries per token at least
+  `min_gap` apart (offending tokens are redrawn): the routing then does not
+  depend on the summation order of the router matmul."""
+  wg = O.cast_act(w_gate, act_dtype)
+  x = O.cast_act(rng.standard_normal((n_tok, m)).astype(np.float32), act_dtype)
+  k = min(3, wg.shape[1])
+  for _ in range(100):
+    logits = O.router_logits(x, wg)
+    if bias is not None:
+      logits = logits + bias
+    top = -np.sort(-logits, axis=-1)[..., :k]
+    bad = ((top[..., :-1] - top[..., 1:]) < min_gap).any(axis=-1)
+    if not bad.any():
+      return x
+    x[bad] = O.cast_act(
+        rng.standard_normal((int(bad.sum()), m)).astype(np.float32), act_dtype)
+  raise AssertionError("could not separate the router logits")
+
+
+def normal_weights(rng, shape, fan_in):
+  return (rng.standard_normal(shape) / np.sqrt(fan_in)).astype(np.float32)
+
+
+def value_tolerance(act_dtype):
+  """Output tolerance of the layer: rtol 1e-4 for float32 (plus an absolute
+  floor for entries that cancel to ~0), rtol 2e-2 / atol 1e-2 for bfloat16."""
+  if act_dtype == "bfloat16":
+    return dict(rtol=2e-2, atol=1e-2)
+  return dict(rtol=1e-4, atol=2e-5)

@@ -1,0 +1,241 @@
+"""End-to-end GPU parity of the layers, called through the mtf-shaped API on
+HipMeshImpl, against the CPU oracle on the same seeded inputs."""
+
+import numpy as np
+import pytest
+import torch
+
+import mesh_amd as mtf
+from mesh_amd.transformer import moe
+from oracle import moe_oracle as O
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+def make_hparams(**kw):
+  hp = dict(
+      moe_gating="top_2", moe_num_experts=8, moe_loss_coef=1e-2,
+      moe_hidden_size=64, moe_group_size=32, moe_min_expert_capacity=4,
+      moe_capacity_factor_train=1.25, moe_capacity_factor_eval=2.0,
+      moe_capacity_factor_second_level=1.0, moe_use_second_place_loss=False,
+      moe_second_policy_train="all", moe_second_policy_eval="all",
+      moe_second_threshold_train=0.2, moe_second_threshold_eval=0.2,
+      moe_dropout_rate=0.0, moe_use_experts_attention=False)
+  hp.update(kw)
+  return moe.HParams(**hp), O.HParams(**hp)
+
+
+def run_v1(x, weights, hp, train, act_dtype, nonpadding=None, activation="relu",
+           num_microbatches=None, variable_dtype=None):
+  """x: float32 array [batch, length, M] of activation-dtype values."""
+  dt = H.ACT_TORCH[act_dtype]
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  b, l, m = x.shape
+  dims = [mtf.Dimension("batch", b), mtf.Dimension("length", l),
+          mtf.Dimension("d_model", m)]
+  xt = mtf.import_tf_tensor(mesh, torch.from_numpy(x).to(dt), mtf.Shape(dims))
+  npad = None
+  if nonpadding is not None:
+    npad = mtf.import_tf_tensor(mesh, torch.from_numpy(nonpadding).to(dt),
+                                mtf.Shape(dims[:2]))
+  n = weights["wo"].shape[-1]
+  vdt = variable_dtype or mtf.VariableDType(torch.float32, torch.float32, dt)
+  with mtf.variable_scope("moe"):
+    y, loss = moe.transformer_moe_layer_v1(
+        xt, mtf.Dimension("d_model", n), hp, train, vdt, nonpadding=npad,
+        activation=activation, num_microbatches=num_microbatches)
+  init = {"moe/top_2_gating/kernel": weights["w_gate"],
+          "moe/wi/kernel": weights["wi"], "moe/wo/kernel": weights["wo"]}
+  lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()}, initial_values=init)
+  out = H.to_np(lowering.export_to_tf_tensor(y))
+  return out, float(H.to_np(lowering.export_to_tf_tensor(loss))), lowering, (xt, y)
+
+
+V1_CASES = [
+    # name, batch, length, M, H, E, group, cf, dtype
+    ("tiny_f32", 2, 64, 16, 64, 8, 32, 1.25, "float32"),
+    ("tiny_bf16", 2, 64, 16, 64, 8, 32, 1.25, "bfloat16"),
+    ("ragged_f32", 3, 50, 24, 40, 5, 64, 1.0, "float32"),
+    ("cfg1_f32", 2, 1024, 512, 2048, 8, 1024, 1.25, "float32"),
+    ("cfg2_quarter_bf16", 4, 1024, 1024, 4096, 32, 1024, 1.25, "bfloat16"),
+]
+
+
+@pytest.mark.parametrize("case", V1_CASES, ids=[c[0] for c in V1_CASES])
+def test_v1_matches_oracle(case):
+  _, b, l, m, hdim, e, group, cf, act_dtype = case
+  rng = np.random.default_rng(101)
+  w = dict(w_gate=H.normal_weights(rng, (m, e), m),
+           wi=H.normal_weights(rng, (e, m, hdim), m),
+           wo=H.normal_weights(rng, (e, hdim, m), hdim))
+  x = H.safe_tokens(rng, b * l, m, w["w_gate"], act_dtype).reshape(b, l, m)
+  hp, ohp = make_hparams(moe_num_experts=e, moe_hidden_size=hdim,
+                         moe_group_size=group, moe_capacity_factor_train=cf)
+  got, got_loss, _, _ = run_v1(x, w, hp, True, act_dtype)
+  want, want_loss, aux = O.moe_layer_v1(x, w["w_gate"], w["wi"], w["wo"], ohp,
+                                        True, act_dtype, dense=b * l <= 4096)
+  assert aux["kept_1"].mean() < 1.0 or cf > 1.2   # the drop path is exercised
+  np.testing.assert_allclose(got, want, **H.value_tolerance(act_dtype))
+  np.testing.assert_allclose(got_loss, want_loss,
+                             rtol=1e-2 if act_dtype == "bfloat16" else 1e-5)
+
+
+def test_v1_skewed_routing_drops_tokens():
+  """Capacity factor 1.0 with a Zipf-biased router (folded into the router
+  weights through a constant input column) overflows the popular experts."""
+  b, l, m, hdim, e = 4, 512, 64, 128, 16
+  rng = np.random.default_rng(103)
+  w = dict(w_gate=H.normal_weights(rng, (m, e), m),
+           wi=H.normal_weights(rng, (e, m, hdim), m),
+           wo=H.normal_weights(rng, (e, hdim, m), hdim))
+  w["w_gate"][0] = H.zipf_bias(rng, e)
+  x = H.safe_tokens(rng, b * l, m, w["w_gate"], "bfloat16",
+                    ones_column=True).reshape(b, l, m)
+  hp, ohp = make_hparams(moe_num_experts=e, moe_hidden_size=hdim,
+                         moe_group_size=512, moe_capacity_factor_train=1.0)
+  got, _, _, _ = run_v1(x, w, hp, True, "bfloat16")
+  want, _, aux = O.moe_layer_v1(x, w["w_gate"], w["wi"], w["wo"], ohp, True,
+                                "bfloat16", dense=True)
+  assert aux["kept_1"].mean() < 0.9 and aux["kept_2"].mean() < 0.8
+  dropped = ~(aux["kept_1"] | aux["kept_2"]).reshape(got.shape[:2])
+  assert dropped.any() and (got[dropped] == 0).all()
+  np.testing.assert_allclose(got, want, **H.value_tolerance("bfloat16"))
+
+
+@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
+def test_v1_nonpadding_eval_and_policies(act_dtype):
+  b, l, m, hdim, e = 2, 96, 32, 64, 4
+  rng = np.random.default_rng(107)
+  w = dict(w_gate=H.normal_weights(rng, (m, e), m),
+           wi=H.normal_weights(rng, (e, m, hdim), m),
+           wo=H.normal_weights(rng, (e, hdim, m), hdim))
+  x = H.safe_tokens(rng, b * l, m, w["w_gate"], act_dtype).reshape(b, l, m)
+  nonpadding = (rng.random((b, l)) < 0.8).astype(np.float32)
+  for policy, thr in (("all", 0.2), ("none", 0.2), ("threshold", 0.35)):
+    hp, ohp = make_hparams(
+        moe_num_experts=e, moe_hidden_size=hdim, moe_group_size=48,
+        moe_second_policy_eval=policy, moe_second_threshold_eval=thr,
+        moe_use_second_place_loss=True, moe_capacity_factor_eval=1.5)
+    got, got_loss, _, _ = run_v1(x, w, hp, False, act_dtype,
+                                 nonpadding=nonpadding, activation="gelu",
+                                 num_microbatches=2)
+    want, want_loss, aux = O.moe_layer_v1(
+        x, w["w_gate"], w["wi"], w["wo"], ohp, False, act_dtype,
+        nonpadding=nonpadding, activation="gelu", num_microbatches=2)
+    if policy == "threshold":
+      g2 = O.top_2_gating(aux["logits"], 10 ** 6)["gate_2"]
+      assert np.abs(g2 - np.float32(thr)).min() > 1e-5
+    np.testing.assert_allclose(got, want, **H.value_tolerance(act_dtype))
+    assert (got[nonpadding == 0] == 0).all()
+    np.testing.assert_allclose(got_loss, want_loss,
+                               rtol=1e-2 if act_dtype == "bfloat16" else 1e-5)
+
+
+def test_v1_rerun_with_new_inputs():
+  """Lowering.run(feeds) re-executes the layer with the variables in place."""
+  b, l, m, hdim, e = 2, 64, 16, 32, 4
+  rng = np.random.default_rng(109)
+  w = dict(w_gate=H.normal_weights(rng, (m, e), m),
+           wi=H.normal_weights(rng, (e, m, hdim), m),
+           wo=H.normal_weights(rng, (e, hdim, m), hdim))
+  x1 = H.safe_tokens(rng, b * l, m, w["w_gate"], "float32").reshape(b, l, m)
+  x2 = H.safe_tokens(rng, b * l, m, w["w_gate"], "float32").reshape(b, l, m)
+  hp, ohp = make_hparams(moe_num_experts=e, moe_hidden_size=hdim)
+  _, _, lowering, (xt, y) = run_v1(x1, w, hp, True, "float32")
+  lowering.run({xt: torch.from_numpy(x2)})
+  got = H.to_np(lowering.export_to_tf_tensor(y))
+  want, _, _ = O.moe_layer_v1(x2, w["w_gate"], w["wi"], w["wo"], ohp, True)
+  np.testing.assert_allclose(got, want, **H.value_tolerance("float32"))
+
+
+def run_v2(x, weights, hp, train, act_dtype, nonpadding=None):
+  dt = H.ACT_TORCH[act_dtype]
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  names = ["outer_batch", "batch", "length", "d_model"][4 - x.ndim:]
+  dims = [mtf.Dimension(nm, s) for nm, s in zip(names, x.shape)]
+  xt = mtf.import_tf_tensor(mesh, torch.from_numpy(x).to(dt), mtf.Shape(dims))
+  npad = None
+  if nonpadding is not None:
+    npad = mtf.import_tf_tensor(mesh, torch.from_numpy(nonpadding).to(dt),
+                                mtf.Shape(dims[:-1]))
+  n = weights["wo"].shape[-1]
+  vdt = mtf.VariableDType(torch.float32, torch.float32, dt)
+  with mtf.variable_scope("moe2d"):
+    y, loss = moe.transformer_moe_layer_v2(
+        xt, mtf.Dimension("d_model", n), hp, train, vdt, nonpadding=npad)
+  init = {"moe2d/outer_gating/kernel": weights["w_outer"],
+          "moe2d/inner_gating/kernel": weights["w_inner"],
+          "moe2d/wi/kernel": weights["wi"], "moe2d/wo/kernel": weights["wo"]}
+  lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()}, initial_values=init)
+  return (H.to_np(lowering.export_to_tf_tensor(y)),
+          float(H.to_np(lowering.export_to_tf_tensor(loss))))
+
+
+def v2_weights(rng, m, hdim, xe, ye):
+  return dict(w_outer=H.normal_weights(rng, (m, xe), m),
+              w_inner=H.normal_weights(rng, (xe, m, ye), m),
+              wi=H.normal_weights(rng, (ye, xe, m, hdim), m),
+              wo=H.normal_weights(rng, (ye, xe, hdim, m), hdim))
+
+
+def inner_gap_ok(aux, min_gap=1e-4):
+  """True if no inner-level row that is actually routed has a near-tie."""
+  logits = aux["logits_inner"]
+  imp = aux["importance_inner"].reshape(logits.shape[:2])
+  top = -np.sort(-logits, axis=-1)[..., :3]
+  gaps = (top[..., :-1] - top[..., 1:]).min(axis=-1)
+  return bool((gaps[imp > 0] > min_gap).all())
+
+
+V2_CASES = [
+    ("f32", (2, 64, 16), 32, 4, 4, 32, 1.25, 1.25, "float32"),
+    ("bf16", (2, 64, 16), 32, 4, 4, 32, 1.25, 1.0, "bfloat16"),
+    ("outer_batch_f32", (1, 4, 96, 24), 48, 3, 5, 64, 2.0, 1.5, "float32"),
+    ("mid_bf16", (8, 256, 128), 256, 4, 8, 256, 1.25, 1.25, "bfloat16"),
+]
+
+
+@pytest.mark.parametrize("case", V2_CASES, ids=[c[0] for c in V2_CASES])
+def test_v2_matches_oracle(case):
+  _, shape, hdim, xe, ye, group, cf, cf2, act_dtype = case
+  m = shape[-1]
+  n_tok = int(np.prod(shape[:-1]))
+  hp, ohp = make_hparams(moe_num_experts=[xe, ye], moe_hidden_size=hdim,
+                         moe_group_size=group, moe_capacity_factor_train=cf,
+                         moe_capacity_factor_second_level=cf2)
+  for seed in range(211, 231):   # first seed without an inner-level near-tie
+    rng = np.random.default_rng(seed)
+    w = v2_weights(rng, m, hdim, xe, ye)
+    x = H.safe_tokens(rng, n_tok, m, w["w_outer"], act_dtype).reshape(shape)
+    want, want_loss, aux = O.moe_layer_v2(
+        x, w["w_outer"], w["w_inner"], w["wi"], w["wo"], ohp, True, act_dtype,
+        dense=n_tok <= 1024)
+    if inner_gap_ok(aux):
+      break
+  assert inner_gap_ok(aux)
+  got, got_loss = run_v2(x, w, hp, True, act_dtype)
+  np.testing.assert_allclose(got, want, **H.value_tolerance(act_dtype))
+  np.testing.assert_allclose(got_loss, want_loss,
+                             rtol=1e-2 if act_dtype == "bfloat16" else 1e-5)
+
+
+def test_v2_nonpadding():
+  shape, hdim, xe, ye = (2, 80, 16), 32, 2, 4
+  rng = np.random.default_rng(223)
+  w = v2_weights(rng, 16, hdim, xe, ye)
+  x = H.safe_tokens(rng, 160, 16, w["w_outer"], "float32").reshape(shape)
+  nonpadding = (rng.random(shape[:-1]) < 0.7).astype(np.float32)
+  hp, ohp = make_hparams(moe_num_experts=[xe, ye], moe_hidden_size=hdim,
+                         moe_group_size=40, moe_capacity_factor_train=2.0,
+                         moe_capacity_factor_second_level=2.0)
+  want, want_loss, aux = O.moe_layer_v2(
+      x, w["w_outer"], w["w_inner"], w["wi"], w["wo"], ohp, True, "float32",
+      nonpadding=nonpadding)
+  assert inner_gap_ok(aux)
+  got, got_loss = run_v2(x, w, hp, True, "float32", nonpadding=nonpadding)
+  np.testing.assert_allclose(got, want, **H.value_tolerance("float32"))
+  assert (got[nonpadding == 0] == 0).all()
+  np.testing.assert_allclose(got_loss, want_loss, rtol=1e-5)
