@@ -1,0 +1,279 @@
+"""Benchmark: forward pass of the top-2 Mixture-of-Experts layer on one MI355X.
+
+  python bench.py [--gpus 1] [--steps K] [--warmup W] [--config 1..5]
+
+A step is one forward pass of the layer (router -> top-2 gating -> dispatch ->
+expert FFN -> combine) over one batch of synthetic tokens that is already
+resident in HBM, run through the mtf-shaped API on HipMeshImpl.  Prints ONE
+JSON line: whole-job tokens/s, the roofline of the dominant kernel (the expert
+grouped GEMM, against the bf16 dense MFMA peak), per-stage timings, and the CPU
+restatement of the reference lowering timed on a bounded sample of the same
+workload on this machine's host cores.
+"""
+
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+  sys.path.insert(0, ROOT)
+
+# MI355X published peaks
+HBM_PEAK_GBS = 8000.0
+MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}
+
+# The five workloads of the benchmark definition.  `cf2` is
+# moe_capacity_factor_second_level (hierarchical layer only).
+CONFIGS = {
+    1: dict(name="cfg1 v1 fp32 2048 tok, d_model 512, d_ff 2048, 8 experts",
+            layer="v1", dtype="f32", batch=2, length=1024, group=1024, M=512,
+            H=2048, E=8, cf=1.25),
+    2: dict(name="cfg2 v1 bf16 16384 tok, d_model 1024, d_ff 4096, 32 experts",
+            layer="v1", dtype="bf16", batch=16, length=1024, group=1024,
+            M=1024, H=4096, E=32, cf=1.25),
+    3: dict(name="cfg3 v1 bf16 skewed 32768 tok, d_model 1024, d_ff 4096, "
+                 "64 experts, Zipf(1.2) router bias scaled to 3.0",
+            layer="v1", dtype="bf16", batch=16, length=2048, group=2048,
+            M=1024, H=4096, E=64, cf=1.0, skew=True),
+    4: dict(name="cfg4 v1 bf16 65536 tok, d_model 4096, d_ff 16384, 64 experts",
+            layer="v1", dtype="bf16", batch=32, length=2048, group=2048,
+            M=4096, H=16384, E=64, cf=2.0),
+    5: dict(name="cfg5 v2 bf16 32768 tok, d_model 2048, d_ff 8192, 8x16 experts",
+            layer="v2", dtype="bf16", batch=32, length=1024, group=1024,
+            M=2048, H=8192, E=[8, 16], cf=1.25, cf2=1.25),
+}
+
+
+def hparams_dict(cfg):
+  return dict(
+      moe_gating="top_2", moe_num_experts=cfg["E"], moe_loss_coef=1e-2,
+      moe_hidden_size=cfg["H"], moe_group_size=cfg["group"],
+      moe_min_expert_capacity=4, moe_capacity_factor_train=cfg["cf"],
+      moe_capacity_factor_eval=cfg["cf"],
+      moe_capacity_factor_second_level=cfg.get("cf2", 1.0),
+      moe_use_second_place_loss=False, moe_second_policy_train="all",
+      moe_second_policy_eval="all", moe_second_threshold_train=0.2,
+      moe_second_threshold_eval=0.2, moe_dropout_rate=0.0,
+      moe_use_experts_attention=False)
+
+
+def normal_init(fan_in, seed):
+  """N(0, 1/sqrt(fan_in)) generated on the device, one leading index at a time
+  so that a 8 GiB variable never needs a float32 temporary of its full size."""
+  import torch
+
+  def init(sizes, dtype, device):
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+    out = torch.empty(sizes, dtype=dtype, device=device)
+    flat = out.reshape(sizes[0], -1) if len(sizes) > 2 else out.reshape(1, -1)
+    for i in range(flat.shape[0]):
+      row = torch.randn(flat.shape[1], generator=gen, device=device,
+                        dtype=torch.float32)
+      flat[i] = (row / math.sqrt(fan_in)).to(dtype)
+    return out
+  return init
+
+
+def build(cfg, device):
+  """Builds the graph for `cfg` through the mtf-shaped API and lowers it once.
+  Returns (lowering, x Tensor, y Tensor, loss Tensor)."""
+  import torch
+  import mesh_amd as mtf
+  from mesh_amd.transformer import moe
+
+  dt = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float32
+  m, h = cfg["M"], cfg["H"]
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  gen = torch.Generator(device=device)
+  gen.manual_seed(1)
+  x_val = torch.randn((cfg["batch"], cfg["length"], m), generator=gen,
+                      device=device, dtype=torch.float32).to(dt)
+  dims = [mtf.Dimension("batch", cfg["batch"]),
+          mtf.Dimension("length", cfg["length"]), mtf.Dimension("d_model", m)]
+  hp = moe.HParams(**hparams_dict(cfg))
+  vdt = mtf.VariableDType(dt, dt, dt)
+  init = {}
+  if cfg["layer"] == "v1":
+    if cfg.get("skew"):
+      # Zipf(s=1.2) rank profile scaled to 3.0, added to the router logits.  The
+      # reference router has no bias term: feature 0 of every token is set to 1
+      # and row 0 of the router kernel carries the bias.
+      x_val[..., 0] = 1.0
+    init["moe/top_2_gating/kernel"] = normal_init(m, 2)
+    init["moe/wi/kernel"] = normal_init(m, 3)
+    init["moe/wo/kernel"] = normal_init(h, 4)
+  else:
+    init["moe/outer_gating/kernel"] = normal_init(m, 2)
+    init["moe/inner_gating/kernel"] = normal_init(m, 5)
+    init["moe/wi/kernel"] = normal_init(m, 3)
+    init["moe/wo/kernel"] = normal_init(h, 4)
+  x = mtf.import_tf_tensor(mesh, x_val, mtf.Shape(dims))
+  with mtf.variable_scope("moe"):
+    if cfg["layer"] == "v1":
+      y, loss = moe.transformer_moe_layer_v1(x, dims[-1], hp, True, vdt)
+    else:
+      y, loss = moe.transformer_moe_layer_v2(x, dims[-1], hp, True, vdt)
+  if cfg.get("skew"):
+    base = init["moe/top_2_gating/kernel"]
+
+    def skewed(sizes, dtype, dev):
+      w = base(sizes, dtype, dev)
+      perm = torch.randperm(sizes[1], generator=gen, device=dev) + 1
+      w[0] = (3.0 * perm.double() ** -1.2).to(dtype)
+      return w
+    init["moe/top_2_gating/kernel"] = skewed
+  lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl(device=device)},
+                          initial_values=init)
+  return lowering, x, y, loss
+
+
+def stage_model(cfg, kept_pairs, slots):
+  """Algorithmic bytes / flops per step of each stage (v1 layer): what a
+  perfect implementation has to move or compute."""
+  b = 2 if cfg["dtype"] == "bf16" else 4
+  t = cfg["batch"] * cfg["length"]
+  m, h, e = cfg["M"], cfg["H"], cfg["E"]
+  r = kept_pairs
+  return {
+      "router_logits": dict(bytes=t * m * b + m * e * b + t * e * 4),
+      "top2_gating": dict(bytes=t * (4 * e + 26)),
+      "dispatch": dict(bytes=t * m * b + r * m * b + 18 * t),
+      "combine": dict(bytes=r * m * b + t * m * b + 26 * t),
+      "expert_ffn": dict(flops=4 * r * m * h, padded_flops=4 * slots * m * h),
+  }
+
+
+def cpu_baseline(cfg):
+  """Times the CPU restatement of the reference lowering (dense one-hot
+  dispatch/combine einsums, S x S cumsum matmul, per-expert matmuls) on a
+  bounded sample: ONE group of the workload, with one expert's weight matrices
+  shared by all experts so that host memory stays bounded."""
+  import numpy as np
+  from oracle import moe_oracle as O
+  if cfg["layer"] != "v1":
+    return None
+  rng = np.random.default_rng(0)
+  m, h, e, s = cfg["M"], cfg["H"], cfg["E"], cfg["group"]
+  act = "bfloat16" if cfg["dtype"] == "bf16" else "float32"
+  x = O.cast_act(rng.standard_normal((1, s, m), dtype=np.float32), act)
+  wg = (rng.standard_normal((m, e), dtype=np.float32) / np.sqrt(m))
+  wi1 = O.cast_act(rng.standard_normal((1, m, h), dtype=np.float32)
+                   / np.float32(np.sqrt(m)), act)
+  wo1 = O.cast_act(rng.standard_normal((1, h, m), dtype=np.float32)
+                   / np.float32(np.sqrt(h)), act)
+  wi = np.broadcast_to(wi1, (e, m, h))
+  wo = np.broadcast_to(wo1, (e, h, m))
+  hp = O.HParams(**hparams_dict(cfg))
+  threads = os.cpu_count()
+  try:
+    from threadpoolctl import threadpool_info
+    blas = [p["num_threads"] for p in threadpool_info()
+            if p.get("user_api") == "blas"]
+    if blas:
+      threads = max(blas)
+  except Exception:  # pylint: disable=broad-except
+    pass
+  t0 = time.perf_counter()
+  O.moe_layer_v1(x, wg, wi, wo, hp, True, act, dense=True,
+                 weights_are_cast=True)
+  dt = time.perf_counter() - t0
+  return dict(value=s / dt, unit="tokens/s", cores=int(threads), kind="port",
+              sample="1 of %d groups (%d tokens, all %d experts, dense "
+                     "formulation, one expert's weights shared by all "
+                     "experts), %.1f s"
+                     % (cfg["batch"] * cfg["length"] // s, s, e, dt))
+
+
+def main():
+  ap = argparse.ArgumentParser()
+  ap.add_argument("--gpus", type=int, default=1)
+  ap.add_argument("--steps", type=int, default=10)
+  ap.add_argument("--warmup", type=int, default=3)
+  ap.add_argument("--config", type=int, default=4, choices=sorted(CONFIGS))
+  ap.add_argument("--no-cpu-baseline", action="store_true")
+  args = ap.parse_args()
+  if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
+    print("bench.py measures ONE GPU: this layer runs on a single-device mesh "
+          "(no collectives are built); --gpus %d is not supported" % args.gpus,
+          file=sys.stderr)
+    sys.exit(2)
+
+  import torch
+  from mesh_amd import moe_hip
+  cfg = CONFIGS[args.config]
+  device = torch.device("cuda:0")
+  torch.cuda.set_device(device)
+  lowering, x, y, loss = build(cfg, device)   # first execution
+  for _ in range(args.warmup):
+    lowering.run()
+  torch.cuda.synchronize()
+  with moe_hip.StageTimer() as timer:
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+      lowering.run()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    stages = timer.totals()
+    routings = timer.routing
+  ms_per_step = (t1 - t0) * 1e3 / args.steps
+  tokens = cfg["batch"] * cfg["length"]
+  out_ok = bool(torch.isfinite(lowering.export_to_tf_tensor(y).float()).all())
+
+  result = {
+      "metric": "MoE layer fwd tokens/sec @1 GPU",
+      "value": tokens / (ms_per_step * 1e-3), "unit": "tokens/s",
+      "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+      "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
+      "vs_baseline": None, "dtype": cfg["dtype"], "data": "synthetic",
+      "config": {"workload": cfg["name"], "layer": cfg["layer"],
+                 "tokens": tokens, "output_finite": out_ok},
+  }
+  if cfg["layer"] == "v1":
+    r = routings[-1]
+    kept = int(r.fill.sum().item())
+    slots = r.fill.numel() * r.capacity
+    model = stage_model(cfg, kept, slots)
+    per_stage = {}
+    for name, (calls, ms) in stages.items():
+      ms_step = ms / args.steps
+      entry = {"ms_per_step": ms_step, "launches_per_step": calls / args.steps}
+      if "bytes" in model.get(name, {}):
+        gbs = model[name]["bytes"] / (ms_step * 1e-3) / 1e9
+        entry.update(algorithmic_bytes=model[name]["bytes"], GBps=gbs,
+                     frac_hbm_peak=gbs / HBM_PEAK_GBS)
+      per_stage[name] = entry
+    ffn_ms = stages["expert_ffn"][1] / args.steps
+    # the expert FFN is two launches of the same grouped-GEMM kernel with the
+    # same flop count; `achieved` prices the average launch
+    flops_per_launch = model["expert_ffn"]["flops"] / 2
+    achieved = flops_per_launch / (ffn_ms / 2 * 1e-3) / 1e12
+    peak = MFMA_PEAK_TFLOPS[cfg["dtype"]]
+    result["roofline"] = {
+        "kernel": "grouped expert GEMM (expert_ffn, 2 launches/step)",
+        "bound": "mfma", "achieved": achieved, "peak": peak,
+        "unit": "TFLOP/s", "frac": achieved / peak, "traffic": None,
+        "flops_per_launch": flops_per_launch,
+        "avg_launch_ms": ffn_ms / 2,
+        "padded_frac": (model["expert_ffn"]["padded_flops"] / 2
+                        / (ffn_ms / 2 * 1e-3) / 1e12) / peak}
+    result["stages"] = per_stage
+    result["config"].update(kept_pairs=kept, slots=slots,
+                            capacity=r.capacity)
+  else:
+    result["roofline"] = None
+    result["stages"] = {k: {"ms_per_step": v[1] / args.steps,
+                            "launches_per_step": v[0] / args.steps}
+                        for k, v in stages.items()}
+  result["cpu_baseline"] = (None if args.no_cpu_baseline
+                            else cpu_baseline(cfg))
+  print(json.dumps(result))
+
+
+if __name__ == "__main__":
+  main()

@@ -18,12 +18,16 @@ typedef __attribute__((ext_vector_type(16))) float f32x16_t;
 // bf16 MFMA kernel.
 // Block tile BM x BN, K step BK, 4 wavefronts in a 2 x 2 grid, each owning a
 // (BM/2) x (BN/2) sub-tile made of 32 x 32 MFMA tiles.  LDS rows hold BK bf16
-// plus 8 bf16 of padding, which makes the 16-byte fragment reads of 16
+// plus 8 bf16 of padding, which makes the 16-byte fragment reads of
 // consecutive rows hit disjoint banks.
 //
-// MFMA 32x32x16 operand layout (per lane l): A row l%32, k = 8*(l/32)..+7;
-// B column l%32, same k; accumulator register r holds row
-// 8*(r/4) + 4*(l/32) + r%4, column l%32.
+// The weight tile is fed as the MFMA "A" operand and the activation tile as
+// "B", i.e. each MFMA produces a 32(n) x 32(m) block of C^T.  Per lane l the
+// operands are row/column l%32 with k = 8*(l/32)..+7, and accumulator register
+// r holds n = 8*(r/4) + 4*(l/32) + r%4 for m = l%32: four consecutive output
+// columns per lane, which the epilogue packs into one 8-byte LDS write.  The
+// finished tile is staged in LDS and written out with 16-byte row-contiguous
+// stores.
 // ---------------------------------------------------------------------------
 template <int BM, int BN, int BK>
 struct GemmCfg {
@@ -34,21 +38,33 @@ struct GemmCfg {
   static constexpr int CPR = BK / 8;  // 16-byte chunks per tile row
   static constexpr int A_CHUNKS = BM * CPR / THREADS;
   static constexpr int B_CHUNKS = BN * CPR / THREADS;
-  static constexpr size_t LDS_BYTES = 2ull * (BM + BN) * LDK * sizeof(bf16_t);
+  static constexpr int LDC = BN + 4;  // padded row of the staged C tile
+  static constexpr size_t LOOP_BYTES = 2ull * (BM + BN) * LDK * sizeof(bf16_t);
+  static constexpr size_t EPI_BYTES = (size_t)BM * LDC * sizeof(bf16_t);
+  static constexpr size_t LDS_BYTES =
+      LOOP_BYTES > EPI_BYTES ? LOOP_BYTES : EPI_BYTES;
 };
 
-template <int BM, int BN, int BK>
+__device__ __forceinline__ uint32_t pack2_bf16(float a, float b, bool relu) {
+  uint32_t lo = f32_to_bf16(a), hi = f32_to_bf16(b);
+  if (relu) {  // relu of the rounded value: clear negatives (sign bit set)
+    if (lo & 0x8000u) lo = 0;
+    if (hi & 0x8000u) hi = 0;
+  }
+  return lo | (hi << 16);
+}
+
+template <int BM, int BN, int BK, bool RELU>
 __global__ __launch_bounds__(256) void grouped_gemm_bf16_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
-    bf16_t* __restrict__ Cout, int R, int N, int K, int tiles_m, int tiles_n,
-    int act) {
+    bf16_t* __restrict__ Cout, int R, int N, int K, int tiles_m, int tiles_n) {
   using Cfg = GemmCfg<BM, BN, BK>;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   bf16_t* As = reinterpret_cast<bf16_t*>(smem_raw);  // [2][BM][LDK]
   bf16_t* Bs = As + 2 * BM * Cfg::LDK;               // [2][BN][LDK]
 
-  // tile decode: consecutive blocks walk the N tiles of one (expert, M tile)
-  // so that blocks resident together share the A panel and stream B once.
+  // tile decode: consecutive blocks walk the M tiles of one (expert, N tile),
+  // so blocks resident together share the weight panel.
   const int tiles_per_e = tiles_m * tiles_n;
   const int e = blockIdx.x / tiles_per_e;
   const int rem = blockIdx.x - e * tiles_per_e;
@@ -135,29 +151,42 @@ __global__ __launch_bounds__(256) void grouped_gemm_bf16_kernel(
       for (int i = 0; i < Cfg::TM; ++i)
 #pragma unroll
         for (int j = 0; j < Cfg::TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(af[i], bfr[j], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[j], af[i], acc[i][j], 0, 0, 0);
     }
     if (kt + 1 < nk) store_lds(buf ^ 1);
     __syncthreads();
   }
 
-  // epilogue: round to bf16, activation on the rounded value, store
-  const int col_l = lane & 31;
-  const int row_l = (lane >> 5) * 4;
+  // epilogue: round (and relu), stage the tile in LDS, coalesced stores
+  bf16_t* Cs = reinterpret_cast<bf16_t*>(smem_raw);  // [BM][LDC]
+  const int m_l = lane & 31;
+  const int n_l = (lane >> 5) * 4;
 #pragma unroll
   for (int i = 0; i < Cfg::TM; ++i) {
 #pragma unroll
     for (int j = 0; j < Cfg::TN; ++j) {
-      const int col = col0 + wn * Cfg::WTN + j * 32 + col_l;
 #pragma unroll
-      for (int r = 0; r < 16; ++r) {
-        const int row = row0 + wm * Cfg::WTM + i * 32 + 8 * (r / 4) + row_l + (r % 4);
-        if (row < R && col < N) {
-          float v = round_to<bf16_t>(acc[i][j][r]);
-          if (act != MESH_MOE_ACT_LINEAR) v = apply_activation(v, act);
-          Ce[(int64_t)row * N + col] = f32_to_bf16(v);
-        }
+      for (int q = 0; q < 4; ++q) {
+        const int row = wm * Cfg::WTM + i * 32 + m_l;
+        const int col = wn * Cfg::WTN + j * 32 + 8 * q + n_l;
+        uint2 v;
+        v.x = pack2_bf16(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], RELU);
+        v.y = pack2_bf16(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3], RELU);
+        *reinterpret_cast<uint2*>(Cs + row * Cfg::LDC + col) = v;
       }
+    }
+  }
+  __syncthreads();
+  constexpr int CPR_C = BN / 8;  // 16-byte chunks per output row
+#pragma unroll 4
+  for (int c = tid; c < BM * CPR_C; c += Cfg::THREADS) {
+    const int r = c / CPR_C, cc = (c % CPR_C) * 8;
+    const int grow = row0 + r, gcol = col0 + cc;
+    if (grow < R && gcol < N) {
+      const uint2* s = reinterpret_cast<const uint2*>(Cs + r * Cfg::LDC + cc);
+      uint2 lo = s[0], hi = s[1];
+      *reinterpret_cast<uint4*>(Ce + (int64_t)grow * N + gcol) =
+          make_uint4(lo.x, lo.y, hi.x, hi.y);
     }
   }
 }
@@ -167,10 +196,10 @@ __global__ __launch_bounds__(256) void grouped_gemm_bf16_kernel(
 // 64 x 64 tile, 16-deep K step, each thread a 4 x 4 patch, float32 accumulate
 // in k order.
 // ---------------------------------------------------------------------------
-template <typename T>
+template <typename T, bool RELU>
 __global__ __launch_bounds__(256) void grouped_gemm_simple_kernel(
     const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ Cout,
-    int R, int N, int K, int tiles_m, int tiles_n, int act) {
+    int R, int N, int K, int tiles_m, int tiles_n) {
   __shared__ float As[16][64 + 4];
   __shared__ float Bs[16][64 + 4];
   const int tiles_per_e = tiles_m * tiles_n;
@@ -220,38 +249,60 @@ __global__ __launch_bounds__(256) void grouped_gemm_simple_kernel(
       int col = col0 + tx * 4 + j;
       if (row < R && col < N) {
         float v = round_to<T>(acc[i][j]);
-        if (act != MESH_MOE_ACT_LINEAR) v = apply_activation(v, act);
+        if (RELU) v = v > 0.f ? v : 0.f;
         store_f32<T>(Ce + (int64_t)row * N + col, v);
       }
     }
   }
 }
 
+// In-place activation on an already rounded tensor, for the activations that
+// are not fused into the GEMM epilogue (everything except relu / linear).
+template <typename T>
+__global__ __launch_bounds__(256) void activation_kernel(T* __restrict__ h,
+                                                         int64_t n, int act) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += stride)
+    store_f32<T>(h + i, apply_activation(load_f32<T>(h + i), act));
+}
+
 template <int BM, int BN, int BK>
 static int launch_mfma(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
-                       int R, int N, int K, int act, hipStream_t st) {
+                       int R, int N, int K, bool relu, hipStream_t st) {
   using Cfg = GemmCfg<BM, BN, BK>;
   const int tiles_m = (R + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   const int64_t blocks = (int64_t)tiles_m * tiles_n * E;
   MOE_REQUIRE(blocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
               "expert_ffn: too many tiles (%lld)", (long long)blocks);
-  auto k = grouped_gemm_bf16_kernel<BM, BN, BK>;
-  MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
-  k<<<(unsigned)blocks, 256, Cfg::LDS_BYTES, st>>>(A, B, C, R, N, K, tiles_m,
-                                                    tiles_n, act);
+  if (relu) {
+    auto k = grouped_gemm_bf16_kernel<BM, BN, BK, true>;
+    MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
+    k<<<(unsigned)blocks, 256, Cfg::LDS_BYTES, st>>>(A, B, C, R, N, K, tiles_m,
+                                                      tiles_n);
+  } else {
+    auto k = grouped_gemm_bf16_kernel<BM, BN, BK, false>;
+    MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
+    k<<<(unsigned)blocks, 256, Cfg::LDS_BYTES, st>>>(A, B, C, R, N, K, tiles_m,
+                                                      tiles_n);
+  }
   MOE_CHECK_LAUNCH("expert_ffn (mfma)");
   return 0;
 }
 
 template <typename T>
 static int launch_simple(const T* A, const T* B, T* C, int E, int R, int N,
-                         int K, int act, hipStream_t st) {
+                         int K, bool relu, hipStream_t st) {
   const int tiles_m = (R + 63) / 64, tiles_n = (N + 63) / 64;
   const int64_t blocks = (int64_t)tiles_m * tiles_n * E;
   MOE_REQUIRE(blocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
               "expert_ffn: too many tiles (%lld)", (long long)blocks);
-  grouped_gemm_simple_kernel<T><<<(unsigned)blocks, 256, 0, st>>>(
-      A, B, C, R, N, K, tiles_m, tiles_n, act);
+  if (relu)
+    grouped_gemm_simple_kernel<T, true><<<(unsigned)blocks, 256, 0, st>>>(
+        A, B, C, R, N, K, tiles_m, tiles_n);
+  else
+    grouped_gemm_simple_kernel<T, false><<<(unsigned)blocks, 256, 0, st>>>(
+        A, B, C, R, N, K, tiles_m, tiles_n);
   MOE_CHECK_LAUNCH("expert_ffn (fma)");
   return 0;
 }
@@ -259,18 +310,36 @@ static int launch_simple(const T* A, const T* B, T* C, int E, int R, int N,
 // C[e] = act(A[e] . B[e]^T) for every expert.
 static int grouped_gemm(const void* A, const void* B, void* C, int E, int R,
                         int N, int K, int act, int dtype, hipStream_t st) {
-  if (dtype == MESH_MOE_F32)
-    return launch_simple<float>((const float*)A, (const float*)B, (float*)C, E,
-                                R, N, K, act, st);
-  const bool mfma_ok = (K % 8 == 0) && (((uintptr_t)A | (uintptr_t)B) % 16 == 0);
-  if (!mfma_ok)
-    return launch_simple<bf16_t>((const bf16_t*)A, (const bf16_t*)B,
-                                 (bf16_t*)C, E, R, N, K, act, st);
-  if (R >= 1024 && N >= 1024)
-    return launch_mfma<256, 256, 64>((const bf16_t*)A, (const bf16_t*)B,
-                                     (bf16_t*)C, E, R, N, K, act, st);
-  return launch_mfma<128, 128, 64>((const bf16_t*)A, (const bf16_t*)B,
-                                   (bf16_t*)C, E, R, N, K, act, st);
+  const bool relu = act == MESH_MOE_ACT_RELU;
+  int rc;
+  if (dtype == MESH_MOE_F32) {
+    rc = launch_simple<float>((const float*)A, (const float*)B, (float*)C, E,
+                              R, N, K, relu, st);
+  } else {
+    const bool mfma_ok =
+        (K % 8 == 0) && (N % 8 == 0) &&
+        (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) % 16 == 0);
+    if (!mfma_ok)
+      rc = launch_simple<bf16_t>((const bf16_t*)A, (const bf16_t*)B,
+                                 (bf16_t*)C, E, R, N, K, relu, st);
+    else if (R >= 1024 && N >= 1024)
+      rc = launch_mfma<256, 256, 64>((const bf16_t*)A, (const bf16_t*)B,
+                                     (bf16_t*)C, E, R, N, K, relu, st);
+    else
+      rc = launch_mfma<128, 128, 64>((const bf16_t*)A, (const bf16_t*)B,
+                                     (bf16_t*)C, E, R, N, K, relu, st);
+  }
+  if (rc != 0) return rc;
+  if (act != MESH_MOE_ACT_RELU && act != MESH_MOE_ACT_LINEAR) {
+    const int64_t n = (int64_t)E * R * N;
+    const int blocks = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
+    if (dtype == MESH_MOE_F32)
+      activation_kernel<float><<<blocks, 256, 0, st>>>((float*)C, n, act);
+    else
+      activation_kernel<bf16_t><<<blocks, 256, 0, st>>>((bf16_t*)C, n, act);
+    MOE_CHECK_LAUNCH("expert_ffn (activation)");
+  }
+  return 0;
 }
 
 }  // namespace mesh_moe

@@ -98,8 +98,9 @@ class HipMeshImpl(mtf.MeshImpl):
         if init is None:
           raise ValueError("variable %s has no initializer and no initial "
                            "value" % variable.name)
-        initial_value = init(shape, variable.master_dtype, dev) if callable(
-            init) else init
+        initial_value = init
+      if callable(initial_value):
+        initial_value = initial_value(shape, variable.master_dtype, dev)
       master = torch.as_tensor(initial_value)
       if list(master.shape) != shape:
         raise ValueError("initial value of %s has shape %s, want %s"

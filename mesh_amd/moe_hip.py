@@ -113,6 +113,62 @@ def _stream():
   return torch.cuda.current_stream().cuda_stream
 
 
+class StageTimer(object):
+  """Optional per-stage HIP-event timing of the calls below.
+
+  While a StageTimer is installed (`with StageTimer() as t:`), every stage
+  records a start and an end event on the stream it launches on; `totals()`
+  synchronises and returns {stage: (calls, milliseconds)}.  The last Routing
+  produced is kept in `routing` so that a benchmark can count kept slots.
+  """
+
+  def __init__(self):
+    self.events = []
+    self.routing = []
+
+  def __enter__(self):
+    global _timer
+    self._previous = _timer
+    _timer = self
+    return self
+
+  def __exit__(self, *exc):
+    global _timer
+    _timer = self._previous
+    return False
+
+  def totals(self):
+    torch.cuda.synchronize()
+    out = {}
+    for name, start, end in self.events:
+      calls, ms = out.get(name, (0, 0.0))
+      out[name] = (calls + 1, ms + start.elapsed_time(end))
+    return out
+
+
+_timer = None
+
+
+class _stage(object):
+  """Context manager bracketing one stage with events if a timer is set."""
+
+  def __init__(self, name):
+    self.name = name
+
+  def __enter__(self):
+    if _timer is not None:
+      self.start = torch.cuda.Event(enable_timing=True)
+      self.start.record()
+    return self
+
+  def __exit__(self, *exc):
+    if _timer is not None and exc[0] is None:
+      end = torch.cuda.Event(enable_timing=True)
+      end.record()
+      _timer.events.append((self.name, self.start, end))
+    return False
+
+
 def router_logits(x, w, bias=None, out=None):
   """x [B, T, M] or [T, M]; w [B, M, E] or [M, E] -> float32 logits [.., T, E]."""
   lib = load_library()
@@ -128,8 +184,9 @@ def router_logits(x, w, bias=None, out=None):
     out = torch.empty((b, t, e), dtype=torch.float32, device=x.device)
   op = _dev(out, "logits", torch.float32, (b, t, e))
   bp = None if bias is None else _dev(bias, "bias", torch.float32, (e,))
-  _check(lib.mesh_moe_router_logits(xp, wp, bp, op, b, t, m, e, code,
-                                    _stream()), "router_logits")
+  with _stage("router_logits"):
+    _check(lib.mesh_moe_router_logits(xp, wp, bp, op, b, t, m, e, code,
+                                      _stream()), "router_logits")
   return out[0] if squeeze else out
 
 
@@ -168,14 +225,18 @@ def top2_gating(logits, capacity, importance=None, policy="all",
   loss = torch.empty((1,), dtype=torch.float32, device=dev)
   ws_bytes = lib.mesh_moe_gating_workspace_bytes(g, s, e)
   ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
-  _check(lib.mesh_moe_top2_gating(
-      lp, ip, icode, int(bool(importance_from_slot_gate)), up, g, s, e,
-      int(capacity), POLICIES[policy],
-      float(threshold), int(bool(use_second_place_loss)),
-      int(num_microbatches or 1), idx.data_ptr(), pos.data_ptr(),
-      gate.data_ptr(), kept.data_ptr(), fill.data_ptr(), loss.data_ptr(),
-      ws.data_ptr(), ws_bytes, _stream()), "top2_gating")
-  return Routing(idx, pos, gate, kept, fill, loss, int(capacity), e)
+  with _stage("top2_gating"):
+    _check(lib.mesh_moe_top2_gating(
+        lp, ip, icode, int(bool(importance_from_slot_gate)), up, g, s, e,
+        int(capacity), POLICIES[policy],
+        float(threshold), int(bool(use_second_place_loss)),
+        int(num_microbatches or 1), idx.data_ptr(), pos.data_ptr(),
+        gate.data_ptr(), kept.data_ptr(), fill.data_ptr(), loss.data_ptr(),
+        ws.data_ptr(), ws_bytes, _stream()), "top2_gating")
+  r = Routing(idx, pos, gate, kept, fill, loss, int(capacity), e)
+  if _timer is not None:
+    _timer.routing.append(r)
+  return r
 
 
 def dispatch(x, r, want_slot_gate=False, out=None):
@@ -191,14 +252,15 @@ def dispatch(x, r, want_slot_gate=False, out=None):
   slot_gate = None
   if want_slot_gate:
     slot_gate = torch.empty((e, g, c), dtype=torch.float32, device=x.device)
-  _check(lib.mesh_moe_dispatch(
-      xp, _dev(r.idx, "idx", torch.int32, (g, s, 2)),
-      _dev(r.pos, "pos", torch.int32, (g, s, 2)),
-      _dev(r.gate, "gate", torch.float32, (g, s, 2)),
-      _dev(r.kept, "kept", torch.uint8, (g, s, 2)),
-      _dev(r.fill, "fill", torch.int32, (g, e)), op,
-      None if slot_gate is None else slot_gate.data_ptr(),
-      g, s, e, c, m, code, _stream()), "dispatch")
+  with _stage("dispatch"):
+    _check(lib.mesh_moe_dispatch(
+        xp, _dev(r.idx, "idx", torch.int32, (g, s, 2)),
+        _dev(r.pos, "pos", torch.int32, (g, s, 2)),
+        _dev(r.gate, "gate", torch.float32, (g, s, 2)),
+        _dev(r.kept, "kept", torch.uint8, (g, s, 2)),
+        _dev(r.fill, "fill", torch.int32, (g, e)), op,
+        None if slot_gate is None else slot_gate.data_ptr(),
+        g, s, e, c, m, code, _stream()), "dispatch")
   return (out, slot_gate) if want_slot_gate else out
 
 
@@ -233,9 +295,10 @@ def expert_ffn(expert_in, wi_packed, wo_packed, activation="relu", h=None,
     y = torch.empty((e, rows, n), dtype=dt, device=expert_in.device)
   hp = _dev(h, "h", dt, (e, rows, hdim))
   yp = _dev(y, "y", dt, (e, rows, n))
-  _check(lib.mesh_moe_expert_ffn(ip, wip, wop, hp, yp, e, rows, m, hdim, n,
-                                 ACTIVATIONS[activation], code, _stream()),
-         "expert_ffn")
+  with _stage("expert_ffn"):
+    _check(lib.mesh_moe_expert_ffn(ip, wip, wop, hp, yp, e, rows, m, hdim, n,
+                                   ACTIVATIONS[activation], code, _stream()),
+           "expert_ffn")
   return y
 
 
@@ -252,10 +315,11 @@ def combine(y, r, group_size, out=None):
   if out is None:
     out = torch.empty((g, s, n), dtype=y.dtype, device=y.device)
   op = _dev(out, "out", y.dtype, (g, s, n))
-  _check(lib.mesh_moe_combine(
-      yp, _dev(r.idx, "idx", torch.int32, (g, s, 2)),
-      _dev(r.pos, "pos", torch.int32, (g, s, 2)),
-      _dev(r.gate, "gate", torch.float32, (g, s, 2)),
-      _dev(r.kept, "kept", torch.uint8, (g, s, 2)), op, g, s, e, c, n, code,
-      _stream()), "combine")
+  with _stage("combine"):
+    _check(lib.mesh_moe_combine(
+        yp, _dev(r.idx, "idx", torch.int32, (g, s, 2)),
+        _dev(r.pos, "pos", torch.int32, (g, s, 2)),
+        _dev(r.gate, "gate", torch.float32, (g, s, 2)),
+        _dev(r.kept, "kept", torch.uint8, (g, s, 2)), op, g, s, e, c, n, code,
+        _stream()), "combine")
   return out

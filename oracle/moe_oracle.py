@@ -431,7 +431,7 @@ def expert_ffn(expert_in, wi, wo, activation, act_dtype):
 def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
                  nonpadding=None, activation="relu", num_microbatches=None,
                  logit_bias=None, second_uniform=None, dense=True,
-                 mesh_dim_size=1):
+                 mesh_dim_size=1, weights_are_cast=False):
   """transformer_moe_layer_v1 forward (transformer/moe.py:191-525).
 
   x: [batch..., length, M] float32 array holding activation-dtype values.
@@ -467,8 +467,10 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
   r = top_2_gating(logits, c_, importance, policy, threshold,
                    hp.moe_use_second_place_loss, num_microbatches, act_dtype,
                    second_uniform, dense=dense)
-  wi_a = cast_act(wi, act_dtype)
-  wo_a = cast_act(wo, act_dtype)
+  # weights_are_cast: the caller already holds activation-dtype values (lets
+  # the CPU-baseline timing pass one expert's matrix broadcast to all experts)
+  wi_a = wi if weights_are_cast else cast_act(wi, act_dtype)
+  wo_a = wo if weights_are_cast else cast_act(wo, act_dtype)
   if dense:
     disp = r["dispatch"].reshape(g_, s_, e_ * c_)
     expert_in = np.matmul(disp.transpose(0, 2, 1), xg)           # [G, EC, M]
