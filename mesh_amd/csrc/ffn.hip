@@ -63,11 +63,18 @@ __global__ __launch_bounds__(256) void grouped_gemm_bf16_kernel(
   bf16_t* As = reinterpret_cast<bf16_t*>(smem_raw);  // [2][BM][LDK]
   bf16_t* Bs = As + 2 * BM * Cfg::LDK;               // [2][BN][LDK]
 
-  // tile decode: consecutive blocks walk the M tiles of one (expert, N tile),
-  // so blocks resident together share the weight panel.
+  // Workgroups are handed to the 8 XCDs round-robin (block b runs on XCD
+  // b % 8) and each XCD has its own L2.  Renumber so that every XCD works on a
+  // contiguous range of logical tiles; logical tiles walk the M tiles of one
+  // (expert, N tile), so the tiles resident on an XCD at one time share a few
+  // weight panels and all of the expert's activation rows through that L2.
+  const int nblk = gridDim.x;
+  const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+  const int q = nblk >> 3, rmd = nblk & 7;
+  const int logical = xcd * q + min(xcd, rmd) + local;
   const int tiles_per_e = tiles_m * tiles_n;
-  const int e = blockIdx.x / tiles_per_e;
-  const int rem = blockIdx.x - e * tiles_per_e;
+  const int e = logical / tiles_per_e;
+  const int rem = logical - e * tiles_per_e;
   const int tn = rem / tiles_m;
   const int tm = rem - tn * tiles_m;
   const int row0 = tm * BM, col0 = tn * BN;
@@ -89,8 +96,8 @@ __global__ __launch_bounds__(256) void grouped_gemm_bf16_kernel(
       int r = c / Cfg::CPR, kc = c % Cfg::CPR;
       int gr = min(row0 + r, R - 1);
       int gk = k0 + kc * 8;
-      areg[i] = gk < K ? *reinterpret_cast<const uint4*>(Ae + (int64_t)gr * K + gk)
-                       : make_uint4(0, 0, 0, 0);
+      uint4 v = *reinterpret_cast<const uint4*>(Ae + (int64_t)gr * K + min(gk, K - 8));
+      areg[i] = gk < K ? v : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
     for (int i = 0; i < Cfg::B_CHUNKS; ++i) {
@@ -98,8 +105,8 @@ __global__ __launch_bounds__(256) void grouped_gemm_bf16_kernel(
       int r = c / Cfg::CPR, kc = c % Cfg::CPR;
       int gr = min(col0 + r, N - 1);
       int gk = k0 + kc * 8;
-      breg[i] = gk < K ? *reinterpret_cast<const uint4*>(Be + (int64_t)gr * K + gk)
-                       : make_uint4(0, 0, 0, 0);
+      uint4 v = *reinterpret_cast<const uint4*>(Be + (int64_t)gr * K + min(gk, K - 8));
+      breg[i] = gk < K ? v : make_uint4(0, 0, 0, 0);
     }
   };
   auto store_lds = [&](int buf) {

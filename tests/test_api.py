@@ -1,0 +1,272 @@
+"""Host-side contract of the mtf-shaped API (no GPU needed): signatures,
+defaults, dimension and variable names, error types, and that the C-ABI library
+loads and exports every symbol the header declares."""
+
+import ctypes
+import inspect
+import os
+import re
+
+import pytest
+import torch
+
+import mesh_amd as mtf
+from mesh_amd import moe_hip
+from mesh_amd.transformer import moe
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def hparams(**kw):
+  hp = dict(
+      moe_gating="top_2", moe_num_experts=8, moe_loss_coef=1e-2,
+      moe_hidden_size=64, moe_group_size=32, moe_min_expert_capacity=4,
+      moe_capacity_factor_train=1.25, moe_capacity_factor_eval=2.0,
+      moe_capacity_factor_second_level=1.0, moe_use_second_place_loss=False,
+      moe_second_policy_train="all", moe_second_policy_eval="all",
+      moe_second_threshold_train=0.2, moe_second_threshold_eval=0.2,
+      moe_dropout_rate=0.0, moe_use_experts_attention=False)
+  hp.update(kw)
+  return moe.HParams(**hp)
+
+
+def graph_input(shape=(2, 64, 16), names=("batch", "length", "d_model"),
+                dtype=torch.float32):
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  dims = [mtf.Dimension(n, s) for n, s in zip(names, shape)]
+  x = mtf.import_tf_tensor(mesh, torch.zeros(shape, dtype=dtype), mtf.Shape(dims))
+  return graph, mesh, x, dims
+
+
+def param_list(fn):
+  return [(p.name, p.default) for p in inspect.signature(fn).parameters.values()]
+
+
+def test_layer_signatures_match_reference():
+  """transformer/moe.py:191-194 and :528-530."""
+  E = inspect.Parameter.empty
+  assert param_list(moe.transformer_moe_layer_v1) == [
+      ("inputs", E), ("output_dim", E), ("hparams", E), ("train", E),
+      ("variable_dtype", E), ("layout", None), ("mesh_shape", None),
+      ("nonpadding", None), ("activation", mtf.relu),
+      ("num_microbatches", None)]
+  assert param_list(moe.transformer_moe_layer_v2) == [
+      ("inputs", E), ("output_dim", E), ("hparams", E), ("train", E),
+      ("variable_dtype", E), ("layout", None), ("mesh_shape", None),
+      ("nonpadding", None), ("num_microbatches", None)]
+  assert param_list(moe._split_into_groups) == [
+      ("n", E), ("max_group_size", E), ("mesh_dim_size", E)]
+
+
+def test_moe1d_moe2d_constructor_defaults():
+  """transformer/moe.py:40-64 and :134-147."""
+  assert param_list(moe.MoE1D.__init__)[1:] == [
+      ("num_experts", 16), ("loss_coef", 1e-2), ("hidden_size", 4096),
+      ("group_size", 1024), ("capacity_factor_train", 1.25),
+      ("capacity_factor_eval", 2.0), ("use_second_place_loss", False),
+      ("second_policy_train", "random"), ("second_policy_eval", "random"),
+      ("second_threshold_train", 0.2), ("second_threshold_eval", 0.2),
+      ("dropout_rate", 0.0), ("activation", "relu"), ("moe_gating", "top_2"),
+      ("min_expert_capacity", 4), ("switch_policy_train", "input_jitter"),
+      ("switch_policy_eval", "input_jitter"), ("switch_dropout", 0.1),
+      ("switch_temperature", 1.0), ("switch_jitter", 1e-2), ("ntlb_top_k", 4),
+      ("output_dim", None), ("use_experts_attention", False), ("z_loss", None)]
+  assert param_list(moe.MoE2D.__init__)[1:] == [
+      ("expert_x", 8), ("expert_y", 8), ("loss_coef", 1e-2),
+      ("hidden_size", 4096), ("group_size", 1024),
+      ("capacity_factor_train", 1.25), ("capacity_factor_eval", 2.0),
+      ("capacity_factor_second_level", 1.0), ("use_second_place_loss", False),
+      ("second_policy_train", "random"), ("second_policy_eval", "random"),
+      ("second_threshold_train", 0.2), ("second_threshold_eval", 0.2)]
+  hp = moe.MoE1D(num_experts=4)._hparams
+  assert hp.moe_num_experts == 4 and hp.moe_gating == "top_2"
+  assert moe.MoE2D()._hparams.moe_num_experts == [8, 8]
+
+
+def test_default_hparams():
+  hp = moe.HParams()
+  moe.set_default_moe_hparams(hp)
+  assert (hp.moe_num_experts, hp.moe_hidden_size, hp.moe_group_size) == (16, 4096, 1024)
+  assert hp.moe_capacity_factor_train == 1.25 and hp.moe_capacity_factor_eval == 2.0
+  assert hp.moe_second_policy_train == "random" and hp.moe_gating == "top_2"
+
+
+def test_split_into_groups():
+  assert moe._split_into_groups(65536, 2048, 1) == (32, 2048)
+  assert moe._split_into_groups(5120, 1024, 1) == (5, 1024)
+  # the search starts at n // max_group_size groups, so (as in the reference)
+  # a group can exceed max_group_size when that count already divides n
+  assert moe._split_into_groups(150, 64, 1) == (2, 75)
+  assert moe._split_into_groups(150, 49, 1) == (3, 50)
+  assert moe._split_into_groups(96, 32, 4) == (4, 24)
+  with pytest.raises(ValueError):
+    moe._split_into_groups(10, 4, 3)
+
+
+def test_v1_graph_names_and_shapes():
+  graph, _, x, dims = graph_input()
+  with mtf.variable_scope("layer_0"):
+    y, loss = moe.transformer_moe_layer_v1(
+        x, dims[-1], hparams(), True, mtf.VariableDType(torch.float32))
+  assert y.shape == mtf.Shape(dims) and loss.shape == mtf.Shape([])
+  got = {v.name: v.shape.to_string for v in graph.all_variables}
+  assert got == {
+      "layer_0/top_2_gating/kernel": "Shape[d_model=16, expert_unsplit=8]",
+      "layer_0/wi/kernel": "Shape[experts=8, d_model=16, expert_hidden=64]",
+      "layer_0/wo/kernel": "Shape[experts=8, expert_hidden=64, d_model=16]"}
+  op = [o for o in graph.operations if isinstance(o, moe.MoEV1Operation)][0]
+  assert op.inputs[0].shape.dimension_names == [
+      "outer_batch", "batch", "group", "d_model"]
+  assert op.inputs[0].shape.to_integer_list == [1, 4, 32, 16]
+  assert op._capacity == 5          # max(min(32, int(32 * 1.25 / 8)), 4)
+
+
+def test_v2_graph_names_and_shapes():
+  graph, _, x, dims = graph_input()
+  with mtf.variable_scope("moe2d"):
+    y, _ = moe.transformer_moe_layer_v2(
+        x, dims[-1], hparams(moe_num_experts=[4, 2]), True,
+        mtf.VariableDType(torch.float32))
+  assert y.shape == mtf.Shape(dims)
+  got = {v.name: v.shape.to_string for v in graph.all_variables}
+  assert got == {
+      "moe2d/outer_gating/kernel": "Shape[d_model=16, expert_x_unsplit=4]",
+      "moe2d/inner_gating/kernel":
+          "Shape[expert_x=4, d_model=16, expert_y_unsplit=2]",
+      "moe2d/wi/kernel":
+          "Shape[expert_y=2, expert_x=4, d_model=16, expert_hidden=64]",
+      "moe2d/wo/kernel":
+          "Shape[expert_y=2, expert_x=4, expert_hidden=64, d_model=16]"}
+  op = [o for o in graph.operations if isinstance(o, moe.MoEV2Operation)][0]
+  assert op.inputs[0].shape.dimension_names == [
+      "outer_batch", "batch", "group_size_x", "d_model"]
+  # x=4, y=2, c=max(min(32, int(32*1.25/4)), 4)=10, 4*10=40 slots -> h0=2,t=20 ...
+  assert op._dims[:3] == (4, 2, 10)
+  assert op._dims[3] * op._dims[4] == 4 * 10
+
+
+def test_error_behaviour():
+  _, _, x, dims = graph_input()
+  vdt = mtf.VariableDType(torch.float32)
+  with pytest.raises(ValueError, match="unknown hparams.moe_gating"):
+    moe.transformer_moe_layer_v1(x, dims[-1], hparams(moe_gating="top_3"), True, vdt)
+  with pytest.raises(ValueError, match="unknown hparams.moe_gating"):
+    moe.transformer_moe_layer_v2(
+        x, dims[-1], hparams(moe_gating="switch", moe_num_experts=[2, 2]), True, vdt)
+  with pytest.raises(ValueError, match="Unknown policy"):
+    moe.transformer_moe_layer_v1(
+        x, dims[-1], hparams(moe_second_policy_train="sometimes"), True, vdt)
+  with pytest.raises(NotImplementedError):
+    moe.transformer_moe_layer_v1(x, dims[-1], hparams(moe_gating="switch"), True, vdt)
+  with pytest.raises(NotImplementedError):
+    moe.transformer_moe_layer_v1(x, dims[-1], hparams(moe_dropout_rate=0.1), True, vdt)
+  with pytest.raises(ValueError, match="not a multiple of mesh_dim_size"):
+    moe.transformer_moe_layer_v1(
+        x, dims[-1], hparams(), True, vdt, layout="batch:rows", mesh_shape="rows:3")
+
+  class Model(object):
+    ensemble_dim = mtf.Dimension("ensemble", 2)
+
+  class Context(object):
+    model = Model()
+  with pytest.raises(NotImplementedError, match="ensembles"):
+    moe.MoE1D().call(Context(), x)
+  with pytest.raises(NotImplementedError, match="ensembles"):
+    moe.MoE2D().call(Context(), x)
+
+
+def test_moe1d_call_adds_length_dim_and_loss():
+  graph, _, x, dims = graph_input(shape=(6, 16), names=("batch", "d_model"))
+
+  class Model(object):
+    ensemble_dim = None
+    model_dim = dims[-1]
+    layout = None
+    mesh_shape = None
+
+  class Context(object):
+    model = Model()
+    length_dim = mtf.Dimension("length", 64)
+    train = True
+    variable_dtype = mtf.VariableDType(torch.float32)
+    nonpadding = None
+    num_microbatches = None
+    losses = []
+  layer = moe.MoE1D(num_experts=2, hidden_size=8, group_size=4,
+                    second_policy_train="all")
+  y = layer.call(Context(), x)
+  assert y.shape == x.shape and len(Context.losses) == 1
+  op = [o for o in graph.operations if isinstance(o, moe.MoEV1Operation)][0]
+  assert op.inputs[0].shape.to_integer_list == [1, 1, 6, 16]
+
+
+def test_shape_and_layout_helpers():
+  s = mtf.convert_to_shape("rows:2,cols:4")
+  assert s.size == 8 and s.dimension_names == ["rows", "cols"]
+  assert mtf.tensor_dim_to_mesh_dim_size(
+      "batch:rows", "rows:2,cols:4", mtf.Dimension("batch", 8)) == 2
+  assert mtf.tensor_dim_to_mesh_dim_size(None, None, mtf.Dimension("batch", 8)) == 1
+  with pytest.raises(ValueError):
+    mtf.Shape([mtf.Dimension("a", 1), mtf.Dimension("a", 2)])
+  impl = mtf.MeshImpl("rows:2", "batch:rows")
+  assert impl.slice_shape(mtf.Shape([("batch", 8), ("d", 3)])) == [4, 3]
+  with pytest.raises(ValueError):
+    impl.slice_shape(mtf.Shape([("batch", 7)]))
+
+
+def test_mesh_impl_interface():
+  """The plugin methods an Operation's lower() may call
+  (mesh_tensorflow/ops.py:867-1340) exist on HipMeshImpl."""
+  for name in ("slicewise", "einsum", "allreduce", "allconcat", "alltoall",
+               "receive", "import_tf_tensor", "export_to_tf_tensor",
+               "slice_shape", "slice_begin", "slice_size", "laid_out_size",
+               "tensor_layout", "tensor_dimension_to_mesh_axis", "make_slices",
+               "combine_slices", "random"):
+    assert callable(getattr(mtf.HipMeshImpl, name)), name
+  for name in ("shape", "ndims", "size", "layout_rules", "devices",
+               "supports_control_dependencies"):
+    assert isinstance(getattr(mtf.HipMeshImpl, name), property), name
+  for name in ("tensor_list", "all_slices", "slice_shape"):
+    assert isinstance(getattr(mtf.HipMeshImpl.LaidOutTensor, name), property)
+  assert hasattr(mtf.HipMeshImpl.LaidOutTensor, "to_laid_out_tensor")
+  assert hasattr(mtf.HipMeshImpl.LaidOutTensor, "from_tensor_list")
+  for name in ("laid_out_tensor", "copy_master_to_slices",
+               "copy_slices_to_master", "assign_to_slices"):
+    assert hasattr(mtf.HipMeshImpl.LaidOutVariable, name)
+
+
+def test_no_cpu_fallback():
+  if torch.cuda.is_available():
+    pytest.skip("a GPU is visible")
+  with pytest.raises(RuntimeError, match="needs a GPU"):
+    mtf.HipMeshImpl()
+  with pytest.raises(moe_hip.MoeHipError):
+    moe_hip.router_logits(torch.zeros(4, 8), torch.zeros(8, 2))
+  with pytest.raises(moe_hip.MoeHipError, match="not found"):
+    moe_hip.load_library("/nonexistent/libmesh_moe_hip.so")
+
+
+def test_library_exports_every_declared_symbol():
+  header = open(os.path.join(ROOT, "include", "mesh_moe.h")).read()
+  declared = set(re.findall(r"\b(mesh_moe_[a-z0-9_]+)\s*\(", header))
+  assert declared == set(moe_hip.EXPORTS)
+  if not os.path.exists(moe_hip.LIB_PATH):
+    from mesh_amd.csrc import build
+    build.build_library(verbose=False)
+  lib = ctypes.CDLL(moe_hip.LIB_PATH)
+  for name in declared:
+    assert getattr(lib, name) is not None
+  lib.mesh_moe_abi_version.restype = ctypes.c_int
+  assert lib.mesh_moe_abi_version() == moe_hip.ABI_VERSION
+  lib.mesh_moe_gating_workspace_bytes.restype = ctypes.c_size_t
+  assert lib.mesh_moe_gating_workspace_bytes(32, 2048, 64) > 0
+
+
+def test_product_does_not_import_the_oracle():
+  pkg = os.path.join(ROOT, "mesh_amd")
+  for dirpath, _, files in os.walk(pkg):
+    for f in files:
+      if f.endswith((".py", ".hip", ".h", ".cpp")):
+        text = open(os.path.join(dirpath, f)).read()
+        assert "oracle" not in text, os.path.join(dirpath, f)

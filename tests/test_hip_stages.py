@@ -197,3 +197,99 @@ def test_rejects_bad_arguments(hip):
   with pytest.raises(hip.MoeHipError):
     hip.router_logits(torch.zeros((4, 8), device="cuda"),
                       torch.zeros((9, 2), device="cuda"))
+
+
+def test_gating_golden_fixture(hip):
+  """The committed golden vectors (tests/golden/top2_gating_small.json)."""
+  import json
+  import os
+  path = os.path.join(os.path.dirname(__file__), "golden",
+                      "top2_gating_small.json")
+  with open(path) as f:
+    gold = json.load(f)
+  logits = np.array(gold["logits"], np.float32)
+  got = H.routing_to_np(hip.top2_gating(torch.from_numpy(logits).cuda(),
+                                        gold["capacity"]))
+  for k in ("index_1", "index_2", "pos_1", "pos_2"):
+    np.testing.assert_array_equal(got[k], np.array(gold[k]), err_msg=k)
+  for k in ("kept_1", "kept_2"):
+    np.testing.assert_array_equal(got[k], np.array(gold[k], bool), err_msg=k)
+  np.testing.assert_allclose(got["gate_1"], np.array(gold["gate_1"]), rtol=1e-5)
+  np.testing.assert_allclose(got["gate_2"], np.array(gold["gate_2"]), rtol=1e-5,
+                             atol=1e-7)
+  np.testing.assert_allclose(got["loss"], gold["loss"], rtol=2e-5)
+
+
+# Full benchmark sizes: (G, S, E, C, M) of configurations 3 and 4.  The oracle
+# is too slow here, so the checks are size-independent properties.
+FULL_SIZES = [(16, 2048, 64, 32, 1024, True), (32, 2048, 64, 64, 4096, False)]
+
+
+@pytest.mark.parametrize("size", FULL_SIZES, ids=["cfg3", "cfg4"])
+def test_full_size_routing_properties(hip, size):
+  g, s, e, c, m, skew = size
+  gen = torch.Generator(device="cuda")
+  gen.manual_seed(5)
+  logits = torch.randn((g, s, e), generator=gen, device="cuda")
+  if skew:
+    ranks = torch.randperm(e, generator=gen, device="cuda").double() + 1
+    logits = logits + (3.0 * ranks ** -1.2).float()
+  r = hip.top2_gating(logits, c)
+  idx, pos, kept = r.idx.long(), r.pos.long(), r.kept.bool()
+  # first / second expert: argmax and argmax-with-first-removed of the logits
+  # (softmax is monotone; ties have measure zero for continuous random logits)
+  top2 = logits.topk(2, dim=-1).indices
+  assert torch.equal(idx, top2)
+  # every (group, expert) fills slots 0..fill-1 exactly once, fill <= C
+  gi = torch.arange(g, device="cuda").view(g, 1, 1).expand(g, s, 2)
+  slot = (gi * e + idx) * c + pos
+  used = torch.zeros(g * e * c, dtype=torch.int32, device="cuda")
+  used.scatter_add_(0, slot[kept], torch.ones_like(slot[kept], dtype=torch.int32))
+  assert int(used.max()) <= 1
+  used = used.view(g, e, c)
+  fill = r.fill.long()
+  assert int(fill.max()) <= c
+  want_used = (torch.arange(c, device="cuda").view(1, 1, c) < fill.unsqueeze(-1))
+  assert torch.equal(used.bool(), want_used)
+  assert torch.equal(used.sum(-1), fill)
+  # kept <=> position below capacity, for every competing choice
+  assert torch.equal(kept, pos < c)
+  # first choices of an expert precede its second choices
+  first_count = torch.zeros(g * e, dtype=torch.long, device="cuda")
+  k1 = kept[..., 0]
+  first_count.scatter_add_(0, (gi[..., 0] * e + idx[..., 0])[k1],
+                           torch.ones(int(k1.sum()), dtype=torch.long,
+                                      device="cuda"))
+  base2 = first_count[(gi[..., 1] * e + idx[..., 1])]
+  assert bool((pos[..., 1] >= base2).all())
+  # positions grow with the token index within (group, expert, choice)
+  for k in range(2):
+    key = (idx[..., k] * s + torch.arange(s, device="cuda").view(1, s))
+    order = key.argsort(dim=1, stable=True)
+    sorted_pos = pos[..., k].gather(1, order)
+    sorted_e = idx[..., k].gather(1, order)
+    same = sorted_e[:, 1:] == sorted_e[:, :-1]
+    assert bool(((sorted_pos[:, 1:] - sorted_pos[:, :-1])[same] == 1).all())
+  if skew:
+    assert float(kept.float().mean()) < 0.8       # the drop path is exercised
+  # gates: normalised pair sums to one where both kept
+  both = kept.all(-1)
+  assert torch.allclose(r.gate.sum(-1)[both], torch.ones((), device="cuda"),
+                        atol=1e-5)
+
+  # dispatch -> combine with identity experts: out = (w1 + w2) * x
+  x = torch.randn((g, s, m), generator=gen, device="cuda").to(torch.bfloat16)
+  ein, slot_gate = hip.dispatch(x, r, want_slot_gate=True)
+  w = r.gate.to(torch.bfloat16).float() * kept.float()
+  # checksum: every kept choice copies its row exactly once
+  n_copies = (kept & (w != 0)).sum(-1).double()
+  want_sum = (x.double().sum(-1) * n_copies).sum()
+  got_sum = ein.double().sum()
+  assert abs(float(got_sum - want_sum)) <= 1e-6 * float(x.double().abs().sum())
+  assert torch.equal(ein.view(e, g, c, m)[~want_used.permute(1, 0, 2)],
+                     torch.zeros((), dtype=torch.bfloat16, device="cuda").expand(
+                         int((~want_used).sum()), m))
+  assert abs(float(slot_gate.double().sum() - w.double().sum())) < 1e-3
+  out = hip.combine(ein, r, s)
+  want = (w[..., 0:1] * x.float() + w[..., 1:2] * x.float()).to(torch.bfloat16)
+  assert torch.equal(out, want)

@@ -1,0 +1,407 @@
+"""Pins the CPU oracle (the reference holds no golden vectors for its MoE file):
+each function is checked against brute force, closed forms, float64 library
+routines or hand-worked cases, chosen so that a dropped term, a wrong index or a
+transposed operand fails."""
+
+import json
+import os
+
+import numpy as np
+import pytest
+import scipy.special
+
+from oracle import moe_oracle as O
+
+GOLDEN = os.path.join(os.path.dirname(__file__), "golden")
+
+
+# ---- host integer logic ------------------------------------------------------
+def test_split_into_groups_brute_force():
+  """Defining constraints of transformer/moe.py:1555-1557: group_size is the
+  largest divisor arrangement with group_size <= max and num_groups a multiple
+  of mesh_dim_size (when n allows)."""
+  for n in list(range(1, 200)) + [1024, 2048, 4096, 5120, 65536]:
+    for max_group in (1, 3, 16, 100, 1024, 2048):
+      for mesh in (1, 2, 4, 8):
+        if n % mesh:
+          with pytest.raises(ValueError):
+            O.split_into_groups(n, max_group, mesh)
+          continue
+        g, s = O.split_into_groups(n, max_group, mesh)
+        assert g * s == n and g % mesh == 0
+        # brute force: smallest admissible num_groups >= max(1, n // max_group)
+        want = next(k for k in range(max(1, n // max_group), n + 1)
+                    if k % mesh == 0 and n % k == 0)
+        assert g == want
+        if n % max_group == 0 and (n // max_group) % mesh == 0:
+          assert s == max_group
+
+
+def test_capacity_table():
+  """The five benchmark configurations (S, cf, E, min=4) -> C."""
+  assert O.expert_capacity(1024, 1.25, 8, 4) == 160
+  assert O.expert_capacity(1024, 1.25, 32, 4) == 40
+  assert O.expert_capacity(2048, 1.0, 64, 4) == 32
+  assert O.expert_capacity(2048, 2.0, 64, 4) == 64
+  assert O.expert_capacity(1024, 1.25, 16, 4) == 80
+  assert O.expert_capacity(1024, 1.0, 16, 4) == 64
+  assert O.expert_capacity(8, 1.0, 64, 4) == 4       # floor at min capacity
+  assert O.expert_capacity(16, 100.0, 2, 4) == 16    # never above group size
+  assert O.split_into_groups(8 * 32 * 160 // 8, 1024, 1) == (5, 1024)
+
+
+# ---- float primitives --------------------------------------------------------
+def test_round_bf16_matches_torch():
+  import torch
+  rng = np.random.default_rng(0)
+  a = np.concatenate([
+      rng.standard_normal(10000).astype(np.float32) * 10.0 ** rng.integers(-20, 20, 10000),
+      np.array([0.0, -0.0, 1.0, 1.00390625, 1.01171875, np.inf, -np.inf,
+                3.3895e38, 1e-45], np.float32)])
+  want = torch.from_numpy(a).to(torch.bfloat16).float().numpy()
+  np.testing.assert_array_equal(O.round_bf16(a), want)
+  assert np.isnan(O.round_bf16(np.float32(np.nan)))
+
+
+def test_softmax_against_float64():
+  rng = np.random.default_rng(1)
+  x = (rng.standard_normal((50, 7, 33)) * 4).astype(np.float32)
+  p = O.softmax(x)
+  want = scipy.special.softmax(x.astype(np.float64), axis=-1)
+  np.testing.assert_allclose(p, want, rtol=2e-6)
+  np.testing.assert_allclose(p.sum(-1), 1.0, atol=1e-6)
+  # equal logits -> equal gates, whatever exp/log round to
+  eq = O.softmax(np.full((3, 8), 1.7, np.float32))
+  assert (eq == eq[:, :1]).all()
+  # large offsets do not overflow
+  assert np.isfinite(O.softmax(x + np.float32(1e4))).all()
+
+
+def test_seq_sum_is_sequential():
+  a = np.array([1e8, 1.0, -1e8, 1.0], np.float32)
+  assert O.seq_sum(a) == np.float32(1.0)     # ((1e8 + 1) - 1e8) + 1 in float32
+  rng = np.random.default_rng(2)
+  x = rng.standard_normal((4, 9)).astype(np.float32)
+  want = np.zeros(4, np.float32)
+  for j in range(9):
+    want = want + x[:, j]
+  np.testing.assert_array_equal(O.seq_sum(x), want)
+
+
+def test_cumsum_dense_equals_index_form():
+  rng = np.random.default_rng(3)
+  x = (rng.random((3, 40, 6)) < 0.3).astype(np.float32)
+  a, b = O.cumsum_exclusive(x, dense=True), O.cumsum_exclusive(x)
+  np.testing.assert_array_equal(a, b)
+  assert (a[:, 0] == 0).all()
+  np.testing.assert_array_equal(a[:, 1:], np.cumsum(x, axis=1)[:, :-1])
+
+
+# ---- top-2 selection -----------------------------------------------------------
+def test_top2_against_stable_argsort():
+  rng = np.random.default_rng(4)
+  logits = rng.standard_normal((5, 64, 12)).astype(np.float32)
+  r = O.top_2_gating(logits, 1000)
+  p = O.softmax(logits)
+  order = np.argsort(-p, axis=-1, kind="stable")
+  np.testing.assert_array_equal(r["index_1"], order[..., 0])
+  np.testing.assert_array_equal(r["index_2"], order[..., 1])
+  g1 = np.take_along_axis(p, order[..., :1], -1)[..., 0]
+  g2 = np.take_along_axis(p, order[..., 1:2], -1)[..., 0]
+  np.testing.assert_allclose(r["gate_1"], g1 / (g1 + g2 + 1e-9), rtol=1e-6)
+  np.testing.assert_allclose(r["gate_1"] + r["gate_2"], 1.0, atol=1e-6)
+
+
+def test_top2_exact_ties_lowest_index_wins():
+  logits = np.zeros((1, 4, 5), np.float32)
+  logits[0, 1, [2, 4]] = 1.0          # two-way tie for first
+  logits[0, 2, 3] = 2.0               # clear first, four-way tie for second
+  r = O.top_2_gating(logits, 100)
+  np.testing.assert_array_equal(r["index_1"][0], [0, 2, 3, 0])
+  np.testing.assert_array_equal(r["index_2"][0], [1, 4, 0, 1])
+
+
+def test_two_experts_always_both():
+  rng = np.random.default_rng(5)
+  r = O.top_2_gating(rng.standard_normal((2, 30, 2)).astype(np.float32), 100)
+  assert (r["index_1"] != r["index_2"]).all()
+  assert r["kept_1"].all() and r["kept_2"].all()
+
+
+# ---- capacity positions --------------------------------------------------------
+def test_hand_worked_capacity_case():
+  """One group, S=6, E=3, C=2; worked by hand from transformer/moe.py:1472-1496."""
+  big, mid = 5.0, 3.0
+  idx1 = [0, 0, 1, 0, 2, 1]
+  idx2 = [1, 2, 0, 1, 0, 0]
+  logits = np.zeros((1, 6, 3), np.float32)
+  for s, (a, b) in enumerate(zip(idx1, idx2)):
+    logits[0, s, a], logits[0, s, b] = big, mid
+  r = O.top_2_gating(logits, 2)
+  np.testing.assert_array_equal(r["index_1"][0], idx1)
+  np.testing.assert_array_equal(r["index_2"][0], idx2)
+  np.testing.assert_array_equal(r["pos_1"][0], [0, 1, 0, 2, 0, 1])
+  np.testing.assert_array_equal(r["kept_1"][0], [1, 1, 1, 0, 1, 1])
+  np.testing.assert_array_equal(r["pos_2"][0], [2, 1, 2, 3, 3, 4])
+  np.testing.assert_array_equal(r["kept_2"][0], [0, 1, 0, 0, 0, 0])
+  np.testing.assert_array_equal(r["fill"][0], [2, 2, 2])
+  # token 3 lost both choices; token 0 keeps its un-renormalised first gate
+  assert r["gate_1"][0, 3] == 0 and r["gate_2"][0, 3] == 0
+  p = O.softmax(logits)[0, 0]
+  np.testing.assert_allclose(r["gate_1"][0, 0], p[0] / (p[0] + p[1] + 1e-9),
+                             rtol=1e-6)
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_capacity_against_sequential_loop(seed):
+  rng = np.random.default_rng(100 + seed)
+  g, s, e = 3, int(rng.integers(5, 90)), int(rng.integers(2, 9))
+  c = int(rng.integers(1, 2 * s // e + 2))
+  logits = rng.standard_normal((g, s, e)).astype(np.float32)
+  imp = None
+  if seed % 2:
+    imp = rng.choice(np.array([0.0, 0.5, 1.0], np.float32), size=(g, s))
+  for dense in (False, True):
+    r = O.top_2_gating(logits, c, importance=imp, dense=dense)
+    sel1 = np.ones((g, s), bool) if imp is None else imp == 1.0
+    sel2 = np.ones((g, s), bool) if imp is None else imp > 0
+    p1, k1, p2, k2, fill = O.routing_sequential(r["index_1"], r["index_2"],
+                                                sel1, sel2, e, c)
+    np.testing.assert_array_equal(r["kept_1"], k1)
+    np.testing.assert_array_equal(r["kept_2"], k2)
+    np.testing.assert_array_equal(r["pos_1"], p1)
+    np.testing.assert_array_equal(r["pos_2"], p2)
+    np.testing.assert_array_equal(r["fill"], fill)
+
+
+def test_capacity_invariants():
+  rng = np.random.default_rng(7)
+  g, s, e, c = 4, 200, 8, 30
+  r = O.top_2_gating(rng.standard_normal((g, s, e)).astype(np.float32), c)
+  for gi in range(g):
+    for ex in range(e):
+      pos = np.concatenate([
+          r["pos_1"][gi][(r["index_1"][gi] == ex) & r["kept_1"][gi]],
+          r["pos_2"][gi][(r["index_2"][gi] == ex) & r["kept_2"][gi]]])
+      assert sorted(pos.tolist()) == list(range(len(pos))) and len(pos) <= c
+      assert len(pos) == r["fill"][gi, ex]
+      first = r["pos_1"][gi][(r["index_1"][gi] == ex) & r["kept_1"][gi]]
+      assert (np.diff(first) > 0).all()
+  # nothing is dropped when capacity covers both choices of every token
+  r = O.top_2_gating(rng.standard_normal((g, s, e)).astype(np.float32), 2 * s)
+  assert r["kept_1"].all() and r["kept_2"].all()
+  # all tokens to one expert: exactly the first C survive
+  one = np.zeros((1, 50, 4), np.float32)
+  one[..., 2] = 5.0
+  r = O.top_2_gating(one, 7)
+  np.testing.assert_array_equal(r["kept_1"][0], np.arange(50) < 7)
+
+
+def test_importance_semantics():
+  """importance 1 -> up to two experts; 0 < importance < 1 -> best expert only,
+  at second priority, gate ~ 1; importance 0 -> nowhere
+  (transformer/moe.py:1347-1355, :1401-1411)."""
+  rng = np.random.default_rng(8)
+  logits = rng.standard_normal((1, 9, 4)).astype(np.float32)
+  imp = np.array([[1, 0.5, 0, 1, 0.5, 0.3, 1, 0, 1]], np.float32)
+  r = O.top_2_gating(logits, 100, importance=imp)
+  half = (imp > 0) & (imp < 1)
+  assert (r["index_2"][half] == r["index_1"][half]).all()
+  assert not r["kept_1"][half].any() and r["kept_2"][half].all()
+  np.testing.assert_allclose(r["gate_2"][half], 1.0, atol=1e-6)
+  assert not r["kept_1"][imp == 0].any() and not r["kept_2"][imp == 0].any()
+  assert r["kept_1"][imp == 1].all() and r["kept_2"][imp == 1].all()
+
+
+def test_second_policies():
+  rng = np.random.default_rng(9)
+  logits = rng.standard_normal((2, 60, 6)).astype(np.float32)
+  base = O.top_2_gating(logits, 1000)
+  none = O.top_2_gating(logits, 1000, policy="none")
+  assert not none["kept_2"].any() and none["kept_1"].all()
+  thr = O.top_2_gating(logits, 1000, policy="threshold", threshold=0.3)
+  np.testing.assert_array_equal(thr["kept_2"], base["gate_2"] > np.float32(0.3))
+  u = rng.random((2, 60)).astype(np.float32)
+  rnd = O.top_2_gating(logits, 1000, policy="random", threshold=0.25,
+                       second_uniform=u)
+  np.testing.assert_array_equal(rnd["kept_2"],
+                                u < base["gate_2"] * np.float32(4.0))
+  with pytest.raises(ValueError):
+    O.top_2_gating(logits, 10, policy="sometimes")
+
+
+# ---- dense tensors, dispatch, combine -----------------------------------------
+@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
+def test_dense_tensors_match_index_record(act_dtype):
+  rng = np.random.default_rng(10)
+  g, s, e, c, m = 2, 40, 5, 9, 8
+  logits = rng.standard_normal((g, s, e)).astype(np.float32)
+  r = O.top_2_gating(logits, c, act_dtype=act_dtype, dense=True)
+  w1, w2 = O.combine_weights(r, act_dtype)
+  rebuilt = np.zeros((g, s, e, c), np.float32)
+  for gi in range(g):
+    for si in range(s):
+      if r["kept_1"][gi, si]:
+        rebuilt[gi, si, r["index_1"][gi, si], r["pos_1"][gi, si]] += w1[gi, si]
+      if r["kept_2"][gi, si]:
+        rebuilt[gi, si, r["index_2"][gi, si], r["pos_2"][gi, si]] += w2[gi, si]
+  np.testing.assert_array_equal(r["combine"], rebuilt)
+  np.testing.assert_array_equal(r["dispatch"], (rebuilt != 0).astype(np.float32))
+  assert (r["dispatch"].sum(axis=1) <= 1).all()         # one token per slot
+  x = O.cast_act(rng.standard_normal((g, s, m)).astype(np.float32), act_dtype)
+  np.testing.assert_array_equal(
+      O.dispatch_gather(x, r, e, c, act_dtype),
+      np.einsum("gsm,gsec->egcm", x, r["dispatch"]).astype(np.float32))
+  y = O.cast_act(rng.standard_normal((e, g, c, m)).astype(np.float32), act_dtype)
+  dense_out = np.einsum("egcn,gsec->gsn", y.astype(np.float64),
+                        r["combine"].astype(np.float64))
+  got = O.combine_gather(y, r, act_dtype)
+  tol = 1e-2 if act_dtype == "bfloat16" else 1e-6
+  np.testing.assert_allclose(got, dense_out, rtol=tol, atol=tol)
+
+
+def test_expert_ffn_against_float64():
+  rng = np.random.default_rng(11)
+  e, rows, m, h, n = 3, 17, 12, 20, 10
+  x = rng.standard_normal((e, rows, m)).astype(np.float32)
+  wi = rng.standard_normal((e, m, h)).astype(np.float32)
+  wo = rng.standard_normal((e, h, n)).astype(np.float32)
+  got = O.expert_ffn(x, wi, wo, "relu", "float32")
+  want = np.zeros((e, rows, n))
+  for k in range(e):   # explicit per-expert loops: a transposed operand fails
+    hid = np.maximum(x[k].astype(np.float64) @ wi[k].astype(np.float64), 0)
+    want[k] = hid @ wo[k].astype(np.float64)
+  np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-4)
+  lin = O.expert_ffn(x, wi, wo, "linear", "float32")
+  assert not np.allclose(lin, got)
+
+
+def test_balanced_routing_loss_is_one():
+  """Perfectly balanced first choices with uniform gates: density = proxy = 1/E,
+  loss = mean(1/E^2) * E^2 = 1 (transformer/moe.py:1420-1424)."""
+  e, s = 8, 64
+  logits = np.zeros((2, s, e), np.float32)
+  r = O.top_2_gating(logits, 1000)
+  # uniform gates but argmax always 0 -> density_1 = [1,0,..]: loss = 1/E * E = 1
+  np.testing.assert_allclose(r["loss"], 1.0, rtol=1e-6)
+  # truly balanced: token s prefers expert s % E by a hair (gates ~uniform)
+  logits[:, np.arange(s), np.arange(s) % e] = 1e-4
+  r = O.top_2_gating(logits, 1000)
+  np.testing.assert_allclose(r["loss"], 1.0, rtol=1e-4)
+  # all mass on one expert: density = proxy = 1 for it -> loss = E
+  logits = np.zeros((1, s, e), np.float32)
+  logits[..., 3] = 30.0
+  np.testing.assert_allclose(O.top_2_gating(logits, 1000)["loss"], e, rtol=1e-5)
+  # microbatches divide, the second-place loss adds half of a second term
+  a = O.top_2_gating(logits, 1000, num_microbatches=4)["loss"]
+  np.testing.assert_allclose(a, e / 4, rtol=1e-5)
+
+
+# ---- the layers ----------------------------------------------------------------
+def _hp(**kw):
+  base = dict(moe_second_policy_train="all", moe_second_policy_eval="all")
+  base.update(kw)
+  return O.default_hparams(**base)
+
+
+@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
+def test_v1_dense_equals_index_form(act_dtype):
+  rng = np.random.default_rng(12)
+  b, l, m, h, e = 2, 48, 16, 24, 4
+  x = rng.standard_normal((b, l, m)).astype(np.float32)
+  wg = rng.standard_normal((m, e)).astype(np.float32)
+  wi = rng.standard_normal((e, m, h)).astype(np.float32) / 4
+  wo = rng.standard_normal((e, h, m)).astype(np.float32) / 5
+  hp = _hp(moe_num_experts=e, moe_hidden_size=h, moe_group_size=32,
+           moe_capacity_factor_train=1.0)
+  nonpad = (rng.random((b, l)) < 0.8).astype(np.float32)
+  d, dl, aux = O.moe_layer_v1(x, wg, wi, wo, hp, True, act_dtype,
+                              nonpadding=nonpad, dense=True)
+  i, il, _ = O.moe_layer_v1(x, wg, wi, wo, hp, True, act_dtype,
+                            nonpadding=nonpad, dense=False)
+  tol = 1e-2 if act_dtype == "bfloat16" else 1e-5
+  np.testing.assert_allclose(d, i, rtol=tol, atol=tol)
+  assert dl == il and aux["num_groups"] == 3 and aux["group_size"] == 32
+  assert (d[nonpad == 0] == 0).all()
+  # a token that lost both choices outputs exactly zero
+  lost = ~(aux["kept_1"] | aux["kept_2"]).reshape(b, l)
+  assert (d[lost] == 0).all()
+
+
+def test_v1_single_expert_is_a_dense_ffn():
+  """E = 2 identical experts, capacity for everything: gates sum to 1, so the
+  layer equals one feed-forward network applied to every token."""
+  rng = np.random.default_rng(13)
+  b, l, m, h = 1, 16, 8, 12
+  x = rng.standard_normal((b, l, m)).astype(np.float32)
+  wi1 = rng.standard_normal((m, h)).astype(np.float32)
+  wo1 = rng.standard_normal((h, m)).astype(np.float32)
+  hp = _hp(moe_num_experts=2, moe_hidden_size=h, moe_group_size=16,
+           moe_capacity_factor_train=4.0)
+  out, _, _ = O.moe_layer_v1(x, rng.standard_normal((m, 2)).astype(np.float32),
+                             np.stack([wi1, wi1]), np.stack([wo1, wo1]), hp, True)
+  want = np.maximum(x.astype(np.float64) @ wi1, 0) @ wo1
+  np.testing.assert_allclose(out, want, rtol=1e-4, atol=1e-4)
+
+
+def test_v2_with_one_outer_expert_reduces_to_v1():
+  """x = 1 outer group with capacity for every token: the outer level passes
+  every token through with gate 1/(1+1e-9) rounding to 1, importance 1, and the
+  inner level is a v1 layer over the same tokens in the same order."""
+  rng = np.random.default_rng(14)
+  b, l, m, h, ye = 2, 32, 8, 16, 4
+  x = rng.standard_normal((b, l, m)).astype(np.float32)
+  w_outer = rng.standard_normal((m, 1)).astype(np.float32)
+  w_inner = rng.standard_normal((1, m, ye)).astype(np.float32)
+  wi = rng.standard_normal((ye, 1, m, h)).astype(np.float32) / 3
+  wo = rng.standard_normal((ye, 1, h, m)).astype(np.float32) / 4
+  hp2 = _hp(moe_num_experts=[1, ye], moe_hidden_size=h, moe_group_size=32,
+            moe_capacity_factor_train=1.0, moe_capacity_factor_second_level=1.5,
+            moe_min_expert_capacity=1)
+  out2, loss2, aux = O.moe_layer_v2(x, w_outer, w_inner, wi, wo, hp2, True)
+  assert aux["capacity_x"] == 32 and aux["groups_y"] == (2, 32)
+  assert aux["outer"]["kept_1"].all()
+  hp1 = _hp(moe_num_experts=ye, moe_hidden_size=h, moe_group_size=32,
+            moe_capacity_factor_train=1.5, moe_min_expert_capacity=1)
+  out1, loss1, _ = O.moe_layer_v1(x, w_inner[0], wi[:, 0], wo[:, 0], hp1, True)
+  np.testing.assert_allclose(out2, out1, rtol=1e-5, atol=1e-6)
+  # outer loss with one expert: density = proxy = 1 -> 1; total = (1 + inner)
+  np.testing.assert_allclose(loss2, (1.0 + loss1 / 1e-2) * 1e-2, rtol=1e-5)
+
+
+def test_v2_importance_mapping():
+  """importance = 0.5 * ((w > 0.5) + (w > 0)) on the slot weights
+  (transformer/moe.py:725-727)."""
+  w = np.array([0.0, 0.3, 0.5, 0.7], np.float32)
+  imp = np.float32(0.5) * ((w > 0.5).astype(np.float32) + (w > 0).astype(np.float32))
+  np.testing.assert_array_equal(imp, [0.0, 0.5, 0.5, 1.0])
+  rng = np.random.default_rng(15)
+  x = rng.standard_normal((2, 64, 8)).astype(np.float32)
+  hp = _hp(moe_num_experts=[4, 4], moe_hidden_size=8, moe_group_size=32)
+  _, _, aux = O.moe_layer_v2(
+      x, rng.standard_normal((8, 4)).astype(np.float32),
+      rng.standard_normal((4, 8, 4)).astype(np.float32),
+      rng.standard_normal((4, 4, 8, 8)).astype(np.float32),
+      rng.standard_normal((4, 4, 8, 8)).astype(np.float32), hp, True)
+  imp = aux["importance_inner"]
+  assert set(np.unique(imp)) <= {0.0, 0.5, 1.0}
+  n_first = int(aux["outer"]["kept_1"].sum())
+  # every kept first choice has gate > 0.5 here (no exact ties), so it becomes 1.0
+  assert int((imp == 1.0).sum()) == n_first
+  assert int((imp == 0.5).sum()) == int(aux["outer"]["kept_2"].sum())
+
+
+def test_golden_fixture():
+  """Small committed input/output vectors of the oracle itself (guards the
+  oracle against accidental edits; generated by tests/golden/make_golden.py)."""
+  path = os.path.join(GOLDEN, "top2_gating_small.json")
+  with open(path) as f:
+    gold = json.load(f)
+  logits = np.array(gold["logits"], np.float32)
+  r = O.top_2_gating(logits, gold["capacity"])
+  for k in ("index_1", "index_2", "pos_1", "pos_2"):
+    np.testing.assert_array_equal(r[k], np.array(gold[k]))
+  np.testing.assert_array_equal(r["kept_1"], np.array(gold["kept_1"], bool))
+  np.testing.assert_array_equal(r["kept_2"], np.array(gold["kept_2"], bool))
+  np.testing.assert_allclose(r["gate_1"], np.array(gold["gate_1"]), rtol=1e-6)
+  np.testing.assert_allclose(r["loss"], gold["loss"], rtol=1e-6)
