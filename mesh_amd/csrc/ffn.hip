@@ -7,6 +7,8 @@
 // K-contiguous, C [R, N] = A . B^T.  The bf16 kernel uses
 // v_mfma_f32_32x32x16_bf16 with LDS double buffering; float32 and odd shapes
 // use a plain FMA tile kernel.
+#include <stdlib.h>
+
 #include "common.h"
 
 namespace mesh_moe {
@@ -199,6 +201,209 @@ __global__ __launch_bounds__(256) void grouped_gemm_bf16_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// bf16 MFMA kernel with direct global -> LDS loads and an NS-stage ring.
+//
+// Same tiling and MFMA operand roles as the kernel above, but the K loop is fed
+// by global_load_lds_dwordx4: every lane names its own 16 global bytes and the
+// wavefront's 64 x 16 bytes land contiguously in LDS without passing through
+// registers.  The loads for K tile kt+NS-1 are issued while tile kt is being
+// multiplied; a partial vmcnt wait plus one bare s_barrier per K tile publishes
+// the oldest tile.
+//
+// One load instruction fetches 8 rows x 128 bytes (BK = 64 bf16): 8 consecutive
+// lanes read one full 128-byte line of a row, which is what the memory
+// pipeline coalesces best (lanes that stride across rows run ~4x slower).
+// LDS therefore holds plain 128-byte rows, and bank conflicts are avoided by
+// an XOR swizzle of the 16-byte chunk index applied on the GLOBAL side: the
+// lane that fills LDS slot (row, p) loads chunk p ^ swz(row), with
+// swz(row) = (row & 7) ^ ((row >> 3) & 1).  The MFMA fragment read of 16
+// consecutive rows at one chunk then touches 16 distinct 16-byte columns of a
+// 256-byte window (and any 8 consecutive rows 8 distinct columns of 128 bytes).
+// Requires K % 64 == 0 and per-expert operand sizes below 2^30 elements.
+// ---------------------------------------------------------------------------
+typedef __attribute__((address_space(3))) void lds_void_t;
+typedef const __attribute__((address_space(1))) void glb_void_t;
+
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+  // s_waitcnt with expcnt / lgkmcnt left at "no wait"
+  __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+}
+
+template <int BM, int BN, int NS>
+struct DmaCfg {
+  static constexpr int BK = 64;
+  static constexpr int THREADS = 256;
+  static constexpr int WTM = BM / 2, WTN = BN / 2;
+  static constexpr int TM = WTM / 32, TN = WTN / 32;
+  static constexpr int ROW_BYTES = BK * 2;             // 128
+  static constexpr int A_INSTR = (BM / 8) / 4;         // per wavefront
+  static constexpr int B_INSTR = (BN / 8) / 4;
+  static constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES;
+  static constexpr int STAGE_BYTES = A_BYTES + B_BYTES;
+  static constexpr int LDC = BN + 4;
+  static constexpr size_t LOOP_BYTES = (size_t)NS * STAGE_BYTES;
+  static constexpr size_t EPI_BYTES = (size_t)BM * LDC * sizeof(bf16_t);
+  static constexpr size_t LDS_BYTES =
+      LOOP_BYTES > EPI_BYTES ? LOOP_BYTES : EPI_BYTES;
+};
+
+__device__ __forceinline__ int lds_swizzle(int row) {
+  return (row & 7) ^ ((row >> 3) & 1);
+}
+
+template <int BM, int BN, int NS, bool RELU>
+__global__ __launch_bounds__(256) void grouped_gemm_bf16_dma_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
+    bf16_t* __restrict__ Cout, int R, int N, int K, int tiles_m, int tiles_n) {
+  using Cfg = DmaCfg<BM, BN, NS>;
+  constexpr int BK = Cfg::BK;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+
+  const int nblk = gridDim.x;
+  const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+  const int per_xcd = nblk >> 3, extra = nblk & 7;
+  const int logical = xcd * per_xcd + min(xcd, extra) + local;
+  const int tiles_per_e = tiles_m * tiles_n;
+  const int e = logical / tiles_per_e;
+  const int rem = logical - e * tiles_per_e;
+  const int tn = rem / tiles_m;
+  const int tm = rem - tn * tiles_m;
+  const int row0 = tm * BM, col0 = tn * BN;
+  const bf16_t* Ae = A + (int64_t)e * R * K;
+  const bf16_t* Be = B + (int64_t)e * N * K;
+  bf16_t* Ce = Cout + (int64_t)e * R * N;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  // Element offsets of the 16 bytes this lane fetches in each of its load
+  // instructions.  Instruction q of an operand covers tile rows 8q .. 8q+7;
+  // lane l fills LDS slot (row 8q + l/8, column l%8).  Wavefront w issues
+  // q = w, w + 4, ...
+  int a_off[Cfg::A_INSTR], b_off[Cfg::B_INSTR];
+#pragma unroll
+  for (int j = 0; j < Cfg::A_INSTR; ++j) {
+    const int row = (wave + 4 * j) * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ lds_swizzle(row);
+    a_off[j] = min(row0 + row, R - 1) * K + chunk * 8;
+  }
+#pragma unroll
+  for (int j = 0; j < Cfg::B_INSTR; ++j) {
+    const int row = (wave + 4 * j) * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ lds_swizzle(row);
+    b_off[j] = min(col0 + row, N - 1) * K + chunk * 8;
+  }
+  auto issue_stage = [&](int kt, int slot) {
+    unsigned char* sa = smem_raw + slot * Cfg::STAGE_BYTES;
+    unsigned char* sb = sa + Cfg::A_BYTES;
+    const bf16_t* ak = Ae + kt * BK;
+    const bf16_t* bk = Be + kt * BK;
+#pragma unroll
+    for (int j = 0; j < Cfg::A_INSTR; ++j)
+      __builtin_amdgcn_global_load_lds(
+          (glb_void_t*)(ak + a_off[j]),
+          (lds_void_t*)(sa + (wave + 4 * j) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int j = 0; j < Cfg::B_INSTR; ++j)
+      __builtin_amdgcn_global_load_lds(
+          (glb_void_t*)(bk + b_off[j]),
+          (lds_void_t*)(sb + (wave + 4 * j) * 1024), 16, 0, 0);
+  };
+
+  f32x16_t acc[Cfg::TM][Cfg::TN];
+#pragma unroll
+  for (int i = 0; i < Cfg::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < Cfg::TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  // Fragment reads: this lane reads row l % 32 of each 32-row MFMA tile of its
+  // wavefront's sub-tile, chunk 2*kk + l/32 of the K tile, at the swizzled
+  // column.  The swizzle depends only on the low four row bits, which every
+  // MFMA tile of the sub-tile shares.
+  const int fr = lane & 31, fc = lane >> 5;
+  int a_frag[BK / 16], b_frag[BK / 16];
+#pragma unroll
+  for (int kk = 0; kk < BK / 16; ++kk) {
+    const int col = ((kk * 2 + fc) ^ lds_swizzle(fr)) * 16;
+    a_frag[kk] = (wm * Cfg::WTM + fr) * Cfg::ROW_BYTES + col;
+    b_frag[kk] = (wn * Cfg::WTN + fr) * Cfg::ROW_BYTES + col;
+  }
+
+  const int nk = K / BK;
+  constexpr int LPS = Cfg::A_INSTR + Cfg::B_INSTR;  // loads per stage per lane
+#pragma unroll
+  for (int s = 0; s < NS - 1; ++s)
+    if (s < nk) issue_stage(s, s);
+  for (int kt = 0; kt < nk; ++kt) {
+    // tile kt must have landed; the NS-2 younger stages may stay in flight
+    if (kt + NS - 2 < nk) wait_vmcnt<(NS - 2) * LPS>();
+    else wait_vmcnt<0>();
+    // bare s_barrier: __syncthreads() would add a fence that drains every
+    // load in flight, including the stages that are meant to stay in flight
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (kt + NS - 1 < nk) issue_stage(kt + NS - 1, (kt + NS - 1) % NS);
+    const unsigned char* sa = smem_raw + (kt % NS) * Cfg::STAGE_BYTES;
+    const unsigned char* sb = sa + Cfg::A_BYTES;
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; ++kk) {
+      bf16x8_t af[Cfg::TM], bfr[Cfg::TN];
+#pragma unroll
+      for (int i = 0; i < Cfg::TM; ++i)
+        af[i] = *reinterpret_cast<const bf16x8_t*>(sa + a_frag[kk] + i * 32 * Cfg::ROW_BYTES);
+#pragma unroll
+      for (int j = 0; j < Cfg::TN; ++j)
+        bfr[j] = *reinterpret_cast<const bf16x8_t*>(sb + b_frag[kk] + j * 32 * Cfg::ROW_BYTES);
+#pragma unroll
+      for (int i = 0; i < Cfg::TM; ++i)
+#pragma unroll
+        for (int j = 0; j < Cfg::TN; ++j)
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[j], af[i], acc[i][j], 0, 0, 0);
+    }
+  }
+  __syncthreads();
+
+  // epilogue: round (and relu), stage the tile in LDS, coalesced stores
+  bf16_t* Cs = reinterpret_cast<bf16_t*>(smem_raw);  // [BM][LDC]
+  const int m_l = lane & 31;
+  const int n_l = (lane >> 5) * 4;
+#pragma unroll
+  for (int i = 0; i < Cfg::TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < Cfg::TN; ++j) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int row = wm * Cfg::WTM + i * 32 + m_l;
+        const int col = wn * Cfg::WTN + j * 32 + 8 * q + n_l;
+        uint2 v;
+        v.x = pack2_bf16(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], RELU);
+        v.y = pack2_bf16(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3], RELU);
+        *reinterpret_cast<uint2*>(Cs + row * Cfg::LDC + col) = v;
+      }
+    }
+  }
+  __syncthreads();
+  constexpr int CPR_C = BN / 8;  // 16-byte chunks per output row
+#pragma unroll 4
+  for (int c = tid; c < BM * CPR_C; c += Cfg::THREADS) {
+    const int r = c / CPR_C, cc = (c % CPR_C) * 8;
+    const int grow = row0 + r, gcol = col0 + cc;
+    if (grow < R && gcol < N) {
+      const uint2* s = reinterpret_cast<const uint2*>(Cs + r * Cfg::LDC + cc);
+      uint2 lo = s[0], hi = s[1];
+      *reinterpret_cast<uint4*>(Ce + (int64_t)grow * N + gcol) =
+          make_uint4(lo.x, lo.y, hi.x, hi.y);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Plain FMA tile kernel (float32, and bf16 shapes the MFMA kernel rejects):
 // 64 x 64 tile, 16-deep K step, each thread a 4 x 4 patch, float32 accumulate
 // in k order.
@@ -297,6 +502,29 @@ static int launch_mfma(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
   return 0;
 }
 
+template <int BM, int BN, int NS>
+static int launch_dma(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
+                      int R, int N, int K, bool relu, hipStream_t st) {
+  using Cfg = DmaCfg<BM, BN, NS>;
+  const int tiles_m = (R + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
+  const int64_t blocks = (int64_t)tiles_m * tiles_n * E;
+  MOE_REQUIRE(blocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
+              "expert_ffn: too many tiles (%lld)", (long long)blocks);
+  if (relu) {
+    auto k = grouped_gemm_bf16_dma_kernel<BM, BN, NS, true>;
+    MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
+    k<<<(unsigned)blocks, 256, Cfg::LDS_BYTES, st>>>(A, B, C, R, N, K, tiles_m,
+                                                      tiles_n);
+  } else {
+    auto k = grouped_gemm_bf16_dma_kernel<BM, BN, NS, false>;
+    MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
+    k<<<(unsigned)blocks, 256, Cfg::LDS_BYTES, st>>>(A, B, C, R, N, K, tiles_m,
+                                                      tiles_n);
+  }
+  MOE_CHECK_LAUNCH("expert_ffn (mfma, direct-to-LDS)");
+  return 0;
+}
+
 template <typename T>
 static int launch_simple(const T* A, const T* B, T* C, int E, int R, int N,
                          int K, bool relu, hipStream_t st) {
@@ -314,6 +542,17 @@ static int launch_simple(const T* A, const T* B, T* C, int E, int R, int N,
   return 0;
 }
 
+// Development knob: MESH_MOE_GEMM_VARIANT=0 selects the register-staged
+// large-tile kernel instead of the direct-to-LDS one.
+static int gemm_variant() {
+  static int v = -1;
+  if (v < 0) {
+    const char* s = getenv("MESH_MOE_GEMM_VARIANT");
+    v = s ? atoi(s) : 1;
+  }
+  return v;
+}
+
 // C[e] = act(A[e] . B[e]^T) for every expert.
 static int grouped_gemm(const void* A, const void* B, void* C, int E, int R,
                         int N, int K, int act, int dtype, hipStream_t st) {
@@ -329,7 +568,12 @@ static int grouped_gemm(const void* A, const void* B, void* C, int E, int R,
     if (!mfma_ok)
       rc = launch_simple<bf16_t>((const bf16_t*)A, (const bf16_t*)B,
                                  (bf16_t*)C, E, R, N, K, relu, st);
-    else if (R >= 1024 && N >= 1024)
+    else if (R >= 1024 && N >= 1024 && gemm_variant() != 0 && K % 64 == 0 &&
+             (int64_t)R * K < (1LL << 30) && (int64_t)N * K < (1LL << 30)) {
+      const bf16_t *a = (const bf16_t*)A, *b = (const bf16_t*)B;
+      bf16_t* c = (bf16_t*)C;
+      rc = launch_dma<256, 256, 2>(a, b, c, E, R, N, K, relu, st);
+    } else if (R >= 1024 && N >= 1024)
       rc = launch_mfma<256, 256, 64>((const bf16_t*)A, (const bf16_t*)B,
                                      (bf16_t*)C, E, R, N, K, relu, st);
     else
