@@ -334,37 +334,59 @@ __global__ __launch_bounds__(256) void grouped_gemm_bf16_dma_kernel(
     b_frag[kk] = (wn * Cfg::WTN + fr) * Cfg::ROW_BYTES + col;
   }
 
+  // K loop, NS = 2 slots.  The MFMA fragments are double buffered in registers:
+  // while the 16 MFMAs of step kk run, the 8 fragment reads of step kk+1 are in
+  // flight.  The hand-over to the next K tile happens before the MFMAs of the
+  // LAST step of a tile: once this lane holds that step's fragments it no
+  // longer needs the tile's LDS slot, so it waits for its own loads of the next
+  // tile, meets the other wavefronts at a bare s_barrier (__syncthreads() would
+  // add a fence that also drains the loads that are meant to stay in flight),
+  // issues the loads of tile kt+2 into the slot just freed and reads the first
+  // fragments of tile kt+1 -- all of it hidden behind the last 16 MFMAs.
+  static_assert(NS == 2, "the K loop is written for two LDS slots");
+  constexpr int KSTEPS = BK / 16;
   const int nk = K / BK;
-  constexpr int LPS = Cfg::A_INSTR + Cfg::B_INSTR;  // loads per stage per lane
-#pragma unroll
-  for (int s = 0; s < NS - 1; ++s)
-    if (s < nk) issue_stage(s, s);
-  for (int kt = 0; kt < nk; ++kt) {
-    // tile kt must have landed; the NS-2 younger stages may stay in flight
-    if (kt + NS - 2 < nk) wait_vmcnt<(NS - 2) * LPS>();
-    else wait_vmcnt<0>();
-    // bare s_barrier: __syncthreads() would add a fence that drains every
-    // load in flight, including the stages that are meant to stay in flight
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-    if (kt + NS - 1 < nk) issue_stage(kt + NS - 1, (kt + NS - 1) % NS);
-    const unsigned char* sa = smem_raw + (kt % NS) * Cfg::STAGE_BYTES;
+  bf16x8_t fa[2][Cfg::TM], fb[2][Cfg::TN];
+  auto read_frags = [&](int slot, int kk, int buf) {
+    const unsigned char* sa = smem_raw + slot * Cfg::STAGE_BYTES;
     const unsigned char* sb = sa + Cfg::A_BYTES;
 #pragma unroll
-    for (int kk = 0; kk < BK / 16; ++kk) {
-      bf16x8_t af[Cfg::TM], bfr[Cfg::TN];
+    for (int i = 0; i < Cfg::TM; ++i)
+      fa[buf][i] = *reinterpret_cast<const bf16x8_t*>(sa + a_frag[kk] + i * 32 * Cfg::ROW_BYTES);
 #pragma unroll
-      for (int i = 0; i < Cfg::TM; ++i)
-        af[i] = *reinterpret_cast<const bf16x8_t*>(sa + a_frag[kk] + i * 32 * Cfg::ROW_BYTES);
+    for (int j = 0; j < Cfg::TN; ++j)
+      fb[buf][j] = *reinterpret_cast<const bf16x8_t*>(sb + b_frag[kk] + j * 32 * Cfg::ROW_BYTES);
+  };
+
+  issue_stage(0, 0);
+  wait_vmcnt<0>();
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+  if (nk > 1) issue_stage(1, 1);
+  read_frags(0, 0, 0);
+  for (int kt = 0; kt < nk; ++kt) {
+    const int slot = kt & 1;
 #pragma unroll
-      for (int j = 0; j < Cfg::TN; ++j)
-        bfr[j] = *reinterpret_cast<const bf16x8_t*>(sb + b_frag[kk] + j * 32 * Cfg::ROW_BYTES);
+    for (int kk = 0; kk < KSTEPS; ++kk) {
+      const int cur = kk & 1, nxt = cur ^ 1;
+      if (kk + 1 < KSTEPS) {
+        read_frags(slot, kk + 1, nxt);
+      } else if (kt + 1 < nk) {
+        // fragments of the last step are in registers (lgkmcnt 0) and this
+        // lane's loads of tile kt+1 have landed (vmcnt 0)
+        __builtin_amdgcn_s_waitcnt(0x0070);
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        if (kt + 2 < nk) issue_stage(kt + 2, slot);
+        read_frags(slot ^ 1, 0, nxt);
+      }
 #pragma unroll
       for (int i = 0; i < Cfg::TM; ++i)
 #pragma unroll
         for (int j = 0; j < Cfg::TN; ++j)
-          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(bfr[j], af[i], acc[i][j], 0, 0, 0);
+          acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][j], fa[cur][i], acc[i][j], 0, 0, 0);
     }
   }
   __syncthreads();
