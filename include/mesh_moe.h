@@ -65,11 +65,15 @@ const char* mesh_moe_last_error(void);
  * batch > 1 is the inner level of the hierarchical layer, where every outer
  * expert has its own router (outer_expert_dims, moe.py:743-753).
  *   x [batch, tokens, M] dtype; w [batch, M, E] dtype; logits [batch,tokens,E]
+ *   w_packed [batch, E, M] dtype or NULL: the same weights K-contiguous (see
+ *   mesh_moe_pack_weights).  When given (bf16, M % 64 == 0, E % 4 == 0) the
+ *   projection runs on the matrix cores and is bound by reading x once.
  * `bias` is a benchmark hook (skewed-routing stress); the reference has none.
  */
-int mesh_moe_router_logits(const void* x, const void* w, const float* bias,
-                           float* logits, int batch, int64_t tokens, int M,
-                           int E, int dtype, void* stream);
+int mesh_moe_router_logits(const void* x, const void* w, const void* w_packed,
+                           const float* bias, float* logits, int batch,
+                           int64_t tokens, int M, int E, int dtype,
+                           void* stream);
 
 /* Bytes of scratch mesh_moe_top2_gating needs for (G, S, E). */
 size_t mesh_moe_gating_workspace_bytes(int G, int S, int E);

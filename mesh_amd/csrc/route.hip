@@ -77,6 +77,129 @@ __global__ __launch_bounds__(256) void router_logits_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// Router logits on the matrix cores (bf16 inputs, packed router weights
+// wp[b][e][m]).  logits^T tile = wp tile (experts as MFMA rows) x x tile (tokens
+// as MFMA columns): lane l ends up with token l % 32 of its wavefront and, per
+// 32-expert tile, experts 8*(r/4) + 4*(l/32) + r%4 in accumulator register r.
+// bf16 x bf16 products are exact in float32, so this is the float32 matmul of
+// the reference on bf16-rounded operands up to summation order.
+//
+// A block is 4 wavefronts x 32 tokens; x and wp K tiles (64 deep) are brought
+// into a two-slot LDS ring by global_load_lds_dwordx4 with the same
+// 128-byte-row XOR swizzle as the expert GEMM.  The kernel is bound by reading
+// x once from HBM.
+// ---------------------------------------------------------------------------
+typedef __attribute__((ext_vector_type(8))) __bf16 rl_bf16x8_t;
+typedef __attribute__((ext_vector_type(16))) float rl_f32x16_t;
+typedef __attribute__((address_space(3))) void rl_lds_void_t;
+typedef const __attribute__((address_space(1))) void rl_glb_void_t;
+
+__device__ __forceinline__ int rl_swizzle(int row) {
+  return (row & 7) ^ ((row >> 3) & 1);
+}
+
+template <int NT>  // number of 32-expert tiles: E <= 32 * NT
+__global__ __launch_bounds__(256) void router_mfma_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ wp,
+    const float* __restrict__ bias, float* __restrict__ logits, int tokens,
+    int M, int E) {
+  constexpr int TOK = 128, BK = 64, ROWB = 128;
+  constexpr int X_BYTES = TOK * ROWB, W_BYTES = NT * 32 * ROWB;
+  constexpr int STAGE = X_BYTES + W_BYTES;
+  extern __shared__ __attribute__((aligned(16))) unsigned char rl_smem[];
+  const int b = blockIdx.y;
+  const int t0 = blockIdx.x * TOK;
+  const bf16_t* xb = x + (int64_t)b * tokens * M;
+  const bf16_t* wb = wp + (int64_t)b * E * M;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+  // load instruction q covers tile rows 8q..8q+7; lane l fills slot
+  // (row 8q + l/8, column l%8) and fetches chunk (l%8) ^ swizzle(row)
+  int x_off[4], w_off[NT];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int row = (wave + 4 * j) * 8 + (lane >> 3);
+    x_off[j] = min(t0 + row, tokens - 1) * M + (((lane & 7) ^ rl_swizzle(row)) * 8);
+  }
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    const int row = (wave + 4 * j) * 8 + (lane >> 3);
+    w_off[j] = min(row, E - 1) * M + (((lane & 7) ^ rl_swizzle(row)) * 8);
+  }
+  auto issue = [&](int kt, int slot) {
+    unsigned char* sx = rl_smem + slot * STAGE;
+    unsigned char* sw = sx + X_BYTES;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      __builtin_amdgcn_global_load_lds(
+          (rl_glb_void_t*)(xb + kt * BK + x_off[j]),
+          (rl_lds_void_t*)(sx + (wave + 4 * j) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+      __builtin_amdgcn_global_load_lds(
+          (rl_glb_void_t*)(wb + kt * BK + w_off[j]),
+          (rl_lds_void_t*)(sw + (wave + 4 * j) * 1024), 16, 0, 0);
+  };
+
+  rl_f32x16_t acc[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[j][r] = 0.f;
+
+  const int fr = lane & 31, fc = lane >> 5;
+  int x_frag[4], w_frag[4];
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) {
+    const int col = ((kk * 2 + fc) ^ rl_swizzle(fr)) * 16;
+    x_frag[kk] = (wave * 32 + fr) * ROWB + col;
+    w_frag[kk] = fr * ROWB + col;
+  }
+  const int nk = M / BK;
+  issue(0, 0);
+  for (int kt = 0; kt < nk; ++kt) {
+    const int slot = kt & 1;
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (kt + 1 < nk) issue(kt + 1, slot ^ 1);
+    const unsigned char* sx = rl_smem + slot * STAGE;
+    const unsigned char* sw = sx + X_BYTES;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      const rl_bf16x8_t xf = *reinterpret_cast<const rl_bf16x8_t*>(sx + x_frag[kk]);
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        const rl_bf16x8_t wf =
+            *reinterpret_cast<const rl_bf16x8_t*>(sw + w_frag[kk] + j * 32 * ROWB);
+        acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, xf, acc[j], 0, 0, 0);
+      }
+    }
+  }
+  const int t = t0 + wave * 32 + (lane & 31);
+  if (t < tokens) {
+    float* out = logits + ((int64_t)b * tokens + t) * E;
+#pragma unroll
+    for (int j = 0; j < NT; ++j) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int e0 = j * 32 + 8 * q + 4 * (lane >> 5);
+        if (e0 < E) {  // E % 4 == 0, so the four experts are in range together
+          float4 v = make_float4(acc[j][4 * q], acc[j][4 * q + 1],
+                                 acc[j][4 * q + 2], acc[j][4 * q + 3]);
+          if (bias != nullptr) {
+            v.x += bias[e0]; v.y += bias[e0 + 1];
+            v.z += bias[e0 + 2]; v.w += bias[e0 + 3];
+          }
+          *reinterpret_cast<float4*>(out + e0) = v;
+        }
+      }
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Gating step 1: per token softmax, top-2, gate normalisation, second-place
 // policy; per block column sums of the balancing-loss proxies.
 // Grid (blocks per group, G); one thread per token; the logits tile is staged
@@ -349,10 +472,23 @@ static int gate_tokens_per_block(int E) {
 
 using namespace mesh_moe;
 
+template <int NT>
+static int launch_router_mfma(const bf16_t* x, const bf16_t* wp,
+                              const float* bias, float* logits, int batch,
+                              int tokens, int M, int E, hipStream_t st) {
+  const size_t smem = 2 * (128 * 128 + (size_t)NT * 32 * 128);
+  auto k = router_mfma_kernel<NT>;
+  MOE_ALLOW_LDS(k, smem);
+  dim3 grid((unsigned)((tokens + 127) / 128), (unsigned)batch);
+  k<<<grid, 256, smem, st>>>(x, wp, bias, logits, tokens, M, E);
+  MOE_CHECK_LAUNCH("router_logits (mfma)");
+  return 0;
+}
+
 extern "C" int mesh_moe_router_logits(const void* x, const void* w,
-                                      const float* bias, float* logits,
-                                      int batch, int64_t tokens, int M, int E,
-                                      int dtype, void* stream) {
+                                      const void* w_packed, const float* bias,
+                                      float* logits, int batch, int64_t tokens,
+                                      int M, int E, int dtype, void* stream) {
   MOE_REQUIRE(x && w && logits, MESH_MOE_E_ARG, "router_logits: null pointer");
   MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG, "router_logits: bad dtype %d",
               dtype);
@@ -364,6 +500,18 @@ extern "C" int mesh_moe_router_logits(const void* x, const void* w,
   MOE_REQUIRE(batch <= 65535, MESH_MOE_E_UNSUPPORTED,
               "router_logits: batch=%d > 65535", batch);
   if (tokens == 0) return 0;
+  if (dtype == MESH_MOE_BF16 && w_packed != nullptr && M % 64 == 0 &&
+      E % 4 == 0 && tokens * (int64_t)M < (1LL << 31) &&
+      (((uintptr_t)x | (uintptr_t)w_packed | (uintptr_t)logits) % 16 == 0)) {
+    const bf16_t* xb = (const bf16_t*)x;
+    const bf16_t* wp = (const bf16_t*)w_packed;
+    hipStream_t s2 = (hipStream_t)stream;
+    if (E <= 32)
+      return launch_router_mfma<1>(xb, wp, bias, logits, batch, (int)tokens, M, E, s2);
+    if (E <= 64)
+      return launch_router_mfma<2>(xb, wp, bias, logits, batch, (int)tokens, M, E, s2);
+    return launch_router_mfma<4>(xb, wp, bias, logits, batch, (int)tokens, M, E, s2);
+  }
   const int ept = (E + 3) / 4;
   dim3 grid((unsigned)((tokens + RL_TOK - 1) / RL_TOK), (unsigned)batch);
   size_t smem = sizeof(float) * (RL_TOK * (RL_KC + 1) + (size_t)RL_KC * E);

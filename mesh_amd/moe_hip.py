@@ -29,7 +29,7 @@ _SIGNATURES = {
     "mesh_moe_abi_version": (ctypes.c_int, []),
     "mesh_moe_last_error": (ctypes.c_char_p, []),
     "mesh_moe_router_logits": (ctypes.c_int, [
-        _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
+        _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, _vp]),
     "mesh_moe_gating_workspace_bytes": (ctypes.c_size_t, [
         ctypes.c_int, ctypes.c_int, ctypes.c_int]),
@@ -169,12 +169,15 @@ class _stage(object):
     return False
 
 
-def router_logits(x, w, bias=None, out=None):
-  """x [B, T, M] or [T, M]; w [B, M, E] or [M, E] -> float32 logits [.., T, E]."""
+def router_logits(x, w, bias=None, out=None, w_packed=None):
+  """x [B, T, M] or [T, M]; w [B, M, E] or [M, E] -> float32 logits [.., T, E].
+  w_packed, if given, is pack_weights(w): [B, E, M] (or [E, M])."""
   lib = load_library()
   squeeze = x.dim() == 2
   if squeeze:
     x, w = x.unsqueeze(0), w.unsqueeze(0)
+    if w_packed is not None and w_packed.dim() == 2:
+      w_packed = w_packed.unsqueeze(0)
   b, t, m = x.shape
   e = w.shape[-1]
   code = dtype_code(x.dtype)
@@ -184,8 +187,10 @@ def router_logits(x, w, bias=None, out=None):
     out = torch.empty((b, t, e), dtype=torch.float32, device=x.device)
   op = _dev(out, "logits", torch.float32, (b, t, e))
   bp = None if bias is None else _dev(bias, "bias", torch.float32, (e,))
+  pp = None if w_packed is None else _dev(w_packed, "w_packed", x.dtype,
+                                          (b, e, m))
   with _stage("router_logits"):
-    _check(lib.mesh_moe_router_logits(xp, wp, bp, op, b, t, m, e, code,
+    _check(lib.mesh_moe_router_logits(xp, wp, pp, bp, op, b, t, m, e, code,
                                       _stream()), "router_logits")
   return out[0] if squeeze else out
 

@@ -161,6 +161,7 @@ class MoEV1Operation(mtf.Operation):
     dt = x.dtype
     wi_p = _packed(lowering, wi, dt)
     wo_p = _packed(lowering, wo, dt)
+    wg_p = _packed(lowering, w_gate, dt)[0]            # [E, M]
     o_, g_, s_, m_ = x.shape.to_integer_list
     n_ = self.outputs[0].shape.dims[-1].size
     e_, c_ = self._num_experts, self._capacity
@@ -168,7 +169,8 @@ class MoEV1Operation(mtf.Operation):
 
     def fn(x_s, wg_s, imp_s=None):
       xg = x_s.reshape(groups, s_, m_)
-      logits = moe_hip.router_logits(xg.reshape(groups * s_, m_), wg_s)
+      logits = moe_hip.router_logits(xg.reshape(groups * s_, m_), wg_s,
+                                     w_packed=wg_p)
       if imp_s is not None:
         imp_s = imp_s.reshape(groups, s_)
       r = self._gating.run(logits.reshape(groups, s_, e_), c_, imp_s)
@@ -306,6 +308,8 @@ class MoEV2Operation(mtf.Operation):
     dt = x.dtype
     wi_p = _packed(lowering, wi, dt)      # [y*x, hidden, m]
     wo_p = _packed(lowering, wo, dt)      # [y*x, n, hidden]
+    w_outer_p = _packed(lowering, w_outer, dt)[0]      # [x, m]
+    w_inner_p = _packed(lowering, w_inner, dt)         # [x, y, m]
     a0, g1, s_, m_ = x.shape.to_integer_list
     n_ = self.outputs[0].shape.dims[-1].size
     x_e, y_e, c_, h0, t_, d_ = self._dims
@@ -314,14 +318,16 @@ class MoEV2Operation(mtf.Operation):
     def fn(x_s, wo_s, wi_s, imp_s=None):
       xg = x_s.reshape(ag, s_, m_)
       # outer level
-      logits_x = moe_hip.router_logits(xg.reshape(ag * s_, m_), wo_s)
+      logits_x = moe_hip.router_logits(xg.reshape(ag * s_, m_), wo_s,
+                                       w_packed=w_outer_p)
       if imp_s is not None:
         imp_s = imp_s.reshape(ag, s_)
       rx = self._gating.run(logits_x.reshape(ag, s_, x_e), c_, imp_s)
       ein_x, slot_gate = moe_hip.dispatch(xg, rx, want_slot_gate=True)
       # inner level: each outer expert's a0*g*c slots become h0 groups of t
       inputs_y = ein_x.reshape(x_e, h0 * t_, m_)
-      logits_y = moe_hip.router_logits(inputs_y, wi_s)      # [x, h0*t, y]
+      logits_y = moe_hip.router_logits(inputs_y, wi_s,
+                                       w_packed=w_inner_p)  # [x, h0*t, y]
       ry = self._gating.run(logits_y.reshape(x_e * h0, t_, y_e), d_,
                             slot_gate.reshape(x_e * h0, t_),
                             importance_from_slot_gate=True)

@@ -115,6 +115,28 @@ def test_router_logits(hip, act_dtype, shape):
                                     H.to_gpu(w, act_dtype),
                                     bias=torch.from_numpy(bias).cuda()))
   np.testing.assert_allclose(got_b, want + bias, rtol=1e-5, atol=2e-5)
+  # packed router weights: the matrix-core path for bf16 (when M % 64 == 0 and
+  # E % 4 == 0), the same FMA kernel otherwise
+  wg = H.to_gpu(w, act_dtype)
+  wp = hip.pack_weights(wg.unsqueeze(0), wg.dtype)[0]
+  got_p = H.to_np(hip.router_logits(H.to_gpu(x, act_dtype), wg, w_packed=wp,
+                                    bias=torch.from_numpy(bias).cuda()))
+  np.testing.assert_allclose(got_p, want + bias, rtol=1e-5, atol=2e-5)
+
+
+def test_router_logits_mfma_shapes(hip):
+  """Matrix-core router: ragged token counts, E = 4 .. 128, batched weights."""
+  rng = np.random.default_rng(31)
+  for b, t, m, e in [(1, 1, 64, 4), (1, 127, 128, 32), (3, 300, 192, 20),
+                     (2, 129, 64, 128), (1, 2048, 1024, 64)]:
+    x = O.round_bf16(rng.standard_normal((b, t, m)).astype(np.float32))
+    w = O.round_bf16((rng.standard_normal((b, m, e)) / np.sqrt(m)).astype(np.float32))
+    want = np.matmul(x.astype(np.float64), w.astype(np.float64))
+    wg = H.to_gpu(w, "bfloat16")
+    got = H.to_np(hip.router_logits(H.to_gpu(x, "bfloat16"), wg,
+                                    w_packed=hip.pack_weights(wg, wg.dtype)))
+    np.testing.assert_allclose(got, want, rtol=1e-5, atol=2e-5,
+                               err_msg=str((b, t, m, e)))
 
 
 def test_router_logits_batched(hip):
