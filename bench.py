@@ -161,7 +161,11 @@ def cpu_baseline(cfg):
   rng = np.random.default_rng(0)
   m, h, e, s = cfg["M"], cfg["H"], cfg["E"], cfg["group"]
   act = "bfloat16" if cfg["dtype"] == "bf16" else "float32"
-  x = O.cast_act(rng.standard_normal((1, s, m), dtype=np.float32), act)
+  total_groups = cfg["batch"] * cfg["length"] // s
+  # size the sample for roughly 10-30 s of host work (~7e11 flop/s measured on 16 cores)
+  flops_per_group = 4.0 * e * max(4, min(s, int(s * cfg["cf"] / e))) * m * h
+  n_groups = int(max(1, min(total_groups, round(1e13 / flops_per_group))))
+  x = O.cast_act(rng.standard_normal((n_groups, s, m), dtype=np.float32), act)
   wg = (rng.standard_normal((m, e), dtype=np.float32) / np.sqrt(m))
   wi1 = O.cast_act(rng.standard_normal((1, m, h), dtype=np.float32)
                    / np.float32(np.sqrt(m)), act)
@@ -183,11 +187,12 @@ def cpu_baseline(cfg):
   O.moe_layer_v1(x, wg, wi, wo, hp, True, act, dense=True,
                  weights_are_cast=True)
   dt = time.perf_counter() - t0
-  return dict(value=s / dt, unit="tokens/s", cores=int(threads), kind="port",
-              sample="1 of %d groups (%d tokens, all %d experts, dense "
+  return dict(value=n_groups * s / dt, unit="tokens/s", cores=int(threads),
+              kind="port",
+              sample="%d of %d groups (%d tokens, all %d experts, dense "
                      "formulation, one expert's weights shared by all "
                      "experts), %.1f s"
-                     % (cfg["batch"] * cfg["length"] // s, s, e, dt))
+                     % (n_groups, total_groups, n_groups * s, e, dt))
 
 
 def main():
