@@ -9,6 +9,8 @@
 // use a plain FMA tile kernel.
 #include <stdlib.h>
 
+#include <type_traits>
+
 #include "common.h"
 
 namespace mesh_moe {
@@ -365,21 +367,25 @@ __global__ __launch_bounds__(256) void grouped_gemm_bf16_dma_kernel(
   asm volatile("" ::: "memory");
   if (nk > 1) issue_stage(1, 1);
   read_frags(0, 0, 0);
-  for (int kt = 0; kt < nk; ++kt) {
+  // One K tile.  LAST = the final tile (no hand-over).  The body is free of
+  // branches so that the scheduling hints below see one basic block; past the
+  // end of K the hand-over simply re-fetches the last tile into the free slot.
+  auto k_tile = [&](int kt, auto last_tag) {
+    constexpr bool LAST = decltype(last_tag)::value;
     const int slot = kt & 1;
 #pragma unroll
     for (int kk = 0; kk < KSTEPS; ++kk) {
       const int cur = kk & 1, nxt = cur ^ 1;
       if (kk + 1 < KSTEPS) {
         read_frags(slot, kk + 1, nxt);
-      } else if (kt + 1 < nk) {
+      } else if (!LAST) {
         // fragments of the last step are in registers (lgkmcnt 0) and this
         // lane's loads of tile kt+1 have landed (vmcnt 0)
         __builtin_amdgcn_s_waitcnt(0x0070);
         asm volatile("" ::: "memory");
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        if (kt + 2 < nk) issue_stage(kt + 2, slot);
+        issue_stage(min(kt + 2, nk - 1), slot);
         read_frags(slot ^ 1, 0, nxt);
       }
 #pragma unroll
@@ -387,8 +393,27 @@ __global__ __launch_bounds__(256) void grouped_gemm_bf16_dma_kernel(
 #pragma unroll
         for (int j = 0; j < Cfg::TN; ++j)
           acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[cur][j], fa[cur][i], acc[i][j], 0, 0, 0);
+      // Spread the memory instructions of this step between its MFMAs instead
+      // of letting them queue up in front (masks: 0x8 MFMA, 0x20 VMEM read,
+      // 0x100 LDS read).
+      if (kk + 1 < KSTEPS) {
+#pragma unroll
+        for (int g = 0; g < Cfg::TM + Cfg::TN; ++g) {
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+        }
+      } else if (!LAST) {
+#pragma unroll
+        for (int g = 0; g < Cfg::TM + Cfg::TN; ++g) {
+          __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
+          __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+          __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+      }
     }
-  }
+  };
+  for (int kt = 0; kt + 1 < nk; ++kt) k_tile(kt, std::false_type{});
+  k_tile(nk - 1, std::true_type{});
   __syncthreads();
 
   // epilogue: round (and relu), stage the tile in LDS, coalesced stores
