@@ -396,17 +396,20 @@ __global__ __launch_bounds__(256) void grouped_gemm_bf16_dma_kernel(
       // Spread the memory instructions of this step between its MFMAs instead
       // of letting them queue up in front (masks: 0x8 MFMA, 0x20 VMEM read,
       // 0x100 LDS read).
+      constexpr int READS = Cfg::TM + Cfg::TN;
+      constexpr int MFMA_PER_READ = Cfg::TM * Cfg::TN / READS;
+      constexpr int LOADS = Cfg::A_INSTR + Cfg::B_INSTR;
       if (kk + 1 < KSTEPS) {
 #pragma unroll
-        for (int g = 0; g < Cfg::TM + Cfg::TN; ++g) {
+        for (int g = 0; g < READS; ++g) {
           __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
+          __builtin_amdgcn_sched_group_barrier(0x008, MFMA_PER_READ, 0);
         }
       } else if (!LAST) {
 #pragma unroll
-        for (int g = 0; g < Cfg::TM + Cfg::TN; ++g) {
+        for (int g = 0; g < READS; ++g) {
           __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-          __builtin_amdgcn_sched_group_barrier(0x020, 2, 0);
+          __builtin_amdgcn_sched_group_barrier(0x020, (LOADS + READS - 1) / READS, 0);
           __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
         }
       }
@@ -615,11 +618,17 @@ static int grouped_gemm(const void* A, const void* B, void* C, int E, int R,
     if (!mfma_ok)
       rc = launch_simple<bf16_t>((const bf16_t*)A, (const bf16_t*)B,
                                  (bf16_t*)C, E, R, N, K, relu, st);
-    else if (R >= 1024 && N >= 1024 && gemm_variant() != 0 && K % 64 == 0 &&
+    else if (N >= 256 && R >= 128 && gemm_variant() != 0 && K % 64 == 0 &&
              (int64_t)R * K < (1LL << 30) && (int64_t)N * K < (1LL << 30)) {
+      // direct-to-LDS kernels; 256-row tiles unless 128-row tiles waste fewer
+      // padded rows (e.g. 640 rows per expert: 5 x 128 instead of 3 x 256)
       const bf16_t *a = (const bf16_t*)A, *b = (const bf16_t*)B;
       bf16_t* c = (bf16_t*)C;
-      rc = launch_dma<256, 256, 2>(a, b, c, E, R, N, K, relu, st);
+      const int pad256 = (R + 255) / 256 * 256, pad128 = (R + 127) / 128 * 128;
+      if (pad128 < pad256)
+        rc = launch_dma<128, 256, 2>(a, b, c, E, R, N, K, relu, st);
+      else
+        rc = launch_dma<256, 256, 2>(a, b, c, E, R, N, K, relu, st);
     } else if (R >= 1024 && N >= 1024)
       rc = launch_mfma<256, 256, 64>((const bf16_t*)A, (const bf16_t*)B,
                                      (bf16_t*)C, E, R, N, K, relu, st);
