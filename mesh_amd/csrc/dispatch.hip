@@ -60,11 +60,24 @@ __global__ __launch_bounds__(256) void dispatch_kernel(
       uint4* d0 = reinterpret_cast<uint4*>(dst[0]);
       uint4* d1 = reinterpret_cast<uint4*>(dst[1]);
       const uint4 z = make_uint4(0, 0, 0, 0);
-#pragma unroll 4
-      for (int i = lane; i < nv; i += 64) {
-        uint4 v = s4[i];
-        if (d0) d0[i] = zero[0] ? z : v;
-        if (d1) d1[i] = zero[1] ? z : v;
+      // four independent 16-byte loads in flight per lane before any store
+      constexpr int UN = 4;
+      const bool has0 = d0 != nullptr, has1 = d1 != nullptr;
+      for (int base = lane; base < nv; base += 64 * UN) {
+        uint4 v[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+          const int i = base + u * 64;
+          v[u] = i < nv ? s4[i] : z;
+        }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+          const int i = base + u * 64;
+          if (i < nv) {
+            if (has0) d0[i] = zero[0] ? z : v[u];
+            if (has1) d1[i] = zero[1] ? z : v[u];
+          }
+        }
       }
     } else {
       for (int i = lane; i < M; i += 64) {
@@ -161,11 +174,22 @@ __global__ __launch_bounds__(256) void combine_kernel(
     const uint4* a4 = reinterpret_cast<const uint4*>(src[0]);
     const uint4* b4 = reinterpret_cast<const uint4*>(src[1]);
     const uint4 z = make_uint4(0, 0, 0, 0);
-#pragma unroll 4
-    for (int i = lane; i < nv; i += 64) {
-      uint4 a = a4 ? a4[i] : z;
-      uint4 b = b4 ? b4[i] : z;
-      d4[i] = combine_vec<T>(a, b, w[0], w[1]);
+    // all loads of a batch are issued before the first use
+    constexpr int UN = 4;
+    const bool has_a = a4 != nullptr, has_b = b4 != nullptr;
+    for (int base = lane; base < nv; base += 64 * UN) {
+      uint4 a[UN], b[UN];
+#pragma unroll
+      for (int u = 0; u < UN; ++u) {
+        const int i = base + u * 64;
+        a[u] = (has_a && i < nv) ? a4[i] : z;
+        b[u] = (has_b && i < nv) ? b4[i] : z;
+      }
+#pragma unroll
+      for (int u = 0; u < UN; ++u) {
+        const int i = base + u * 64;
+        if (i < nv) d4[i] = combine_vec<T>(a[u], b[u], w[0], w[1]);
+      }
     }
   } else {
     for (int i = lane; i < N; i += 64) {
