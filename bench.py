@@ -22,6 +22,13 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 if ROOT not in sys.path:
   sys.path.insert(0, ROOT)
 
+# Bytes crossing the L2 <-> fabric boundary per grouped-GEMM launch, from
+# `rocprofv3 --pmc FETCH_SIZE` and `--pmc WRITE_SIZE` runs of this script
+# (scaled by what the same counters read for a 1 GiB copy: 2.0 and 1.0; the
+# summary with the commands is profiles/hbm_traffic_cfg4_pmc.txt).  Mean of the
+# wi and wo launches.  Measured offline: the counters cannot be read from here.
+MEASURED_GEMM_TRAFFIC_BYTES = {4: 29.8e9}
+
 # MI355X published peaks
 HBM_PEAK_GBS = 8000.0
 MFMA_PEAK_TFLOPS = {"bf16": 2500.0, "f32": 157.3}
@@ -143,6 +150,8 @@ def stage_model(cfg, kept_pairs, slots):
   return {
       "router_logits": dict(bytes=t * m * b + m * e * b + t * e * 4),
       "top2_gating": dict(bytes=t * (4 * e + 26)),
+      # fused projection + gating: the logits never reach HBM
+      "router_top2_gating": dict(bytes=t * m * b + m * e * b + 26 * t),
       "dispatch": dict(bytes=t * m * b + r * m * b + 18 * t),
       "combine": dict(bytes=r * m * b + t * m * b + 26 * t),
       "expert_ffn": dict(flops=4 * r * m * h, padded_flops=4 * slots * m * h),
@@ -262,7 +271,8 @@ def main():
     result["roofline"] = {
         "kernel": "grouped expert GEMM (expert_ffn, 2 launches/step)",
         "bound": "mfma", "achieved": achieved, "peak": peak,
-        "unit": "TFLOP/s", "frac": achieved / peak, "traffic": None,
+        "unit": "TFLOP/s", "frac": achieved / peak,
+        "traffic": MEASURED_GEMM_TRAFFIC_BYTES.get(args.config),
         "flops_per_launch": flops_per_launch,
         "avg_launch_ms": ffn_ms / 2,
         "padded_frac": (model["expert_ffn"]["padded_flops"] / 2

@@ -112,6 +112,27 @@ int mesh_moe_top2_gating(const float* logits, const void* importance,
                          void* stream);
 
 /*
+ * Router projection and top-2 gating in one call: what _top_2_gating does from
+ * `to_float(inputs)` to the per-token assignment (transformer/moe.py:1384-1496),
+ * with the logits kept in LDS between the matrix-core projection and the
+ * softmax / top-2 step (they are written to `logits` [G,S,E] only if it is not
+ * NULL).  Arguments are those of mesh_moe_router_logits (packed weights only)
+ * followed by those of mesh_moe_top2_gating; batch * tokens == G * S and each
+ * weight set covers whole groups.
+ * Returns MESH_MOE_E_UNSUPPORTED (nothing launched) unless dtype is bf16,
+ * M % 64 == 0, E % 4 == 0, E <= 128 and S % 128 == 0; callers then use the two
+ * separate entry points.
+ */
+int mesh_moe_router_top2_gating(
+    const void* x, const void* w_packed, const float* bias, float* logits,
+    int batch, int64_t tokens, int M, int dtype, const void* importance,
+    int importance_dtype, int importance_from_slot_gate,
+    const float* second_uniform, int G, int S, int E, int C, int policy,
+    double threshold, int use_second_place_loss, int num_microbatches,
+    int32_t* idx, int32_t* pos, float* gate, uint8_t* kept, int32_t* fill,
+    float* loss, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
  * Dispatch: expert_in[e,g,c,:] = x[g,s,:] for the token holding slot (e,g,c),
  * zero rows for empty slots.  Replaces the one-hot dispatch einsum
  * (transformer/moe.py:443-447; a slot whose activation-dtype gate is exactly

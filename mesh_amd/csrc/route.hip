@@ -220,30 +220,19 @@ struct GateParams {
 // bit 0 of the step-1 `kept` byte: the token competes for a slot (mask_k after
 // importance and policy); bit 1 (second choice only): mask_2 before the policy,
 // which is what the second-place loss counts (moe.py:1430).
+//
+// gate_select_tile does the work for `ntok` tokens (tokens t0 .. of group g,
+// block `blk` of the group) whose logits already sit in LDS as tile[ntok][ld];
+// every thread of the block must call it.
 template <typename IT>
-__global__ __launch_bounds__(256) void gate_select_kernel(
-    const float* __restrict__ logits, const IT* __restrict__ importance,
-    const float* __restrict__ second_uniform, GateParams p,
-    int32_t* __restrict__ idx, int32_t* __restrict__ pos,
+__device__ __forceinline__ void gate_select_tile(
+    float* tile, float* isone, int ld, int ntok, int g, int blk, int t0,
+    const IT* __restrict__ importance, const float* __restrict__ second_uniform,
+    const GateParams& p, int32_t* __restrict__ idx, int32_t* __restrict__ pos,
     float* __restrict__ gate, uint8_t* __restrict__ kept,
     float* __restrict__ part1, float* __restrict__ part2) {
-  extern __shared__ float smem[];
   const int E = p.E, S = p.S;
-  const int ld = E + 1;
-  float* tile = smem;                                  // [tt][E+1]
-  float* isone = smem + (size_t)p.tt * ld;             // [tt]
-  const int g = blockIdx.y;
-  const int blk = blockIdx.x;
-  const int t0 = blk * p.tt;
-  const int ntok = min(p.tt, S - t0);
   const int tid = threadIdx.x;
-  const float* src = logits + ((int64_t)g * S + t0) * E;
-  for (int i = tid; i < ntok * E; i += blockDim.x) {
-    int r = i / E, c = i - r * E;
-    tile[r * ld + c] = src[i];
-  }
-  __syncthreads();
-
   float qscale = 0.f;
   int i1 = 0;
   bool sel1 = false;
@@ -326,6 +315,151 @@ __global__ __launch_bounds__(256) void gate_select_kernel(
       part2[((int64_t)g * p.nblk + blk) * E + e] = s;
     }
   }
+}
+
+template <typename IT>
+__global__ __launch_bounds__(256) void gate_select_kernel(
+    const float* __restrict__ logits, const IT* __restrict__ importance,
+    const float* __restrict__ second_uniform, GateParams p,
+    int32_t* __restrict__ idx, int32_t* __restrict__ pos,
+    float* __restrict__ gate, uint8_t* __restrict__ kept,
+    float* __restrict__ part1, float* __restrict__ part2) {
+  extern __shared__ float smem[];
+  const int E = p.E, S = p.S;
+  const int ld = E + 1;
+  float* tile = smem;                                  // [tt][E+1]
+  float* isone = smem + (size_t)p.tt * ld;             // [tt]
+  const int g = blockIdx.y;
+  const int blk = blockIdx.x;
+  const int t0 = blk * p.tt;
+  const int ntok = min(p.tt, S - t0);
+  const int tid = threadIdx.x;
+  const float* src = logits + ((int64_t)g * S + t0) * E;
+  for (int i = tid; i < ntok * E; i += blockDim.x) {
+    int r = i / E, c = i - r * E;
+    tile[r * ld + c] = src[i];
+  }
+  __syncthreads();
+  gate_select_tile<IT>(tile, isone, ld, ntok, g, blk, t0, importance,
+                       second_uniform, p, idx, pos, gate, kept, part1, part2);
+}
+
+// ---------------------------------------------------------------------------
+// Router projection fused with gating step 1: the K loop of router_mfma_kernel,
+// then the block's 128 x E logits go from the accumulators to LDS (never to
+// HBM unless `logits` is given) and gate_select_tile runs on them.  Needs the
+// group size to be a multiple of 128 so that a block's tokens share a group.
+// ---------------------------------------------------------------------------
+template <int NT, typename IT>
+__global__ __launch_bounds__(256) void router_gate_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ wp,
+    const float* __restrict__ bias, float* __restrict__ logits,
+    int64_t tokens_total, int M, const IT* __restrict__ importance,
+    const float* __restrict__ second_uniform, GateParams p,
+    int32_t* __restrict__ idx, int32_t* __restrict__ pos,
+    float* __restrict__ gate, uint8_t* __restrict__ kept,
+    float* __restrict__ part1, float* __restrict__ part2,
+    int tokens_per_batch) {
+  constexpr int TOK = 128, BK = 64, ROWB = 128;
+  constexpr int X_BYTES = TOK * ROWB, W_BYTES = NT * 32 * ROWB;
+  constexpr int STAGE = X_BYTES + W_BYTES;
+  extern __shared__ __attribute__((aligned(16))) unsigned char rl_smem[];
+  const int E = p.E;
+  const int64_t tok0 = (int64_t)blockIdx.x * TOK;       // first token, flat
+  const int b = (int)(tok0 / tokens_per_batch);         // router weight set
+  const bf16_t* xb = x + tok0 * M;
+  const bf16_t* wb = wp + (int64_t)b * E * M;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+
+  int x_off[4], w_off[NT];
+#pragma unroll
+  for (int j = 0; j < 4; ++j) {
+    const int row = (wave + 4 * j) * 8 + (lane >> 3);
+    x_off[j] = row * M + (((lane & 7) ^ rl_swizzle(row)) * 8);
+  }
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+    const int row = (wave + 4 * j) * 8 + (lane >> 3);
+    w_off[j] = min(row, E - 1) * M + (((lane & 7) ^ rl_swizzle(row)) * 8);
+  }
+  auto issue = [&](int kt, int slot) {
+    unsigned char* sx = rl_smem + slot * STAGE;
+    unsigned char* sw = sx + X_BYTES;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+      __builtin_amdgcn_global_load_lds(
+          (rl_glb_void_t*)(xb + kt * BK + x_off[j]),
+          (rl_lds_void_t*)(sx + (wave + 4 * j) * 1024), 16, 0, 0);
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+      __builtin_amdgcn_global_load_lds(
+          (rl_glb_void_t*)(wb + kt * BK + w_off[j]),
+          (rl_lds_void_t*)(sw + (wave + 4 * j) * 1024), 16, 0, 0);
+  };
+  rl_f32x16_t acc[NT];
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[j][r] = 0.f;
+  const int fr = lane & 31, fc = lane >> 5;
+  int x_frag[4], w_frag[4];
+#pragma unroll
+  for (int kk = 0; kk < 4; ++kk) {
+    const int col = ((kk * 2 + fc) ^ rl_swizzle(fr)) * 16;
+    x_frag[kk] = (wave * 32 + fr) * ROWB + col;
+    w_frag[kk] = fr * ROWB + col;
+  }
+  const int nk = M / BK;
+  issue(0, 0);
+  for (int kt = 0; kt < nk; ++kt) {
+    const int slot = kt & 1;
+    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+    if (kt + 1 < nk) issue(kt + 1, slot ^ 1);
+    const unsigned char* sx = rl_smem + slot * STAGE;
+    const unsigned char* sw = sx + X_BYTES;
+#pragma unroll
+    for (int kk = 0; kk < 4; ++kk) {
+      const rl_bf16x8_t xf = *reinterpret_cast<const rl_bf16x8_t*>(sx + x_frag[kk]);
+#pragma unroll
+      for (int j = 0; j < NT; ++j) {
+        const rl_bf16x8_t wf =
+            *reinterpret_cast<const rl_bf16x8_t*>(sw + w_frag[kk] + j * 32 * ROWB);
+        acc[j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(wf, xf, acc[j], 0, 0, 0);
+      }
+    }
+  }
+  __syncthreads();  // every wavefront is done with the ring: reuse it
+
+  // accumulators -> LDS logits tile [128][E + 1]
+  float* tile = reinterpret_cast<float*>(rl_smem);
+  const int ld = E + 1;
+  float* isone = tile + TOK * ld;
+  const int trow = wave * 32 + (lane & 31);
+#pragma unroll
+  for (int j = 0; j < NT; ++j) {
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int e0 = j * 32 + 8 * q + 4 * (lane >> 5);
+      if (e0 < E) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          float v = acc[j][4 * q + r];
+          if (bias != nullptr) v += bias[e0 + r];
+          tile[trow * ld + e0 + r] = v;
+          if (logits != nullptr) logits[(tok0 + trow) * E + e0 + r] = v;
+        }
+      }
+    }
+  }
+  __syncthreads();
+  const int g = (int)(tok0 / p.S);
+  const int t0 = (int)(tok0 - (int64_t)g * p.S);
+  gate_select_tile<IT>(tile, isone, ld, TOK, g, t0 / TOK, t0, importance,
+                       second_uniform, p, idx, pos, gate, kept, part1, part2);
+  (void)tokens_total;
 }
 
 // ---------------------------------------------------------------------------
@@ -529,22 +663,30 @@ extern "C" int mesh_moe_router_logits(const void* x, const void* w,
   return 0;
 }
 
-extern "C" size_t mesh_moe_gating_workspace_bytes(int G, int S, int E) {
-  if (G < 1 || S < 1 || E < 1) return 0;
-  const int tt = gate_tokens_per_block(E);
-  const size_t nblk = (size_t)(S + tt - 1) / tt;
-  return sizeof(float) * (2 * (size_t)G * nblk * E + 2 * (size_t)G) + 256;
+// Gating steps 2 and 3 (capacity positions, balancing loss) for every group.
+static int launch_capacity_and_loss(const GateParams& p, int32_t* idx,
+                                    int32_t* pos, float* gate, uint8_t* kept,
+                                    int32_t* fill, float* loss,
+                                    const float* part1, const float* part2,
+                                    float* gsum, hipStream_t st) {
+  int el = 2;
+  while (el < p.E) el *= 2;
+  size_t smem = sizeof(int32_t) * (CAP_THREADS + 3 * (size_t)el) +
+                sizeof(float) * 2 * (size_t)el +
+                sizeof(int16_t) * 3 * (size_t)p.S;
+  MOE_ALLOW_LDS(gate_capacity_kernel, smem);
+  gate_capacity_kernel<<<p.G, CAP_THREADS, smem, st>>>(
+      p, idx, pos, gate, kept, fill, part1, part2, gsum, el);
+  MOE_CHECK_LAUNCH("gate_capacity");
+  gate_loss_kernel<<<1, 64, 0, st>>>(p, gsum, loss);
+  MOE_CHECK_LAUNCH("gate_loss");
+  return 0;
 }
 
-extern "C" int mesh_moe_top2_gating(
-    const float* logits, const void* importance, int importance_dtype,
-    int importance_from_slot_gate, const float* second_uniform, int G, int S,
-    int E, int C, int policy,
-    double threshold, int use_second_place_loss, int num_microbatches,
-    int32_t* idx, int32_t* pos, float* gate, uint8_t* kept, int32_t* fill,
-    float* loss, void* workspace, size_t workspace_bytes, void* stream) {
-  MOE_REQUIRE(logits && idx && pos && gate && kept && fill && loss && workspace,
-              MESH_MOE_E_ARG, "top2_gating: null pointer");
+static int check_gating_args(int G, int S, int E, int C, int policy,
+                             const float* second_uniform,
+                             const void* importance, int importance_dtype,
+                             size_t workspace_bytes) {
   MOE_REQUIRE(G >= 1 && S >= 1 && C >= 1, MESH_MOE_E_ARG,
               "top2_gating: bad sizes G=%d S=%d C=%d", G, S, C);
   MOE_REQUIRE(E >= 2 && E <= 512, MESH_MOE_E_UNSUPPORTED,
@@ -563,6 +705,13 @@ extern "C" int mesh_moe_top2_gating(
   MOE_REQUIRE(workspace_bytes >= mesh_moe_gating_workspace_bytes(G, S, E),
               MESH_MOE_E_ARG, "top2_gating: workspace too small (%zu < %zu)",
               workspace_bytes, mesh_moe_gating_workspace_bytes(G, S, E));
+  return 0;
+}
+
+static GateParams make_gate_params(int G, int S, int E, int C, int policy,
+                                   double threshold, int use_second_place_loss,
+                                   int num_microbatches,
+                                   int importance_from_slot_gate, int tt) {
   GateParams p;
   p.G = G; p.S = S; p.E = E; p.C = C;
   p.policy = policy;
@@ -571,8 +720,53 @@ extern "C" int mesh_moe_top2_gating(
   p.use_second_place_loss = use_second_place_loss ? 1 : 0;
   p.num_microbatches = num_microbatches;
   p.importance_from_slot_gate = importance_from_slot_gate ? 1 : 0;
-  p.tt = gate_tokens_per_block(E);
-  p.nblk = (S + p.tt - 1) / p.tt;
+  p.tt = tt;
+  p.nblk = (S + tt - 1) / tt;
+  return p;
+}
+
+template <int NT, typename IT>
+static int launch_router_gate(const bf16_t* x, const bf16_t* wp,
+                              const float* bias, float* logits, int64_t tokens,
+                              int M, const void* importance,
+                              const float* second_uniform, const GateParams& p,
+                              int32_t* idx, int32_t* pos, float* gate,
+                              uint8_t* kept, float* part1, float* part2,
+                              int tokens_per_batch, hipStream_t st) {
+  const size_t ring = 2 * (128 * 128 + (size_t)NT * 32 * 128);
+  const size_t tile = sizeof(float) * (128 * (size_t)(p.E + 1) + 128);
+  const size_t smem = ring > tile ? ring : tile;
+  auto k = router_gate_kernel<NT, IT>;
+  MOE_ALLOW_LDS(k, smem);
+  k<<<(unsigned)(tokens / 128), 256, smem, st>>>(
+      x, wp, bias, logits, tokens, M, (const IT*)importance, second_uniform, p,
+      idx, pos, gate, kept, part1, part2, tokens_per_batch);
+  MOE_CHECK_LAUNCH("router_gate");
+  return 0;
+}
+
+extern "C" size_t mesh_moe_gating_workspace_bytes(int G, int S, int E) {
+  if (G < 1 || S < 1 || E < 1) return 0;
+  const size_t nblk = (size_t)(S + 63) / 64;  // smallest token block of any path
+  return sizeof(float) * (2 * (size_t)G * nblk * E + 2 * (size_t)G) + 256;
+}
+
+extern "C" int mesh_moe_top2_gating(
+    const float* logits, const void* importance, int importance_dtype,
+    int importance_from_slot_gate, const float* second_uniform, int G, int S,
+    int E, int C, int policy,
+    double threshold, int use_second_place_loss, int num_microbatches,
+    int32_t* idx, int32_t* pos, float* gate, uint8_t* kept, int32_t* fill,
+    float* loss, void* workspace, size_t workspace_bytes, void* stream) {
+  MOE_REQUIRE(logits && idx && pos && gate && kept && fill && loss && workspace,
+              MESH_MOE_E_ARG, "top2_gating: null pointer");
+  if (int rc = check_gating_args(G, S, E, C, policy, second_uniform, importance,
+                                 importance_dtype, workspace_bytes))
+    return rc;
+  GateParams p = make_gate_params(G, S, E, C, policy, threshold,
+                                  use_second_place_loss, num_microbatches,
+                                  importance_from_slot_gate,
+                                  gate_tokens_per_block(E));
   hipStream_t st = (hipStream_t)stream;
   uintptr_t wsp = ((uintptr_t)workspace + 255) & ~(uintptr_t)255;
   float* part1 = (float*)wsp;
@@ -597,18 +791,62 @@ extern "C" int mesh_moe_top2_gating(
     }
     MOE_CHECK_LAUNCH("gate_select");
   }
-  {
-    int el = 2;
-    while (el < E) el *= 2;
-    size_t smem = sizeof(int32_t) * (CAP_THREADS + 3 * (size_t)el) +
-                  sizeof(float) * 2 * (size_t)el +
-                  sizeof(int16_t) * 3 * (size_t)S;
-    MOE_ALLOW_LDS(gate_capacity_kernel, smem);
-    gate_capacity_kernel<<<G, CAP_THREADS, smem, st>>>(
-        p, idx, pos, gate, kept, fill, part1, part2, gsum, el);
-    MOE_CHECK_LAUNCH("gate_capacity");
-  }
-  gate_loss_kernel<<<1, 64, 0, st>>>(p, gsum, loss);
-  MOE_CHECK_LAUNCH("gate_loss");
-  return 0;
+  return launch_capacity_and_loss(p, idx, pos, gate, kept, fill, loss, part1,
+                                  part2, gsum, st);
+}
+
+extern "C" int mesh_moe_router_top2_gating(
+    const void* x, const void* w_packed, const float* bias, float* logits,
+    int batch, int64_t tokens, int M, int dtype, const void* importance,
+    int importance_dtype, int importance_from_slot_gate,
+    const float* second_uniform, int G, int S, int E, int C, int policy,
+    double threshold, int use_second_place_loss, int num_microbatches,
+    int32_t* idx, int32_t* pos, float* gate, uint8_t* kept, int32_t* fill,
+    float* loss, void* workspace, size_t workspace_bytes, void* stream) {
+  MOE_REQUIRE(x && w_packed && idx && pos && gate && kept && fill && loss &&
+                  workspace, MESH_MOE_E_ARG, "router_top2_gating: null pointer");
+  if (int rc = check_gating_args(G, S, E, C, policy, second_uniform, importance,
+                                 importance_dtype, workspace_bytes))
+    return rc;
+  MOE_REQUIRE(batch >= 1 && (int64_t)batch * tokens == (int64_t)G * S,
+              MESH_MOE_E_ARG,
+              "router_top2_gating: batch*tokens=%lld != G*S=%lld",
+              (long long)batch * tokens, (long long)G * S);
+  MOE_REQUIRE(dtype == MESH_MOE_BF16 && M % 64 == 0 && E % 4 == 0 && E <= 128 &&
+                  S % 128 == 0 && tokens % S == 0 &&
+                  (int64_t)128 * M < (1LL << 31) &&
+                  (((uintptr_t)x | (uintptr_t)w_packed) % 16 == 0),
+              MESH_MOE_E_UNSUPPORTED,
+              "router_top2_gating: the fused kernel needs bf16, M %% 64 == 0, "
+              "E %% 4 == 0, E <= 128, S %% 128 == 0 (M=%d E=%d S=%d dtype=%d); "
+              "use router_logits + top2_gating", M, E, S, dtype);
+  GateParams p = make_gate_params(G, S, E, C, policy, threshold,
+                                  use_second_place_loss, num_microbatches,
+                                  importance_from_slot_gate, 128);
+  hipStream_t st = (hipStream_t)stream;
+  uintptr_t wsp = ((uintptr_t)workspace + 255) & ~(uintptr_t)255;
+  float* part1 = (float*)wsp;
+  float* part2 = part1 + (size_t)G * p.nblk * E;
+  float* gsum = part2 + (size_t)G * p.nblk * E;
+  const bf16_t* xb = (const bf16_t*)x;
+  const bf16_t* wp = (const bf16_t*)w_packed;
+  const int64_t total = (int64_t)G * S;
+  const bool imp_bf16 = importance && importance_dtype == MESH_MOE_BF16;
+  int rc;
+#define MOE_ROUTER_GATE(NT)                                                    \
+  (imp_bf16 ? launch_router_gate<NT, bf16_t>(xb, wp, bias, logits, total, M,   \
+                                             importance, second_uniform, p,    \
+                                             idx, pos, gate, kept, part1,      \
+                                             part2, (int)tokens, st)           \
+            : launch_router_gate<NT, float>(xb, wp, bias, logits, total, M,    \
+                                            importance, second_uniform, p,     \
+                                            idx, pos, gate, kept, part1,       \
+                                            part2, (int)tokens, st))
+  if (E <= 32) rc = MOE_ROUTER_GATE(1);
+  else if (E <= 64) rc = MOE_ROUTER_GATE(2);
+  else rc = MOE_ROUTER_GATE(4);
+#undef MOE_ROUTER_GATE
+  if (rc != 0) return rc;
+  return launch_capacity_and_loss(p, idx, pos, gate, kept, fill, loss, part1,
+                                  part2, gsum, st);
 }

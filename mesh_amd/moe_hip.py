@@ -38,6 +38,12 @@ _SIGNATURES = {
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_double, ctypes.c_int,
         ctypes.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_size_t,
         _vp]),
+    "mesh_moe_router_top2_gating": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
+        ctypes.c_int, _vp, ctypes.c_int, ctypes.c_int, _vp, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_double, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, _vp, _vp,
+        _vp, _vp, ctypes.c_size_t, _vp]),
     "mesh_moe_dispatch": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
@@ -242,6 +248,69 @@ def top2_gating(logits, capacity, importance=None, policy="all",
   if _timer is not None:
     _timer.routing.append(r)
   return r
+
+
+def fused_gating_supported(x, num_experts, group_size):
+  """True if mesh_moe_router_top2_gating has a kernel for this case."""
+  return (x.dtype == torch.bfloat16 and x.shape[-1] % 64 == 0 and
+          num_experts % 4 == 0 and num_experts <= 128 and group_size % 128 == 0)
+
+
+def router_top2_gating(x, w_packed, group_size, capacity, importance=None,
+                       policy="all", threshold=0.2,
+                       use_second_place_loss=False, num_microbatches=None,
+                       second_uniform=None, importance_from_slot_gate=False,
+                       bias=None, want_logits=False):
+  """Router projection + top-2 gating in one launch sequence.
+
+  x [B, T, M] bf16 with w_packed [B, E, M] (one router per leading index), the
+  B*T tokens forming groups of `group_size`.  Returns Routing over
+  [G = B*T/group_size, group_size] (and the logits if want_logits)."""
+  lib = load_library()
+  if policy not in POLICIES:
+    raise ValueError("Unknown policy %s" % policy)
+  b, t, m = x.shape
+  e = w_packed.shape[1]
+  s = int(group_size)
+  if (b * t) % s or t % s:
+    raise MoeHipError("tokens per router (%d) must be whole groups of %d"
+                      % (t, s))
+  g = b * t // s
+  dev = x.device
+  xp = _dev(x, "x", torch.bfloat16)
+  wp = _dev(w_packed, "w_packed", torch.bfloat16, (b, e, m))
+  bp = None if bias is None else _dev(bias, "bias", torch.float32, (e,))
+  ip, icode = None, F32
+  if importance is not None:
+    icode = dtype_code(importance.dtype)
+    ip = _dev(importance, "importance", None, (g, s))
+  up = None
+  if second_uniform is not None:
+    up = _dev(second_uniform, "second_uniform", torch.float32, (g, s))
+  logits = None
+  if want_logits:
+    logits = torch.empty((g, s, e), dtype=torch.float32, device=dev)
+  idx = torch.empty((g, s, 2), dtype=torch.int32, device=dev)
+  pos = torch.empty((g, s, 2), dtype=torch.int32, device=dev)
+  gate = torch.empty((g, s, 2), dtype=torch.float32, device=dev)
+  kept = torch.empty((g, s, 2), dtype=torch.uint8, device=dev)
+  fill = torch.empty((g, e), dtype=torch.int32, device=dev)
+  loss = torch.empty((1,), dtype=torch.float32, device=dev)
+  ws_bytes = lib.mesh_moe_gating_workspace_bytes(g, s, e)
+  ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
+  with _stage("router_top2_gating"):
+    _check(lib.mesh_moe_router_top2_gating(
+        xp, wp, bp, None if logits is None else logits.data_ptr(), b, t, m,
+        BF16, ip, icode, int(bool(importance_from_slot_gate)), up, g, s, e,
+        int(capacity), POLICIES[policy], float(threshold),
+        int(bool(use_second_place_loss)), int(num_microbatches or 1),
+        idx.data_ptr(), pos.data_ptr(), gate.data_ptr(), kept.data_ptr(),
+        fill.data_ptr(), loss.data_ptr(), ws.data_ptr(), ws_bytes, _stream()),
+        "router_top2_gating")
+  r = Routing(idx, pos, gate, kept, fill, loss, int(capacity), e)
+  if _timer is not None:
+    _timer.routing.append(r)
+  return (r, logits) if want_logits else r
 
 
 def dispatch(x, r, want_slot_gate=False, out=None):

@@ -117,6 +117,29 @@ class _GatingSpec(object):
     self.use_second_place_loss = bool(hparams.moe_use_second_place_loss)
     self.num_microbatches = num_microbatches
 
+  def route(self, x, w, w_packed, group_size, num_experts, capacity,
+            importance=None, importance_from_slot_gate=False):
+    """Router projection + gating of x [B, T, M] with routers w [B, M, E]
+    (w_packed [B, E, M]); the B*T tokens form groups of group_size.  One fused
+    launch sequence where the library has a kernel for the case, otherwise the
+    projection and the gating as two calls."""
+    b, t, _ = x.shape
+    groups = b * t // group_size
+    if moe_hip.fused_gating_supported(x, num_experts, group_size):
+      uniform = None
+      if self.policy == "random":
+        uniform = torch.rand((groups, group_size), dtype=torch.float32,
+                             device=x.device)
+      return moe_hip.router_top2_gating(
+          x, w_packed, group_size, capacity, importance=importance,
+          policy=self.policy, threshold=self.threshold,
+          use_second_place_loss=self.use_second_place_loss,
+          num_microbatches=self.num_microbatches, second_uniform=uniform,
+          importance_from_slot_gate=importance_from_slot_gate)
+    logits = moe_hip.router_logits(x, w, w_packed=w_packed)
+    return self.run(logits.reshape(groups, group_size, num_experts), capacity,
+                    importance, importance_from_slot_gate)
+
   def run(self, logits, capacity, importance=None,
           importance_from_slot_gate=False):
     uniform = None
@@ -161,7 +184,7 @@ class MoEV1Operation(mtf.Operation):
     dt = x.dtype
     wi_p = _packed(lowering, wi, dt)
     wo_p = _packed(lowering, wo, dt)
-    wg_p = _packed(lowering, w_gate, dt)[0]            # [E, M]
+    wg_p = _packed(lowering, w_gate, dt)               # [1, E, M]
     o_, g_, s_, m_ = x.shape.to_integer_list
     n_ = self.outputs[0].shape.dims[-1].size
     e_, c_ = self._num_experts, self._capacity
@@ -169,11 +192,10 @@ class MoEV1Operation(mtf.Operation):
 
     def fn(x_s, wg_s, imp_s=None):
       xg = x_s.reshape(groups, s_, m_)
-      logits = moe_hip.router_logits(xg.reshape(groups * s_, m_), wg_s,
-                                     w_packed=wg_p)
       if imp_s is not None:
         imp_s = imp_s.reshape(groups, s_)
-      r = self._gating.run(logits.reshape(groups, s_, e_), c_, imp_s)
+      r = self._gating.route(xg.reshape(1, groups * s_, m_),
+                             wg_s.reshape(1, m_, e_), wg_p, s_, e_, c_, imp_s)
       expert_in = moe_hip.dispatch(xg, r)
       y = moe_hip.expert_ffn(expert_in.reshape(e_, groups * c_, m_), wi_p,
                              wo_p, self._activation)
@@ -308,7 +330,7 @@ class MoEV2Operation(mtf.Operation):
     dt = x.dtype
     wi_p = _packed(lowering, wi, dt)      # [y*x, hidden, m]
     wo_p = _packed(lowering, wo, dt)      # [y*x, n, hidden]
-    w_outer_p = _packed(lowering, w_outer, dt)[0]      # [x, m]
+    w_outer_p = _packed(lowering, w_outer, dt)         # [1, x, m]
     w_inner_p = _packed(lowering, w_inner, dt)         # [x, y, m]
     a0, g1, s_, m_ = x.shape.to_integer_list
     n_ = self.outputs[0].shape.dims[-1].size
@@ -318,19 +340,17 @@ class MoEV2Operation(mtf.Operation):
     def fn(x_s, wo_s, wi_s, imp_s=None):
       xg = x_s.reshape(ag, s_, m_)
       # outer level
-      logits_x = moe_hip.router_logits(xg.reshape(ag * s_, m_), wo_s,
-                                       w_packed=w_outer_p)
       if imp_s is not None:
         imp_s = imp_s.reshape(ag, s_)
-      rx = self._gating.run(logits_x.reshape(ag, s_, x_e), c_, imp_s)
+      rx = self._gating.route(xg.reshape(1, ag * s_, m_),
+                              wo_s.reshape(1, m_, x_e), w_outer_p, s_, x_e, c_,
+                              imp_s)
       ein_x, slot_gate = moe_hip.dispatch(xg, rx, want_slot_gate=True)
       # inner level: each outer expert's a0*g*c slots become h0 groups of t
       inputs_y = ein_x.reshape(x_e, h0 * t_, m_)
-      logits_y = moe_hip.router_logits(inputs_y, wi_s,
-                                       w_packed=w_inner_p)  # [x, h0*t, y]
-      ry = self._gating.run(logits_y.reshape(x_e * h0, t_, y_e), d_,
-                            slot_gate.reshape(x_e * h0, t_),
-                            importance_from_slot_gate=True)
+      ry = self._gating.route(inputs_y, wi_s, w_inner_p, t_, y_e, d_,
+                              slot_gate.reshape(x_e * h0, t_),
+                              importance_from_slot_gate=True)
       ein_y = moe_hip.dispatch(inputs_y.reshape(x_e * h0, t_, m_), ry)
       # experts: weights are [y, x, ...]; rows of (y, x) are its h0*d slots
       yy = moe_hip.expert_ffn(ein_y.reshape(y_e * x_e, h0 * d_, m_), wi_p,

@@ -315,3 +315,47 @@ def test_full_size_routing_properties(hip, size):
   out = hip.combine(ein, r, s)
   want = (w[..., 0:1] * x.float() + w[..., 1:2] * x.float()).to(torch.bfloat16)
   assert torch.equal(out, want)
+
+
+@pytest.mark.parametrize("case", [
+    # routers, groups per router, S, M, E, C
+    (1, 2, 256, 128, 8, 70), (1, 3, 128, 64, 64, 5), (2, 2, 384, 192, 20, 40),
+    (4, 1, 128, 64, 128, 3), (1, 16, 1024, 1024, 32, 40)])
+def test_router_top2_gating_fused(hip, case):
+  """The fused router + gating entry point against the oracle (and against the
+  two-call path): bf16 tokens whose router logits do not nearly tie."""
+  b, gpr, s, m, e, c = case
+  rng = np.random.default_rng(41)
+  w = O.round_bf16((rng.standard_normal((b, m, e)) / np.sqrt(m)).astype(np.float32))
+  x = np.stack([H.safe_tokens(rng, gpr * s, m, w[i], "bfloat16") for i in range(b)])
+  imp = rng.choice(np.array([0.0, 0.5, 1.0], np.float32), size=(b * gpr, s),
+                   p=[0.1, 0.2, 0.7])
+  logits = np.matmul(x, w).astype(np.float32).reshape(b * gpr, s, e)
+  xg, wg = H.to_gpu(x, "bfloat16"), H.to_gpu(w, "bfloat16")
+  wp = hip.pack_weights(wg, wg.dtype)
+  assert hip.fused_gating_supported(xg, e, s)
+  for importance in (None, imp):
+    want = O.top_2_gating(logits, c, importance=importance,
+                          use_second_place_loss=True, num_microbatches=2)
+    r, got_logits = hip.router_top2_gating(
+        xg, wp, s, c, importance=None if importance is None else H.to_gpu(importance),
+        use_second_place_loss=True, num_microbatches=2, want_logits=True)
+    np.testing.assert_allclose(H.to_np(got_logits), logits, rtol=1e-5, atol=2e-5)
+    got = H.routing_to_np(r)
+    H.assert_routing_equal(got, want, gate_rtol=2e-5)
+    np.testing.assert_allclose(got["loss"], want["loss"], rtol=5e-5)
+    # same record as the two separate calls fed the fused kernel's logits
+    r2 = hip.top2_gating(got_logits, c,
+                         importance=None if importance is None else H.to_gpu(importance),
+                         use_second_place_loss=True, num_microbatches=2)
+    for a_, b_ in ((r.idx, r2.idx), (r.pos, r2.pos), (r.kept, r2.kept),
+                   (r.fill, r2.fill), (r.gate, r2.gate)):
+      assert torch.equal(a_, b_)
+
+
+def test_router_top2_gating_rejects_unsupported(hip):
+  x = torch.zeros((1, 96, 64), dtype=torch.bfloat16, device="cuda")
+  wp = torch.zeros((1, 8, 64), dtype=torch.bfloat16, device="cuda")
+  assert not hip.fused_gating_supported(x, 8, 96)
+  with pytest.raises(hip.MoeHipError, match="fused kernel needs"):
+    hip.router_top2_gating(x, wp, 96, 4)
