@@ -230,13 +230,13 @@ __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
-template <int BM, int BN, int WN>  // WN = wavefronts along N (2 x WN in all)
+template <int BM, int BN, int WN, int WM = 2>  // WM x WN wavefronts
 struct DmaCfg {
   static constexpr int BK = 64;
   static constexpr int NS = 2;                         // LDS slots
-  static constexpr int WAVES = 2 * WN;
+  static constexpr int WAVES = WM * WN;
   static constexpr int THREADS = 64 * WAVES;
-  static constexpr int WTM = BM / 2, WTN = BN / WN;
+  static constexpr int WTM = BM / WM, WTN = BN / WN;
   static constexpr int TM = WTM / 32, TN = WTN / 32;
   static constexpr int ROW_BYTES = BK * 2;             // 128
   static constexpr int A_INSTR = (BM / 8) / WAVES;     // per wavefront
@@ -254,11 +254,11 @@ __device__ __forceinline__ int lds_swizzle(int row) {
   return (row & 7) ^ ((row >> 3) & 1);
 }
 
-template <int BM, int BN, int WN, bool RELU>
-__global__ __launch_bounds__(128 * WN) void grouped_gemm_bf16_dma_kernel(
+template <int BM, int BN, int WN, bool RELU, int WM = 2>
+__global__ __launch_bounds__(64 * WM * WN) void grouped_gemm_bf16_dma_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
     bf16_t* __restrict__ Cout, int R, int N, int K, int tiles_m, int tiles_n) {
-  using Cfg = DmaCfg<BM, BN, WN>;
+  using Cfg = DmaCfg<BM, BN, WN, WM>;
   constexpr int BK = Cfg::BK;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
 
@@ -551,21 +551,21 @@ static int launch_mfma(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
   return 0;
 }
 
-template <int BM, int BN, int WN>
+template <int BM, int BN, int WN, int WM = 2>
 static int launch_dma(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
                       int R, int N, int K, bool relu, hipStream_t st) {
-  using Cfg = DmaCfg<BM, BN, WN>;
+  using Cfg = DmaCfg<BM, BN, WN, WM>;
   const int tiles_m = (R + BM - 1) / BM, tiles_n = (N + BN - 1) / BN;
   const int64_t blocks = (int64_t)tiles_m * tiles_n * E;
   MOE_REQUIRE(blocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
               "expert_ffn: too many tiles (%lld)", (long long)blocks);
   if (relu) {
-    auto k = grouped_gemm_bf16_dma_kernel<BM, BN, WN, true>;
+    auto k = grouped_gemm_bf16_dma_kernel<BM, BN, WN, true, WM>;
     MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
     k<<<(unsigned)blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(A, B, C, R, N, K, tiles_m,
                                                       tiles_n);
   } else {
-    auto k = grouped_gemm_bf16_dma_kernel<BM, BN, WN, false>;
+    auto k = grouped_gemm_bf16_dma_kernel<BM, BN, WN, false, WM>;
     MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
     k<<<(unsigned)blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(A, B, C, R, N, K, tiles_m,
                                                       tiles_n);
