@@ -416,6 +416,9 @@ __global__ __launch_bounds__(64 * WM * WN) void grouped_gemm_bf16_dma_kernel(
   };
   for (int kt = 0; kt + 1 < nk; ++kt) k_tile(kt, std::false_type{});
   k_tile(nk - 1, std::true_type{});
+  // the epilogue reuses the ring: no direct-to-LDS load may still be in flight
+  // (the last hand-over re-fetches a tile nobody reads)
+  wait_vmcnt<0>();
   __syncthreads();
 
   // epilogue: round (and relu), stage the tile in LDS, coalesced stores
