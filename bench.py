@@ -57,7 +57,9 @@ CONFIGS = {
 
 def hparams_dict(cfg):
   return dict(
-      moe_gating="top_2", moe_num_experts=cfg["E"], moe_loss_coef=1e-2,
+      moe_gating=cfg.get("gating", "top_2"), moe_switch_policy_train="argmax",
+      moe_switch_policy_eval="argmax", moe_z_loss=None,
+      moe_num_experts=cfg["E"], moe_loss_coef=1e-2,
       moe_hidden_size=cfg["H"], moe_group_size=cfg["group"],
       moe_min_expert_capacity=4, moe_capacity_factor_train=cfg["cf"],
       moe_capacity_factor_eval=cfg["cf"],
@@ -112,7 +114,9 @@ def build(cfg, device):
       # reference router has no bias term: feature 0 of every token is set to 1
       # and row 0 of the router kernel carries the bias.
       x_val[..., 0] = 1.0
-    init["moe/top_2_gating/kernel"] = normal_init(m, 2)
+    router = "moe/%s/kernel" % ("switch_gating" if cfg.get("gating") == "switch"
+                                else "top_2_gating")
+    init[router] = normal_init(m, 2)
     init["moe/wi/kernel"] = normal_init(m, 3)
     init["moe/wo/kernel"] = normal_init(h, 4)
   else:
@@ -127,14 +131,14 @@ def build(cfg, device):
     else:
       y, loss = moe.transformer_moe_layer_v2(x, dims[-1], hp, True, vdt)
   if cfg.get("skew"):
-    base = init["moe/top_2_gating/kernel"]
+    base = init[router]
 
     def skewed(sizes, dtype, dev):
       w = base(sizes, dtype, dev)
       perm = torch.randperm(sizes[1], generator=gen, device=dev) + 1
       w[0] = (3.0 * perm.double() ** -1.2).to(dtype)
       return w
-    init["moe/top_2_gating/kernel"] = skewed
+    init[router] = skewed
   lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl(device=device)},
                           initial_values=init)
   return lowering, x, y, loss
@@ -152,6 +156,8 @@ def stage_model(cfg, kept_pairs, slots):
       "top2_gating": dict(bytes=t * (4 * e + 26)),
       # fused projection + gating: the logits never reach HBM
       "router_top2_gating": dict(bytes=t * m * b + m * e * b + 26 * t),
+      "switch_gating": dict(bytes=t * (4 * e + 26)),
+      "router_switch_gating": dict(bytes=t * m * b + m * e * b + 26 * t),
       "dispatch": dict(bytes=t * m * b + r * m * b + 18 * t),
       "combine": dict(bytes=r * m * b + t * m * b + 26 * t),
       "expert_ffn": dict(flops=4 * r * m * h, padded_flops=4 * slots * m * h),
@@ -210,6 +216,9 @@ def main():
   ap.add_argument("--steps", type=int, default=10)
   ap.add_argument("--warmup", type=int, default=3)
   ap.add_argument("--config", type=int, default=4, choices=sorted(CONFIGS))
+  ap.add_argument("--gating", default="top_2", choices=["top_2", "switch"],
+                  help="router of the v1 configs (the benchmark definition "
+                       "uses top_2)")
   ap.add_argument("--no-cpu-baseline", action="store_true")
   args = ap.parse_args()
   if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -220,7 +229,13 @@ def main():
 
   import torch
   from mesh_amd import moe_hip
-  cfg = CONFIGS[args.config]
+  cfg = dict(CONFIGS[args.config])
+  if args.gating != "top_2":
+    if cfg["layer"] != "v1":
+      print("--gating applies to the v1 configs only", file=sys.stderr)
+      sys.exit(2)
+    cfg["gating"] = args.gating
+    cfg["name"] += ", %s gating" % args.gating
   device = torch.device("cuda:0")
   torch.cuda.set_device(device)
   lowering, x, y, loss = build(cfg, device)   # first execution
@@ -272,7 +287,8 @@ def main():
         "kernel": "grouped expert GEMM (expert_ffn, 2 launches/step)",
         "bound": "mfma", "achieved": achieved, "peak": peak,
         "unit": "TFLOP/s", "frac": achieved / peak,
-        "traffic": MEASURED_GEMM_TRAFFIC_BYTES.get(args.config),
+        "traffic": (MEASURED_GEMM_TRAFFIC_BYTES.get(args.config)
+                    if args.gating == "top_2" else None),
         "flops_per_launch": flops_per_launch,
         "avg_launch_ms": ffn_ms / 2,
         "padded_frac": (model["expert_ffn"]["padded_flops"] / 2

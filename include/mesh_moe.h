@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 1
+#define MESH_MOE_ABI_VERSION 2
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -131,6 +131,46 @@ int mesh_moe_router_top2_gating(
     double threshold, int use_second_place_loss, int num_microbatches,
     int32_t* idx, int32_t* pos, float* gate, uint8_t* kept, int32_t* fill,
     float* loss, void* workspace, size_t workspace_bytes, void* stream);
+
+/*
+ * Switch (top-1) gating from router logits: softmax, arg-max expert, raw
+ * probability as the gate, per-group capacity positions with overflow drop,
+ * load-balancing loss and (optionally) the router z-loss.
+ * Replaces _switch_gating after the router projection for its deterministic
+ * policies -- "argmax", and "input_dropout" / "input_jitter" outside training
+ * (transformer/moe.py:1207-1306; z-loss :1253-1266).
+ * The per-token record has the layout of mesh_moe_top2_gating with the second
+ * choice never kept (kept[..,1] = 0, gate[..,1] = 0), so mesh_moe_dispatch and
+ * mesh_moe_combine apply unchanged.
+ *   importance [G,S] of importance_dtype or NULL: only tokens with
+ *               importance == 1 are routed (moe.py:1226-1231)
+ *   use_z_loss != 0 adds z_loss_coef * sum_t(logsumexp_t^2 * (imp_t == 1)) /
+ *               (#(imp == 1) * num_microbatches); the caller passes it only
+ *               when training with hparams.moe_z_loss set
+ *   loss [1]  float32, before moe_loss_coef
+ * Limits as mesh_moe_top2_gating; workspace from
+ * mesh_moe_gating_workspace_bytes.
+ */
+int mesh_moe_switch_gating(const float* logits, const void* importance,
+                           int importance_dtype, int G, int S, int E, int C,
+                           int use_z_loss, double z_loss_coef,
+                           int num_microbatches, int32_t* idx, int32_t* pos,
+                           float* gate, uint8_t* kept, int32_t* fill,
+                           float* loss, void* workspace,
+                           size_t workspace_bytes, void* stream);
+
+/*
+ * Router projection + switch gating in one call (transformer/moe.py:1200-1306);
+ * the switch counterpart of mesh_moe_router_top2_gating, same shape limits and
+ * the same MESH_MOE_E_UNSUPPORTED convention.
+ */
+int mesh_moe_router_switch_gating(
+    const void* x, const void* w_packed, const float* bias, float* logits,
+    int batch, int64_t tokens, int M, int dtype, const void* importance,
+    int importance_dtype, int G, int S, int E, int C, int use_z_loss,
+    double z_loss_coef, int num_microbatches, int32_t* idx, int32_t* pos,
+    float* gate, uint8_t* kept, int32_t* fill, float* loss, void* workspace,
+    size_t workspace_bytes, void* stream);
 
 /*
  * Dispatch: expert_in[e,g,c,:] = x[g,s,:] for the token holding slot (e,g,c),

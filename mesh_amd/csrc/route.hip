@@ -215,7 +215,15 @@ struct GateParams {
   int importance_from_slot_gate;  // importance = 0.5*((w>0.5)+(w>0))
   int tt;    // tokens per block of step 1
   int nblk;  // blocks per group of step 1
+  int router;          // ROUTER_TOP2 or ROUTER_SWITCH
+  int has_importance;  // switch loss: the proxy is masked per token
+  int use_z_loss;      // switch: add z_loss_coef * z_loss (moe.py:1253-1266)
+  float z_loss_coef;
 };
+
+constexpr int ROUTER_TOP2 = 0;    // _top_2_gating, moe.py:1312-1513
+constexpr int ROUTER_SWITCH = 1;  // _switch_gating, moe.py:1176-1309
+constexpr int GSUM = 4;  // floats per group: loss term 1, term 2, #(imp==1), z
 
 // bit 0 of the step-1 `kept` byte: the token competes for a slot (mask_k after
 // importance and policy); bit 1 (second choice only): mask_2 before the policy,
@@ -233,7 +241,7 @@ __device__ __forceinline__ void gate_select_tile(
     float* __restrict__ part1, float* __restrict__ part2) {
   const int E = p.E, S = p.S;
   const int tid = threadIdx.x;
-  float qscale = 0.f;
+  float qscale = 0.f, zterm = 0.f;
   int i1 = 0;
   bool sel1 = false;
   if (tid < ntok) {
@@ -252,6 +260,25 @@ __device__ __forceinline__ void gate_select_tile(
       if (pe > g1) { g1 = pe; i1 = e; }                     // first argmax
     }
     sel1 = true;
+    if (p.router == ROUTER_SWITCH) {
+      // one choice, raw probability as the gate (moe.py:1207-1228); the load
+      // balancing loss counts every token's arg-max (density_1 is taken
+      // before the importance mask, moe.py:1224) and an unmasked proxy
+      if (importance != nullptr)
+        sel1 = (load_f32<IT>(importance + t) == 1.0f);
+      if (!sel1) g1 = g1 * 0.0f;
+      idx[t * 2 + 0] = i1;
+      idx[t * 2 + 1] = 0;
+      pos[t * 2 + 0] = 0;
+      pos[t * 2 + 1] = 0;
+      gate[t * 2 + 0] = g1;
+      gate[t * 2 + 1] = 0.0f;
+      kept[t * 2 + 0] = (sel1 ? 1 : 0) | 2;   // bit 1: counted by density_1
+      kept[t * 2 + 1] = 0;
+      isone[tid] = 1.0f;
+      const float lse = -neglse;                            // reduce_logsumexp
+      zterm = sel1 ? lse * lse : 0.0f;                      // moe.py:1256-1259
+    } else {
     bool sel2 = true;
     if (importance != nullptr) {
       float imp = load_f32<IT>(importance + t);
@@ -291,6 +318,7 @@ __device__ __forceinline__ void gate_select_tile(
     kept[t * 2 + 1] = (sel2 ? 1 : 0) | (sel2_loss ? 2 : 0);
     isone[tid] = sel1 ? 1.0f : 0.0f;
     qscale = 1.0f / (qsum + 1e-9f);                         // moe.py:1433-1434
+    }
   }
   __syncthreads();
   // density_1_proxy partial: sum over the block's tokens of p * (imp == 1)
@@ -299,7 +327,21 @@ __device__ __forceinline__ void gate_select_tile(
     for (int r = 0; r < ntok; ++r) s += tile[r * ld + e] * isone[r];
     part1[((int64_t)g * p.nblk + blk) * E + e] = s;
   }
-  if (p.use_second_place_loss) {
+  if (p.router == ROUTER_SWITCH) {
+    // per-block sums for the z-loss: column 0 = sum of logsumexp^2 over the
+    // tokens with importance 1, column 1 = how many those are
+    __syncthreads();
+    if (tid < ntok) {
+      tile[tid * ld + 0] = zterm;
+      tile[tid * ld + 1] = sel1 ? 1.0f : 0.0f;
+    }
+    __syncthreads();
+    if (tid < 2) {
+      float s = 0.f;
+      for (int r = 0; r < ntok; ++r) s += tile[r * ld + tid];
+      part2[((int64_t)g * p.nblk + blk) * E + tid] = s;
+    }
+  } else if (p.use_second_place_loss) {
     __syncthreads();
     if (tid < ntok) {
       float* row = tile + tid * ld;
@@ -488,14 +530,18 @@ __global__ __launch_bounds__(CAP_THREADS) void gate_capacity_kernel(
   const int g = blockIdx.x;
   const int tid = threadIdx.x;
   const int64_t base = (int64_t)g * S;
-  const bool loss2 = p.use_second_place_loss != 0;
+  const bool sw = p.router == ROUTER_SWITCH;
+  // a third count per expert: the second-place loss's mask_2 before the
+  // policy (top-2), or every token's arg-max for density_1 (switch)
+  const bool loss2 = p.use_second_place_loss != 0 || sw;
   for (int s = tid; s < S; s += CAP_THREADS) {
     int64_t t = base + s;
     int a = idx[t * 2], b = idx[t * 2 + 1];
     uint8_t k1 = kept[t * 2], k2 = kept[t * 2 + 1];
     c1[s] = (k1 & 1) ? (int16_t)a : (int16_t)-1;
     c2[s] = (k2 & 1) ? (int16_t)b : (int16_t)-1;
-    if (loss2) c2l[s] = (k2 & 2) ? (int16_t)b : (int16_t)-1;
+    if (sw) c2l[s] = (k1 & 2) ? (int16_t)a : (int16_t)-1;
+    else if (loss2) c2l[s] = (k2 & 2) ? (int16_t)b : (int16_t)-1;
   }
   __syncthreads();
   const int e = tid % el;
@@ -563,8 +609,11 @@ __global__ __launch_bounds__(CAP_THREADS) void gate_capacity_kernel(
     float proxy = 0.f;
     for (int b = 0; b < p.nblk; ++b)
       proxy += part1[((int64_t)g * p.nblk + b) * E + tid];
-    prod[tid] = (proxy * inv_s) * ((float)t1 * inv_s);       // moe.py:1420-1423
-    if (loss2) {
+    // density_1: competing first choices (top-2, moe.py:1420-1423) or every
+    // token's arg-max (switch, moe.py:1224-1225)
+    const int dens = sw ? tot[2 * el + tid] : t1;
+    prod[tid] = (proxy * inv_s) * ((float)dens * inv_s);
+    if (loss2 && !sw) {
       float proxy2 = 0.f;
       for (int b = 0; b < p.nblk; ++b)
         proxy2 += part2[((int64_t)g * p.nblk + b) * E + tid];
@@ -573,12 +622,20 @@ __global__ __launch_bounds__(CAP_THREADS) void gate_capacity_kernel(
   }
   __syncthreads();
   if (tid == 0) {
-    float s1 = 0.f, s2 = 0.f;
+    float s1 = 0.f, s2 = 0.f, n_one = 0.f, z = 0.f;
     for (int k = 0; k < E; ++k) s1 += prod[k];
-    if (loss2)
+    if (loss2 && !sw)
       for (int k = 0; k < E; ++k) s2 += prod[el + k];
-    gsum[g * 2] = s1;
-    gsum[g * 2 + 1] = s2;
+    if (sw) {
+      for (int b = 0; b < p.nblk; ++b) {
+        z += part2[((int64_t)g * p.nblk + b) * E + 0];
+        n_one += part2[((int64_t)g * p.nblk + b) * E + 1];
+      }
+    }
+    gsum[g * GSUM] = s1;
+    gsum[g * GSUM + 1] = s2;
+    gsum[g * GSUM + 2] = n_one;
+    gsum[g * GSUM + 3] = z;
   }
 }
 
@@ -586,10 +643,38 @@ __global__ void gate_loss_kernel(GateParams p, const float* __restrict__ gsum,
                                  float* __restrict__ loss) {
   if (threadIdx.x != 0 || blockIdx.x != 0) return;
   float s1 = 0.f, s2 = 0.f;
-  for (int g = 0; g < p.G; ++g) { s1 += gsum[g * 2]; s2 += gsum[g * 2 + 1]; }
+  for (int g = 0; g < p.G; ++g) {
+    s1 += gsum[g * GSUM];
+    s2 += gsum[g * GSUM + 1];
+  }
   const float inv_ge = (float)(1.0 / ((double)p.G * (double)p.E));
   const float ee = (float)((double)p.E * (double)p.E);
-  float l = (s1 * inv_ge) * ee;                              // moe.py:1423-1424
+  float l;
+  if (p.router == ROUTER_SWITCH) {
+    if (p.has_importance) {
+      // mean over [G,E,S] of proxy[g,e] * (imp[g,s] == 1) * density[g,e]
+      // (moe.py:1229-1234): each group's term counts once per such token
+      float sm = 0.f;
+      for (int g = 0; g < p.G; ++g) sm += gsum[g * GSUM] * gsum[g * GSUM + 2];
+      l = (sm * (float)(1.0 / ((double)p.G * (double)p.E * (double)p.S))) * ee;
+    } else {
+      l = (s1 * inv_ge) * ee;
+    }
+    if (p.num_microbatches > 1)
+      l = l * (float)(1.0 / (double)p.num_microbatches);     // moe.py:1235-1238
+    if (p.use_z_loss) {                                      // moe.py:1253-1266
+      float z = 0.f, n = 0.f;
+      for (int g = 0; g < p.G; ++g) {
+        z += gsum[g * GSUM + 3];
+        n += gsum[g * GSUM + 2];
+      }
+      const float mb = (float)(p.num_microbatches > 0 ? p.num_microbatches : 1);
+      l = l + p.z_loss_coef * (z / (n * mb));
+    }
+    loss[0] = l;
+    return;
+  }
+  l = (s1 * inv_ge) * ee;                                    // moe.py:1423-1424
   if (p.use_second_place_loss) l = l + ((s2 * inv_ge) * ee) * 0.5f;
   if (p.num_microbatches > 1)
     l = l * (float)(1.0 / (double)p.num_microbatches);       // moe.py:1439-1442
@@ -722,6 +807,23 @@ static GateParams make_gate_params(int G, int S, int E, int C, int policy,
   p.importance_from_slot_gate = importance_from_slot_gate ? 1 : 0;
   p.tt = tt;
   p.nblk = (S + tt - 1) / tt;
+  p.router = ROUTER_TOP2;
+  p.has_importance = 0;
+  p.use_z_loss = 0;
+  p.z_loss_coef = 0.f;
+  return p;
+}
+
+static GateParams make_switch_params(int G, int S, int E, int C,
+                                     const void* importance, int use_z_loss,
+                                     double z_loss_coef, int num_microbatches,
+                                     int tt) {
+  GateParams p = make_gate_params(G, S, E, C, MESH_MOE_SECOND_NONE, 0.0, 0,
+                                  num_microbatches, 0, tt);
+  p.router = ROUTER_SWITCH;
+  p.has_importance = importance != nullptr;
+  p.use_z_loss = use_z_loss ? 1 : 0;
+  p.z_loss_coef = (float)z_loss_coef;
   return p;
 }
 
@@ -748,82 +850,70 @@ static int launch_router_gate(const bf16_t* x, const bf16_t* wp,
 extern "C" size_t mesh_moe_gating_workspace_bytes(int G, int S, int E) {
   if (G < 1 || S < 1 || E < 1) return 0;
   const size_t nblk = (size_t)(S + 63) / 64;  // smallest token block of any path
-  return sizeof(float) * (2 * (size_t)G * nblk * E + 2 * (size_t)G) + 256;
+  return sizeof(float) * (2 * (size_t)G * nblk * E + GSUM * (size_t)G) + 256;
 }
 
-extern "C" int mesh_moe_top2_gating(
-    const float* logits, const void* importance, int importance_dtype,
-    int importance_from_slot_gate, const float* second_uniform, int G, int S,
-    int E, int C, int policy,
-    double threshold, int use_second_place_loss, int num_microbatches,
-    int32_t* idx, int32_t* pos, float* gate, uint8_t* kept, int32_t* fill,
-    float* loss, void* workspace, size_t workspace_bytes, void* stream) {
-  MOE_REQUIRE(logits && idx && pos && gate && kept && fill && loss && workspace,
-              MESH_MOE_E_ARG, "top2_gating: null pointer");
-  if (int rc = check_gating_args(G, S, E, C, policy, second_uniform, importance,
-                                 importance_dtype, workspace_bytes))
-    return rc;
-  GateParams p = make_gate_params(G, S, E, C, policy, threshold,
-                                  use_second_place_loss, num_microbatches,
-                                  importance_from_slot_gate,
-                                  gate_tokens_per_block(E));
-  hipStream_t st = (hipStream_t)stream;
+// Gating from logits: step 1 (softmax / choices) then steps 2 and 3.
+static int run_gating(const GateParams& p, const float* logits,
+                      const void* importance, int importance_dtype,
+                      const float* second_uniform, int32_t* idx, int32_t* pos,
+                      float* gate, uint8_t* kept, int32_t* fill, float* loss,
+                      void* workspace, hipStream_t st) {
+  const int G = p.G, E = p.E;
   uintptr_t wsp = ((uintptr_t)workspace + 255) & ~(uintptr_t)255;
   float* part1 = (float*)wsp;
   float* part2 = part1 + (size_t)G * p.nblk * E;
   float* gsum = part2 + (size_t)G * p.nblk * E;
-
-  {
-    dim3 grid((unsigned)p.nblk, (unsigned)G);
-    size_t smem = sizeof(float) * ((size_t)p.tt * (E + 1) + p.tt);
-    if (importance && importance_dtype == MESH_MOE_BF16) {
-      auto k = gate_select_kernel<bf16_t>;
-      MOE_ALLOW_LDS(k, smem);
-      k<<<grid, p.tt, smem, st>>>(logits, (const bf16_t*)importance,
-                                  second_uniform, p, idx, pos, gate, kept,
-                                  part1, part2);
-    } else {
-      auto k = gate_select_kernel<float>;
-      MOE_ALLOW_LDS(k, smem);
-      k<<<grid, p.tt, smem, st>>>(logits, (const float*)importance,
-                                  second_uniform, p, idx, pos, gate, kept,
-                                  part1, part2);
-    }
-    MOE_CHECK_LAUNCH("gate_select");
+  dim3 grid((unsigned)p.nblk, (unsigned)G);
+  size_t smem = sizeof(float) * ((size_t)p.tt * (E + 1) + p.tt);
+  if (importance && importance_dtype == MESH_MOE_BF16) {
+    auto k = gate_select_kernel<bf16_t>;
+    MOE_ALLOW_LDS(k, smem);
+    k<<<grid, p.tt, smem, st>>>(logits, (const bf16_t*)importance,
+                                second_uniform, p, idx, pos, gate, kept, part1,
+                                part2);
+  } else {
+    auto k = gate_select_kernel<float>;
+    MOE_ALLOW_LDS(k, smem);
+    k<<<grid, p.tt, smem, st>>>(logits, (const float*)importance,
+                                second_uniform, p, idx, pos, gate, kept, part1,
+                                part2);
   }
+  MOE_CHECK_LAUNCH("gate_select");
   return launch_capacity_and_loss(p, idx, pos, gate, kept, fill, loss, part1,
                                   part2, gsum, st);
 }
 
-extern "C" int mesh_moe_router_top2_gating(
-    const void* x, const void* w_packed, const float* bias, float* logits,
-    int batch, int64_t tokens, int M, int dtype, const void* importance,
-    int importance_dtype, int importance_from_slot_gate,
-    const float* second_uniform, int G, int S, int E, int C, int policy,
-    double threshold, int use_second_place_loss, int num_microbatches,
-    int32_t* idx, int32_t* pos, float* gate, uint8_t* kept, int32_t* fill,
-    float* loss, void* workspace, size_t workspace_bytes, void* stream) {
-  MOE_REQUIRE(x && w_packed && idx && pos && gate && kept && fill && loss &&
-                  workspace, MESH_MOE_E_ARG, "router_top2_gating: null pointer");
-  if (int rc = check_gating_args(G, S, E, C, policy, second_uniform, importance,
-                                 importance_dtype, workspace_bytes))
-    return rc;
+// Shape limits of the fused projection + gating kernel.
+static int check_fused_router_args(const char* who, const void* x,
+                                   const void* w_packed, int batch,
+                                   int64_t tokens, int M, int dtype, int G,
+                                   int S, int E) {
   MOE_REQUIRE(batch >= 1 && (int64_t)batch * tokens == (int64_t)G * S,
-              MESH_MOE_E_ARG,
-              "router_top2_gating: batch*tokens=%lld != G*S=%lld",
+              MESH_MOE_E_ARG, "%s: batch*tokens=%lld != G*S=%lld", who,
               (long long)batch * tokens, (long long)G * S);
   MOE_REQUIRE(dtype == MESH_MOE_BF16 && M % 64 == 0 && E % 4 == 0 && E <= 128 &&
                   S % 128 == 0 && tokens % S == 0 &&
                   (int64_t)128 * M < (1LL << 31) &&
                   (((uintptr_t)x | (uintptr_t)w_packed) % 16 == 0),
               MESH_MOE_E_UNSUPPORTED,
-              "router_top2_gating: the fused kernel needs bf16, M %% 64 == 0, "
+              "%s: the fused kernel needs bf16, M %% 64 == 0, "
               "E %% 4 == 0, E <= 128, S %% 128 == 0 (M=%d E=%d S=%d dtype=%d); "
-              "use router_logits + top2_gating", M, E, S, dtype);
-  GateParams p = make_gate_params(G, S, E, C, policy, threshold,
-                                  use_second_place_loss, num_microbatches,
-                                  importance_from_slot_gate, 128);
-  hipStream_t st = (hipStream_t)stream;
+              "use router_logits + the logits-in gating call", who, M, E, S,
+              dtype);
+  return 0;
+}
+
+// Fused projection + gating step 1 (p.tt must be 128), then steps 2 and 3.
+static int run_router_gating(const GateParams& p, const void* x,
+                             const void* w_packed, const float* bias,
+                             float* logits, int64_t tokens, int M,
+                             const void* importance, int importance_dtype,
+                             const float* second_uniform, int32_t* idx,
+                             int32_t* pos, float* gate, uint8_t* kept,
+                             int32_t* fill, float* loss, void* workspace,
+                             hipStream_t st) {
+  const int G = p.G, S = p.S, E = p.E;
   uintptr_t wsp = ((uintptr_t)workspace + 255) & ~(uintptr_t)255;
   float* part1 = (float*)wsp;
   float* part2 = part1 + (size_t)G * p.nblk * E;
@@ -849,4 +939,90 @@ extern "C" int mesh_moe_router_top2_gating(
   if (rc != 0) return rc;
   return launch_capacity_and_loss(p, idx, pos, gate, kept, fill, loss, part1,
                                   part2, gsum, st);
+}
+
+extern "C" int mesh_moe_top2_gating(
+    const float* logits, const void* importance, int importance_dtype,
+    int importance_from_slot_gate, const float* second_uniform, int G, int S,
+    int E, int C, int policy,
+    double threshold, int use_second_place_loss, int num_microbatches,
+    int32_t* idx, int32_t* pos, float* gate, uint8_t* kept, int32_t* fill,
+    float* loss, void* workspace, size_t workspace_bytes, void* stream) {
+  MOE_REQUIRE(logits && idx && pos && gate && kept && fill && loss && workspace,
+              MESH_MOE_E_ARG, "top2_gating: null pointer");
+  if (int rc = check_gating_args(G, S, E, C, policy, second_uniform, importance,
+                                 importance_dtype, workspace_bytes))
+    return rc;
+  GateParams p = make_gate_params(G, S, E, C, policy, threshold,
+                                  use_second_place_loss, num_microbatches,
+                                  importance_from_slot_gate,
+                                  gate_tokens_per_block(E));
+  return run_gating(p, logits, importance, importance_dtype, second_uniform,
+                    idx, pos, gate, kept, fill, loss, workspace,
+                    (hipStream_t)stream);
+}
+
+extern "C" int mesh_moe_router_top2_gating(
+    const void* x, const void* w_packed, const float* bias, float* logits,
+    int batch, int64_t tokens, int M, int dtype, const void* importance,
+    int importance_dtype, int importance_from_slot_gate,
+    const float* second_uniform, int G, int S, int E, int C, int policy,
+    double threshold, int use_second_place_loss, int num_microbatches,
+    int32_t* idx, int32_t* pos, float* gate, uint8_t* kept, int32_t* fill,
+    float* loss, void* workspace, size_t workspace_bytes, void* stream) {
+  MOE_REQUIRE(x && w_packed && idx && pos && gate && kept && fill && loss &&
+                  workspace, MESH_MOE_E_ARG, "router_top2_gating: null pointer");
+  if (int rc = check_gating_args(G, S, E, C, policy, second_uniform, importance,
+                                 importance_dtype, workspace_bytes))
+    return rc;
+  if (int rc = check_fused_router_args("router_top2_gating", x, w_packed, batch,
+                                       tokens, M, dtype, G, S, E))
+    return rc;
+  GateParams p = make_gate_params(G, S, E, C, policy, threshold,
+                                  use_second_place_loss, num_microbatches,
+                                  importance_from_slot_gate, 128);
+  return run_router_gating(p, x, w_packed, bias, logits, tokens, M, importance,
+                           importance_dtype, second_uniform, idx, pos, gate,
+                           kept, fill, loss, workspace, (hipStream_t)stream);
+}
+
+extern "C" int mesh_moe_switch_gating(
+    const float* logits, const void* importance, int importance_dtype, int G,
+    int S, int E, int C, int use_z_loss, double z_loss_coef,
+    int num_microbatches, int32_t* idx, int32_t* pos, float* gate,
+    uint8_t* kept, int32_t* fill, float* loss, void* workspace,
+    size_t workspace_bytes, void* stream) {
+  MOE_REQUIRE(logits && idx && pos && gate && kept && fill && loss && workspace,
+              MESH_MOE_E_ARG, "switch_gating: null pointer");
+  if (int rc = check_gating_args(G, S, E, C, MESH_MOE_SECOND_NONE, nullptr,
+                                 importance, importance_dtype, workspace_bytes))
+    return rc;
+  GateParams p = make_switch_params(G, S, E, C, importance, use_z_loss,
+                                    z_loss_coef, num_microbatches,
+                                    gate_tokens_per_block(E));
+  return run_gating(p, logits, importance, importance_dtype, nullptr, idx, pos,
+                    gate, kept, fill, loss, workspace, (hipStream_t)stream);
+}
+
+extern "C" int mesh_moe_router_switch_gating(
+    const void* x, const void* w_packed, const float* bias, float* logits,
+    int batch, int64_t tokens, int M, int dtype, const void* importance,
+    int importance_dtype, int G, int S, int E, int C, int use_z_loss,
+    double z_loss_coef, int num_microbatches, int32_t* idx, int32_t* pos,
+    float* gate, uint8_t* kept, int32_t* fill, float* loss, void* workspace,
+    size_t workspace_bytes, void* stream) {
+  MOE_REQUIRE(x && w_packed && idx && pos && gate && kept && fill && loss &&
+                  workspace, MESH_MOE_E_ARG,
+              "router_switch_gating: null pointer");
+  if (int rc = check_gating_args(G, S, E, C, MESH_MOE_SECOND_NONE, nullptr,
+                                 importance, importance_dtype, workspace_bytes))
+    return rc;
+  if (int rc = check_fused_router_args("router_switch_gating", x, w_packed,
+                                       batch, tokens, M, dtype, G, S, E))
+    return rc;
+  GateParams p = make_switch_params(G, S, E, C, importance, use_z_loss,
+                                    z_loss_coef, num_microbatches, 128);
+  return run_router_gating(p, x, w_packed, bias, logits, tokens, M, importance,
+                           importance_dtype, nullptr, idx, pos, gate, kept,
+                           fill, loss, workspace, (hipStream_t)stream);
 }

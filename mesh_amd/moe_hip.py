@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -44,6 +44,16 @@ _SIGNATURES = {
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_double, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, _vp, _vp,
         _vp, _vp, ctypes.c_size_t, _vp]),
+    "mesh_moe_switch_gating": (ctypes.c_int, [
+        _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_double, ctypes.c_int, _vp, _vp,
+        _vp, _vp, _vp, _vp, _vp, ctypes.c_size_t, _vp]),
+    "mesh_moe_router_switch_gating": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
+        ctypes.c_int, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_double,
+        ctypes.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_size_t,
+        _vp]),
     "mesh_moe_dispatch": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
@@ -307,6 +317,85 @@ def router_top2_gating(x, w_packed, group_size, capacity, importance=None,
         idx.data_ptr(), pos.data_ptr(), gate.data_ptr(), kept.data_ptr(),
         fill.data_ptr(), loss.data_ptr(), ws.data_ptr(), ws_bytes, _stream()),
         "router_top2_gating")
+  r = Routing(idx, pos, gate, kept, fill, loss, int(capacity), e)
+  if _timer is not None:
+    _timer.routing.append(r)
+  return (r, logits) if want_logits else r
+
+
+def _routing_buffers(lib, g, s, e, dev):
+  idx = torch.empty((g, s, 2), dtype=torch.int32, device=dev)
+  pos = torch.empty((g, s, 2), dtype=torch.int32, device=dev)
+  gate = torch.empty((g, s, 2), dtype=torch.float32, device=dev)
+  kept = torch.empty((g, s, 2), dtype=torch.uint8, device=dev)
+  fill = torch.empty((g, e), dtype=torch.int32, device=dev)
+  loss = torch.empty((1,), dtype=torch.float32, device=dev)
+  ws_bytes = lib.mesh_moe_gating_workspace_bytes(g, s, e)
+  ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
+  return idx, pos, gate, kept, fill, loss, ws, ws_bytes
+
+
+def switch_gating(logits, capacity, importance=None, z_loss=None,
+                  num_microbatches=None):
+  """logits float32 [G, S, E] -> Routing for switch (top-1) gating.
+
+  z_loss: coefficient of the router z-loss, or None to leave it out (the
+  caller passes it only when training, transformer/moe.py:1253)."""
+  lib = load_library()
+  g, s, e = logits.shape
+  lp = _dev(logits, "logits", torch.float32)
+  ip, icode = None, F32
+  if importance is not None:
+    icode = dtype_code(importance.dtype)
+    ip = _dev(importance, "importance", None, (g, s))
+  idx, pos, gate, kept, fill, loss, ws, ws_bytes = _routing_buffers(
+      lib, g, s, e, logits.device)
+  with _stage("switch_gating"):
+    _check(lib.mesh_moe_switch_gating(
+        lp, ip, icode, g, s, e, int(capacity), int(z_loss is not None),
+        float(z_loss or 0.0), int(num_microbatches or 1), idx.data_ptr(),
+        pos.data_ptr(), gate.data_ptr(), kept.data_ptr(), fill.data_ptr(),
+        loss.data_ptr(), ws.data_ptr(), ws_bytes, _stream()), "switch_gating")
+  r = Routing(idx, pos, gate, kept, fill, loss, int(capacity), e)
+  if _timer is not None:
+    _timer.routing.append(r)
+  return r
+
+
+def router_switch_gating(x, w_packed, group_size, capacity, importance=None,
+                         z_loss=None, num_microbatches=None, bias=None,
+                         want_logits=False):
+  """Router projection + switch gating in one launch sequence; arguments as
+  router_top2_gating / switch_gating."""
+  lib = load_library()
+  b, t, m = x.shape
+  e = w_packed.shape[1]
+  s = int(group_size)
+  if (b * t) % s or t % s:
+    raise MoeHipError("tokens per router (%d) must be whole groups of %d"
+                      % (t, s))
+  g = b * t // s
+  dev = x.device
+  xp = _dev(x, "x", torch.bfloat16)
+  wp = _dev(w_packed, "w_packed", torch.bfloat16, (b, e, m))
+  bp = None if bias is None else _dev(bias, "bias", torch.float32, (e,))
+  ip, icode = None, F32
+  if importance is not None:
+    icode = dtype_code(importance.dtype)
+    ip = _dev(importance, "importance", None, (g, s))
+  logits = None
+  if want_logits:
+    logits = torch.empty((g, s, e), dtype=torch.float32, device=dev)
+  idx, pos, gate, kept, fill, loss, ws, ws_bytes = _routing_buffers(
+      lib, g, s, e, dev)
+  with _stage("router_switch_gating"):
+    _check(lib.mesh_moe_router_switch_gating(
+        xp, wp, bp, None if logits is None else logits.data_ptr(), b, t, m,
+        BF16, ip, icode, g, s, e, int(capacity), int(z_loss is not None),
+        float(z_loss or 0.0), int(num_microbatches or 1), idx.data_ptr(),
+        pos.data_ptr(), gate.data_ptr(), kept.data_ptr(), fill.data_ptr(),
+        loss.data_ptr(), ws.data_ptr(), ws_bytes, _stream()),
+        "router_switch_gating")
   r = Routing(idx, pos, gate, kept, fill, loss, int(capacity), e)
   if _timer is not None:
     _timer.routing.append(r)

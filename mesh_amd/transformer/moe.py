@@ -21,7 +21,7 @@ from mesh_amd import layers as mtf_layers
 from mesh_amd import moe_hip
 from mesh_amd import ops as mtf
 
-_OTHER_GATINGS = ("switch", "ntlb", "switch_max", "expert_selection")
+_OTHER_GATINGS = ("ntlb", "switch_max", "expert_selection")
 
 
 class HParams(object):
@@ -89,11 +89,12 @@ def _activation_name(activation):
 
 
 def _check_gating(hparams):
-  if hparams.moe_gating == "top_2":
+  if hparams.moe_gating in ("top_2", "switch"):
     return
   if hparams.moe_gating in _OTHER_GATINGS:
     raise NotImplementedError(
-        "moe_gating=%s is not implemented (top_2 only)" % hparams.moe_gating)
+        "moe_gating=%s is not implemented (top_2 and switch only)"
+        % hparams.moe_gating)
   raise ValueError("unknown hparams.moe_gating=%s" % hparams.moe_gating)
 
 
@@ -152,6 +153,48 @@ class _GatingSpec(object):
         use_second_place_loss=self.use_second_place_loss,
         num_microbatches=self.num_microbatches, second_uniform=uniform,
         importance_from_slot_gate=importance_from_slot_gate)
+
+
+class _SwitchGatingSpec(object):
+  """Static configuration of one _switch_gating call (moe.py:1176-1309) for
+  its deterministic policies: "argmax", and "input_dropout" / "input_jitter"
+  when not training, where the reference applies no perturbation
+  (moe.py:1192-1199)."""
+
+  def __init__(self, hparams, train, num_microbatches, has_importance):
+    policy = (hparams.moe_switch_policy_train if train
+              else hparams.moe_switch_policy_eval)
+    if policy == "sample" or (train and policy in ("input_dropout",
+                                                   "input_jitter")):
+      raise NotImplementedError(
+          "switch policy %r draws random numbers (%s) and is not implemented"
+          % (policy, "training" if train else "sampling"))
+    if policy not in ("argmax", "input_dropout", "input_jitter"):
+      raise ValueError("Unknown Switch gating policy %s" % policy)
+    self.z_loss = None
+    if train and getattr(hparams, "moe_z_loss", None) is not None:
+      # the reference evaluates equal(importance, 1.0) and
+      # denom * num_microbatches unconditionally (moe.py:1260-1264)
+      if not has_importance or not num_microbatches:
+        raise ValueError("moe_z_loss needs nonpadding and num_microbatches")
+      self.z_loss = float(hparams.moe_z_loss)
+    self.num_microbatches = num_microbatches
+
+  def route(self, x, w, w_packed, group_size, num_experts, capacity,
+            importance=None, importance_from_slot_gate=False):
+    """Same contract as _GatingSpec.route."""
+    assert not importance_from_slot_gate
+    b, t, _ = x.shape
+    groups = b * t // group_size
+    if moe_hip.fused_gating_supported(x, num_experts, group_size):
+      return moe_hip.router_switch_gating(
+          x, w_packed, group_size, capacity, importance=importance,
+          z_loss=self.z_loss, num_microbatches=self.num_microbatches)
+    logits = moe_hip.router_logits(x, w, w_packed=w_packed)
+    return moe_hip.switch_gating(
+        logits.reshape(groups, group_size, num_experts), capacity,
+        importance=importance, z_loss=self.z_loss,
+        num_microbatches=self.num_microbatches)
 
 
 def _packed(lowering, kernel_tensor, dtype):
@@ -215,7 +258,8 @@ def transformer_moe_layer_v1(
     layout=None, mesh_shape=None, nonpadding=None, activation=mtf.relu,
     num_microbatches=None):
   """Local mixture of experts: each position goes to 0-2 experts chosen by a
-  learned top-2 gate, with a fixed per-group capacity per expert.
+  learned top-2 gate (moe_gating="top_2") or to 0-1 experts chosen by a switch
+  gate (moe_gating="switch"), with a fixed per-group capacity per expert.
 
   Args:
     inputs: a mtf.Tensor with shape [batch_dim(s), length_dim, input_dim]
@@ -224,7 +268,8 @@ def transformer_moe_layer_v1(
       moe_group_size, moe_capacity_factor_train/eval, moe_min_expert_capacity,
       moe_gating, moe_dropout_rate, moe_use_experts_attention, moe_loss_coef,
       moe_use_second_place_loss, moe_second_policy_train/eval,
-      moe_second_threshold_train/eval)
+      moe_second_threshold_train/eval; for switch gating
+      moe_switch_policy_train/eval and moe_z_loss)
     train: a boolean
     variable_dtype: a mtf.VariableDType
     layout: optional - an input to mtf.convert_to_layout_rules
@@ -281,13 +326,19 @@ def transformer_moe_layer_v1(
                               "implemented (moe_dropout_rate must be 0)")
   if hparams.moe_use_experts_attention:
     raise NotImplementedError("moe_use_experts_attention is not implemented")
-  gating = _GatingSpec(hparams, train, num_microbatches)
+  if hparams.moe_gating == "switch":
+    gating = _SwitchGatingSpec(hparams, train, num_microbatches,
+                               nonpadding is not None)
+    router_name = "switch_gating"                       # moe.py:1179
+  else:
+    gating = _GatingSpec(hparams, train, num_microbatches)
+    router_name = "top_2_gating"                        # moe.py:1314
   act_name = _activation_name(activation)
 
   # variables, named and shaped as the reference's dense layers create them
   w_gate = mtf_layers.get_dense_kernel_weights(
       inputs, [experts_dim_unsplit], [input_dim], [], None,
-      name="top_2_gating", variable_dtype=variable_dtype)
+      name=router_name, variable_dtype=variable_dtype)
   wi = mtf_layers.get_dense_kernel_weights(
       inputs, [hidden_dim], [input_dim], [experts_dim], None, name="wi",
       variable_dtype=variable_dtype)

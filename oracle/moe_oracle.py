@@ -21,6 +21,11 @@ MoE file, and its TensorFlow dependency cannot run here):
   dispatch / combine einsums          gather/scatter form vs np.einsum
   expert FFN                          float64 matmul
   aux loss                            balanced-routing closed form (= 1.0)
+  switch_gating                       sequential integer loop, raw-probability
+                                      gate vs float64 softmax, closed forms for
+                                      the loss (balanced: = fraction of tokens
+                                      with importance 1) and the z-loss
+                                      (constant logits c: (c + log E)^2 / mb)
   v2                                  x=1 outer expert reduces to v1
 
 PARITY UNPINNED against TensorFlow itself (only running the reference could
@@ -267,6 +272,97 @@ def top_2_gating(logits, capacity, importance=None, policy="all",
   return out
 
 
+# ----------------------------------------------------------------------------
+# _switch_gating  (transformer/moe.py:1176-1309)
+# ----------------------------------------------------------------------------
+def switch_gating(logits, capacity, importance=None, train=False, z_loss=None,
+                  num_microbatches=None, act_dtype="float32", dense=False):
+  """Everything in _switch_gating after the router projection, for the
+  deterministic policies ("argmax"; "input_dropout" / "input_jitter" when not
+  training, where they change nothing, moe.py:1192-1199).
+
+  Same arguments and result dict as top_2_gating; the second-choice entries
+  are all "not kept" so that dispatch_gather / combine_gather apply unchanged.
+  The gate is the raw softmax probability of the chosen expert (no
+  normalisation).  z_loss (hparams.moe_z_loss) is added only when training
+  (moe.py:1253); the reference then needs `importance` and `num_microbatches`
+  (it evaluates equal(importance, 1.0) and denom * num_microbatches
+  unconditionally, moe.py:1260-1264) and so does this function.
+  """
+  logits = np.asarray(logits, dtype=F32)
+  g_, s_, e_ = logits.shape
+  cap_f = F32(float(capacity))
+
+  raw_gates = softmax(logits)                                    # :1207
+  expert_gate, expert_index = top_1(raw_gates)                   # :1210
+  expert_mask = one_hot(expert_index, e_)                        # :1221
+
+  # load balancing loss (:1224-1238).  density_1 is taken BEFORE the
+  # importance mask; density_1_proxy [G,E] times (importance == 1) [G,S]
+  # broadcasts to [G,E,S] and the mean runs over all three dims.
+  inv_s = F32(1.0 / s_)
+  density_1 = seq_sum(expert_mask, axis=-2) * inv_s              # [G,E]
+  density_1_proxy = seq_sum(raw_gates, axis=-2) * inv_s          # [G,E]
+  is_one = None
+  if importance is not None:
+    importance = np.asarray(importance, dtype=F32)
+    is_one = (importance == F32(1.0)).astype(F32)                # [G,S]
+    expert_mask = expert_mask * is_one[..., None]                # :1227
+    expert_gate = expert_gate * is_one                           # :1228
+    density_1_proxy = density_1_proxy[:, :, None] * is_one[:, None, :]
+    prod = density_1_proxy * density_1[:, :, None]               # [G,E,S]
+    # G*E*S terms: tf.reduce_sum's order is Eigen's tree, whose error does not
+    # grow with the length as a sequential float32 sum's would; a float64
+    # accumulation rounded once stands in for it
+    total = F32(prod.sum(dtype=np.float64))
+  else:
+    prod = density_1_proxy * density_1
+    total = seq_sum(prod.reshape(-1))
+  loss = total * F32(1.0 / prod.size)                            # reduce_mean
+  loss = loss * F32(float(e_ * e_))
+  if num_microbatches and num_microbatches > 1:                  # :1235-1238
+    loss = loss * F32(1.0 / num_microbatches)
+
+  if train and z_loss is not None:                               # :1253-1266
+    if is_one is None or not num_microbatches:
+      raise ValueError("z_loss needs importance and num_microbatches "
+                       "(moe.py:1260-1264)")
+    m = logits.max(axis=-1, keepdims=True)                       # :5510-5520
+    log_z = np.log(seq_sum(np.exp(logits + (-m)).astype(F32), axis=-1)
+                   ).astype(F32) + m[..., 0]
+    z = (log_z * log_z) * is_one                                 # square, mask
+    denom = seq_sum(is_one.reshape(-1))
+    z = seq_sum(z.reshape(-1)) / (denom * F32(num_microbatches))
+    loss = loss + F32(z_loss) * z                                # :1266
+
+  # capacity assignment (:1268-1291)
+  position_in_expert = cumsum_exclusive(expert_mask, dense) * expert_mask
+  expert_mask = expert_mask * (position_in_expert < cap_f).astype(F32)
+  expert_mask_flat = seq_sum(expert_mask, axis=-1)               # [G,S]
+  expert_gate = expert_gate * expert_mask_flat                   # :1291
+
+  pos_full = position_in_expert.astype(np.int32)                 # [G,S,E]
+  pos_1 = np.take_along_axis(pos_full, expert_index[..., None], -1)[..., 0]
+  zeros_i = np.zeros_like(expert_index)
+  out = dict(
+      index_1=expert_index, index_2=zeros_i, pos_1=pos_1, pos_2=zeros_i,
+      kept_1=expert_mask_flat > 0, kept_2=np.zeros(expert_index.shape, bool),
+      gate_1=expert_gate, gate_2=np.zeros_like(expert_gate),
+      fill=seq_sum(expert_mask, axis=-2).astype(np.int32),
+      loss=cast_act(loss, act_dtype)[()])                        # :1304
+  if dense:
+    # one_hot(to_int32(position_in_expert)) is taken per expert ([G,S,E] ->
+    # [G,S,E,C]); non-chosen experts have position 0 but a zero one_hot(index)
+    combine = (                                                  # :1293-1299
+        (expert_gate * expert_mask_flat)[..., None, None]
+        * one_hot(expert_index, e_)[..., None]
+        * one_hot(pos_full, capacity))
+    combine = cast_act(combine, act_dtype)                       # :1302
+    out["combine"] = combine
+    out["dispatch"] = (combine != 0).astype(F32)                 # :1305-1306
+  return out
+
+
 def routing_sequential(index_1, index_2, sel_1, sel_2, num_experts, capacity):
   """Integer brute force for moe.py:1472-1496, one token at a time.
 
@@ -392,7 +488,10 @@ def default_hparams(**overrides):
       moe_use_second_place_loss=False,
       moe_second_policy_train="random", moe_second_policy_eval="random",
       moe_second_threshold_train=0.2, moe_second_threshold_eval=0.2,
-      moe_dropout_rate=0.0, moe_use_experts_attention=False)
+      moe_dropout_rate=0.0, moe_use_experts_attention=False,
+      moe_switch_policy_train="input_jitter",
+      moe_switch_policy_eval="input_jitter", moe_switch_dropout=0.1,
+      moe_switch_temperature=1.0, moe_switch_jitter=1e-2, moe_z_loss=None)
   hp.update(overrides)
   return HParams(**hp)
 
@@ -444,7 +543,7 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
 
   Returns (output [batch..., length, N], loss scalar, aux dict).
   """
-  if hp.moe_gating != "top_2":
+  if hp.moe_gating not in ("top_2", "switch"):
     raise ValueError("unknown hparams.moe_gating=%s" % hp.moe_gating)
   x = cast_act(x, act_dtype)
   lead = x.shape[:-1]
@@ -463,10 +562,19 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
   logits = router_logits(xg, wg)
   if logit_bias is not None:
     logits = logits + np.asarray(logit_bias, F32)
-  policy, threshold = _policy(hp, train)
-  r = top_2_gating(logits, c_, importance, policy, threshold,
-                   hp.moe_use_second_place_loss, num_microbatches, act_dtype,
-                   second_uniform, dense=dense)
+  if hp.moe_gating == "switch":                                  # :393-402
+    sw = hp.moe_switch_policy_train if train else hp.moe_switch_policy_eval
+    if sw == "sample" or (train and sw in ("input_dropout", "input_jitter")):
+      raise NotImplementedError("switch policy %r draws random numbers" % sw)
+    if sw not in ("argmax", "input_dropout", "input_jitter"):
+      raise ValueError("Unknown Switch gating policy %s" % sw)
+    r = switch_gating(logits, c_, importance, train, hp.moe_z_loss,
+                      num_microbatches, act_dtype, dense=dense)
+  else:
+    policy, threshold = _policy(hp, train)
+    r = top_2_gating(logits, c_, importance, policy, threshold,
+                     hp.moe_use_second_place_loss, num_microbatches, act_dtype,
+                     second_uniform, dense=dense)
   # weights_are_cast: the caller already holds activation-dtype values (lets
   # the CPU-baseline timing pass one expert's matrix broadcast to all experts)
   wi_a = wi if weights_are_cast else cast_act(wi, act_dtype)

@@ -1,4 +1,5 @@
-"""Writes tests/golden/top2_gating_small.json from the CPU oracle.
+"""Writes tests/golden/top2_gating_small.json and switch_gating_small.json from
+the CPU oracle.
 
 The reference holds no test, golden vector or fixture for its MoE file, and its
 TensorFlow dependency is not installed, so these vectors come from the oracle
@@ -31,6 +32,18 @@ def main():
   for k in ("gate_1", "gate_2"):
     out[k] = [[float(v) for v in row] for row in r[k]]
   with open(os.path.join(HERE, "top2_gating_small.json"), "w") as f:
+    json.dump(out, f)
+
+  # switch gating on the same logits, with a padding mask and the z-loss
+  imp = (rng.random((g, s)) < 0.8).astype(np.float32)
+  r = O.switch_gating(logits, c, importance=imp, train=True, z_loss=1e-2,
+                      num_microbatches=2)
+  out = dict(capacity=c, logits=logits.tolist(), importance=imp.tolist(),
+             z_loss=1e-2, num_microbatches=2, loss=float(r["loss"]))
+  for k in ("index_1", "pos_1", "kept_1"):
+    out[k] = r[k].astype(int).tolist()
+  out["gate_1"] = [[float(v) for v in row] for row in r["gate_1"]]
+  with open(os.path.join(HERE, "switch_gating_small.json"), "w") as f:
     json.dump(out, f)
 
 

@@ -104,6 +104,21 @@ def test_split_into_groups():
     moe._split_into_groups(10, 4, 3)
 
 
+def test_v1_switch_graph_names():
+  """The switch router's variable lives under "switch_gating" (the `name`
+  default of _switch_gating, transformer/moe.py:1179)."""
+  graph, _, x, dims = graph_input()
+  hp = hparams(moe_gating="switch", moe_switch_policy_train="argmax",
+               moe_switch_policy_eval="argmax", moe_z_loss=None)
+  with mtf.variable_scope("layer_0"):
+    y, loss = moe.transformer_moe_layer_v1(
+        x, dims[-1], hp, True, mtf.VariableDType(torch.float32))
+  assert y.shape == mtf.Shape(dims) and loss.shape == mtf.Shape([])
+  names = sorted(v.name for v in graph.all_variables)
+  assert names == ["layer_0/switch_gating/kernel", "layer_0/wi/kernel",
+                   "layer_0/wo/kernel"]
+
+
 def test_v1_graph_names_and_shapes():
   graph, _, x, dims = graph_input()
   with mtf.variable_scope("layer_0"):
@@ -158,7 +173,20 @@ def test_error_behaviour():
     moe.transformer_moe_layer_v1(
         x, dims[-1], hparams(moe_second_policy_train="sometimes"), True, vdt)
   with pytest.raises(NotImplementedError):
+    moe.transformer_moe_layer_v1(x, dims[-1], hparams(moe_gating="ntlb"), True, vdt)
+  # switch gating reads its own hyperparameters, as the reference does
+  with pytest.raises(AttributeError, match="moe_switch_policy_train"):
     moe.transformer_moe_layer_v1(x, dims[-1], hparams(moe_gating="switch"), True, vdt)
+  sw = dict(moe_gating="switch", moe_switch_policy_train="argmax",
+            moe_switch_policy_eval="sample", moe_z_loss=None)
+  with pytest.raises(NotImplementedError, match="random numbers"):
+    moe.transformer_moe_layer_v1(x, dims[-1], hparams(**sw), False, vdt)
+  with pytest.raises(ValueError, match="Unknown Switch gating policy"):
+    moe.transformer_moe_layer_v1(
+        x, dims[-1], hparams(**dict(sw, moe_switch_policy_train="best")), True, vdt)
+  with pytest.raises(ValueError, match="moe_z_loss needs"):
+    moe.transformer_moe_layer_v1(
+        x, dims[-1], hparams(**dict(sw, moe_z_loss=1e-3)), True, vdt)
   with pytest.raises(NotImplementedError):
     moe.transformer_moe_layer_v1(x, dims[-1], hparams(moe_dropout_rate=0.1), True, vdt)
   with pytest.raises(ValueError, match="not a multiple of mesh_dim_size"):

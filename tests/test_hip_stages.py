@@ -359,3 +359,125 @@ def test_router_top2_gating_rejects_unsupported(hip):
   assert not hip.fused_gating_supported(x, 8, 96)
   with pytest.raises(hip.MoeHipError, match="fused kernel needs"):
     hip.router_top2_gating(x, wp, 96, 4)
+
+
+# ---- switch (top-1) gating ------------------------------------------------------
+@pytest.mark.parametrize("shape", [(2, 1024, 8, 160), (16, 2048, 64, 32),
+                                   (3, 77, 5, 7), (1, 1, 2, 1),
+                                   (2, 130, 200, 4), (1, 4096, 64, 70)])
+def test_switch_gating_random_logits(hip, shape):
+  g, s, e, c = shape
+  rng = np.random.default_rng(1000 + hash(shape) % 1000)
+  logits = H.safe_logits(rng, g, s, e, scale=1.5)
+  want = O.switch_gating(logits, c)
+  got = H.routing_to_np(hip.switch_gating(torch.from_numpy(logits).cuda(), c))
+  H.assert_routing_equal(got, want)
+  np.testing.assert_allclose(got["loss"], want["loss"], rtol=2e-5)
+
+
+def test_switch_gating_exact_ties(hip):
+  g, s, e, c = 3, 500, 64, 9
+  rng = np.random.default_rng(8)
+  logits = H.random_logits(rng, g, s, e, scale=0.6, quantum=0.25)
+  want = O.switch_gating(logits, c)
+  got = H.routing_to_np(hip.switch_gating(torch.from_numpy(logits).cuda(), c))
+  H.assert_routing_equal(got, want)
+
+
+@pytest.mark.parametrize("imp_dtype", ["float32", "bfloat16"])
+def test_switch_gating_importance_and_z_loss(hip, imp_dtype):
+  g, s, e, c = 4, 320, 16, 24
+  rng = np.random.default_rng(12)
+  logits = H.safe_logits(rng, g, s, e)
+  imp = rng.choice(np.array([0.0, 0.5, 1.0], np.float32), size=(g, s),
+                   p=[0.2, 0.2, 0.6])
+  lg = torch.from_numpy(logits).cuda()
+  for z, mb in ((None, None), (1e-3, 1), (0.5, 4)):
+    want = O.switch_gating(logits, c, importance=imp, train=True, z_loss=z,
+                           num_microbatches=mb)
+    got = H.routing_to_np(hip.switch_gating(
+        lg, c, importance=H.to_gpu(imp, imp_dtype), z_loss=z,
+        num_microbatches=mb))
+    H.assert_routing_equal(got, want)
+    np.testing.assert_allclose(got["loss"], want["loss"], rtol=2e-5)
+  # only importance == 1 rows are routed
+  assert not got["kept_1"][imp != 1.0].any()
+  assert (got["gate_1"][imp != 1.0] == 0).all()
+  # z-loss closed form through the kernel: constant logits c0 give
+  # (c0 + log E)^2 / microbatches whatever the mask
+  const = torch.full((g, s, e), 1.5, dtype=torch.float32, device="cuda")
+  a = hip.switch_gating(const, c, importance=H.to_gpu(imp), z_loss=0.1,
+                        num_microbatches=2).loss.item()
+  b = hip.switch_gating(const, c, importance=H.to_gpu(imp),
+                        num_microbatches=2).loss.item()
+  np.testing.assert_allclose(a - b, 0.1 * (1.5 + np.log(e)) ** 2 / 2, rtol=1e-4)
+
+
+@pytest.mark.parametrize("case", [
+    (1, 2, 256, 128, 8, 70), (2, 2, 384, 192, 20, 40), (1, 16, 1024, 1024, 32, 40)])
+def test_router_switch_gating_fused(hip, case):
+  b, gpr, s, m, e, c = case
+  rng = np.random.default_rng(43)
+  w = O.round_bf16((rng.standard_normal((b, m, e)) / np.sqrt(m)).astype(np.float32))
+  x = np.stack([H.safe_tokens(rng, gpr * s, m, w[i], "bfloat16") for i in range(b)])
+  imp = rng.choice(np.array([0.0, 1.0], np.float32), size=(b * gpr, s),
+                   p=[0.2, 0.8])
+  logits = np.matmul(x, w).astype(np.float32).reshape(b * gpr, s, e)
+  xg, wg = H.to_gpu(x, "bfloat16"), H.to_gpu(w, "bfloat16")
+  wp = hip.pack_weights(wg, wg.dtype)
+  for importance, z in ((None, None), (imp, 1e-2)):
+    want = O.switch_gating(logits, c, importance=importance, train=True,
+                           z_loss=z, num_microbatches=2)
+    gi = None if importance is None else H.to_gpu(importance)
+    r, got_logits = hip.router_switch_gating(
+        xg, wp, s, c, importance=gi, z_loss=z, num_microbatches=2,
+        want_logits=True)
+    np.testing.assert_allclose(H.to_np(got_logits), logits, rtol=1e-5, atol=2e-5)
+    got = H.routing_to_np(r)
+    H.assert_routing_equal(got, want, gate_rtol=2e-5)
+    np.testing.assert_allclose(got["loss"], want["loss"], rtol=5e-5)
+    r2 = hip.switch_gating(got_logits, c, importance=gi, z_loss=z,
+                           num_microbatches=2)
+    for a_, b_ in ((r.idx, r2.idx), (r.pos, r2.pos), (r.kept, r2.kept),
+                   (r.fill, r2.fill), (r.gate, r2.gate)):
+      assert torch.equal(a_, b_)
+
+
+def test_switch_dispatch_combine_roundtrip(hip):
+  """Switch routing record through the unchanged dispatch / combine kernels."""
+  g, s, e, c, m = 2, 256, 8, 40, 64
+  rng = np.random.default_rng(44)
+  logits = H.safe_logits(rng, g, s, e)
+  x = rng.standard_normal((g, s, m)).astype(np.float32)
+  want_r = O.switch_gating(logits, c)
+  r = hip.switch_gating(torch.from_numpy(logits).cuda(), c)
+  xg = H.to_gpu(x)
+  expert_in = hip.dispatch(xg, r)
+  np.testing.assert_array_equal(H.to_np(expert_in),
+                                O.dispatch_gather(x, want_r, e, c, "float32"))
+  out = hip.combine(expert_in, r, s)
+  np.testing.assert_allclose(
+      H.to_np(out), O.combine_gather(H.to_np(expert_in), want_r, "float32"),
+      rtol=1e-6, atol=1e-7)
+
+
+def test_switch_gating_golden_fixture(hip):
+  """The committed golden vectors (tests/golden/switch_gating_small.json)."""
+  import json
+  import os
+  path = os.path.join(os.path.dirname(__file__), "golden",
+                      "switch_gating_small.json")
+  with open(path) as f:
+    gold = json.load(f)
+  logits = np.array(gold["logits"], np.float32)
+  imp = np.array(gold["importance"], np.float32)
+  got = H.routing_to_np(hip.switch_gating(
+      torch.from_numpy(logits).cuda(), gold["capacity"],
+      importance=H.to_gpu(imp), z_loss=gold["z_loss"],
+      num_microbatches=gold["num_microbatches"]))
+  for k in ("index_1", "pos_1"):
+    np.testing.assert_array_equal(got[k], np.array(gold[k]), err_msg=k)
+  np.testing.assert_array_equal(got["kept_1"], np.array(gold["kept_1"], bool))
+  np.testing.assert_allclose(got["gate_1"], np.array(gold["gate_1"]), rtol=1e-5,
+                             atol=1e-7)
+  np.testing.assert_allclose(got["loss"], gold["loss"], rtol=2e-5)

@@ -46,7 +46,8 @@ def run_v1(x, weights, hp, train, act_dtype, nonpadding=None, activation="relu",
     y, loss = moe.transformer_moe_layer_v1(
         xt, mtf.Dimension("d_model", n), hp, train, vdt, nonpadding=npad,
         activation=activation, num_microbatches=num_microbatches)
-  init = {"moe/top_2_gating/kernel": weights["w_gate"],
+  router = "switch_gating" if hp.moe_gating == "switch" else "top_2_gating"
+  init = {"moe/%s/kernel" % router: weights["w_gate"],
           "moe/wi/kernel": weights["wi"], "moe/wo/kernel": weights["wo"]}
   lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()}, initial_values=init)
   out = H.to_np(lowering.export_to_tf_tensor(y))
@@ -239,3 +240,84 @@ def test_v2_nonpadding():
   np.testing.assert_allclose(got, want, **H.value_tolerance("float32"))
   assert (got[nonpadding == 0] == 0).all()
   np.testing.assert_allclose(got_loss, want_loss, rtol=1e-5)
+
+
+# ---- switch gating ------------------------------------------------------------
+SWITCH_HP = dict(moe_gating="switch", moe_switch_policy_train="argmax",
+                 moe_switch_policy_eval="input_jitter", moe_switch_dropout=0.1,
+                 moe_switch_temperature=1.0, moe_switch_jitter=1e-2,
+                 moe_z_loss=None)
+
+
+@pytest.mark.parametrize("case", V1_CASES[:3] + V1_CASES[4:],
+                         ids=[c[0] for c in V1_CASES[:3] + V1_CASES[4:]])
+def test_v1_switch_matches_oracle(case):
+  _, b, l, m, hdim, e, group, cf, act_dtype = case
+  rng = np.random.default_rng(301)
+  w = dict(w_gate=H.normal_weights(rng, (m, e), m),
+           wi=H.normal_weights(rng, (e, m, hdim), m),
+           wo=H.normal_weights(rng, (e, hdim, m), hdim))
+  x = H.safe_tokens(rng, b * l, m, w["w_gate"], act_dtype).reshape(b, l, m)
+  hp, ohp = make_hparams(moe_num_experts=e, moe_hidden_size=hdim,
+                         moe_group_size=group, moe_capacity_factor_eval=cf,
+                         **SWITCH_HP)
+  got, got_loss, _, _ = run_v1(x, w, hp, False, act_dtype)
+  want, want_loss, aux = O.moe_layer_v1(x, w["w_gate"], w["wi"], w["wo"], ohp,
+                                        False, act_dtype, dense=b * l <= 4096)
+  assert not aux["kept_1"].all()                 # the drop path is exercised
+  np.testing.assert_allclose(got, want, **H.value_tolerance(act_dtype))
+  np.testing.assert_allclose(got_loss, want_loss,
+                             rtol=1e-2 if act_dtype == "bfloat16" else 1e-4)
+  # dropped tokens output exactly zero
+  assert (got.reshape(-1, m)[~aux["kept_1"].reshape(-1)] == 0).all()
+
+
+def test_v1_switch_train_z_loss_and_nonpadding():
+  b, l, m, hdim, e = 2, 96, 32, 48, 4
+  rng = np.random.default_rng(302)
+  w = dict(w_gate=H.normal_weights(rng, (m, e), m),
+           wi=H.normal_weights(rng, (e, m, hdim), m),
+           wo=H.normal_weights(rng, (e, hdim, m), hdim))
+  x = H.safe_tokens(rng, b * l, m, w["w_gate"], "float32").reshape(b, l, m)
+  nonpad = (rng.random((b, l)) < 0.8).astype(np.float32)
+  kw = dict(SWITCH_HP, moe_z_loss=1e-2)
+  hp, ohp = make_hparams(moe_num_experts=e, moe_hidden_size=hdim,
+                         moe_group_size=64, moe_capacity_factor_train=1.0, **kw)
+  got, got_loss, _, _ = run_v1(x, w, hp, True, "float32", nonpadding=nonpad,
+                               num_microbatches=2)
+  want, want_loss, aux = O.moe_layer_v1(x, w["w_gate"], w["wi"], w["wo"], ohp,
+                                        True, "float32", nonpadding=nonpad,
+                                        num_microbatches=2)
+  np.testing.assert_allclose(got, want, **H.value_tolerance("float32"))
+  np.testing.assert_allclose(got_loss, want_loss, rtol=1e-4)
+  assert (got[nonpad == 0] == 0).all()
+  # the z-loss is part of the loss: without it the value differs
+  hp0, _ = make_hparams(moe_num_experts=e, moe_hidden_size=hdim,
+                        moe_group_size=64, moe_capacity_factor_train=1.0,
+                        **SWITCH_HP)
+  _, loss0, _, _ = run_v1(x, w, hp0, True, "float32", nonpadding=nonpad,
+                          num_microbatches=2)
+  assert got_loss > loss0
+
+
+def test_v1_switch_rejections():
+  x = np.zeros((1, 32, 16), np.float32)
+  w = dict(w_gate=np.zeros((16, 4), np.float32),
+           wi=np.zeros((4, 16, 8), np.float32),
+           wo=np.zeros((4, 8, 16), np.float32))
+  base = dict(moe_num_experts=4, moe_hidden_size=8, moe_group_size=32)
+  hp, _ = make_hparams(**dict(base, **dict(SWITCH_HP,
+                                          moe_switch_policy_eval="sample")))
+  with pytest.raises(NotImplementedError, match="random"):
+    run_v1(x, w, hp, False, "float32")
+  hp, _ = make_hparams(**dict(base, **dict(SWITCH_HP,
+                                          moe_switch_policy_train="input_jitter")))
+  with pytest.raises(NotImplementedError, match="random"):
+    run_v1(x, w, hp, True, "float32")
+  hp, _ = make_hparams(**dict(base, **dict(SWITCH_HP,
+                                          moe_switch_policy_eval="bogus")))
+  with pytest.raises(ValueError, match="Unknown Switch gating policy"):
+    run_v1(x, w, hp, False, "float32")
+  hp, _ = make_hparams(**dict(base, **dict(SWITCH_HP, moe_z_loss=1e-3)))
+  with pytest.raises(ValueError, match="moe_z_loss needs"):
+    run_v1(x, w, hp, True, "float32")

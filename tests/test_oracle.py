@@ -297,6 +297,159 @@ def test_balanced_routing_loss_is_one():
   np.testing.assert_allclose(a, e / 4, rtol=1e-5)
 
 
+# ---- switch (top-1) gating ------------------------------------------------------
+@pytest.mark.parametrize("seed", range(4))
+def test_switch_against_sequential_loop_and_float64(seed):
+  """One choice per token: positions/drops against a per-token integer loop
+  written from transformer/moe.py:1268-1291, the gate against a float64 softmax
+  (raw probability of the arg-max expert, not normalised)."""
+  rng = np.random.default_rng(300 + seed)
+  g, s, e = 3, int(rng.integers(5, 90)), int(rng.integers(2, 9))
+  c = int(rng.integers(1, s // e + 3))
+  logits = rng.standard_normal((g, s, e)).astype(np.float32)
+  imp = None
+  if seed % 2:
+    imp = rng.choice(np.array([0.0, 0.5, 1.0], np.float32), size=(g, s))
+  p64 = scipy.special.softmax(logits.astype(np.float64), axis=-1)
+  for dense in (False, True):
+    r = O.switch_gating(logits, c, importance=imp, dense=dense)
+    np.testing.assert_array_equal(r["index_1"], p64.argmax(-1))
+    assert not r["kept_2"].any() and not r["gate_2"].any()
+    for gi in range(g):
+      count = [0] * e
+      for si in range(s):
+        ex = int(r["index_1"][gi, si])
+        competes = imp is None or imp[gi, si] == 1.0
+        if not competes:
+          assert not r["kept_1"][gi, si] and r["gate_1"][gi, si] == 0
+          continue
+        slot = count[ex]
+        count[ex] += 1
+        assert r["pos_1"][gi, si] == slot
+        assert r["kept_1"][gi, si] == (slot < c)
+        want = p64[gi, si, ex] if slot < c else 0.0
+        np.testing.assert_allclose(r["gate_1"][gi, si], want, rtol=2e-6)
+      np.testing.assert_array_equal(r["fill"][gi], np.minimum(count, c))
+
+
+def test_switch_first_choice_equals_top2_first_choice():
+  """The first-choice bookkeeping of the two routers is the same code path in
+  the reference (moe.py:1268-1275 vs :1472-1476): same experts, positions and
+  drops; only the gate differs (raw probability vs normalised pair)."""
+  rng = np.random.default_rng(31)
+  logits = rng.standard_normal((2, 120, 6)).astype(np.float32)
+  imp = rng.choice(np.array([0.0, 1.0], np.float32), size=(2, 120))
+  a = O.switch_gating(logits, 17, importance=imp)
+  b = O.top_2_gating(logits, 17, importance=imp, policy="none")
+  for k in ("index_1", "kept_1", "fill"):
+    np.testing.assert_array_equal(a[k], b[k])
+  np.testing.assert_array_equal(a["pos_1"][a["kept_1"]], b["pos_1"][b["kept_1"]])
+  p = O.softmax(logits)
+  np.testing.assert_array_equal(a["gate_1"][a["kept_1"]],
+                                p.max(-1)[a["kept_1"]])
+
+
+def test_switch_loss_closed_forms():
+  """density_1 is taken before the importance mask and the proxy is multiplied
+  by (importance == 1) per token (moe.py:1224-1234): with uniform gates and
+  balanced arg-max the loss is the fraction of tokens with importance 1."""
+  e, s = 8, 64
+  logits = np.zeros((2, s, e), np.float32)
+  logits[:, np.arange(s), np.arange(s) % e] = 1e-4
+  np.testing.assert_allclose(O.switch_gating(logits, 1000)["loss"], 1.0,
+                             rtol=1e-4)
+  imp = np.ones((2, s), np.float32)
+  imp[0, :16] = 0.0
+  imp[1, :32] = 0.5
+  r = O.switch_gating(logits, 1000, importance=imp)
+  np.testing.assert_allclose(r["loss"], (48 + 32) / 128.0, rtol=1e-4)
+  # all mass on one expert -> E; microbatches divide
+  one = np.zeros((1, s, e), np.float32)
+  one[..., 3] = 30.0
+  np.testing.assert_allclose(O.switch_gating(one, 1000)["loss"], e, rtol=1e-5)
+  np.testing.assert_allclose(
+      O.switch_gating(one, 1000, num_microbatches=4)["loss"], e / 4, rtol=1e-5)
+
+
+def test_switch_z_loss_closed_form():
+  """Constant logits c: logsumexp = c + log E for every token, so
+  z_loss = (c + log E)^2 / num_microbatches whatever the mask
+  (moe.py:1253-1266); added only when training."""
+  e, s, c0 = 4, 32, 1.5
+  logits = np.full((2, s, e), c0, np.float32)
+  imp = np.ones((2, s), np.float32)
+  imp[1, ::3] = 0.0
+  base = O.switch_gating(logits, 100, importance=imp, train=True,
+                         num_microbatches=2)["loss"]
+  got = O.switch_gating(logits, 100, importance=imp, train=True, z_loss=0.1,
+                        num_microbatches=2)["loss"]
+  np.testing.assert_allclose(got - base, 0.1 * (c0 + np.log(e)) ** 2 / 2,
+                             rtol=1e-5)
+  evalv = O.switch_gating(logits, 100, importance=imp, train=False, z_loss=0.1,
+                          num_microbatches=2)["loss"]
+  assert evalv == base
+  # masked tokens do not contribute: give them huge logits
+  big = logits.copy()
+  big[1, ::3] = 40.0
+  got2 = O.switch_gating(big, 100, importance=imp, train=True, z_loss=0.1,
+                         num_microbatches=2)
+  base2 = O.switch_gating(big, 100, importance=imp, train=True,
+                          num_microbatches=2)
+  np.testing.assert_allclose(got2["loss"] - base2["loss"],
+                             0.1 * (c0 + np.log(e)) ** 2 / 2, rtol=1e-4)
+  with pytest.raises(ValueError):
+    O.switch_gating(logits, 100, train=True, z_loss=0.1, num_microbatches=2)
+
+
+@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
+def test_switch_dense_tensors_match_index_record(act_dtype):
+  rng = np.random.default_rng(33)
+  g, s, e, c = 2, 40, 5, 6
+  logits = rng.standard_normal((g, s, e)).astype(np.float32)
+  r = O.switch_gating(logits, c, act_dtype=act_dtype, dense=True)
+  want = np.zeros((g, s, e, c), np.float32)
+  w = O.cast_act(r["gate_1"], act_dtype)
+  for gi in range(g):
+    for si in range(s):
+      if r["kept_1"][gi, si]:
+        want[gi, si, r["index_1"][gi, si], r["pos_1"][gi, si]] = w[gi, si]
+  np.testing.assert_array_equal(r["combine"], want)
+  np.testing.assert_array_equal(r["dispatch"], (want != 0).astype(np.float32))
+  assert (r["dispatch"].sum(axis=1) <= 1).all()      # one token per slot
+
+
+def test_v1_switch_dense_equals_index_form():
+  rng = np.random.default_rng(34)
+  b, l, m, h, e = 2, 48, 16, 24, 4
+  x = rng.standard_normal((b, l, m)).astype(np.float32)
+  wg = rng.standard_normal((m, e)).astype(np.float32)
+  wi = rng.standard_normal((e, m, h)).astype(np.float32) / 4
+  wo = rng.standard_normal((e, h, m)).astype(np.float32) / 5
+  hp = O.default_hparams(moe_gating="switch", moe_num_experts=e,
+                         moe_hidden_size=h, moe_group_size=32,
+                         moe_capacity_factor_eval=1.0)
+  nonpad = (rng.random((b, l)) < 0.8).astype(np.float32)
+  d, dl, aux = O.moe_layer_v1(x, wg, wi, wo, hp, False, nonpadding=nonpad,
+                              dense=True)
+  i, il, _ = O.moe_layer_v1(x, wg, wi, wo, hp, False, nonpadding=nonpad,
+                            dense=False)
+  np.testing.assert_allclose(d, i, rtol=1e-5, atol=1e-5)
+  assert dl == il
+  assert (d[nonpad == 0] == 0).all()
+  assert (d[~aux["kept_1"].reshape(b, l)] == 0).all()
+  # a token that kept its slot gets gate * FFN_e(x): check one by hand
+  t = int(np.flatnonzero(aux["kept_1"].reshape(-1))[0])
+  ex = int(aux["index_1"].reshape(-1)[t])
+  xt = x.reshape(-1, m)[t].astype(np.float64)
+  ref = np.maximum(xt @ wi[ex].astype(np.float64), 0) @ wo[ex].astype(np.float64)
+  np.testing.assert_allclose(d.reshape(-1, m)[t],
+                             aux["gate_1"].reshape(-1)[t] * ref, rtol=1e-4,
+                             atol=1e-5)
+  hp.moe_switch_policy_eval = "sample"
+  with pytest.raises(NotImplementedError):
+    O.moe_layer_v1(x, wg, wi, wo, hp, False)
+
+
 # ---- the layers ----------------------------------------------------------------
 def _hp(**kw):
   base = dict(moe_second_policy_train="all", moe_second_policy_eval="all")
@@ -403,5 +556,20 @@ def test_golden_fixture():
     np.testing.assert_array_equal(r[k], np.array(gold[k]))
   np.testing.assert_array_equal(r["kept_1"], np.array(gold["kept_1"], bool))
   np.testing.assert_array_equal(r["kept_2"], np.array(gold["kept_2"], bool))
+  np.testing.assert_allclose(r["gate_1"], np.array(gold["gate_1"]), rtol=1e-6)
+  np.testing.assert_allclose(r["loss"], gold["loss"], rtol=1e-6)
+
+
+def test_switch_golden_fixture():
+  path = os.path.join(GOLDEN, "switch_gating_small.json")
+  with open(path) as f:
+    gold = json.load(f)
+  r = O.switch_gating(np.array(gold["logits"], np.float32), gold["capacity"],
+                      importance=np.array(gold["importance"], np.float32),
+                      train=True, z_loss=gold["z_loss"],
+                      num_microbatches=gold["num_microbatches"])
+  for k in ("index_1", "pos_1"):
+    np.testing.assert_array_equal(r[k], np.array(gold[k]))
+  np.testing.assert_array_equal(r["kept_1"], np.array(gold["kept_1"], bool))
   np.testing.assert_allclose(r["gate_1"], np.array(gold["gate_1"]), rtol=1e-6)
   np.testing.assert_allclose(r["loss"], gold["loss"], rtol=1e-6)
