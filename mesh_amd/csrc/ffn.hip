@@ -456,6 +456,260 @@ __global__ __launch_bounds__(64 * WM * WN) void grouped_gemm_bf16_dma_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// bf16 MFMA kernel for 256 x 256 tiles with SPREAD direct-to-LDS loads.
+//
+// Same tile, wavefront grid (2 x 4, 128 x 64 sub-tiles), LDS image and
+// fragment reads as grouped_gemm_bf16_dma_kernel<256, 256, 4, RELU, 2>; the
+// difference is when the loads are issued.  A wavefront that issues its eight
+// loads of a K tile back to back sits in that burst for ~0.7 us (the memory
+// pipeline accepts them only as fast as earlier requests drain), and because
+// the wavefronts of a block hand over together, the MFMA pipes idle meanwhile.
+// Here the 160 KB of LDS hold two slots for the token tile and THREE for the
+// weight tile, which lets every MFMA step carry exactly two loads:
+//
+//   step 0 of tile t:  token loads 2,3 of tile t+1
+//   step 1, step 2:    weight loads 0,1 / 2,3 of tile t+2   (two tiles ahead)
+//   step 3 (after the hand-over barrier): token loads 0,1 of tile t+2
+//
+// vmcnt counts in issue order, so the hand-over of tile t waits with vmcnt(4):
+// everything up to the token loads of tile t+1 has landed, the four weight
+// loads of tile t+2 stay in flight.
+// ---------------------------------------------------------------------------
+struct RingCfg {
+  static constexpr int BM = 256, BN = 256, BK = 64, WM = 2, WN = 4;
+  static constexpr int WAVES = WM * WN, THREADS = 64 * WAVES;
+  static constexpr int WTM = BM / WM, WTN = BN / WN;
+  static constexpr int TM = WTM / 32, TN = WTN / 32;
+  static constexpr int ROW_BYTES = BK * 2;
+  static constexpr int A_INSTR = (BM / 8) / WAVES, B_INSTR = (BN / 8) / WAVES;
+  static constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES;
+  static constexpr int A_SLOTS = 2, B_SLOTS = 3;
+  static constexpr int B_BASE = A_SLOTS * A_BYTES;
+  static constexpr int LDC = BN + 4;
+  static constexpr size_t LOOP_BYTES = (size_t)A_SLOTS * A_BYTES + (size_t)B_SLOTS * B_BYTES;
+  static constexpr size_t EPI_BYTES = (size_t)BM * LDC * sizeof(bf16_t);
+  static constexpr size_t LDS_BYTES = LOOP_BYTES > EPI_BYTES ? LOOP_BYTES : EPI_BYTES;
+  static_assert(A_INSTR == 4 && B_INSTR == 4, "load schedule assumes 4 + 4");
+};
+
+template <bool RELU, bool DEEP_B>
+__global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
+    bf16_t* __restrict__ Cout, int R, int N, int K, int tiles_m, int tiles_n) {
+  using Cfg = RingCfg;
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, WN = Cfg::WN;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+
+  const int nblk = gridDim.x;
+  const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+  const int per_xcd = nblk >> 3, extra = nblk & 7;
+  const int logical = xcd * per_xcd + min(xcd, extra) + local;
+  const int tiles_per_e = tiles_m * tiles_n;
+  const int e = logical / tiles_per_e;
+  const int rem = logical - e * tiles_per_e;
+  const int tn = rem / tiles_m;
+  const int tm = rem - tn * tiles_m;
+  const int row0 = tm * BM, col0 = tn * BN;
+  const bf16_t* Ae = A + (int64_t)e * R * K;
+  const bf16_t* Be = B + (int64_t)e * N * K;
+  bf16_t* Ce = Cout + (int64_t)e * R * N;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int wm = wave / WN, wn = wave % WN;
+
+  int a_off[Cfg::A_INSTR], b_off[Cfg::B_INSTR];
+#pragma unroll
+  for (int j = 0; j < Cfg::A_INSTR; ++j) {
+    const int row = (wave + Cfg::WAVES * j) * 8 + (lane >> 3);
+    const int chunk = (lane & 7) ^ lds_swizzle(row);
+    a_off[j] = min(row0 + row, R - 1) * K + chunk * 8;
+    b_off[j] = min(col0 + row, N - 1) * K + chunk * 8;
+  }
+  const int nk = K / BK;
+  // load j of the token (A) / weight (B) tile kt; kt past the end re-fetches
+  // the last tile into a slot nobody reads any more
+  // The operand with two slots ("near", fetched one tile ahead) sits at LDS
+  // offset 0, the one with three slots ("far", two tiles ahead) behind it.
+  // DEEP_B: the weight tile is the far operand, else the token tile.
+  constexpr int FAR_BASE = 2 * Cfg::A_BYTES;
+  const bf16_t* near_g = DEEP_B ? Ae : Be;
+  const bf16_t* far_g = DEEP_B ? Be : Ae;
+  auto load_near = [&](int kt, int j) {
+    const int slot = kt & 1;
+    kt = min(kt, nk - 1);
+    __builtin_amdgcn_global_load_lds(
+        (glb_void_t*)(near_g + kt * BK + (DEEP_B ? a_off[j] : b_off[j])),
+        (lds_void_t*)(smem_raw + slot * Cfg::A_BYTES +
+                      (wave + Cfg::WAVES * j) * 1024), 16, 0, 0);
+  };
+  auto load_far = [&](int kt, int slot, int j) {
+    kt = min(kt, nk - 1);
+    __builtin_amdgcn_global_load_lds(
+        (glb_void_t*)(far_g + kt * BK + (DEEP_B ? b_off[j] : a_off[j])),
+        (lds_void_t*)(smem_raw + FAR_BASE + slot * Cfg::B_BYTES +
+                      (wave + Cfg::WAVES * j) * 1024), 16, 0, 0);
+  };
+
+  f32x16_t acc[Cfg::TM][Cfg::TN];
+#pragma unroll
+  for (int i = 0; i < Cfg::TM; ++i)
+#pragma unroll
+    for (int j = 0; j < Cfg::TN; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const int fr = lane & 31, fc = lane >> 5;
+  int a_frag[BK / 16], b_frag[BK / 16];
+#pragma unroll
+  for (int kk = 0; kk < BK / 16; ++kk) {
+    const int col = ((kk * 2 + fc) ^ lds_swizzle(fr)) * 16;
+    a_frag[kk] = (wm * Cfg::WTM + fr) * Cfg::ROW_BYTES + col;
+    b_frag[kk] = (wn * Cfg::WTN + fr) * Cfg::ROW_BYTES + col;
+  }
+  constexpr int KSTEPS = BK / 16;
+  bf16x8_t fa[2][Cfg::TM], fb[2][Cfg::TN];
+  // fragment read n of a step: 0..TM-1 token rows, TM..TM+TN-1 weight rows
+  auto read_frag = [&](int nslot, int fslot, int kk, int buf, int n) {
+    const int a_base = DEEP_B ? nslot * Cfg::A_BYTES : FAR_BASE + fslot * Cfg::A_BYTES;
+    const int b_base = DEEP_B ? FAR_BASE + fslot * Cfg::B_BYTES : nslot * Cfg::B_BYTES;
+    if (n < Cfg::TM)
+      fa[buf][n] = *reinterpret_cast<const bf16x8_t*>(
+          smem_raw + a_base + a_frag[kk] + n * 32 * Cfg::ROW_BYTES);
+    else
+      fb[buf][n - Cfg::TM] = *reinterpret_cast<const bf16x8_t*>(
+          smem_raw + b_base + b_frag[kk] + (n - Cfg::TM) * 32 * Cfg::ROW_BYTES);
+  };
+  auto mfma = [&](int buf, int n) {
+    const int i = n / Cfg::TN, j = n % Cfg::TN;
+    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][j], fa[buf][i],
+                                                        acc[i][j], 0, 0, 0);
+  };
+  // nothing moves across: the instruction order below is the issue order
+  auto fence = [&]() { __builtin_amdgcn_sched_barrier(0); };
+  // fragment reads in the order the MFMAs (token tile i = n / TN outer, weight
+  // tile j = n % TN inner) first need them: a0 b0 b1 a1 a2 a3
+  constexpr int RD[6] = {0, Cfg::TM, Cfg::TM + 1, 1, 2, 3};
+
+  // prologue: tile 0 (8 loads), weight tile 1 (4), token loads 0,1 of tile 1
+#pragma unroll
+  for (int j = 0; j < 4; ++j) load_near(0, j);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) load_far(0, 0, j);
+#pragma unroll
+  for (int j = 0; j < 4; ++j) load_far(1, 1, j);
+  load_near(1, 0);
+  load_near(1, 1);
+  wait_vmcnt<6>();
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+#pragma unroll
+  for (int n = 0; n < 6; ++n) read_frag(0, 0, 0, 0, n);
+
+  // bslot = kt % 3, kept incrementally
+  int bslot = 0;
+  auto k_tile = [&](int kt, auto last_tag) {
+    constexpr bool LAST = decltype(last_tag)::value;
+    const int aslot = kt & 1;
+    const int bnext = bslot == 2 ? 0 : bslot + 1;       // slot of tile kt+1
+    const int bnext2 = bnext == 2 ? 0 : bnext + 1;      // slot of tile kt+2
+#pragma unroll
+    for (int kk = 0; kk < KSTEPS; ++kk) {
+      const int cur = kk & 1, nxt = cur ^ 1;
+      auto load = [&](int which) {   // the two loads this step carries
+        if (LAST) return;
+        if (kk == 0) load_near(kt + 1, 2 + which);
+        if (kk == 1) load_far(kt + 2, bnext2, which);
+        if (kk == 2) load_far(kt + 2, bnext2, 2 + which);
+        if (kk == 3) load_near(kt + 2, which);
+      };
+      if (kk + 1 < KSTEPS) {
+        // 6 fragment reads of step kk+1 (in the order its MFMAs need them),
+        // 2 loads, 8 MFMAs of step kk
+        fence();
+        read_frag(aslot, bslot, kk + 1, nxt, RD[0]);
+        read_frag(aslot, bslot, kk + 1, nxt, RD[1]);
+        mfma(cur, 0); fence();
+        read_frag(aslot, bslot, kk + 1, nxt, RD[2]);
+        mfma(cur, 1); fence();
+        load(0);
+        mfma(cur, 2); fence();
+        read_frag(aslot, bslot, kk + 1, nxt, RD[3]);
+        mfma(cur, 3); fence();
+        read_frag(aslot, bslot, kk + 1, nxt, RD[4]);
+        mfma(cur, 4); fence();
+        load(1);
+        mfma(cur, 5); fence();
+        read_frag(aslot, bslot, kk + 1, nxt, RD[5]);
+        mfma(cur, 6); fence();
+        mfma(cur, 7); fence();
+      } else if (!LAST) {
+        // this lane holds the last step's fragments (lgkmcnt 0); everything
+        // but the four weight loads of tile kt+2 has landed (vmcnt 4)
+        fence();
+        __builtin_amdgcn_s_waitcnt((4 & 15) | (0 << 8) | (7 << 4));
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        fence();
+        load(0);
+        mfma(cur, 0); fence();
+        load(1);
+        mfma(cur, 1); fence();
+#pragma unroll
+        for (int n = 0; n < 6; ++n) {
+          read_frag(aslot ^ 1, bnext, 0, nxt, RD[n]);
+          mfma(cur, 2 + n); fence();
+        }
+      } else {
+#pragma unroll
+        for (int n = 0; n < 8; ++n) mfma(cur, n);
+      }
+    }
+    bslot = bnext;
+  };
+  for (int kt = 0; kt + 1 < nk; ++kt) k_tile(kt, std::false_type{});
+  k_tile(nk - 1, std::true_type{});
+  // the epilogue reuses the ring: no direct-to-LDS load may still be in flight
+  wait_vmcnt<0>();
+  __syncthreads();
+
+  bf16_t* Cs = reinterpret_cast<bf16_t*>(smem_raw);  // [BM][LDC]
+  const int m_l = lane & 31;
+  const int n_l = (lane >> 5) * 4;
+#pragma unroll
+  for (int i = 0; i < Cfg::TM; ++i) {
+#pragma unroll
+    for (int j = 0; j < Cfg::TN; ++j) {
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int row = wm * Cfg::WTM + i * 32 + m_l;
+        const int col = wn * Cfg::WTN + j * 32 + 8 * q + n_l;
+        uint2 v;
+        v.x = pack2_bf16(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], RELU);
+        v.y = pack2_bf16(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3], RELU);
+        *reinterpret_cast<uint2*>(Cs + row * Cfg::LDC + col) = v;
+      }
+    }
+  }
+  __syncthreads();
+  constexpr int CPR_C = BN / 8;
+#pragma unroll 4
+  for (int c = tid; c < BM * CPR_C; c += Cfg::THREADS) {
+    const int r = c / CPR_C, cc = (c % CPR_C) * 8;
+    const int grow = row0 + r, gcol = col0 + cc;
+    if (grow < R && gcol < N) {
+      const uint2* sp = reinterpret_cast<const uint2*>(Cs + r * Cfg::LDC + cc);
+      uint2 lo = sp[0], hi = sp[1];
+      *reinterpret_cast<uint4*>(Ce + (int64_t)grow * N + gcol) =
+          make_uint4(lo.x, lo.y, hi.x, hi.y);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Plain FMA tile kernel (float32, and bf16 shapes the MFMA kernel rejects):
 // 64 x 64 tile, 16-deep K step, each thread a 4 x 4 patch, float32 accumulate
 // in k order.
@@ -577,6 +831,29 @@ static int launch_dma(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
   return 0;
 }
 
+static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
+                       int R, int N, int K, bool relu, hipStream_t st) {
+  using Cfg = RingCfg;
+  const int tiles_m = (R + Cfg::BM - 1) / Cfg::BM;
+  const int tiles_n = (N + Cfg::BN - 1) / Cfg::BN;
+  const int64_t blocks = (int64_t)tiles_m * tiles_n * E;
+  MOE_REQUIRE(blocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
+              "expert_ffn: too many tiles (%lld)", (long long)blocks);
+  if (relu) {
+    auto k = grouped_gemm_bf16_ring_kernel<true, true>;
+    MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
+    k<<<(unsigned)blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(A, B, C, R, N, K,
+                                                              tiles_m, tiles_n);
+  } else {
+    auto k = grouped_gemm_bf16_ring_kernel<false, true>;
+    MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
+    k<<<(unsigned)blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(A, B, C, R, N, K,
+                                                              tiles_m, tiles_n);
+  }
+  MOE_CHECK_LAUNCH("expert_ffn (mfma, spread direct-to-LDS loads)");
+  return 0;
+}
+
 template <typename T>
 static int launch_simple(const T* A, const T* B, T* C, int E, int R, int N,
                          int K, bool relu, hipStream_t st) {
@@ -616,12 +893,12 @@ static int grouped_gemm(const void* A, const void* B, void* C, int E, int R,
       const bf16_t *a = (const bf16_t*)A, *b = (const bf16_t*)B;
       bf16_t* c = (bf16_t*)C;
       const int pad256 = (R + 255) / 256 * 256, pad128 = (R + 127) / 128 * 128;
-      // 256 x 256 tiles run 8 wavefronts (two per SIMD, 128 x 64 sub-tiles):
-      // measured ~2-3 % faster than 4 wavefronts with 128 x 128 sub-tiles
+      // 256 x 256 tiles run 8 wavefronts (two per SIMD, 128 x 64 sub-tiles)
+      // with the loads spread over the MFMA steps
       if (pad128 < pad256)
         rc = launch_dma<128, 256, 2>(a, b, c, E, R, N, K, relu, st);
       else
-        rc = launch_dma<256, 256, 4>(a, b, c, E, R, N, K, relu, st);
+        rc = launch_ring(a, b, c, E, R, N, K, relu, st);
     } else if (R >= 1024 && N >= 1024)
       rc = launch_mfma<256, 256, 64>((const bf16_t*)A, (const bf16_t*)B,
                                      (bf16_t*)C, E, R, N, K, relu, st);
