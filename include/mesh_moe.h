@@ -136,14 +136,21 @@ int mesh_moe_router_top2_gating(
  * Switch (top-1) gating from router logits: softmax, arg-max expert, raw
  * probability as the gate, per-group capacity positions with overflow drop,
  * load-balancing loss and (optionally) the router z-loss.
- * Replaces _switch_gating after the router projection for its deterministic
- * policies -- "argmax", and "input_dropout" / "input_jitter" outside training
- * (transformer/moe.py:1207-1306; z-loss :1253-1266).
+ * Replaces _switch_gating and _switch_max_gating after the router projection
+ * for their deterministic policies -- "argmax", and "input_dropout" /
+ * "input_jitter" outside training (transformer/moe.py:1207-1306, :976-1051;
+ * z-loss :1253-1266).
  * The per-token record has the layout of mesh_moe_top2_gating with the second
  * choice never kept (kept[..,1] = 0, gate[..,1] = 0), so mesh_moe_dispatch and
  * mesh_moe_combine apply unchanged.
  *   importance [G,S] of importance_dtype or NULL: only tokens with
  *               importance == 1 are routed (moe.py:1226-1231)
+ *   slots_by_gate  0: an expert's slots go to its choosers in token order,
+ *               overflow dropped (_switch_gating, moe.py:1268-1291);
+ *               1: to the `C` choosers with the largest gate, slot c holding
+ *               the (c+1)-th largest, equal gates in token order
+ *               (_switch_max_gating, transformer/moe.py:1033-1039, the top_k
+ *               of ops.py:4934-4942); pos then is that rank
  *   use_z_loss != 0 adds z_loss_coef * sum_t(logsumexp_t^2 * (imp_t == 1)) /
  *               (#(imp == 1) * num_microbatches); the caller passes it only
  *               when training with hparams.moe_z_loss set
@@ -153,7 +160,8 @@ int mesh_moe_router_top2_gating(
  */
 int mesh_moe_switch_gating(const float* logits, const void* importance,
                            int importance_dtype, int G, int S, int E, int C,
-                           int use_z_loss, double z_loss_coef,
+                           int slots_by_gate, int use_z_loss,
+                           double z_loss_coef,
                            int num_microbatches, int32_t* idx, int32_t* pos,
                            float* gate, uint8_t* kept, int32_t* fill,
                            float* loss, void* workspace,
@@ -167,10 +175,10 @@ int mesh_moe_switch_gating(const float* logits, const void* importance,
 int mesh_moe_router_switch_gating(
     const void* x, const void* w_packed, const float* bias, float* logits,
     int batch, int64_t tokens, int M, int dtype, const void* importance,
-    int importance_dtype, int G, int S, int E, int C, int use_z_loss,
-    double z_loss_coef, int num_microbatches, int32_t* idx, int32_t* pos,
-    float* gate, uint8_t* kept, int32_t* fill, float* loss, void* workspace,
-    size_t workspace_bytes, void* stream);
+    int importance_dtype, int G, int S, int E, int C, int slots_by_gate,
+    int use_z_loss, double z_loss_coef, int num_microbatches, int32_t* idx,
+    int32_t* pos, float* gate, uint8_t* kept, int32_t* fill, float* loss,
+    void* workspace, size_t workspace_bytes, void* stream);
 
 /*
  * Dispatch: expert_in[e,g,c,:] = x[g,s,:] for the token holding slot (e,g,c),

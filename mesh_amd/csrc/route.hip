@@ -219,6 +219,7 @@ struct GateParams {
   int has_importance;  // switch loss: the proxy is masked per token
   int use_z_loss;      // switch: add z_loss_coef * z_loss (moe.py:1253-1266)
   float z_loss_coef;
+  int rank_by_gate;    // switch_max: slots by descending gate (moe.py:1033-1039)
 };
 
 constexpr int ROUTER_TOP2 = 0;    // _top_2_gating, moe.py:1312-1513
@@ -527,6 +528,9 @@ __global__ __launch_bounds__(CAP_THREADS) void gate_capacity_kernel(
   int16_t* c1 = reinterpret_cast<int16_t*>(prod + 2 * el);  // [S]
   int16_t* c2 = c1 + S;                                      // [S]
   int16_t* c2l = c2 + S;                                     // [S] (loss only)
+  // first-choice gates of the group, for the by-gate slot order; float-aligned
+  // because 3 * S int16 may end on an odd 2-byte boundary
+  float* gl = reinterpret_cast<float*>(c2l + S + (S & 1));    // [S]
   const int g = blockIdx.x;
   const int tid = threadIdx.x;
   const int64_t base = (int64_t)g * S;
@@ -542,6 +546,7 @@ __global__ __launch_bounds__(CAP_THREADS) void gate_capacity_kernel(
     c2[s] = (k2 & 1) ? (int16_t)b : (int16_t)-1;
     if (sw) c2l[s] = (k1 & 2) ? (int16_t)a : (int16_t)-1;
     else if (loss2) c2l[s] = (k2 & 2) ? (int16_t)b : (int16_t)-1;
+    if (p.rank_by_gate) gl[s] = gate[t * 2];
   }
   __syncthreads();
   const int e = tid % el;
@@ -565,7 +570,8 @@ __global__ __launch_bounds__(CAP_THREADS) void gate_capacity_kernel(
       if (k < chunk) before += v;
     }
     int running = before + (round == 0 ? 0 : count1);
-    for (int s = s_begin; s < s_end; ++s) {
+    const bool in_token_order = !(p.rank_by_gate && round == 0);
+    for (int s = s_begin; in_token_order && s < s_end; ++s) {
       if (ch[s] == e) {
         int64_t t = base + s;
         const bool ok = running < C;
@@ -578,6 +584,27 @@ __global__ __launch_bounds__(CAP_THREADS) void gate_capacity_kernel(
     if (chunk == 0 && e < E) tot[round * el + e] = total;
     if (round == 0) count1 = min(total, C);
     __syncthreads();
+  }
+  if (p.rank_by_gate) {
+    // switch_max: expert e keeps its C choosers with the largest gate; slot =
+    // rank by (gate descending, token ascending), the order of tf.math.top_k
+    for (int s = tid; s < S; s += CAP_THREADS) {
+      const int ex = c1[s];
+      if (ex < 0) continue;
+      const float gs = gl[s];
+      int rank = 0;
+      for (int s2 = 0; s2 < S; ++s2) {
+        if (c1[s2] == ex) {
+          const float g2 = gl[s2];
+          rank += (g2 > gs || (g2 == gs && s2 < s)) ? 1 : 0;
+        }
+      }
+      const int64_t t = base + s;
+      const bool ok = rank < C;
+      pos[t * 2] = rank;
+      kept[t * 2] = ok ? 1 : 0;
+      if (!ok) gate[t * 2] = gs * 0.0f;
+    }
   }
   // tokens that did not compete: mask_k_flat = 0 -> gate_k * 0, kept = 0
   for (int s = tid; s < S; s += CAP_THREADS) {
@@ -758,7 +785,8 @@ static int launch_capacity_and_loss(const GateParams& p, int32_t* idx,
   while (el < p.E) el *= 2;
   size_t smem = sizeof(int32_t) * (CAP_THREADS + 3 * (size_t)el) +
                 sizeof(float) * 2 * (size_t)el +
-                sizeof(int16_t) * 3 * (size_t)p.S;
+                sizeof(int16_t) * (3 * (size_t)p.S + 1) +
+                (p.rank_by_gate ? sizeof(float) * (size_t)p.S : 0);
   MOE_ALLOW_LDS(gate_capacity_kernel, smem);
   gate_capacity_kernel<<<p.G, CAP_THREADS, smem, st>>>(
       p, idx, pos, gate, kept, fill, part1, part2, gsum, el);
@@ -811,19 +839,21 @@ static GateParams make_gate_params(int G, int S, int E, int C, int policy,
   p.has_importance = 0;
   p.use_z_loss = 0;
   p.z_loss_coef = 0.f;
+  p.rank_by_gate = 0;
   return p;
 }
 
 static GateParams make_switch_params(int G, int S, int E, int C,
-                                     const void* importance, int use_z_loss,
-                                     double z_loss_coef, int num_microbatches,
-                                     int tt) {
+                                     const void* importance, int slots_by_gate,
+                                     int use_z_loss, double z_loss_coef,
+                                     int num_microbatches, int tt) {
   GateParams p = make_gate_params(G, S, E, C, MESH_MOE_SECOND_NONE, 0.0, 0,
                                   num_microbatches, 0, tt);
   p.router = ROUTER_SWITCH;
   p.has_importance = importance != nullptr;
   p.use_z_loss = use_z_loss ? 1 : 0;
   p.z_loss_coef = (float)z_loss_coef;
+  p.rank_by_gate = slots_by_gate ? 1 : 0;
   return p;
 }
 
@@ -988,7 +1018,7 @@ extern "C" int mesh_moe_router_top2_gating(
 
 extern "C" int mesh_moe_switch_gating(
     const float* logits, const void* importance, int importance_dtype, int G,
-    int S, int E, int C, int use_z_loss, double z_loss_coef,
+    int S, int E, int C, int slots_by_gate, int use_z_loss, double z_loss_coef,
     int num_microbatches, int32_t* idx, int32_t* pos, float* gate,
     uint8_t* kept, int32_t* fill, float* loss, void* workspace,
     size_t workspace_bytes, void* stream) {
@@ -997,8 +1027,8 @@ extern "C" int mesh_moe_switch_gating(
   if (int rc = check_gating_args(G, S, E, C, MESH_MOE_SECOND_NONE, nullptr,
                                  importance, importance_dtype, workspace_bytes))
     return rc;
-  GateParams p = make_switch_params(G, S, E, C, importance, use_z_loss,
-                                    z_loss_coef, num_microbatches,
+  GateParams p = make_switch_params(G, S, E, C, importance, slots_by_gate,
+                                    use_z_loss, z_loss_coef, num_microbatches,
                                     gate_tokens_per_block(E));
   return run_gating(p, logits, importance, importance_dtype, nullptr, idx, pos,
                     gate, kept, fill, loss, workspace, (hipStream_t)stream);
@@ -1007,8 +1037,9 @@ extern "C" int mesh_moe_switch_gating(
 extern "C" int mesh_moe_router_switch_gating(
     const void* x, const void* w_packed, const float* bias, float* logits,
     int batch, int64_t tokens, int M, int dtype, const void* importance,
-    int importance_dtype, int G, int S, int E, int C, int use_z_loss,
-    double z_loss_coef, int num_microbatches, int32_t* idx, int32_t* pos,
+    int importance_dtype, int G, int S, int E, int C, int slots_by_gate,
+    int use_z_loss, double z_loss_coef, int num_microbatches, int32_t* idx,
+    int32_t* pos,
     float* gate, uint8_t* kept, int32_t* fill, float* loss, void* workspace,
     size_t workspace_bytes, void* stream) {
   MOE_REQUIRE(x && w_packed && idx && pos && gate && kept && fill && loss &&
@@ -1020,8 +1051,9 @@ extern "C" int mesh_moe_router_switch_gating(
   if (int rc = check_fused_router_args("router_switch_gating", x, w_packed,
                                        batch, tokens, M, dtype, G, S, E))
     return rc;
-  GateParams p = make_switch_params(G, S, E, C, importance, use_z_loss,
-                                    z_loss_coef, num_microbatches, 128);
+  GateParams p = make_switch_params(G, S, E, C, importance, slots_by_gate,
+                                    use_z_loss, z_loss_coef, num_microbatches,
+                                    128);
   return run_router_gating(p, x, w_packed, bias, logits, tokens, M, importance,
                            importance_dtype, nullptr, idx, pos, gate, kept,
                            fill, loss, workspace, (hipStream_t)stream);

@@ -46,14 +46,15 @@ _SIGNATURES = {
         _vp, _vp, ctypes.c_size_t, _vp]),
     "mesh_moe_switch_gating": (ctypes.c_int, [
         _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
-        ctypes.c_int, ctypes.c_int, ctypes.c_double, ctypes.c_int, _vp, _vp,
-        _vp, _vp, _vp, _vp, _vp, ctypes.c_size_t, _vp]),
-    "mesh_moe_router_switch_gating": (ctypes.c_int, [
-        _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
-        ctypes.c_int, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_double,
         ctypes.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_size_t,
         _vp]),
+    "mesh_moe_router_switch_gating": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
+        ctypes.c_int, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_double, ctypes.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+        ctypes.c_size_t, _vp]),
     "mesh_moe_dispatch": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
@@ -336,11 +337,13 @@ def _routing_buffers(lib, g, s, e, dev):
 
 
 def switch_gating(logits, capacity, importance=None, z_loss=None,
-                  num_microbatches=None):
+                  num_microbatches=None, slots_by_gate=False):
   """logits float32 [G, S, E] -> Routing for switch (top-1) gating.
 
   z_loss: coefficient of the router z-loss, or None to leave it out (the
-  caller passes it only when training, transformer/moe.py:1253)."""
+  caller passes it only when training, transformer/moe.py:1253).
+  slots_by_gate: an expert keeps its choosers with the largest gate instead of
+  the earliest ones (_switch_max_gating, transformer/moe.py:1033-1039)."""
   lib = load_library()
   g, s, e = logits.shape
   lp = _dev(logits, "logits", torch.float32)
@@ -352,8 +355,9 @@ def switch_gating(logits, capacity, importance=None, z_loss=None,
       lib, g, s, e, logits.device)
   with _stage("switch_gating"):
     _check(lib.mesh_moe_switch_gating(
-        lp, ip, icode, g, s, e, int(capacity), int(z_loss is not None),
-        float(z_loss or 0.0), int(num_microbatches or 1), idx.data_ptr(),
+        lp, ip, icode, g, s, e, int(capacity), int(bool(slots_by_gate)),
+        int(z_loss is not None), float(z_loss or 0.0),
+        int(num_microbatches or 1), idx.data_ptr(),
         pos.data_ptr(), gate.data_ptr(), kept.data_ptr(), fill.data_ptr(),
         loss.data_ptr(), ws.data_ptr(), ws_bytes, _stream()), "switch_gating")
   r = Routing(idx, pos, gate, kept, fill, loss, int(capacity), e)
@@ -364,7 +368,7 @@ def switch_gating(logits, capacity, importance=None, z_loss=None,
 
 def router_switch_gating(x, w_packed, group_size, capacity, importance=None,
                          z_loss=None, num_microbatches=None, bias=None,
-                         want_logits=False):
+                         want_logits=False, slots_by_gate=False):
   """Router projection + switch gating in one launch sequence; arguments as
   router_top2_gating / switch_gating."""
   lib = load_library()
@@ -391,8 +395,9 @@ def router_switch_gating(x, w_packed, group_size, capacity, importance=None,
   with _stage("router_switch_gating"):
     _check(lib.mesh_moe_router_switch_gating(
         xp, wp, bp, None if logits is None else logits.data_ptr(), b, t, m,
-        BF16, ip, icode, g, s, e, int(capacity), int(z_loss is not None),
-        float(z_loss or 0.0), int(num_microbatches or 1), idx.data_ptr(),
+        BF16, ip, icode, g, s, e, int(capacity), int(bool(slots_by_gate)),
+        int(z_loss is not None), float(z_loss or 0.0),
+        int(num_microbatches or 1), idx.data_ptr(),
         pos.data_ptr(), gate.data_ptr(), kept.data_ptr(), fill.data_ptr(),
         loss.data_ptr(), ws.data_ptr(), ws_bytes, _stream()),
         "router_switch_gating")

@@ -21,7 +21,7 @@ from mesh_amd import layers as mtf_layers
 from mesh_amd import moe_hip
 from mesh_amd import ops as mtf
 
-_OTHER_GATINGS = ("ntlb", "switch_max", "expert_selection")
+_OTHER_GATINGS = ("ntlb", "expert_selection")
 
 
 class HParams(object):
@@ -89,11 +89,11 @@ def _activation_name(activation):
 
 
 def _check_gating(hparams):
-  if hparams.moe_gating in ("top_2", "switch"):
+  if hparams.moe_gating in ("top_2", "switch", "switch_max"):
     return
   if hparams.moe_gating in _OTHER_GATINGS:
     raise NotImplementedError(
-        "moe_gating=%s is not implemented (top_2 and switch only)"
+        "moe_gating=%s is not implemented (top_2, switch and switch_max only)"
         % hparams.moe_gating)
   raise ValueError("unknown hparams.moe_gating=%s" % hparams.moe_gating)
 
@@ -156,12 +156,13 @@ class _GatingSpec(object):
 
 
 class _SwitchGatingSpec(object):
-  """Static configuration of one _switch_gating call (moe.py:1176-1309) for
-  its deterministic policies: "argmax", and "input_dropout" / "input_jitter"
-  when not training, where the reference applies no perturbation
-  (moe.py:1192-1199)."""
+  """Static configuration of one _switch_gating (moe.py:1176-1309) or
+  _switch_max_gating (moe.py:943-1054) call for the deterministic policies:
+  "argmax", and "input_dropout" / "input_jitter" when not training, where the
+  reference applies no perturbation (moe.py:1192-1199)."""
 
   def __init__(self, hparams, train, num_microbatches, has_importance):
+    self.slots_by_gate = hparams.moe_gating == "switch_max"
     policy = (hparams.moe_switch_policy_train if train
               else hparams.moe_switch_policy_eval)
     if policy == "sample" or (train and policy in ("input_dropout",
@@ -171,8 +172,9 @@ class _SwitchGatingSpec(object):
           % (policy, "training" if train else "sampling"))
     if policy not in ("argmax", "input_dropout", "input_jitter"):
       raise ValueError("Unknown Switch gating policy %s" % policy)
-    self.z_loss = None
-    if train and getattr(hparams, "moe_z_loss", None) is not None:
+    self.z_loss = None                     # _switch_max_gating has no z-loss
+    if (train and not self.slots_by_gate and
+        getattr(hparams, "moe_z_loss", None) is not None):
       # the reference evaluates equal(importance, 1.0) and
       # denom * num_microbatches unconditionally (moe.py:1260-1264)
       if not has_importance or not num_microbatches:
@@ -189,12 +191,14 @@ class _SwitchGatingSpec(object):
     if moe_hip.fused_gating_supported(x, num_experts, group_size):
       return moe_hip.router_switch_gating(
           x, w_packed, group_size, capacity, importance=importance,
-          z_loss=self.z_loss, num_microbatches=self.num_microbatches)
+          z_loss=self.z_loss, num_microbatches=self.num_microbatches,
+          slots_by_gate=self.slots_by_gate)
     logits = moe_hip.router_logits(x, w, w_packed=w_packed)
     return moe_hip.switch_gating(
         logits.reshape(groups, group_size, num_experts), capacity,
         importance=importance, z_loss=self.z_loss,
-        num_microbatches=self.num_microbatches)
+        num_microbatches=self.num_microbatches,
+        slots_by_gate=self.slots_by_gate)
 
 
 def _packed(lowering, kernel_tensor, dtype):
@@ -326,10 +330,10 @@ def transformer_moe_layer_v1(
                               "implemented (moe_dropout_rate must be 0)")
   if hparams.moe_use_experts_attention:
     raise NotImplementedError("moe_use_experts_attention is not implemented")
-  if hparams.moe_gating == "switch":
+  if hparams.moe_gating in ("switch", "switch_max"):
     gating = _SwitchGatingSpec(hparams, train, num_microbatches,
                                nonpadding is not None)
-    router_name = "switch_gating"                       # moe.py:1179
+    router_name = hparams.moe_gating + "_gating"        # moe.py:1178, :945
   else:
     gating = _GatingSpec(hparams, train, num_microbatches)
     router_name = "top_2_gating"                        # moe.py:1314

@@ -26,6 +26,10 @@ MoE file, and its TensorFlow dependency cannot run here):
                                       the loss (balanced: = fraction of tokens
                                       with importance 1) and the z-loss
                                       (constant logits c: (c + log E)^2 / mb)
+  switch_max_gating                   repeated arg-max selection (the k < 5
+                                      lowering of mtf.top_k) vs the stable
+                                      sort, per-expert brute force, equality
+                                      with switch_gating when nothing overflows
   v2                                  x=1 outer expert reduces to v1
 
 PARITY UNPINNED against TensorFlow itself (only running the reference could
@@ -363,6 +367,86 @@ def switch_gating(logits, capacity, importance=None, train=False, z_loss=None,
   return out
 
 
+# ----------------------------------------------------------------------------
+# _switch_max_gating  (transformer/moe.py:943-1054)
+# ----------------------------------------------------------------------------
+def top_k_lowest_index_first(x, k, axis):
+  """tf.math.top_k along `axis` as mtf.top_k lowers it (ops.py:4934-4942; for
+  1 < k < 5 mtf uses repeated top_1 with the taken entries pushed to -1e9,
+  ops.py:4988-5017, which selects the same entries): the k largest values in
+  descending order, equal values in ascending index order (the documented
+  tie rule of tf.math.top_k).  Returns (values, indices) with k last."""
+  x = np.moveaxis(np.asarray(x), axis, -1)
+  order = np.argsort(-x, axis=-1, kind="stable")[..., :k].astype(np.int32)
+  return np.take_along_axis(x, order, -1), order
+
+
+def switch_max_gating(logits, capacity, importance=None,
+                      num_microbatches=None, act_dtype="float32", dense=False):
+  """Everything in _switch_max_gating after the router projection, for the
+  deterministic policies (as switch_gating).
+
+  Choice, gate and loss are those of _switch_gating (no z-loss here); the
+  slots differ: expert e keeps, per group, the `capacity` tokens that chose it
+  with the LARGEST gate, slot c holding the (c+1)-th largest
+  (top_k over the group dim of expert_mask * expert_gate, moe.py:1033-1039).
+  A slot whose selected value is 0 (fewer choosers than slots) combines with
+  weight 0 and is therefore not dispatched.  Same result dict as
+  switch_gating; pos_1 is the slot, meaningful where kept_1.
+  """
+  logits = np.asarray(logits, dtype=F32)
+  g_, s_, e_ = logits.shape
+  raw_gates = softmax(logits)                                    # :976
+  expert_gate, expert_index = top_1(raw_gates)                   # :979
+  expert_mask = one_hot(expert_index, e_)                        # :990
+  inv_s = F32(1.0 / s_)
+  density_1 = seq_sum(expert_mask, axis=-2) * inv_s              # :994
+  density_1_proxy = seq_sum(raw_gates, axis=-2) * inv_s          # :995
+  if importance is not None:                                     # :996-1000
+    importance = np.asarray(importance, dtype=F32)
+    is_one = (importance == F32(1.0)).astype(F32)
+    expert_mask = expert_mask * is_one[..., None]
+    expert_gate = expert_gate * is_one
+    density_1_proxy = density_1_proxy[:, :, None] * is_one[:, None, :]
+    prod = density_1_proxy * density_1[:, :, None]
+    total = F32(prod.sum(dtype=np.float64))    # see switch_gating
+  else:
+    prod = density_1_proxy * density_1
+    total = seq_sum(prod.reshape(-1))
+  loss = total * F32(1.0 / prod.size)
+  loss = loss * F32(float(e_ * e_))                              # :1001-1003
+  if num_microbatches and num_microbatches > 1:
+    loss = loss * F32(1.0 / num_microbatches)
+
+  expert_masked_probs = expert_mask * expert_gate[..., None]     # :1033 [G,S,E]
+  probs, tokens = top_k_lowest_index_first(expert_masked_probs, capacity, 1)
+  # probs, tokens: [G, E, C]
+  kept = np.zeros((g_, s_), bool)
+  pos_1 = np.zeros((g_, s_), np.int32)
+  gate_1 = np.zeros((g_, s_), F32)
+  fill = np.zeros((g_, e_), np.int32)
+  for g in range(g_):
+    for e in range(e_):
+      for c in range(capacity):
+        if probs[g, e, c] > 0:
+          t = tokens[g, e, c]
+          kept[g, t], pos_1[g, t], gate_1[g, t] = True, c, probs[g, e, c]
+          fill[g, e] += 1
+  zeros_i = np.zeros_like(expert_index)
+  out = dict(
+      index_1=expert_index, index_2=zeros_i, pos_1=pos_1, pos_2=zeros_i,
+      kept_1=kept, kept_2=np.zeros((g_, s_), bool),
+      gate_1=gate_1, gate_2=np.zeros((g_, s_), F32), fill=fill,
+      loss=cast_act(loss, act_dtype)[()])                        # :1049
+  if dense:
+    dispatch = one_hot(tokens, s_)                               # [G,E,C,S]
+    combine = dispatch * probs[..., None]                        # :1038-1039
+    combine = cast_act(combine.transpose(0, 3, 1, 2), act_dtype)  # [G,S,E,C]
+    out["combine"] = combine
+    out["dispatch"] = (combine != 0).astype(F32)                 # :1050-1051
+  return out
+
+
 def routing_sequential(index_1, index_2, sel_1, sel_2, num_experts, capacity):
   """Integer brute force for moe.py:1472-1496, one token at a time.
 
@@ -543,7 +627,7 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
 
   Returns (output [batch..., length, N], loss scalar, aux dict).
   """
-  if hp.moe_gating not in ("top_2", "switch"):
+  if hp.moe_gating not in ("top_2", "switch", "switch_max"):
     raise ValueError("unknown hparams.moe_gating=%s" % hp.moe_gating)
   x = cast_act(x, act_dtype)
   lead = x.shape[:-1]
@@ -562,14 +646,18 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
   logits = router_logits(xg, wg)
   if logit_bias is not None:
     logits = logits + np.asarray(logit_bias, F32)
-  if hp.moe_gating == "switch":                                  # :393-402
+  if hp.moe_gating in ("switch", "switch_max"):                  # :393-424
     sw = hp.moe_switch_policy_train if train else hp.moe_switch_policy_eval
     if sw == "sample" or (train and sw in ("input_dropout", "input_jitter")):
       raise NotImplementedError("switch policy %r draws random numbers" % sw)
     if sw not in ("argmax", "input_dropout", "input_jitter"):
       raise ValueError("Unknown Switch gating policy %s" % sw)
-    r = switch_gating(logits, c_, importance, train, hp.moe_z_loss,
-                      num_microbatches, act_dtype, dense=dense)
+    if hp.moe_gating == "switch":
+      r = switch_gating(logits, c_, importance, train, hp.moe_z_loss,
+                        num_microbatches, act_dtype, dense=dense)
+    else:
+      r = switch_max_gating(logits, c_, importance, num_microbatches,
+                            act_dtype, dense=dense)
   else:
     policy, threshold = _policy(hp, train)
     r = top_2_gating(logits, c_, importance, policy, threshold,

@@ -46,7 +46,8 @@ def run_v1(x, weights, hp, train, act_dtype, nonpadding=None, activation="relu",
     y, loss = moe.transformer_moe_layer_v1(
         xt, mtf.Dimension("d_model", n), hp, train, vdt, nonpadding=npad,
         activation=activation, num_microbatches=num_microbatches)
-  router = "switch_gating" if hp.moe_gating == "switch" else "top_2_gating"
+  router = {"switch": "switch_gating", "switch_max": "switch_max_gating"}.get(
+      hp.moe_gating, "top_2_gating")
   init = {"moe/%s/kernel" % router: weights["w_gate"],
           "moe/wi/kernel": weights["wi"], "moe/wo/kernel": weights["wo"]}
   lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()}, initial_values=init)
@@ -321,3 +322,36 @@ def test_v1_switch_rejections():
   hp, _ = make_hparams(**dict(base, **dict(SWITCH_HP, moe_z_loss=1e-3)))
   with pytest.raises(ValueError, match="moe_z_loss needs"):
     run_v1(x, w, hp, True, "float32")
+
+
+def test_v1_switch_max_matches_oracle():
+  """switch_max end to end.  Which tokens an over-subscribed expert keeps
+  depends on gates that the two implementations compute with different exp
+  routines: the seed is chosen so that no expert's C-th and (C+1)-th gate are
+  within 1e-5 of each other (checked on the oracle's values)."""
+  b, l, m, hdim, e, group = 2, 128, 32, 64, 4, 64
+  for seed in range(303, 323):
+    rng = np.random.default_rng(seed)
+    w = dict(w_gate=H.normal_weights(rng, (m, e), m),
+             wi=H.normal_weights(rng, (e, m, hdim), m),
+             wo=H.normal_weights(rng, (e, hdim, m), hdim))
+    x = H.safe_tokens(rng, b * l, m, w["w_gate"], "float32").reshape(b, l, m)
+    hp, ohp = make_hparams(moe_num_experts=e, moe_hidden_size=hdim,
+                           moe_group_size=group, moe_capacity_factor_eval=0.75,
+                           **dict(SWITCH_HP, moe_gating="switch_max"))
+    want, want_loss, aux = O.moe_layer_v1(x, w["w_gate"], w["wi"], w["wo"], ohp,
+                                          False, "float32")
+    p = O.softmax(aux["logits"]).max(-1)
+    gaps_ok = True
+    for gi in range(aux["num_groups"]):
+      for ex in range(e):
+        v = -np.sort(-p[gi][aux["index_1"][gi] == ex])
+        c = aux["capacity"]
+        if len(v) > c and (v[c - 1] - v[c]) < 1e-5:
+          gaps_ok = False
+    if gaps_ok:
+      break
+  assert gaps_ok and not aux["kept_1"].all()
+  got, got_loss, _, _ = run_v1(x, w, hp, False, "float32")
+  np.testing.assert_allclose(got, want, **H.value_tolerance("float32"))
+  np.testing.assert_allclose(got_loss, want_loss, rtol=1e-4)

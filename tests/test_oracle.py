@@ -450,6 +450,84 @@ def test_v1_switch_dense_equals_index_form():
     O.moe_layer_v1(x, wg, wi, wo, hp, False)
 
 
+# ---- switch_max gating ----------------------------------------------------------
+def test_top_k_matches_iterative_top_1():
+  """mtf.top_k lowers 1 < k < 5 as repeated top_1 with the taken entries pushed
+  down by 1e9 (ops.py:4988-5017) and other k as tf.math.top_k (lower index first
+  on ties): both select what the stable descending sort selects."""
+  rng = np.random.default_rng(51)
+  x = np.round(rng.random((3, 40, 5)) * 6) / 6        # many exact ties
+  x = x.astype(np.float32)
+  for k in (1, 2, 4, 7):
+    vals, idx = O.top_k_lowest_index_first(x, k, axis=1)      # over the 40
+    y = x.copy()
+    for i in range(k):
+      m = y.max(axis=1)
+      am = y.argmax(axis=1)                                    # first max
+      np.testing.assert_array_equal(idx[..., i], am)
+      np.testing.assert_array_equal(vals[..., i], np.take_along_axis(x, am[:, None, :], 1)[:, 0, :])
+      np.put_along_axis(y, am[:, None, :], -1e9, axis=1)
+      del m
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_switch_max_brute_force(seed):
+  """Per (group, expert): the tokens that chose the expert, sorted by gate
+  descending (token order on ties), fill slots 0..C-1; the rest are dropped."""
+  rng = np.random.default_rng(400 + seed)
+  g, s, e = 2, int(rng.integers(6, 80)), int(rng.integers(2, 7))
+  c = int(rng.integers(1, s // e + 3))
+  scale = 0.0 if seed == 3 else 1.0                    # seed 3: all gates tie
+  logits = (rng.standard_normal((g, s, e)) * scale).astype(np.float32)
+  imp = None
+  if seed % 2:
+    imp = rng.choice(np.array([0.0, 0.5, 1.0], np.float32), size=(g, s))
+  p = O.softmax(logits)
+  for dense in (False, True):
+    r = O.switch_max_gating(logits, c, importance=imp, dense=dense)
+    np.testing.assert_array_equal(r["index_1"], p.argmax(-1))
+    for gi in range(g):
+      for ex in range(e):
+        chose = [t for t in range(s) if r["index_1"][gi, t] == ex and
+                 (imp is None or imp[gi, t] == 1.0)]
+        chose.sort(key=lambda t: (-p[gi, t, ex], t))
+        for rank, t in enumerate(chose):
+          assert r["kept_1"][gi, t] == (rank < c)
+          if rank < c:
+            assert r["pos_1"][gi, t] == rank
+            assert r["gate_1"][gi, t] == p[gi, t, ex]
+          else:
+            assert r["gate_1"][gi, t] == 0
+        assert r["fill"][gi, ex] == min(len(chose), c)
+    if imp is not None:
+      assert not r["kept_1"][imp != 1.0].any()
+    if dense:
+      want = np.zeros((g, s, e, c), np.float32)
+      kk = r["kept_1"]
+      for gi, t in zip(*np.nonzero(kk)):
+        want[gi, t, r["index_1"][gi, t], r["pos_1"][gi, t]] = r["gate_1"][gi, t]
+      np.testing.assert_array_equal(r["combine"], want)
+      np.testing.assert_array_equal(r["dispatch"], (want != 0).astype(np.float32))
+
+
+def test_switch_max_equals_switch_without_overflow():
+  """With room for every token the two routers keep the same tokens with the
+  same gates and the same loss; only the slot order differs."""
+  rng = np.random.default_rng(52)
+  logits = rng.standard_normal((2, 50, 4)).astype(np.float32)
+  a = O.switch_gating(logits, 50)
+  b = O.switch_max_gating(logits, 50)
+  for k in ("index_1", "kept_1", "fill"):
+    np.testing.assert_array_equal(a[k], b[k])
+  np.testing.assert_array_equal(a["gate_1"], b["gate_1"])
+  assert a["loss"] == b["loss"]
+  # under overflow switch_max keeps the confident tokens, switch the early ones
+  c = 5
+  a, b = O.switch_gating(logits, c), O.switch_max_gating(logits, c)
+  np.testing.assert_array_equal(a["fill"], b["fill"])
+  assert b["gate_1"].sum() > a["gate_1"].sum()
+
+
 # ---- the layers ----------------------------------------------------------------
 def _hp(**kw):
   base = dict(moe_second_policy_train="all", moe_second_policy_eval="all")
