@@ -571,3 +571,37 @@ def test_router_switch_max_fused(hip):
         assert p[gi][kept, ex].min() >= p[gi][mine & ~kept, ex].max() * (1 - 1e-6)
       order = np.argsort(got["pos_1"][gi][kept])
       assert (np.diff(got["gate_1"][gi][kept][order]) <= 0).all()
+
+
+# ---- expert FFN at the full benchmark sizes ---------------------------------------
+@pytest.mark.parametrize("size", [(64, 512, 1024, 4096), (64, 2048, 4096, 16384)],
+                         ids=["cfg3", "cfg4"])
+def test_full_size_expert_ffn_properties(hip, size):
+  """(E, rows per expert, M, H) of configurations 3 and 4.  The oracle is too
+  slow here: row blocks sampled from the first, a middle and the last expert
+  are checked against float32 matmuls of the same bf16 operands (tile mapping,
+  K loop, epilogue at the real grid size), and two exact properties hold on the
+  whole output: scaling the tokens by 2 scales the output by 2 bit for bit,
+  and an expert whose token rows are zero outputs zeros."""
+  e, r, m, hdim = size
+  gen = torch.Generator(device="cuda")
+  gen.manual_seed(17)
+  x = torch.randn((e, r, m), generator=gen, device="cuda").to(torch.bfloat16)
+  wi = torch.empty((e, hdim, m), dtype=torch.bfloat16, device="cuda")
+  wo = torch.empty((e, m, hdim), dtype=torch.bfloat16, device="cuda")
+  for i in range(e):                         # packed layout [E, N, K] directly
+    wi[i] = (torch.randn((hdim, m), generator=gen, device="cuda") / m ** 0.5).to(torch.bfloat16)
+    wo[i] = (torch.randn((m, hdim), generator=gen, device="cuda") / hdim ** 0.5).to(torch.bfloat16)
+  x[e // 2 + 1].zero_()
+  y = hip.expert_ffn(x, wi, wo, "relu")
+  assert bool(torch.isfinite(y.float()).all())
+  for ei, r0 in ((0, 0), (e // 2, r // 2 - 37), (e - 1, r - 64), (e - 1, 0)):
+    xs = x[ei, r0:r0 + 64].float()
+    h_ref = torch.relu(xs @ wi[ei].float().t()).to(torch.bfloat16).float()
+    y_ref = h_ref @ wo[ei].float().t()
+    err = (y[ei, r0:r0 + 64].float() - y_ref).abs().max().item()
+    scale = y_ref.abs().max().item()
+    assert err <= 2e-2 * scale, (ei, r0, err, scale)
+  assert not bool(y[e // 2 + 1].any())
+  y2 = hip.expert_ffn(x * 2, wi, wo, "relu")
+  assert torch.equal(y2, y * 2)
