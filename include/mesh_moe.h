@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 2
+#define MESH_MOE_ABI_VERSION 3
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -235,6 +235,110 @@ int mesh_moe_expert_ffn(const void* expert_in, const void* wi_packed,
 int mesh_moe_combine(const void* y, const int32_t* idx, const int32_t* pos,
                      const float* gate, const uint8_t* kept, void* out, int G,
                      int S, int E, int C, int N, int dtype, void* stream);
+
+/*
+ * ---------------------------------------------------------------------------
+ * Backward.  The reference has no hand-written backward for the layer:
+ * mtf.gradients (mesh_tensorflow/ops.py:5254-5291) assembles it from the
+ * gradients of the einsums and element-wise ops the layer is built from
+ * (EinsumOperation.gradient ops.py:2846-2854, TopKOperation.gradient
+ * ops.py:4916-4920, softmax ops.py:5493-5541).  The entry points below are
+ * those einsum gradients with the one-hot tensors replaced by the routing
+ * record.  Gradient tensors have the activation dtype; the gating runs in
+ * float32 as in the forward pass.  Order of calls for one layer:
+ * combine_backward, expert_ffn_backward, gating_backward,
+ * router_backward_weights, dispatch_backward.
+ * ---------------------------------------------------------------------------
+ */
+
+/*
+ * Backward of the combine einsum (transformer/moe.py:509-510):
+ *   dy[e,g,c,:]  = w * dout[g,s,:] for the token in slot (e,g,c), zero rows for
+ *                  empty slots (w = its activation-dtype combine weight)
+ *   dgate[g,s,k] = <dout[g,s,:], y[idx_k,g,pos_k,:]>, 0 where not kept
+ *   dout [G,S,N] dtype; y, dy [E,G,C,N] dtype; dgate [G,S,2] float32
+ */
+int mesh_moe_combine_backward(const void* dout, const void* y,
+                              const int32_t* idx, const int32_t* pos,
+                              const float* gate, const uint8_t* kept,
+                              const int32_t* fill, void* dy, float* dgate,
+                              int G, int S, int E, int C, int N, int dtype,
+                              void* stream);
+
+/* Bytes of scratch mesh_moe_expert_ffn_backward needs. */
+size_t mesh_moe_expert_ffn_backward_workspace_bytes(int E, int R, int M, int H,
+                                                    int N, int dtype);
+
+/*
+ * Backward of the two expert einsums (transformer/moe.py:469-486), ReLU or
+ * linear experts:
+ *   dh = (dy . wo^T) * (h > 0);  dwo = h^T . dy
+ *   dexpert_in = dh . wi^T;      dwi = expert_in^T . dh
+ *   expert_in [E,R,M], h [E,R,H] (as mesh_moe_expert_ffn left it), dy [E,R,N]
+ *   wi [E,M,H], wo [E,H,N]: the variables' own layout (NOT the packed one)
+ *   dexpert_in [E,R,M]; dwi [E,M,H]; dwo [E,H,N]; everything of `dtype`
+ * Four grouped GEMMs on the forward kernels plus four transposes.
+ */
+int mesh_moe_expert_ffn_backward(const void* expert_in, const void* h,
+                                 const void* dy, const void* wi,
+                                 const void* wo, void* dexpert_in, void* dwi,
+                                 void* dwo, int E, int R, int M, int H, int N,
+                                 int activation, int dtype, void* workspace,
+                                 size_t workspace_bytes, void* stream);
+
+/* Bytes of scratch mesh_moe_gating_backward needs. */
+size_t mesh_moe_gating_backward_workspace_bytes(int G, int E);
+
+/*
+ * Backward of the gating (transformer/moe.py:1391-1496 for router 0 = top-2,
+ * :1207-1306 for router 1 = switch / switch_max): d(logits) from the
+ * gradients of the two combine weights and of the layer's returned loss.
+ *   logits [G,S,E] float32 (the forward values), importance as in the forward
+ *   idx, kept [G,S,2] from the forward; dgate [G,S,2] float32 from
+ *   mesh_moe_combine_backward
+ *   d_loss [1] float32 ON THE DEVICE: gradient w.r.t. the returned loss
+ *   (balancing loss * moe_loss_coef); loss_scale = moe_loss_coef
+ *   use_z_loss / z_loss_coef / num_microbatches as in the forward call
+ *   dlogits [G,S,E] float32
+ * The second-place loss (moe_use_second_place_loss) is not covered.
+ */
+int mesh_moe_gating_backward(const float* logits, const void* importance,
+                             int importance_dtype, const int32_t* idx,
+                             const uint8_t* kept, const float* dgate,
+                             const float* d_loss, double loss_scale, int G,
+                             int S, int E, int router, int use_z_loss,
+                             double z_loss_coef, int num_microbatches,
+                             float* dlogits, void* workspace,
+                             size_t workspace_bytes, void* stream);
+
+/*
+ * Backward of the router projection w.r.t. its kernel
+ * (transformer/moe.py:1384-1390): dw_gate[m,e] = sum_t float(x[t,m]) *
+ * dlogits[t,e], float32 accumulate, stored in dtype.
+ *   x [tokens,M] dtype; dlogits [tokens,E] float32; dw_gate [M,E] dtype
+ *   workspace: M*E float32
+ */
+int mesh_moe_router_backward_weights(const void* x, const float* dlogits,
+                                     void* dw_gate, float* workspace,
+                                     int64_t tokens, int M, int E, int dtype,
+                                     void* stream);
+
+/*
+ * Backward of the dispatch einsum (transformer/moe.py:443-447) plus, when
+ * dlogits is given, of the router projection w.r.t. the tokens:
+ *   dx[g,s,:] = sum over the dispatched choices k of dexpert_in[idx_k,g,pos_k,:]
+ *               + dlogits[g,s,:] . w_gate^T
+ * float32 accumulate, one rounding.  The dispatch tensor itself carries no
+ * gradient (it is a bool cast, moe.py:1510-1511).
+ *   dexpert_in [E,G,C,M] dtype; dlogits [G,S,E] float32 or NULL;
+ *   w_gate_packed [E,M] dtype (NULL iff dlogits is); dx [G,S,M] dtype
+ */
+int mesh_moe_dispatch_backward(const void* dexpert_in, const int32_t* idx,
+                               const int32_t* pos, const float* gate,
+                               const uint8_t* kept, const float* dlogits,
+                               const void* w_gate_packed, void* dx, int G,
+                               int S, int E, int C, int M, int dtype,
+                               void* stream);
 
 #ifdef __cplusplus
 }

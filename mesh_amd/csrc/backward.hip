@@ -1,0 +1,567 @@
+// Backward of the Mixture-of-Experts layer for gfx950: the token-side kernels.
+//
+// The reference has no backward code of its own for the layer: mtf.gradients
+// (mesh_tensorflow/ops.py:5254-5291) assembles it from the gradients of the
+// einsums and element-wise ops the layer is built from
+// (EinsumOperation.gradient ops.py:2846-2854, TopKOperation.gradient
+// ops.py:4916-4920, softmax ops.py:5493-5541).  With the one-hot
+// dispatch / combine tensors of transformer/moe.py:1499-1511 replaced by the
+// per-token routing record, those einsum gradients become the gathers and
+// scatters below.  The expert feed-forward backward (four grouped GEMMs) lives
+// next to the forward GEMM.
+#include "common.h"
+
+namespace mesh_moe {
+
+constexpr int BW_ROWS_PER_BLOCK = 4;  // one wavefront per row, 256 threads
+
+template <typename T>
+struct Vec16B {
+  static constexpr int N = 16 / sizeof(T);
+};
+
+__device__ __forceinline__ void unpack16(const uint4& v, float (&f)[4], float) {
+  f[0] = __uint_as_float(v.x); f[1] = __uint_as_float(v.y);
+  f[2] = __uint_as_float(v.z); f[3] = __uint_as_float(v.w);
+}
+__device__ __forceinline__ void unpack16(const uint4& v, float (&f)[8], bf16_t) {
+  f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
+  f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
+  f[4] = __uint_as_float(v.z << 16); f[5] = __uint_as_float(v.z & 0xffff0000u);
+  f[6] = __uint_as_float(v.w << 16); f[7] = __uint_as_float(v.w & 0xffff0000u);
+}
+__device__ __forceinline__ uint4 pack16(const float (&f)[4], float) {
+  return make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]),
+                    __float_as_uint(f[2]), __float_as_uint(f[3]));
+}
+__device__ __forceinline__ uint4 pack16(const float (&f)[8], bf16_t) {
+  uint4 r;
+  r.x = (uint32_t)f32_to_bf16(f[0]) | ((uint32_t)f32_to_bf16(f[1]) << 16);
+  r.y = (uint32_t)f32_to_bf16(f[2]) | ((uint32_t)f32_to_bf16(f[3]) << 16);
+  r.z = (uint32_t)f32_to_bf16(f[4]) | ((uint32_t)f32_to_bf16(f[5]) << 16);
+  r.w = (uint32_t)f32_to_bf16(f[6]) | ((uint32_t)f32_to_bf16(f[7]) << 16);
+  return r;
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+  return v;
+}
+
+// ---------------------------------------------------------------------------
+// combine backward.  Forward: out[t] = w1 * y[slot1] + w2 * y[slot2] with
+// w_k the activation-dtype gate (transformer/moe.py:509-510).  Hence
+//   dy[slot_k]  = w_k * dout[t]            (rounded to the activation dtype)
+//   dgate[t,k]  = <dout[t], y[slot_k]>     (float32), 0 where not kept
+// Jobs [0, T): tokens; jobs [T, T + G*E): zero rows for the slots >= fill.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void combine_backward_kernel(
+    const T* __restrict__ dout, const T* __restrict__ y,
+    const int32_t* __restrict__ idx, const int32_t* __restrict__ pos,
+    const float* __restrict__ gate, const uint8_t* __restrict__ kept,
+    const int32_t* __restrict__ fill, T* __restrict__ dy,
+    float* __restrict__ dgate, int G, int S, int E, int C, int N,
+    int64_t T_tokens, bool vec) {
+  constexpr int VN = Vec16B<T>::N;
+  const int lane = threadIdx.x & 63;
+  const int64_t job =
+      (int64_t)blockIdx.x * BW_ROWS_PER_BLOCK + (threadIdx.x >> 6);
+  if (job >= T_tokens + (int64_t)G * E) return;
+  if (job >= T_tokens) {
+    const int64_t ge = job - T_tokens;
+    const int g = (int)(ge / E), e = (int)(ge % E);
+    for (int c = fill[ge]; c < C; ++c) {
+      T* d = dy + (((int64_t)e * G + g) * C + c) * N;
+      if (vec) {
+        uint4* d4 = reinterpret_cast<uint4*>(d);
+        for (int i = lane; i < N / VN; i += 64) d4[i] = make_uint4(0, 0, 0, 0);
+      } else {
+        for (int i = lane; i < N; i += 64) d[i] = (T)0;
+      }
+    }
+    return;
+  }
+  const int64_t t = job;
+  const int g = (int)(t / S);
+  const T* yrow[2] = {nullptr, nullptr};
+  T* drow[2] = {nullptr, nullptr};
+  float w[2] = {0.f, 0.f};
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    if (kept[t * 2 + k]) {
+      const int64_t slot =
+          ((int64_t)idx[t * 2 + k] * G + g) * C + pos[t * 2 + k];
+      yrow[k] = y + slot * N;
+      drow[k] = dy + slot * N;
+      w[k] = round_to<T>(gate[t * 2 + k]);
+    }
+  }
+  float dot[2] = {0.f, 0.f};
+  const T* drc = dout + t * N;
+  if (vec) {
+    const uint4* d4 = reinterpret_cast<const uint4*>(drc);
+    for (int i = lane; i < N / VN; i += 64) {
+      float d[VN];
+      unpack16(d4[i], d, T());
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        if (yrow[k] == nullptr) continue;
+        float yv[VN], o[VN];
+        unpack16(reinterpret_cast<const uint4*>(yrow[k])[i], yv, T());
+#pragma unroll
+        for (int j = 0; j < VN; ++j) {
+          dot[k] += d[j] * yv[j];
+          o[j] = w[k] * d[j];
+        }
+        reinterpret_cast<uint4*>(drow[k])[i] = pack16(o, T());
+      }
+    }
+  } else {
+    for (int i = lane; i < N; i += 64) {
+      const float d = load_f32<T>(drc + i);
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        if (yrow[k] == nullptr) continue;
+        dot[k] += d * load_f32<T>(yrow[k] + i);
+        store_f32<T>(drow[k] + i, w[k] * d);
+      }
+    }
+  }
+  dot[0] = wave_sum(dot[0]);
+  dot[1] = wave_sum(dot[1]);
+  if (lane == 0) {
+    dgate[t * 2 + 0] = yrow[0] ? dot[0] : 0.f;
+    dgate[t * 2 + 1] = yrow[1] ? dot[1] : 0.f;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// dispatch backward (+ router projection backward w.r.t. the tokens).
+// Forward: expert_in[slot_k] = x[t] for every dispatched choice (a kept choice
+// whose activation-dtype gate is non-zero, transformer/moe.py:443-447,
+// :1510-1511) and logits[t] = float(x[t]) . w_gate (moe.py:1384-1390).  Hence
+//   dx[t] = sum_k dispatched_k * dexpert_in[slot_k] + dlogits[t] . w_gate^T
+// float32 accumulate, one rounding.  w_gate comes K-contiguous ([E, M]).
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void dispatch_backward_kernel(
+    const T* __restrict__ dxe, const int32_t* __restrict__ idx,
+    const int32_t* __restrict__ pos, const float* __restrict__ gate,
+    const uint8_t* __restrict__ kept, const float* __restrict__ dlogits,
+    const T* __restrict__ wgp, T* __restrict__ dx, int G, int S, int E, int C,
+    int M, int64_t T_tokens, bool vec) {
+  constexpr int VN = Vec16B<T>::N;
+  const int lane = threadIdx.x & 63;
+  const int64_t t =
+      (int64_t)blockIdx.x * BW_ROWS_PER_BLOCK + (threadIdx.x >> 6);
+  if (t >= T_tokens) return;
+  const int g = (int)(t / S);
+  const T* src[2] = {nullptr, nullptr};
+#pragma unroll
+  for (int k = 0; k < 2; ++k) {
+    if (kept[t * 2 + k] && round_to<T>(gate[t * 2 + k]) != 0.0f) {
+      const int64_t slot =
+          ((int64_t)idx[t * 2 + k] * G + g) * C + pos[t * 2 + k];
+      src[k] = dxe + slot * M;
+    }
+  }
+  const float* dl = dlogits ? dlogits + t * E : nullptr;
+  T* dst = dx + t * M;
+  if (vec) {
+    for (int i = lane; i < M / VN; i += 64) {
+      float acc[VN];
+#pragma unroll
+      for (int j = 0; j < VN; ++j) acc[j] = 0.f;
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        if (src[k] == nullptr) continue;
+        float v[VN];
+        unpack16(reinterpret_cast<const uint4*>(src[k])[i], v, T());
+#pragma unroll
+        for (int j = 0; j < VN; ++j) acc[j] += v[j];
+      }
+      if (dl != nullptr) {
+        for (int e = 0; e < E; ++e) {
+          const float d = dl[e];
+          float v[VN];
+          unpack16(reinterpret_cast<const uint4*>(wgp + (int64_t)e * M)[i], v,
+                   T());
+#pragma unroll
+          for (int j = 0; j < VN; ++j) acc[j] += d * v[j];
+        }
+      }
+      reinterpret_cast<uint4*>(dst)[i] = pack16(acc, T());
+    }
+  } else {
+    for (int i = lane; i < M; i += 64) {
+      float acc = 0.f;
+      if (src[0]) acc += load_f32<T>(src[0] + i);
+      if (src[1]) acc += load_f32<T>(src[1] + i);
+      if (dl != nullptr)
+        for (int e = 0; e < E; ++e)
+          acc += dl[e] * load_f32<T>(wgp + (int64_t)e * M + i);
+      store_f32<T>(dst + i, acc);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
+// gating backward.
+// Step 1, one block per group: how many tokens count for density_1 of each
+// expert and how many tokens have importance 1.
+// Step 2, one thread per token: d(logits) from d(gates) and d(loss).
+// ---------------------------------------------------------------------------
+struct GateBackwardParams {
+  int G, S, E;
+  int router;           // 0 = top-2, 1 = switch / switch_max
+  int has_importance;
+  int num_microbatches;
+  int use_z_loss;
+  float z_loss_coef;
+  float loss_scale;     // moe_loss_coef as the activation dtype holds it
+};
+
+template <typename IT>
+__global__ __launch_bounds__(256) void gate_count_kernel(
+    GateBackwardParams p, const int32_t* __restrict__ idx,
+    const IT* __restrict__ importance, int32_t* __restrict__ counts,
+    float* __restrict__ n_one) {
+  extern __shared__ int32_t cnt[];  // [E] + 1
+  const int g = blockIdx.x;
+  for (int e = threadIdx.x; e <= p.E; e += blockDim.x) cnt[e] = 0;
+  __syncthreads();
+  for (int s = threadIdx.x; s < p.S; s += blockDim.x) {
+    const int64_t t = (int64_t)g * p.S + s;
+    bool one = true;
+    if (importance != nullptr) one = load_f32<IT>(importance + t) == 1.0f;
+    if (one) atomicAdd(&cnt[p.E], 1);
+    // top-2: density_1 counts mask_1 after the importance mask
+    // (moe.py:1402-1420); switch: every token's arg-max (moe.py:1224)
+    if (one || p.router == 1) atomicAdd(&cnt[idx[t * 2]], 1);
+  }
+  __syncthreads();
+  for (int e = threadIdx.x; e < p.E; e += blockDim.x)
+    counts[(int64_t)g * p.E + e] = cnt[e];
+  if (threadIdx.x == 0) n_one[g] = (float)cnt[p.E];
+}
+
+template <typename IT>
+__global__ __launch_bounds__(256) void gating_backward_kernel(
+    GateBackwardParams p, const float* __restrict__ logits,
+    const IT* __restrict__ importance, const int32_t* __restrict__ idx,
+    const uint8_t* __restrict__ kept, const float* __restrict__ dgate,
+    const float* __restrict__ d_loss, const int32_t* __restrict__ counts,
+    const float* __restrict__ n_one, float* __restrict__ dlogits) {
+  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  const int64_t T_tokens = (int64_t)p.G * p.S;
+  if (t >= T_tokens) return;
+  const int E = p.E, S = p.S;
+  const int g = (int)(t / S);
+  const float* row = logits + t * E;
+  float* out = dlogits + t * E;
+  // softmax exactly as the forward kernel computes it
+  float m = row[0];
+  for (int e = 1; e < E; ++e) m = fmaxf(m, row[e]);
+  const float negm = -m;
+  float s = 0.f;
+  for (int e = 0; e < E; ++e) s += expf(row[e] + negm);
+  const float lse = logf(s) + m;
+  const float neglse = -lse;
+  float m1 = 1.0f;
+  if (importance != nullptr)
+    m1 = load_f32<IT>(importance + t) == 1.0f ? 1.0f : 0.0f;
+  const int i1 = idx[t * 2], i2 = idx[t * 2 + 1];
+  const float k1 = kept[t * 2] ? 1.0f : 0.0f, k2 = kept[t * 2 + 1] ? 1.0f : 0.0f;
+  const float mb =
+      p.num_microbatches > 1 ? (float)(1.0 / (double)p.num_microbatches) : 1.0f;
+  const float dl = d_loss[0] * p.loss_scale;
+  const float inv_s = (float)(1.0 / (double)S);
+  const float ee = (float)((double)E * (double)E);
+  float add1 = 0.f, add2 = 0.f;  // d(p[i1]), d(p[i2]) from the gates
+  float coef;                    // d(p[e]) = coef * counts[g,e] from the loss
+  if (p.router == 0) {
+    const float p1 = expf(row[i1] + neglse), p2 = expf(row[i2] + neglse);
+    const float g1 = p1 * m1;
+    const float same = (i2 == i1) ? m1 : 0.0f;
+    const float g2 = p2 * (1.0f - same);
+    const float dg1n = dgate[t * 2] * k1, dg2n = dgate[t * 2 + 1] * k2;
+    const float rec = 1.0f / ((g1 + g2) + 1e-9f);
+    const float common = (dg1n * g1 + dg2n * g2) * rec * rec;
+    add1 = (dg1n * rec - common) * m1;
+    add2 = (dg2n * rec - common) * (1.0f - same);
+    // loss = mean_{g,e}(mean_s(p * m1) * density_1) * E^2, density = count / S
+    coef = dl * mb * ee * (float)(1.0 / ((double)p.G * (double)E)) * inv_s *
+           inv_s * m1;
+  } else {
+    add1 = dgate[t * 2] * k1 * m1;
+    if (p.has_importance)
+      coef = dl * mb * ee *
+             (float)(1.0 / ((double)p.G * (double)E * (double)S)) * n_one[g] *
+             inv_s * inv_s;
+    else
+      coef = dl * mb * ee * (float)(1.0 / ((double)p.G * (double)E)) * inv_s *
+             inv_s;
+  }
+  const int32_t* cg = counts + (int64_t)g * E;
+  // inner = sum_e p[e] * dp[e]
+  float inner = 0.f;
+  for (int e = 0; e < E; ++e) {
+    const float pe = expf(row[e] + neglse);
+    float dp = coef * (float)cg[e];
+    if (e == i1) dp += add1;
+    if (p.router == 0 && e == i2) dp += add2;
+    inner += pe * dp;
+  }
+  float zfac = 0.f;
+  if (p.use_z_loss) {  // d/dx of z_coef * sum(lse^2 * m1) / (n * microbatches)
+    float n = 0.f;
+    for (int gg = 0; gg < p.G; ++gg) n += n_one[gg];
+    const float mbz = (float)(p.num_microbatches > 0 ? p.num_microbatches : 1);
+    zfac = (d_loss[0] * p.loss_scale * p.z_loss_coef * 2.0f) * lse * m1 /
+           (n * mbz);
+  }
+  for (int e = 0; e < E; ++e) {
+    const float pe = expf(row[e] + neglse);
+    float dp = coef * (float)cg[e];
+    if (e == i1) dp += add1;
+    if (p.router == 0 && e == i2) dp += add2;
+    out[e] = pe * (dp - inner) + zfac * pe;
+  }
+}
+
+// ---------------------------------------------------------------------------
+// router projection backward w.r.t. the kernel: dw[m,e] = sum_t x[t,m] *
+// dlogits[t,e], float32.  Block (m tile of 64, chunk of tokens, chunk of 64
+// experts) accumulates 64 x 64 partial sums, thread (m = tid % 64, 16 experts),
+// and adds them to the float32 accumulator with atomics.
+// ---------------------------------------------------------------------------
+constexpr int WG_TOK = 1024;  // tokens per block
+constexpr int WG_BATCH = 32;  // tokens staged in LDS at a time
+
+template <typename T>
+__global__ __launch_bounds__(256) void router_wgrad_kernel(
+    const T* __restrict__ x, const float* __restrict__ dlogits,
+    float* __restrict__ acc_out, int64_t T_tokens, int M, int E) {
+  __shared__ float xs[WG_BATCH][64 + 1];
+  __shared__ float ds[WG_BATCH][64];
+  const int m0 = blockIdx.x * 64, e0 = blockIdx.z * 64;
+  const int64_t t0 = (int64_t)blockIdx.y * WG_TOK;
+  const int64_t t1 = t0 + WG_TOK < T_tokens ? t0 + WG_TOK : T_tokens;
+  const int tid = threadIdx.x;
+  const int ml = tid & 63, eg = tid >> 6;  // experts e0 + eg*16 .. +15
+  float acc[16];
+#pragma unroll
+  for (int j = 0; j < 16; ++j) acc[j] = 0.f;
+  for (int64_t tb = t0; tb < t1; tb += WG_BATCH) {
+    for (int i = tid; i < WG_BATCH * 64; i += 256) {
+      const int r = i >> 6, c = i & 63;
+      const int64_t t = tb + r;
+      const bool ok = t < t1;
+      xs[r][c] = (ok && m0 + c < M) ? load_f32<T>(x + t * M + m0 + c) : 0.f;
+      ds[r][c] = (ok && e0 + c < E) ? dlogits[t * E + e0 + c] : 0.f;
+    }
+    __syncthreads();
+#pragma unroll 4
+    for (int r = 0; r < WG_BATCH; ++r) {
+      const float xv = xs[r][ml];
+#pragma unroll
+      for (int j = 0; j < 16; ++j) acc[j] += xv * ds[r][eg * 16 + j];
+    }
+    __syncthreads();
+  }
+  if (m0 + ml < M) {
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+      const int e = e0 + eg * 16 + j;
+      if (e < E) atomicAdd(acc_out + (int64_t)(m0 + ml) * E + e, acc[j]);
+    }
+  }
+}
+
+__global__ void fill_f32_kernel(float* p, int64_t n, float v) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += stride)
+    p[i] = v;
+}
+
+template <typename T>
+__global__ void convert_f32_kernel(const float* src, T* dst, int64_t n) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += stride)
+    store_f32<T>(dst + i, src[i]);
+}
+
+static bool bw_aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
+
+}  // namespace mesh_moe
+
+using namespace mesh_moe;
+
+extern "C" int mesh_moe_combine_backward(
+    const void* dout, const void* y, const int32_t* idx, const int32_t* pos,
+    const float* gate, const uint8_t* kept, const int32_t* fill, void* dy,
+    float* dgate, int G, int S, int E, int C, int N, int dtype, void* stream) {
+  MOE_REQUIRE(dout && y && idx && pos && gate && kept && fill && dy && dgate,
+              MESH_MOE_E_ARG, "combine_backward: null pointer");
+  MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG,
+              "combine_backward: bad dtype %d", dtype);
+  MOE_REQUIRE(G >= 1 && S >= 1 && E >= 1 && C >= 1 && N >= 1, MESH_MOE_E_ARG,
+              "combine_backward: bad sizes G=%d S=%d E=%d C=%d N=%d", G, S, E,
+              C, N);
+  const int64_t T_tokens = (int64_t)G * S;
+  const int64_t njobs = T_tokens + (int64_t)G * E;
+  const int64_t nblocks = (njobs + BW_ROWS_PER_BLOCK - 1) / BW_ROWS_PER_BLOCK;
+  MOE_REQUIRE(nblocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
+              "combine_backward: too many rows (%lld)", (long long)njobs);
+  const bool vec = ((size_t)N * dtype_size(dtype)) % 16 == 0 &&
+                   bw_aligned16(dout) && bw_aligned16(y) && bw_aligned16(dy);
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == MESH_MOE_F32)
+    combine_backward_kernel<float><<<(unsigned)nblocks, 256, 0, st>>>(
+        (const float*)dout, (const float*)y, idx, pos, gate, kept, fill,
+        (float*)dy, dgate, G, S, E, C, N, T_tokens, vec);
+  else
+    combine_backward_kernel<bf16_t><<<(unsigned)nblocks, 256, 0, st>>>(
+        (const bf16_t*)dout, (const bf16_t*)y, idx, pos, gate, kept, fill,
+        (bf16_t*)dy, dgate, G, S, E, C, N, T_tokens, vec);
+  MOE_CHECK_LAUNCH("combine_backward");
+  return 0;
+}
+
+extern "C" int mesh_moe_dispatch_backward(
+    const void* dexpert_in, const int32_t* idx, const int32_t* pos,
+    const float* gate, const uint8_t* kept, const float* dlogits,
+    const void* w_gate_packed, void* dx, int G, int S, int E, int C, int M,
+    int dtype, void* stream) {
+  MOE_REQUIRE(dexpert_in && idx && pos && gate && kept && dx, MESH_MOE_E_ARG,
+              "dispatch_backward: null pointer");
+  MOE_REQUIRE((dlogits == nullptr) == (w_gate_packed == nullptr),
+              MESH_MOE_E_ARG,
+              "dispatch_backward: dlogits and w_gate_packed go together");
+  MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG,
+              "dispatch_backward: bad dtype %d", dtype);
+  MOE_REQUIRE(G >= 1 && S >= 1 && E >= 1 && C >= 1 && M >= 1, MESH_MOE_E_ARG,
+              "dispatch_backward: bad sizes G=%d S=%d E=%d C=%d M=%d", G, S, E,
+              C, M);
+  const int64_t T_tokens = (int64_t)G * S;
+  const int64_t nblocks =
+      (T_tokens + BW_ROWS_PER_BLOCK - 1) / BW_ROWS_PER_BLOCK;
+  MOE_REQUIRE(nblocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
+              "dispatch_backward: too many rows (%lld)", (long long)T_tokens);
+  const bool vec = ((size_t)M * dtype_size(dtype)) % 16 == 0 &&
+                   bw_aligned16(dexpert_in) && bw_aligned16(dx) &&
+                   (w_gate_packed == nullptr || bw_aligned16(w_gate_packed));
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == MESH_MOE_F32)
+    dispatch_backward_kernel<float><<<(unsigned)nblocks, 256, 0, st>>>(
+        (const float*)dexpert_in, idx, pos, gate, kept, dlogits,
+        (const float*)w_gate_packed, (float*)dx, G, S, E, C, M, T_tokens, vec);
+  else
+    dispatch_backward_kernel<bf16_t><<<(unsigned)nblocks, 256, 0, st>>>(
+        (const bf16_t*)dexpert_in, idx, pos, gate, kept, dlogits,
+        (const bf16_t*)w_gate_packed, (bf16_t*)dx, G, S, E, C, M, T_tokens,
+        vec);
+  MOE_CHECK_LAUNCH("dispatch_backward");
+  return 0;
+}
+
+extern "C" size_t mesh_moe_gating_backward_workspace_bytes(int G, int E) {
+  if (G < 1 || E < 1) return 0;
+  return sizeof(int32_t) * (size_t)G * E + sizeof(float) * (size_t)G + 256;
+}
+
+extern "C" int mesh_moe_gating_backward(
+    const float* logits, const void* importance, int importance_dtype,
+    const int32_t* idx, const uint8_t* kept, const float* dgate,
+    const float* d_loss, double loss_scale, int G, int S, int E, int router,
+    int use_z_loss, double z_loss_coef, int num_microbatches, float* dlogits,
+    void* workspace, size_t workspace_bytes, void* stream) {
+  MOE_REQUIRE(logits && idx && kept && dgate && d_loss && dlogits && workspace,
+              MESH_MOE_E_ARG, "gating_backward: null pointer");
+  MOE_REQUIRE(G >= 1 && S >= 1 && E >= 2 && E <= 512 && G <= 65535,
+              MESH_MOE_E_ARG, "gating_backward: bad sizes G=%d S=%d E=%d", G, S,
+              E);
+  MOE_REQUIRE(router == 0 || router == 1, MESH_MOE_E_ARG,
+              "gating_backward: unknown router %d", router);
+  MOE_REQUIRE(!importance || valid_dtype(importance_dtype), MESH_MOE_E_ARG,
+              "gating_backward: bad importance dtype %d", importance_dtype);
+  MOE_REQUIRE(workspace_bytes >= mesh_moe_gating_backward_workspace_bytes(G, E),
+              MESH_MOE_E_ARG, "gating_backward: workspace too small");
+  GateBackwardParams p;
+  p.G = G; p.S = S; p.E = E;
+  p.router = router;
+  p.has_importance = importance != nullptr;
+  p.num_microbatches = num_microbatches;
+  p.use_z_loss = (use_z_loss && router == 1) ? 1 : 0;
+  p.z_loss_coef = (float)z_loss_coef;
+  p.loss_scale = (float)loss_scale;
+  uintptr_t wsp = ((uintptr_t)workspace + 255) & ~(uintptr_t)255;
+  int32_t* counts = (int32_t*)wsp;
+  float* n_one = (float*)(counts + (size_t)G * E);
+  hipStream_t st = (hipStream_t)stream;
+  const size_t smem = sizeof(int32_t) * ((size_t)E + 1);
+  const int64_t T_tokens = (int64_t)G * S;
+  const unsigned blocks = (unsigned)((T_tokens + 255) / 256);
+  if (importance && importance_dtype == MESH_MOE_BF16) {
+    gate_count_kernel<bf16_t><<<G, 256, smem, st>>>(
+        p, idx, (const bf16_t*)importance, counts, n_one);
+    MOE_CHECK_LAUNCH("gating_backward (count)");
+    gating_backward_kernel<bf16_t><<<blocks, 256, 0, st>>>(
+        p, logits, (const bf16_t*)importance, idx, kept, dgate, d_loss, counts,
+        n_one, dlogits);
+  } else {
+    gate_count_kernel<float><<<G, 256, smem, st>>>(
+        p, idx, (const float*)importance, counts, n_one);
+    MOE_CHECK_LAUNCH("gating_backward (count)");
+    gating_backward_kernel<float><<<blocks, 256, 0, st>>>(
+        p, logits, (const float*)importance, idx, kept, dgate, d_loss, counts,
+        n_one, dlogits);
+  }
+  MOE_CHECK_LAUNCH("gating_backward");
+  return 0;
+}
+
+extern "C" int mesh_moe_router_backward_weights(const void* x,
+                                                const float* dlogits,
+                                                void* dw_gate,
+                                                float* workspace,
+                                                int64_t tokens, int M, int E,
+                                                int dtype, void* stream) {
+  MOE_REQUIRE(x && dlogits && dw_gate && workspace, MESH_MOE_E_ARG,
+              "router_backward_weights: null pointer");
+  MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG,
+              "router_backward_weights: bad dtype %d", dtype);
+  MOE_REQUIRE(tokens >= 1 && M >= 1 && E >= 1, MESH_MOE_E_ARG,
+              "router_backward_weights: bad sizes tokens=%lld M=%d E=%d",
+              (long long)tokens, M, E);
+  const int64_t chunks = (tokens + WG_TOK - 1) / WG_TOK;
+  MOE_REQUIRE(chunks <= 65535 && (E + 63) / 64 <= 65535,
+              MESH_MOE_E_UNSUPPORTED,
+              "router_backward_weights: too many tokens (%lld)",
+              (long long)tokens);
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t n = (int64_t)M * E;
+  const unsigned fb = (unsigned)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+  fill_f32_kernel<<<fb, 256, 0, st>>>(workspace, n, 0.0f);
+  MOE_CHECK_LAUNCH("router_backward_weights (clear)");
+  dim3 grid((unsigned)((M + 63) / 64), (unsigned)chunks,
+            (unsigned)((E + 63) / 64));
+  if (dtype == MESH_MOE_F32) {
+    router_wgrad_kernel<float><<<grid, 256, 0, st>>>(
+        (const float*)x, dlogits, workspace, tokens, M, E);
+    MOE_CHECK_LAUNCH("router_backward_weights");
+    convert_f32_kernel<float><<<fb, 256, 0, st>>>(workspace, (float*)dw_gate, n);
+  } else {
+    router_wgrad_kernel<bf16_t><<<grid, 256, 0, st>>>(
+        (const bf16_t*)x, dlogits, workspace, tokens, M, E);
+    MOE_CHECK_LAUNCH("router_backward_weights");
+    convert_f32_kernel<bf16_t><<<fb, 256, 0, st>>>(workspace, (bf16_t*)dw_gate,
+                                                  n);
+  }
+  MOE_CHECK_LAUNCH("router_backward_weights (convert)");
+  return 0;
+}

@@ -785,6 +785,19 @@ __global__ __launch_bounds__(256) void activation_kernel(T* __restrict__ h,
     store_f32<T>(h + i, apply_activation(load_f32<T>(h + i), act));
 }
 
+// dh = (h > 0) ? dh : 0 -- the ReLU of the forward pass seen from behind
+// (h is the stored, already rounded activation: positive iff the
+// pre-activation rounded to a positive value).
+template <typename T>
+__global__ __launch_bounds__(256) void relu_mask_kernel(T* __restrict__ dh,
+                                                        const T* __restrict__ h,
+                                                        int64_t n) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += stride)
+    if (!(load_f32<T>(h + i) > 0.f)) dh[i] = (T)0;
+}
+
 template <int BM, int BN, int BK>
 static int launch_mfma(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
                        int R, int N, int K, bool relu, hipStream_t st) {
@@ -941,5 +954,85 @@ extern "C" int mesh_moe_expert_ffn(const void* expert_in, const void* wi_packed,
                         st);
   if (rc != 0) return rc;
   return grouped_gemm(h, wo_packed, y, E, R, N, H, MESH_MOE_ACT_LINEAR, dtype,
+                      st);
+}
+
+// Elements of the scratch mesh_moe_expert_ffn_backward needs: dh [E,R,H], one
+// [E,H,R] transpose buffer (h^T, then dh^T) and one [E,max(M,N),R] buffer
+// (dy^T, then expert_in^T).
+static size_t ffn_backward_elems(int E, int R, int M, int H, int N) {
+  const size_t mn = (size_t)(M > N ? M : N);
+  return (size_t)E * R * H * 2 + (size_t)E * R * mn;
+}
+
+extern "C" size_t mesh_moe_expert_ffn_backward_workspace_bytes(int E, int R,
+                                                               int M, int H,
+                                                               int N,
+                                                               int dtype) {
+  if (E < 1 || R < 1 || M < 1 || H < 1 || N < 1 || !valid_dtype(dtype))
+    return 0;
+  return ffn_backward_elems(E, R, M, H, N) * dtype_size(dtype) + 3 * 256;
+}
+
+extern "C" int mesh_moe_expert_ffn_backward(
+    const void* expert_in, const void* h, const void* dy, const void* wi,
+    const void* wo, void* dexpert_in, void* dwi, void* dwo, int E, int R,
+    int M, int H, int N, int activation, int dtype, void* workspace,
+    size_t workspace_bytes, void* stream) {
+  MOE_REQUIRE(expert_in && h && dy && wi && wo && dexpert_in && dwi && dwo &&
+                  workspace, MESH_MOE_E_ARG,
+              "expert_ffn_backward: null pointer");
+  MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG,
+              "expert_ffn_backward: bad dtype %d", dtype);
+  MOE_REQUIRE(E >= 1 && R >= 1 && M >= 1 && H >= 1 && N >= 1, MESH_MOE_E_ARG,
+              "expert_ffn_backward: bad sizes E=%d R=%d M=%d H=%d N=%d", E, R,
+              M, H, N);
+  MOE_REQUIRE(activation == MESH_MOE_ACT_RELU ||
+                  activation == MESH_MOE_ACT_LINEAR, MESH_MOE_E_UNSUPPORTED,
+              "expert_ffn_backward: only relu and linear experts (got %d): the "
+              "other activations need the pre-activation, which is not kept",
+              activation);
+  MOE_REQUIRE(workspace_bytes >= mesh_moe_expert_ffn_backward_workspace_bytes(
+                                     E, R, M, H, N, dtype),
+              MESH_MOE_E_ARG, "expert_ffn_backward: workspace too small");
+  const size_t es = dtype_size(dtype);
+  auto up = [](uintptr_t v) { return (v + 255) & ~(uintptr_t)255; };
+  unsigned char* dh = (unsigned char*)up((uintptr_t)workspace);
+  unsigned char* tr_h = (unsigned char*)up((uintptr_t)(dh + (size_t)E * R * H * es));
+  unsigned char* tr_mn = (unsigned char*)up((uintptr_t)(tr_h + (size_t)E * R * H * es));
+  hipStream_t st = (hipStream_t)stream;
+  int rc;
+  // dh = dy . wo^T  (wo in its variable layout [E, H, N] is K-contiguous here)
+  rc = grouped_gemm(dy, wo, dh, E, R, H, N, MESH_MOE_ACT_LINEAR, dtype, st);
+  if (rc != 0) return rc;
+  if (activation == MESH_MOE_ACT_RELU) {
+    const int64_t n = (int64_t)E * R * H;
+    const int blocks = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
+    if (dtype == MESH_MOE_F32)
+      relu_mask_kernel<float><<<blocks, 256, 0, st>>>((float*)dh,
+                                                      (const float*)h, n);
+    else
+      relu_mask_kernel<bf16_t><<<blocks, 256, 0, st>>>((bf16_t*)dh,
+                                                       (const bf16_t*)h, n);
+    MOE_CHECK_LAUNCH("expert_ffn_backward (relu mask)");
+  }
+  // dexpert_in = dh . wi^T  (wi in its variable layout [E, M, H])
+  rc = grouped_gemm(dh, wi, dexpert_in, E, R, M, H, MESH_MOE_ACT_LINEAR, dtype,
+                    st);
+  if (rc != 0) return rc;
+  // dwo [E, H, N] = h^T . dy: both operands transposed to token-contiguous
+  rc = mesh_moe_pack_weights(h, tr_h, E, R, H, dtype, dtype, stream);
+  if (rc != 0) return rc;
+  rc = mesh_moe_pack_weights(dy, tr_mn, E, R, N, dtype, dtype, stream);
+  if (rc != 0) return rc;
+  rc = grouped_gemm(tr_h, tr_mn, dwo, E, H, N, R, MESH_MOE_ACT_LINEAR, dtype,
+                    st);
+  if (rc != 0) return rc;
+  // dwi [E, M, H] = expert_in^T . dh
+  rc = mesh_moe_pack_weights(expert_in, tr_mn, E, R, M, dtype, dtype, stream);
+  if (rc != 0) return rc;
+  rc = mesh_moe_pack_weights(dh, tr_h, E, R, H, dtype, dtype, stream);
+  if (rc != 0) return rc;
+  return grouped_gemm(tr_mn, tr_h, dwi, E, M, H, R, MESH_MOE_ACT_LINEAR, dtype,
                       st);
 }

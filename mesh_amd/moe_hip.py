@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 2
+ABI_VERSION = 3
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -66,6 +66,29 @@ _SIGNATURES = {
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
     "mesh_moe_combine": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
+    "mesh_moe_combine_backward": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        _vp]),
+    "mesh_moe_expert_ffn_backward_workspace_bytes": (ctypes.c_size_t, [
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int]),
+    "mesh_moe_expert_ffn_backward": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        _vp, ctypes.c_size_t, _vp]),
+    "mesh_moe_gating_backward_workspace_bytes": (ctypes.c_size_t, [
+        ctypes.c_int, ctypes.c_int]),
+    "mesh_moe_gating_backward": (ctypes.c_int, [
+        _vp, _vp, ctypes.c_int, _vp, _vp, _vp, _vp, ctypes.c_double,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_double, ctypes.c_int, _vp, _vp, ctypes.c_size_t, _vp]),
+    "mesh_moe_router_backward_weights": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, _vp]),
+    "mesh_moe_dispatch_backward": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
 }
 EXPORTS = sorted(_SIGNATURES)
@@ -491,3 +514,123 @@ def combine(y, r, group_size, out=None):
         _dev(r.kept, "kept", torch.uint8, (g, s, 2)), op, g, s, e, c, n, code,
         _stream()), "combine")
   return out
+
+
+# ----------------------------------------------------------------------------
+# backward
+# ----------------------------------------------------------------------------
+def _routing_ptrs(r, g, s):
+  return (_dev(r.idx, "idx", torch.int32, (g, s, 2)),
+          _dev(r.pos, "pos", torch.int32, (g, s, 2)),
+          _dev(r.gate, "gate", torch.float32, (g, s, 2)),
+          _dev(r.kept, "kept", torch.uint8, (g, s, 2)))
+
+
+def combine_backward(dout, y, r):
+  """dout [G, S, N], y [E, G, C, N] -> (dy [E, G, C, N], dgate [G, S, 2])."""
+  lib = load_library()
+  g, s, n = dout.shape
+  e, _, c, _ = y.shape
+  dt = y.dtype
+  dy = torch.empty_like(y)
+  dgate = torch.empty((g, s, 2), dtype=torch.float32, device=y.device)
+  ip, pp, gp, kp = _routing_ptrs(r, g, s)
+  with _stage("combine_backward"):
+    _check(lib.mesh_moe_combine_backward(
+        _dev(dout, "dout", dt, (g, s, n)), _dev(y, "y", dt, (e, g, c, n)),
+        ip, pp, gp, kp, _dev(r.fill, "fill", torch.int32, (g, e)),
+        dy.data_ptr(), dgate.data_ptr(), g, s, e, c, n, dtype_code(dt),
+        _stream()), "combine_backward")
+  return dy, dgate
+
+
+def expert_ffn_backward(expert_in, h, dy, wi, wo, activation="relu"):
+  """expert_in [E,R,M], h [E,R,H], dy [E,R,N]; wi [E,M,H], wo [E,H,N] in the
+  variables' own layout -> (dexpert_in [E,R,M], dwi [E,M,H], dwo [E,H,N])."""
+  lib = load_library()
+  if activation not in ACTIVATIONS:
+    raise ValueError("unsupported expert activation %r" % (activation,))
+  e, rows, m = expert_in.shape
+  hdim, n = wo.shape[1], wo.shape[2]
+  dt = expert_in.dtype
+  code = dtype_code(dt)
+  dev = expert_in.device
+  dxe = torch.empty((e, rows, m), dtype=dt, device=dev)
+  dwi = torch.empty((e, m, hdim), dtype=dt, device=dev)
+  dwo = torch.empty((e, hdim, n), dtype=dt, device=dev)
+  ws_bytes = lib.mesh_moe_expert_ffn_backward_workspace_bytes(
+      e, rows, m, hdim, n, code)
+  ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
+  with _stage("expert_ffn_backward"):
+    _check(lib.mesh_moe_expert_ffn_backward(
+        _dev(expert_in, "expert_in"), _dev(h, "h", dt, (e, rows, hdim)),
+        _dev(dy, "dy", dt, (e, rows, n)), _dev(wi, "wi", dt, (e, m, hdim)),
+        _dev(wo, "wo", dt, (e, hdim, n)), dxe.data_ptr(), dwi.data_ptr(),
+        dwo.data_ptr(), e, rows, m, hdim, n, ACTIVATIONS[activation], code,
+        ws.data_ptr(), ws_bytes, _stream()), "expert_ffn_backward")
+  return dxe, dwi, dwo
+
+
+def gating_backward(logits, r, dgate, d_loss, loss_scale, router="top_2",
+                    importance=None, z_loss=None, num_microbatches=None):
+  """d(logits) [G, S, E] float32.  d_loss: float32 tensor of one element on the
+  device (gradient w.r.t. the layer's returned loss); loss_scale:
+  moe_loss_coef."""
+  lib = load_library()
+  g, s, e = logits.shape
+  dev = logits.device
+  ip, icode = None, F32
+  if importance is not None:
+    icode = dtype_code(importance.dtype)
+    ip = _dev(importance, "importance", None, (g, s))
+  dlogits = torch.empty((g, s, e), dtype=torch.float32, device=dev)
+  ws_bytes = lib.mesh_moe_gating_backward_workspace_bytes(g, e)
+  ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=dev)
+  with _stage("gating_backward"):
+    _check(lib.mesh_moe_gating_backward(
+        _dev(logits, "logits", torch.float32), ip, icode,
+        _dev(r.idx, "idx", torch.int32, (g, s, 2)),
+        _dev(r.kept, "kept", torch.uint8, (g, s, 2)),
+        _dev(dgate, "dgate", torch.float32, (g, s, 2)),
+        _dev(d_loss, "d_loss", torch.float32), float(loss_scale), g, s, e,
+        0 if router == "top_2" else 1, int(z_loss is not None),
+        float(z_loss or 0.0), int(num_microbatches or 1), dlogits.data_ptr(),
+        ws.data_ptr(), ws_bytes, _stream()), "gating_backward")
+  return dlogits
+
+
+def router_backward_weights(x, dlogits):
+  """x [T, M], dlogits [T, E] float32 -> dw_gate [M, E] of x's dtype."""
+  lib = load_library()
+  t, m = x.shape
+  e = dlogits.shape[-1]
+  out = torch.empty((m, e), dtype=x.dtype, device=x.device)
+  ws = torch.empty((m, e), dtype=torch.float32, device=x.device)
+  with _stage("router_backward_weights"):
+    _check(lib.mesh_moe_router_backward_weights(
+        _dev(x, "x"), _dev(dlogits, "dlogits", torch.float32, (t, e)),
+        out.data_ptr(), ws.data_ptr(), t, m, e, dtype_code(x.dtype),
+        _stream()), "router_backward_weights")
+  return out
+
+
+def dispatch_backward(dexpert_in, r, group_size, dlogits=None,
+                      w_gate_packed=None):
+  """dexpert_in [E, G, C, M] (+ dlogits [G, S, E], w_gate_packed [E, M]) ->
+  dx [G, S, M]."""
+  lib = load_library()
+  e, g, c, m = dexpert_in.shape
+  s = group_size
+  dt = dexpert_in.dtype
+  dx = torch.empty((g, s, m), dtype=dt, device=dexpert_in.device)
+  ip, pp, gp, kp = _routing_ptrs(r, g, s)
+  dlp = wgp = None
+  if dlogits is not None:
+    dlp = _dev(dlogits, "dlogits", torch.float32, (g, s, e))
+    wgp = _dev(w_gate_packed, "w_gate_packed", dt, (e, m))
+  with _stage("dispatch_backward"):
+    _check(lib.mesh_moe_dispatch_backward(
+        _dev(dexpert_in, "dexpert_in"), ip, pp, gp, kp, dlp, wgp,
+        dx.data_ptr(), g, s, e, c, m, dtype_code(dt), _stream()),
+        "dispatch_backward")
+  return dx

@@ -30,6 +30,9 @@ MoE file, and its TensorFlow dependency cannot run here):
                                       lowering of mtf.top_k) vs the stable
                                       sort, per-expert brute force, equality
                                       with switch_gating when nothing overflows
+  gating_backward,                    central differences of an independent
+  moe_layer_v1_backward               float64 forward with the routing held
+                                      fixed (tests/test_oracle.py)
   v2                                  x=1 outer expert reduces to v1
 
 PARITY UNPINNED against TensorFlow itself (only running the reference could
@@ -688,6 +691,169 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
              num_groups=g_, group_size=s_, capacity=c_)
   return (out.reshape(lead + (n_,)),
           _scale_loss(r["loss"], hp.moe_loss_coef, act_dtype), aux)
+
+
+# ----------------------------------------------------------------------------
+# backward of transformer_moe_layer_v1
+# ----------------------------------------------------------------------------
+def gating_backward(logits, r, gating, d_gate_1, d_gate_2, d_loss,
+                    importance=None, num_microbatches=None, z_loss=None):
+  """d(logits) of _top_2_gating / _switch_gating / _switch_max_gating.
+
+  The reference obtains it from the gradients of the ops the gating is built
+  from: top_1 routes the gradient of a gate to the arg-max entry
+  (TopKOperation.gradient, ops.py:4916-4920); one_hot, cumsum-of-masks,
+  comparisons and the bool cast that makes the dispatch tensor have no
+  gradient; divide/add/multiply are the usual rules (ops.py:2044-2084);
+  softmax = exp(x - logsumexp(x)) (ops.py:5493-5541).
+
+  d_gate_k [G,S]: gradient w.r.t. the combine weight gate_k * mask_k_flat
+  (float32, zero where not kept); d_loss: gradient w.r.t. the balancing loss
+  before moe_loss_coef.  Returns float32 [G,S,E].
+  """
+  logits = np.asarray(logits, dtype=F32)
+  g_, s_, e_ = logits.shape
+  p = softmax(logits)
+  rows = np.arange(g_)[:, None], np.arange(s_)[None, :]
+  i1 = r["index_1"]
+  one = np.ones((g_, s_), F32)
+  m1 = one if importance is None else (
+      np.asarray(importance, F32) == F32(1.0)).astype(F32)
+  mb = F32(1.0 / num_microbatches) if (num_microbatches and
+                                       num_microbatches > 1) else F32(1.0)
+  dp = np.zeros_like(p)
+  d_loss = F32(d_loss)
+  inv_s = F32(1.0 / s_)
+  ee = F32(float(e_ * e_))
+  if gating == "top_2":
+    i2 = r["index_2"]
+    g1 = p[rows + (i1,)] * m1
+    same = (i2 == i1).astype(F32) * m1
+    g2 = p[rows + (i2,)] * (one - same)
+    dg1n = np.asarray(d_gate_1, F32) * r["kept_1"]
+    dg2n = np.asarray(d_gate_2, F32) * r["kept_2"]
+    rec = F32(1.0) / ((g1 + g2) + F32(1e-9))                     # moe.py:1413
+    common = (dg1n * g1 + dg2n * g2) * rec * rec
+    dg1 = dg1n * rec - common
+    dg2 = dg2n * rec - common
+    np.add.at(dp, rows + (i1,), dg1 * m1)
+    np.add.at(dp, rows + (i2,), dg2 * (one - same))
+    # loss = mean_{g,e}(mean_s(p * m1) * density_1) * E^2   (moe.py:1420-1424)
+    density = seq_sum(one_hot(i1, e_) * m1[..., None], axis=-2) * inv_s
+    coef = d_loss * mb * ee * F32(1.0 / (g_ * e_))
+    dp += (coef * density * inv_s)[:, None, :] * m1[..., None]
+    return (p * (dp - (p * dp).sum(-1, keepdims=True))).astype(F32)
+  if gating not in ("switch", "switch_max"):
+    raise ValueError("unknown gating %r" % (gating,))
+  np.add.at(dp, rows + (i1,), np.asarray(d_gate_1, F32) * r["kept_1"] * m1)
+  # loss = mean(mean_s(p)[g,e] * m1[g,s] * density_1[g,e]) * E^2 with density_1
+  # counting every token (moe.py:1224-1234)
+  density = seq_sum(one_hot(i1, e_), axis=-2) * inv_s
+  if importance is None:
+    coef = d_loss * mb * ee * F32(1.0 / (g_ * e_))
+    dproxy = coef * density
+  else:
+    coef = d_loss * mb * ee * F32(1.0 / (g_ * e_ * s_))
+    dproxy = coef * density * m1.sum(-1, dtype=F32)[:, None]
+  dp += (dproxy * inv_s)[:, None, :]
+  dlogits = p * (dp - (p * dp).sum(-1, keepdims=True))
+  if z_loss is not None:                                        # moe.py:1253-1266
+    m = logits.max(-1, keepdims=True)
+    lse = (np.log(np.exp(logits - m).sum(-1)) + m[..., 0]).astype(F32)
+    denom = m1.sum(dtype=F32) * F32(num_microbatches)
+    dlogits = dlogits + ((d_loss * F32(z_loss) * F32(2.0)) * lse * m1
+                         / denom)[..., None] * p
+  return dlogits.astype(F32)
+
+
+def moe_layer_v1_backward(x, w_gate, wi, wo, hp, train, act_dtype, d_out,
+                          d_loss=0.0, nonpadding=None, activation="relu",
+                          num_microbatches=None, logit_bias=None):
+  """Gradients of (outputs, loss) of moe_layer_v1 w.r.t. x and the three
+  kernels, given d_out [batch..., length, N] and the scalar d_loss.
+
+  Follows what mtf.gradients (ops.py:5254-5291) assembles from the layer's ops:
+  the combine / dispatch einsums and the two expert einsums back-propagate as
+  einsums with the same one-hot tensors (EinsumOperation.gradient,
+  ops.py:2846-2854), i.e. as the gather / scatter of the routing record;
+  gradients are tensors of the activation dtype (cast gradients cast back,
+  ops.py:1945-1962), float32 inside the gating.  The dispatch tensor is a
+  bool cast of the combine tensor and carries no gradient (moe.py:1510-1511).
+  The second-place loss is not covered.
+
+  Returns dict(dx, dw_gate, dwi, dwo) holding activation-dtype values.
+  """
+  if hp.moe_use_second_place_loss:
+    raise NotImplementedError("backward of the second-place loss")
+  if activation not in ("relu", "linear", None):
+    raise NotImplementedError("backward of activation %r" % (activation,))
+  _, _, aux = moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype,
+                           nonpadding=nonpadding, activation=activation,
+                           num_microbatches=num_microbatches,
+                           logit_bias=logit_bias, dense=False)
+  x = cast_act(x, act_dtype)
+  lead, m_ = x.shape[:-1], x.shape[-1]
+  g_, s_, c_ = aux["num_groups"], aux["group_size"], aux["capacity"]
+  e_ = hp.moe_num_experts
+  xg = x.reshape(g_, s_, m_)
+  wg_a, wi_a, wo_a = (cast_act(w, act_dtype) for w in (w_gate, wi, wo))
+  n_ = wo_a.shape[-1]
+  dout = cast_act(np.asarray(d_out, F32), act_dtype).reshape(g_, s_, n_)
+  y = aux["expert_out"]                                          # [E,G,C,N]
+  expert_in = aux["expert_in"]                                   # [E,G,C,M]
+  w1, w2 = combine_weights(aux, act_dtype)
+
+  # combine backward: d(weights) and d(expert outputs)
+  dy = np.zeros_like(y)
+  dgate = []
+  for k, w in (("1", w1), ("2", w2)):
+    dgk = np.zeros((g_, s_), F32)
+    sel = aux["kept_" + k]
+    gi, si = np.nonzero(sel)
+    ei, ci = aux["index_" + k][gi, si], aux["pos_" + k][gi, si]
+    dgk[gi, si] = (dout[gi, si] * y[ei, gi, ci]).sum(-1, dtype=F32)
+    dy[ei, gi, ci] = cast_act(w[gi, si][:, None] * dout[gi, si], act_dtype)
+    dgate.append(dgk)
+
+  # expert FFN backward (float32 accumulate, activation-dtype results)
+  r_ = g_ * c_
+  xe = expert_in.reshape(e_, r_, m_)
+  h = cast_act(np.matmul(xe, wi_a), act_dtype)
+  if activation == "relu":
+    h = cast_act(np.maximum(h, F32(0.0)), act_dtype)
+  dy2 = dy.reshape(e_, r_, n_)
+  dh = cast_act(np.matmul(dy2, wo_a.transpose(0, 2, 1)), act_dtype)
+  if activation == "relu":
+    dh = dh * (h > 0)
+  dwo = cast_act(np.matmul(h.transpose(0, 2, 1), dy2), act_dtype)
+  dxe = cast_act(np.matmul(dh, wi_a.transpose(0, 2, 1)), act_dtype)
+  dwi = cast_act(np.matmul(xe.transpose(0, 2, 1), dh), act_dtype)
+  dxe = dxe.reshape(e_, g_, c_, m_)
+
+  # dispatch backward: a token gathers the rows of the slots it was sent to
+  dx = np.zeros((g_, s_, m_), F32)
+  for k, w in (("1", w1), ("2", w2)):
+    sel = aux["kept_" + k] & (w != 0)
+    gi, si = np.nonzero(sel)
+    dx[gi, si] += dxe[aux["index_" + k][gi, si], gi, aux["pos_" + k][gi, si]]
+
+  # gating and router backward
+  importance = None
+  if nonpadding is not None:
+    importance = cast_act(np.broadcast_to(nonpadding, lead), act_dtype)
+    importance = importance.reshape(g_, s_)
+  z = hp.moe_z_loss if (train and hp.moe_gating == "switch") else None
+  # the returned loss is aux * moe_loss_coef in the activation dtype
+  d_aux = F32(cast_act(F32(d_loss), act_dtype)
+              * cast_act(F32(hp.moe_loss_coef), act_dtype))
+  dlogits = gating_backward(aux["logits"], aux, hp.moe_gating, dgate[0],
+                            dgate[1], d_aux, importance, num_microbatches, z)
+  dwg = np.matmul(xg.reshape(-1, m_).T.astype(F32),
+                  dlogits.reshape(-1, e_)).astype(F32)
+  dx = dx + np.matmul(dlogits, wg_a.T.astype(F32))
+  return dict(dx=cast_act(dx, act_dtype).reshape(lead + (m_,)),
+              dw_gate=cast_act(dwg, act_dtype), dwi=dwi, dwo=dwo,
+              dlogits=dlogits, dgate=np.stack(dgate, -1), aux=aux)
 
 
 def moe_layer_v2(x, w_outer, w_inner, wi, wo, hp, train, act_dtype="float32",

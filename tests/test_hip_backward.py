@@ -1,0 +1,115 @@
+"""GPU parity of the backward C-ABI entry points against the CPU oracle's
+backward (itself pinned by central differences in tests/test_oracle.py)."""
+
+import numpy as np
+import pytest
+import torch
+
+from oracle import moe_oracle as O
+from tests import helpers as H
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def hip():
+  from mesh_amd import moe_hip
+  moe_hip.load_library()
+  return moe_hip
+
+
+def _hp(**kw):
+  base = dict(moe_second_policy_train="all", moe_second_policy_eval="all",
+              moe_switch_policy_train="argmax", moe_switch_policy_eval="argmax")
+  base.update(kw)
+  return O.default_hparams(**base)
+
+
+def run_backward(hip, x, w, hp, act_dtype, d_out, d_loss, nonpad, mb):
+  """The forward and backward call sequence of one v1 layer through the C ABI
+  (what MoEV1Operation and its gradient do), on [G, S, M] tokens."""
+  g, s, m = x.shape
+  e, hdim = hp.moe_num_experts, hp.moe_hidden_size
+  n = w["wo"].shape[-1]
+  c = O.expert_capacity(s, hp.moe_capacity_factor_train, e,
+                        hp.moe_min_expert_capacity)
+  xg = H.to_gpu(x, act_dtype)
+  wg, wi, wo = (H.to_gpu(O.cast_act(w[k], act_dtype), act_dtype)
+                for k in ("w_gate", "wi", "wo"))
+  imp = None if nonpad is None else H.to_gpu(nonpad, act_dtype)
+  wg_p = hip.pack_weights(wg.reshape(1, m, e), wg.dtype)
+  wi_p, wo_p = hip.pack_weights(wi, wi.dtype), hip.pack_weights(wo, wo.dtype)
+  logits = hip.router_logits(xg.reshape(1, g * s, m), wg.reshape(1, m, e),
+                             w_packed=wg_p).reshape(g, s, e)
+  gating = hp.moe_gating
+  z = hp.moe_z_loss if gating == "switch" else None
+  if gating == "top_2":
+    r = hip.top2_gating(logits, c, importance=imp, num_microbatches=mb)
+  else:
+    r = hip.switch_gating(logits, c, importance=imp, z_loss=z,
+                          num_microbatches=mb,
+                          slots_by_gate=gating == "switch_max")
+  expert_in = hip.dispatch(xg, r)
+  h = torch.empty((e, g * c, hdim), dtype=xg.dtype, device="cuda")
+  y = hip.expert_ffn(expert_in.reshape(e, g * c, m), wi_p, wo_p, "relu", h=h)
+  # backward
+  dout = H.to_gpu(d_out, act_dtype)
+  dy, dgate = hip.combine_backward(dout, y.reshape(e, g, c, n), r)
+  dxe, dwi, dwo = hip.expert_ffn_backward(
+      expert_in.reshape(e, g * c, m), h, dy.reshape(e, g * c, n), wi, wo, "relu")
+  dl = torch.tensor([d_loss], dtype=H.ACT_TORCH[act_dtype]).float().cuda()
+  scale = torch.tensor(hp.moe_loss_coef, dtype=H.ACT_TORCH[act_dtype]).item()
+  dlogits = hip.gating_backward(logits, r, dgate, dl, scale, router=gating,
+                                importance=imp, z_loss=z, num_microbatches=mb)
+  dwg = hip.router_backward_weights(xg.reshape(g * s, m),
+                                    dlogits.reshape(g * s, e))
+  dx = hip.dispatch_backward(dxe.reshape(e, g, c, m), r, s, dlogits,
+                             wg_p.reshape(e, m))
+  return dict(dx=H.to_np(dx), dw_gate=H.to_np(dwg), dwi=H.to_np(dwi),
+              dwo=H.to_np(dwo), dlogits=H.to_np(dlogits), dgate=H.to_np(dgate))
+
+
+CASES = [
+    # gating, G, S, M, H, E, cf, dtype, nonpadding
+    ("top_2", 2, 64, 16, 24, 4, 1.0, "float32", True),
+    ("top_2", 3, 50, 24, 40, 5, 1.25, "float32", False),
+    ("top_2", 2, 128, 64, 128, 8, 1.0, "bfloat16", True),
+    ("switch", 2, 64, 16, 24, 4, 1.0, "float32", True),
+    ("switch", 2, 128, 64, 128, 8, 1.25, "bfloat16", False),
+    ("switch_max", 2, 64, 16, 24, 4, 0.75, "float32", True),
+    ("top_2", 2, 256, 256, 512, 8, 1.0, "bfloat16", True),   # MFMA GEMM paths
+]
+
+
+@pytest.mark.parametrize("case", CASES, ids=[
+    "%s-%s-%d" % (c[0], c[7], i) for i, c in enumerate(CASES)])
+def test_backward_matches_oracle(hip, case):
+  gating, g, s, m, hdim, e, cf, act_dtype, use_np = case
+  rng = np.random.default_rng(71)
+  w = dict(w_gate=H.normal_weights(rng, (m, e), m),
+           wi=H.normal_weights(rng, (e, m, hdim), m),
+           wo=H.normal_weights(rng, (e, hdim, m), hdim))
+  x = H.safe_tokens(rng, g * s, m, w["w_gate"], act_dtype).reshape(g, s, m)
+  nonpad = (rng.random((g, s)) < 0.85).astype(np.float32) if use_np else None
+  d_out = O.cast_act(rng.standard_normal((g, s, m)).astype(np.float32), act_dtype)
+  d_loss, mb = 1.5, 2
+  hp = _hp(moe_gating=gating, moe_num_experts=e, moe_hidden_size=hdim,
+           moe_group_size=s, moe_capacity_factor_train=cf, moe_loss_coef=0.25,
+           moe_z_loss=0.1 if (gating == "switch" and use_np) else None)
+  want = O.moe_layer_v1_backward(x, w["w_gate"], w["wi"], w["wo"], hp, True,
+                                 act_dtype, d_out, d_loss, nonpadding=nonpad,
+                                 num_microbatches=mb)
+  got = run_backward(hip, x, w, hp, act_dtype, d_out, d_loss, nonpad, mb)
+  tol = H.value_tolerance(act_dtype)
+  np.testing.assert_allclose(got["dgate"], want["dgate"], rtol=1e-2 if
+                             act_dtype == "bfloat16" else 1e-4, atol=1e-3 if
+                             act_dtype == "bfloat16" else 1e-5)
+  scale = np.abs(want["dlogits"]).max()
+  np.testing.assert_allclose(got["dlogits"], want["dlogits"],
+                             rtol=2e-2 if act_dtype == "bfloat16" else 1e-3,
+                             atol=(1e-2 if act_dtype == "bfloat16" else 1e-5) * scale)
+  for k in ("dx", "dw_gate", "dwi", "dwo"):
+    ref = want[k].reshape(got[k].shape)
+    atol = tol["atol"] * max(1.0, np.abs(ref).max())
+    np.testing.assert_allclose(got[k], ref, rtol=tol["rtol"], atol=atol,
+                               err_msg=k)

@@ -651,3 +651,81 @@ def test_switch_golden_fixture():
   np.testing.assert_array_equal(r["kept_1"], np.array(gold["kept_1"], bool))
   np.testing.assert_allclose(r["gate_1"], np.array(gold["gate_1"]), rtol=1e-6)
   np.testing.assert_allclose(r["loss"], gold["loss"], rtol=1e-6)
+
+
+# ---- backward -------------------------------------------------------------------
+def _f64_layer(x, wg, wi, wo, aux, gating, m1, coef, mb, z_loss):
+  """Independent float64 forward of the v1 layer with the ROUTING HELD FIXED
+  (experts, kept masks and density counts taken from `aux`): a smooth function
+  of (x, wg, wi, wo) whose central differences pin the oracle's backward."""
+  g, s, _ = x.shape
+  e = wg.shape[1]
+  logits = x @ wg
+  p = scipy.special.softmax(logits, axis=-1)
+  rows = np.arange(g)[:, None], np.arange(s)[None, :]
+  i1, i2 = aux["index_1"], aux["index_2"]
+  k1, k2 = aux["kept_1"].astype(np.float64), aux["kept_2"].astype(np.float64)
+
+  def ffn(idx):
+    h = np.maximum(np.einsum("gsm,gsmh->gsh", x, wi[idx]), 0.0)
+    return np.einsum("gsh,gshn->gsn", h, wo[idx])
+  onehot1 = (i1[..., None] == np.arange(e)).astype(np.float64)
+  if gating == "top_2":
+    g1 = p[rows + (i1,)] * m1
+    g2 = p[rows + (i2,)] * (1.0 - (i2 == i1) * m1)
+    den = g1 + g2 + 1e-9
+    out = ((g1 / den * k1)[..., None] * ffn(i1)
+           + (g2 / den * k2)[..., None] * ffn(i2))
+    density = (onehot1 * m1[..., None]).mean(1)
+    proxy = (p * m1[..., None]).mean(1)
+    aux_loss = (proxy * density).mean() * e * e / mb
+  else:
+    out = (p[rows + (i1,)] * m1 * k1)[..., None] * ffn(i1)
+    density = onehot1.mean(1)
+    proxy = p.mean(1)
+    aux_loss = (proxy[:, :, None] * m1[:, None, :] * density[:, :, None]
+                ).mean() * e * e / mb
+    if z_loss is not None:
+      lse = scipy.special.logsumexp(logits, axis=-1)
+      aux_loss = aux_loss + z_loss * (lse ** 2 * m1).sum() / (m1.sum() * mb)
+  return out, aux_loss * coef
+
+
+@pytest.mark.parametrize("gating", ["top_2", "switch", "switch_max"])
+def test_backward_against_central_differences(gating):
+  rng = np.random.default_rng(61)
+  b, l, m, h, e, group = 2, 24, 6, 10, 4, 24
+  x = rng.standard_normal((b, l, m)).astype(np.float32)
+  wg = rng.standard_normal((m, e)).astype(np.float32)
+  wi = (rng.standard_normal((e, m, h)) / 2).astype(np.float32)
+  wo = (rng.standard_normal((e, h, m)) / 3).astype(np.float32)
+  nonpad = (rng.random((b, l)) < 0.8).astype(np.float32)
+  d_out = rng.standard_normal((b, l, m)).astype(np.float32)
+  d_loss, mb = 1.7, 2
+  hp = _hp(moe_gating=gating, moe_num_experts=e, moe_hidden_size=h,
+           moe_group_size=group, moe_capacity_factor_train=1.2,
+           moe_min_expert_capacity=2, moe_loss_coef=0.5,
+           moe_switch_policy_train="argmax",
+           moe_z_loss=0.3 if gating == "switch" else None)
+  got = O.moe_layer_v1_backward(x, wg, wi, wo, hp, True, "float32", d_out,
+                                d_loss, nonpadding=nonpad, num_microbatches=mb)
+  aux = got["aux"]
+  assert not (aux["kept_1"] | aux["kept_2"]).all()     # drops are exercised
+  m1 = (nonpad.reshape(aux["kept_1"].shape) == 1).astype(np.float64)
+  z = hp.moe_z_loss if gating == "switch" else None
+
+  def scalar(xv, wgv, wiv, wov):
+    out, loss = _f64_layer(xv.reshape(b, l, m), wgv, wiv, wov, aux, gating, m1,
+                           0.5, mb, z)
+    return (out * d_out.reshape(out.shape)).sum() + d_loss * loss
+  base = [a.astype(np.float64) for a in (x.reshape(b, l, m), wg, wi, wo)]
+  grads = [got["dx"].reshape(b, l, m), got["dw_gate"], got["dwi"], got["dwo"]]
+  eps = 1e-6
+  for which in range(4):
+    for trial in range(3):
+      d = rng.standard_normal(base[which].shape)
+      plus = [a + eps * d if i == which else a for i, a in enumerate(base)]
+      minus = [a - eps * d if i == which else a for i, a in enumerate(base)]
+      fd = (scalar(*plus) - scalar(*minus)) / (2 * eps)
+      an = float((grads[which].astype(np.float64) * d).sum())
+      assert abs(fd - an) <= 2e-4 * max(1.0, abs(fd)), (which, trial, fd, an)
