@@ -399,6 +399,16 @@ class Operation(object):
         ", ".join(t.to_string for t in self._inputs),
         ", ".join(t.to_string for t in self._outputs))
 
+  @property
+  def has_gradient(self):
+    """Operations with a floating-point first output back-propagate
+    (mesh_tensorflow/ops.py:1478-1482)."""
+    return bool(self._outputs) and self._outputs[0].dtype.is_floating_point
+
+  def gradient(self, unused_grad_ys):
+    raise NotImplementedError(
+        "Gradient not implemented for %s" % type(self).__name__)
+
   def lower(self, lowering):
     raise NotImplementedError("Lower not implemented")
 
@@ -602,11 +612,20 @@ class SlicewiseOperation(Operation):
   def __init__(self, tf_fn, inputs, output_shapes, output_dtypes,
                splittable_dims=None, grad_function=None, name=None):
     super(SlicewiseOperation, self).__init__(inputs, name=name or "slicewise")
-    del splittable_dims, grad_function
+    del splittable_dims
+    self._grad_function = grad_function
     self._tf_fn = tf_fn
     self._outputs = [Tensor(self, convert_to_shape(s), d, index=i)
                      for i, (s, d) in enumerate(zip(output_shapes,
                                                     output_dtypes))]
+
+  @property
+  def has_gradient(self):
+    return self._grad_function is not None
+
+  def gradient(self, grad_ys):
+    # the reference calls grad_function(op, *grad_ys) (ops.py:1705-1708)
+    return self._grad_function(self, *grad_ys)
 
   def lower(self, lowering):
     mesh_impl = lowering.mesh_impl(self)
@@ -637,7 +656,9 @@ def cwise(tf_fn, xs, output_dtype=None, grad_function=None, name=None):
 def cast(x, dtype, name="cast"):
   if dtype == x.dtype:
     return x
-  return cwise(lambda t: t.to(dtype), [x], output_dtype=dtype, name=name)
+  # the gradient of a cast casts back (mesh_tensorflow/ops.py:1945-1962)
+  return cwise(lambda t: t.to(dtype), [x], output_dtype=dtype, name=name,
+               grad_function=lambda op, dy: [cast(dy, op.inputs[0].dtype)])
 
 
 def to_float(x, name="to_float"):
@@ -660,7 +681,8 @@ def add(x1, x2, output_shape=None, name=None):
   del output_shape
   if not isinstance(x2, Tensor):
     c = _scalar_in(x1.dtype, x2)
-    return cwise(lambda t: t + c, [x1], name=name or "scalar_add")
+    return cwise(lambda t: t + c, [x1], name=name or "scalar_add",
+                 grad_function=lambda op, dy: [dy])
   if not isinstance(x1, Tensor):
     return add(x2, x1)
   big, small = (x1, x2) if x1.shape.ndims >= x2.shape.ndims else (x2, x1)
@@ -675,8 +697,12 @@ def add(x1, x2, output_shape=None, name=None):
 
   def fn(a, b):
     return a + b.reshape(view).to(a.dtype)
+  grad = None
+  if big.shape == small.shape and big.dtype == small.dtype:
+    grad = lambda op, dy: [dy, dy]     # what accumulating gradients needs
   return slicewise(fn, [big, small], output_shape=big.shape,
-                   output_dtype=big.dtype, name=name or "add")
+                   output_dtype=big.dtype, name=name or "add",
+                   grad_function=grad)
 
 
 def multiply(x1, x2, output_shape=None, name=None):
@@ -688,7 +714,8 @@ def multiply(x1, x2, output_shape=None, name=None):
   if isinstance(x2, Tensor):
     raise NotImplementedError("Tensor * Tensor is not part of this subset")
   c = _scalar_in(x1.dtype, x2)
-  return cwise(lambda t: t * c, [x1], name=name or "scalar_mul")
+  return cwise(lambda t: t * c, [x1], name=name or "scalar_mul",
+               grad_function=lambda op, dy: [multiply(dy, x2)])
 
 
 class ReshapeOperation(Operation):
@@ -701,6 +728,9 @@ class ReshapeOperation(Operation):
       raise ValueError("Cannot reshape Tensor %s to shape %s - sizes differ."
                        % (x, new_shape))
     self._outputs = [Tensor(self, new_shape, x.dtype)]
+
+  def gradient(self, grad_ys):
+    return [reshape(grad_ys[0], self.inputs[0].shape)]
 
   def lower(self, lowering):
     mesh_impl = lowering.mesh_impl(self)
@@ -860,6 +890,36 @@ def get_variable(mesh, name, shape, dtype=float32, master_dtype=None,
     raise ValueError("Variable %s already exists" % full)
   return Variable(mesh, name, convert_to_shape(shape), dtype, initializer,
                   trainable, **kwargs).outputs[0]
+
+
+def gradients(ys, xs, grad_ys=None, operations=None):
+  """mtf.gradients (mesh_tensorflow/ops.py:5254-5291): gradient Tensors of the
+  sum of `ys` (weighted by grad_ys) w.r.t. each of `xs`, built by walking the
+  graph backwards and calling Operation.gradient.  None for an x nothing
+  depends on."""
+  if operations is None:
+    operations = ys[0].graph.operations
+  if not grad_ys:
+    grad_ys = [Constant(y.mesh, 1.0, y.shape, y.dtype).outputs[0] for y in ys]
+  downstream = set(xs)
+  for op in operations:
+    if op.has_gradient:
+      if set(op.inputs) & downstream:
+        downstream |= set(op.outputs)
+  tensor_to_gradient = {y: g for y, g in zip(ys, grad_ys) if g is not None}
+  for op in operations[::-1]:
+    grad_outputs = [tensor_to_gradient.get(out) for out in op.outputs]
+    if (op.has_gradient and any(g is not None for g in grad_outputs)
+        and (set(op.inputs) & downstream)):
+      with variable_scope(op.name + "/gradients"):
+        input_grads = op.gradient(grad_outputs)
+        for inp, grad in zip(op.inputs, input_grads):
+          if inp in downstream and grad is not None:
+            if inp in tensor_to_gradient:
+              tensor_to_gradient[inp] = tensor_to_gradient[inp] + grad
+            else:
+              tensor_to_gradient[inp] = grad
+  return [tensor_to_gradient.get(x, None) for x in xs]
 
 
 def relu(x, name="relu"):

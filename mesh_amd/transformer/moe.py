@@ -118,12 +118,17 @@ class _GatingSpec(object):
     self.use_second_place_loss = bool(hparams.moe_use_second_place_loss)
     self.num_microbatches = num_microbatches
 
+  router = "top_2"
+  z_loss = None
+
   def route(self, x, w, w_packed, group_size, num_experts, capacity,
-            importance=None, importance_from_slot_gate=False):
+            importance=None, importance_from_slot_gate=False,
+            want_logits=False):
     """Router projection + gating of x [B, T, M] with routers w [B, M, E]
     (w_packed [B, E, M]); the B*T tokens form groups of group_size.  One fused
     launch sequence where the library has a kernel for the case, otherwise the
-    projection and the gating as two calls."""
+    projection and the gating as two calls.  Returns the Routing, and the
+    float32 logits [G, S, E] too if want_logits."""
     b, t, _ = x.shape
     groups = b * t // group_size
     if moe_hip.fused_gating_supported(x, num_experts, group_size):
@@ -136,10 +141,12 @@ class _GatingSpec(object):
           policy=self.policy, threshold=self.threshold,
           use_second_place_loss=self.use_second_place_loss,
           num_microbatches=self.num_microbatches, second_uniform=uniform,
-          importance_from_slot_gate=importance_from_slot_gate)
+          importance_from_slot_gate=importance_from_slot_gate,
+          want_logits=want_logits)
     logits = moe_hip.router_logits(x, w, w_packed=w_packed)
-    return self.run(logits.reshape(groups, group_size, num_experts), capacity,
-                    importance, importance_from_slot_gate)
+    logits = logits.reshape(groups, group_size, num_experts)
+    r = self.run(logits, capacity, importance, importance_from_slot_gate)
+    return (r, logits) if want_logits else r
 
   def run(self, logits, capacity, importance=None,
           importance_from_slot_gate=False):
@@ -182,8 +189,12 @@ class _SwitchGatingSpec(object):
       self.z_loss = float(hparams.moe_z_loss)
     self.num_microbatches = num_microbatches
 
+  router = "switch"
+  use_second_place_loss = False
+
   def route(self, x, w, w_packed, group_size, num_experts, capacity,
-            importance=None, importance_from_slot_gate=False):
+            importance=None, importance_from_slot_gate=False,
+            want_logits=False):
     """Same contract as _GatingSpec.route."""
     assert not importance_from_slot_gate
     b, t, _ = x.shape
@@ -192,13 +203,14 @@ class _SwitchGatingSpec(object):
       return moe_hip.router_switch_gating(
           x, w_packed, group_size, capacity, importance=importance,
           z_loss=self.z_loss, num_microbatches=self.num_microbatches,
-          slots_by_gate=self.slots_by_gate)
+          slots_by_gate=self.slots_by_gate, want_logits=want_logits)
     logits = moe_hip.router_logits(x, w, w_packed=w_packed)
-    return moe_hip.switch_gating(
-        logits.reshape(groups, group_size, num_experts), capacity,
-        importance=importance, z_loss=self.z_loss,
+    logits = logits.reshape(groups, group_size, num_experts)
+    r = moe_hip.switch_gating(
+        logits, capacity, importance=importance, z_loss=self.z_loss,
         num_microbatches=self.num_microbatches,
         slots_by_gate=self.slots_by_gate)
+    return (r, logits) if want_logits else r
 
 
 def _packed(lowering, kernel_tensor, dtype):
@@ -221,9 +233,29 @@ class MoEV1Operation(mtf.Operation):
     self._gating = gating
     self._activation = activation
     self._num_experts = wi.shape.dims[0].size
+    self._save_for_backward = False
     out_shape = mtf.Shape(inputs.shape.dims[:-1] + [output_dim])
     self._outputs = [mtf.Tensor(self, out_shape, inputs.dtype, index=0),
                      mtf.Tensor(self, mtf.Shape([]), inputs.dtype, index=1)]
+
+  def gradient(self, grad_ys):
+    """Gradients w.r.t. (inputs, gate kernel, wi, wo[, importance]) from those
+    of (outputs, loss); importance carries none."""
+    if self._gating.use_second_place_loss:
+      raise NotImplementedError(
+          "backward of the second-place loss is not implemented")
+    if self._activation not in ("relu", "linear"):
+      raise NotImplementedError(
+          "backward of expert activation %r is not implemented (the "
+          "pre-activation is not kept)" % (self._activation,))
+    self._save_for_backward = True
+    d_out, d_loss = grad_ys
+    if d_out is None:
+      d_out = mtf.zeros(self.mesh, self.outputs[0].shape, self.outputs[0].dtype)
+    if d_loss is None:
+      d_loss = mtf.zeros(self.mesh, mtf.Shape([]), self.outputs[1].dtype)
+    grads = MoEV1GradOperation(self, d_out, d_loss).outputs
+    return grads + [None] * (len(self.inputs) - 4)
 
   def lower(self, lowering):
     mesh_impl = lowering.mesh_impl(self)
@@ -237,16 +269,31 @@ class MoEV1Operation(mtf.Operation):
     e_, c_ = self._num_experts, self._capacity
     groups = o_ * g_
 
+    save = self._save_for_backward
+    saved = {}
+
     def fn(x_s, wg_s, imp_s=None):
       xg = x_s.reshape(groups, s_, m_)
       if imp_s is not None:
         imp_s = imp_s.reshape(groups, s_)
       r = self._gating.route(xg.reshape(1, groups * s_, m_),
-                             wg_s.reshape(1, m_, e_), wg_p, s_, e_, c_, imp_s)
+                             wg_s.reshape(1, m_, e_), wg_p, s_, e_, c_, imp_s,
+                             want_logits=save)
+      logits = None
+      if save:
+        r, logits = r
       expert_in = moe_hip.dispatch(xg, r)
+      h = None
+      if save:
+        h = torch.empty((e_, groups * c_, wi_p.shape[1]), dtype=dt,
+                        device=xg.device)
       y = moe_hip.expert_ffn(expert_in.reshape(e_, groups * c_, m_), wi_p,
-                             wo_p, self._activation)
+                             wo_p, self._activation, h=h)
       out = moe_hip.combine(y.reshape(e_, groups, c_, n_), r, s_)
+      if save:
+        # what the gradient operation reads (activations of this step)
+        saved.update(x=xg, routing=r, logits=logits, importance=imp_s,
+                     expert_in=expert_in, h=h, y=y, w_gate_packed=wg_p)
       return out.reshape(o_, g_, s_, n_), r.loss.to(dt).reshape(())
 
     args = [lowering.tensors[x], lowering.tensors[w_gate]]
@@ -255,6 +302,70 @@ class MoEV1Operation(mtf.Operation):
     out, loss = mesh_impl.slicewise(fn, *args)
     lowering.set_tensor_lowering(self.outputs[0], out)
     lowering.set_tensor_lowering(self.outputs[1], loss)
+    lowering.operations[self] = saved
+
+
+class MoEV1GradOperation(mtf.Operation):
+  """Backward of MoEV1Operation: (d outputs, d loss) -> gradients of the
+  tokens and of the three kernels, in the activation dtype.
+
+  The reference gets these from mtf.gradients over the layer's einsums
+  (mesh_tensorflow/ops.py:5254-5291, :2846-2854); here they are one call
+  sequence into the HIP library on the activations the forward operation
+  kept."""
+
+  def __init__(self, forward, d_out, d_loss, name="moe_v1_grad"):
+    super(MoEV1GradOperation, self).__init__(
+        forward.inputs[:4] + [d_out, d_loss], name=name)
+    self._forward = forward
+    self._outputs = [mtf.Tensor(self, t.shape, t.dtype, index=i)
+                     for i, t in enumerate(forward.inputs[:4])]
+
+  @property
+  def has_gradient(self):
+    return False
+
+  def lower(self, lowering):
+    mesh_impl = lowering.mesh_impl(self)
+    fwd = self._forward
+    x, w_gate, wi, wo = fwd.inputs[:4]
+    o_, g_, s_, m_ = x.shape.to_integer_list
+    e_, c_ = fwd._num_experts, fwd._capacity
+    n_ = fwd.outputs[0].shape.dims[-1].size
+    groups = o_ * g_
+    gating = fwd._gating
+
+    def fn(wi_s, wo_s, dout_s, dloss_s):
+      sv = lowering.operations[fwd]
+      if not sv:
+        raise ValueError("the forward operation kept no activations: build "
+                         "the gradient before lowering the graph")
+      r = sv["routing"]
+      dy, dgate = moe_hip.combine_backward(
+          dout_s.reshape(groups, s_, n_).contiguous(),
+          sv["y"].reshape(e_, groups, c_, n_), r)
+      dxe, dwi, dwo = moe_hip.expert_ffn_backward(
+          sv["expert_in"].reshape(e_, groups * c_, m_), sv["h"],
+          dy.reshape(e_, groups * c_, n_), wi_s, wo_s, fwd._activation)
+      dlogits = moe_hip.gating_backward(
+          sv["logits"], r, dgate, dloss_s.reshape(1).float(), 1.0,
+          router=gating.router,
+          importance=sv["importance"], z_loss=gating.z_loss,
+          num_microbatches=gating.num_microbatches)
+      dwg = moe_hip.router_backward_weights(
+          sv["x"].reshape(groups * s_, m_), dlogits.reshape(groups * s_, e_))
+      dx = moe_hip.dispatch_backward(
+          dxe.reshape(e_, groups, c_, m_), r, s_, dlogits,
+          sv["w_gate_packed"].reshape(e_, m_))
+      return dx.reshape(o_, g_, s_, m_), dwg, dwi, dwo
+
+    ins = self.inputs
+    outs = mesh_impl.slicewise(fn, lowering.tensors[ins[2]],
+                               lowering.tensors[ins[3]],
+                               lowering.tensors[ins[4]],
+                               lowering.tensors[ins[5]])
+    for t, v in zip(self.outputs, outs):
+      lowering.set_tensor_lowering(t, v)
 
 
 def transformer_moe_layer_v1(

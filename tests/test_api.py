@@ -298,3 +298,35 @@ def test_product_does_not_import_the_oracle():
       if f.endswith((".py", ".hip", ".h", ".cpp")):
         text = open(os.path.join(dirpath, f)).read()
         assert "oracle" not in text, os.path.join(dirpath, f)
+
+
+def test_gradients_builds_the_backward_operation():
+  """mtf.gradients (mesh_tensorflow/ops.py:5254-5291) over the layer: one
+  gradient per requested tensor with that tensor's shape and dtype, None for a
+  tensor nothing depends on, and the forward operation told to keep its
+  activations.  Graph construction only, no GPU."""
+  graph, mesh, x, dims = graph_input()
+  with mtf.variable_scope("moe"):
+    y, loss = moe.transformer_moe_layer_v1(
+        x, dims[-1], hparams(), True, mtf.VariableDType(torch.float32))
+  variables = [v.outputs[0] for v in graph.trainable_variables]
+  other = mtf.import_tf_tensor(mesh, torch.zeros(3), mtf.Shape([mtf.Dimension("z", 3)]))
+  grads = mtf.gradients([y, loss], [x] + variables + [other])
+  assert grads[-1] is None
+  for t, g in zip([x] + variables, grads[:-1]):
+    assert g.shape == t.shape and g.dtype == t.dtype
+  fwd = [o for o in graph.operations if isinstance(o, moe.MoEV1Operation)][0]
+  assert fwd._save_for_backward
+  assert any(isinstance(o, moe.MoEV1GradOperation) for o in graph.operations)
+  with pytest.raises(NotImplementedError, match="second-place loss"):
+    g2, _, x2, d2 = graph_input()
+    y2, l2 = moe.transformer_moe_layer_v1(
+        x2, d2[-1], hparams(moe_use_second_place_loss=True), True,
+        mtf.VariableDType(torch.float32))
+    mtf.gradients([y2], [x2])
+  with pytest.raises(NotImplementedError, match="Gradient not implemented"):
+    g3, _, x3, d3 = graph_input()
+    y3, _ = moe.transformer_moe_layer_v2(
+        x3, d3[-1], hparams(moe_num_experts=[2, 2]), True,
+        mtf.VariableDType(torch.float32))
+    mtf.gradients([y3], [x3])

@@ -355,3 +355,72 @@ def test_v1_switch_max_matches_oracle():
   got, got_loss, _, _ = run_v1(x, w, hp, False, "float32")
   np.testing.assert_allclose(got, want, **H.value_tolerance("float32"))
   np.testing.assert_allclose(got_loss, want_loss, rtol=1e-4)
+
+
+# ---- gradients through the mtf-shaped API -------------------------------------
+@pytest.mark.parametrize("case", [
+    ("top_2", "float32", 101), ("top_2", "bfloat16", 102),
+    ("switch", "float32", 103), ("switch_max", "float32", 104)],
+    ids=lambda c: "%s-%s" % (c[0], c[1]))
+def test_v1_gradients_match_oracle(case):
+  """mtf.gradients over the layer (outputs and loss) against the oracle's
+  backward, which central differences pin in tests/test_oracle.py."""
+  gating, act_dtype, seed = case
+  b, l, m, hdim, e, group = 2, 64, 32, 48, 4, 32
+  rng = np.random.default_rng(seed)
+  w = dict(w_gate=H.normal_weights(rng, (m, e), m),
+           wi=H.normal_weights(rng, (e, m, hdim), m),
+           wo=H.normal_weights(rng, (e, hdim, m), hdim))
+  x = H.safe_tokens(rng, b * l, m, w["w_gate"], act_dtype).reshape(b, l, m)
+  nonpad = (rng.random((b, l)) < 0.85).astype(np.float32)
+  d_out = O.cast_act(rng.standard_normal((b, l, m)).astype(np.float32), act_dtype)
+  kw = dict(moe_num_experts=e, moe_hidden_size=hdim, moe_group_size=group,
+            moe_capacity_factor_train=1.0, moe_loss_coef=0.25)
+  if gating != "top_2":
+    kw.update(SWITCH_HP, moe_gating=gating,
+              moe_z_loss=0.1 if gating == "switch" else None)
+  hp, ohp = make_hparams(**kw)
+  dt = H.ACT_TORCH[act_dtype]
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  dims = [mtf.Dimension("batch", b), mtf.Dimension("length", l),
+          mtf.Dimension("d_model", m)]
+  xt = mtf.import_tf_tensor(mesh, torch.from_numpy(x).to(dt), mtf.Shape(dims))
+  npad = mtf.import_tf_tensor(mesh, torch.from_numpy(nonpad).to(dt),
+                              mtf.Shape(dims[:2]))
+  with mtf.variable_scope("moe"):
+    y, loss = moe.transformer_moe_layer_v1(
+        xt, dims[-1], hp, True, mtf.VariableDType(torch.float32, torch.float32, dt),
+        nonpadding=npad, num_microbatches=2)
+  variables = graph.trainable_variables
+  assert [v.name.split("/")[-2] for v in variables][1:] == ["wi", "wo"]
+  dyt = mtf.import_tf_tensor(mesh, torch.from_numpy(d_out).to(dt), mtf.Shape(dims))
+  dlt = mtf.import_tf_tensor(mesh, torch.tensor(1.5, dtype=dt), mtf.Shape([]))
+  grads = mtf.gradients([y, loss], [xt] + [v.outputs[0] for v in variables],
+                        grad_ys=[dyt, dlt])
+  router = {"switch": "switch_gating", "switch_max": "switch_max_gating"}.get(
+      gating, "top_2_gating")
+  init = {"moe/%s/kernel" % router: w["w_gate"], "moe/wi/kernel": w["wi"],
+          "moe/wo/kernel": w["wo"]}
+  lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()}, initial_values=init)
+  got = [H.to_np(lowering.export_to_tf_tensor(g)) for g in grads]
+  want = O.moe_layer_v1_backward(x, w["w_gate"], w["wi"], w["wo"], ohp, True,
+                                 act_dtype, d_out, 1.5, nonpadding=nonpad,
+                                 num_microbatches=2)
+  assert not (want["aux"]["kept_1"] | want["aux"]["kept_2"]).all()
+  tol = H.value_tolerance(act_dtype)
+  for g_, k in zip(got, ("dx", "dw_gate", "dwi", "dwo")):
+    ref = want[k].reshape(g_.shape)
+    np.testing.assert_allclose(
+        g_, ref, rtol=tol["rtol"], atol=tol["atol"] * max(1.0, np.abs(ref).max()),
+        err_msg=k)
+  # a second step re-runs forward and backward on new tokens
+  x2 = H.safe_tokens(rng, b * l, m, w["w_gate"], act_dtype).reshape(b, l, m)
+  lowering.run({xt: torch.from_numpy(x2).to(dt).cuda()})
+  want2 = O.moe_layer_v1_backward(x2, w["w_gate"], w["wi"], w["wo"], ohp, True,
+                                  act_dtype, d_out, 1.5, nonpadding=nonpad,
+                                  num_microbatches=2)
+  got2 = H.to_np(lowering.export_to_tf_tensor(grads[2]))
+  np.testing.assert_allclose(
+      got2, want2["dwi"], rtol=tol["rtol"],
+      atol=tol["atol"] * max(1.0, np.abs(want2["dwi"]).max()))
