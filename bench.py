@@ -88,9 +88,11 @@ def normal_init(fan_in, seed):
   return init
 
 
-def build(cfg, device):
+def build(cfg, device, backward=False):
   """Builds the graph for `cfg` through the mtf-shaped API and lowers it once.
-  Returns (lowering, x Tensor, y Tensor, loss Tensor)."""
+  With backward=True the graph also holds mtf.gradients of (outputs, loss)
+  w.r.t. the tokens and the kernels.  Returns (lowering, x Tensor, y Tensor,
+  loss Tensor)."""
   import torch
   import mesh_amd as mtf
   from mesh_amd.transformer import moe
@@ -139,6 +141,13 @@ def build(cfg, device):
       w[0] = (3.0 * perm.double() ** -1.2).to(dtype)
       return w
     init[router] = skewed
+  if backward:
+    d_out = mtf.import_tf_tensor(
+        mesh, torch.randn(x_val.shape, generator=gen, device=device,
+                          dtype=torch.float32).to(dt), mtf.Shape(dims))
+    mtf.gradients([y, loss],
+                  [x] + [v.outputs[0] for v in graph.trainable_variables],
+                  grad_ys=[d_out, None])
   lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl(device=device)},
                           initial_values=init)
   return lowering, x, y, loss
@@ -161,6 +170,13 @@ def stage_model(cfg, kept_pairs, slots):
       "dispatch": dict(bytes=t * m * b + r * m * b + 18 * t),
       "combine": dict(bytes=r * m * b + t * m * b + 26 * t),
       "expert_ffn": dict(flops=4 * r * m * h, padded_flops=4 * slots * m * h),
+      # backward (only timed with --backward)
+      "combine_backward": dict(bytes=t * m * b + 2 * r * m * b + 34 * t),
+      "dispatch_backward": dict(bytes=r * m * b + t * m * b + t * e * 4 + 26 * t),
+      "gating_backward": dict(bytes=t * (8 * e + 18)),
+      "router_backward_weights": dict(bytes=t * m * b + t * e * 4),
+      "expert_ffn_backward": dict(flops=8 * r * m * h,
+                                  padded_flops=8 * slots * m * h),
   }
 
 
@@ -219,6 +235,9 @@ def main():
   ap.add_argument("--gating", default="top_2", choices=["top_2", "switch"],
                   help="router of the v1 configs (the benchmark definition "
                        "uses top_2)")
+  ap.add_argument("--backward", action="store_true",
+                  help="time forward + backward (v1 configs); the metric is "
+                       "then named accordingly and is not the benchmark's")
   ap.add_argument("--no-cpu-baseline", action="store_true")
   args = ap.parse_args()
   if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -238,7 +257,10 @@ def main():
     cfg["name"] += ", %s gating" % args.gating
   device = torch.device("cuda:0")
   torch.cuda.set_device(device)
-  lowering, x, y, loss = build(cfg, device)   # first execution
+  if args.backward and cfg["layer"] != "v1":
+    print("--backward applies to the v1 configs only", file=sys.stderr)
+    sys.exit(2)
+  lowering, x, y, loss = build(cfg, device, args.backward)   # first execution
   for _ in range(args.warmup):
     lowering.run()
   torch.cuda.synchronize()
@@ -255,7 +277,8 @@ def main():
   out_ok = bool(torch.isfinite(lowering.export_to_tf_tensor(y).float()).all())
 
   result = {
-      "metric": "MoE layer fwd tokens/sec @1 GPU",
+      "metric": ("MoE layer fwd+bwd tokens/sec @1 GPU" if args.backward
+                 else "MoE layer fwd tokens/sec @1 GPU"),
       "value": tokens / (ms_per_step * 1e-3), "unit": "tokens/s",
       "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
       "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
@@ -294,6 +317,13 @@ def main():
         "padded_frac": (model["expert_ffn"]["padded_flops"] / 2
                         / (ffn_ms / 2 * 1e-3) / 1e12) / peak}
     result["stages"] = per_stage
+    if args.backward:
+      bw_ms = stages["expert_ffn_backward"][1] / args.steps
+      bw = model["expert_ffn_backward"]
+      per_stage["expert_ffn_backward"].update(
+          TFLOPs=bw["flops"] / (bw_ms * 1e-3) / 1e12,
+          frac_mfma_peak=bw["flops"] / (bw_ms * 1e-3) / 1e12 / peak,
+          padded_frac=bw["padded_flops"] / (bw_ms * 1e-3) / 1e12 / peak)
     result["config"].update(kept_pairs=kept, slots=slots,
                             capacity=r.capacity)
   else:
@@ -301,7 +331,7 @@ def main():
     result["stages"] = {k: {"ms_per_step": v[1] / args.steps,
                             "launches_per_step": v[0] / args.steps}
                         for k, v in stages.items()}
-  result["cpu_baseline"] = (None if args.no_cpu_baseline
+  result["cpu_baseline"] = (None if (args.no_cpu_baseline or args.backward)
                             else cpu_baseline(cfg))
   print(json.dumps(result))
 
