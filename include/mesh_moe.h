@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 3
+#define MESH_MOE_ABI_VERSION 4
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -235,6 +235,62 @@ int mesh_moe_expert_ffn(const void* expert_in, const void* wi_packed,
 int mesh_moe_combine(const void* y, const int32_t* idx, const int32_t* pos,
                      const float* gate, const uint8_t* kept, void* out, int G,
                      int S, int E, int C, int N, int dtype, void* stream);
+
+/*
+ * ---------------------------------------------------------------------------
+ * Expert-selection ("expert choice") gating: every expert picks, per group,
+ * the C tokens it likes best (_expert_selection_gating,
+ * transformer/moe.py:1057-1173).  A token can sit in the slots of several
+ * experts or of none, so the record is per slot:
+ *   slot_token  [G,E,C] int32    token (index within the group) of each slot
+ *   slot_weight [G,E,C] float32  its combine weight before the dtype cast
+ *   tok_slot    [G,S,E] int16    slot the token holds at expert e, -1 if none
+ * ---------------------------------------------------------------------------
+ */
+
+/* Bytes of scratch mesh_moe_expert_choice_gating needs. */
+size_t mesh_moe_expert_choice_workspace_bytes(int G, int S, int E, int C);
+
+/*
+ * Gating from router logits (transformer/moe.py:1092-1147): -1e9 on the logits
+ * of tokens with importance 0, softmax over the GROUP dim, per (group, expert)
+ * the C largest probabilities in descending order with equal ones in token
+ * order (top_k, ops.py:4934-4942), weights divided by max(#experts that chose
+ * the token, 1) if `normalize`, and the loss
+ * mean(mean_e(p)^2 * (importance == 1) * sum_s importance) * S.
+ *   logits [G,S,E] float32; importance [G,S] of importance_dtype or NULL
+ *   (NULL = all ones; the reference requires it, moe.py:1138-1140)
+ *   loss [1] float32 before moe_loss_coef
+ * Limits: C <= S <= 32768.
+ */
+int mesh_moe_expert_choice_gating(const float* logits, const void* importance,
+                                  int importance_dtype, int G, int S, int E,
+                                  int C, int normalize, int num_microbatches,
+                                  int32_t* slot_token, float* slot_weight,
+                                  int16_t* tok_slot, float* loss,
+                                  void* workspace, size_t workspace_bytes,
+                                  void* stream);
+
+/*
+ * Dispatch by slot: expert_in[e,g,c,:] = x[g, slot_token[g,e,c], :]
+ * (transformer/moe.py:443-447 with the one-hot dispatch tensor of :1105-1106,
+ * which is 1 for every slot whatever its weight, :1169-1170).
+ *   x [G,S,M] dtype; expert_in [E,G,C,M] dtype
+ */
+int mesh_moe_slot_dispatch(const void* x, const int32_t* slot_token,
+                           void* expert_in, int G, int S, int E, int C, int M,
+                           int dtype, void* stream);
+
+/*
+ * Combine by slot: out[g,s,:] = sum over the experts e that chose token s of
+ * w * y[e,g,tok_slot[g,s,e],:], w the activation-dtype-rounded slot weight;
+ * float32 accumulate in expert order, one rounding; zero rows for tokens
+ * nobody chose (transformer/moe.py:509-510).
+ *   y [E,G,C,N] dtype; out [G,S,N] dtype
+ */
+int mesh_moe_slot_combine(const void* y, const int16_t* tok_slot,
+                          const float* slot_weight, void* out, int G, int S,
+                          int E, int C, int N, int dtype, void* stream);
 
 /*
  * ---------------------------------------------------------------------------

@@ -9,7 +9,8 @@ import sys
 from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-SOURCES = ["abi.hip", "route.hip", "dispatch.hip", "ffn.hip", "backward.hip"]
+SOURCES = ["abi.hip", "route.hip", "dispatch.hip", "ffn.hip", "backward.hip",
+           "expert_choice.hip"]
 LIB_NAME = "libmesh_moe_hip.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)
 
@@ -32,7 +33,7 @@ def _compile(src):
 def build_library(verbose=True):
   """Compiles every kernel source and links the shared library in-tree."""
   os.makedirs(os.path.join(HERE, "build"), exist_ok=True)
-  with ThreadPoolExecutor(max_workers=5) as pool:
+  with ThreadPoolExecutor(max_workers=6) as pool:
     objs = list(pool.map(_compile, SOURCES))
   cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB_PATH]
   subprocess.run(cmd + objs, check=True, cwd=HERE)

@@ -1,0 +1,350 @@
+// Expert-selection ("expert choice") gating for gfx950: every expert picks, per
+// group, the `capacity` tokens it likes best
+// (mesh_tensorflow/transformer/moe.py:1057-1173, _expert_selection_gating).
+//
+// A token can sit in the slots of several experts or of none, so the routing
+// record is per SLOT, not per token:
+//   slot_token  [G,E,C] int32   token (index within the group) of each slot
+//   slot_weight [G,E,C] float32 combine weight of that slot
+//   tok_slot    [G,S,E] int16   slot the token holds at expert e, -1 if none
+// and the dispatch / combine einsums (moe.py:443-447, :509-510) become a gather
+// per slot and a sum over the (at most E) slots of a token.
+#include "common.h"
+
+namespace mesh_moe {
+
+struct ChoiceParams {
+  int G, S, E, C;
+  int normalize;  // divide by the number of experts that chose the token
+  int num_microbatches;
+};
+
+__global__ void choice_clear_kernel(int32_t* num_routed, int64_t n_tok,
+                                    int16_t* tok_slot, int64_t n_ts) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n_ts;
+       i += stride) {
+    tok_slot[i] = (int16_t)-1;
+    if (i < n_tok) num_routed[i] = 0;
+  }
+}
+
+__device__ __forceinline__ float block_reduce(float v, float* red, bool is_max) {
+  // 256 threads = 4 wavefronts
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    const float o = __shfl_xor(v, off, 64);
+    v = is_max ? fmaxf(v, o) : v + o;
+  }
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  float r = red[0];
+  for (int w = 1; w < 4; ++w) r = is_max ? fmaxf(r, red[w]) : r + red[w];
+  return r;
+}
+
+// One block per (expert, group): softmax over the group's tokens
+// (moe.py:1094-1098; tokens with importance 0 get -1e9 first), then the C
+// largest probabilities in descending order, equal ones in token order (the
+// order of tf.math.top_k, ops.py:4934-4942): rank = number of tokens that beat
+// this one.
+template <typename IT>
+__global__ __launch_bounds__(256) void choice_select_kernel(
+    ChoiceParams p, const float* __restrict__ logits,
+    const IT* __restrict__ importance, int32_t* __restrict__ slot_token,
+    float* __restrict__ slot_prob, int16_t* __restrict__ tok_slot,
+    int32_t* __restrict__ num_routed, float* __restrict__ lse_out) {
+  extern __shared__ float pr[];  // [S] + 4
+  float* red = pr + p.S;
+  const int e = blockIdx.x, g = blockIdx.y;
+  const int S = p.S, E = p.E, C = p.C;
+  const int tid = threadIdx.x;
+  const int64_t base = (int64_t)g * S;
+  float m = -INFINITY;
+  for (int s = tid; s < S; s += 256) {
+    float x = logits[(base + s) * E + e];
+    if (importance != nullptr && load_f32<IT>(importance + base + s) == 0.0f)
+      x = x + (-1e9f);
+    pr[s] = x;
+    m = fmaxf(m, x);
+  }
+  m = block_reduce(m, red, true);
+  const float negm = -m;
+  float sum = 0.f;
+  for (int s = tid; s < S; s += 256) sum += expf(pr[s] + negm);
+  sum = block_reduce(sum, red, false);
+  const float lse = logf(sum) + m;
+  const float neglse = -lse;
+  __syncthreads();
+  for (int s = tid; s < S; s += 256) pr[s] = expf(pr[s] + neglse);
+  if (tid == 0) lse_out[(int64_t)g * E + e] = lse;
+  __syncthreads();
+  for (int s = tid; s < S; s += 256) {
+    const float ps = pr[s];
+    int rank = 0;
+    for (int s2 = 0; s2 < S; ++s2) {
+      const float p2 = pr[s2];
+      rank += (p2 > ps || (p2 == ps && s2 < s)) ? 1 : 0;
+    }
+    if (rank < C) {
+      const int64_t slot = ((int64_t)g * E + e) * C + rank;
+      slot_token[slot] = s;
+      slot_prob[slot] = ps;
+      tok_slot[(base + s) * E + e] = (int16_t)rank;
+      atomicAdd(num_routed + base + s, 1);
+    }
+  }
+}
+
+// One block per group: combine weights (probability over the number of experts
+// that chose the token, moe.py:1119-1123) and the group's term of the loss
+// mean(agg^2 * sum_s importance) * S with agg = mean_e p * (importance == 1)
+// (moe.py:1125-1147).
+template <typename IT>
+__global__ __launch_bounds__(256) void choice_finish_kernel(
+    ChoiceParams p, const float* __restrict__ logits,
+    const IT* __restrict__ importance, const float* __restrict__ lse,
+    const float* __restrict__ slot_prob, const int16_t* __restrict__ tok_slot,
+    const int32_t* __restrict__ num_routed, float* __restrict__ slot_weight,
+    float* __restrict__ gsum) {
+  __shared__ float red[4];
+  const int g = blockIdx.x;
+  const int S = p.S, E = p.E, C = p.C;
+  const int64_t base = (int64_t)g * S;
+  const float inv_e = (float)(1.0 / (double)E);
+  float sq = 0.f, imp_sum = 0.f;
+  for (int s = threadIdx.x; s < S; s += 256) {
+    const int64_t t = base + s;
+    float imp = 1.0f;
+    if (importance != nullptr) imp = load_f32<IT>(importance + t);
+    const float mask = imp == 0.0f ? -1e9f : 0.0f;
+    const float recip =
+        p.normalize ? 1.0f / fmaxf((float)num_routed[t], 1.0f) : 1.0f;
+    float agg = 0.f;
+    for (int e = 0; e < E; ++e) {
+      float x = logits[t * E + e];
+      if (imp == 0.0f) x = x + mask;
+      agg += expf(x + (-lse[(int64_t)g * E + e]));
+      const int c = tok_slot[t * E + e];
+      if (c >= 0) {
+        const int64_t slot = ((int64_t)g * E + e) * C + c;
+        slot_weight[slot] = slot_prob[slot] * recip;
+      }
+    }
+    agg = (agg * inv_e) * (imp == 1.0f ? 1.0f : 0.0f);
+    sq += agg * agg;
+    imp_sum += imp;
+  }
+  sq = block_reduce(sq, red, false);
+  imp_sum = block_reduce(imp_sum, red, false);
+  if (threadIdx.x == 0) gsum[g] = sq * imp_sum;
+}
+
+__global__ void choice_loss_kernel(ChoiceParams p, const float* __restrict__ gsum,
+                                   float* __restrict__ loss) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  float s = 0.f;
+  for (int g = 0; g < p.G; ++g) s += gsum[g];
+  float l = (s * (float)(1.0 / ((double)p.G * (double)p.S))) * (float)p.S;
+  if (p.num_microbatches > 1)
+    l = l * (float)(1.0 / (double)p.num_microbatches);
+  loss[0] = l;
+}
+
+constexpr int CH_ROWS = 4;  // wavefronts (rows) per block
+
+// expert_in[e,g,c,:] = x[g, slot_token[g,e,c], :]
+template <typename T>
+__global__ __launch_bounds__(256) void slot_dispatch_kernel(
+    const T* __restrict__ x, const int32_t* __restrict__ slot_token,
+    T* __restrict__ expert_in, int G, int S, int E, int C, int M,
+    int64_t n_slots, bool vec) {
+  const int lane = threadIdx.x & 63;
+  const int64_t j = (int64_t)blockIdx.x * CH_ROWS + (threadIdx.x >> 6);
+  if (j >= n_slots) return;
+  // j enumerates the destination [E,G,C]
+  const int c = (int)(j % C);
+  const int g = (int)((j / C) % G);
+  const int e = (int)(j / ((int64_t)C * G));
+  const int s = slot_token[((int64_t)g * E + e) * C + c];
+  const T* src = x + ((int64_t)g * S + s) * M;
+  T* dst = expert_in + j * M;
+  if (vec) {
+    const uint4* s4 = reinterpret_cast<const uint4*>(src);
+    uint4* d4 = reinterpret_cast<uint4*>(dst);
+    const int nv = M / (16 / (int)sizeof(T));
+    for (int i = lane; i < nv; i += 64) d4[i] = s4[i];
+  } else {
+    for (int i = lane; i < M; i += 64) dst[i] = src[i];
+  }
+}
+
+// out[g,s,:] = sum_e w * y[e,g,tok_slot[g,s,e],:] over the experts that chose
+// the token, float32 accumulate in expert order, one rounding.
+template <typename T>
+__global__ __launch_bounds__(256) void slot_combine_kernel(
+    const T* __restrict__ y, const int16_t* __restrict__ tok_slot,
+    const float* __restrict__ slot_weight, T* __restrict__ out, int G, int S,
+    int E, int C, int N, int64_t T_tokens) {
+  const int lane = threadIdx.x & 63;
+  const int64_t t = (int64_t)blockIdx.x * CH_ROWS + (threadIdx.x >> 6);
+  if (t >= T_tokens) return;
+  const int g = (int)(t / S);
+  const int16_t* ts = tok_slot + t * E;
+  T* dst = out + t * N;
+  for (int i0 = 0; i0 < N; i0 += 64 * 4) {
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int e = 0; e < E; ++e) {
+      const int c = ts[e];
+      if (c < 0) continue;
+      const int64_t slot = ((int64_t)g * E + e) * C + c;
+      const float w = round_to<T>(slot_weight[slot]);
+      const T* row = y + (((int64_t)e * G + g) * C + c) * N;
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        const int i = i0 + u * 64 + lane;
+        if (i < N) acc[u] += w * load_f32<T>(row + i);
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int i = i0 + u * 64 + lane;
+      if (i < N) store_f32<T>(dst + i, acc[u]);
+    }
+  }
+}
+
+}  // namespace mesh_moe
+
+using namespace mesh_moe;
+
+extern "C" size_t mesh_moe_expert_choice_workspace_bytes(int G, int S, int E,
+                                                         int C) {
+  if (G < 1 || S < 1 || E < 1 || C < 1) return 0;
+  return sizeof(int32_t) * (size_t)G * S + sizeof(float) * (size_t)G * E +
+         sizeof(float) * (size_t)G * E * C + sizeof(float) * (size_t)G +
+         4 * 256;
+}
+
+extern "C" int mesh_moe_expert_choice_gating(
+    const float* logits, const void* importance, int importance_dtype, int G,
+    int S, int E, int C, int normalize, int num_microbatches,
+    int32_t* slot_token, float* slot_weight, int16_t* tok_slot, float* loss,
+    void* workspace, size_t workspace_bytes, void* stream) {
+  MOE_REQUIRE(logits && slot_token && slot_weight && tok_slot && loss &&
+                  workspace, MESH_MOE_E_ARG,
+              "expert_choice_gating: null pointer");
+  MOE_REQUIRE(G >= 1 && S >= 1 && E >= 1 && C >= 1, MESH_MOE_E_ARG,
+              "expert_choice_gating: bad sizes G=%d S=%d E=%d C=%d", G, S, E,
+              C);
+  MOE_REQUIRE(C <= S, MESH_MOE_E_ARG,
+              "expert_choice_gating: capacity %d > group size %d", C, S);
+  MOE_REQUIRE(S <= 32768 && E <= 65535 && G <= 65535, MESH_MOE_E_UNSUPPORTED,
+              "expert_choice_gating: S=%d > 32768 or E, G > 65535", S);
+  MOE_REQUIRE(!importance || valid_dtype(importance_dtype), MESH_MOE_E_ARG,
+              "expert_choice_gating: bad importance dtype %d",
+              importance_dtype);
+  MOE_REQUIRE(workspace_bytes >=
+                  mesh_moe_expert_choice_workspace_bytes(G, S, E, C),
+              MESH_MOE_E_ARG, "expert_choice_gating: workspace too small");
+  ChoiceParams p;
+  p.G = G; p.S = S; p.E = E; p.C = C;
+  p.normalize = normalize ? 1 : 0;
+  p.num_microbatches = num_microbatches;
+  auto up = [](uintptr_t v) { return (v + 255) & ~(uintptr_t)255; };
+  int32_t* num_routed = (int32_t*)up((uintptr_t)workspace);
+  float* lse = (float*)up((uintptr_t)(num_routed + (size_t)G * S));
+  float* slot_prob = (float*)up((uintptr_t)(lse + (size_t)G * E));
+  float* gsum = (float*)up((uintptr_t)(slot_prob + (size_t)G * E * C));
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t n_tok = (int64_t)G * S, n_ts = n_tok * E;
+  const unsigned cb = (unsigned)((n_ts + 255) / 256 < 8192 ? (n_ts + 255) / 256
+                                                            : 8192);
+  choice_clear_kernel<<<cb, 256, 0, st>>>(num_routed, n_tok, tok_slot, n_ts);
+  MOE_CHECK_LAUNCH("expert_choice_gating (clear)");
+  const size_t smem = sizeof(float) * ((size_t)S + 4);
+  dim3 grid((unsigned)E, (unsigned)G);
+  const bool bf = importance && importance_dtype == MESH_MOE_BF16;
+  if (bf) {
+    auto k = choice_select_kernel<bf16_t>;
+    MOE_ALLOW_LDS(k, smem);
+    k<<<grid, 256, smem, st>>>(p, logits, (const bf16_t*)importance, slot_token,
+                               slot_prob, tok_slot, num_routed, lse);
+  } else {
+    auto k = choice_select_kernel<float>;
+    MOE_ALLOW_LDS(k, smem);
+    k<<<grid, 256, smem, st>>>(p, logits, (const float*)importance, slot_token,
+                               slot_prob, tok_slot, num_routed, lse);
+  }
+  MOE_CHECK_LAUNCH("expert_choice_gating (select)");
+  if (bf)
+    choice_finish_kernel<bf16_t><<<G, 256, 0, st>>>(
+        p, logits, (const bf16_t*)importance, lse, slot_prob, tok_slot,
+        num_routed, slot_weight, gsum);
+  else
+    choice_finish_kernel<float><<<G, 256, 0, st>>>(
+        p, logits, (const float*)importance, lse, slot_prob, tok_slot,
+        num_routed, slot_weight, gsum);
+  MOE_CHECK_LAUNCH("expert_choice_gating (finish)");
+  choice_loss_kernel<<<1, 64, 0, st>>>(p, gsum, loss);
+  MOE_CHECK_LAUNCH("expert_choice_gating (loss)");
+  return 0;
+}
+
+extern "C" int mesh_moe_slot_dispatch(const void* x, const int32_t* slot_token,
+                                      void* expert_in, int G, int S, int E,
+                                      int C, int M, int dtype, void* stream) {
+  MOE_REQUIRE(x && slot_token && expert_in, MESH_MOE_E_ARG,
+              "slot_dispatch: null pointer");
+  MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG, "slot_dispatch: bad dtype %d",
+              dtype);
+  MOE_REQUIRE(G >= 1 && S >= 1 && E >= 1 && C >= 1 && M >= 1, MESH_MOE_E_ARG,
+              "slot_dispatch: bad sizes G=%d S=%d E=%d C=%d M=%d", G, S, E, C,
+              M);
+  const int64_t n_slots = (int64_t)G * E * C;
+  const int64_t nblocks = (n_slots + CH_ROWS - 1) / CH_ROWS;
+  MOE_REQUIRE(nblocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
+              "slot_dispatch: too many slots (%lld)", (long long)n_slots);
+  const bool vec = ((size_t)M * dtype_size(dtype)) % 16 == 0 &&
+                   ((uintptr_t)x & 15) == 0 && ((uintptr_t)expert_in & 15) == 0;
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == MESH_MOE_F32)
+    slot_dispatch_kernel<float><<<(unsigned)nblocks, 256, 0, st>>>(
+        (const float*)x, slot_token, (float*)expert_in, G, S, E, C, M, n_slots,
+        vec);
+  else
+    slot_dispatch_kernel<bf16_t><<<(unsigned)nblocks, 256, 0, st>>>(
+        (const bf16_t*)x, slot_token, (bf16_t*)expert_in, G, S, E, C, M,
+        n_slots, vec);
+  MOE_CHECK_LAUNCH("slot_dispatch");
+  return 0;
+}
+
+extern "C" int mesh_moe_slot_combine(const void* y, const int16_t* tok_slot,
+                                     const float* slot_weight, void* out,
+                                     int G, int S, int E, int C, int N,
+                                     int dtype, void* stream) {
+  MOE_REQUIRE(y && tok_slot && slot_weight && out, MESH_MOE_E_ARG,
+              "slot_combine: null pointer");
+  MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG, "slot_combine: bad dtype %d",
+              dtype);
+  MOE_REQUIRE(G >= 1 && S >= 1 && E >= 1 && C >= 1 && N >= 1, MESH_MOE_E_ARG,
+              "slot_combine: bad sizes G=%d S=%d E=%d C=%d N=%d", G, S, E, C,
+              N);
+  const int64_t T_tokens = (int64_t)G * S;
+  const int64_t nblocks = (T_tokens + CH_ROWS - 1) / CH_ROWS;
+  MOE_REQUIRE(nblocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
+              "slot_combine: too many rows (%lld)", (long long)T_tokens);
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == MESH_MOE_F32)
+    slot_combine_kernel<float><<<(unsigned)nblocks, 256, 0, st>>>(
+        (const float*)y, tok_slot, slot_weight, (float*)out, G, S, E, C, N,
+        T_tokens);
+  else
+    slot_combine_kernel<bf16_t><<<(unsigned)nblocks, 256, 0, st>>>(
+        (const bf16_t*)y, tok_slot, slot_weight, (bf16_t*)out, G, S, E, C, N,
+        T_tokens);
+  MOE_CHECK_LAUNCH("slot_combine");
+  return 0;
+}

@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -90,6 +90,18 @@ _SIGNATURES = {
     "mesh_moe_dispatch_backward": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
+    "mesh_moe_expert_choice_workspace_bytes": (ctypes.c_size_t, [
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "mesh_moe_expert_choice_gating": (ctypes.c_int, [
+        _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, _vp, _vp,
+        ctypes.c_size_t, _vp]),
+    "mesh_moe_slot_dispatch": (ctypes.c_int, [
+        _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, _vp]),
+    "mesh_moe_slot_combine": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
 }
 EXPORTS = sorted(_SIGNATURES)
 
@@ -634,3 +646,72 @@ def dispatch_backward(dexpert_in, r, group_size, dlogits=None,
         dx.data_ptr(), g, s, e, c, m, dtype_code(dt), _stream()),
         "dispatch_backward")
   return dx
+
+
+# ----------------------------------------------------------------------------
+# expert-selection ("expert choice") gating
+# ----------------------------------------------------------------------------
+class SlotRouting(object):
+  """Per-slot routing record written by expert_choice_gating."""
+
+  def __init__(self, slot_token, slot_weight, tok_slot, loss, capacity,
+               num_experts):
+    self.slot_token, self.slot_weight = slot_token, slot_weight
+    self.tok_slot, self.loss = tok_slot, loss
+    self.capacity, self.num_experts = capacity, num_experts
+
+
+def expert_choice_gating(logits, capacity, importance=None, normalize=True,
+                         num_microbatches=None):
+  """logits float32 [G, S, E] -> SlotRouting."""
+  lib = load_library()
+  g, s, e = logits.shape
+  c = int(capacity)
+  dev = logits.device
+  ip, icode = None, F32
+  if importance is not None:
+    icode = dtype_code(importance.dtype)
+    ip = _dev(importance, "importance", None, (g, s))
+  slot_token = torch.empty((g, e, c), dtype=torch.int32, device=dev)
+  slot_weight = torch.empty((g, e, c), dtype=torch.float32, device=dev)
+  tok_slot = torch.empty((g, s, e), dtype=torch.int16, device=dev)
+  loss = torch.empty((1,), dtype=torch.float32, device=dev)
+  ws_bytes = lib.mesh_moe_expert_choice_workspace_bytes(g, s, e, c)
+  ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
+  with _stage("expert_choice_gating"):
+    _check(lib.mesh_moe_expert_choice_gating(
+        _dev(logits, "logits", torch.float32), ip, icode, g, s, e, c,
+        int(bool(normalize)), int(num_microbatches or 1),
+        slot_token.data_ptr(), slot_weight.data_ptr(), tok_slot.data_ptr(),
+        loss.data_ptr(), ws.data_ptr(), ws_bytes, _stream()),
+        "expert_choice_gating")
+  return SlotRouting(slot_token, slot_weight, tok_slot, loss, c, e)
+
+
+def slot_dispatch(x, r):
+  """x [G, S, M] -> expert_in [E, G, C, M], one token row per slot."""
+  lib = load_library()
+  g, s, m = x.shape
+  e, c = r.num_experts, r.capacity
+  out = torch.empty((e, g, c, m), dtype=x.dtype, device=x.device)
+  with _stage("slot_dispatch"):
+    _check(lib.mesh_moe_slot_dispatch(
+        _dev(x, "x"), _dev(r.slot_token, "slot_token", torch.int32, (g, e, c)),
+        out.data_ptr(), g, s, e, c, m, dtype_code(x.dtype), _stream()),
+        "slot_dispatch")
+  return out
+
+
+def slot_combine(y, r, group_size):
+  """y [E, G, C, N] -> out [G, S, N]."""
+  lib = load_library()
+  e, g, c, n = y.shape
+  s = group_size
+  out = torch.empty((g, s, n), dtype=y.dtype, device=y.device)
+  with _stage("slot_combine"):
+    _check(lib.mesh_moe_slot_combine(
+        _dev(y, "y"), _dev(r.tok_slot, "tok_slot", torch.int16, (g, s, e)),
+        _dev(r.slot_weight, "slot_weight", torch.float32, (g, e, c)),
+        out.data_ptr(), g, s, e, c, n, dtype_code(y.dtype), _stream()),
+        "slot_combine")
+  return out

@@ -21,7 +21,7 @@ from mesh_amd import layers as mtf_layers
 from mesh_amd import moe_hip
 from mesh_amd import ops as mtf
 
-_OTHER_GATINGS = ("ntlb", "expert_selection")
+_OTHER_GATINGS = ("ntlb",)
 
 
 class HParams(object):
@@ -89,11 +89,12 @@ def _activation_name(activation):
 
 
 def _check_gating(hparams):
-  if hparams.moe_gating in ("top_2", "switch", "switch_max"):
+  if hparams.moe_gating in ("top_2", "switch", "switch_max",
+                            "expert_selection"):
     return
   if hparams.moe_gating in _OTHER_GATINGS:
     raise NotImplementedError(
-        "moe_gating=%s is not implemented (top_2, switch and switch_max only)"
+        "moe_gating=%s is not implemented"
         % hparams.moe_gating)
   raise ValueError("unknown hparams.moe_gating=%s" % hparams.moe_gating)
 
@@ -213,6 +214,41 @@ class _SwitchGatingSpec(object):
     return (r, logits) if want_logits else r
 
 
+class _ExpertSelectionGatingSpec(object):
+  """Static configuration of one _expert_selection_gating call
+  (moe.py:1057-1173): experts choose tokens.  The routing record is per slot
+  (moe_hip.SlotRouting), so the layer dispatches and combines by slot."""
+
+  router = "expert_selection"
+  use_second_place_loss = False
+  z_loss = None
+
+  def __init__(self, hparams, train, num_microbatches, has_importance):
+    policy = (hparams.moe_switch_policy_train if train
+              else hparams.moe_switch_policy_eval)
+    if train and policy in ("input_dropout", "input_jitter"):
+      raise NotImplementedError(
+          "switch policy %r draws random numbers while training and is not "
+          "implemented" % (policy,))
+    if not has_importance:
+      # the reference sums `importance` for its loss (moe.py:1138-1140)
+      raise ValueError("expert_selection gating needs nonpadding")
+    self.num_microbatches = num_microbatches
+
+  def route(self, x, w, w_packed, group_size, num_experts, capacity,
+            importance=None, importance_from_slot_gate=False,
+            want_logits=False):
+    assert not importance_from_slot_gate
+    b, t, _ = x.shape
+    groups = b * t // group_size
+    logits = moe_hip.router_logits(x, w, w_packed=w_packed)
+    logits = logits.reshape(groups, group_size, num_experts)
+    r = moe_hip.expert_choice_gating(
+        logits, capacity, importance=importance,
+        num_microbatches=self.num_microbatches)
+    return (r, logits) if want_logits else r
+
+
 def _packed(lowering, kernel_tensor, dtype):
   """K-contiguous copy of an expert kernel variable, cached on the variable."""
   return lowering.variables[kernel_tensor.operation].packed(dtype)
@@ -241,6 +277,9 @@ class MoEV1Operation(mtf.Operation):
   def gradient(self, grad_ys):
     """Gradients w.r.t. (inputs, gate kernel, wi, wo[, importance]) from those
     of (outputs, loss); importance carries none."""
+    if self._gating.router == "expert_selection":
+      raise NotImplementedError(
+          "backward of expert_selection gating is not implemented")
     if self._gating.use_second_place_loss:
       raise NotImplementedError(
           "backward of the second-place loss is not implemented")
@@ -282,14 +321,18 @@ class MoEV1Operation(mtf.Operation):
       logits = None
       if save:
         r, logits = r
-      expert_in = moe_hip.dispatch(xg, r)
+      by_slot = isinstance(r, moe_hip.SlotRouting)
+      expert_in = (moe_hip.slot_dispatch(xg, r) if by_slot
+                   else moe_hip.dispatch(xg, r))
       h = None
       if save:
         h = torch.empty((e_, groups * c_, wi_p.shape[1]), dtype=dt,
                         device=xg.device)
       y = moe_hip.expert_ffn(expert_in.reshape(e_, groups * c_, m_), wi_p,
                              wo_p, self._activation, h=h)
-      out = moe_hip.combine(y.reshape(e_, groups, c_, n_), r, s_)
+      y4 = y.reshape(e_, groups, c_, n_)
+      out = (moe_hip.slot_combine(y4, r, s_) if by_slot
+             else moe_hip.combine(y4, r, s_))
       if save:
         # what the gradient operation reads (activations of this step)
         saved.update(x=xg, routing=r, logits=logits, importance=imp_s,
@@ -441,7 +484,11 @@ def transformer_moe_layer_v1(
                               "implemented (moe_dropout_rate must be 0)")
   if hparams.moe_use_experts_attention:
     raise NotImplementedError("moe_use_experts_attention is not implemented")
-  if hparams.moe_gating in ("switch", "switch_max"):
+  if hparams.moe_gating == "expert_selection":
+    gating = _ExpertSelectionGatingSpec(hparams, train, num_microbatches,
+                                        nonpadding is not None)
+    router_name = "expert_selection_gating"             # moe.py:1061
+  elif hparams.moe_gating in ("switch", "switch_max"):
     gating = _SwitchGatingSpec(hparams, train, num_microbatches,
                                nonpadding is not None)
     router_name = hparams.moe_gating + "_gating"        # moe.py:1178, :945

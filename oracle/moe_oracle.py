@@ -30,6 +30,10 @@ MoE file, and its TensorFlow dependency cannot run here):
                                       lowering of mtf.top_k) vs the stable
                                       sort, per-expert brute force, equality
                                       with switch_gating when nothing overflows
+  expert_selection_gating             per-expert stable sort brute force,
+                                      weights of a token sum to sum(p)/count,
+                                      closed-form loss (uniform logits: 1.0),
+                                      dense tensors vs slot record
   gating_backward,                    central differences of an independent
   moe_layer_v1_backward               float64 forward with the routing held
                                       fixed (tests/test_oracle.py)
@@ -450,6 +454,81 @@ def switch_max_gating(logits, capacity, importance=None,
   return out
 
 
+# ----------------------------------------------------------------------------
+# _expert_selection_gating  (transformer/moe.py:1057-1173)
+# ----------------------------------------------------------------------------
+def expert_selection_gating(logits, capacity, importance,
+                            num_microbatches=None, act_dtype="float32",
+                            normalize_by_num_experts_routed=True, dense=False):
+  """Everything in _expert_selection_gating after the router projection, for
+  the policies that draw no random numbers: every expert picks the `capacity`
+  tokens of each group it likes best.
+
+  The softmax runs over the GROUP dim (per expert, over tokens); tokens with
+  importance 0 get -1e9 added to their logits first (moe.py:1094-1097).  A
+  token may be chosen by several experts or by none; its combine weights are
+  the chosen probabilities divided by max(#experts that chose it, 1)
+  (moe.py:1119-1123).  `importance` is required, as in the reference, whose
+  loss sums it (moe.py:1138-1140).
+
+  Returns dict(slot_token int32 [G,E,C] (token of each slot), slot_weight
+  float32 [G,E,C] (combine weight before the activation-dtype cast), loss,
+  and with dense=True combine / dispatch [G,S,E,C]).
+  """
+  logits = np.asarray(logits, dtype=F32)
+  g_, s_, e_ = logits.shape
+  importance = np.asarray(importance, dtype=F32)
+  logits = logits + ((importance == F32(0.0)).astype(F32) * F32(-1e9))[..., None]
+  # softmax over the group dim (ops.py:5493-5541 with reduced_dim = group)
+  raw_gates = np.moveaxis(softmax(np.moveaxis(logits, 1, -1)), -1, 1)  # [G,S,E]
+  probs, tokens = top_k_lowest_index_first(raw_gates, capacity, 1)    # [G,E,C]
+  dispatch = one_hot(tokens, s_)                                 # [G,E,C,S]
+  combine = dispatch * probs[..., None]                          # :1115
+  slot_weight = probs
+  if normalize_by_num_experts_routed:                            # :1119-1123
+    num_routed = dispatch.sum(axis=(1, 2), dtype=F32)            # [G,S]
+    recip = (F32(1.0) / np.maximum(num_routed, F32(1.0))).astype(F32)
+    combine = combine * recip[:, None, None, :]
+    slot_weight = probs * np.take_along_axis(
+        recip[:, None, :].repeat(e_, 1), tokens, -1)
+  # load balancing loss (:1125-1147)
+  agg = seq_sum(raw_gates, axis=-1) * F32(1.0 / e_)              # [G,S]
+  agg = agg * (importance == F32(1.0)).astype(F32)
+  true_group_size = seq_sum(importance, axis=-1)                 # [G]
+  prod = (agg * agg) * true_group_size[:, None]
+  loss = seq_sum(prod.reshape(-1)) * F32(1.0 / prod.size)
+  loss = loss * F32(float(s_))
+  if num_microbatches and num_microbatches > 1:
+    loss = loss * F32(1.0 / num_microbatches)
+  out = dict(slot_token=tokens, slot_weight=slot_weight.astype(F32),
+             loss=cast_act(loss, act_dtype)[()])
+  if dense:
+    out["combine"] = cast_act(combine.transpose(0, 3, 1, 2), act_dtype)
+    out["dispatch"] = dispatch.transpose(0, 3, 1, 2).astype(F32)  # :1169-1170
+  return out
+
+
+def slot_dispatch(x, r):
+  """expert_in[e, g, c, :] = x[g, slot_token[g, e, c], :] (the dispatch einsum
+  with a one-hot per slot, moe.py:443-447)."""
+  g_ = x.shape[0]
+  tok = r["slot_token"]                                          # [G,E,C]
+  return x[np.arange(g_)[:, None, None], tok].transpose(1, 0, 2, 3)
+
+
+def slot_combine(y, r, group_size, act_dtype):
+  """out[g, s, :] = sum over the slots holding token s of w * y[e, g, c, :]
+  with w the activation-dtype combine weight (moe.py:509-510); float32
+  accumulate in (expert, slot) order, one rounding."""
+  e_, g_, c_, n_ = y.shape
+  w = cast_act(r["slot_weight"], act_dtype)
+  out = np.zeros((g_, group_size, n_), F32)
+  for g in range(g_):
+    for e in range(e_):
+      np.add.at(out[g], r["slot_token"][g, e], w[g, e][:, None] * y[e, g])
+  return cast_act(out, act_dtype)
+
+
 def routing_sequential(index_1, index_2, sel_1, sel_2, num_experts, capacity):
   """Integer brute force for moe.py:1472-1496, one token at a time.
 
@@ -630,7 +709,7 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
 
   Returns (output [batch..., length, N], loss scalar, aux dict).
   """
-  if hp.moe_gating not in ("top_2", "switch", "switch_max"):
+  if hp.moe_gating not in ("top_2", "switch", "switch_max", "expert_selection"):
     raise ValueError("unknown hparams.moe_gating=%s" % hp.moe_gating)
   x = cast_act(x, act_dtype)
   lead = x.shape[:-1]
@@ -649,6 +728,37 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
   logits = router_logits(xg, wg)
   if logit_bias is not None:
     logits = logits + np.asarray(logit_bias, F32)
+  if hp.moe_gating == "expert_selection":                        # :425-438
+    sw = hp.moe_switch_policy_train if train else hp.moe_switch_policy_eval
+    if train and sw in ("input_dropout", "input_jitter"):
+      raise NotImplementedError("switch policy %r draws random numbers" % sw)
+    if importance is None:
+      raise ValueError("expert_selection gating needs nonpadding "
+                       "(moe.py:1138-1140)")
+    r = expert_selection_gating(logits, c_, importance, num_microbatches,
+                                act_dtype, dense=dense)
+    wi_a = wi if weights_are_cast else cast_act(wi, act_dtype)
+    wo_a = wo if weights_are_cast else cast_act(wo, act_dtype)
+    if dense:
+      disp = r["dispatch"].reshape(g_, s_, e_ * c_)
+      expert_in = cast_act(np.matmul(disp.transpose(0, 2, 1), xg), act_dtype)
+      expert_in = expert_in.reshape(g_, e_, c_, m_).transpose(1, 0, 2, 3)
+    else:
+      expert_in = slot_dispatch(xg, r)
+    y = expert_ffn(expert_in.reshape(e_, g_ * c_, m_), wi_a, wo_a, activation,
+                   act_dtype)
+    n_ = y.shape[-1]
+    y = y.reshape(e_, g_, c_, n_)
+    if dense:
+      comb = r["combine"].reshape(g_, s_, e_ * c_)
+      yg = y.transpose(1, 0, 2, 3).reshape(g_, e_ * c_, n_)
+      out = cast_act(np.matmul(comb, yg), act_dtype)
+    else:
+      out = slot_combine(y, r, s_, act_dtype)
+    aux = dict(r, logits=logits, expert_in=expert_in, expert_out=y,
+               num_groups=g_, group_size=s_, capacity=c_)
+    return (out.reshape(lead + (n_,)),
+            _scale_loss(r["loss"], hp.moe_loss_coef, act_dtype), aux)
   if hp.moe_gating in ("switch", "switch_max"):                  # :393-424
     sw = hp.moe_switch_policy_train if train else hp.moe_switch_policy_eval
     if sw == "sample" or (train and sw in ("input_dropout", "input_jitter")):

@@ -605,3 +605,90 @@ def test_full_size_expert_ffn_properties(hip, size):
   assert not bool(y[e // 2 + 1].any())
   y2 = hip.expert_ffn(x * 2, wi, wo, "relu")
   assert torch.equal(y2, y * 2)
+
+
+# ---- expert-selection (expert choice) gating ---------------------------------------
+def _column_gaps_ok(logits, imp, min_gap=1e-4):
+  """No two unmasked tokens of a group have logits for the same expert closer
+  than min_gap: their probabilities then rank the same way whatever the last
+  ulp of exp/log."""
+  g, s, e = logits.shape
+  for gi in range(g):
+    keep = imp[gi] != 0
+    col = np.sort(logits[gi][keep], axis=0)
+    if (np.diff(col, axis=0) < min_gap).any():
+      return False
+  return True
+
+
+@pytest.mark.parametrize("shape", [(2, 64, 4, 8), (3, 77, 5, 20), (2, 1024, 8, 256),
+                                   (16, 2048, 64, 32), (1, 300, 130, 7)])
+def test_expert_choice_gating(hip, shape):
+  g, s, e, c = shape
+  rng = np.random.default_rng(3000 + hash(shape) % 1000)
+  # per (group, expert) a shuffled grid of logits with spacing 6 / S plus a
+  # jitter below a quarter of it: no two tokens of a column nearly tie
+  step = 6.0 / s
+  grid = (np.arange(s) - s / 2) * step
+  logits = np.empty((g, s, e), np.float32)
+  for gi in range(g):
+    for ex in range(e):
+      logits[gi, :, ex] = rng.permutation(grid) + rng.uniform(-step / 4, step / 4, s)
+  imp = rng.choice(np.array([0.0, 0.5, 1.0], np.float32), size=(g, s),
+                   p=[0.1, 0.1, 0.8])
+  assert _column_gaps_ok(logits, imp, min_gap=step / 4)
+  want = O.expert_selection_gating(logits, c, imp, num_microbatches=2)
+  for imp_dtype in ("float32", "bfloat16"):
+    r = hip.expert_choice_gating(torch.from_numpy(logits).cuda(), c,
+                                 importance=H.to_gpu(imp, imp_dtype),
+                                 num_microbatches=2)
+    np.testing.assert_array_equal(H.to_np(r.slot_token), want["slot_token"])
+    np.testing.assert_allclose(H.to_np(r.slot_weight), want["slot_weight"],
+                               rtol=2e-5, atol=1e-30)
+    np.testing.assert_allclose(H.to_np(r.loss)[0], want["loss"], rtol=5e-5)
+    # tok_slot is the inverse of slot_token
+    ts = H.to_np(r.tok_slot)
+    inv = np.full((g, s, e), -1, np.int16)
+    for gi in range(g):
+      for ex in range(e):
+        inv[gi, want["slot_token"][gi, ex], ex] = np.arange(c)
+    np.testing.assert_array_equal(ts, inv)
+
+
+def test_expert_choice_exact_ties_token_order(hip):
+  g, s, e, c = 2, 96, 4, 30
+  rng = np.random.default_rng(10)
+  logits = (np.round(rng.standard_normal((g, s, e)) * 2) / 2).astype(np.float32)
+  imp = np.ones((g, s), np.float32)
+  want = O.expert_selection_gating(logits, c, imp)
+  r = hip.expert_choice_gating(torch.from_numpy(logits).cuda(), c,
+                               importance=H.to_gpu(imp))
+  # equal logits give bit-equal probabilities in either implementation and
+  # unequal ones differ by >= 0.5, so the slots must agree exactly
+  np.testing.assert_array_equal(H.to_np(r.slot_token), want["slot_token"])
+
+
+@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
+def test_slot_dispatch_combine(hip, act_dtype):
+  g, s, e, c, m = 2, 128, 8, 40, 72
+  rng = np.random.default_rng(11)
+  logits = (rng.standard_normal((g, s, e)) * 1.5).astype(np.float32)
+  imp = np.ones((g, s), np.float32)
+  want_r = O.expert_selection_gating(logits, c, imp)
+  r = hip.expert_choice_gating(torch.from_numpy(logits).cuda(), c,
+                               importance=H.to_gpu(imp))
+  assert np.array_equal(H.to_np(r.slot_token), want_r["slot_token"])
+  x = O.cast_act(rng.standard_normal((g, s, m)).astype(np.float32), act_dtype)
+  ein = hip.slot_dispatch(H.to_gpu(x, act_dtype), r)
+  np.testing.assert_array_equal(H.to_np(ein), O.slot_dispatch(x, want_r))
+  y = O.cast_act(rng.standard_normal((e, g, c, m)).astype(np.float32), act_dtype)
+  out = hip.slot_combine(H.to_gpu(y, act_dtype), r, s)
+  # the kernel's own weights (they match the oracle's to float32 round-off;
+  # a bf16 rounding boundary could otherwise flip a weight by one bf16 ulp)
+  r_np = dict(slot_token=want_r["slot_token"], slot_weight=H.to_np(r.slot_weight))
+  np.testing.assert_allclose(H.to_np(out), O.slot_combine(y, r_np, s, act_dtype),
+                             **H.value_tolerance(act_dtype))
+  chosen = np.zeros((g, s), bool)
+  for gi in range(g):
+    chosen[gi][want_r["slot_token"][gi].reshape(-1)] = True
+  assert (H.to_np(out)[~chosen] == 0).all()

@@ -424,3 +424,51 @@ def test_v1_gradients_match_oracle(case):
   np.testing.assert_allclose(
       got2, want2["dwi"], rtol=tol["rtol"],
       atol=tol["atol"] * max(1.0, np.abs(want2["dwi"]).max()))
+
+
+def test_v1_expert_selection_matches_oracle():
+  b, l, m, hdim, e, group = 2, 128, 32, 64, 4, 64
+  rng = np.random.default_rng(401)
+  w = dict(w_gate=H.normal_weights(rng, (m, e), m),
+           wi=H.normal_weights(rng, (e, m, hdim), m),
+           wo=H.normal_weights(rng, (e, hdim, m), hdim))
+  nonpad = (rng.random((b, l)) < 0.85).astype(np.float32)
+  hp, ohp = make_hparams(moe_num_experts=e, moe_hidden_size=hdim,
+                         moe_group_size=group, moe_capacity_factor_eval=1.0,
+                         **dict(SWITCH_HP, moe_gating="expert_selection"))
+  # tokens whose router logits keep every expert's ranking unambiguous
+  for _ in range(50):
+    x = rng.standard_normal((b, l, m)).astype(np.float32)
+    logits = O.router_logits(x.reshape(-1, group, m), w["w_gate"])
+    ok = True
+    for gi in range(logits.shape[0]):
+      keep = nonpad.reshape(-1, group)[gi] != 0
+      if (np.diff(np.sort(logits[gi][keep], axis=0), axis=0) < 1e-4).any():
+        ok = False
+    if ok:
+      break
+  assert ok
+  want, want_loss, aux = O.moe_layer_v1(x, w["w_gate"], w["wi"], w["wo"], ohp,
+                                        False, "float32", nonpadding=nonpad)
+  wi = dict(w)
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  dims = [mtf.Dimension("batch", b), mtf.Dimension("length", l),
+          mtf.Dimension("d_model", m)]
+  xt = mtf.import_tf_tensor(mesh, torch.from_numpy(x), mtf.Shape(dims))
+  npad = mtf.import_tf_tensor(mesh, torch.from_numpy(nonpad), mtf.Shape(dims[:2]))
+  with mtf.variable_scope("moe"):
+    y, loss = moe.transformer_moe_layer_v1(
+        xt, dims[-1], hp, False, mtf.VariableDType(torch.float32), nonpadding=npad)
+  names = sorted(v.name for v in graph.all_variables)
+  assert names[0] == "moe/expert_selection_gating/kernel"
+  lowering = mtf.Lowering(
+      graph, {mesh: mtf.HipMeshImpl()},
+      initial_values={"moe/expert_selection_gating/kernel": wi["w_gate"],
+                      "moe/wi/kernel": wi["wi"], "moe/wo/kernel": wi["wo"]})
+  got = H.to_np(lowering.export_to_tf_tensor(y))
+  np.testing.assert_allclose(got, want, **H.value_tolerance("float32"))
+  np.testing.assert_allclose(float(H.to_np(lowering.export_to_tf_tensor(loss))),
+                             want_loss, rtol=1e-4)
+  with pytest.raises(ValueError, match="needs nonpadding"):
+    run_v1(x, w, hp, False, "float32")

@@ -528,6 +528,108 @@ def test_switch_max_equals_switch_without_overflow():
   assert b["gate_1"].sum() > a["gate_1"].sum()
 
 
+# ---- expert_selection gating ------------------------------------------------------
+@pytest.mark.parametrize("seed", range(3))
+def test_expert_selection_brute_force(seed):
+  """Per (group, expert): softmax over the group's tokens in float64, tokens
+  sorted by probability descending (token order on ties), the first C fill the
+  slots; a token's weights are its probabilities over the number of experts
+  that chose it (transformer/moe.py:1099-1123)."""
+  rng = np.random.default_rng(500 + seed)
+  g, s, e = 2, int(rng.integers(8, 60)), int(rng.integers(2, 6))
+  c = int(rng.integers(1, s // 2))
+  quantum = 0.5 if seed == 2 else 0.0                   # seed 2: exact ties
+  logits = rng.standard_normal((g, s, e)).astype(np.float32)
+  if quantum:
+    logits = (np.round(logits / quantum) * quantum).astype(np.float32)
+  imp = rng.choice(np.array([0.0, 1.0], np.float32), size=(g, s), p=[0.2, 0.8])
+  masked = logits.astype(np.float64) + (imp == 0)[..., None] * -1e9
+  p64 = scipy.special.softmax(masked, axis=1)
+  for dense in (False, True):
+    r = O.expert_selection_gating(logits, c, imp, dense=dense)
+    count = np.zeros((g, s), int)
+    for gi in range(g):
+      for ex in range(e):
+        order = sorted(range(s), key=lambda t: (-O.F32(p64[gi, t, ex]), t))
+        if not quantum:
+          np.testing.assert_array_equal(r["slot_token"][gi, ex], order[:c])
+        count[gi][r["slot_token"][gi, ex]] += 1
+    for gi in range(g):
+      for ex in range(e):
+        tok = r["slot_token"][gi, ex]
+        np.testing.assert_allclose(
+            r["slot_weight"][gi, ex], p64[gi, tok, ex] / count[gi, tok],
+            rtol=3e-6, atol=1e-30)
+        # probabilities descend along the slots, ties in token order
+        pv = p64[gi, tok, ex]
+        assert (np.diff(pv) <= 1e-12).all()
+        if quantum:
+          same = np.isclose(np.diff(pv), 0, atol=1e-15)
+          assert (np.diff(tok)[same] > 0).all()
+    if dense:
+      want = np.zeros((g, s, e, c), np.float32)
+      disp = np.zeros((g, s, e, c), np.float32)
+      for gi in range(g):
+        for ex in range(e):
+          want[gi, r["slot_token"][gi, ex], ex, np.arange(c)] = \
+              r["slot_weight"][gi, ex]
+          disp[gi, r["slot_token"][gi, ex], ex, np.arange(c)] = 1.0
+      np.testing.assert_allclose(r["combine"], want, rtol=1e-6)
+      # the dispatch tensor is the one-hot itself, whatever the weight
+      np.testing.assert_array_equal(r["dispatch"], disp)
+      assert (r["dispatch"].sum(axis=1) == 1).all()     # every slot is filled
+
+
+def test_expert_selection_loss_closed_forms():
+  """loss = mean_{g,s}(agg^2 * sum_s importance) * S with agg = mean_e p
+  (moe.py:1125-1147).  Uniform logits: p = 1/n over the n unmasked tokens,
+  loss = 1 whatever the mask; all mass on one token: loss = S."""
+  s, e = 32, 4
+  ones = np.ones((2, s), np.float32)
+  np.testing.assert_allclose(
+      O.expert_selection_gating(np.zeros((2, s, e), np.float32), 4, ones)["loss"],
+      1.0, rtol=1e-5)
+  imp = ones.copy()
+  imp[:, ::2] = 0.0
+  np.testing.assert_allclose(
+      O.expert_selection_gating(np.zeros((2, s, e), np.float32), 4, imp)["loss"],
+      1.0, rtol=1e-5)
+  peak = np.zeros((1, s, e), np.float32)
+  peak[0, 5] = 60.0
+  np.testing.assert_allclose(
+      O.expert_selection_gating(peak, 4, ones[:1])["loss"], s, rtol=1e-5)
+  np.testing.assert_allclose(
+      O.expert_selection_gating(peak, 4, ones[:1], num_microbatches=4)["loss"],
+      s / 4, rtol=1e-5)
+
+
+def test_v1_expert_selection_dense_equals_index_form():
+  rng = np.random.default_rng(53)
+  b, l, m, h, e = 2, 48, 16, 24, 4
+  x = rng.standard_normal((b, l, m)).astype(np.float32)
+  wg = rng.standard_normal((m, e)).astype(np.float32)
+  wi = rng.standard_normal((e, m, h)).astype(np.float32) / 4
+  wo = rng.standard_normal((e, h, m)).astype(np.float32) / 5
+  hp = O.default_hparams(moe_gating="expert_selection", moe_num_experts=e,
+                         moe_hidden_size=h, moe_group_size=32,
+                         moe_capacity_factor_eval=2.0,
+                         moe_switch_policy_eval="argmax")
+  nonpad = (rng.random((b, l)) < 0.8).astype(np.float32)
+  d, dl, aux = O.moe_layer_v1(x, wg, wi, wo, hp, False, nonpadding=nonpad,
+                              dense=True)
+  i, il, _ = O.moe_layer_v1(x, wg, wi, wo, hp, False, nonpadding=nonpad,
+                            dense=False)
+  np.testing.assert_allclose(d, i, rtol=1e-5, atol=1e-6)
+  assert dl == il and aux["capacity"] == 16
+  # tokens nobody chose output zero; a chosen one is the weighted FFN sum
+  chosen = np.zeros((aux["num_groups"], aux["group_size"]), bool)
+  for gi in range(aux["num_groups"]):
+    chosen[gi][aux["slot_token"][gi].reshape(-1)] = True
+  assert (d.reshape(chosen.shape + (m,))[~chosen] == 0).all() and chosen.any()
+  with pytest.raises(ValueError):
+    O.moe_layer_v1(x, wg, wi, wo, hp, False)
+
+
 # ---- the layers ----------------------------------------------------------------
 def _hp(**kw):
   base = dict(moe_second_policy_train="all", moe_second_policy_eval="all")
