@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 4
+#define MESH_MOE_ABI_VERSION 5
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -225,6 +225,18 @@ int mesh_moe_expert_ffn(const void* expert_in, const void* wi_packed,
                         const void* wo_packed, void* h, void* y, int E, int R,
                         int M, int H, int N, int activation, int dtype,
                         void* stream);
+
+/*
+ * One expert projection: y = act(a . w) per expert, float32 accumulate -- the
+ * grouped GEMM mesh_moe_expert_ffn runs twice.  Replaces a single
+ * mtf.layers.dense with expert_dims (layers.py:129-208), e.g. the "q_wo" and
+ * "k_wo" projections of the same hidden tensor when moe_use_experts_attention
+ * is set (transformer/moe.py:482-520).
+ *   a [E,R,K] dtype; w_packed [E,N,K] dtype (see pack_weights); y [E,R,N] dtype
+ */
+int mesh_moe_expert_linear(const void* a, const void* w_packed, void* y, int E,
+                           int R, int K, int N, int activation, int dtype,
+                           void* stream);
 
 /*
  * Combine: out[g,s,:] = w1 * y[idx1,g,pos1,:] + w2 * y[idx2,g,pos2,:] with

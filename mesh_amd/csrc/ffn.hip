@@ -957,6 +957,22 @@ extern "C" int mesh_moe_expert_ffn(const void* expert_in, const void* wi_packed,
                       st);
 }
 
+extern "C" int mesh_moe_expert_linear(const void* a, const void* w_packed,
+                                      void* y, int E, int R, int K, int N,
+                                      int activation, int dtype, void* stream) {
+  MOE_REQUIRE(a && w_packed && y, MESH_MOE_E_ARG, "expert_linear: null pointer");
+  MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG, "expert_linear: bad dtype %d",
+              dtype);
+  MOE_REQUIRE(E >= 1 && R >= 1 && K >= 1 && N >= 1, MESH_MOE_E_ARG,
+              "expert_linear: bad sizes E=%d R=%d K=%d N=%d", E, R, K, N);
+  MOE_REQUIRE(activation >= MESH_MOE_ACT_LINEAR &&
+                  activation <= MESH_MOE_ACT_SWISH,
+              MESH_MOE_E_ARG, "expert_linear: unknown activation %d",
+              activation);
+  return grouped_gemm(a, w_packed, y, E, R, N, K, activation, dtype,
+                      (hipStream_t)stream);
+}
+
 // Elements of the scratch mesh_moe_expert_ffn_backward needs: dh [E,R,H], one
 // [E,H,R] transpose buffer (h^T, then dh^T) and one [E,max(M,N),R] buffer
 // (dy^T, then expert_in^T).

@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 4
+ABI_VERSION = 5
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -64,6 +64,9 @@ _SIGNATURES = {
     "mesh_moe_expert_ffn": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
+    "mesh_moe_expert_linear": (ctypes.c_int, [
+        _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, _vp]),
     "mesh_moe_combine": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
@@ -502,6 +505,24 @@ def expert_ffn(expert_in, wi_packed, wo_packed, activation="relu", h=None,
     _check(lib.mesh_moe_expert_ffn(ip, wip, wop, hp, yp, e, rows, m, hdim, n,
                                    ACTIVATIONS[activation], code, _stream()),
            "expert_ffn")
+  return y
+
+
+def expert_linear(a, w_packed, activation="linear", y=None):
+  """a [E, R, K]; w_packed [E, N, K] -> y [E, R, N] = act(a . w) per expert."""
+  lib = load_library()
+  if activation not in ACTIVATIONS:
+    raise ValueError("unsupported expert activation %r" % (activation,))
+  e, rows, k = a.shape
+  n = w_packed.shape[1]
+  dt = a.dtype
+  if y is None:
+    y = torch.empty((e, rows, n), dtype=dt, device=a.device)
+  with _stage("expert_linear"):
+    _check(lib.mesh_moe_expert_linear(
+        _dev(a, "a"), _dev(w_packed, "w_packed", dt, (e, n, k)),
+        _dev(y, "y", dt, (e, rows, n)), e, rows, k, n, ACTIVATIONS[activation],
+        dtype_code(dt), _stream()), "expert_linear")
   return y
 
 

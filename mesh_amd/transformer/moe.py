@@ -8,11 +8,13 @@ reference expands the layer into ~100 graph primitives and dense one-hot
 [G,S,E,C] tensors, each layer here is ONE Operation whose slice function calls
 the HIP kernels: router -> top-2 gating -> dispatch -> expert FFN -> combine.
 
-Built: moe_gating="top_2" with every second-place policy, nonpadding /
-importance, the second-place loss, float32 and bfloat16.  Not built (they
-raise NotImplementedError): the other routers of the reference's file,
-expert dropout while training, moe_use_experts_attention, gated (list)
-activations, and a mesh with more than one device.
+Built: moe_gating "top_2" (every second-place policy, the second-place loss),
+"switch", "switch_max" and "expert_selection" for the policies that draw no
+random numbers; nonpadding / importance; moe_use_experts_attention; float32 and
+bfloat16; mtf.gradients over the v1 layer (top_2 / switch / switch_max, ReLU or
+linear experts).  Not built (they raise NotImplementedError): moe_gating
+"ntlb", expert dropout while training, gated (list) activations, gradients of
+the v2 layer, and a mesh with more than one device.
 """
 
 import torch
@@ -260,11 +262,17 @@ class MoEV1Operation(mtf.Operation):
   replaced by output_dim, scalar balancing loss before moe_loss_coef)."""
 
   def __init__(self, inputs, w_gate, wi, wo, importance, output_dim, capacity,
-               gating, activation, name="moe_v1"):
+               gating, activation, k_wo=None, name="moe_v1"):
+    """With k_wo (moe_use_experts_attention, moe.py:514-522) `wo` is the "q_wo"
+    kernel, the operation has a second output projection of the same hidden
+    tensor and its outputs are (q, loss, k)."""
     ins = [inputs, w_gate, wi, wo] + ([importance] if importance is not None
                                       else [])
+    if k_wo is not None:
+      ins.append(k_wo)
     super(MoEV1Operation, self).__init__(ins, name=name)
     self._has_importance = importance is not None
+    self._k_wo = k_wo
     self._capacity = capacity
     self._gating = gating
     self._activation = activation
@@ -273,10 +281,15 @@ class MoEV1Operation(mtf.Operation):
     out_shape = mtf.Shape(inputs.shape.dims[:-1] + [output_dim])
     self._outputs = [mtf.Tensor(self, out_shape, inputs.dtype, index=0),
                      mtf.Tensor(self, mtf.Shape([]), inputs.dtype, index=1)]
+    if k_wo is not None:
+      self._outputs.append(mtf.Tensor(self, out_shape, inputs.dtype, index=2))
 
   def gradient(self, grad_ys):
     """Gradients w.r.t. (inputs, gate kernel, wi, wo[, importance]) from those
     of (outputs, loss); importance carries none."""
+    if self._k_wo is not None:
+      raise NotImplementedError(
+          "backward with moe_use_experts_attention is not implemented")
     if self._gating.router == "expert_selection":
       raise NotImplementedError(
           "backward of expert_selection gating is not implemented")
@@ -303,6 +316,8 @@ class MoEV1Operation(mtf.Operation):
     wi_p = _packed(lowering, wi, dt)
     wo_p = _packed(lowering, wo, dt)
     wg_p = _packed(lowering, w_gate, dt)               # [1, E, M]
+    kwo_p = (_packed(lowering, self._k_wo, dt) if self._k_wo is not None
+             else None)
     o_, g_, s_, m_ = x.shape.to_integer_list
     n_ = self.outputs[0].shape.dims[-1].size
     e_, c_ = self._num_experts, self._capacity
@@ -325,7 +340,7 @@ class MoEV1Operation(mtf.Operation):
       expert_in = (moe_hip.slot_dispatch(xg, r) if by_slot
                    else moe_hip.dispatch(xg, r))
       h = None
-      if save:
+      if save or kwo_p is not None:
         h = torch.empty((e_, groups * c_, wi_p.shape[1]), dtype=dt,
                         device=xg.device)
       y = moe_hip.expert_ffn(expert_in.reshape(e_, groups * c_, m_), wi_p,
@@ -337,14 +352,21 @@ class MoEV1Operation(mtf.Operation):
         # what the gradient operation reads (activations of this step)
         saved.update(x=xg, routing=r, logits=logits, importance=imp_s,
                      expert_in=expert_in, h=h, y=y, w_gate_packed=wg_p)
-      return out.reshape(o_, g_, s_, n_), r.loss.to(dt).reshape(())
+      outs = (out.reshape(o_, g_, s_, n_), r.loss.to(dt).reshape(()))
+      if kwo_p is not None:
+        # the "k" projection of the same hidden tensor (moe.py:514-520)
+        yk = moe_hip.expert_linear(h, kwo_p).reshape(e_, groups, c_, n_)
+        out_k = (moe_hip.slot_combine(yk, r, s_) if by_slot
+                 else moe_hip.combine(yk, r, s_))
+        outs = outs + (out_k.reshape(o_, g_, s_, n_),)
+      return outs
 
     args = [lowering.tensors[x], lowering.tensors[w_gate]]
     if self._has_importance:
       args.append(lowering.tensors[self.inputs[4]])
-    out, loss = mesh_impl.slicewise(fn, *args)
-    lowering.set_tensor_lowering(self.outputs[0], out)
-    lowering.set_tensor_lowering(self.outputs[1], loss)
+    outs = mesh_impl.slicewise(fn, *args)
+    for t, v in zip(self.outputs, outs):
+      lowering.set_tensor_lowering(t, v)
     lowering.operations[self] = saved
 
 
@@ -482,8 +504,6 @@ def transformer_moe_layer_v1(
   if hparams.moe_dropout_rate != 0.0 and train:
     raise NotImplementedError("expert dropout while training is not "
                               "implemented (moe_dropout_rate must be 0)")
-  if hparams.moe_use_experts_attention:
-    raise NotImplementedError("moe_use_experts_attention is not implemented")
   if hparams.moe_gating == "expert_selection":
     gating = _ExpertSelectionGatingSpec(hparams, train, num_microbatches,
                                         nonpadding is not None)
@@ -504,6 +524,20 @@ def transformer_moe_layer_v1(
   wi = mtf_layers.get_dense_kernel_weights(
       inputs, [hidden_dim], [input_dim], [experts_dim], None, name="wi",
       variable_dtype=variable_dtype)
+  if hparams.moe_use_experts_attention:
+    # two output projections of the same hidden tensor (moe.py:514-522)
+    q_wo = mtf_layers.get_dense_kernel_weights(
+        inputs, [output_dim], [hidden_dim], [experts_dim], None, name="q_wo",
+        variable_dtype=variable_dtype)
+    k_wo = mtf_layers.get_dense_kernel_weights(
+        inputs, [output_dim], [hidden_dim], [experts_dim], None, name="k_wo",
+        variable_dtype=variable_dtype)
+    q, loss, k = MoEV1Operation(
+        inputs, w_gate, wi, q_wo, nonpadding, output_dim, expert_capacity,
+        gating, act_name, k_wo=k_wo).outputs
+    outputs = [mtf.reshape(t, batch_and_length_dims + [output_dim])
+               for t in (q, k)]
+    return outputs, loss * hparams.moe_loss_coef
   wo = mtf_layers.get_dense_kernel_weights(
       inputs, [output_dim], [hidden_dim], [experts_dim], None, name="wo",
       variable_dtype=variable_dtype)
@@ -755,7 +789,10 @@ class MoE1D(object):
     if context.losses is not None:
       context.losses.append(loss)
     if not has_length_dim:
-      y = mtf.reshape(y, x_shape)
+      if self._hparams.moe_use_experts_attention:
+        y = [mtf.reshape(y_out, x_shape) for y_out in y]
+      else:
+        y = mtf.reshape(y, x_shape)
     return y
 
 

@@ -696,7 +696,7 @@ def expert_ffn(expert_in, wi, wo, activation, act_dtype):
 def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
                  nonpadding=None, activation="relu", num_microbatches=None,
                  logit_bias=None, second_uniform=None, dense=True,
-                 mesh_dim_size=1, weights_are_cast=False):
+                 mesh_dim_size=1, weights_are_cast=False, k_wo=None):
   """transformer_moe_layer_v1 forward (transformer/moe.py:191-525).
 
   x: [batch..., length, M] float32 array holding activation-dtype values.
@@ -706,9 +706,27 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
   the skewed-routing config; the reference router has no bias).
   dense=True follows the reference dataflow literally (one-hot [G,S,E,C]
   tensors, einsums); dense=False uses the index form.
+  k_wo [E, H, N]: with hparams.moe_use_experts_attention `wo` is the "q_wo"
+  kernel and k_wo the "k_wo" kernel of a second output projection of the same
+  hidden tensor (moe.py:514-522); the output is then the list [q, k].
 
   Returns (output [batch..., length, N], loss scalar, aux dict).
   """
+  if getattr(hp, "moe_use_experts_attention", False):
+    if k_wo is None:
+      raise ValueError("moe_use_experts_attention needs the k_wo kernel")
+    import copy
+    hp1 = copy.copy(hp)
+    hp1.moe_use_experts_attention = False
+    kw = dict(nonpadding=nonpadding, activation=activation,
+              num_microbatches=num_microbatches, logit_bias=logit_bias,
+              second_uniform=second_uniform, dense=dense,
+              mesh_dim_size=mesh_dim_size, weights_are_cast=weights_are_cast)
+    # the two outputs share everything up to the hidden tensor, so each equals
+    # the plain layer with its own output kernel
+    q, loss, aux = moe_layer_v1(x, w_gate, wi, wo, hp1, train, act_dtype, **kw)
+    k, _, _ = moe_layer_v1(x, w_gate, wi, k_wo, hp1, train, act_dtype, **kw)
+    return [q, k], loss, aux
   if hp.moe_gating not in ("top_2", "switch", "switch_max", "expert_selection"):
     raise ValueError("unknown hparams.moe_gating=%s" % hp.moe_gating)
   x = cast_act(x, act_dtype)

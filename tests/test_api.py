@@ -300,6 +300,21 @@ def test_product_does_not_import_the_oracle():
         assert "oracle" not in text, os.path.join(dirpath, f)
 
 
+def test_experts_attention_graph():
+  """moe_use_experts_attention returns [q, k] and creates "q_wo" / "k_wo"
+  instead of "wo" (transformer/moe.py:514-522)."""
+  graph, _, x, dims = graph_input()
+  with mtf.variable_scope("att"):
+    outs, loss = moe.transformer_moe_layer_v1(
+        x, dims[-1], hparams(moe_use_experts_attention=True), True,
+        mtf.VariableDType(torch.float32))
+  assert isinstance(outs, list) and [o.shape for o in outs] == [mtf.Shape(dims)] * 2
+  assert loss.shape == mtf.Shape([])
+  assert sorted(v.name for v in graph.all_variables) == [
+      "att/k_wo/kernel", "att/q_wo/kernel", "att/top_2_gating/kernel",
+      "att/wi/kernel"]
+
+
 def test_gradients_builds_the_backward_operation():
   """mtf.gradients (mesh_tensorflow/ops.py:5254-5291) over the layer: one
   gradient per requested tensor with that tensor's shape and dtype, None for a

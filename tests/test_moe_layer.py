@@ -472,3 +472,48 @@ def test_v1_expert_selection_matches_oracle():
                              want_loss, rtol=1e-4)
   with pytest.raises(ValueError, match="needs nonpadding"):
     run_v1(x, w, hp, False, "float32")
+
+
+@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
+def test_v1_experts_attention(act_dtype):
+  """moe_use_experts_attention: two output projections ("q_wo", "k_wo") of the
+  same hidden tensor (transformer/moe.py:514-522)."""
+  b, l, m, hdim, e, group = 2, 64, 64, 128, 4, 32
+  rng = np.random.default_rng(501)
+  w = dict(w_gate=H.normal_weights(rng, (m, e), m),
+           wi=H.normal_weights(rng, (e, m, hdim), m),
+           wo=H.normal_weights(rng, (e, hdim, m), hdim))
+  k_wo = H.normal_weights(rng, (e, hdim, m), hdim)
+  x = H.safe_tokens(rng, b * l, m, w["w_gate"], act_dtype).reshape(b, l, m)
+  hp, ohp = make_hparams(moe_num_experts=e, moe_hidden_size=hdim,
+                         moe_group_size=group, moe_use_experts_attention=True)
+  dt = H.ACT_TORCH[act_dtype]
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  dims = [mtf.Dimension("batch", b), mtf.Dimension("length", l),
+          mtf.Dimension("d_model", m)]
+  xt = mtf.import_tf_tensor(mesh, torch.from_numpy(x).to(dt), mtf.Shape(dims))
+  with mtf.variable_scope("moe"):
+    outs, loss = moe.transformer_moe_layer_v1(
+        xt, dims[-1], hp, True, mtf.VariableDType(torch.float32, torch.float32, dt))
+  assert isinstance(outs, list) and len(outs) == 2
+  assert sorted(v.name for v in graph.all_variables) == [
+      "moe/k_wo/kernel", "moe/q_wo/kernel", "moe/top_2_gating/kernel",
+      "moe/wi/kernel"]
+  lowering = mtf.Lowering(
+      graph, {mesh: mtf.HipMeshImpl()},
+      initial_values={"moe/top_2_gating/kernel": w["w_gate"],
+                      "moe/wi/kernel": w["wi"], "moe/q_wo/kernel": w["wo"],
+                      "moe/k_wo/kernel": k_wo})
+  q, k = (H.to_np(lowering.export_to_tf_tensor(t)) for t in outs)
+  want, want_loss, _ = O.moe_layer_v1(x, w["w_gate"], w["wi"], w["wo"], ohp,
+                                      True, act_dtype, dense=False, k_wo=k_wo)
+  np.testing.assert_allclose(q, want[0], **H.value_tolerance(act_dtype))
+  np.testing.assert_allclose(k, want[1], **H.value_tolerance(act_dtype))
+  # each output is bit for bit the plain layer with that output kernel
+  hp_plain, _ = make_hparams(moe_num_experts=e, moe_hidden_size=hdim,
+                             moe_group_size=group)
+  plain_k, _, _, _ = run_v1(x, dict(w, wo=k_wo), hp_plain, True, act_dtype)
+  np.testing.assert_array_equal(k, plain_k)
+  with pytest.raises(NotImplementedError, match="experts_attention"):
+    mtf.gradients([outs[0]], [xt])
