@@ -894,6 +894,50 @@ def gating_backward(logits, r, gating, d_gate_1, d_gate_2, d_loss,
   return dlogits.astype(F32)
 
 
+def combine_backward(dout, y, r, act_dtype):
+  """Backward of the combine einsum (moe.py:509-510) in gather form.
+  dout [G,S,N], y [E,G,C,N] -> dy [E,G,C,N] (activation dtype; zero rows for
+  empty slots), dgate [G,S,2] float32 (zero where not kept)."""
+  g_, s_, _ = dout.shape
+  dy = np.zeros_like(y)
+  dgate = np.zeros((g_, s_, 2), F32)
+  for ki, (k, w) in enumerate(zip("12", combine_weights(r, act_dtype))):
+    gi, si = np.nonzero(r["kept_" + k])
+    ei, ci = r["index_" + k][gi, si], r["pos_" + k][gi, si]
+    dgate[gi, si, ki] = (dout[gi, si] * y[ei, gi, ci]).sum(-1, dtype=F32)
+    dy[ei, gi, ci] = cast_act(w[gi, si][:, None] * dout[gi, si], act_dtype)
+  return dy, dgate
+
+
+def dispatch_backward(dxe, r, act_dtype):
+  """Backward of the dispatch einsum (moe.py:443-447): a token gathers the
+  rows of the slots it was dispatched to.  dxe [E,G,C,M] -> float32 [G,S,M]
+  (not yet rounded: the router's share is added before the cast)."""
+  _, g_, _, m_ = dxe.shape
+  s_ = r["kept_1"].shape[1]
+  dx = np.zeros((g_, s_, m_), F32)
+  for k, w in zip("12", combine_weights(r, act_dtype)):
+    gi, si = np.nonzero(r["kept_" + k] & (w != 0))
+    dx[gi, si] += dxe[r["index_" + k][gi, si], gi, r["pos_" + k][gi, si]]
+  return dx
+
+
+def expert_ffn_backward(xe, wi_a, wo_a, dy, activation, act_dtype):
+  """Backward of the two expert einsums (moe.py:469-486): float32 accumulate,
+  activation-dtype results.  xe [E,R,M], dy [E,R,N]; returns
+  (dxe [E,R,M], dwi [E,M,H], dwo [E,H,N])."""
+  h = cast_act(np.matmul(xe, wi_a), act_dtype)
+  if activation == "relu":
+    h = cast_act(np.maximum(h, F32(0.0)), act_dtype)
+  dh = cast_act(np.matmul(dy, wo_a.transpose(0, 2, 1)), act_dtype)
+  if activation == "relu":
+    dh = dh * (h > 0)
+  dwo = cast_act(np.matmul(h.transpose(0, 2, 1), dy), act_dtype)
+  dxe = cast_act(np.matmul(dh, wi_a.transpose(0, 2, 1)), act_dtype)
+  dwi = cast_act(np.matmul(xe.transpose(0, 2, 1), dh), act_dtype)
+  return dxe, dwi, dwo
+
+
 def moe_layer_v1_backward(x, w_gate, wi, wo, hp, train, act_dtype, d_out,
                           d_loss=0.0, nonpadding=None, activation="relu",
                           num_microbatches=None, logit_bias=None):
@@ -929,41 +973,13 @@ def moe_layer_v1_backward(x, w_gate, wi, wo, hp, train, act_dtype, d_out,
   dout = cast_act(np.asarray(d_out, F32), act_dtype).reshape(g_, s_, n_)
   y = aux["expert_out"]                                          # [E,G,C,N]
   expert_in = aux["expert_in"]                                   # [E,G,C,M]
-  w1, w2 = combine_weights(aux, act_dtype)
 
-  # combine backward: d(weights) and d(expert outputs)
-  dy = np.zeros_like(y)
-  dgate = []
-  for k, w in (("1", w1), ("2", w2)):
-    dgk = np.zeros((g_, s_), F32)
-    sel = aux["kept_" + k]
-    gi, si = np.nonzero(sel)
-    ei, ci = aux["index_" + k][gi, si], aux["pos_" + k][gi, si]
-    dgk[gi, si] = (dout[gi, si] * y[ei, gi, ci]).sum(-1, dtype=F32)
-    dy[ei, gi, ci] = cast_act(w[gi, si][:, None] * dout[gi, si], act_dtype)
-    dgate.append(dgk)
-
-  # expert FFN backward (float32 accumulate, activation-dtype results)
+  dy, dgate = combine_backward(dout, y, aux, act_dtype)
   r_ = g_ * c_
-  xe = expert_in.reshape(e_, r_, m_)
-  h = cast_act(np.matmul(xe, wi_a), act_dtype)
-  if activation == "relu":
-    h = cast_act(np.maximum(h, F32(0.0)), act_dtype)
-  dy2 = dy.reshape(e_, r_, n_)
-  dh = cast_act(np.matmul(dy2, wo_a.transpose(0, 2, 1)), act_dtype)
-  if activation == "relu":
-    dh = dh * (h > 0)
-  dwo = cast_act(np.matmul(h.transpose(0, 2, 1), dy2), act_dtype)
-  dxe = cast_act(np.matmul(dh, wi_a.transpose(0, 2, 1)), act_dtype)
-  dwi = cast_act(np.matmul(xe.transpose(0, 2, 1), dh), act_dtype)
-  dxe = dxe.reshape(e_, g_, c_, m_)
-
-  # dispatch backward: a token gathers the rows of the slots it was sent to
-  dx = np.zeros((g_, s_, m_), F32)
-  for k, w in (("1", w1), ("2", w2)):
-    sel = aux["kept_" + k] & (w != 0)
-    gi, si = np.nonzero(sel)
-    dx[gi, si] += dxe[aux["index_" + k][gi, si], gi, aux["pos_" + k][gi, si]]
+  dxe, dwi, dwo = expert_ffn_backward(
+      expert_in.reshape(e_, r_, m_), wi_a, wo_a, dy.reshape(e_, r_, n_),
+      activation, act_dtype)
+  dx = dispatch_backward(dxe.reshape(e_, g_, c_, m_), aux, act_dtype)
 
   # gating and router backward
   importance = None
@@ -974,14 +990,15 @@ def moe_layer_v1_backward(x, w_gate, wi, wo, hp, train, act_dtype, d_out,
   # the returned loss is aux * moe_loss_coef in the activation dtype
   d_aux = F32(cast_act(F32(d_loss), act_dtype)
               * cast_act(F32(hp.moe_loss_coef), act_dtype))
-  dlogits = gating_backward(aux["logits"], aux, hp.moe_gating, dgate[0],
-                            dgate[1], d_aux, importance, num_microbatches, z)
+  dlogits = gating_backward(aux["logits"], aux, hp.moe_gating, dgate[..., 0],
+                            dgate[..., 1], d_aux, importance, num_microbatches,
+                            z)
   dwg = np.matmul(xg.reshape(-1, m_).T.astype(F32),
                   dlogits.reshape(-1, e_)).astype(F32)
   dx = dx + np.matmul(dlogits, wg_a.T.astype(F32))
   return dict(dx=cast_act(dx, act_dtype).reshape(lead + (m_,)),
               dw_gate=cast_act(dwg, act_dtype), dwi=dwi, dwo=dwo,
-              dlogits=dlogits, dgate=np.stack(dgate, -1), aux=aux)
+              dlogits=dlogits, dgate=dgate, aux=aux)
 
 
 def moe_layer_v2(x, w_outer, w_inner, wi, wo, hp, train, act_dtype="float32",
@@ -1086,5 +1103,71 @@ def moe_layer_v2(x, w_outer, w_inner, wi, wo, hp, train, act_dtype="float32",
   loss = cast_act(rx["loss"] + ry["loss"], act_dtype)            # :801
   aux = dict(outer=rx, inner=ry, capacity_x=c_, capacity_y=d_,
              groups_x=(g1, s_), groups_y=(h0, t_), importance_inner=imp2,
-             logits_outer=logits_x, logits_inner=logits_y)
+             importance_outer=importance, logits_outer=logits_x,
+             logits_inner=logits_y, expert_in_x=ein, expert_in_y=ein_y,
+             expert_out_y=yy, expert_out_x=eo_x)
   return out, _scale_loss(loss, hp.moe_loss_coef, act_dtype), aux
+
+
+def moe_layer_v2_backward(x, w_outer, w_inner, wi, wo, hp, train, act_dtype,
+                          d_out, d_loss=0.0, nonpadding=None,
+                          num_microbatches=None):
+  """Gradients of (outputs, loss) of moe_layer_v2 w.r.t. x and the four
+  kernels: the v1 pieces applied twice, inner level first.  The importance of
+  the inner level is a comparison of the slot weights (moe.py:725-727) and
+  carries no gradient.  Returns dict(dx, dw_outer, dw_inner, dwi, dwo)."""
+  if hp.moe_use_second_place_loss:
+    raise NotImplementedError("backward of the second-place loss")
+  _, _, aux = moe_layer_v2(x, w_outer, w_inner, wi, wo, hp, train, act_dtype,
+                           nonpadding=nonpadding,
+                           num_microbatches=num_microbatches, dense=False)
+  x = cast_act(x, act_dtype)
+  orig_shape = x.shape
+  m_ = x.shape[-1]
+  rx, ry = aux["outer"], aux["inner"]
+  x_e, y_e = hp.moe_num_experts
+  c_, d_ = aux["capacity_x"], aux["capacity_y"]
+  h0, t_ = aux["groups_y"]
+  ag, s_ = rx["kept_1"].shape
+  xg = x.reshape(ag, s_, m_)
+  wo_a, wi_a = cast_act(wo, act_dtype), cast_act(wi, act_dtype)
+  w_out_a, w_in_a = cast_act(w_outer, act_dtype), cast_act(w_inner, act_dtype)
+  h_dim, n_ = wi_a.shape[-1], wo_a.shape[-1]
+  dout = cast_act(np.asarray(d_out, F32), act_dtype).reshape(ag, s_, n_)
+  d_aux = F32(cast_act(F32(d_loss), act_dtype)
+              * cast_act(F32(hp.moe_loss_coef), act_dtype))
+
+  # outer combine, then inner combine
+  d_eo_x, dgate_x = combine_backward(dout, aux["expert_out_x"], rx, act_dtype)
+  d_out_y = d_eo_x.reshape(x_e * h0, t_, n_)
+  dyy, dgate_y = combine_backward(d_out_y, aux["expert_out_y"], ry, act_dtype)
+  # experts
+  ein_y = aux["expert_in_y"].reshape(y_e * x_e, h0 * d_, m_)
+  dein_y, dwi, dwo = expert_ffn_backward(
+      ein_y, wi_a.reshape(y_e * x_e, m_, h_dim),
+      wo_a.reshape(y_e * x_e, h_dim, n_), dyy.reshape(y_e * x_e, h0 * d_, n_),
+      "relu", act_dtype)
+  # inner gating, router and dispatch
+  imp_in = aux["importance_inner"].reshape(x_e * h0, t_)
+  dlogits_y = gating_backward(aux["logits_inner"], ry, "top_2",
+                              dgate_y[..., 0], dgate_y[..., 1], d_aux, imp_in,
+                              num_microbatches)
+  inputs_y = aux["expert_in_x"].reshape(x_e, h0 * t_, m_)
+  dl_y = dlogits_y.reshape(x_e, h0 * t_, y_e)
+  dw_inner = np.matmul(inputs_y.transpose(0, 2, 1).astype(F32), dl_y)
+  dxin = dispatch_backward(dein_y.reshape(y_e, x_e * h0, d_, m_), ry, act_dtype)
+  dxin = dxin.reshape(x_e, h0 * t_, m_) + np.matmul(
+      dl_y, w_in_a.transpose(0, 2, 1).astype(F32))
+  d_ein = cast_act(dxin, act_dtype).reshape(x_e, ag, c_, m_)
+  # outer gating, router and dispatch
+  dlogits_x = gating_backward(aux["logits_outer"], rx, "top_2",
+                              dgate_x[..., 0], dgate_x[..., 1], d_aux,
+                              aux["importance_outer"], num_microbatches)
+  dw_outer = np.matmul(xg.reshape(-1, m_).T.astype(F32),
+                       dlogits_x.reshape(-1, x_e))
+  dx = dispatch_backward(d_ein, rx, act_dtype) + np.matmul(
+      dlogits_x, w_out_a.T.astype(F32))
+  return dict(dx=cast_act(dx, act_dtype).reshape(orig_shape),
+              dw_outer=cast_act(dw_outer, act_dtype),
+              dw_inner=cast_act(dw_inner, act_dtype),
+              dwi=dwi.reshape(wi_a.shape), dwo=dwo.reshape(wo_a.shape), aux=aux)

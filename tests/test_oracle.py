@@ -831,3 +831,98 @@ def test_backward_against_central_differences(gating):
       fd = (scalar(*plus) - scalar(*minus)) / (2 * eps)
       an = float((grads[which].astype(np.float64) * d).sum())
       assert abs(fd - an) <= 2e-4 * max(1.0, abs(fd)), (which, trial, fd, an)
+
+
+def _f64_layer_v2(x, w_outer, w_inner, wi, wo, aux, m1_outer, coef, mb):
+  """Independent float64 forward of the hierarchical layer with the routing of
+  BOTH levels held fixed (experts, kept masks, slots, inner importance and
+  density counts from `aux`), written per (token, choice) pair."""
+  rx, ry = aux["outer"], aux["inner"]
+  ag, s = rx["kept_1"].shape
+  x_e, y_e = w_inner.shape[0], w_inner.shape[2]
+  c = aux["capacity_x"]
+  h0, t_ = aux["groups_y"]
+  imp_in = (aux["importance_inner"].reshape(x_e * h0, t_) == 1).astype(np.float64)
+
+  def gates(p, i1, i2, m1, k1, k2):
+    g1 = p[i1] * m1
+    g2 = p[i2] * (1.0 - (i2 == i1) * m1)
+    den = g1 + g2 + 1e-9
+    return g1 / den * k1, g2 / den * k2
+
+  n = wo.shape[-1]
+  out = np.zeros((ag, s, n))
+  px = scipy.special.softmax(x @ w_outer, axis=-1)               # [ag,s,X]
+  py_sum = np.zeros((x_e * h0, y_e))                             # inner proxy
+  for gi in range(ag):
+    for si in range(s):
+      gx = gates(px[gi, si], rx["index_1"][gi, si], rx["index_2"][gi, si],
+                 m1_outer[gi, si], float(rx["kept_1"][gi, si]),
+                 float(rx["kept_2"][gi, si]))
+      for k in range(2):
+        if not rx["kept_%d" % (k + 1)][gi, si]:
+          continue
+        xe = int(rx["index_%d" % (k + 1)][gi, si])
+        slot = gi * c + int(rx["pos_%d" % (k + 1)][gi, si])      # in [0, ag*c)
+        hh, tt = divmod(slot, t_)
+        row = xe * h0 + hh
+        v = x[gi, si]
+        py = scipy.special.softmax(v @ w_inner[xe])
+        py_sum[row] += py * imp_in[row, tt]
+        gy = gates(py, ry["index_1"][row, tt], ry["index_2"][row, tt],
+                   imp_in[row, tt], float(ry["kept_1"][row, tt]),
+                   float(ry["kept_2"][row, tt]))
+        acc = np.zeros(n)
+        for kk in range(2):
+          ye = int(ry["index_%d" % (kk + 1)][row, tt])
+          acc += gy[kk] * (np.maximum(v @ wi[ye, xe], 0.0) @ wo[ye, xe])
+        out[gi, si] += gx[k] * acc
+  # losses with the density counts fixed
+  e1 = (rx["index_1"][..., None] == np.arange(x_e)) * m1_outer[..., None]
+  loss_x = ((px * m1_outer[..., None]).mean(1) * e1.mean(1)).mean() * x_e * x_e
+  e2 = (ry["index_1"][..., None] == np.arange(y_e)) * imp_in[..., None]
+  # empty outer slots hold zero rows: their softmax is uniform but their
+  # importance is 0, so they add nothing to the inner proxy
+  loss_y = ((py_sum / t_) * e2.mean(1)).mean() * y_e * y_e
+  return out, (loss_x + loss_y) / mb * coef
+
+
+def test_v2_backward_against_central_differences():
+  rng = np.random.default_rng(62)
+  b, l, m, h = 2, 16, 5, 7
+  x_e, y_e = 2, 3
+  x = rng.standard_normal((b, l, m)).astype(np.float32)
+  w_outer = rng.standard_normal((m, x_e)).astype(np.float32)
+  w_inner = rng.standard_normal((x_e, m, y_e)).astype(np.float32)
+  wi = (rng.standard_normal((y_e, x_e, m, h)) / 2).astype(np.float32)
+  wo = (rng.standard_normal((y_e, x_e, h, m)) / 3).astype(np.float32)
+  nonpad = (rng.random((b, l)) < 0.85).astype(np.float32)
+  d_out = rng.standard_normal((b, l, m)).astype(np.float32)
+  d_loss, mb = 1.3, 2
+  hp = _hp(moe_num_experts=[x_e, y_e], moe_hidden_size=h, moe_group_size=16,
+           moe_capacity_factor_train=1.5, moe_capacity_factor_second_level=1.0,
+           moe_min_expert_capacity=2, moe_loss_coef=0.5)
+  got = O.moe_layer_v2_backward(x, w_outer, w_inner, wi, wo, hp, True,
+                                "float32", d_out, d_loss, nonpadding=nonpad,
+                                num_microbatches=mb)
+  aux = got["aux"]
+  rx, ry = aux["outer"], aux["inner"]
+  assert not (rx["kept_1"] | rx["kept_2"]).all() or not ry["kept_2"].all()
+  ag, s = rx["kept_1"].shape
+  m1 = (nonpad.reshape(ag, s) == 1).astype(np.float64)
+
+  def scalar(xv, a, bq, cq, dq):
+    out, loss = _f64_layer_v2(xv.reshape(ag, s, m), a, bq, cq, dq, aux, m1,
+                              0.5, mb)
+    return (out * d_out.reshape(out.shape)).sum() + d_loss * loss
+  base = [a.astype(np.float64) for a in (x, w_outer, w_inner, wi, wo)]
+  grads = [got["dx"], got["dw_outer"], got["dw_inner"], got["dwi"], got["dwo"]]
+  eps = 1e-6
+  for which in range(5):
+    for trial in range(2):
+      d = rng.standard_normal(base[which].shape)
+      plus = [a + eps * d if i == which else a for i, a in enumerate(base)]
+      minus = [a - eps * d if i == which else a for i, a in enumerate(base)]
+      fd = (scalar(*plus) - scalar(*minus)) / (2 * eps)
+      an = float((grads[which].astype(np.float64) * d).sum())
+      assert abs(fd - an) <= 1e-4 * max(1.0, abs(fd)), (which, trial, fd, an)
