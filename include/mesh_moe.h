@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 5
+#define MESH_MOE_ABI_VERSION 6
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -361,7 +361,8 @@ size_t mesh_moe_gating_backward_workspace_bytes(int G, int E);
  * Backward of the gating (transformer/moe.py:1391-1496 for router 0 = top-2,
  * :1207-1306 for router 1 = switch / switch_max): d(logits) from the
  * gradients of the two combine weights and of the layer's returned loss.
- *   logits [G,S,E] float32 (the forward values), importance as in the forward
+ *   logits [G,S,E] float32 (the forward values), importance and
+ *   importance_from_slot_gate as in the forward
  *   idx, kept [G,S,2] from the forward; dgate [G,S,2] float32 from
  *   mesh_moe_combine_backward
  *   d_loss [1] float32 ON THE DEVICE: gradient w.r.t. the returned loss
@@ -371,7 +372,8 @@ size_t mesh_moe_gating_backward_workspace_bytes(int G, int E);
  * The second-place loss (moe_use_second_place_loss) is not covered.
  */
 int mesh_moe_gating_backward(const float* logits, const void* importance,
-                             int importance_dtype, const int32_t* idx,
+                             int importance_dtype,
+                             int importance_from_slot_gate, const int32_t* idx,
                              const uint8_t* kept, const float* dgate,
                              const float* d_loss, double loss_scale, int G,
                              int S, int E, int router, int use_z_loss,
@@ -399,14 +401,17 @@ int mesh_moe_router_backward_weights(const void* x, const float* dlogits,
  * float32 accumulate, one rounding.  The dispatch tensor itself carries no
  * gradient (it is a bool cast, moe.py:1510-1511).
  *   dexpert_in [E,G,C,M] dtype; dlogits [G,S,E] float32 or NULL;
- *   w_gate_packed [E,M] dtype (NULL iff dlogits is); dx [G,S,M] dtype
+ *   w_gate_packed [G / groups_per_router, E, M] dtype (NULL iff dlogits is):
+ *   one router per groups_per_router consecutive groups (G for a single
+ *   router; the inner level of the hierarchical layer has one per outer
+ *   expert, moe.py:743-753); dx [G,S,M] dtype
  */
 int mesh_moe_dispatch_backward(const void* dexpert_in, const int32_t* idx,
                                const int32_t* pos, const float* gate,
                                const uint8_t* kept, const float* dlogits,
-                               const void* w_gate_packed, void* dx, int G,
-                               int S, int E, int C, int M, int dtype,
-                               void* stream);
+                               const void* w_gate_packed,
+                               int groups_per_router, void* dx, int G, int S,
+                               int E, int C, int M, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -143,7 +143,9 @@ __global__ __launch_bounds__(256) void combine_backward_kernel(
 // whose activation-dtype gate is non-zero, transformer/moe.py:443-447,
 // :1510-1511) and logits[t] = float(x[t]) . w_gate (moe.py:1384-1390).  Hence
 //   dx[t] = sum_k dispatched_k * dexpert_in[slot_k] + dlogits[t] . w_gate^T
-// float32 accumulate, one rounding.  w_gate comes K-contiguous ([E, M]).
+// float32 accumulate, one rounding.  w_gate comes K-contiguous ([E, M]), one
+// per `groups_per_router` consecutive groups (the inner level of the
+// hierarchical layer has a router per outer expert, moe.py:743-753).
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void dispatch_backward_kernel(
@@ -151,13 +153,14 @@ __global__ __launch_bounds__(256) void dispatch_backward_kernel(
     const int32_t* __restrict__ pos, const float* __restrict__ gate,
     const uint8_t* __restrict__ kept, const float* __restrict__ dlogits,
     const T* __restrict__ wgp, T* __restrict__ dx, int G, int S, int E, int C,
-    int M, int64_t T_tokens, bool vec) {
+    int M, int64_t T_tokens, int groups_per_router, bool vec) {
   constexpr int VN = Vec16B<T>::N;
   const int lane = threadIdx.x & 63;
   const int64_t t =
       (int64_t)blockIdx.x * BW_ROWS_PER_BLOCK + (threadIdx.x >> 6);
   if (t >= T_tokens) return;
   const int g = (int)(t / S);
+  if (wgp != nullptr) wgp += (int64_t)(g / groups_per_router) * E * M;
   const T* src[2] = {nullptr, nullptr};
 #pragma unroll
   for (int k = 0; k < 2; ++k) {
@@ -217,6 +220,7 @@ struct GateBackwardParams {
   int G, S, E;
   int router;           // 0 = top-2, 1 = switch / switch_max
   int has_importance;
+  int importance_from_slot_gate;  // importance = 0.5*((w>0.5)+(w>0))
   int num_microbatches;
   int use_z_loss;
   float z_loss_coef;
@@ -235,7 +239,11 @@ __global__ __launch_bounds__(256) void gate_count_kernel(
   for (int s = threadIdx.x; s < p.S; s += blockDim.x) {
     const int64_t t = (int64_t)g * p.S + s;
     bool one = true;
-    if (importance != nullptr) one = load_f32<IT>(importance + t) == 1.0f;
+    if (importance != nullptr) {
+      const float imp = load_f32<IT>(importance + t);
+      // from a slot weight w: 0.5*((w>0.5)+(w>0)) == 1  <=>  w > 0.5
+      one = p.importance_from_slot_gate ? imp > 0.5f : imp == 1.0f;
+    }
     if (one) atomicAdd(&cnt[p.E], 1);
     // top-2: density_1 counts mask_1 after the importance mask
     // (moe.py:1402-1420); switch: every token's arg-max (moe.py:1224)
@@ -270,8 +278,10 @@ __global__ __launch_bounds__(256) void gating_backward_kernel(
   const float lse = logf(s) + m;
   const float neglse = -lse;
   float m1 = 1.0f;
-  if (importance != nullptr)
-    m1 = load_f32<IT>(importance + t) == 1.0f ? 1.0f : 0.0f;
+  if (importance != nullptr) {
+    const float imp = load_f32<IT>(importance + t);
+    m1 = (p.importance_from_slot_gate ? imp > 0.5f : imp == 1.0f) ? 1.0f : 0.0f;
+  }
   const int i1 = idx[t * 2], i2 = idx[t * 2 + 1];
   const float k1 = kept[t * 2] ? 1.0f : 0.0f, k2 = kept[t * 2 + 1] ? 1.0f : 0.0f;
   const float mb =
@@ -435,10 +445,15 @@ extern "C" int mesh_moe_combine_backward(
 extern "C" int mesh_moe_dispatch_backward(
     const void* dexpert_in, const int32_t* idx, const int32_t* pos,
     const float* gate, const uint8_t* kept, const float* dlogits,
-    const void* w_gate_packed, void* dx, int G, int S, int E, int C, int M,
-    int dtype, void* stream) {
+    const void* w_gate_packed, int groups_per_router, void* dx, int G, int S,
+    int E, int C, int M, int dtype, void* stream) {
   MOE_REQUIRE(dexpert_in && idx && pos && gate && kept && dx, MESH_MOE_E_ARG,
               "dispatch_backward: null pointer");
+  MOE_REQUIRE(w_gate_packed == nullptr ||
+                  (groups_per_router >= 1 && G % groups_per_router == 0),
+              MESH_MOE_E_ARG,
+              "dispatch_backward: G=%d is not a multiple of "
+              "groups_per_router=%d", G, groups_per_router);
   MOE_REQUIRE((dlogits == nullptr) == (w_gate_packed == nullptr),
               MESH_MOE_E_ARG,
               "dispatch_backward: dlogits and w_gate_packed go together");
@@ -459,12 +474,13 @@ extern "C" int mesh_moe_dispatch_backward(
   if (dtype == MESH_MOE_F32)
     dispatch_backward_kernel<float><<<(unsigned)nblocks, 256, 0, st>>>(
         (const float*)dexpert_in, idx, pos, gate, kept, dlogits,
-        (const float*)w_gate_packed, (float*)dx, G, S, E, C, M, T_tokens, vec);
+        (const float*)w_gate_packed, (float*)dx, G, S, E, C, M, T_tokens,
+        groups_per_router, vec);
   else
     dispatch_backward_kernel<bf16_t><<<(unsigned)nblocks, 256, 0, st>>>(
         (const bf16_t*)dexpert_in, idx, pos, gate, kept, dlogits,
         (const bf16_t*)w_gate_packed, (bf16_t*)dx, G, S, E, C, M, T_tokens,
-        vec);
+        groups_per_router, vec);
   MOE_CHECK_LAUNCH("dispatch_backward");
   return 0;
 }
@@ -476,8 +492,9 @@ extern "C" size_t mesh_moe_gating_backward_workspace_bytes(int G, int E) {
 
 extern "C" int mesh_moe_gating_backward(
     const float* logits, const void* importance, int importance_dtype,
-    const int32_t* idx, const uint8_t* kept, const float* dgate,
-    const float* d_loss, double loss_scale, int G, int S, int E, int router,
+    int importance_from_slot_gate, const int32_t* idx, const uint8_t* kept,
+    const float* dgate, const float* d_loss, double loss_scale, int G, int S,
+    int E, int router,
     int use_z_loss, double z_loss_coef, int num_microbatches, float* dlogits,
     void* workspace, size_t workspace_bytes, void* stream) {
   MOE_REQUIRE(logits && idx && kept && dgate && d_loss && dlogits && workspace,
@@ -495,6 +512,7 @@ extern "C" int mesh_moe_gating_backward(
   p.G = G; p.S = S; p.E = E;
   p.router = router;
   p.has_importance = importance != nullptr;
+  p.importance_from_slot_gate = importance_from_slot_gate ? 1 : 0;
   p.num_microbatches = num_microbatches;
   p.use_z_loss = (use_z_loss && router == 1) ? 1 : 0;
   p.z_loss_coef = (float)z_loss_coef;

@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 5
+ABI_VERSION = 6
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -84,15 +84,17 @@ _SIGNATURES = {
     "mesh_moe_gating_backward_workspace_bytes": (ctypes.c_size_t, [
         ctypes.c_int, ctypes.c_int]),
     "mesh_moe_gating_backward": (ctypes.c_int, [
-        _vp, _vp, ctypes.c_int, _vp, _vp, _vp, _vp, ctypes.c_double,
+        _vp, _vp, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, _vp,
+        ctypes.c_double,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_double, ctypes.c_int, _vp, _vp, ctypes.c_size_t, _vp]),
     "mesh_moe_router_backward_weights": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, _vp]),
     "mesh_moe_dispatch_backward": (ctypes.c_int, [
-        _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
-        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
+        _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        _vp]),
     "mesh_moe_expert_choice_workspace_bytes": (ctypes.c_size_t, [
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "mesh_moe_expert_choice_gating": (ctypes.c_int, [
@@ -605,7 +607,8 @@ def expert_ffn_backward(expert_in, h, dy, wi, wo, activation="relu"):
 
 
 def gating_backward(logits, r, dgate, d_loss, loss_scale, router="top_2",
-                    importance=None, z_loss=None, num_microbatches=None):
+                    importance=None, z_loss=None, num_microbatches=None,
+                    importance_from_slot_gate=False):
   """d(logits) [G, S, E] float32.  d_loss: float32 tensor of one element on the
   device (gradient w.r.t. the layer's returned loss); loss_scale:
   moe_loss_coef."""
@@ -622,6 +625,7 @@ def gating_backward(logits, r, dgate, d_loss, loss_scale, router="top_2",
   with _stage("gating_backward"):
     _check(lib.mesh_moe_gating_backward(
         _dev(logits, "logits", torch.float32), ip, icode,
+        int(bool(importance_from_slot_gate)),
         _dev(r.idx, "idx", torch.int32, (g, s, 2)),
         _dev(r.kept, "kept", torch.uint8, (g, s, 2)),
         _dev(dgate, "dgate", torch.float32, (g, s, 2)),
@@ -649,8 +653,8 @@ def router_backward_weights(x, dlogits):
 
 def dispatch_backward(dexpert_in, r, group_size, dlogits=None,
                       w_gate_packed=None):
-  """dexpert_in [E, G, C, M] (+ dlogits [G, S, E], w_gate_packed [E, M]) ->
-  dx [G, S, M]."""
+  """dexpert_in [E, G, C, M] (+ dlogits [G, S, E], w_gate_packed [B, E, M] with
+  one router per G / B consecutive groups) -> dx [G, S, M]."""
   lib = load_library()
   e, g, c, m = dexpert_in.shape
   s = group_size
@@ -658,12 +662,19 @@ def dispatch_backward(dexpert_in, r, group_size, dlogits=None,
   dx = torch.empty((g, s, m), dtype=dt, device=dexpert_in.device)
   ip, pp, gp, kp = _routing_ptrs(r, g, s)
   dlp = wgp = None
+  gpr = g
   if dlogits is not None:
     dlp = _dev(dlogits, "dlogits", torch.float32, (g, s, e))
-    wgp = _dev(w_gate_packed, "w_gate_packed", dt, (e, m))
+    if w_gate_packed.dim() == 2:
+      w_gate_packed = w_gate_packed.reshape(1, e, m)
+    routers = w_gate_packed.shape[0]
+    if g % routers:
+      raise MoeHipError("dispatch_backward: %d groups, %d routers" % (g, routers))
+    gpr = g // routers
+    wgp = _dev(w_gate_packed, "w_gate_packed", dt, (routers, e, m))
   with _stage("dispatch_backward"):
     _check(lib.mesh_moe_dispatch_backward(
-        _dev(dexpert_in, "dexpert_in"), ip, pp, gp, kp, dlp, wgp,
+        _dev(dexpert_in, "dexpert_in"), ip, pp, gp, kp, dlp, wgp, gpr,
         dx.data_ptr(), g, s, e, c, m, dtype_code(dt), _stream()),
         "dispatch_backward")
   return dx

@@ -12,9 +12,9 @@ Built: moe_gating "top_2" (every second-place policy, the second-place loss),
 "switch", "switch_max" and "expert_selection" for the policies that draw no
 random numbers; nonpadding / importance; moe_use_experts_attention; float32 and
 bfloat16; mtf.gradients over the v1 layer (top_2 / switch / switch_max, ReLU or
-linear experts).  Not built (they raise NotImplementedError): moe_gating
-"ntlb", expert dropout while training, gated (list) activations, gradients of
-the v2 layer, and a mesh with more than one device.
+linear experts) and the v2 layer.  Not built (they raise NotImplementedError): moe_gating
+"ntlb", expert dropout while training, gated (list) activations, and a mesh
+with more than one device.
 """
 
 import torch
@@ -567,9 +567,25 @@ class MoEV2Operation(mtf.Operation):
     self._has_importance = importance is not None
     self._dims = dims
     self._gating = gating
+    self._save_for_backward = False
     out_shape = mtf.Shape(inputs.shape.dims[:-1] + [output_dim])
     self._outputs = [mtf.Tensor(self, out_shape, inputs.dtype, index=0),
                      mtf.Tensor(self, mtf.Shape([]), inputs.dtype, index=1)]
+
+  def gradient(self, grad_ys):
+    """Gradients w.r.t. (inputs, outer / inner gate kernels, wi, wo
+    [, importance]) from those of (outputs, loss)."""
+    if self._gating.use_second_place_loss:
+      raise NotImplementedError(
+          "backward of the second-place loss is not implemented")
+    self._save_for_backward = True
+    d_out, d_loss = grad_ys
+    if d_out is None:
+      d_out = mtf.zeros(self.mesh, self.outputs[0].shape, self.outputs[0].dtype)
+    if d_loss is None:
+      d_loss = mtf.zeros(self.mesh, mtf.Shape([]), self.outputs[1].dtype)
+    grads = MoEV2GradOperation(self, d_out, d_loss).outputs
+    return grads + [None] * (len(self.inputs) - 5)
 
   def lower(self, lowering):
     mesh_impl = lowering.mesh_impl(self)
@@ -584,6 +600,9 @@ class MoEV2Operation(mtf.Operation):
     x_e, y_e, c_, h0, t_, d_ = self._dims
     ag = a0 * g1
 
+    save = self._save_for_backward
+    saved = {}
+
     def fn(x_s, wo_s, wi_s, imp_s=None):
       xg = x_s.reshape(ag, s_, m_)
       # outer level
@@ -591,20 +610,35 @@ class MoEV2Operation(mtf.Operation):
         imp_s = imp_s.reshape(ag, s_)
       rx = self._gating.route(xg.reshape(1, ag * s_, m_),
                               wo_s.reshape(1, m_, x_e), w_outer_p, s_, x_e, c_,
-                              imp_s)
+                              imp_s, want_logits=save)
+      logits_x = None
+      if save:
+        rx, logits_x = rx
       ein_x, slot_gate = moe_hip.dispatch(xg, rx, want_slot_gate=True)
       # inner level: each outer expert's a0*g*c slots become h0 groups of t
       inputs_y = ein_x.reshape(x_e, h0 * t_, m_)
       ry = self._gating.route(inputs_y, wi_s, w_inner_p, t_, y_e, d_,
                               slot_gate.reshape(x_e * h0, t_),
-                              importance_from_slot_gate=True)
+                              importance_from_slot_gate=True, want_logits=save)
+      logits_y = None
+      if save:
+        ry, logits_y = ry
       ein_y = moe_hip.dispatch(inputs_y.reshape(x_e * h0, t_, m_), ry)
       # experts: weights are [y, x, ...]; rows of (y, x) are its h0*d slots
+      h = None
+      if save:
+        h = torch.empty((y_e * x_e, h0 * d_, wi_p.shape[1]), dtype=dt,
+                        device=xg.device)
       yy = moe_hip.expert_ffn(ein_y.reshape(y_e * x_e, h0 * d_, m_), wi_p,
-                              wo_p, "relu")
+                              wo_p, "relu", h=h)
       out_y = moe_hip.combine(yy.reshape(y_e, x_e * h0, d_, n_), ry, t_)
       out = moe_hip.combine(out_y.reshape(x_e, ag, c_, n_), rx, s_)
       loss = (rx.loss.to(dt) + ry.loss.to(dt)).reshape(())
+      if save:
+        saved.update(x=xg, rx=rx, ry=ry, logits_x=logits_x, logits_y=logits_y,
+                     importance=imp_s, slot_gate=slot_gate, inputs_y=inputs_y,
+                     ein_y=ein_y, h=h, yy=yy, out_y=out_y,
+                     w_outer_packed=w_outer_p, w_inner_packed=w_inner_p)
       return out.reshape(a0, g1, s_, n_), loss
 
     args = [lowering.tensors[x], lowering.tensors[w_outer],
@@ -614,6 +648,87 @@ class MoEV2Operation(mtf.Operation):
     out, loss = mesh_impl.slicewise(fn, *args)
     lowering.set_tensor_lowering(self.outputs[0], out)
     lowering.set_tensor_lowering(self.outputs[1], loss)
+    lowering.operations[self] = saved
+
+
+class MoEV2GradOperation(mtf.Operation):
+  """Backward of MoEV2Operation: the v1 call sequence twice, inner level first
+  (combine outer, combine inner, experts, inner gating / router / dispatch,
+  outer gating / router / dispatch).  The inner importance is a comparison of
+  slot weights (moe.py:725-727) and carries no gradient."""
+
+  def __init__(self, forward, d_out, d_loss, name="moe_v2_grad"):
+    super(MoEV2GradOperation, self).__init__(
+        forward.inputs[:5] + [d_out, d_loss], name=name)
+    self._forward = forward
+    self._outputs = [mtf.Tensor(self, t.shape, t.dtype, index=i)
+                     for i, t in enumerate(forward.inputs[:5])]
+
+  @property
+  def has_gradient(self):
+    return False
+
+  def lower(self, lowering):
+    mesh_impl = lowering.mesh_impl(self)
+    fwd = self._forward
+    x = fwd.inputs[0]
+    a0, g1, s_, m_ = x.shape.to_integer_list
+    n_ = fwd.outputs[0].shape.dims[-1].size
+    x_e, y_e, c_, h0, t_, d_ = fwd._dims
+    ag = a0 * g1
+    gating = fwd._gating
+
+    def fn(wi_s, wo_s, dout_s, dloss_s):
+      sv = lowering.operations[fwd]
+      if not sv:
+        raise ValueError("the forward operation kept no activations: build "
+                         "the gradient before lowering the graph")
+      rx, ry = sv["rx"], sv["ry"]
+      dl = dloss_s.reshape(1).float()
+      hdim = wi_s.shape[-1]
+      d_eo_x, dgate_x = moe_hip.combine_backward(
+          dout_s.reshape(ag, s_, n_).contiguous(),
+          sv["out_y"].reshape(x_e, ag, c_, n_), rx)
+      dyy, dgate_y = moe_hip.combine_backward(
+          d_eo_x.reshape(x_e * h0, t_, n_),
+          sv["yy"].reshape(y_e, x_e * h0, d_, n_), ry)
+      dein_y, dwi, dwo = moe_hip.expert_ffn_backward(
+          sv["ein_y"].reshape(y_e * x_e, h0 * d_, m_), sv["h"],
+          dyy.reshape(y_e * x_e, h0 * d_, n_),
+          wi_s.reshape(y_e * x_e, m_, hdim), wo_s.reshape(y_e * x_e, hdim, n_),
+          "relu")
+      dlogits_y = moe_hip.gating_backward(
+          sv["logits_y"], ry, dgate_y, dl, 1.0, router="top_2",
+          importance=sv["slot_gate"].reshape(x_e * h0, t_),
+          num_microbatches=gating.num_microbatches,
+          importance_from_slot_gate=True)
+      inputs_y = sv["inputs_y"]                           # [x, h0*t, m]
+      dl_y = dlogits_y.reshape(x_e, h0 * t_, y_e)
+      dw_inner = torch.stack([
+          moe_hip.router_backward_weights(inputs_y[i], dl_y[i])
+          for i in range(x_e)])                           # [x, m, y]
+      d_inputs_y = moe_hip.dispatch_backward(
+          dein_y.reshape(y_e, x_e * h0, d_, m_), ry, t_, dlogits_y,
+          sv["w_inner_packed"])
+      dlogits_x = moe_hip.gating_backward(
+          sv["logits_x"], rx, dgate_x, dl, 1.0, router="top_2",
+          importance=sv["importance"],
+          num_microbatches=gating.num_microbatches)
+      dw_outer = moe_hip.router_backward_weights(
+          sv["x"].reshape(ag * s_, m_), dlogits_x.reshape(ag * s_, x_e))
+      dx = moe_hip.dispatch_backward(
+          d_inputs_y.reshape(x_e, ag, c_, m_), rx, s_, dlogits_x,
+          sv["w_outer_packed"])
+      return (dx.reshape(a0, g1, s_, m_), dw_outer, dw_inner,
+              dwi.reshape(wi_s.shape), dwo.reshape(wo_s.shape))
+
+    ins = self.inputs
+    outs = mesh_impl.slicewise(fn, lowering.tensors[ins[3]],
+                               lowering.tensors[ins[4]],
+                               lowering.tensors[ins[5]],
+                               lowering.tensors[ins[6]])
+    for t, v in zip(self.outputs, outs):
+      lowering.set_tensor_lowering(t, v)
 
 
 def transformer_moe_layer_v2(

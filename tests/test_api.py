@@ -339,9 +339,11 @@ def test_gradients_builds_the_backward_operation():
         x2, d2[-1], hparams(moe_use_second_place_loss=True), True,
         mtf.VariableDType(torch.float32))
     mtf.gradients([y2], [x2])
-  with pytest.raises(NotImplementedError, match="Gradient not implemented"):
-    g3, _, x3, d3 = graph_input()
-    y3, _ = moe.transformer_moe_layer_v2(
-        x3, d3[-1], hparams(moe_num_experts=[2, 2]), True,
-        mtf.VariableDType(torch.float32))
-    mtf.gradients([y3], [x3])
+  g3, _, x3, d3 = graph_input()
+  y3, l3 = moe.transformer_moe_layer_v2(
+      x3, d3[-1], hparams(moe_num_experts=[2, 2]), True,
+      mtf.VariableDType(torch.float32))
+  v3 = [v.outputs[0] for v in g3.trainable_variables]
+  grads3 = mtf.gradients([y3, l3], [x3] + v3)
+  assert [g.shape for g in grads3] == [t.shape for t in [x3] + v3]
+  assert any(isinstance(o, moe.MoEV2GradOperation) for o in g3.operations)

@@ -517,3 +517,59 @@ def test_v1_experts_attention(act_dtype):
   np.testing.assert_array_equal(k, plain_k)
   with pytest.raises(NotImplementedError, match="experts_attention"):
     mtf.gradients([outs[0]], [xt])
+
+
+@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
+def test_v2_gradients_match_oracle(act_dtype):
+  """mtf.gradients over the hierarchical layer against the oracle's backward
+  (pinned by central differences in tests/test_oracle.py)."""
+  b, l, m, hdim, xe, ye, group = 2, 64, 32, 48, 2, 4, 32
+  hp, ohp = make_hparams(moe_num_experts=[xe, ye], moe_hidden_size=hdim,
+                         moe_group_size=group, moe_capacity_factor_train=1.25,
+                         moe_capacity_factor_second_level=1.0,
+                         moe_loss_coef=0.25)
+  for seed in range(601, 621):   # first seed without an inner-level near-tie
+    rng = np.random.default_rng(seed)
+    w = v2_weights(rng, m, hdim, xe, ye)
+    x = H.safe_tokens(rng, b * l, m, w["w_outer"], act_dtype).reshape(b, l, m)
+    nonpad = (rng.random((b, l)) < 0.9).astype(np.float32)
+    _, _, aux = O.moe_layer_v2(x, w["w_outer"], w["w_inner"], w["wi"], w["wo"],
+                               ohp, True, act_dtype, nonpadding=nonpad,
+                               dense=False)
+    if inner_gap_ok(aux):
+      break
+  assert inner_gap_ok(aux)
+  d_out = O.cast_act(rng.standard_normal((b, l, m)).astype(np.float32), act_dtype)
+  dt = H.ACT_TORCH[act_dtype]
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  dims = [mtf.Dimension("batch", b), mtf.Dimension("length", l),
+          mtf.Dimension("d_model", m)]
+  xt = mtf.import_tf_tensor(mesh, torch.from_numpy(x).to(dt), mtf.Shape(dims))
+  npad = mtf.import_tf_tensor(mesh, torch.from_numpy(nonpad).to(dt),
+                              mtf.Shape(dims[:2]))
+  with mtf.variable_scope("moe2d"):
+    y, loss = moe.transformer_moe_layer_v2(
+        xt, dims[-1], hp, True, mtf.VariableDType(torch.float32, torch.float32, dt),
+        nonpadding=npad, num_microbatches=2)
+  variables = graph.trainable_variables
+  assert [v.name.split("/")[-2] for v in variables] == [
+      "outer_gating", "inner_gating", "wi", "wo"]
+  dyt = mtf.import_tf_tensor(mesh, torch.from_numpy(d_out).to(dt), mtf.Shape(dims))
+  dlt = mtf.import_tf_tensor(mesh, torch.tensor(1.5, dtype=dt), mtf.Shape([]))
+  grads = mtf.gradients([y, loss], [xt] + [v.outputs[0] for v in variables],
+                        grad_ys=[dyt, dlt])
+  init = {"moe2d/outer_gating/kernel": w["w_outer"],
+          "moe2d/inner_gating/kernel": w["w_inner"],
+          "moe2d/wi/kernel": w["wi"], "moe2d/wo/kernel": w["wo"]}
+  lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()}, initial_values=init)
+  got = [H.to_np(lowering.export_to_tf_tensor(g)) for g in grads]
+  want = O.moe_layer_v2_backward(x, w["w_outer"], w["w_inner"], w["wi"], w["wo"],
+                                 ohp, True, act_dtype, d_out, 1.5,
+                                 nonpadding=nonpad, num_microbatches=2)
+  tol = H.value_tolerance(act_dtype)
+  for g_, k in zip(got, ("dx", "dw_outer", "dw_inner", "dwi", "dwo")):
+    ref = want[k].reshape(g_.shape)
+    np.testing.assert_allclose(
+        g_, ref, rtol=tol["rtol"], atol=tol["atol"] * max(1.0, np.abs(ref).max()),
+        err_msg=k)
