@@ -188,7 +188,11 @@ def test_dispatch_combine(hip, act_dtype, shape):
     ("float32", "linear")])
 @pytest.mark.parametrize("shape", [(3, 320, 64, 128, 64), (2, 100, 72, 200, 40),
                                    (2, 1100, 128, 1152, 1024),
-                                   (1, 40, 30, 50, 20)])
+                                   (1, 40, 30, 50, 20),
+                                   # 256-row tiles with 1, 2, 3 and 5 K tiles,
+                                   # ragged rows and a ragged last column tile
+                                   (2, 512, 64, 256, 256), (1, 256, 128, 320, 256),
+                                   (2, 700, 192, 256, 512)])
 def test_expert_ffn(hip, act_dtype, activation, shape):
   e, rows, m, hdim, n = shape
   rng = np.random.default_rng(29)
