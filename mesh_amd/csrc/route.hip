@@ -556,9 +556,9 @@ __global__ __launch_bounds__(CAP_THREADS) void gate_capacity_kernel(
   const int s_begin = min(S, chunk * clen);
   const int s_end = min(S, s_begin + clen);
 
-  int count1 = 0;  // kept first choices of expert e (valid after round 0)
-  for (int round = 0; round < 2; ++round) {
-    const int16_t* ch = round == 0 ? c1 : c2;
+  int count1 = 0;  // kept first choices of expert e (valid after choice 0)
+  for (int choice = 0; choice < 2; ++choice) {
+    const int16_t* ch = choice == 0 ? c1 : c2;
     int c = 0;
     for (int s = s_begin; s < s_end; ++s) c += (ch[s] == e);
     cnt[chunk * el + e] = c;
@@ -569,20 +569,20 @@ __global__ __launch_bounds__(CAP_THREADS) void gate_capacity_kernel(
       total += v;
       if (k < chunk) before += v;
     }
-    int running = before + (round == 0 ? 0 : count1);
-    const bool in_token_order = !(p.rank_by_gate && round == 0);
+    int running = before + (choice == 0 ? 0 : count1);
+    const bool in_token_order = !(p.rank_by_gate && choice == 0);
     for (int s = s_begin; in_token_order && s < s_end; ++s) {
       if (ch[s] == e) {
         int64_t t = base + s;
         const bool ok = running < C;
-        pos[t * 2 + round] = running;
-        kept[t * 2 + round] = ok ? 1 : 0;
-        if (!ok) gate[t * 2 + round] = gate[t * 2 + round] * 0.0f;
+        pos[t * 2 + choice] = running;
+        kept[t * 2 + choice] = ok ? 1 : 0;
+        if (!ok) gate[t * 2 + choice] = gate[t * 2 + choice] * 0.0f;
         ++running;
       }
     }
-    if (chunk == 0 && e < E) tot[round * el + e] = total;
-    if (round == 0) count1 = min(total, C);
+    if (chunk == 0 && e < E) tot[choice * el + e] = total;
+    if (choice == 0) count1 = min(total, C);
     __syncthreads();
   }
   if (p.rank_by_gate) {
