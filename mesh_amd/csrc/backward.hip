@@ -36,10 +36,10 @@ __device__ __forceinline__ uint4 pack16(const float (&f)[4], float) {
 }
 __device__ __forceinline__ uint4 pack16(const float (&f)[8], bf16_t) {
   uint4 r;
-  r.x = (uint32_t)f32_to_bf16(f[0]) | ((uint32_t)f32_to_bf16(f[1]) << 16);
-  r.y = (uint32_t)f32_to_bf16(f[2]) | ((uint32_t)f32_to_bf16(f[3]) << 16);
-  r.z = (uint32_t)f32_to_bf16(f[4]) | ((uint32_t)f32_to_bf16(f[5]) << 16);
-  r.w = (uint32_t)f32_to_bf16(f[6]) | ((uint32_t)f32_to_bf16(f[7]) << 16);
+  r.x = f32x2_to_bf16x2(f[0], f[1]);
+  r.y = f32x2_to_bf16x2(f[2], f[3]);
+  r.z = f32x2_to_bf16x2(f[4], f[5]);
+  r.w = f32x2_to_bf16x2(f[6], f[7]);
   return r;
 }
 

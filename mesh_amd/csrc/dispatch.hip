@@ -115,7 +115,7 @@ __device__ __forceinline__ void fma2_bf16(uint32_t a, uint32_t b, float w1,
   float b0 = __uint_as_float(b << 16), b1 = __uint_as_float(b & 0xffff0000u);
   float r0 = w1 * a0 + w2 * b0;
   float r1 = w1 * a1 + w2 * b1;
-  out = (uint32_t)f32_to_bf16(r0) | ((uint32_t)f32_to_bf16(r1) << 16);
+  out = f32x2_to_bf16x2(r0, r1);
 }
 
 template <typename T>

@@ -15,6 +15,7 @@ namespace mesh_moe {
 
 typedef __attribute__((ext_vector_type(8))) __bf16 bf16x8_t;
 typedef __attribute__((ext_vector_type(16))) float f32x16_t;
+typedef __attribute__((ext_vector_type(4))) uint32_t u32x4_t;
 
 // ---------------------------------------------------------------------------
 // bf16 MFMA kernel.
@@ -47,13 +48,14 @@ struct GemmCfg {
       LOOP_BYTES > EPI_BYTES ? LOOP_BYTES : EPI_BYTES;
 };
 
+// relu commutes with the rounding (which keeps the sign; -0 and +0 both end as
+// +0), so it is applied to the float32 accumulators
 __device__ __forceinline__ uint32_t pack2_bf16(float a, float b, bool relu) {
-  uint32_t lo = f32_to_bf16(a), hi = f32_to_bf16(b);
-  if (relu) {  // relu of the rounded value: clear negatives (sign bit set)
-    if (lo & 0x8000u) lo = 0;
-    if (hi & 0x8000u) hi = 0;
+  if (relu) {
+    a = fmaxf(a, 0.f);
+    b = fmaxf(b, 0.f);
   }
-  return lo | (hi << 16);
+  return f32x2_to_bf16x2(a, b);
 }
 
 template <int BM, int BN, int BK, bool RELU>
@@ -485,80 +487,106 @@ struct RingCfg {
   static constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES;
   static constexpr int A_SLOTS = 2, B_SLOTS = 3;
   static constexpr int B_BASE = A_SLOTS * A_BYTES;
-  static constexpr int LDC = BN + 4;
   static constexpr size_t LOOP_BYTES = (size_t)A_SLOTS * A_BYTES + (size_t)B_SLOTS * B_BYTES;
-  static constexpr size_t EPI_BYTES = (size_t)BM * LDC * sizeof(bf16_t);
-  static constexpr size_t LDS_BYTES = LOOP_BYTES > EPI_BYTES ? LOOP_BYTES : EPI_BYTES;
+  static constexpr size_t LDS_BYTES = LOOP_BYTES;  // the epilogue stages inside
   static_assert(A_INSTR == 4 && B_INSTR == 4, "load schedule assumes 4 + 4");
 };
 
-template <bool RELU, bool DEEP_B>
+template <bool RELU>
 __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
-    bf16_t* __restrict__ Cout, int R, int N, int K, int tiles_m, int tiles_n) {
+    bf16_t* __restrict__ Cout, int R, int N, int K, int tiles_m, int tiles_n,
+    int total_tiles) {
   using Cfg = RingCfg;
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, WN = Cfg::WN;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
 
+  // PERSISTENT blocks: one per CU, each walks a strided list of tiles, so that
+  // block start-up and the first loads of a tile overlap the previous tile's
+  // epilogue.  Block b runs on XCD b % 8; an XCD owns a contiguous range of
+  // logical tiles and its blocks take them round-robin, which keeps the tiles
+  // resident on an XCD at any moment consecutive (shared panels in its L2).
   const int nblk = gridDim.x;
-  const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
-  const int per_xcd = nblk >> 3, extra = nblk & 7;
-  const int logical = xcd * per_xcd + min(xcd, extra) + local;
-  const int tiles_per_e = tiles_m * tiles_n;
-  const int e = logical / tiles_per_e;
-  const int rem = logical - e * tiles_per_e;
-  const int tn = rem / tiles_m;
-  const int tm = rem - tn * tiles_m;
-  const int row0 = tm * BM, col0 = tn * BN;
-  const bf16_t* Ae = A + (int64_t)e * R * K;
-  const bf16_t* Be = B + (int64_t)e * N * K;
-  bf16_t* Ce = Cout + (int64_t)e * R * N;
+  int tile, tile_end, tile_step;
+  if ((nblk & 7) == 0) {
+    const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
+    const int per_xcd = total_tiles >> 3, extra = total_tiles & 7;
+    const int begin = xcd * per_xcd + min(xcd, extra);
+    tile_end = begin + per_xcd + (xcd < extra ? 1 : 0);
+    tile = begin + local;
+    tile_step = nblk >> 3;
+  } else {
+    tile = blockIdx.x;
+    tile_end = total_tiles;
+    tile_step = nblk;
+  }
+  if (tile >= tile_end) return;
 
   const int tid = threadIdx.x;
   const int lane = tid & 63;
   const int wave = tid >> 6;
   const int wm = wave / WN, wn = wave % WN;
-
-  int a_off[Cfg::A_INSTR], b_off[Cfg::B_INSTR];
-#pragma unroll
-  for (int j = 0; j < Cfg::A_INSTR; ++j) {
-    const int row = (wave + Cfg::WAVES * j) * 8 + (lane >> 3);
-    const int chunk = (lane & 7) ^ lds_swizzle(row);
-    a_off[j] = min(row0 + row, R - 1) * K + chunk * 8;
-    b_off[j] = min(col0 + row, N - 1) * K + chunk * 8;
-  }
+  const int tiles_per_e = tiles_m * tiles_n;
   const int nk = K / BK;
-  // load j of the token (A) / weight (B) tile kt; kt past the end re-fetches
-  // the last tile into a slot nobody reads any more
-  // The operand with two slots ("near", fetched one tile ahead) sits at LDS
-  // offset 0, the one with three slots ("far", two tiles ahead) behind it.
-  // DEEP_B: the weight tile is the far operand, else the token tile.
-  constexpr int FAR_BASE = 2 * Cfg::A_BYTES;
-  const bf16_t* near_g = DEEP_B ? Ae : Be;
-  const bf16_t* far_g = DEEP_B ? Be : Ae;
-  auto load_near = [&](int kt, int j) {
+
+  // per-tile state
+  int row0, col0;
+  const bf16_t *Ae, *Be;
+  bf16_t* Ce;
+  int a_off[Cfg::A_INSTR], b_off[Cfg::B_INSTR];
+  auto set_tile = [&](int logical) {
+    const int e = logical / tiles_per_e;
+    const int rem = logical - e * tiles_per_e;
+    const int tn = rem / tiles_m;
+    const int tm = rem - tn * tiles_m;
+    row0 = tm * BM;
+    col0 = tn * BN;
+    Ae = A + (int64_t)e * R * K;
+    Be = B + (int64_t)e * N * K;
+    Ce = Cout + (int64_t)e * R * N;
+#pragma unroll
+    for (int j = 0; j < Cfg::A_INSTR; ++j) {
+      const int row = (wave + Cfg::WAVES * j) * 8 + (lane >> 3);
+      const int chunk = (lane & 7) ^ lds_swizzle(row);
+      a_off[j] = min(row0 + row, R - 1) * K + chunk * 8;
+      b_off[j] = min(col0 + row, N - 1) * K + chunk * 8;
+    }
+  };
+  // load j of the token (A, two slots at LDS offset 0) / weight (B, three
+  // slots behind them) tile kt; kt past the end re-fetches the last tile into
+  // a slot nobody reads any more
+  constexpr int B_BASE = Cfg::B_BASE;
+  auto load_a = [&](int kt, int j) {
     const int slot = kt & 1;
     kt = min(kt, nk - 1);
     __builtin_amdgcn_global_load_lds(
-        (glb_void_t*)(near_g + kt * BK + (DEEP_B ? a_off[j] : b_off[j])),
+        (glb_void_t*)(Ae + kt * BK + a_off[j]),
         (lds_void_t*)(smem_raw + slot * Cfg::A_BYTES +
                       (wave + Cfg::WAVES * j) * 1024), 16, 0, 0);
   };
-  auto load_far = [&](int kt, int slot, int j) {
+  auto load_b = [&](int kt, int slot, int j) {
     kt = min(kt, nk - 1);
     __builtin_amdgcn_global_load_lds(
-        (glb_void_t*)(far_g + kt * BK + (DEEP_B ? b_off[j] : a_off[j])),
-        (lds_void_t*)(smem_raw + FAR_BASE + slot * Cfg::B_BYTES +
+        (glb_void_t*)(Be + kt * BK + b_off[j]),
+        (lds_void_t*)(smem_raw + B_BASE + slot * Cfg::B_BYTES +
                       (wave + Cfg::WAVES * j) * 1024), 16, 0, 0);
+  };
+  // the first loads of a tile except weight tile 1, whose slot the epilogue of
+  // the previous tile still uses as staging area
+  auto prologue_head = [&]() {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) load_a(0, j);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) load_b(0, 0, j);
+    load_a(1, 0);
+    load_a(1, 1);
+  };
+  auto prologue_tail = [&]() {
+#pragma unroll
+    for (int j = 0; j < 4; ++j) load_b(1, 1, j);
   };
 
   f32x16_t acc[Cfg::TM][Cfg::TN];
-#pragma unroll
-  for (int i = 0; i < Cfg::TM; ++i)
-#pragma unroll
-    for (int j = 0; j < Cfg::TN; ++j)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
   const int fr = lane & 31, fc = lane >> 5;
   int a_frag[BK / 16], b_frag[BK / 16];
@@ -571,15 +599,14 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
   constexpr int KSTEPS = BK / 16;
   bf16x8_t fa[2][Cfg::TM], fb[2][Cfg::TN];
   // fragment read n of a step: 0..TM-1 token rows, TM..TM+TN-1 weight rows
-  auto read_frag = [&](int nslot, int fslot, int kk, int buf, int n) {
-    const int a_base = DEEP_B ? nslot * Cfg::A_BYTES : FAR_BASE + fslot * Cfg::A_BYTES;
-    const int b_base = DEEP_B ? FAR_BASE + fslot * Cfg::B_BYTES : nslot * Cfg::B_BYTES;
+  auto read_frag = [&](int aslot, int bslot, int kk, int buf, int n) {
     if (n < Cfg::TM)
       fa[buf][n] = *reinterpret_cast<const bf16x8_t*>(
-          smem_raw + a_base + a_frag[kk] + n * 32 * Cfg::ROW_BYTES);
+          smem_raw + aslot * Cfg::A_BYTES + a_frag[kk] + n * 32 * Cfg::ROW_BYTES);
     else
       fb[buf][n - Cfg::TM] = *reinterpret_cast<const bf16x8_t*>(
-          smem_raw + b_base + b_frag[kk] + (n - Cfg::TM) * 32 * Cfg::ROW_BYTES);
+          smem_raw + B_BASE + bslot * Cfg::B_BYTES + b_frag[kk] +
+          (n - Cfg::TM) * 32 * Cfg::ROW_BYTES);
   };
   auto mfma = [&](int buf, int n) {
     const int i = n / Cfg::TN, j = n % Cfg::TN;
@@ -591,22 +618,6 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
   // fragment reads in the order the MFMAs (token tile i = n / TN outer, weight
   // tile j = n % TN inner) first need them: a0 b0 b1 a1 a2 a3
   constexpr int RD[6] = {0, Cfg::TM, Cfg::TM + 1, 1, 2, 3};
-
-  // prologue: tile 0 (8 loads), weight tile 1 (4), token loads 0,1 of tile 1
-#pragma unroll
-  for (int j = 0; j < 4; ++j) load_near(0, j);
-#pragma unroll
-  for (int j = 0; j < 4; ++j) load_far(0, 0, j);
-#pragma unroll
-  for (int j = 0; j < 4; ++j) load_far(1, 1, j);
-  load_near(1, 0);
-  load_near(1, 1);
-  wait_vmcnt<6>();
-  asm volatile("" ::: "memory");
-  __builtin_amdgcn_s_barrier();
-  asm volatile("" ::: "memory");
-#pragma unroll
-  for (int n = 0; n < 6; ++n) read_frag(0, 0, 0, 0, n);
 
   // bslot = kt % 3, kept incrementally
   int bslot = 0;
@@ -620,10 +631,10 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
       const int cur = kk & 1, nxt = cur ^ 1;
       auto load = [&](int which) {   // the two loads this step carries
         if (LAST) return;
-        if (kk == 0) load_near(kt + 1, 2 + which);
-        if (kk == 1) load_far(kt + 2, bnext2, which);
-        if (kk == 2) load_far(kt + 2, bnext2, 2 + which);
-        if (kk == 3) load_near(kt + 2, which);
+        if (kk == 0) load_a(kt + 1, 2 + which);
+        if (kk == 1) load_b(kt + 2, bnext2, which);
+        if (kk == 2) load_b(kt + 2, bnext2, 2 + which);
+        if (kk == 3) load_a(kt + 2, which);
       };
       if (kk + 1 < KSTEPS) {
         // 6 fragment reads of step kk+1 (in the order its MFMAs need them),
@@ -670,42 +681,97 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
     }
     bslot = bnext;
   };
-  for (int kt = 0; kt + 1 < nk; ++kt) k_tile(kt, std::false_type{});
-  k_tile(nk - 1, std::true_type{});
-  // the epilogue reuses the ring: no direct-to-LDS load may still be in flight
-  wait_vmcnt<0>();
-  __syncthreads();
 
-  bf16_t* Cs = reinterpret_cast<bf16_t*>(smem_raw);  // [BM][LDC]
+  // Epilogue staging: two passes of 128 output rows (64 from each half of the
+  // tile, so that all eight wavefronts write), exactly the last two weight
+  // slots, which are free once the K loop is over.  Rows are 512 bytes, a
+  // multiple of the bank count, so 16-byte chunk c of staging row r lives at
+  // chunk c ^ (r & 31): the writes of a wavefront (32 rows x 8 bytes, twice)
+  // and its reads (2 rows x 32 chunks) both spread over all banks.
+  constexpr int EPI_ROWS = 128;
+  constexpr int EPI_ROW_BYTES = BN * 2;
+  constexpr int EPI_BASE = B_BASE + Cfg::B_BYTES;
+  static_assert(EPI_BASE + EPI_ROWS * EPI_ROW_BYTES <= (int)Cfg::LOOP_BYTES,
+                "epilogue staging exceeds the ring");
+  static_assert(BN == 256 && Cfg::WM == 2 && Cfg::TM == 4, "epilogue layout");
+  unsigned char* Cs = smem_raw + EPI_BASE;
   const int m_l = lane & 31;
-  const int n_l = (lane >> 5) * 4;
+  const int half = lane >> 5;   // which 8 bytes of a 16-byte chunk
+  constexpr int CPR_C = BN / 8;  // 16-byte chunks per output row
+
+  set_tile(tile);
+  prologue_head();
+  prologue_tail();
+  for (;;) {
 #pragma unroll
-  for (int i = 0; i < Cfg::TM; ++i) {
+    for (int i = 0; i < Cfg::TM; ++i)
 #pragma unroll
-    for (int j = 0; j < Cfg::TN; ++j) {
+      for (int j = 0; j < Cfg::TN; ++j)
 #pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const int row = wm * Cfg::WTM + i * 32 + m_l;
-        const int col = wn * Cfg::WTN + j * 32 + 8 * q + n_l;
-        uint2 v;
-        v.x = pack2_bf16(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], RELU);
-        v.y = pack2_bf16(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3], RELU);
-        *reinterpret_cast<uint2*>(Cs + row * Cfg::LDC + col) = v;
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    // K tile 0 has landed: only weight tile 1 (4 loads) and token loads 0,1 of
+    // tile 1 may still be in flight
+    wait_vmcnt<6>();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int n = 0; n < 6; ++n) read_frag(0, 0, 0, 0, RD[n]);
+    bslot = 0;
+    for (int kt = 0; kt + 1 < nk; ++kt) k_tile(kt, std::false_type{});
+    k_tile(nk - 1, std::true_type{});
+
+    // Every wavefront is done with the ring and no direct-to-LDS load is in
+    // flight (the last hand-over re-fetched a tile nobody reads).
+    wait_vmcnt<0>();
+    __syncthreads();
+    const int out_row0 = row0, out_col0 = col0;
+    bf16_t* out_c = Ce;
+    const int next = tile + tile_step;
+    const bool has_next = next < tile_end;
+    if (has_next) {
+      // the next tile's first loads fly while this tile is written out
+      set_tile(next);
+      prologue_head();
+    }
+    // round (and relu), stage in LDS, coalesced 16-byte stores
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+#pragma unroll
+      for (int ii = 0; ii < 2; ++ii) {
+        const int i = pass * 2 + ii;
+        const int srow = wm * 64 + ii * 32 + m_l;
+#pragma unroll
+        for (int j = 0; j < Cfg::TN; ++j) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int chunk = (wn * Cfg::WTN + j * 32 + 8 * q) / 8;
+            uint2 v;
+            v.x = pack2_bf16(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], RELU);
+            v.y = pack2_bf16(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3], RELU);
+            *reinterpret_cast<uint2*>(Cs + srow * EPI_ROW_BYTES +
+                                      ((chunk ^ m_l) * 16) + half * 8) = v;
+          }
+        }
       }
+      __syncthreads();
+#pragma unroll
+      for (int c = tid; c < EPI_ROWS * CPR_C; c += Cfg::THREADS) {
+        const int srow = c / CPR_C, chunk = c % CPR_C;
+        // staging row -> tile row: 64 rows of each half of the tile
+        const int grow = out_row0 + (srow >> 6) * 128 + pass * 64 + (srow & 63);
+        const int gcol = out_col0 + chunk * 8;
+        if (grow < R && gcol < N) {
+          const u32x4_t v = *reinterpret_cast<const u32x4_t*>(
+              Cs + srow * EPI_ROW_BYTES + ((chunk ^ (srow & 31)) * 16));
+          *reinterpret_cast<u32x4_t*>(out_c + (int64_t)grow * N + gcol) = v;
+        }
+      }
+      __syncthreads();
     }
-  }
-  __syncthreads();
-  constexpr int CPR_C = BN / 8;
-#pragma unroll 4
-  for (int c = tid; c < BM * CPR_C; c += Cfg::THREADS) {
-    const int r = c / CPR_C, cc = (c % CPR_C) * 8;
-    const int grow = row0 + r, gcol = col0 + cc;
-    if (grow < R && gcol < N) {
-      const uint2* sp = reinterpret_cast<const uint2*>(Cs + r * Cfg::LDC + cc);
-      uint2 lo = sp[0], hi = sp[1];
-      *reinterpret_cast<uint4*>(Ce + (int64_t)grow * N + gcol) =
-          make_uint4(lo.x, lo.y, hi.x, hi.y);
-    }
+    if (!has_next) break;
+    tile = next;
+    prologue_tail();   // the staging area is free again
   }
 }
 
@@ -849,19 +915,32 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
   using Cfg = RingCfg;
   const int tiles_m = (R + Cfg::BM - 1) / Cfg::BM;
   const int tiles_n = (N + Cfg::BN - 1) / Cfg::BN;
-  const int64_t blocks = (int64_t)tiles_m * tiles_n * E;
-  MOE_REQUIRE(blocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
-              "expert_ffn: too many tiles (%lld)", (long long)blocks);
+  const int64_t tiles = (int64_t)tiles_m * tiles_n * E;
+  MOE_REQUIRE(tiles <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
+              "expert_ffn: too many tiles (%lld)", (long long)tiles);
+  // one persistent block per CU (a block takes all of a CU's LDS)
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) !=
+            hipSuccess || n < 1) {
+      set_error("expert_ffn: cannot query the number of compute units");
+      return MESH_MOE_E_HIP;
+    }
+    cus = n;
+  }
+  const unsigned blocks = (unsigned)(tiles < cus ? tiles : cus);
   if (relu) {
-    auto k = grouped_gemm_bf16_ring_kernel<true, true>;
+    auto k = grouped_gemm_bf16_ring_kernel<true>;
     MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
-    k<<<(unsigned)blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(A, B, C, R, N, K,
-                                                              tiles_m, tiles_n);
+    k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(A, B, C, R, N, K, tiles_m,
+                                                    tiles_n, (int)tiles);
   } else {
-    auto k = grouped_gemm_bf16_ring_kernel<false, true>;
+    auto k = grouped_gemm_bf16_ring_kernel<false>;
     MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
-    k<<<(unsigned)blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(A, B, C, R, N, K,
-                                                              tiles_m, tiles_n);
+    k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(A, B, C, R, N, K, tiles_m,
+                                                    tiles_n, (int)tiles);
   }
   MOE_CHECK_LAUNCH("expert_ffn (mfma, spread direct-to-LDS loads)");
   return 0;
