@@ -578,12 +578,12 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
     for (int j = 0; j < 4; ++j) load_a(0, j);
 #pragma unroll
     for (int j = 0; j < 4; ++j) load_b(0, 0, j);
-    load_a(1, 0);
-    load_a(1, 1);
   };
   auto prologue_tail = [&]() {
 #pragma unroll
     for (int j = 0; j < 4; ++j) load_b(1, 1, j);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) load_a(1, j);
   };
 
   f32x16_t acc[Cfg::TM][Cfg::TN];
@@ -629,11 +629,14 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
 #pragma unroll
     for (int kk = 0; kk < KSTEPS; ++kk) {
       const int cur = kk & 1, nxt = cur ^ 1;
-      auto load = [&](int which) {   // the two loads this step carries
+      // The loads a step carries: the four weight loads of tile kt+2 over
+      // steps 0..2, all four token loads of tile kt+2 right behind the
+      // hand-over barrier that frees their slot (a full K tile ahead of use).
+      auto load = [&](int which) {
         if (LAST) return;
-        if (kk == 0) load_a(kt + 1, 2 + which);
-        if (kk == 1) load_b(kt + 2, bnext2, which);
-        if (kk == 2) load_b(kt + 2, bnext2, 2 + which);
+        if (kk == 0) load_b(kt + 2, bnext2, which);
+        if (kk == 1 && which == 0) load_b(kt + 2, bnext2, 2);
+        if (kk == 2 && which == 0) load_b(kt + 2, bnext2, 3);
         if (kk == 3) load_a(kt + 2, which);
       };
       if (kk + 1 < KSTEPS) {
@@ -665,15 +668,16 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
         fence();
-        load(0);
-        mfma(cur, 0); fence();
-        load(1);
-        mfma(cur, 1); fence();
+        // fragment reads first: a load right behind the barrier would queue
+        // up with the other wavefronts' and hold this one's MFMAs back
 #pragma unroll
         for (int n = 0; n < 6; ++n) {
           read_frag(aslot ^ 1, bnext, 0, nxt, RD[n]);
-          mfma(cur, 2 + n); fence();
+          if (n >= 2) load(n - 2);
+          mfma(cur, n); fence();
         }
+        mfma(cur, 6); fence();
+        mfma(cur, 7); fence();
       } else {
 #pragma unroll
         for (int n = 0; n < 8; ++n) mfma(cur, n);
@@ -709,9 +713,8 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
       for (int j = 0; j < Cfg::TN; ++j)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-    // K tile 0 has landed: only weight tile 1 (4 loads) and token loads 0,1 of
-    // tile 1 may still be in flight
-    wait_vmcnt<6>();
+    // K tile 0 has landed: only tile 1 (4 + 4 loads) may still be in flight
+    wait_vmcnt<8>();
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
