@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 6
+#define MESH_MOE_ABI_VERSION 7
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -249,6 +249,27 @@ int mesh_moe_combine(const void* y, const int32_t* idx, const int32_t* pos,
                      int S, int E, int C, int N, int dtype, void* stream);
 
 /*
+ * "No token left behind" gating (_ntlb_gating, transformer/moe.py:804-940)
+ * after the router projection: every token names its top_k experts
+ * (mtf.top_k, ops.py:4964-5015); round i offers the tokens no expert has
+ * taken yet, in token order, to their i-th expert, which takes them while its
+ * total stays within the capacity (moe.py:903-934).  A token is routed at
+ * most once, with the raw softmax probability of the expert that took it as
+ * the gate.  The record has the [G,S,2] layout of the other routers with the
+ * second choice never kept, so dispatch, the FFN and combine apply unchanged;
+ * idx[g,s,0] of a token nobody took is its first candidate.  The loss is
+ * E^2 * mean(density_1_proxy * density_1) over [G,k,E] (and over the group dim
+ * when `importance` is given, moe.py:845-860).  top_k <= 8.
+ */
+size_t mesh_moe_ntlb_workspace_bytes(int G, int S, int E, int top_k);
+int mesh_moe_ntlb_gating(const float* logits, const void* importance,
+                         int importance_dtype, int G, int S, int E, int C,
+                         int top_k, int num_microbatches, int32_t* idx,
+                         int32_t* pos, float* gate, uint8_t* kept,
+                         int32_t* fill, float* loss, void* workspace,
+                         size_t workspace_bytes, void* stream);
+
+/*
  * ---------------------------------------------------------------------------
  * Expert-selection ("expert choice") gating: every expert picks, per group,
  * the C tokens it likes best (_expert_selection_gating,
@@ -359,7 +380,8 @@ size_t mesh_moe_gating_backward_workspace_bytes(int G, int E);
 
 /*
  * Backward of the gating (transformer/moe.py:1391-1496 for router 0 = top-2,
- * :1207-1306 for router 1 = switch / switch_max): d(logits) from the
+ * :1207-1306 for router 1 = switch / switch_max, :831-934 for router 2 = ntlb
+ * with its top_k; top_k is ignored otherwise): d(logits) from the
  * gradients of the two combine weights and of the layer's returned loss.
  *   logits [G,S,E] float32 (the forward values), importance and
  *   importance_from_slot_gate as in the forward
@@ -376,8 +398,9 @@ int mesh_moe_gating_backward(const float* logits, const void* importance,
                              int importance_from_slot_gate, const int32_t* idx,
                              const uint8_t* kept, const float* dgate,
                              const float* d_loss, double loss_scale, int G,
-                             int S, int E, int router, int use_z_loss,
-                             double z_loss_coef, int num_microbatches,
+                             int S, int E, int router, int top_k,
+                             int use_z_loss, double z_loss_coef,
+                             int num_microbatches,
                              float* dlogits, void* workspace,
                              size_t workspace_bytes, void* stream);
 

@@ -218,7 +218,8 @@ __global__ __launch_bounds__(256) void dispatch_backward_kernel(
 // ---------------------------------------------------------------------------
 struct GateBackwardParams {
   int G, S, E;
-  int router;           // 0 = top-2, 1 = switch / switch_max
+  int router;           // 0 = top-2, 1 = switch / switch_max, 2 = ntlb
+  int top_k;            // ntlb: candidates per token
   int has_importance;
   int importance_from_slot_gate;  // importance = 0.5*((w>0.5)+(w>0))
   int num_microbatches;
@@ -227,11 +228,13 @@ struct GateBackwardParams {
   float loss_scale;     // moe_loss_coef as the activation dtype holds it
 };
 
+constexpr int GB_MAX_K = 8;
+
 template <typename IT>
 __global__ __launch_bounds__(256) void gate_count_kernel(
-    GateBackwardParams p, const int32_t* __restrict__ idx,
-    const IT* __restrict__ importance, int32_t* __restrict__ counts,
-    float* __restrict__ n_one) {
+    GateBackwardParams p, const float* __restrict__ logits,
+    const int32_t* __restrict__ idx, const IT* __restrict__ importance,
+    int32_t* __restrict__ counts, float* __restrict__ n_one) {
   extern __shared__ int32_t cnt[];  // [E] + 1
   const int g = blockIdx.x;
   for (int e = threadIdx.x; e <= p.E; e += blockDim.x) cnt[e] = 0;
@@ -245,6 +248,36 @@ __global__ __launch_bounds__(256) void gate_count_kernel(
       one = p.importance_from_slot_gate ? imp > 0.5f : imp == 1.0f;
     }
     if (one) atomicAdd(&cnt[p.E], 1);
+    if (p.router == 2) {
+      // ntlb: one density per round, every token's top_k candidates
+      // (moe.py:839-847); the probabilities and the repeated first-arg-max are
+      // those of the forward kernel, so the candidates are the same
+      const float* row = logits + t * p.E;
+      float m = row[0];
+      for (int e = 1; e < p.E; ++e) m = fmaxf(m, row[e]);
+      const float negm = -m;
+      float sum = 0.f;
+      for (int e = 0; e < p.E; ++e) sum += expf(row[e] + negm);
+      const float neglse = -(logf(sum) + m);
+      int ids[GB_MAX_K];
+#pragma unroll
+      for (int i = 0; i < GB_MAX_K; ++i) {
+        if (i < p.top_k) {
+          float best = -1.f;
+          int bi = 0;
+          for (int e = 0; e < p.E; ++e) {
+            bool taken = false;
+#pragma unroll
+            for (int j = 0; j < GB_MAX_K; ++j) taken |= (j < i && ids[j] == e);
+            const float v = taken ? -2.f : expf(row[e] + neglse);
+            if (v > best) { best = v; bi = e; }
+          }
+          ids[i] = bi;
+          atomicAdd(&cnt[bi], 1);
+        }
+      }
+      continue;
+    }
     // top-2: density_1 counts mask_1 after the importance mask
     // (moe.py:1402-1420); switch: every token's arg-max (moe.py:1224)
     if (one || p.router == 1) atomicAdd(&cnt[idx[t * 2]], 1);
@@ -305,14 +338,17 @@ __global__ __launch_bounds__(256) void gating_backward_kernel(
     coef = dl * mb * ee * (float)(1.0 / ((double)p.G * (double)E)) * inv_s *
            inv_s * m1;
   } else {
+    // switch: the gate is the arg-max probability; ntlb: the probability of
+    // the candidate that took the token, and the loss averages over the
+    // top_k rounds as well (moe.py:845-856)
     add1 = dgate[t * 2] * k1 * m1;
+    const double terms =
+        (double)p.G * (double)E * (p.router == 2 ? (double)p.top_k : 1.0);
     if (p.has_importance)
-      coef = dl * mb * ee *
-             (float)(1.0 / ((double)p.G * (double)E * (double)S)) * n_one[g] *
+      coef = dl * mb * ee * (float)(1.0 / (terms * (double)S)) * n_one[g] *
              inv_s * inv_s;
     else
-      coef = dl * mb * ee * (float)(1.0 / ((double)p.G * (double)E)) * inv_s *
-             inv_s;
+      coef = dl * mb * ee * (float)(1.0 / terms) * inv_s * inv_s;
   }
   const int32_t* cg = counts + (int64_t)g * E;
   // inner = sum_e p[e] * dp[e]
@@ -494,7 +530,7 @@ extern "C" int mesh_moe_gating_backward(
     const float* logits, const void* importance, int importance_dtype,
     int importance_from_slot_gate, const int32_t* idx, const uint8_t* kept,
     const float* dgate, const float* d_loss, double loss_scale, int G, int S,
-    int E, int router,
+    int E, int router, int top_k,
     int use_z_loss, double z_loss_coef, int num_microbatches, float* dlogits,
     void* workspace, size_t workspace_bytes, void* stream) {
   MOE_REQUIRE(logits && idx && kept && dgate && d_loss && dlogits && workspace,
@@ -502,8 +538,11 @@ extern "C" int mesh_moe_gating_backward(
   MOE_REQUIRE(G >= 1 && S >= 1 && E >= 2 && E <= 512 && G <= 65535,
               MESH_MOE_E_ARG, "gating_backward: bad sizes G=%d S=%d E=%d", G, S,
               E);
-  MOE_REQUIRE(router == 0 || router == 1, MESH_MOE_E_ARG,
+  MOE_REQUIRE(router >= 0 && router <= 2, MESH_MOE_E_ARG,
               "gating_backward: unknown router %d", router);
+  MOE_REQUIRE(router != 2 || (top_k >= 1 && top_k <= E && top_k <= GB_MAX_K),
+              MESH_MOE_E_ARG, "gating_backward: top_k=%d with %d experts "
+              "(at most %d)", top_k, E, GB_MAX_K);
   MOE_REQUIRE(!importance || valid_dtype(importance_dtype), MESH_MOE_E_ARG,
               "gating_backward: bad importance dtype %d", importance_dtype);
   MOE_REQUIRE(workspace_bytes >= mesh_moe_gating_backward_workspace_bytes(G, E),
@@ -511,6 +550,7 @@ extern "C" int mesh_moe_gating_backward(
   GateBackwardParams p;
   p.G = G; p.S = S; p.E = E;
   p.router = router;
+  p.top_k = top_k;
   p.has_importance = importance != nullptr;
   p.importance_from_slot_gate = importance_from_slot_gate ? 1 : 0;
   p.num_microbatches = num_microbatches;
@@ -526,14 +566,14 @@ extern "C" int mesh_moe_gating_backward(
   const unsigned blocks = (unsigned)((T_tokens + 255) / 256);
   if (importance && importance_dtype == MESH_MOE_BF16) {
     gate_count_kernel<bf16_t><<<G, 256, smem, st>>>(
-        p, idx, (const bf16_t*)importance, counts, n_one);
+        p, logits, idx, (const bf16_t*)importance, counts, n_one);
     MOE_CHECK_LAUNCH("gating_backward (count)");
     gating_backward_kernel<bf16_t><<<blocks, 256, 0, st>>>(
         p, logits, (const bf16_t*)importance, idx, kept, dgate, d_loss, counts,
         n_one, dlogits);
   } else {
     gate_count_kernel<float><<<G, 256, smem, st>>>(
-        p, idx, (const float*)importance, counts, n_one);
+        p, logits, idx, (const float*)importance, counts, n_one);
     MOE_CHECK_LAUNCH("gating_backward (count)");
     gating_backward_kernel<float><<<blocks, 256, 0, st>>>(
         p, logits, (const float*)importance, idx, kept, dgate, d_loss, counts,

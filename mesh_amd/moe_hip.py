@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -55,6 +55,12 @@ _SIGNATURES = {
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_double, ctypes.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
         ctypes.c_size_t, _vp]),
+    "mesh_moe_ntlb_workspace_bytes": (ctypes.c_size_t, [
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "mesh_moe_ntlb_gating": (ctypes.c_int, [
+        _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, _vp, _vp,
+        _vp, _vp, ctypes.c_size_t, _vp]),
     "mesh_moe_dispatch": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
@@ -87,7 +93,8 @@ _SIGNATURES = {
         _vp, _vp, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, _vp,
         ctypes.c_double,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
-        ctypes.c_double, ctypes.c_int, _vp, _vp, ctypes.c_size_t, _vp]),
+        ctypes.c_int, ctypes.c_double, ctypes.c_int, _vp, _vp, ctypes.c_size_t,
+        _vp]),
     "mesh_moe_router_backward_weights": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, _vp]),
@@ -406,6 +413,35 @@ def switch_gating(logits, capacity, importance=None, z_loss=None,
   return r
 
 
+def ntlb_gating(logits, capacity, top_k, importance=None,
+                num_microbatches=None):
+  """logits float32 [G, S, E] -> Routing for "no token left behind" gating
+  (_ntlb_gating, transformer/moe.py:804-940): top_k candidates per token, one
+  round per candidate rank, each token routed at most once."""
+  lib = load_library()
+  g, s, e = logits.shape
+  lp = _dev(logits, "logits", torch.float32)
+  ip, icode = None, F32
+  if importance is not None:
+    icode = dtype_code(importance.dtype)
+    ip = _dev(importance, "importance", None, (g, s))
+  idx, pos, gate, kept, fill, loss, _, _ = _routing_buffers(
+      lib, g, s, e, logits.device)
+  ws_bytes = lib.mesh_moe_ntlb_workspace_bytes(g, s, e, int(top_k))
+  ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8,
+                   device=logits.device)
+  with _stage("ntlb_gating"):
+    _check(lib.mesh_moe_ntlb_gating(
+        lp, ip, icode, g, s, e, int(capacity), int(top_k),
+        int(num_microbatches or 1), idx.data_ptr(), pos.data_ptr(),
+        gate.data_ptr(), kept.data_ptr(), fill.data_ptr(), loss.data_ptr(),
+        ws.data_ptr(), ws_bytes, _stream()), "ntlb_gating")
+  r = Routing(idx, pos, gate, kept, fill, loss, int(capacity), e)
+  if _timer is not None:
+    _timer.routing.append(r)
+  return r
+
+
 def router_switch_gating(x, w_packed, group_size, capacity, importance=None,
                          z_loss=None, num_microbatches=None, bias=None,
                          want_logits=False, slots_by_gate=False):
@@ -608,10 +644,11 @@ def expert_ffn_backward(expert_in, h, dy, wi, wo, activation="relu"):
 
 def gating_backward(logits, r, dgate, d_loss, loss_scale, router="top_2",
                     importance=None, z_loss=None, num_microbatches=None,
-                    importance_from_slot_gate=False):
+                    importance_from_slot_gate=False, top_k=0):
   """d(logits) [G, S, E] float32.  d_loss: float32 tensor of one element on the
   device (gradient w.r.t. the layer's returned loss); loss_scale:
-  moe_loss_coef."""
+  moe_loss_coef.  router: "top_2", "switch" (also switch_max) or "ntlb" (then
+  top_k = moe_ntlb_top_k)."""
   lib = load_library()
   g, s, e = logits.shape
   dev = logits.device
@@ -630,7 +667,9 @@ def gating_backward(logits, r, dgate, d_loss, loss_scale, router="top_2",
         _dev(r.kept, "kept", torch.uint8, (g, s, 2)),
         _dev(dgate, "dgate", torch.float32, (g, s, 2)),
         _dev(d_loss, "d_loss", torch.float32), float(loss_scale), g, s, e,
-        0 if router == "top_2" else 1, int(z_loss is not None),
+        {"top_2": 0, "switch": 1, "switch_max": 1, "ntlb": 2}[router],
+        int(top_k),
+        int(z_loss is not None),
         float(z_loss or 0.0), int(num_microbatches or 1), dlogits.data_ptr(),
         ws.data_ptr(), ws_bytes, _stream()), "gating_backward")
   return dlogits

@@ -30,6 +30,12 @@ MoE file, and its TensorFlow dependency cannot run here):
                                       lowering of mtf.top_k) vs the stable
                                       sort, per-expert brute force, equality
                                       with switch_gating when nothing overflows
+  ntlb_gating                         walk over (round, token) with one
+                                      counter per expert, a hand-worked case
+                                      (4 tokens, 3 experts, capacity 1),
+                                      k = 1 equals switch_gating, closed-form
+                                      loss (uniform router: 1.0 for any k),
+                                      dense tensors vs record
   expert_selection_gating             per-expert stable sort brute force,
                                       weights of a token sum to sum(p)/count,
                                       closed-form loss (uniform logits: 1.0),
@@ -455,6 +461,98 @@ def switch_max_gating(logits, capacity, importance=None,
 
 
 # ----------------------------------------------------------------------------
+# _ntlb_gating  (transformer/moe.py:804-940)
+# ----------------------------------------------------------------------------
+def ntlb_gating(logits, capacity, top_k, importance=None,
+                num_microbatches=None, act_dtype="float32", dense=False):
+  """Everything in _ntlb_gating ("no token left behind") after the router
+  projection, for the deterministic policies (as switch_gating).
+
+  Every token names its `top_k` best experts (mtf.top_k, moe.py:839-842).
+  Round i offers the still unrouted tokens to their i-th expert in token
+  order; an expert takes them while its running total, carried over from the
+  earlier rounds, stays within `capacity` (moe.py:905-934).  A token is routed
+  at most once; its gate is the raw softmax probability of the expert that
+  took it.  Same result dict as switch_gating, plus `round` [G,S] (which of
+  its choices took the token, -1 if none) and `topk_index` [G,S,k].
+  """
+  logits = np.asarray(logits, dtype=F32)
+  g_, s_, e_ = logits.shape
+  k_ = int(top_k)
+  if not 1 <= k_ <= e_:
+    raise ValueError("moe_ntlb_top_k=%d with %d experts" % (k_, e_))
+  raw_gates = softmax(logits)                                    # :831
+  expert_gate, expert_index = top_k_lowest_index_first(raw_gates, k_, -1)
+  expert_mask = one_hot(expert_index, e_)                        # [G,S,k,E]
+
+  # load balancing loss (:845-861): density_1 [G,k,E] before the importance
+  # mask; the proxy [G,E] times (importance == 1) [G,S] broadcasts, and the
+  # mean runs over every dim of the product
+  inv_s = F32(1.0 / s_)
+  density_1 = seq_sum(expert_mask, axis=1) * inv_s               # [G,k,E]
+  density_1_proxy = seq_sum(raw_gates, axis=-2) * inv_s          # [G,E]
+  if importance is not None:
+    importance = np.asarray(importance, dtype=F32)
+    is_one = (importance == F32(1.0)).astype(F32)                # [G,S]
+    expert_mask = expert_mask * is_one[..., None, None]          # :850
+    expert_gate = expert_gate * is_one[..., None]                # :851
+    proxy = density_1_proxy[:, :, None] * is_one[:, None, :]     # [G,E,S]
+    prod = proxy[:, None, :, :] * density_1[..., None]           # [G,k,E,S]
+    total = F32(prod.sum(dtype=np.float64))    # see switch_gating
+  else:
+    prod = density_1_proxy[:, None, :] * density_1               # [G,k,E]
+    total = seq_sum(prod.reshape(-1))
+  loss = total * F32(1.0 / prod.size)
+  loss = loss * F32(float(e_ * e_))                              # :854-856
+  if num_microbatches and num_microbatches > 1:                  # :857-860
+    loss = loss * F32(1.0 / num_microbatches)
+
+  cap_f = F32(float(capacity))
+  cum_tokens = np.zeros((g_, e_), F32)                           # :897-898
+  left = np.ones((g_, s_), F32)                                  # :899-900
+  index_1 = expert_index[..., 0].copy()
+  pos_1 = np.zeros((g_, s_), np.int32)
+  gate_1 = np.zeros((g_, s_), F32)
+  kept_1 = np.zeros((g_, s_), bool)
+  rnd = np.full((g_, s_), -1, np.int32)
+  combine = np.zeros((g_, s_, e_, capacity), F32) if dense else None
+  for i in range(k_):                                            # :903-934
+    mask_i = expert_mask[:, :, i, :] * left[..., None]           # [G,S,E]
+    cumulative = cum_tokens[:, None, :] + np.cumsum(mask_i, axis=1, dtype=F32)
+    within = (cumulative <= cap_f).astype(F32)                   # :913-914
+    out_i = mask_i * within
+    cum_tokens = cum_tokens + seq_sum(out_i, axis=1)
+    out_flat = seq_sum(out_i, axis=-1)                           # [G,S]
+    left = left + (-out_flat)
+    position = cumulative - F32(1.0)                             # [G,S,E]
+    took = out_flat > 0
+    idx_i = expert_index[:, :, i]
+    pos_i = np.take_along_axis(position, idx_i[..., None], -1)[..., 0]
+    index_1[took] = idx_i[took]
+    pos_1[took] = pos_i[took].astype(np.int32)
+    gate_1[took] = expert_gate[:, :, i][took]
+    kept_1 |= took
+    rnd[took] = i
+    if dense:
+      combine = combine + (                                      # :927-932
+          (expert_gate[:, :, i] * out_flat)[..., None, None]
+          * one_hot(idx_i, e_)[..., None]
+          * one_hot(position.astype(np.int32), capacity))
+  zeros_i = np.zeros((g_, s_), np.int32)
+  out = dict(
+      index_1=index_1, index_2=zeros_i, pos_1=pos_1, pos_2=zeros_i,
+      kept_1=kept_1, kept_2=np.zeros((g_, s_), bool),
+      gate_1=gate_1, gate_2=np.zeros((g_, s_), F32),
+      fill=cum_tokens.astype(np.int32), round=rnd, topk_index=expert_index,
+      loss=cast_act(loss, act_dtype)[()])                        # :937
+  if dense:
+    combine = cast_act(combine, act_dtype)                       # :936
+    out["combine"] = combine
+    out["dispatch"] = (combine != 0).astype(F32)                 # :938-939
+  return out
+
+
+# ----------------------------------------------------------------------------
 # _expert_selection_gating  (transformer/moe.py:1057-1173)
 # ----------------------------------------------------------------------------
 def expert_selection_gating(logits, capacity, importance,
@@ -657,7 +755,8 @@ def default_hparams(**overrides):
       moe_dropout_rate=0.0, moe_use_experts_attention=False,
       moe_switch_policy_train="input_jitter",
       moe_switch_policy_eval="input_jitter", moe_switch_dropout=0.1,
-      moe_switch_temperature=1.0, moe_switch_jitter=1e-2, moe_z_loss=None)
+      moe_switch_temperature=1.0, moe_switch_jitter=1e-2, moe_z_loss=None,
+      moe_ntlb_top_k=4)
   hp.update(overrides)
   return HParams(**hp)
 
@@ -727,7 +826,8 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
     q, loss, aux = moe_layer_v1(x, w_gate, wi, wo, hp1, train, act_dtype, **kw)
     k, _, _ = moe_layer_v1(x, w_gate, wi, k_wo, hp1, train, act_dtype, **kw)
     return [q, k], loss, aux
-  if hp.moe_gating not in ("top_2", "switch", "switch_max", "expert_selection"):
+  if hp.moe_gating not in ("top_2", "switch", "switch_max", "ntlb",
+                          "expert_selection"):
     raise ValueError("unknown hparams.moe_gating=%s" % hp.moe_gating)
   x = cast_act(x, act_dtype)
   lead = x.shape[:-1]
@@ -777,7 +877,7 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
                num_groups=g_, group_size=s_, capacity=c_)
     return (out.reshape(lead + (n_,)),
             _scale_loss(r["loss"], hp.moe_loss_coef, act_dtype), aux)
-  if hp.moe_gating in ("switch", "switch_max"):                  # :393-424
+  if hp.moe_gating in ("switch", "switch_max", "ntlb"):          # :393-424
     sw = hp.moe_switch_policy_train if train else hp.moe_switch_policy_eval
     if sw == "sample" or (train and sw in ("input_dropout", "input_jitter")):
       raise NotImplementedError("switch policy %r draws random numbers" % sw)
@@ -786,6 +886,9 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
     if hp.moe_gating == "switch":
       r = switch_gating(logits, c_, importance, train, hp.moe_z_loss,
                         num_microbatches, act_dtype, dense=dense)
+    elif hp.moe_gating == "ntlb":
+      r = ntlb_gating(logits, c_, hp.moe_ntlb_top_k, importance,
+                      num_microbatches, act_dtype, dense=dense)
     else:
       r = switch_max_gating(logits, c_, importance, num_microbatches,
                             act_dtype, dense=dense)
@@ -826,7 +929,8 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
 # ----------------------------------------------------------------------------
 def gating_backward(logits, r, gating, d_gate_1, d_gate_2, d_loss,
                     importance=None, num_microbatches=None, z_loss=None):
-  """d(logits) of _top_2_gating / _switch_gating / _switch_max_gating.
+  """d(logits) of _top_2_gating / _switch_gating / _switch_max_gating /
+  _ntlb_gating.
 
   The reference obtains it from the gradients of the ops the gating is built
   from: top_1 routes the gradient of a gate to the arg-max entry
@@ -871,17 +975,28 @@ def gating_backward(logits, r, gating, d_gate_1, d_gate_2, d_loss,
     coef = d_loss * mb * ee * F32(1.0 / (g_ * e_))
     dp += (coef * density * inv_s)[:, None, :] * m1[..., None]
     return (p * (dp - (p * dp).sum(-1, keepdims=True))).astype(F32)
-  if gating not in ("switch", "switch_max"):
+  if gating not in ("switch", "switch_max", "ntlb"):
     raise ValueError("unknown gating %r" % (gating,))
+  # index_1 is the expert that took the token: the arg-max (switch) or the
+  # candidate of the round that placed it (ntlb: mtf.top_k routes the gradient
+  # of each value to its entry, ops.py:4916-4920, :5009-5015)
   np.add.at(dp, rows + (i1,), np.asarray(d_gate_1, F32) * r["kept_1"] * m1)
   # loss = mean(mean_s(p)[g,e] * m1[g,s] * density_1[g,e]) * E^2 with density_1
-  # counting every token (moe.py:1224-1234)
-  density = seq_sum(one_hot(i1, e_), axis=-2) * inv_s
+  # counting every token (moe.py:1224-1234); ntlb has one density per round and
+  # the mean runs over the rounds too (moe.py:845-856)
+  if gating == "ntlb":
+    k_ = r["topk_index"].shape[-1]
+    density = seq_sum(one_hot(r["topk_index"], e_).sum(axis=2, dtype=F32),
+                      axis=-2) * inv_s
+    terms = g_ * e_ * k_
+  else:
+    density = seq_sum(one_hot(i1, e_), axis=-2) * inv_s
+    terms = g_ * e_
   if importance is None:
-    coef = d_loss * mb * ee * F32(1.0 / (g_ * e_))
+    coef = d_loss * mb * ee * F32(1.0 / terms)
     dproxy = coef * density
   else:
-    coef = d_loss * mb * ee * F32(1.0 / (g_ * e_ * s_))
+    coef = d_loss * mb * ee * F32(1.0 / (terms * s_))
     dproxy = coef * density * m1.sum(-1, dtype=F32)[:, None]
   dp += (dproxy * inv_s)[:, None, :]
   dlogits = p * (dp - (p * dp).sum(-1, keepdims=True))

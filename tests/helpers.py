@@ -25,24 +25,24 @@ def random_logits(rng, g, s, e, scale=1.0, quantum=None):
   return x
 
 
-def safe_logits(rng, g, s, e, scale=1.0, bias=None, min_gap=1e-4):
-  """Random logits whose three largest entries per row differ by at least
-  `min_gap` (rows that do not are redrawn), so that the top-2 choice does not
-  depend on the last ulps of exp/log."""
+def safe_logits(rng, g, s, e, scale=1.0, bias=None, min_gap=1e-4, top=3):
+  """Random logits whose `top` largest entries per row differ by at least
+  `min_gap` (rows that do not are redrawn), so that the choice of the first
+  top - 1 experts does not depend on the last ulps of exp/log."""
   x = random_logits(rng, g, s, e, scale)
   if bias is not None:
     x = x + bias
-  k = min(3, e)
+  k = min(top, e)
   for _ in range(100):
-    top = -np.sort(-x, axis=-1)[..., :k]
-    bad = ((top[..., :-1] - top[..., 1:]) < min_gap).any(axis=-1)
+    best = -np.sort(-x, axis=-1)[..., :k]
+    bad = ((best[..., :-1] - best[..., 1:]) < min_gap).any(axis=-1)
     if not bad.any():
       return x
     fresh = random_logits(rng, 1, int(bad.sum()), e, scale)[0]
     if bias is not None:
       fresh = fresh + bias
     x[bad] = fresh
-  raise AssertionError("could not separate the top-3 logits")
+  raise AssertionError("could not separate the top logits")
 
 
 def min_relative_gap(p, k=3):
@@ -80,14 +80,14 @@ def assert_routing_equal(got, want, gate_rtol=1e-5):
 
 
 def safe_tokens(rng, n_tok, m, w_gate, act_dtype, bias=None, min_gap=1e-3,
-                ones_column=False):
+                ones_column=False, top=3):
   """x [n_tok, m] ~ N(0,1) in the activation dtype such that the router logits
-  x . w_gate (+ bias) have their three largest entries per token at least
+  x . w_gate (+ bias) have their `top` largest entries per token at least
   `min_gap` apart (offending tokens are redrawn): the routing then does not
   depend on the summation order of the router matmul."""
   wg = O.cast_act(w_gate, act_dtype)
   x = O.cast_act(rng.standard_normal((n_tok, m)).astype(np.float32), act_dtype)
-  k = min(3, wg.shape[1])
+  k = min(top, wg.shape[1])
   for _ in range(100):
     logits = O.router_logits(x, wg)
     if bias is not None:

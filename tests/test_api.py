@@ -119,6 +119,23 @@ def test_v1_switch_graph_names():
                    "layer_0/wo/kernel"]
 
 
+def test_v1_ntlb_graph_names():
+  """The ntlb router's variable lives under "ntlb_gating" (the `name` default
+  of _ntlb_gating, transformer/moe.py:812)."""
+  graph, _, x, dims = graph_input()
+  hp = hparams(moe_gating="ntlb", moe_switch_policy_train="argmax",
+               moe_switch_policy_eval="argmax", moe_ntlb_top_k=3)
+  with mtf.variable_scope("layer_0"):
+    y, loss = moe.transformer_moe_layer_v1(
+        x, dims[-1], hp, True, mtf.VariableDType(torch.float32))
+  assert y.shape == mtf.Shape(dims) and loss.shape == mtf.Shape([])
+  names = sorted(v.name for v in graph.all_variables)
+  assert names == ["layer_0/ntlb_gating/kernel", "layer_0/wi/kernel",
+                   "layer_0/wo/kernel"]
+  op = [o for o in graph.operations if isinstance(o, moe.MoEV1Operation)][0]
+  assert op._gating.top_k == 3
+
+
 def test_v1_graph_names_and_shapes():
   graph, _, x, dims = graph_input()
   with mtf.variable_scope("layer_0"):
@@ -172,8 +189,13 @@ def test_error_behaviour():
   with pytest.raises(ValueError, match="Unknown policy"):
     moe.transformer_moe_layer_v1(
         x, dims[-1], hparams(moe_second_policy_train="sometimes"), True, vdt)
-  with pytest.raises(NotImplementedError):
+  # ntlb reads the switch policy first, as the reference does (moe.py:816-819)
+  with pytest.raises(AttributeError, match="moe_switch_policy_train"):
     moe.transformer_moe_layer_v1(x, dims[-1], hparams(moe_gating="ntlb"), True, vdt)
+  nt = dict(moe_gating="ntlb", moe_switch_policy_train="input_jitter",
+            moe_switch_policy_eval="argmax", moe_ntlb_top_k=2)
+  with pytest.raises(NotImplementedError, match="random numbers"):
+    moe.transformer_moe_layer_v1(x, dims[-1], hparams(**nt), True, vdt)
   # switch gating reads its own hyperparameters, as the reference does
   with pytest.raises(AttributeError, match="moe_switch_policy_train"):
     moe.transformer_moe_layer_v1(x, dims[-1], hparams(moe_gating="switch"), True, vdt)

@@ -45,6 +45,9 @@ def run_backward(hip, x, w, hp, act_dtype, d_out, d_loss, nonpad, mb):
   z = hp.moe_z_loss if gating == "switch" else None
   if gating == "top_2":
     r = hip.top2_gating(logits, c, importance=imp, num_microbatches=mb)
+  elif gating == "ntlb":
+    r = hip.ntlb_gating(logits, c, hp.moe_ntlb_top_k, importance=imp,
+                        num_microbatches=mb)
   else:
     r = hip.switch_gating(logits, c, importance=imp, z_loss=z,
                           num_microbatches=mb,
@@ -59,8 +62,10 @@ def run_backward(hip, x, w, hp, act_dtype, d_out, d_loss, nonpad, mb):
       expert_in.reshape(e, g * c, m), h, dy.reshape(e, g * c, n), wi, wo, "relu")
   dl = torch.tensor([d_loss], dtype=H.ACT_TORCH[act_dtype]).float().cuda()
   scale = torch.tensor(hp.moe_loss_coef, dtype=H.ACT_TORCH[act_dtype]).item()
-  dlogits = hip.gating_backward(logits, r, dgate, dl, scale, router=gating,
-                                importance=imp, z_loss=z, num_microbatches=mb)
+  dlogits = hip.gating_backward(
+      logits, r, dgate, dl, scale,
+      router="switch" if gating == "switch_max" else gating,
+      top_k=hp.moe_ntlb_top_k, importance=imp, z_loss=z, num_microbatches=mb)
   dwg = hip.router_backward_weights(xg.reshape(g * s, m),
                                     dlogits.reshape(g * s, e))
   dx = hip.dispatch_backward(dxe.reshape(e, g, c, m), r, s, dlogits,
@@ -78,6 +83,8 @@ CASES = [
     ("switch", 2, 128, 64, 128, 8, 1.25, "bfloat16", False),
     ("switch_max", 2, 64, 16, 24, 4, 0.75, "float32", True),
     ("top_2", 2, 256, 256, 512, 8, 1.0, "bfloat16", True),   # MFMA GEMM paths
+    ("ntlb", 2, 96, 16, 24, 6, 1.0, "float32", True),
+    ("ntlb", 2, 128, 64, 128, 8, 0.75, "bfloat16", False),
 ]
 
 
@@ -89,16 +96,22 @@ def test_backward_matches_oracle(hip, case):
   w = dict(w_gate=H.normal_weights(rng, (m, e), m),
            wi=H.normal_weights(rng, (e, m, hdim), m),
            wo=H.normal_weights(rng, (e, hdim, m), hdim))
-  x = H.safe_tokens(rng, g * s, m, w["w_gate"], act_dtype).reshape(g, s, m)
+  if gating == "ntlb":
+    w["w_gate"][:, 0] *= 3.0          # a popular expert: later rounds matter
+  x = H.safe_tokens(rng, g * s, m, w["w_gate"], act_dtype,
+                    top=4 if gating == "ntlb" else 3).reshape(g, s, m)
   nonpad = (rng.random((g, s)) < 0.85).astype(np.float32) if use_np else None
   d_out = O.cast_act(rng.standard_normal((g, s, m)).astype(np.float32), act_dtype)
   d_loss, mb = 1.5, 2
   hp = _hp(moe_gating=gating, moe_num_experts=e, moe_hidden_size=hdim,
            moe_group_size=s, moe_capacity_factor_train=cf, moe_loss_coef=0.25,
+           moe_ntlb_top_k=3,
            moe_z_loss=0.1 if (gating == "switch" and use_np) else None)
   want = O.moe_layer_v1_backward(x, w["w_gate"], w["wi"], w["wo"], hp, True,
                                  act_dtype, d_out, d_loss, nonpadding=nonpad,
                                  num_microbatches=mb)
+  if gating == "ntlb":
+    assert (want["aux"]["round"] > 0).any()
   got = run_backward(hip, x, w, hp, act_dtype, d_out, d_loss, nonpad, mb)
   tol = H.value_tolerance(act_dtype)
   np.testing.assert_allclose(got["dgate"], want["dgate"], rtol=1e-2 if

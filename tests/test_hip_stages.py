@@ -497,6 +497,76 @@ def _assert_switch_max_equal(got, want):
   assert not got["gate_2"].any()
 
 
+# ---- ntlb ("no token left behind") gating ---------------------------------------
+@pytest.mark.parametrize("shape", [(2, 1024, 8, 100, 2), (8, 2048, 64, 30, 4),
+                                   (3, 77, 5, 12, 3), (1, 1, 2, 1, 1),
+                                   (2, 131, 200, 1, 4), (1, 4096, 64, 60, 8),
+                                   (2, 512, 16, 512, 4), (4, 300, 6, 40, 6)])
+def test_ntlb_gating_random_logits(hip, shape):
+  """Skewed router (a Zipf bias) so that the popular experts overflow in round
+  0 and the later rounds route what is left."""
+  g, s, e, c, k = shape
+  rng = np.random.default_rng(3000 + sum(shape))
+  logits = H.safe_logits(rng, g, s, e, scale=1.5,
+                         bias=H.zipf_bias(rng, e, scale=2.0), top=k + 1)
+  imp = rng.choice(np.array([0.0, 0.5, 1.0], np.float32), size=(g, s),
+                   p=[0.1, 0.1, 0.8])
+  lg = torch.from_numpy(logits).cuda()
+  for importance, mb in ((None, None), (imp, 2)):
+    want = O.ntlb_gating(logits, c, k, importance=importance,
+                         num_microbatches=mb)
+    got = H.routing_to_np(hip.ntlb_gating(
+        lg, c, k, importance=None if importance is None else H.to_gpu(importance),
+        num_microbatches=mb))
+    H.assert_routing_equal(got, want)
+    np.testing.assert_allclose(got["loss"], want["loss"], rtol=2e-5)
+  if s > 64 and k > 1 and c * e < s:
+    assert (want["round"] > 0).any()       # the later rounds did something
+  assert not got["kept_1"][imp != 1.0].any()
+
+
+def test_ntlb_gating_exact_ties(hip):
+  """Logits on a coarse grid: equal probabilities within a row go to the lower
+  expert index first (repeated first-arg-max, ops.py:5009-5014)."""
+  g, s, e, c, k = 3, 500, 16, 20, 4
+  rng = np.random.default_rng(31)
+  logits = H.random_logits(rng, g, s, e, scale=0.6, quantum=0.25)
+  want = O.ntlb_gating(logits, c, k)
+  got = H.routing_to_np(hip.ntlb_gating(torch.from_numpy(logits).cuda(), c, k))
+  H.assert_routing_equal(got, want)
+  np.testing.assert_allclose(got["loss"], want["loss"], rtol=2e-5)
+
+
+def test_ntlb_dispatch_combine_roundtrip(hip):
+  """The record drives the unchanged dispatch / combine kernels: with identity
+  experts the output is gate * x for routed tokens and 0 for the others."""
+  g, s, e, c, m, k = 2, 256, 8, 24, 64, 3
+  rng = np.random.default_rng(32)
+  logits = H.safe_logits(rng, g, s, e, scale=1.5,
+                         bias=H.zipf_bias(rng, e, scale=2.0), top=k + 1)
+  x = rng.standard_normal((g, s, m)).astype(np.float32)
+  r = hip.ntlb_gating(torch.from_numpy(logits).cuda(), c, k)
+  xe = hip.dispatch(H.to_gpu(x), r)
+  out = H.to_np(hip.combine(xe, r, s))
+  rec = H.routing_to_np(r)
+  want = x * (rec["gate_1"] * rec["kept_1"])[..., None]
+  np.testing.assert_allclose(out, want, rtol=1e-6, atol=1e-7)
+  ref = O.ntlb_gating(logits, c, k)
+  np.testing.assert_array_equal(
+      H.to_np(xe), O.dispatch_gather(x, ref, e, c, "float32"))
+
+
+def test_ntlb_gating_rejections(hip):
+  lg = torch.zeros((1, 8, 4), dtype=torch.float32, device="cuda")
+  with pytest.raises(hip.MoeHipError, match="top_k=5 with 4 experts"):
+    hip.ntlb_gating(lg, 2, 5)
+  with pytest.raises(hip.MoeHipError, match="top_k=0"):
+    hip.ntlb_gating(lg, 2, 0)
+  big = torch.zeros((1, 8, 16), dtype=torch.float32, device="cuda")
+  with pytest.raises(hip.MoeHipError, match="top_k=9 > 8"):
+    hip.ntlb_gating(big, 2, 9)
+
+
 @pytest.mark.parametrize("shape", [(2, 1024, 8, 160), (16, 2048, 64, 32),
                                    (3, 77, 5, 7), (1, 1, 2, 1),
                                    (2, 131, 200, 4), (1, 4096, 64, 40)])

@@ -46,8 +46,8 @@ def run_v1(x, weights, hp, train, act_dtype, nonpadding=None, activation="relu",
     y, loss = moe.transformer_moe_layer_v1(
         xt, mtf.Dimension("d_model", n), hp, train, vdt, nonpadding=npad,
         activation=activation, num_microbatches=num_microbatches)
-  router = {"switch": "switch_gating", "switch_max": "switch_max_gating"}.get(
-      hp.moe_gating, "top_2_gating")
+  router = {"switch": "switch_gating", "switch_max": "switch_max_gating",
+            "ntlb": "ntlb_gating"}.get(hp.moe_gating, "top_2_gating")
   init = {"moe/%s/kernel" % router: weights["w_gate"],
           "moe/wi/kernel": weights["wi"], "moe/wo/kernel": weights["wo"]}
   lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()}, initial_values=init)
@@ -324,6 +324,41 @@ def test_v1_switch_rejections():
     run_v1(x, w, hp, True, "float32")
 
 
+@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
+def test_v1_ntlb_matches_oracle(act_dtype):
+  """ntlb end to end with a skewed router, so that round 0 overflows and the
+  later rounds place tokens; nonpadding masks some tokens out."""
+  b, l, m, hdim, e, group, k = 2, 256, 64, 128, 8, 128, 3
+  rng = np.random.default_rng(305)
+  w = dict(w_gate=H.normal_weights(rng, (m, e), m),
+           wi=H.normal_weights(rng, (e, m, hdim), m),
+           wo=H.normal_weights(rng, (e, hdim, m), hdim))
+  w["w_gate"][:, 0] *= 3.0                          # expert 0 is popular
+  x = H.safe_tokens(rng, b * l, m, w["w_gate"], act_dtype,
+                    top=k + 1).reshape(b, l, m)
+  nonpad = (rng.random((b, l)) < 0.85).astype(np.float32)
+  hp, ohp = make_hparams(moe_num_experts=e, moe_hidden_size=hdim,
+                         moe_group_size=group, moe_capacity_factor_eval=1.0,
+                         moe_ntlb_top_k=k,
+                         **dict(SWITCH_HP, moe_gating="ntlb"))
+  got, got_loss, _, _ = run_v1(x, w, hp, False, act_dtype, nonpadding=nonpad,
+                               num_microbatches=2)
+  want, want_loss, aux = O.moe_layer_v1(x, w["w_gate"], w["wi"], w["wo"], ohp,
+                                        False, act_dtype, nonpadding=nonpad,
+                                        num_microbatches=2, dense=True)
+  assert (aux["round"] > 0).any() and not aux["kept_1"].all()
+  np.testing.assert_allclose(got, want, **H.value_tolerance(act_dtype))
+  np.testing.assert_allclose(got_loss, want_loss,
+                             rtol=1e-2 if act_dtype == "bfloat16" else 1e-4)
+  assert (got.reshape(-1, m)[~aux["kept_1"].reshape(-1)] == 0).all()
+  hp_j, _ = make_hparams(moe_num_experts=e, moe_hidden_size=hdim,
+                         moe_group_size=group, moe_ntlb_top_k=k,
+                         **dict(SWITCH_HP, moe_gating="ntlb",
+                                moe_switch_policy_train="input_jitter"))
+  with pytest.raises(NotImplementedError, match="random"):
+    run_v1(x, w, hp_j, True, act_dtype)
+
+
 def test_v1_switch_max_matches_oracle():
   """switch_max end to end.  Which tokens an over-subscribed expert keeps
   depends on gates that the two implementations compute with different exp
@@ -360,7 +395,8 @@ def test_v1_switch_max_matches_oracle():
 # ---- gradients through the mtf-shaped API -------------------------------------
 @pytest.mark.parametrize("case", [
     ("top_2", "float32", 101), ("top_2", "bfloat16", 102),
-    ("switch", "float32", 103), ("switch_max", "float32", 104)],
+    ("switch", "float32", 103), ("switch_max", "float32", 104),
+    ("ntlb", "float32", 105)],
     ids=lambda c: "%s-%s" % (c[0], c[1]))
 def test_v1_gradients_match_oracle(case):
   """mtf.gradients over the layer (outputs and loss) against the oracle's
@@ -371,13 +407,14 @@ def test_v1_gradients_match_oracle(case):
   w = dict(w_gate=H.normal_weights(rng, (m, e), m),
            wi=H.normal_weights(rng, (e, m, hdim), m),
            wo=H.normal_weights(rng, (e, hdim, m), hdim))
-  x = H.safe_tokens(rng, b * l, m, w["w_gate"], act_dtype).reshape(b, l, m)
+  x = H.safe_tokens(rng, b * l, m, w["w_gate"], act_dtype,
+                    top=4).reshape(b, l, m)
   nonpad = (rng.random((b, l)) < 0.85).astype(np.float32)
   d_out = O.cast_act(rng.standard_normal((b, l, m)).astype(np.float32), act_dtype)
   kw = dict(moe_num_experts=e, moe_hidden_size=hdim, moe_group_size=group,
             moe_capacity_factor_train=1.0, moe_loss_coef=0.25)
   if gating != "top_2":
-    kw.update(SWITCH_HP, moe_gating=gating,
+    kw.update(SWITCH_HP, moe_gating=gating, moe_ntlb_top_k=3,
               moe_z_loss=0.1 if gating == "switch" else None)
   hp, ohp = make_hparams(**kw)
   dt = H.ACT_TORCH[act_dtype]
@@ -398,8 +435,8 @@ def test_v1_gradients_match_oracle(case):
   dlt = mtf.import_tf_tensor(mesh, torch.tensor(1.5, dtype=dt), mtf.Shape([]))
   grads = mtf.gradients([y, loss], [xt] + [v.outputs[0] for v in variables],
                         grad_ys=[dyt, dlt])
-  router = {"switch": "switch_gating", "switch_max": "switch_max_gating"}.get(
-      gating, "top_2_gating")
+  router = {"switch": "switch_gating", "switch_max": "switch_max_gating",
+            "ntlb": "ntlb_gating"}.get(gating, "top_2_gating")
   init = {"moe/%s/kernel" % router: w["w_gate"], "moe/wi/kernel": w["wi"],
           "moe/wo/kernel": w["wo"]}
   lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()}, initial_values=init)
@@ -415,7 +452,8 @@ def test_v1_gradients_match_oracle(case):
         g_, ref, rtol=tol["rtol"], atol=tol["atol"] * max(1.0, np.abs(ref).max()),
         err_msg=k)
   # a second step re-runs forward and backward on new tokens
-  x2 = H.safe_tokens(rng, b * l, m, w["w_gate"], act_dtype).reshape(b, l, m)
+  x2 = H.safe_tokens(rng, b * l, m, w["w_gate"], act_dtype,
+                     top=4).reshape(b, l, m)
   lowering.run({xt: torch.from_numpy(x2).to(dt).cuda()})
   want2 = O.moe_layer_v1_backward(x2, w["w_gate"], w["wi"], w["wo"], ohp, True,
                                   act_dtype, d_out, 1.5, nonpadding=nonpad,

@@ -450,6 +450,178 @@ def test_v1_switch_dense_equals_index_form():
     O.moe_layer_v1(x, wg, wi, wo, hp, False)
 
 
+# ---- ntlb ("no token left behind") gating ---------------------------------------
+def _ntlb_by_token_walk(p64, k, c, imp):
+  """transformer/moe.py:903-934 as a walk over (round, token): round i offers
+  the unrouted tokens, in token order, to their i-th best expert; the expert's
+  counter for the round starts at what it holds and counts every offer, taken
+  or not; an offer is taken while the counter stays within the capacity."""
+  g, s, e = p64.shape
+  order = np.argsort(-p64, axis=-1, kind="stable")[..., :k]
+  routed = np.full((g, s), -1)
+  slot = np.zeros((g, s), int)
+  held = np.zeros((g, e), int)
+  for gi in range(g):
+    for i in range(k):
+      offered = held[gi].copy()
+      for si in range(s):
+        if routed[gi, si] >= 0 or (imp is not None and imp[gi, si] != 1.0):
+          continue
+        ex = order[gi, si, i]
+        offered[ex] += 1
+        if offered[ex] <= c:
+          routed[gi, si], slot[gi, si] = i, offered[ex] - 1
+          held[gi, ex] += 1
+  return order, routed, slot, held
+
+
+@pytest.mark.parametrize("seed", range(6))
+def test_ntlb_against_token_walk_and_float64(seed):
+  rng = np.random.default_rng(900 + seed)
+  g, s, e = 3, int(rng.integers(30, 80)), int(rng.integers(3, 7))
+  k = 1 + seed % 4 if seed % 4 < e else e
+  c = s // e + 1
+  # expert 0 is everybody's favourite: it overflows in round 0 while the
+  # others keep room for the later rounds
+  logits = (2 * rng.standard_normal((g, s, e))).astype(np.float32)
+  logits[..., 0] += 2.0
+  imp = None
+  if seed % 2:
+    imp = rng.choice(np.array([0.0, 0.5, 1.0, 1.0, 1.0, 1.0, 1.0], np.float32),
+                     size=(g, s))
+  p64 = scipy.special.softmax(logits.astype(np.float64), axis=-1)
+  order, routed, slot, held = _ntlb_by_token_walk(p64, k, c, imp)
+  for dense in (False, True):
+    r = O.ntlb_gating(logits, c, k, importance=imp, dense=dense)
+    np.testing.assert_array_equal(r["topk_index"], order)
+    np.testing.assert_array_equal(r["round"], routed)
+    np.testing.assert_array_equal(r["kept_1"], routed >= 0)
+    np.testing.assert_array_equal(r["fill"], held)
+    assert not r["kept_2"].any() and not r["gate_2"].any()
+    took = routed >= 0
+    ex = np.take_along_axis(order, np.maximum(routed, 0)[..., None], -1)[..., 0]
+    np.testing.assert_array_equal(r["index_1"][took], ex[took])
+    np.testing.assert_array_equal(r["pos_1"][took], slot[took])
+    want = np.take_along_axis(p64, ex[..., None], -1)[..., 0] * took
+    np.testing.assert_allclose(r["gate_1"], want, rtol=2e-6)
+  # the capacity leaves first choices unserved, so later rounds matter
+  assert (routed != 0).any()
+  if k > 1:
+    assert (routed > 0).any()
+
+
+def test_ntlb_hand_worked_case():
+  """4 tokens, 3 experts, capacity 1, k = 2.  First choices 0,0,1,0; second
+  choices 1,2,0,1.  Round 0: token 0 takes expert 0, token 1 overflows it,
+  token 2 takes expert 1, token 3 overflows.  Round 1: token 1 -> expert 2
+  (free), token 3 -> expert 1 (full) -> dropped."""
+  big, mid, low = 3.0, 1.0, -2.0
+  logits = np.array([[[big, mid, low], [big, low, mid], [mid, big, low],
+                      [big, mid, low]]], np.float32)
+  r = O.ntlb_gating(logits, 1, 2, dense=True)
+  p = scipy.special.softmax(logits.astype(np.float64), axis=-1)[0]
+  np.testing.assert_array_equal(r["kept_1"][0], [True, True, True, False])
+  np.testing.assert_array_equal(r["index_1"][0][:3], [0, 2, 1])
+  np.testing.assert_array_equal(r["round"][0], [0, 1, 0, -1])
+  np.testing.assert_array_equal(r["pos_1"][0][:3], [0, 0, 0])
+  np.testing.assert_allclose(r["gate_1"][0], [p[0, 0], p[1, 2], p[2, 1], 0],
+                             rtol=2e-6)
+  np.testing.assert_array_equal(r["fill"][0], [1, 1, 1])
+  want = np.zeros((4, 3, 1), np.float32)
+  want[0, 0, 0], want[1, 2, 0], want[2, 1, 0] = r["gate_1"][0][:3]
+  np.testing.assert_array_equal(r["combine"][0], want)
+
+
+def test_ntlb_with_one_choice_is_switch():
+  """k = 1: the one round is _switch_gating's capacity rule (an offer counts
+  whether or not it is taken, moe.py:1268-1276 and :908-914) and the loss is
+  the same expression."""
+  rng = np.random.default_rng(910)
+  logits = rng.standard_normal((2, 50, 4)).astype(np.float32)
+  imp = rng.choice(np.array([0.0, 1.0], np.float32), size=(2, 50))
+  for importance in (None, imp):
+    a = O.ntlb_gating(logits, 7, 1, importance=importance, num_microbatches=3)
+    b = O.switch_gating(logits, 7, importance=importance, num_microbatches=3)
+    for key in ("kept_1", "gate_1", "fill"):
+      np.testing.assert_array_equal(a[key], b[key])
+    np.testing.assert_array_equal(a["index_1"][a["kept_1"]],
+                                  b["index_1"][b["kept_1"]])
+    np.testing.assert_array_equal(a["pos_1"][a["kept_1"]],
+                                  b["pos_1"][b["kept_1"]])
+    np.testing.assert_allclose(a["loss"], b["loss"], rtol=1e-6)
+
+
+def test_ntlb_loss_closed_forms():
+  """loss = E^2 * mean over [G,k,E] of proxy[g,e] * density[g,i,e]
+  (moe.py:845-856).  Uniform router: proxy = 1/E, and each round's density
+  sums to 1 over the experts, so the loss is E^2 * (1/E) * 1/E = 1 for any k.
+  With importance the product gains the group dim and the mean the factor
+  mean(importance == 1)."""
+  g, s, e, k = 2, 24, 4, 3
+  r = O.ntlb_gating(np.zeros((g, s, e), np.float32), 100, k)
+  np.testing.assert_allclose(r["loss"], 1.0, rtol=1e-6)
+  # uniform router: every token names experts 0..k-1 in this order
+  np.testing.assert_array_equal(r["topk_index"][0, 0], np.arange(k))
+  imp = np.ones((g, s), np.float32)
+  imp[:, : s // 4] = 0.0
+  r2 = O.ntlb_gating(np.zeros((g, s, e), np.float32), 100, k, importance=imp)
+  np.testing.assert_allclose(r2["loss"], 0.75, rtol=1e-6)
+  rng = np.random.default_rng(911)
+  logits = rng.standard_normal((g, s, e)).astype(np.float32)
+  p = scipy.special.softmax(logits.astype(np.float64), axis=-1)
+  order = np.argsort(-p, axis=-1, kind="stable")[..., :k]
+  dens = np.stack([(order[..., i, None] == np.arange(e)).mean(axis=1)
+                   for i in range(k)], axis=1)               # [G,k,E]
+  want = e * e * (p.mean(axis=1)[:, None, :] * dens).mean()
+  got = O.ntlb_gating(logits, 5, k, num_microbatches=2)["loss"]
+  np.testing.assert_allclose(got, want / 2, rtol=1e-5)
+
+
+@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
+def test_ntlb_dense_tensors_match_index_record(act_dtype):
+  rng = np.random.default_rng(912)
+  g, s, e, c, k = 2, 40, 5, 5, 3
+  logits = (2 * rng.standard_normal((g, s, e))).astype(np.float32)
+  r = O.ntlb_gating(logits, c, k, act_dtype=act_dtype, dense=True)
+  want = np.zeros((g, s, e, c), np.float32)
+  w = O.cast_act(r["gate_1"], act_dtype)
+  for gi in range(g):
+    for si in range(s):
+      if r["kept_1"][gi, si]:
+        want[gi, si, r["index_1"][gi, si], r["pos_1"][gi, si]] = w[gi, si]
+  np.testing.assert_array_equal(r["combine"], want)
+  np.testing.assert_array_equal(r["dispatch"], (want != 0).astype(np.float32))
+  assert (r["dispatch"].sum(axis=1) <= 1).all()      # one token per slot
+  assert (r["round"] > 0).any()
+
+
+def test_v1_ntlb_dense_equals_index_form():
+  rng = np.random.default_rng(913)
+  b, l, m, h, e = 2, 48, 16, 24, 4
+  x = rng.standard_normal((b, l, m)).astype(np.float32)
+  wg = rng.standard_normal((m, e)).astype(np.float32)
+  wi = rng.standard_normal((e, m, h)).astype(np.float32) / 4
+  wo = rng.standard_normal((e, h, m)).astype(np.float32) / 5
+  hp = O.default_hparams(moe_gating="ntlb", moe_num_experts=e,
+                         moe_hidden_size=h, moe_group_size=32,
+                         moe_capacity_factor_eval=1.0, moe_ntlb_top_k=2)
+  nonpad = (rng.random((b, l)) < 0.8).astype(np.float32)
+  d, dl, aux = O.moe_layer_v1(x, wg, wi, wo, hp, False, nonpadding=nonpad,
+                              dense=True)
+  i, il, _ = O.moe_layer_v1(x, wg, wi, wo, hp, False, nonpadding=nonpad,
+                            dense=False)
+  np.testing.assert_allclose(d, i, rtol=1e-5, atol=1e-5)
+  assert dl == il
+  assert (d[nonpad == 0] == 0).all()
+  t = int(np.flatnonzero(aux["round"].reshape(-1) == 1)[0])   # a second choice
+  ex = int(aux["index_1"].reshape(-1)[t])
+  xt = x.reshape(-1, m)[t].astype(np.float64)
+  ref = np.maximum(xt @ wi[ex].astype(np.float64), 0) @ wo[ex].astype(np.float64)
+  np.testing.assert_allclose(d.reshape(-1, m)[t],
+                             aux["gate_1"].reshape(-1)[t] * ref, rtol=1e-4,
+                             atol=1e-5)
+
+
 # ---- switch_max gating ----------------------------------------------------------
 def test_top_k_matches_iterative_top_1():
   """mtf.top_k lowers 1 < k < 5 as repeated top_1 with the taken entries pushed
@@ -781,6 +953,13 @@ def _f64_layer(x, wg, wi, wo, aux, gating, m1, coef, mb, z_loss):
     density = (onehot1 * m1[..., None]).mean(1)
     proxy = (p * m1[..., None]).mean(1)
     aux_loss = (proxy * density).mean() * e * e / mb
+  elif gating == "ntlb":
+    out = (p[rows + (i1,)] * m1 * k1)[..., None] * ffn(i1)
+    topk = aux["topk_index"]                                  # [G,S,k] fixed
+    density = (topk[..., None] == np.arange(e)).mean(1)       # [G,k,E]
+    proxy = p.mean(1)                                         # [G,E]
+    aux_loss = (proxy[:, None, :, None] * m1[:, None, None, :]
+                * density[..., None]).mean() * e * e / mb
   else:
     out = (p[rows + (i1,)] * m1 * k1)[..., None] * ffn(i1)
     density = onehot1.mean(1)
@@ -793,7 +972,7 @@ def _f64_layer(x, wg, wi, wo, aux, gating, m1, coef, mb, z_loss):
   return out, aux_loss * coef
 
 
-@pytest.mark.parametrize("gating", ["top_2", "switch", "switch_max"])
+@pytest.mark.parametrize("gating", ["top_2", "switch", "switch_max", "ntlb"])
 def test_backward_against_central_differences(gating):
   rng = np.random.default_rng(61)
   b, l, m, h, e, group = 2, 24, 6, 10, 4, 24
@@ -807,12 +986,14 @@ def test_backward_against_central_differences(gating):
   hp = _hp(moe_gating=gating, moe_num_experts=e, moe_hidden_size=h,
            moe_group_size=group, moe_capacity_factor_train=1.2,
            moe_min_expert_capacity=2, moe_loss_coef=0.5,
-           moe_switch_policy_train="argmax",
+           moe_switch_policy_train="argmax", moe_ntlb_top_k=3,
            moe_z_loss=0.3 if gating == "switch" else None)
   got = O.moe_layer_v1_backward(x, wg, wi, wo, hp, True, "float32", d_out,
                                 d_loss, nonpadding=nonpad, num_microbatches=mb)
   aux = got["aux"]
   assert not (aux["kept_1"] | aux["kept_2"]).all()     # drops are exercised
+  if gating == "ntlb":
+    assert (aux["round"] > 0).any()        # tokens placed by a later choice
   m1 = (nonpad.reshape(aux["kept_1"].shape) == 1).astype(np.float64)
   z = hp.moe_z_loss if gating == "switch" else None
 
