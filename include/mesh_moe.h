@@ -436,6 +436,46 @@ int mesh_moe_dispatch_backward(const void* dexpert_in, const int32_t* idx,
                                int groups_per_router, void* dx, int G, int S,
                                int E, int C, int M, int dtype, void* stream);
 
+/*
+ * ---------------------------------------------------------------------------
+ * The rest of a transformer block around the layer (the LayerStack sublayers
+ * and SelfAttention of mesh_tensorflow/transformer/transformer.py and
+ * transformer_layers.py).  Dense projections use mesh_moe_expert_linear with
+ * E = 1.
+ * ---------------------------------------------------------------------------
+ */
+
+/*
+ * RMS normalisation (sublayer_rms_norm, transformer/transformer.py:493-516):
+ * y = x * rsqrt(mean(square(x)) + epsilon) * scale over the last dim, one
+ * rounding to dtype per reference op, float32 accumulation.
+ *   x, y [rows,M] dtype; scale [M] dtype
+ */
+int mesh_moe_rms_norm(const void* x, const void* scale, void* y, int64_t rows,
+                      int M, double epsilon, int dtype, void* stream);
+
+/* Bytes of scratch mesh_moe_self_attention needs. */
+size_t mesh_moe_self_attention_workspace_bytes(int B, int L, int H, int D,
+                                               int dtype);
+
+/*
+ * Multi-head dot-product self-attention after the q/k/v projections
+ * (attention.attention with float32_logits, transformer/attention.py:27-88):
+ * float32 logits q . k (no scaling: the reference folds 1/sqrt(d_kv) into the
+ * query kernel's initialiser, attention.py:436-439), keys after the query
+ * masked when `causal` (the autoregressive bias of
+ * transformer_layers.py:289-296 via attention.py:830-842), float32 softmax,
+ * weights cast to dtype, outputs = weights . v.
+ *   q, k, v, out [B,L,H*D] dtype (heads and d_kv combined as the reference's
+ *   combine_dims does); bf16 needs L and D multiples of 8.
+ * The logits and weights of all heads live in the workspace
+ * (B*H*L*L*(4 + sizeof dtype) bytes).
+ */
+int mesh_moe_self_attention(const void* q, const void* k, const void* v,
+                            void* out, int B, int L, int H, int D, int causal,
+                            int dtype, void* workspace, size_t workspace_bytes,
+                            void* stream);
+
 #ifdef __cplusplus
 }
 #endif

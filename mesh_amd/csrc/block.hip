@@ -1,0 +1,245 @@
+// The rest of a transformer block around the Mixture-of-Experts layer, for
+// gfx950: RMS normalisation and multi-head self-attention.
+//
+// rms_norm follows sublayer_rms_norm, mesh_tensorflow/transformer/
+// transformer.py:493-516: x * rsqrt(mean(square(x)) + epsilon) * scale, one
+// rounding to the activation dtype per reference op, float32 accumulation.
+//
+// self_attention follows attention.attention, mesh_tensorflow/transformer/
+// attention.py:27-88 with float32_logits (the default): logits = q . k in
+// float32, plus a -1e9 bias where a key is not visible (attention.py:830-842),
+// mtf.softmax in float32 (ops.py:5493-5541), weights cast to the activation
+// dtype, outputs = weights . v.  The scaling 1/sqrt(d_kv) is folded into the
+// query kernel's initialiser by the reference (attention.py:436-439), so none
+// is applied here.
+#include "common.h"
+
+namespace mesh_moe {
+
+// ---------------------------------------------------------------------------
+// RMS norm: one wavefront per row.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void rms_norm_kernel(
+    const T* __restrict__ x, const T* __restrict__ scale, T* __restrict__ y,
+    int64_t rows, int M, float inv_m, float eps) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const T* xr = x + row * M;
+  float sum = 0.f;
+  for (int i = lane; i < M; i += 64) {
+    const float v = load_f32<T>(xr + i);
+    sum += round_to<T>(v * v);                              // mtf.square
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+  const float total = round_to<T>(sum);                     // reduce_sum
+  const float mean = round_to<T>(total * inv_m);            // * (1 / M)
+  const float var = round_to<T>(mean + eps);                // + epsilon
+  const float r = round_to<T>(1.0f / sqrtf(var));           // rsqrt
+  T* yr = y + row * M;
+  for (int i = lane; i < M; i += 64) {
+    const float v = load_f32<T>(xr + i);
+    const float s = load_f32<T>(scale + i);
+    store_f32<T>(yr + i, round_to<T>(v * r) * s);
+  }
+}
+
+// ---------------------------------------------------------------------------
+// [B, L, H*D] -> [B*H, L, D]  (heads to the front)
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ void split_heads_kernel(const T* __restrict__ in, T* __restrict__ out,
+                                   int B, int L, int H, int D) {
+  const int64_t n = (int64_t)B * L * H * D;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += stride) {
+    const int d = (int)(i % D);
+    int64_t r = i / D;
+    const int l = (int)(r % L);
+    r /= L;
+    const int h = (int)(r % H);
+    const int b = (int)(r / H);
+    out[i] = in[(((int64_t)b * L + l) * H + h) * D + d];
+  }
+}
+
+// [B*H, L, D] -> [B, L, H*D]
+template <typename T>
+__global__ void merge_heads_kernel(const T* __restrict__ in, T* __restrict__ out,
+                                   int B, int L, int H, int D) {
+  const int64_t n = (int64_t)B * L * H * D;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += stride) {
+    const int d = (int)(i % D);
+    int64_t r = i / D;
+    const int h = (int)(r % H);
+    r /= H;
+    const int l = (int)(r % L);
+    const int b = (int)(r / L);
+    out[i] = in[(((int64_t)b * H + h) * L + l) * D + d];
+  }
+}
+
+// [B, L, H*D] -> [B*H, D, L]: the values as the K-contiguous second operand of
+// weights . v.  32 x 32 tiles through LDS so both sides are coalesced.
+template <typename T>
+__global__ __launch_bounds__(256) void transpose_heads_kernel(
+    const T* __restrict__ in, T* __restrict__ out, int B, int L, int H, int D) {
+  __shared__ T tile[32][33];
+  const int bh = blockIdx.z, b = bh / H, h = bh % H;
+  const int l0 = blockIdx.x * 32, d0 = blockIdx.y * 32;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;   // 32 x 8
+  for (int r = ty; r < 32; r += 8) {
+    const int l = l0 + r, d = d0 + tx;
+    if (l < L && d < D)
+      tile[r][tx] = in[(((int64_t)b * L + l) * H + h) * D + d];
+  }
+  __syncthreads();
+  for (int r = ty; r < 32; r += 8) {
+    const int d = d0 + r, l = l0 + tx;
+    if (l < L && d < D) out[((int64_t)bh * D + d) * L + l] = tile[tx][r];
+  }
+}
+
+// ---------------------------------------------------------------------------
+// Row softmax of the logits [BH, L, L] (float32) into weights of the
+// activation dtype; with `causal`, query i sees keys 0..i.  One wavefront per
+// row; the operation order is mtf.softmax's: exp(x - (log(sum(exp(x - max))) +
+// max)).  A key that is not visible carries logit + (-1e9), whose exp is
+// exactly 0 in float32, so it is left out of max and sum.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void attention_softmax_kernel(
+    const float* __restrict__ logits, T* __restrict__ weights, int64_t rows,
+    int L, int causal) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int i = (int)(row % L);
+  const int visible = causal ? i + 1 : L;
+  const float* xr = logits + row * L;
+  float m = -INFINITY;
+  for (int j = lane; j < visible; j += 64) m = fmaxf(m, xr[j]);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+  const float negm = -m;
+  float sum = 0.f;
+  for (int j = lane; j < visible; j += 64) sum += expf(xr[j] + negm);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+  const float neglse = -(logf(sum) + m);
+  T* wr = weights + row * L;
+  for (int j = lane; j < L; j += 64)
+    store_f32<T>(wr + j, j < visible ? expf(xr[j] + neglse) : 0.0f);
+}
+
+template <typename T>
+static int run_attention(const T* q, const T* k, const T* v, T* out, int B,
+                         int L, int H, int D, int causal, int dtype,
+                         void* workspace, hipStream_t st) {
+  const int BH = B * H;
+  const size_t hd = (size_t)BH * L * D, ll = (size_t)BH * L * L;
+  auto up = [](uintptr_t p) { return (p + 255) & ~(uintptr_t)255; };
+  T* qh = (T*)up((uintptr_t)workspace);
+  T* kh = (T*)up((uintptr_t)(qh + hd));
+  T* vt = (T*)up((uintptr_t)(kh + hd));
+  T* oh = (T*)up((uintptr_t)(vt + hd));
+  float* logits = (float*)up((uintptr_t)(oh + hd));
+  T* weights = (T*)up((uintptr_t)(logits + ll));
+  const int64_t n = (int64_t)hd;
+  const unsigned eb = (unsigned)((n + 255) / 256 < 65536 ? (n + 255) / 256
+                                                         : 65536);
+  split_heads_kernel<T><<<eb, 256, 0, st>>>(q, qh, B, L, H, D);
+  MOE_CHECK_LAUNCH("self_attention (split q)");
+  split_heads_kernel<T><<<eb, 256, 0, st>>>(k, kh, B, L, H, D);
+  MOE_CHECK_LAUNCH("self_attention (split k)");
+  dim3 tg((unsigned)((L + 31) / 32), (unsigned)((D + 31) / 32), (unsigned)BH);
+  transpose_heads_kernel<T><<<tg, 256, 0, st>>>(v, vt, B, L, H, D);
+  MOE_CHECK_LAUNCH("self_attention (transpose v)");
+  int rc = batched_gemm_nt(qh, kh, logits, BH, L, L, D, dtype, true, st);
+  if (rc != 0) return rc;
+  const int64_t rows = (int64_t)BH * L;
+  attention_softmax_kernel<T><<<(unsigned)((rows + 3) / 4), 256, 0, st>>>(
+      logits, weights, rows, L, causal);
+  MOE_CHECK_LAUNCH("self_attention (softmax)");
+  rc = batched_gemm_nt(weights, vt, oh, BH, L, D, L, dtype, false, st);
+  if (rc != 0) return rc;
+  merge_heads_kernel<T><<<eb, 256, 0, st>>>(oh, out, B, L, H, D);
+  MOE_CHECK_LAUNCH("self_attention (merge)");
+  return 0;
+}
+
+}  // namespace mesh_moe
+
+using namespace mesh_moe;
+
+extern "C" int mesh_moe_rms_norm(const void* x, const void* scale, void* y,
+                                 int64_t rows, int M, double epsilon, int dtype,
+                                 void* stream) {
+  MOE_REQUIRE(x && scale && y, MESH_MOE_E_ARG, "rms_norm: null pointer");
+  MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG, "rms_norm: bad dtype %d",
+              dtype);
+  MOE_REQUIRE(rows >= 1 && M >= 1, MESH_MOE_E_ARG,
+              "rms_norm: bad sizes rows=%lld M=%d", (long long)rows, M);
+  const int64_t blocks = (rows + 3) / 4;
+  MOE_REQUIRE(blocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
+              "rms_norm: too many rows (%lld)", (long long)rows);
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == MESH_MOE_F32) {
+    rms_norm_kernel<float><<<(unsigned)blocks, 256, 0, st>>>(
+        (const float*)x, (const float*)scale, (float*)y, rows, M,
+        (float)(1.0 / (double)M), (float)epsilon);
+  } else {
+    // Python scalars reach the reference's ops rounded to the tensor dtype
+    const float inv_m = round_bf16_host((float)(1.0 / (double)M));
+    const float eps = round_bf16_host((float)epsilon);
+    rms_norm_kernel<bf16_t><<<(unsigned)blocks, 256, 0, st>>>(
+        (const bf16_t*)x, (const bf16_t*)scale, (bf16_t*)y, rows, M, inv_m,
+        eps);
+  }
+  MOE_CHECK_LAUNCH("rms_norm");
+  return 0;
+}
+
+extern "C" size_t mesh_moe_self_attention_workspace_bytes(int B, int L, int H,
+                                                          int D, int dtype) {
+  if (B < 1 || L < 1 || H < 1 || D < 1 || !valid_dtype(dtype)) return 0;
+  const size_t b = dtype_size(dtype);
+  const size_t hd = (size_t)B * H * L * D, ll = (size_t)B * H * L * L;
+  return 4 * hd * b + ll * 4 + ll * b + 7 * 256;
+}
+
+extern "C" int mesh_moe_self_attention(const void* q, const void* k,
+                                       const void* v, void* out, int B, int L,
+                                       int H, int D, int causal, int dtype,
+                                       void* workspace, size_t workspace_bytes,
+                                       void* stream) {
+  MOE_REQUIRE(q && k && v && out && workspace, MESH_MOE_E_ARG,
+              "self_attention: null pointer");
+  MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG,
+              "self_attention: bad dtype %d", dtype);
+  MOE_REQUIRE(B >= 1 && L >= 1 && H >= 1 && D >= 1, MESH_MOE_E_ARG,
+              "self_attention: bad sizes B=%d L=%d H=%d D=%d", B, L, H, D);
+  MOE_REQUIRE((int64_t)B * H <= 65535, MESH_MOE_E_UNSUPPORTED,
+              "self_attention: batch * heads = %lld > 65535",
+              (long long)B * H);
+  MOE_REQUIRE(dtype == MESH_MOE_F32 || (L % 8 == 0 && D % 8 == 0),
+              MESH_MOE_E_UNSUPPORTED,
+              "self_attention: bfloat16 needs length and d_kv multiples of 8 "
+              "(L=%d D=%d)", L, D);
+  MOE_REQUIRE(workspace_bytes >=
+                  mesh_moe_self_attention_workspace_bytes(B, L, H, D, dtype),
+              MESH_MOE_E_ARG, "self_attention: workspace too small");
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == MESH_MOE_F32)
+    return run_attention<float>((const float*)q, (const float*)k,
+                                (const float*)v, (float*)out, B, L, H, D,
+                                causal ? 1 : 0, dtype, workspace, st);
+  return run_attention<bf16_t>((const bf16_t*)q, (const bf16_t*)k,
+                               (const bf16_t*)v, (bf16_t*)out, B, L, H, D,
+                               causal ? 1 : 0, dtype, workspace, st);
+}

@@ -4,6 +4,7 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 #include <stdio.h>
+#include <string.h>
 
 #include "../../include/mesh_moe.h"
 
@@ -11,6 +12,12 @@ namespace mesh_moe {
 
 // Per-thread error text returned by mesh_moe_last_error().
 void set_error(const char* fmt, ...);
+
+// Batched C[e] = A[e] . B[e]^T (ffn.hip): A [E,R,K], B [E,N,K] of `dtype`
+// (MESH_MOE_F32 / MESH_MOE_BF16), C [E,R,N] of `dtype`, or float32 when
+// out_f32.  Float32 accumulation on the matrix cores for bf16.
+int batched_gemm_nt(const void* A, const void* B, void* C, int E, int R, int N,
+                    int K, int dtype, bool out_f32, hipStream_t st);
 
 #define MOE_REQUIRE(cond, code, ...)      \
   do {                                    \
@@ -56,6 +63,16 @@ static inline size_t dtype_size(int d) { return d == MESH_MOE_BF16 ? 2 : 4; }
 
 // ---- bfloat16 as raw bits -------------------------------------------------
 typedef uint16_t bf16_t;
+
+// host side: a finite float32 rounded to the nearest bfloat16 (ties to even)
+static inline float round_bf16_host(float f) {
+  uint32_t u;
+  memcpy(&u, &f, 4);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  u &= 0xffff0000u;
+  memcpy(&f, &u, 4);
+  return f;
+}
 
 __device__ __forceinline__ float bf16_to_f32(bf16_t v) {
   return __uint_as_float(((uint32_t)v) << 16);

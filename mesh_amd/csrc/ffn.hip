@@ -58,10 +58,11 @@ __device__ __forceinline__ uint32_t pack2_bf16(float a, float b, bool relu) {
   return f32x2_to_bf16x2(a, b);
 }
 
-template <int BM, int BN, int BK, bool RELU>
+template <int BM, int BN, int BK, bool RELU, bool OUT_F32 = false>
 __global__ __launch_bounds__(256) void grouped_gemm_bf16_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
-    bf16_t* __restrict__ Cout, int R, int N, int K, int tiles_m, int tiles_n) {
+    void* __restrict__ Cvoid, int R, int N, int K, int tiles_m, int tiles_n) {
+  bf16_t* Cout = reinterpret_cast<bf16_t*>(Cvoid);
   using Cfg = GemmCfg<BM, BN, BK>;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   bf16_t* As = reinterpret_cast<bf16_t*>(smem_raw);  // [2][BM][LDK]
@@ -168,10 +169,36 @@ __global__ __launch_bounds__(256) void grouped_gemm_bf16_kernel(
     __syncthreads();
   }
 
-  // epilogue: round (and relu), stage the tile in LDS, coalesced stores
-  bf16_t* Cs = reinterpret_cast<bf16_t*>(smem_raw);  // [BM][LDC]
   const int m_l = lane & 31;
   const int n_l = (lane >> 5) * 4;
+  if (OUT_F32) {
+    // float32 result (attention logits, which the reference keeps in float32):
+    // every lane owns 4 consecutive columns per register group
+    float* Cf = reinterpret_cast<float*>(Cvoid) + (int64_t)e * R * N;
+#pragma unroll
+    for (int i = 0; i < Cfg::TM; ++i) {
+#pragma unroll
+      for (int j = 0; j < Cfg::TN; ++j) {
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const int grow = row0 + wm * Cfg::WTM + i * 32 + m_l;
+          const int gcol = col0 + wn * Cfg::WTN + j * 32 + 8 * q + n_l;
+          if (grow < R && gcol < N) {
+            float4 v = make_float4(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1],
+                                   acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+            if (RELU) {
+              v.x = fmaxf(v.x, 0.f); v.y = fmaxf(v.y, 0.f);
+              v.z = fmaxf(v.z, 0.f); v.w = fmaxf(v.w, 0.f);
+            }
+            *reinterpret_cast<float4*>(Cf + (int64_t)grow * N + gcol) = v;
+          }
+        }
+      }
+    }
+    return;
+  }
+  // epilogue: round (and relu), stage the tile in LDS, coalesced stores
+  bf16_t* Cs = reinterpret_cast<bf16_t*>(smem_raw);  // [BM][LDC]
 #pragma unroll
   for (int i = 0; i < Cfg::TM; ++i) {
 #pragma unroll
@@ -1011,6 +1038,30 @@ static int grouped_gemm(const void* A, const void* B, void* C, int E, int R,
       activation_kernel<bf16_t><<<blocks, 256, 0, st>>>((bf16_t*)C, n, act);
     MOE_CHECK_LAUNCH("expert_ffn (activation)");
   }
+  return 0;
+}
+
+// Batched C[e] = A[e] . B[e]^T for the other source files (attention): `dtype`
+// operands, `dtype` result or, with out_f32, a float32 result.
+int batched_gemm_nt(const void* A, const void* B, void* C, int E, int R, int N,
+                    int K, int dtype, bool out_f32, hipStream_t st) {
+  if (dtype == MESH_MOE_F32 || !out_f32)
+    return grouped_gemm(A, B, C, E, R, N, K, MESH_MOE_ACT_LINEAR, dtype, st);
+  MOE_REQUIRE(K % 8 == 0 && N % 8 == 0 &&
+                  (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) % 16 == 0),
+              MESH_MOE_E_UNSUPPORTED,
+              "batched_gemm_nt: float32 result needs K and N multiples of 8 "
+              "(K=%d N=%d) and 16-byte aligned operands", K, N);
+  using Cfg = GemmCfg<128, 128, 64>;
+  const int tiles_m = (R + 127) / 128, tiles_n = (N + 127) / 128;
+  const int64_t blocks = (int64_t)tiles_m * tiles_n * E;
+  MOE_REQUIRE(blocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
+              "batched_gemm_nt: too many tiles (%lld)", (long long)blocks);
+  auto k = grouped_gemm_bf16_kernel<128, 128, 64, false, true>;
+  MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
+  k<<<(unsigned)blocks, 256, Cfg::LDS_BYTES, st>>>(
+      (const bf16_t*)A, (const bf16_t*)B, C, R, N, K, tiles_m, tiles_n);
+  MOE_CHECK_LAUNCH("batched_gemm_nt (mfma, float32 result)");
   return 0;
 }
 

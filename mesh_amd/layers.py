@@ -1,11 +1,12 @@
-"""Weight creation for dense layers, as the Mixture-of-Experts layers use it.
+"""Dense layers as the Mixture-of-Experts layers and the transformer block
+around them use them.
 
-Mirrors the part of mesh_tensorflow/layers.py the MoE path touches:
+Mirrors the part of mesh_tensorflow/layers.py those paths touch:
 get_dense_kernel_weights (layers.py:211-253: variable `<name>/kernel` of shape
-expert_dims + reduced_dims + new_dims) and VarianceScalingInitializer
-(layers.py:310-369: truncated normal with stddev sqrt(scale / fan_in)).
-The matmul itself is not here: the MoE operations consume the variables
-directly.
+expert_dims + reduced_dims + new_dims), VarianceScalingInitializer
+(layers.py:310-369: truncated normal with stddev sqrt(scale / fan_in)), and
+dense / dense_product without bias (layers.py:112-160, :256-295).  The MoE
+operations consume their variables directly.
 """
 
 import torch
@@ -33,6 +34,26 @@ def truncated_normal_initializer(stddev=1.0, seed=None):
                                 b=2 * stddev, generator=gen)
     return t.to(dtype)
   return init
+
+
+def random_normal_initializer(stddev=1.0, seed=None):
+  """Normal(0, stddev), like tf.random_normal_initializer.  Returns
+  f(sizes, dtype, device)."""
+  def init(sizes, dtype, device):
+    gen = None
+    if seed is not None:
+      gen = torch.Generator(device=device)
+      gen.manual_seed(seed)
+    t = torch.empty(sizes, dtype=torch.float32, device=device)
+    t.normal_(0.0, stddev, generator=gen)
+    return t.to(dtype)
+  return init
+
+
+def ones_initializer():
+  """tf.ones_initializer.  Returns f(sizes, dtype, device)."""
+  return lambda sizes, dtype, device: torch.ones(sizes, dtype=dtype,
+                                                 device=device)
 
 
 def random_uniform_initializer(minval, maxval, seed=None):
@@ -98,3 +119,85 @@ def get_dense_kernel_weights(x, new_dims, reduced_dims, expert_dims,
     return mtf.get_variable(x.mesh, "kernel", w_shape,
                             initializer=kernel_initializer,
                             dtype=variable_dtype)
+
+
+class DenseOperation(mtf.Operation):
+  """y = activation(x . kernel) over the last dim of x: the einsum (+ relu) of
+  mtf.layers.dense without bias (mesh_tensorflow/layers.py:112-160) as one
+  operation on the matrix cores.  The kernel is read from the variable's
+  K-contiguous packed copy."""
+
+  def __init__(self, x, kernel, new_dims, activation, name=None):
+    super(DenseOperation, self).__init__([x, kernel], name=name or "dense")
+    self._activation = activation
+    shape = mtf.Shape(x.shape.dims[:-1] + list(new_dims))
+    self._outputs = [mtf.Tensor(self, shape, x.dtype)]
+
+  def lower(self, lowering):
+    from mesh_amd import moe_hip
+    x, kernel = self.inputs
+    mesh_impl = lowering.mesh_impl(self)
+    packed = lowering.variables[kernel.operation].packed(x.dtype)
+    sizes = self.outputs[0].shape.to_integer_list
+    act = self._activation
+
+    def fn(xs):
+      return moe_hip.dense(xs.contiguous(), packed, act).reshape(sizes)
+    lowering.set_tensor_lowering(
+        self.outputs[0], mesh_impl.slicewise(fn, lowering.tensors[x]))
+
+
+def _activation_name(activation):
+  if activation is None or activation == "linear":
+    return None
+  name = activation if isinstance(activation, str) else getattr(
+      activation, "__name__", None)
+  if name != "relu":
+    raise NotImplementedError("dense activation %r is not implemented"
+                              % (activation,))
+  return name
+
+
+def dense(x, new_dims, reduced_dims=None, expert_dims=None, use_bias=True,
+          activation=None, master_dtype=mtf.float32, slice_dtype=mtf.float32,
+          variable_dtype=None, kernel_initializer=None, kernel_weights=None,
+          name=None):
+  """mtf.layers.dense (mesh_tensorflow/layers.py:112-160) for the case the
+  transformer layers use: no bias, no expert dims, the reduced dims being the
+  trailing dims of x; activation None / "linear" / relu.  The variable is
+  `<name>/kernel` with shape reduced_dims + new_dims."""
+  if isinstance(new_dims, mtf.Dimension) or not isinstance(new_dims,
+                                                           (list, tuple)):
+    new_dims = [new_dims]
+  new_dims = [mtf.convert_to_dimension(d) for d in new_dims]
+  if reduced_dims is None:
+    reduced_dims = x.shape.dims[-1:]
+  reduced_dims = list(reduced_dims)
+  if use_bias:
+    raise NotImplementedError("dense with a bias is not implemented")
+  if expert_dims:
+    raise NotImplementedError("dense with expert (ensemble) dims is not "
+                              "implemented; the MoE layers have their own op")
+  if kernel_weights is not None:
+    raise NotImplementedError("dense with external kernel_weights")
+  if len(reduced_dims) != 1 or len(new_dims) != 1:
+    raise NotImplementedError("dense over several reduced or new dims")
+  if x.shape.dims[-1] != reduced_dims[0]:
+    raise NotImplementedError("the reduced dim must be the last dim of x")
+  act = _activation_name(activation)
+  w = get_dense_kernel_weights(x, new_dims, reduced_dims, [],
+                               kernel_initializer, name, variable_dtype,
+                               master_dtype, slice_dtype)
+  return DenseOperation(x, w, new_dims, act, name=name).outputs[0]
+
+
+def dense_product(x, reduced_dims, new_dims, activation_functions=None,
+                  name="dense_product", **kwargs):
+  """mtf.layers.dense_product (mesh_tensorflow/layers.py:256-295) with one
+  factor; gated (list) activations are not implemented."""
+  if isinstance(activation_functions, list):
+    if len(activation_functions) != 1:
+      raise NotImplementedError("gated (list) activations are not implemented")
+    activation_functions = activation_functions[0]
+  return dense(x, new_dims=new_dims, reduced_dims=reduced_dims,
+               activation=activation_functions, name=name, **kwargs)

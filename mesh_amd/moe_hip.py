@@ -114,6 +114,14 @@ _SIGNATURES = {
     "mesh_moe_slot_combine": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
+    "mesh_moe_rms_norm": (ctypes.c_int, [
+        _vp, _vp, _vp, ctypes.c_int64, ctypes.c_int, ctypes.c_double,
+        ctypes.c_int, _vp]),
+    "mesh_moe_self_attention_workspace_bytes": (ctypes.c_size_t, [
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "mesh_moe_self_attention": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
 }
 EXPORTS = sorted(_SIGNATURES)
 
@@ -785,4 +793,51 @@ def slot_combine(y, r, group_size):
         _dev(r.slot_weight, "slot_weight", torch.float32, (g, e, c)),
         out.data_ptr(), g, s, e, c, n, dtype_code(y.dtype), _stream()),
         "slot_combine")
+  return out
+
+
+# ---- the rest of a transformer block ----------------------------------------
+def rms_norm(x, scale, epsilon=1e-6):
+  """x [..., M], scale [M] of x's dtype -> x * rsqrt(mean(x^2) + eps) * scale
+  (sublayer_rms_norm, transformer/transformer.py:493-516)."""
+  lib = load_library()
+  m = x.shape[-1]
+  rows = x.numel() // m
+  out = torch.empty_like(x)
+  with _stage("rms_norm"):
+    _check(lib.mesh_moe_rms_norm(
+        _dev(x, "x"), _dev(scale, "scale", x.dtype, (m,)), out.data_ptr(),
+        rows, m, float(epsilon), dtype_code(x.dtype), _stream()), "rms_norm")
+  return out
+
+
+def dense(x, w_packed, activation=None):
+  """x [..., K] times a packed kernel [1, N, K] -> [..., N]
+  (mtf.layers.dense without bias: one einsum, ops.py / layers.py:112-160)."""
+  k = x.shape[-1]
+  n = w_packed.shape[1]
+  y = expert_linear(x.reshape(1, -1, k), w_packed, activation)
+  return y.reshape(tuple(x.shape[:-1]) + (n,))
+
+
+def self_attention(q, k, v, num_heads, causal):
+  """q, k, v [B, L, H*D] -> [B, L, H*D] (attention.attention with float32
+  logits, transformer/attention.py:27-88)."""
+  lib = load_library()
+  b, l, hd = q.shape
+  if hd % num_heads:
+    raise MoeHipError("q channels %d not divisible by %d heads"
+                      % (hd, num_heads))
+  d = hd // num_heads
+  code = dtype_code(q.dtype)
+  out = torch.empty_like(q)
+  ws_bytes = lib.mesh_moe_self_attention_workspace_bytes(b, l, num_heads, d,
+                                                         code)
+  ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=q.device)
+  with _stage("self_attention"):
+    _check(lib.mesh_moe_self_attention(
+        _dev(q, "q"), _dev(k, "k", q.dtype, (b, l, hd)),
+        _dev(v, "v", q.dtype, (b, l, hd)), out.data_ptr(), b, l, num_heads, d,
+        int(bool(causal)), code, ws.data_ptr(), ws_bytes, _stream()),
+        "self_attention")
   return out

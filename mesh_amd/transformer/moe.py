@@ -22,6 +22,7 @@ import torch
 from mesh_amd import layers as mtf_layers
 from mesh_amd import moe_hip
 from mesh_amd import ops as mtf
+from mesh_amd.transformer import transformer
 
 _OTHER_GATINGS = ()
 
@@ -862,7 +863,7 @@ def transformer_moe_layer_v2(
   return output, loss * hparams.moe_loss_coef
 
 
-class MoE1D(object):
+class MoE1D(transformer.TransformerLayer):
   """Mixture of Experts Layer (transformer layer adapter, moe.py:37-128)."""
 
   def __init__(self,
@@ -948,7 +949,7 @@ class MoE1D(object):
     return y
 
 
-class MoE2D(object):
+class MoE2D(transformer.TransformerLayer):
   """Hierarchical Mixture of Experts Layer (moe.py:131-188).  Unlike the
   reference's constructor this one also sets moe_min_expert_capacity (= 4, the
   MoE1D default), which transformer_moe_layer_v2 reads."""

@@ -1,0 +1,351 @@
+"""The layer-stack part of mesh_tensorflow/transformer/transformer.py that a
+Mixture-of-Experts transformer block needs: TransformerLayer, Context,
+LayerStack with its sublayers (RMS norm, layer call, dropout, residual,
+padding mask), make_layer_stack, and the layer-stack call of Unitransformer.
+
+Not here: embeddings, vocabularies, logits and losses of Unitransformer /
+Bitransformer, decoding ("first_part" / "incremental" modes), dropout while
+training, ensembles, packed sequences (sequence_id tensors).
+"""
+
+from mesh_amd import layers as mtf_layers
+from mesh_amd import ops as mtf
+
+TRAIN = "train"   # tf.estimator.ModeKeys.TRAIN
+EVAL = "eval"     # tf.estimator.ModeKeys.EVAL
+
+
+class _Position(object):
+  """Stands for mtf.range(mesh, length_dim, int32), the value Unitransformer
+  gives read_priority and write_priority of an autoregressive model
+  (transformer.py:1032-1040): position a sees position b iff a >= b."""
+
+  def __repr__(self):
+    return "POSITION"
+
+
+POSITION = _Position()
+
+
+class TransformerLayer(object):
+  """Base class of the layers (transformer.py:56-105): the constructor records
+  hyperparameters, call(context, x) builds the layer and its variables."""
+
+  def call(self, context, x):
+    raise NotImplementedError("Not implemented")
+
+  def set_name(self, name):
+    self._name = name
+
+  @property
+  def name(self):
+    return getattr(self, "_name", None)
+
+
+class Context(object):
+  """What layers need at call time (transformer.py:107-311), for the "train"
+  and "eval" modes.  read_priority / write_priority are None (every position
+  sees every position) or POSITION (autoregressive); sequence_id is None or 1
+  (no padding)."""
+
+  def __init__(self, model, mesh, batch_dims, length_dim, variable_dtype,
+               beam_dim=None, mode=TRAIN, position=None,
+               position_is_default=False, sequence_id=None,
+               subsequence_id=None, states=None, new_states=None, losses=None,
+               initial_position=None, layer_outputs=None, encoder_output=None,
+               encoder_sequence_id=None, constant_states=None,
+               shared_params=None, encoder_layer_outputs=None,
+               write_priority=None, read_priority=None, inputs=None,
+               encoder_inputs=None, num_microbatches=1):
+    if mode not in (TRAIN, EVAL):
+      raise NotImplementedError("mode %r (decoding) is not implemented"
+                                % (mode,))
+    if beam_dim is not None or encoder_output is not None:
+      raise NotImplementedError("beam search / encoder-decoder attention")
+    for pr in (write_priority, read_priority):
+      if pr is not None and pr is not POSITION:
+        raise NotImplementedError(
+            "read/write priorities other than the position")
+    if (write_priority is None) != (read_priority is None):
+      raise ValueError("read_priority and write_priority go together")
+    self.model = model
+    self.mesh = mesh
+    self.batch_dims = batch_dims
+    self.length_dim = length_dim
+    self.variable_dtype = variable_dtype
+    self.beam_dim = beam_dim
+    self.mode = mode
+    self.position = position
+    self.position_is_default = position_is_default
+    self.sequence_id = sequence_id
+    self.subsequence_id = subsequence_id
+    self.states = states
+    self.new_states = new_states
+    self.losses = losses
+    self.initial_position = initial_position
+    self.layer_outputs = layer_outputs if layer_outputs is not None else []
+    self.encoder_output = encoder_output
+    self.encoder_sequence_id = encoder_sequence_id
+    self.constant_states = constant_states
+    self.shared_params = shared_params or {}
+    self.layer_index = 0
+    self.encoder_layer_outputs = encoder_layer_outputs
+    self.cache = {}
+    self.write_priority = write_priority
+    self.read_priority = read_priority
+    self.inputs = inputs
+    self.encoder_inputs = encoder_inputs
+    self.num_microbatches = num_microbatches
+
+  @property
+  def train(self):
+    return self.mode == TRAIN
+
+  @property
+  def activation_dtype(self):
+    return self.variable_dtype.activation_dtype
+
+  @property
+  def nonpadding(self):
+    """Zeros in padding positions and ones elsewhere (transformer.py:297-306)."""
+    if self.sequence_id is None:
+      return None
+    if isinstance(self.sequence_id, int) and self.sequence_id == 1:
+      return 1
+    raise NotImplementedError("sequence_id tensors (packed or padded "
+                              "sequences) are not implemented")
+
+
+class RmsNormOperation(mtf.Operation):
+  """x * rsqrt(mean(square(x)) + epsilon) * scale over the last dim: the five
+  ops of sublayer_rms_norm (transformer.py:493-516) in one kernel."""
+
+  def __init__(self, x, scale, epsilon, name=None):
+    super(RmsNormOperation, self).__init__([x, scale], name=name or "rms_norm")
+    if scale.shape.dims != x.shape.dims[-1:]:
+      raise ValueError("scale %s does not match the last dim of %s"
+                       % (scale.shape, x.shape))
+    self._epsilon = float(epsilon)
+    self._outputs = [mtf.Tensor(self, x.shape, x.dtype)]
+
+  def lower(self, lowering):
+    from mesh_amd import moe_hip
+    mesh_impl = lowering.mesh_impl(self)
+    eps = self._epsilon
+
+    def fn(x, scale):
+      return moe_hip.rms_norm(x.contiguous(), scale.contiguous(), eps)
+    lowering.set_tensor_lowering(
+        self.outputs[0],
+        mesh_impl.slicewise(fn, *[lowering.tensors[t] for t in self.inputs]))
+
+
+def sublayer_call_layer(x, layer_stack, context):
+  """transformer.py:462-466."""
+  x = sublayer_mask_padding(x, layer_stack, context)
+  layer = context.current_layer
+  with mtf.variable_scope(layer.__class__.__name__):
+    return layer.call(context, x)
+
+
+def sublayer_mask_padding(x, layer_stack, context):
+  """Zeroes the padding positions (transformer.py:469-489); without a
+  sequence_id tensor there is nothing to mask."""
+  del layer_stack
+  if isinstance(context.sequence_id, mtf.Tensor):
+    raise NotImplementedError("sequence_id tensors are not implemented")
+  return x
+
+
+def sublayer_rms_norm(x, layer_stack, context, epsilon=1e-6, name="rms_norm"):
+  """RMS normalisation with a learned scale `<name>/scale` [d_model]
+  (transformer.py:493-516)."""
+  del layer_stack
+  model_dim = context.model.model_dim
+  if context.model.ensemble_dims:
+    raise NotImplementedError("ensembles are not implemented")
+  with mtf.variable_scope(name):
+    scale = mtf.get_variable(context.mesh, "scale", mtf.Shape([model_dim]),
+                             initializer=mtf_layers.ones_initializer(),
+                             dtype=context.variable_dtype)
+  return RmsNormOperation(x, scale, epsilon, name=name).outputs[0]
+
+
+def sublayer_legacy_rms_norm(x, layer_stack, context):
+  """transformer.py:519-522."""
+  return sublayer_rms_norm(x, layer_stack, context, name="layer_norm")
+
+
+def sublayer_legacy_final_rms_norm(x, layer_stack, context):
+  """transformer.py:525-528."""
+  return sublayer_rms_norm(x, layer_stack, context, name="final_layer_norm")
+
+
+def sublayer_residual(x, layer_stack, context):
+  """transformer.py:584-587."""
+  del layer_stack
+  return x + context.current_layer_input
+
+
+def sublayer_dropout(x, layer_stack, context, dropout_rate=0.0):
+  """transformer.py:590-599; dropout while training draws random numbers and
+  is not implemented."""
+  del layer_stack
+  if context.train and dropout_rate > 0:
+    raise NotImplementedError("dropout while training is not implemented")
+  return x
+
+
+def sublayer_legacy_dropout(x, layer_stack, context):
+  """transformer.py:627-636."""
+  return sublayer_dropout(x, layer_stack, context,
+                          dropout_rate=layer_stack.dropout_rate)
+
+
+class LayerStack(TransformerLayer):
+  """A stack of layers with residual connections and norms
+  (transformer.py:314-457).  The default sublayers are those of the
+  reference's defaults.gin."""
+
+  def __init__(self, layers, sublayers_initial=None, sublayers_per_layer=None,
+               sublayers_final=None, dropout_rate=None, norm_epsilon=None,
+               recompute_grads=False):
+    if recompute_grads:
+      raise NotImplementedError("recompute_grads is not implemented")
+    self._layers = layers
+    self._sublayers_initial = sublayers_initial
+    self._sublayers_per_layer = sublayers_per_layer
+    self._sublayers_final = sublayers_final
+    if (dropout_rate is not None) != (norm_epsilon is not None):
+      raise ValueError(
+          "LayerStack.dropout_rate and LayerStack.norm_epsilon should either "
+          "be both not None (legacy mode) or both None (normal mode)")
+    if dropout_rate is not None:
+      # legacy mode, for old checkpoints' variable names (transformer.py:383-406)
+      self.dropout_rate = dropout_rate
+      self.norm_epsilon = norm_epsilon
+      self._sublayers_initial = [sublayer_legacy_dropout]
+      self._sublayers_per_layer = [sublayer_legacy_rms_norm,
+                                   sublayer_call_layer,
+                                   sublayer_legacy_dropout, sublayer_residual]
+      self._sublayers_final = [sublayer_legacy_final_rms_norm,
+                               sublayer_legacy_dropout]
+    else:
+      if self._sublayers_initial is None:
+        self._sublayers_initial = [sublayer_dropout]
+      if self._sublayers_per_layer is None:
+        self._sublayers_per_layer = [sublayer_rms_norm, sublayer_call_layer,
+                                     sublayer_dropout, sublayer_residual]
+      if self._sublayers_final is None:
+        self._sublayers_final = [sublayer_rms_norm, sublayer_dropout]
+
+  def call(self, context, x):
+    """transformer.py:408-428."""
+    x = self._call_sublayers(self._sublayers_initial, x, context)
+    context.layer_outputs.append(x)
+    for lnum, layer in enumerate(self._layers):
+      with mtf.variable_scope(layer.name or ""):
+        x = self._layer_fn(x, layer, context)
+      if lnum != len(self._layers) - 1:
+        context.layer_outputs.append(x)
+      context.layer_index += 1
+    x = self._call_sublayers(self._sublayers_final, x, context)
+    x = sublayer_mask_padding(x, self, context)
+    context.layer_outputs.append(x)
+    return x
+
+  def _call_sublayers(self, sublayers, x, context):
+    for s in sublayers:
+      x = s(x, self, context)
+    return x
+
+  def _layer_fn(self, x, layer, context):
+    context.current_layer = layer
+    context.current_layer_input = x
+    y = self._call_sublayers(self._sublayers_per_layer, x, context)
+    if y.shape != x.shape:
+      raise ValueError("Layer %s returned misshaped output x=%s y=%s"
+                       % (layer.__class__.__name__, x, y))
+    return y
+
+  @property
+  def num_layers(self):
+    return len(self.layers)
+
+  @property
+  def layers(self):
+    return self._layers
+
+
+def make_layer_stack(layers, num_layers=6, block_scope=True,
+                     layer_stack_cls=LayerStack):
+  """transformer.py:1876-1948: `layers` lists, per block, classes or
+  (class, name, kwargs) tuples; the names are block_%03d/layer_%03d or
+  layer_%03d."""
+  layer_stack = []
+  for block in range(num_layers):
+    for n, cls in enumerate(layers):
+      name = None
+      kwargs = {}
+      if isinstance(cls, (list, tuple)):
+        for x in cls:
+          if isinstance(x, str):
+            name = x
+          elif isinstance(x, dict):
+            kwargs = x
+          else:
+            cls = x
+      if block_scope:
+        name = "block_{:03d}/{}".format(block, name or "layer_{:03d}".format(n))
+      else:
+        name = name or "layer_{:03d}".format(len(layer_stack))
+      layer = cls(**kwargs)
+      layer.set_name(name)
+      layer_stack.append(layer)
+  return layer_stack_cls(layer_stack)
+
+
+class Unitransformer(object):
+  """The layer-stack call of the reference's Unitransformer
+  (transformer.py:696-1075) on activations that are already embedded: model
+  dims, the Context, and LayerStack.call under the model's name scope."""
+
+  def __init__(self, layer_stack, d_model=1024, name="transformer",
+               autoregressive=False, layout=None, mesh_shape=None,
+               ensemble=None):
+    if ensemble:
+      raise NotImplementedError("ensembles are not implemented")
+    self.layer_stack = layer_stack
+    self.model_dim = mtf.Dimension("d_model", d_model)
+    self.name = name
+    self.autoregressive = autoregressive
+    self.layout = layout
+    self.mesh_shape = mesh_shape
+    self.ensemble_dim = None
+
+  @property
+  def ensemble_dims(self):
+    return []
+
+  @property
+  def fully_autoregressive(self):
+    return self.autoregressive
+
+  def call_layers(self, x, variable_dtype, mode=EVAL, num_microbatches=1,
+                  sequence_id=None):
+    """x [batch dims..., length, d_model] -> (y, losses).  The Context is the
+    one _call_internal builds (transformer.py:1032-1062): read and write
+    priorities are the position for an autoregressive model."""
+    if x.shape.dims[-1] != self.model_dim:
+      raise ValueError("x %s does not end in %s" % (x.shape, self.model_dim))
+    priority = POSITION if self.autoregressive else None
+    losses = []
+    context = Context(
+        model=self, mesh=x.mesh, batch_dims=x.shape.dims[:-2],
+        length_dim=x.shape.dims[-2], variable_dtype=variable_dtype, mode=mode,
+        position_is_default=True, sequence_id=sequence_id, losses=losses,
+        write_priority=priority, read_priority=priority,
+        num_microbatches=num_microbatches)
+    with mtf.variable_scope(self.name):
+      y = self.layer_stack.call(context, x)
+    return y, losses

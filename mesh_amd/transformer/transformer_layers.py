@@ -1,0 +1,97 @@
+"""DenseReluDense and SelfAttention as mesh_tensorflow/transformer/
+transformer_layers.py defines them, for training / evaluation on one device.
+"""
+
+from mesh_amd import layers as mtf_layers
+from mesh_amd import ops as mtf
+from mesh_amd.transformer import attention
+from mesh_amd.transformer import transformer
+
+
+class DenseReluDense(transformer.TransformerLayer):
+  """Two dense layers with an activation on the hidden layer
+  (transformer_layers.py:36-76): variables wi/kernel [d_model, d_ff] and
+  wo/kernel [d_ff, d_model]."""
+
+  def __init__(self, hidden_size=4096, dropout_rate=0.0, activation="relu",
+               use_bias=False):
+    self.hidden_size = hidden_size
+    self.dropout_rate = dropout_rate
+    self.activation = activation
+    self.use_bias = use_bias
+
+  def call(self, context, x, losses=None):
+    del losses
+    io_channels = x.shape.dims[-1]
+    hidden_channels = mtf.Dimension("d_ff", self.hidden_size)
+    if context.model.ensemble_dims:
+      raise NotImplementedError("ensembles are not implemented")
+    h = mtf_layers.dense_product(
+        x, reduced_dims=x.shape.dims[-1:], new_dims=hidden_channels,
+        activation_functions=self.activation, use_bias=self.use_bias,
+        variable_dtype=context.variable_dtype, name="wi")
+    if context.train and self.dropout_rate != 0.0:
+      raise NotImplementedError("dropout while training is not implemented")
+    return mtf_layers.dense(
+        h, io_channels, use_bias=self.use_bias, activation=None,
+        variable_dtype=context.variable_dtype, reduced_dims=h.shape.dims[-1:],
+        name="wo")
+
+
+class SelfAttention(transformer.TransformerLayer):
+  """Multi-head self-attention (transformer_layers.py:151-357) with the default
+  parameters: no relative position bias, separate k and v, combined dims.
+  Visibility comes from the context: read/write priorities (autoregressive
+  models) or none."""
+
+  def __init__(self, num_heads=8, num_memory_heads=0, key_value_size=128,
+               shared_kv=False, dropout_rate=0.0, attention_kwargs=None,
+               relative_attention_type=None,
+               relative_attention_num_buckets=32, attention_func=None,
+               combine_dims=True, keep_query_heads_dims=False,
+               fold_scaling_into_initializer=True):
+    if (num_memory_heads or shared_kv or attention_kwargs or
+        relative_attention_type is not None or attention_func is not None or
+        not combine_dims or keep_query_heads_dims):
+      raise NotImplementedError(
+          "only the default SelfAttention options are implemented")
+    self.num_heads = num_heads
+    self.key_value_size = key_value_size
+    self.dropout_rate = dropout_rate
+    self.relative_attention_num_buckets = relative_attention_num_buckets
+    self.fold_scaling_into_initializer = fold_scaling_into_initializer
+
+  @property
+  def kv_dim(self):
+    return mtf.Dimension("d_kv", self.key_value_size)
+
+  def make_params(self, context):
+    """transformer_layers.py:79-149 (attention_params)."""
+    heads = ([mtf.Dimension("heads", self.num_heads)]
+             if self.num_heads > 1 else None)
+    return attention.AttentionParams(
+        context.mesh, query_input_dim=context.model.model_dim,
+        memory_input_dim=context.model.model_dim,
+        output_dim=context.model.model_dim, key_dim=self.kv_dim,
+        value_dim=self.kv_dim, query_heads_dims=heads,
+        memory_heads_dims=heads, variable_dtype=context.variable_dtype,
+        ensemble_dim=context.model.ensemble_dim,
+        fold_scaling_into_initializer=self.fold_scaling_into_initializer)
+
+  def call(self, context, x, losses=None):
+    """transformer_layers.py:223-271 for the train / eval modes."""
+    del losses
+    if context.train and self.dropout_rate != 0.0:
+      raise NotImplementedError("dropout while training is not implemented")
+    if isinstance(context.sequence_id, mtf.Tensor) or isinstance(
+        context.subsequence_id, mtf.Tensor):
+      raise NotImplementedError("sequence_id tensors are not implemented")
+    params = self.make_params(context)
+    q = params.compute_q(x)
+    k = params.compute_k(x)
+    v = params.compute_v(x)
+    # read_priority >= write_priority (transformer_layers.py:289-296)
+    causal = context.read_priority is transformer.POSITION
+    o = attention.SelfAttentionOperation(q, k, v, params.num_heads,
+                                         causal).outputs[0]
+    return params.compute_output(o, output_shape=x.shape)

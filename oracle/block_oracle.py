@@ -1,0 +1,133 @@
+"""CPU restatement of the transformer block around the Mixture-of-Experts
+layer: RMS norm, dense layers, multi-head self-attention and the LayerStack
+that chains them with residual connections.
+
+TEST INFRASTRUCTURE ONLY -- never imported by the product package.
+
+NumPy float32 arithmetic with one rounding to the activation dtype per
+reference op (float32 accumulation inside reductions and matmuls), as in
+moe_oracle.  What pins each function (tests/test_block_oracle.py):
+
+  rms_norm         float64 closed form; unit scale and constant rows give
+                   x / |x| exactly representable cases
+  dense            float64 matmul
+  self_attention   float64 per-head softmax(q k^T + mask) v; causality (an
+                   output does not change when later positions change); zero
+                   queries give the running mean of the values
+  layer_stack      zero output kernels reduce the stack to its final norm;
+                   one layer by hand
+
+PARITY UNPINNED against TensorFlow itself: the order of float32 accumulation
+inside TF's reductions and matmuls, and for bfloat16 whether TF's reduce_sum
+rounds partial sums (here: one rounding of a float32 sum).
+
+Citations are to files under the reference tree (mesh_tensorflow/...).
+"""
+
+import numpy as np
+
+from oracle import moe_oracle as O
+
+F32 = np.float32
+
+
+def _r(a, act_dtype):
+  return O.cast_act(np.asarray(a, F32), act_dtype)
+
+
+def rms_norm(x, scale, act_dtype="float32", epsilon=1e-6):
+  """sublayer_rms_norm (transformer/transformer.py:493-516):
+  variance = reduce_mean(square(x), d_model); x * rsqrt(variance + eps) * scale.
+  reduce_mean is reduce_sum times the Python float 1/M (ops.py:4807-4808);
+  Python scalars enter an op rounded to the tensor dtype."""
+  x = _r(x, act_dtype)
+  scale = _r(scale, act_dtype)
+  m = x.shape[-1]
+  sq = _r(x * x, act_dtype)                                      # square
+  total = _r(O.seq_sum(sq, axis=-1), act_dtype)                  # reduce_sum
+  mean = _r(total * _r(F32(1.0 / m), act_dtype), act_dtype)      # * (1 / M)
+  var = _r(mean + _r(F32(epsilon), act_dtype), act_dtype)        # + epsilon
+  r = _r(F32(1.0) / np.sqrt(var, dtype=F32), act_dtype)          # rsqrt
+  y = _r(x * r[..., None], act_dtype)                            # x * rsqrt
+  return _r(y * scale, act_dtype)                                # * scale
+
+
+def dense(x, w, act_dtype="float32", activation=None):
+  """mtf.layers.dense without bias (layers.py:112-160): einsum over the last
+  dim of x with float32 accumulation, result in the activation dtype, then
+  the activation as its own op."""
+  y = _r(np.matmul(_r(x, act_dtype), _r(w, act_dtype)), act_dtype)
+  if activation == "relu":
+    y = np.maximum(y, F32(0.0))
+  elif activation not in (None, "linear"):
+    raise ValueError("activation %r" % (activation,))
+  return y
+
+
+def self_attention(x, wq, wk, wv, wo, num_heads, causal, act_dtype="float32"):
+  """SelfAttention.call for the train / eval modes with the default options
+  (transformer/transformer_layers.py:223-271) around attention.attention with
+  float32 logits (transformer/attention.py:27-88).
+
+  x [B, L, d_model]; wq, wk, wv [d_model, H*D]; wo [H*D, d_model].  q, k, v are
+  activation-dtype tensors; logits = q . k in float32 (+ -1e9 where the key is
+  not visible, attention.py:830-842; the bias is cast to the logits' dtype,
+  :78-79); weights = mtf.softmax(logits) in float32, cast to the activation
+  dtype; outputs = weights . v.  No 1/sqrt(d_kv) factor: it is folded into the
+  initialiser of wq (attention.py:436-439).
+  """
+  x = _r(x, act_dtype)
+  b, l, _ = x.shape
+  hd = wq.shape[1]
+  d = hd // num_heads
+  q = dense(x, wq, act_dtype).reshape(b, l, num_heads, d)
+  k = dense(x, wk, act_dtype).reshape(b, l, num_heads, d)
+  v = dense(x, wv, act_dtype).reshape(b, l, num_heads, d)
+  logits = np.einsum("blhd,bmhd->bhlm", q, k).astype(F32)        # float32
+  if causal:
+    pos = np.arange(l)
+    hidden = (pos[None, :] > pos[:, None]).astype(F32)           # key > query
+    logits = logits + hidden * F32(-1e9)
+  weights = _r(O.softmax(logits), act_dtype)                     # cast to v's
+  o = _r(np.einsum("bhlm,bmhd->blhd", weights, v), act_dtype)
+  return dense(o.reshape(b, l, hd), wo, act_dtype)
+
+
+def dense_relu_dense(x, wi, wo, act_dtype="float32"):
+  """DenseReluDense.call (transformer/transformer_layers.py:55-76)."""
+  return dense(dense(x, wi, act_dtype, "relu"), wo, act_dtype)
+
+
+def layer_stack(x, layers, final_scale, act_dtype="float32",
+                autoregressive=False, train=False):
+  """LayerStack.call with the default sublayers (transformer/transformer.py:
+  408-428 and the defaults quoted at :346-358): per layer
+  x + layer(rms_norm(x)); a final rms_norm.  Dropout rates are 0.
+
+  layers: list of dicts with "kind" in {"attention", "dense_relu_dense",
+  "moe"}, "scale" (the layer's rms_norm scale) and the layer's weights:
+    attention: wq, wk, wv, wo, num_heads
+    dense_relu_dense: wi, wo
+    moe: w_gate, wi, wo, hparams (an O.HParams); optional num_microbatches
+  Returns (y, losses) with one loss per MoE layer.
+  """
+  x = _r(x, act_dtype)
+  losses = []
+  for layer in layers:
+    h = rms_norm(x, layer["scale"], act_dtype)
+    kind = layer["kind"]
+    if kind == "attention":
+      y = self_attention(h, layer["wq"], layer["wk"], layer["wv"], layer["wo"],
+                         layer["num_heads"], autoregressive, act_dtype)
+    elif kind == "dense_relu_dense":
+      y = dense_relu_dense(h, layer["wi"], layer["wo"], act_dtype)
+    elif kind == "moe":
+      y, loss, _ = O.moe_layer_v1(
+          h, layer["w_gate"], layer["wi"], layer["wo"], layer["hparams"],
+          train, act_dtype, num_microbatches=layer.get("num_microbatches"),
+          dense=False)
+      losses.append(loss)
+    else:
+      raise ValueError("layer kind %r" % (kind,))
+    x = _r(y + x, act_dtype)                                     # residual
+  return rms_norm(x, final_scale, act_dtype), losses

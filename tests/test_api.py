@@ -369,3 +369,106 @@ def test_gradients_builds_the_backward_operation():
   grads3 = mtf.gradients([y3, l3], [x3] + v3)
   assert [g.shape for g in grads3] == [t.shape for t in [x3] + v3]
   assert any(isinstance(o, moe.MoEV2GradOperation) for o in g3.operations)
+
+
+# ---- the transformer block around the layer -------------------------------------
+def _lm_moe_stack():
+  from mesh_amd.transformer import transformer, transformer_layers
+  return transformer.make_layer_stack(
+      [transformer_layers.SelfAttention,
+       (moe.MoE1D, dict(num_experts=4, hidden_size=64, group_size=16,
+                        second_policy_train="all", second_policy_eval="all")),
+       (transformer_layers.SelfAttention, dict(num_heads=4, key_value_size=8)),
+       (transformer_layers.DenseReluDense, dict(hidden_size=64))],
+      num_layers=1, block_scope=False)
+
+
+def test_layer_stack_graph_names_and_shapes():
+  """The block of transformer/gin/models/lm_moe.gin:11-16: variable names and
+  shapes are the reference's (rms_norm/scale per layer and at the end,
+  SelfAttention/{q,k,v,o} with heads and d_kv combined, attention.py:410-414)."""
+  from mesh_amd.transformer import transformer
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  dims = [mtf.Dimension("batch", 2), mtf.Dimension("length", 16),
+          mtf.Dimension("d_model", 32)]
+  x = mtf.import_tf_tensor(mesh, torch.zeros(2, 16, 32), mtf.Shape(dims))
+  model = transformer.Unitransformer(_lm_moe_stack(), d_model=32,
+                                     name="decoder", autoregressive=True)
+  y, losses = model.call_layers(x, mtf.VariableDType(torch.float32))
+  assert y.shape == x.shape and len(losses) == 1
+  got = {v.name: v.shape.to_string for v in graph.all_variables}
+  assert got == {
+      "decoder/layer_000/rms_norm/scale": "Shape[d_model=32]",
+      "decoder/layer_000/SelfAttention/q": "Shape[d_model=32, heads=1024]",
+      "decoder/layer_000/SelfAttention/k": "Shape[d_model=32, heads=1024]",
+      "decoder/layer_000/SelfAttention/v": "Shape[d_model=32, heads=1024]",
+      "decoder/layer_000/SelfAttention/o": "Shape[heads=1024, d_model=32]",
+      "decoder/layer_001/rms_norm/scale": "Shape[d_model=32]",
+      "decoder/layer_001/MoE1D/top_2_gating/kernel":
+          "Shape[d_model=32, expert_unsplit=4]",
+      "decoder/layer_001/MoE1D/wi/kernel":
+          "Shape[experts=4, d_model=32, expert_hidden=64]",
+      "decoder/layer_001/MoE1D/wo/kernel":
+          "Shape[experts=4, expert_hidden=64, d_model=32]",
+      "decoder/layer_002/rms_norm/scale": "Shape[d_model=32]",
+      "decoder/layer_002/SelfAttention/q": "Shape[d_model=32, heads=32]",
+      "decoder/layer_002/SelfAttention/k": "Shape[d_model=32, heads=32]",
+      "decoder/layer_002/SelfAttention/v": "Shape[d_model=32, heads=32]",
+      "decoder/layer_002/SelfAttention/o": "Shape[heads=32, d_model=32]",
+      "decoder/layer_003/rms_norm/scale": "Shape[d_model=32]",
+      "decoder/layer_003/DenseReluDense/wi/kernel": "Shape[d_model=32, d_ff=64]",
+      "decoder/layer_003/DenseReluDense/wo/kernel": "Shape[d_ff=64, d_model=32]",
+      "decoder/rms_norm/scale": "Shape[d_model=32]"}
+
+
+def test_layer_stack_names_with_block_scope_and_legacy_mode():
+  from mesh_amd.transformer import transformer, transformer_layers
+  stack = transformer.make_layer_stack(
+      [transformer_layers.SelfAttention,
+       (transformer_layers.DenseReluDense, "feedforward", {"hidden_size": 8})],
+      num_layers=2)
+  assert [l.name for l in stack.layers] == [
+      "block_000/layer_000", "block_000/feedforward",
+      "block_001/layer_000", "block_001/feedforward"]
+  legacy = transformer.LayerStack(stack.layers, dropout_rate=0.0,
+                                  norm_epsilon=1e-6)
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  dims = [mtf.Dimension("batch", 1), mtf.Dimension("length", 8),
+          mtf.Dimension("d_model", 16)]
+  x = mtf.import_tf_tensor(mesh, torch.zeros(1, 8, 16), mtf.Shape(dims))
+  model = transformer.Unitransformer(legacy, d_model=16, name="encoder")
+  model.call_layers(x, mtf.VariableDType(torch.float32))
+  names = [v.name for v in graph.all_variables]
+  assert "encoder/block_000/layer_000/layer_norm/scale" in names
+  assert "encoder/final_layer_norm/scale" in names
+  with pytest.raises(ValueError, match="legacy mode"):
+    transformer.LayerStack(stack.layers, dropout_rate=0.1)
+
+
+def test_block_rejections():
+  from mesh_amd.transformer import transformer, transformer_layers
+  with pytest.raises(NotImplementedError):
+    transformer_layers.SelfAttention(relative_attention_type="bias")
+  with pytest.raises(NotImplementedError):
+    transformer_layers.SelfAttention(shared_kv=True)
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  dims = [mtf.Dimension("batch", 1), mtf.Dimension("length", 8),
+          mtf.Dimension("d_model", 16)]
+  x = mtf.import_tf_tensor(mesh, torch.zeros(1, 8, 16), mtf.Shape(dims))
+  vdt = mtf.VariableDType(torch.float32)
+  model = transformer.Unitransformer(None, d_model=16)
+  with pytest.raises(NotImplementedError, match="decoding"):
+    transformer.Context(model, mesh, dims[:1], dims[1], vdt, mode="incremental")
+  stack = transformer.make_layer_stack(
+      [(transformer_layers.DenseReluDense,
+        dict(hidden_size=8, dropout_rate=0.1))], num_layers=1)
+  model = transformer.Unitransformer(stack, d_model=16)
+  with pytest.raises(NotImplementedError, match="dropout"):
+    model.call_layers(x, vdt, mode="train")
+  ctx = transformer.Context(model, mesh, dims[:1], dims[1], vdt, sequence_id=1)
+  assert ctx.nonpadding == 1 and not isinstance(ctx.nonpadding, mtf.Tensor)
+  with pytest.raises(ValueError, match="does not end in"):
+    model.call_layers(mtf.reshape(x, [dims[0], dims[2], dims[1]]), vdt)

@@ -1,0 +1,162 @@
+"""Pins of oracle/block_oracle.py: float64 closed forms, invariants and
+hand-worked cases for the transformer block around the MoE layer."""
+
+import numpy as np
+import pytest
+import scipy.special
+
+from oracle import block_oracle as B
+from oracle import moe_oracle as O
+
+
+def test_rms_norm_against_float64():
+  rng = np.random.default_rng(1)
+  x = rng.standard_normal((3, 7, 48)).astype(np.float32) * 3
+  scale = rng.standard_normal(48).astype(np.float32)
+  x64 = x.astype(np.float64)
+  want = x64 / np.sqrt((x64 ** 2).mean(-1, keepdims=True) + 1e-6) * scale
+  np.testing.assert_allclose(B.rms_norm(x, scale), want, rtol=2e-6, atol=1e-7)
+  # a row of equal entries c normalises to sign(c) (eps aside)
+  const = np.full((1, 16), -4.0, np.float32)
+  np.testing.assert_allclose(B.rms_norm(const, np.ones(16, np.float32)),
+                             -np.ones((1, 16)), rtol=1e-6)
+  # scale-invariance: rms_norm(a x) = rms_norm(x) for a > 0 (eps negligible)
+  np.testing.assert_allclose(B.rms_norm(8 * x, scale), B.rms_norm(x, scale),
+                             rtol=1e-5, atol=1e-6)
+
+
+def test_rms_norm_bf16_rounds_every_op():
+  rng = np.random.default_rng(2)
+  x = O.round_bf16(rng.standard_normal((5, 64)).astype(np.float32))
+  scale = O.round_bf16(1 + 0.1 * rng.standard_normal(64).astype(np.float32))
+  y = B.rms_norm(x, scale, "bfloat16")
+  np.testing.assert_array_equal(y, O.round_bf16(y))
+  x64 = x.astype(np.float64)
+  want = x64 / np.sqrt((x64 ** 2).mean(-1, keepdims=True) + 1e-6) * scale
+  # six bf16 roundings in a row: within a few bf16 ulps of the exact value
+  np.testing.assert_allclose(y, want, rtol=3e-2, atol=1e-3)
+
+
+def test_dense_against_float64():
+  rng = np.random.default_rng(3)
+  x = rng.standard_normal((2, 9, 24)).astype(np.float32)
+  w = rng.standard_normal((24, 40)).astype(np.float32)
+  want = x.astype(np.float64) @ w.astype(np.float64)
+  np.testing.assert_allclose(B.dense(x, w), want, rtol=1e-5, atol=1e-5)
+  np.testing.assert_allclose(B.dense(x, w, activation="relu"),
+                             np.maximum(want, 0), rtol=1e-5, atol=1e-5)
+
+
+def _attention64(x, wq, wk, wv, wo, heads, causal):
+  b, l, _ = x.shape
+  d = wq.shape[1] // heads
+  x, wq, wk, wv, wo = (a.astype(np.float64) for a in (x, wq, wk, wv, wo))
+  out = np.zeros((b, l, wq.shape[1]))
+  for bi in range(b):
+    for h in range(heads):
+      sl = slice(h * d, (h + 1) * d)
+      q, k, v = x[bi] @ wq[:, sl], x[bi] @ wk[:, sl], x[bi] @ wv[:, sl]
+      s = q @ k.T
+      if causal:
+        s = np.where(np.tril(np.ones((l, l), bool)), s, -np.inf)
+      out[bi, :, sl] = scipy.special.softmax(s, axis=-1) @ v
+  return out @ wo
+
+
+@pytest.mark.parametrize("causal", [False, True])
+def test_self_attention_against_float64(causal):
+  rng = np.random.default_rng(4)
+  b, l, m, heads, d = 2, 12, 16, 3, 4
+  x = rng.standard_normal((b, l, m)).astype(np.float32)
+  wq, wk, wv = (rng.standard_normal((m, heads * d)).astype(np.float32) / 3
+                for _ in range(3))
+  wo = rng.standard_normal((heads * d, m)).astype(np.float32) / 3
+  got = B.self_attention(x, wq, wk, wv, wo, heads, causal)
+  np.testing.assert_allclose(got, _attention64(x, wq, wk, wv, wo, heads, causal),
+                             rtol=2e-5, atol=2e-5)
+
+
+def test_self_attention_causality_and_uniform_case():
+  rng = np.random.default_rng(5)
+  b, l, m, heads, d = 1, 10, 8, 2, 4
+  x = rng.standard_normal((b, l, m)).astype(np.float32)
+  wq, wk, wv = (rng.standard_normal((m, heads * d)).astype(np.float32)
+                for _ in range(3))
+  wo = np.eye(heads * d, m, dtype=np.float32)
+  base = B.self_attention(x, wq, wk, wv, wo, heads, True)
+  x2 = x.copy()
+  x2[:, 6:] = rng.standard_normal((b, 4, m))
+  moved = B.self_attention(x2, wq, wk, wv, wo, heads, True)
+  np.testing.assert_array_equal(base[:, :6], moved[:, :6])     # the past is fixed
+  assert np.abs(base[:, 6:] - moved[:, 6:]).max() > 1e-3
+  full = B.self_attention(x2, wq, wk, wv, wo, heads, False)
+  assert np.abs(full[:, :6] - base[:, :6]).max() > 1e-3         # not so unmasked
+  # zero queries: uniform weights, output t = mean of the values 0..t
+  out = B.self_attention(x, np.zeros_like(wq), wk, wv, wo, heads, True)
+  v = x[0].astype(np.float64) @ wv.astype(np.float64)
+  want = np.cumsum(v, axis=0) / np.arange(1, l + 1)[:, None]
+  np.testing.assert_allclose(out[0], want, rtol=1e-5, atol=1e-5)
+
+
+def test_self_attention_bf16_close_to_float32():
+  rng = np.random.default_rng(6)
+  b, l, m, heads, d = 2, 16, 32, 2, 8
+  x = O.round_bf16(rng.standard_normal((b, l, m)).astype(np.float32))
+  ws = [O.round_bf16(rng.standard_normal(s).astype(np.float32) / 5)
+        for s in ((m, heads * d),) * 3 + ((heads * d, m),)]
+  a = B.self_attention(x, *ws, heads, True, "bfloat16")
+  np.testing.assert_array_equal(a, O.round_bf16(a))
+  f = B.self_attention(x, *ws, heads, True, "float32")
+  np.testing.assert_allclose(a, f, rtol=5e-2, atol=5e-2)
+
+
+def _stack_weights(rng, m, e, hdim, heads, d):
+  def n(*shape):
+    return (rng.standard_normal(shape) / np.sqrt(shape[-2])).astype(np.float32)
+  att = dict(kind="attention", num_heads=heads, wq=n(m, heads * d),
+             wk=n(m, heads * d), wv=n(m, heads * d), wo=n(heads * d, m),
+             scale=(1 + 0.1 * rng.standard_normal(m)).astype(np.float32))
+  hp = O.default_hparams(moe_num_experts=e, moe_hidden_size=hdim,
+                         moe_group_size=16, moe_second_policy_eval="all",
+                         moe_capacity_factor_eval=2.0)
+  moe = dict(kind="moe", w_gate=n(m, e), wi=n(e, m, hdim), wo=n(e, hdim, m),
+             hparams=hp,
+             scale=(1 + 0.1 * rng.standard_normal(m)).astype(np.float32))
+  ffn = dict(kind="dense_relu_dense", wi=n(m, hdim), wo=n(hdim, m),
+             scale=(1 + 0.1 * rng.standard_normal(m)).astype(np.float32))
+  return [att, moe, dict(att), ffn]
+
+
+def test_layer_stack_by_hand_and_zero_kernels():
+  rng = np.random.default_rng(7)
+  b, l, m = 2, 16, 24
+  layers = _stack_weights(rng, m, 4, 32, 2, 8)
+  final = (1 + 0.1 * rng.standard_normal(m)).astype(np.float32)
+  x = rng.standard_normal((b, l, m)).astype(np.float32)
+  y, losses = B.layer_stack(x, layers, final, autoregressive=True)
+  assert len(losses) == 1 and y.shape == x.shape
+  # by hand: chain the pieces
+  h = x
+  a = layers[0]
+  h = h + B.self_attention(B.rms_norm(h, a["scale"]), a["wq"], a["wk"], a["wv"],
+                           a["wo"], 2, True)
+  mo = layers[1]
+  out, loss, _ = O.moe_layer_v1(B.rms_norm(h, mo["scale"]), mo["w_gate"],
+                                mo["wi"], mo["wo"], mo["hparams"], False,
+                                dense=False)
+  h = h + out
+  a = layers[2]
+  h = h + B.self_attention(B.rms_norm(h, a["scale"]), a["wq"], a["wk"], a["wv"],
+                           a["wo"], 2, True)
+  f = layers[3]
+  h = h + B.dense_relu_dense(B.rms_norm(h, f["scale"]), f["wi"], f["wo"])
+  np.testing.assert_allclose(y, B.rms_norm(h, final), rtol=1e-6, atol=1e-6)
+  assert losses[0] == loss
+  # all output kernels zero: every layer adds 0 and the stack is its final norm
+  zeroed = []
+  for layer in layers:
+    z = dict(layer)
+    z["wo"] = np.zeros_like(layer["wo"])
+    zeroed.append(z)
+  y0, _ = B.layer_stack(x, zeroed, final)
+  np.testing.assert_array_equal(y0, B.rms_norm(x, final))
