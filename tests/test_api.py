@@ -472,3 +472,29 @@ def test_block_rejections():
   assert ctx.nonpadding == 1 and not isinstance(ctx.nonpadding, mtf.Tensor)
   with pytest.raises(ValueError, match="does not end in"):
     model.call_layers(mtf.reshape(x, [dims[0], dims[2], dims[1]]), vdt)
+
+
+# ---- checkpoints ----------------------------------------------------------------
+def test_plan_restore_selection_logic():
+  """utils.py:948-972: the filter applies to checkpoint names, the mapping to
+  graph names, and only variables that pass should_load are candidates."""
+  from mesh_amd import checkpoint
+  graph = ["decoder/layer_001/MoE1D/wi/kernel", "decoder/layer_001/MoE1D/wo/kernel",
+           "decoder/rms_norm/scale", "decoder/extra/bias"]
+  ckpt = ["decoder/layer_001/MoE1D/wi/kernel", "decoder/layer_001/MoE1D/wo/kernel",
+          "decoder/rms_norm/scale", "decoder/rms_norm/scale_slot_v", "global_step"]
+  r = checkpoint.plan_restore(graph, ckpt)
+  assert r.restored == {n: n for n in graph[:3]}
+  assert r.in_checkpoint_not_in_graph == ["decoder/rms_norm/scale_slot_v",
+                                          "global_step"]
+  assert r.in_graph_not_in_checkpoint == ["decoder/extra/bias"]
+  r = checkpoint.plan_restore(graph, ckpt, variable_filter=r"MoE1D")
+  assert sorted(r.restored) == graph[:2]
+  assert r.in_graph_not_in_checkpoint == ["decoder/extra/bias",
+                                          "decoder/rms_norm/scale"]
+  r = checkpoint.plan_restore(
+      ["student/" + n for n in graph], ckpt,
+      variable_mapping=lambda n: n[len("student/"):],
+      should_load=lambda n: "rms_norm" not in n)
+  assert r.restored == {"student/" + n: n for n in graph[:2]}
+  assert "decoder/rms_norm/scale" in r.in_checkpoint_not_in_graph

@@ -226,3 +226,52 @@ def test_layer_stack_bfloat16():
   ok = np.isclose(got, want, rtol=5e-2, atol=5e-2).all(axis=-1)
   assert ok.mean() >= 0.95, ok.mean()
   np.testing.assert_allclose(got_loss, want_loss, rtol=2e-2)
+
+
+def test_checkpoint_round_trip(tmp_path):
+  """Variables saved by name to an .npz archive and restored into a freshly
+  initialised lowering of the same graph reproduce the outputs; a filter
+  restores only the matching names; a wrong shape raises."""
+  from mesh_amd import checkpoint
+  b, l, m, e, hdim, heads, d, group = 1, 32, 32, 4, 48, 2, 16, 32
+  rng = np.random.default_rng(31)
+  layers, final = _build_stack(rng, m, e, hdim, heads, d, group)
+  x = rng.standard_normal((b, l, m)).astype(np.float32)
+
+  def build():
+    graph = mtf.Graph()
+    mesh = mtf.Mesh(graph, "mesh")
+    dims = [mtf.Dimension("batch", b), mtf.Dimension("length", l),
+            mtf.Dimension("d_model", m)]
+    xt = mtf.import_tf_tensor(mesh, torch.from_numpy(x), mtf.Shape(dims))
+    stack = transformer.make_layer_stack(
+        [(transformer_layers.SelfAttention,
+          dict(num_heads=heads, key_value_size=d)),
+         (moe.MoE1D, dict(num_experts=e, hidden_size=hdim, group_size=group,
+                          second_policy_train="all", second_policy_eval="all")),
+         (transformer_layers.DenseReluDense, dict(hidden_size=hdim))],
+        num_layers=1, block_scope=False)
+    model = transformer.Unitransformer(stack, d_model=m, name="decoder")
+    y, _ = model.call_layers(xt, mtf.VariableDType(torch.float32))
+    lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()})
+    return lowering, y
+
+  low_a, y_a = build()                       # random initial values
+  out_a = H.to_np(low_a.export_to_tf_tensor(y_a))
+  path = str(tmp_path / "model.npz")
+  saved = checkpoint.save_variables(low_a, path)
+  assert "decoder/layer_001/MoE1D/top_2_gating/kernel" in saved
+  low_b, y_b = build()                       # other random values
+  assert np.abs(H.to_np(low_b.export_to_tf_tensor(y_b)) - out_a).max() > 1e-3
+  report = checkpoint.restore_variables(low_b, path)
+  assert sorted(report.restored) == sorted(saved)
+  assert not report.in_graph_not_in_checkpoint
+  low_b.run()
+  np.testing.assert_array_equal(H.to_np(low_b.export_to_tf_tensor(y_b)), out_a)
+  low_c, _ = build()
+  report = checkpoint.restore_variables(low_c, saved, variable_filter="MoE1D")
+  assert sorted(report.restored) == sorted(n for n in saved if "MoE1D" in n)
+  bad = dict(saved)
+  bad["decoder/rms_norm/scale"] = np.ones(m + 1, np.float32)
+  with pytest.raises(ValueError, match="has shape"):
+    checkpoint.restore_variables(low_c, bad)
