@@ -42,72 +42,63 @@ class TransformerLayer(object):
     return getattr(self, "_name", None)
 
 
+# Context fields that only decoding, beam search, encoder-decoder attention or
+# parameter sharing use; accepted for signature compatibility, must stay None.
+_UNUSED_CONTEXT_FIELDS = (
+    "beam_dim", "subsequence_id", "states", "new_states", "initial_position",
+    "encoder_output", "encoder_sequence_id", "constant_states",
+    "shared_params", "encoder_layer_outputs", "inputs", "encoder_inputs")
+
+
 class Context(object):
   """What layers need at call time (transformer.py:107-311), for the "train"
   and "eval" modes.  read_priority / write_priority are None (every position
   sees every position) or POSITION (autoregressive); sequence_id is None or 1
-  (no padding)."""
+  (no padding).  The reference's remaining constructor arguments
+  (_UNUSED_CONTEXT_FIELDS) are accepted as keywords and must be None."""
 
   def __init__(self, model, mesh, batch_dims, length_dim, variable_dtype,
-               beam_dim=None, mode=TRAIN, position=None,
-               position_is_default=False, sequence_id=None,
-               subsequence_id=None, states=None, new_states=None, losses=None,
-               initial_position=None, layer_outputs=None, encoder_output=None,
-               encoder_sequence_id=None, constant_states=None,
-               shared_params=None, encoder_layer_outputs=None,
-               write_priority=None, read_priority=None, inputs=None,
-               encoder_inputs=None, num_microbatches=1):
+               mode=TRAIN, position=None, position_is_default=False,
+               sequence_id=None, losses=None, layer_outputs=None,
+               write_priority=None, read_priority=None, num_microbatches=1,
+               **unused):
     if mode not in (TRAIN, EVAL):
       raise NotImplementedError("mode %r (decoding) is not implemented"
                                 % (mode,))
-    if beam_dim is not None or encoder_output is not None:
-      raise NotImplementedError("beam search / encoder-decoder attention")
-    for pr in (write_priority, read_priority):
-      if pr is not None and pr is not POSITION:
-        raise NotImplementedError(
-            "read/write priorities other than the position")
+    for key, value in unused.items():
+      if key not in _UNUSED_CONTEXT_FIELDS:
+        raise TypeError("Context got an unexpected argument %r" % key)
+      if value is not None:
+        raise NotImplementedError("Context.%s is not implemented" % key)
     if (write_priority is None) != (read_priority is None):
       raise ValueError("read_priority and write_priority go together")
-    self.model = model
-    self.mesh = mesh
-    self.batch_dims = batch_dims
-    self.length_dim = length_dim
+    if write_priority not in (None, POSITION) or read_priority not in (
+        None, POSITION):
+      raise NotImplementedError("read/write priorities other than the position")
+    for key in _UNUSED_CONTEXT_FIELDS:
+      setattr(self, key, None)
+    self.shared_params = {}
+    self.model, self.mesh = model, mesh
+    self.batch_dims, self.length_dim = batch_dims, length_dim
     self.variable_dtype = variable_dtype
-    self.beam_dim = beam_dim
     self.mode = mode
-    self.position = position
-    self.position_is_default = position_is_default
+    self.position, self.position_is_default = position, position_is_default
     self.sequence_id = sequence_id
-    self.subsequence_id = subsequence_id
-    self.states = states
-    self.new_states = new_states
     self.losses = losses
-    self.initial_position = initial_position
-    self.layer_outputs = layer_outputs if layer_outputs is not None else []
-    self.encoder_output = encoder_output
-    self.encoder_sequence_id = encoder_sequence_id
-    self.constant_states = constant_states
-    self.shared_params = shared_params or {}
-    self.layer_index = 0
-    self.encoder_layer_outputs = encoder_layer_outputs
-    self.cache = {}
-    self.write_priority = write_priority
-    self.read_priority = read_priority
-    self.inputs = inputs
-    self.encoder_inputs = encoder_inputs
+    self.layer_outputs = [] if layer_outputs is None else layer_outputs
+    self.write_priority, self.read_priority = write_priority, read_priority
     self.num_microbatches = num_microbatches
+    self.layer_index = 0
+    self.cache = {}            # values shared between layers
 
-  @property
-  def train(self):
-    return self.mode == TRAIN
-
-  @property
-  def activation_dtype(self):
-    return self.variable_dtype.activation_dtype
+  train = property(lambda self: self.mode == TRAIN)
+  activation_dtype = property(
+      lambda self: self.variable_dtype.activation_dtype)
 
   @property
   def nonpadding(self):
-    """Zeros in padding positions and ones elsewhere (transformer.py:297-306)."""
+    """Zeros in padding positions and ones elsewhere (transformer.py:297-306):
+    None without a sequence_id, the integer 1 when sequence_id == 1."""
     if self.sequence_id is None:
       return None
     if isinstance(self.sequence_id, int) and self.sequence_id == 1:
@@ -277,32 +268,39 @@ class LayerStack(TransformerLayer):
     return self._layers
 
 
+def _layer_spec(spec):
+  """A class, or a list / tuple holding a class and optionally a name (str)
+  and constructor arguments (dict), in any order."""
+  if not isinstance(spec, (list, tuple)):
+    return spec, None, {}
+  cls, name, kwargs = None, None, {}
+  for item in spec:
+    if isinstance(item, str):
+      name = item
+    elif isinstance(item, dict):
+      kwargs = item
+    else:
+      cls = item
+  return cls, name, kwargs
+
+
 def make_layer_stack(layers, num_layers=6, block_scope=True,
                      layer_stack_cls=LayerStack):
-  """transformer.py:1876-1948: `layers` lists, per block, classes or
-  (class, name, kwargs) tuples; the names are block_%03d/layer_%03d or
-  layer_%03d."""
-  layer_stack = []
+  """transformer.py:1876-1948: `layers` describes one block, repeated
+  num_layers times.  Layer names are block_%03d/<name or layer_%03d> with
+  block_scope, else <name> or layer_%03d counted over the whole stack."""
+  built = []
   for block in range(num_layers):
-    for n, cls in enumerate(layers):
-      name = None
-      kwargs = {}
-      if isinstance(cls, (list, tuple)):
-        for x in cls:
-          if isinstance(x, str):
-            name = x
-          elif isinstance(x, dict):
-            kwargs = x
-          else:
-            cls = x
+    for n, spec in enumerate(layers):
+      cls, name, kwargs = _layer_spec(spec)
       if block_scope:
-        name = "block_{:03d}/{}".format(block, name or "layer_{:03d}".format(n))
-      else:
-        name = name or "layer_{:03d}".format(len(layer_stack))
+        name = "block_%03d/%s" % (block, name or "layer_%03d" % n)
+      elif not name:
+        name = "layer_%03d" % len(built)
       layer = cls(**kwargs)
       layer.set_name(name)
-      layer_stack.append(layer)
-  return layer_stack_cls(layer_stack)
+      built.append(layer)
+  return layer_stack_cls(built)
 
 
 class Unitransformer(object):
