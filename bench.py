@@ -153,6 +153,44 @@ def build(cfg, device, backward=False):
   return lowering, x, y, loss
 
 
+def build_block(cfg, device):
+  """The block of mesh_tensorflow/transformer/gin/models/lm_moe.gin:11-16
+  (SelfAttention, MoE1D, SelfAttention, DenseReluDense; autoregressive, eval
+  mode) around the layer of `cfg`: d_kv 128, d_model / 128 heads, d_ff and the
+  experts' hidden size = cfg's H.  Variables keep their own initialisers
+  (random normal).  Returns (lowering, x Tensor, y Tensor, None)."""
+  import torch
+  import mesh_amd as mtf
+  from mesh_amd.transformer import moe, transformer, transformer_layers
+
+  dt = torch.bfloat16 if cfg["dtype"] == "bf16" else torch.float32
+  m = cfg["M"]
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  gen = torch.Generator(device=device)
+  gen.manual_seed(1)
+  x_val = torch.randn((cfg["batch"], cfg["length"], m), generator=gen,
+                      device=device, dtype=torch.float32).to(dt)
+  dims = [mtf.Dimension("batch", cfg["batch"]),
+          mtf.Dimension("length", cfg["length"]), mtf.Dimension("d_model", m)]
+  x = mtf.import_tf_tensor(mesh, x_val, mtf.Shape(dims))
+  attention = (transformer_layers.SelfAttention,
+               dict(num_heads=max(1, m // 128), key_value_size=128))
+  stack = transformer.make_layer_stack(
+      [attention,
+       (moe.MoE1D, dict(num_experts=cfg["E"], hidden_size=cfg["H"],
+                        group_size=cfg["group"], capacity_factor_eval=cfg["cf"],
+                        second_policy_eval="all", second_policy_train="all")),
+       attention,
+       (transformer_layers.DenseReluDense, dict(hidden_size=cfg["H"]))],
+      num_layers=1, block_scope=False)
+  model = transformer.Unitransformer(stack, d_model=m, name="decoder",
+                                     autoregressive=True)
+  y, _ = model.call_layers(x, mtf.VariableDType(dt, dt, dt), mode="eval")
+  lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl(device=device)})
+  return lowering, x, y, None
+
+
 def stage_model(cfg, kept_pairs, slots):
   """Algorithmic bytes / flops per step of each stage (v1 layer): what a
   perfect implementation has to move or compute."""
@@ -238,6 +276,10 @@ def main():
   ap.add_argument("--backward", action="store_true",
                   help="time forward + backward (v1 configs); the metric is "
                        "then named accordingly and is not the benchmark's")
+  ap.add_argument("--block", action="store_true",
+                  help="time the transformer block around the layer "
+                       "(attention, MoE1D, attention, DenseReluDense; v1 "
+                       "configs); not the benchmark's metric")
   ap.add_argument("--no-cpu-baseline", action="store_true")
   args = ap.parse_args()
   if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -260,7 +302,14 @@ def main():
   if args.backward and cfg["layer"] != "v1":
     print("--backward applies to the v1 configs only", file=sys.stderr)
     sys.exit(2)
-  lowering, x, y, loss = build(cfg, device, args.backward)   # first execution
+  if args.block and (cfg["layer"] != "v1" or args.backward or
+                     args.gating != "top_2"):
+    print("--block applies to the v1 configs, forward, top_2", file=sys.stderr)
+    sys.exit(2)
+  if args.block:
+    lowering, x, y, loss = build_block(cfg, device)
+  else:
+    lowering, x, y, loss = build(cfg, device, args.backward)  # first execution
   for _ in range(args.warmup):
     lowering.run()
   torch.cuda.synchronize()
@@ -276,6 +325,26 @@ def main():
   tokens = cfg["batch"] * cfg["length"]
   out_ok = bool(torch.isfinite(lowering.export_to_tf_tensor(y).float()).all())
 
+  if args.block:
+    # attention + MoE1D + attention + DenseReluDense: per-stage times only
+    heads = max(1, cfg["M"] // 128)
+    print(json.dumps({
+        "metric": "MoE transformer block fwd tokens/sec @1 GPU",
+        "value": tokens / (ms_per_step * 1e-3), "unit": "tokens/s",
+        "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True,
+        "scaling": "weak", "vs_baseline": None, "dtype": cfg["dtype"],
+        "data": "synthetic",
+        "config": {"workload": "lm_moe block (attention, MoE1D, attention, "
+                               "DenseReluDense) around " + cfg["name"],
+                   "tokens": tokens, "heads": heads, "d_kv": 128,
+                   "output_finite": out_ok},
+        "roofline": None,
+        "stages": {k: {"ms_per_step": v[1] / args.steps,
+                       "launches_per_step": v[0] / args.steps}
+                   for k, v in stages.items()},
+        "cpu_baseline": None}))
+    return
   result = {
       "metric": ("MoE layer fwd+bwd tokens/sec @1 GPU" if args.backward
                  else "MoE layer fwd tokens/sec @1 GPU"),

@@ -468,8 +468,11 @@ size_t mesh_moe_self_attention_workspace_bytes(int B, int L, int H, int D,
  * weights cast to dtype, outputs = weights . v.
  *   q, k, v, out [B,L,H*D] dtype (heads and d_kv combined as the reference's
  *   combine_dims does); bf16 needs L and D multiples of 8.
- * The logits and weights of all heads live in the workspace
- * (B*H*L*L*(4 + sizeof dtype) bytes).
+ * bf16 with D = 64 or 128 runs one fused kernel (logits stay on chip, the
+ * division by the softmax sum comes after the weights are rounded; workspace =
+ * a transposed copy of v).  Other cases run the three-step form whose logits
+ * and weights of all heads live in the workspace (B*H*L*L*(4 + sizeof dtype)
+ * bytes).
  */
 int mesh_moe_self_attention(const void* q, const void* k, const void* v,
                             void* out, int B, int L, int H, int D, int causal,

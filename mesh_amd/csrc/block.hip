@@ -22,12 +22,53 @@ namespace mesh_moe {
 template <typename T>
 __global__ __launch_bounds__(256) void rms_norm_kernel(
     const T* __restrict__ x, const T* __restrict__ scale, T* __restrict__ y,
-    int64_t rows, int M, float inv_m, float eps) {
+    int64_t rows, int M, float inv_m, float eps, bool vec16) {
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
   const T* xr = x + row * M;
+  T* yr = y + row * M;
   float sum = 0.f;
+  if (sizeof(T) == 2 && vec16) {
+    // bf16 rows in 16-byte pieces: 8 values per lane and step
+    const uint4* xv = reinterpret_cast<const uint4*>(xr);
+    const uint4* sv = reinterpret_cast<const uint4*>(scale);
+    uint4* yv = reinterpret_cast<uint4*>(yr);
+    const int chunks = M / 8;
+    for (int c = lane; c < chunks; c += 64) {
+      const uint4 p = xv[c];
+      const uint32_t w[4] = {p.x, p.y, p.z, p.w};
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float a = __uint_as_float(w[j] << 16);
+        const float b = __uint_as_float(w[j] & 0xffff0000u);
+        sum += round_to<T>(a * a);
+        sum += round_to<T>(b * b);
+      }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+    const float total = round_to<T>(sum);
+    const float mean = round_to<T>(total * inv_m);
+    const float var = round_to<T>(mean + eps);
+    const float r = round_to<T>(1.0f / sqrtf(var));
+    for (int c = lane; c < chunks; c += 64) {
+      const uint4 p = xv[c], q = sv[c];
+      const uint32_t w[4] = {p.x, p.y, p.z, p.w};
+      const uint32_t g[4] = {q.x, q.y, q.z, q.w};
+      uint32_t o[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float a = __uint_as_float(w[j] << 16);
+        const float b = __uint_as_float(w[j] & 0xffff0000u);
+        const float sa = __uint_as_float(g[j] << 16);
+        const float sb = __uint_as_float(g[j] & 0xffff0000u);
+        o[j] = f32x2_to_bf16x2(round_to<T>(a * r) * sa, round_to<T>(b * r) * sb);
+      }
+      yv[c] = make_uint4(o[0], o[1], o[2], o[3]);
+    }
+    return;
+  }
   for (int i = lane; i < M; i += 64) {
     const float v = load_f32<T>(xr + i);
     sum += round_to<T>(v * v);                              // mtf.square
@@ -38,7 +79,6 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(
   const float mean = round_to<T>(total * inv_m);            // * (1 / M)
   const float var = round_to<T>(mean + eps);                // + epsilon
   const float r = round_to<T>(1.0f / sqrtf(var));           // rsqrt
-  T* yr = y + row * M;
   for (int i = lane; i < M; i += 64) {
     const float v = load_f32<T>(xr + i);
     const float s = load_f32<T>(scale + i);
@@ -192,14 +232,17 @@ extern "C" int mesh_moe_rms_norm(const void* x, const void* scale, void* y,
   if (dtype == MESH_MOE_F32) {
     rms_norm_kernel<float><<<(unsigned)blocks, 256, 0, st>>>(
         (const float*)x, (const float*)scale, (float*)y, rows, M,
-        (float)(1.0 / (double)M), (float)epsilon);
+        (float)(1.0 / (double)M), (float)epsilon, false);
   } else {
     // Python scalars reach the reference's ops rounded to the tensor dtype
     const float inv_m = round_bf16_host((float)(1.0 / (double)M));
     const float eps = round_bf16_host((float)epsilon);
+    const bool vec16 =
+        M % 8 == 0 &&
+        (((uintptr_t)x | (uintptr_t)scale | (uintptr_t)y) % 16 == 0);
     rms_norm_kernel<bf16_t><<<(unsigned)blocks, 256, 0, st>>>(
         (const bf16_t*)x, (const bf16_t*)scale, (bf16_t*)y, rows, M, inv_m,
-        eps);
+        eps, vec16);
   }
   MOE_CHECK_LAUNCH("rms_norm");
   return 0;
@@ -208,6 +251,9 @@ extern "C" int mesh_moe_rms_norm(const void* x, const void* scale, void* y,
 extern "C" size_t mesh_moe_self_attention_workspace_bytes(int B, int L, int H,
                                                           int D, int dtype) {
   if (B < 1 || L < 1 || H < 1 || D < 1 || !valid_dtype(dtype)) return 0;
+  if (flash_attention_supported(L, H, D, dtype, nullptr, nullptr, nullptr,
+                                nullptr))
+    return flash_attention_workspace_bytes(B, L, H, D);
   const size_t b = dtype_size(dtype);
   const size_t hd = (size_t)B * H * L * D, ll = (size_t)B * H * L * L;
   return 4 * hd * b + ll * 4 + ll * b + 7 * 256;
@@ -235,6 +281,15 @@ extern "C" int mesh_moe_self_attention(const void* q, const void* k,
                   mesh_moe_self_attention_workspace_bytes(B, L, H, D, dtype),
               MESH_MOE_E_ARG, "self_attention: workspace too small");
   hipStream_t st = (hipStream_t)stream;
+  if (flash_attention_supported(L, H, D, dtype, nullptr, nullptr, nullptr,
+                                nullptr)) {
+    // fused kernel: the logits stay on chip
+    MOE_REQUIRE(flash_attention_supported(L, H, D, dtype, q, k, v, out),
+                MESH_MOE_E_UNSUPPORTED,
+                "self_attention: q, k, v, out must be 16-byte aligned");
+    return flash_attention(q, k, v, out, B, L, H, D, causal ? 1 : 0, workspace,
+                           st);
+  }
   if (dtype == MESH_MOE_F32)
     return run_attention<float>((const float*)q, (const float*)k,
                                 (const float*)v, (float*)out, B, L, H, D,

@@ -19,6 +19,14 @@ void set_error(const char* fmt, ...);
 int batched_gemm_nt(const void* A, const void* B, void* C, int E, int R, int N,
                     int K, int dtype, bool out_f32, hipStream_t st);
 
+// Fused self-attention (attention.hip): q, k, v, out [B,L,H*D] bf16.
+bool flash_attention_supported(int L, int H, int D, int dtype, const void* q,
+                               const void* k, const void* v, const void* out);
+size_t flash_attention_workspace_bytes(int B, int L, int H, int D);
+int flash_attention(const void* q, const void* k, const void* v, void* out,
+                    int B, int L, int H, int D, int causal, void* workspace,
+                    hipStream_t st);
+
 #define MOE_REQUIRE(cond, code, ...)      \
   do {                                    \
     if (!(cond)) {                        \

@@ -65,9 +65,11 @@ def test_dense(hip, shape, act_dtype):
 
 
 ATT_CASES = [
-    # B, L, heads, d_kv, d_model
+    # B, L, heads, d_kv, d_model; bf16 with d_kv 64 / 128 runs the fused kernel
     (2, 12, 3, 4, 16), (1, 128, 4, 32, 64), (2, 200, 2, 64, 48),
-    (1, 512, 8, 128, 256), (3, 64, 1, 16, 32),
+    (1, 512, 8, 128, 256), (3, 64, 1, 16, 32), (2, 8, 2, 128, 32),
+    (1, 72, 3, 64, 64), (2, 1000, 2, 128, 128), (1, 2048, 2, 128, 128),
+    (3, 328, 1, 64, 32),
 ]
 
 
