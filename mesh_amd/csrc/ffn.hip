@@ -1009,7 +1009,7 @@ static int grouped_gemm(const void* A, const void* B, void* C, int E, int R,
       rc = launch_simple<bf16_t>((const bf16_t*)A, (const bf16_t*)B,
                                  (bf16_t*)C, E, R, N, K, relu, st);
     else if (N >= 256 && R >= 128 && K % 64 == 0 &&
-             (int64_t)R * K < (1LL << 30) && (int64_t)N * K < (1LL << 30)) {
+             (int64_t)R * K < (1LL << 31) && (int64_t)N * K < (1LL << 31)) {
       // direct-to-LDS kernels; 256-row tiles unless 128-row tiles waste fewer
       // padded rows (e.g. 640 rows per expert: 5 x 128 instead of 3 x 256)
       const bf16_t *a = (const bf16_t*)A, *b = (const bf16_t*)B;

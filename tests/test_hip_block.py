@@ -277,3 +277,25 @@ def test_checkpoint_round_trip(tmp_path):
   bad["decoder/rms_norm/scale"] = np.ones(m + 1, np.float32)
   with pytest.raises(ValueError, match="has shape"):
     checkpoint.restore_variables(low_c, bad)
+
+
+def test_dense_rows_beyond_2_to_the_30_elements(hip):
+  """A dense layer whose input has more than 2^30 elements (98304 tokens x
+  16384 channels): the direct-to-LDS kernels address rows with 32-bit element
+  offsets, which must hold up to 2^31.  Checked on the first and last rows
+  against a float32 matmul of those rows."""
+  rows, k, n = 98304, 16384, 256
+  gen = torch.Generator(device="cuda")
+  gen.manual_seed(5)
+  x = torch.empty((1, rows, k), dtype=torch.bfloat16, device="cuda")
+  for i in range(0, rows, 8192):     # in pieces: no float32 copy of 6 GB
+    x[0, i:i + 8192] = torch.randn((8192, k), generator=gen,
+                                   device="cuda").to(torch.bfloat16)
+  w = (torch.randn((k, n), generator=gen, device="cuda") / k ** 0.5).to(
+      torch.bfloat16)
+  wp = hip.pack_weights(w.reshape(1, k, n), torch.bfloat16)
+  y = hip.dense(x, wp, None)
+  for sl in (slice(0, 64), slice(rows - 64, rows), slice(65500, 65600)):
+    want = x[0, sl].float() @ w.float()
+    np.testing.assert_allclose(H.to_np(y[0, sl]), H.to_np(want), rtol=2e-2,
+                               atol=2e-2)
