@@ -251,7 +251,7 @@ int mesh_moe_combine(const void* y, const int32_t* idx, const int32_t* pos,
 /*
  * "No token left behind" gating (_ntlb_gating, transformer/moe.py:804-940)
  * after the router projection: every token names its top_k experts
- * (mtf.top_k, ops.py:4964-5015); round i offers the tokens no expert has
+ * (mtf.top_k, ops.py:4964-5015); pass i offers the tokens no expert has
  * taken yet, in token order, to their i-th expert, which takes them while its
  * total stays within the capacity (moe.py:903-934).  A token is routed at
  * most once, with the raw softmax probability of the expert that took it as

@@ -249,7 +249,7 @@ __global__ __launch_bounds__(256) void gate_count_kernel(
     }
     if (one) atomicAdd(&cnt[p.E], 1);
     if (p.router == 2) {
-      // ntlb: one density per round, every token's top_k candidates
+      // ntlb: one density per pass, every token's top_k candidates
       // (moe.py:839-847); the probabilities and the repeated first-arg-max are
       // those of the forward kernel, so the candidates are the same
       const float* row = logits + t * p.E;
@@ -340,7 +340,7 @@ __global__ __launch_bounds__(256) void gating_backward_kernel(
   } else {
     // switch: the gate is the arg-max probability; ntlb: the probability of
     // the candidate that took the token, and the loss averages over the
-    // top_k rounds as well (moe.py:845-856)
+    // top_k passes as well (moe.py:845-856)
     add1 = dgate[t * 2] * k1 * m1;
     const double terms =
         (double)p.G * (double)E * (p.router == 2 ? (double)p.top_k : 1.0);

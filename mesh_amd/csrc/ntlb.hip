@@ -3,7 +3,7 @@
 // Follows _ntlb_gating, mesh_tensorflow/transformer/moe.py:804-940, after the
 // router projection: float32 softmax in the operation order of mtf.softmax
 // (ops.py:5493-5541), the top_k experts of every token (mtf.top_k,
-// ops.py:4964-5015: repeated first-arg-max), then top_k rounds in which the
+// ops.py:4964-5015: repeated first-arg-max), then top_k passes in which the
 // still unrouted tokens are offered, in token order, to their next expert
 // (moe.py:903-934).  The dense [G,S,k,E] masks and the cumsum over the group
 // are replaced by per-token candidate lists and integer counting; the result
@@ -106,13 +106,13 @@ __global__ __launch_bounds__(256) void ntlb_select_kernel(
 
 // ---------------------------------------------------------------------------
 // Step 2: one block per group.  Thread (e = tid % el, chunk = tid / el), as in
-// the capacity kernel of the other routers.  Round i: every thread counts the
+// the capacity kernel of the other routers.  Pass i: every thread counts the
 // offers to expert e in its chunk of tokens (unrouted tokens with importance 1
 // whose i-th candidate is e), an exclusive prefix over the chunks gives the
 // chunk's starting count on top of what the expert holds, and a second walk
 // takes the offers whose running count stays within the capacity
 // (moe.py:908-916: the count includes the offers that are turned down).  Each
-// token is visited by exactly one thread per round.
+// token is visited by exactly one thread per pass.
 // ---------------------------------------------------------------------------
 __global__ __launch_bounds__(NTLB_THREADS) void ntlb_assign_kernel(
     NtlbParams p, const int16_t* __restrict__ cand_idx,
@@ -158,7 +158,7 @@ __global__ __launch_bounds__(NTLB_THREADS) void ntlb_assign_kernel(
   const int s_end = min(S, s_begin + clen);
   for (int i = 0; i < K; ++i) {
     const int16_t* ch = cand + (size_t)i * S;
-    // density_1 of this round counts every token (moe.py:847 precedes the
+    // density_1 of this pass counts every token (moe.py:847 precedes the
     // importance mask), the offers only the open ones
     int all = 0, c = 0;
     for (int s = s_begin; s < s_end; ++s) {
@@ -201,7 +201,7 @@ __global__ __launch_bounds__(NTLB_THREADS) void ntlb_assign_kernel(
     __syncthreads();
   }
   if (tid < E) fill[(int64_t)g * E + tid] = held[tid];
-  // the group's share of the loss: sum over rounds and experts of
+  // the group's share of the loss: sum over passes and experts of
   // proxy[e] * density[i][e] (moe.py:848, :854)
   if (tid < E) {
     float proxy = 0.f;

@@ -425,7 +425,7 @@ def ntlb_gating(logits, capacity, top_k, importance=None,
                 num_microbatches=None):
   """logits float32 [G, S, E] -> Routing for "no token left behind" gating
   (_ntlb_gating, transformer/moe.py:804-940): top_k candidates per token, one
-  round per candidate rank, each token routed at most once."""
+  pass per candidate rank, each token routed at most once."""
   lib = load_library()
   g, s, e = logits.shape
   lp = _dev(logits, "logits", torch.float32)

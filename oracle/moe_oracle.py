@@ -30,7 +30,7 @@ MoE file, and its TensorFlow dependency cannot run here):
                                       lowering of mtf.top_k) vs the stable
                                       sort, per-expert brute force, equality
                                       with switch_gating when nothing overflows
-  ntlb_gating                         walk over (round, token) with one
+  ntlb_gating                         walk over (pass, token) with one
                                       counter per expert, a hand-worked case
                                       (4 tokens, 3 experts, capacity 1),
                                       k = 1 equals switch_gating, closed-form
@@ -469,11 +469,11 @@ def ntlb_gating(logits, capacity, top_k, importance=None,
   projection, for the deterministic policies (as switch_gating).
 
   Every token names its `top_k` best experts (mtf.top_k, moe.py:839-842).
-  Round i offers the still unrouted tokens to their i-th expert in token
+  Pass i offers the still unrouted tokens to their i-th expert in token
   order; an expert takes them while its running total, carried over from the
-  earlier rounds, stays within `capacity` (moe.py:905-934).  A token is routed
+  earlier passes, stays within `capacity` (moe.py:905-934).  A token is routed
   at most once; its gate is the raw softmax probability of the expert that
-  took it.  Same result dict as switch_gating, plus `round` [G,S] (which of
+  took it.  Same result dict as switch_gating, plus `taken_in_pass` [G,S] (which of
   its choices took the token, -1 if none) and `topk_index` [G,S,k].
   """
   logits = np.asarray(logits, dtype=F32)
@@ -543,7 +543,7 @@ def ntlb_gating(logits, capacity, top_k, importance=None,
       index_1=index_1, index_2=zeros_i, pos_1=pos_1, pos_2=zeros_i,
       kept_1=kept_1, kept_2=np.zeros((g_, s_), bool),
       gate_1=gate_1, gate_2=np.zeros((g_, s_), F32),
-      fill=cum_tokens.astype(np.int32), round=rnd, topk_index=expert_index,
+      fill=cum_tokens.astype(np.int32), taken_in_pass=rnd, topk_index=expert_index,
       loss=cast_act(loss, act_dtype)[()])                        # :937
   if dense:
     combine = cast_act(combine, act_dtype)                       # :936
@@ -978,12 +978,12 @@ def gating_backward(logits, r, gating, d_gate_1, d_gate_2, d_loss,
   if gating not in ("switch", "switch_max", "ntlb"):
     raise ValueError("unknown gating %r" % (gating,))
   # index_1 is the expert that took the token: the arg-max (switch) or the
-  # candidate of the round that placed it (ntlb: mtf.top_k routes the gradient
+  # candidate of the pass that placed it (ntlb: mtf.top_k routes the gradient
   # of each value to its entry, ops.py:4916-4920, :5009-5015)
   np.add.at(dp, rows + (i1,), np.asarray(d_gate_1, F32) * r["kept_1"] * m1)
   # loss = mean(mean_s(p)[g,e] * m1[g,s] * density_1[g,e]) * E^2 with density_1
-  # counting every token (moe.py:1224-1234); ntlb has one density per round and
-  # the mean runs over the rounds too (moe.py:845-856)
+  # counting every token (moe.py:1224-1234); ntlb has one density per pass and
+  # the mean runs over the passes too (moe.py:845-856)
   if gating == "ntlb":
     k_ = r["topk_index"].shape[-1]
     density = seq_sum(one_hot(r["topk_index"], e_).sum(axis=2, dtype=F32),

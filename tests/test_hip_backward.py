@@ -97,7 +97,7 @@ def test_backward_matches_oracle(hip, case):
            wi=H.normal_weights(rng, (e, m, hdim), m),
            wo=H.normal_weights(rng, (e, hdim, m), hdim))
   if gating == "ntlb":
-    w["w_gate"][:, 0] *= 3.0          # a popular expert: later rounds matter
+    w["w_gate"][:, 0] *= 3.0          # a popular expert: later passes matter
   x = H.safe_tokens(rng, g * s, m, w["w_gate"], act_dtype,
                     top=4 if gating == "ntlb" else 3).reshape(g, s, m)
   nonpad = (rng.random((g, s)) < 0.85).astype(np.float32) if use_np else None
@@ -111,7 +111,7 @@ def test_backward_matches_oracle(hip, case):
                                  act_dtype, d_out, d_loss, nonpadding=nonpad,
                                  num_microbatches=mb)
   if gating == "ntlb":
-    assert (want["aux"]["round"] > 0).any()
+    assert (want["aux"]["taken_in_pass"] > 0).any()
   got = run_backward(hip, x, w, hp, act_dtype, d_out, d_loss, nonpad, mb)
   tol = H.value_tolerance(act_dtype)
   np.testing.assert_allclose(got["dgate"], want["dgate"], rtol=1e-2 if

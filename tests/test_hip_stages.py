@@ -503,8 +503,8 @@ def _assert_switch_max_equal(got, want):
                                    (2, 131, 200, 1, 4), (1, 4096, 64, 60, 8),
                                    (2, 512, 16, 512, 4), (4, 300, 6, 40, 6)])
 def test_ntlb_gating_random_logits(hip, shape):
-  """Skewed router (a Zipf bias) so that the popular experts overflow in round
-  0 and the later rounds route what is left."""
+  """Skewed router (a Zipf bias) so that the popular experts overflow in pass
+  0 and the later passes route what is left."""
   g, s, e, c, k = shape
   rng = np.random.default_rng(3000 + sum(shape))
   logits = H.safe_logits(rng, g, s, e, scale=1.5,
@@ -521,7 +521,7 @@ def test_ntlb_gating_random_logits(hip, shape):
     H.assert_routing_equal(got, want)
     np.testing.assert_allclose(got["loss"], want["loss"], rtol=2e-5)
   if s > 64 and k > 1 and c * e < s:
-    assert (want["round"] > 0).any()       # the later rounds did something
+    assert (want["taken_in_pass"] > 0).any()       # the later passes did something
   assert not got["kept_1"][imp != 1.0].any()
 
 

@@ -326,8 +326,8 @@ def test_v1_switch_rejections():
 
 @pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
 def test_v1_ntlb_matches_oracle(act_dtype):
-  """ntlb end to end with a skewed router, so that round 0 overflows and the
-  later rounds place tokens; nonpadding masks some tokens out."""
+  """ntlb end to end with a skewed router, so that pass 0 overflows and the
+  later passes place tokens; nonpadding masks some tokens out."""
   b, l, m, hdim, e, group, k = 2, 256, 64, 128, 8, 128, 3
   rng = np.random.default_rng(305)
   w = dict(w_gate=H.normal_weights(rng, (m, e), m),
@@ -346,7 +346,7 @@ def test_v1_ntlb_matches_oracle(act_dtype):
   want, want_loss, aux = O.moe_layer_v1(x, w["w_gate"], w["wi"], w["wo"], ohp,
                                         False, act_dtype, nonpadding=nonpad,
                                         num_microbatches=2, dense=True)
-  assert (aux["round"] > 0).any() and not aux["kept_1"].all()
+  assert (aux["taken_in_pass"] > 0).any() and not aux["kept_1"].all()
   np.testing.assert_allclose(got, want, **H.value_tolerance(act_dtype))
   np.testing.assert_allclose(got_loss, want_loss,
                              rtol=1e-2 if act_dtype == "bfloat16" else 1e-4)

@@ -452,9 +452,9 @@ def test_v1_switch_dense_equals_index_form():
 
 # ---- ntlb ("no token left behind") gating ---------------------------------------
 def _ntlb_by_token_walk(p64, k, c, imp):
-  """transformer/moe.py:903-934 as a walk over (round, token): round i offers
+  """transformer/moe.py:903-934 as a walk over (pass, token): pass i offers
   the unrouted tokens, in token order, to their i-th best expert; the expert's
-  counter for the round starts at what it holds and counts every offer, taken
+  counter for the pass starts at what it holds and counts every offer, taken
   or not; an offer is taken while the counter stays within the capacity."""
   g, s, e = p64.shape
   order = np.argsort(-p64, axis=-1, kind="stable")[..., :k]
@@ -481,8 +481,8 @@ def test_ntlb_against_token_walk_and_float64(seed):
   g, s, e = 3, int(rng.integers(30, 80)), int(rng.integers(3, 7))
   k = 1 + seed % 4 if seed % 4 < e else e
   c = s // e + 1
-  # expert 0 is everybody's favourite: it overflows in round 0 while the
-  # others keep room for the later rounds
+  # expert 0 is everybody's favourite: it overflows in pass 0 while the
+  # others keep room for the later passes
   logits = (2 * rng.standard_normal((g, s, e))).astype(np.float32)
   logits[..., 0] += 2.0
   imp = None
@@ -494,7 +494,7 @@ def test_ntlb_against_token_walk_and_float64(seed):
   for dense in (False, True):
     r = O.ntlb_gating(logits, c, k, importance=imp, dense=dense)
     np.testing.assert_array_equal(r["topk_index"], order)
-    np.testing.assert_array_equal(r["round"], routed)
+    np.testing.assert_array_equal(r["taken_in_pass"], routed)
     np.testing.assert_array_equal(r["kept_1"], routed >= 0)
     np.testing.assert_array_equal(r["fill"], held)
     assert not r["kept_2"].any() and not r["gate_2"].any()
@@ -504,7 +504,7 @@ def test_ntlb_against_token_walk_and_float64(seed):
     np.testing.assert_array_equal(r["pos_1"][took], slot[took])
     want = np.take_along_axis(p64, ex[..., None], -1)[..., 0] * took
     np.testing.assert_allclose(r["gate_1"], want, rtol=2e-6)
-  # the capacity leaves first choices unserved, so later rounds matter
+  # the capacity leaves first choices unserved, so later passes matter
   assert (routed != 0).any()
   if k > 1:
     assert (routed > 0).any()
@@ -512,8 +512,8 @@ def test_ntlb_against_token_walk_and_float64(seed):
 
 def test_ntlb_hand_worked_case():
   """4 tokens, 3 experts, capacity 1, k = 2.  First choices 0,0,1,0; second
-  choices 1,2,0,1.  Round 0: token 0 takes expert 0, token 1 overflows it,
-  token 2 takes expert 1, token 3 overflows.  Round 1: token 1 -> expert 2
+  choices 1,2,0,1.  Pass 0: token 0 takes expert 0, token 1 overflows it,
+  token 2 takes expert 1, token 3 overflows.  Pass 1: token 1 -> expert 2
   (free), token 3 -> expert 1 (full) -> dropped."""
   big, mid, low = 3.0, 1.0, -2.0
   logits = np.array([[[big, mid, low], [big, low, mid], [mid, big, low],
@@ -522,7 +522,7 @@ def test_ntlb_hand_worked_case():
   p = scipy.special.softmax(logits.astype(np.float64), axis=-1)[0]
   np.testing.assert_array_equal(r["kept_1"][0], [True, True, True, False])
   np.testing.assert_array_equal(r["index_1"][0][:3], [0, 2, 1])
-  np.testing.assert_array_equal(r["round"][0], [0, 1, 0, -1])
+  np.testing.assert_array_equal(r["taken_in_pass"][0], [0, 1, 0, -1])
   np.testing.assert_array_equal(r["pos_1"][0][:3], [0, 0, 0])
   np.testing.assert_allclose(r["gate_1"][0], [p[0, 0], p[1, 2], p[2, 1], 0],
                              rtol=2e-6)
@@ -553,7 +553,7 @@ def test_ntlb_with_one_choice_is_switch():
 
 def test_ntlb_loss_closed_forms():
   """loss = E^2 * mean over [G,k,E] of proxy[g,e] * density[g,i,e]
-  (moe.py:845-856).  Uniform router: proxy = 1/E, and each round's density
+  (moe.py:845-856).  Uniform router: proxy = 1/E, and each pass's density
   sums to 1 over the experts, so the loss is E^2 * (1/E) * 1/E = 1 for any k.
   With importance the product gains the group dim and the mean the factor
   mean(importance == 1)."""
@@ -592,7 +592,7 @@ def test_ntlb_dense_tensors_match_index_record(act_dtype):
   np.testing.assert_array_equal(r["combine"], want)
   np.testing.assert_array_equal(r["dispatch"], (want != 0).astype(np.float32))
   assert (r["dispatch"].sum(axis=1) <= 1).all()      # one token per slot
-  assert (r["round"] > 0).any()
+  assert (r["taken_in_pass"] > 0).any()
 
 
 def test_v1_ntlb_dense_equals_index_form():
@@ -613,7 +613,7 @@ def test_v1_ntlb_dense_equals_index_form():
   np.testing.assert_allclose(d, i, rtol=1e-5, atol=1e-5)
   assert dl == il
   assert (d[nonpad == 0] == 0).all()
-  t = int(np.flatnonzero(aux["round"].reshape(-1) == 1)[0])   # a second choice
+  t = int(np.flatnonzero(aux["taken_in_pass"].reshape(-1) == 1)[0])   # a second choice
   ex = int(aux["index_1"].reshape(-1)[t])
   xt = x.reshape(-1, m)[t].astype(np.float64)
   ref = np.maximum(xt @ wi[ex].astype(np.float64), 0) @ wo[ex].astype(np.float64)
@@ -993,7 +993,7 @@ def test_backward_against_central_differences(gating):
   aux = got["aux"]
   assert not (aux["kept_1"] | aux["kept_2"]).all()     # drops are exercised
   if gating == "ntlb":
-    assert (aux["round"] > 0).any()        # tokens placed by a later choice
+    assert (aux["taken_in_pass"] > 0).any()        # tokens placed by a later choice
   m1 = (nonpad.reshape(aux["kept_1"].shape) == 1).astype(np.float64)
   z = hp.moe_z_loss if gating == "switch" else None
 
