@@ -9,8 +9,8 @@ reference expands the layer into ~100 graph primitives and dense one-hot
 the HIP kernels: router -> top-2 gating -> dispatch -> expert FFN -> combine.
 
 Built: moe_gating "top_2" (every second-place policy, the second-place loss),
-"switch", "switch_max", "ntlb" and "expert_selection" for the policies that
-draw no random numbers; nonpadding / importance; moe_use_experts_attention; float32 and
+"switch", "switch_max", "ntlb" and "expert_selection" (switch policies
+"argmax", "input_jitter", "input_dropout"; not "sample"); nonpadding / importance; moe_use_experts_attention; float32 and
 bfloat16; mtf.gradients over the v1 layer (top_2 / switch / switch_max / ntlb,
 ReLU or linear experts) and the v2 layer.  Not built (they raise NotImplementedError):
 expert dropout while training, gated (list) activations, gradients of the
@@ -166,23 +166,78 @@ class _GatingSpec(object):
         importance_from_slot_gate=importance_from_slot_gate)
 
 
+class _GateInputNoise(object):
+  """The random multiplier the switch-family routers put on their input while
+  training (hparams.moe_switch_policy_train):
+
+  "input_jitter": u in [1 - eps, 1 + eps), eps = moe_switch_jitter
+  (mtf.layers.multiplicative_jitter, layers.py:1949-1952);
+  "input_dropout": (u < keep_prob) / keep_prob with keep_prob = 1 -
+  moe_switch_dropout (mtf.dropout, ops.py:5864-5872).
+  _switch_gating and _expert_selection_gating apply it to to_float(inputs)
+  (moe.py:1189-1199, :1071-1078); _ntlb_gating knows only the jitter and
+  applies it in the activation dtype (moe.py:821-822).  Only the router sees
+  the perturbed tokens.  The uniform numbers come from torch's generator on the
+  device (the reference's come from TensorFlow's)."""
+
+  def __init__(self, hparams, train, in_float32, allow_dropout=True):
+    policy = (hparams.moe_switch_policy_train if train
+              else hparams.moe_switch_policy_eval)
+    self.kind = None
+    if train and policy == "input_jitter" and hparams.moe_switch_jitter != 0:
+      self.kind = "jitter"
+      self.eps = float(hparams.moe_switch_jitter)
+    elif train and policy == "input_dropout" and allow_dropout and (
+        hparams.moe_switch_dropout != 0):
+      self.kind = "dropout"
+      self.keep = 1.0 - float(hparams.moe_switch_dropout)
+    self.in_float32 = in_float32
+    self.last = None          # (router input, multiplier) of the last step
+
+  def apply(self, x):
+    """x [B, T, M] -> the router's input (float32 or x's dtype)."""
+    self.last = None
+    if self.kind is None:
+      return x
+    u = torch.rand(x.shape, dtype=torch.float32, device=x.device)
+    if self.kind == "jitter":
+      mult = (1.0 - self.eps) + u * (2.0 * self.eps)
+    else:
+      mult = (u < self.keep).to(torch.float32) / self.keep
+    if self.in_float32:
+      x_gate = x.to(torch.float32) * mult
+    else:
+      mult = mult.to(x.dtype)
+      x_gate = x * mult
+    self.last = (x_gate, mult)
+    return x_gate
+
+
+def _router_logits(x_gate, w, w_packed):
+  """Router projection of a possibly float32 (perturbed) input with kernels of
+  the activation dtype: the kernels are cast up, no packed copy is used."""
+  if x_gate.dtype == w.dtype:
+    return moe_hip.router_logits(x_gate, w, w_packed=w_packed)
+  return moe_hip.router_logits(x_gate.contiguous(), w.to(x_gate.dtype))
+
+
 class _SwitchGatingSpec(object):
   """Static configuration of one _switch_gating (moe.py:1176-1309) or
-  _switch_max_gating (moe.py:943-1054) call for the deterministic policies:
-  "argmax", and "input_dropout" / "input_jitter" when not training, where the
-  reference applies no perturbation (moe.py:1192-1199)."""
+  _switch_max_gating (moe.py:943-1054) call for the policies "argmax",
+  "input_dropout" and "input_jitter" (the perturbations apply while training,
+  moe.py:1192-1199)."""
 
   def __init__(self, hparams, train, num_microbatches, has_importance):
     self.slots_by_gate = hparams.moe_gating == "switch_max"
     policy = (hparams.moe_switch_policy_train if train
               else hparams.moe_switch_policy_eval)
-    if policy == "sample" or (train and policy in ("input_dropout",
-                                                   "input_jitter")):
+    if policy == "sample":
       raise NotImplementedError(
-          "switch policy %r draws random numbers (%s) and is not implemented"
-          % (policy, "training" if train else "sampling"))
+          "switch policy %r (sampling the expert) is not implemented"
+          % (policy,))
     if policy not in ("argmax", "input_dropout", "input_jitter"):
       raise ValueError("Unknown Switch gating policy %s" % policy)
+    self.noise = _GateInputNoise(hparams, train, in_float32=True)
     self.z_loss = None                     # _switch_max_gating has no z-loss
     if (train and not self.slots_by_gate and
         getattr(hparams, "moe_z_loss", None) is not None):
@@ -203,12 +258,14 @@ class _SwitchGatingSpec(object):
     assert not importance_from_slot_gate
     b, t, _ = x.shape
     groups = b * t // group_size
-    if moe_hip.fused_gating_supported(x, num_experts, group_size):
+    x_gate = self.noise.apply(x)
+    if x_gate is x and moe_hip.fused_gating_supported(x, num_experts,
+                                                      group_size):
       return moe_hip.router_switch_gating(
           x, w_packed, group_size, capacity, importance=importance,
           z_loss=self.z_loss, num_microbatches=self.num_microbatches,
           slots_by_gate=self.slots_by_gate, want_logits=want_logits)
-    logits = moe_hip.router_logits(x, w, w_packed=w_packed)
+    logits = _router_logits(x_gate, w, w_packed)
     logits = logits.reshape(groups, group_size, num_experts)
     r = moe_hip.switch_gating(
         logits, capacity, importance=importance, z_loss=self.z_loss,
@@ -218,8 +275,8 @@ class _SwitchGatingSpec(object):
 
 
 class _NtlbGatingSpec(object):
-  """Static configuration of one _ntlb_gating call (moe.py:804-940) for the
-  policies that draw no random numbers (as _SwitchGatingSpec)."""
+  """Static configuration of one _ntlb_gating call (moe.py:804-940); the only
+  policy it knows is "input_jitter" while training."""
 
   router = "ntlb"
   use_second_place_loss = False
@@ -228,10 +285,9 @@ class _NtlbGatingSpec(object):
   def __init__(self, hparams, train, num_microbatches, has_importance):
     policy = (hparams.moe_switch_policy_train if train
               else hparams.moe_switch_policy_eval)
-    if train and policy == "input_jitter":               # moe.py:821-822
-      raise NotImplementedError(
-          "switch policy %r draws random numbers while training and is not "
-          "implemented" % (policy,))
+    del policy                                          # moe.py:816-822
+    self.noise = _GateInputNoise(hparams, train, in_float32=False,
+                                 allow_dropout=False)
     self.top_k = int(hparams.moe_ntlb_top_k)
     self.num_microbatches = num_microbatches
 
@@ -242,7 +298,7 @@ class _NtlbGatingSpec(object):
     assert not importance_from_slot_gate
     b, t, _ = x.shape
     groups = b * t // group_size
-    logits = moe_hip.router_logits(x, w, w_packed=w_packed)
+    logits = _router_logits(self.noise.apply(x), w, w_packed)
     logits = logits.reshape(groups, group_size, num_experts)
     r = moe_hip.ntlb_gating(logits, capacity, self.top_k,
                             importance=importance,
@@ -262,10 +318,8 @@ class _ExpertSelectionGatingSpec(object):
   def __init__(self, hparams, train, num_microbatches, has_importance):
     policy = (hparams.moe_switch_policy_train if train
               else hparams.moe_switch_policy_eval)
-    if train and policy in ("input_dropout", "input_jitter"):
-      raise NotImplementedError(
-          "switch policy %r draws random numbers while training and is not "
-          "implemented" % (policy,))
+    del policy                                          # moe.py:1064-1078
+    self.noise = _GateInputNoise(hparams, train, in_float32=True)
     if not has_importance:
       # the reference sums `importance` for its loss (moe.py:1138-1140)
       raise ValueError("expert_selection gating needs nonpadding")
@@ -277,7 +331,7 @@ class _ExpertSelectionGatingSpec(object):
     assert not importance_from_slot_gate
     b, t, _ = x.shape
     groups = b * t // group_size
-    logits = moe_hip.router_logits(x, w, w_packed=w_packed)
+    logits = _router_logits(self.noise.apply(x), w, w_packed)
     logits = logits.reshape(groups, group_size, num_experts)
     r = moe_hip.expert_choice_gating(
         logits, capacity, importance=importance,
@@ -384,8 +438,11 @@ class MoEV1Operation(mtf.Operation):
              else moe_hip.combine(y4, r, s_))
       if save:
         # what the gradient operation reads (activations of this step)
+        noise = getattr(self._gating, "noise", None)
+        gate_in = noise.last if noise is not None else None
         saved.update(x=xg, routing=r, logits=logits, importance=imp_s,
-                     expert_in=expert_in, h=h, y=y, w_gate_packed=wg_p)
+                     expert_in=expert_in, h=h, y=y, w_gate_packed=wg_p,
+                     gate_in=gate_in, w_gate=wg_s)
       outs = (out.reshape(o_, g_, s_, n_), r.loss.to(dt).reshape(()))
       if kwo_p is not None:
         # the "k" projection of the same hidden tensor (moe.py:514-520)
@@ -451,11 +508,29 @@ class MoEV1GradOperation(mtf.Operation):
           router=gating.router, top_k=getattr(gating, "top_k", 0),
           importance=sv["importance"], z_loss=gating.z_loss,
           num_microbatches=gating.num_microbatches)
-      dwg = moe_hip.router_backward_weights(
-          sv["x"].reshape(groups * s_, m_), dlogits.reshape(groups * s_, e_))
-      dx = moe_hip.dispatch_backward(
-          dxe.reshape(e_, groups, c_, m_), r, s_, dlogits,
-          sv["w_gate_packed"].reshape(e_, m_))
+      tokens = groups * s_
+      if sv["gate_in"] is None:
+        dwg = moe_hip.router_backward_weights(
+            sv["x"].reshape(tokens, m_), dlogits.reshape(tokens, e_))
+        dx = moe_hip.dispatch_backward(
+            dxe.reshape(e_, groups, c_, m_), r, s_, dlogits,
+            sv["w_gate_packed"].reshape(e_, m_))
+      else:
+        # the router saw x * mult (a constant of the graph): its kernel's
+        # gradient uses that input, and its share of d(tokens) is
+        # (dlogits . w_gate^T) * mult
+        x_gate, mult = sv["gate_in"]
+        dt = sv["x"].dtype
+        dwg = moe_hip.router_backward_weights(
+            x_gate.reshape(tokens, m_).contiguous(),
+            dlogits.reshape(tokens, e_)).to(dt)
+        dx = moe_hip.dispatch_backward(dxe.reshape(e_, groups, c_, m_), r, s_)
+        w32 = sv["w_gate"].reshape(1, m_, e_).to(torch.float32).contiguous()
+        dx_router = moe_hip.expert_linear(
+            dlogits.reshape(1, tokens, e_), w32, "linear")   # [1, T, M]
+        dx = (dx.reshape(tokens, m_).to(torch.float32) +
+              dx_router.reshape(tokens, m_) *
+              mult.reshape(tokens, m_).to(torch.float32)).to(dt)
       return dx.reshape(o_, g_, s_, m_), dwg, dwi, dwo
 
     ins = self.inputs

@@ -792,10 +792,48 @@ def expert_ffn(expert_in, wi, wo, activation, act_dtype):
   return cast_act(np.matmul(h, wo), act_dtype)
 
 
+def perturb_gate_inputs(xg, hp, train, act_dtype, gate_noise):
+  """The router's input under hparams.moe_switch_policy_*:
+
+  _switch_gating / _expert_selection_gating (moe.py:1189-1199, :1071-1078):
+  gate_inputs = to_float(inputs); "input_dropout" multiplies by
+  (u < keep_prob) / keep_prob while training (mtf.dropout, ops.py:5864-5872),
+  "input_jitter" by u in [1 - eps, 1 + eps) while training
+  (mtf.layers.multiplicative_jitter, layers.py:1949-1952).
+  _ntlb_gating (moe.py:821-822) knows only the jitter and applies it in the
+  activation dtype.
+
+  gate_noise stands in for the random tensor u ~ U[0, 1) of xg's shape (the
+  reference draws it from TensorFlow's generator).  Returns (gate inputs,
+  the multiplier or None).
+  """
+  policy = hp.moe_switch_policy_train if train else hp.moe_switch_policy_eval
+  ntlb = hp.moe_gating == "ntlb"
+  jitter = train and policy == "input_jitter"
+  dropout = train and policy == "input_dropout" and not ntlb
+  if not (jitter or dropout):
+    return xg, None
+  if gate_noise is None:
+    raise NotImplementedError(
+        "switch policy %r needs the random tensor (gate_noise)" % policy)
+  u = np.asarray(gate_noise, F32).reshape(xg.shape)
+  if jitter:
+    eps = F32(hp.moe_switch_jitter)
+    if ntlb:       # random_uniform(dtype = activation dtype), product rounded
+      mult = cast_act((F32(1.0) - eps) + u * (F32(2.0) * eps), act_dtype)
+      return cast_act(xg * mult, act_dtype), mult
+    mult = (F32(1.0) - eps) + u * (F32(2.0) * eps)
+    return (xg.astype(F32) * mult).astype(F32), mult
+  keep = F32(1.0 - hp.moe_switch_dropout)
+  mult = (u < keep).astype(F32) / keep
+  return (xg.astype(F32) * mult).astype(F32), mult
+
+
 def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
                  nonpadding=None, activation="relu", num_microbatches=None,
                  logit_bias=None, second_uniform=None, dense=True,
-                 mesh_dim_size=1, weights_are_cast=False, k_wo=None):
+                 mesh_dim_size=1, weights_are_cast=False, k_wo=None,
+                 gate_noise=None):
   """transformer_moe_layer_v1 forward (transformer/moe.py:191-525).
 
   x: [batch..., length, M] float32 array holding activation-dtype values.
@@ -843,13 +881,16 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
     importance = cast_act(np.broadcast_to(nonpadding, lead), act_dtype)
     importance = importance.reshape(g_, s_)
   wg = cast_act(w_gate, act_dtype)
-  logits = router_logits(xg, wg)
+  gate_mult = None
+  if hp.moe_gating in ("switch", "switch_max", "ntlb", "expert_selection"):
+    x_gate, gate_mult = perturb_gate_inputs(xg, hp, train, act_dtype,
+                                            gate_noise)
+    logits = router_logits(x_gate, wg)
+  else:
+    logits = router_logits(xg, wg)
   if logit_bias is not None:
     logits = logits + np.asarray(logit_bias, F32)
   if hp.moe_gating == "expert_selection":                        # :425-438
-    sw = hp.moe_switch_policy_train if train else hp.moe_switch_policy_eval
-    if train and sw in ("input_dropout", "input_jitter"):
-      raise NotImplementedError("switch policy %r draws random numbers" % sw)
     if importance is None:
       raise ValueError("expert_selection gating needs nonpadding "
                        "(moe.py:1138-1140)")
@@ -879,7 +920,7 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
             _scale_loss(r["loss"], hp.moe_loss_coef, act_dtype), aux)
   if hp.moe_gating in ("switch", "switch_max", "ntlb"):          # :393-424
     sw = hp.moe_switch_policy_train if train else hp.moe_switch_policy_eval
-    if sw == "sample" or (train and sw in ("input_dropout", "input_jitter")):
+    if sw == "sample":
       raise NotImplementedError("switch policy %r draws random numbers" % sw)
     if sw not in ("argmax", "input_dropout", "input_jitter"):
       raise ValueError("Unknown Switch gating policy %s" % sw)
@@ -919,7 +960,7 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
   else:
     out = combine_gather(y, r, act_dtype)
   aux = dict(r, logits=logits, expert_in=expert_in, expert_out=y,
-             num_groups=g_, group_size=s_, capacity=c_)
+             num_groups=g_, group_size=s_, capacity=c_, gate_mult=gate_mult)
   return (out.reshape(lead + (n_,)),
           _scale_loss(r["loss"], hp.moe_loss_coef, act_dtype), aux)
 
@@ -1055,7 +1096,8 @@ def expert_ffn_backward(xe, wi_a, wo_a, dy, activation, act_dtype):
 
 def moe_layer_v1_backward(x, w_gate, wi, wo, hp, train, act_dtype, d_out,
                           d_loss=0.0, nonpadding=None, activation="relu",
-                          num_microbatches=None, logit_bias=None):
+                          num_microbatches=None, logit_bias=None,
+                          gate_noise=None):
   """Gradients of (outputs, loss) of moe_layer_v1 w.r.t. x and the three
   kernels, given d_out [batch..., length, N] and the scalar d_loss.
 
@@ -1077,7 +1119,8 @@ def moe_layer_v1_backward(x, w_gate, wi, wo, hp, train, act_dtype, d_out,
   _, _, aux = moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype,
                            nonpadding=nonpadding, activation=activation,
                            num_microbatches=num_microbatches,
-                           logit_bias=logit_bias, dense=False)
+                           logit_bias=logit_bias, dense=False,
+                           gate_noise=gate_noise)
   x = cast_act(x, act_dtype)
   lead, m_ = x.shape[:-1], x.shape[-1]
   g_, s_, c_ = aux["num_groups"], aux["group_size"], aux["capacity"]
@@ -1108,9 +1151,18 @@ def moe_layer_v1_backward(x, w_gate, wi, wo, hp, train, act_dtype, d_out,
   dlogits = gating_backward(aux["logits"], aux, hp.moe_gating, dgate[..., 0],
                             dgate[..., 1], d_aux, importance, num_microbatches,
                             z)
-  dwg = np.matmul(xg.reshape(-1, m_).T.astype(F32),
+  # the router saw the perturbed inputs x * mult (perturb_gate_inputs); the
+  # multiplier is a constant of the graph
+  mult = aux.get("gate_mult")
+  x_gate = xg.astype(F32) if mult is None else (
+      cast_act(xg * mult, act_dtype) if hp.moe_gating == "ntlb"
+      else xg.astype(F32) * mult)
+  dwg = np.matmul(x_gate.reshape(-1, m_).T.astype(F32),
                   dlogits.reshape(-1, e_)).astype(F32)
-  dx = dx + np.matmul(dlogits, wg_a.T.astype(F32))
+  dx_router = np.matmul(dlogits, wg_a.T.astype(F32))
+  if mult is not None:
+    dx_router = dx_router * mult
+  dx = dx + dx_router
   return dict(dx=cast_act(dx, act_dtype).reshape(lead + (m_,)),
               dw_gate=cast_act(dwg, act_dtype), dwi=dwi, dwo=dwo,
               dlogits=dlogits, dgate=dgate, aux=aux)

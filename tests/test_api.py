@@ -192,16 +192,17 @@ def test_error_behaviour():
   # ntlb reads the switch policy first, as the reference does (moe.py:816-819)
   with pytest.raises(AttributeError, match="moe_switch_policy_train"):
     moe.transformer_moe_layer_v1(x, dims[-1], hparams(moe_gating="ntlb"), True, vdt)
+  # the jitter reads its own hyperparameter, as the reference does
   nt = dict(moe_gating="ntlb", moe_switch_policy_train="input_jitter",
             moe_switch_policy_eval="argmax", moe_ntlb_top_k=2)
-  with pytest.raises(NotImplementedError, match="random numbers"):
+  with pytest.raises(AttributeError, match="moe_switch_jitter"):
     moe.transformer_moe_layer_v1(x, dims[-1], hparams(**nt), True, vdt)
   # switch gating reads its own hyperparameters, as the reference does
   with pytest.raises(AttributeError, match="moe_switch_policy_train"):
     moe.transformer_moe_layer_v1(x, dims[-1], hparams(moe_gating="switch"), True, vdt)
   sw = dict(moe_gating="switch", moe_switch_policy_train="argmax",
             moe_switch_policy_eval="sample", moe_z_loss=None)
-  with pytest.raises(NotImplementedError, match="random numbers"):
+  with pytest.raises(NotImplementedError, match="sampling"):
     moe.transformer_moe_layer_v1(x, dims[-1], hparams(**sw), False, vdt)
   with pytest.raises(ValueError, match="Unknown Switch gating policy"):
     moe.transformer_moe_layer_v1(

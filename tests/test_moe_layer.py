@@ -309,12 +309,8 @@ def test_v1_switch_rejections():
   base = dict(moe_num_experts=4, moe_hidden_size=8, moe_group_size=32)
   hp, _ = make_hparams(**dict(base, **dict(SWITCH_HP,
                                           moe_switch_policy_eval="sample")))
-  with pytest.raises(NotImplementedError, match="random"):
+  with pytest.raises(NotImplementedError, match="sampling"):
     run_v1(x, w, hp, False, "float32")
-  hp, _ = make_hparams(**dict(base, **dict(SWITCH_HP,
-                                          moe_switch_policy_train="input_jitter")))
-  with pytest.raises(NotImplementedError, match="random"):
-    run_v1(x, w, hp, True, "float32")
   hp, _ = make_hparams(**dict(base, **dict(SWITCH_HP,
                                           moe_switch_policy_eval="bogus")))
   with pytest.raises(ValueError, match="Unknown Switch gating policy"):
@@ -351,12 +347,53 @@ def test_v1_ntlb_matches_oracle(act_dtype):
   np.testing.assert_allclose(got_loss, want_loss,
                              rtol=1e-2 if act_dtype == "bfloat16" else 1e-4)
   assert (got.reshape(-1, m)[~aux["kept_1"].reshape(-1)] == 0).all()
-  hp_j, _ = make_hparams(moe_num_experts=e, moe_hidden_size=hdim,
-                         moe_group_size=group, moe_ntlb_top_k=k,
-                         **dict(SWITCH_HP, moe_gating="ntlb",
-                                moe_switch_policy_train="input_jitter"))
-  with pytest.raises(NotImplementedError, match="random"):
-    run_v1(x, w, hp_j, True, act_dtype)
+
+
+@pytest.mark.parametrize("case", [
+    ("switch", "input_jitter", "float32"), ("switch", "input_jitter", "bfloat16"),
+    ("switch", "input_dropout", "float32"), ("ntlb", "input_jitter", "bfloat16"),
+    ("switch_max", "input_dropout", "bfloat16")],
+    ids=lambda c: "-".join(c))
+def test_v1_router_input_noise_matches_oracle(case):
+  """Training with the perturbing switch policies: the layer draws u ~ U[0,1)
+  of the tokens' shape from torch's generator on the device as its first random
+  call; re-seeding reproduces the tensor for the oracle."""
+  gating, policy, act_dtype = case
+  b, l, m, hdim, e, group = 2, 96, 32, 48, 4, 48
+  rng = np.random.default_rng(331)
+  w = dict(w_gate=H.normal_weights(rng, (m, e), m),
+           wi=H.normal_weights(rng, (e, m, hdim), m),
+           wo=H.normal_weights(rng, (e, hdim, m), hdim))
+  x = O.cast_act(rng.standard_normal((b, l, m)).astype(np.float32), act_dtype)
+  kw = dict(SWITCH_HP, moe_gating=gating, moe_switch_policy_train=policy,
+            moe_switch_jitter=0.25, moe_switch_dropout=0.3, moe_ntlb_top_k=2)
+  hp, ohp = make_hparams(moe_num_experts=e, moe_hidden_size=hdim,
+                         moe_group_size=group, moe_capacity_factor_train=1.0,
+                         **kw)
+  torch.manual_seed(99)
+  got, got_loss, _, _ = run_v1(x, w, hp, True, act_dtype, num_microbatches=2)
+  torch.manual_seed(99)
+  u = torch.rand((1, b * l, m), dtype=torch.float32, device="cuda")
+  noise = u.cpu().numpy().reshape(b, l, m)
+  want, want_loss, aux = O.moe_layer_v1(x, w["w_gate"], w["wi"], w["wo"], ohp,
+                                        True, act_dtype, num_microbatches=2,
+                                        dense=False, gate_noise=noise)
+  assert aux["gate_mult"] is not None
+  plain, _, aux0 = O.moe_layer_v1(
+      x, w["w_gate"], w["wi"], w["wo"],
+      make_hparams(moe_num_experts=e, moe_hidden_size=hdim,
+                   moe_group_size=group, moe_capacity_factor_train=1.0,
+                   **dict(kw, moe_switch_policy_train="argmax"))[1],
+      True, act_dtype, num_microbatches=2, dense=False)
+  assert (aux["index_1"] != aux0["index_1"]).any()    # the noise changed routes
+  np.testing.assert_allclose(got, want, **H.value_tolerance(act_dtype))
+  np.testing.assert_allclose(got_loss, want_loss,
+                             rtol=1e-2 if act_dtype == "bfloat16" else 1e-4)
+  # evaluation draws nothing: same result whatever the generator's state
+  a, _, _, _ = run_v1(x, w, hp, False, act_dtype)
+  torch.manual_seed(5)
+  c, _, _, _ = run_v1(x, w, hp, False, act_dtype)
+  np.testing.assert_array_equal(a, c)
 
 
 def test_v1_switch_max_matches_oracle():
@@ -396,12 +433,15 @@ def test_v1_switch_max_matches_oracle():
 @pytest.mark.parametrize("case", [
     ("top_2", "float32", 101), ("top_2", "bfloat16", 102),
     ("switch", "float32", 103), ("switch_max", "float32", 104),
-    ("ntlb", "float32", 105)],
+    ("ntlb", "float32", 105), ("switch+input_jitter", "float32", 106),
+    ("switch+input_dropout", "bfloat16", 107),
+    ("ntlb+input_jitter", "float32", 108)],
     ids=lambda c: "%s-%s" % (c[0], c[1]))
 def test_v1_gradients_match_oracle(case):
   """mtf.gradients over the layer (outputs and loss) against the oracle's
   backward, which central differences pin in tests/test_oracle.py."""
   gating, act_dtype, seed = case
+  gating, _, noise_policy = gating.partition("+")
   b, l, m, hdim, e, group = 2, 64, 32, 48, 4, 32
   rng = np.random.default_rng(seed)
   w = dict(w_gate=H.normal_weights(rng, (m, e), m),
@@ -416,6 +456,9 @@ def test_v1_gradients_match_oracle(case):
   if gating != "top_2":
     kw.update(SWITCH_HP, moe_gating=gating, moe_ntlb_top_k=3,
               moe_z_loss=0.1 if gating == "switch" else None)
+  if noise_policy:
+    kw.update(moe_switch_policy_train=noise_policy, moe_switch_jitter=0.25,
+              moe_switch_dropout=0.3)
   hp, ohp = make_hparams(**kw)
   dt = H.ACT_TORCH[act_dtype]
   graph = mtf.Graph()
@@ -439,11 +482,17 @@ def test_v1_gradients_match_oracle(case):
             "ntlb": "ntlb_gating"}.get(gating, "top_2_gating")
   init = {"moe/%s/kernel" % router: w["w_gate"], "moe/wi/kernel": w["wi"],
           "moe/wo/kernel": w["wo"]}
+  torch.manual_seed(seed)
   lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()}, initial_values=init)
   got = [H.to_np(lowering.export_to_tf_tensor(g)) for g in grads]
+  noise = None
+  if noise_policy:         # the layer's first random call, reproduced
+    torch.manual_seed(seed)
+    noise = torch.rand((1, b * l, m), dtype=torch.float32,
+                       device="cuda").cpu().numpy().reshape(b, l, m)
   want = O.moe_layer_v1_backward(x, w["w_gate"], w["wi"], w["wo"], ohp, True,
                                  act_dtype, d_out, 1.5, nonpadding=nonpad,
-                                 num_microbatches=2)
+                                 num_microbatches=2, gate_noise=noise)
   assert not (want["aux"]["kept_1"] | want["aux"]["kept_2"]).all()
   tol = H.value_tolerance(act_dtype)
   for g_, k in zip(got, ("dx", "dw_gate", "dwi", "dwo")):
@@ -451,6 +500,8 @@ def test_v1_gradients_match_oracle(case):
     np.testing.assert_allclose(
         g_, ref, rtol=tol["rtol"], atol=tol["atol"] * max(1.0, np.abs(ref).max()),
         err_msg=k)
+  if noise_policy:
+    return        # a second step would draw new noise
   # a second step re-runs forward and backward on new tokens
   x2 = H.safe_tokens(rng, b * l, m, w["w_gate"], act_dtype,
                      top=4).reshape(b, l, m)

@@ -928,13 +928,13 @@ def test_switch_golden_fixture():
 
 
 # ---- backward -------------------------------------------------------------------
-def _f64_layer(x, wg, wi, wo, aux, gating, m1, coef, mb, z_loss):
+def _f64_layer(x, wg, wi, wo, aux, gating, m1, coef, mb, z_loss, mult=None):
   """Independent float64 forward of the v1 layer with the ROUTING HELD FIXED
   (experts, kept masks and density counts taken from `aux`): a smooth function
   of (x, wg, wi, wo) whose central differences pin the oracle's backward."""
   g, s, _ = x.shape
   e = wg.shape[1]
-  logits = x @ wg
+  logits = (x if mult is None else x * mult) @ wg     # the router's own input
   p = scipy.special.softmax(logits, axis=-1)
   rows = np.arange(g)[:, None], np.arange(s)[None, :]
   i1, i2 = aux["index_1"], aux["index_2"]
@@ -972,8 +972,11 @@ def _f64_layer(x, wg, wi, wo, aux, gating, m1, coef, mb, z_loss):
   return out, aux_loss * coef
 
 
-@pytest.mark.parametrize("gating", ["top_2", "switch", "switch_max", "ntlb"])
+@pytest.mark.parametrize("gating", ["top_2", "switch", "switch_max", "ntlb",
+                                    "switch+jitter", "switch+dropout",
+                                    "ntlb+jitter"])
 def test_backward_against_central_differences(gating):
+  gating, _, perturb = gating.partition("+")
   rng = np.random.default_rng(61)
   b, l, m, h, e, group = 2, 24, 6, 10, 4, 24
   x = rng.standard_normal((b, l, m)).astype(np.float32)
@@ -986,11 +989,18 @@ def test_backward_against_central_differences(gating):
   hp = _hp(moe_gating=gating, moe_num_experts=e, moe_hidden_size=h,
            moe_group_size=group, moe_capacity_factor_train=1.2,
            moe_min_expert_capacity=2, moe_loss_coef=0.5,
-           moe_switch_policy_train="argmax", moe_ntlb_top_k=3,
+           moe_switch_policy_train=("input_" + perturb) if perturb else "argmax",
+           moe_switch_jitter=0.3, moe_switch_dropout=0.25, moe_ntlb_top_k=3,
            moe_z_loss=0.3 if gating == "switch" else None)
+  noise = rng.random((b, l, m)).astype(np.float32) if perturb else None
   got = O.moe_layer_v1_backward(x, wg, wi, wo, hp, True, "float32", d_out,
-                                d_loss, nonpadding=nonpad, num_microbatches=mb)
+                                d_loss, nonpadding=nonpad, num_microbatches=mb,
+                                gate_noise=noise)
   aux = got["aux"]
+  mult = None
+  if perturb:
+    mult = aux["gate_mult"].astype(np.float64).reshape(b, l, m)
+    assert np.abs(mult - 1).max() > 0.05
   assert not (aux["kept_1"] | aux["kept_2"]).all()     # drops are exercised
   if gating == "ntlb":
     assert (aux["taken_in_pass"] > 0).any()        # tokens placed by a later choice
@@ -999,7 +1009,7 @@ def test_backward_against_central_differences(gating):
 
   def scalar(xv, wgv, wiv, wov):
     out, loss = _f64_layer(xv.reshape(b, l, m), wgv, wiv, wov, aux, gating, m1,
-                           0.5, mb, z)
+                           0.5, mb, z, mult)
     return (out * d_out.reshape(out.shape)).sum() + d_loss * loss
   base = [a.astype(np.float64) for a in (x.reshape(b, l, m), wg, wi, wo)]
   grads = [got["dx"].reshape(b, l, m), got["dw_gate"], got["dwi"], got["dwo"]]
@@ -1107,3 +1117,51 @@ def test_v2_backward_against_central_differences():
       fd = (scalar(*plus) - scalar(*minus)) / (2 * eps)
       an = float((grads[which].astype(np.float64) * d).sum())
       assert abs(fd - an) <= 1e-4 * max(1.0, abs(fd)), (which, trial, fd, an)
+
+
+def test_gate_input_perturbations():
+  """moe.py:1189-1199: the router (only) sees perturbed inputs while training.
+  jitter eps = 0 and eval mode change nothing; dropout with every u below
+  keep_prob scales the router's input, hence its logits, by 1 / keep_prob; the
+  experts always see the unperturbed tokens."""
+  rng = np.random.default_rng(77)
+  b, l, m, h, e = 2, 32, 8, 12, 4
+  x = rng.standard_normal((b, l, m)).astype(np.float32)
+  wg = rng.standard_normal((m, e)).astype(np.float32)
+  wi = rng.standard_normal((e, m, h)).astype(np.float32) / 3
+  wo = rng.standard_normal((e, h, m)).astype(np.float32) / 3
+  noise = rng.random((b, l, m)).astype(np.float32)
+  kw = dict(moe_gating="switch", moe_num_experts=e, moe_hidden_size=h,
+            moe_group_size=32, moe_switch_policy_eval="input_jitter")
+  base = O.moe_layer_v1(x, wg, wi, wo, _hp(moe_switch_policy_train="argmax", **kw),
+                        True, dense=False)
+  same = O.moe_layer_v1(x, wg, wi, wo,
+                        _hp(moe_switch_policy_train="input_jitter",
+                            moe_switch_jitter=0.0, **kw), True, dense=False,
+                        gate_noise=noise)
+  np.testing.assert_array_equal(base[0], same[0])
+  ev = O.moe_layer_v1(x, wg, wi, wo,
+                      _hp(moe_switch_policy_train="input_jitter", **kw), False,
+                      dense=False)                    # eval: no noise needed
+  assert ev[2]["gate_mult"] is None
+  jit = O.moe_layer_v1(x, wg, wi, wo,
+                       _hp(moe_switch_policy_train="input_jitter",
+                           moe_switch_jitter=0.5, **kw), True, dense=False,
+                       gate_noise=noise)
+  mult = jit[2]["gate_mult"]
+  assert mult.min() >= 0.5 and mult.max() < 1.5
+  np.testing.assert_allclose(jit[2]["logits"].reshape(b, l, e),
+                             (x.astype(np.float64) * mult.reshape(b, l, m)) @ wg,
+                             rtol=1e-5, atol=1e-5)
+  np.testing.assert_array_equal(                       # experts see x itself
+      jit[2]["expert_in"][jit[2]["index_1"][0, 0], 0, jit[2]["pos_1"][0, 0]]
+      if jit[2]["kept_1"][0, 0] else x[0, 0], x[0, 0])
+  drop = O.moe_layer_v1(x, wg, wi, wo,
+                        _hp(moe_switch_policy_train="input_dropout",
+                            moe_switch_dropout=0.2, **kw), True, dense=False,
+                        gate_noise=np.zeros_like(noise))
+  np.testing.assert_allclose(drop[2]["logits"], base[2]["logits"] / 0.8,
+                             rtol=1e-5, atol=1e-6)
+  with pytest.raises(NotImplementedError, match="gate_noise"):
+    O.moe_layer_v1(x, wg, wi, wo,
+                   _hp(moe_switch_policy_train="input_jitter", **kw), True)
