@@ -40,6 +40,12 @@ MoE file, and its TensorFlow dependency cannot run here):
                                       weights of a token sum to sum(p)/count,
                                       closed-form loss (uniform logits: 1.0),
                                       dense tensors vs slot record
+  perturb_gate_inputs                 closed forms (eps = 0 and eval change
+                                      nothing, all-kept dropout scales the
+                                      logits by 1 / keep_prob), the experts
+                                      see the unperturbed tokens; backward by
+                                      central differences with the multiplier
+                                      held fixed
   gating_backward,                    central differences of an independent
   moe_layer_v1_backward               float64 forward with the routing held
                                       fixed (tests/test_oracle.py)
@@ -47,7 +53,8 @@ MoE file, and its TensorFlow dependency cannot run here):
 
 PARITY UNPINNED against TensorFlow itself (only running the reference could
 pin these): near-tie behaviour of argmax after TF's exp/log, the accumulation
-order of TF's bf16 einsum, and the "random" second-place policy's RNG stream.
+order of TF's bf16 einsum, and the random streams (the "random" second-place
+policy, the router input noise): the uniform numbers are explicit inputs here.
 
 Citations are to files under the reference tree (mesh_tensorflow/...).
 """
