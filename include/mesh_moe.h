@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 7
+#define MESH_MOE_ABI_VERSION 8
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -137,12 +137,17 @@ int mesh_moe_router_top2_gating(
  * probability as the gate, per-group capacity positions with overflow drop,
  * load-balancing loss and (optionally) the router z-loss.
  * Replaces _switch_gating and _switch_max_gating after the router projection
- * for their deterministic policies -- "argmax", and "input_dropout" /
- * "input_jitter" outside training (transformer/moe.py:1207-1306, :976-1051;
- * z-loss :1253-1266).
+ * (transformer/moe.py:1207-1306, :976-1051; z-loss :1253-1266).  The policies
+ * "input_dropout" / "input_jitter" change the projection's input, which is
+ * the caller's business; policy "sample" passes choice_logits.
  * The per-token record has the layout of mesh_moe_top2_gating with the second
  * choice never kept (kept[..,1] = 0, gate[..,1] = 0), so mesh_moe_dispatch and
  * mesh_moe_combine apply unchanged.
+ *   choice_logits [G,S,E] float32 or NULL: when given, a token's expert is
+ *               the first arg-max of its row here instead of the arg-max of
+ *               the probabilities, and the gate is the probability of that
+ *               expert (policy "sample", moe.py:1213-1216: the caller passes
+ *               logits + Gumbel noise * temperature, ops.py:5070-5086)
  *   importance [G,S] of importance_dtype or NULL: only tokens with
  *               importance == 1 are routed (moe.py:1226-1231)
  *   slots_by_gate  0: an expert's slots go to its choosers in token order,
@@ -158,8 +163,9 @@ int mesh_moe_router_top2_gating(
  * Limits as mesh_moe_top2_gating; workspace from
  * mesh_moe_gating_workspace_bytes.
  */
-int mesh_moe_switch_gating(const float* logits, const void* importance,
-                           int importance_dtype, int G, int S, int E, int C,
+int mesh_moe_switch_gating(const float* logits, const float* choice_logits,
+                           const void* importance, int importance_dtype, int G,
+                           int S, int E, int C,
                            int slots_by_gate, int use_z_loss,
                            double z_loss_coef,
                            int num_microbatches, int32_t* idx, int32_t* pos,

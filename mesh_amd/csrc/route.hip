@@ -261,6 +261,21 @@ __device__ __forceinline__ void gate_select_tile(
       if (pe > g1) { g1 = pe; i1 = e; }                     // first argmax
     }
     sel1 = true;
+    if (p.router == ROUTER_SWITCH && second_uniform != nullptr) {
+      // policy "sample" (moe.py:1213-1216): the expert is the first arg-max of
+      // the caller's choice logits [G,S,E] (router logits plus Gumbel noise
+      // times the temperature, ops.py:5070-5086), which arrive through the
+      // pointer the top-2 mode uses for its uniform samples; the gate is the
+      // softmax probability of that expert (mtf.gather of raw_gates)
+      const float* ch = second_uniform + t * E;
+      float best = ch[0];
+      i1 = 0;
+      for (int e = 1; e < E; ++e) {
+        const float v = ch[e];
+        if (v > best) { best = v; i1 = e; }
+      }
+      g1 = row[i1];
+    }
     if (p.router == ROUTER_SWITCH) {
       // one choice, raw probability as the gate (moe.py:1207-1228); the load
       // balancing loss counts every token's arg-max (density_1 is taken
@@ -1017,8 +1032,9 @@ extern "C" int mesh_moe_router_top2_gating(
 }
 
 extern "C" int mesh_moe_switch_gating(
-    const float* logits, const void* importance, int importance_dtype, int G,
-    int S, int E, int C, int slots_by_gate, int use_z_loss, double z_loss_coef,
+    const float* logits, const float* choice_logits, const void* importance,
+    int importance_dtype, int G, int S, int E, int C, int slots_by_gate,
+    int use_z_loss, double z_loss_coef,
     int num_microbatches, int32_t* idx, int32_t* pos, float* gate,
     uint8_t* kept, int32_t* fill, float* loss, void* workspace,
     size_t workspace_bytes, void* stream) {
@@ -1030,8 +1046,9 @@ extern "C" int mesh_moe_switch_gating(
   GateParams p = make_switch_params(G, S, E, C, importance, slots_by_gate,
                                     use_z_loss, z_loss_coef, num_microbatches,
                                     gate_tokens_per_block(E));
-  return run_gating(p, logits, importance, importance_dtype, nullptr, idx, pos,
-                    gate, kept, fill, loss, workspace, (hipStream_t)stream);
+  return run_gating(p, logits, importance, importance_dtype, choice_logits,
+                    idx, pos, gate, kept, fill, loss, workspace,
+                    (hipStream_t)stream);
 }
 
 extern "C" int mesh_moe_router_switch_gating(

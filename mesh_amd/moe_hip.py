@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -45,7 +45,7 @@ _SIGNATURES = {
         ctypes.c_double, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, _vp, _vp,
         _vp, _vp, ctypes.c_size_t, _vp]),
     "mesh_moe_switch_gating": (ctypes.c_int, [
-        _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_double,
         ctypes.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_size_t,
         _vp]),
@@ -392,8 +392,13 @@ def _routing_buffers(lib, g, s, e, dev):
 
 
 def switch_gating(logits, capacity, importance=None, z_loss=None,
-                  num_microbatches=None, slots_by_gate=False):
+                  num_microbatches=None, slots_by_gate=False,
+                  choice_logits=None):
   """logits float32 [G, S, E] -> Routing for switch (top-1) gating.
+
+  choice_logits float32 [G, S, E]: when given, the expert of a token is the
+  first arg-max of its row there (policy "sample", transformer/moe.py:1213-1216)
+  and the gate is the softmax probability of that expert.
 
   z_loss: coefficient of the router z-loss, or None to leave it out (the
   caller passes it only when training, transformer/moe.py:1253).
@@ -409,8 +414,10 @@ def switch_gating(logits, capacity, importance=None, z_loss=None,
   idx, pos, gate, kept, fill, loss, ws, ws_bytes = _routing_buffers(
       lib, g, s, e, logits.device)
   with _stage("switch_gating"):
+    cp = None if choice_logits is None else _dev(
+        choice_logits, "choice_logits", torch.float32, (g, s, e))
     _check(lib.mesh_moe_switch_gating(
-        lp, ip, icode, g, s, e, int(capacity), int(bool(slots_by_gate)),
+        lp, cp, ip, icode, g, s, e, int(capacity), int(bool(slots_by_gate)),
         int(z_loss is not None), float(z_loss or 0.0),
         int(num_microbatches or 1), idx.data_ptr(),
         pos.data_ptr(), gate.data_ptr(), kept.data_ptr(), fill.data_ptr(),

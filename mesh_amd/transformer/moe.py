@@ -9,8 +9,8 @@ reference expands the layer into ~100 graph primitives and dense one-hot
 the HIP kernels: router -> top-2 gating -> dispatch -> expert FFN -> combine.
 
 Built: moe_gating "top_2" (every second-place policy, the second-place loss),
-"switch", "switch_max", "ntlb" and "expert_selection" (switch policies
-"argmax", "input_jitter", "input_dropout"; not "sample"); nonpadding / importance; moe_use_experts_attention; float32 and
+"switch", "switch_max", "ntlb" and "expert_selection" with their switch
+policies ("argmax", "sample", "input_jitter", "input_dropout"); nonpadding / importance; moe_use_experts_attention; float32 and
 bfloat16; mtf.gradients over the v1 layer (top_2 / switch / switch_max / ntlb,
 ReLU or linear experts) and the v2 layer.  Not built (they raise NotImplementedError):
 expert dropout while training, gated (list) activations, gradients of the
@@ -223,7 +223,7 @@ def _router_logits(x_gate, w, w_packed):
 
 class _SwitchGatingSpec(object):
   """Static configuration of one _switch_gating (moe.py:1176-1309) or
-  _switch_max_gating (moe.py:943-1054) call for the policies "argmax",
+  _switch_max_gating (moe.py:943-1054) call: policies "argmax", "sample",
   "input_dropout" and "input_jitter" (the perturbations apply while training,
   moe.py:1192-1199)."""
 
@@ -231,12 +231,11 @@ class _SwitchGatingSpec(object):
     self.slots_by_gate = hparams.moe_gating == "switch_max"
     policy = (hparams.moe_switch_policy_train if train
               else hparams.moe_switch_policy_eval)
-    if policy == "sample":
-      raise NotImplementedError(
-          "switch policy %r (sampling the expert) is not implemented"
-          % (policy,))
-    if policy not in ("argmax", "input_dropout", "input_jitter"):
+    if policy not in ("argmax", "input_dropout", "input_jitter", "sample"):
       raise ValueError("Unknown Switch gating policy %s" % policy)
+    # policy "sample" (moe.py:1213-1216): temperature 0 is the arg-max
+    self.temperature = (float(hparams.moe_switch_temperature)
+                        if policy == "sample" else 0.0)
     self.noise = _GateInputNoise(hparams, train, in_float32=True)
     self.z_loss = None                     # _switch_max_gating has no z-loss
     if (train and not self.slots_by_gate and
@@ -259,18 +258,25 @@ class _SwitchGatingSpec(object):
     b, t, _ = x.shape
     groups = b * t // group_size
     x_gate = self.noise.apply(x)
-    if x_gate is x and moe_hip.fused_gating_supported(x, num_experts,
-                                                      group_size):
+    if (x_gate is x and self.temperature == 0.0 and
+        moe_hip.fused_gating_supported(x, num_experts, group_size)):
       return moe_hip.router_switch_gating(
           x, w_packed, group_size, capacity, importance=importance,
           z_loss=self.z_loss, num_microbatches=self.num_microbatches,
           slots_by_gate=self.slots_by_gate, want_logits=want_logits)
     logits = _router_logits(x_gate, w, w_packed)
     logits = logits.reshape(groups, group_size, num_experts)
+    choice = None
+    if self.temperature != 0.0:
+      # mtf.sample_with_temperature (ops.py:5070-5086): Gumbel noise from
+      # u in [1e-9, 1), arg-max of logits + noise * temperature
+      u = torch.rand(logits.shape, dtype=torch.float32, device=logits.device)
+      u = 1e-9 + u * (1.0 - 1e-9)
+      choice = logits + (-torch.log(-torch.log(u))) * self.temperature
     r = moe_hip.switch_gating(
         logits, capacity, importance=importance, z_loss=self.z_loss,
         num_microbatches=self.num_microbatches,
-        slots_by_gate=self.slots_by_gate)
+        slots_by_gate=self.slots_by_gate, choice_logits=choice)
     return (r, logits) if want_logits else r
 
 

@@ -299,8 +299,22 @@ def top_2_gating(logits, capacity, importance=None, policy="all",
 # ----------------------------------------------------------------------------
 # _switch_gating  (transformer/moe.py:1176-1309)
 # ----------------------------------------------------------------------------
+def sample_choice_logits(logits, temperature, uniform):
+  """mtf.sample_with_temperature before its argmax (ops.py:5070-5086): logits +
+  g * temperature with Gumbel noise g = -log(-log(u)), u in [1e-9, 1).
+  `uniform` stands in for random_uniform's U[0, 1) draw."""
+  logits = np.asarray(logits, F32)
+  if temperature == 0.0:
+    return logits
+  tiny = F32(1e-9)
+  u = tiny + np.asarray(uniform, F32) * (F32(1.0) - tiny)
+  g = -np.log(-np.log(u).astype(F32)).astype(F32)
+  return (logits + g * F32(temperature)).astype(F32)
+
+
 def switch_gating(logits, capacity, importance=None, train=False, z_loss=None,
-                  num_microbatches=None, act_dtype="float32", dense=False):
+                  num_microbatches=None, act_dtype="float32", dense=False,
+                  choice_logits=None):
   """Everything in _switch_gating after the router projection, for the
   deterministic policies ("argmax"; "input_dropout" / "input_jitter" when not
   training, where they change nothing, moe.py:1192-1199).
@@ -318,7 +332,12 @@ def switch_gating(logits, capacity, importance=None, train=False, z_loss=None,
   cap_f = F32(float(capacity))
 
   raw_gates = softmax(logits)                                    # :1207
-  expert_gate, expert_index = top_1(raw_gates)                   # :1210
+  if choice_logits is None:
+    expert_gate, expert_index = top_1(raw_gates)                 # :1210
+  else:    # policy "sample" (:1213-1216): argmax elsewhere, gate gathered
+    expert_index = np.argmax(np.asarray(choice_logits, F32), -1).astype(np.int32)
+    expert_gate = np.take_along_axis(raw_gates, expert_index[..., None],
+                                     -1)[..., 0]
   expert_mask = one_hot(expert_index, e_)                        # :1221
 
   # load balancing loss (:1224-1238).  density_1 is taken BEFORE the
@@ -402,7 +421,8 @@ def top_k_lowest_index_first(x, k, axis):
 
 
 def switch_max_gating(logits, capacity, importance=None,
-                      num_microbatches=None, act_dtype="float32", dense=False):
+                      num_microbatches=None, act_dtype="float32", dense=False,
+                      choice_logits=None):
   """Everything in _switch_max_gating after the router projection, for the
   deterministic policies (as switch_gating).
 
@@ -417,7 +437,12 @@ def switch_max_gating(logits, capacity, importance=None,
   logits = np.asarray(logits, dtype=F32)
   g_, s_, e_ = logits.shape
   raw_gates = softmax(logits)                                    # :976
-  expert_gate, expert_index = top_1(raw_gates)                   # :979
+  if choice_logits is None:
+    expert_gate, expert_index = top_1(raw_gates)                 # :979
+  else:                                                          # :982-985
+    expert_index = np.argmax(np.asarray(choice_logits, F32), -1).astype(np.int32)
+    expert_gate = np.take_along_axis(raw_gates, expert_index[..., None],
+                                     -1)[..., 0]
   expert_mask = one_hot(expert_index, e_)                        # :990
   inv_s = F32(1.0 / s_)
   density_1 = seq_sum(expert_mask, axis=-2) * inv_s              # :994
@@ -840,7 +865,7 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
                  nonpadding=None, activation="relu", num_microbatches=None,
                  logit_bias=None, second_uniform=None, dense=True,
                  mesh_dim_size=1, weights_are_cast=False, k_wo=None,
-                 gate_noise=None):
+                 gate_noise=None, sample_uniform=None):
   """transformer_moe_layer_v1 forward (transformer/moe.py:191-525).
 
   x: [batch..., length, M] float32 array holding activation-dtype values.
@@ -865,7 +890,8 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
     kw = dict(nonpadding=nonpadding, activation=activation,
               num_microbatches=num_microbatches, logit_bias=logit_bias,
               second_uniform=second_uniform, dense=dense,
-              mesh_dim_size=mesh_dim_size, weights_are_cast=weights_are_cast)
+              mesh_dim_size=mesh_dim_size, weights_are_cast=weights_are_cast,
+              gate_noise=gate_noise, sample_uniform=sample_uniform)
     # the two outputs share everything up to the hidden tensor, so each equals
     # the plain layer with its own output kernel
     q, loss, aux = moe_layer_v1(x, w_gate, wi, wo, hp1, train, act_dtype, **kw)
@@ -927,19 +953,27 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
             _scale_loss(r["loss"], hp.moe_loss_coef, act_dtype), aux)
   if hp.moe_gating in ("switch", "switch_max", "ntlb"):          # :393-424
     sw = hp.moe_switch_policy_train if train else hp.moe_switch_policy_eval
-    if sw == "sample":
-      raise NotImplementedError("switch policy %r draws random numbers" % sw)
-    if sw not in ("argmax", "input_dropout", "input_jitter"):
+    if sw not in ("argmax", "input_dropout", "input_jitter", "sample"):
       raise ValueError("Unknown Switch gating policy %s" % sw)
+    choice = None
+    if sw == "sample" and hp.moe_gating != "ntlb" and (
+        hp.moe_switch_temperature != 0.0):
+      if sample_uniform is None:
+        raise NotImplementedError(
+            "switch policy 'sample' needs the random tensor (sample_uniform)")
+      choice = sample_choice_logits(
+          logits, hp.moe_switch_temperature,
+          np.asarray(sample_uniform, F32).reshape(logits.shape))
     if hp.moe_gating == "switch":
       r = switch_gating(logits, c_, importance, train, hp.moe_z_loss,
-                        num_microbatches, act_dtype, dense=dense)
+                        num_microbatches, act_dtype, dense=dense,
+                        choice_logits=choice)
     elif hp.moe_gating == "ntlb":
       r = ntlb_gating(logits, c_, hp.moe_ntlb_top_k, importance,
                       num_microbatches, act_dtype, dense=dense)
     else:
       r = switch_max_gating(logits, c_, importance, num_microbatches,
-                            act_dtype, dense=dense)
+                            act_dtype, dense=dense, choice_logits=choice)
   else:
     policy, threshold = _policy(hp, train)
     r = top_2_gating(logits, c_, importance, policy, threshold,
@@ -1104,7 +1138,7 @@ def expert_ffn_backward(xe, wi_a, wo_a, dy, activation, act_dtype):
 def moe_layer_v1_backward(x, w_gate, wi, wo, hp, train, act_dtype, d_out,
                           d_loss=0.0, nonpadding=None, activation="relu",
                           num_microbatches=None, logit_bias=None,
-                          gate_noise=None):
+                          gate_noise=None, sample_uniform=None):
   """Gradients of (outputs, loss) of moe_layer_v1 w.r.t. x and the three
   kernels, given d_out [batch..., length, N] and the scalar d_loss.
 
@@ -1127,7 +1161,8 @@ def moe_layer_v1_backward(x, w_gate, wi, wo, hp, train, act_dtype, d_out,
                            nonpadding=nonpadding, activation=activation,
                            num_microbatches=num_microbatches,
                            logit_bias=logit_bias, dense=False,
-                           gate_noise=gate_noise)
+                           gate_noise=gate_noise,
+                           sample_uniform=sample_uniform)
   x = cast_act(x, act_dtype)
   lead, m_ = x.shape[:-1], x.shape[-1]
   g_, s_, c_ = aux["num_groups"], aux["group_size"], aux["capacity"]

@@ -202,7 +202,8 @@ def test_error_behaviour():
     moe.transformer_moe_layer_v1(x, dims[-1], hparams(moe_gating="switch"), True, vdt)
   sw = dict(moe_gating="switch", moe_switch_policy_train="argmax",
             moe_switch_policy_eval="sample", moe_z_loss=None)
-  with pytest.raises(NotImplementedError, match="sampling"):
+  # sampling reads its temperature, as the reference does (moe.py:1214-1215)
+  with pytest.raises(AttributeError, match="moe_switch_temperature"):
     moe.transformer_moe_layer_v1(x, dims[-1], hparams(**sw), False, vdt)
   with pytest.raises(ValueError, match="Unknown Switch gating policy"):
     moe.transformer_moe_layer_v1(

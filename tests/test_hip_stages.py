@@ -379,6 +379,26 @@ def test_switch_gating_random_logits(hip, shape):
   np.testing.assert_allclose(got["loss"], want["loss"], rtol=2e-5)
 
 
+def test_switch_gating_choice_logits(hip):
+  """Policy "sample": experts from the arg-max of separate choice logits, gates
+  from the probabilities, for both slot orders."""
+  g, s, e, c = 3, 400, 16, 30
+  rng = np.random.default_rng(14)
+  logits = H.safe_logits(rng, g, s, e)
+  u = rng.random((g, s, e)).astype(np.float32)
+  choice = O.sample_choice_logits(logits, 1.0, u)
+  imp = rng.choice(np.array([0.0, 1.0], np.float32), size=(g, s), p=[0.2, 0.8])
+  lg, ch = torch.from_numpy(logits).cuda(), torch.from_numpy(choice).cuda()
+  want = O.switch_gating(logits, c, importance=imp, choice_logits=choice)
+  assert (want["index_1"] != logits.argmax(-1)).mean() > 0.2
+  got = H.routing_to_np(hip.switch_gating(lg, c, importance=H.to_gpu(imp),
+                                          choice_logits=ch))
+  H.assert_routing_equal(got, want)
+  np.testing.assert_allclose(got["loss"], want["loss"], rtol=2e-5)
+  with pytest.raises(hip.MoeHipError, match="choice_logits"):
+    hip.switch_gating(lg, c, choice_logits=ch[:, :, :8].contiguous())
+
+
 def test_switch_gating_exact_ties(hip):
   g, s, e, c = 3, 500, 64, 9
   rng = np.random.default_rng(8)

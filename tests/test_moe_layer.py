@@ -308,10 +308,6 @@ def test_v1_switch_rejections():
            wo=np.zeros((4, 8, 16), np.float32))
   base = dict(moe_num_experts=4, moe_hidden_size=8, moe_group_size=32)
   hp, _ = make_hparams(**dict(base, **dict(SWITCH_HP,
-                                          moe_switch_policy_eval="sample")))
-  with pytest.raises(NotImplementedError, match="sampling"):
-    run_v1(x, w, hp, False, "float32")
-  hp, _ = make_hparams(**dict(base, **dict(SWITCH_HP,
                                           moe_switch_policy_eval="bogus")))
   with pytest.raises(ValueError, match="Unknown Switch gating policy"):
     run_v1(x, w, hp, False, "float32")
@@ -352,7 +348,8 @@ def test_v1_ntlb_matches_oracle(act_dtype):
 @pytest.mark.parametrize("case", [
     ("switch", "input_jitter", "float32"), ("switch", "input_jitter", "bfloat16"),
     ("switch", "input_dropout", "float32"), ("ntlb", "input_jitter", "bfloat16"),
-    ("switch_max", "input_dropout", "bfloat16")],
+    ("switch_max", "input_dropout", "bfloat16"),
+    ("switch", "sample", "float32"), ("switch_max", "sample", "bfloat16")],
     ids=lambda c: "-".join(c))
 def test_v1_router_input_noise_matches_oracle(case):
   """Training with the perturbing switch policies: the layer draws u ~ U[0,1)
@@ -366,19 +363,26 @@ def test_v1_router_input_noise_matches_oracle(case):
            wo=H.normal_weights(rng, (e, hdim, m), hdim))
   x = O.cast_act(rng.standard_normal((b, l, m)).astype(np.float32), act_dtype)
   kw = dict(SWITCH_HP, moe_gating=gating, moe_switch_policy_train=policy,
-            moe_switch_jitter=0.25, moe_switch_dropout=0.3, moe_ntlb_top_k=2)
+            moe_switch_jitter=0.25, moe_switch_dropout=0.3, moe_ntlb_top_k=2,
+            moe_switch_temperature=1.5)
   hp, ohp = make_hparams(moe_num_experts=e, moe_hidden_size=hdim,
                          moe_group_size=group, moe_capacity_factor_train=1.0,
                          **kw)
   torch.manual_seed(99)
   got, got_loss, _, _ = run_v1(x, w, hp, True, act_dtype, num_microbatches=2)
   torch.manual_seed(99)
-  u = torch.rand((1, b * l, m), dtype=torch.float32, device="cuda")
-  noise = u.cpu().numpy().reshape(b, l, m)
+  noise = su = None
+  if policy == "sample":
+    su = torch.rand((b * l // group, group, e), dtype=torch.float32,
+                    device="cuda").cpu().numpy()
+  else:
+    noise = torch.rand((1, b * l, m), dtype=torch.float32,
+                       device="cuda").cpu().numpy().reshape(b, l, m)
   want, want_loss, aux = O.moe_layer_v1(x, w["w_gate"], w["wi"], w["wo"], ohp,
                                         True, act_dtype, num_microbatches=2,
-                                        dense=False, gate_noise=noise)
-  assert aux["gate_mult"] is not None
+                                        dense=False, gate_noise=noise,
+                                        sample_uniform=su)
+  assert (aux["gate_mult"] is not None) == (policy != "sample")
   plain, _, aux0 = O.moe_layer_v1(
       x, w["w_gate"], w["wi"], w["wo"],
       make_hparams(moe_num_experts=e, moe_hidden_size=hdim,
@@ -389,6 +393,8 @@ def test_v1_router_input_noise_matches_oracle(case):
   np.testing.assert_allclose(got, want, **H.value_tolerance(act_dtype))
   np.testing.assert_allclose(got_loss, want_loss,
                              rtol=1e-2 if act_dtype == "bfloat16" else 1e-4)
+  if policy == "sample":
+    return          # the eval policy of SWITCH_HP is another one
   # evaluation draws nothing: same result whatever the generator's state
   a, _, _, _ = run_v1(x, w, hp, False, act_dtype)
   torch.manual_seed(5)

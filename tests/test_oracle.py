@@ -974,7 +974,7 @@ def _f64_layer(x, wg, wi, wo, aux, gating, m1, coef, mb, z_loss, mult=None):
 
 @pytest.mark.parametrize("gating", ["top_2", "switch", "switch_max", "ntlb",
                                     "switch+jitter", "switch+dropout",
-                                    "ntlb+jitter"])
+                                    "ntlb+jitter", "switch+sample"])
 def test_backward_against_central_differences(gating):
   gating, _, perturb = gating.partition("+")
   rng = np.random.default_rng(61)
@@ -989,16 +989,21 @@ def test_backward_against_central_differences(gating):
   hp = _hp(moe_gating=gating, moe_num_experts=e, moe_hidden_size=h,
            moe_group_size=group, moe_capacity_factor_train=1.2,
            moe_min_expert_capacity=2, moe_loss_coef=0.5,
-           moe_switch_policy_train=("input_" + perturb) if perturb else "argmax",
+           moe_switch_policy_train=("sample" if perturb == "sample" else
+                                    "input_" + perturb) if perturb else "argmax",
+           moe_switch_temperature=2.0,
            moe_switch_jitter=0.3, moe_switch_dropout=0.25, moe_ntlb_top_k=3,
            moe_z_loss=0.3 if gating == "switch" else None)
   noise = rng.random((b, l, m)).astype(np.float32) if perturb else None
+  su = rng.random((b * l // group, group, e)).astype(np.float32)
   got = O.moe_layer_v1_backward(x, wg, wi, wo, hp, True, "float32", d_out,
                                 d_loss, nonpadding=nonpad, num_microbatches=mb,
-                                gate_noise=noise)
+                                gate_noise=noise, sample_uniform=su)
   aux = got["aux"]
   mult = None
-  if perturb:
+  if perturb == "sample":       # sampled experts differ from the arg-max
+    assert (aux["index_1"] != aux["logits"].argmax(-1)).any()
+  elif perturb:
     mult = aux["gate_mult"].astype(np.float64).reshape(b, l, m)
     assert np.abs(mult - 1).max() > 0.05
   assert not (aux["kept_1"] | aux["kept_2"]).all()     # drops are exercised
@@ -1165,3 +1170,36 @@ def test_gate_input_perturbations():
   with pytest.raises(NotImplementedError, match="gate_noise"):
     O.moe_layer_v1(x, wg, wi, wo,
                    _hp(moe_switch_policy_train="input_jitter", **kw), True)
+
+
+def test_switch_sample_policy():
+  """moe.py:1213-1216 with ops.py:5070-5086: the expert is the arg-max of
+  logits + Gumbel(u) * temperature, the gate the softmax probability of that
+  expert.  Temperature 0 is the arg-max policy; u -> 1 at one expert (a huge
+  Gumbel value) forces that expert."""
+  rng = np.random.default_rng(88)
+  g, s, e, c = 2, 40, 5, 100
+  logits = rng.standard_normal((g, s, e)).astype(np.float32)
+  u = rng.random((g, s, e)).astype(np.float32)
+  np.testing.assert_array_equal(O.sample_choice_logits(logits, 0.0, u), logits)
+  ch = O.sample_choice_logits(logits, 1.5, u)
+  u64 = 1e-9 + u.astype(np.float64) * (1 - 1e-9)
+  np.testing.assert_allclose(ch, logits - 1.5 * np.log(-np.log(u64)),
+                             rtol=1e-4, atol=1e-4)   # float32 logs of u near 1
+  forced = np.full((g, s, e), 0.5, np.float32)
+  target = rng.integers(0, e, size=(g, s))
+  np.put_along_axis(forced, target[..., None], np.float32(1 - 1e-7), -1)
+  r = O.switch_gating(logits, c,
+                      choice_logits=O.sample_choice_logits(logits, 50.0, forced))
+  np.testing.assert_array_equal(r["index_1"], target)
+  p = scipy.special.softmax(logits.astype(np.float64), -1)
+  np.testing.assert_allclose(
+      r["gate_1"], np.take_along_axis(p, target[..., None], -1)[..., 0],
+      rtol=2e-6)
+  # the loss counts the sampled experts
+  dens = (target[..., None] == np.arange(e)).mean(1)
+  np.testing.assert_allclose(r["loss"], e * e * (p.mean(1) * dens).mean(),
+                             rtol=1e-5)
+  rm = O.switch_max_gating(logits, s, choice_logits=O.sample_choice_logits(
+      logits, 50.0, forced))
+  np.testing.assert_array_equal(rm["index_1"], target)
