@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 8
+#define MESH_MOE_ABI_VERSION 9
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -243,6 +243,28 @@ int mesh_moe_expert_ffn(const void* expert_in, const void* wi_packed,
 int mesh_moe_expert_linear(const void* a, const void* w_packed, void* y, int E,
                            int R, int K, int N, int activation, int dtype,
                            void* stream);
+
+/* Bytes of scratch mesh_moe_dispatched_expert_ffn needs. */
+size_t mesh_moe_dispatched_expert_ffn_workspace_bytes(int G, int E, int C,
+                                                      int M);
+
+/*
+ * mesh_moe_dispatch + mesh_moe_expert_ffn in one call that never writes
+ * expert_in: the first GEMM fetches each slot's token row straight from x
+ * through a slot -> token map built from the routing record (empty slots and
+ * kept choices whose gate rounds to 0 read a zero row).  Same h and y as the
+ * two calls.  For callers that do not need expert_in afterwards (inference;
+ * the backward reads it).  bf16 only, and only where the first GEMM
+ * ([G*C, M] x [M, H] per expert) fits the 256 x 256 direct-to-LDS kernel;
+ * otherwise MESH_MOE_E_UNSUPPORTED with nothing launched: make the two calls.
+ *   x [G,S,M] dtype; idx, pos, gate, kept as written by the gating calls
+ *   h [E,G*C,H], y [E,G*C,N] dtype
+ */
+int mesh_moe_dispatched_expert_ffn(
+    const void* x, const int32_t* idx, const int32_t* pos, const float* gate,
+    const uint8_t* kept, const void* wi_packed, const void* wo_packed, void* h,
+    void* y, void* workspace, size_t workspace_bytes, int G, int S, int E, int C,
+    int M, int H, int N, int activation, int dtype, void* stream);
 
 /*
  * Combine: out[g,s,:] = w1 * y[idx1,g,pos1,:] + w2 * y[idx2,g,pos2,:] with

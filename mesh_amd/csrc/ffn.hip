@@ -519,11 +519,16 @@ struct RingCfg {
   static_assert(A_INSTR == 4 && B_INSTR == 4, "load schedule assumes 4 + 4");
 };
 
-template <bool RELU>
+// GATHER: the rows of expert e's first operand are not A[e][r] but rows of a
+// shared token matrix, A[row_map[e * R + r]] (row_map < 0: the all-zero row
+// `zero_row`): the dispatch of the Mixture-of-Experts layer folded into the
+// first expert GEMM's loads.
+template <bool RELU, bool GATHER = false>
 __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
     bf16_t* __restrict__ Cout, int R, int N, int K, int tiles_m, int tiles_n,
-    int total_tiles) {
+    int total_tiles, const int32_t* __restrict__ row_map = nullptr,
+    const bf16_t* __restrict__ zero_row = nullptr) {
   using Cfg = RingCfg;
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, WN = Cfg::WN;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -560,7 +565,8 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
   int row0, col0;
   const bf16_t *Ae, *Be;
   bf16_t* Ce;
-  int a_off[Cfg::A_INSTR], b_off[Cfg::B_INSTR];
+  typename std::conditional<GATHER, int64_t, int>::type a_off[Cfg::A_INSTR];
+  int b_off[Cfg::B_INSTR];
   auto set_tile = [&](int logical) {
     const int e = logical / tiles_per_e;
     const int rem = logical - e * tiles_per_e;
@@ -568,14 +574,20 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
     const int tm = rem - tn * tiles_m;
     row0 = tm * BM;
     col0 = tn * BN;
-    Ae = A + (int64_t)e * R * K;
+    Ae = GATHER ? A : A + (int64_t)e * R * K;
     Be = B + (int64_t)e * N * K;
     Ce = Cout + (int64_t)e * R * N;
 #pragma unroll
     for (int j = 0; j < Cfg::A_INSTR; ++j) {
       const int row = (wave + Cfg::WAVES * j) * 8 + (lane >> 3);
       const int chunk = (lane & 7) ^ lds_swizzle(row);
-      a_off[j] = min(row0 + row, R - 1) * K + chunk * 8;
+      if constexpr (GATHER) {
+        const int src = row_map[(int64_t)e * R + min(row0 + row, R - 1)];
+        a_off[j] = (src >= 0 ? (int64_t)src * K : (int64_t)(zero_row - A)) +
+                   chunk * 8;
+      } else {
+        a_off[j] = min(row0 + row, R - 1) * K + chunk * 8;
+      }
       b_off[j] = min(col0 + row, N - 1) * K + chunk * 8;
     }
   };
@@ -941,7 +953,9 @@ static int launch_dma(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
 }
 
 static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
-                       int R, int N, int K, bool relu, hipStream_t st) {
+                       int R, int N, int K, bool relu, hipStream_t st,
+                       const int32_t* row_map = nullptr,
+                       const bf16_t* zero_row = nullptr) {
   using Cfg = RingCfg;
   const int tiles_m = (R + Cfg::BM - 1) / Cfg::BM;
   const int tiles_n = (N + Cfg::BN - 1) / Cfg::BN;
@@ -961,16 +975,31 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
     cus = n;
   }
   const unsigned blocks = (unsigned)(tiles < cus ? tiles : cus);
+  if (row_map != nullptr) {
+    if (relu) {
+      auto k = grouped_gemm_bf16_ring_kernel<true, true>;
+      MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
+      k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
+          A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, row_map, zero_row);
+    } else {
+      auto k = grouped_gemm_bf16_ring_kernel<false, true>;
+      MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
+      k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
+          A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, row_map, zero_row);
+    }
+    MOE_CHECK_LAUNCH("expert_ffn (mfma, gathered rows)");
+    return 0;
+  }
   if (relu) {
-    auto k = grouped_gemm_bf16_ring_kernel<true>;
+    auto k = grouped_gemm_bf16_ring_kernel<true, false>;
     MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
-    k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(A, B, C, R, N, K, tiles_m,
-                                                    tiles_n, (int)tiles);
+    k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
+        A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr);
   } else {
-    auto k = grouped_gemm_bf16_ring_kernel<false>;
+    auto k = grouped_gemm_bf16_ring_kernel<false, false>;
     MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
-    k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(A, B, C, R, N, K, tiles_m,
-                                                    tiles_n, (int)tiles);
+    k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
+        A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr);
   }
   MOE_CHECK_LAUNCH("expert_ffn (mfma, spread direct-to-LDS loads)");
   return 0;
@@ -1086,6 +1115,100 @@ extern "C" int mesh_moe_expert_ffn(const void* expert_in, const void* wi_packed,
   int rc = grouped_gemm(expert_in, wi_packed, h, E, R, H, M, activation, dtype,
                         st);
   if (rc != 0) return rc;
+  return grouped_gemm(h, wo_packed, y, E, R, N, H, MESH_MOE_ACT_LINEAR, dtype,
+                      st);
+}
+
+// ---------------------------------------------------------------------------
+// Dispatch folded into the first expert GEMM: slot -> token map.
+// ---------------------------------------------------------------------------
+__global__ void slot_map_clear_kernel(int32_t* map, int64_t n, bf16_t* zero_row,
+                                      int m) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  const int64_t i0 = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  for (int64_t i = i0; i < n; i += stride) map[i] = -1;
+  for (int64_t i = i0; i < m; i += stride) zero_row[i] = 0;
+}
+
+// one thread per (token, choice): a kept choice whose activation-dtype gate is
+// not 0 owns slot [idx][g][pos] (transformer/moe.py:1510-1511: the dispatch
+// tensor is the combine tensor cast to bool)
+__global__ void slot_map_kernel(const int32_t* __restrict__ idx,
+                                const int32_t* __restrict__ pos,
+                                const float* __restrict__ gate,
+                                const uint8_t* __restrict__ kept,
+                                int32_t* __restrict__ map, int64_t tokens,
+                                int S, int C, int64_t rows_per_expert) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= tokens * 2) return;
+  if (!kept[i] || round_to<bf16_t>(gate[i]) == 0.0f) return;
+  const int64_t t = i >> 1;
+  const int64_t g = t / S;
+  map[(int64_t)idx[i] * rows_per_expert + g * C + pos[i]] = (int32_t)t;
+}
+
+static bool ring_path_applies(int R, int N, int K) {
+  const int pad256 = (R + 255) / 256 * 256, pad128 = (R + 127) / 128 * 128;
+  return N >= 256 && R >= 128 && K % 64 == 0 && K % 8 == 0 && N % 8 == 0 &&
+         pad128 >= pad256 && (int64_t)N * K < (1LL << 31);
+}
+
+extern "C" size_t mesh_moe_dispatched_expert_ffn_workspace_bytes(int G, int E,
+                                                                 int C, int M) {
+  if (G < 1 || E < 1 || C < 1 || M < 1) return 0;
+  return sizeof(int32_t) * (size_t)E * G * C + sizeof(bf16_t) * (size_t)M + 512;
+}
+
+extern "C" int mesh_moe_dispatched_expert_ffn(
+    const void* x, const int32_t* idx, const int32_t* pos, const float* gate,
+    const uint8_t* kept, const void* wi_packed, const void* wo_packed, void* h,
+    void* y, void* workspace, size_t workspace_bytes, int G, int S, int E, int C,
+    int M, int H, int N, int activation, int dtype, void* stream) {
+  MOE_REQUIRE(x && idx && pos && gate && kept && wi_packed && wo_packed && h &&
+                  y && workspace, MESH_MOE_E_ARG,
+              "dispatched_expert_ffn: null pointer");
+  MOE_REQUIRE(G >= 1 && S >= 1 && E >= 1 && C >= 1 && M >= 1 && H >= 1 && N >= 1,
+              MESH_MOE_E_ARG, "dispatched_expert_ffn: bad sizes");
+  MOE_REQUIRE(activation >= MESH_MOE_ACT_LINEAR &&
+                  activation <= MESH_MOE_ACT_SWISH,
+              MESH_MOE_E_ARG, "dispatched_expert_ffn: unknown activation %d",
+              activation);
+  const int64_t rows = (int64_t)G * C;
+  MOE_REQUIRE(dtype == MESH_MOE_BF16 && rows <= 0x7fffffffLL &&
+                  (int64_t)G * S <= 0x7fffffffLL &&
+                  ring_path_applies((int)rows, H, M) &&
+                  (((uintptr_t)x | (uintptr_t)wi_packed | (uintptr_t)h) % 16 == 0),
+              MESH_MOE_E_UNSUPPORTED,
+              "dispatched_expert_ffn: needs bf16 and a first GEMM the 256 x 256 "
+              "direct-to-LDS kernel takes (rows=%lld M=%d H=%d)",
+              (long long)rows, M, H);
+  MOE_REQUIRE(workspace_bytes >=
+                  mesh_moe_dispatched_expert_ffn_workspace_bytes(G, E, C, M),
+              MESH_MOE_E_ARG, "dispatched_expert_ffn: workspace too small");
+  hipStream_t st = (hipStream_t)stream;
+  const int R = (int)rows;
+  int32_t* map = (int32_t*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+  bf16_t* zero_row =
+      (bf16_t*)(((uintptr_t)(map + (size_t)E * R) + 255) & ~(uintptr_t)255);
+  const int64_t n_map = (int64_t)E * R;
+  const unsigned cb = (unsigned)((n_map + 255) / 256 < 4096 ? (n_map + 255) / 256
+                                                            : 4096);
+  slot_map_clear_kernel<<<cb, 256, 0, st>>>(map, n_map, zero_row, M);
+  MOE_CHECK_LAUNCH("dispatched_expert_ffn (clear)");
+  const int64_t pairs = (int64_t)G * S * 2;
+  slot_map_kernel<<<(unsigned)((pairs + 255) / 256), 256, 0, st>>>(
+      idx, pos, gate, kept, map, (int64_t)G * S, S, C, rows);
+  MOE_CHECK_LAUNCH("dispatched_expert_ffn (slot map)");
+  const bool relu = activation == MESH_MOE_ACT_RELU;
+  int rc = launch_ring((const bf16_t*)x, (const bf16_t*)wi_packed, (bf16_t*)h,
+                       E, R, H, M, relu, st, map, zero_row);
+  if (rc != 0) return rc;
+  if (!relu && activation != MESH_MOE_ACT_LINEAR) {
+    const int64_t n = (int64_t)E * R * H;
+    const int blocks = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
+    activation_kernel<bf16_t><<<blocks, 256, 0, st>>>((bf16_t*)h, n, activation);
+    MOE_CHECK_LAUNCH("dispatched_expert_ffn (activation)");
+  }
   return grouped_gemm(h, wo_packed, y, E, R, N, H, MESH_MOE_ACT_LINEAR, dtype,
                       st);
 }

@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -69,6 +69,12 @@ _SIGNATURES = {
         ctypes.c_int, _vp]),
     "mesh_moe_expert_ffn": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
+    "mesh_moe_dispatched_expert_ffn_workspace_bytes": (ctypes.c_size_t, [
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "mesh_moe_dispatched_expert_ffn": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_size_t,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
     "mesh_moe_expert_linear": (ctypes.c_int, [
         _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
@@ -558,6 +564,41 @@ def expert_ffn(expert_in, wi_packed, wo_packed, activation="relu", h=None,
     _check(lib.mesh_moe_expert_ffn(ip, wip, wop, hp, yp, e, rows, m, hdim, n,
                                    ACTIVATIONS[activation], code, _stream()),
            "expert_ffn")
+  return y
+
+
+E_UNSUPPORTED = -2
+
+
+def dispatched_expert_ffn(x, r, wi_packed, wo_packed, activation="relu"):
+  """dispatch + expert_ffn without materialising expert_in: x [G, S, M], the
+  Routing r -> y [E, G*C, N], or None where the library has no such kernel for
+  the case (the caller then makes the two calls)."""
+  lib = load_library()
+  if activation not in ACTIVATIONS:
+    raise ValueError("unsupported expert activation %r" % (activation,))
+  g, s, m = x.shape
+  e, c = r.num_experts, r.capacity
+  hdim, n = wi_packed.shape[1], wo_packed.shape[1]
+  dt = x.dtype
+  if dt != torch.bfloat16:
+    return None
+  dev = x.device
+  h = torch.empty((e, g * c, hdim), dtype=dt, device=dev)
+  y = torch.empty((e, g * c, n), dtype=dt, device=dev)
+  ws_bytes = lib.mesh_moe_dispatched_expert_ffn_workspace_bytes(g, e, c, m)
+  ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
+  with _stage("expert_ffn"):
+    rc = lib.mesh_moe_dispatched_expert_ffn(
+        _dev(x, "x"), _dev(r.idx, "idx", torch.int32, (g, s, 2)),
+        r.pos.data_ptr(), r.gate.data_ptr(), r.kept.data_ptr(),
+        _dev(wi_packed, "wi_packed", dt, (e, hdim, m)),
+        _dev(wo_packed, "wo_packed", dt, (e, n, hdim)), h.data_ptr(),
+        y.data_ptr(), ws.data_ptr(), ws_bytes, g, s, e, c, m, hdim, n,
+        ACTIVATIONS[activation], dtype_code(dt), _stream())
+  if rc == E_UNSUPPORTED:
+    return None
+  _check(rc, "dispatched_expert_ffn")
   return y
 
 

@@ -431,14 +431,20 @@ class MoEV1Operation(mtf.Operation):
       if save:
         r, logits = r
       by_slot = isinstance(r, moe_hip.SlotRouting)
-      expert_in = (moe_hip.slot_dispatch(xg, r) if by_slot
-                   else moe_hip.dispatch(xg, r))
-      h = None
-      if save or kwo_p is not None:
-        h = torch.empty((e_, groups * c_, wi_p.shape[1]), dtype=dt,
-                        device=xg.device)
-      y = moe_hip.expert_ffn(expert_in.reshape(e_, groups * c_, m_), wi_p,
-                             wo_p, self._activation, h=h)
+      y = None
+      if not (save or by_slot or kwo_p is not None):
+        # nobody reads expert_in afterwards: fold the dispatch into the first
+        # expert GEMM where the library can
+        y = moe_hip.dispatched_expert_ffn(xg, r, wi_p, wo_p, self._activation)
+      if y is None:
+        expert_in = (moe_hip.slot_dispatch(xg, r) if by_slot
+                     else moe_hip.dispatch(xg, r))
+        h = None
+        if save or kwo_p is not None:
+          h = torch.empty((e_, groups * c_, wi_p.shape[1]), dtype=dt,
+                          device=xg.device)
+        y = moe_hip.expert_ffn(expert_in.reshape(e_, groups * c_, m_), wi_p,
+                               wo_p, self._activation, h=h)
       y4 = y.reshape(e_, groups, c_, n_)
       out = (moe_hip.slot_combine(y4, r, s_) if by_slot
              else moe_hip.combine(y4, r, s_))

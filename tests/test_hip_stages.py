@@ -786,3 +786,37 @@ def test_slot_dispatch_combine(hip, act_dtype):
   for gi in range(g):
     chosen[gi][want_r["slot_token"][gi].reshape(-1)] = True
   assert (H.to_np(out)[~chosen] == 0).all()
+
+
+@pytest.mark.parametrize("shape", [(4, 512, 8, 128, 256, 512, 256),
+                                   (2, 1024, 16, 128, 128, 384, 128),
+                                   (5, 300, 4, 180, 64, 256, 64)])
+def test_dispatched_expert_ffn_equals_two_calls(hip, shape):
+  """The dispatch folded into the first expert GEMM gives bit-identical h-free
+  outputs to mesh_moe_dispatch + mesh_moe_expert_ffn (same kernel, same
+  operands, rows fetched through the slot map), including empty slots and
+  kept choices whose bf16 gate is 0."""
+  g, s, e, c, m, hdim, n = shape
+  rng = np.random.default_rng(sum(shape))
+  logits = H.safe_logits(rng, g, s, e, scale=1.5,
+                         bias=H.zipf_bias(rng, e, scale=2.0))
+  x = H.to_gpu(rng.standard_normal((g, s, m)).astype(np.float32), "bfloat16")
+  wi = H.to_gpu(H.normal_weights(rng, (e, m, hdim), m), "bfloat16")
+  wo = H.to_gpu(H.normal_weights(rng, (e, hdim, n), hdim), "bfloat16")
+  wi_p = hip.pack_weights(wi, torch.bfloat16)
+  wo_p = hip.pack_weights(wo, torch.bfloat16)
+  r = hip.top2_gating(torch.from_numpy(logits).cuda(), c)
+  r.gate[0, 0, 0] = 0.0            # a kept choice with gate 0: dispatches zeros
+  assert int((r.fill < c).sum()) > 0                   # some empty slots
+  want = hip.expert_ffn(hip.dispatch(x, r).reshape(e, g * c, m), wi_p, wo_p,
+                        "relu")
+  got = hip.dispatched_expert_ffn(x, r, wi_p, wo_p, "relu")
+  assert got is not None
+  assert torch.equal(got, want)
+  # float32, and row counts that 128-row tiles serve better (320 rows here):
+  # the library declines and the caller makes the two calls
+  assert hip.dispatched_expert_ffn(x.float(), r, wi_p.float(), wo_p.float(),
+                                   "relu") is None
+  if g * c == 256:
+    r2 = hip.top2_gating(torch.from_numpy(logits).cuda(), c + 32)
+    assert hip.dispatched_expert_ffn(x, r2, wi_p, wo_p, "relu") is None
