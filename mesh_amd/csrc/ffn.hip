@@ -1119,6 +1119,8 @@ extern "C" int mesh_moe_expert_ffn(const void* expert_in, const void* wi_packed,
                       st);
 }
 
+namespace mesh_moe {
+
 // ---------------------------------------------------------------------------
 // Dispatch folded into the first expert GEMM: slot -> token map.
 // ---------------------------------------------------------------------------
@@ -1152,6 +1154,8 @@ static bool ring_path_applies(int R, int N, int K) {
   return N >= 256 && R >= 128 && K % 64 == 0 && K % 8 == 0 && N % 8 == 0 &&
          pad128 >= pad256 && (int64_t)N * K < (1LL << 31);
 }
+
+}  // namespace mesh_moe
 
 extern "C" size_t mesh_moe_dispatched_expert_ffn_workspace_bytes(int G, int E,
                                                                  int C, int M) {
