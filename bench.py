@@ -280,6 +280,10 @@ def main():
                   help="time the transformer block around the layer "
                        "(attention, MoE1D, attention, DenseReluDense; v1 "
                        "configs); not the benchmark's metric")
+  ap.add_argument("--graph", action="store_true",
+                  help="time replays of a recorded HIP graph of the step "
+                       "(Lowering.capture) instead of eager runs; the per-stage "
+                       "times still come from eager runs")
   ap.add_argument("--no-cpu-baseline", action="store_true")
   args = ap.parse_args()
   if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -322,6 +326,16 @@ def main():
     stages = timer.totals()
     routings = timer.routing
   ms_per_step = (t1 - t0) * 1e3 / args.steps
+  if args.graph:
+    step = lowering.capture()
+    for _ in range(args.warmup):
+      step.replay()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(args.steps):
+      step.replay()
+    torch.cuda.synchronize()
+    ms_per_step = (time.perf_counter() - t0) * 1e3 / args.steps
   tokens = cfg["batch"] * cfg["length"]
   out_ok = bool(torch.isfinite(lowering.export_to_tf_tensor(y).float()).all())
 
@@ -353,7 +367,8 @@ def main():
       "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak",
       "vs_baseline": None, "dtype": cfg["dtype"], "data": "synthetic",
       "config": {"workload": cfg["name"], "layer": cfg["layer"],
-                 "tokens": tokens, "output_finite": out_ok},
+                 "tokens": tokens, "output_finite": out_ok,
+                 "hip_graph": bool(args.graph)},
   }
   if cfg["layer"] == "v1":
     r = routings[-1]

@@ -554,6 +554,33 @@ class Lowering(object):
   def fed_value(self, tensor, default):
     return self._feeds.get(tensor, default)
 
+  def capture(self):
+    """Records one `run()` into a HIP graph and returns a CapturedStep whose
+    `replay(feeds)` re-executes it with one graph launch instead of one launch
+    per kernel (what pays when the step is launch-bound: small layers).
+
+    Every imported tensor gets a static device buffer that the recorded
+    kernels read; `replay` copies new values into those buffers first.  The
+    outputs live in the graph's memory pool: `export_to_tf_tensor` returns the
+    tensors the last replay wrote.  Variables are read in place, so an
+    assignment between replays is seen.  The library allocates nothing and
+    uses no memset nodes, which is what makes its launches capturable.
+    """
+    statics = {}
+    for op in self.graph.operations:
+      if isinstance(op, ImportOperation):
+        t = op.outputs[0]
+        statics[t] = self.tensors[t].to_laid_out_tensor().tensor_list[0].clone()
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):     # warm-up outside the capture
+      self.run(statics)
+    torch.cuda.current_stream().wait_stream(side)
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+      self.run(statics)
+    return CapturedStep(graph, statics)
+
   def mesh_impl(self, m):
     if not isinstance(m, Mesh):
       m = m.mesh
@@ -600,6 +627,24 @@ class Lowering(object):
       raise ValueError(
           "Wrong slice shape: correct_shape = %s actual shape = %s"
           % (correct_shape, actual_shape))
+
+
+class CapturedStep(object):
+  """A recorded step of a Lowering (Lowering.capture)."""
+
+  def __init__(self, graph, statics):
+    self._graph = graph
+    self._statics = statics
+
+  def replay(self, feeds=None):
+    """feeds: {imported Tensor: torch tensor of the same shape}; tensors not
+    fed keep the values of the previous replay."""
+    for tensor, value in (feeds or {}).items():
+      if tensor not in self._statics:
+        raise ValueError("%s is not an imported tensor of the recorded graph"
+                         % (tensor,))
+      self._statics[tensor].copy_(torch.as_tensor(value))
+    self._graph.replay()
 
 
 # ----------------------------------------------------------------------------
