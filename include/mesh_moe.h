@@ -249,8 +249,9 @@ size_t mesh_moe_dispatched_expert_ffn_workspace_bytes(int G, int E, int C,
                                                       int M);
 
 /*
- * mesh_moe_dispatch + mesh_moe_expert_ffn in one call that never writes
- * expert_in: the first GEMM fetches each slot's token row straight from x
+ * mesh_moe_dispatch + mesh_moe_expert_ffn in one call (the dispatch einsum
+ * and the two expert einsums, transformer/moe.py:443-447 and :469-486) that
+ * never writes expert_in: the first GEMM fetches each slot's token row straight from x
  * through a slot -> token map built from the routing record (empty slots and
  * kept choices whose gate rounds to 0 read a zero row).  Same h and y as the
  * two calls.  For callers that do not need expert_in afterwards (inference;
