@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 9
+#define MESH_MOE_ABI_VERSION 10
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -244,6 +244,22 @@ int mesh_moe_expert_linear(const void* a, const void* w_packed, void* y, int E,
                            int R, int K, int N, int activation, int dtype,
                            void* stream);
 
+/*
+ * What the layer does to the hidden tensor between the two expert einsums, in
+ * place on n elements of `dtype`, each product rounded once:
+ *   factor  != NULL: h *= factor -- one more factor of mtf.layers.dense_product
+ *            (layers.py:256-295) when the expert activation is a list (gated
+ *            units, transformer/moe.py:469-475)
+ *   uniform != NULL: h *= noise, noise = (uniform < keep_prob) / keep_prob with
+ *            keep_prob and the quotient rounded to `dtype` -- mtf.dropout
+ *            (ops.py:5832-5872) under hparams.moe_dropout_rate
+ *            (transformer/moe.py:477-479); uniform [n] dtype in [0, 1)
+ *   noise_out [n] dtype or NULL: the noise, kept for the backward pass
+ */
+int mesh_moe_hidden_product(void* h, const void* factor, const void* uniform,
+                            float keep_prob, void* noise_out, int64_t n,
+                            int dtype, void* stream);
+
 /* Bytes of scratch mesh_moe_dispatched_expert_ffn needs. */
 size_t mesh_moe_dispatched_expert_ffn_workspace_bytes(int G, int E, int C,
                                                       int M);
@@ -390,18 +406,22 @@ size_t mesh_moe_expert_ffn_backward_workspace_bytes(int E, int R, int M, int H,
 /*
  * Backward of the two expert einsums (transformer/moe.py:469-486), ReLU or
  * linear experts:
- *   dh = (dy . wo^T) * (h > 0);  dwo = h^T . dy
- *   dexpert_in = dh . wi^T;      dwi = expert_in^T . dh
- *   expert_in [E,R,M], h [E,R,H] (as mesh_moe_expert_ffn left it), dy [E,R,N]
+ *   dh = (dy . wo^T) * dh_scale * (h > 0);  dwo = h^T . dy
+ *   dexpert_in = dh . wi^T;                 dwi = expert_in^T . dh
+ *   expert_in [E,R,M], h [E,R,H] (as mesh_moe_expert_ffn left it, after the
+ *   hidden dropout if there was one), dy [E,R,N]
  *   wi [E,M,H], wo [E,H,N]: the variables' own layout (NOT the packed one)
+ *   dh_scale [E,R,H] dtype or NULL: the dropout noise mesh_moe_hidden_product
+ *   wrote (transformer/moe.py:477-479)
  *   dexpert_in [E,R,M]; dwi [E,M,H]; dwo [E,H,N]; everything of `dtype`
  * Four grouped GEMMs on the forward kernels plus four transposes.
  */
 int mesh_moe_expert_ffn_backward(const void* expert_in, const void* h,
                                  const void* dy, const void* wi,
-                                 const void* wo, void* dexpert_in, void* dwi,
-                                 void* dwo, int E, int R, int M, int H, int N,
-                                 int activation, int dtype, void* workspace,
+                                 const void* wo, const void* dh_scale,
+                                 void* dexpert_in, void* dwi, void* dwo, int E,
+                                 int R, int M, int H, int N, int activation,
+                                 int dtype, void* workspace,
                                  size_t workspace_bytes, void* stream);
 
 /* Bytes of scratch mesh_moe_gating_backward needs. */

@@ -893,17 +893,46 @@ __global__ __launch_bounds__(256) void activation_kernel(T* __restrict__ h,
     store_f32<T>(h + i, apply_activation(load_f32<T>(h + i), act));
 }
 
-// dh = (h > 0) ? dh : 0 -- the ReLU of the forward pass seen from behind
-// (h is the stored, already rounded activation: positive iff the
-// pre-activation rounded to a positive value).
+// dh = dh * scale (when given), then dh = (h > 0) ? dh : 0 for ReLU experts --
+// the hidden dropout and the ReLU of the forward pass seen from behind (h is
+// the stored, already rounded activation: positive iff the pre-activation
+// rounded to a positive value and the element was not dropped).
 template <typename T>
-__global__ __launch_bounds__(256) void relu_mask_kernel(T* __restrict__ dh,
-                                                        const T* __restrict__ h,
-                                                        int64_t n) {
+__global__ __launch_bounds__(256) void hidden_grad_kernel(
+    T* __restrict__ dh, const T* __restrict__ h, const T* __restrict__ scale,
+    bool relu, int64_t n) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
-       i += stride)
-    if (!(load_f32<T>(h + i) > 0.f)) dh[i] = (T)0;
+       i += stride) {
+    if (relu && !(load_f32<T>(h + i) > 0.f)) {
+      dh[i] = (T)0;
+    } else if (scale) {
+      store_f32<T>(dh + i, load_f32<T>(dh + i) * load_f32<T>(scale + i));
+    }
+  }
+}
+
+// h = h * factor (when given), then dropout: noise = (u < keep) ? inv_keep : 0,
+// h = h * noise, each product rounded once to T.
+template <typename T>
+__global__ __launch_bounds__(256) void hidden_product_kernel(
+    T* __restrict__ h, const T* __restrict__ factor,
+    const T* __restrict__ uniform, float keep, float inv_keep,
+    T* __restrict__ noise_out, int64_t n) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += stride) {
+    float v = load_f32<T>(h + i);
+    if (factor) {
+      store_f32<T>(h + i, v * load_f32<T>(factor + i));
+      v = load_f32<T>(h + i);
+    }
+    if (uniform) {
+      const float noise = load_f32<T>(uniform + i) < keep ? inv_keep : 0.f;
+      store_f32<T>(h + i, v * noise);
+      if (noise_out) store_f32<T>(noise_out + i, noise);
+    } 
+  }
 }
 
 template <int BM, int BN, int BK>
@@ -1233,6 +1262,37 @@ extern "C" int mesh_moe_expert_linear(const void* a, const void* w_packed,
                       (hipStream_t)stream);
 }
 
+extern "C" int mesh_moe_hidden_product(void* h, const void* factor,
+                                       const void* uniform, float keep_prob,
+                                       void* noise_out, int64_t n, int dtype,
+                                       void* stream) {
+  MOE_REQUIRE(h, MESH_MOE_E_ARG, "hidden_product: null pointer");
+  MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG,
+              "hidden_product: bad dtype %d", dtype);
+  MOE_REQUIRE(n >= 1, MESH_MOE_E_ARG, "hidden_product: bad size n=%lld",
+              (long long)n);
+  MOE_REQUIRE(!noise_out || uniform, MESH_MOE_E_ARG,
+              "hidden_product: noise_out without uniform");
+  MOE_REQUIRE(!uniform || (keep_prob > 0.f && keep_prob <= 1.f), MESH_MOE_E_ARG,
+              "hidden_product: keep_prob %g outside (0, 1]", (double)keep_prob);
+  if (!factor && !uniform) return 0;
+  hipStream_t st = (hipStream_t)stream;
+  const int blocks = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
+  if (dtype == MESH_MOE_F32) {
+    hidden_product_kernel<float><<<blocks, 256, 0, st>>>(
+        (float*)h, (const float*)factor, (const float*)uniform, keep_prob,
+        1.f / keep_prob, (float*)noise_out, n);
+  } else {
+    // the threshold and 1 / keep_prob are scalars of the activation dtype
+    const float keep = round_bf16_host(keep_prob);
+    hidden_product_kernel<bf16_t><<<blocks, 256, 0, st>>>(
+        (bf16_t*)h, (const bf16_t*)factor, (const bf16_t*)uniform, keep,
+        round_bf16_host(1.f / keep), (bf16_t*)noise_out, n);
+  }
+  MOE_CHECK_LAUNCH("hidden_product");
+  return 0;
+}
+
 // Elements of the scratch mesh_moe_expert_ffn_backward needs: dh [E,R,H], one
 // [E,H,R] transpose buffer (h^T, then dh^T) and one [E,max(M,N),R] buffer
 // (dy^T, then expert_in^T).
@@ -1252,7 +1312,8 @@ extern "C" size_t mesh_moe_expert_ffn_backward_workspace_bytes(int E, int R,
 
 extern "C" int mesh_moe_expert_ffn_backward(
     const void* expert_in, const void* h, const void* dy, const void* wi,
-    const void* wo, void* dexpert_in, void* dwi, void* dwo, int E, int R,
+    const void* wo, const void* dh_scale, void* dexpert_in, void* dwi,
+    void* dwo, int E, int R,
     int M, int H, int N, int activation, int dtype, void* workspace,
     size_t workspace_bytes, void* stream) {
   MOE_REQUIRE(expert_in && h && dy && wi && wo && dexpert_in && dwi && dwo &&
@@ -1281,16 +1342,17 @@ extern "C" int mesh_moe_expert_ffn_backward(
   // dh = dy . wo^T  (wo in its variable layout [E, H, N] is K-contiguous here)
   rc = grouped_gemm(dy, wo, dh, E, R, H, N, MESH_MOE_ACT_LINEAR, dtype, st);
   if (rc != 0) return rc;
-  if (activation == MESH_MOE_ACT_RELU) {
+  if (activation == MESH_MOE_ACT_RELU || dh_scale) {
     const int64_t n = (int64_t)E * R * H;
+    const bool relu = activation == MESH_MOE_ACT_RELU;
     const int blocks = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
     if (dtype == MESH_MOE_F32)
-      relu_mask_kernel<float><<<blocks, 256, 0, st>>>((float*)dh,
-                                                      (const float*)h, n);
+      hidden_grad_kernel<float><<<blocks, 256, 0, st>>>(
+          (float*)dh, (const float*)h, (const float*)dh_scale, relu, n);
     else
-      relu_mask_kernel<bf16_t><<<blocks, 256, 0, st>>>((bf16_t*)dh,
-                                                       (const bf16_t*)h, n);
-    MOE_CHECK_LAUNCH("expert_ffn_backward (relu mask)");
+      hidden_grad_kernel<bf16_t><<<blocks, 256, 0, st>>>(
+          (bf16_t*)dh, (const bf16_t*)h, (const bf16_t*)dh_scale, relu, n);
+    MOE_CHECK_LAUNCH("expert_ffn_backward (hidden mask)");
   }
   // dexpert_in = dh . wi^T  (wi in its variable layout [E, M, H])
   rc = grouped_gemm(dh, wi, dexpert_in, E, R, M, H, MESH_MOE_ACT_LINEAR, dtype,

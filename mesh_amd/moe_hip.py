@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -89,8 +89,10 @@ _SIGNATURES = {
     "mesh_moe_expert_ffn_backward_workspace_bytes": (ctypes.c_size_t, [
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_int]),
+    "mesh_moe_hidden_product": (ctypes.c_int, [
+        _vp, _vp, _vp, ctypes.c_float, _vp, ctypes.c_int64, ctypes.c_int, _vp]),
     "mesh_moe_expert_ffn_backward": (ctypes.c_int, [
-        _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
+        _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         _vp, ctypes.c_size_t, _vp]),
     "mesh_moe_gating_backward_workspace_bytes": (ctypes.c_size_t, [
@@ -671,9 +673,30 @@ def combine_backward(dout, y, r):
   return dy, dgate
 
 
-def expert_ffn_backward(expert_in, h, dy, wi, wo, activation="relu"):
+def hidden_product(h, factor=None, uniform=None, keep_prob=1.0,
+                   want_noise=False):
+  """In place on h (any shape, contiguous): h *= factor, then the dropout
+  h *= (uniform < keep_prob) / keep_prob.  Returns the noise tensor when
+  want_noise, else None."""
+  lib = load_library()
+  dt = h.dtype
+  noise = torch.empty_like(h) if (want_noise and uniform is not None) else None
+  with _stage("hidden_product"):
+    _check(lib.mesh_moe_hidden_product(
+        _dev(h, "h"),
+        _dev(factor, "factor", dt, tuple(h.shape)) if factor is not None else None,
+        _dev(uniform, "uniform", dt, tuple(h.shape)) if uniform is not None
+        else None,
+        float(keep_prob), noise.data_ptr() if noise is not None else None,
+        h.numel(), dtype_code(dt), _stream()), "hidden_product")
+  return noise
+
+
+def expert_ffn_backward(expert_in, h, dy, wi, wo, activation="relu",
+                        dh_scale=None):
   """expert_in [E,R,M], h [E,R,H], dy [E,R,N]; wi [E,M,H], wo [E,H,N] in the
-  variables' own layout -> (dexpert_in [E,R,M], dwi [E,M,H], dwo [E,H,N])."""
+  variables' own layout -> (dexpert_in [E,R,M], dwi [E,M,H], dwo [E,H,N]).
+  dh_scale [E,R,H]: the hidden dropout's noise, if there was one."""
   lib = load_library()
   if activation not in ACTIVATIONS:
     raise ValueError("unsupported expert activation %r" % (activation,))
@@ -692,7 +715,9 @@ def expert_ffn_backward(expert_in, h, dy, wi, wo, activation="relu"):
     _check(lib.mesh_moe_expert_ffn_backward(
         _dev(expert_in, "expert_in"), _dev(h, "h", dt, (e, rows, hdim)),
         _dev(dy, "dy", dt, (e, rows, n)), _dev(wi, "wi", dt, (e, m, hdim)),
-        _dev(wo, "wo", dt, (e, hdim, n)), dxe.data_ptr(), dwi.data_ptr(),
+        _dev(wo, "wo", dt, (e, hdim, n)),
+        _dev(dh_scale, "dh_scale", dt, (e, rows, hdim))
+        if dh_scale is not None else None, dxe.data_ptr(), dwi.data_ptr(),
         dwo.data_ptr(), e, rows, m, hdim, n, ACTIVATIONS[activation], code,
         ws.data_ptr(), ws_bytes, _stream()), "expert_ffn_backward")
   return dxe, dwi, dwo

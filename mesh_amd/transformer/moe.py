@@ -73,22 +73,25 @@ def _expert_capacity(group_size, capacity_factor, num_experts, min_capacity):
   return max(capacity, min_capacity)
 
 
-def _activation_name(activation):
-  """mtf.relu / "relu" / None / "linear" -> name understood by the kernels."""
-  if isinstance(activation, (list, tuple)):
-    if len(activation) != 1:
-      raise NotImplementedError(
-          "products of several dense layers (gated activations) are not "
-          "implemented: %r" % (activation,))
-    activation = activation[0]
-  if activation is None or activation == "linear":
-    return "linear"
-  name = activation if isinstance(activation, str) else getattr(
-      activation, "__name__", None)
-  if name not in moe_hip.ACTIVATIONS:
-    raise NotImplementedError("expert activation %r is not implemented"
-                              % (activation,))
-  return name
+def _activation_names(activation):
+  """mtf.relu / "relu" / None / "linear", or a list of those (the factors of
+  mtf.layers.dense_product, layers.py:279-295) -> names understood by the
+  kernels, one per factor."""
+  if not isinstance(activation, (list, tuple)):
+    activation = [activation]
+  if not activation:
+    raise ValueError("empty list of expert activations")
+  names = []
+  for a in activation:
+    if a is None or a == "linear":
+      names.append("linear")
+      continue
+    name = a if isinstance(a, str) else getattr(a, "__name__", None)
+    if name not in moe_hip.ACTIVATIONS:
+      raise NotImplementedError("expert activation %r is not implemented"
+                                % (a,))
+    names.append(name)
+  return names
 
 
 def _check_gating(hparams):
@@ -356,20 +359,37 @@ class MoEV1Operation(mtf.Operation):
   replaced by output_dim, scalar balancing loss before moe_loss_coef)."""
 
   def __init__(self, inputs, w_gate, wi, wo, importance, output_dim, capacity,
-               gating, activation, k_wo=None, name="moe_v1"):
+               gating, activation, k_wo=None, hidden_keep_prob=None,
+               name="moe_v1"):
     """With k_wo (moe_use_experts_attention, moe.py:514-522) `wo` is the "q_wo"
     kernel, the operation has a second output projection of the same hidden
-    tensor and its outputs are (q, loss, k)."""
+    tensor and its outputs are (q, loss, k).
+
+    `wi` and `activation` may be lists of the same length: the hidden tensor
+    is then the product of act_i(expert_in . wi_i) (moe.py:469-475).
+    hidden_keep_prob: keep probability of the dropout on the hidden tensor
+    (moe.py:477-479), None for none."""
+    wis = list(wi) if isinstance(wi, (list, tuple)) else [wi]
+    acts = (list(activation) if isinstance(activation, (list, tuple))
+            else [activation])
+    if len(wis) != len(acts):
+      raise ValueError("%d wi kernels for %d activations"
+                       % (len(wis), len(acts)))
+    wi = wis[0]
     ins = [inputs, w_gate, wi, wo] + ([importance] if importance is not None
                                       else [])
     if k_wo is not None:
       ins.append(k_wo)
+    ins.extend(wis[1:])
     super(MoEV1Operation, self).__init__(ins, name=name)
     self._has_importance = importance is not None
     self._k_wo = k_wo
     self._capacity = capacity
     self._gating = gating
-    self._activation = activation
+    self._activation = acts[0]
+    self._more_wi = wis[1:]
+    self._more_activations = acts[1:]
+    self._hidden_keep_prob = hidden_keep_prob
     self._num_experts = wi.shape.dims[0].size
     self._save_for_backward = False
     out_shape = mtf.Shape(inputs.shape.dims[:-1] + [output_dim])
@@ -390,6 +410,10 @@ class MoEV1Operation(mtf.Operation):
     if self._gating.use_second_place_loss:
       raise NotImplementedError(
           "backward of the second-place loss is not implemented")
+    if self._more_wi:
+      raise NotImplementedError(
+          "backward of a product of several dense layers (gated expert "
+          "activations) is not implemented")
     if self._activation not in ("relu", "linear"):
       raise NotImplementedError(
           "backward of expert activation %r is not implemented (the "
@@ -412,6 +436,9 @@ class MoEV1Operation(mtf.Operation):
     wg_p = _packed(lowering, w_gate, dt)               # [1, E, M]
     kwo_p = (_packed(lowering, self._k_wo, dt) if self._k_wo is not None
              else None)
+    more_wi_p = [_packed(lowering, t, dt) for t in self._more_wi]
+    keep_prob = self._hidden_keep_prob
+    plain_hidden = not more_wi_p and keep_prob is None
     o_, g_, s_, m_ = x.shape.to_integer_list
     n_ = self.outputs[0].shape.dims[-1].size
     e_, c_ = self._num_experts, self._capacity
@@ -432,29 +459,43 @@ class MoEV1Operation(mtf.Operation):
         r, logits = r
       by_slot = isinstance(r, moe_hip.SlotRouting)
       y = None
-      if not (save or by_slot or kwo_p is not None):
+      noise = None
+      if not (save or by_slot or kwo_p is not None) and plain_hidden:
         # nobody reads expert_in afterwards: fold the dispatch into the first
         # expert GEMM where the library can
         y = moe_hip.dispatched_expert_ffn(xg, r, wi_p, wo_p, self._activation)
       if y is None:
         expert_in = (moe_hip.slot_dispatch(xg, r) if by_slot
                      else moe_hip.dispatch(xg, r))
+        expert_in = expert_in.reshape(e_, groups * c_, m_)
+      if y is None and plain_hidden:
         h = None
         if save or kwo_p is not None:
           h = torch.empty((e_, groups * c_, wi_p.shape[1]), dtype=dt,
                           device=xg.device)
-        y = moe_hip.expert_ffn(expert_in.reshape(e_, groups * c_, m_), wi_p,
-                               wo_p, self._activation, h=h)
+        y = moe_hip.expert_ffn(expert_in, wi_p, wo_p, self._activation, h=h)
+      elif y is None:
+        # the hidden tensor is worked on between the two projections: the
+        # other factors of the product, then the dropout
+        h = moe_hip.expert_linear(expert_in, wi_p, self._activation)
+        for w_p, act in zip(more_wi_p, self._more_activations):
+          moe_hip.hidden_product(
+              h, factor=moe_hip.expert_linear(expert_in, w_p, act))
+        if keep_prob is not None:
+          u = torch.rand(h.shape, dtype=dt, device=h.device)
+          noise = moe_hip.hidden_product(h, uniform=u, keep_prob=keep_prob,
+                                         want_noise=save)
+        y = moe_hip.expert_linear(h, wo_p)
       y4 = y.reshape(e_, groups, c_, n_)
       out = (moe_hip.slot_combine(y4, r, s_) if by_slot
              else moe_hip.combine(y4, r, s_))
       if save:
         # what the gradient operation reads (activations of this step)
-        noise = getattr(self._gating, "noise", None)
-        gate_in = noise.last if noise is not None else None
+        gate_noise = getattr(self._gating, "noise", None)
+        gate_in = gate_noise.last if gate_noise is not None else None
         saved.update(x=xg, routing=r, logits=logits, importance=imp_s,
                      expert_in=expert_in, h=h, y=y, w_gate_packed=wg_p,
-                     gate_in=gate_in, w_gate=wg_s)
+                     gate_in=gate_in, w_gate=wg_s, hidden_noise=noise)
       outs = (out.reshape(o_, g_, s_, n_), r.loss.to(dt).reshape(()))
       if kwo_p is not None:
         # the "k" projection of the same hidden tensor (moe.py:514-520)
@@ -514,7 +555,8 @@ class MoEV1GradOperation(mtf.Operation):
           sv["y"].reshape(e_, groups, c_, n_), r)
       dxe, dwi, dwo = moe_hip.expert_ffn_backward(
           sv["expert_in"].reshape(e_, groups * c_, m_), sv["h"],
-          dy.reshape(e_, groups * c_, n_), wi_s, wo_s, fwd._activation)
+          dy.reshape(e_, groups * c_, n_), wi_s, wo_s, fwd._activation,
+          dh_scale=sv["hidden_noise"])
       dlogits = moe_hip.gating_backward(
           sv["logits"], r, dgate, dloss_s.reshape(1).float(), 1.0,
           router=gating.router, top_k=getattr(gating, "top_k", 0),
@@ -622,9 +664,9 @@ def transformer_moe_layer_v1(
     nonpadding = mtf.reshape(nonpadding, moe_input_dims[:-1])
 
   _check_gating(hparams)
+  hidden_keep_prob = None
   if hparams.moe_dropout_rate != 0.0 and train:
-    raise NotImplementedError("expert dropout while training is not "
-                              "implemented (moe_dropout_rate must be 0)")
+    hidden_keep_prob = 1.0 - hparams.moe_dropout_rate   # moe.py:477-479
   if hparams.moe_gating == "expert_selection":
     gating = _ExpertSelectionGatingSpec(hparams, train, num_microbatches,
                                         nonpadding is not None)
@@ -640,15 +682,18 @@ def transformer_moe_layer_v1(
   else:
     gating = _GatingSpec(hparams, train, num_microbatches)
     router_name = "top_2_gating"                        # moe.py:1314
-  act_name = _activation_name(activation)
+  act_names = _activation_names(activation)
 
   # variables, named and shaped as the reference's dense layers create them
   w_gate = mtf_layers.get_dense_kernel_weights(
       inputs, [experts_dim_unsplit], [input_dim], [], None,
       name=router_name, variable_dtype=variable_dtype)
-  wi = mtf_layers.get_dense_kernel_weights(
-      inputs, [hidden_dim], [input_dim], [experts_dim], None, name="wi",
-      variable_dtype=variable_dtype)
+  # one kernel per factor of the product, "wi" or "wi_0", "wi_1", ...
+  # (layers.py:293)
+  wi = [mtf_layers.get_dense_kernel_weights(
+      inputs, [hidden_dim], [input_dim], [experts_dim], None,
+      name="wi_%d" % i if len(act_names) > 1 else "wi",
+      variable_dtype=variable_dtype) for i in range(len(act_names))]
   if hparams.moe_use_experts_attention:
     # two output projections of the same hidden tensor (moe.py:514-522)
     q_wo = mtf_layers.get_dense_kernel_weights(
@@ -659,7 +704,8 @@ def transformer_moe_layer_v1(
         variable_dtype=variable_dtype)
     q, loss, k = MoEV1Operation(
         inputs, w_gate, wi, q_wo, nonpadding, output_dim, expert_capacity,
-        gating, act_name, k_wo=k_wo).outputs
+        gating, act_names, k_wo=k_wo,
+        hidden_keep_prob=hidden_keep_prob).outputs
     outputs = [mtf.reshape(t, batch_and_length_dims + [output_dim])
                for t in (q, k)]
     return outputs, loss * hparams.moe_loss_coef
@@ -669,7 +715,7 @@ def transformer_moe_layer_v1(
 
   output, loss = MoEV1Operation(
       inputs, w_gate, wi, wo, nonpadding, output_dim, expert_capacity, gating,
-      act_name).outputs
+      act_names, hidden_keep_prob=hidden_keep_prob).outputs
   output = mtf.reshape(output, batch_and_length_dims + [output_dim])
   return output, loss * hparams.moe_loss_coef
 

@@ -46,6 +46,14 @@ MoE file, and its TensorFlow dependency cannot run here):
                                       see the unperturbed tokens; backward by
                                       central differences with the multiplier
                                       held fixed
+  expert_hidden (products of dense    independent float64 evaluation per
+  layers), hidden_dropout_noise       activation pair, factors commute, a zero
+                                      linear factor zeroes the output; the
+                                      noise against torch's arithmetic in the
+                                      tensor's dtype, strict threshold, keep
+                                      0.5 with everything kept = twice the
+                                      plain layer; backward through the
+                                      dropout by central differences
   gating_backward,                    central differences of an independent
   moe_layer_v1_backward               float64 forward with the routing held
                                       fixed (tests/test_oracle.py)
@@ -54,7 +62,8 @@ MoE file, and its TensorFlow dependency cannot run here):
 PARITY UNPINNED against TensorFlow itself (only running the reference could
 pin these): near-tie behaviour of argmax after TF's exp/log, the accumulation
 order of TF's bf16 einsum, and the random streams (the "random" second-place
-policy, the router input noise): the uniform numbers are explicit inputs here.
+policy, the router input noise, the hidden dropout): the uniform numbers are
+explicit inputs here.
 
 Citations are to files under the reference tree (mesh_tensorflow/...).
 """
@@ -814,13 +823,43 @@ def _scale_loss(loss, coef, act_dtype):
                   act_dtype)[()]
 
 
-def expert_ffn(expert_in, wi, wo, activation, act_dtype):
+def hidden_dropout_noise(uniform, keep_prob, act_dtype):
+  """mtf.dropout's multiplier (ops.py:5864-5872) for a tensor of the activation
+  dtype: cast(uniform < keep_prob) / keep_prob, where `uniform` holds
+  activation-dtype values in [0, 1) and keep_prob is a scalar of that dtype, so
+  both it and the quotient are rounded to it."""
+  keep = cast_act(F32(keep_prob), act_dtype)
+  u = cast_act(np.asarray(uniform, F32), act_dtype)
+  return cast_act((u < keep).astype(F32) / keep, act_dtype)
+
+
+def expert_hidden(expert_in, wi, activation, act_dtype, hidden_noise=None):
+  """The experts' hidden tensor (moe.py:469-479): the product over the factors
+  of mtf.layers.dense_product (layers.py:279-295) of act_i(expert_in . wi_i),
+  times the dropout noise.  wi / activation: one kernel [E, M, H] and one
+  name, or lists of the same length.  Every op rounds to the activation dtype.
+  """
+  wis = list(wi) if isinstance(wi, (list, tuple)) else [wi]
+  acts = (list(activation) if isinstance(activation, (list, tuple))
+          else [activation])
+  if len(wis) != len(acts):
+    raise ValueError("%d kernels for %d activations" % (len(wis), len(acts)))
+  h = None
+  for w, a in zip(wis, acts):
+    f = cast_act(np.matmul(expert_in, w), act_dtype)
+    f = cast_act(ACTIVATIONS[a](f), act_dtype)
+    h = f if h is None else cast_act(h * f, act_dtype)
+  if hidden_noise is not None:
+    h = cast_act(h * hidden_noise, act_dtype)
+  return h
+
+
+def expert_ffn(expert_in, wi, wo, activation, act_dtype, hidden_noise=None):
   """h = act(expert_in . wi), y = h . wo per expert (moe.py:469-486).
-  expert_in [E, R, M], wi [E, M, H], wo [E, H, N]; float32 accumulate, results
-  rounded to the activation dtype."""
-  act = ACTIVATIONS[activation]
-  h = cast_act(np.matmul(expert_in, wi), act_dtype)
-  h = cast_act(act(h), act_dtype)
+  expert_in [E, R, M], wi [E, M, H] (or a list, see expert_hidden),
+  wo [E, H, N]; float32 accumulate, results rounded to the activation dtype.
+  hidden_noise [E, R, H]: the dropout multiplier on h, if any."""
+  h = expert_hidden(expert_in, wi, activation, act_dtype, hidden_noise)
   return cast_act(np.matmul(h, wo), act_dtype)
 
 
@@ -861,11 +900,17 @@ def perturb_gate_inputs(xg, hp, train, act_dtype, gate_noise):
   return (xg.astype(F32) * mult).astype(F32), mult
 
 
+def _cast_kernels(w, act_dtype):
+  if isinstance(w, (list, tuple)):
+    return [cast_act(v, act_dtype) for v in w]
+  return cast_act(w, act_dtype)
+
+
 def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
                  nonpadding=None, activation="relu", num_microbatches=None,
                  logit_bias=None, second_uniform=None, dense=True,
                  mesh_dim_size=1, weights_are_cast=False, k_wo=None,
-                 gate_noise=None, sample_uniform=None):
+                 gate_noise=None, sample_uniform=None, hidden_uniform=None):
   """transformer_moe_layer_v1 forward (transformer/moe.py:191-525).
 
   x: [batch..., length, M] float32 array holding activation-dtype values.
@@ -878,6 +923,10 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
   k_wo [E, H, N]: with hparams.moe_use_experts_attention `wo` is the "q_wo"
   kernel and k_wo the "k_wo" kernel of a second output projection of the same
   hidden tensor (moe.py:514-522); the output is then the list [q, k].
+  wi / activation may be lists of the same length (gated units, see
+  expert_hidden).  hidden_uniform [E, G*C, H]: the uniform numbers of the
+  dropout on the hidden tensor, needed when train and hp.moe_dropout_rate != 0
+  (moe.py:477-479).
 
   Returns (output [batch..., length, N], loss scalar, aux dict).
   """
@@ -891,7 +940,8 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
               num_microbatches=num_microbatches, logit_bias=logit_bias,
               second_uniform=second_uniform, dense=dense,
               mesh_dim_size=mesh_dim_size, weights_are_cast=weights_are_cast,
-              gate_noise=gate_noise, sample_uniform=sample_uniform)
+              gate_noise=gate_noise, sample_uniform=sample_uniform,
+              hidden_uniform=hidden_uniform)
     # the two outputs share everything up to the hidden tensor, so each equals
     # the plain layer with its own output kernel
     q, loss, aux = moe_layer_v1(x, w_gate, wi, wo, hp1, train, act_dtype, **kw)
@@ -914,6 +964,14 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
     importance = cast_act(np.broadcast_to(nonpadding, lead), act_dtype)
     importance = importance.reshape(g_, s_)
   wg = cast_act(w_gate, act_dtype)
+  hidden_noise = None
+  if train and getattr(hp, "moe_dropout_rate", 0.0) != 0.0:
+    if hidden_uniform is None:
+      raise NotImplementedError(
+          "moe_dropout_rate while training needs the random tensor "
+          "(hidden_uniform)")
+    hidden_noise = hidden_dropout_noise(
+        hidden_uniform, 1.0 - hp.moe_dropout_rate, act_dtype)
   gate_mult = None
   if hp.moe_gating in ("switch", "switch_max", "ntlb", "expert_selection"):
     x_gate, gate_mult = perturb_gate_inputs(xg, hp, train, act_dtype,
@@ -929,7 +987,7 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
                        "(moe.py:1138-1140)")
     r = expert_selection_gating(logits, c_, importance, num_microbatches,
                                 act_dtype, dense=dense)
-    wi_a = wi if weights_are_cast else cast_act(wi, act_dtype)
+    wi_a = wi if weights_are_cast else _cast_kernels(wi, act_dtype)
     wo_a = wo if weights_are_cast else cast_act(wo, act_dtype)
     if dense:
       disp = r["dispatch"].reshape(g_, s_, e_ * c_)
@@ -938,7 +996,7 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
     else:
       expert_in = slot_dispatch(xg, r)
     y = expert_ffn(expert_in.reshape(e_, g_ * c_, m_), wi_a, wo_a, activation,
-                   act_dtype)
+                   act_dtype, hidden_noise)
     n_ = y.shape[-1]
     y = y.reshape(e_, g_, c_, n_)
     if dense:
@@ -981,7 +1039,7 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
                      second_uniform, dense=dense)
   # weights_are_cast: the caller already holds activation-dtype values (lets
   # the CPU-baseline timing pass one expert's matrix broadcast to all experts)
-  wi_a = wi if weights_are_cast else cast_act(wi, act_dtype)
+  wi_a = wi if weights_are_cast else _cast_kernels(wi, act_dtype)
   wo_a = wo if weights_are_cast else cast_act(wo, act_dtype)
   if dense:
     disp = r["dispatch"].reshape(g_, s_, e_ * c_)
@@ -991,7 +1049,7 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
   else:
     expert_in = dispatch_gather(xg, r, e_, c_, act_dtype)
   y = expert_ffn(expert_in.reshape(e_, g_ * c_, m_), wi_a, wo_a, activation,
-                 act_dtype)
+                 act_dtype, hidden_noise)
   n_ = y.shape[-1]
   y = y.reshape(e_, g_, c_, n_)
   if dense:
@@ -1119,16 +1177,23 @@ def dispatch_backward(dxe, r, act_dtype):
   return dx
 
 
-def expert_ffn_backward(xe, wi_a, wo_a, dy, activation, act_dtype):
+def expert_ffn_backward(xe, wi_a, wo_a, dy, activation, act_dtype,
+                        hidden_noise=None):
   """Backward of the two expert einsums (moe.py:469-486): float32 accumulate,
   activation-dtype results.  xe [E,R,M], dy [E,R,N]; returns
-  (dxe [E,R,M], dwi [E,M,H], dwo [E,H,N])."""
-  h = cast_act(np.matmul(xe, wi_a), act_dtype)
+  (dxe [E,R,M], dwi [E,M,H], dwo [E,H,N]).  hidden_noise [E,R,H]: the dropout
+  multiplier on the hidden tensor (moe.py:477-479), a constant of the graph."""
+  pre = cast_act(np.matmul(xe, wi_a), act_dtype)
+  h = pre
   if activation == "relu":
     h = cast_act(np.maximum(h, F32(0.0)), act_dtype)
+  if hidden_noise is not None:
+    h = cast_act(h * hidden_noise, act_dtype)
   dh = cast_act(np.matmul(dy, wo_a.transpose(0, 2, 1)), act_dtype)
+  if hidden_noise is not None:
+    dh = cast_act(dh * hidden_noise, act_dtype)
   if activation == "relu":
-    dh = dh * (h > 0)
+    dh = dh * (pre > 0)
   dwo = cast_act(np.matmul(h.transpose(0, 2, 1), dy), act_dtype)
   dxe = cast_act(np.matmul(dh, wi_a.transpose(0, 2, 1)), act_dtype)
   dwi = cast_act(np.matmul(xe.transpose(0, 2, 1), dh), act_dtype)
@@ -1138,7 +1203,8 @@ def expert_ffn_backward(xe, wi_a, wo_a, dy, activation, act_dtype):
 def moe_layer_v1_backward(x, w_gate, wi, wo, hp, train, act_dtype, d_out,
                           d_loss=0.0, nonpadding=None, activation="relu",
                           num_microbatches=None, logit_bias=None,
-                          gate_noise=None, sample_uniform=None):
+                          gate_noise=None, sample_uniform=None,
+                          hidden_uniform=None):
   """Gradients of (outputs, loss) of moe_layer_v1 w.r.t. x and the three
   kernels, given d_out [batch..., length, N] and the scalar d_loss.
 
@@ -1155,6 +1221,8 @@ def moe_layer_v1_backward(x, w_gate, wi, wo, hp, train, act_dtype, d_out,
   """
   if hp.moe_use_second_place_loss:
     raise NotImplementedError("backward of the second-place loss")
+  if isinstance(wi, (list, tuple)) or isinstance(activation, (list, tuple)):
+    raise NotImplementedError("backward of a product of dense layers")
   if activation not in ("relu", "linear", None):
     raise NotImplementedError("backward of activation %r" % (activation,))
   _, _, aux = moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype,
@@ -1162,7 +1230,12 @@ def moe_layer_v1_backward(x, w_gate, wi, wo, hp, train, act_dtype, d_out,
                            num_microbatches=num_microbatches,
                            logit_bias=logit_bias, dense=False,
                            gate_noise=gate_noise,
-                           sample_uniform=sample_uniform)
+                           sample_uniform=sample_uniform,
+                           hidden_uniform=hidden_uniform)
+  hidden_noise = None
+  if train and getattr(hp, "moe_dropout_rate", 0.0) != 0.0:
+    hidden_noise = hidden_dropout_noise(
+        hidden_uniform, 1.0 - hp.moe_dropout_rate, act_dtype)
   x = cast_act(x, act_dtype)
   lead, m_ = x.shape[:-1], x.shape[-1]
   g_, s_, c_ = aux["num_groups"], aux["group_size"], aux["capacity"]
@@ -1178,7 +1251,7 @@ def moe_layer_v1_backward(x, w_gate, wi, wo, hp, train, act_dtype, d_out,
   r_ = g_ * c_
   dxe, dwi, dwo = expert_ffn_backward(
       expert_in.reshape(e_, r_, m_), wi_a, wo_a, dy.reshape(e_, r_, n_),
-      activation, act_dtype)
+      activation, act_dtype, hidden_noise)
   dx = dispatch_backward(dxe.reshape(e_, g_, c_, m_), aux, act_dtype)
 
   # gating and router backward

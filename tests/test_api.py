@@ -119,6 +119,31 @@ def test_v1_switch_graph_names():
                    "layer_0/wo/kernel"]
 
 
+def test_v1_gated_activation_graph_names():
+  """A list of activations makes one "wi_<i>" dense layer per factor
+  (mtf.layers.dense_product, layers.py:293); a list of one keeps "wi"."""
+  graph, _, x, dims = graph_input()
+  with mtf.variable_scope("layer_0"):
+    y, _ = moe.transformer_moe_layer_v1(
+        x, dims[-1], hparams(), True, mtf.VariableDType(torch.float32),
+        activation=["gelu", "linear"])
+  assert y.shape == mtf.Shape(dims)
+  names = sorted(v.name for v in graph.all_variables)
+  assert names == ["layer_0/top_2_gating/kernel", "layer_0/wi_0/kernel",
+                   "layer_0/wi_1/kernel", "layer_0/wo/kernel"]
+  op = y.operation.inputs[0].operation
+  assert [op._activation] + op._more_activations == ["gelu", "linear"]
+  with pytest.raises(NotImplementedError, match="product of several"):
+    mtf.gradients([y], [x])
+  graph2, _, x2, dims2 = graph_input()
+  with mtf.variable_scope("layer_0"):
+    moe.transformer_moe_layer_v1(
+        x2, dims2[-1], hparams(), True, mtf.VariableDType(torch.float32),
+        activation=[mtf.relu])
+  assert sorted(v.name for v in graph2.all_variables) == [
+      "layer_0/top_2_gating/kernel", "layer_0/wi/kernel", "layer_0/wo/kernel"]
+
+
 def test_v1_ntlb_graph_names():
   """The ntlb router's variable lives under "ntlb_gating" (the `name` default
   of _ntlb_gating, transformer/moe.py:812)."""
@@ -211,8 +236,15 @@ def test_error_behaviour():
   with pytest.raises(ValueError, match="moe_z_loss needs"):
     moe.transformer_moe_layer_v1(
         x, dims[-1], hparams(**dict(sw, moe_z_loss=1e-3)), True, vdt)
-  with pytest.raises(NotImplementedError):
-    moe.transformer_moe_layer_v1(x, dims[-1], hparams(moe_dropout_rate=0.1), True, vdt)
+  # dropout on the hidden tensor while training builds (moe.py:477-479)
+  with mtf.variable_scope("dropout_train"):
+    out, _ = moe.transformer_moe_layer_v1(
+        x, dims[-1], hparams(moe_dropout_rate=0.1), True, vdt)
+  assert out.operation.inputs[0].operation._hidden_keep_prob == 0.9
+  with mtf.variable_scope("dropout_eval"):
+    out, _ = moe.transformer_moe_layer_v1(
+        x, dims[-1], hparams(moe_dropout_rate=0.1), False, vdt)
+  assert out.operation.inputs[0].operation._hidden_keep_prob is None
   with pytest.raises(ValueError, match="not a multiple of mesh_dim_size"):
     moe.transformer_moe_layer_v1(
         x, dims[-1], hparams(), True, vdt, layout="batch:rows", mesh_shape="rows:3")

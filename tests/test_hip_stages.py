@@ -820,3 +820,61 @@ def test_dispatched_expert_ffn_equals_two_calls(hip, shape):
   if g * c == 256:
     r2 = hip.top2_gating(torch.from_numpy(logits).cuda(), c + 32)
     assert hip.dispatched_expert_ffn(x, r2, wi_p, wo_p, "relu") is None
+
+
+@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("activation", ["relu", "linear"])
+def test_hidden_product_and_dropout_backward(hip, act_dtype, activation):
+  """mesh_moe_hidden_product (a second factor, then dropout) and the backward
+  of the expert einsums with the dropout noise, against the oracle."""
+  e, rows, m, hdim, n = 3, 70, 24, 40, 16
+  keep = 0.7
+  rng = np.random.default_rng(17)
+  cast = lambda a: O.cast_act(a.astype(np.float32), act_dtype)
+  xe = cast(rng.standard_normal((e, rows, m)))
+  wi = cast(H.normal_weights(rng, (e, m, hdim), m))
+  wi2 = cast(H.normal_weights(rng, (e, m, hdim), m))
+  wo = cast(H.normal_weights(rng, (e, hdim, n), hdim))
+  dy = cast(rng.standard_normal((e, rows, n)))
+  u = cast(rng.random((e, rows, hdim)))
+  u = np.minimum(u, np.float32(0.99))          # bf16 rounding may reach 1.0
+  u[0, 0, 0] = O.cast_act(np.float32(keep), act_dtype)   # the threshold itself
+  dt = H.ACT_TORCH[act_dtype]
+  g = lambda a: H.to_gpu(a, act_dtype)
+  wi_p, wi2_p = hip.pack_weights(g(wi), dt), hip.pack_weights(g(wi2), dt)
+  noise_want = O.hidden_dropout_noise(u, keep, act_dtype)
+  assert noise_want[0, 0, 0] == 0
+  tol = H.value_tolerance(act_dtype)
+
+  # two factors and dropout, forward
+  h = hip.expert_linear(g(xe), wi_p, activation)
+  f = hip.expert_linear(g(xe), wi2_p, "sigmoid")
+  assert hip.hidden_product(h, factor=f) is None
+  noise = hip.hidden_product(h, uniform=g(u), keep_prob=keep, want_noise=True)
+  np.testing.assert_array_equal(H.to_np(noise), noise_want)
+  h_want = O.expert_hidden(xe, [wi, wi2], [activation, "sigmoid"], act_dtype,
+                           noise_want)
+  np.testing.assert_allclose(H.to_np(h), h_want, **tol)
+  assert (H.to_np(h)[noise_want == 0] == 0).all()
+
+  # one factor and dropout, forward and backward
+  h = hip.expert_linear(g(xe), wi_p, activation)
+  noise = hip.hidden_product(h, uniform=g(u), keep_prob=keep, want_noise=True)
+  dxe, dwi, dwo = hip.expert_ffn_backward(g(xe), h, g(dy), g(wi), g(wo),
+                                          activation, dh_scale=noise)
+  want = O.expert_ffn_backward(xe, wi, wo, dy, activation, act_dtype,
+                               noise_want)
+  plain = O.expert_ffn_backward(xe, wi, wo, dy, activation, act_dtype)
+  assert np.abs(want[1] - plain[1]).max() > 0.05
+  for got_, want_, name in zip((dxe, dwi, dwo), want, ("dxe", "dwi", "dwo")):
+    np.testing.assert_allclose(
+        H.to_np(got_), want_, rtol=tol["rtol"],
+        atol=tol["atol"] * max(1.0, np.abs(want_).max()), err_msg=name)
+  # nothing to do / bad arguments
+  h0 = h.clone()
+  hip.hidden_product(h)
+  assert torch.equal(h, h0)
+  with pytest.raises(hip.MoeHipError):
+    hip.hidden_product(h, uniform=g(u), keep_prob=0.0)
+  with pytest.raises(hip.MoeHipError):
+    hip.hidden_product(h, factor=f[:, :1])

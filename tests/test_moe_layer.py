@@ -47,9 +47,15 @@ def run_v1(x, weights, hp, train, act_dtype, nonpadding=None, activation="relu",
         xt, mtf.Dimension("d_model", n), hp, train, vdt, nonpadding=npad,
         activation=activation, num_microbatches=num_microbatches)
   router = {"switch": "switch_gating", "switch_max": "switch_max_gating",
-            "ntlb": "ntlb_gating"}.get(hp.moe_gating, "top_2_gating")
+            "ntlb": "ntlb_gating",
+            "expert_selection": "expert_selection_gating"}.get(
+                hp.moe_gating, "top_2_gating")
   init = {"moe/%s/kernel" % router: weights["w_gate"],
-          "moe/wi/kernel": weights["wi"], "moe/wo/kernel": weights["wo"]}
+          "moe/wo/kernel": weights["wo"]}
+  if isinstance(weights["wi"], list):
+    init.update(("moe/wi_%d/kernel" % i, v) for i, v in enumerate(weights["wi"]))
+  else:
+    init["moe/wi/kernel"] = weights["wi"]
   lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()}, initial_values=init)
   out = H.to_np(lowering.export_to_tf_tensor(y))
   return out, float(H.to_np(lowering.export_to_tf_tensor(loss))), lowering, (xt, y)
@@ -133,6 +139,78 @@ def test_v1_nonpadding_eval_and_policies(act_dtype):
     assert (got[nonpadding == 0] == 0).all()
     np.testing.assert_allclose(got_loss, want_loss,
                                rtol=1e-2 if act_dtype == "bfloat16" else 1e-5)
+
+
+def run_v1_attention(x, weights, hp, train, act_dtype, nonpadding, activation):
+  """The layer with moe_use_experts_attention: returns [q, k] arrays."""
+  dt = H.ACT_TORCH[act_dtype]
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  b, l, m = x.shape
+  dims = [mtf.Dimension("batch", b), mtf.Dimension("length", l),
+          mtf.Dimension("d_model", m)]
+  xt = mtf.import_tf_tensor(mesh, torch.from_numpy(x).to(dt), mtf.Shape(dims))
+  npad = mtf.import_tf_tensor(mesh, torch.from_numpy(nonpadding).to(dt),
+                              mtf.Shape(dims[:2]))
+  with mtf.variable_scope("moe"):
+    outs, _ = moe.transformer_moe_layer_v1(
+        xt, dims[-1], hp, train,
+        mtf.VariableDType(torch.float32, torch.float32, dt), nonpadding=npad,
+        activation=activation)
+  init = {"moe/top_2_gating/kernel": weights["w_gate"],
+          "moe/q_wo/kernel": weights["wo"], "moe/k_wo/kernel": weights["k_wo"]}
+  init.update(("moe/wi_%d/kernel" % i, v) for i, v in enumerate(weights["wi"]))
+  lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()}, initial_values=init)
+  return [H.to_np(lowering.export_to_tf_tensor(t)) for t in outs]
+
+
+@pytest.mark.parametrize("case", [
+    (["gelu", "linear"], "float32", "top_2"),
+    (["gelu", "linear"], "bfloat16", "top_2"),
+    (["linear", "sigmoid"], "bfloat16", "switch"),
+    (["relu", "swish", "tanh"], "float32", "expert_selection"),
+    (["relu", "linear"], "bfloat16", "top_2+experts_attention")],
+    ids=lambda c: "%s-%s-%s" % ("*".join(c[0]), c[1], c[2]))
+def test_v1_gated_activations_match_oracle(case):
+  """A list of activations: the hidden tensor is the product of one dense layer
+  per entry (gated units), variables "wi_0", "wi_1", ..."""
+  acts, act_dtype, gating = case
+  gating, _, attention = gating.partition("+")
+  b, l, m, hdim, e, group = 2, 96, 32, 64, 4, 48
+  rng = np.random.default_rng(211)
+  w = dict(w_gate=H.normal_weights(rng, (m, e), m),
+           wi=[H.normal_weights(rng, (e, m, hdim), m) for _ in acts],
+           wo=H.normal_weights(rng, (e, hdim, m), hdim))
+  x = H.safe_tokens(rng, b * l, m, w["w_gate"], act_dtype).reshape(b, l, m)
+  nonpad = (rng.random((b, l)) < 0.9).astype(np.float32)
+  kw = dict(moe_num_experts=e, moe_hidden_size=hdim, moe_group_size=group,
+            moe_capacity_factor_eval=1.0)
+  if gating != "top_2":
+    kw.update(SWITCH_HP, moe_gating=gating)
+  if attention:
+    kw.update(moe_use_experts_attention=True)
+    w["k_wo"] = H.normal_weights(rng, (e, hdim, m), hdim)
+  hp, ohp = make_hparams(**kw)
+  if attention:
+    got = run_v1_attention(x, w, hp, False, act_dtype, nonpad, acts)
+    want, _, _ = O.moe_layer_v1(x, w["w_gate"], w["wi"], w["wo"], ohp, False,
+                                act_dtype, nonpadding=nonpad, activation=acts,
+                                dense=False, k_wo=w["k_wo"])
+    for g_, w_ in zip(got, want):
+      np.testing.assert_allclose(g_, w_, **H.value_tolerance(act_dtype))
+    return
+  got, got_loss, _, _ = run_v1(x, w, hp, False, act_dtype, nonpadding=nonpad,
+                               activation=acts)
+  want, want_loss, aux = O.moe_layer_v1(
+      x, w["w_gate"], w["wi"], w["wo"], ohp, False, act_dtype,
+      nonpadding=nonpad, activation=acts, dense=False)
+  single, _, _ = O.moe_layer_v1(
+      x, w["w_gate"], w["wi"][0], w["wo"], ohp, False, act_dtype,
+      nonpadding=nonpad, activation=acts[0], dense=False)
+  assert np.abs(want - single).max() > 0.05      # the other factors matter
+  np.testing.assert_allclose(got, want, **H.value_tolerance(act_dtype))
+  np.testing.assert_allclose(got_loss, want_loss,
+                             rtol=1e-2 if act_dtype == "bfloat16" else 1e-5)
 
 
 def test_v1_rerun_with_new_inputs():
@@ -441,13 +519,19 @@ def test_v1_switch_max_matches_oracle():
     ("switch", "float32", 103), ("switch_max", "float32", 104),
     ("ntlb", "float32", 105), ("switch+input_jitter", "float32", 106),
     ("switch+input_dropout", "bfloat16", 107),
-    ("ntlb+input_jitter", "float32", 108)],
+    ("ntlb+input_jitter", "float32", 108),
+    ("top_2+hidden_dropout", "float32", 109),
+    ("top_2+hidden_dropout", "bfloat16", 110),
+    ("switch+hidden_dropout", "float32", 111)],
     ids=lambda c: "%s-%s" % (c[0], c[1]))
 def test_v1_gradients_match_oracle(case):
   """mtf.gradients over the layer (outputs and loss) against the oracle's
   backward, which central differences pin in tests/test_oracle.py."""
   gating, act_dtype, seed = case
   gating, _, noise_policy = gating.partition("+")
+  hidden_dropout = noise_policy == "hidden_dropout"
+  if hidden_dropout:
+    noise_policy = ""
   b, l, m, hdim, e, group = 2, 64, 32, 48, 4, 32
   rng = np.random.default_rng(seed)
   w = dict(w_gate=H.normal_weights(rng, (m, e), m),
@@ -465,6 +549,8 @@ def test_v1_gradients_match_oracle(case):
   if noise_policy:
     kw.update(moe_switch_policy_train=noise_policy, moe_switch_jitter=0.25,
               moe_switch_dropout=0.3)
+  if hidden_dropout:
+    kw.update(moe_dropout_rate=0.25)
   hp, ohp = make_hparams(**kw)
   dt = H.ACT_TORCH[act_dtype]
   graph = mtf.Graph()
@@ -496,17 +582,37 @@ def test_v1_gradients_match_oracle(case):
     torch.manual_seed(seed)
     noise = torch.rand((1, b * l, m), dtype=torch.float32,
                        device="cuda").cpu().numpy().reshape(b, l, m)
+  hu = None
+  if hidden_dropout:       # likewise: uniforms of the hidden tensor's shape
+    torch.manual_seed(seed)
+    cap = O.expert_capacity(group, 1.0, e, 4)
+    hu = torch.rand((e, (b * l // group) * cap, hdim), dtype=dt,
+                    device="cuda").float().cpu().numpy()
   want = O.moe_layer_v1_backward(x, w["w_gate"], w["wi"], w["wo"], ohp, True,
                                  act_dtype, d_out, 1.5, nonpadding=nonpad,
-                                 num_microbatches=2, gate_noise=noise)
+                                 num_microbatches=2, gate_noise=noise,
+                                 hidden_uniform=hu)
   assert not (want["aux"]["kept_1"] | want["aux"]["kept_2"]).all()
+  if hidden_dropout:
+    out_got = H.to_np(lowering.export_to_tf_tensor(y))
+    out_want, _, _ = O.moe_layer_v1(x, w["w_gate"], w["wi"], w["wo"], ohp, True,
+                                    act_dtype, nonpadding=nonpad,
+                                    num_microbatches=2, dense=False,
+                                    hidden_uniform=hu)
+    out_plain, _, _ = O.moe_layer_v1(
+        x, w["w_gate"], w["wi"], w["wo"],
+        make_hparams(**dict(kw, moe_dropout_rate=0.0))[1], True, act_dtype,
+        nonpadding=nonpad, num_microbatches=2, dense=False)
+    assert np.abs(out_want - out_plain).max() > 0.05     # units were dropped
+    np.testing.assert_allclose(out_got, out_want,
+                               **H.value_tolerance(act_dtype))
   tol = H.value_tolerance(act_dtype)
   for g_, k in zip(got, ("dx", "dw_gate", "dwi", "dwo")):
     ref = want[k].reshape(g_.shape)
     np.testing.assert_allclose(
         g_, ref, rtol=tol["rtol"], atol=tol["atol"] * max(1.0, np.abs(ref).max()),
         err_msg=k)
-  if noise_policy:
+  if noise_policy or hidden_dropout:
     return        # a second step would draw new noise
   # a second step re-runs forward and backward on new tokens
   x2 = H.safe_tokens(rng, b * l, m, w["w_gate"], act_dtype,

@@ -927,8 +927,94 @@ def test_switch_golden_fixture():
   np.testing.assert_allclose(r["loss"], gold["loss"], rtol=1e-6)
 
 
+def test_gated_expert_hidden_against_float64():
+  """Product of dense layers (gated units): an independent float64 evaluation,
+  the one-factor list equals the plain layer, and a zero kernel in one linear
+  factor zeroes the output."""
+  rng = np.random.default_rng(77)
+  e, r, m, h, n = 3, 10, 6, 8, 5
+  xe = rng.standard_normal((e, r, m)).astype(np.float32)
+  wi0 = rng.standard_normal((e, m, h)).astype(np.float32)
+  wi1 = rng.standard_normal((e, m, h)).astype(np.float32)
+  wo = rng.standard_normal((e, h, n)).astype(np.float32)
+  x64, a64, b64, o64 = (v.astype(np.float64) for v in (xe, wi0, wi1, wo))
+  for acts, f0, f1 in (
+      (["gelu", "linear"], None, lambda v: v),
+      (["linear", "sigmoid"], lambda v: v, scipy.special.expit),
+      (["relu", "swish"], lambda v: np.maximum(v, 0),
+       lambda v: v * scipy.special.expit(v)),
+      (["tanh", "relu"], np.tanh, lambda v: np.maximum(v, 0))):
+    if f0 is None:      # tanh-approximated gelu, ops.py gelu
+      f0 = lambda v: 0.5 * v * (1 + np.tanh(
+          np.sqrt(2 / np.pi) * (v + 0.044715 * v ** 3)))
+    want = (f0(x64 @ a64) * f1(x64 @ b64)) @ o64
+    got = O.expert_ffn(xe, [wi0, wi1], wo, acts, "float32")
+    np.testing.assert_allclose(got, want, rtol=2e-4, atol=2e-4)
+    # the factors commute
+    swapped = O.expert_ffn(xe, [wi1, wi0], wo, acts[::-1], "float32")
+    np.testing.assert_allclose(swapped, got, rtol=1e-5, atol=1e-5)
+  np.testing.assert_array_equal(
+      O.expert_ffn(xe, [wi0], wo, ["relu"], "bfloat16"),
+      O.expert_ffn(xe, wi0, wo, "relu", "bfloat16"))
+  np.testing.assert_array_equal(
+      O.expert_ffn(xe, [wi0, np.zeros_like(wi1)], wo, ["relu", "linear"],
+                   "float32"), np.zeros((e, r, n), np.float32))
+  with pytest.raises(ValueError):
+    O.expert_ffn(xe, [wi0, wi1], wo, ["relu"], "float32")
+
+
+@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
+def test_hidden_dropout_noise(act_dtype):
+  """The dropout multiplier: zero or 1 / keep_prob in the tensor's dtype, strict
+  comparison, scalars rounded to that dtype (checked against torch's own
+  arithmetic in that dtype)."""
+  import torch
+  tdt = torch.float32 if act_dtype == "float32" else torch.bfloat16
+  rng = np.random.default_rng(5)
+  for keep in (0.5, 0.9, 0.75, 0.3):
+    u = O.cast_act(rng.random((4, 50, 7)).astype(np.float32), act_dtype)
+    keep_t = torch.tensor(keep, dtype=tdt)
+    u[0, 0, 0] = float(keep_t)                          # not strictly below
+    u[0, 0, 1] = 0.0
+    noise = O.hidden_dropout_noise(u, keep, act_dtype)
+    want = ((torch.from_numpy(u).to(tdt) < keep_t).to(tdt) / keep_t).float().numpy()
+    np.testing.assert_array_equal(noise, want)
+    assert noise[0, 0, 0] == 0 and noise[0, 0, 1] > 1
+    assert set(np.unique(noise)) == {0.0, float(torch.tensor(1.0, dtype=tdt) / keep_t)}
+    assert abs(noise.mean() - 1.0) < 0.15
+  # the layer: dropped hidden units change the output, evaluation ignores it,
+  # and keep_prob -> noise of all ones is the plain layer
+  e, m, hdim, group = 4, 8, 12, 32
+  x = rng.standard_normal((2, 32, m)).astype(np.float32)
+  wg = rng.standard_normal((m, e)).astype(np.float32)
+  wi = rng.standard_normal((e, m, hdim)).astype(np.float32)
+  wo = rng.standard_normal((e, hdim, m)).astype(np.float32)
+  hp = _hp(moe_num_experts=e, moe_hidden_size=hdim, moe_group_size=group,
+           moe_dropout_rate=0.5)
+  hp0 = _hp(moe_num_experts=e, moe_hidden_size=hdim, moe_group_size=group)
+  cap = O.expert_capacity(group, hp.moe_capacity_factor_train, e,
+                          hp.moe_min_expert_capacity)
+  hu = rng.random((e, 2 * cap, hdim)).astype(np.float32)
+  plain, _, _ = O.moe_layer_v1(x, wg, wi, wo, hp0, True, act_dtype, dense=False)
+  with pytest.raises(NotImplementedError):
+    O.moe_layer_v1(x, wg, wi, wo, hp, True, act_dtype, dense=False)
+  dropped, _, _ = O.moe_layer_v1(x, wg, wi, wo, hp, True, act_dtype,
+                                 dense=False, hidden_uniform=hu)
+  assert np.abs(dropped - plain).max() > 0.1
+  ev, _, _ = O.moe_layer_v1(x, wg, wi, wo, hp, False, act_dtype, dense=False)
+  ev0, _, _ = O.moe_layer_v1(x, wg, wi, wo, hp0, False, act_dtype, dense=False)
+  np.testing.assert_array_equal(ev, ev0)
+  # all units kept with keep_prob 0.5: exactly twice the plain hidden tensor,
+  # hence (a power of two) exactly twice the plain output
+  twice, _, _ = O.moe_layer_v1(x, wg, wi, wo, hp, True, act_dtype, dense=False,
+                               hidden_uniform=np.zeros_like(hu))
+  np.testing.assert_allclose(twice, 2 * plain, rtol=1e-2 if act_dtype ==
+                             "bfloat16" else 1e-5, atol=1e-5)
+
+
 # ---- backward -------------------------------------------------------------------
-def _f64_layer(x, wg, wi, wo, aux, gating, m1, coef, mb, z_loss, mult=None):
+def _f64_layer(x, wg, wi, wo, aux, gating, m1, coef, mb, z_loss, mult=None,
+               hidden_noise=None):
   """Independent float64 forward of the v1 layer with the ROUTING HELD FIXED
   (experts, kept masks and density counts taken from `aux`): a smooth function
   of (x, wg, wi, wo) whose central differences pin the oracle's backward."""
@@ -940,16 +1026,19 @@ def _f64_layer(x, wg, wi, wo, aux, gating, m1, coef, mb, z_loss, mult=None):
   i1, i2 = aux["index_1"], aux["index_2"]
   k1, k2 = aux["kept_1"].astype(np.float64), aux["kept_2"].astype(np.float64)
 
-  def ffn(idx):
+  def ffn(idx, pos=None):
     h = np.maximum(np.einsum("gsm,gsmh->gsh", x, wi[idx]), 0.0)
+    if hidden_noise is not None:          # [E, G, C, H], per expert slot
+      cap = hidden_noise.shape[2]
+      h = h * hidden_noise[idx, np.arange(g)[:, None], np.minimum(pos, cap - 1)]
     return np.einsum("gsh,gshn->gsn", h, wo[idx])
   onehot1 = (i1[..., None] == np.arange(e)).astype(np.float64)
   if gating == "top_2":
     g1 = p[rows + (i1,)] * m1
     g2 = p[rows + (i2,)] * (1.0 - (i2 == i1) * m1)
     den = g1 + g2 + 1e-9
-    out = ((g1 / den * k1)[..., None] * ffn(i1)
-           + (g2 / den * k2)[..., None] * ffn(i2))
+    out = ((g1 / den * k1)[..., None] * ffn(i1, aux["pos_1"])
+           + (g2 / den * k2)[..., None] * ffn(i2, aux["pos_2"]))
     density = (onehot1 * m1[..., None]).mean(1)
     proxy = (p * m1[..., None]).mean(1)
     aux_loss = (proxy * density).mean() * e * e / mb
@@ -974,9 +1063,13 @@ def _f64_layer(x, wg, wi, wo, aux, gating, m1, coef, mb, z_loss, mult=None):
 
 @pytest.mark.parametrize("gating", ["top_2", "switch", "switch_max", "ntlb",
                                     "switch+jitter", "switch+dropout",
-                                    "ntlb+jitter", "switch+sample"])
+                                    "ntlb+jitter", "switch+sample",
+                                    "top_2+hidden"])
 def test_backward_against_central_differences(gating):
   gating, _, perturb = gating.partition("+")
+  hidden = perturb == "hidden"      # dropout on the experts' hidden tensor
+  if hidden:
+    perturb = ""
   rng = np.random.default_rng(61)
   b, l, m, h, e, group = 2, 24, 6, 10, 4, 24
   x = rng.standard_normal((b, l, m)).astype(np.float32)
@@ -993,12 +1086,22 @@ def test_backward_against_central_differences(gating):
                                     "input_" + perturb) if perturb else "argmax",
            moe_switch_temperature=2.0,
            moe_switch_jitter=0.3, moe_switch_dropout=0.25, moe_ntlb_top_k=3,
-           moe_z_loss=0.3 if gating == "switch" else None)
+           moe_z_loss=0.3 if gating == "switch" else None,
+           moe_dropout_rate=0.4 if hidden else 0.0)
   noise = rng.random((b, l, m)).astype(np.float32) if perturb else None
   su = rng.random((b * l // group, group, e)).astype(np.float32)
+  hu = hnoise = None
+  if hidden:
+    groups = b * l // group
+    cap = O.expert_capacity(group, 1.2, e, 2)
+    hu = rng.random((e, groups * cap, h)).astype(np.float32)
+    hnoise = ((hu < np.float32(0.6)) / np.float32(0.6)).astype(
+        np.float64).reshape(e, groups, cap, h)
+    assert 0.3 < (hnoise == 0).mean() < 0.5
   got = O.moe_layer_v1_backward(x, wg, wi, wo, hp, True, "float32", d_out,
                                 d_loss, nonpadding=nonpad, num_microbatches=mb,
-                                gate_noise=noise, sample_uniform=su)
+                                gate_noise=noise, sample_uniform=su,
+                                hidden_uniform=hu)
   aux = got["aux"]
   mult = None
   if perturb == "sample":       # sampled experts differ from the arg-max
@@ -1014,7 +1117,7 @@ def test_backward_against_central_differences(gating):
 
   def scalar(xv, wgv, wiv, wov):
     out, loss = _f64_layer(xv.reshape(b, l, m), wgv, wiv, wov, aux, gating, m1,
-                           0.5, mb, z, mult)
+                           0.5, mb, z, mult, hnoise)
     return (out * d_out.reshape(out.shape)).sum() + d_loss * loss
   base = [a.astype(np.float64) for a in (x.reshape(b, l, m), wg, wi, wo)]
   grads = [got["dx"].reshape(b, l, m), got["dw_gate"], got["dwi"], got["dwo"]]
