@@ -85,7 +85,7 @@ __global__ __launch_bounds__(256) void router_logits_kernel(
 // the reference on bf16-rounded operands up to summation order.
 //
 // A block is 4 wavefronts x 32 tokens; x and wp K tiles (64 deep) are brought
-// into a two-slot LDS ring by global_load_lds_dwordx4 with the same
+// into a three-slot LDS ring by global_load_lds_dwordx4 with the same
 // 128-byte-row XOR swizzle as the expert GEMM.  The kernel is bound by reading
 // x once from HBM.
 // ---------------------------------------------------------------------------
@@ -126,18 +126,26 @@ __global__ __launch_bounds__(256) void router_mfma_kernel(
     const int row = (wave + 4 * j) * 8 + (lane >> 3);
     w_off[j] = min(row, E - 1) * M + (((lane & 7) ^ rl_swizzle(row)) * 8);
   }
+  // Block b walks the K tiles starting at tile b % nk and wraps around: the
+  // blocks run in step, and with rows a power of two apart all of them asking
+  // for the same 128-byte column of their rows at the same moment lands on
+  // few memory channels (measured: 20 % slower).
+  const int nk = M / BK;
+  const int rot = (int)(blockIdx.x % (unsigned)nk);
   auto issue = [&](int kt, int slot) {
     unsigned char* sx = rl_smem + slot * STAGE;
     unsigned char* sw = sx + X_BYTES;
+    int kq = kt + rot;
+    if (kq >= nk) kq -= nk;
 #pragma unroll
     for (int j = 0; j < 4; ++j)
       __builtin_amdgcn_global_load_lds(
-          (rl_glb_void_t*)(xb + kt * BK + x_off[j]),
+          (rl_glb_void_t*)(xb + kq * BK + x_off[j]),
           (rl_lds_void_t*)(sx + (wave + 4 * j) * 1024), 16, 0, 0);
 #pragma unroll
     for (int j = 0; j < NT; ++j)
       __builtin_amdgcn_global_load_lds(
-          (rl_glb_void_t*)(wb + kt * BK + w_off[j]),
+          (rl_glb_void_t*)(wb + kq * BK + w_off[j]),
           (rl_lds_void_t*)(sw + (wave + 4 * j) * 1024), 16, 0, 0);
   };
 
@@ -155,16 +163,26 @@ __global__ __launch_bounds__(256) void router_mfma_kernel(
     x_frag[kk] = (wave * 32 + fr) * ROWB + col;
     w_frag[kk] = fr * ROWB + col;
   }
-  const int nk = M / BK;
+  // Three slots, two K tiles in flight: the loop is bound by the latency of
+  // one round trip to HBM per K tile, so what it moves per second is the bytes
+  // it keeps in flight.  vmcnt retires in issue order: leaving the newest
+  // tile's 4 + NT loads outstanding means tile kt has landed.  Passing the
+  // barrier of step kt also means every wavefront has finished reading slot
+  // (kt - 1) % 3, which the loads of tile kt + 2 then overwrite.
   issue(0, 0);
+  if (nk > 1) issue(1, 1);
+  int slot = 0;
   for (int kt = 0; kt < nk; ++kt) {
-    const int slot = kt & 1;
-    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+    if (kt + 1 < nk)
+      __builtin_amdgcn_s_waitcnt(0x0070 | (4 + NT));  // vmcnt(4+NT) lgkmcnt(0)
+    else
+      __builtin_amdgcn_s_waitcnt(0x0070);             // vmcnt(0) lgkmcnt(0)
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    if (kt + 1 < nk) issue(kt + 1, slot ^ 1);
+    if (kt + 2 < nk) issue(kt + 2, slot == 0 ? 2 : slot - 1);
     const unsigned char* sx = rl_smem + slot * STAGE;
+    slot = slot == 2 ? 0 : slot + 1;
     const unsigned char* sw = sx + X_BYTES;
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
@@ -440,18 +458,26 @@ __global__ __launch_bounds__(256) void router_gate_kernel(
     const int row = (wave + 4 * j) * 8 + (lane >> 3);
     w_off[j] = min(row, E - 1) * M + (((lane & 7) ^ rl_swizzle(row)) * 8);
   }
+  // Block b walks the K tiles starting at tile b % nk and wraps around: the
+  // blocks run in step, and with rows a power of two apart all of them asking
+  // for the same 128-byte column of their rows at the same moment lands on
+  // few memory channels (measured: 20 % slower).
+  const int nk = M / BK;
+  const int rot = (int)(blockIdx.x % (unsigned)nk);
   auto issue = [&](int kt, int slot) {
     unsigned char* sx = rl_smem + slot * STAGE;
     unsigned char* sw = sx + X_BYTES;
+    int kq = kt + rot;
+    if (kq >= nk) kq -= nk;
 #pragma unroll
     for (int j = 0; j < 4; ++j)
       __builtin_amdgcn_global_load_lds(
-          (rl_glb_void_t*)(xb + kt * BK + x_off[j]),
+          (rl_glb_void_t*)(xb + kq * BK + x_off[j]),
           (rl_lds_void_t*)(sx + (wave + 4 * j) * 1024), 16, 0, 0);
 #pragma unroll
     for (int j = 0; j < NT; ++j)
       __builtin_amdgcn_global_load_lds(
-          (rl_glb_void_t*)(wb + kt * BK + w_off[j]),
+          (rl_glb_void_t*)(wb + kq * BK + w_off[j]),
           (rl_lds_void_t*)(sw + (wave + 4 * j) * 1024), 16, 0, 0);
   };
   rl_f32x16_t acc[NT];
@@ -467,16 +493,26 @@ __global__ __launch_bounds__(256) void router_gate_kernel(
     x_frag[kk] = (wave * 32 + fr) * ROWB + col;
     w_frag[kk] = fr * ROWB + col;
   }
-  const int nk = M / BK;
+  // Three slots, two K tiles in flight: the loop is bound by the latency of
+  // one round trip to HBM per K tile, so what it moves per second is the bytes
+  // it keeps in flight.  vmcnt retires in issue order: leaving the newest
+  // tile's 4 + NT loads outstanding means tile kt has landed.  Passing the
+  // barrier of step kt also means every wavefront has finished reading slot
+  // (kt - 1) % 3, which the loads of tile kt + 2 then overwrite.
   issue(0, 0);
+  if (nk > 1) issue(1, 1);
+  int slot = 0;
   for (int kt = 0; kt < nk; ++kt) {
-    const int slot = kt & 1;
-    __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0)
+    if (kt + 1 < nk)
+      __builtin_amdgcn_s_waitcnt(0x0070 | (4 + NT));  // vmcnt(4+NT) lgkmcnt(0)
+    else
+      __builtin_amdgcn_s_waitcnt(0x0070);             // vmcnt(0) lgkmcnt(0)
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
-    if (kt + 1 < nk) issue(kt + 1, slot ^ 1);
+    if (kt + 2 < nk) issue(kt + 2, slot == 0 ? 2 : slot - 1);
     const unsigned char* sx = rl_smem + slot * STAGE;
+    slot = slot == 2 ? 0 : slot + 1;
     const unsigned char* sw = sx + X_BYTES;
 #pragma unroll
     for (int kk = 0; kk < 4; ++kk) {
@@ -737,7 +773,7 @@ template <int NT>
 static int launch_router_mfma(const bf16_t* x, const bf16_t* wp,
                               const float* bias, float* logits, int batch,
                               int tokens, int M, int E, hipStream_t st) {
-  const size_t smem = 2 * (128 * 128 + (size_t)NT * 32 * 128);
+  const size_t smem = 3 * (128 * 128 + (size_t)NT * 32 * 128);
   auto k = router_mfma_kernel<NT>;
   MOE_ALLOW_LDS(k, smem);
   dim3 grid((unsigned)((tokens + 127) / 128), (unsigned)batch);
@@ -880,7 +916,7 @@ static int launch_router_gate(const bf16_t* x, const bf16_t* wp,
                               int32_t* idx, int32_t* pos, float* gate,
                               uint8_t* kept, float* part1, float* part2,
                               int tokens_per_batch, hipStream_t st) {
-  const size_t ring = 2 * (128 * 128 + (size_t)NT * 32 * 128);
+  const size_t ring = 3 * (128 * 128 + (size_t)NT * 32 * 128);
   const size_t tile = sizeof(float) * (128 * (size_t)(p.E + 1) + 128);
   const size_t smem = ring > tile ? ring : tile;
   auto k = router_gate_kernel<NT, IT>;
