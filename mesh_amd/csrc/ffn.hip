@@ -251,6 +251,8 @@ __global__ __launch_bounds__(256) void grouped_gemm_bf16_kernel(
 // Requires K % 64 == 0 and per-expert operand sizes below 2^30 elements.
 // ---------------------------------------------------------------------------
 typedef __attribute__((address_space(3))) void lds_void_t;
+typedef short i16x4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) i16x4_t lds_i16x4_t;
 typedef const __attribute__((address_space(1))) void glb_void_t;
 
 template <int N>
@@ -504,6 +506,17 @@ __global__ __launch_bounds__(64 * WM * WN) void grouped_gemm_bf16_dma_kernel(
 // everything up to the token loads of tile t+1 has landed, the four weight
 // loads of tile t+2 stay in flight.
 // ---------------------------------------------------------------------------
+// Two ds_read_b64_tr_b16 at byte offsets OFF and OFF + 2048 from LDS address
+// `addr` (see the K-major variant of the ring kernel).
+template <int OFF>
+__device__ __forceinline__ void lds_read_tr16_pair(uint32_t addr, i16x4_t& lo,
+                                                   i16x4_t& hi) {
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2"
+               : "=v"(lo) : "v"(addr), "n"(OFF));
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2"
+               : "=v"(hi) : "v"(addr), "n"(OFF + 2048));
+}
+
 struct RingCfg {
   static constexpr int BM = 256, BN = 256, BK = 64, WM = 2, WN = 4;
   static constexpr int WAVES = WM * WN, THREADS = 64 * WAVES;
@@ -523,7 +536,17 @@ struct RingCfg {
 // shared token matrix, A[row_map[e * R + r]] (row_map < 0: the all-zero row
 // `zero_row`): the dispatch of the Mixture-of-Experts layer folded into the
 // first expert GEMM's loads.
-template <bool RELU, bool GATHER = false>
+//
+// KMAJOR: both operands are stored with the reduction index outermost,
+// A[e][k][r] and B[e][k][n] (C = A^T . B, the weight gradients of the expert
+// einsums: the reduction runs over token rows).  A K tile is then 64 rows of
+// 256 consecutive elements; it goes to LDS as it lies in memory (row k at byte
+// 512 k, the 64-byte units of a row XOR-ed with k % 4 against bank
+// conflicts) and the MFMA operands, which need 8 consecutive k per lane, are
+// read with ds_read_b64_tr_b16: within 16 lanes, lane t addresses the 8 bytes
+// at (row t / 4, elements 4 (t % 4) ..) of a 4 x 16 block and lane i receives
+// the block's column i.  R, N multiples of 8.
+template <bool RELU, bool GATHER = false, bool KMAJOR = false>
 __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
     bf16_t* __restrict__ Cout, int R, int N, int K, int tiles_m, int tiles_n,
@@ -579,6 +602,17 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
     Ce = Cout + (int64_t)e * R * N;
 #pragma unroll
     for (int j = 0; j < Cfg::A_INSTR; ++j) {
+      if constexpr (KMAJOR) {
+        // instruction q = wave + WAVES * j fills tile rows 2q and 2q + 1; lane
+        // l fills 16-byte position l % 32 of its row with the chunk that
+        // belongs there under the unit swizzle
+        const int krow = (wave + Cfg::WAVES * j) * 2 + (lane >> 5);
+        const int p = lane & 31;
+        const int chunk = ((((p >> 2) ^ (krow & 3)) << 2) | (p & 3)) * 8;
+        a_off[j] = krow * R + min(row0 + chunk, R - 8);
+        b_off[j] = krow * N + min(col0 + chunk, N - 8);
+        continue;
+      }
       const int row = (wave + Cfg::WAVES * j) * 8 + (lane >> 3);
       const int chunk = (lane & 7) ^ lds_swizzle(row);
       if constexpr (GATHER) {
@@ -599,14 +633,14 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
     const int slot = kt & 1;
     kt = min(kt, nk - 1);
     __builtin_amdgcn_global_load_lds(
-        (glb_void_t*)(Ae + kt * BK + a_off[j]),
+        (glb_void_t*)(Ae + kt * (KMAJOR ? BK * R : BK) + a_off[j]),
         (lds_void_t*)(smem_raw + slot * Cfg::A_BYTES +
                       (wave + Cfg::WAVES * j) * 1024), 16, 0, 0);
   };
   auto load_b = [&](int kt, int slot, int j) {
     kt = min(kt, nk - 1);
     __builtin_amdgcn_global_load_lds(
-        (glb_void_t*)(Be + kt * BK + b_off[j]),
+        (glb_void_t*)(Be + kt * (KMAJOR ? BK * N : BK) + b_off[j]),
         (lds_void_t*)(smem_raw + B_BASE + slot * Cfg::B_BYTES +
                       (wave + Cfg::WAVES * j) * 1024), 16, 0, 0);
   };
@@ -629,16 +663,65 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
 
   const int fr = lane & 31, fc = lane >> 5;
   int a_frag[BK / 16], b_frag[BK / 16];
+  if constexpr (KMAJOR) {
+    // byte offset of this lane's 8 bytes for 32-column block n of its
+    // wavefront's sub-tile, at step 0 / first half: a_frag[n], b_frag[n]
+    static_assert(Cfg::TM <= BK / 16 && Cfg::TN <= BK / 16, "offset arrays");
+    const int t = lane & 15, g = lane >> 4;
+    const int inner = ((g & 1) * 16 + 4 * (t & 3)) * 2 +
+                      ((g >> 1) * 8 + (t >> 2)) * 512;
 #pragma unroll
-  for (int kk = 0; kk < BK / 16; ++kk) {
-    const int col = ((kk * 2 + fc) ^ lds_swizzle(fr)) * 16;
-    a_frag[kk] = (wm * Cfg::WTM + fr) * Cfg::ROW_BYTES + col;
-    b_frag[kk] = (wn * Cfg::WTN + fr) * Cfg::ROW_BYTES + col;
+    for (int n = 0; n < Cfg::TM; ++n)
+      a_frag[n] = (((wm * Cfg::TM + n) ^ (t >> 2)) * 64) + inner;
+#pragma unroll
+    for (int n = 0; n < Cfg::TN; ++n)
+      b_frag[n] = (((wn * Cfg::TN + n) ^ (t >> 2)) * 64) + inner;
+  } else {
+#pragma unroll
+    for (int kk = 0; kk < BK / 16; ++kk) {
+      const int col = ((kk * 2 + fc) ^ lds_swizzle(fr)) * 16;
+      a_frag[kk] = (wm * Cfg::WTM + fr) * Cfg::ROW_BYTES + col;
+      b_frag[kk] = (wn * Cfg::WTN + fr) * Cfg::ROW_BYTES + col;
+    }
   }
   constexpr int KSTEPS = BK / 16;
   bf16x8_t fa[2][Cfg::TM], fb[2][Cfg::TN];
+  // 8 consecutive k of one column of a K-major tile: two transposed reads at
+  // LDS byte address `at` + 8192 kk (+ 2048 for the second four).  Written as
+  // asm because the compiler puts a vmcnt(0) in front of the builtin form (it
+  // takes the read for a possible LDS store racing the direct-to-LDS loads),
+  // which would drain the loads that are meant to stay in flight.  The
+  // compiler therefore does not know when the data arrives: wait_frags()
+  // (lgkmcnt(0)) stands before the MFMAs that use it.
+  const uint32_t lds0 = (uint32_t)(size_t)(lds_void_t*)smem_raw;
+  auto read_tr = [&](uint32_t at, int kk) {
+    i16x4_t lo, hi;
+    switch (kk) {
+      case 0: lds_read_tr16_pair<0>(at, lo, hi); break;
+      case 1: lds_read_tr16_pair<8192>(at, lo, hi); break;
+      case 2: lds_read_tr16_pair<16384>(at, lo, hi); break;
+      default: lds_read_tr16_pair<24576>(at, lo, hi); break;
+    }
+    return __builtin_bit_cast(
+        bf16x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+  };
+  auto wait_frags = [&]() {
+    if constexpr (KMAJOR) {
+      __builtin_amdgcn_sched_barrier(0);
+      __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0) only
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  };
   // fragment read n of a step: 0..TM-1 token rows, TM..TM+TN-1 weight rows
   auto read_frag = [&](int aslot, int bslot, int kk, int buf, int n) {
+    if constexpr (KMAJOR) {
+      if (n < Cfg::TM)
+        fa[buf][n] = read_tr(lds0 + aslot * Cfg::A_BYTES + a_frag[n], kk);
+      else
+        fb[buf][n - Cfg::TM] = read_tr(
+            lds0 + B_BASE + bslot * Cfg::B_BYTES + b_frag[n - Cfg::TM], kk);
+      return;
+    }
     if (n < Cfg::TM)
       fa[buf][n] = *reinterpret_cast<const bf16x8_t*>(
           smem_raw + aslot * Cfg::A_BYTES + a_frag[kk] + n * 32 * Cfg::ROW_BYTES);
@@ -682,6 +765,7 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
         // 6 fragment reads of step kk+1 (in the order its MFMAs need them),
         // 2 loads, 8 MFMAs of step kk
         fence();
+        wait_frags();
         read_frag(aslot, bslot, kk + 1, nxt, RD[0]);
         read_frag(aslot, bslot, kk + 1, nxt, RD[1]);
         mfma(cur, 0); fence();
@@ -718,6 +802,7 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
         mfma(cur, 6); fence();
         mfma(cur, 7); fence();
       } else {
+        wait_frags();
 #pragma unroll
         for (int n = 0; n < 8; ++n) mfma(cur, n);
       }
@@ -981,6 +1066,52 @@ static int launch_dma(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
   return 0;
 }
 
+// Compute units of the current device (one persistent block per CU: a block
+// takes all of a CU's LDS); 0 on failure.
+static int compute_units() {
+  static int cus = 0;
+  if (cus == 0) {
+    int dev = 0, n = 0;
+    if (hipGetDevice(&dev) != hipSuccess ||
+        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) !=
+            hipSuccess || n < 1) {
+      set_error("expert_ffn: cannot query the number of compute units");
+      return 0;
+    }
+    cus = n;
+  }
+  return cus;
+}
+
+// C[e] [R, N] = A[e]^T . B[e] with A[e] [K, R] and B[e] [K, N] (both with the
+// reduction index outermost); true if the K-major ring kernel takes the shape.
+static bool kmajor_path_applies(const void* A, const void* B, const void* C,
+                                int R, int N, int K, int dtype) {
+  return dtype == MESH_MOE_BF16 && K % RingCfg::BK == 0 && K >= RingCfg::BK &&
+         R % 8 == 0 && N % 8 == 0 && R >= 128 && N >= 128 &&
+         (int64_t)R * K < (1LL << 31) && (int64_t)N * K < (1LL << 31) &&
+         (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15) == 0;
+}
+
+static int launch_ring_kmajor(const bf16_t* A, const bf16_t* B, bf16_t* C,
+                              int E, int R, int N, int K, hipStream_t st) {
+  using Cfg = RingCfg;
+  const int tiles_m = (R + Cfg::BM - 1) / Cfg::BM;
+  const int tiles_n = (N + Cfg::BN - 1) / Cfg::BN;
+  const int64_t tiles = (int64_t)tiles_m * tiles_n * E;
+  MOE_REQUIRE(tiles <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
+              "expert_ffn_backward: too many tiles (%lld)", (long long)tiles);
+  const int cus = compute_units();
+  if (cus == 0) return MESH_MOE_E_HIP;
+  const unsigned blocks = (unsigned)(tiles < cus ? tiles : cus);
+  auto k = grouped_gemm_bf16_ring_kernel<false, false, true>;
+  MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
+  k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
+      A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr);
+  MOE_CHECK_LAUNCH("expert_ffn_backward (mfma, K-major operands)");
+  return 0;
+}
+
 static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
                        int R, int N, int K, bool relu, hipStream_t st,
                        const int32_t* row_map = nullptr,
@@ -991,18 +1122,8 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
   const int64_t tiles = (int64_t)tiles_m * tiles_n * E;
   MOE_REQUIRE(tiles <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
               "expert_ffn: too many tiles (%lld)", (long long)tiles);
-  // one persistent block per CU (a block takes all of a CU's LDS)
-  static int cus = 0;
-  if (cus == 0) {
-    int dev = 0, n = 0;
-    if (hipGetDevice(&dev) != hipSuccess ||
-        hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) !=
-            hipSuccess || n < 1) {
-      set_error("expert_ffn: cannot query the number of compute units");
-      return MESH_MOE_E_HIP;
-    }
-    cus = n;
-  }
+  const int cus = compute_units();
+  if (cus == 0) return MESH_MOE_E_HIP;
   const unsigned blocks = (unsigned)(tiles < cus ? tiles : cus);
   if (row_map != nullptr) {
     if (relu) {
@@ -1358,7 +1479,17 @@ extern "C" int mesh_moe_expert_ffn_backward(
   rc = grouped_gemm(dh, wi, dexpert_in, E, R, M, H, MESH_MOE_ACT_LINEAR, dtype,
                     st);
   if (rc != 0) return rc;
-  // dwo [E, H, N] = h^T . dy: both operands transposed to token-contiguous
+  // dwo [E, H, N] = h^T . dy and dwi [E, M, H] = expert_in^T . dh: the
+  // reduction runs over token rows, the outermost index of both operands
+  if (kmajor_path_applies(h, dy, dwo, H, N, R, dtype) &&
+      kmajor_path_applies(expert_in, dh, dwi, M, H, R, dtype)) {
+    rc = launch_ring_kmajor((const bf16_t*)h, (const bf16_t*)dy, (bf16_t*)dwo,
+                            E, H, N, R, st);
+    if (rc != 0) return rc;
+    return launch_ring_kmajor((const bf16_t*)expert_in, (const bf16_t*)dh,
+                              (bf16_t*)dwi, E, M, H, R, st);
+  }
+  // otherwise: both operands transposed to token-contiguous copies first
   rc = mesh_moe_pack_weights(h, tr_h, E, R, H, dtype, dtype, stream);
   if (rc != 0) return rc;
   rc = mesh_moe_pack_weights(dy, tr_mn, E, R, N, dtype, dtype, stream);

@@ -878,3 +878,34 @@ def test_hidden_product_and_dropout_backward(hip, act_dtype, activation):
     hip.hidden_product(h, uniform=g(u), keep_prob=0.0)
   with pytest.raises(hip.MoeHipError):
     hip.hidden_product(h, factor=f[:, :1])
+
+
+@pytest.mark.parametrize("shape", [(2, 128, 256, 512, 256), (3, 192, 136, 264, 136),
+                                   (1, 2048, 512, 1024, 256), (2, 64, 256, 256, 128),
+                                   (2, 96, 256, 256, 256)])
+def test_expert_ffn_backward_weight_gradients_bf16(hip, shape):
+  """bf16 weight gradients dwi = expert_in^T . dh and dwo = h^T . dy: the
+  reduction runs over token rows.  Row counts that are multiples of 64 take the
+  kernel that reads both operands as they lie in memory (transposing LDS
+  reads); the last shape takes the path through transposed copies.  Both
+  against float32 matmuls of the same bf16 operands."""
+  e, rows, m, hdim, n = shape
+  rng = np.random.default_rng(sum(shape))
+  g = lambda a: H.to_gpu(O.cast_act(a.astype(np.float32), "bfloat16"), "bfloat16")
+  xe = g(rng.standard_normal((e, rows, m)))
+  wi = g(H.normal_weights(rng, (e, m, hdim), m))
+  wo = g(H.normal_weights(rng, (e, hdim, n), hdim))
+  dy = g(rng.standard_normal((e, rows, n)))
+  wi_p = hip.pack_weights(wi, torch.bfloat16)
+  h = hip.expert_linear(xe, wi_p, "relu")
+  dxe, dwi, dwo = hip.expert_ffn_backward(xe, h, dy, wi, wo, "relu")
+  dh = (torch.bmm(dy.float(), wo.float().transpose(1, 2)).to(torch.bfloat16).float()
+        * (h > 0))
+  want_dwo = torch.bmm(h.float().transpose(1, 2), dy.float())
+  want_dwi = torch.bmm(xe.float().transpose(1, 2), dh)
+  want_dxe = torch.bmm(dh, wi.float().transpose(1, 2))
+  for got, want, name in ((dwo, want_dwo, "dwo"), (dwi, want_dwi, "dwi"),
+                          (dxe, want_dxe, "dxe")):
+    scale = float(want.abs().max())
+    np.testing.assert_allclose(H.to_np(got), H.to_np(want), rtol=2e-2,
+                               atol=1e-2 * scale, err_msg=name)
