@@ -546,12 +546,18 @@ struct RingCfg {
 // read with ds_read_b64_tr_b16: within 16 lanes, lane t addresses the 8 bytes
 // at (row t / 4, elements 4 (t % 4) ..) of a 4 x 16 block and lane i receives
 // the block's column i.  R, N multiples of 8.
-template <bool RELU, bool GATHER = false, bool KMAJOR = false>
+//
+// MASKED: element (e, r, n) of the result is stored as zero unless
+// mask_src[e][r][n] > 0 (the backward of a ReLU whose output is mask_src,
+// applied while the tile is written out).
+template <bool RELU, bool GATHER = false, bool KMAJOR = false,
+          bool MASKED = false>
 __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
     bf16_t* __restrict__ Cout, int R, int N, int K, int tiles_m, int tiles_n,
     int total_tiles, const int32_t* __restrict__ row_map = nullptr,
-    const bf16_t* __restrict__ zero_row = nullptr) {
+    const bf16_t* __restrict__ zero_row = nullptr,
+    const bf16_t* __restrict__ mask_src = nullptr) {
   using Cfg = RingCfg;
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, WN = Cfg::WN;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -889,8 +895,20 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
         const int grow = out_row0 + (srow >> 6) * 128 + pass * 64 + (srow & 63);
         const int gcol = out_col0 + chunk * 8;
         if (grow < R && gcol < N) {
-          const u32x4_t v = *reinterpret_cast<const u32x4_t*>(
+          u32x4_t v = *reinterpret_cast<const u32x4_t*>(
               Cs + srow * EPI_ROW_BYTES + ((chunk ^ (srow & 31)) * 16));
+          if constexpr (MASKED) {
+            const u32x4_t hm = *reinterpret_cast<const u32x4_t*>(
+                mask_src + (out_c - Cout) + (int64_t)grow * N + gcol);
+#pragma unroll
+            for (int q = 0; q < 4; ++q) {
+              const uint32_t keep =
+                  (__builtin_bit_cast(float, hm[q] << 16) > 0.f ? 0xffffu : 0u) |
+                  (__builtin_bit_cast(float, hm[q] & 0xffff0000u) > 0.f
+                       ? 0xffff0000u : 0u);
+              v[q] &= keep;
+            }
+          }
           *reinterpret_cast<u32x4_t*>(out_c + (int64_t)grow * N + gcol) = v;
         }
       }
@@ -1107,7 +1125,8 @@ static int launch_ring_kmajor(const bf16_t* A, const bf16_t* B, bf16_t* C,
   auto k = grouped_gemm_bf16_ring_kernel<false, false, true>;
   MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
   k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
-      A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr);
+      A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr,
+        nullptr);
   MOE_CHECK_LAUNCH("expert_ffn_backward (mfma, K-major operands)");
   return 0;
 }
@@ -1115,7 +1134,8 @@ static int launch_ring_kmajor(const bf16_t* A, const bf16_t* B, bf16_t* C,
 static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
                        int R, int N, int K, bool relu, hipStream_t st,
                        const int32_t* row_map = nullptr,
-                       const bf16_t* zero_row = nullptr) {
+                       const bf16_t* zero_row = nullptr,
+                       const bf16_t* mask_src = nullptr) {
   using Cfg = RingCfg;
   const int tiles_m = (R + Cfg::BM - 1) / Cfg::BM;
   const int tiles_n = (N + Cfg::BN - 1) / Cfg::BN;
@@ -1125,17 +1145,30 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
   const int cus = compute_units();
   if (cus == 0) return MESH_MOE_E_HIP;
   const unsigned blocks = (unsigned)(tiles < cus ? tiles : cus);
+  if (mask_src != nullptr) {
+    MOE_REQUIRE(!relu && row_map == nullptr, MESH_MOE_E_ARG,
+                "expert_ffn: masked result with relu or gathered rows");
+    auto k = grouped_gemm_bf16_ring_kernel<false, false, false, true>;
+    MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
+    k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
+        A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr,
+        mask_src);
+    MOE_CHECK_LAUNCH("expert_ffn (mfma, masked result)");
+    return 0;
+  }
   if (row_map != nullptr) {
     if (relu) {
       auto k = grouped_gemm_bf16_ring_kernel<true, true>;
       MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
       k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
-          A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, row_map, zero_row);
+          A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, row_map, zero_row,
+          nullptr);
     } else {
       auto k = grouped_gemm_bf16_ring_kernel<false, true>;
       MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
       k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
-          A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, row_map, zero_row);
+          A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, row_map, zero_row,
+          nullptr);
     }
     MOE_CHECK_LAUNCH("expert_ffn (mfma, gathered rows)");
     return 0;
@@ -1144,12 +1177,14 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
     auto k = grouped_gemm_bf16_ring_kernel<true, false>;
     MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
     k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
-        A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr);
+        A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr,
+        nullptr);
   } else {
     auto k = grouped_gemm_bf16_ring_kernel<false, false>;
     MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
     k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
-        A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr);
+        A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr,
+        nullptr);
   }
   MOE_CHECK_LAUNCH("expert_ffn (mfma, spread direct-to-LDS loads)");
   return 0;
@@ -1173,10 +1208,16 @@ static int launch_simple(const T* A, const T* B, T* C, int E, int R, int N,
 }
 
 // C[e] = act(A[e] . B[e]^T) for every expert.
+// relu_mask_src (same shape and dtype as C): the kernels that can zero the
+// elements of C whose mask_src element is not positive while they write C do so
+// and set *mask_applied; otherwise the caller runs the mask as a pass of its own.
 static int grouped_gemm(const void* A, const void* B, void* C, int E, int R,
-                        int N, int K, int act, int dtype, hipStream_t st) {
+                        int N, int K, int act, int dtype, hipStream_t st,
+                        const void* relu_mask_src = nullptr,
+                        bool* mask_applied = nullptr) {
   const bool relu = act == MESH_MOE_ACT_RELU;
   int rc;
+  if (mask_applied) *mask_applied = false;
   if (dtype == MESH_MOE_F32) {
     rc = launch_simple<float>((const float*)A, (const float*)B, (float*)C, E,
                               R, N, K, relu, st);
@@ -1196,10 +1237,16 @@ static int grouped_gemm(const void* A, const void* B, void* C, int E, int R,
       const int pad256 = (R + 255) / 256 * 256, pad128 = (R + 127) / 128 * 128;
       // 256 x 256 tiles run 8 wavefronts (two per SIMD, 128 x 64 sub-tiles)
       // with the loads spread over the MFMA steps
-      if (pad128 < pad256)
+      if (pad128 < pad256) {
         rc = launch_dma<128, 256, 2>(a, b, c, E, R, N, K, relu, st);
-      else
+      } else if (relu_mask_src != nullptr && mask_applied != nullptr && !relu &&
+                 ((uintptr_t)relu_mask_src % 16) == 0) {
+        rc = launch_ring(a, b, c, E, R, N, K, false, st, nullptr, nullptr,
+                         (const bf16_t*)relu_mask_src);
+        *mask_applied = rc == 0;
+      } else {
         rc = launch_ring(a, b, c, E, R, N, K, relu, st);
+      }
     } else if (R >= 1024 && N >= 1024)
       rc = launch_mfma<256, 256, 64>((const bf16_t*)A, (const bf16_t*)B,
                                      (bf16_t*)C, E, R, N, K, relu, st);
@@ -1461,9 +1508,13 @@ extern "C" int mesh_moe_expert_ffn_backward(
   hipStream_t st = (hipStream_t)stream;
   int rc;
   // dh = dy . wo^T  (wo in its variable layout [E, H, N] is K-contiguous here)
-  rc = grouped_gemm(dy, wo, dh, E, R, H, N, MESH_MOE_ACT_LINEAR, dtype, st);
+  // (the ReLU mask rides on the stores of this GEMM where its kernel can)
+  bool masked = false;
+  rc = grouped_gemm(dy, wo, dh, E, R, H, N, MESH_MOE_ACT_LINEAR, dtype, st,
+                    activation == MESH_MOE_ACT_RELU && !dh_scale ? h : nullptr,
+                    &masked);
   if (rc != 0) return rc;
-  if (activation == MESH_MOE_ACT_RELU || dh_scale) {
+  if (!masked && (activation == MESH_MOE_ACT_RELU || dh_scale)) {
     const int64_t n = (int64_t)E * R * H;
     const bool relu = activation == MESH_MOE_ACT_RELU;
     const int blocks = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
