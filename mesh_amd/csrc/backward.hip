@@ -210,6 +210,84 @@ __global__ __launch_bounds__(256) void dispatch_backward_kernel(
   }
 }
 
+// The same with the router's share for FOUR tokens per wavefront: a 16-byte
+// piece of a router kernel row, once loaded, serves all four (the one-token
+// kernel reads the whole router kernel, E * M elements, per token, which is
+// what bounds it).  The four tokens' d(logits) sit in LDS as [e][4], so one
+// broadcast read per expert feeds 4 x 8 multiply-adds.  Needs 16-byte rows,
+// E <= DBR_MAX_E and S % 4 == 0 (the four tokens share a group).
+constexpr int DBR_TOK = 4;
+constexpr int DBR_MAX_E = 128;
+
+template <typename T>
+__global__ __launch_bounds__(256) void dispatch_backward_router4_kernel(
+    const T* __restrict__ dxe, const int32_t* __restrict__ idx,
+    const int32_t* __restrict__ pos, const float* __restrict__ gate,
+    const uint8_t* __restrict__ kept, const float* __restrict__ dlogits,
+    const T* __restrict__ wgp, T* __restrict__ dx, int G, int S, int E, int C,
+    int M, int64_t T_tokens, int groups_per_router) {
+  constexpr int VN = Vec16B<T>::N;
+  __shared__ __attribute__((aligned(16))) float dls[4][DBR_MAX_E][DBR_TOK];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t t0 = ((int64_t)blockIdx.x * 4 + wave) * DBR_TOK;
+  if (t0 >= T_tokens) return;          // whole wavefronts leave: no barrier below
+  const int g = (int)(t0 / S);
+  wgp += (int64_t)(g / groups_per_router) * E * M;
+  const T* src[DBR_TOK][2];
+#pragma unroll
+  for (int j = 0; j < DBR_TOK; ++j) {
+    const int64_t t = t0 + j;
+#pragma unroll
+    for (int k = 0; k < 2; ++k) {
+      src[j][k] = nullptr;
+      if (t < T_tokens && kept[t * 2 + k] &&
+          round_to<T>(gate[t * 2 + k]) != 0.0f) {
+        const int64_t slot =
+            ((int64_t)idx[t * 2 + k] * G + g) * C + pos[t * 2 + k];
+        src[j][k] = dxe + slot * M;
+      }
+    }
+  }
+  // this wavefront's d(logits) -> LDS, transposed to [e][token]
+  for (int i = lane; i < E * DBR_TOK; i += 64) {
+    const int j = i / E, e = i - j * E;
+    dls[wave][e][j] = t0 + j < T_tokens ? dlogits[(t0 + j) * E + e] : 0.f;
+  }
+  // (same wavefront writes and reads: program order is enough within a wave)
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+  __builtin_amdgcn_wave_barrier();
+  for (int i = lane; i < M / VN; i += 64) {
+    float acc[DBR_TOK][VN];
+#pragma unroll
+    for (int j = 0; j < DBR_TOK; ++j) {
+#pragma unroll
+      for (int q = 0; q < VN; ++q) acc[j][q] = 0.f;
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        if (src[j][k] == nullptr) continue;
+        float v[VN];
+        unpack16(reinterpret_cast<const uint4*>(src[j][k])[i], v, T());
+#pragma unroll
+        for (int q = 0; q < VN; ++q) acc[j][q] += v[q];
+      }
+    }
+    for (int e = 0; e < E; ++e) {
+      float w[VN];
+      unpack16(reinterpret_cast<const uint4*>(wgp + (int64_t)e * M)[i], w, T());
+      const float4 d4 = *reinterpret_cast<const float4*>(&dls[wave][e][0]);
+      const float d[DBR_TOK] = {d4.x, d4.y, d4.z, d4.w};
+#pragma unroll
+      for (int j = 0; j < DBR_TOK; ++j)
+#pragma unroll
+        for (int q = 0; q < VN; ++q) acc[j][q] = fmaf(d[j], w[q], acc[j][q]);
+    }
+#pragma unroll
+    for (int j = 0; j < DBR_TOK; ++j)
+      if (t0 + j < T_tokens)
+        reinterpret_cast<uint4*>(dx + (t0 + j) * M)[i] = pack16(acc[j], T());
+  }
+}
+
 // ---------------------------------------------------------------------------
 // gating backward.
 // Step 1, one block per group: how many tokens count for density_1 of each
@@ -379,49 +457,111 @@ __global__ __launch_bounds__(256) void gating_backward_kernel(
 
 // ---------------------------------------------------------------------------
 // router projection backward w.r.t. the kernel: dw[m,e] = sum_t x[t,m] *
-// dlogits[t,e], float32.  Block (m tile of 64, chunk of tokens, chunk of 64
-// experts) accumulates 64 x 64 partial sums, thread (m = tid % 64, 16 experts),
-// and adds them to the float32 accumulator with atomics.
+// dlogits[t,e], float32.  Block (m tile of 256, chunk of tokens, chunk of 64
+// experts) accumulates 256 x 64 partial sums and adds them to the float32
+// accumulator with atomics.  Thread (m group = tid % 64, expert group =
+// tid / 64) owns a 4 x 16 patch: per staged token one 16-byte LDS read of x
+// and four (broadcast) of dlogits feed 64 multiply-adds.
 // ---------------------------------------------------------------------------
 constexpr int WG_TOK = 1024;  // tokens per block
 constexpr int WG_BATCH = 32;  // tokens staged in LDS at a time
+constexpr int WG_M = 256;     // kernel rows per block
 
 template <typename T>
 __global__ __launch_bounds__(256) void router_wgrad_kernel(
     const T* __restrict__ x, const float* __restrict__ dlogits,
-    float* __restrict__ acc_out, int64_t T_tokens, int M, int E) {
-  __shared__ float xs[WG_BATCH][64 + 1];
-  __shared__ float ds[WG_BATCH][64];
-  const int m0 = blockIdx.x * 64, e0 = blockIdx.z * 64;
+    float* __restrict__ acc_out, int64_t T_tokens, int M, int E, bool vec) {
+  __shared__ __attribute__((aligned(16))) float xs[WG_BATCH][WG_M];
+  __shared__ __attribute__((aligned(16))) float ds[WG_BATCH][64];
+  const int m0 = blockIdx.x * WG_M, e0 = blockIdx.z * 64;
   const int64_t t0 = (int64_t)blockIdx.y * WG_TOK;
   const int64_t t1 = t0 + WG_TOK < T_tokens ? t0 + WG_TOK : T_tokens;
   const int tid = threadIdx.x;
-  const int ml = tid & 63, eg = tid >> 6;  // experts e0 + eg*16 .. +15
-  float acc[16];
+  const int mg = tid & 63, eg = tid >> 6;  // rows m0 + 4 mg .., experts e0 + 16 eg ..
+  float acc[4][16];
 #pragma unroll
-  for (int j = 0; j < 16; ++j) acc[j] = 0.f;
+  for (int i = 0; i < 4; ++i)
+#pragma unroll
+    for (int j = 0; j < 16; ++j) acc[i][j] = 0.f;
   for (int64_t tb = t0; tb < t1; tb += WG_BATCH) {
-    for (int i = tid; i < WG_BATCH * 64; i += 256) {
-      const int r = i >> 6, c = i & 63;
-      const int64_t t = tb + r;
-      const bool ok = t < t1;
-      xs[r][c] = (ok && m0 + c < M) ? load_f32<T>(x + t * M + m0 + c) : 0.f;
-      ds[r][c] = (ok && e0 + c < E) ? dlogits[t * E + e0 + c] : 0.f;
+    if (vec) {
+      // 16-byte pieces, all of a thread's loads in flight before the first
+      // LDS write
+      constexpr int VN = Vec16B<T>::N;
+      constexpr int XP = WG_BATCH * WG_M / VN / 256;   // pieces of x per thread
+      uint4 xv[XP];
+      float4 dv[2];
+#pragma unroll
+      for (int u = 0; u < XP; ++u) {
+        const int i = tid + u * 256;
+        const int r = i / (WG_M / VN), c = (i % (WG_M / VN)) * VN;
+        const int64_t t = tb + r;
+        xv[u] = (t < t1 && m0 + c < M)
+                    ? *reinterpret_cast<const uint4*>(x + t * M + m0 + c)
+                    : make_uint4(0, 0, 0, 0);
+      }
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int i = tid + u * 256;
+        const int r = i >> 4, c = (i & 15) * 4;
+        const int64_t t = tb + r;
+        dv[u] = (t < t1 && e0 + c < E)
+                    ? *reinterpret_cast<const float4*>(dlogits + t * E + e0 + c)
+                    : make_float4(0.f, 0.f, 0.f, 0.f);
+      }
+#pragma unroll
+      for (int u = 0; u < XP; ++u) {
+        const int i = tid + u * 256;
+        const int r = i / (WG_M / VN), c = (i % (WG_M / VN)) * VN;
+        float f[VN];
+        unpack16(xv[u], f, T());
+#pragma unroll
+        for (int q = 0; q < VN; ++q) xs[r][c + q] = f[q];
+      }
+#pragma unroll
+      for (int u = 0; u < 2; ++u) {
+        const int i = tid + u * 256;
+        *reinterpret_cast<float4*>(&ds[i >> 4][(i & 15) * 4]) = dv[u];
+      }
+    } else {
+      for (int i = tid; i < WG_BATCH * WG_M; i += 256) {
+        const int r = i / WG_M, c = i % WG_M;
+        const int64_t t = tb + r;
+        xs[r][c] = (t < t1 && m0 + c < M) ? load_f32<T>(x + t * M + m0 + c) : 0.f;
+      }
+      for (int i = tid; i < WG_BATCH * 64; i += 256) {
+        const int r = i >> 6, c = i & 63;
+        const int64_t t = tb + r;
+        ds[r][c] = (t < t1 && e0 + c < E) ? dlogits[t * E + e0 + c] : 0.f;
+      }
     }
     __syncthreads();
-#pragma unroll 4
+#pragma unroll 2
     for (int r = 0; r < WG_BATCH; ++r) {
-      const float xv = xs[r][ml];
+      const float4 xv = *reinterpret_cast<const float4*>(&xs[r][mg * 4]);
+      const float xa[4] = {xv.x, xv.y, xv.z, xv.w};
 #pragma unroll
-      for (int j = 0; j < 16; ++j) acc[j] += xv * ds[r][eg * 16 + j];
+      for (int q = 0; q < 4; ++q) {
+        const float4 dv = *reinterpret_cast<const float4*>(&ds[r][eg * 16 + q * 4]);
+        const float da[4] = {dv.x, dv.y, dv.z, dv.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+          for (int j = 0; j < 4; ++j)
+            acc[i][q * 4 + j] = fmaf(xa[i], da[j], acc[i][q * 4 + j]);
+      }
     }
     __syncthreads();
   }
-  if (m0 + ml < M) {
 #pragma unroll
-    for (int j = 0; j < 16; ++j) {
-      const int e = e0 + eg * 16 + j;
-      if (e < E) atomicAdd(acc_out + (int64_t)(m0 + ml) * E + e, acc[j]);
+  for (int i = 0; i < 4; ++i) {
+    const int m = m0 + mg * 4 + i;
+    if (m < M) {
+#pragma unroll
+      for (int j = 0; j < 16; ++j) {
+        const int e = e0 + eg * 16 + j;
+        if (e < E) atomicAdd(acc_out + (int64_t)m * E + e, acc[i][j]);
+      }
     }
   }
 }
@@ -507,6 +647,21 @@ extern "C" int mesh_moe_dispatch_backward(
                    bw_aligned16(dexpert_in) && bw_aligned16(dx) &&
                    (w_gate_packed == nullptr || bw_aligned16(w_gate_packed));
   hipStream_t st = (hipStream_t)stream;
+  if (vec && dlogits != nullptr && E <= DBR_MAX_E && S % DBR_TOK == 0) {
+    const int64_t nb4 = (T_tokens + 4 * DBR_TOK - 1) / (4 * DBR_TOK);
+    if (dtype == MESH_MOE_F32)
+      dispatch_backward_router4_kernel<float><<<(unsigned)nb4, 256, 0, st>>>(
+          (const float*)dexpert_in, idx, pos, gate, kept, dlogits,
+          (const float*)w_gate_packed, (float*)dx, G, S, E, C, M, T_tokens,
+          groups_per_router);
+    else
+      dispatch_backward_router4_kernel<bf16_t><<<(unsigned)nb4, 256, 0, st>>>(
+          (const bf16_t*)dexpert_in, idx, pos, gate, kept, dlogits,
+          (const bf16_t*)w_gate_packed, (bf16_t*)dx, G, S, E, C, M, T_tokens,
+          groups_per_router);
+    MOE_CHECK_LAUNCH("dispatch_backward (router share, 4 tokens per wavefront)");
+    return 0;
+  }
   if (dtype == MESH_MOE_F32)
     dispatch_backward_kernel<float><<<(unsigned)nblocks, 256, 0, st>>>(
         (const float*)dexpert_in, idx, pos, gate, kept, dlogits,
@@ -606,16 +761,20 @@ extern "C" int mesh_moe_router_backward_weights(const void* x,
   const unsigned fb = (unsigned)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
   fill_f32_kernel<<<fb, 256, 0, st>>>(workspace, n, 0.0f);
   MOE_CHECK_LAUNCH("router_backward_weights (clear)");
-  dim3 grid((unsigned)((M + 63) / 64), (unsigned)chunks,
+  dim3 grid((unsigned)((M + WG_M - 1) / WG_M), (unsigned)chunks,
             (unsigned)((E + 63) / 64));
+  // 16-byte loads: rows of x and of dlogits start 16-byte aligned and hold
+  // whole pieces
+  const bool vec = ((size_t)M * dtype_size(dtype)) % 16 == 0 && E % 4 == 0 &&
+                   bw_aligned16(x) && bw_aligned16(dlogits);
   if (dtype == MESH_MOE_F32) {
     router_wgrad_kernel<float><<<grid, 256, 0, st>>>(
-        (const float*)x, dlogits, workspace, tokens, M, E);
+        (const float*)x, dlogits, workspace, tokens, M, E, vec);
     MOE_CHECK_LAUNCH("router_backward_weights");
     convert_f32_kernel<float><<<fb, 256, 0, st>>>(workspace, (float*)dw_gate, n);
   } else {
     router_wgrad_kernel<bf16_t><<<grid, 256, 0, st>>>(
-        (const bf16_t*)x, dlogits, workspace, tokens, M, E);
+        (const bf16_t*)x, dlogits, workspace, tokens, M, E, vec);
     MOE_CHECK_LAUNCH("router_backward_weights");
     convert_f32_kernel<bf16_t><<<fb, 256, 0, st>>>(workspace, (bf16_t*)dw_gate,
                                                   n);
