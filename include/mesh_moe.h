@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 10
+#define MESH_MOE_ABI_VERSION 11
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -414,7 +414,9 @@ size_t mesh_moe_expert_ffn_backward_workspace_bytes(int E, int R, int M, int H,
  *   dh_scale [E,R,H] dtype or NULL: the dropout noise mesh_moe_hidden_product
  *   wrote (transformer/moe.py:477-479)
  *   dexpert_in [E,R,M]; dwi [E,M,H]; dwo [E,H,N]; everything of `dtype`
- * Four grouped GEMMs on the forward kernels plus four transposes.
+ * Four grouped GEMMs on the forward kernels; the weight gradients read both
+ * operands as they are (reduction index outermost) where the kernel takes the
+ * shape (bf16, R a multiple of 64), through transposed copies otherwise.
  */
 int mesh_moe_expert_ffn_backward(const void* expert_in, const void* h,
                                  const void* dy, const void* wi,
@@ -438,9 +440,9 @@ size_t mesh_moe_gating_backward_workspace_bytes(int G, int E);
  *   mesh_moe_combine_backward
  *   d_loss [1] float32 ON THE DEVICE: gradient w.r.t. the returned loss
  *   (balancing loss * moe_loss_coef); loss_scale = moe_loss_coef
- *   use_z_loss / z_loss_coef / num_microbatches as in the forward call
+ *   use_second_place_loss (router 0 only, moe.py:1425-1438) / use_z_loss /
+ *   z_loss_coef / num_microbatches as in the forward call
  *   dlogits [G,S,E] float32
- * The second-place loss (moe_use_second_place_loss) is not covered.
  */
 int mesh_moe_gating_backward(const float* logits, const void* importance,
                              int importance_dtype,
@@ -448,6 +450,7 @@ int mesh_moe_gating_backward(const float* logits, const void* importance,
                              const uint8_t* kept, const float* dgate,
                              const float* d_loss, double loss_scale, int G,
                              int S, int E, int router, int top_k,
+                             int use_second_place_loss,
                              int use_z_loss, double z_loss_coef,
                              int num_microbatches,
                              float* dlogits, void* workspace,

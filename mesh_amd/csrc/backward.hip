@@ -298,6 +298,7 @@ struct GateBackwardParams {
   int G, S, E;
   int router;           // 0 = top-2, 1 = switch / switch_max, 2 = ntlb
   int top_k;            // ntlb: candidates per token
+  int use_second_place_loss;  // top-2: the loss has the density_2 term too
   int has_importance;
   int importance_from_slot_gate;  // importance = 0.5*((w>0.5)+(w>0))
   int num_microbatches;
@@ -313,17 +314,19 @@ __global__ __launch_bounds__(256) void gate_count_kernel(
     GateBackwardParams p, const float* __restrict__ logits,
     const int32_t* __restrict__ idx, const IT* __restrict__ importance,
     int32_t* __restrict__ counts, float* __restrict__ n_one) {
-  extern __shared__ int32_t cnt[];  // [E] + 1
+  extern __shared__ int32_t cnt[];  // [E] + 1 + [E]
+  int32_t* cnt2 = cnt + p.E + 1;    // second choices (second-place loss)
   const int g = blockIdx.x;
-  for (int e = threadIdx.x; e <= p.E; e += blockDim.x) cnt[e] = 0;
+  for (int e = threadIdx.x; e <= 2 * p.E; e += blockDim.x) cnt[e] = 0;
   __syncthreads();
   for (int s = threadIdx.x; s < p.S; s += blockDim.x) {
     const int64_t t = (int64_t)g * p.S + s;
-    bool one = true;
+    bool one = true, positive = true;
     if (importance != nullptr) {
       const float imp = load_f32<IT>(importance + t);
       // from a slot weight w: 0.5*((w>0.5)+(w>0)) == 1  <=>  w > 0.5
       one = p.importance_from_slot_gate ? imp > 0.5f : imp == 1.0f;
+      positive = imp > 0.0f;    // either form: 0.5*((w>0.5)+(w>0)) > 0 <=> w > 0
     }
     if (one) atomicAdd(&cnt[p.E], 1);
     if (p.router == 2) {
@@ -359,10 +362,16 @@ __global__ __launch_bounds__(256) void gate_count_kernel(
     // top-2: density_1 counts mask_1 after the importance mask
     // (moe.py:1402-1420); switch: every token's arg-max (moe.py:1224)
     if (one || p.router == 1) atomicAdd(&cnt[idx[t * 2]], 1);
+    // density_2 counts mask_2 = one_hot(index_2) * (importance > 0), before
+    // the second-choice policy and the capacity (moe.py:1409-1411, :1429)
+    if (p.use_second_place_loss && positive)
+      atomicAdd(&cnt2[idx[t * 2 + 1]], 1);
   }
   __syncthreads();
-  for (int e = threadIdx.x; e < p.E; e += blockDim.x)
+  for (int e = threadIdx.x; e < p.E; e += blockDim.x) {
     counts[(int64_t)g * p.E + e] = cnt[e];
+    counts[((int64_t)p.G + g) * p.E + e] = cnt2[e];
+  }
   if (threadIdx.x == 0) n_one[g] = (float)cnt[p.E];
 }
 
@@ -429,15 +438,35 @@ __global__ __launch_bounds__(256) void gating_backward_kernel(
       coef = dl * mb * ee * (float)(1.0 / terms) * inv_s * inv_s;
   }
   const int32_t* cg = counts + (int64_t)g * E;
-  // inner = sum_e p[e] * dp[e]
-  float inner = 0.f;
-  for (int e = 0; e < E; ++e) {
-    const float pe = expf(row[e] + neglse);
+  // Second-place loss (moe.py:1426-1438): 0.5 * E^2 * mean_{g,e}(mean_s(n) *
+  // density_2) with n = q / (sum(q) + 1e-9), q = p * (1 - mask_1):
+  // d/dq[e] = c2[e] * rq - (sum_f c2[f] q[f]) * rq^2, c2 = coef2 * count_2.
+  const int32_t* cg2 = counts + ((int64_t)p.G + g) * E;
+  const bool loss2 = p.router == 0 && p.use_second_place_loss;
+  float coef2 = 0.f, rq = 0.f, aq = 0.f;
+  if (loss2) {
+    coef2 = dl * mb * 0.5f * ee * (float)(1.0 / ((double)p.G * (double)E)) *
+            inv_s * inv_s;
+    float q = 0.f, a = 0.f;
+    for (int e = 0; e < E; ++e) {
+      const float qe = expf(row[e] + neglse) * (e == i1 ? 1.0f - m1 : 1.0f);
+      q += qe;
+      a += coef2 * (float)cg2[e] * qe;
+    }
+    rq = 1.0f / (q + 1e-9f);
+    aq = a * rq * rq;
+  }
+  auto dprob = [&](int e) {
     float dp = coef * (float)cg[e];
     if (e == i1) dp += add1;
     if (p.router == 0 && e == i2) dp += add2;
-    inner += pe * dp;
-  }
+    if (loss2)
+      dp += (e == i1 ? 1.0f - m1 : 1.0f) * (coef2 * (float)cg2[e] * rq - aq);
+    return dp;
+  };
+  // inner = sum_e p[e] * dp[e]
+  float inner = 0.f;
+  for (int e = 0; e < E; ++e) inner += expf(row[e] + neglse) * dprob(e);
   float zfac = 0.f;
   if (p.use_z_loss) {  // d/dx of z_coef * sum(lse^2 * m1) / (n * microbatches)
     float n = 0.f;
@@ -448,10 +477,7 @@ __global__ __launch_bounds__(256) void gating_backward_kernel(
   }
   for (int e = 0; e < E; ++e) {
     const float pe = expf(row[e] + neglse);
-    float dp = coef * (float)cg[e];
-    if (e == i1) dp += add1;
-    if (p.router == 0 && e == i2) dp += add2;
-    out[e] = pe * (dp - inner) + zfac * pe;
+    out[e] = pe * (dprob(e) - inner) + zfac * pe;
   }
 }
 
@@ -678,14 +704,15 @@ extern "C" int mesh_moe_dispatch_backward(
 
 extern "C" size_t mesh_moe_gating_backward_workspace_bytes(int G, int E) {
   if (G < 1 || E < 1) return 0;
-  return sizeof(int32_t) * (size_t)G * E + sizeof(float) * (size_t)G + 256;
+  // counts of first and of second choices [2][G][E], tokens of importance 1 [G]
+  return sizeof(int32_t) * 2 * (size_t)G * E + sizeof(float) * (size_t)G + 256;
 }
 
 extern "C" int mesh_moe_gating_backward(
     const float* logits, const void* importance, int importance_dtype,
     int importance_from_slot_gate, const int32_t* idx, const uint8_t* kept,
     const float* dgate, const float* d_loss, double loss_scale, int G, int S,
-    int E, int router, int top_k,
+    int E, int router, int top_k, int use_second_place_loss,
     int use_z_loss, double z_loss_coef, int num_microbatches, float* dlogits,
     void* workspace, size_t workspace_bytes, void* stream) {
   MOE_REQUIRE(logits && idx && kept && dgate && d_loss && dlogits && workspace,
@@ -706,6 +733,7 @@ extern "C" int mesh_moe_gating_backward(
   p.G = G; p.S = S; p.E = E;
   p.router = router;
   p.top_k = top_k;
+  p.use_second_place_loss = (use_second_place_loss && router == 0) ? 1 : 0;
   p.has_importance = importance != nullptr;
   p.importance_from_slot_gate = importance_from_slot_gate ? 1 : 0;
   p.num_microbatches = num_microbatches;
@@ -714,9 +742,9 @@ extern "C" int mesh_moe_gating_backward(
   p.loss_scale = (float)loss_scale;
   uintptr_t wsp = ((uintptr_t)workspace + 255) & ~(uintptr_t)255;
   int32_t* counts = (int32_t*)wsp;
-  float* n_one = (float*)(counts + (size_t)G * E);
+  float* n_one = (float*)(counts + 2 * (size_t)G * E);
   hipStream_t st = (hipStream_t)stream;
-  const size_t smem = sizeof(int32_t) * ((size_t)E + 1);
+  const size_t smem = sizeof(int32_t) * (2 * (size_t)E + 1);
   const int64_t T_tokens = (int64_t)G * S;
   const unsigned blocks = (unsigned)((T_tokens + 255) / 256);
   if (importance && importance_dtype == MESH_MOE_BF16) {

@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -101,8 +101,8 @@ _SIGNATURES = {
         _vp, _vp, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, _vp,
         ctypes.c_double,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
-        ctypes.c_int, ctypes.c_double, ctypes.c_int, _vp, _vp, ctypes.c_size_t,
-        _vp]),
+        ctypes.c_int, ctypes.c_int, ctypes.c_double, ctypes.c_int, _vp, _vp,
+        ctypes.c_size_t, _vp]),
     "mesh_moe_router_backward_weights": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, _vp]),
@@ -725,7 +725,8 @@ def expert_ffn_backward(expert_in, h, dy, wi, wo, activation="relu",
 
 def gating_backward(logits, r, dgate, d_loss, loss_scale, router="top_2",
                     importance=None, z_loss=None, num_microbatches=None,
-                    importance_from_slot_gate=False, top_k=0):
+                    importance_from_slot_gate=False, top_k=0,
+                    use_second_place_loss=False):
   """d(logits) [G, S, E] float32.  d_loss: float32 tensor of one element on the
   device (gradient w.r.t. the layer's returned loss); loss_scale:
   moe_loss_coef.  router: "top_2", "switch" (also switch_max) or "ntlb" (then
@@ -749,7 +750,7 @@ def gating_backward(logits, r, dgate, d_loss, loss_scale, router="top_2",
         _dev(dgate, "dgate", torch.float32, (g, s, 2)),
         _dev(d_loss, "d_loss", torch.float32), float(loss_scale), g, s, e,
         {"top_2": 0, "switch": 1, "switch_max": 1, "ntlb": 2}[router],
-        int(top_k),
+        int(top_k), int(bool(use_second_place_loss)),
         int(z_loss is not None),
         float(z_loss or 0.0), int(num_microbatches or 1), dlogits.data_ptr(),
         ws.data_ptr(), ws_bytes, _stream()), "gating_backward")

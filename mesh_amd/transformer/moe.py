@@ -407,9 +407,6 @@ class MoEV1Operation(mtf.Operation):
     if self._gating.router == "expert_selection":
       raise NotImplementedError(
           "backward of expert_selection gating is not implemented")
-    if self._gating.use_second_place_loss:
-      raise NotImplementedError(
-          "backward of the second-place loss is not implemented")
     if self._more_wi:
       raise NotImplementedError(
           "backward of a product of several dense layers (gated expert "
@@ -561,7 +558,8 @@ class MoEV1GradOperation(mtf.Operation):
           sv["logits"], r, dgate, dloss_s.reshape(1).float(), 1.0,
           router=gating.router, top_k=getattr(gating, "top_k", 0),
           importance=sv["importance"], z_loss=gating.z_loss,
-          num_microbatches=gating.num_microbatches)
+          num_microbatches=gating.num_microbatches,
+          use_second_place_loss=gating.use_second_place_loss)
       tokens = groups * s_
       if sv["gate_in"] is None:
         dwg = moe_hip.router_backward_weights(
@@ -746,9 +744,6 @@ class MoEV2Operation(mtf.Operation):
   def gradient(self, grad_ys):
     """Gradients w.r.t. (inputs, outer / inner gate kernels, wi, wo
     [, importance]) from those of (outputs, loss)."""
-    if self._gating.use_second_place_loss:
-      raise NotImplementedError(
-          "backward of the second-place loss is not implemented")
     self._save_for_backward = True
     d_out, d_loss = grad_ys
     if d_out is None:
@@ -872,7 +867,8 @@ class MoEV2GradOperation(mtf.Operation):
           sv["logits_y"], ry, dgate_y, dl, 1.0, router="top_2",
           importance=sv["slot_gate"].reshape(x_e * h0, t_),
           num_microbatches=gating.num_microbatches,
-          importance_from_slot_gate=True)
+          importance_from_slot_gate=True,
+          use_second_place_loss=gating.use_second_place_loss)
       inputs_y = sv["inputs_y"]                           # [x, h0*t, m]
       dl_y = dlogits_y.reshape(x_e, h0 * t_, y_e)
       dw_inner = torch.stack([
@@ -884,7 +880,8 @@ class MoEV2GradOperation(mtf.Operation):
       dlogits_x = moe_hip.gating_backward(
           sv["logits_x"], rx, dgate_x, dl, 1.0, router="top_2",
           importance=sv["importance"],
-          num_microbatches=gating.num_microbatches)
+          num_microbatches=gating.num_microbatches,
+          use_second_place_loss=gating.use_second_place_loss)
       dw_outer = moe_hip.router_backward_weights(
           sv["x"].reshape(ag * s_, m_), dlogits_x.reshape(ag * s_, x_e))
       dx = moe_hip.dispatch_backward(

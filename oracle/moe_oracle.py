@@ -56,7 +56,9 @@ MoE file, and its TensorFlow dependency cannot run here):
                                       dropout by central differences
   gating_backward,                    central differences of an independent
   moe_layer_v1_backward               float64 forward with the routing held
-                                      fixed (tests/test_oracle.py)
+                                      fixed (tests/test_oracle.py), every
+                                      router, the second-place loss, the
+                                      noise policies and the hidden dropout
   v2                                  x=1 outer expert reduces to v1
 
 PARITY UNPINNED against TensorFlow itself (only running the reference could
@@ -1068,7 +1070,8 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
 # backward of transformer_moe_layer_v1
 # ----------------------------------------------------------------------------
 def gating_backward(logits, r, gating, d_gate_1, d_gate_2, d_loss,
-                    importance=None, num_microbatches=None, z_loss=None):
+                    importance=None, num_microbatches=None, z_loss=None,
+                    use_second_place_loss=False):
   """d(logits) of _top_2_gating / _switch_gating / _switch_max_gating /
   _ntlb_gating.
 
@@ -1114,6 +1117,20 @@ def gating_backward(logits, r, gating, d_gate_1, d_gate_2, d_loss,
     density = seq_sum(one_hot(i1, e_) * m1[..., None], axis=-2) * inv_s
     coef = d_loss * mb * ee * F32(1.0 / (g_ * e_))
     dp += (coef * density * inv_s)[:, None, :] * m1[..., None]
+    if use_second_place_loss:
+      # loss_2 * 0.5 = 0.5 E^2 mean_{g,e}(mean_s(n) * density_2), n = q /
+      # (sum_e q + 1e-9), q = p * (1 - mask_1) (moe.py:1405, :1426-1438);
+      # density_2 counts mask_2 before the second-choice policy and has no
+      # gradient
+      keep = one[..., None] - one_hot(i1, e_) * m1[..., None]
+      q = p * keep
+      m2 = one if importance is None else (
+          np.asarray(importance, F32) > F32(0.0)).astype(F32)
+      density_2 = seq_sum(one_hot(i2, e_) * m2[..., None], axis=-2) * inv_s
+      a = (coef * F32(0.5) * density_2 * inv_s)[:, None, :]     # d/dn [G,1,E]
+      rq = F32(1.0) / (q.sum(-1, keepdims=True) + F32(1e-9))
+      dq = a * rq - (a * q).sum(-1, keepdims=True) * rq * rq
+      dp += dq * keep
     return (p * (dp - (p * dp).sum(-1, keepdims=True))).astype(F32)
   if gating not in ("switch", "switch_max", "ntlb"):
     raise ValueError("unknown gating %r" % (gating,))
@@ -1215,12 +1232,9 @@ def moe_layer_v1_backward(x, w_gate, wi, wo, hp, train, act_dtype, d_out,
   gradients are tensors of the activation dtype (cast gradients cast back,
   ops.py:1945-1962), float32 inside the gating.  The dispatch tensor is a
   bool cast of the combine tensor and carries no gradient (moe.py:1510-1511).
-  The second-place loss is not covered.
 
   Returns dict(dx, dw_gate, dwi, dwo) holding activation-dtype values.
   """
-  if hp.moe_use_second_place_loss:
-    raise NotImplementedError("backward of the second-place loss")
   if isinstance(wi, (list, tuple)) or isinstance(activation, (list, tuple)):
     raise NotImplementedError("backward of a product of dense layers")
   if activation not in ("relu", "linear", None):
@@ -1265,7 +1279,7 @@ def moe_layer_v1_backward(x, w_gate, wi, wo, hp, train, act_dtype, d_out,
               * cast_act(F32(hp.moe_loss_coef), act_dtype))
   dlogits = gating_backward(aux["logits"], aux, hp.moe_gating, dgate[..., 0],
                             dgate[..., 1], d_aux, importance, num_microbatches,
-                            z)
+                            z, hp.moe_use_second_place_loss)
   # the router saw the perturbed inputs x * mult (perturb_gate_inputs); the
   # multiplier is a constant of the graph
   mult = aux.get("gate_mult")
@@ -1398,8 +1412,6 @@ def moe_layer_v2_backward(x, w_outer, w_inner, wi, wo, hp, train, act_dtype,
   kernels: the v1 pieces applied twice, inner level first.  The importance of
   the inner level is a comparison of the slot weights (moe.py:725-727) and
   carries no gradient.  Returns dict(dx, dw_outer, dw_inner, dwi, dwo)."""
-  if hp.moe_use_second_place_loss:
-    raise NotImplementedError("backward of the second-place loss")
   _, _, aux = moe_layer_v2(x, w_outer, w_inner, wi, wo, hp, train, act_dtype,
                            nonpadding=nonpadding,
                            num_microbatches=num_microbatches, dense=False)
@@ -1433,7 +1445,8 @@ def moe_layer_v2_backward(x, w_outer, w_inner, wi, wo, hp, train, act_dtype,
   imp_in = aux["importance_inner"].reshape(x_e * h0, t_)
   dlogits_y = gating_backward(aux["logits_inner"], ry, "top_2",
                               dgate_y[..., 0], dgate_y[..., 1], d_aux, imp_in,
-                              num_microbatches)
+                              num_microbatches,
+                              use_second_place_loss=hp.moe_use_second_place_loss)
   inputs_y = aux["expert_in_x"].reshape(x_e, h0 * t_, m_)
   dl_y = dlogits_y.reshape(x_e, h0 * t_, y_e)
   dw_inner = np.matmul(inputs_y.transpose(0, 2, 1).astype(F32), dl_y)
@@ -1444,7 +1457,8 @@ def moe_layer_v2_backward(x, w_outer, w_inner, wi, wo, hp, train, act_dtype,
   # outer gating, router and dispatch
   dlogits_x = gating_backward(aux["logits_outer"], rx, "top_2",
                               dgate_x[..., 0], dgate_x[..., 1], d_aux,
-                              aux["importance_outer"], num_microbatches)
+                              aux["importance_outer"], num_microbatches,
+                              use_second_place_loss=hp.moe_use_second_place_loss)
   dw_outer = np.matmul(xg.reshape(-1, m_).T.astype(F32),
                        dlogits_x.reshape(-1, x_e))
   dx = dispatch_backward(d_ein, rx, act_dtype) + np.matmul(

@@ -389,12 +389,18 @@ def test_gradients_builds_the_backward_operation():
   fwd = [o for o in graph.operations if isinstance(o, moe.MoEV1Operation)][0]
   assert fwd._save_for_backward
   assert any(isinstance(o, moe.MoEV1GradOperation) for o in graph.operations)
-  with pytest.raises(NotImplementedError, match="second-place loss"):
+  with pytest.raises(NotImplementedError, match="pre-activation"):
     g2, _, x2, d2 = graph_input()
     y2, l2 = moe.transformer_moe_layer_v1(
-        x2, d2[-1], hparams(moe_use_second_place_loss=True), True,
-        mtf.VariableDType(torch.float32))
+        x2, d2[-1], hparams(), True, mtf.VariableDType(torch.float32),
+        activation="gelu")
     mtf.gradients([y2], [x2])
+  # the second-place loss has a gradient like the rest of the gating
+  g2, _, x2, d2 = graph_input()
+  y2, l2 = moe.transformer_moe_layer_v1(
+      x2, d2[-1], hparams(moe_use_second_place_loss=True), True,
+      mtf.VariableDType(torch.float32))
+  assert mtf.gradients([y2, l2], [x2])[0].shape == x2.shape
   g3, _, x3, d3 = graph_input()
   y3, l3 = moe.transformer_moe_layer_v2(
       x3, d3[-1], hparams(moe_num_experts=[2, 2]), True,

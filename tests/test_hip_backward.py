@@ -126,3 +126,39 @@ def test_backward_matches_oracle(hip, case):
     atol = tol["atol"] * max(1.0, np.abs(ref).max())
     np.testing.assert_allclose(got[k], ref, rtol=tol["rtol"], atol=atol,
                                err_msg=k)
+
+
+@pytest.mark.parametrize("use_importance", [False, True])
+def test_gating_backward_second_place_loss(hip, use_importance):
+  """d(logits) of the balancing loss alone (zero gate gradients), with the
+  second-place term: against the oracle, and the term is not negligible."""
+  g, s, e, c = 3, 96, 8, 16
+  rng = np.random.default_rng(91)
+  logits = H.safe_logits(rng, g, s, e, scale=1.5)
+  imp = None
+  if use_importance:
+    imp = rng.choice([0.0, 0.5, 1.0], size=(g, s), p=[0.2, 0.2, 0.6]).astype(np.float32)
+  r_o = O.top_2_gating(logits, c, importance=imp, policy="threshold",
+                       threshold=0.3, use_second_place_loss=True,
+                       num_microbatches=2)
+  zeros = np.zeros((g, s), np.float32)
+  want = O.gating_backward(logits, r_o, "top_2", zeros, zeros, 0.7, imp, 2,
+                           use_second_place_loss=True)
+  without = O.gating_backward(logits, r_o, "top_2", zeros, zeros, 0.7, imp, 2)
+  assert np.abs(want - without).max() > 0.2 * np.abs(want).max()
+  lg = torch.from_numpy(logits).cuda()
+  ig = None if imp is None else torch.from_numpy(imp).cuda()
+  r = hip.top2_gating(lg, c, importance=ig, policy="threshold", threshold=0.3,
+                      use_second_place_loss=True, num_microbatches=2)
+  np.testing.assert_allclose(float(r.loss), r_o["loss"], rtol=1e-5)
+  dgate = torch.zeros((g, s, 2), dtype=torch.float32, device="cuda")
+  dl = torch.tensor([0.7], dtype=torch.float32, device="cuda")
+  got = hip.gating_backward(lg, r, dgate, dl, 1.0, router="top_2",
+                            importance=ig, num_microbatches=2,
+                            use_second_place_loss=True)
+  np.testing.assert_allclose(H.to_np(got), want, rtol=1e-3,
+                             atol=1e-5 * np.abs(want).max())
+  got0 = hip.gating_backward(lg, r, dgate, dl, 1.0, router="top_2",
+                             importance=ig, num_microbatches=2)
+  np.testing.assert_allclose(H.to_np(got0), without, rtol=1e-3,
+                             atol=1e-5 * np.abs(without).max())

@@ -522,7 +522,9 @@ def test_v1_switch_max_matches_oracle():
     ("ntlb+input_jitter", "float32", 108),
     ("top_2+hidden_dropout", "float32", 109),
     ("top_2+hidden_dropout", "bfloat16", 110),
-    ("switch+hidden_dropout", "float32", 111)],
+    ("switch+hidden_dropout", "float32", 111),
+    ("top_2+second_place_loss", "float32", 112),
+    ("top_2+second_place_loss", "bfloat16", 113)],
     ids=lambda c: "%s-%s" % (c[0], c[1]))
 def test_v1_gradients_match_oracle(case):
   """mtf.gradients over the layer (outputs and loss) against the oracle's
@@ -530,7 +532,8 @@ def test_v1_gradients_match_oracle(case):
   gating, act_dtype, seed = case
   gating, _, noise_policy = gating.partition("+")
   hidden_dropout = noise_policy == "hidden_dropout"
-  if hidden_dropout:
+  loss2 = noise_policy == "second_place_loss"
+  if hidden_dropout or loss2:
     noise_policy = ""
   b, l, m, hdim, e, group = 2, 64, 32, 48, 4, 32
   rng = np.random.default_rng(seed)
@@ -551,6 +554,9 @@ def test_v1_gradients_match_oracle(case):
               moe_switch_dropout=0.3)
   if hidden_dropout:
     kw.update(moe_dropout_rate=0.25)
+  if loss2:
+    kw.update(moe_use_second_place_loss=True, moe_second_policy_train="threshold",
+              moe_second_threshold_train=0.3)
   hp, ohp = make_hparams(**kw)
   dt = H.ACT_TORCH[act_dtype]
   graph = mtf.Graph()
@@ -720,15 +726,18 @@ def test_v1_experts_attention(act_dtype):
     mtf.gradients([outs[0]], [xt])
 
 
-@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
-def test_v2_gradients_match_oracle(act_dtype):
+@pytest.mark.parametrize("case", [("float32", False), ("bfloat16", False),
+                                  ("float32", True)],
+                         ids=["float32", "bfloat16", "float32-second_place_loss"])
+def test_v2_gradients_match_oracle(case):
   """mtf.gradients over the hierarchical layer against the oracle's backward
   (pinned by central differences in tests/test_oracle.py)."""
+  act_dtype, loss2 = case
   b, l, m, hdim, xe, ye, group = 2, 64, 32, 48, 2, 4, 32
   hp, ohp = make_hparams(moe_num_experts=[xe, ye], moe_hidden_size=hdim,
                          moe_group_size=group, moe_capacity_factor_train=1.25,
                          moe_capacity_factor_second_level=1.0,
-                         moe_loss_coef=0.25)
+                         moe_loss_coef=0.25, moe_use_second_place_loss=loss2)
   for seed in range(601, 621):   # first seed without an inner-level near-tie
     rng = np.random.default_rng(seed)
     w = v2_weights(rng, m, hdim, xe, ye)

@@ -1014,7 +1014,7 @@ def test_hidden_dropout_noise(act_dtype):
 
 # ---- backward -------------------------------------------------------------------
 def _f64_layer(x, wg, wi, wo, aux, gating, m1, coef, mb, z_loss, mult=None,
-               hidden_noise=None):
+               hidden_noise=None, density_2=None):
   """Independent float64 forward of the v1 layer with the ROUTING HELD FIXED
   (experts, kept masks and density counts taken from `aux`): a smooth function
   of (x, wg, wi, wo) whose central differences pin the oracle's backward."""
@@ -1041,7 +1041,12 @@ def _f64_layer(x, wg, wi, wo, aux, gating, m1, coef, mb, z_loss, mult=None,
            + (g2 / den * k2)[..., None] * ffn(i2, aux["pos_2"]))
     density = (onehot1 * m1[..., None]).mean(1)
     proxy = (p * m1[..., None]).mean(1)
-    aux_loss = (proxy * density).mean() * e * e / mb
+    aux_loss = (proxy * density).mean() * e * e
+    if density_2 is not None:     # the second-place term, its density held fixed
+      q = p * (1.0 - onehot1 * m1[..., None])
+      proxy_2 = (q / (q.sum(-1, keepdims=True) + 1e-9)).mean(1)
+      aux_loss = aux_loss + 0.5 * (proxy_2 * density_2).mean() * e * e
+    aux_loss = aux_loss / mb
   elif gating == "ntlb":
     out = (p[rows + (i1,)] * m1 * k1)[..., None] * ffn(i1)
     topk = aux["topk_index"]                                  # [G,S,k] fixed
@@ -1064,11 +1069,12 @@ def _f64_layer(x, wg, wi, wo, aux, gating, m1, coef, mb, z_loss, mult=None,
 @pytest.mark.parametrize("gating", ["top_2", "switch", "switch_max", "ntlb",
                                     "switch+jitter", "switch+dropout",
                                     "ntlb+jitter", "switch+sample",
-                                    "top_2+hidden"])
+                                    "top_2+hidden", "top_2+loss2"])
 def test_backward_against_central_differences(gating):
   gating, _, perturb = gating.partition("+")
   hidden = perturb == "hidden"      # dropout on the experts' hidden tensor
-  if hidden:
+  loss2 = perturb == "loss2"        # moe_use_second_place_loss
+  if hidden or loss2:
     perturb = ""
   rng = np.random.default_rng(61)
   b, l, m, h, e, group = 2, 24, 6, 10, 4, 24
@@ -1087,7 +1093,10 @@ def test_backward_against_central_differences(gating):
            moe_switch_temperature=2.0,
            moe_switch_jitter=0.3, moe_switch_dropout=0.25, moe_ntlb_top_k=3,
            moe_z_loss=0.3 if gating == "switch" else None,
-           moe_dropout_rate=0.4 if hidden else 0.0)
+           moe_dropout_rate=0.4 if hidden else 0.0,
+           moe_use_second_place_loss=loss2,
+           moe_second_policy_train="threshold" if loss2 else "all",
+           moe_second_threshold_train=0.3)
   noise = rng.random((b, l, m)).astype(np.float32) if perturb else None
   su = rng.random((b * l // group, group, e)).astype(np.float32)
   hu = hnoise = None
@@ -1114,10 +1123,17 @@ def test_backward_against_central_differences(gating):
     assert (aux["taken_in_pass"] > 0).any()        # tokens placed by a later choice
   m1 = (nonpad.reshape(aux["kept_1"].shape) == 1).astype(np.float64)
   z = hp.moe_z_loss if gating == "switch" else None
+  density_2 = None
+  if loss2:
+    # counted before the second-choice policy, which drops some of them here
+    m2 = (nonpad.reshape(aux["kept_1"].shape) > 0)
+    assert (m2 & ~aux["kept_2"]).any()
+    density_2 = ((aux["index_2"][..., None] == np.arange(e))
+                 * m2[..., None]).mean(1)
 
   def scalar(xv, wgv, wiv, wov):
     out, loss = _f64_layer(xv.reshape(b, l, m), wgv, wiv, wov, aux, gating, m1,
-                           0.5, mb, z, mult, hnoise)
+                           0.5, mb, z, mult, hnoise, density_2)
     return (out * d_out.reshape(out.shape)).sum() + d_loss * loss
   base = [a.astype(np.float64) for a in (x.reshape(b, l, m), wg, wi, wo)]
   grads = [got["dx"].reshape(b, l, m), got["dw_gate"], got["dwi"], got["dwo"]]
