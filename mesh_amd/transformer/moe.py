@@ -399,11 +399,9 @@ class MoEV1Operation(mtf.Operation):
       self._outputs.append(mtf.Tensor(self, out_shape, inputs.dtype, index=2))
 
   def gradient(self, grad_ys):
-    """Gradients w.r.t. (inputs, gate kernel, wi, wo[, importance]) from those
-    of (outputs, loss); importance carries none."""
-    if self._k_wo is not None:
-      raise NotImplementedError(
-          "backward with moe_use_experts_attention is not implemented")
+    """Gradients w.r.t. (inputs, gate kernel, wi, wo[, importance][, k_wo])
+    from those of (outputs, loss[, second outputs]); importance carries
+    none."""
     if self._gating.router == "expert_selection":
       raise NotImplementedError(
           "backward of expert_selection gating is not implemented")
@@ -416,13 +414,21 @@ class MoEV1Operation(mtf.Operation):
           "backward of expert activation %r is not implemented (the "
           "pre-activation is not kept)" % (self._activation,))
     self._save_for_backward = True
-    d_out, d_loss = grad_ys
+    d_out, d_loss = grad_ys[:2]
     if d_out is None:
       d_out = mtf.zeros(self.mesh, self.outputs[0].shape, self.outputs[0].dtype)
     if d_loss is None:
       d_loss = mtf.zeros(self.mesh, mtf.Shape([]), self.outputs[1].dtype)
-    grads = MoEV1GradOperation(self, d_out, d_loss).outputs
-    return grads + [None] * (len(self.inputs) - 4)
+    d_k = None
+    if self._k_wo is not None:
+      d_k = grad_ys[2]
+      if d_k is None:
+        d_k = mtf.zeros(self.mesh, self.outputs[2].shape, self.outputs[2].dtype)
+    grads = MoEV1GradOperation(self, d_out, d_loss, d_k).outputs
+    by_input = dict(zip(self.inputs[:4], grads[:4]))
+    if self._k_wo is not None:
+      by_input[self._k_wo] = grads[4]
+    return [by_input.get(t) for t in self.inputs]
 
   def lower(self, lowering):
     mesh_impl = lowering.mesh_impl(self)
@@ -497,6 +503,8 @@ class MoEV1Operation(mtf.Operation):
       if kwo_p is not None:
         # the "k" projection of the same hidden tensor (moe.py:514-520)
         yk = moe_hip.expert_linear(h, kwo_p).reshape(e_, groups, c_, n_)
+        if save:
+          saved.update(yk=yk)
         out_k = (moe_hip.slot_combine(yk, r, s_) if by_slot
                  else moe_hip.combine(yk, r, s_))
         outs = outs + (out_k.reshape(o_, g_, s_, n_),)
@@ -520,12 +528,20 @@ class MoEV1GradOperation(mtf.Operation):
   sequence into the HIP library on the activations the forward operation
   kept."""
 
-  def __init__(self, forward, d_out, d_loss, name="moe_v1_grad"):
-    super(MoEV1GradOperation, self).__init__(
-        forward.inputs[:4] + [d_out, d_loss], name=name)
+  def __init__(self, forward, d_out, d_loss, d_k=None, name="moe_v1_grad"):
+    """d_k: gradient of the second outputs of a layer with
+    moe_use_experts_attention; the operation then has a fifth output, the
+    gradient of the "k_wo" kernel."""
+    ins = forward.inputs[:4] + [d_out, d_loss]
+    wrt = forward.inputs[:4]
+    if d_k is not None:
+      ins = ins + [forward._k_wo, d_k]
+      wrt = wrt + [forward._k_wo]
+    super(MoEV1GradOperation, self).__init__(ins, name=name)
     self._forward = forward
+    self._has_k = d_k is not None
     self._outputs = [mtf.Tensor(self, t.shape, t.dtype, index=i)
-                     for i, t in enumerate(forward.inputs[:4])]
+                     for i, t in enumerate(wrt)]
 
   @property
   def has_gradient(self):
@@ -541,7 +557,7 @@ class MoEV1GradOperation(mtf.Operation):
     groups = o_ * g_
     gating = fwd._gating
 
-    def fn(wi_s, wo_s, dout_s, dloss_s):
+    def fn(wi_s, wo_s, dout_s, dloss_s, kwo_s=None, dk_s=None):
       sv = lowering.operations[fwd]
       if not sv:
         raise ValueError("the forward operation kept no activations: build "
@@ -554,6 +570,19 @@ class MoEV1GradOperation(mtf.Operation):
           sv["expert_in"].reshape(e_, groups * c_, m_), sv["h"],
           dy.reshape(e_, groups * c_, n_), wi_s, wo_s, fwd._activation,
           dh_scale=sv["hidden_noise"])
+      dkwo = None
+      if kwo_s is not None:
+        # the second projection of the same hidden tensor: its share of every
+        # gradient adds to the first one's (the hidden tensor and the combine
+        # weights have two consumers)
+        dyk, dgate_k = moe_hip.combine_backward(
+            dk_s.reshape(groups, s_, n_).contiguous(),
+            sv["yk"].reshape(e_, groups, c_, n_), r)
+        dxe_k, dwi_k, dkwo = moe_hip.expert_ffn_backward(
+            sv["expert_in"].reshape(e_, groups * c_, m_), sv["h"],
+            dyk.reshape(e_, groups * c_, n_), wi_s, kwo_s, fwd._activation,
+            dh_scale=sv["hidden_noise"])
+        dxe, dwi, dgate = dxe + dxe_k, dwi + dwi_k, dgate + dgate_k
       dlogits = moe_hip.gating_backward(
           sv["logits"], r, dgate, dloss_s.reshape(1).float(), 1.0,
           router=gating.router, top_k=getattr(gating, "top_k", 0),
@@ -583,13 +612,14 @@ class MoEV1GradOperation(mtf.Operation):
         dx = (dx.reshape(tokens, m_).to(torch.float32) +
               dx_router.reshape(tokens, m_) *
               mult.reshape(tokens, m_).to(torch.float32)).to(dt)
-      return dx.reshape(o_, g_, s_, m_), dwg, dwi, dwo
+      res = (dx.reshape(o_, g_, s_, m_), dwg, dwi, dwo)
+      return res + (dkwo,) if kwo_s is not None else res
 
     ins = self.inputs
-    outs = mesh_impl.slicewise(fn, lowering.tensors[ins[2]],
-                               lowering.tensors[ins[3]],
-                               lowering.tensors[ins[4]],
-                               lowering.tensors[ins[5]])
+    args = [lowering.tensors[ins[i]] for i in (2, 3, 4, 5)]
+    if self._has_k:
+      args += [lowering.tensors[ins[6]], lowering.tensors[ins[7]]]
+    outs = mesh_impl.slicewise(fn, *args)
     for t, v in zip(self.outputs, outs):
       lowering.set_tensor_lowering(t, v)
 

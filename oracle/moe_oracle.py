@@ -1221,7 +1221,7 @@ def moe_layer_v1_backward(x, w_gate, wi, wo, hp, train, act_dtype, d_out,
                           d_loss=0.0, nonpadding=None, activation="relu",
                           num_microbatches=None, logit_bias=None,
                           gate_noise=None, sample_uniform=None,
-                          hidden_uniform=None):
+                          hidden_uniform=None, k_wo=None):
   """Gradients of (outputs, loss) of moe_layer_v1 w.r.t. x and the three
   kernels, given d_out [batch..., length, N] and the scalar d_loss.
 
@@ -1233,8 +1233,29 @@ def moe_layer_v1_backward(x, w_gate, wi, wo, hp, train, act_dtype, d_out,
   ops.py:1945-1962), float32 inside the gating.  The dispatch tensor is a
   bool cast of the combine tensor and carries no gradient (moe.py:1510-1511).
 
+  With hparams.moe_use_experts_attention (k_wo given, d_out = [d_q, d_k]) the
+  two outputs are two plain layers that share everything but the output kernel
+  (moe_layer_v1), so every shared gradient is the sum of the two layers'
+  (mtf.gradients adds the gradients of a tensor's consumers, ops.py:5276-5283)
+  and "dk_wo" is the second layer's dwo.
+
   Returns dict(dx, dw_gate, dwi, dwo) holding activation-dtype values.
   """
+  if getattr(hp, "moe_use_experts_attention", False):
+    import copy
+    hp1 = copy.copy(hp)
+    hp1.moe_use_experts_attention = False
+    kw = dict(nonpadding=nonpadding, activation=activation,
+              num_microbatches=num_microbatches, logit_bias=logit_bias,
+              gate_noise=gate_noise, sample_uniform=sample_uniform,
+              hidden_uniform=hidden_uniform)
+    q = moe_layer_v1_backward(x, w_gate, wi, wo, hp1, train, act_dtype,
+                              d_out[0], d_loss, **kw)
+    k = moe_layer_v1_backward(x, w_gate, wi, k_wo, hp1, train, act_dtype,
+                              d_out[1], 0.0, **kw)
+    out = {n: cast_act(q[n] + k[n], act_dtype) for n in ("dx", "dw_gate", "dwi")}
+    out.update(dwo=q["dwo"], dk_wo=k["dwo"], aux=q["aux"])
+    return out
   if isinstance(wi, (list, tuple)) or isinstance(activation, (list, tuple)):
     raise NotImplementedError("backward of a product of dense layers")
   if activation not in ("relu", "linear", None):

@@ -722,8 +722,60 @@ def test_v1_experts_attention(act_dtype):
                              moe_group_size=group)
   plain_k, _, _, _ = run_v1(x, dict(w, wo=k_wo), hp_plain, True, act_dtype)
   np.testing.assert_array_equal(k, plain_k)
-  with pytest.raises(NotImplementedError, match="experts_attention"):
-    mtf.gradients([outs[0]], [xt])
+
+
+@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
+def test_v1_experts_attention_gradients(act_dtype):
+  """Gradients through both outputs of the layer with
+  moe_use_experts_attention: the shared tensors get the sum of the two
+  projections' shares."""
+  b, l, m, hdim, e, group = 2, 64, 32, 48, 4, 32
+  rng = np.random.default_rng(521)
+  w = dict(w_gate=H.normal_weights(rng, (m, e), m),
+           wi=H.normal_weights(rng, (e, m, hdim), m),
+           wo=H.normal_weights(rng, (e, hdim, m), hdim))
+  k_wo = H.normal_weights(rng, (e, hdim, m), hdim)
+  x = H.safe_tokens(rng, b * l, m, w["w_gate"], act_dtype).reshape(b, l, m)
+  d_q, d_k = (O.cast_act(rng.standard_normal((b, l, m)).astype(np.float32),
+                         act_dtype) for _ in range(2))
+  hp, ohp = make_hparams(moe_num_experts=e, moe_hidden_size=hdim,
+                         moe_group_size=group, moe_use_experts_attention=True,
+                         moe_capacity_factor_train=1.0, moe_loss_coef=0.25)
+  dt = H.ACT_TORCH[act_dtype]
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  dims = [mtf.Dimension("batch", b), mtf.Dimension("length", l),
+          mtf.Dimension("d_model", m)]
+  imp = lambda a, shape: mtf.import_tf_tensor(
+      mesh, torch.from_numpy(np.asarray(a, np.float32)).to(dt), mtf.Shape(shape))
+  xt = imp(x, dims)
+  with mtf.variable_scope("moe"):
+    outs, loss = moe.transformer_moe_layer_v1(
+        xt, dims[-1], hp, True, mtf.VariableDType(torch.float32, torch.float32, dt))
+  by_name = {v.name: v.outputs[0] for v in graph.trainable_variables}
+  names = ["moe/top_2_gating/kernel", "moe/wi/kernel", "moe/q_wo/kernel",
+           "moe/k_wo/kernel"]
+  grads = mtf.gradients(outs + [loss], [xt] + [by_name[n] for n in names],
+                        grad_ys=[imp(d_q, dims), imp(d_k, dims), imp(1.5, [])])
+  lowering = mtf.Lowering(
+      graph, {mesh: mtf.HipMeshImpl()},
+      initial_values=dict(zip(names, (w["w_gate"], w["wi"], w["wo"], k_wo))))
+  got = [H.to_np(lowering.export_to_tf_tensor(g)) for g in grads]
+  want = O.moe_layer_v1_backward(x, w["w_gate"], w["wi"], w["wo"], ohp, True,
+                                 act_dtype, [d_q, d_k], 1.5, k_wo=k_wo)
+  assert not (want["aux"]["kept_1"] & want["aux"]["kept_2"]).all()
+  only_q = O.moe_layer_v1_backward(
+      x, w["w_gate"], w["wi"], w["wo"],
+      make_hparams(moe_num_experts=e, moe_hidden_size=hdim, moe_group_size=group,
+                   moe_capacity_factor_train=1.0, moe_loss_coef=0.25)[1],
+      True, act_dtype, d_q, 1.5)
+  assert np.abs(want["dx"] - only_q["dx"]).max() > 0.1   # the k branch matters
+  tol = H.value_tolerance(act_dtype)
+  for g_, k in zip(got, ("dx", "dw_gate", "dwi", "dwo", "dk_wo")):
+    ref = want[k].reshape(g_.shape)
+    np.testing.assert_allclose(
+        g_, ref, rtol=tol["rtol"], atol=tol["atol"] * max(1.0, np.abs(ref).max()),
+        err_msg=k)
 
 
 @pytest.mark.parametrize("case", [("float32", False), ("bfloat16", False),
