@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 11
+#define MESH_MOE_ABI_VERSION 12
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -425,6 +425,45 @@ int mesh_moe_expert_ffn_backward(const void* expert_in, const void* h,
                                  int R, int M, int H, int N, int activation,
                                  int dtype, void* workspace,
                                  size_t workspace_bytes, void* stream);
+
+/* Bytes of scratch mesh_moe_expert_linear_backward needs. */
+size_t mesh_moe_expert_linear_backward_workspace_bytes(int E, int R, int K,
+                                                       int N, int dtype);
+
+/*
+ * Backward of one expert projection y = a . w (mtf.layers.dense with
+ * expert_dims, layers.py:129-208; EinsumOperation.gradient, ops.py:2846-2854):
+ *   da = dy . w^T;  dw = a^T . dy
+ *   a [E,R,K], dy [E,R,N], w [E,K,N] (the variable's own layout), da [E,R,K]
+ *   (NULL: not wanted), dw [E,K,N]; everything of `dtype`
+ * With mesh_moe_activation_backward this is what the layer's backward is made
+ * of when the experts are not plain ReLU / linear layers (products of several
+ * dense layers, other activations: transformer/moe.py:469-475).
+ */
+int mesh_moe_expert_linear_backward(const void* a, const void* dy,
+                                    const void* w, void* da, void* dw, int E,
+                                    int R, int K, int N, int dtype,
+                                    void* workspace, size_t workspace_bytes,
+                                    void* stream);
+
+/*
+ * out = act(pre) on n elements of `dtype`: the activation of a dense layer
+ * (ops.py:1818-1921) as a step of its own, for callers that keep the
+ * pre-activation for the backward pass (mesh_moe_expert_linear with that
+ * activation gives the same values).
+ */
+int mesh_moe_activation(const void* pre, void* out, int64_t n, int activation,
+                        int dtype, void* stream);
+
+/*
+ * dpre = dh * factor * act'(pre) on n elements of `dtype` (float32 arithmetic,
+ * one rounding): the gradient of a dense layer's activation from its
+ * pre-activation (ops.py:1818-1921), times the other factors of a product of
+ * dense layers (factor NULL: none).
+ */
+int mesh_moe_activation_backward(const void* dh, const void* pre,
+                                 const void* factor, void* dpre, int64_t n,
+                                 int activation, int dtype, void* stream);
 
 /* Bytes of scratch mesh_moe_gating_backward needs. */
 size_t mesh_moe_gating_backward_workspace_bytes(int G, int E);

@@ -996,6 +996,16 @@ __global__ __launch_bounds__(256) void activation_kernel(T* __restrict__ h,
     store_f32<T>(h + i, apply_activation(load_f32<T>(h + i), act));
 }
 
+// out = act(pre), element by element (what activation_kernel does in place).
+template <typename T>
+__global__ __launch_bounds__(256) void activation_copy_kernel(
+    const T* __restrict__ pre, T* __restrict__ out, int64_t n, int act) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += stride)
+    store_f32<T>(out + i, apply_activation(load_f32<T>(pre + i), act));
+}
+
 // dh = dh * scale (when given), then dh = (h > 0) ? dh : 0 for ReLU experts --
 // the hidden dropout and the ReLU of the forward pass seen from behind (h is
 // the stored, already rounded activation: positive iff the pre-activation
@@ -1035,6 +1045,48 @@ __global__ __launch_bounds__(256) void hidden_product_kernel(
       store_f32<T>(h + i, v * noise);
       if (noise_out) store_f32<T>(noise_out + i, noise);
     } 
+  }
+}
+
+// d(act(v)) / dv in float32, from the pre-activation v.
+__device__ __forceinline__ float activation_derivative(float v, int act) {
+  switch (act) {
+    case MESH_MOE_ACT_RELU:
+      return v > 0.f ? 1.0f : 0.0f;
+    case MESH_MOE_ACT_GELU: {
+      const float k = 0.7978845608028654f;
+      const float t = tanhf(k * (v + 0.044715f * v * v * v));
+      const float du = k * (1.0f + 3.0f * 0.044715f * v * v);
+      return 0.5f * (1.0f + t) + 0.5f * v * (1.0f - t * t) * du;
+    }
+    case MESH_MOE_ACT_SIGMOID: {
+      const float sg = 1.0f / (1.0f + expf(-v));
+      return sg * (1.0f - sg);
+    }
+    case MESH_MOE_ACT_TANH: {
+      const float t = tanhf(v);
+      return 1.0f - t * t;
+    }
+    case MESH_MOE_ACT_SWISH: {
+      const float sg = 1.0f / (1.0f + expf(-v));
+      return sg + v * sg * (1.0f - sg);
+    }
+    default:
+      return 1.0f;
+  }
+}
+
+// dpre = dh * factor * act'(pre), float32 arithmetic, one rounding.
+template <typename T>
+__global__ __launch_bounds__(256) void activation_backward_kernel(
+    const T* __restrict__ dh, const T* __restrict__ pre,
+    const T* __restrict__ factor, T* __restrict__ dpre, int64_t n, int act) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += stride) {
+    float g = load_f32<T>(dh + i);
+    if (factor) g *= load_f32<T>(factor + i);
+    store_f32<T>(dpre + i, g * activation_derivative(load_f32<T>(pre + i), act));
   }
 }
 
@@ -1459,6 +1511,102 @@ extern "C" int mesh_moe_hidden_product(void* h, const void* factor,
   }
   MOE_CHECK_LAUNCH("hidden_product");
   return 0;
+}
+
+extern "C" int mesh_moe_activation(const void* pre, void* out, int64_t n,
+                                   int activation, int dtype, void* stream) {
+  MOE_REQUIRE(pre && out, MESH_MOE_E_ARG, "activation: null pointer");
+  MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG, "activation: bad dtype %d",
+              dtype);
+  MOE_REQUIRE(n >= 1, MESH_MOE_E_ARG, "activation: bad size n=%lld",
+              (long long)n);
+  MOE_REQUIRE(activation >= MESH_MOE_ACT_LINEAR &&
+                  activation <= MESH_MOE_ACT_SWISH,
+              MESH_MOE_E_ARG, "activation: unknown activation %d", activation);
+  hipStream_t st = (hipStream_t)stream;
+  const int blocks = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
+  if (dtype == MESH_MOE_F32)
+    activation_copy_kernel<float><<<blocks, 256, 0, st>>>(
+        (const float*)pre, (float*)out, n, activation);
+  else
+    activation_copy_kernel<bf16_t><<<blocks, 256, 0, st>>>(
+        (const bf16_t*)pre, (bf16_t*)out, n, activation);
+  MOE_CHECK_LAUNCH("activation");
+  return 0;
+}
+
+extern "C" int mesh_moe_activation_backward(const void* dh, const void* pre,
+                                            const void* factor, void* dpre,
+                                            int64_t n, int activation,
+                                            int dtype, void* stream) {
+  MOE_REQUIRE(dh && pre && dpre, MESH_MOE_E_ARG,
+              "activation_backward: null pointer");
+  MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG,
+              "activation_backward: bad dtype %d", dtype);
+  MOE_REQUIRE(n >= 1, MESH_MOE_E_ARG, "activation_backward: bad size n=%lld",
+              (long long)n);
+  MOE_REQUIRE(activation >= MESH_MOE_ACT_LINEAR &&
+                  activation <= MESH_MOE_ACT_SWISH,
+              MESH_MOE_E_ARG, "activation_backward: unknown activation %d",
+              activation);
+  hipStream_t st = (hipStream_t)stream;
+  const int blocks = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
+  if (dtype == MESH_MOE_F32)
+    activation_backward_kernel<float><<<blocks, 256, 0, st>>>(
+        (const float*)dh, (const float*)pre, (const float*)factor,
+        (float*)dpre, n, activation);
+  else
+    activation_backward_kernel<bf16_t><<<blocks, 256, 0, st>>>(
+        (const bf16_t*)dh, (const bf16_t*)pre, (const bf16_t*)factor,
+        (bf16_t*)dpre, n, activation);
+  MOE_CHECK_LAUNCH("activation_backward");
+  return 0;
+}
+
+extern "C" size_t mesh_moe_expert_linear_backward_workspace_bytes(int E, int R,
+                                                                  int K, int N,
+                                                                  int dtype) {
+  if (E < 1 || R < 1 || K < 1 || N < 1 || !valid_dtype(dtype)) return 0;
+  return ((size_t)E * R * K + (size_t)E * R * N) * dtype_size(dtype) + 2 * 256;
+}
+
+extern "C" int mesh_moe_expert_linear_backward(
+    const void* a, const void* dy, const void* w, void* da, void* dw, int E,
+    int R, int K, int N, int dtype, void* workspace, size_t workspace_bytes,
+    void* stream) {
+  MOE_REQUIRE(a && dy && w && dw && workspace, MESH_MOE_E_ARG,
+              "expert_linear_backward: null pointer");
+  MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG,
+              "expert_linear_backward: bad dtype %d", dtype);
+  MOE_REQUIRE(E >= 1 && R >= 1 && K >= 1 && N >= 1, MESH_MOE_E_ARG,
+              "expert_linear_backward: bad sizes E=%d R=%d K=%d N=%d", E, R, K,
+              N);
+  MOE_REQUIRE(workspace_bytes >=
+                  mesh_moe_expert_linear_backward_workspace_bytes(E, R, K, N,
+                                                                  dtype),
+              MESH_MOE_E_ARG, "expert_linear_backward: workspace too small");
+  hipStream_t st = (hipStream_t)stream;
+  int rc;
+  if (da != nullptr) {
+    // da = dy . w^T  (w in its variable layout [E, K, N] is K-contiguous here)
+    rc = grouped_gemm(dy, w, da, E, R, K, N, MESH_MOE_ACT_LINEAR, dtype, st);
+    if (rc != 0) return rc;
+  }
+  // dw [E, K, N] = a^T . dy: the reduction runs over the rows of both operands
+  if (kmajor_path_applies(a, dy, dw, K, N, R, dtype))
+    return launch_ring_kmajor((const bf16_t*)a, (const bf16_t*)dy, (bf16_t*)dw,
+                              E, K, N, R, st);
+  const size_t es = dtype_size(dtype);
+  auto up = [](uintptr_t v) { return (v + 255) & ~(uintptr_t)255; };
+  unsigned char* tr_a = (unsigned char*)up((uintptr_t)workspace);
+  unsigned char* tr_dy =
+      (unsigned char*)up((uintptr_t)(tr_a + (size_t)E * R * K * es));
+  rc = mesh_moe_pack_weights(a, tr_a, E, R, K, dtype, dtype, stream);
+  if (rc != 0) return rc;
+  rc = mesh_moe_pack_weights(dy, tr_dy, E, R, N, dtype, dtype, stream);
+  if (rc != 0) return rc;
+  return grouped_gemm(tr_a, tr_dy, dw, E, K, N, R, MESH_MOE_ACT_LINEAR, dtype,
+                      st);
 }
 
 // Elements of the scratch mesh_moe_expert_ffn_backward needs: dh [E,R,H], one

@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 11
+ABI_VERSION = 12
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -95,6 +95,15 @@ _SIGNATURES = {
         _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         _vp, ctypes.c_size_t, _vp]),
+    "mesh_moe_expert_linear_backward_workspace_bytes": (ctypes.c_size_t, [
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "mesh_moe_expert_linear_backward": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
+    "mesh_moe_activation": (ctypes.c_int, [
+        _vp, _vp, ctypes.c_int64, ctypes.c_int, ctypes.c_int, _vp]),
+    "mesh_moe_activation_backward": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, ctypes.c_int64, ctypes.c_int, ctypes.c_int, _vp]),
     "mesh_moe_gating_backward_workspace_bytes": (ctypes.c_size_t, [
         ctypes.c_int, ctypes.c_int]),
     "mesh_moe_gating_backward": (ctypes.c_int, [
@@ -721,6 +730,58 @@ def expert_ffn_backward(expert_in, h, dy, wi, wo, activation="relu",
         dwo.data_ptr(), e, rows, m, hdim, n, ACTIVATIONS[activation], code,
         ws.data_ptr(), ws_bytes, _stream()), "expert_ffn_backward")
   return dxe, dwi, dwo
+
+
+def expert_linear_backward(a, dy, w, want_da=True):
+  """Backward of y = a . w per expert: a [E,R,K], dy [E,R,N], w [E,K,N] in the
+  variable's own layout -> (da [E,R,K] or None, dw [E,K,N])."""
+  lib = load_library()
+  e, rows, k = a.shape
+  n = w.shape[2]
+  dt = a.dtype
+  code = dtype_code(dt)
+  da = torch.empty((e, rows, k), dtype=dt, device=a.device) if want_da else None
+  dw = torch.empty((e, k, n), dtype=dt, device=a.device)
+  ws_bytes = lib.mesh_moe_expert_linear_backward_workspace_bytes(
+      e, rows, k, n, code)
+  ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=a.device)
+  with _stage("expert_linear_backward"):
+    _check(lib.mesh_moe_expert_linear_backward(
+        _dev(a, "a"), _dev(dy, "dy", dt, (e, rows, n)),
+        _dev(w, "w", dt, (e, k, n)), da.data_ptr() if want_da else None,
+        dw.data_ptr(), e, rows, k, n, code, ws.data_ptr(), ws_bytes,
+        _stream()), "expert_linear_backward")
+  return da, dw
+
+
+def activation(pre, activation):
+  """act(pre), a new tensor."""
+  lib = load_library()
+  if activation not in ACTIVATIONS:
+    raise ValueError("unsupported expert activation %r" % (activation,))
+  out = torch.empty_like(pre)
+  with _stage("activation"):
+    _check(lib.mesh_moe_activation(
+        _dev(pre, "pre"), out.data_ptr(), pre.numel(), ACTIVATIONS[activation],
+        dtype_code(pre.dtype), _stream()), "activation")
+  return out
+
+
+def activation_backward(dh, pre, activation, factor=None):
+  """dh * factor * act'(pre), a new tensor of pre's shape and dtype."""
+  lib = load_library()
+  if activation not in ACTIVATIONS:
+    raise ValueError("unsupported expert activation %r" % (activation,))
+  dt = pre.dtype
+  out = torch.empty_like(pre)
+  with _stage("activation_backward"):
+    _check(lib.mesh_moe_activation_backward(
+        _dev(dh, "dh", dt, tuple(pre.shape)), _dev(pre, "pre"),
+        _dev(factor, "factor", dt, tuple(pre.shape))
+        if factor is not None else None,
+        out.data_ptr(), pre.numel(), ACTIVATIONS[activation], dtype_code(dt),
+        _stream()), "activation_backward")
+  return out
 
 
 def gating_backward(logits, r, dgate, d_loss, loss_scale, router="top_2",

@@ -390,6 +390,10 @@ class MoEV1Operation(mtf.Operation):
     self._more_wi = wis[1:]
     self._more_activations = acts[1:]
     self._hidden_keep_prob = hidden_keep_prob
+    # experts that are not one ReLU / linear layer: the backward pass needs the
+    # pre-activation of every factor
+    self._general_hidden = bool(self._more_wi) or (
+        self._activation not in ("relu", "linear"))
     self._num_experts = wi.shape.dims[0].size
     self._save_for_backward = False
     out_shape = mtf.Shape(inputs.shape.dims[:-1] + [output_dim])
@@ -405,14 +409,6 @@ class MoEV1Operation(mtf.Operation):
     if self._gating.router == "expert_selection":
       raise NotImplementedError(
           "backward of expert_selection gating is not implemented")
-    if self._more_wi:
-      raise NotImplementedError(
-          "backward of a product of several dense layers (gated expert "
-          "activations) is not implemented")
-    if self._activation not in ("relu", "linear"):
-      raise NotImplementedError(
-          "backward of expert activation %r is not implemented (the "
-          "pre-activation is not kept)" % (self._activation,))
     self._save_for_backward = True
     d_out, d_loss = grad_ys[:2]
     if d_out is None:
@@ -424,10 +420,8 @@ class MoEV1Operation(mtf.Operation):
       d_k = grad_ys[2]
       if d_k is None:
         d_k = mtf.zeros(self.mesh, self.outputs[2].shape, self.outputs[2].dtype)
-    grads = MoEV1GradOperation(self, d_out, d_loss, d_k).outputs
-    by_input = dict(zip(self.inputs[:4], grads[:4]))
-    if self._k_wo is not None:
-      by_input[self._k_wo] = grads[4]
+    grad_op = MoEV1GradOperation(self, d_out, d_loss, d_k)
+    by_input = dict(zip(grad_op.wrt, grad_op.outputs))
     return [by_input.get(t) for t in self.inputs]
 
   def lower(self, lowering):
@@ -441,7 +435,8 @@ class MoEV1Operation(mtf.Operation):
              else None)
     more_wi_p = [_packed(lowering, t, dt) for t in self._more_wi]
     keep_prob = self._hidden_keep_prob
-    plain_hidden = not more_wi_p and keep_prob is None
+    keep_pre = self._save_for_backward and self._general_hidden
+    plain_hidden = not more_wi_p and keep_prob is None and not keep_pre
     o_, g_, s_, m_ = x.shape.to_integer_list
     n_ = self.outputs[0].shape.dims[-1].size
     e_, c_ = self._num_experts, self._capacity
@@ -480,10 +475,21 @@ class MoEV1Operation(mtf.Operation):
       elif y is None:
         # the hidden tensor is worked on between the two projections: the
         # other factors of the product, then the dropout
-        h = moe_hip.expert_linear(expert_in, wi_p, self._activation)
-        for w_p, act in zip(more_wi_p, self._more_activations):
-          moe_hip.hidden_product(
-              h, factor=moe_hip.expert_linear(expert_in, w_p, act))
+        pres, factors = [], []
+        for w_p, act in zip([wi_p] + more_wi_p,
+                            [self._activation] + self._more_activations):
+          if keep_pre:
+            pres.append(moe_hip.expert_linear(expert_in, w_p, "linear"))
+            factors.append(moe_hip.activation(pres[-1], act))
+          else:
+            factors.append(moe_hip.expert_linear(expert_in, w_p, act))
+        h = factors[0].clone() if (keep_pre and len(factors) > 1) else factors[0]
+        for f in factors[1:]:
+          moe_hip.hidden_product(h, factor=f)
+        if keep_pre:
+          if len(factors) == 1 and keep_prob is not None:
+            factors[0] = None       # h is about to be changed in place
+          saved.update(pre=pres, factors=factors)
         if keep_prob is not None:
           u = torch.rand(h.shape, dtype=dt, device=h.device)
           noise = moe_hip.hidden_product(h, uniform=u, keep_prob=keep_prob,
@@ -537,9 +543,13 @@ class MoEV1GradOperation(mtf.Operation):
     if d_k is not None:
       ins = ins + [forward._k_wo, d_k]
       wrt = wrt + [forward._k_wo]
+    # the kernels of the other factors of a product of dense layers
+    ins = ins + forward._more_wi
+    wrt = wrt + forward._more_wi
     super(MoEV1GradOperation, self).__init__(ins, name=name)
     self._forward = forward
     self._has_k = d_k is not None
+    self.wrt = wrt          # the tensors the outputs are gradients of
     self._outputs = [mtf.Tensor(self, t.shape, t.dtype, index=i)
                      for i, t in enumerate(wrt)]
 
@@ -557,7 +567,37 @@ class MoEV1GradOperation(mtf.Operation):
     groups = o_ * g_
     gating = fwd._gating
 
-    def fn(wi_s, wo_s, dout_s, dloss_s, kwo_s=None, dk_s=None):
+    has_k, n_more = self._has_k, len(fwd._more_wi)
+    activations = [fwd._activation] + fwd._more_activations
+
+    def general_hidden_backward(sv, dys, wos, wis):
+      """Experts that are not one ReLU / linear layer: h = noise * prod_i
+      act_i(expert_in . wi_i).  dys / wos: the gradient and the kernel of every
+      output projection of h.  Returns (dexpert_in, [dwi_i], [dwo_j])."""
+      xe = sv["expert_in"].reshape(e_, groups * c_, m_)
+      dh, dwos = None, []
+      for dy_j, wo_j in zip(dys, wos):
+        dh_j, dwo_j = moe_hip.expert_linear_backward(sv["h"], dy_j, wo_j)
+        dh = dh_j if dh is None else dh + dh_j
+        dwos.append(dwo_j)
+      if sv["hidden_noise"] is not None:
+        moe_hip.hidden_product(dh, factor=sv["hidden_noise"])
+      dxe, dwis = None, []
+      for i, act in enumerate(activations):
+        g = dh
+        for j, f in enumerate(sv["factors"]):
+          if j != i:
+            g = g.clone() if g is dh else g
+            moe_hip.hidden_product(g, factor=f)
+        dpre = moe_hip.activation_backward(g, sv["pre"][i], act)
+        dxe_i, dwi_i = moe_hip.expert_linear_backward(xe, dpre, wis[i])
+        dxe = dxe_i if dxe is None else dxe + dxe_i
+        dwis.append(dwi_i)
+      return dxe, dwis, dwos
+
+    def fn(wi_s, wo_s, dout_s, dloss_s, *rest):
+      kwo_s, dk_s = rest[:2] if has_k else (None, None)
+      more_wi_s = list(rest[2 if has_k else 0:])
       sv = lowering.operations[fwd]
       if not sv:
         raise ValueError("the forward operation kept no activations: build "
@@ -566,11 +606,26 @@ class MoEV1GradOperation(mtf.Operation):
       dy, dgate = moe_hip.combine_backward(
           dout_s.reshape(groups, s_, n_).contiguous(),
           sv["y"].reshape(e_, groups, c_, n_), r)
-      dxe, dwi, dwo = moe_hip.expert_ffn_backward(
-          sv["expert_in"].reshape(e_, groups * c_, m_), sv["h"],
-          dy.reshape(e_, groups * c_, n_), wi_s, wo_s, fwd._activation,
-          dh_scale=sv["hidden_noise"])
-      dkwo = None
+      if fwd._general_hidden:
+        dys, wos = [dy.reshape(e_, groups * c_, n_)], [wo_s]
+        if has_k:
+          dyk, dgate_k = moe_hip.combine_backward(
+              dk_s.reshape(groups, s_, n_).contiguous(),
+              sv["yk"].reshape(e_, groups, c_, n_), r)
+          dys.append(dyk.reshape(e_, groups * c_, n_))
+          wos.append(kwo_s)
+          dgate = dgate + dgate_k
+        dxe, dwis, dwos = general_hidden_backward(sv, dys, wos,
+                                                  [wi_s] + more_wi_s)
+        dwi, dwo = dwis[0], dwos[0]
+        dkwo = dwos[1] if has_k else None
+        kwo_s = None                        # its share is in already
+      else:
+        dxe, dwi, dwo = moe_hip.expert_ffn_backward(
+            sv["expert_in"].reshape(e_, groups * c_, m_), sv["h"],
+            dy.reshape(e_, groups * c_, n_), wi_s, wo_s, fwd._activation,
+            dh_scale=sv["hidden_noise"])
+        dkwo, dwis = None, [dwi]
       if kwo_s is not None:
         # the second projection of the same hidden tensor: its share of every
         # gradient adds to the first one's (the hidden tensor and the combine
@@ -613,12 +668,13 @@ class MoEV1GradOperation(mtf.Operation):
               dx_router.reshape(tokens, m_) *
               mult.reshape(tokens, m_).to(torch.float32)).to(dt)
       res = (dx.reshape(o_, g_, s_, m_), dwg, dwi, dwo)
-      return res + (dkwo,) if kwo_s is not None else res
+      if has_k:
+        res = res + (dkwo,)
+      return res + tuple(dwis[1:])
 
     ins = self.inputs
     args = [lowering.tensors[ins[i]] for i in (2, 3, 4, 5)]
-    if self._has_k:
-      args += [lowering.tensors[ins[6]], lowering.tensors[ins[7]]]
+    args += [lowering.tensors[t] for t in ins[6:]]
     outs = mesh_impl.slicewise(fn, *args)
     for t, v in zip(self.outputs, outs):
       lowering.set_tensor_lowering(t, v)

@@ -1194,27 +1194,72 @@ def dispatch_backward(dxe, r, act_dtype):
   return dx
 
 
+def _gelu_grad(x):
+  k = F32(np.sqrt(2 / np.pi))
+  t = np.tanh(k * (x + F32(0.044715) * x * x * x)).astype(F32)
+  du = k * (F32(1.0) + F32(3 * 0.044715) * x * x)
+  return F32(0.5) * (F32(1.0) + t) + F32(0.5) * x * (F32(1.0) - t * t) * du
+
+
+def _sigmoid(x):
+  return (F32(1) / (F32(1) + np.exp(-x))).astype(F32)
+
+
+# d act(x) / dx from the pre-activation, float32
+ACTIVATION_GRADS = {
+    "relu": lambda x: (x > 0).astype(F32),
+    "linear": lambda x: np.ones_like(x, dtype=F32),
+    None: lambda x: np.ones_like(x, dtype=F32),
+    "gelu": _gelu_grad,
+    "sigmoid": lambda x: _sigmoid(x) * (F32(1) - _sigmoid(x)),
+    "tanh": lambda x: F32(1) - np.tanh(x).astype(F32) ** 2,
+    "swish": lambda x: _sigmoid(x) + x * _sigmoid(x) * (F32(1) - _sigmoid(x)),
+}
+
+
 def expert_ffn_backward(xe, wi_a, wo_a, dy, activation, act_dtype,
                         hidden_noise=None):
-  """Backward of the two expert einsums (moe.py:469-486): float32 accumulate,
+  """Backward of the expert einsums (moe.py:469-486): float32 accumulate,
   activation-dtype results.  xe [E,R,M], dy [E,R,N]; returns
   (dxe [E,R,M], dwi [E,M,H], dwo [E,H,N]).  hidden_noise [E,R,H]: the dropout
-  multiplier on the hidden tensor (moe.py:477-479), a constant of the graph."""
-  pre = cast_act(np.matmul(xe, wi_a), act_dtype)
-  h = pre
-  if activation == "relu":
-    h = cast_act(np.maximum(h, F32(0.0)), act_dtype)
+  multiplier on the hidden tensor (moe.py:477-479), a constant of the graph.
+
+  wi_a / activation may be lists (a product of dense layers, layers.py:279-295;
+  dwi is then a list): with f_i = act_i(pre_i), pre_i = xe . wi_i,
+  h = noise * prod_i f_i, the gradient reaching pre_i is
+  dh * noise * prod_{j != i} f_j * act_i'(pre_i); the derivative of an
+  activation is taken in float32 from the (rounded) pre-activation and the
+  product is rounded once (the reference differentiates the primitives an
+  activation is built from, each rounding its result: a few more roundings in
+  bfloat16, nothing else)."""
+  is_list = isinstance(wi_a, (list, tuple))
+  wis = list(wi_a) if is_list else [wi_a]
+  acts = list(activation) if isinstance(activation, (list, tuple)) else [activation]
+  if len(wis) != len(acts):
+    raise ValueError("%d kernels for %d activations" % (len(wis), len(acts)))
+  pres = [cast_act(np.matmul(xe, w), act_dtype) for w in wis]
+  fs = [cast_act(ACTIVATIONS[a](p), act_dtype) for a, p in zip(acts, pres)]
+  h = fs[0]
+  for f in fs[1:]:
+    h = cast_act(h * f, act_dtype)
   if hidden_noise is not None:
     h = cast_act(h * hidden_noise, act_dtype)
   dh = cast_act(np.matmul(dy, wo_a.transpose(0, 2, 1)), act_dtype)
   if hidden_noise is not None:
     dh = cast_act(dh * hidden_noise, act_dtype)
-  if activation == "relu":
-    dh = dh * (pre > 0)
   dwo = cast_act(np.matmul(h.transpose(0, 2, 1), dy), act_dtype)
-  dxe = cast_act(np.matmul(dh, wi_a.transpose(0, 2, 1)), act_dtype)
-  dwi = cast_act(np.matmul(xe.transpose(0, 2, 1), dh), act_dtype)
-  return dxe, dwi, dwo
+  dxe = np.zeros_like(xe, dtype=F32)
+  dwis = []
+  for i, (w, a, p) in enumerate(zip(wis, acts, pres)):
+    g = dh
+    for j, f in enumerate(fs):
+      if j != i:
+        g = cast_act(g * f, act_dtype)
+    dpre = cast_act(g * ACTIVATION_GRADS[a](p), act_dtype)
+    part = cast_act(np.matmul(dpre, w.transpose(0, 2, 1)), act_dtype)
+    dxe = part if i == 0 else cast_act(dxe + part, act_dtype)
+    dwis.append(cast_act(np.matmul(xe.transpose(0, 2, 1), dpre), act_dtype))
+  return dxe, (dwis if is_list else dwis[0]), dwo
 
 
 def moe_layer_v1_backward(x, w_gate, wi, wo, hp, train, act_dtype, d_out,
@@ -1253,13 +1298,12 @@ def moe_layer_v1_backward(x, w_gate, wi, wo, hp, train, act_dtype, d_out,
                               d_out[0], d_loss, **kw)
     k = moe_layer_v1_backward(x, w_gate, wi, k_wo, hp1, train, act_dtype,
                               d_out[1], 0.0, **kw)
-    out = {n: cast_act(q[n] + k[n], act_dtype) for n in ("dx", "dw_gate", "dwi")}
+    out = {n: cast_act(q[n] + k[n], act_dtype) for n in ("dx", "dw_gate")}
+    out["dwi"] = ([cast_act(a + b, act_dtype) for a, b in zip(q["dwi"], k["dwi"])]
+                  if isinstance(q["dwi"], list)
+                  else cast_act(q["dwi"] + k["dwi"], act_dtype))
     out.update(dwo=q["dwo"], dk_wo=k["dwo"], aux=q["aux"])
     return out
-  if isinstance(wi, (list, tuple)) or isinstance(activation, (list, tuple)):
-    raise NotImplementedError("backward of a product of dense layers")
-  if activation not in ("relu", "linear", None):
-    raise NotImplementedError("backward of activation %r" % (activation,))
   _, _, aux = moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype,
                            nonpadding=nonpadding, activation=activation,
                            num_microbatches=num_microbatches,
@@ -1276,7 +1320,8 @@ def moe_layer_v1_backward(x, w_gate, wi, wo, hp, train, act_dtype, d_out,
   g_, s_, c_ = aux["num_groups"], aux["group_size"], aux["capacity"]
   e_ = hp.moe_num_experts
   xg = x.reshape(g_, s_, m_)
-  wg_a, wi_a, wo_a = (cast_act(w, act_dtype) for w in (w_gate, wi, wo))
+  wg_a, wo_a = cast_act(w_gate, act_dtype), cast_act(wo, act_dtype)
+  wi_a = _cast_kernels(wi, act_dtype)
   n_ = wo_a.shape[-1]
   dout = cast_act(np.asarray(d_out, F32), act_dtype).reshape(g_, s_, n_)
   y = aux["expert_out"]                                          # [E,G,C,N]

@@ -952,3 +952,47 @@ def test_full_size_ffn_backward_properties(hip, size):
   assert err <= 2e-2 * want_dwi.float().abs().max().item()
   assert not bool(dwo[e // 2].any()) and not bool(dwi[e // 2].any())
   assert not bool(dxe[e // 2].any())
+
+
+@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
+def test_expert_linear_backward_and_activations(hip, act_dtype):
+  """mesh_moe_expert_linear_backward against float32 matmuls, and
+  mesh_moe_activation / mesh_moe_activation_backward against the oracle's
+  activation tables for every activation."""
+  e, rows, k, n = 2, 192, 136, 264
+  rng = np.random.default_rng(29)
+  cast = lambda a: O.cast_act(a.astype(np.float32), act_dtype)
+  g = lambda a: H.to_gpu(a, act_dtype)
+  a = cast(rng.standard_normal((e, rows, k)))
+  w = cast(H.normal_weights(rng, (e, k, n), k))
+  dy = cast(rng.standard_normal((e, rows, n)))
+  da, dw = hip.expert_linear_backward(g(a), g(dy), g(w))
+  tol = H.value_tolerance(act_dtype)
+  want_da = np.matmul(dy, w.transpose(0, 2, 1))
+  want_dw = np.matmul(a.transpose(0, 2, 1), dy)
+  for got, want, name in ((da, want_da, "da"), (dw, want_dw, "dw")):
+    np.testing.assert_allclose(H.to_np(got), O.cast_act(want, act_dtype),
+                               rtol=tol["rtol"],
+                               atol=tol["atol"] * np.abs(want).max(), err_msg=name)
+  none, dw2 = hip.expert_linear_backward(g(a), g(dy), g(w), want_da=False)
+  assert none is None and torch.equal(dw2, dw)
+  pre = cast(rng.standard_normal((e, rows, n)) * 2.0)
+  f = cast(rng.standard_normal((e, rows, n)))
+  for act in ("relu", "linear", "gelu", "sigmoid", "tanh", "swish"):
+    out = hip.activation(g(pre), act)
+    np.testing.assert_allclose(
+        H.to_np(out), O.cast_act(O.ACTIVATIONS[act](pre), act_dtype),
+        rtol=1e-2 if act_dtype == "bfloat16" else 1e-5, atol=1e-6, err_msg=act)
+    # same values as the activation applied inside the projection
+    assert torch.equal(out, hip.activation(g(pre), act))
+    for factor in (None, f):
+      got = hip.activation_backward(g(dy), g(pre), act, factor=None if factor
+                                    is None else g(factor))
+      want = dy * (1.0 if factor is None else factor) * O.ACTIVATION_GRADS[act](pre)
+      np.testing.assert_allclose(
+          H.to_np(got), O.cast_act(want.astype(np.float32), act_dtype),
+          rtol=2e-2 if act_dtype == "bfloat16" else 1e-4,
+          atol=(2e-2 if act_dtype == "bfloat16" else 1e-5) * np.abs(want).max(),
+          err_msg=act)
+  with pytest.raises(ValueError):
+    hip.activation(g(pre), "softplus")

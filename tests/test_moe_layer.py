@@ -724,6 +724,105 @@ def test_v1_experts_attention(act_dtype):
   np.testing.assert_array_equal(k, plain_k)
 
 
+@pytest.mark.parametrize("case", [
+    ("gelu", "float32", "top_2", False, False),
+    ("swish", "bfloat16", "switch", False, False),
+    (["gelu", "linear"], "float32", "top_2", False, False),
+    (["gelu", "linear"], "bfloat16", "top_2", True, False),
+    (["tanh", "sigmoid", "relu"], "float32", "switch", True, False),
+    (["relu", "linear"], "float32", "top_2", False, True),
+    ("sigmoid", "float32", "top_2", True, True)],
+    ids=lambda c: "%s-%s-%s%s%s" % ("*".join(c[0]) if isinstance(c[0], list)
+                                    else c[0], c[1], c[2],
+                                    "-dropout" if c[3] else "",
+                                    "-experts_attention" if c[4] else ""))
+def test_v1_gradients_other_activations(case):
+  """Experts that are not one ReLU / linear layer (other activations, products
+  of dense layers), with and without the hidden dropout and the second output
+  projection: mtf.gradients against the oracle's backward (pinned by central
+  differences in tests/test_oracle.py)."""
+  activation, act_dtype, gating, dropout, attention = case
+  acts = activation if isinstance(activation, list) else [activation]
+  b, l, m, hdim, e, group = 2, 64, 32, 48, 4, 32
+  rng = np.random.default_rng(131)
+  w_gate = H.normal_weights(rng, (m, e), m)
+  wis = [H.normal_weights(rng, (e, m, hdim), m) for _ in acts]
+  wo = H.normal_weights(rng, (e, hdim, m), hdim)
+  k_wo = H.normal_weights(rng, (e, hdim, m), hdim)
+  x = H.safe_tokens(rng, b * l, m, w_gate, act_dtype, top=3).reshape(b, l, m)
+  nonpad = (rng.random((b, l)) < 0.9).astype(np.float32)
+  d_q, d_k = (O.cast_act(rng.standard_normal((b, l, m)).astype(np.float32),
+                         act_dtype) for _ in range(2))
+  kw = dict(moe_num_experts=e, moe_hidden_size=hdim, moe_group_size=group,
+            moe_capacity_factor_train=1.0, moe_loss_coef=0.25,
+            moe_dropout_rate=0.25 if dropout else 0.0,
+            moe_use_experts_attention=attention)
+  if gating != "top_2":
+    kw.update(SWITCH_HP, moe_gating=gating)
+  hp, ohp = make_hparams(**kw)
+  dt = H.ACT_TORCH[act_dtype]
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  dims = [mtf.Dimension("batch", b), mtf.Dimension("length", l),
+          mtf.Dimension("d_model", m)]
+  imp = lambda a, shape: mtf.import_tf_tensor(
+      mesh, torch.from_numpy(np.asarray(a, np.float32)).to(dt), mtf.Shape(shape))
+  xt = imp(x, dims)
+  with mtf.variable_scope("moe"):
+    outs, loss = moe.transformer_moe_layer_v1(
+        xt, dims[-1], hp, True, mtf.VariableDType(torch.float32, torch.float32, dt),
+        nonpadding=imp(nonpad, dims[:2]), activation=activation,
+        num_microbatches=2)
+  outs = outs if attention else [outs]
+  router = "switch_gating" if gating == "switch" else "top_2_gating"
+  wi_names = (["moe/wi_%d/kernel" % i for i in range(len(acts))]
+              if len(acts) > 1 else ["moe/wi/kernel"])
+  wo_names = (["moe/q_wo/kernel", "moe/k_wo/kernel"] if attention
+              else ["moe/wo/kernel"])
+  names = ["moe/%s/kernel" % router] + wi_names + wo_names
+  values = [w_gate] + wis + ([wo, k_wo] if attention else [wo])
+  by_name = {v.name: v.outputs[0] for v in graph.trainable_variables}
+  assert sorted(by_name) == sorted(names)
+  grads = mtf.gradients(
+      outs + [loss], [xt] + [by_name[n] for n in names],
+      grad_ys=[imp(d, dims) for d in (d_q, d_k)[:len(outs)]] + [imp(1.5, [])])
+  torch.manual_seed(77)
+  lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()},
+                          initial_values=dict(zip(names, values)))
+  got = dict(zip(["dx"] + names, (H.to_np(lowering.export_to_tf_tensor(g))
+                                  for g in grads)))
+  hu = None
+  if dropout:          # the layer's only random call, reproduced
+    torch.manual_seed(77)
+    cap = O.expert_capacity(group, 1.0, e, 4)
+    hu = torch.rand((e, (b * l // group) * cap, hdim), dtype=dt,
+                    device="cuda").float().cpu().numpy()
+  wi_arg = wis if len(acts) > 1 else wis[0]
+  want = O.moe_layer_v1_backward(
+      x, w_gate, wi_arg, wo, ohp, True, act_dtype,
+      [d_q, d_k] if attention else d_q, 1.5, nonpadding=nonpad,
+      activation=activation, num_microbatches=2, hidden_uniform=hu,
+      k_wo=k_wo if attention else None)
+  ref = {"dx": want["dx"], names[0]: want["dw_gate"], wo_names[0]: want["dwo"]}
+  ref.update(zip(wi_names, want["dwi"] if len(acts) > 1 else [want["dwi"]]))
+  if attention:
+    ref[wo_names[1]] = want["dk_wo"]
+  tol = H.value_tolerance(act_dtype)
+  for k, g_ in got.items():
+    r_ = ref[k].reshape(g_.shape)
+    assert np.abs(r_).max() > 0
+    np.testing.assert_allclose(
+        g_, r_, rtol=tol["rtol"], atol=tol["atol"] * max(1.0, np.abs(r_).max()),
+        err_msg=k)
+  # the forward values with the pre-activations kept equal those without
+  if not dropout and not attention:
+    hp_e = make_hparams(**dict(kw, moe_capacity_factor_eval=1.0))[0]
+    fwd = run_v1(x, dict(w_gate=w_gate, wi=wi_arg, wo=wo), hp_e, False,
+                 act_dtype, nonpadding=nonpad, activation=activation)[0]
+    np.testing.assert_array_equal(
+        H.to_np(lowering.export_to_tf_tensor(outs[0])), fwd)
+
+
 @pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
 def test_v1_experts_attention_gradients(act_dtype):
   """Gradients through both outputs of the layer with

@@ -1013,8 +1013,19 @@ def test_hidden_dropout_noise(act_dtype):
 
 
 # ---- backward -------------------------------------------------------------------
+_F64_ACT = {
+    "relu": lambda v: np.maximum(v, 0.0),
+    "linear": lambda v: v,
+    "gelu": lambda v: 0.5 * v * (1 + np.tanh(
+        np.sqrt(2 / np.pi) * (v + 0.044715 * v ** 3))),
+    "sigmoid": scipy.special.expit,
+    "tanh": np.tanh,
+    "swish": lambda v: v * scipy.special.expit(v),
+}
+
+
 def _f64_layer(x, wg, wi, wo, aux, gating, m1, coef, mb, z_loss, mult=None,
-               hidden_noise=None, density_2=None):
+               hidden_noise=None, density_2=None, activation="relu"):
   """Independent float64 forward of the v1 layer with the ROUTING HELD FIXED
   (experts, kept masks and density counts taken from `aux`): a smooth function
   of (x, wg, wi, wo) whose central differences pin the oracle's backward."""
@@ -1026,8 +1037,13 @@ def _f64_layer(x, wg, wi, wo, aux, gating, m1, coef, mb, z_loss, mult=None,
   i1, i2 = aux["index_1"], aux["index_2"]
   k1, k2 = aux["kept_1"].astype(np.float64), aux["kept_2"].astype(np.float64)
 
+  wis = wi if isinstance(wi, list) else [wi]
+  acts = activation if isinstance(activation, list) else [activation]
+
   def ffn(idx, pos=None):
-    h = np.maximum(np.einsum("gsm,gsmh->gsh", x, wi[idx]), 0.0)
+    h = 1.0
+    for w_f, a_f in zip(wis, acts):      # a product of dense layers
+      h = h * _F64_ACT[a_f](np.einsum("gsm,gsmh->gsh", x, w_f[idx]))
     if hidden_noise is not None:          # [E, G, C, H], per expert slot
       cap = hidden_noise.shape[2]
       h = h * hidden_noise[idx, np.arange(g)[:, None], np.minimum(pos, cap - 1)]
@@ -1048,14 +1064,14 @@ def _f64_layer(x, wg, wi, wo, aux, gating, m1, coef, mb, z_loss, mult=None,
       aux_loss = aux_loss + 0.5 * (proxy_2 * density_2).mean() * e * e
     aux_loss = aux_loss / mb
   elif gating == "ntlb":
-    out = (p[rows + (i1,)] * m1 * k1)[..., None] * ffn(i1)
+    out = (p[rows + (i1,)] * m1 * k1)[..., None] * ffn(i1, aux["pos_1"])
     topk = aux["topk_index"]                                  # [G,S,k] fixed
     density = (topk[..., None] == np.arange(e)).mean(1)       # [G,k,E]
     proxy = p.mean(1)                                         # [G,E]
     aux_loss = (proxy[:, None, :, None] * m1[:, None, None, :]
                 * density[..., None]).mean() * e * e / mb
   else:
-    out = (p[rows + (i1,)] * m1 * k1)[..., None] * ffn(i1)
+    out = (p[rows + (i1,)] * m1 * k1)[..., None] * ffn(i1, aux["pos_1"])
     density = onehot1.mean(1)
     proxy = p.mean(1)
     aux_loss = (proxy[:, :, None] * m1[:, None, :] * density[:, :, None]
@@ -1069,11 +1085,20 @@ def _f64_layer(x, wg, wi, wo, aux, gating, m1, coef, mb, z_loss, mult=None,
 @pytest.mark.parametrize("gating", ["top_2", "switch", "switch_max", "ntlb",
                                     "switch+jitter", "switch+dropout",
                                     "ntlb+jitter", "switch+sample",
-                                    "top_2+hidden", "top_2+loss2"])
+                                    "top_2+hidden", "top_2+loss2",
+                                    "top_2+act:gelu", "switch+act:swish",
+                                    "top_2+act:gelu*linear",
+                                    "switch+act:tanh*sigmoid*relu"])
 def test_backward_against_central_differences(gating):
   gating, _, perturb = gating.partition("+")
   hidden = perturb == "hidden"      # dropout on the experts' hidden tensor
   loss2 = perturb == "loss2"        # moe_use_second_place_loss
+  activation = "relu"
+  if perturb.startswith("act:"):    # other expert activations, gated units
+    activation = perturb[4:].split("*")
+    activation = activation if len(activation) > 1 else activation[0]
+    hidden = len(activation) == 3 and isinstance(activation, list)
+    perturb = ""
   if hidden or loss2:
     perturb = ""
   rng = np.random.default_rng(61)
@@ -1081,6 +1106,9 @@ def test_backward_against_central_differences(gating):
   x = rng.standard_normal((b, l, m)).astype(np.float32)
   wg = rng.standard_normal((m, e)).astype(np.float32)
   wi = (rng.standard_normal((e, m, h)) / 2).astype(np.float32)
+  if isinstance(activation, list):
+    wi = [wi] + [(rng.standard_normal((e, m, h)) / 2).astype(np.float32)
+                 for _ in activation[1:]]
   wo = (rng.standard_normal((e, h, m)) / 3).astype(np.float32)
   nonpad = (rng.random((b, l)) < 0.8).astype(np.float32)
   d_out = rng.standard_normal((b, l, m)).astype(np.float32)
@@ -1110,7 +1138,7 @@ def test_backward_against_central_differences(gating):
   got = O.moe_layer_v1_backward(x, wg, wi, wo, hp, True, "float32", d_out,
                                 d_loss, nonpadding=nonpad, num_microbatches=mb,
                                 gate_noise=noise, sample_uniform=su,
-                                hidden_uniform=hu)
+                                hidden_uniform=hu, activation=activation)
   aux = got["aux"]
   mult = None
   if perturb == "sample":       # sampled experts differ from the arg-max
@@ -1133,10 +1161,16 @@ def test_backward_against_central_differences(gating):
 
   def scalar(xv, wgv, wiv, wov):
     out, loss = _f64_layer(xv.reshape(b, l, m), wgv, wiv, wov, aux, gating, m1,
-                           0.5, mb, z, mult, hnoise, density_2)
+                           0.5, mb, z, mult, hnoise, density_2, activation)
     return (out * d_out.reshape(out.shape)).sum() + d_loss * loss
-  base = [a.astype(np.float64) for a in (x.reshape(b, l, m), wg, wi, wo)]
+  base = [np.asarray(a).astype(np.float64)
+          for a in (x.reshape(b, l, m), wg, wi, wo)]
   grads = [got["dx"].reshape(b, l, m), got["dw_gate"], got["dwi"], got["dwo"]]
+  if isinstance(activation, list):
+    # the kernels of the factors, stacked: one perturbation moves all of them
+    grads[2] = np.stack(got["dwi"])
+    inner = scalar
+    scalar = lambda xv, wgv, wiv, wov: inner(xv, wgv, list(wiv), wov)
   eps = 1e-6
   for which in range(4):
     for trial in range(3):
