@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 12
+#define MESH_MOE_ABI_VERSION 13
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -369,6 +369,45 @@ int mesh_moe_slot_dispatch(const void* x, const int32_t* slot_token,
 int mesh_moe_slot_combine(const void* y, const int16_t* tok_slot,
                           const float* slot_weight, void* out, int G, int S,
                           int E, int C, int N, int dtype, void* stream);
+
+/*
+ * Backward of the per-slot record (expert-selection gating).  The reference
+ * gets these from mtf.gradients over the same einsums and over
+ * _expert_selection_gating (transformer/moe.py:443-447, :509-510, :1094-1147):
+ *
+ * mesh_moe_slot_combine_backward: dy[e,g,c,:] = w * dout[g, token of the slot,:]
+ *   with w the slot's combine weight as `dtype` holds it; dweight [G,E,C]
+ *   float32 = <dout[g,token,:], y[e,g,c,:]>.
+ * mesh_moe_slot_dispatch_backward: dx[g,s,:] = sum over the slots holding the
+ *   token of dexpert_in[e,g,c,:] (+ dlogits[g,s,:] . w_gate^T when dlogits and
+ *   w_gate_packed [E,M] are given), float32 accumulate, one rounding.
+ * mesh_moe_expert_choice_backward: d(logits) [G,S,E] float32 from dweight and
+ *   from the gradient of the returned loss (d_loss [1] float32 on the device,
+ *   loss_scale = moe_loss_coef): the softmax runs over the group's tokens per
+ *   expert, a chosen probability is divided by the number of experts that chose
+ *   the token (no gradient through that count), the loss goes through
+ *   agg = mean_e p * (importance == 1).
+ */
+int mesh_moe_slot_combine_backward(const void* dout, const void* y,
+                                   const int32_t* slot_token,
+                                   const float* slot_weight, void* dy,
+                                   float* dweight, int G, int S, int E, int C,
+                                   int N, int dtype, void* stream);
+int mesh_moe_slot_dispatch_backward(const void* dexpert_in,
+                                    const int16_t* tok_slot,
+                                    const float* dlogits,
+                                    const void* w_gate_packed, void* dx, int G,
+                                    int S, int E, int C, int M, int dtype,
+                                    void* stream);
+size_t mesh_moe_expert_choice_backward_workspace_bytes(int G, int S, int E);
+int mesh_moe_expert_choice_backward(const float* logits, const void* importance,
+                                    int importance_dtype,
+                                    const int16_t* tok_slot,
+                                    const float* dweight, const float* d_loss,
+                                    double loss_scale, int G, int S, int E,
+                                    int C, int normalize, int num_microbatches,
+                                    float* dlogits, void* workspace,
+                                    size_t workspace_bytes, void* stream);
 
 /*
  * ---------------------------------------------------------------------------

@@ -215,6 +215,196 @@ __global__ __launch_bounds__(256) void slot_combine_kernel(
   }
 }
 
+// ---------------------------------------------------------------------------
+// Backward.
+// ---------------------------------------------------------------------------
+
+// dy[e,g,c,:] = w * dout[g, slot_token[g,e,c], :] (w = the slot's combine weight
+// as the activation dtype holds it), dweight[g,e,c] = <dout[g,token,:],
+// y[e,g,c,:]> in float32.  One wavefront per slot.
+template <typename T>
+__global__ __launch_bounds__(256) void slot_combine_backward_kernel(
+    const T* __restrict__ dout, const T* __restrict__ y,
+    const int32_t* __restrict__ slot_token,
+    const float* __restrict__ slot_weight, T* __restrict__ dy,
+    float* __restrict__ dweight, int G, int S, int E, int C, int N,
+    int64_t n_slots) {
+  const int lane = threadIdx.x & 63;
+  const int64_t j = (int64_t)blockIdx.x * CH_ROWS + (threadIdx.x >> 6);
+  if (j >= n_slots) return;
+  // j enumerates [E,G,C] (the layout of y and dy)
+  const int c = (int)(j % C);
+  const int g = (int)((j / C) % G);
+  const int e = (int)(j / ((int64_t)C * G));
+  const int64_t slot = ((int64_t)g * E + e) * C + c;
+  const float w = round_to<T>(slot_weight[slot]);
+  const T* drow = dout + ((int64_t)g * S + slot_token[slot]) * N;
+  const T* yrow = y + j * N;
+  T* dst = dy + j * N;
+  float dot = 0.f;
+  for (int i = lane; i < N; i += 64) {
+    const float d = load_f32<T>(drow + i);
+    dot += d * load_f32<T>(yrow + i);
+    store_f32<T>(dst + i, w * d);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
+  if (lane == 0) dweight[slot] = dot;
+}
+
+// dx[g,s,:] = sum over the experts that chose the token of dexpert_in[e,g,c,:]
+// (+ dlogits[g,s,:] . w_gate^T when the router's share is wanted), float32
+// accumulate in expert order, one rounding.  One wavefront per token.
+template <typename T>
+__global__ __launch_bounds__(256) void slot_dispatch_backward_kernel(
+    const T* __restrict__ dxe, const int16_t* __restrict__ tok_slot,
+    const float* __restrict__ dlogits, const T* __restrict__ wgp,
+    T* __restrict__ dx, int G, int S, int E, int C, int M, int64_t T_tokens) {
+  const int lane = threadIdx.x & 63;
+  const int64_t t = (int64_t)blockIdx.x * CH_ROWS + (threadIdx.x >> 6);
+  if (t >= T_tokens) return;
+  const int g = (int)(t / S);
+  const int16_t* ts = tok_slot + t * E;
+  const float* dl = dlogits ? dlogits + t * E : nullptr;
+  T* dst = dx + t * M;
+  for (int i0 = 0; i0 < M; i0 += 64 * 4) {
+    float acc[4] = {0.f, 0.f, 0.f, 0.f};
+    for (int e = 0; e < E; ++e) {
+      const int c = ts[e];
+      if (c >= 0) {
+        const T* row = dxe + (((int64_t)e * G + g) * C + c) * M;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int i = i0 + u * 64 + lane;
+          if (i < M) acc[u] += load_f32<T>(row + i);
+        }
+      }
+    }
+    if (dl != nullptr) {
+      for (int e = 0; e < E; ++e) {
+        const float d = dl[e];
+        const T* row = wgp + (int64_t)e * M;
+#pragma unroll
+        for (int u = 0; u < 4; ++u) {
+          const int i = i0 + u * 64 + lane;
+          if (i < M) acc[u] = fmaf(d, load_f32<T>(row + i), acc[u]);
+        }
+      }
+    }
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+      const int i = i0 + u * 64 + lane;
+      if (i < M) store_f32<T>(dst + i, acc[u]);
+    }
+  }
+}
+
+// log-sum-exp over the group's tokens of every (group, expert) column, as the
+// forward pass computes it.  One block per (expert, group).
+template <typename IT>
+__global__ __launch_bounds__(256) void choice_lse_kernel(
+    ChoiceParams p, const float* __restrict__ logits,
+    const IT* __restrict__ importance, float* __restrict__ lse_out) {
+  __shared__ float red[4];
+  const int e = blockIdx.x, g = blockIdx.y;
+  const int S = p.S, E = p.E;
+  const int64_t base = (int64_t)g * S;
+  auto value = [&](int s) {
+    float x = logits[(base + s) * E + e];
+    if (importance != nullptr && load_f32<IT>(importance + base + s) == 0.0f)
+      x = x + (-1e9f);
+    return x;
+  };
+  float m = -INFINITY;
+  for (int s = threadIdx.x; s < S; s += 256) m = fmaxf(m, value(s));
+  m = block_reduce(m, red, true);
+  const float negm = -m;
+  float sum = 0.f;
+  for (int s = threadIdx.x; s < S; s += 256) sum += expf(value(s) + negm);
+  sum = block_reduce(sum, red, false);
+  if (threadIdx.x == 0) lse_out[(int64_t)g * E + e] = logf(sum) + m;
+}
+
+// One block per group: per token 1 / max(#experts that chose it, 1) and the
+// loss's share of d(p[g,s,e]) (the same for every e):
+// d_loss * 2 * agg * sum_s(importance) * (importance == 1) / (E * G * mb).
+template <typename IT>
+__global__ __launch_bounds__(256) void choice_backward_token_kernel(
+    ChoiceParams p, const float* __restrict__ logits,
+    const IT* __restrict__ importance, const float* __restrict__ lse,
+    const int16_t* __restrict__ tok_slot, const float* __restrict__ d_loss,
+    float loss_scale, float* __restrict__ recip_out,
+    float* __restrict__ dloss_out) {
+  __shared__ float red[4];
+  const int g = blockIdx.x;
+  const int S = p.S, E = p.E;
+  const int64_t base = (int64_t)g * S;
+  const float inv_e = (float)(1.0 / (double)E);
+  float imp_sum = 0.f;
+  for (int s = threadIdx.x; s < S; s += 256)
+    imp_sum += importance != nullptr ? load_f32<IT>(importance + base + s) : 1.0f;
+  imp_sum = block_reduce(imp_sum, red, false);
+  const float mb =
+      p.num_microbatches > 1 ? (float)(1.0 / (double)p.num_microbatches) : 1.0f;
+  const float coef = d_loss[0] * loss_scale * mb * (float)(2.0 / (double)p.G) *
+                     imp_sum * inv_e;
+  for (int s = threadIdx.x; s < S; s += 256) {
+    const int64_t t = base + s;
+    float imp = 1.0f;
+    if (importance != nullptr) imp = load_f32<IT>(importance + t);
+    float agg = 0.f;
+    int routed = 0;
+    for (int e = 0; e < E; ++e) {
+      float x = logits[t * E + e];
+      if (imp == 0.0f) x = x + (-1e9f);
+      agg += expf(x + (-lse[(int64_t)g * E + e]));
+      routed += tok_slot[t * E + e] >= 0 ? 1 : 0;
+    }
+    const float is_one = imp == 1.0f ? 1.0f : 0.0f;
+    agg = (agg * inv_e) * is_one;
+    recip_out[t] = p.normalize ? 1.0f / fmaxf((float)routed, 1.0f) : 1.0f;
+    dloss_out[t] = coef * agg * is_one;
+  }
+}
+
+// One block per (expert, group): d(logits[g,:,e]) = p * (dp - sum_s p * dp),
+// dp = dweight[slot] / #experts of the token (chosen tokens) + the loss's share.
+template <typename IT>
+__global__ __launch_bounds__(256) void choice_backward_column_kernel(
+    ChoiceParams p, const float* __restrict__ logits,
+    const IT* __restrict__ importance, const float* __restrict__ lse,
+    const int16_t* __restrict__ tok_slot, const float* __restrict__ dweight,
+    const float* __restrict__ recip, const float* __restrict__ dloss_tok,
+    float* __restrict__ dlogits) {
+  __shared__ float red[4];
+  const int e = blockIdx.x, g = blockIdx.y;
+  const int S = p.S, E = p.E, C = p.C;
+  const int64_t base = (int64_t)g * S;
+  const float neglse = -lse[(int64_t)g * E + e];
+  auto prob_and_dp = [&](int s, float& dp) {
+    const int64_t t = base + s;
+    float x = logits[t * E + e];
+    if (importance != nullptr && load_f32<IT>(importance + t) == 0.0f)
+      x = x + (-1e9f);
+    dp = dloss_tok[t];
+    const int c = tok_slot[t * E + e];
+    if (c >= 0) dp += dweight[((int64_t)g * E + e) * C + c] * recip[t];
+    return expf(x + neglse);
+  };
+  float inner = 0.f;
+  for (int s = threadIdx.x; s < S; s += 256) {
+    float dp;
+    const float ps = prob_and_dp(s, dp);
+    inner += ps * dp;
+  }
+  inner = block_reduce(inner, red, false);
+  for (int s = threadIdx.x; s < S; s += 256) {
+    float dp;
+    const float ps = prob_and_dp(s, dp);
+    dlogits[(base + s) * E + e] = ps * (dp - inner);
+  }
+}
+
 }  // namespace mesh_moe
 
 using namespace mesh_moe;
@@ -346,5 +536,126 @@ extern "C" int mesh_moe_slot_combine(const void* y, const int16_t* tok_slot,
         (const bf16_t*)y, tok_slot, slot_weight, (bf16_t*)out, G, S, E, C, N,
         T_tokens);
   MOE_CHECK_LAUNCH("slot_combine");
+  return 0;
+}
+
+extern "C" int mesh_moe_slot_combine_backward(
+    const void* dout, const void* y, const int32_t* slot_token,
+    const float* slot_weight, void* dy, float* dweight, int G, int S, int E,
+    int C, int N, int dtype, void* stream) {
+  MOE_REQUIRE(dout && y && slot_token && slot_weight && dy && dweight,
+              MESH_MOE_E_ARG, "slot_combine_backward: null pointer");
+  MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG,
+              "slot_combine_backward: bad dtype %d", dtype);
+  MOE_REQUIRE(G >= 1 && S >= 1 && E >= 1 && C >= 1 && N >= 1, MESH_MOE_E_ARG,
+              "slot_combine_backward: bad sizes G=%d S=%d E=%d C=%d N=%d", G, S,
+              E, C, N);
+  const int64_t n_slots = (int64_t)G * E * C;
+  const int64_t nblocks = (n_slots + CH_ROWS - 1) / CH_ROWS;
+  MOE_REQUIRE(nblocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
+              "slot_combine_backward: too many slots (%lld)",
+              (long long)n_slots);
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == MESH_MOE_F32)
+    slot_combine_backward_kernel<float><<<(unsigned)nblocks, 256, 0, st>>>(
+        (const float*)dout, (const float*)y, slot_token, slot_weight,
+        (float*)dy, dweight, G, S, E, C, N, n_slots);
+  else
+    slot_combine_backward_kernel<bf16_t><<<(unsigned)nblocks, 256, 0, st>>>(
+        (const bf16_t*)dout, (const bf16_t*)y, slot_token, slot_weight,
+        (bf16_t*)dy, dweight, G, S, E, C, N, n_slots);
+  MOE_CHECK_LAUNCH("slot_combine_backward");
+  return 0;
+}
+
+extern "C" int mesh_moe_slot_dispatch_backward(
+    const void* dexpert_in, const int16_t* tok_slot, const float* dlogits,
+    const void* w_gate_packed, void* dx, int G, int S, int E, int C, int M,
+    int dtype, void* stream) {
+  MOE_REQUIRE(dexpert_in && tok_slot && dx, MESH_MOE_E_ARG,
+              "slot_dispatch_backward: null pointer");
+  MOE_REQUIRE((dlogits == nullptr) == (w_gate_packed == nullptr),
+              MESH_MOE_E_ARG,
+              "slot_dispatch_backward: dlogits and w_gate_packed go together");
+  MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG,
+              "slot_dispatch_backward: bad dtype %d", dtype);
+  MOE_REQUIRE(G >= 1 && S >= 1 && E >= 1 && C >= 1 && M >= 1, MESH_MOE_E_ARG,
+              "slot_dispatch_backward: bad sizes G=%d S=%d E=%d C=%d M=%d", G,
+              S, E, C, M);
+  const int64_t T_tokens = (int64_t)G * S;
+  const int64_t nblocks = (T_tokens + CH_ROWS - 1) / CH_ROWS;
+  MOE_REQUIRE(nblocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
+              "slot_dispatch_backward: too many rows (%lld)",
+              (long long)T_tokens);
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == MESH_MOE_F32)
+    slot_dispatch_backward_kernel<float><<<(unsigned)nblocks, 256, 0, st>>>(
+        (const float*)dexpert_in, tok_slot, dlogits,
+        (const float*)w_gate_packed, (float*)dx, G, S, E, C, M, T_tokens);
+  else
+    slot_dispatch_backward_kernel<bf16_t><<<(unsigned)nblocks, 256, 0, st>>>(
+        (const bf16_t*)dexpert_in, tok_slot, dlogits,
+        (const bf16_t*)w_gate_packed, (bf16_t*)dx, G, S, E, C, M, T_tokens);
+  MOE_CHECK_LAUNCH("slot_dispatch_backward");
+  return 0;
+}
+
+extern "C" size_t mesh_moe_expert_choice_backward_workspace_bytes(int G, int S,
+                                                                  int E) {
+  if (G < 1 || S < 1 || E < 1) return 0;
+  return sizeof(float) * ((size_t)G * E + 2 * (size_t)G * S) + 3 * 256;
+}
+
+extern "C" int mesh_moe_expert_choice_backward(
+    const float* logits, const void* importance, int importance_dtype,
+    const int16_t* tok_slot, const float* dweight, const float* d_loss,
+    double loss_scale, int G, int S, int E, int C, int normalize,
+    int num_microbatches, float* dlogits, void* workspace,
+    size_t workspace_bytes, void* stream) {
+  MOE_REQUIRE(logits && tok_slot && dweight && d_loss && dlogits && workspace,
+              MESH_MOE_E_ARG, "expert_choice_backward: null pointer");
+  MOE_REQUIRE(G >= 1 && S >= 1 && E >= 1 && C >= 1 && C <= S, MESH_MOE_E_ARG,
+              "expert_choice_backward: bad sizes G=%d S=%d E=%d C=%d", G, S, E,
+              C);
+  MOE_REQUIRE(E <= 65535 && G <= 65535, MESH_MOE_E_UNSUPPORTED,
+              "expert_choice_backward: E or G > 65535");
+  MOE_REQUIRE(!importance || valid_dtype(importance_dtype), MESH_MOE_E_ARG,
+              "expert_choice_backward: bad importance dtype %d",
+              importance_dtype);
+  MOE_REQUIRE(workspace_bytes >=
+                  mesh_moe_expert_choice_backward_workspace_bytes(G, S, E),
+              MESH_MOE_E_ARG, "expert_choice_backward: workspace too small");
+  ChoiceParams p;
+  p.G = G; p.S = S; p.E = E; p.C = C;
+  p.normalize = normalize ? 1 : 0;
+  p.num_microbatches = num_microbatches;
+  auto up = [](uintptr_t v) { return (v + 255) & ~(uintptr_t)255; };
+  float* lse = (float*)up((uintptr_t)workspace);
+  float* recip = (float*)up((uintptr_t)(lse + (size_t)G * E));
+  float* dloss_tok = (float*)up((uintptr_t)(recip + (size_t)G * S));
+  hipStream_t st = (hipStream_t)stream;
+  dim3 grid((unsigned)E, (unsigned)G);
+  if (importance && importance_dtype == MESH_MOE_BF16) {
+    const bf16_t* imp = (const bf16_t*)importance;
+    choice_lse_kernel<bf16_t><<<grid, 256, 0, st>>>(p, logits, imp, lse);
+    MOE_CHECK_LAUNCH("expert_choice_backward (lse)");
+    choice_backward_token_kernel<bf16_t><<<G, 256, 0, st>>>(
+        p, logits, imp, lse, tok_slot, d_loss, (float)loss_scale, recip,
+        dloss_tok);
+    MOE_CHECK_LAUNCH("expert_choice_backward (tokens)");
+    choice_backward_column_kernel<bf16_t><<<grid, 256, 0, st>>>(
+        p, logits, imp, lse, tok_slot, dweight, recip, dloss_tok, dlogits);
+  } else {
+    const float* imp = (const float*)importance;
+    choice_lse_kernel<float><<<grid, 256, 0, st>>>(p, logits, imp, lse);
+    MOE_CHECK_LAUNCH("expert_choice_backward (lse)");
+    choice_backward_token_kernel<float><<<G, 256, 0, st>>>(
+        p, logits, imp, lse, tok_slot, d_loss, (float)loss_scale, recip,
+        dloss_tok);
+    MOE_CHECK_LAUNCH("expert_choice_backward (tokens)");
+    choice_backward_column_kernel<float><<<grid, 256, 0, st>>>(
+        p, logits, imp, lse, tok_slot, dweight, recip, dloss_tok, dlogits);
+  }
+  MOE_CHECK_LAUNCH("expert_choice_backward (columns)");
   return 0;
 }

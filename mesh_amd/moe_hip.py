@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 12
+ABI_VERSION = 13
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -104,6 +104,18 @@ _SIGNATURES = {
         _vp, _vp, ctypes.c_int64, ctypes.c_int, ctypes.c_int, _vp]),
     "mesh_moe_activation_backward": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, ctypes.c_int64, ctypes.c_int, ctypes.c_int, _vp]),
+    "mesh_moe_slot_combine_backward": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
+    "mesh_moe_slot_dispatch_backward": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
+    "mesh_moe_expert_choice_backward_workspace_bytes": (ctypes.c_size_t, [
+        ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "mesh_moe_expert_choice_backward": (ctypes.c_int, [
+        _vp, _vp, ctypes.c_int, _vp, _vp, _vp, ctypes.c_double, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        _vp, _vp, ctypes.c_size_t, _vp]),
     "mesh_moe_gating_backward_workspace_bytes": (ctypes.c_size_t, [
         ctypes.c_int, ctypes.c_int]),
     "mesh_moe_gating_backward": (ctypes.c_int, [
@@ -976,3 +988,70 @@ def self_attention(q, k, v, num_heads, causal):
         int(bool(causal)), code, ws.data_ptr(), ws_bytes, _stream()),
         "self_attention")
   return out
+
+
+def slot_combine_backward(dout, y, r):
+  """dout [G,S,N], y [E,G,C,N], r a SlotRouting -> (dy [E,G,C,N],
+  dweight [G,E,C] float32)."""
+  lib = load_library()
+  e, g, c, n = y.shape
+  s = dout.shape[1]
+  dt = y.dtype
+  dy = torch.empty_like(y)
+  dweight = torch.empty((g, e, c), dtype=torch.float32, device=y.device)
+  with _stage("slot_combine_backward"):
+    _check(lib.mesh_moe_slot_combine_backward(
+        _dev(dout, "dout", dt, (g, s, n)), _dev(y, "y"),
+        _dev(r.slot_token, "slot_token", torch.int32, (g, e, c)),
+        _dev(r.slot_weight, "slot_weight", torch.float32, (g, e, c)),
+        dy.data_ptr(), dweight.data_ptr(), g, s, e, c, n, dtype_code(dt),
+        _stream()), "slot_combine_backward")
+  return dy, dweight
+
+
+def slot_dispatch_backward(dxe, r, group_size, dlogits=None,
+                           w_gate_packed=None):
+  """dxe [E,G,C,M] -> dx [G,S,M]; with dlogits [G,S,E] float32 and the packed
+  router kernel [E,M] the router's share is added."""
+  lib = load_library()
+  e, g, c, m = dxe.shape
+  s = group_size
+  dt = dxe.dtype
+  dx = torch.empty((g, s, m), dtype=dt, device=dxe.device)
+  with _stage("slot_dispatch_backward"):
+    _check(lib.mesh_moe_slot_dispatch_backward(
+        _dev(dxe, "dxe"),
+        _dev(r.tok_slot, "tok_slot", torch.int16, (g, s, e)),
+        _dev(dlogits, "dlogits", torch.float32, (g, s, e))
+        if dlogits is not None else None,
+        _dev(w_gate_packed, "w_gate_packed", dt, (e, m))
+        if w_gate_packed is not None else None,
+        dx.data_ptr(), g, s, e, c, m, dtype_code(dt), _stream()),
+        "slot_dispatch_backward")
+  return dx
+
+
+def expert_choice_backward(logits, r, dweight, d_loss, loss_scale,
+                           importance=None, normalize=True,
+                           num_microbatches=None):
+  """d(logits) [G,S,E] float32 of expert_choice_gating."""
+  lib = load_library()
+  g, s, e = logits.shape
+  c = r.capacity
+  ip, icode = None, F32
+  if importance is not None:
+    icode = dtype_code(importance.dtype)
+    ip = _dev(importance, "importance", None, (g, s))
+  dlogits = torch.empty((g, s, e), dtype=torch.float32, device=logits.device)
+  ws_bytes = lib.mesh_moe_expert_choice_backward_workspace_bytes(g, s, e)
+  ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=logits.device)
+  with _stage("expert_choice_backward"):
+    _check(lib.mesh_moe_expert_choice_backward(
+        _dev(logits, "logits", torch.float32), ip, icode,
+        _dev(r.tok_slot, "tok_slot", torch.int16, (g, s, e)),
+        _dev(dweight, "dweight", torch.float32, (g, e, c)),
+        _dev(d_loss, "d_loss", torch.float32, (1,)), float(loss_scale), g, s, e,
+        c, int(bool(normalize)), int(num_microbatches or 1),
+        dlogits.data_ptr(), ws.data_ptr(), ws_bytes, _stream()),
+        "expert_choice_backward")
+  return dlogits

@@ -406,9 +406,6 @@ class MoEV1Operation(mtf.Operation):
     """Gradients w.r.t. (inputs, gate kernel, wi, wo[, importance][, k_wo])
     from those of (outputs, loss[, second outputs]); importance carries
     none."""
-    if self._gating.router == "expert_selection":
-      raise NotImplementedError(
-          "backward of expert_selection gating is not implemented")
     self._save_for_backward = True
     d_out, d_loss = grad_ys[:2]
     if d_out is None:
@@ -603,13 +600,16 @@ class MoEV1GradOperation(mtf.Operation):
         raise ValueError("the forward operation kept no activations: build "
                          "the gradient before lowering the graph")
       r = sv["routing"]
-      dy, dgate = moe_hip.combine_backward(
+      by_slot = isinstance(r, moe_hip.SlotRouting)
+      combine_backward = (moe_hip.slot_combine_backward if by_slot
+                          else moe_hip.combine_backward)
+      dy, dgate = combine_backward(
           dout_s.reshape(groups, s_, n_).contiguous(),
           sv["y"].reshape(e_, groups, c_, n_), r)
       if fwd._general_hidden:
         dys, wos = [dy.reshape(e_, groups * c_, n_)], [wo_s]
         if has_k:
-          dyk, dgate_k = moe_hip.combine_backward(
+          dyk, dgate_k = combine_backward(
               dk_s.reshape(groups, s_, n_).contiguous(),
               sv["yk"].reshape(e_, groups, c_, n_), r)
           dys.append(dyk.reshape(e_, groups * c_, n_))
@@ -630,7 +630,7 @@ class MoEV1GradOperation(mtf.Operation):
         # the second projection of the same hidden tensor: its share of every
         # gradient adds to the first one's (the hidden tensor and the combine
         # weights have two consumers)
-        dyk, dgate_k = moe_hip.combine_backward(
+        dyk, dgate_k = combine_backward(
             dk_s.reshape(groups, s_, n_).contiguous(),
             sv["yk"].reshape(e_, groups, c_, n_), r)
         dxe_k, dwi_k, dkwo = moe_hip.expert_ffn_backward(
@@ -638,17 +638,25 @@ class MoEV1GradOperation(mtf.Operation):
             dyk.reshape(e_, groups * c_, n_), wi_s, kwo_s, fwd._activation,
             dh_scale=sv["hidden_noise"])
         dxe, dwi, dgate = dxe + dxe_k, dwi + dwi_k, dgate + dgate_k
-      dlogits = moe_hip.gating_backward(
-          sv["logits"], r, dgate, dloss_s.reshape(1).float(), 1.0,
-          router=gating.router, top_k=getattr(gating, "top_k", 0),
-          importance=sv["importance"], z_loss=gating.z_loss,
-          num_microbatches=gating.num_microbatches,
-          use_second_place_loss=gating.use_second_place_loss)
+      if by_slot:
+        dlogits = moe_hip.expert_choice_backward(
+            sv["logits"], r, dgate, dloss_s.reshape(1).float(), 1.0,
+            importance=sv["importance"],
+            num_microbatches=gating.num_microbatches)
+        dispatch_backward = moe_hip.slot_dispatch_backward
+      else:
+        dlogits = moe_hip.gating_backward(
+            sv["logits"], r, dgate, dloss_s.reshape(1).float(), 1.0,
+            router=gating.router, top_k=getattr(gating, "top_k", 0),
+            importance=sv["importance"], z_loss=gating.z_loss,
+            num_microbatches=gating.num_microbatches,
+            use_second_place_loss=gating.use_second_place_loss)
+        dispatch_backward = moe_hip.dispatch_backward
       tokens = groups * s_
       if sv["gate_in"] is None:
         dwg = moe_hip.router_backward_weights(
             sv["x"].reshape(tokens, m_), dlogits.reshape(tokens, e_))
-        dx = moe_hip.dispatch_backward(
+        dx = dispatch_backward(
             dxe.reshape(e_, groups, c_, m_), r, s_, dlogits,
             sv["w_gate_packed"].reshape(e_, m_))
       else:
@@ -660,7 +668,7 @@ class MoEV1GradOperation(mtf.Operation):
         dwg = moe_hip.router_backward_weights(
             x_gate.reshape(tokens, m_).contiguous(),
             dlogits.reshape(tokens, e_)).to(dt)
-        dx = moe_hip.dispatch_backward(dxe.reshape(e_, groups, c_, m_), r, s_)
+        dx = dispatch_backward(dxe.reshape(e_, groups, c_, m_), r, s_)
         w32 = sv["w_gate"].reshape(1, m_, e_).to(torch.float32).contiguous()
         dx_router = moe_hip.expert_linear(
             dlogits.reshape(1, tokens, e_), w32, "linear")   # [1, T, M]

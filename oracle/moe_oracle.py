@@ -57,8 +57,10 @@ MoE file, and its TensorFlow dependency cannot run here):
   gating_backward,                    central differences of an independent
   moe_layer_v1_backward               float64 forward with the routing held
                                       fixed (tests/test_oracle.py), every
-                                      router, the second-place loss, the
-                                      noise policies and the hidden dropout
+                                      router (expert selection included), the
+                                      second-place loss, the noise policies,
+                                      the hidden dropout, other activations
+                                      and products of dense layers
   v2                                  x=1 outer expert reduces to v1
 
 PARITY UNPINNED against TensorFlow itself (only running the reference could
@@ -1008,7 +1010,7 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
     else:
       out = slot_combine(y, r, s_, act_dtype)
     aux = dict(r, logits=logits, expert_in=expert_in, expert_out=y,
-               num_groups=g_, group_size=s_, capacity=c_)
+               num_groups=g_, group_size=s_, capacity=c_, gate_mult=gate_mult)
     return (out.reshape(lead + (n_,)),
             _scale_loss(r["loss"], hp.moe_loss_coef, act_dtype), aux)
   if hp.moe_gating in ("switch", "switch_max", "ntlb"):          # :393-424
@@ -1164,6 +1166,70 @@ def gating_backward(logits, r, gating, d_gate_1, d_gate_2, d_loss,
     dlogits = dlogits + ((d_loss * F32(z_loss) * F32(2.0)) * lse * m1
                          / denom)[..., None] * p
   return dlogits.astype(F32)
+
+
+def expert_selection_gating_backward(logits, r, importance, d_slot_weight,
+                                     d_loss, num_microbatches=None,
+                                     normalize_by_num_experts_routed=True):
+  """d(logits) of _expert_selection_gating (moe.py:1094-1147).
+
+  The probabilities are a softmax over the GROUP's tokens, one column per
+  expert.  A slot's combine weight is the probability it was chosen with over
+  max(#experts that chose the token, 1); top_k routes the gradient of a chosen
+  value to its entry (ops.py:4916-4920, :5009-5015), the count comes from
+  one-hot tensors and has no gradient.  The loss mean(agg^2 * sum(importance))
+  * S with agg = mean_e p * (importance == 1) differentiates through agg.
+
+  d_slot_weight [G,E,C]: gradient w.r.t. the float32 combine weight of each
+  slot; d_loss: gradient w.r.t. the loss before moe_loss_coef.  Returns float32
+  [G,S,E].
+  """
+  logits = np.asarray(logits, dtype=F32)
+  g_, s_, e_ = logits.shape
+  importance = np.asarray(importance, dtype=F32)
+  masked = logits + ((importance == F32(0.0)).astype(F32) * F32(-1e9))[..., None]
+  p = np.moveaxis(softmax(np.moveaxis(masked, 1, -1)), -1, 1)    # [G,S,E]
+  tok = r["slot_token"]                                          # [G,E,C]
+  gi = np.arange(g_)[:, None, None]
+  ei = np.arange(e_)[None, :, None]
+  recip = np.ones((g_, s_), F32)
+  if normalize_by_num_experts_routed:
+    num_routed = np.zeros((g_, s_), F32)
+    np.add.at(num_routed, (np.broadcast_to(gi, tok.shape), tok), F32(1.0))
+    recip = (F32(1.0) / np.maximum(num_routed, F32(1.0))).astype(F32)
+  dp = np.zeros_like(p)
+  dp[gi, tok, ei] = np.asarray(d_slot_weight, F32) * recip[gi, tok]
+  is_one = (importance == F32(1.0)).astype(F32)
+  agg = p.sum(-1, dtype=F32) * F32(1.0 / e_) * is_one
+  tgs = importance.sum(-1, dtype=F32)                            # [G]
+  mb = F32(1.0 / num_microbatches) if (num_microbatches and
+                                       num_microbatches > 1) else F32(1.0)
+  dagg = F32(d_loss) * mb * F32(2.0 / g_) * agg * tgs[:, None]
+  dp += (dagg * is_one * F32(1.0 / e_))[..., None]
+  return (p * (dp - (p * dp).sum(1, keepdims=True))).astype(F32)
+
+
+def slot_combine_backward(dout, y, r, act_dtype):
+  """Backward of the combine einsum for a per-slot record: dy [E,G,C,N] =
+  w * dout[token of the slot] (activation dtype), d_slot_weight [G,E,C] =
+  <dout[token], y[slot]> (float32)."""
+  e_, g_, c_, _ = y.shape
+  w = cast_act(r["slot_weight"], act_dtype)                      # [G,E,C]
+  rows = dout[np.arange(g_)[:, None, None], r["slot_token"]]     # [G,E,C,N]
+  dy = cast_act(w[..., None] * rows, act_dtype).transpose(1, 0, 2, 3)
+  dw = (rows * y.transpose(1, 0, 2, 3)).sum(-1, dtype=F32)
+  return dy, dw
+
+
+def slot_dispatch_backward(dxe, r, group_size):
+  """Backward of the dispatch einsum for a per-slot record: a token gathers
+  the rows of all slots that hold it.  dxe [E,G,C,M] -> float32 [G,S,M]."""
+  e_, g_, c_, m_ = dxe.shape
+  dx = np.zeros((g_, group_size, m_), F32)
+  for g in range(g_):
+    for e in range(e_):
+      np.add.at(dx[g], r["slot_token"][g, e], dxe[e, g].astype(F32))
+  return dx
 
 
 def combine_backward(dout, y, r, act_dtype):
@@ -1327,12 +1393,19 @@ def moe_layer_v1_backward(x, w_gate, wi, wo, hp, train, act_dtype, d_out,
   y = aux["expert_out"]                                          # [E,G,C,N]
   expert_in = aux["expert_in"]                                   # [E,G,C,M]
 
-  dy, dgate = combine_backward(dout, y, aux, act_dtype)
+  by_slot = hp.moe_gating == "expert_selection"
+  if by_slot:
+    dy, dgate = slot_combine_backward(dout, y, aux, act_dtype)
+  else:
+    dy, dgate = combine_backward(dout, y, aux, act_dtype)
   r_ = g_ * c_
   dxe, dwi, dwo = expert_ffn_backward(
       expert_in.reshape(e_, r_, m_), wi_a, wo_a, dy.reshape(e_, r_, n_),
       activation, act_dtype, hidden_noise)
-  dx = dispatch_backward(dxe.reshape(e_, g_, c_, m_), aux, act_dtype)
+  if by_slot:
+    dx = slot_dispatch_backward(dxe.reshape(e_, g_, c_, m_), aux, s_)
+  else:
+    dx = dispatch_backward(dxe.reshape(e_, g_, c_, m_), aux, act_dtype)
 
   # gating and router backward
   importance = None
@@ -1343,9 +1416,13 @@ def moe_layer_v1_backward(x, w_gate, wi, wo, hp, train, act_dtype, d_out,
   # the returned loss is aux * moe_loss_coef in the activation dtype
   d_aux = F32(cast_act(F32(d_loss), act_dtype)
               * cast_act(F32(hp.moe_loss_coef), act_dtype))
-  dlogits = gating_backward(aux["logits"], aux, hp.moe_gating, dgate[..., 0],
-                            dgate[..., 1], d_aux, importance, num_microbatches,
-                            z, hp.moe_use_second_place_loss)
+  if by_slot:
+    dlogits = expert_selection_gating_backward(
+        aux["logits"], aux, importance, dgate, d_aux, num_microbatches)
+  else:
+    dlogits = gating_backward(aux["logits"], aux, hp.moe_gating, dgate[..., 0],
+                              dgate[..., 1], d_aux, importance,
+                              num_microbatches, z, hp.moe_use_second_place_loss)
   # the router saw the perturbed inputs x * mult (perturb_gate_inputs); the
   # multiplier is a constant of the graph
   mult = aux.get("gate_mult")

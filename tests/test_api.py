@@ -389,17 +389,6 @@ def test_gradients_builds_the_backward_operation():
   fwd = [o for o in graph.operations if isinstance(o, moe.MoEV1Operation)][0]
   assert fwd._save_for_backward
   assert any(isinstance(o, moe.MoEV1GradOperation) for o in graph.operations)
-  with pytest.raises(NotImplementedError, match="expert_selection"):
-    g2, _, x2, d2 = graph_input()
-    np2 = mtf.import_tf_tensor(g2.meshes[0] if hasattr(g2, "meshes") else x2.mesh,
-                               torch.ones(x2.shape.to_integer_list[:-1]),
-                               mtf.Shape(d2[:-1]))
-    y2, l2 = moe.transformer_moe_layer_v1(
-        x2, d2[-1], hparams(moe_gating="expert_selection",
-                            moe_switch_policy_train="argmax",
-                            moe_switch_policy_eval="argmax"), True,
-        mtf.VariableDType(torch.float32), nonpadding=np2)
-    mtf.gradients([y2], [x2])
   # the second-place loss has a gradient like the rest of the gating
   g2, _, x2, d2 = graph_input()
   y2, l2 = moe.transformer_moe_layer_v1(

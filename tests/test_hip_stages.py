@@ -996,3 +996,55 @@ def test_expert_linear_backward_and_activations(hip, act_dtype):
           err_msg=act)
   with pytest.raises(ValueError):
     hip.activation(g(pre), "softplus")
+
+
+@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
+def test_expert_choice_backward_stages(hip, act_dtype):
+  """The three backward entry points of the per-slot record against the
+  oracle: combine backward, dispatch backward (with and without the router's
+  share), and d(logits) of the gating (importance 0 / 0.5 / 1, two
+  microbatches)."""
+  g, s, e, c, m = 3, 96, 6, 20, 40
+  rng = np.random.default_rng(13)
+  logits = (rng.standard_normal((g, s, e)) * 1.5).astype(np.float32)
+  imp = rng.choice([0.0, 0.5, 1.0], size=(g, s), p=[0.15, 0.15, 0.7]).astype(np.float32)
+  want_r = O.expert_selection_gating(logits, c, imp, num_microbatches=2)
+  lg = torch.from_numpy(logits).cuda()
+  r = hip.expert_choice_gating(lg, c, importance=H.to_gpu(imp), num_microbatches=2)
+  assert np.array_equal(H.to_np(r.slot_token), want_r["slot_token"])
+  r_np = dict(slot_token=want_r["slot_token"], slot_weight=H.to_np(r.slot_weight))
+  cast = lambda a: O.cast_act(a.astype(np.float32), act_dtype)
+  tol = H.value_tolerance(act_dtype)
+  dout, y = cast(rng.standard_normal((g, s, m))), cast(rng.standard_normal((e, g, c, m)))
+  dy, dw = hip.slot_combine_backward(H.to_gpu(dout, act_dtype),
+                                     H.to_gpu(y, act_dtype), r)
+  want_dy, want_dw = O.slot_combine_backward(dout, y, r_np, act_dtype)
+  np.testing.assert_allclose(H.to_np(dy), want_dy, **tol)
+  np.testing.assert_allclose(H.to_np(dw), want_dw, rtol=1e-4, atol=1e-4)
+  dxe = cast(rng.standard_normal((e, g, c, m)))
+  dx = hip.slot_dispatch_backward(H.to_gpu(dxe, act_dtype), r, s)
+  want_dx = O.slot_dispatch_backward(dxe, r_np, s)
+  np.testing.assert_allclose(H.to_np(dx), O.cast_act(want_dx, act_dtype),
+                             rtol=tol["rtol"], atol=tol["atol"] * 4)
+  held = np.zeros((g, s), bool)
+  for gi in range(g):
+    held[gi][want_r["slot_token"][gi].reshape(-1)] = True
+  assert (~held).any() and (H.to_np(dx)[~held] == 0).all()
+  dweight = rng.standard_normal((g, e, c)).astype(np.float32)
+  want_dl = O.expert_selection_gating_backward(logits, r_np, imp, dweight, 0.7, 2)
+  assert np.abs(want_dl).max() > 0
+  dl = hip.expert_choice_backward(
+      lg, r, torch.from_numpy(dweight).cuda(),
+      torch.tensor([0.7], dtype=torch.float32, device="cuda"), 1.0,
+      importance=H.to_gpu(imp), num_microbatches=2)
+  np.testing.assert_allclose(H.to_np(dl), want_dl, rtol=1e-3,
+                             atol=1e-5 * np.abs(want_dl).max())
+  assert (H.to_np(dl)[imp == 0] == 0).all()          # masked tokens: p = 0
+  # with the router's share
+  wg = cast(H.normal_weights(rng, (m, e), m))
+  wg_p = hip.pack_weights(H.to_gpu(wg, act_dtype).reshape(1, m, e),
+                          H.ACT_TORCH[act_dtype]).reshape(e, m)
+  dx2 = hip.slot_dispatch_backward(H.to_gpu(dxe, act_dtype), r, s, dl, wg_p)
+  want2 = want_dx + np.matmul(H.to_np(dl), wg.T)
+  np.testing.assert_allclose(H.to_np(dx2), O.cast_act(want2, act_dtype),
+                             rtol=tol["rtol"], atol=tol["atol"] * 4)

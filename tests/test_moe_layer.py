@@ -731,7 +731,10 @@ def test_v1_experts_attention(act_dtype):
     (["gelu", "linear"], "bfloat16", "top_2", True, False),
     (["tanh", "sigmoid", "relu"], "float32", "switch", True, False),
     (["relu", "linear"], "float32", "top_2", False, True),
-    ("sigmoid", "float32", "top_2", True, True)],
+    ("sigmoid", "float32", "top_2", True, True),
+    ("relu", "float32", "expert_selection", False, False),
+    ("relu", "bfloat16", "expert_selection", True, False),
+    (["gelu", "linear"], "float32", "expert_selection", False, True)],
     ids=lambda c: "%s-%s-%s%s%s" % ("*".join(c[0]) if isinstance(c[0], list)
                                     else c[0], c[1], c[2],
                                     "-dropout" if c[3] else "",
@@ -751,6 +754,17 @@ def test_v1_gradients_other_activations(case):
   k_wo = H.normal_weights(rng, (e, hdim, m), hdim)
   x = H.safe_tokens(rng, b * l, m, w_gate, act_dtype, top=3).reshape(b, l, m)
   nonpad = (rng.random((b, l)) < 0.9).astype(np.float32)
+  if gating == "expert_selection":
+    # tokens whose router logits keep every expert's ranking of the group's
+    # tokens unambiguous (the experts choose, per column)
+    for _ in range(200):
+      x = O.cast_act(rng.standard_normal((b, l, m)).astype(np.float32), act_dtype)
+      lg = O.router_logits(x.reshape(-1, group, m), O.cast_act(w_gate, act_dtype))
+      gaps = [np.diff(np.sort(lg[gi][nonpad.reshape(-1, group)[gi] != 0], axis=0),
+                      axis=0).min() for gi in range(lg.shape[0])]
+      if min(gaps) > 1e-4:    # both implementations see the same rounded inputs
+        break
+    assert min(gaps) > 1e-4
   d_q, d_k = (O.cast_act(rng.standard_normal((b, l, m)).astype(np.float32),
                          act_dtype) for _ in range(2))
   kw = dict(moe_num_experts=e, moe_hidden_size=hdim, moe_group_size=group,
@@ -774,7 +788,9 @@ def test_v1_gradients_other_activations(case):
         nonpadding=imp(nonpad, dims[:2]), activation=activation,
         num_microbatches=2)
   outs = outs if attention else [outs]
-  router = "switch_gating" if gating == "switch" else "top_2_gating"
+  router = {"switch": "switch_gating",
+            "expert_selection": "expert_selection_gating"}.get(
+                gating, "top_2_gating")
   wi_names = (["moe/wi_%d/kernel" % i for i in range(len(acts))]
               if len(acts) > 1 else ["moe/wi/kernel"])
   wo_names = (["moe/q_wo/kernel", "moe/k_wo/kernel"] if attention

@@ -1032,6 +1032,27 @@ def _f64_layer(x, wg, wi, wo, aux, gating, m1, coef, mb, z_loss, mult=None,
   g, s, _ = x.shape
   e = wg.shape[1]
   logits = (x if mult is None else x * mult) @ wg     # the router's own input
+  if gating == "expert_selection":
+    # every expert holds `capacity` slots; softmax over the group's tokens per
+    # expert; chosen[g,s,e] and the number of experts per token held fixed
+    imp = aux["_importance"].astype(np.float64)
+    pc = scipy.special.softmax(logits + (imp == 0)[..., None] * -1e9, axis=1)
+    chosen = np.zeros((g, s, e))
+    for gi in range(g):
+      for ei in range(e):
+        chosen[gi, aux["slot_token"][gi, ei], ei] = 1.0
+    recip = 1.0 / np.maximum(chosen.sum(-1), 1.0)
+    out = 0.0
+    for ei in range(e):
+      h = 1.0
+      for w_f, a_f in zip(wi if isinstance(wi, list) else [wi],
+                          activation if isinstance(activation, list)
+                          else [activation]):
+        h = h * _F64_ACT[a_f](x @ w_f[ei])
+      out = out + (chosen[..., ei] * pc[..., ei] * recip)[..., None] * (h @ wo[ei])
+    agg = pc.mean(-1) * (imp == 1)
+    aux_loss = (agg ** 2 * imp.sum(-1, keepdims=True)).mean() * s / mb
+    return out, aux_loss * coef
   p = scipy.special.softmax(logits, axis=-1)
   rows = np.arange(g)[:, None], np.arange(s)[None, :]
   i1, i2 = aux["index_1"], aux["index_2"]
@@ -1088,7 +1109,9 @@ def _f64_layer(x, wg, wi, wo, aux, gating, m1, coef, mb, z_loss, mult=None,
                                     "top_2+hidden", "top_2+loss2",
                                     "top_2+act:gelu", "switch+act:swish",
                                     "top_2+act:gelu*linear",
-                                    "switch+act:tanh*sigmoid*relu"])
+                                    "switch+act:tanh*sigmoid*relu",
+                                    "expert_selection",
+                                    "expert_selection+jitter"])
 def test_backward_against_central_differences(gating):
   gating, _, perturb = gating.partition("+")
   hidden = perturb == "hidden"      # dropout on the experts' hidden tensor
@@ -1141,6 +1164,31 @@ def test_backward_against_central_differences(gating):
                                 hidden_uniform=hu, activation=activation)
   aux = got["aux"]
   mult = None
+  if gating == "expert_selection":
+    aux = dict(aux, _importance=nonpad.reshape(b, l))
+    counts = np.zeros((b, l))
+    for gi in range(b):
+      for ei in range(e):
+        counts[gi, aux["slot_token"][gi, ei]] += 1
+    assert (counts == 0).any() and (counts > 1).any()    # none / several experts
+    if perturb:
+      mult = aux["gate_mult"].astype(np.float64).reshape(b, l, m)
+    m1 = z = None
+    def scalar(xv, wgv, wiv, wov):
+      out, loss = _f64_layer(xv.reshape(b, l, m), wgv, wiv, wov, aux, gating,
+                             None, 0.5, mb, None, mult)
+      return (out * d_out.reshape(out.shape)).sum() + d_loss * loss
+    base = [a.astype(np.float64) for a in (x.reshape(b, l, m), wg, wi, wo)]
+    grads = [got["dx"].reshape(b, l, m), got["dw_gate"], got["dwi"], got["dwo"]]
+    for which in range(4):
+      for trial in range(3):
+        d = rng.standard_normal(base[which].shape)
+        plus = [a + 1e-6 * d if i == which else a for i, a in enumerate(base)]
+        minus = [a - 1e-6 * d if i == which else a for i, a in enumerate(base)]
+        fd = (scalar(*plus) - scalar(*minus)) / 2e-6
+        an = float((grads[which].astype(np.float64) * d).sum())
+        assert abs(fd - an) <= 2e-4 * max(1.0, abs(fd)), (which, trial, fd, an)
+    return
   if perturb == "sample":       # sampled experts differ from the arg-max
     assert (aux["index_1"] != aux["logits"].argmax(-1)).any()
   elif perturb:
