@@ -23,14 +23,23 @@
 // go straight from the accumulator registers into the second product's
 // operand registers: MFMA step u of O^T uses registers 8*(u%2) .. +7 of key
 // sub-tile u/2, which makes its 16 k-indices the keys 16u + {0-3, 8-11} for
-// the lower half-wave and 16u + {4-7, 12-15} for the upper one; the V^T
-// operand is read from LDS as two 8-byte pieces in that same key order, so no
-// data moves between lanes.
+// the lower half-wave and 16u + {4-7, 12-15} for the upper one.  The V^T
+// operand comes from the V tile as it lies in memory (rows = keys) through
+// ds_read_b64_tr_b16: within 16 lanes, lane t addresses the 8 bytes at (key row
+// t / 4, elements 4 (t % 4) ..) of a 4 x 16 block and lane i receives column i,
+// i.e. four consecutive keys of one d -- two such reads are exactly the 4 + 4
+// keys of a step, so no data moves between lanes and V is never transposed in
+// memory.
 //
-// K and V^T tiles (V^T [B*H, d_kv, L] is written by a transpose kernel first)
-// reach a two-stage LDS ring through global_load_lds_dwordx4 with XOR-swizzled
-// 16-byte chunks; the queries of a wavefront stay in registers.
+// K and V tiles reach a two-stage LDS ring through global_load_lds_dwordx4; K
+// rows with XOR-swizzled 16-byte chunks, V rows with their 64-byte units
+// XOR-ed by the key index (bank conflicts of the transposing reads); the
+// queries of a wavefront stay in registers.  The transposing reads are inline
+// asm: the compiler puts a vmcnt(0) in front of the builtin form, which would
+// drain the next tile's loads; lgkmcnt(0) stands before the MFMAs that use
+// their results.
 #include "common.h"
+#include <type_traits>
 
 namespace mesh_moe {
 
@@ -46,8 +55,11 @@ struct FlashCfg {
   static constexpr int BQ = 128, BK = 64, WAVES = 4, THREADS = 64 * WAVES;
   static constexpr int K_ROW = D * 2;              // bytes per key row
   static constexpr int K_BYTES = BK * K_ROW;
-  static constexpr int V_ROW = BK * 2;             // bytes per row of V^T
-  static constexpr int V_BYTES = D * V_ROW;
+  static constexpr int V_ROW = D * 2;              // bytes per key row of V
+  static constexpr int V_BYTES = BK * V_ROW;
+  static constexpr int V_RPI = 1024 / V_ROW;       // key rows per load instr
+  static constexpr int VCH = V_ROW / 16;           // 16-byte chunks per row
+  static constexpr int V_UNITS = V_ROW / 64;       // 64-byte units per row
   static constexpr int STAGE = K_BYTES + V_BYTES;
   static constexpr int LDS_BYTES = 2 * STAGE;
   static constexpr int KCH = K_ROW / 16;           // 16-byte chunks per key row
@@ -64,14 +76,35 @@ template <int KCH>
 __device__ __forceinline__ int fa_kswz(int row) {
   return KCH == 16 ? (row & 15) : ((row & 7) ^ ((row >> 3) & 1));
 }
+// 64-byte unit p of key row `row` of the V tile holds unit p ^ fa_vswz(row):
+// the four rows a transposing read touches land on different banks
+template <int UNITS>
 __device__ __forceinline__ int fa_vswz(int row) {
-  return (row & 7) ^ ((row >> 3) & 1);
+  return UNITS == 4 ? (row & 3) : ((row >> 1) & 1);
+}
+
+typedef short fa_i16x4_t __attribute__((ext_vector_type(4)));
+
+// ds_read_b64_tr_b16 at LDS byte address `addr` + OFF
+template <int OFF>
+__device__ __forceinline__ fa_i16x4_t fa_lds_read_tr16(uint32_t addr) {
+  fa_i16x4_t v;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2"
+               : "=v"(v) : "v"(addr), "n"(OFF));
+  return v;
+}
+
+// 2^x as one v_exp_f32 (results below the normal range flush to 0, which is
+// what a softmax weight that small is anyway; exp2f() spends four more
+// instructions on that range)
+__device__ __forceinline__ float fa_exp2(float x) {
+  return __builtin_amdgcn_exp2f(x);
 }
 
 template <int D, bool CAUSAL>
 __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
-    const bf16_t* __restrict__ vt, bf16_t* __restrict__ out, int L, int H) {
+    const bf16_t* __restrict__ v, bf16_t* __restrict__ out, int L, int H) {
   using Cfg = FlashCfg<D>;
   extern __shared__ __attribute__((aligned(16))) unsigned char fa_smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -83,7 +116,7 @@ __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
   const int64_t row_stride = (int64_t)H * D;               // elements
   const bf16_t* qb = q + ((int64_t)b * L) * row_stride + (int64_t)h * D;
   const bf16_t* kb = k + ((int64_t)b * L) * row_stride + (int64_t)h * D;
-  const bf16_t* vb = vt + (int64_t)bh * D * L;
+  const bf16_t* vb = v + ((int64_t)b * L) * row_stride + (int64_t)h * D;
   bf16_t* ob = out + ((int64_t)b * L) * row_stride + (int64_t)h * D;
 
   const int n_ktiles_all = (L + Cfg::BK - 1) / Cfg::BK;
@@ -101,7 +134,7 @@ __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
       qf[s] = *reinterpret_cast<const fa_bf16x8_t*>(qr + s * 16);
   }
 
-  // direct-to-LDS loads of one K tile and one V^T tile
+  // direct-to-LDS loads of one K tile and one V tile
   auto load_tile = [&](int kt, int buf) {
     const int key0 = kt * Cfg::BK;
     unsigned char* base = fa_smem + buf * Cfg::STAGE;
@@ -119,10 +152,11 @@ __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
 #pragma unroll
     for (int j = 0; j < Cfg::V_INSTR; ++j) {
       const int g = wave * Cfg::V_INSTR + j;
-      const int row = g * 8 + (lane >> 3);                  // d
-      const int c = (lane & 7) ^ fa_vswz(row);
+      const int row = g * Cfg::V_RPI + lane / Cfg::VCH;     // key
+      const int p = lane % Cfg::VCH;
+      const int c = (((p >> 2) ^ fa_vswz<Cfg::V_UNITS>(row)) << 2) | (p & 3);
       const bf16_t* src =
-          vb + (int64_t)row * L + min(key0 + c * 8, L - 8);
+          vb + (int64_t)min(key0 + row, L - 1) * row_stride + c * 8;
       __builtin_amdgcn_global_load_lds(
           (fa_glb_void_t*)src,
           (fa_lds_void_t*)(base + Cfg::K_BYTES + g * 1024), 16, 0, 0);
@@ -149,8 +183,11 @@ __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
     if (kt + 1 < n_ktiles) load_tile(kt + 1, buf ^ 1);
     const int key0 = kt * Cfg::BK;
     // (a wavefront whose queries all precede this tile still runs it: every
-    // weight comes out 0, and the loop body stays one straight line, which
-    // measured faster than skipping)
+    // weight comes out 0, which measured faster than skipping)
+    // mask: diagonal and last tiles only, behind a branch the tiles in between
+    // do not take
+    const bool need_mask =
+        (CAUSAL && key0 + Cfg::BK - 1 > qw_first) || key0 + Cfg::BK > L;
     {
       const unsigned char* ks = fa_smem + buf * Cfg::STAGE;
       const unsigned char* vs = ks + Cfg::K_BYTES;
@@ -171,25 +208,29 @@ __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
               kf, qf[s], acc_s[sub], 0, 0, 0);
         }
       }
-      // mask (diagonal and last tiles only) and row maximum
-      const bool need_mask =
-          (CAUSAL && key0 + Cfg::BK - 1 > qw_first) || key0 + Cfg::BK > L;
-      float mx = NEG;
+      // mask and row maximum
+      if (need_mask) {
+        // (the empty asm keeps the compiler from turning the branch into 64
+        // selects that every tile would execute)
+        asm volatile("" ::: "memory");
 #pragma unroll
-      for (int sub = 0; sub < 2; ++sub) {
+        for (int sub = 0; sub < 2; ++sub) {
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          if (need_mask) {
+          for (int r = 0; r < 16; ++r) {
             const int key = key0 + sub * 32 + 8 * (r / 4) + 4 * half + (r % 4);
             const bool ok = key < L && (!CAUSAL || key <= my_q);
             if (!ok) acc_s[sub][r] = NEG;
           }
-          mx = fmaxf(mx, acc_s[sub][r]);
         }
       }
+      float mx = NEG;
+#pragma unroll
+      for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) mx = fmaxf(mx, acc_s[sub][r]);
       mx = fmaxf(mx, __shfl_xor(mx, 32));
       const float m_new = fmaxf(m_run, mx);
-      const float alpha = exp2f((m_run - m_new) * LOG2E);
+      const float alpha = fa_exp2((m_run - m_new) * LOG2E);
       const float mneg = -m_new * LOG2E;
       m_run = m_new;
       float psum = 0.f;
@@ -200,8 +241,8 @@ __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
 #pragma unroll
         for (int c = 0; c < 4; ++c) {
           const int r = 8 * (u & 1) + 2 * c;
-          const float p0 = exp2f(fmaf(acc_s[u >> 1][r], LOG2E, mneg));
-          const float p1 = exp2f(fmaf(acc_s[u >> 1][r + 1], LOG2E, mneg));
+          const float p0 = fa_exp2(fmaf(acc_s[u >> 1][r], LOG2E, mneg));
+          const float p1 = fa_exp2(fmaf(acc_s[u >> 1][r + 1], LOG2E, mneg));
           psum += p0 + p1;
           w[c] = f32x2_to_bf16x2(p0, p1);
         }
@@ -213,21 +254,53 @@ __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
       for (int dt = 0; dt < Cfg::DT; ++dt)
 #pragma unroll
         for (int r = 0; r < 16; ++r) acc_o[dt][r] *= alpha;
-      // O^T += V^T . P
+      // O^T += V^T . P: the V^T operand of step u, block dt is two
+      // transposing reads of 4 key rows x 16 d each (per 16 lanes)
+      {
+        const uint32_t lds0 = (uint32_t)(size_t)(fa_lds_void_t*)fa_smem;
+        const int t16 = lane & 15, g16 = lane >> 4;
+        const int krow = 4 * (g16 >> 1) + (t16 >> 2);        // + 16 u (+ 8)
+        const int dcol = (g16 & 1) * 16 + 4 * (t16 & 3);      // + 32 dt
+        // row krow + 16 u + 8 j has the same fa_vswz as krow (multiples of 4
+        // or 8 are added), so the unit swizzle is a per-lane constant
+        const int sw = fa_vswz<Cfg::V_UNITS>(krow);
+        uint32_t vaddr[Cfg::DT];
 #pragma unroll
-      for (int dt = 0; dt < Cfg::DT; ++dt) {
-        const int row = dt * 32 + l32;
-        const unsigned char* vr = vs + row * Cfg::V_ROW + half * 8;
-        const int sw = fa_vswz(row);
+        for (int dt = 0; dt < Cfg::DT; ++dt) {
+          const int col = dt * 32 + dcol;                     // element index
+          vaddr[dt] = lds0 + buf * Cfg::STAGE + Cfg::K_BYTES +
+                      krow * Cfg::V_ROW + (((col >> 5) ^ sw) << 6) +
+                      (col & 31) * 2;
+        }
+        fa_i16x4_t vlo[2][4], vhi[2][4];
+        auto read_v = [&](int dt, int slot) {
+          const uint32_t a = vaddr[dt];
+          vlo[slot][0] = fa_lds_read_tr16<0 * Cfg::V_ROW>(a);
+          vhi[slot][0] = fa_lds_read_tr16<8 * Cfg::V_ROW>(a);
+          vlo[slot][1] = fa_lds_read_tr16<16 * Cfg::V_ROW>(a);
+          vhi[slot][1] = fa_lds_read_tr16<24 * Cfg::V_ROW>(a);
+          vlo[slot][2] = fa_lds_read_tr16<32 * Cfg::V_ROW>(a);
+          vhi[slot][2] = fa_lds_read_tr16<40 * Cfg::V_ROW>(a);
+          vlo[slot][3] = fa_lds_read_tr16<48 * Cfg::V_ROW>(a);
+          vhi[slot][3] = fa_lds_read_tr16<56 * Cfg::V_ROW>(a);
+        };
+        read_v(0, 0);
 #pragma unroll
-        for (int u = 0; u < 4; ++u) {
-          const fa_u32x2_t lo = *reinterpret_cast<const fa_u32x2_t*>(
-              vr + (((2 * u) ^ sw) * 16));
-          const fa_u32x2_t hi = *reinterpret_cast<const fa_u32x2_t*>(
-              vr + (((2 * u + 1) ^ sw) * 16));
-          fa_u32x4_t both = {lo.x, lo.y, hi.x, hi.y};
-          acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
-              __builtin_bit_cast(fa_bf16x8_t, both), pf[u], acc_o[dt], 0, 0, 0);
+        for (int dt = 0; dt < Cfg::DT; ++dt) {
+          const int cur = dt & 1;
+          __builtin_amdgcn_sched_barrier(0);
+          __builtin_amdgcn_s_waitcnt(0xc07f);      // lgkmcnt(0): block dt is here
+          __builtin_amdgcn_sched_barrier(0);
+          if (dt + 1 < Cfg::DT) read_v(dt + 1, cur ^ 1);
+#pragma unroll
+          for (int u = 0; u < 4; ++u) {
+            const fa_bf16x8_t vf = __builtin_bit_cast(
+                fa_bf16x8_t, __builtin_shufflevector(vlo[cur][u], vhi[cur][u], 0,
+                                                     1, 2, 3, 4, 5, 6, 7));
+            acc_o[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
+                vf, pf[u], acc_o[dt], 0, 0, 0);
+          }
+          __builtin_amdgcn_sched_barrier(0);
         }
       }
     }
@@ -256,28 +329,8 @@ __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
   }
 }
 
-// [B, L, H*D] -> [B*H, D, L]
-__global__ __launch_bounds__(256) void fa_transpose_v_kernel(
-    const bf16_t* __restrict__ in, bf16_t* __restrict__ out, int L, int H,
-    int D) {
-  __shared__ bf16_t tile[32][33];
-  const int bh = blockIdx.z, b = bh / H, h = bh % H;
-  const int l0 = blockIdx.x * 32, d0 = blockIdx.y * 32;
-  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
-  for (int r = ty; r < 32; r += 8) {
-    const int l = l0 + r, d = d0 + tx;
-    if (l < L && d < D)
-      tile[r][tx] = in[(((int64_t)b * L + l) * H + h) * D + d];
-  }
-  __syncthreads();
-  for (int r = ty; r < 32; r += 8) {
-    const int d = d0 + r, l = l0 + tx;
-    if (l < L && d < D) out[((int64_t)bh * D + d) * L + l] = tile[tx][r];
-  }
-}
-
 template <int D>
-static int launch_flash(const bf16_t* q, const bf16_t* k, const bf16_t* vt,
+static int launch_flash(const bf16_t* q, const bf16_t* k, const bf16_t* v,
                         bf16_t* out, int B, int L, int H, int causal,
                         hipStream_t st) {
   using Cfg = FlashCfg<D>;
@@ -285,11 +338,11 @@ static int launch_flash(const bf16_t* q, const bf16_t* k, const bf16_t* vt,
   if (causal) {
     auto kern = flash_attention_kernel<D, true>;
     MOE_ALLOW_LDS(kern, Cfg::LDS_BYTES);
-    kern<<<grid, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(q, k, vt, out, L, H);
+    kern<<<grid, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(q, k, v, out, L, H);
   } else {
     auto kern = flash_attention_kernel<D, false>;
     MOE_ALLOW_LDS(kern, Cfg::LDS_BYTES);
-    kern<<<grid, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(q, k, vt, out, L, H);
+    kern<<<grid, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(q, k, v, out, L, H);
   }
   MOE_CHECK_LAUNCH("self_attention (fused)");
   return 0;
@@ -304,22 +357,20 @@ bool flash_attention_supported(int L, int H, int D, int dtype, const void* q,
 }
 
 size_t flash_attention_workspace_bytes(int B, int L, int H, int D) {
-  return (size_t)B * H * D * L * sizeof(bf16_t) + 256;
+  (void)B; (void)L; (void)H; (void)D;
+  return 256;     // the fused kernel needs no scratch
 }
 
 int flash_attention(const void* q, const void* k, const void* v, void* out,
                     int B, int L, int H, int D, int causal, void* workspace,
                     hipStream_t st) {
-  bf16_t* vt = (bf16_t*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
-  dim3 tg((unsigned)((L + 31) / 32), (unsigned)((D + 31) / 32),
-          (unsigned)(B * H));
-  fa_transpose_v_kernel<<<tg, 256, 0, st>>>((const bf16_t*)v, vt, L, H, D);
-  MOE_CHECK_LAUNCH("self_attention (transpose v)");
+  (void)workspace;
   if (D == 128)
-    return launch_flash<128>((const bf16_t*)q, (const bf16_t*)k, vt,
-                             (bf16_t*)out, B, L, H, causal, st);
-  return launch_flash<64>((const bf16_t*)q, (const bf16_t*)k, vt, (bf16_t*)out,
-                          B, L, H, causal, st);
+    return launch_flash<128>((const bf16_t*)q, (const bf16_t*)k,
+                             (const bf16_t*)v, (bf16_t*)out, B, L, H, causal,
+                             st);
+  return launch_flash<64>((const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v,
+                          (bf16_t*)out, B, L, H, causal, st);
 }
 
 }  // namespace mesh_moe
