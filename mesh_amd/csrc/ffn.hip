@@ -496,11 +496,13 @@ __global__ __launch_bounds__(64 * WM * WN) void grouped_gemm_bf16_dma_kernel(
 // pipeline accepts them only as fast as earlier requests drain), and because
 // the wavefronts of a block hand over together, the MFMA pipes idle meanwhile.
 // Here the 160 KB of LDS hold two slots for the token tile and THREE for the
-// weight tile, which lets every MFMA step carry exactly two loads:
+// weight tile, which lets the loads of tile t+2 ride on the MFMA steps of
+// tile t, pinned between its MFMAs:
 //
-//   step 0 of tile t:  token loads 2,3 of tile t+1
-//   step 1, step 2:    weight loads 0,1 / 2,3 of tile t+2   (two tiles ahead)
-//   step 3 (after the hand-over barrier): token loads 0,1 of tile t+2
+//   step 0:            weight loads 0,1 of tile t+2   (two tiles ahead)
+//   step 1, step 2:    weight load 2 / weight load 3 of tile t+2
+//   step 3 (after the hand-over barrier that frees their slot, behind the
+//           first fragment reads of tile t+1): the four token loads of tile t+2
 //
 // vmcnt counts in issue order, so the hand-over of tile t waits with vmcnt(4):
 // everything up to the token loads of tile t+1 has landed, the four weight
