@@ -25,11 +25,13 @@ class AttentionParams(object):
                combine_dims=True, ensemble_dim=None,
                keep_query_heads_dims=False,
                fold_scaling_into_initializer=True, make_attention_vars=True):
-    if shared_kv or no_query or not combine_dims or ensemble_dim or \
-        keep_query_heads_dims or not make_attention_vars:
+    if no_query or not combine_dims or ensemble_dim or keep_query_heads_dims:
       raise NotImplementedError(
-          "only the default attention parameters are implemented (separate "
-          "k and v, combined dims, no ensemble)")
+          "only the default attention parameters are implemented (combined "
+          "dims, no ensemble)")
+    if shared_kv and make_attention_vars:
+      raise NotImplementedError(
+          "a shared \"kv\" kernel is only implemented for ExpertsAttention")
     if key_dim != value_dim:
       raise NotImplementedError("key_dim != value_dim")
     query_heads_dims = list(query_heads_dims or [])
@@ -45,6 +47,8 @@ class AttentionParams(object):
     self.query_heads_dims = query_heads_dims
     self.memory_heads_dims = memory_heads_dims
     self.variable_dtype = variable_dtype
+    self.shared_kv = shared_kv
+    self.make_attention_vars = make_attention_vars
     self.fold_scaling_into_initializer = fold_scaling_into_initializer
     self.num_heads = query_heads_dims[0].size if query_heads_dims else 1
     first = (query_heads_dims + [key_dim])[0].name
@@ -57,12 +61,18 @@ class AttentionParams(object):
     o_std = combined.size ** -0.5
 
     normal = mtf_layers.random_normal_initializer
-    self.wq = mtf.get_variable(mesh, "q", [query_input_dim, combined],
-                               initializer=normal(stddev), dtype=variable_dtype)
-    self.wk = mtf.get_variable(mesh, "k", [memory_input_dim, combined],
-                               initializer=normal(kv_std), dtype=variable_dtype)
-    self.wv = mtf.get_variable(mesh, "v", [memory_input_dim, combined],
-                               initializer=normal(kv_std), dtype=variable_dtype)
+    # the q / k / v kernels are not needed by ExpertsAttention
+    # (attention.py:443-468)
+    if make_attention_vars:
+      self.wq = mtf.get_variable(mesh, "q", [query_input_dim, combined],
+                                 initializer=normal(stddev),
+                                 dtype=variable_dtype)
+      self.wk = mtf.get_variable(mesh, "k", [memory_input_dim, combined],
+                                 initializer=normal(kv_std),
+                                 dtype=variable_dtype)
+      self.wv = mtf.get_variable(mesh, "v", [memory_input_dim, combined],
+                                 initializer=normal(kv_std),
+                                 dtype=variable_dtype)
     self.wo = mtf.get_variable(mesh, "o", [combined, output_dim],
                                initializer=normal(o_std), dtype=variable_dtype)
 
@@ -91,6 +101,81 @@ class AttentionParams(object):
       raise ValueError("attention output %s, expected %s"
                        % (y.shape, output_shape))
     return y
+
+
+class ExpertsAttentionParams(AttentionParams):
+  """Attention parameters whose queries and keys come out of a
+  Mixture-of-Experts layer (attention.py:594-692): a MoE1D with
+  use_experts_attention projects the antecedent to [q, k] through two output
+  kernels of the same experts ("q_wo", "k_wo"), the keys are also the values
+  (shared_kv) and only the output kernel "o" is a variable of its own.  The
+  queries are scaled by d_kv ** -0.5 after the layer (attention.py:664-665).
+
+  The reference passes `switch_top_k` to a MoE1D constructor that has no such
+  argument (transformer/moe.py:44-66), so its version cannot be constructed;
+  here the value goes to `ntlb_top_k`, the only top-k the layer has."""
+
+  def __init__(self, mesh, query_input_dim, memory_input_dim, output_dim,
+               key_dim, value_dim, query_heads_dims, memory_heads_dims,
+               variable_dtype, shared_kv=False, no_query=False,
+               combine_dims=True, ensemble_dim=None,
+               keep_query_heads_dims=False,
+               fold_scaling_into_initializer=True, context=None,
+               experts_hparams=None):
+    super(ExpertsAttentionParams, self).__init__(
+        mesh=mesh, query_input_dim=query_input_dim,
+        memory_input_dim=memory_input_dim, output_dim=output_dim,
+        key_dim=key_dim, value_dim=value_dim,
+        query_heads_dims=query_heads_dims, memory_heads_dims=memory_heads_dims,
+        variable_dtype=variable_dtype, shared_kv=shared_kv, no_query=no_query,
+        combine_dims=combine_dims, ensemble_dim=ensemble_dim,
+        keep_query_heads_dims=keep_query_heads_dims,
+        fold_scaling_into_initializer=fold_scaling_into_initializer,
+        make_attention_vars=False)
+    self.context = context
+    if not combine_dims:
+      raise ValueError("self.combine_dims must be True for ExpertsAttention")
+    if not shared_kv:
+      raise ValueError("self.shared_kv must be True for ExpertsAttention")
+    from mesh_amd.transformer import moe
+    hp = experts_hparams
+    self.moe_layer = moe.MoE1D(
+        moe_gating=hp.moe_gating, num_experts=hp.num_experts,
+        loss_coef=hp.loss_coef, group_size=hp.group_size,
+        min_expert_capacity=hp.min_expert_capacity,
+        capacity_factor_train=hp.capacity_factor_train,
+        capacity_factor_eval=hp.capacity_factor_eval,
+        switch_policy_train=hp.switch_policy_train,
+        switch_policy_eval=hp.switch_policy_eval,
+        switch_dropout=hp.switch_dropout,
+        switch_temperature=hp.switch_temperature,
+        switch_jitter=hp.switch_jitter, ntlb_top_k=hp.switch_top_k,
+        hidden_size=hp.hidden_size, output_dim=self.combined_dim,
+        use_experts_attention=hp.use_experts_attention)
+    self._q = self._k = None
+
+  def _compute_merge_qkv(self, antecedent):
+    """q and k in one call of the experts layer (query and memory antecedent
+    are taken to be the same, attention.py:657-667)."""
+    q, k = self.moe_layer.call(self.context, antecedent)
+    self._q = q * (self.key_dim.size ** -0.5)
+    self._k = k
+
+  def compute_q(self, query_antecedent):
+    self._compute_merge_qkv(query_antecedent)
+    return self._q
+
+  def compute_k(self, memory_antecedent):
+    del memory_antecedent
+    return self._k
+
+  def compute_kv(self, memory_antecedent):
+    del memory_antecedent
+    return self._k
+
+  def compute_v(self, memory_antecedent):
+    del memory_antecedent
+    raise NotImplementedError("ExpertsAttention uses shared_kv = True.")
 
 
 class SelfAttentionOperation(mtf.Operation):

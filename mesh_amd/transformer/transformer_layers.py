@@ -44,18 +44,23 @@ class SelfAttention(transformer.TransformerLayer):
   Visibility comes from the context: read/write priorities (autoregressive
   models) or none."""
 
+  _shared_kv_implemented = False     # a "kv" kernel of its own is not
+
   def __init__(self, num_heads=8, num_memory_heads=0, key_value_size=128,
                shared_kv=False, dropout_rate=0.0, attention_kwargs=None,
                relative_attention_type=None,
                relative_attention_num_buckets=32, attention_func=None,
                combine_dims=True, keep_query_heads_dims=False,
                fold_scaling_into_initializer=True):
-    if (num_memory_heads or shared_kv or attention_kwargs or
+    if (num_memory_heads or attention_kwargs or
         relative_attention_type is not None or attention_func is not None or
-        not combine_dims or keep_query_heads_dims):
+        not combine_dims or keep_query_heads_dims or
+        (shared_kv and not self._shared_kv_implemented)):
       raise NotImplementedError(
           "only the default SelfAttention options are implemented")
     self.num_heads = num_heads
+    self.shared_kv = shared_kv
+    self.combine_dims = combine_dims
     self.key_value_size = key_value_size
     self.dropout_rate = dropout_rate
     self.relative_attention_num_buckets = relative_attention_num_buckets
@@ -75,7 +80,7 @@ class SelfAttention(transformer.TransformerLayer):
         output_dim=context.model.model_dim, key_dim=self.kv_dim,
         value_dim=self.kv_dim, query_heads_dims=heads,
         memory_heads_dims=heads, variable_dtype=context.variable_dtype,
-        ensemble_dim=context.model.ensemble_dim,
+        shared_kv=self.shared_kv, ensemble_dim=context.model.ensemble_dim,
         fold_scaling_into_initializer=self.fold_scaling_into_initializer)
 
   def call(self, context, x, losses=None):
@@ -88,10 +93,58 @@ class SelfAttention(transformer.TransformerLayer):
       raise NotImplementedError("sequence_id tensors are not implemented")
     params = self.make_params(context)
     q = params.compute_q(x)
-    k = params.compute_k(x)
-    v = params.compute_v(x)
+    if self.shared_kv:                       # transformer_layers.py:246-249
+      k = v = params.compute_kv(x)
+    else:
+      k = params.compute_k(x)
+      v = params.compute_v(x)
     # read_priority >= write_priority (transformer_layers.py:289-296)
     causal = context.read_priority is transformer.POSITION
     o = attention.SelfAttentionOperation(q, k, v, params.num_heads,
                                          causal).outputs[0]
     return params.compute_output(o, output_shape=x.shape)
+
+
+class ExpertsSelfAttention(SelfAttention):
+  """Self-attention whose queries and keys (= values) are computed by a
+  Mixture-of-Experts layer (transformer_layers.py:383-459).  `shared_kv=True`
+  must be passed, as to the reference's.  Variables under the layer's scope:
+  the experts layer's "<router>_gating/kernel", "wi/kernel", "q_wo/kernel",
+  "k_wo/kernel" and the attention output kernel "o"."""
+
+  _shared_kv_implemented = True      # the keys the experts compute are the values
+
+  def __init__(self, num_experts=16, loss_coef=1e-2, group_size=1024,
+               capacity_factor_train=1.25, capacity_factor_eval=2.0,
+               moe_gating="switch", min_expert_capacity=4,
+               switch_policy_train="input_jitter",
+               switch_policy_eval="input_jitter", switch_dropout=0.0,
+               switch_temperature=1.0, switch_jitter=1e-2, switch_top_k=4,
+               hidden_size=3072, use_experts_attention=True, **kwargs):
+    super(ExpertsSelfAttention, self).__init__(**kwargs)
+    from mesh_amd.transformer import moe
+    self._hparams = moe.HParams(
+        moe_gating=moe_gating, num_experts=num_experts, loss_coef=loss_coef,
+        group_size=group_size, min_expert_capacity=min_expert_capacity,
+        capacity_factor_train=capacity_factor_train,
+        capacity_factor_eval=capacity_factor_eval,
+        switch_policy_train=switch_policy_train,
+        switch_policy_eval=switch_policy_eval, switch_dropout=switch_dropout,
+        switch_temperature=switch_temperature, switch_jitter=switch_jitter,
+        switch_top_k=switch_top_k, hidden_size=hidden_size,
+        use_experts_attention=use_experts_attention)
+
+  def make_params(self, context):
+    heads = ([mtf.Dimension("heads", self.num_heads)]
+             if self.num_heads > 1 else None)
+    return attention.ExpertsAttentionParams(
+        context.mesh, query_input_dim=context.model.model_dim,
+        memory_input_dim=context.model.model_dim,
+        output_dim=context.model.model_dim, key_dim=self.kv_dim,
+        value_dim=self.kv_dim, query_heads_dims=heads,
+        memory_heads_dims=heads, variable_dtype=context.variable_dtype,
+        shared_kv=self.shared_kv, no_query=False,
+        ensemble_dim=context.model.ensemble_dim,
+        combine_dims=self.combine_dims,
+        fold_scaling_into_initializer=self.fold_scaling_into_initializer,
+        context=context, experts_hparams=self._hparams)

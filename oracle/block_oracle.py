@@ -93,6 +93,42 @@ def self_attention(x, wq, wk, wv, wo, num_heads, causal, act_dtype="float32"):
   return dense(o.reshape(b, l, hd), wo, act_dtype)
 
 
+def _attention_core(q, k, v, num_heads, causal, act_dtype):
+  """attention.attention with float32 logits (attention.py:27-88) on
+  [B, L, H*D] activation-dtype tensors -> [B, L, H*D]."""
+  b, l, hd = q.shape
+  d = hd // num_heads
+  q, k, v = (t.reshape(b, l, num_heads, d) for t in (q, k, v))
+  logits = np.einsum("blhd,bmhd->bhlm", q, k).astype(F32)
+  if causal:
+    pos = np.arange(l)
+    logits = logits + (pos[None, :] > pos[:, None]).astype(F32) * F32(-1e9)
+  weights = _r(O.softmax(logits), act_dtype)
+  return _r(np.einsum("bhlm,bmhd->blhd", weights, v), act_dtype).reshape(b, l, hd)
+
+
+def experts_self_attention(x, w_gate, wi, q_wo, k_wo, wo, hparams, num_heads,
+                           causal, act_dtype="float32", train=False,
+                           num_microbatches=None):
+  """ExpertsSelfAttention.call (transformer/transformer_layers.py:383-459 with
+  attention.ExpertsAttentionParams, attention.py:594-692): a Mixture-of-Experts
+  layer with moe_use_experts_attention projects x to [q, k] (two output
+  kernels of the same experts, moe.py:514-522); q is scaled by d_kv ** -0.5
+  (a Python scalar times a tensor: the scalar is rounded to the tensor's
+  dtype); the keys are also the values; "o" projects the result back.
+
+  hparams: an O.HParams for the experts layer (moe_use_experts_attention set).
+  Returns (y [B, L, d_model], loss of the experts layer)."""
+  x = _r(x, act_dtype)
+  (q, k), loss, _ = O.moe_layer_v1(x, w_gate, wi, q_wo, hparams, train,
+                                   act_dtype, k_wo=k_wo, dense=False,
+                                   num_microbatches=num_microbatches)
+  d = q.shape[-1] // num_heads
+  q = _r(q * _r(F32(d ** -0.5), act_dtype), act_dtype)
+  o = _attention_core(q, k, k, num_heads, causal, act_dtype)
+  return dense(o, wo, act_dtype), loss
+
+
 def dense_relu_dense(x, wi, wo, act_dtype="float32"):
   """DenseReluDense.call (transformer/transformer_layers.py:55-76)."""
   return dense(dense(x, wi, act_dtype, "relu"), wo, act_dtype)

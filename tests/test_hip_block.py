@@ -299,3 +299,80 @@ def test_dense_rows_beyond_2_to_the_30_elements(hip):
     want = x[0, sl].float() @ w.float()
     np.testing.assert_allclose(H.to_np(y[0, sl]), H.to_np(want), rtol=2e-2,
                                atol=2e-2)
+
+
+@pytest.mark.parametrize("case", [("float32", True), ("bfloat16", False)],
+                         ids=["float32-causal", "bfloat16"])
+def test_experts_self_attention_layer(case):
+  """ExpertsSelfAttention in a layer stack: queries and keys (= values) come
+  out of a switch-gated experts layer with two output kernels, the scaled
+  queries attend, "o" projects back; against the oracle."""
+  act_dtype, autoregressive = case
+  b, l, m, e, hdim, heads, d, group = 2, 64, 64, 4, 96, 4, 16, 32
+  rng = np.random.default_rng(31)
+  n = lambda *shape: H.normal_weights(rng, shape, shape[-2])
+  w = dict(w_gate=n(m, e), wi=n(e, m, hdim), q_wo=n(e, hdim, heads * d),
+           k_wo=n(e, hdim, heads * d), o=n(heads * d, m))
+  scale = (1 + 0.1 * rng.standard_normal(m)).astype(np.float32)
+  final = (1 + 0.1 * rng.standard_normal(m)).astype(np.float32)
+  # tokens whose normalised form keeps every router decision clear
+  for _ in range(100):
+    x = O.cast_act(rng.standard_normal((b, l, m)).astype(np.float32), act_dtype)
+    xn = B.rms_norm(x, scale, act_dtype)
+    lg = np.sort(O.router_logits(xn.reshape(-1, group, m),
+                                 O.cast_act(w["w_gate"], act_dtype)), axis=-1)
+    if (lg[..., -1] - lg[..., -2]).min() > (2e-2 if act_dtype == "bfloat16"
+                                           else 1e-3):
+      break
+  hp_kw = dict(moe_gating="switch", moe_num_experts=e, moe_hidden_size=hdim,
+               moe_group_size=group, moe_capacity_factor_eval=1.25,
+               moe_switch_policy_train="argmax", moe_switch_policy_eval="argmax",
+               moe_use_experts_attention=True, moe_min_expert_capacity=4,
+               moe_loss_coef=1e-2)
+  ohp = O.default_hparams(**hp_kw)
+  dt = H.ACT_TORCH[act_dtype]
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  dims = [mtf.Dimension("batch", b), mtf.Dimension("length", l),
+          mtf.Dimension("d_model", m)]
+  xt = mtf.import_tf_tensor(mesh, torch.from_numpy(x).to(dt), mtf.Shape(dims))
+  stack = transformer.make_layer_stack(
+      [(transformer_layers.ExpertsSelfAttention,
+        dict(num_heads=heads, key_value_size=d, shared_kv=True, num_experts=e,
+             hidden_size=hdim, group_size=group, capacity_factor_eval=1.25,
+             switch_policy_train="argmax", switch_policy_eval="argmax"))],
+      num_layers=1, block_scope=False)
+  model = transformer.Unitransformer(stack, d_model=m, name="decoder",
+                                     autoregressive=autoregressive)
+  y, losses = model.call_layers(
+      xt, mtf.VariableDType(torch.float32, torch.float32, dt), mode="eval")
+  p = "decoder/layer_000/ExpertsSelfAttention/"
+  init = {"decoder/rms_norm/scale": final,
+          "decoder/layer_000/rms_norm/scale": scale,
+          p + "switch_gating/kernel": w["w_gate"], p + "wi/kernel": w["wi"],
+          p + "q_wo/kernel": w["q_wo"], p + "k_wo/kernel": w["k_wo"],
+          p + "o": w["o"]}
+  assert sorted(init) == sorted(v.name for v in graph.all_variables)
+  lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()}, initial_values=init)
+  got = H.to_np(lowering.export_to_tf_tensor(y))
+  assert len(losses) == 1
+  got_loss = float(H.to_np(lowering.export_to_tf_tensor(losses[0])))
+  # the oracle's stack: x + layer(rms_norm(x)), then the final rms_norm
+  att, want_loss = B.experts_self_attention(
+      B.rms_norm(x, scale, act_dtype), w["w_gate"], w["wi"], w["q_wo"],
+      w["k_wo"], w["o"], ohp, heads, autoregressive, act_dtype)
+  want = B.rms_norm(O.cast_act(x + att, act_dtype), final, act_dtype)
+  tol = dict(rtol=2e-4, atol=2e-4) if act_dtype == "float32" else dict(
+      rtol=5e-2, atol=5e-2)
+  np.testing.assert_allclose(got, want, **tol)
+  np.testing.assert_allclose(got_loss, want_loss,
+                             rtol=1e-4 if act_dtype == "float32" else 2e-2)
+  with pytest.raises(ValueError, match="shared_kv must be True"):
+    g2 = mtf.Graph()
+    x2 = mtf.import_tf_tensor(mtf.Mesh(g2, "mesh"), torch.zeros(b, l, m),
+                              mtf.Shape(dims))
+    st2 = transformer.make_layer_stack(
+        [(transformer_layers.ExpertsSelfAttention, dict(num_heads=heads))],
+        num_layers=1, block_scope=False)
+    transformer.Unitransformer(st2, d_model=m, name="decoder").call_layers(
+        x2, mtf.VariableDType(torch.float32), mode="eval")
