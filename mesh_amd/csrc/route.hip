@@ -566,12 +566,36 @@ __global__ __launch_bounds__(256) void router_gate_kernel(
 // ---------------------------------------------------------------------------
 constexpr int CAP_THREADS = 1024;
 
+// How many of the eight int16 expert ids in v equal e (0 <= e < 1024; an id of
+// -1, "not competing", never does).
+__device__ __forceinline__ int cap_match8(const uint4& v, int e) {
+  const uint32_t w[4] = {v.x, v.y, v.z, v.w};
+  const uint32_t ue = (uint32_t)e;
+  int n = 0;
+#pragma unroll
+  for (int j = 0; j < 4; ++j)
+    n += ((w[j] & 0xffffu) == ue ? 1 : 0) + ((w[j] >> 16) == ue ? 1 : 0);
+  return n;
+}
+
+// Number of entries of ch[s_begin, s_end) equal to e; with `vec` the range
+// starts 16-byte aligned and is read eight ids at a time.
+__device__ __forceinline__ int cap_count(const int16_t* ch, int s_begin,
+                                         int s_end, int e, bool vec) {
+  int c = 0, s = s_begin;
+  if (vec)
+    for (; s + 8 <= s_end; s += 8)
+      c += cap_match8(*reinterpret_cast<const uint4*>(ch + s), e);
+  for (; s < s_end; ++s) c += (ch[s] == e);
+  return c;
+}
+
 __global__ __launch_bounds__(CAP_THREADS) void gate_capacity_kernel(
     GateParams p, const int32_t* __restrict__ idx, int32_t* __restrict__ pos,
     float* __restrict__ gate, uint8_t* __restrict__ kept,
     int32_t* __restrict__ fill, const float* __restrict__ part1,
     const float* __restrict__ part2, float* __restrict__ gsum, int el) {
-  extern __shared__ int32_t smem_i[];
+  extern __shared__ __attribute__((aligned(16))) int32_t smem_i[];
   const int S = p.S, E = p.E, C = p.C;
   int32_t* cnt = smem_i;                        // [nchunks][el] = CAP_THREADS
   int32_t* tot = cnt + CAP_THREADS;             // [3][el]: total1,total2,loss2
@@ -606,13 +630,14 @@ __global__ __launch_bounds__(CAP_THREADS) void gate_capacity_kernel(
   const int clen = (S + nchunks - 1) / nchunks;
   const int s_begin = min(S, chunk * clen);
   const int s_end = min(S, s_begin + clen);
+  // 16-byte reads of the id arrays: c1 starts 4096 + 20 * el bytes into LDS,
+  // c2 and c2l S and 2 S ids later, a chunk clen ids after the previous one
+  const bool vec = (el % 4 == 0) && (S % 8 == 0) && (clen % 8 == 0);
 
   int count1 = 0;  // kept first choices of expert e (valid after choice 0)
   for (int choice = 0; choice < 2; ++choice) {
     const int16_t* ch = choice == 0 ? c1 : c2;
-    int c = 0;
-    for (int s = s_begin; s < s_end; ++s) c += (ch[s] == e);
-    cnt[chunk * el + e] = c;
+    cnt[chunk * el + e] = cap_count(ch, s_begin, s_end, e, vec);
     __syncthreads();
     int before = 0, total = 0;
     for (int k = 0; k < nchunks; ++k) {
@@ -623,6 +648,12 @@ __global__ __launch_bounds__(CAP_THREADS) void gate_capacity_kernel(
     int running = before + (choice == 0 ? 0 : count1);
     const bool in_token_order = !(p.rank_by_gate && choice == 0);
     for (int s = s_begin; in_token_order && s < s_end; ++s) {
+      // eight ids at a time where none of them is e (most of the time)
+      if (vec && (s & 7) == 0 && s + 8 <= s_end &&
+          cap_match8(*reinterpret_cast<const uint4*>(ch + s), e) == 0) {
+        s += 7;
+        continue;
+      }
       if (ch[s] == e) {
         int64_t t = base + s;
         const bool ok = running < C;
@@ -667,9 +698,7 @@ __global__ __launch_bounds__(CAP_THREADS) void gate_capacity_kernel(
     }
   }
   if (loss2) {
-    int c = 0;
-    for (int s = s_begin; s < s_end; ++s) c += (c2l[s] == e);
-    cnt[chunk * el + e] = c;
+    cnt[chunk * el + e] = cap_count(c2l, s_begin, s_end, e, vec);
     __syncthreads();
     if (chunk == 0 && e < E) {
       int total = 0;
@@ -678,42 +707,62 @@ __global__ __launch_bounds__(CAP_THREADS) void gate_capacity_kernel(
     }
     __syncthreads();
   }
-  // per-expert outputs and the group's share of the balancing loss
+  // per-expert outputs and the group's share of the balancing loss.  The
+  // per-block partial sums of the select step are summed in block order; they
+  // come through LDS (`cnt` is free now), nchunks blocks at a time, so that
+  // the loads of one batch fly together instead of one after the other.
+  float* stage = reinterpret_cast<float*>(cnt);          // [nchunks][el]
+  auto sum_blocks = [&](const float* part) {
+    float acc = 0.f;
+    for (int b0 = 0; b0 < p.nblk; b0 += nchunks) {
+      const int bb = b0 + chunk;
+      const float v = (bb < p.nblk && e < E)
+                          ? part[((int64_t)g * p.nblk + bb) * E + e] : 0.f;
+      __syncthreads();
+      stage[chunk * el + e] = v;
+      __syncthreads();
+      if (tid < E)
+        for (int k = 0; k < nchunks && b0 + k < p.nblk; ++k)
+          acc += stage[k * el + tid];
+    }
+    return acc;                                          // valid for tid < E
+  };
+  const float proxy = sum_blocks(part1);
+  float proxy2 = 0.f, zsum = 0.f, n_one_sum = 0.f;
+  if (loss2 && !sw) proxy2 = sum_blocks(part2);
+  if (sw) {
+    // columns 0 and 1 of part2: sum of logsumexp^2 and the number of tokens of
+    // importance 1; thread e sums column e
+    const float colsum = sum_blocks(part2);
+    __syncthreads();
+    if (tid < 2) stage[tid] = colsum;
+    __syncthreads();
+    zsum = stage[0];
+    n_one_sum = E > 1 ? stage[1] : 0.f;
+    __syncthreads();
+  }
   if (tid < E) {
     const int t1 = tot[tid], t2 = tot[el + tid];
     const int k1 = min(t1, C);
     fill[(int64_t)g * E + tid] = k1 + min(t2, C - k1);
     const float inv_s = (float)(1.0 / (double)S);
-    float proxy = 0.f;
-    for (int b = 0; b < p.nblk; ++b)
-      proxy += part1[((int64_t)g * p.nblk + b) * E + tid];
     // density_1: competing first choices (top-2, moe.py:1420-1423) or every
     // token's arg-max (switch, moe.py:1224-1225)
     const int dens = sw ? tot[2 * el + tid] : t1;
     prod[tid] = (proxy * inv_s) * ((float)dens * inv_s);
-    if (loss2 && !sw) {
-      float proxy2 = 0.f;
-      for (int b = 0; b < p.nblk; ++b)
-        proxy2 += part2[((int64_t)g * p.nblk + b) * E + tid];
+    if (loss2 && !sw)
       prod[el + tid] = (proxy2 * inv_s) * ((float)tot[2 * el + tid] * inv_s);
-    }
   }
   __syncthreads();
   if (tid == 0) {
-    float s1 = 0.f, s2 = 0.f, n_one = 0.f, z = 0.f;
+    float s1 = 0.f, s2 = 0.f;
     for (int k = 0; k < E; ++k) s1 += prod[k];
     if (loss2 && !sw)
       for (int k = 0; k < E; ++k) s2 += prod[el + k];
-    if (sw) {
-      for (int b = 0; b < p.nblk; ++b) {
-        z += part2[((int64_t)g * p.nblk + b) * E + 0];
-        n_one += part2[((int64_t)g * p.nblk + b) * E + 1];
-      }
-    }
     gsum[g * GSUM] = s1;
     gsum[g * GSUM + 1] = s2;
-    gsum[g * GSUM + 2] = n_one;
-    gsum[g * GSUM + 3] = z;
+    gsum[g * GSUM + 2] = sw ? n_one_sum : 0.f;
+    gsum[g * GSUM + 3] = sw ? zsum : 0.f;
   }
 }
 
