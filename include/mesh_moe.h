@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 13
+#define MESH_MOE_ABI_VERSION 14
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -56,6 +56,16 @@ extern "C" {
 
 int mesh_moe_abi_version(void);
 const char* mesh_moe_last_error(void);
+
+/*
+ * CRC-32C (Castagnoli) of data[0, n) continued from `crc` (0 to start): the
+ * checksum TensorFlow's tensor-bundle checkpoint files carry for every table
+ * block and every tensor (tensorflow/core/lib/hash/crc32c.h `Extend`; TensorFlow
+ * is the reference's dependency and is not vendored in it).  Host code; `data`
+ * is a host pointer.  The reference reaches those files through tf.train
+ * (mesh_tensorflow/transformer/utils.py:947-972, tf.train.init_from_checkpoint).
+ */
+uint32_t mesh_moe_crc32c(uint32_t crc, const void* data, size_t n);
 
 /*
  * Router projection: logits[b,t,e] = sum_m float(x[b,t,m]) * float(w[b,m,e])

@@ -9,17 +9,21 @@ mapping, a should-load predicate) and the two hooks around TensorFlow's saver
 (mesh_tensorflow/ops.py:5740-5779: masters are copied to slices after a
 restore, slices to masters before a save).
 
-A checkpoint is a mapping name -> array, or the path of a NumPy `.npz` archive
-of such a mapping.  TensorFlow's own tensor-bundle files are not read here;
-`{name: reader.get_tensor(name) for name in names}` from
-tf.train.load_checkpoint converts one.
+A checkpoint is a mapping name -> array, the path of a NumPy `.npz` archive of
+such a mapping, the prefix of a TensorFlow tensor bundle (`model.ckpt-1000`
+beside `model.ckpt-1000.index` and `.data-*`), or a directory whose `checkpoint`
+file names such a prefix (mesh_amd/tensor_bundle.py reads and writes the
+bundles without TensorFlow).
 """
 
 import collections
+import os
 import re
 
 import numpy as np
 import torch
+
+from mesh_amd import tensor_bundle
 
 RestoreReport = collections.namedtuple(
     "RestoreReport",
@@ -53,9 +57,16 @@ def plan_restore(graph_names, checkpoint_names, variable_filter=None,
 
 
 def _open(checkpoint):
-  if isinstance(checkpoint, str):
-    return np.load(checkpoint, allow_pickle=False)
-  return checkpoint
+  if not isinstance(checkpoint, str):
+    return checkpoint
+  if os.path.isdir(checkpoint):
+    prefix = tensor_bundle.latest_checkpoint(checkpoint)
+    if prefix is None:
+      raise ValueError("no checkpoint state file in %s" % checkpoint)
+    return tensor_bundle.BundleReader(prefix)
+  if os.path.exists(checkpoint + ".index"):
+    return tensor_bundle.BundleReader(checkpoint)
+  return np.load(checkpoint, allow_pickle=False)
 
 
 def restore_variables(lowering, checkpoint, variable_filter=None,
@@ -84,7 +95,9 @@ def restore_variables(lowering, checkpoint, variable_filter=None,
 def save_variables(lowering, path=None):
   """Copies slices to masters (MtfCheckpointSaverListener.before_save,
   ops.py:5740-5757) and returns {name: float32 / integer NumPy array of the
-  master}; with `path`, also writes them as an `.npz` archive."""
+  master}.  With a `path` ending in `.npz` also writes them as a NumPy
+  archive; with any other `path`, as a TensorFlow tensor bundle of that prefix,
+  and points the directory's `checkpoint` file at it."""
   lowering.copy_slices_to_masters()
   out = {}
   for variable, laid_out in lowering.variables.items():
@@ -92,6 +105,9 @@ def save_variables(lowering, path=None):
     if master.dtype == torch.bfloat16:
       master = master.float()
     out[variable.name] = master.cpu().numpy()
-  if path is not None:
+  if path is not None and path.endswith(".npz"):
     np.savez(path, **out)
+  elif path is not None:
+    tensor_bundle.write_bundle(path, out)
+    tensor_bundle.write_checkpoint_state(path)
   return out

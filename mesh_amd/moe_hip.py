@@ -22,12 +22,14 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 13
+ABI_VERSION = 14
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
     "mesh_moe_abi_version": (ctypes.c_int, []),
     "mesh_moe_last_error": (ctypes.c_char_p, []),
+    "mesh_moe_crc32c": (ctypes.c_uint32, [
+        ctypes.c_uint32, ctypes.c_void_p, ctypes.c_size_t]),
     "mesh_moe_router_logits": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, _vp]),

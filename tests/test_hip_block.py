@@ -2,6 +2,8 @@
 self-attention) and of a whole LayerStack with a MoE layer in it against
 oracle/block_oracle.py."""
 
+import os
+
 import numpy as np
 import pytest
 import torch
@@ -231,8 +233,9 @@ def test_layer_stack_bfloat16():
 
 
 def test_checkpoint_round_trip(tmp_path):
-  """Variables saved by name to an .npz archive and restored into a freshly
-  initialised lowering of the same graph reproduce the outputs; a filter
+  """Variables saved by name to an .npz archive, or to a tensor bundle, and
+  restored into a freshly initialised lowering of the same graph reproduce the
+  outputs; a filter
   restores only the matching names; a wrong shape raises."""
   from mesh_amd import checkpoint
   b, l, m, e, hdim, heads, d, group = 1, 32, 32, 4, 48, 2, 16, 32
@@ -270,6 +273,20 @@ def test_checkpoint_round_trip(tmp_path):
   assert not report.in_graph_not_in_checkpoint
   low_b.run()
   np.testing.assert_array_equal(H.to_np(low_b.export_to_tf_tensor(y_b)), out_a)
+  # the same through a TensorFlow tensor bundle: by prefix, then by directory
+  prefix = str(tmp_path / "run" / "model.ckpt-100")
+  checkpoint.save_variables(low_a, prefix)
+  assert os.path.exists(prefix + ".index")
+  assert os.path.exists(prefix + ".data-00000-of-00001")
+  for source in (prefix, str(tmp_path / "run")):
+    low_d, y_d = build()
+    report = checkpoint.restore_variables(low_d, source)
+    assert sorted(report.restored) == sorted(saved)
+    low_d.run()
+    np.testing.assert_array_equal(H.to_np(low_d.export_to_tf_tensor(y_d)),
+                                  out_a)
+  with pytest.raises(ValueError, match="no checkpoint state"):
+    checkpoint.restore_variables(low_b, str(tmp_path))
   low_c, _ = build()
   report = checkpoint.restore_variables(low_c, saved, variable_filter="MoE1D")
   assert sorted(report.restored) == sorted(n for n in saved if "MoE1D" in n)
