@@ -560,9 +560,12 @@ __global__ __launch_bounds__(256) void router_gate_kernel(
 // Gating step 2: capacity positions for one group per block (moe.py:1472-1496).
 // Thread (e = tid % EL, chunk = tid / EL) counts, over its chunk of the
 // group's tokens, those whose choice is expert e; an exclusive prefix over the
-// chunks gives each chunk's starting slot; a second walk assigns positions in
-// token order.  Second choices start after the kept first choices of the same
-// expert.  The token's expert ids live in LDS as int16 (-1 = not competing).
+// chunks gives the slot of each chunk's first chooser of e.  Then one thread
+// per token adds the number of earlier choosers of its expert inside its own
+// chunk: every lane runs the same short loop, where a walk per (expert, chunk)
+// would have each wave step through every token of the chunk.  Second choices
+// start after the kept first choices of the same expert.  The token's expert
+// ids live in LDS as int16 (-1 = not competing).
 // ---------------------------------------------------------------------------
 constexpr int CAP_THREADS = 1024;
 
@@ -598,7 +601,8 @@ __global__ __launch_bounds__(CAP_THREADS) void gate_capacity_kernel(
   extern __shared__ __attribute__((aligned(16))) int32_t smem_i[];
   const int S = p.S, E = p.E, C = p.C;
   int32_t* cnt = smem_i;                        // [nchunks][el] = CAP_THREADS
-  int32_t* tot = cnt + CAP_THREADS;             // [3][el]: total1,total2,loss2
+  int32_t* pre = cnt + CAP_THREADS;             // [nchunks][el]: first slots
+  int32_t* tot = pre + CAP_THREADS;             // [3][el]: total1,total2,loss2
   float* prod = reinterpret_cast<float*>(tot + 3 * el);  // [2][el]
   int16_t* c1 = reinterpret_cast<int16_t*>(prod + 2 * el);  // [S]
   int16_t* c2 = c1 + S;                                      // [S]
@@ -630,7 +634,7 @@ __global__ __launch_bounds__(CAP_THREADS) void gate_capacity_kernel(
   const int clen = (S + nchunks - 1) / nchunks;
   const int s_begin = min(S, chunk * clen);
   const int s_end = min(S, s_begin + clen);
-  // 16-byte reads of the id arrays: c1 starts 4096 + 20 * el bytes into LDS,
+  // 16-byte reads of the id arrays: c1 starts 8192 + 20 * el bytes into LDS,
   // c2 and c2l S and 2 S ids later, a chunk clen ids after the previous one
   const bool vec = (el % 4 == 0) && (S % 8 == 0) && (clen % 8 == 0);
 
@@ -645,26 +649,22 @@ __global__ __launch_bounds__(CAP_THREADS) void gate_capacity_kernel(
       total += v;
       if (k < chunk) before += v;
     }
-    int running = before + (choice == 0 ? 0 : count1);
-    const bool in_token_order = !(p.rank_by_gate && choice == 0);
-    for (int s = s_begin; in_token_order && s < s_end; ++s) {
-      // eight ids at a time where none of them is e (most of the time)
-      if (vec && (s & 7) == 0 && s + 8 <= s_end &&
-          cap_match8(*reinterpret_cast<const uint4*>(ch + s), e) == 0) {
-        s += 7;
-        continue;
-      }
-      if (ch[s] == e) {
-        int64_t t = base + s;
-        const bool ok = running < C;
-        pos[t * 2 + choice] = running;
-        kept[t * 2 + choice] = ok ? 1 : 0;
-        if (!ok) gate[t * 2 + choice] = gate[t * 2 + choice] * 0.0f;
-        ++running;
-      }
-    }
+    pre[chunk * el + e] = before + (choice == 0 ? 0 : count1);
     if (chunk == 0 && e < E) tot[choice * el + e] = total;
     if (choice == 0) count1 = min(total, C);
+    __syncthreads();
+    const bool in_token_order = !(p.rank_by_gate && choice == 0);
+    for (int s = tid; in_token_order && s < S; s += CAP_THREADS) {
+      const int ex = ch[s];
+      if (ex < 0) continue;
+      const int ck = s / clen;
+      const int slot = pre[ck * el + ex] + cap_count(ch, ck * clen, s, ex, vec);
+      const int64_t t = base + s;
+      const bool ok = slot < C;
+      pos[t * 2 + choice] = slot;
+      kept[t * 2 + choice] = ok ? 1 : 0;
+      if (!ok) gate[t * 2 + choice] = gate[t * 2 + choice] * 0.0f;
+    }
     __syncthreads();
   }
   if (p.rank_by_gate) {
@@ -883,7 +883,7 @@ static int launch_capacity_and_loss(const GateParams& p, int32_t* idx,
                                     float* gsum, hipStream_t st) {
   int el = 2;
   while (el < p.E) el *= 2;
-  size_t smem = sizeof(int32_t) * (CAP_THREADS + 3 * (size_t)el) +
+  size_t smem = sizeof(int32_t) * (2 * CAP_THREADS + 3 * (size_t)el) +
                 sizeof(float) * 2 * (size_t)el +
                 sizeof(int16_t) * (3 * (size_t)p.S + 1) +
                 (p.rank_by_gate ? sizeof(float) * (size_t)p.S : 0);
