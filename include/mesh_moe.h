@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 14
+#define MESH_MOE_ABI_VERSION 15
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -584,6 +584,23 @@ int mesh_moe_dispatch_backward(const void* dexpert_in, const int32_t* idx,
  * E = 1.
  * ---------------------------------------------------------------------------
  */
+
+/*
+ * Dropout whose noise is broadcast over some dimensions of x
+ * (mtf.dropout with a noise_shape, mesh_tensorflow/ops.py:5832-5872, as called by
+ * sublayer_dropout, transformer/transformer.py:590-599, by dense_relu_dense,
+ * layers.py:1176-1178, and on the attention weights, transformer/attention.py:82-84):
+ * x and out [outer, mid, inner], uniform / noise_in / noise_out [outer, inner].
+ *   out[o, m, i] = x[o, m, i] * noise[o, i]
+ *   noise = (uniform < keep_prob) ? 1 / keep_prob : 0   (threshold and quotient
+ *           rounded to `dtype`, as scalars of the tensor's type are there)
+ * or noise = noise_in (the backward pass: dx = dy * noise).  Exactly one of
+ * uniform and noise_in is non-NULL; noise_out may be NULL; out does not overlap x.
+ */
+int mesh_moe_broadcast_dropout(const void* x, const void* uniform,
+                               const void* noise_in, float keep_prob, void* out,
+                               void* noise_out, int64_t outer, int64_t mid,
+                               int64_t inner, int dtype, void* stream);
 
 /*
  * RMS normalisation (sublayer_rms_norm, transformer/transformer.py:493-516):

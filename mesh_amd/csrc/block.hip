@@ -213,9 +213,107 @@ static int run_attention(const T* q, const T* k, const T* v, T* out, int B,
   return 0;
 }
 
+// Dropout with the noise broadcast over the middle of three index ranges
+// (ops.py:5832-5872 with a noise_shape that leaves dimensions of x out):
+// out[o, m, i] = x[o, m, i] * noise[o, i], noise = (uniform < keep) ? 1 / keep
+// : 0, or `noise_in` as given.  One thread per (o, m) row piece of up to eight
+// consecutive i; bf16 rows whose length is a multiple of eight move 16 bytes.
+template <typename T>
+__global__ __launch_bounds__(256) void broadcast_dropout_kernel(
+    const T* __restrict__ x, const T* __restrict__ uniform,
+    const T* __restrict__ noise_in, float keep, float inv_keep,
+    T* __restrict__ out, T* __restrict__ noise_out, int64_t outer, int64_t mid,
+    int64_t inner, bool vec8) {
+  const int64_t step = vec8 ? 8 : 1;
+  const int64_t per_row = inner / step;
+  const int64_t total = outer * mid * per_row;
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t w = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; w < total;
+       w += stride) {
+    const int64_t i0 = (w % per_row) * step;
+    const int64_t om = w / per_row;
+    const int64_t o = om / mid;
+    const int64_t xi = om * inner + i0;
+    const int64_t ni = o * inner + i0;
+    const bool writes_noise = noise_out != nullptr && om % mid == 0;
+    if (vec8) {
+      const uint4 xv = *reinterpret_cast<const uint4*>(x + xi);
+      const uint4 sv = *reinterpret_cast<const uint4*>(
+          (noise_in ? noise_in : uniform) + ni);
+      const bf16_t* xs = reinterpret_cast<const bf16_t*>(&xv);
+      const bf16_t* ss = reinterpret_cast<const bf16_t*>(&sv);
+      uint4 ov, nv;
+      bf16_t* os = reinterpret_cast<bf16_t*>(&ov);
+      bf16_t* ns = reinterpret_cast<bf16_t*>(&nv);
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const float sj = load_f32<bf16_t>(ss + j);
+        const float noise = noise_in ? sj : (sj < keep ? inv_keep : 0.f);
+        store_f32<bf16_t>(ns + j, noise);
+        store_f32<bf16_t>(os + j, load_f32<bf16_t>(xs + j) * noise);
+      }
+      *reinterpret_cast<uint4*>(out + xi) = ov;
+      if (writes_noise) *reinterpret_cast<uint4*>(noise_out + ni) = nv;
+    } else {
+      const float sj = load_f32<T>((noise_in ? noise_in : uniform) + ni);
+      const float noise = noise_in ? sj : (sj < keep ? inv_keep : 0.f);
+      store_f32<T>(out + xi, load_f32<T>(x + xi) * noise);
+      if (writes_noise) store_f32<T>(noise_out + ni, noise);
+    }
+  }
+}
+
 }  // namespace mesh_moe
 
 using namespace mesh_moe;
+
+extern "C" int mesh_moe_broadcast_dropout(const void* x, const void* uniform,
+                                          const void* noise_in, float keep_prob,
+                                          void* out, void* noise_out,
+                                          int64_t outer, int64_t mid,
+                                          int64_t inner, int dtype,
+                                          void* stream) {
+  MOE_REQUIRE(x && out, MESH_MOE_E_ARG, "broadcast_dropout: null pointer");
+  MOE_REQUIRE((uniform != nullptr) != (noise_in != nullptr), MESH_MOE_E_ARG,
+              "broadcast_dropout: exactly one of uniform and noise_in");
+  MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG,
+              "broadcast_dropout: bad dtype %d", dtype);
+  MOE_REQUIRE(outer >= 1 && mid >= 1 && inner >= 1, MESH_MOE_E_ARG,
+              "broadcast_dropout: bad sizes %lld x %lld x %lld",
+              (long long)outer, (long long)mid, (long long)inner);
+  MOE_REQUIRE(noise_in || (keep_prob > 0.f && keep_prob <= 1.f), MESH_MOE_E_ARG,
+              "broadcast_dropout: keep_prob %g outside (0, 1]", keep_prob);
+  MOE_REQUIRE(outer <= (int64_t)1 << 40 && mid <= (int64_t)1 << 40 &&
+                  inner <= (int64_t)1 << 40 &&
+                  (double)outer * (double)mid * (double)inner < 9.0e18,
+              MESH_MOE_E_UNSUPPORTED, "broadcast_dropout: too many elements");
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == MESH_MOE_F32) {
+    const int64_t total = outer * mid * inner;
+    const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256
+                                                         : 65536);
+    broadcast_dropout_kernel<float><<<blocks, 256, 0, st>>>(
+        (const float*)x, (const float*)uniform, (const float*)noise_in,
+        keep_prob, 1.f / keep_prob, (float*)out, (float*)noise_out, outer, mid,
+        inner, false);
+  } else {
+    const uintptr_t ptrs = (uintptr_t)x | (uintptr_t)uniform |
+                           (uintptr_t)noise_in | (uintptr_t)out |
+                           (uintptr_t)noise_out;
+    const bool vec8 = inner % 8 == 0 && ptrs % 16 == 0;
+    const int64_t total = outer * mid * (vec8 ? inner / 8 : inner);
+    const int blocks = (int)((total + 255) / 256 < 65536 ? (total + 255) / 256
+                                                         : 65536);
+    // the threshold and 1 / keep_prob are scalars of the activation dtype
+    const float keep = round_bf16_host(keep_prob);
+    broadcast_dropout_kernel<bf16_t><<<blocks, 256, 0, st>>>(
+        (const bf16_t*)x, (const bf16_t*)uniform, (const bf16_t*)noise_in, keep,
+        round_bf16_host(1.f / keep), (bf16_t*)out, (bf16_t*)noise_out, outer,
+        mid, inner, vec8);
+  }
+  MOE_CHECK_LAUNCH("broadcast_dropout");
+  return 0;
+}
 
 extern "C" int mesh_moe_rms_norm(const void* x, const void* scale, void* y,
                                  int64_t rows, int M, double epsilon, int dtype,

@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 14
+ABI_VERSION = 15
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -102,6 +102,9 @@ _SIGNATURES = {
     "mesh_moe_expert_linear_backward": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
+    "mesh_moe_broadcast_dropout": (ctypes.c_int, [
+        _vp, _vp, _vp, ctypes.c_float, _vp, _vp, ctypes.c_int64, ctypes.c_int64,
+        ctypes.c_int64, ctypes.c_int, _vp]),
     "mesh_moe_activation": (ctypes.c_int, [
         _vp, _vp, ctypes.c_int64, ctypes.c_int, ctypes.c_int, _vp]),
     "mesh_moe_activation_backward": (ctypes.c_int, [
@@ -946,6 +949,37 @@ def slot_combine(y, r, group_size):
 
 
 # ---- the rest of a transformer block ----------------------------------------
+def broadcast_dropout(x, sizes, uniform=None, noise=None, keep_prob=1.0,
+                      want_noise=False):
+  """mtf.dropout with a noise_shape (ops.py:5832-5872).  x is contiguous and
+  is read as [outer, mid, inner] = sizes; uniform or noise has outer * inner
+  elements and is broadcast over mid.  Returns (out, noise or None)."""
+  lib = load_library()
+  outer, mid, inner = (int(v) for v in sizes)
+  if outer * mid * inner != x.numel():
+    raise MoeHipError("sizes %s do not cover %d elements"
+                      % ((outer, mid, inner), x.numel()))
+  if (uniform is None) == (noise is None):
+    raise MoeHipError("exactly one of uniform and noise")
+  dt = x.dtype
+  given = uniform if uniform is not None else noise
+  if given.numel() != outer * inner:
+    raise MoeHipError("noise has %d elements, expected %d"
+                      % (given.numel(), outer * inner))
+  out = torch.empty_like(x)
+  noise_out = (torch.empty_like(uniform)
+               if (want_noise and uniform is not None) else None)
+  with _stage("broadcast_dropout"):
+    _check(lib.mesh_moe_broadcast_dropout(
+        _dev(x, "x"),
+        _dev(uniform, "uniform", dt) if uniform is not None else None,
+        _dev(noise, "noise", dt) if noise is not None else None,
+        float(keep_prob), out.data_ptr(),
+        noise_out.data_ptr() if noise_out is not None else None,
+        outer, mid, inner, dtype_code(dt), _stream()), "broadcast_dropout")
+  return out, (noise_out if uniform is not None else noise)
+
+
 def rms_norm(x, scale, epsilon=1e-6):
   """x [..., M], scale [M] of x's dtype -> x * rsqrt(mean(x^2) + eps) * scale
   (sublayer_rms_norm, transformer/transformer.py:493-516)."""

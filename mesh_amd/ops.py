@@ -971,6 +971,109 @@ def relu(x, name="relu"):
   return cwise(torch.relu, [x], name=name)
 
 
+def _dropout_sizes(shape, noise_shape):
+  """x's dimensions as (outer, mid, inner) sizes, `mid` covering the one run of
+  consecutive dimensions that noise_shape leaves out."""
+  missing = [d for d in noise_shape.dims if d not in shape.dims]
+  if missing:
+    raise ValueError("noise_shape %s is not a subset of %s"
+                     % (noise_shape, shape))
+  flags = [d in noise_shape.dims for d in shape.dims]
+  if [d for d in shape.dims if d in noise_shape.dims] != noise_shape.dims:
+    raise NotImplementedError(
+        "dropout noise_shape %s orders its dimensions differently from %s"
+        % (noise_shape, shape))
+  if all(flags):
+    return 1, 1, shape.size
+  first = flags.index(False)
+  last = len(flags) - 1 - flags[::-1].index(False)
+  if any(flags[first:last + 1]):
+    raise NotImplementedError(
+        "dropout noise broadcast over dimensions of %s that are not "
+        "consecutive (noise_shape %s)" % (shape, noise_shape))
+  sizes = shape.to_integer_list
+  return (list_product(sizes[:first]), list_product(sizes[first:last + 1]),
+          list_product(sizes[last + 1:]))
+
+
+class DropoutOperation(Operation):
+  """x * noise, noise = (uniform < keep_prob) / keep_prob drawn in x's dtype
+  over noise_shape and broadcast over x's other dimensions
+  (mesh_tensorflow/ops.py:5832-5872).  The uniform numbers come from torch's
+  generator on the device, or from `uniform` (a tensor of outer * inner
+  elements) when it is set before lowering; `noise` holds the multiplier of
+  the last lowering."""
+
+  def __init__(self, x, keep_prob, noise_shape, name=None):
+    # checked first: a constructor that raises must not leave its operation
+    # in the graph
+    self.sizes = _dropout_sizes(x.shape, noise_shape)
+    super(DropoutOperation, self).__init__([x], name=name or "dropout")
+    self.keep_prob = keep_prob
+    self.noise_shape = noise_shape
+    self._outputs = [Tensor(self, x.shape, x.dtype)]
+    self.uniform = None
+    self.noise = None
+
+  def gradient(self, grad_ys):
+    return [DropoutGradOperation(self, grad_ys[0]).outputs[0]]
+
+  def lower(self, lowering):
+    from mesh_amd import moe_hip  # pylint: disable=g-import-not-at-top
+    outer, _, inner = self.sizes
+
+    def fn(t):
+      u = self.uniform
+      if u is None:
+        u = torch.rand((outer, inner), dtype=t.dtype, device=t.device)
+      out, self.noise = moe_hip.broadcast_dropout(
+          t.contiguous(), self.sizes, uniform=u.to(t.dtype).contiguous(),
+          keep_prob=self.keep_prob, want_noise=True)
+      return out
+    lowering.set_tensor_lowering(
+        self.outputs[0], lowering.mesh_impl(self).slicewise(
+            fn, lowering.tensors[self.inputs[0]]))
+
+
+class DropoutGradOperation(Operation):
+  """dx = dy * noise with the multiplier the forward lowering drew."""
+
+  def __init__(self, forward, dy, name=None):
+    super(DropoutGradOperation, self).__init__(
+        [dy, forward.outputs[0]], name=name or "dropout_grad")
+    self._forward = forward
+    self._outputs = [Tensor(self, dy.shape, dy.dtype)]
+
+  def lower(self, lowering):
+    from mesh_amd import moe_hip  # pylint: disable=g-import-not-at-top
+    forward = self._forward
+
+    def fn(dy, unused_y):
+      return moe_hip.broadcast_dropout(dy.contiguous(), forward.sizes,
+                                       noise=forward.noise)[0]
+    lowering.set_tensor_lowering(
+        self.outputs[0], lowering.mesh_impl(self).slicewise(
+            fn, *[lowering.tensors[x] for x in self.inputs]))
+
+
+def dropout(x, is_training, keep_prob=None, rate=None, noise_shape=None,
+            name=None):
+  """mtf.dropout (mesh_tensorflow/ops.py:5832-5872): identity unless training;
+  kept elements are scaled by 1 / keep_prob."""
+  if (keep_prob is None) == (rate is None):
+    raise ValueError("exactly one of keep_prob and rate should be set")
+  if keep_prob is None:
+    keep_prob = 1.0 - rate
+  noise_shape = convert_to_shape(noise_shape)
+  if noise_shape is None:
+    noise_shape = x.shape
+  if keep_prob == 1.0 or not is_training:
+    return x
+  if not x.dtype.is_floating_point:
+    raise NotImplementedError("dropout of an integer tensor")
+  return DropoutOperation(x, keep_prob, noise_shape, name=name).outputs[0]
+
+
 def to_numpy(t):
   """Torch tensor -> float32/int NumPy array on the host."""
   t = t.detach()

@@ -179,11 +179,13 @@ def sublayer_residual(x, layer_stack, context):
 
 
 def sublayer_dropout(x, layer_stack, context, dropout_rate=0.0):
-  """transformer.py:590-599; dropout while training draws random numbers and
-  is not implemented."""
+  """transformer.py:590-599: while training, one noise value per (batch
+  entry, channel), shared by the positions of a sequence."""
   del layer_stack
   if context.train and dropout_rate > 0:
-    raise NotImplementedError("dropout while training is not implemented")
+    return mtf.dropout(
+        x, context.train, rate=dropout_rate,
+        noise_shape=mtf.Shape(context.batch_dims + [context.model.model_dim]))
   return x
 
 

@@ -30,8 +30,9 @@ class DenseReluDense(transformer.TransformerLayer):
         x, reduced_dims=x.shape.dims[-1:], new_dims=hidden_channels,
         activation_functions=self.activation, use_bias=self.use_bias,
         variable_dtype=context.variable_dtype, name="wi")
-    if context.train and self.dropout_rate != 0.0:
-      raise NotImplementedError("dropout while training is not implemented")
+    if context.train and self.dropout_rate != 0.0:   # transformer_layers.py:67-69
+      h = mtf.dropout(h, context.train, keep_prob=1.0 - self.dropout_rate,
+                      noise_shape=h.shape - context.length_dim)
     return mtf_layers.dense(
         h, io_channels, use_bias=self.use_bias, activation=None,
         variable_dtype=context.variable_dtype, reduced_dims=h.shape.dims[-1:],
@@ -83,11 +84,23 @@ class SelfAttention(transformer.TransformerLayer):
         shared_kv=self.shared_kv, ensemble_dim=context.model.ensemble_dim,
         fold_scaling_into_initializer=self.fold_scaling_into_initializer)
 
+  def _attention_dropout(self, context, v, num_heads):
+    """Dropout of the attention weights with one noise value per (batch entry,
+    head, memory position), shared by the queries (attention.py:82-84 with
+    dropout_broadcast_dims = [length], transformer_layers.py:210-212):
+    sum_k weights[b,h,q,k] * noise[b,h,k] * v[b,k,h,:] is the undropped
+    attention over v * noise, so the noise goes onto the values."""
+    batch_length = v.shape.dims[:-1]
+    heads = mtf.Dimension("heads", num_heads)
+    per_head = mtf.Dimension("d_kv", v.shape.dims[-1].size // num_heads)
+    split = mtf.reshape(v, mtf.Shape(batch_length + [heads, per_head]))
+    split = mtf.dropout(split, context.train, keep_prob=1.0 - self.dropout_rate,
+                        noise_shape=mtf.Shape(batch_length + [heads]))
+    return mtf.reshape(split, v.shape)
+
   def call(self, context, x, losses=None):
     """transformer_layers.py:223-271 for the train / eval modes."""
     del losses
-    if context.train and self.dropout_rate != 0.0:
-      raise NotImplementedError("dropout while training is not implemented")
     if isinstance(context.sequence_id, mtf.Tensor) or isinstance(
         context.subsequence_id, mtf.Tensor):
       raise NotImplementedError("sequence_id tensors are not implemented")
@@ -100,6 +113,8 @@ class SelfAttention(transformer.TransformerLayer):
       v = params.compute_v(x)
     # read_priority >= write_priority (transformer_layers.py:289-296)
     causal = context.read_priority is transformer.POSITION
+    if context.train and self.dropout_rate != 0.0:
+      v = self._attention_dropout(context, v, params.num_heads)
     o = attention.SelfAttentionOperation(q, k, v, params.num_heads,
                                          causal).outputs[0]
     return params.compute_output(o, output_shape=x.shape)

@@ -16,6 +16,9 @@ moe_oracle.  What pins each function (tests/test_block_oracle.py):
                    queries give the running mean of the values
   layer_stack      zero output kernels reduce the stack to its final norm;
                    one layer by hand
+  dropout noise    (broadcast_dropout and the noise arguments) noise of ones
+                   is the identity; float64 product; noise on the attention
+                   weights equals noise on the values
 
 PARITY UNPINNED against TensorFlow itself: the order of float32 accumulation
 inside TF's reductions and matmuls, and for bfloat16 whether TF's reduce_sum
@@ -64,7 +67,16 @@ def dense(x, w, act_dtype="float32", activation=None):
   return y
 
 
-def self_attention(x, wq, wk, wv, wo, num_heads, causal, act_dtype="float32"):
+def broadcast_dropout(x, noise, axis, act_dtype="float32"):
+  """mtf.dropout's product x * noise (ops.py:5872) with the noise broadcast
+  over `axis` of x (a noise_shape without that dimension); `noise` is
+  O.hidden_dropout_noise of the uniform draw."""
+  return _r(_r(x, act_dtype) * np.expand_dims(_r(noise, act_dtype), axis),
+            act_dtype)
+
+
+def self_attention(x, wq, wk, wv, wo, num_heads, causal, act_dtype="float32",
+                   weights_noise=None):
   """SelfAttention.call for the train / eval modes with the default options
   (transformer/transformer_layers.py:223-271) around attention.attention with
   float32 logits (transformer/attention.py:27-88).
@@ -74,7 +86,9 @@ def self_attention(x, wq, wk, wv, wo, num_heads, causal, act_dtype="float32"):
   not visible, attention.py:830-842; the bias is cast to the logits' dtype,
   :78-79); weights = mtf.softmax(logits) in float32, cast to the activation
   dtype; outputs = weights . v.  No 1/sqrt(d_kv) factor: it is folded into the
-  initialiser of wq (attention.py:436-439).
+  initialiser of wq (attention.py:436-439).  weights_noise [B, H, L]: the
+  dropout multiplier of the weights, one value per memory position, shared by
+  the queries (attention.py:82-84 with dropout_broadcast_dims = [length]).
   """
   x = _r(x, act_dtype)
   b, l, _ = x.shape
@@ -89,6 +103,8 @@ def self_attention(x, wq, wk, wv, wo, num_heads, causal, act_dtype="float32"):
     hidden = (pos[None, :] > pos[:, None]).astype(F32)           # key > query
     logits = logits + hidden * F32(-1e9)
   weights = _r(O.softmax(logits), act_dtype)                     # cast to v's
+  if weights_noise is not None:
+    weights = broadcast_dropout(weights, weights_noise, 2, act_dtype)
   o = _r(np.einsum("bhlm,bmhd->blhd", weights, v), act_dtype)
   return dense(o.reshape(b, l, hd), wo, act_dtype)
 
@@ -129,16 +145,28 @@ def experts_self_attention(x, w_gate, wi, q_wo, k_wo, wo, hparams, num_heads,
   return dense(o, wo, act_dtype), loss
 
 
-def dense_relu_dense(x, wi, wo, act_dtype="float32"):
-  """DenseReluDense.call (transformer/transformer_layers.py:55-76)."""
-  return dense(dense(x, wi, act_dtype, "relu"), wo, act_dtype)
+def dense_relu_dense(x, wi, wo, act_dtype="float32", hidden_noise=None):
+  """DenseReluDense.call (transformer/transformer_layers.py:55-76);
+  hidden_noise [B, d_ff]: the dropout multiplier of the hidden tensor, shared
+  by the positions of a sequence (:67-69)."""
+  h = dense(x, wi, act_dtype, "relu")
+  if hidden_noise is not None:
+    h = broadcast_dropout(h, hidden_noise, -2, act_dtype)
+  return dense(h, wo, act_dtype)
 
 
 def layer_stack(x, layers, final_scale, act_dtype="float32",
-                autoregressive=False, train=False):
+                autoregressive=False, train=False, initial_noise=None,
+                final_noise=None):
   """LayerStack.call with the default sublayers (transformer/transformer.py:
   408-428 and the defaults quoted at :346-358): per layer
-  x + layer(rms_norm(x)); a final rms_norm.  Dropout rates are 0.
+  dropout(x) first; per layer x + dropout(layer(rms_norm(x))); at the end
+  dropout(rms_norm(x)).  Each dropout multiplies by a noise tensor
+  [B, d_model] shared by the positions of a sequence (sublayer_dropout,
+  transformer.py:590-599) and is skipped when its noise is None:
+  initial_noise, final_noise, and per layer "sublayer_noise"; a layer's own
+  dropout takes "weights_noise" (attention) or "hidden_noise"
+  (dense_relu_dense).
 
   layers: list of dicts with "kind" in {"attention", "dense_relu_dense",
   "moe"}, "scale" (the layer's rms_norm scale) and the layer's weights:
@@ -148,15 +176,19 @@ def layer_stack(x, layers, final_scale, act_dtype="float32",
   Returns (y, losses) with one loss per MoE layer.
   """
   x = _r(x, act_dtype)
+  if initial_noise is not None:
+    x = broadcast_dropout(x, initial_noise, -2, act_dtype)
   losses = []
   for layer in layers:
     h = rms_norm(x, layer["scale"], act_dtype)
     kind = layer["kind"]
     if kind == "attention":
       y = self_attention(h, layer["wq"], layer["wk"], layer["wv"], layer["wo"],
-                         layer["num_heads"], autoregressive, act_dtype)
+                         layer["num_heads"], autoregressive, act_dtype,
+                         layer.get("weights_noise"))
     elif kind == "dense_relu_dense":
-      y = dense_relu_dense(h, layer["wi"], layer["wo"], act_dtype)
+      y = dense_relu_dense(h, layer["wi"], layer["wo"], act_dtype,
+                           layer.get("hidden_noise"))
     elif kind == "moe":
       y, loss, _ = O.moe_layer_v1(
           h, layer["w_gate"], layer["wi"], layer["wo"], layer["hparams"],
@@ -165,5 +197,10 @@ def layer_stack(x, layers, final_scale, act_dtype="float32",
       losses.append(loss)
     else:
       raise ValueError("layer kind %r" % (kind,))
+    if layer.get("sublayer_noise") is not None:
+      y = broadcast_dropout(y, layer["sublayer_noise"], -2, act_dtype)
     x = _r(y + x, act_dtype)                                     # residual
-  return rms_norm(x, final_scale, act_dtype), losses
+  y = rms_norm(x, final_scale, act_dtype)
+  if final_noise is not None:
+    y = broadcast_dropout(y, final_noise, -2, act_dtype)
+  return y, losses

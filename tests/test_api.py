@@ -500,8 +500,13 @@ def test_block_rejections():
       [(transformer_layers.DenseReluDense,
         dict(hidden_size=8, dropout_rate=0.1))], num_layers=1)
   model = transformer.Unitransformer(stack, d_model=16)
-  with pytest.raises(NotImplementedError, match="dropout"):
-    model.call_layers(x, vdt, mode="train")
+  # dropout while training builds mtf.dropout with the noise shared along length
+  y, _ = model.call_layers(x, vdt, mode="train")
+  drops = [op for op in graph.operations
+           if isinstance(op, mtf.DropoutOperation)]
+  assert len(drops) == 1 and drops[0].keep_prob == 0.9
+  assert drops[0].noise_shape.dimension_names == ["batch", "d_ff"]
+  assert drops[0].sizes == (1, 8, 8) and y.shape == x.shape
   ctx = transformer.Context(model, mesh, dims[:1], dims[1], vdt, sequence_id=1)
   assert ctx.nonpadding == 1 and not isinstance(ctx.nonpadding, mtf.Tensor)
   with pytest.raises(ValueError, match="does not end in"):

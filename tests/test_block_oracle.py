@@ -160,3 +160,62 @@ def test_layer_stack_by_hand_and_zero_kernels():
     zeroed.append(z)
   y0, _ = B.layer_stack(x, zeroed, final)
   np.testing.assert_array_equal(y0, B.rms_norm(x, final))
+
+
+def test_dropout_noise_arguments():
+  """The dropout hooks of the block oracle: noise of ones changes nothing; the
+  product against float64; noise on the attention weights (what the reference
+  does) equals noise on the values (what the fused kernel is given)."""
+  rng = np.random.default_rng(9)
+  b, l, m, heads, d, hid = 2, 10, 16, 2, 4, 12
+  x = rng.standard_normal((b, l, m)).astype(np.float32)
+  noise = O.hidden_dropout_noise(rng.random((b, m)), 0.75, "float32")
+  assert set(np.unique(noise)) == {np.float32(0), np.float32(1 / 0.75)}
+  got = B.broadcast_dropout(x, noise, -2)
+  np.testing.assert_allclose(got, x.astype(np.float64) * noise[:, None, :],
+                             rtol=1e-6)
+  assert (got[:, :, noise[0] == 0][0] == 0).all()
+  np.testing.assert_array_equal(B.broadcast_dropout(x, np.ones((b, m)), -2), x)
+  # bf16: threshold and quotient are bf16 scalars
+  nb = O.hidden_dropout_noise(rng.random((b, m)), 0.9, "bfloat16")
+  assert set(np.unique(nb)) <= {np.float32(0), np.float32(1.109375)}
+  wq, wk, wv = (rng.standard_normal((m, heads * d)).astype(np.float32) / 3
+                for _ in range(3))
+  wo = rng.standard_normal((heads * d, m)).astype(np.float32) / 3
+  ones = np.ones((b, heads, l), np.float32)
+  np.testing.assert_array_equal(
+      B.self_attention(x, wq, wk, wv, wo, heads, True, weights_noise=ones),
+      B.self_attention(x, wq, wk, wv, wo, heads, True))
+  wn = O.hidden_dropout_noise(rng.random((b, heads, l)), 0.6, "float32")
+  got = B.self_attention(x, wq, wk, wv, wo, heads, False, weights_noise=wn)
+  # float64, with the noise on the values instead: v[b, k, h, :] * noise[b, h, k]
+  x64 = x.astype(np.float64)
+  want = np.zeros((b, l, heads * d))
+  for bi in range(b):
+    for h in range(heads):
+      sl = slice(h * d, (h + 1) * d)
+      q, k, v = x64[bi] @ wq[:, sl], x64[bi] @ wk[:, sl], x64[bi] @ wv[:, sl]
+      want[bi, :, sl] = scipy.special.softmax(q @ k.T, axis=-1) @ (
+          v * wn[bi, h][:, None])
+  np.testing.assert_allclose(got, want @ wo.astype(np.float64), rtol=2e-5,
+                             atol=2e-5)
+  wi = rng.standard_normal((m, hid)).astype(np.float32) / 4
+  wo2 = rng.standard_normal((hid, m)).astype(np.float32) / 4
+  hn = O.hidden_dropout_noise(rng.random((b, hid)), 0.5, "float32")
+  got = B.dense_relu_dense(x, wi, wo2, hidden_noise=hn)
+  want = (np.maximum(x64 @ wi, 0) * hn[:, None, :]) @ wo2
+  np.testing.assert_allclose(got, want, rtol=2e-5, atol=2e-5)
+  # the stack: by hand with one dense layer
+  scale = np.ones(m, np.float32)
+  layer = dict(kind="dense_relu_dense", scale=scale, wi=wi, wo=wo2,
+               hidden_noise=hn, sublayer_noise=noise)
+  first = O.hidden_dropout_noise(rng.random((b, m)), 0.8, "float32")
+  last = O.hidden_dropout_noise(rng.random((b, m)), 0.8, "float32")
+  y, _ = B.layer_stack(x, [layer], scale, initial_noise=first, final_noise=last)
+  h = B.broadcast_dropout(x, first, -2)
+  h = h + B.broadcast_dropout(
+      B.dense_relu_dense(B.rms_norm(h, scale), wi, wo2, hidden_noise=hn),
+      noise, -2)
+  np.testing.assert_allclose(
+      y, B.broadcast_dropout(B.rms_norm(h, scale), last, -2), rtol=1e-6,
+      atol=1e-6)

@@ -393,3 +393,178 @@ def test_experts_self_attention_layer(case):
         num_layers=1, block_scope=False)
     transformer.Unitransformer(st2, d_model=m, name="decoder").call_layers(
         x2, mtf.VariableDType(torch.float32), mode="eval")
+
+
+@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
+def test_broadcast_dropout_entry(hip, act_dtype):
+  """mesh_moe_broadcast_dropout: x [outer, mid, inner] times the noise of a
+  uniform draw [outer, inner], against the oracle; then the same multiplier
+  passed back in (the backward pass)."""
+  dt = H.ACT_TORCH[act_dtype]
+  rng = np.random.default_rng(41)
+  for outer, mid, inner, keep in ((3, 5, 16, 0.75), (2, 7, 24, 0.9),
+                                  (6, 4, 1, 0.5), (1, 1, 40, 0.9),
+                                  (2, 3, 5, 0.6), (4, 33, 256, 0.9)):
+    x = O.cast_act(rng.standard_normal((outer, mid, inner)).astype(np.float32),
+                   act_dtype)
+    u = O.cast_act(rng.random((outer, inner)).astype(np.float32), act_dtype)
+    noise = O.hidden_dropout_noise(u, keep, act_dtype)
+    want = B.broadcast_dropout(x, noise, 1, act_dtype)
+    xt = torch.from_numpy(x).to(dt).cuda()
+    got, got_noise = hip.broadcast_dropout(
+        xt, (outer, mid, inner), uniform=torch.from_numpy(u).to(dt).cuda(),
+        keep_prob=keep, want_noise=True)
+    np.testing.assert_array_equal(H.to_np(got_noise), noise)
+    np.testing.assert_array_equal(H.to_np(got), want)
+    assert 0 < (noise == 0).sum() < noise.size or noise.size < 8
+    dy = O.cast_act(rng.standard_normal(x.shape).astype(np.float32), act_dtype)
+    back, same = hip.broadcast_dropout(torch.from_numpy(dy).to(dt).cuda(),
+                                       (outer, mid, inner), noise=got_noise)
+    assert same is got_noise
+    np.testing.assert_array_equal(
+        H.to_np(back), B.broadcast_dropout(dy, noise, 1, act_dtype))
+  with pytest.raises(hip.MoeHipError, match="exactly one"):
+    hip.broadcast_dropout(xt, (4, 33, 256))
+  with pytest.raises(hip.MoeHipError, match="do not cover"):
+    hip.broadcast_dropout(xt, (4, 33, 255), noise=got_noise)
+  with pytest.raises(hip.MoeHipError, match="keep_prob"):
+    hip.broadcast_dropout(xt, (4, 33, 256),
+                          uniform=torch.zeros((4, 256), dtype=dt,
+                                              device="cuda"), keep_prob=0.0)
+
+
+def test_dropout_operation_and_gradient():
+  """mtf.dropout through the graph: noise shared along `length`, the saved
+  multiplier, the gradient, and the cases that return x or raise."""
+  b, l, m = 2, 6, 16
+  rng = np.random.default_rng(42)
+  x = rng.standard_normal((b, l, m)).astype(np.float32)
+  dy = rng.standard_normal((b, l, m)).astype(np.float32)
+  u = rng.random((b, m)).astype(np.float32)
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  dims = [mtf.Dimension("batch", b), mtf.Dimension("length", l),
+          mtf.Dimension("d_model", m)]
+  xt = mtf.import_tf_tensor(mesh, torch.from_numpy(x), mtf.Shape(dims))
+  dyt = mtf.import_tf_tensor(mesh, torch.from_numpy(dy), mtf.Shape(dims))
+  assert mtf.dropout(xt, False, rate=0.5) is xt
+  assert mtf.dropout(xt, True, keep_prob=1.0) is xt
+  with pytest.raises(ValueError, match="exactly one"):
+    mtf.dropout(xt, True)
+  with pytest.raises(ValueError, match="exactly one"):
+    mtf.dropout(xt, True, keep_prob=0.5, rate=0.5)
+  with pytest.raises(ValueError, match="not a subset"):
+    mtf.dropout(xt, True, rate=0.5,
+                noise_shape=mtf.Shape([mtf.Dimension("other", 3)]))
+  y = mtf.dropout(xt, True, rate=0.25,
+                  noise_shape=mtf.Shape([dims[0], dims[2]]))
+  op = y.operation
+  assert op.sizes == (b, l, m)
+  op.uniform = torch.from_numpy(u).cuda()
+  y_all = mtf.dropout(xt, True, keep_prob=0.5)            # noise of x's shape
+  assert y_all.operation.sizes == (1, 1, b * l * m)
+  y_last = mtf.dropout(xt, True, keep_prob=0.5,
+                       noise_shape=mtf.Shape(dims[:2]))   # shared by channels
+  assert y_last.operation.sizes == (b * l, m, 1)
+  (dx,) = mtf.gradients([y], [xt], [dyt])
+  lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()})
+  noise = O.hidden_dropout_noise(u, 0.75, "float32")
+  np.testing.assert_array_equal(H.to_np(op.noise), noise)
+  np.testing.assert_array_equal(H.to_np(lowering.export_to_tf_tensor(y)),
+                                B.broadcast_dropout(x, noise, 1))
+  np.testing.assert_array_equal(H.to_np(lowering.export_to_tf_tensor(dx)),
+                                B.broadcast_dropout(dy, noise, 1))
+  got = H.to_np(lowering.export_to_tf_tensor(y_all))
+  n_all = H.to_np(y_all.operation.noise).reshape(x.shape)
+  assert set(np.unique(n_all)) == {0.0, 2.0}
+  np.testing.assert_array_equal(got, x * n_all)
+  got = H.to_np(lowering.export_to_tf_tensor(y_last))
+  n_last = H.to_np(y_last.operation.noise).reshape(b, l, 1)
+  np.testing.assert_array_equal(got, x * n_last)
+  # a 4-d tensor with noise over dimensions 0 and 2 leaves two separate runs out
+  graph2 = mtf.Graph()
+  mesh2 = mtf.Mesh(graph2, "mesh")
+  d4 = dims + [mtf.Dimension("extra", 2)]
+  x4 = mtf.import_tf_tensor(mesh2, torch.zeros((b, l, m, 2)), mtf.Shape(d4))
+  with pytest.raises(NotImplementedError, match="not consecutive"):
+    mtf.dropout(x4, True, rate=0.5, noise_shape=mtf.Shape([d4[0], d4[2]]))
+
+
+def test_layer_stack_with_dropout():
+  """A training-mode stack with every dropout of the block switched on: the
+  sublayer dropouts (noise per batch entry and channel), the attention
+  weights' (noise per batch entry, head and memory position, applied to the
+  values here) and DenseReluDense's hidden one; the oracle gets the multipliers
+  the lowering drew."""
+  import functools
+  b, l, m, e, hdim, heads, d, group = 2, 64, 64, 4, 96, 4, 16, 32
+  rng = np.random.default_rng(43)
+  layers, final = _build_stack(rng, m, e, hdim, heads, d, group)
+  layers = [layers[0], layers[3], layers[1]]      # attention, dense, MoE
+  x = rng.standard_normal((b, l, m)).astype(np.float32)
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  dims = [mtf.Dimension("batch", b), mtf.Dimension("length", l),
+          mtf.Dimension("d_model", m)]
+  xt = mtf.import_tf_tensor(mesh, torch.from_numpy(x), mtf.Shape(dims))
+  drop = functools.partial(transformer.sublayer_dropout, dropout_rate=0.2)
+  stack_cls = functools.partial(
+      transformer.LayerStack, sublayers_initial=[drop],
+      sublayers_per_layer=[transformer.sublayer_rms_norm,
+                           transformer.sublayer_call_layer, drop,
+                           transformer.sublayer_residual],
+      sublayers_final=[transformer.sublayer_rms_norm, drop])
+  stack = transformer.make_layer_stack(
+      [(transformer_layers.SelfAttention,
+        dict(num_heads=heads, key_value_size=d, dropout_rate=0.3)),
+       (transformer_layers.DenseReluDense,
+        dict(hidden_size=hdim, dropout_rate=0.4)),
+       (moe.MoE1D, dict(num_experts=e, hidden_size=hdim, group_size=group,
+                        second_policy_train="all", second_policy_eval="all",
+                        capacity_factor_train=2.0))],
+      num_layers=1, block_scope=False, layer_stack_cls=stack_cls)
+  model = transformer.Unitransformer(stack, d_model=m, name="decoder",
+                                     autoregressive=True)
+  y, losses = model.call_layers(
+      xt, mtf.VariableDType(torch.float32), mode="train")
+  init = {"decoder/rms_norm/scale": final}
+  for i, (layer, cls) in enumerate(zip(layers, ("SelfAttention",
+                                                "DenseReluDense", "MoE1D"))):
+    p = "decoder/layer_%03d/" % i
+    init[p + "rms_norm/scale"] = layer["scale"]
+    if cls == "SelfAttention":
+      for k in "qkvo":
+        init[p + cls + "/" + k] = layer["w" + k]
+    elif cls == "MoE1D":
+      init[p + cls + "/top_2_gating/kernel"] = layer["w_gate"]
+      init[p + cls + "/wi/kernel"] = layer["wi"]
+      init[p + cls + "/wo/kernel"] = layer["wo"]
+    else:
+      init[p + cls + "/wi/kernel"] = layer["wi"]
+      init[p + cls + "/wo/kernel"] = layer["wo"]
+  lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()}, initial_values=init)
+  got = H.to_np(lowering.export_to_tf_tensor(y))
+  drops = [op for op in graph.operations
+           if isinstance(op, mtf.DropoutOperation)]
+  # graph order: initial; attention's, its sublayer's; hidden, its sublayer's;
+  # the MoE layer's sublayer's; final
+  assert [op.keep_prob for op in drops] == [0.8, 0.7, 0.8, 0.6, 0.8, 0.8, 0.8]
+  noises = [H.to_np(op.noise) for op in drops]
+  assert noises[1].shape == (b * l * heads, 1)
+  layers[0] = dict(layers[0], sublayer_noise=noises[2],
+                   weights_noise=noises[1].reshape(b, l, heads).transpose(
+                       0, 2, 1))
+  layers[1] = dict(layers[1], hidden_noise=noises[3], sublayer_noise=noises[4])
+  hp = O.default_hparams(
+      moe_num_experts=e, moe_hidden_size=hdim, moe_group_size=group,
+      moe_second_policy_eval="all", moe_second_policy_train="all",
+      moe_capacity_factor_train=2.0)
+  layers[2] = dict(layers[2], sublayer_noise=noises[5], hparams=hp)
+  want, want_loss = B.layer_stack(x, layers, final, "float32", True, True,
+                                  initial_noise=noises[0],
+                                  final_noise=noises[6])
+  for noise, keep in zip(noises, (0.8, 0.7, 0.8, 0.6, 0.8, 0.8, 0.8)):
+    assert 0.3 < (noise == 0).mean() / (1 - keep) < 2.0
+  np.testing.assert_allclose(got, want, rtol=2e-4, atol=2e-4)
+  got_loss = [float(H.to_np(lowering.export_to_tf_tensor(t))) for t in losses]
+  np.testing.assert_allclose(got_loss, want_loss, rtol=1e-4)
