@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 15
+#define MESH_MOE_ABI_VERSION 16
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -584,6 +584,41 @@ int mesh_moe_dispatch_backward(const void* dexpert_in, const int32_t* idx,
  * E = 1.
  * ---------------------------------------------------------------------------
  */
+
+/*
+ * Backward passes of the block's operations.  The reference has no code for
+ * them: mtf.gradients differentiates the einsum, reduce and cwise operations
+ * these forward kernels fuse (mesh_tensorflow/ops.py:2846-2854 einsum,
+ * :1478-1482 gradient hook), so each entry states the derivative it computes.
+ * Float32 arithmetic on the stored operands, one rounding to `dtype`.
+ *
+ * mesh_moe_rms_norm_backward (sublayer_rms_norm, transformer/transformer.py:
+ * 493-516): y = x * r * scale with r = rsqrt(mean(x^2) + epsilon);
+ *   dx = r * g - x * r^3 * mean(g * x),  g = dy * scale;   dscale = sum_rows dy * x * r.
+ * x, dy, dx [rows, M]; scale, dscale [M].
+ *
+ * mesh_moe_softmax_backward (mtf.softmax, ops.py:5539-5541): from the output w,
+ *   dlogits = w * (dw - sum_k dw * w) over the last dim; [rows, L] each.
+ *
+ * mesh_moe_attention_weights (transformer/attention.py:76-81): the weights
+ * softmax(q . k + visibility) the fused forward kernel never stores, recomputed
+ * for the backward pass: q, k [B, L, H*D] -> weights [B*H, L, L] in `dtype`
+ * (float32 logits and softmax, as in the forward pass).
+ */
+size_t mesh_moe_rms_norm_backward_workspace_bytes(int64_t rows, int M);
+int mesh_moe_rms_norm_backward(const void* x, const void* scale, const void* dy,
+                               void* dx, void* dscale, int64_t rows, int M,
+                               double epsilon, int dtype, void* workspace,
+                               size_t workspace_bytes, void* stream);
+int mesh_moe_softmax_backward(const void* weights, const void* dweights,
+                              void* dlogits, int64_t rows, int L, int dtype,
+                              void* stream);
+size_t mesh_moe_attention_weights_workspace_bytes(int B, int L, int H, int D,
+                                                  int dtype);
+int mesh_moe_attention_weights(const void* q, const void* k, void* weights,
+                               int B, int L, int H, int D, int causal,
+                               int dtype, void* workspace,
+                               size_t workspace_bytes, void* stream);
 
 /*
  * Dropout whose noise is broadcast over some dimensions of x

@@ -213,6 +213,129 @@ static int run_attention(const T* q, const T* k, const T* v, T* out, int B,
   return 0;
 }
 
+// ---------------------------------------------------------------------------
+// Backward of the RMS norm y = x * r * scale, r = rsqrt(mean(x^2) + eps):
+// with g = dy * scale, dx = r * g - x * r^3 * mean(g * x).  One wavefront per
+// row, float32 arithmetic, one rounding; r goes to rstd[row] for the scale's
+// gradient dscale[j] = sum_rows dy * x * r.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void rms_norm_backward_kernel(
+    const T* __restrict__ x, const T* __restrict__ scale,
+    const T* __restrict__ dy, T* __restrict__ dx, float* __restrict__ rstd,
+    int64_t rows, int M, float inv_m, float eps) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const T* xr = x + row * M;
+  const T* gr = dy + row * M;
+  float sumsq = 0.f, dot = 0.f;
+  for (int i = lane; i < M; i += 64) {
+    const float v = load_f32<T>(xr + i);
+    sumsq = fmaf(v, v, sumsq);
+    dot = fmaf(load_f32<T>(gr + i) * load_f32<T>(scale + i), v, dot);
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) {
+    sumsq += __shfl_xor(sumsq, off);
+    dot += __shfl_xor(dot, off);
+  }
+  const float r = 1.0f / sqrtf(sumsq * inv_m + eps);
+  const float c = r * r * r * dot * inv_m;
+  if (lane == 0) rstd[row] = r;
+  T* outr = dx + row * M;
+  for (int i = lane; i < M; i += 64) {
+    const float v = load_f32<T>(xr + i);
+    const float g = load_f32<T>(gr + i) * load_f32<T>(scale + i);
+    store_f32<T>(outr + i, g * r - v * c);
+  }
+}
+
+// partial[chunk, j] = sum over the chunk's rows of dy * x * rstd
+template <typename T>
+__global__ __launch_bounds__(256) void rms_norm_dscale_partial_kernel(
+    const T* __restrict__ x, const T* __restrict__ dy,
+    const float* __restrict__ rstd, float* __restrict__ partial, int64_t rows,
+    int M, int64_t rows_per_chunk) {
+  const int j = blockIdx.x * 256 + threadIdx.x;
+  if (j >= M) return;
+  const int64_t r0 = (int64_t)blockIdx.y * rows_per_chunk;
+  const int64_t r1 = r0 + rows_per_chunk < rows ? r0 + rows_per_chunk : rows;
+  float acc = 0.f;
+  for (int64_t r = r0; r < r1; ++r)
+    acc = fmaf(load_f32<T>(dy + r * M + j) * load_f32<T>(x + r * M + j),
+               rstd[r], acc);
+  partial[(int64_t)blockIdx.y * M + j] = acc;
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void rms_norm_dscale_final_kernel(
+    const float* __restrict__ partial, T* __restrict__ dscale, int chunks,
+    int M) {
+  const int j = blockIdx.x * 256 + threadIdx.x;
+  if (j >= M) return;
+  float acc = 0.f;
+  for (int c = 0; c < chunks; ++c) acc += partial[(int64_t)c * M + j];
+  store_f32<T>(dscale + j, acc);
+}
+
+static int rms_norm_dscale_chunks(int64_t rows) {
+  const int64_t c = (rows + 255) / 256;
+  return (int)(c < 1 ? 1 : (c > 256 ? 256 : c));
+}
+
+// ---------------------------------------------------------------------------
+// Backward of a softmax over the last dim from its output:
+// dlogits = w * (dw - sum_k dw * w).  One wavefront per row, float32
+// arithmetic, one rounding.  Where w is 0 (keys that are not visible) so is
+// the result.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void softmax_backward_kernel(
+    const T* __restrict__ w, const T* __restrict__ dw, T* __restrict__ dlogits,
+    int64_t rows, int L) {
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const T* wr = w + row * L;
+  const T* dr = dw + row * L;
+  float dot = 0.f;
+  for (int j = lane; j < L; j += 64)
+    dot = fmaf(load_f32<T>(dr + j), load_f32<T>(wr + j), dot);
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off);
+  T* outr = dlogits + row * L;
+  for (int j = lane; j < L; j += 64)
+    store_f32<T>(outr + j, load_f32<T>(wr + j) * (load_f32<T>(dr + j) - dot));
+}
+
+// The attention weights alone, heads to the front: weights [B*H, L, L].
+template <typename T>
+static int run_attention_weights(const T* q, const T* k, T* weights, int B,
+                                 int L, int H, int D, int causal, int dtype,
+                                 void* workspace, hipStream_t st) {
+  const int BH = B * H;
+  const size_t hd = (size_t)BH * L * D;
+  auto up = [](uintptr_t p) { return (p + 255) & ~(uintptr_t)255; };
+  T* qh = (T*)up((uintptr_t)workspace);
+  T* kh = (T*)up((uintptr_t)(qh + hd));
+  float* logits = (float*)up((uintptr_t)(kh + hd));
+  const int64_t n = (int64_t)hd;
+  const unsigned eb = (unsigned)((n + 255) / 256 < 65536 ? (n + 255) / 256
+                                                         : 65536);
+  split_heads_kernel<T><<<eb, 256, 0, st>>>(q, qh, B, L, H, D);
+  MOE_CHECK_LAUNCH("attention_weights (split q)");
+  split_heads_kernel<T><<<eb, 256, 0, st>>>(k, kh, B, L, H, D);
+  MOE_CHECK_LAUNCH("attention_weights (split k)");
+  int rc = batched_gemm_nt(qh, kh, logits, BH, L, L, D, dtype, true, st);
+  if (rc != 0) return rc;
+  const int64_t rows = (int64_t)BH * L;
+  attention_softmax_kernel<T><<<(unsigned)((rows + 3) / 4), 256, 0, st>>>(
+      logits, weights, rows, L, causal);
+  MOE_CHECK_LAUNCH("attention_weights (softmax)");
+  return 0;
+}
+
 // Dropout with the noise broadcast over the middle of three index ranges
 // (ops.py:5832-5872 with a noise_shape that leaves dimensions of x out):
 // out[o, m, i] = x[o, m, i] * noise[o, i], noise = (uniform < keep) ? 1 / keep
@@ -313,6 +436,133 @@ extern "C" int mesh_moe_broadcast_dropout(const void* x, const void* uniform,
   }
   MOE_CHECK_LAUNCH("broadcast_dropout");
   return 0;
+}
+
+extern "C" size_t mesh_moe_rms_norm_backward_workspace_bytes(int64_t rows,
+                                                            int M) {
+  if (rows < 1 || M < 1) return 0;
+  return ((size_t)rows * 4 + 255) / 256 * 256 +
+         (size_t)rms_norm_dscale_chunks(rows) * (size_t)M * 4;
+}
+
+extern "C" int mesh_moe_rms_norm_backward(const void* x, const void* scale,
+                                          const void* dy, void* dx,
+                                          void* dscale, int64_t rows, int M,
+                                          double epsilon, int dtype,
+                                          void* workspace,
+                                          size_t workspace_bytes,
+                                          void* stream) {
+  MOE_REQUIRE(x && scale && dy && dx && dscale && workspace, MESH_MOE_E_ARG,
+              "rms_norm_backward: null pointer");
+  MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG,
+              "rms_norm_backward: bad dtype %d", dtype);
+  MOE_REQUIRE(rows >= 1 && M >= 1, MESH_MOE_E_ARG,
+              "rms_norm_backward: bad sizes rows=%lld M=%d", (long long)rows,
+              M);
+  const int64_t blocks = (rows + 3) / 4;
+  MOE_REQUIRE(blocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
+              "rms_norm_backward: too many rows (%lld)", (long long)rows);
+  MOE_REQUIRE(workspace_bytes >=
+                  mesh_moe_rms_norm_backward_workspace_bytes(rows, M),
+              MESH_MOE_E_ARG, "rms_norm_backward: workspace too small");
+  hipStream_t st = (hipStream_t)stream;
+  float* rstd = (float*)workspace;
+  float* partial =
+      (float*)((char*)workspace + ((size_t)rows * 4 + 255) / 256 * 256);
+  const int chunks = rms_norm_dscale_chunks(rows);
+  const int64_t per_chunk = (rows + chunks - 1) / chunks;
+  const dim3 pg((unsigned)((M + 255) / 256), (unsigned)chunks);
+  const float inv_m = (float)(1.0 / (double)M);
+  if (dtype == MESH_MOE_F32) {
+    rms_norm_backward_kernel<float><<<(unsigned)blocks, 256, 0, st>>>(
+        (const float*)x, (const float*)scale, (const float*)dy, (float*)dx,
+        rstd, rows, M, inv_m, (float)epsilon);
+    MOE_CHECK_LAUNCH("rms_norm_backward");
+    rms_norm_dscale_partial_kernel<float><<<pg, 256, 0, st>>>(
+        (const float*)x, (const float*)dy, rstd, partial, rows, M, per_chunk);
+    MOE_CHECK_LAUNCH("rms_norm_backward (dscale partial)");
+    rms_norm_dscale_final_kernel<float><<<pg.x, 256, 0, st>>>(
+        partial, (float*)dscale, chunks, M);
+  } else {
+    rms_norm_backward_kernel<bf16_t><<<(unsigned)blocks, 256, 0, st>>>(
+        (const bf16_t*)x, (const bf16_t*)scale, (const bf16_t*)dy, (bf16_t*)dx,
+        rstd, rows, M, inv_m, round_bf16_host((float)epsilon));
+    MOE_CHECK_LAUNCH("rms_norm_backward");
+    rms_norm_dscale_partial_kernel<bf16_t><<<pg, 256, 0, st>>>(
+        (const bf16_t*)x, (const bf16_t*)dy, rstd, partial, rows, M, per_chunk);
+    MOE_CHECK_LAUNCH("rms_norm_backward (dscale partial)");
+    rms_norm_dscale_final_kernel<bf16_t><<<pg.x, 256, 0, st>>>(
+        partial, (bf16_t*)dscale, chunks, M);
+  }
+  MOE_CHECK_LAUNCH("rms_norm_backward (dscale)");
+  return 0;
+}
+
+extern "C" int mesh_moe_softmax_backward(const void* weights,
+                                         const void* dweights, void* dlogits,
+                                         int64_t rows, int L, int dtype,
+                                         void* stream) {
+  MOE_REQUIRE(weights && dweights && dlogits, MESH_MOE_E_ARG,
+              "softmax_backward: null pointer");
+  MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG,
+              "softmax_backward: bad dtype %d", dtype);
+  MOE_REQUIRE(rows >= 1 && L >= 1, MESH_MOE_E_ARG,
+              "softmax_backward: bad sizes rows=%lld L=%d", (long long)rows, L);
+  const int64_t blocks = (rows + 3) / 4;
+  MOE_REQUIRE(blocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
+              "softmax_backward: too many rows (%lld)", (long long)rows);
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == MESH_MOE_F32)
+    softmax_backward_kernel<float><<<(unsigned)blocks, 256, 0, st>>>(
+        (const float*)weights, (const float*)dweights, (float*)dlogits, rows,
+        L);
+  else
+    softmax_backward_kernel<bf16_t><<<(unsigned)blocks, 256, 0, st>>>(
+        (const bf16_t*)weights, (const bf16_t*)dweights, (bf16_t*)dlogits, rows,
+        L);
+  MOE_CHECK_LAUNCH("softmax_backward");
+  return 0;
+}
+
+extern "C" size_t mesh_moe_attention_weights_workspace_bytes(int B, int L,
+                                                             int H, int D,
+                                                             int dtype) {
+  if (B < 1 || L < 1 || H < 1 || D < 1 || !valid_dtype(dtype)) return 0;
+  const size_t b = dtype_size(dtype);
+  const size_t hd = (size_t)B * H * L * D, ll = (size_t)B * H * L * L;
+  return 2 * hd * b + ll * 4 + 4 * 256;
+}
+
+extern "C" int mesh_moe_attention_weights(const void* q, const void* k,
+                                          void* weights, int B, int L, int H,
+                                          int D, int causal, int dtype,
+                                          void* workspace,
+                                          size_t workspace_bytes,
+                                          void* stream) {
+  MOE_REQUIRE(q && k && weights && workspace, MESH_MOE_E_ARG,
+              "attention_weights: null pointer");
+  MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG,
+              "attention_weights: bad dtype %d", dtype);
+  MOE_REQUIRE(B >= 1 && L >= 1 && H >= 1 && D >= 1, MESH_MOE_E_ARG,
+              "attention_weights: bad sizes B=%d L=%d H=%d D=%d", B, L, H, D);
+  MOE_REQUIRE((int64_t)B * H <= 65535, MESH_MOE_E_UNSUPPORTED,
+              "attention_weights: batch * heads = %lld > 65535",
+              (long long)B * H);
+  MOE_REQUIRE(dtype == MESH_MOE_F32 || (L % 8 == 0 && D % 8 == 0),
+              MESH_MOE_E_UNSUPPORTED,
+              "attention_weights: bfloat16 needs length and d_kv multiples of "
+              "8 (L=%d D=%d)", L, D);
+  MOE_REQUIRE(workspace_bytes >=
+                  mesh_moe_attention_weights_workspace_bytes(B, L, H, D, dtype),
+              MESH_MOE_E_ARG, "attention_weights: workspace too small");
+  hipStream_t st = (hipStream_t)stream;
+  if (dtype == MESH_MOE_F32)
+    return run_attention_weights<float>((const float*)q, (const float*)k,
+                                        (float*)weights, B, L, H, D,
+                                        causal ? 1 : 0, dtype, workspace, st);
+  return run_attention_weights<bf16_t>((const bf16_t*)q, (const bf16_t*)k,
+                                       (bf16_t*)weights, B, L, H, D,
+                                       causal ? 1 : 0, dtype, workspace, st);
 }
 
 extern "C" int mesh_moe_rms_norm(const void* x, const void* scale, void* y,

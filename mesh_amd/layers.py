@@ -146,6 +146,44 @@ class DenseOperation(mtf.Operation):
     lowering.set_tensor_lowering(
         self.outputs[0], mesh_impl.slicewise(fn, lowering.tensors[x]))
 
+  def gradient(self, grad_ys):
+    return list(DenseGradOperation(self, grad_ys[0]).outputs)
+
+
+class DenseGradOperation(mtf.Operation):
+  """(dx, dkernel) of a DenseOperation: what mtf.gradients derives from the
+  einsum (mesh_tensorflow/ops.py:2846-2854) and the relu of layers.dense, as
+  dpre = dy * (y > 0), dx = dpre . kernel^T, dkernel = x^T . dpre on the
+  grouped GEMM with one group."""
+
+  def __init__(self, forward, dy, name=None):
+    x, kernel = forward.inputs
+    super(DenseGradOperation, self).__init__(
+        [dy, x, kernel, forward.outputs[0]], name=name or "dense_grad")
+    self._relu = forward._activation == "relu"   # pylint: disable=protected-access
+    if forward._activation not in (None, "relu"):  # pylint: disable=protected-access
+      raise NotImplementedError("gradient of dense with activation %r"
+                                % (forward._activation,))  # pylint: disable=protected-access
+    self._outputs = [mtf.Tensor(self, x.shape, x.dtype, index=0),
+                     mtf.Tensor(self, kernel.shape, kernel.dtype, index=1)]
+
+  def lower(self, lowering):
+    from mesh_amd import moe_hip
+    mesh_impl = lowering.mesh_impl(self)
+    relu = self._relu
+    k = self.inputs[1].shape.dims[-1].size
+    kernel_sizes = self.inputs[2].shape.to_integer_list
+
+    def fn(dy, x, w, y):
+      w2 = w.to(x.dtype).reshape(k, -1)
+      dx, dw = moe_hip.dense_backward(x.contiguous(), w2, dy.contiguous(),
+                                      y if relu else None)
+      return dx, dw.reshape(kernel_sizes).to(w.dtype)
+    dx, dw = mesh_impl.slicewise(
+        fn, *[lowering.tensors[t] for t in self.inputs])
+    lowering.set_tensor_lowering(self.outputs[0], dx)
+    lowering.set_tensor_lowering(self.outputs[1], dw)
+
 
 def _activation_name(activation):
   if activation is None or activation == "linear":

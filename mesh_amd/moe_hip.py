@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 15
+ABI_VERSION = 16
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -101,6 +101,18 @@ _SIGNATURES = {
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "mesh_moe_expert_linear_backward": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
+    "mesh_moe_rms_norm_backward_workspace_bytes": (ctypes.c_size_t, [
+        ctypes.c_int64, ctypes.c_int]),
+    "mesh_moe_rms_norm_backward": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, _vp, ctypes.c_int64, ctypes.c_int, ctypes.c_double,
+        ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
+    "mesh_moe_softmax_backward": (ctypes.c_int, [
+        _vp, _vp, _vp, ctypes.c_int64, ctypes.c_int, ctypes.c_int, _vp]),
+    "mesh_moe_attention_weights_workspace_bytes": (ctypes.c_size_t, [
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "mesh_moe_attention_weights": (ctypes.c_int, [
+        _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
     "mesh_moe_broadcast_dropout": (ctypes.c_int, [
         _vp, _vp, _vp, ctypes.c_float, _vp, _vp, ctypes.c_int64, ctypes.c_int64,
@@ -1091,3 +1103,99 @@ def expert_choice_backward(logits, r, dweight, d_loss, loss_scale,
         dlogits.data_ptr(), ws.data_ptr(), ws_bytes, _stream()),
         "expert_choice_backward")
   return dlogits
+
+
+# ---- backward of the block's operations ----------------------------------------
+def rms_norm_backward(x, scale, dy, epsilon=1e-6):
+  """Backward of rms_norm: x, dy [..., M], scale [M] -> (dx, dscale)."""
+  lib = load_library()
+  m = x.shape[-1]
+  rows = x.numel() // m
+  dt = x.dtype
+  dx = torch.empty_like(x)
+  dscale = torch.empty_like(scale)
+  ws_bytes = lib.mesh_moe_rms_norm_backward_workspace_bytes(rows, m)
+  ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=x.device)
+  with _stage("rms_norm_backward"):
+    _check(lib.mesh_moe_rms_norm_backward(
+        _dev(x, "x"), _dev(scale, "scale", dt, (m,)),
+        _dev(dy, "dy", dt, tuple(x.shape)), dx.data_ptr(), dscale.data_ptr(),
+        rows, m, float(epsilon), dtype_code(dt), ws.data_ptr(), ws_bytes,
+        _stream()), "rms_norm_backward")
+  return dx, dscale
+
+
+def dense_backward(x, w, dy, y=None, want_dx=True):
+  """Backward of y = act(x . w): x [..., K], w [K, N] in the variable's own
+  layout, dy [..., N]; with `y` (the forward output) the activation was relu.
+  Returns (dx or None, dw [K, N])."""
+  k = x.shape[-1]
+  n = w.shape[-1]
+  x3 = x.reshape(1, -1, k)
+  dy3 = dy.reshape(1, -1, n)
+  if y is not None:     # relu: y > 0 exactly where the pre-activation is
+    dy3 = activation_backward(dy3.contiguous(), y.reshape(1, -1, n), "relu")
+  dx, dw = expert_linear_backward(x3.contiguous(), dy3.contiguous(),
+                                  w.reshape(1, k, n).contiguous(),
+                                  want_da=want_dx)
+  return (dx.reshape(x.shape) if want_dx else None), dw.reshape(k, n)
+
+
+def attention_weights(q, k, num_heads, causal):
+  """q, k [B, L, H*D] -> softmax(q . k + visibility) [B*H, L, L] in q's dtype."""
+  lib = load_library()
+  b, l, hd = q.shape
+  d = hd // num_heads
+  code = dtype_code(q.dtype)
+  weights = torch.empty((b * num_heads, l, l), dtype=q.dtype, device=q.device)
+  ws_bytes = lib.mesh_moe_attention_weights_workspace_bytes(b, l, num_heads, d,
+                                                            code)
+  ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=q.device)
+  with _stage("attention_weights"):
+    _check(lib.mesh_moe_attention_weights(
+        _dev(q, "q"), _dev(k, "k", q.dtype, (b, l, hd)), weights.data_ptr(), b,
+        l, num_heads, d, 1 if causal else 0, code, ws.data_ptr(), ws_bytes,
+        _stream()), "attention_weights")
+  return weights
+
+
+def softmax_backward(weights, dweights):
+  """dlogits = w * (dw - sum_k dw * w) over the last dim."""
+  lib = load_library()
+  l = weights.shape[-1]
+  out = torch.empty_like(weights)
+  with _stage("softmax_backward"):
+    _check(lib.mesh_moe_softmax_backward(
+        _dev(weights, "weights"),
+        _dev(dweights, "dweights", weights.dtype, tuple(weights.shape)),
+        out.data_ptr(), weights.numel() // l, l, dtype_code(weights.dtype),
+        _stream()), "softmax_backward")
+  return out
+
+
+def self_attention_backward(q, k, v, dout, num_heads, causal):
+  """Backward of self_attention: q, k, v, dout [B, L, H*D] -> (dq, dk, dv).
+  The weights are recomputed ([B*H, L, L], which the forward kernel never
+  stores); every product runs on the grouped GEMM with one (batch, head) pair
+  per group:
+    dweights = dout . v^T,  dv = weights^T . dout    (one linear backward)
+    dlogits  = softmax backward
+    dq = dlogits . k,       dk = dlogits^T . q
+  Heads move to the front and back with torch permutes."""
+  b, l, hd = q.shape
+  h = num_heads
+  d = hd // h
+  def heads_first(t):
+    return t.reshape(b, l, h, d).permute(0, 2, 1, 3).reshape(b * h, l, d) \
+        .contiguous()
+  def heads_last(t):
+    return t.reshape(b, h, l, d).permute(0, 2, 1, 3).reshape(b, l, hd) \
+        .contiguous()
+  qh, kh, vh, doh = (heads_first(t) for t in (q, k, v, dout))
+  weights = attention_weights(q, k, h, causal)
+  dweights, dvh = expert_linear_backward(weights, doh, vh)
+  dlogits = softmax_backward(weights, dweights)
+  del weights, dweights
+  dqh = expert_linear(dlogits, pack_weights(kh, q.dtype))
+  _, dkh = expert_linear_backward(dlogits, qh, vh, want_da=False)
+  return heads_last(dqh), heads_last(dkh), heads_last(dvh)

@@ -208,3 +208,38 @@ class SelfAttentionOperation(mtf.Operation):
     lowering.set_tensor_lowering(
         self.outputs[0],
         mesh_impl.slicewise(fn, *[lowering.tensors[t] for t in self.inputs]))
+
+  def gradient(self, grad_ys):
+    return list(SelfAttentionGradOperation(self, grad_ys[0]).outputs)
+
+
+class SelfAttentionGradOperation(mtf.Operation):
+  """(dq, dk, dv) of a SelfAttentionOperation: the gradients of the two
+  einsums and the softmax of attention.attention (attention.py:76-87), with
+  the weights recomputed."""
+
+  def __init__(self, forward, dout, name=None):
+    q, k, v = forward.inputs
+    super(SelfAttentionGradOperation, self).__init__(
+        [dout, q, k, v], name=name or "attention_grad")
+    self._num_heads = forward._num_heads   # pylint: disable=protected-access
+    self._causal = forward._causal         # pylint: disable=protected-access
+    self._outputs = [mtf.Tensor(self, t.shape, t.dtype, index=i)
+                     for i, t in enumerate((q, k, v))]
+
+  def lower(self, lowering):
+    from mesh_amd import moe_hip
+    mesh_impl = lowering.mesh_impl(self)
+    sizes = self.outputs[0].shape.to_integer_list
+    length, channels = sizes[-2], sizes[-1]
+    heads, causal = self._num_heads, self._causal
+
+    def fn(dout, q, k, v):
+      d3, q3, k3, v3 = (t.reshape(-1, length, channels).contiguous()
+                        for t in (dout, q, k, v))
+      return tuple(t.reshape(sizes) for t in moe_hip.self_attention_backward(
+          q3, k3, v3, d3, heads, causal))
+    grads = mesh_impl.slicewise(
+        fn, *[lowering.tensors[t] for t in self.inputs])
+    for out, value in zip(self.outputs, grads):
+      lowering.set_tensor_lowering(out, value)

@@ -130,6 +130,35 @@ class RmsNormOperation(mtf.Operation):
         self.outputs[0],
         mesh_impl.slicewise(fn, *[lowering.tensors[t] for t in self.inputs]))
 
+  def gradient(self, grad_ys):
+    return list(RmsNormGradOperation(self, grad_ys[0]).outputs)
+
+
+class RmsNormGradOperation(mtf.Operation):
+  """(dx, dscale) of an RmsNormOperation."""
+
+  def __init__(self, forward, dy, name=None):
+    x, scale = forward.inputs
+    super(RmsNormGradOperation, self).__init__(
+        [dy, x, scale], name=name or "rms_norm_grad")
+    self._epsilon = forward._epsilon   # pylint: disable=protected-access
+    self._outputs = [mtf.Tensor(self, x.shape, x.dtype, index=0),
+                     mtf.Tensor(self, scale.shape, scale.dtype, index=1)]
+
+  def lower(self, lowering):
+    from mesh_amd import moe_hip
+    mesh_impl = lowering.mesh_impl(self)
+    eps = self._epsilon
+
+    def fn(dy, x, scale):
+      dx, dscale = moe_hip.rms_norm_backward(
+          x.contiguous(), scale.to(x.dtype).contiguous(), dy.contiguous(), eps)
+      return dx, dscale.to(scale.dtype)
+    dx, dscale = mesh_impl.slicewise(
+        fn, *[lowering.tensors[t] for t in self.inputs])
+    lowering.set_tensor_lowering(self.outputs[0], dx)
+    lowering.set_tensor_lowering(self.outputs[1], dscale)
+
 
 def sublayer_call_layer(x, layer_stack, context):
   """transformer.py:462-466."""

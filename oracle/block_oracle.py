@@ -204,3 +204,64 @@ def layer_stack(x, layers, final_scale, act_dtype="float32",
   if final_noise is not None:
     y = broadcast_dropout(y, final_noise, -2, act_dtype)
   return y, losses
+
+
+# --- backward passes ----------------------------------------------------------
+# The reference has no code of its own for these: mtf.gradients differentiates
+# the einsum / reduce / cwise operations of the forward graph (ops.py:2846-2854
+# and the gradient methods of the cwise operations).  They are restated as the
+# derivatives of the forward formulas above, in float32 on the stored
+# (activation-dtype) operands with one rounding per tensor that reaches memory,
+# and pinned by float64 finite differences of the forward formulas.
+
+def rms_norm_backward(x, scale, dy, act_dtype="float32", epsilon=1e-6):
+  """(dx, dscale) of rms_norm: with r = rsqrt(mean(x^2) + eps), g = dy * scale:
+  dx = r g - x r^3 mean(g x), dscale = sum over rows of dy x r."""
+  x, scale, dy = _r(x, act_dtype), _r(scale, act_dtype), _r(dy, act_dtype)
+  eps = _r(F32(epsilon), act_dtype)
+  m = x.shape[-1]
+  r = F32(1.0) / np.sqrt((x * x).sum(-1, keepdims=True, dtype=F32) / F32(m)
+                         + eps, dtype=F32)
+  g = dy * scale
+  dot = (g * x).sum(-1, keepdims=True, dtype=F32) / F32(m)
+  dx = g * r - x * (r * r * r * dot)
+  dscale = (dy * x * r).reshape(-1, m).sum(0, dtype=F32)
+  return _r(dx, act_dtype), _r(dscale, act_dtype)
+
+
+def dense_backward(x, w, dy, act_dtype="float32", activation=None):
+  """(dx, dw) of dense: dpre = dy (times (y > 0) after a relu), dx = dpre w^T,
+  dw = x^T dpre over all leading dims."""
+  x, w, dy = _r(x, act_dtype), _r(w, act_dtype), _r(dy, act_dtype)
+  if activation == "relu":
+    dy = _r(dy * (dense(x, w, act_dtype, "relu") > 0), act_dtype)
+  elif activation not in (None, "linear"):
+    raise ValueError("activation %r" % (activation,))
+  k, n = w.shape
+  dx = _r(np.matmul(dy, w.T), act_dtype)
+  dw = _r(np.matmul(x.reshape(-1, k).T, dy.reshape(-1, n)), act_dtype)
+  return dx, dw
+
+
+def attention_core_backward(q, k, v, dout, num_heads, causal,
+                            act_dtype="float32"):
+  """(dq, dk, dv) of _attention_core on [B, L, H*D] tensors: the weights as
+  the forward pass rounds them; dweights = dout v^T, dv = weights^T dout,
+  dlogits = weights (dweights - sum_k dweights weights), dq = dlogits k,
+  dk = dlogits^T q."""
+  b, l, hd = q.shape
+  d = hd // num_heads
+  q, k, v, dout = (_r(t, act_dtype).reshape(b, l, num_heads, d)
+                   for t in (q, k, v, dout))
+  logits = np.einsum("blhd,bmhd->bhlm", q, k).astype(F32)
+  if causal:
+    pos = np.arange(l)
+    logits = logits + (pos[None, :] > pos[:, None]).astype(F32) * F32(-1e9)
+  weights = _r(O.softmax(logits), act_dtype)
+  dweights = _r(np.einsum("blhd,bmhd->bhlm", dout, v), act_dtype)
+  dv = _r(np.einsum("bhlm,blhd->bmhd", weights, dout), act_dtype)
+  dot = (dweights * weights).sum(-1, keepdims=True, dtype=F32)
+  dlogits = _r(weights * (dweights - dot), act_dtype)
+  dq = _r(np.einsum("bhlm,bmhd->blhd", dlogits, k), act_dtype)
+  dk = _r(np.einsum("bhlm,blhd->bmhd", dlogits, q), act_dtype)
+  return tuple(t.reshape(b, l, hd) for t in (dq, dk, dv))

@@ -219,3 +219,68 @@ def test_dropout_noise_arguments():
   np.testing.assert_allclose(
       y, B.broadcast_dropout(B.rms_norm(h, scale), last, -2), rtol=1e-6,
       atol=1e-6)
+
+
+def _fd(fn, arg, direction, eps=1e-6):
+  """Central difference of the scalar fn along `direction` in float64."""
+  return (fn(arg + eps * direction) - fn(arg - eps * direction)) / (2 * eps)
+
+
+def test_backward_passes_against_float64_finite_differences():
+  """Each backward restatement against central differences of a float64
+  forward: <grad, direction> = d/dt loss(arg + t direction)."""
+  rng = np.random.default_rng(11)
+  b, l, m, heads, d = 2, 7, 12, 3, 4
+  f64 = lambda *s: rng.standard_normal(s)
+  x, dy, scale = f64(b, l, m), f64(b, l, m), 1 + 0.3 * f64(m)
+
+  def rms64(x_, s_):
+    return x_ / np.sqrt((x_ * x_).mean(-1, keepdims=True) + 1e-6) * s_
+  dx, ds = B.rms_norm_backward(x, scale, dy)
+  u, us = f64(b, l, m), f64(m)
+  np.testing.assert_allclose(
+      (dx * u).sum(), _fd(lambda a: (rms64(a, scale) * dy).sum(), x, u),
+      rtol=2e-4)
+  np.testing.assert_allclose(
+      (ds * us).sum(), _fd(lambda s_: (rms64(x, s_) * dy).sum(), scale, us),
+      rtol=2e-4)
+  # a dropped mean term would leave dx with a component along x
+  np.testing.assert_allclose(
+      (B.rms_norm_backward(x, np.ones(m), x)[0]), 0, atol=2e-5)
+
+  w, dyn = f64(m, 9) / 3, f64(b, l, 9)
+  for act in (None, "relu"):
+    fwd = lambda x_, w_: (np.maximum(x_ @ w_, 0) if act else x_ @ w_)
+    dxd, dw = B.dense_backward(x, w, dyn, activation=act)
+    uw = f64(m, 9)
+    np.testing.assert_allclose(
+        (dxd * u).sum(), _fd(lambda a: (fwd(a, w) * dyn).sum(), x, u),
+        rtol=2e-4)
+    np.testing.assert_allclose(
+        (dw * uw).sum(), _fd(lambda a: (fwd(x, a) * dyn).sum(), w, uw),
+        rtol=2e-4)
+
+  q, k, v, do = (f64(b, l, heads * d) for _ in range(4))
+
+  def core64(q_, k_, v_, causal):
+    out = np.zeros((b, l, heads * d))
+    for bi in range(b):
+      for h in range(heads):
+        sl = slice(h * d, (h + 1) * d)
+        s = q_[bi, :, sl] @ k_[bi, :, sl].T
+        if causal:
+          s = np.where(np.tril(np.ones((l, l), bool)), s, -np.inf)
+        out[bi, :, sl] = scipy.special.softmax(s, axis=-1) @ v_[bi, :, sl]
+    return out
+  for causal in (False, True):
+    dq, dk, dv = B.attention_core_backward(q, k, v, do, heads, causal)
+    uq = f64(b, l, heads * d)
+    for grad, which in ((dq, 0), (dk, 1), (dv, 2)):
+      def loss(a, which=which):
+        args = [q, k, v]
+        args[which] = a
+        return (core64(*args, causal) * do).sum()
+      np.testing.assert_allclose((grad * uq).sum(),
+                                 _fd(loss, (q, k, v)[which], uq), rtol=5e-4)
+    if causal:       # the first query sees one key: a softmax of one element
+      np.testing.assert_allclose(dq[:, 0], 0, atol=1e-6)

@@ -568,3 +568,124 @@ def test_layer_stack_with_dropout():
   np.testing.assert_allclose(got, want, rtol=2e-4, atol=2e-4)
   got_loss = [float(H.to_np(lowering.export_to_tf_tensor(t))) for t in losses]
   np.testing.assert_allclose(got_loss, want_loss, rtol=1e-4)
+
+
+@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
+def test_block_backward_entries(hip, act_dtype):
+  """rms_norm_backward, dense_backward (with and without relu) and
+  self_attention_backward (both visibility modes) against the oracle."""
+  dt = H.ACT_TORCH[act_dtype]
+  tol = dict(rtol=2e-4, atol=2e-4) if act_dtype == "float32" else dict(
+      rtol=3e-2, atol=3e-2)
+  rng = np.random.default_rng(51)
+  dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dt).cuda()
+  rnd = lambda *s: O.cast_act(rng.standard_normal(s).astype(np.float32),
+                              act_dtype)
+  for rows, m in ((37, 48), (1024, 256), (5, 1000)):
+    x, dy = rnd(rows, m), rnd(rows, m)
+    scale = O.cast_act((1 + 0.2 * rng.standard_normal(m)).astype(np.float32),
+                       act_dtype)
+    dx, ds = hip.rms_norm_backward(dev(x), dev(scale), dev(dy))
+    want_dx, want_ds = B.rms_norm_backward(x, scale, dy, act_dtype)
+    np.testing.assert_allclose(H.to_np(dx), want_dx, **tol)
+    np.testing.assert_allclose(H.to_np(ds), want_ds, rtol=tol["rtol"],
+                               atol=tol["atol"] * rows ** 0.5)
+  b, l, k, n = 2, 64, 128, 192
+  x, dy = rnd(b, l, k), rnd(b, l, n)
+  w = O.cast_act(H.normal_weights(rng, (k, n), k), act_dtype)
+  for act in (None, "relu"):
+    y = B.dense(x, w, act_dtype, act)
+    dx, dw = hip.dense_backward(dev(x), dev(w), dev(dy),
+                                dev(y) if act else None)
+    want_dx, want_dw = B.dense_backward(x, w, dy, act_dtype, act)
+    np.testing.assert_allclose(H.to_np(dx), want_dx, **tol)
+    np.testing.assert_allclose(H.to_np(dw), want_dw, rtol=tol["rtol"],
+                               atol=tol["atol"] * 4)
+  for bsz, length, heads, d, causal in ((2, 64, 4, 16, True),
+                                        (1, 128, 2, 64, False),
+                                        (2, 256, 2, 128, True)):
+    q, kk, v, do = (rnd(bsz, length, heads * d) * np.float32(0.5)
+                    for _ in range(4))
+    q, kk, v, do = (O.cast_act(t, act_dtype) for t in (q, kk, v, do))
+    got = hip.self_attention_backward(dev(q), dev(kk), dev(v), dev(do), heads,
+                                      causal)
+    want = B.attention_core_backward(q, kk, v, do, heads, causal, act_dtype)
+    for g, wnt, name in zip(got, want, "qkv"):
+      np.testing.assert_allclose(H.to_np(g), wnt, err_msg="d" + name, **tol)
+    w_got = hip.attention_weights(dev(q), dev(kk), heads, causal)
+    np.testing.assert_allclose(H.to_np(w_got).sum(-1), 1.0,
+                               rtol=1e-5 if act_dtype == "float32" else 2e-2)
+
+
+def test_layer_stack_gradients():
+  """mtf.gradients through a stack of attention and DenseReluDense layers
+  (RMS norms, residuals, projections): every variable's gradient and the
+  input's against the oracle's per-operation backward passes chained by
+  hand, float32."""
+  b, l, m, hdim, heads, d = 2, 32, 64, 96, 4, 16
+  rng = np.random.default_rng(52)
+  layers, final = _build_stack(rng, m, 4, hdim, heads, d, 32)
+  att, ffn = layers[0], layers[3]
+  x = rng.standard_normal((b, l, m)).astype(np.float32)
+  dy = rng.standard_normal((b, l, m)).astype(np.float32)
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  dims = [mtf.Dimension("batch", b), mtf.Dimension("length", l),
+          mtf.Dimension("d_model", m)]
+  xt = mtf.import_tf_tensor(mesh, torch.from_numpy(x), mtf.Shape(dims))
+  dyt = mtf.import_tf_tensor(mesh, torch.from_numpy(dy), mtf.Shape(dims))
+  stack = transformer.make_layer_stack(
+      [(transformer_layers.SelfAttention,
+        dict(num_heads=heads, key_value_size=d)),
+       (transformer_layers.DenseReluDense, dict(hidden_size=hdim))],
+      num_layers=1, block_scope=False)
+  model = transformer.Unitransformer(stack, d_model=m, name="decoder",
+                                     autoregressive=True)
+  y, _ = model.call_layers(xt, mtf.VariableDType(torch.float32), mode="eval")
+  init = {"decoder/rms_norm/scale": final,
+          "decoder/layer_000/rms_norm/scale": att["scale"],
+          "decoder/layer_001/rms_norm/scale": ffn["scale"],
+          "decoder/layer_001/DenseReluDense/wi/kernel": ffn["wi"],
+          "decoder/layer_001/DenseReluDense/wo/kernel": ffn["wo"]}
+  for kname in "qkvo":
+    init["decoder/layer_000/SelfAttention/" + kname] = att["w" + kname]
+  variables = {v.name: v for v in graph.all_variables}
+  assert sorted(variables) == sorted(init)
+  names = sorted(init)
+  grads = mtf.gradients([y], [xt] + [variables[n].outputs[0] for n in names],
+                        [dyt])
+  lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()}, initial_values=init)
+  got = {n: H.to_np(lowering.export_to_tf_tensor(g))
+         for n, g in zip(["x"] + names, grads)}
+  # the oracle, forward then backward, by hand
+  h1 = B.rms_norm(x, att["scale"])
+  q, k, v = (B.dense(h1, att["w" + c]) for c in "qkv")
+  o = B._attention_core(q, k, v, heads, True, "float32")
+  x1 = x + B.dense(o, att["wo"])
+  h2 = B.rms_norm(x1, ffn["scale"])
+  hid = B.dense(h2, ffn["wi"], activation="relu")
+  x2 = x1 + B.dense(hid, ffn["wo"])
+  want = {}
+  dx2, want["decoder/rms_norm/scale"] = B.rms_norm_backward(x2, final, dy)
+  dhid, want["decoder/layer_001/DenseReluDense/wo/kernel"] = B.dense_backward(
+      hid, ffn["wo"], dx2)
+  dh2, want["decoder/layer_001/DenseReluDense/wi/kernel"] = B.dense_backward(
+      h2, ffn["wi"], dhid, activation="relu")
+  d1, want["decoder/layer_001/rms_norm/scale"] = B.rms_norm_backward(
+      x1, ffn["scale"], dh2)
+  dx1 = dx2 + d1
+  do, want["decoder/layer_000/SelfAttention/o"] = B.dense_backward(
+      o, att["wo"], dx1)
+  dq, dk, dv = B.attention_core_backward(q, k, v, do, heads, True)
+  dh1 = 0
+  for c, g in zip("qkv", (dq, dk, dv)):
+    part, want["decoder/layer_000/SelfAttention/" + c] = B.dense_backward(
+        h1, att["w" + c], g)
+    dh1 = dh1 + part
+  d0, want["decoder/layer_000/rms_norm/scale"] = B.rms_norm_backward(
+      x, att["scale"], dh1)
+  want["x"] = dx1 + d0
+  for name in ["x"] + names:
+    scale = max(1.0, float(np.abs(want[name]).max()))
+    np.testing.assert_allclose(got[name], want[name], rtol=1e-3,
+                               atol=1e-3 * scale, err_msg=name)
