@@ -153,12 +153,14 @@ def build(cfg, device, backward=False):
   return lowering, x, y, loss
 
 
-def build_block(cfg, device):
+def build_block(cfg, device, backward=False):
   """The block of mesh_tensorflow/transformer/gin/models/lm_moe.gin:11-16
   (SelfAttention, MoE1D, SelfAttention, DenseReluDense; autoregressive, eval
   mode) around the layer of `cfg`: d_kv 128, d_model / 128 heads, d_ff and the
   experts' hidden size = cfg's H.  Variables keep their own initialisers
-  (random normal).  Returns (lowering, x Tensor, y Tensor, None)."""
+  (random normal).  With `backward`, also mtf.gradients of the output and the
+  MoE loss w.r.t. the tokens and every variable.  Returns (lowering, x Tensor,
+  y Tensor, None)."""
   import torch
   import mesh_amd as mtf
   from mesh_amd.transformer import moe, transformer, transformer_layers
@@ -186,7 +188,14 @@ def build_block(cfg, device):
       num_layers=1, block_scope=False)
   model = transformer.Unitransformer(stack, d_model=m, name="decoder",
                                      autoregressive=True)
-  y, _ = model.call_layers(x, mtf.VariableDType(dt, dt, dt), mode="eval")
+  y, losses = model.call_layers(x, mtf.VariableDType(dt, dt, dt), mode="eval")
+  if backward:
+    d_out = mtf.import_tf_tensor(
+        mesh, torch.randn(x_val.shape, generator=gen, device=device,
+                          dtype=torch.float32).to(dt), mtf.Shape(dims))
+    mtf.gradients([y] + list(losses),
+                  [x] + [v.outputs[0] for v in graph.trainable_variables],
+                  grad_ys=[d_out] + [None] * len(losses))
   lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl(device=device)})
   return lowering, x, y, None
 
@@ -306,12 +315,11 @@ def main():
   if args.backward and cfg["layer"] != "v1":
     print("--backward applies to the v1 configs only", file=sys.stderr)
     sys.exit(2)
-  if args.block and (cfg["layer"] != "v1" or args.backward or
-                     args.gating != "top_2"):
-    print("--block applies to the v1 configs, forward, top_2", file=sys.stderr)
+  if args.block and (cfg["layer"] != "v1" or args.gating != "top_2"):
+    print("--block applies to the v1 configs, top_2", file=sys.stderr)
     sys.exit(2)
   if args.block:
-    lowering, x, y, loss = build_block(cfg, device)
+    lowering, x, y, loss = build_block(cfg, device, args.backward)
   else:
     lowering, x, y, loss = build(cfg, device, args.backward)  # first execution
   for _ in range(args.warmup):
@@ -343,7 +351,9 @@ def main():
     # attention + MoE1D + attention + DenseReluDense: per-stage times only
     heads = max(1, cfg["M"] // 128)
     print(json.dumps({
-        "metric": "MoE transformer block fwd tokens/sec @1 GPU",
+        "metric": ("MoE transformer block fwd+bwd tokens/sec @1 GPU"
+                   if args.backward
+                   else "MoE transformer block fwd tokens/sec @1 GPU"),
         "value": tokens / (ms_per_step * 1e-3), "unit": "tokens/s",
         "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True,
