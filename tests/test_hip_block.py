@@ -689,3 +689,64 @@ def test_layer_stack_gradients():
     scale = max(1.0, float(np.abs(want[name]).max()))
     np.testing.assert_allclose(got[name], want[name], rtol=1e-3,
                                atol=1e-3 * scale, err_msg=name)
+
+
+def test_layer_stack_gradients_through_moe():
+  """mtf.gradients of the output and the MoE loss through rms_norm -> MoE1D
+  -> residual -> final rms_norm: the block operations' and the MoE layer's
+  backward passes chained by the graph, against the oracles chained by hand."""
+  b, l, m, e, hdim, group = 2, 64, 64, 4, 96, 32
+  rng = np.random.default_rng(53)
+  layers, final = _build_stack(rng, m, e, hdim, 4, 16, group)
+  mo = layers[1]
+  x = rng.standard_normal((b, l, m)).astype(np.float32)
+  dy = rng.standard_normal((b, l, m)).astype(np.float32)
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  dims = [mtf.Dimension("batch", b), mtf.Dimension("length", l),
+          mtf.Dimension("d_model", m)]
+  xt = mtf.import_tf_tensor(mesh, torch.from_numpy(x), mtf.Shape(dims))
+  dyt = mtf.import_tf_tensor(mesh, torch.from_numpy(dy), mtf.Shape(dims))
+  stack = transformer.make_layer_stack(
+      [(moe.MoE1D, dict(num_experts=e, hidden_size=hdim, group_size=group,
+                        second_policy_train="all", second_policy_eval="all",
+                        capacity_factor_eval=2.0))],
+      num_layers=1, block_scope=False)
+  model = transformer.Unitransformer(stack, d_model=m, name="decoder")
+  y, losses = model.call_layers(xt, mtf.VariableDType(torch.float32),
+                                mode="eval")
+  p = "decoder/layer_000/"
+  init = {"decoder/rms_norm/scale": final, p + "rms_norm/scale": mo["scale"],
+          p + "MoE1D/top_2_gating/kernel": mo["w_gate"],
+          p + "MoE1D/wi/kernel": mo["wi"], p + "MoE1D/wo/kernel": mo["wo"]}
+  variables = {v.name: v for v in graph.all_variables}
+  names = sorted(init)
+  assert sorted(variables) == names and len(losses) == 1
+  grads = mtf.gradients([y, losses[0]],
+                        [xt] + [variables[n].outputs[0] for n in names],
+                        [dyt, None])
+  lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()}, initial_values=init)
+  got = {n: H.to_np(lowering.export_to_tf_tensor(g))
+         for n, g in zip(["x"] + names, grads)}
+  hp = mo["hparams"]
+  h = B.rms_norm(x, mo["scale"])
+  out, _, aux = O.moe_layer_v1(h, mo["w_gate"], mo["wi"], mo["wo"], hp, False,
+                               "float32", dense=False)
+  top = -np.sort(-aux["logits"], axis=-1)[..., :3]
+  assert ((top[..., :-1] - top[..., 1:]) > 1e-4).all()   # no near-tied routing
+  x1 = x + out
+  want = {}
+  dx1, want["decoder/rms_norm/scale"] = B.rms_norm_backward(x1, final, dy)
+  # the loss reaches the graph multiplied by moe_loss_coef inside the layer;
+  # its gradient is seeded with 1
+  g = O.moe_layer_v1_backward(h, mo["w_gate"], mo["wi"], mo["wo"], hp, False,
+                              "float32", dx1, d_loss=1.0)
+  want[p + "MoE1D/top_2_gating/kernel"] = g["dw_gate"]
+  want[p + "MoE1D/wi/kernel"] = g["dwi"]
+  want[p + "MoE1D/wo/kernel"] = g["dwo"]
+  d0, want[p + "rms_norm/scale"] = B.rms_norm_backward(x, mo["scale"], g["dx"])
+  want["x"] = dx1 + d0
+  for name in ["x"] + names:
+    scale = max(1.0, float(np.abs(want[name]).max()))
+    np.testing.assert_allclose(got[name], want[name], rtol=1e-3,
+                               atol=1e-3 * scale, err_msg=name)
