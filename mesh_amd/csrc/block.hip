@@ -177,6 +177,88 @@ __global__ __launch_bounds__(256) void attention_softmax_kernel(
     store_f32<T>(wr + j, j < visible ? expf(xr[j] + neglse) : 0.0f);
 }
 
+// The same softmax for bf16 weights and rows of ITERS * 512 logits: a lane
+// keeps its 8 * ITERS logits in registers (one pass over memory), reads them
+// 32 bytes at a time and writes 16 bytes of weights at a time.
+template <int ITERS>
+__global__ __launch_bounds__(256) void attention_softmax_rows_kernel(
+    const float* __restrict__ logits, bf16_t* __restrict__ weights,
+    int64_t rows, int causal) {
+  constexpr int L = ITERS * 512;
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const int visible = causal ? (int)(row % L) + 1 : L;
+  const float* xr = logits + row * L;
+  float v[ITERS][8];
+  float m = -INFINITY;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int base = (it * 64 + lane) * 8;
+    if (base < visible) {
+      const float4 a = *reinterpret_cast<const float4*>(xr + base);
+      const float4 b = *reinterpret_cast<const float4*>(xr + base + 4);
+      const float t[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        v[it][j] = base + j < visible ? t[j] : -INFINITY;
+        m = fmaxf(m, v[it][j]);
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[it][j] = -INFINITY;
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
+  const float negm = -m;
+  float sum = 0.f;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+    for (int j = 0; j < 8; ++j) sum += expf(v[it][j] + negm);   // exp(-inf) = 0
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+  const float neglse = -(logf(sum) + m);
+  bf16_t* wr = weights + row * L;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int base = (it * 64 + lane) * 8;
+    uint4 o;
+    bf16_t* os = reinterpret_cast<bf16_t*>(&o);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      store_f32<bf16_t>(os + j, expf(v[it][j] + neglse));
+    *reinterpret_cast<uint4*>(wr + base) = o;
+  }
+}
+
+// Picks the register-resident kernel where the row length allows it.
+template <typename T>
+static void launch_attention_softmax(const float* logits, T* weights,
+                                     int64_t rows, int L, int causal,
+                                     hipStream_t st) {
+  const unsigned blocks = (unsigned)((rows + 3) / 4);
+  if constexpr (sizeof(T) == 2) {
+    const bool aligned =
+        (((uintptr_t)logits | (uintptr_t)weights) % 32) == 0;
+    if (aligned && L == 512)
+      return attention_softmax_rows_kernel<1><<<blocks, 256, 0, st>>>(
+          logits, weights, rows, causal);
+    if (aligned && L == 1024)
+      return attention_softmax_rows_kernel<2><<<blocks, 256, 0, st>>>(
+          logits, weights, rows, causal);
+    if (aligned && L == 2048)
+      return attention_softmax_rows_kernel<4><<<blocks, 256, 0, st>>>(
+          logits, weights, rows, causal);
+    if (aligned && L == 4096)
+      return attention_softmax_rows_kernel<8><<<blocks, 256, 0, st>>>(
+          logits, weights, rows, causal);
+  }
+  attention_softmax_kernel<T><<<blocks, 256, 0, st>>>(logits, weights, rows, L,
+                                                      causal);
+}
+
 template <typename T>
 static int run_attention(const T* q, const T* k, const T* v, T* out, int B,
                          int L, int H, int D, int causal, int dtype,
@@ -203,8 +285,7 @@ static int run_attention(const T* q, const T* k, const T* v, T* out, int B,
   int rc = batched_gemm_nt(qh, kh, logits, BH, L, L, D, dtype, true, st);
   if (rc != 0) return rc;
   const int64_t rows = (int64_t)BH * L;
-  attention_softmax_kernel<T><<<(unsigned)((rows + 3) / 4), 256, 0, st>>>(
-      logits, weights, rows, L, causal);
+  launch_attention_softmax<T>(logits, weights, rows, L, causal, st);
   MOE_CHECK_LAUNCH("self_attention (softmax)");
   rc = batched_gemm_nt(weights, vt, oh, BH, L, D, L, dtype, false, st);
   if (rc != 0) return rc;
@@ -309,6 +390,49 @@ __global__ __launch_bounds__(256) void softmax_backward_kernel(
     store_f32<T>(outr + j, load_f32<T>(wr + j) * (load_f32<T>(dr + j) - dot));
 }
 
+// The same for bf16 rows of ITERS * 512 elements, both rows held in registers
+// and moved 16 bytes at a time.
+template <int ITERS>
+__global__ __launch_bounds__(256) void softmax_backward_rows_kernel(
+    const bf16_t* __restrict__ w, const bf16_t* __restrict__ dw,
+    bf16_t* __restrict__ dlogits, int64_t rows) {
+  constexpr int L = ITERS * 512;
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const bf16_t* wr = w + row * L;
+  const bf16_t* dr = dw + row * L;
+  float wv[ITERS][8], dv[ITERS][8];
+  float dot = 0.f;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int base = (it * 64 + lane) * 8;
+    const uint4 a = *reinterpret_cast<const uint4*>(wr + base);
+    const uint4 b = *reinterpret_cast<const uint4*>(dr + base);
+    const bf16_t* as = reinterpret_cast<const bf16_t*>(&a);
+    const bf16_t* bs = reinterpret_cast<const bf16_t*>(&b);
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      wv[it][j] = load_f32<bf16_t>(as + j);
+      dv[it][j] = load_f32<bf16_t>(bs + j);
+      dot = fmaf(dv[it][j], wv[it][j], dot);
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off);
+  bf16_t* outr = dlogits + row * L;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int base = (it * 64 + lane) * 8;
+    uint4 o;
+    bf16_t* os = reinterpret_cast<bf16_t*>(&o);
+#pragma unroll
+    for (int j = 0; j < 8; ++j)
+      store_f32<bf16_t>(os + j, wv[it][j] * (dv[it][j] - dot));
+    *reinterpret_cast<uint4*>(outr + base) = o;
+  }
+}
+
 // The attention weights alone, heads to the front: weights [B*H, L, L].
 template <typename T>
 static int run_attention_weights(const T* q, const T* k, T* weights, int B,
@@ -330,8 +454,7 @@ static int run_attention_weights(const T* q, const T* k, T* weights, int B,
   int rc = batched_gemm_nt(qh, kh, logits, BH, L, L, D, dtype, true, st);
   if (rc != 0) return rc;
   const int64_t rows = (int64_t)BH * L;
-  attention_softmax_kernel<T><<<(unsigned)((rows + 3) / 4), 256, 0, st>>>(
-      logits, weights, rows, L, causal);
+  launch_attention_softmax<T>(logits, weights, rows, L, causal, st);
   MOE_CHECK_LAUNCH("attention_weights (softmax)");
   return 0;
 }
@@ -516,10 +639,24 @@ extern "C" int mesh_moe_softmax_backward(const void* weights,
     softmax_backward_kernel<float><<<(unsigned)blocks, 256, 0, st>>>(
         (const float*)weights, (const float*)dweights, (float*)dlogits, rows,
         L);
-  else
-    softmax_backward_kernel<bf16_t><<<(unsigned)blocks, 256, 0, st>>>(
-        (const bf16_t*)weights, (const bf16_t*)dweights, (bf16_t*)dlogits, rows,
-        L);
+  else {
+    const bf16_t* w = (const bf16_t*)weights;
+    const bf16_t* dw = (const bf16_t*)dweights;
+    bf16_t* dl = (bf16_t*)dlogits;
+    const unsigned nb = (unsigned)blocks;
+    const bool aligned =
+        (((uintptr_t)w | (uintptr_t)dw | (uintptr_t)dl) % 16) == 0;
+    if (aligned && L == 512)
+      softmax_backward_rows_kernel<1><<<nb, 256, 0, st>>>(w, dw, dl, rows);
+    else if (aligned && L == 1024)
+      softmax_backward_rows_kernel<2><<<nb, 256, 0, st>>>(w, dw, dl, rows);
+    else if (aligned && L == 2048)
+      softmax_backward_rows_kernel<4><<<nb, 256, 0, st>>>(w, dw, dl, rows);
+    else if (aligned && L == 4096)
+      softmax_backward_rows_kernel<8><<<nb, 256, 0, st>>>(w, dw, dl, rows);
+    else
+      softmax_backward_kernel<bf16_t><<<nb, 256, 0, st>>>(w, dw, dl, rows, L);
+  }
   MOE_CHECK_LAUNCH("softmax_backward");
   return 0;
 }

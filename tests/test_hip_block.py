@@ -603,7 +603,9 @@ def test_block_backward_entries(hip, act_dtype):
                                atol=tol["atol"] * 4)
   for bsz, length, heads, d, causal in ((2, 64, 4, 16, True),
                                         (1, 128, 2, 64, False),
-                                        (2, 256, 2, 128, True)):
+                                        (2, 256, 2, 128, True),
+                                        (1, 512, 2, 64, True),
+                                        (1, 1024, 1, 64, False)):
     q, kk, v, do = (rnd(bsz, length, heads * d) * np.float32(0.5)
                     for _ in range(4))
     q, kk, v, do = (O.cast_act(t, act_dtype) for t in (q, kk, v, do))
