@@ -16,6 +16,11 @@ moe_oracle.  What pins each function (tests/test_block_oracle.py):
                    queries give the running mean of the values
   layer_stack      zero output kernels reduce the stack to its final norm;
                    one layer by hand
+  rms_norm_backward, dense_backward, attention_core_backward
+                   float64 central differences of the forward formulas along
+                   random directions, for every input; x-direction of the
+                   norm's gradient vanishes when dy = x; the first causal
+                   query's dq is zero
   dropout noise    (broadcast_dropout and the noise arguments) noise of ones
                    is the identity; float64 product; noise on the attention
                    weights equals noise on the values
