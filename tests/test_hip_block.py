@@ -752,3 +752,74 @@ def test_layer_stack_gradients_through_moe():
     scale = max(1.0, float(np.abs(want[name]).max()))
     np.testing.assert_allclose(got[name], want[name], rtol=1e-3,
                                atol=1e-3 * scale, err_msg=name)
+
+
+def test_layer_stack_gradients_bfloat16_follow_float32():
+  """The whole lm_moe block (attention, MoE1D, attention, DenseReluDense) in
+  bfloat16: every gradient is finite, has its variable's shape and points the
+  way the float32 gradient of the same graph does (cosine > 0.97; routing may
+  differ for a few nearly tied tokens)."""
+  b, l, m, e, hdim, heads, d, group = 2, 128, 128, 4, 256, 4, 32, 64
+  rng = np.random.default_rng(54)
+  layers, final = _build_stack(rng, m, e, hdim, heads, d, group)
+  x = O.round_bf16(rng.standard_normal((b, l, m)).astype(np.float32))
+  dy = O.round_bf16(rng.standard_normal((b, l, m)).astype(np.float32))
+
+  def run(dt):
+    graph = mtf.Graph()
+    mesh = mtf.Mesh(graph, "mesh")
+    dims = [mtf.Dimension("batch", b), mtf.Dimension("length", l),
+            mtf.Dimension("d_model", m)]
+    xt = mtf.import_tf_tensor(mesh, torch.from_numpy(x).to(dt), mtf.Shape(dims))
+    dyt = mtf.import_tf_tensor(mesh, torch.from_numpy(dy).to(dt),
+                               mtf.Shape(dims))
+    att = (transformer_layers.SelfAttention,
+           dict(num_heads=heads, key_value_size=d))
+    stack = transformer.make_layer_stack(
+        [att,
+         (moe.MoE1D, dict(num_experts=e, hidden_size=hdim, group_size=group,
+                          second_policy_train="all", second_policy_eval="all",
+                          capacity_factor_eval=2.0)),
+         att, (transformer_layers.DenseReluDense, dict(hidden_size=hdim))],
+        num_layers=1, block_scope=False)
+    model = transformer.Unitransformer(stack, d_model=m, name="decoder",
+                                       autoregressive=True)
+    y, losses = model.call_layers(
+        xt, mtf.VariableDType(torch.float32, torch.float32, dt), mode="eval")
+    init = {"decoder/rms_norm/scale": final}
+    for i, layer in enumerate(layers):
+      p = "decoder/layer_%03d/" % i
+      init[p + "rms_norm/scale"] = layer["scale"]
+      if layer["kind"] == "attention":
+        for kname in "qkvo":
+          init[p + "SelfAttention/" + kname] = layer["w" + kname]
+      elif layer["kind"] == "moe":
+        init[p + "MoE1D/top_2_gating/kernel"] = layer["w_gate"]
+        init[p + "MoE1D/wi/kernel"] = layer["wi"]
+        init[p + "MoE1D/wo/kernel"] = layer["wo"]
+      else:
+        init[p + "DenseReluDense/wi/kernel"] = layer["wi"]
+        init[p + "DenseReluDense/wo/kernel"] = layer["wo"]
+    variables = {v.name: v for v in graph.all_variables}
+    names = sorted(init)
+    grads = mtf.gradients([y] + list(losses),
+                          [xt] + [variables[n].outputs[0] for n in names],
+                          [dyt] + [None] * len(losses))
+    lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()},
+                            initial_values=init)
+    out = {}
+    for n, g in zip(["x"] + names, grads):
+      shape = x.shape if n == "x" else np.shape(init[n])
+      value = H.to_np(lowering.export_to_tf_tensor(g))
+      assert value.shape == tuple(shape), n
+      out[n] = value
+    return out
+
+  ref = run(torch.float32)
+  got = run(torch.bfloat16)
+  for name, want in ref.items():
+    g = got[name].astype(np.float64).ravel()
+    w = want.astype(np.float64).ravel()
+    assert np.isfinite(g).all(), name
+    cos = float(g @ w / (np.linalg.norm(g) * np.linalg.norm(w) + 1e-30))
+    assert cos > 0.97, (name, cos)
