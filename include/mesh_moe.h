@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 16
+#define MESH_MOE_ABI_VERSION 17
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -120,6 +120,33 @@ int mesh_moe_top2_gating(const float* logits, const void* importance,
                          float* gate, uint8_t* kept, int32_t* fill,
                          float* loss, void* workspace, size_t workspace_bytes,
                          void* stream);
+
+/* Size of the scratch array mesh_moe_top2_gating_static_scratch keeps on
+ * every GPU the library runs on, until the process ends. */
+#define MESH_MOE_STATIC_SCRATCH_BYTES (4u << 20)
+
+/*
+ * mesh_moe_top2_gating without the workspace argument.  It has no counterpart
+ * in the reference: it exists for callers that cannot allocate device memory
+ * or carry a workspace around (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  The scratch memory the kernels
+ * need (per-block partial sums of the loss, per-group sums) lives in an array
+ * of MESH_MOE_STATIC_SCRATCH_BYTES that is part of the library's device code;
+ * its address is looked up once per device, on the first call made with that
+ * device current.  The call allocates and frees nothing.
+ * Same arguments, results and limits as mesh_moe_top2_gating, plus:
+ * MESH_MOE_E_UNSUPPORTED (nothing launched) when
+ * mesh_moe_gating_workspace_bytes(G, S, E) > MESH_MOE_STATIC_SCRATCH_BYTES.
+ * Every call on a GPU shares that GPU's array: two calls that overlap in time
+ * on one GPU (different streams, or different threads) race; serialise them.
+ * Nothing in the array has to survive between calls or start at zero.
+ */
+int mesh_moe_top2_gating_static_scratch(
+    const float* logits, const void* importance, int importance_dtype,
+    int importance_from_slot_gate, const float* second_uniform, int G, int S,
+    int E, int C, int policy, double threshold, int use_second_place_loss,
+    int num_microbatches, int32_t* idx, int32_t* pos, float* gate,
+    uint8_t* kept, int32_t* fill, float* loss, void* stream);
 
 /*
  * Router projection and top-2 gating in one call: what _top_2_gating does from

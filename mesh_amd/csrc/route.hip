@@ -5,6 +5,8 @@
 // float32 operation order of mtf.softmax (ops.py:5493-5541) and mtf.top_1
 // (ops.py:4937-4940).  The dense [G,S,E] masks and the S x S cumsum matmul
 // (ops.py:2761-2781) are replaced by a per-token record and integer counting.
+#include <mutex>
+
 #include "common.h"
 
 namespace mesh_moe {
@@ -1069,6 +1071,65 @@ static int run_router_gating(const GateParams& p, const void* x,
   if (rc != 0) return rc;
   return launch_capacity_and_loss(p, idx, pos, gate, kept, fill, loss, part1,
                                   part2, gsum, st);
+}
+
+// ---------------------------------------------------------------------------
+// Scratch memory of mesh_moe_top2_gating_static_scratch: what the other gating
+// calls take from the caller as `workspace`.  Every GPU holds its own copy of
+// the array at its own address; in host code the array's name is only a
+// handle for hipGetSymbolAddress, never a device address.
+// ---------------------------------------------------------------------------
+constexpr size_t STATIC_SCRATCH_BYTES = (size_t)MESH_MOE_STATIC_SCRATCH_BYTES;
+static __device__ __align__(256) unsigned char scratch[STATIC_SCRATCH_BYTES];
+
+constexpr int STATIC_SCRATCH_MAX_DEVICES = 64;
+static std::mutex g_scratch_mutex;
+static void* g_scratch_ptr[STATIC_SCRATCH_MAX_DEVICES] = {};
+
+// Device address of `scratch` on the current device, looked up once per
+// device; nullptr (error text set) if the runtime refuses.
+static void* static_scratch_address() {
+  int dev = -1;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess || dev < 0 || dev >= STATIC_SCRATCH_MAX_DEVICES) {
+    mesh_moe::set_error("static scratch: hipGetDevice gave device %d (%s)", dev,
+                        hipGetErrorString(e));
+    return nullptr;
+  }
+  std::lock_guard<std::mutex> lock(g_scratch_mutex);
+  if (g_scratch_ptr[dev] == nullptr) {
+    void* ptr = nullptr;
+    e = hipGetSymbolAddress((void**)&ptr, HIP_SYMBOL(scratch));
+    if (e != hipSuccess || ptr == nullptr) {
+      mesh_moe::set_error("static scratch: hipGetSymbolAddress: %s",
+                          hipGetErrorString(e));
+      return nullptr;
+    }
+    g_scratch_ptr[dev] = ptr;
+  }
+  return g_scratch_ptr[dev];
+}
+
+extern "C" int mesh_moe_top2_gating_static_scratch(
+    const float* logits, const void* importance, int importance_dtype,
+    int importance_from_slot_gate, const float* second_uniform, int G, int S,
+    int E, int C, int policy, double threshold, int use_second_place_loss,
+    int num_microbatches, int32_t* idx, int32_t* pos, float* gate,
+    uint8_t* kept, int32_t* fill, float* loss, void* stream) {
+  MOE_REQUIRE(G >= 1 && S >= 1 && E >= 1, MESH_MOE_E_ARG,
+              "top2_gating_static_scratch: bad sizes G=%d S=%d E=%d", G, S, E);
+  const size_t need = mesh_moe_gating_workspace_bytes(G, S, E);
+  MOE_REQUIRE(need <= STATIC_SCRATCH_BYTES, MESH_MOE_E_UNSUPPORTED,
+              "top2_gating_static_scratch: G=%d S=%d E=%d needs %zu bytes of "
+              "scratch, the built-in buffer has %zu; use mesh_moe_top2_gating "
+              "with a workspace", G, S, E, need, STATIC_SCRATCH_BYTES);
+  void* ptr = static_scratch_address();
+  if (ptr == nullptr) return MESH_MOE_E_HIP;
+  return mesh_moe_top2_gating(logits, importance, importance_dtype,
+                              importance_from_slot_gate, second_uniform, G, S,
+                              E, C, policy, threshold, use_second_place_loss,
+                              num_microbatches, idx, pos, gate, kept, fill,
+                              loss, ptr, STATIC_SCRATCH_BYTES, stream);
 }
 
 extern "C" int mesh_moe_top2_gating(

@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 16
+ABI_VERSION = 17
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -40,6 +40,10 @@ _SIGNATURES = {
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_double, ctypes.c_int,
         ctypes.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_size_t,
         _vp]),
+    "mesh_moe_top2_gating_static_scratch": (ctypes.c_int, [
+        _vp, _vp, ctypes.c_int, ctypes.c_int, _vp, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_double, ctypes.c_int,
+        ctypes.c_int, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "mesh_moe_router_top2_gating": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int64, ctypes.c_int,
         ctypes.c_int, _vp, ctypes.c_int, ctypes.c_int, _vp, ctypes.c_int,
@@ -360,6 +364,45 @@ def top2_gating(logits, capacity, importance=None, policy="all",
   if _timer is not None:
     _timer.routing.append(r)
   return r
+
+
+STATIC_SCRATCH_BYTES = 4 << 20
+
+
+def top2_gating_static_scratch(logits, capacity, out, importance=None,
+                               policy="all", threshold=0.2,
+                               use_second_place_loss=False,
+                               num_microbatches=None, second_uniform=None,
+                               importance_from_slot_gate=False):
+  """top2_gating into the caller's Routing `out`, on the library's built-in
+  scratch array: neither this function nor the call behind it allocates.
+  Calls that overlap on one GPU race for that array."""
+  lib = load_library()
+  if policy not in POLICIES:
+    raise ValueError("Unknown policy %s" % policy)
+  g, s, e = logits.shape
+  lp = _dev(logits, "logits", torch.float32)
+  ip, icode = None, F32
+  if importance is not None:
+    icode = dtype_code(importance.dtype)
+    ip = _dev(importance, "importance", None, (g, s))
+  up = None
+  if second_uniform is not None:
+    up = _dev(second_uniform, "second_uniform", torch.float32, (g, s))
+  ptrs = [_dev(out.idx, "idx", torch.int32, (g, s, 2)),
+          _dev(out.pos, "pos", torch.int32, (g, s, 2)),
+          _dev(out.gate, "gate", torch.float32, (g, s, 2)),
+          _dev(out.kept, "kept", torch.uint8, (g, s, 2)),
+          _dev(out.fill, "fill", torch.int32, (g, e)),
+          _dev(out.loss, "loss", torch.float32, (1,))]
+  with _stage("top2_gating"):
+    _check(lib.mesh_moe_top2_gating_static_scratch(
+        lp, ip, icode, int(bool(importance_from_slot_gate)), up, g, s, e,
+        int(capacity), POLICIES[policy], float(threshold),
+        int(bool(use_second_place_loss)), int(num_microbatches or 1),
+        *ptrs, _stream()), "top2_gating_static_scratch")
+  out.capacity, out.num_experts = int(capacity), e
+  return out
 
 
 def fused_gating_supported(x, num_experts, group_size):
