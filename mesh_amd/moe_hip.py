@@ -653,10 +653,12 @@ def expert_ffn(expert_in, wi_packed, wo_packed, activation="relu", h=None,
 E_UNSUPPORTED = -2
 
 
-def dispatched_expert_ffn(x, r, wi_packed, wo_packed, activation="relu"):
+def dispatched_expert_ffn(x, r, wi_packed, wo_packed, activation="relu",
+                          h=None):
   """dispatch + expert_ffn without materialising expert_in: x [G, S, M], the
   Routing r -> y [E, G*C, N], or None where the library has no such kernel for
-  the case (the caller then makes the two calls)."""
+  the case (the caller then makes the two calls).  h [E, G*C, H], if given,
+  receives the hidden tensor."""
   lib = load_library()
   if activation not in ACTIVATIONS:
     raise ValueError("unsupported expert activation %r" % (activation,))
@@ -667,7 +669,9 @@ def dispatched_expert_ffn(x, r, wi_packed, wo_packed, activation="relu"):
   if dt != torch.bfloat16:
     return None
   dev = x.device
-  h = torch.empty((e, g * c, hdim), dtype=dt, device=dev)
+  if h is None:
+    h = torch.empty((e, g * c, hdim), dtype=dt, device=dev)
+  _dev(h, "h", dt, (e, g * c, hdim))
   y = torch.empty((e, g * c, n), dtype=dt, device=dev)
   ws_bytes = lib.mesh_moe_dispatched_expert_ffn_workspace_bytes(g, e, c, m)
   ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)

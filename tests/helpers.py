@@ -111,3 +111,73 @@ def value_tolerance(act_dtype):
   if act_dtype == "bfloat16":
     return dict(rtol=2e-2, atol=1e-2)
   return dict(rtol=1e-4, atol=2e-5)
+
+
+def assert_routing_properties(r, logits, importance=None):
+  """Size-independent properties of a top-2 Routing `r` (GPU tensors) computed
+  from float32 `logits` [G, S, E] (GPU): what the definition of the capacity
+  assignment (transformer/moe.py:1397-1496) fixes without running the oracle.
+  importance [G, S] float32 with values in {0, 0.5, 1} or None.  Returns the
+  boolean slot occupancy [G, E, C]."""
+  g, s, e = logits.shape
+  c = r.capacity
+  dev = logits.device
+  idx, pos, kept = r.idx.long(), r.pos.long(), r.kept.bool()
+  # first / second expert: argmax and argmax-with-first-removed of the logits
+  # (softmax is monotone; ties have measure zero for continuous random logits)
+  top2 = logits.topk(2, dim=-1).indices
+  if importance is None:
+    assert torch.equal(idx, top2)
+    competing = torch.ones((g, s, 2), dtype=torch.bool, device=dev)
+  else:
+    one = importance == 1.0
+    half = (importance > 0) & ~one
+    assert torch.equal(idx[one], top2[one])
+    # 0 < importance < 1: the best expert, offered as a second choice
+    assert torch.equal(idx[half][:, 1], top2[half][:, 0])
+    competing = torch.stack([one, one | half], dim=-1)
+    assert not bool(kept[~competing].any())
+    assert not bool(r.gate[~competing].any())
+  # every (group, expert) fills slots 0..fill-1 exactly once, fill <= C
+  gi = torch.arange(g, device=dev).view(g, 1, 1).expand(g, s, 2)
+  slot = (gi * e + idx) * c + pos
+  used = torch.zeros(g * e * c, dtype=torch.int32, device=dev)
+  used.scatter_add_(0, slot[kept], torch.ones_like(slot[kept], dtype=torch.int32))
+  assert int(used.max()) <= 1
+  used = used.view(g, e, c)
+  fill = r.fill.long()
+  assert int(fill.max()) <= c
+  want_used = (torch.arange(c, device=dev).view(1, 1, c) < fill.unsqueeze(-1))
+  assert torch.equal(used.bool(), want_used)
+  assert torch.equal(used.sum(-1), fill)
+  # kept <=> position below capacity, for every competing choice
+  assert torch.equal(kept, (pos < c) & competing)
+  # first choices of an expert precede its second choices
+  first_count = torch.zeros(g * e, dtype=torch.long, device=dev)
+  k1 = kept[..., 0]
+  first_count.scatter_add_(0, (gi[..., 0] * e + idx[..., 0])[k1],
+                           torch.ones(int(k1.sum()), dtype=torch.long,
+                                      device=dev))
+  c2 = competing[..., 1]
+  key2 = (gi[..., 1] * e + idx[..., 1])
+  assert bool((pos[..., 1] >= first_count[key2])[c2].all())
+  first_second = torch.full((g * e,), 1 << 40, dtype=torch.long, device=dev)
+  first_second.scatter_reduce_(0, key2[c2], pos[..., 1][c2], reduce="amin")
+  has_second = first_second < (1 << 40)
+  assert torch.equal(first_second[has_second], first_count[has_second])
+  # positions grow by one per competing chooser, in token order, within
+  # (group, expert, choice); choices that do not compete are set aside under
+  # an expert id of their own
+  for k in range(2):
+    ek = torch.where(competing[..., k], idx[..., k], torch.full_like(idx[..., k], e))
+    key = ek * s + torch.arange(s, device=dev).view(1, s)
+    order = key.argsort(dim=1, stable=True)
+    sorted_pos = pos[..., k].gather(1, order)
+    sorted_e = ek.gather(1, order)
+    same = (sorted_e[:, 1:] == sorted_e[:, :-1]) & (sorted_e[:, 1:] < e)
+    assert bool(((sorted_pos[:, 1:] - sorted_pos[:, :-1])[same] == 1).all())
+  # gates: the normalised pair sums to one where both are kept
+  both = kept.all(-1)
+  assert torch.allclose(r.gate.sum(-1)[both], torch.ones((), device=dev),
+                        atol=1e-5)
+  return want_used

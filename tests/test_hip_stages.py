@@ -261,47 +261,10 @@ def test_full_size_routing_properties(hip, size):
     ranks = torch.randperm(e, generator=gen, device="cuda").double() + 1
     logits = logits + (3.0 * ranks ** -1.2).float()
   r = hip.top2_gating(logits, c)
-  idx, pos, kept = r.idx.long(), r.pos.long(), r.kept.bool()
-  # first / second expert: argmax and argmax-with-first-removed of the logits
-  # (softmax is monotone; ties have measure zero for continuous random logits)
-  top2 = logits.topk(2, dim=-1).indices
-  assert torch.equal(idx, top2)
-  # every (group, expert) fills slots 0..fill-1 exactly once, fill <= C
-  gi = torch.arange(g, device="cuda").view(g, 1, 1).expand(g, s, 2)
-  slot = (gi * e + idx) * c + pos
-  used = torch.zeros(g * e * c, dtype=torch.int32, device="cuda")
-  used.scatter_add_(0, slot[kept], torch.ones_like(slot[kept], dtype=torch.int32))
-  assert int(used.max()) <= 1
-  used = used.view(g, e, c)
-  fill = r.fill.long()
-  assert int(fill.max()) <= c
-  want_used = (torch.arange(c, device="cuda").view(1, 1, c) < fill.unsqueeze(-1))
-  assert torch.equal(used.bool(), want_used)
-  assert torch.equal(used.sum(-1), fill)
-  # kept <=> position below capacity, for every competing choice
-  assert torch.equal(kept, pos < c)
-  # first choices of an expert precede its second choices
-  first_count = torch.zeros(g * e, dtype=torch.long, device="cuda")
-  k1 = kept[..., 0]
-  first_count.scatter_add_(0, (gi[..., 0] * e + idx[..., 0])[k1],
-                           torch.ones(int(k1.sum()), dtype=torch.long,
-                                      device="cuda"))
-  base2 = first_count[(gi[..., 1] * e + idx[..., 1])]
-  assert bool((pos[..., 1] >= base2).all())
-  # positions grow with the token index within (group, expert, choice)
-  for k in range(2):
-    key = (idx[..., k] * s + torch.arange(s, device="cuda").view(1, s))
-    order = key.argsort(dim=1, stable=True)
-    sorted_pos = pos[..., k].gather(1, order)
-    sorted_e = idx[..., k].gather(1, order)
-    same = sorted_e[:, 1:] == sorted_e[:, :-1]
-    assert bool(((sorted_pos[:, 1:] - sorted_pos[:, :-1])[same] == 1).all())
+  want_used = H.assert_routing_properties(r, logits)
+  kept = r.kept.bool()
   if skew:
     assert float(kept.float().mean()) < 0.8       # the drop path is exercised
-  # gates: normalised pair sums to one where both kept
-  both = kept.all(-1)
-  assert torch.allclose(r.gate.sum(-1)[both], torch.ones((), device="cuda"),
-                        atol=1e-5)
 
   # dispatch -> combine with identity experts: out = (w1 + w2) * x
   x = torch.randn((g, s, m), generator=gen, device="cuda").to(torch.bfloat16)
@@ -324,17 +287,24 @@ def test_full_size_routing_properties(hip, size):
 @pytest.mark.parametrize("case", [
     # routers, groups per router, S, M, E, C
     (1, 2, 256, 128, 8, 70), (1, 3, 128, 64, 64, 5), (2, 2, 384, 192, 20, 40),
-    (4, 1, 128, 64, 128, 3), (1, 16, 1024, 1024, 32, 40)])
+    (4, 1, 128, 64, 128, 3), (1, 16, 1024, 1024, 32, 40),
+    (1, 32, 2048, 4096, 64, 64)],
+    ids=["e8", "e64", "two_routers", "e128", "cfg2", "cfg4"])
 def test_router_top2_gating_fused(hip, case):
   """The fused router + gating entry point against the oracle (and against the
-  two-call path): bf16 tokens whose router logits do not nearly tie."""
+  two-call path): bf16 tokens whose router logits do not nearly tie.  The last
+  two cases are the full routing shapes of benchmark configurations 2 and 4;
+  the logits the oracle is fed are the float64 product rounded to float32."""
   b, gpr, s, m, e, c = case
   rng = np.random.default_rng(41)
   w = O.round_bf16((rng.standard_normal((b, m, e)) / np.sqrt(m)).astype(np.float32))
   x = np.stack([H.safe_tokens(rng, gpr * s, m, w[i], "bfloat16") for i in range(b)])
   imp = rng.choice(np.array([0.0, 0.5, 1.0], np.float32), size=(b * gpr, s),
                    p=[0.1, 0.2, 0.7])
-  logits = np.matmul(x, w).astype(np.float32).reshape(b * gpr, s, e)
+  logits = np.concatenate([
+      np.matmul(x[:, r0:r0 + 8192].astype(np.float64), w.astype(np.float64))
+      for r0 in range(0, gpr * s, 8192)], axis=1)
+  logits = logits.astype(np.float32).reshape(b * gpr, s, e)
   xg, wg = H.to_gpu(x, "bfloat16"), H.to_gpu(w, "bfloat16")
   wp = hip.pack_weights(wg, wg.dtype)
   assert hip.fused_gating_supported(xg, e, s)
@@ -820,6 +790,39 @@ def test_dispatched_expert_ffn_equals_two_calls(hip, shape):
   if g * c == 256:
     r2 = hip.top2_gating(torch.from_numpy(logits).cuda(), c + 32)
     assert hip.dispatched_expert_ffn(x, r2, wi_p, wo_p, "relu") is None
+
+
+def test_dispatched_expert_ffn_equals_two_calls_cfg4(hip):
+  """The same identity at the full size of benchmark configuration 4 (32 groups
+  of 2048 tokens, 64 experts, capacity 64, d_model 4096, hidden 16384), where
+  the gathered GEMM is the kernel the benchmark times: hidden and output
+  tensors bit for bit equal to dispatch + expert FFN, with empty slots (a
+  biased router leaves some experts short) and kept choices of gate 0."""
+  g, s, e, c, m, hdim = 32, 2048, 64, 64, 4096, 16384
+  gen = torch.Generator(device="cuda")
+  gen.manual_seed(23)
+  logits = torch.randn((g, s, e), generator=gen, device="cuda")
+  ranks = torch.randperm(e, generator=gen, device="cuda").double() + 1
+  logits = logits + (1.5 * ranks ** -1.2).float()
+  x = torch.randn((g, s, m), generator=gen, device="cuda").to(torch.bfloat16)
+  wi = torch.empty((e, hdim, m), dtype=torch.bfloat16, device="cuda")
+  wo = torch.empty((e, m, hdim), dtype=torch.bfloat16, device="cuda")
+  for i in range(e):                         # packed layout [E, N, K] directly
+    wi[i] = (torch.randn((hdim, m), generator=gen, device="cuda") / m ** 0.5).to(torch.bfloat16)
+    wo[i] = (torch.randn((m, hdim), generator=gen, device="cuda") / hdim ** 0.5).to(torch.bfloat16)
+  r = hip.top2_gating(logits, c)
+  r.gate[0, 0, 0] = 0.0
+  r.gate[g - 1, s - 1, 1] = 0.0
+  assert int((r.fill < c).sum()) > 0 and int((r.fill == c).sum()) > 0
+  h_want = torch.empty((e, g * c, hdim), dtype=torch.bfloat16, device="cuda")
+  h_got = torch.empty_like(h_want)
+  want = hip.expert_ffn(hip.dispatch(x, r).reshape(e, g * c, m), wi, wo, "relu",
+                        h=h_want)
+  got = hip.dispatched_expert_ffn(x, r, wi, wo, "relu", h=h_got)
+  assert got is not None
+  assert torch.equal(h_got, h_want)
+  assert torch.equal(got, want)
+  assert bool(torch.isfinite(got.float()).all())
 
 
 @pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])

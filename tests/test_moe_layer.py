@@ -261,6 +261,32 @@ def v2_weights(rng, m, hdim, xe, ye):
               wo=H.normal_weights(rng, (ye, xe, hdim, m), hdim))
 
 
+def safe_tokens_v2(rng, x, w, act_dtype, min_gap=2e-4):
+  """Redraws the rows of x [n_tok, m] whose three largest logits are closer
+  than min_gap under the outer router (1e-3 there, as H.safe_tokens) or under
+  any outer expert's inner router: whichever slots a token lands in, its inner
+  routing then does not depend on the summation order of the projection."""
+  routers = [(O.cast_act(w["w_outer"], act_dtype), 1e-3)] + [
+      (O.cast_act(wi, act_dtype), min_gap) for wi in w["w_inner"]]
+  x = x.copy()
+  todo = np.ones(x.shape[0], bool)
+  for _ in range(100):
+    rows = x[todo]
+    bad = np.zeros(rows.shape[0], bool)
+    for wr, gap in routers:
+      top = -np.sort(-O.router_logits(rows, wr), axis=-1)[..., :3]
+      bad |= ((top[..., :-1] - top[..., 1:]) < gap).any(axis=-1)
+    where = np.flatnonzero(todo)[bad]
+    if where.size == 0:
+      return x
+    x[where] = O.cast_act(
+        rng.standard_normal((where.size, x.shape[1])).astype(np.float32),
+        act_dtype)
+    todo[:] = False
+    todo[where] = True
+  raise AssertionError("could not separate the inner router logits")
+
+
 def inner_gap_ok(aux, min_gap=1e-4):
   """True if no inner-level row that is actually routed has a near-tie."""
   logits = aux["logits_inner"]
@@ -275,6 +301,12 @@ V2_CASES = [
     ("bf16", (2, 64, 16), 32, 4, 4, 32, 1.25, 1.0, "bfloat16"),
     ("outer_batch_f32", (1, 4, 96, 24), 48, 3, 5, 64, 2.0, 1.5, "float32"),
     ("mid_bf16", (8, 256, 128), 256, 4, 8, 256, 1.25, 1.25, "bfloat16"),
+    # the expert grid, group size and capacity factors of benchmark
+    # configuration 5 (8 x 16 experts, groups of 1024, 1.25 at both levels) on
+    # half the tokens and a sixteenth of d_model / hidden size: outer capacity
+    # 160, 16 * 160 slots per outer expert -> 2 inner groups of 1280, inner
+    # capacity 100
+    ("x8y16_bf16", (16, 1024, 128), 512, 8, 16, 1024, 1.25, 1.25, "bfloat16"),
 ]
 
 
@@ -290,6 +322,10 @@ def test_v2_matches_oracle(case):
     rng = np.random.default_rng(seed)
     w = v2_weights(rng, m, hdim, xe, ye)
     x = H.safe_tokens(rng, n_tok, m, w["w_outer"], act_dtype).reshape(shape)
+    if n_tok > 4096:
+      # too many inner rows for a whole seed to be free of near-ties: redraw
+      # the tokens that nearly tie under any outer expert's inner router
+      x = safe_tokens_v2(rng, x.reshape(n_tok, m), w, act_dtype).reshape(shape)
     want, want_loss, aux = O.moe_layer_v2(
         x, w["w_outer"], w["w_inner"], w["wi"], w["wo"], ohp, True, act_dtype,
         dense=n_tok <= 1024)
@@ -300,6 +336,195 @@ def test_v2_matches_oracle(case):
   np.testing.assert_allclose(got, want, **H.value_tolerance(act_dtype))
   np.testing.assert_allclose(got_loss, want_loss,
                              rtol=1e-2 if act_dtype == "bfloat16" else 1e-5)
+
+
+def _device_normal(fan_in, seed):
+  """N(0, 1/sqrt(fan_in)) drawn on the device one leading index at a time."""
+  def init(sizes, dtype, device):
+    gen = torch.Generator(device=device)
+    gen.manual_seed(seed)
+    out = torch.empty(sizes, dtype=dtype, device=device)
+    flat = out.reshape(sizes[0], -1) if len(sizes) > 2 else out.reshape(1, -1)
+    for i in range(flat.shape[0]):
+      row = torch.randn(flat.shape[1], generator=gen, device=device)
+      flat[i] = (row / fan_in ** 0.5).to(dtype)
+    return out
+  return init
+
+
+def _gather_combine(y4, r, group_size):
+  """combine as a gather in torch: y4 [E, G, C, N], one rounding of
+  w1 * y[slot1] + w2 * y[slot2] with the activation-dtype gates."""
+  g = r.idx.shape[0]
+  idx, kept = r.idx.long(), r.kept.bool()
+  pos = r.pos.long().clamp(max=r.capacity - 1)
+  w = r.gate.to(y4.dtype).float() * kept.float()
+  gi = torch.arange(g, device=y4.device).view(g, 1).expand(g, group_size)
+  y1 = y4[idx[..., 0], gi, pos[..., 0]].float()
+  y2 = y4[idx[..., 1], gi, pos[..., 1]].float()
+  return (w[..., 0:1] * y1 + w[..., 1:2] * y2).to(y4.dtype)
+
+
+def _float64_balancing_loss(logits, is_one=None):
+  """mean over [G, E] of mean_s(p * [imp == 1]) * mean_s(mask_1) * E^2
+  (transformer/moe.py:1400-1404, :1420-1424) in float64."""
+  p = torch.softmax(logits.double(), dim=-1)
+  e = logits.shape[-1]
+  mask_1 = torch.nn.functional.one_hot(logits.argmax(-1), e).double()
+  if is_one is not None:
+    p = p * is_one.double().unsqueeze(-1)
+    mask_1 = mask_1 * is_one.double().unsqueeze(-1)
+  return float((p.mean(1) * mask_1.mean(1)).mean() * e * e)
+
+
+def test_v2_cfg5_full_size_properties():
+  """Benchmark configuration 5 at full size: transformer_moe_layer_v2 on 32 x
+  1024 bf16 tokens, 8 x 16 experts, d_model 2048, hidden 8192, capacity factor
+  1.25 at both levels (outer capacity 160; 5120 slots per outer expert -> 5
+  inner groups of 1024, inner capacity 80).  The oracle is too slow here, so
+  the layer's output is tied, bit for bit, to the library's stages run by hand
+  with the logits kept, and each stage is checked through properties: the
+  routing records of both levels (slots unique and contiguous, first choices
+  before second ones, positions in token order), the inner importance in
+  {0, 0.5, 1} with as many of each as the outer level kept first / second
+  choices, dispatch and combine against torch gathers, sampled row blocks of
+  the experts against float32 matmuls, zero rows for tokens dropped
+  everywhere, and both balancing losses against float64."""
+  from mesh_amd import moe_hip as hip
+  b, l, m, hdim, xe, ye = 32, 1024, 2048, 8192, 8, 16
+  s_, c_, h0, t_, d_ = 1024, 160, 5, 1024, 80
+  dt = torch.bfloat16
+  hp, _ = make_hparams(moe_num_experts=[xe, ye], moe_hidden_size=hdim,
+                       moe_group_size=1024, moe_capacity_factor_train=1.25,
+                       moe_capacity_factor_second_level=1.25)
+  gen = torch.Generator(device="cuda")
+  gen.manual_seed(55)
+  x_val = torch.randn((b, l, m), generator=gen, device="cuda").to(dt)
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  dims = [mtf.Dimension("batch", b), mtf.Dimension("length", l),
+          mtf.Dimension("d_model", m)]
+  xt = mtf.import_tf_tensor(mesh, x_val, mtf.Shape(dims))
+  with mtf.variable_scope("moe2d"):
+    y, loss = moe.transformer_moe_layer_v2(
+        xt, dims[-1], hp, True, mtf.VariableDType(dt, dt, dt))
+  init = {"moe2d/outer_gating/kernel": _device_normal(m, 2),
+          "moe2d/inner_gating/kernel": _device_normal(m, 5),
+          "moe2d/wi/kernel": _device_normal(m, 3),
+          "moe2d/wo/kernel": _device_normal(hdim, 4)}
+  with hip.StageTimer() as timer:
+    lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()},
+                            initial_values=init)
+  out = lowering.export_to_tf_tensor(y)
+  got_loss = float(lowering.export_to_tf_tensor(loss).float())
+  assert tuple(out.shape) == (b, l, m) and out.dtype == dt
+  assert bool(torch.isfinite(out.float()).all())
+  rx, ry = timer.routing
+  assert (rx.capacity, rx.num_experts, tuple(rx.idx.shape)) == (c_, xe, (b, s_, 2))
+  assert (ry.capacity, ry.num_experts, tuple(ry.idx.shape)) == (
+      d_, ye, (xe * h0, t_, 2))
+  var = {v.name: lv for v, lv in lowering.variables.items()}
+  w_outer = var["moe2d/outer_gating/kernel"].master            # [m, x]
+  w_inner = var["moe2d/inner_gating/kernel"].master            # [x, m, y]
+  wi_p = var["moe2d/wi/kernel"].packed(dt)                     # [y*x, hidden, m]
+  wo_p = var["moe2d/wo/kernel"].packed(dt)                     # [y*x, m, hidden]
+
+  def same_record(a, b_):
+    return all(torch.equal(getattr(a, k), getattr(b_, k))
+               for k in ("idx", "pos", "gate", "kept", "fill", "loss"))
+
+  # ---- outer level
+  xg = x_val.reshape(b, s_, m)
+  rx2, logits_x = hip.router_top2_gating(
+      xg.reshape(1, b * s_, m), hip.pack_weights(w_outer.reshape(1, m, xe), dt),
+      s_, c_, want_logits=True)
+  assert same_record(rx, rx2)
+  torch.testing.assert_close(logits_x.reshape(b * s_, xe),
+                             xg.reshape(-1, m).float() @ w_outer.float(),
+                             rtol=1e-4, atol=1e-4)
+  used_x = H.assert_routing_properties(rx, logits_x)
+  assert not bool(rx.kept.bool().all())                 # some outer drops
+  kept_x = rx.kept.bool()
+  w_x = rx.gate.to(dt).float() * kept_x.float()
+  ein_x, slot_gate = hip.dispatch(xg, rx, want_slot_gate=True)
+  sel = kept_x & (w_x != 0)
+  gi, si, ki = sel.nonzero(as_tuple=True)
+  ref = torch.zeros_like(ein_x)
+  ref[rx.idx.long()[gi, si, ki], gi, rx.pos.long()[gi, si, ki]] = xg[gi, si]
+  assert torch.equal(ein_x, ref)
+  ref_gate = torch.zeros_like(slot_gate)
+  ref_gate[rx.idx.long()[gi, si, ki], gi, rx.pos.long()[gi, si, ki]] = w_x[gi, si, ki]
+  assert torch.equal(slot_gate, ref_gate)
+  del ref, ref_gate
+
+  # ---- inner level: importance from the slot weights (moe.py:724-727)
+  imp = 0.5 * ((slot_gate > 0.5).float() + (slot_gate > 0).float())
+  imp = imp.reshape(xe * h0, t_)
+  n_one = int((imp == 1.0).sum())
+  n_half = int((imp == 0.5).sum())
+  assert n_one + n_half + int((imp == 0).sum()) == imp.numel()
+  w1, w2 = w_x[..., 0], w_x[..., 1]
+  assert n_one == int((w1 > 0.5).sum())
+  assert n_half == int(((w1 > 0) & (w1 <= 0.5)).sum()) + int((w2 > 0).sum())
+  assert int((imp == 0).sum()) == int((~used_x).sum()) + int(
+      (kept_x & (w_x == 0)).sum())
+  inputs_y = ein_x.reshape(xe, h0 * t_, m)
+  ry2, logits_y = hip.router_top2_gating(
+      inputs_y, hip.pack_weights(w_inner, dt), t_, d_,
+      importance=slot_gate.reshape(xe * h0, t_), importance_from_slot_gate=True,
+      want_logits=True)
+  assert same_record(ry, ry2)
+  ref_logits = torch.bmm(inputs_y.float(), w_inner.float())
+  torch.testing.assert_close(logits_y.reshape(xe, h0 * t_, ye), ref_logits,
+                             rtol=1e-4, atol=1e-4)
+  H.assert_routing_properties(ry, logits_y, importance=imp)
+  assert not bool(ry.kept.bool()[imp == 1.0].all())     # some inner drops
+  ein_y = hip.dispatch(inputs_y.reshape(xe * h0, t_, m), ry)
+  kept_y = ry.kept.bool()
+  w_y = ry.gate.to(dt).float() * kept_y.float()
+  gi, si, ki = (kept_y & (w_y != 0)).nonzero(as_tuple=True)
+  ref = torch.zeros_like(ein_y)
+  ref[ry.idx.long()[gi, si, ki], gi, ry.pos.long()[gi, si, ki]] = (
+      inputs_y.reshape(xe * h0, t_, m)[gi, si])
+  assert torch.equal(ein_y, ref)
+  del ref
+
+  # ---- experts: rows of (y, x) are that pair's h0 * d slots
+  rows = h0 * d_
+  ein = ein_y.reshape(ye * xe, rows, m)
+  yy = hip.expert_ffn(ein, wi_p, wo_p, "relu")
+  for ei, r0 in ((0, 0), (ye * xe // 2, rows // 2 - 37), (ye * xe - 1, rows - 64),
+                 (37, 100)):
+    xs = ein[ei, r0:r0 + 64].float()
+    h_ref = torch.relu(xs @ wi_p[ei].float().t()).to(dt).float()
+    y_ref = h_ref @ wo_p[ei].float().t()
+    err = (yy[ei, r0:r0 + 64].float() - y_ref).abs().max().item()
+    assert err <= 2e-2 * y_ref.abs().max().item(), (ei, r0, err)
+  empty = ~(ein != 0).any(-1)
+  assert bool(empty.any()) and not bool(yy[empty].any())
+
+  # ---- the two combines, and the layer's output
+  out_y = hip.combine(yy.reshape(ye, xe * h0, d_, m), ry, t_)
+  assert torch.equal(out_y, _gather_combine(yy.reshape(ye, xe * h0, d_, m), ry, t_))
+  out_x = hip.combine(out_y.reshape(xe, b, c_, m), rx, s_)
+  assert torch.equal(out_x, _gather_combine(out_y.reshape(xe, b, c_, m), rx, s_))
+  assert torch.equal(out_x.reshape(b, l, m), out)
+  dropped = ~kept_x.any(-1)
+  assert bool(dropped.any()) and not bool(out.reshape(b, s_, m)[dropped].any())
+  # a token kept only in slots that the inner level dropped twice is zero too
+  slot_live = kept_y.any(-1).reshape(xe, b, c_)             # per outer slot
+  pos_x = rx.pos.long().clamp(max=c_ - 1)
+  gi = torch.arange(b, device="cuda").view(b, 1, 1).expand(b, s_, 2)
+  live = (kept_x & slot_live[rx.idx.long(), gi, pos_x]).any(-1)
+  assert bool((~live & ~dropped).any())
+  assert not bool(out.reshape(b, s_, m)[~live].any())
+
+  # ---- losses (moe.py:801: (outer + inner) * moe_loss_coef)
+  want_x = _float64_balancing_loss(logits_x)
+  want_y = _float64_balancing_loss(logits_y, imp == 1.0)
+  np.testing.assert_allclose(float(rx.loss), want_x, rtol=1e-4)
+  np.testing.assert_allclose(float(ry.loss), want_y, rtol=1e-4)
+  np.testing.assert_allclose(got_loss, (want_x + want_y) * 1e-2, rtol=2e-2)
 
 
 def test_v2_nonpadding():
