@@ -182,8 +182,19 @@ class HipMeshImpl(mtf.MeshImpl):
     return self.LaidOutTensor([ret])
 
   def einsum(self, equation, *slices):
-    raise NotImplementedError(
-        "generic einsum is outside the Mixture-of-Experts path")
+    """The hook the reference documents "for custom einsum implementation"
+    (mesh_tensorflow/ops.py:1331-1340; its default is tf.einsum).  Called with
+    the slices themselves, from inside a slice function.  The layers of this
+    package do not come through here: their contractions run on the library's
+    kernels; this serves Operations written against the reference interface."""
+    return torch.einsum(equation, *slices)
+
+  def laid_out_pnum(self):
+    """Processor number: one int32 scalar slice, 0
+    (mesh_tensorflow/placement_mesh_impl.py:327-329, where the
+    slices are Python ints; here a device tensor, like every other slice)."""
+    return self.LaidOutTensor(
+        [torch.zeros((), dtype=torch.int32, device=self._device)])
 
   # collectives on one processor return their input
   def allreduce(self, x, mesh_axes, reduction_fn_string):
@@ -196,6 +207,12 @@ class HipMeshImpl(mtf.MeshImpl):
     return x
 
   def receive(self, x, mesh_axis, source_pcoord):
+    """Processor i receives the slice of processor source_pcoord[i] along
+    mesh_axis, zeros where that is None
+    (mesh_tensorflow/placement_mesh_impl.py:262-289)."""
+    (source,) = source_pcoord
+    if source is None:
+      return self.slicewise(torch.zeros_like, x)
     return x
 
   def import_tf_tensor(self, x, tf_x):

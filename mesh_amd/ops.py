@@ -477,6 +477,81 @@ class MeshImpl(object):
   def einsum(self, equation, *slices):
     raise NotImplementedError("einsum not implemented")
 
+  def slicewise_delay_allreduce(self, fn, *inputs):
+    """slicewise that stays lazy when every input is a pending all-reduce sum
+    (mesh_tensorflow/ops.py:1032-1051).  No operation of this package produces
+    a pending sum (one device: nothing to reduce), so it always evaluates."""
+    return self.slicewise(fn, *inputs)
+
+  def Print(self, x, data, message, **kwargs):  # pylint: disable=invalid-name
+    """The reference's default passes x through with a warning
+    (mesh_tensorflow/ops.py:1053-1067); so does this."""
+    del data, message, kwargs
+    return x
+
+  def allsplit(self, x, mesh_axis, split_axis, which=None):
+    """Inverse of allconcat: every processor keeps the piece of its slice that
+    its coordinate along mesh_axis (or `which`) names
+    (mesh_tensorflow/ops.py:1082-1109)."""
+    if which is None:
+      which = self.laid_out_pcoord(mesh_axis)
+    num_splits = self.shape[mesh_axis].size
+
+    def keep_piece(t, w):
+      piece = t.shape[split_axis] // num_splits
+      return t.narrow(split_axis, int(w) * piece, piece)
+    return self.slicewise(keep_piece, x, which)
+
+  def shift_by_n_processors(self, x, mesh_axis, offset, wrap):
+    """Every processor receives the slice of the one `offset` places before it
+    along mesh_axis (mesh_tensorflow/ops.py:1162-1184)."""
+    n = self.shape[mesh_axis].size
+    source = []
+    for i in range(n):
+      c = i - offset
+      if not 0 <= c < n:
+        c = c % n if wrap else None
+      source.append(c)
+    return self.receive(x, mesh_axis, source)
+
+  def laid_out_pnum(self):
+    raise NotImplementedError("laid_out_pnum not implemented")
+
+  def laid_out_pcoord(self, mesh_axis):
+    """Integer scalar slices holding each processor's coordinate along
+    mesh_axis (mesh_tensorflow/ops.py:1195-1210)."""
+    divisor = list_product(self.shape.to_integer_list[mesh_axis + 1:])
+    modulus = self.shape[mesh_axis].size
+    return self.slicewise(lambda pnum: (pnum // divisor) % modulus,
+                          self.laid_out_pnum())
+
+  def laid_out_slice_num(self, tensor_shape):
+    """Integer scalar slices that are equal exactly where the slices of a
+    tensor of this shape are equal (mesh_tensorflow/ops.py:1212-1230)."""
+    ret = self.slicewise(lambda pnum: pnum * 0, self.laid_out_pnum())
+    for mesh_axis in self.tensor_layout(tensor_shape).tensor_axis_to_mesh_axis:
+      if mesh_axis is not None:
+        size = self.shape[mesh_axis].size
+        ret = self.slicewise(lambda x, pcoord, n=size: x * n + pcoord, ret,
+                             self.laid_out_pcoord(mesh_axis))
+    return ret
+
+  def broadcast_impl(self, old_slices, old_shape, new_shape):
+    """Slices of old_shape -> slices of new_shape, a superset of its dimensions
+    in any order (mesh_tensorflow/ops.py:1232-1247)."""
+    new_slice_shape = self.slice_shape(new_shape)
+    old_names = [d.name for d in old_shape.dims]
+    order = [old_names.index(d.name) for d in new_shape.dims
+             if d.name in old_names]
+    view = [-1 if d.name in old_names else 1 for d in new_shape.dims]
+
+    def expand(t):
+      t = t.permute(order) if order else t
+      sizes = iter(t.shape)
+      return t.reshape([next(sizes) if v < 0 else 1 for v in view]).expand(
+          new_slice_shape).contiguous()
+    return self.slicewise(expand, old_slices)
+
   def allreduce(self, x, mesh_axes, reduction_fn_string):
     raise NotImplementedError("Allreduce not implemented")
 

@@ -178,6 +178,7 @@ def layer_stack(x, layers, final_scale, act_dtype="float32",
     attention: wq, wk, wv, wo, num_heads
     dense_relu_dense: wi, wo
     moe: w_gate, wi, wo, hparams (an O.HParams); optional num_microbatches
+    moe2d: w_outer, w_inner, wi, wo, hparams; optional num_microbatches
   Returns (y, losses) with one loss per MoE layer.
   """
   x = _r(x, act_dtype)
@@ -199,6 +200,13 @@ def layer_stack(x, layers, final_scale, act_dtype="float32",
           h, layer["w_gate"], layer["wi"], layer["wo"], layer["hparams"],
           train, act_dtype, num_microbatches=layer.get("num_microbatches"),
           dense=False)
+      losses.append(loss)
+    elif kind == "moe2d":
+      # MoE2D.call -> transformer_moe_layer_v2 (transformer/moe.py:163-188)
+      y, loss, _ = O.moe_layer_v2(
+          h, layer["w_outer"], layer["w_inner"], layer["wi"], layer["wo"],
+          layer["hparams"], train, act_dtype,
+          num_microbatches=layer.get("num_microbatches"), dense=False)
       losses.append(loss)
     else:
       raise ValueError("layer kind %r" % (kind,))

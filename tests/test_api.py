@@ -302,12 +302,20 @@ def test_shape_and_layout_helpers():
 def test_mesh_impl_interface():
   """The plugin methods an Operation's lower() may call
   (mesh_tensorflow/ops.py:867-1340) exist on HipMeshImpl."""
-  for name in ("slicewise", "einsum", "allreduce", "allconcat", "alltoall",
-               "receive", "import_tf_tensor", "export_to_tf_tensor",
-               "slice_shape", "slice_begin", "slice_size", "laid_out_size",
-               "tensor_layout", "tensor_dimension_to_mesh_axis", "make_slices",
+  for name in ("slicewise", "slicewise_delay_allreduce", "Print", "einsum",
+               "allreduce", "allsplit", "allconcat", "alltoall", "receive",
+               "shift_by_n_processors", "laid_out_pnum", "laid_out_pcoord",
+               "laid_out_slice_num", "broadcast_impl", "import_tf_tensor",
+               "export_to_tf_tensor", "slice_shape", "slice_begin",
+               "slice_size", "laid_out_size", "tensor_layout",
+               "tensor_dimension_to_mesh_axis", "make_slices",
                "combine_slices", "random"):
     assert callable(getattr(mtf.HipMeshImpl, name)), name
+  # what HipMeshImpl must supply itself rather than inherit as a stub
+  for name in ("slicewise", "einsum", "allreduce", "allconcat", "alltoall",
+               "receive", "laid_out_pnum", "import_tf_tensor",
+               "export_to_tf_tensor", "random"):
+    assert name in vars(mtf.HipMeshImpl), name
   for name in ("shape", "ndims", "size", "layout_rules", "devices",
                "supports_control_dependencies"):
     assert isinstance(getattr(mtf.HipMeshImpl, name), property), name

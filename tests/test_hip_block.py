@@ -214,6 +214,67 @@ def test_layer_stack_float32(autoregressive):
   np.testing.assert_allclose(got_loss, want_loss, rtol=1e-4)
 
 
+@pytest.mark.parametrize("train", [False, True])
+def test_layer_stack_with_moe2d(train):
+  """MoE2D.call (transformer/moe.py:163-188) inside a LayerStack: the
+  hierarchical layer behind rms_norm and the residual, followed by a
+  DenseReluDense, against the oracle's transformer_moe_layer_v2; the capacity
+  factor differs between train and eval mode, so both modes are run."""
+  b, l, m, hdim, xe, ye, group = 2, 96, 32, 48, 3, 4, 48
+  rng = np.random.default_rng(27)
+  n = lambda *shape: H.normal_weights(rng, shape, shape[-2])
+  scale = lambda: (1 + 0.1 * rng.standard_normal(m)).astype(np.float32)
+  kw = dict(expert_x=xe, expert_y=ye, hidden_size=hdim, group_size=group,
+            capacity_factor_train=1.25, capacity_factor_eval=2.0,
+            capacity_factor_second_level=1.5, second_policy_train="all",
+            second_policy_eval="all")
+  ohp = O.default_hparams(
+      moe_num_experts=[xe, ye], moe_hidden_size=hdim, moe_group_size=group,
+      moe_capacity_factor_train=1.25, moe_capacity_factor_eval=2.0,
+      moe_capacity_factor_second_level=1.5, moe_second_policy_train="all",
+      moe_second_policy_eval="all", moe_min_expert_capacity=4)
+  layers = [dict(kind="moe2d", w_outer=n(m, xe), w_inner=n(xe, m, ye),
+                 wi=n(ye, xe, m, hdim), wo=n(ye, xe, hdim, m), hparams=ohp,
+                 scale=scale()),
+            dict(kind="dense_relu_dense", wi=n(m, hdim), wo=n(hdim, m),
+                 scale=scale())]
+  final = scale()
+  x = rng.standard_normal((b, l, m)).astype(np.float32)
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  dims = [mtf.Dimension("batch", b), mtf.Dimension("length", l),
+          mtf.Dimension("d_model", m)]
+  xt = mtf.import_tf_tensor(mesh, torch.from_numpy(x), mtf.Shape(dims))
+  stack = transformer.make_layer_stack(
+      [(moe.MoE2D, kw), (transformer_layers.DenseReluDense,
+                         dict(hidden_size=hdim, dropout_rate=0.0))],
+      num_layers=1, block_scope=False)
+  model = transformer.Unitransformer(stack, d_model=m, name="decoder",
+                                     autoregressive=False)
+  y, losses = model.call_layers(
+      xt, mtf.VariableDType(torch.float32, torch.float32, torch.float32),
+      mode="train" if train else "eval")
+  p0, p1 = "decoder/layer_000/", "decoder/layer_001/"
+  init = {"decoder/rms_norm/scale": final,
+          p0 + "rms_norm/scale": layers[0]["scale"],
+          p0 + "MoE2D/outer_gating/kernel": layers[0]["w_outer"],
+          p0 + "MoE2D/inner_gating/kernel": layers[0]["w_inner"],
+          p0 + "MoE2D/wi/kernel": layers[0]["wi"],
+          p0 + "MoE2D/wo/kernel": layers[0]["wo"],
+          p1 + "rms_norm/scale": layers[1]["scale"],
+          p1 + "DenseReluDense/wi/kernel": layers[1]["wi"],
+          p1 + "DenseReluDense/wo/kernel": layers[1]["wo"]}
+  assert sorted(init) == sorted(v.name for v in graph.all_variables)
+  lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()}, initial_values=init)
+  got = H.to_np(lowering.export_to_tf_tensor(y))
+  got_loss = [float(H.to_np(lowering.export_to_tf_tensor(t))) for t in losses]
+  want, want_loss = B.layer_stack(x, layers, final, "float32", False,
+                                  train=train)
+  assert len(got_loss) == 1
+  np.testing.assert_allclose(got, want, rtol=2e-4, atol=2e-4)
+  np.testing.assert_allclose(got_loss, want_loss, rtol=1e-4)
+
+
 def test_layer_stack_bfloat16():
   """In bfloat16 the tokens that reach the router differ by a bf16 ulp here and
   there between the two implementations (different float32 summation orders

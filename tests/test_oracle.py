@@ -297,6 +297,48 @@ def test_balanced_routing_loss_is_one():
   np.testing.assert_allclose(a, e / 4, rtol=1e-5)
 
 
+def test_second_place_loss_forward_value():
+  """moe_use_second_place_loss (transformer/moe.py:1426-1438): a case worked by
+  hand, then random logits against a float64 computation written from the
+  formulas, with importance and microbatches.
+
+  Hand case, one group, S = 2, E = 3: token 0 has probabilities (.5, .3, .2) ->
+  first choice 0, second 1, renormalised remainder (0, .6, .4); token 1 has
+  (.2, .2, .6) -> first 2, second 0 (lowest index of the tie), remainder
+  (.5, .5, 0).  density_1 = (.5, 0, .5), proxy_1 = (.35, .25, .4): loss_1 =
+  (.175 + 0 + .2) / 3 * 9 = 1.125.  density_2 = (.5, .5, 0), proxy_2 =
+  (.25, .55, .2): loss_2 = (.125 + .275 + 0) / 3 * 9 = 1.2.  Total 1.125 +
+  0.5 * 1.2 = 1.725."""
+  p = np.array([[[0.5, 0.3, 0.2], [0.2, 0.2, 0.6]]])
+  logits = np.log(p).astype(np.float32)
+  r = O.top_2_gating(logits, 4, use_second_place_loss=True)
+  assert r["index_1"].tolist() == [[0, 2]] and r["index_2"].tolist() == [[1, 0]]
+  np.testing.assert_allclose(r["loss"], 1.725, rtol=1e-6)
+  np.testing.assert_allclose(O.top_2_gating(logits, 4)["loss"], 1.125, rtol=1e-6)
+  # the policy comes after the loss: it does not change it (moe.py:1444-1467)
+  r = O.top_2_gating(logits, 4, use_second_place_loss=True, policy="none")
+  np.testing.assert_allclose(r["loss"], 1.725, rtol=1e-6)
+
+  rng = np.random.default_rng(77)
+  g, s, e, mb = 3, 40, 6, 4
+  logits = rng.standard_normal((g, s, e)).astype(np.float32) * 1.5
+  imp = rng.choice(np.array([0.0, 0.5, 1.0], np.float32), size=(g, s))
+  got = O.top_2_gating(logits, 5, importance=imp, use_second_place_loss=True,
+                       num_microbatches=mb)
+  pr = scipy.special.softmax(logits.astype(np.float64), axis=-1)
+  one = (imp == 1.0)[..., None]
+  eye = np.eye(e)
+  mask_1 = eye[pr.argmax(-1)] * one
+  q = pr * (1.0 - mask_1)
+  mask_2 = eye[q.argmax(-1)] * (imp > 0)[..., None]
+  loss_1 = ((pr * one).mean(1) * mask_1.mean(1)).mean() * e * e
+  norm = q / (q.sum(-1, keepdims=True) + 1e-9)
+  loss_2 = (norm.mean(1) * mask_2.mean(1)).mean() * e * e
+  np.testing.assert_allclose(got["loss"], (loss_1 + 0.5 * loss_2) / mb,
+                             rtol=2e-6)
+  assert loss_2 > 0.1 * loss_1              # the second term is not negligible
+
+
 # ---- switch (top-1) gating ------------------------------------------------------
 @pytest.mark.parametrize("seed", range(4))
 def test_switch_against_sequential_loop_and_float64(seed):
@@ -1313,6 +1355,17 @@ def test_v2_backward_against_central_differences():
                               0.5, mb)
     return (out * d_out.reshape(out.shape)).sum() + d_loss * loss
   base = [a.astype(np.float64) for a in (x, w_outer, w_inner, wi, wo)]
+  # the forward restatement itself (more than one outer expert) against the
+  # independent float64 forward: output per token and the loss
+  fwd_out, fwd_loss, _ = O.moe_layer_v2(x, w_outer, w_inner, wi, wo, hp, True,
+                                        "float32", nonpadding=nonpad,
+                                        num_microbatches=mb)
+  ref_out, ref_loss = _f64_layer_v2(base[0].reshape(ag, s, m), *base[1:], aux,
+                                    m1, 0.5, mb)
+  assert np.abs(ref_out).max() > 0.1
+  np.testing.assert_allclose(fwd_out.reshape(ref_out.shape), ref_out,
+                             rtol=1e-5, atol=1e-5)
+  np.testing.assert_allclose(fwd_loss, ref_loss, rtol=1e-5)
   grads = [got["dx"], got["dw_outer"], got["dw_inner"], got["dwi"], got["dwo"]]
   eps = 1e-6
   for which in range(5):
