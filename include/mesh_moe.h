@@ -686,7 +686,8 @@ size_t mesh_moe_self_attention_workspace_bytes(int B, int L, int H, int D,
  * transformer_layers.py:289-296 via attention.py:830-842), float32 softmax,
  * weights cast to dtype, outputs = weights . v.
  *   q, k, v, out [B,L,H*D] dtype (heads and d_kv combined as the reference's
- *   combine_dims does); bf16 needs L and D multiples of 8.
+ *   combine_dims does); any L and D (bf16 shapes whose L or D is not a
+ *   multiple of 8 run their two products on a plain tile kernel).
  * bf16 with D = 64 or 128 runs one fused kernel (logits stay on chip, the
  * division by the softmax sum comes after the weights are rounded; workspace =
  * a transposed copy of v).  Other cases run the three-step form whose logits

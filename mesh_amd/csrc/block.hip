@@ -685,10 +685,6 @@ extern "C" int mesh_moe_attention_weights(const void* q, const void* k,
   MOE_REQUIRE((int64_t)B * H <= 65535, MESH_MOE_E_UNSUPPORTED,
               "attention_weights: batch * heads = %lld > 65535",
               (long long)B * H);
-  MOE_REQUIRE(dtype == MESH_MOE_F32 || (L % 8 == 0 && D % 8 == 0),
-              MESH_MOE_E_UNSUPPORTED,
-              "attention_weights: bfloat16 needs length and d_kv multiples of "
-              "8 (L=%d D=%d)", L, D);
   MOE_REQUIRE(workspace_bytes >=
                   mesh_moe_attention_weights_workspace_bytes(B, L, H, D, dtype),
               MESH_MOE_E_ARG, "attention_weights: workspace too small");
@@ -758,10 +754,6 @@ extern "C" int mesh_moe_self_attention(const void* q, const void* k,
   MOE_REQUIRE((int64_t)B * H <= 65535, MESH_MOE_E_UNSUPPORTED,
               "self_attention: batch * heads = %lld > 65535",
               (long long)B * H);
-  MOE_REQUIRE(dtype == MESH_MOE_F32 || (L % 8 == 0 && D % 8 == 0),
-              MESH_MOE_E_UNSUPPORTED,
-              "self_attention: bfloat16 needs length and d_kv multiples of 8 "
-              "(L=%d D=%d)", L, D);
   MOE_REQUIRE(workspace_bytes >=
                   mesh_moe_self_attention_workspace_bytes(B, L, H, D, dtype),
               MESH_MOE_E_ARG, "self_attention: workspace too small");

@@ -927,9 +927,9 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
 // 64 x 64 tile, 16-deep K step, each thread a 4 x 4 patch, float32 accumulate
 // in k order.
 // ---------------------------------------------------------------------------
-template <typename T, bool RELU>
+template <typename T, bool RELU, typename TO = T>
 __global__ __launch_bounds__(256) void grouped_gemm_simple_kernel(
-    const T* __restrict__ A, const T* __restrict__ B, T* __restrict__ Cout,
+    const T* __restrict__ A, const T* __restrict__ B, TO* __restrict__ Cout,
     int R, int N, int K, int tiles_m, int tiles_n) {
   __shared__ float As[16][64 + 4];
   __shared__ float Bs[16][64 + 4];
@@ -940,7 +940,7 @@ __global__ __launch_bounds__(256) void grouped_gemm_simple_kernel(
   const int row0 = tm * 64, col0 = tn * 64;
   const T* Ae = A + (int64_t)e * R * K;
   const T* Be = B + (int64_t)e * N * K;
-  T* Ce = Cout + (int64_t)e * R * N;
+  TO* Ce = Cout + (int64_t)e * R * N;
   const int tid = threadIdx.x;
   const int tx = tid & 15, ty = tid >> 4;
   float acc[4][4];
@@ -979,9 +979,9 @@ __global__ __launch_bounds__(256) void grouped_gemm_simple_kernel(
     for (int j = 0; j < 4; ++j) {
       int col = col0 + tx * 4 + j;
       if (row < R && col < N) {
-        float v = round_to<T>(acc[i][j]);
+        float v = round_to<TO>(acc[i][j]);
         if (RELU) v = v > 0.f ? v : 0.f;
-        store_f32<T>(Ce + (int64_t)row * N + col, v);
+        store_f32<TO>(Ce + (int64_t)row * N + col, v);
       }
     }
   }
@@ -1327,11 +1327,20 @@ int batched_gemm_nt(const void* A, const void* B, void* C, int E, int R, int N,
                     int K, int dtype, bool out_f32, hipStream_t st) {
   if (dtype == MESH_MOE_F32 || !out_f32)
     return grouped_gemm(A, B, C, E, R, N, K, MESH_MOE_ACT_LINEAR, dtype, st);
-  MOE_REQUIRE(K % 8 == 0 && N % 8 == 0 &&
-                  (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) % 16 == 0),
-              MESH_MOE_E_UNSUPPORTED,
-              "batched_gemm_nt: float32 result needs K and N multiples of 8 "
-              "(K=%d N=%d) and 16-byte aligned operands", K, N);
+  if (!(K % 8 == 0 && N % 8 == 0 &&
+        (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) % 16 == 0))) {
+    // shapes the matrix-core kernel does not take (e.g. a key / value size
+    // that is not a multiple of 8): the plain tile kernel, bf16 in, float32 out
+    const int tiles_m = (R + 63) / 64, tiles_n = (N + 63) / 64;
+    const int64_t blocks = (int64_t)tiles_m * tiles_n * E;
+    MOE_REQUIRE(blocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
+                "batched_gemm_nt: too many tiles (%lld)", (long long)blocks);
+    grouped_gemm_simple_kernel<bf16_t, false, float>
+        <<<(unsigned)blocks, 256, 0, st>>>((const bf16_t*)A, (const bf16_t*)B,
+                                           (float*)C, R, N, K, tiles_m, tiles_n);
+    MOE_CHECK_LAUNCH("batched_gemm_nt (fma, float32 result)");
+    return 0;
+  }
   using Cfg = GemmCfg<128, 128, 64>;
   const int tiles_m = (R + 127) / 128, tiles_n = (N + 127) / 128;
   const int64_t blocks = (int64_t)tiles_m * tiles_n * E;

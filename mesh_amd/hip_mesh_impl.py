@@ -121,20 +121,29 @@ class HipMeshImpl(mtf.MeshImpl):
     def slice_shape(self):
       return list(self._slice.shape)
 
+    # Every update below writes into the storage that already exists: a step
+    # recorded into a HIP graph (Lowering.capture) holds the device addresses
+    # of the slice and of its derived copies, and must see the new values.
+
     def copy_master_to_slices(self):
       v = self._variable
-      self._slice = (self._master if v.slice_dtype == v.master_dtype
-                     else self._master.to(v.slice_dtype))
-      self._derived = {}
+      if v.slice_dtype == v.master_dtype:
+        self._slice = self._master
+      elif self._slice is None:
+        self._slice = self._master.to(v.slice_dtype)
+      else:
+        self._slice.copy_(self._master)
+      self._refresh_derived()
 
     def copy_slices_to_master(self):
-      self._master = self._slice.to(self._variable.master_dtype)
+      if self._master is not self._slice:
+        self._master.copy_(self._slice)
 
     def assign_to_slices(self, assign_fn, values, assign_to_tensor_list=None):
       del assign_fn, assign_to_tensor_list
       (value,) = values
-      self._slice = value.to(self._variable.slice_dtype).contiguous()
-      self._derived = {}
+      self._slice.copy_(value)
+      self._refresh_derived()
 
     def assign(self, value):
       """Sets master and slice from an array / tensor (replaces TF
@@ -144,9 +153,18 @@ class HipMeshImpl(mtf.MeshImpl):
       if list(value.shape) != v.shape.to_integer_list:
         raise ValueError("value for %s has shape %s, want %s"
                          % (v.name, list(value.shape), v.shape.to_integer_list))
-      self._master = value.to(device=self._mesh_impl.device,
-                              dtype=v.master_dtype).contiguous()
+      self._master.copy_(value)
       self.copy_master_to_slices()
+
+    def _refresh_derived(self):
+      """Recomputes the derived copies of the slice in place."""
+      for (kind, dtype), t in self._derived.items():
+        if kind == "act":
+          t.copy_(self._slice)
+        else:
+          s = self._slice
+          moe_hip.pack_weights(s.reshape(-1, s.shape[-2], s.shape[-1]), dtype,
+                               out=t)
 
     def activation_tensor(self):
       """Slice cast to the activation dtype (Variable.lower,

@@ -612,11 +612,14 @@ def dispatch(x, r, want_slot_gate=False, out=None):
   return (out, slot_gate) if want_slot_gate else out
 
 
-def pack_weights(w, dtype):
-  """w [E, K, N] (any supported dtype) -> packed [E, N, K] of `dtype`."""
+def pack_weights(w, dtype, out=None):
+  """w [E, K, N] (any supported dtype) -> packed [E, N, K] of `dtype`, into
+  `out` if given."""
   lib = load_library()
   e, k, n = w.shape
-  out = torch.empty((e, n, k), dtype=dtype, device=w.device)
+  if out is None:
+    out = torch.empty((e, n, k), dtype=dtype, device=w.device)
+  _dev(out, "packed", dtype, (e, n, k))
   _check(lib.mesh_moe_pack_weights(
       _dev(w, "w"), out.data_ptr(), e, k, n, dtype_code(w.dtype),
       dtype_code(dtype), _stream()), "pack_weights")

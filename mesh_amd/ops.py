@@ -637,9 +637,11 @@ class Lowering(object):
     Every imported tensor gets a static device buffer that the recorded
     kernels read; `replay` copies new values into those buffers first.  The
     outputs live in the graph's memory pool: `export_to_tf_tensor` returns the
-    tensors the last replay wrote.  Variables are read in place, so an
-    assignment between replays is seen.  The library allocates nothing and
-    uses no memset nodes, which is what makes its launches capturable.
+    tensors the last replay wrote.  Variables are read in place and
+    LaidOutVariable updates its master, slice and packed copies in place
+    (assign, assign_to_slices, copy_master_to_slices, a checkpoint restore),
+    so an assignment between replays is seen.  The library allocates nothing
+    and uses no memset nodes, which is what makes its launches capturable.
     """
     statics = {}
     for op in self.graph.operations:
@@ -654,7 +656,7 @@ class Lowering(object):
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
       self.run(statics)
-    return CapturedStep(graph, statics)
+    return CapturedStep(graph, statics, self, dict(self.tensors))
 
   def mesh_impl(self, m):
     if not isinstance(m, Mesh):
@@ -707,9 +709,11 @@ class Lowering(object):
 class CapturedStep(object):
   """A recorded step of a Lowering (Lowering.capture)."""
 
-  def __init__(self, graph, statics):
+  def __init__(self, graph, statics, lowering, recorded_tensors):
     self._graph = graph
     self._statics = statics
+    self._lowering = lowering
+    self._recorded = recorded_tensors
 
   def replay(self, feeds=None):
     """feeds: {imported Tensor: torch tensor of the same shape}; tensors not
@@ -720,6 +724,9 @@ class CapturedStep(object):
                          % (tensor,))
       self._statics[tensor].copy_(torch.as_tensor(value))
     self._graph.replay()
+    # an eager run() since the capture has rebound the lowering's tensors to
+    # its own results: point them back at what the recorded kernels write
+    self._lowering.tensors.update(self._recorded)
 
 
 # ----------------------------------------------------------------------------

@@ -353,6 +353,16 @@ def _packed(lowering, kernel_tensor, dtype):
   return lowering.variables[kernel_tensor.operation].packed(dtype)
 
 
+def _release_saved(saved):
+  """Called by a gradient operation when it has run: the activations the
+  forward operation kept for it (several GiB at the largest benchmark layer)
+  are dropped once the last gradient operation built on that forward
+  operation has consumed them, instead of living until the next step."""
+  saved["_consumers"] = saved.get("_consumers", 1) - 1
+  if saved["_consumers"] <= 0:
+    saved.clear()
+
+
 class MoEV1Operation(mtf.Operation):
   """The whole of transformer_moe_layer_v1 after the reshape to groups:
   inputs [outer_batch, groups, group, d_model] -> (outputs with d_model
@@ -407,6 +417,7 @@ class MoEV1Operation(mtf.Operation):
     from those of (outputs, loss[, second outputs]); importance carries
     none."""
     self._save_for_backward = True
+    self._num_grad_ops = getattr(self, "_num_grad_ops", 0) + 1
     d_out, d_loss = grad_ys[:2]
     if d_out is None:
       d_out = mtf.zeros(self.mesh, self.outputs[0].shape, self.outputs[0].dtype)
@@ -519,6 +530,8 @@ class MoEV1Operation(mtf.Operation):
     outs = mesh_impl.slicewise(fn, *args)
     for t, v in zip(self.outputs, outs):
       lowering.set_tensor_lowering(t, v)
+    if saved:
+      saved["_consumers"] = getattr(self, "_num_grad_ops", 0)
     lowering.operations[self] = saved
 
 
@@ -684,6 +697,7 @@ class MoEV1GradOperation(mtf.Operation):
     args = [lowering.tensors[ins[i]] for i in (2, 3, 4, 5)]
     args += [lowering.tensors[t] for t in ins[6:]]
     outs = mesh_impl.slicewise(fn, *args)
+    _release_saved(lowering.operations[fwd])
     for t, v in zip(self.outputs, outs):
       lowering.set_tensor_lowering(t, v)
 
@@ -839,6 +853,7 @@ class MoEV2Operation(mtf.Operation):
     """Gradients w.r.t. (inputs, outer / inner gate kernels, wi, wo
     [, importance]) from those of (outputs, loss)."""
     self._save_for_backward = True
+    self._num_grad_ops = getattr(self, "_num_grad_ops", 0) + 1
     d_out, d_loss = grad_ys
     if d_out is None:
       d_out = mtf.zeros(self.mesh, self.outputs[0].shape, self.outputs[0].dtype)
@@ -908,6 +923,8 @@ class MoEV2Operation(mtf.Operation):
     out, loss = mesh_impl.slicewise(fn, *args)
     lowering.set_tensor_lowering(self.outputs[0], out)
     lowering.set_tensor_lowering(self.outputs[1], loss)
+    if saved:
+      saved["_consumers"] = getattr(self, "_num_grad_ops", 0)
     lowering.operations[self] = saved
 
 
@@ -989,6 +1006,7 @@ class MoEV2GradOperation(mtf.Operation):
                                lowering.tensors[ins[4]],
                                lowering.tensors[ins[5]],
                                lowering.tensors[ins[6]])
+    _release_saved(lowering.operations[fwd])
     for t, v in zip(self.outputs, outs):
       lowering.set_tensor_lowering(t, v)
 

@@ -1205,3 +1205,20 @@ def test_captured_step_replays_match_eager(act_dtype):
   # a replay without feeds repeats the last tokens
   step.replay()
   assert torch.equal(lowering.export_to_tf_tensor(y), eager)
+  # new weights between two replays (an optimizer step, a checkpoint restore):
+  # the variable's slice and its packed copies are updated in place, so the
+  # recorded kernels read the new values
+  var = {v.name: lv for v, lv in lowering.variables.items()}
+  for trial in range(2):
+    var["moe/wi/kernel"].assign(H.normal_weights(rng, (e, m, hdim), m))
+    var["moe/top_2_gating/kernel"].assign(H.normal_weights(rng, (m, e), m))
+    var["moe/wo/kernel"].assign_to_slices(
+        None, [torch.from_numpy(H.normal_weights(rng, (e, hdim, m), hdim)).cuda()])
+    torch.cuda.synchronize()
+    step.replay()
+    torch.cuda.synchronize()
+    replayed = lowering.export_to_tf_tensor(y).clone()
+    lowering.run({xt: xv})
+    assert torch.equal(lowering.export_to_tf_tensor(y), replayed), trial
+    assert not torch.equal(replayed, eager)
+    eager = replayed
