@@ -149,13 +149,17 @@ int mesh_moe_top2_gating_static_scratch(
     uint8_t* kept, int32_t* fill, float* loss, void* stream);
 
 /*
- * Router projection and top-2 gating in one call: what _top_2_gating does from
- * `to_float(inputs)` to the per-token assignment (transformer/moe.py:1384-1496),
- * with the logits kept in LDS between the matrix-core projection and the
- * softmax / top-2 step (they are written to `logits` [G,S,E] only if it is not
- * NULL).  Arguments are those of mesh_moe_router_logits (packed weights only)
- * followed by those of mesh_moe_top2_gating; batch * tokens == G * S and each
- * weight set covers whole groups.
+ * Router projection and top-2 gating in one call and ONE kernel launch: what
+ * _top_2_gating does from `to_float(inputs)` to the per-token assignment
+ * (transformer/moe.py:1384-1496).  The logits stay in LDS between the
+ * matrix-core projection and the softmax / top-2 step (they are written to
+ * `logits` [G,S,E] only if it is not NULL); every block ranks the choices of
+ * its 128 tokens with wavefront ballots and publishes per-expert counts, and
+ * the block of a group that finishes last turns them into capacity positions,
+ * `fill` and the group's loss term (no block waits for another).  Arguments
+ * are those of mesh_moe_router_logits (packed weights only) followed by those
+ * of mesh_moe_top2_gating; batch * tokens == G * S and each weight set covers
+ * whole groups.  The workspace may hold anything on entry.
  * Returns MESH_MOE_E_UNSUPPORTED (nothing launched) unless dtype is bf16,
  * M % 64 == 0, E % 4 == 0, E <= 128 and S % 128 == 0; callers then use the two
  * separate entry points.

@@ -5,6 +5,7 @@
 // float32 operation order of mtf.softmax (ops.py:5493-5541) and mtf.top_1
 // (ops.py:4937-4940).  The dense [G,S,E] masks and the S x S cumsum matmul
 // (ops.py:2761-2781) are replaced by a per-token record and integer counting.
+#include <atomic>
 #include <mutex>
 
 #include "common.h"
@@ -225,6 +226,37 @@ __global__ __launch_bounds__(256) void router_mfma_kernel(
 // Grid (blocks per group, G); one thread per token; the logits tile is staged
 // in LDS with row stride E+1 so that per-thread row walks are conflict-free.
 // ---------------------------------------------------------------------------
+// Accesses that are coherent across the GPU's compute dies without a cache
+// flush.  Each die (XCD) has its own L2; an ordinary store may sit there, and
+// an ordinary load may hit a stale line there, until a device-scope fence
+// writes back / invalidates that whole L2 -- too expensive to issue from
+// every block of a kernel whose other blocks are still streaming through the
+// same L2.  A relaxed atomic store / load at device scope is a write-through
+// store / a load that bypasses lines the L2 cannot vouch for.  The blocks of
+// the single-launch gating kernel exchange their data only through these:
+// the writer waits until its stores have completed (vmcnt 0) before it bumps
+// the arrival counter, the reader loads after it has seen the counter.
+template <typename T>
+__device__ __forceinline__ void st_dev(T* p, T v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+template <typename T>
+__device__ __forceinline__ T ld_dev(const T* p) {
+  return __hip_atomic_load(const_cast<T*>(p), __ATOMIC_RELAXED,
+                           __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ unsigned long long pack_i2(int a, int b) {
+  return (unsigned long long)(unsigned)a | ((unsigned long long)(unsigned)b << 32);
+}
+__device__ __forceinline__ unsigned long long pack_f2(float a, float b) {
+  return pack_i2((int)__float_as_uint(a), (int)__float_as_uint(b));
+}
+// this wavefront's global stores (and loads) have completed
+__device__ __forceinline__ void wait_stores() {
+  __builtin_amdgcn_s_waitcnt(0x0f70);   // vmcnt(0), nothing else
+  asm volatile("" ::: "memory");
+}
+
 struct GateParams {
   int G, S, E, C;
   int policy;
@@ -253,13 +285,19 @@ constexpr int GSUM = 4;  // floats per group: loss term 1, term 2, #(imp==1), z
 // gate_select_tile does the work for `ntok` tokens (tokens t0 .. of group g,
 // block `blk` of the group) whose logits already sit in LDS as tile[ntok][ld];
 // every thread of the block must call it.
+//
+// With `ch` (LDS, 3 * ch_stride int16) the expert a token competes for with
+// its first / second choice, and the expert the loss's extra count sees, also
+// go there (-1 = none) for the in-block ranking of the single-launch kernel,
+// which then writes `pos` itself.
 template <typename IT>
 __device__ __forceinline__ void gate_select_tile(
     float* tile, float* isone, int ld, int ntok, int g, int blk, int t0,
     const IT* __restrict__ importance, const float* __restrict__ second_uniform,
     const GateParams& p, int32_t* __restrict__ idx, int32_t* __restrict__ pos,
     float* __restrict__ gate, uint8_t* __restrict__ kept,
-    float* __restrict__ part1, float* __restrict__ part2) {
+    float* __restrict__ part1, float* __restrict__ part2,
+    int16_t* ch = nullptr, int ch_stride = 0) {
   const int E = p.E, S = p.S;
   const int tid = threadIdx.x;
   float qscale = 0.f, zterm = 0.f;
@@ -305,8 +343,14 @@ __device__ __forceinline__ void gate_select_tile(
       if (!sel1) g1 = g1 * 0.0f;
       idx[t * 2 + 0] = i1;
       idx[t * 2 + 1] = 0;
-      pos[t * 2 + 0] = 0;
-      pos[t * 2 + 1] = 0;
+      if (ch == nullptr) {
+        pos[t * 2 + 0] = 0;
+        pos[t * 2 + 1] = 0;
+      } else {
+        ch[tid] = sel1 ? (int16_t)i1 : (int16_t)-1;
+        ch[ch_stride + tid] = -1;
+        ch[2 * ch_stride + tid] = (int16_t)i1;
+      }
       gate[t * 2 + 0] = g1;
       gate[t * 2 + 1] = 0.0f;
       kept[t * 2 + 0] = (sel1 ? 1 : 0) | 2;   // bit 1: counted by density_1
@@ -346,8 +390,14 @@ __device__ __forceinline__ void gate_select_tile(
     }
     idx[t * 2 + 0] = i1;
     idx[t * 2 + 1] = i2;
-    pos[t * 2 + 0] = 0;
-    pos[t * 2 + 1] = 0;
+    if (ch == nullptr) {
+      pos[t * 2 + 0] = 0;
+      pos[t * 2 + 1] = 0;
+    } else {
+      ch[tid] = sel1 ? (int16_t)i1 : (int16_t)-1;
+      ch[ch_stride + tid] = sel2 ? (int16_t)i2 : (int16_t)-1;
+      ch[2 * ch_stride + tid] = sel2_loss ? (int16_t)i2 : (int16_t)-1;
+    }
     gate[t * 2 + 0] = g1n;
     gate[t * 2 + 1] = g2n;
     kept[t * 2 + 0] = sel1 ? 1 : 0;
@@ -395,6 +445,220 @@ __device__ __forceinline__ void gate_select_tile(
   }
 }
 
+// ---------------------------------------------------------------------------
+// gate_select_tile for a block of 256 threads and 128 tokens: two threads per
+// token (adjacent lanes), each owning half of the experts.  The exponentials,
+// two per expert and the bulk of the work, are split between the pair; every
+// float32 sum still runs in expert order (the first thread's partial sum is
+// handed to the second, which continues it), and the first-arg-max of a pair
+// prefers the lower half on ties, so every per-token result is bit for bit
+// that of gate_select_tile.  The per-block column sums for the loss are split
+// over four row ranges.  H2MAX >= E / 2 (E even) bounds the register copy of a
+// thread's logits; colpart: LDS [4][E] floats.
+// ---------------------------------------------------------------------------
+template <int H2MAX, typename IT>
+__device__ __forceinline__ void gate_select_pair_tile(
+    float* tile, float* isone, int ld, int g, int blk, int t0,
+    const IT* __restrict__ importance, const float* __restrict__ second_uniform,
+    const GateParams& p, int32_t* __restrict__ idx, int32_t* __restrict__ pos,
+    float* __restrict__ gate, uint8_t* __restrict__ kept,
+    float* __restrict__ part1, float* __restrict__ part2, int16_t* ch,
+    float* colpart) {
+  constexpr int NTOK = 128;
+  const int E = p.E, S = p.S, H2 = E >> 1;
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int tok = tid >> 1, half = tid & 1;
+  const int eb = half * H2;
+  const bool sw = p.router == ROUTER_SWITCH;
+  float* row = tile + tok * ld;
+  const int64_t t = (int64_t)g * S + t0 + tok;
+  // the other thread of the pair has the strictly better candidate?  (equal
+  // values: the lower half, i.e. the lower expert index, wins)
+  auto take_other = [&](float mine, float other) {
+    return half == 0 ? other > mine : !(mine > other);
+  };
+
+  float xr[H2MAX];
+  float m = -INFINITY;
+#pragma unroll
+  for (int j = 0; j < H2MAX; ++j)
+    if (j < H2) {
+      xr[j] = row[eb + j];
+      m = fmaxf(m, xr[j]);                                  // reduce_max
+    }
+  m = fmaxf(m, __shfl_xor(m, 1));
+  const float negm = -m;
+  float s = 0.f;
+#pragma unroll
+  for (int j = 0; j < H2MAX; ++j)
+    if (j < H2) {
+      const float u = expf(xr[j] + negm);                   // exp
+      if (half == 0) s += u;                                // reduce_sum ...
+      else row[eb + j] = u;
+    }
+  const float s_low = __shfl(s, lane & ~1);
+  if (half == 1) {
+    s = s_low;                                              // ... continued
+    for (int j = 0; j < H2; ++j) s += row[eb + j];
+  }
+  s = __shfl(s, lane | 1);
+  const float neglse = -(logf(s) + m);                      // log + max
+  float g1 = -1.f;
+  int i1 = 0;
+#pragma unroll
+  for (int j = 0; j < H2MAX; ++j)
+    if (j < H2) {
+      const float pe = expf(xr[j] + neglse);                // exp(log_softmax)
+      row[eb + j] = pe;
+      if (pe > g1) { g1 = pe; i1 = eb + j; }                // first argmax
+    }
+  {
+    const float og = __shfl_xor(g1, 1);
+    const int oi = __shfl_xor(i1, 1);
+    if (take_other(g1, og)) { g1 = og; i1 = oi; }
+  }
+  bool sel1 = true;
+  if (sw && second_uniform != nullptr) {
+    // policy "sample": first arg-max of the caller's choice logits
+    const float* cl = second_uniform + t * E;
+    float best = -INFINITY;
+    int bi = eb;
+    for (int j = 0; j < H2; ++j) {
+      const float v = cl[eb + j];
+      if (j == 0 || v > best) { best = v; bi = eb + j; }
+    }
+    const float ob = __shfl_xor(best, 1);
+    const int oi = __shfl_xor(bi, 1);
+    if (take_other(best, ob)) bi = oi;
+    i1 = bi;
+    __syncthreads();           // the partner's half of the row is in LDS
+    g1 = row[i1];
+  }
+  float qscale = 0.f, zterm = 0.f;
+  if (sw) {
+    if (importance != nullptr)
+      sel1 = (load_f32<IT>(importance + t) == 1.0f);
+    if (!sel1) g1 = g1 * 0.0f;
+    if (half == 0) {
+      st_dev(reinterpret_cast<unsigned long long*>(idx + t * 2), pack_i2(i1, 0));
+      st_dev(reinterpret_cast<unsigned long long*>(gate + t * 2),
+             pack_f2(g1, 0.0f));
+    } else {
+      st_dev(reinterpret_cast<uint16_t*>(kept + t * 2),
+             (uint16_t)((sel1 ? 1 : 0) | 2));
+      if (ch == nullptr) {
+        *reinterpret_cast<int2*>(pos + t * 2) = make_int2(0, 0);
+      } else {
+        ch[tok] = sel1 ? (int16_t)i1 : (int16_t)-1;
+        ch[NTOK + tok] = -1;
+        ch[2 * NTOK + tok] = (int16_t)i1;
+      }
+      isone[tok] = 1.0f;
+    }
+    const float lse = -neglse;
+    zterm = sel1 ? lse * lse : 0.0f;
+  } else {
+    bool sel2 = true;
+    if (importance != nullptr) {
+      float imp = load_f32<IT>(importance + t);
+      if (p.importance_from_slot_gate)
+        imp = 0.5f * ((imp > 0.5f ? 1.0f : 0.0f) + (imp > 0.0f ? 1.0f : 0.0f));
+      sel1 = (imp == 1.0f);
+      sel2 = (imp > 0.0f);
+    }
+    if (!sel1) g1 = g1 * 0.0f;
+    float g2 = -1.f, qsum = 0.f;
+    int i2 = 0;
+    for (int j = 0; j < H2; ++j) {
+      const int e = eb + j;
+      const float keep = (sel1 && e == i1) ? 0.0f : 1.0f;
+      const float q = row[e] * keep;
+      if (half == 0) qsum += q;
+      if (q > g2) { g2 = q; i2 = e; }
+    }
+    const float q_low = __shfl(qsum, lane & ~1);
+    if (half == 1) {
+      qsum = q_low;
+      for (int j = 0; j < H2; ++j) {
+        const int e = eb + j;
+        const float keep = (sel1 && e == i1) ? 0.0f : 1.0f;
+        qsum += row[e] * keep;
+      }
+    }
+    qsum = __shfl(qsum, lane | 1);
+    {
+      const float og = __shfl_xor(g2, 1);
+      const int oi = __shfl_xor(i2, 1);
+      if (take_other(g2, og)) { g2 = og; i2 = oi; }
+    }
+    const float denom = (g1 + g2) + 1e-9f;
+    const float r = 1.0f / denom;
+    const float g1n = g1 * r, g2n = g2 * r;
+    const bool sel2_loss = sel2;
+    if (p.policy == MESH_MOE_SECOND_NONE) {
+      sel2 = false;
+    } else if (p.policy == MESH_MOE_SECOND_THRESHOLD) {
+      sel2 = sel2 && (g2n > p.threshold);
+    } else if (p.policy == MESH_MOE_SECOND_RANDOM) {
+      sel2 = sel2 && (second_uniform[t] < g2n * p.inv_threshold);
+    }
+    if (half == 0) {
+      st_dev(reinterpret_cast<unsigned long long*>(idx + t * 2), pack_i2(i1, i2));
+      st_dev(reinterpret_cast<unsigned long long*>(gate + t * 2),
+             pack_f2(g1n, g2n));
+    } else {
+      st_dev(reinterpret_cast<uint16_t*>(kept + t * 2), (uint16_t)(
+          (sel1 ? 1 : 0) | ((sel2 ? 1 : 0) | (sel2_loss ? 2 : 0)) << 8));
+      if (ch == nullptr) {
+        *reinterpret_cast<int2*>(pos + t * 2) = make_int2(0, 0);
+      } else {
+        ch[tok] = sel1 ? (int16_t)i1 : (int16_t)-1;
+        ch[NTOK + tok] = sel2 ? (int16_t)i2 : (int16_t)-1;
+        ch[2 * NTOK + tok] = sel2_loss ? (int16_t)i2 : (int16_t)-1;
+      }
+      isone[tok] = sel1 ? 1.0f : 0.0f;
+    }
+    qscale = 1.0f / (qsum + 1e-9f);
+  }
+  __syncthreads();
+  // column sums over the block's tokens, four row ranges per column
+  auto column_sums = [&](int ncol, bool weighted, float* out) {
+    for (int i = tid; i < 4 * ncol; i += blockDim.x) {
+      const int e = i % ncol, q4 = i / ncol;
+      float acc = 0.f;
+      for (int r = q4 * (NTOK / 4); r < (q4 + 1) * (NTOK / 4); ++r)
+        acc += weighted ? tile[r * ld + e] * isone[r] : tile[r * ld + e];
+      colpart[q4 * ncol + e] = acc;
+    }
+    __syncthreads();
+    for (int e = tid; e < ncol; e += blockDim.x)
+      st_dev(out + ((int64_t)g * p.nblk + blk) * E + e,
+             ((colpart[e] + colpart[ncol + e]) + colpart[2 * ncol + e]) +
+                 colpart[3 * ncol + e]);
+  };
+  column_sums(E, true, part1);       // density_1_proxy: p * (imp == 1)
+  if (sw) {
+    // z-loss: column 0 = sum of logsumexp^2 over the tokens of importance 1,
+    // column 1 = how many those are
+    __syncthreads();
+    if (half == 0) {
+      row[0] = zterm;
+      row[1] = sel1 ? 1.0f : 0.0f;
+    }
+    __syncthreads();
+    column_sums(2, false, part2);
+  } else if (p.use_second_place_loss) {
+    __syncthreads();
+    for (int j = 0; j < H2; ++j) {
+      const int e = eb + j;
+      const float keep = (sel1 && e == i1) ? 0.0f : 1.0f;
+      row[e] = (row[e] * keep) * qscale;
+    }
+    __syncthreads();
+    column_sums(E, false, part2);
+  }
+}
+
 template <typename IT>
 __global__ __launch_bounds__(256) void gate_select_kernel(
     const float* __restrict__ logits, const IT* __restrict__ importance,
@@ -423,6 +687,280 @@ __global__ __launch_bounds__(256) void gate_select_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// Capacity positions and the loss inside the projection kernel's launch.
+//
+// Every block ranks the choices of its own 128 tokens (gate_rank_tile: per
+// expert a wavefront ballot over 64 tokens and the number of set bits below
+// the lane, then the count of the block's other half) and publishes its
+// per-expert counts.  The block of a group that arrives last at the group's
+// counter (gate_group_tail) turns the counts into each block's first slot per
+// expert, finishes every token of the group (slot = first slot of its block +
+// rank in the block; second choices behind the kept first choices), writes
+// `fill` and the group's loss term; the group that finishes last adds the
+// terms up.  Nobody waits for anybody, so the scheme does not depend on which
+// blocks are resident together.
+//
+// A counter is a 64-bit word: call number << 16 | arrivals.  A word that does
+// not carry the current call's number counts as zero, so the workspace may
+// hold anything when the call starts; the last arrival leaves zero behind.
+// ---------------------------------------------------------------------------
+struct GateParams;
+template <bool COHERENT>
+__device__ __forceinline__ void gate_loss_value(const GateParams& p,
+                                                const float* gsum, float* loss);
+
+struct FusedTail {
+  int32_t* bcnt;              // [G][nblk][3][E] per-block counts
+  unsigned long long* gctr;   // [G] arrivals per group
+  unsigned long long* fctr;   // [1] groups done
+  float* gsum;                // [G][GSUM]
+  int32_t* fill;              // [G][E]
+  float* loss;                // [1]
+  unsigned long long call;    // number of this call, < 2^48, never 0
+};
+
+// Puts a counter word into this call's state "no arrivals yet" if it holds
+// zero, which is what the last arrival of the previous use leaves behind.
+// Nobody waits for the result: a word that held something else (a workspace
+// used for the first time) is handled by the arrivals themselves.
+__device__ __forceinline__ void counter_prepare(unsigned long long* word,
+                                                unsigned long long call) {
+  unsigned long long zero = 0ull;
+  (void)__hip_atomic_compare_exchange_strong(
+      word, &zero, call << 16, __ATOMIC_RELAXED, __ATOMIC_RELAXED,
+      __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// true for the last of `expected` arrivals; one thread per arrival.  The
+// common case is one fetch-add on a word that counter_prepare stamped long
+// ago.  An arrival that finds another stamp (its add then changed a word
+// nobody relies on) installs the stamp itself or, if somebody else just did,
+// adds again: every arrival ends with exactly one successful operation on a
+// word that carries this call's stamp.
+__device__ __forceinline__ bool arrive_is_last(unsigned long long* word,
+                                               unsigned long long call,
+                                               unsigned expected) {
+  unsigned long long old = __hip_atomic_fetch_add(
+      word, 1ull, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  if ((old >> 16) == call) return (unsigned)((old + 1) & 0xffffu) == expected;
+  old = __hip_atomic_load(word, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  for (;;) {
+    if ((old >> 16) == call) {
+      old = __hip_atomic_fetch_add(word, 1ull, __ATOMIC_RELAXED,
+                                   __HIP_MEMORY_SCOPE_AGENT);
+      return (unsigned)((old + 1) & 0xffffu) == expected;
+    }
+    const unsigned long long seen = atomicCAS(word, old, (call << 16) | 1ull);
+    if (seen == old) return expected == 1u;
+    old = seen;
+  }
+}
+
+// Ranks of the block's choices.  ch [3][128] int16 in LDS as written by
+// gate_select_tile; wcnt [3][2][E] int32 in LDS.  Wavefront w ranks choice
+// w / 2 of tokens 64 (w % 2) ..; with `loss2` wavefronts 0 and 1 also count
+// the third array.  Writes pos (rank within the block) for competing choices,
+// 0 otherwise, and the block's counts to bcnt_blk [3][E].
+__device__ __forceinline__ void gate_rank_tile(
+    const int16_t* ch, int32_t* wcnt, int E, bool loss2, int64_t tok0,
+    int32_t* __restrict__ pos, int32_t* __restrict__ bcnt_blk) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int c = wave >> 1, half = wave & 1;
+  const int mine = ch[c * 128 + half * 64 + lane];
+  int rank = 0;
+  for (int e0 = 0; e0 < E; e0 += 64) {
+    int cnt = 0;   // lane l: choosers of expert e0 + l in this wavefront
+    const int n = min(64, E - e0);
+    for (int j = 0; j < n; ++j) {
+      const unsigned long long m = __ballot(mine == e0 + j);
+      if (mine == e0 + j)
+        rank = __builtin_amdgcn_mbcnt_hi(
+            (unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0u));
+      if (lane == j) cnt = __popcll(m);
+    }
+    if (lane < n) wcnt[(c * 2 + half) * E + e0 + lane] = cnt;
+  }
+  if (loss2 && c == 0) {
+    const int third = ch[2 * 128 + half * 64 + lane];
+    for (int e0 = 0; e0 < E; e0 += 64) {
+      int cnt = 0;
+      const int n = min(64, E - e0);
+      for (int j = 0; j < n; ++j) {
+        const unsigned long long m = __ballot(third == e0 + j);
+        if (lane == j) cnt = __popcll(m);
+      }
+      if (lane < n) wcnt[(4 + half) * E + e0 + lane] = cnt;
+    }
+  }
+  __syncthreads();
+  if (half == 1 && mine >= 0) rank += wcnt[(c * 2) * E + mine];
+  st_dev(pos + (tok0 + half * 64 + lane) * 2 + c, mine >= 0 ? rank : 0);
+  for (int i = tid; i < 3 * E; i += blockDim.x) {
+    const int cc = i / E, e = i - cc * E;
+    st_dev(bcnt_blk + i, (cc < 2 || loss2) ? wcnt[(cc * 2) * E + e] +
+                                                 wcnt[(cc * 2 + 1) * E + e]
+                                           : 0);
+  }
+}
+
+// What the last block of group g does (all 256 threads; smem is the block's
+// whole dynamic LDS, free by now).  Same results, bit for bit, as
+// gate_capacity_kernel + gate_loss_kernel for slots in token order.
+__device__ __forceinline__ void gate_group_tail(
+    unsigned char* smem, const GateParams& p, const FusedTail& ft, int g,
+    const int32_t* __restrict__ idx, int32_t* __restrict__ pos,
+    float* __restrict__ gate, uint8_t* __restrict__ kept,
+    const float* __restrict__ part1, const float* __restrict__ part2) {
+  const int S = p.S, E = p.E, C = p.C, nblk = p.nblk;
+  const int tid = threadIdx.x;
+  const bool sw = p.router == ROUTER_SWITCH;
+  const bool loss2 = p.use_second_place_loss != 0 || sw;
+  uint16_t* pre1 = reinterpret_cast<uint16_t*>(smem);          // [nblk][E]
+  uint16_t* pre2 = pre1 + (size_t)nblk * E;                    // [nblk][E]
+  int32_t* tot = reinterpret_cast<int32_t*>(
+      smem + (((size_t)nblk * E * 4 + 15) & ~(size_t)15));     // [3][E]
+  float* prod = reinterpret_cast<float*>(tot + 3 * E);         // [2][E]
+  float* misc = prod + 2 * E;                                  // [4]
+  const int32_t* bc = ft.bcnt + (int64_t)g * nblk * 3 * E;
+  const int64_t base = (int64_t)g * S;
+  // Everything here comes from other compute units' stores, i.e. from memory,
+  // one round trip per dependent access: the loads of the three parts (token
+  // records, partial sums of the loss, per-block counts) are issued together
+  // before anything is used.
+  constexpr int U = 8;     // tokens per thread and trip
+  constexpr int PB = 16;   // blocks whose partial sums are fetched up front
+  int2 ex[U], rk[U];
+  float2 gt[U];
+  uint16_t kk[U];
+  auto load_records = [&](int s0) {
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int s = s0 + u * (int)blockDim.x;
+      if (s < S) {
+        const int64_t t = base + s;
+        const unsigned long long e2 =
+            ld_dev(reinterpret_cast<const unsigned long long*>(idx + t * 2));
+        const unsigned long long r2 =
+            ld_dev(reinterpret_cast<const unsigned long long*>(pos + t * 2));
+        const unsigned long long g2 =
+            ld_dev(reinterpret_cast<const unsigned long long*>(gate + t * 2));
+        kk[u] = ld_dev(reinterpret_cast<const uint16_t*>(kept + t * 2));
+        ex[u] = make_int2((int)(unsigned)e2, (int)(e2 >> 32));
+        rk[u] = make_int2((int)(unsigned)r2, (int)(r2 >> 32));
+        gt[u] = make_float2(__uint_as_float((unsigned)g2),
+                            __uint_as_float((unsigned)(g2 >> 32)));
+      }
+    }
+  };
+  load_records(tid);
+  // thread e < E sums column e of part1, threads E .. 2E-1 column e of part2
+  // (second-place loss: E columns; switch: columns 0 and 1), in block order
+  const int pcol = tid < E ? tid : tid - E;
+  const bool sums1 = tid < E;
+  const bool sums2 = !sums1 && tid < 2 * E && loss2 && (!sw || pcol < 2);
+  const float* pcolumn = (sums1 ? part1 : part2) + (int64_t)g * nblk * E + pcol;
+  float pv[PB];
+  if (sums1 || sums2) {
+#pragma unroll
+    for (int b = 0; b < PB; ++b)
+      pv[b] = b < nblk ? ld_dev(pcolumn + (int64_t)b * E) : 0.f;
+  }
+  // first slot of every block per expert: exclusive prefix over the blocks
+  for (int i = tid; i < 3 * E; i += blockDim.x) {
+    const int c = i / E, e = i - c * E;
+    if (c == 2 && !loss2) { tot[i] = 0; continue; }
+    uint16_t* pre = c == 0 ? pre1 : pre2;
+    int run = 0;
+#pragma unroll 16
+    for (int b = 0; b < nblk; ++b) {
+      const int v = ld_dev(bc + ((int64_t)b * 3 + c) * E + e);
+      if (c < 2) pre[b * E + e] = (uint16_t)run;
+      run += v;
+    }
+    tot[i] = run;
+  }
+  float psum = 0.f;
+  if (sums1 || sums2) {
+#pragma unroll
+    for (int b = 0; b < PB; ++b)
+      if (b < nblk) psum += pv[b];
+    for (int b = PB; b < nblk; ++b) psum += ld_dev(pcolumn + (int64_t)b * E);
+  }
+  __syncthreads();
+  for (int s0 = tid; s0 < S; s0 += (int)blockDim.x * U) {
+    if (s0 != tid) load_records(s0);
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int s = s0 + u * (int)blockDim.x;
+      if (s >= S) continue;
+      const int blk = s >> 7;
+      uint16_t kout = 0;
+      if (kk[u] & 1) {
+        const int slot = pre1[blk * E + ex[u].x] + rk[u].x;
+        rk[u].x = slot;
+        if (slot < C) kout |= 1; else gt[u].x = gt[u].x * 0.0f;
+      } else {
+        rk[u].x = 0;
+        gt[u].x = gt[u].x * 0.0f;
+      }
+      if (kk[u] & 0x100) {
+        const int slot = min(tot[ex[u].y], C) + pre2[blk * E + ex[u].y] + rk[u].y;
+        rk[u].y = slot;
+        if (slot < C) kout |= 0x100; else gt[u].y = gt[u].y * 0.0f;
+      } else {
+        rk[u].y = 0;
+        gt[u].y = gt[u].y * 0.0f;
+      }
+      kk[u] = kout;
+    }
+#pragma unroll
+    for (int u = 0; u < U; ++u) {
+      const int s = s0 + u * (int)blockDim.x;
+      if (s < S) {
+        const int64_t t = base + s;
+        *reinterpret_cast<int2*>(pos + t * 2) = rk[u];
+        *reinterpret_cast<uint16_t*>(kept + t * 2) = kk[u];
+        *reinterpret_cast<float2*>(gate + t * 2) = gt[u];
+      }
+    }
+  }
+  // per-expert outputs and the group's share of the balancing loss
+  if (sums2) {
+    if (sw) misc[pcol] = psum;
+    else prod[E + pcol] = psum;      // proxy of the second-place loss, for now
+  }
+  __syncthreads();
+  if (tid < E) {
+    const int t1 = tot[tid], t2 = tot[E + tid];
+    const int k1 = min(t1, C);
+    ft.fill[(int64_t)g * E + tid] = k1 + min(t2, C - k1);
+    const float inv_s = (float)(1.0 / (double)S);
+    const int dens = sw ? tot[2 * E + tid] : t1;
+    prod[tid] = (psum * inv_s) * ((float)dens * inv_s);
+    if (loss2 && !sw)
+      prod[E + tid] = (prod[E + tid] * inv_s) * ((float)tot[2 * E + tid] * inv_s);
+  }
+  __syncthreads();
+  if (tid == 0) {
+    float s1 = 0.f, s2 = 0.f;
+    for (int k = 0; k < E; ++k) s1 += prod[k];
+    if (loss2 && !sw)
+      for (int k = 0; k < E; ++k) s2 += prod[E + k];
+    float* gs = ft.gsum + (int64_t)g * GSUM;
+    st_dev(gs + 0, s1);
+    st_dev(gs + 1, s2);
+    st_dev(gs + 2, sw ? (E > 1 ? misc[1] : 0.f) : 0.f);
+    st_dev(gs + 3, sw ? misc[0] : 0.f);
+    st_dev(ft.gctr + g, 0ull);
+    wait_stores();
+    if (arrive_is_last(ft.fctr, ft.call, (unsigned)p.G)) {
+      st_dev(ft.fctr, 0ull);
+      gate_loss_value<true>(p, ft.gsum, ft.loss);
+    }
+  }
+}
+
+// ---------------------------------------------------------------------------
 // Router projection fused with gating step 1: the K loop of router_mfma_kernel,
 // then the block's 128 x E logits go from the accumulators to LDS (never to
 // HBM unless `logits` is given) and gate_select_tile runs on them.  Needs the
@@ -437,13 +975,19 @@ __global__ __launch_bounds__(256) void router_gate_kernel(
     int32_t* __restrict__ idx, int32_t* __restrict__ pos,
     float* __restrict__ gate, uint8_t* __restrict__ kept,
     float* __restrict__ part1, float* __restrict__ part2,
-    int tokens_per_batch) {
+    int tokens_per_batch, FusedTail ft) {
   constexpr int TOK = 128, BK = 64, ROWB = 128;
   constexpr int X_BYTES = TOK * ROWB, W_BYTES = NT * 32 * ROWB;
   constexpr int STAGE = X_BYTES + W_BYTES;
   extern __shared__ __attribute__((aligned(16))) unsigned char rl_smem[];
+  __shared__ int last_of_group;
   const int E = p.E;
   const int64_t tok0 = (int64_t)blockIdx.x * TOK;       // first token, flat
+  if (ft.bcnt != nullptr && threadIdx.x == 0) {
+    // the first block of a group stamps the group's counter for this call
+    if (tok0 % p.S == 0) counter_prepare(ft.gctr + tok0 / p.S, ft.call);
+    if (blockIdx.x == 0) counter_prepare(ft.fctr, ft.call);
+  }
   const int b = (int)(tok0 / tokens_per_batch);         // router weight set
   const bf16_t* xb = x + tok0 * M;
   const bf16_t* wb = wp + (int64_t)b * E * M;
@@ -553,8 +1097,35 @@ __global__ __launch_bounds__(256) void router_gate_kernel(
   __syncthreads();
   const int g = (int)(tok0 / p.S);
   const int t0 = (int)(tok0 - (int64_t)g * p.S);
-  gate_select_tile<IT>(tile, isone, ld, TOK, g, t0 / TOK, t0, importance,
-                       second_uniform, p, idx, pos, gate, kept, part1, part2);
+  int16_t* ch = reinterpret_cast<int16_t*>(isone + TOK);      // [3][TOK]
+  int32_t* wcnt = reinterpret_cast<int32_t*>(ch + 3 * TOK);   // [3][2][E]
+  float* colpart = reinterpret_cast<float*>(wcnt + 6 * E);    // [4][E]
+  const int blk = t0 / TOK;
+  if (ft.bcnt == nullptr) {
+    // capacity positions and loss follow as launches of their own
+    gate_select_pair_tile<16 * NT, IT>(
+        tile, isone, ld, g, blk, t0, importance, second_uniform, p, idx, pos,
+        gate, kept, part1, part2, nullptr, colpart);
+    return;
+  }
+  gate_select_pair_tile<16 * NT, IT>(
+      tile, isone, ld, g, blk, t0, importance, second_uniform, p, idx, pos,
+      gate, kept, part1, part2, ch, colpart);
+  const bool loss2 = p.use_second_place_loss != 0 || p.router == ROUTER_SWITCH;
+  gate_rank_tile(ch, wcnt, E, loss2, tok0, pos,
+                 ft.bcnt + ((int64_t)g * p.nblk + blk) * 3 * E);
+  // This block's records, counts and partial sums are out (write-through
+  // stores, see st_dev): once every wavefront's stores have completed, one
+  // thread arrives at the group's counter; the last block to arrive finishes
+  // the group.
+  wait_stores();
+  __syncthreads();
+  if (tid == 0)
+    last_of_group =
+        arrive_is_last(ft.gctr + g, ft.call, (unsigned)p.nblk) ? 1 : 0;
+  __syncthreads();
+  if (!last_of_group) return;
+  gate_group_tail(rl_smem, p, ft, g, idx, pos, gate, kept, part1, part2);
   (void)tokens_total;
 }
 
@@ -768,9 +1339,18 @@ __global__ __launch_bounds__(CAP_THREADS) void gate_capacity_kernel(
   }
 }
 
-__global__ void gate_loss_kernel(GateParams p, const float* __restrict__ gsum,
-                                 float* __restrict__ loss) {
-  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+// The balancing loss from the groups' terms; one thread.  COHERENT: the terms
+// were written by other blocks of the same launch (see st_dev).
+template <bool COHERENT>
+__device__ __forceinline__ void gate_loss_value(const GateParams& p,
+                                                const float* gsum_in,
+                                                float* loss) {
+  struct Terms {
+    const float* q;
+    __device__ float operator[](int i) const {
+      return COHERENT ? ld_dev(q + i) : q[i];
+    }
+  } gsum = {gsum_in};
   float s1 = 0.f, s2 = 0.f;
   for (int g = 0; g < p.G; ++g) {
     s1 += gsum[g * GSUM];
@@ -808,6 +1388,12 @@ __global__ void gate_loss_kernel(GateParams p, const float* __restrict__ gsum,
   if (p.num_microbatches > 1)
     l = l * (float)(1.0 / (double)p.num_microbatches);       // moe.py:1439-1442
   loss[0] = l;
+}
+
+__global__ void gate_loss_kernel(GateParams p, const float* __restrict__ gsum,
+                                 float* __restrict__ loss) {
+  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+  gate_loss_value<false>(p, gsum, loss);
 }
 
 static int gate_tokens_per_block(int E) {
@@ -959,6 +1545,12 @@ static GateParams make_switch_params(int G, int S, int E, int C,
   return p;
 }
 
+// LDS the last block of a group needs (gate_group_tail).
+static size_t fused_tail_lds_bytes(int nblk, int E) {
+  return (((size_t)nblk * E * 4 + 15) & ~(size_t)15) +
+         sizeof(int32_t) * 3 * (size_t)E + sizeof(float) * (2 * (size_t)E + 4);
+}
+
 template <int NT, typename IT>
 static int launch_router_gate(const bf16_t* x, const bf16_t* wp,
                               const float* bias, float* logits, int64_t tokens,
@@ -966,23 +1558,37 @@ static int launch_router_gate(const bf16_t* x, const bf16_t* wp,
                               const float* second_uniform, const GateParams& p,
                               int32_t* idx, int32_t* pos, float* gate,
                               uint8_t* kept, float* part1, float* part2,
-                              int tokens_per_batch, hipStream_t st) {
+                              int tokens_per_batch, const FusedTail& ft,
+                              hipStream_t st) {
   const size_t ring = 3 * (128 * 128 + (size_t)NT * 32 * 128);
-  const size_t tile = sizeof(float) * (128 * (size_t)(p.E + 1) + 128);
-  const size_t smem = ring > tile ? ring : tile;
+  // logits tile, importance flags, choices, per-wavefront counts, column sums
+  const size_t tile = sizeof(float) * (128 * (size_t)(p.E + 1) + 128) +
+                      3 * 128 * sizeof(int16_t) +
+                      6 * (size_t)p.E * sizeof(int32_t) +
+                      4 * (size_t)p.E * sizeof(float);
+  size_t smem = ring > tile ? ring : tile;
+  if (ft.bcnt != nullptr) {
+    const size_t tail = fused_tail_lds_bytes(p.nblk, p.E);
+    smem = smem > tail ? smem : tail;
+  }
   auto k = router_gate_kernel<NT, IT>;
   MOE_ALLOW_LDS(k, smem);
   k<<<(unsigned)(tokens / 128), 256, smem, st>>>(
       x, wp, bias, logits, tokens, M, (const IT*)importance, second_uniform, p,
-      idx, pos, gate, kept, part1, part2, tokens_per_batch);
+      idx, pos, gate, kept, part1, part2, tokens_per_batch, ft);
   MOE_CHECK_LAUNCH("router_gate");
   return 0;
 }
 
+// Workspace: per-block partial sums of the loss (2 float arrays), the groups'
+// terms, and for the single-launch kernel per-block counts (3 int32 arrays)
+// and the arrival counters.
 extern "C" size_t mesh_moe_gating_workspace_bytes(int G, int S, int E) {
   if (G < 1 || S < 1 || E < 1) return 0;
   const size_t nblk = (size_t)(S + 63) / 64;  // smallest token block of any path
-  return sizeof(float) * (2 * (size_t)G * nblk * E + GSUM * (size_t)G) + 256;
+  return sizeof(float) * (2 * (size_t)G * nblk * E + GSUM * (size_t)G) +
+         sizeof(int32_t) * 3 * (size_t)G * nblk * E +
+         sizeof(unsigned long long) * ((size_t)G + 1) + 3 * 256;
 }
 
 // Gating from logits: step 1 (softmax / choices) then steps 2 and 3.
@@ -1014,6 +1620,14 @@ static int run_gating(const GateParams& p, const float* logits,
   MOE_CHECK_LAUNCH("gate_select");
   return launch_capacity_and_loss(p, idx, pos, gate, kept, fill, loss, part1,
                                   part2, gsum, st);
+}
+
+// Number of a single-launch gating call: the arrival counters in the
+// workspace are read relative to it (see arrive_is_last).
+static unsigned long long next_call_number() {
+  static std::atomic<unsigned long long> counter{1};
+  unsigned long long n = counter.fetch_add(1, std::memory_order_relaxed);
+  return (n & ((1ull << 48) - 1)) | (1ull << 47);
 }
 
 // Shape limits of the fused projection + gating kernel.
@@ -1054,21 +1668,38 @@ static int run_router_gating(const GateParams& p, const void* x,
   const bf16_t* wp = (const bf16_t*)w_packed;
   const int64_t total = (int64_t)G * S;
   const bool imp_bf16 = importance && importance_dtype == MESH_MOE_BF16;
+  // Slots in token order: positions, fill and loss are finished inside the
+  // same launch by the last block of each group.  Slots by gate (switch_max)
+  // compare every pair of a group's tokens: the capacity kernel does that.
+  FusedTail ft = {};
+  const bool one_launch =
+      !p.rank_by_gate && fused_tail_lds_bytes(p.nblk, E) <= 60 * 1024;
+  if (one_launch) {
+    auto up = [](uintptr_t q) { return (q + 255) & ~(uintptr_t)255; };
+    ft.bcnt = (int32_t*)up((uintptr_t)(gsum + GSUM * (size_t)G));
+    ft.gctr = (unsigned long long*)up(
+        (uintptr_t)(ft.bcnt + 3 * (size_t)G * p.nblk * E));
+    ft.fctr = ft.gctr + G;
+    ft.gsum = gsum;
+    ft.fill = fill;
+    ft.loss = loss;
+    ft.call = next_call_number();
+  }
   int rc;
 #define MOE_ROUTER_GATE(NT)                                                    \
   (imp_bf16 ? launch_router_gate<NT, bf16_t>(xb, wp, bias, logits, total, M,   \
                                              importance, second_uniform, p,    \
                                              idx, pos, gate, kept, part1,      \
-                                             part2, (int)tokens, st)           \
+                                             part2, (int)tokens, ft, st)       \
             : launch_router_gate<NT, float>(xb, wp, bias, logits, total, M,    \
                                             importance, second_uniform, p,     \
                                             idx, pos, gate, kept, part1,       \
-                                            part2, (int)tokens, st))
+                                            part2, (int)tokens, ft, st))
   if (E <= 32) rc = MOE_ROUTER_GATE(1);
   else if (E <= 64) rc = MOE_ROUTER_GATE(2);
   else rc = MOE_ROUTER_GATE(4);
 #undef MOE_ROUTER_GATE
-  if (rc != 0) return rc;
+  if (rc != 0 || one_launch) return rc;
   return launch_capacity_and_loss(p, idx, pos, gate, kept, fill, loss, part1,
                                   part2, gsum, st);
 }
