@@ -76,7 +76,8 @@ __global__ __launch_bounds__(256) void combine_backward_kernel(
       T* d = dy + (((int64_t)e * G + g) * C + c) * N;
       if (vec) {
         uint4* d4 = reinterpret_cast<uint4*>(d);
-        for (int i = lane; i < N / VN; i += 64) d4[i] = make_uint4(0, 0, 0, 0);
+        for (int i = lane; i < N / VN; i += 64)
+          store_streaming(d4 + i, make_uint4(0, 0, 0, 0));
       } else {
         for (int i = lane; i < N; i += 64) d[i] = (T)0;
       }
@@ -104,18 +105,19 @@ __global__ __launch_bounds__(256) void combine_backward_kernel(
     const uint4* d4 = reinterpret_cast<const uint4*>(drc);
     for (int i = lane; i < N / VN; i += 64) {
       float d[VN];
-      unpack16(d4[i], d, T());
+      unpack16(load_streaming(d4 + i), d, T());
 #pragma unroll
       for (int k = 0; k < 2; ++k) {
         if (yrow[k] == nullptr) continue;
         float yv[VN], o[VN];
-        unpack16(reinterpret_cast<const uint4*>(yrow[k])[i], yv, T());
+        unpack16(load_streaming(reinterpret_cast<const uint4*>(yrow[k]) + i), yv,
+                 T());
 #pragma unroll
         for (int j = 0; j < VN; ++j) {
           dot[k] += d[j] * yv[j];
           o[j] = w[k] * d[j];
         }
-        reinterpret_cast<uint4*>(drow[k])[i] = pack16(o, T());
+        store_streaming(reinterpret_cast<uint4*>(drow[k]) + i, pack16(o, T()));
       }
     }
   } else {
@@ -181,7 +183,8 @@ __global__ __launch_bounds__(256) void dispatch_backward_kernel(
       for (int k = 0; k < 2; ++k) {
         if (src[k] == nullptr) continue;
         float v[VN];
-        unpack16(reinterpret_cast<const uint4*>(src[k])[i], v, T());
+        unpack16(load_streaming(reinterpret_cast<const uint4*>(src[k]) + i), v,
+                 T());
 #pragma unroll
         for (int j = 0; j < VN; ++j) acc[j] += v[j];
       }
@@ -195,7 +198,7 @@ __global__ __launch_bounds__(256) void dispatch_backward_kernel(
           for (int j = 0; j < VN; ++j) acc[j] += d * v[j];
         }
       }
-      reinterpret_cast<uint4*>(dst)[i] = pack16(acc, T());
+      store_streaming(reinterpret_cast<uint4*>(dst) + i, pack16(acc, T()));
     }
   } else {
     for (int i = lane; i < M; i += 64) {
@@ -266,7 +269,8 @@ __global__ __launch_bounds__(256) void dispatch_backward_router4_kernel(
       for (int k = 0; k < 2; ++k) {
         if (src[j][k] == nullptr) continue;
         float v[VN];
-        unpack16(reinterpret_cast<const uint4*>(src[j][k])[i], v, T());
+        unpack16(load_streaming(reinterpret_cast<const uint4*>(src[j][k]) + i), v,
+                 T());
 #pragma unroll
         for (int q = 0; q < VN; ++q) acc[j][q] += v[q];
       }
@@ -284,7 +288,8 @@ __global__ __launch_bounds__(256) void dispatch_backward_router4_kernel(
 #pragma unroll
     for (int j = 0; j < DBR_TOK; ++j)
       if (t0 + j < T_tokens)
-        reinterpret_cast<uint4*>(dx + (t0 + j) * M)[i] = pack16(acc[j], T());
+        store_streaming(reinterpret_cast<uint4*>(dx + (t0 + j) * M) + i,
+                        pack16(acc[j], T()));
   }
 }
 

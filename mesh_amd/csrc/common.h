@@ -128,6 +128,30 @@ __device__ __forceinline__ void store_f32<bf16_t>(bf16_t* p, float v) {
   *p = f32_to_bf16(v);
 }
 
+// 16-byte store that does not allocate in the L2 on its way out.  The rows
+// written here are not read again by the same kernel; with ordinary stores
+// the write-back L2 fetched the lines it was about to overwrite and wrote
+// some of them back more than once (measured on the dispatch kernel: 1.68 GB
+// written and 1.04 GB read for 1.07 GB / 0.54 GB of named traffic; with these
+// stores 1.14 GB / 0.54 GB, and 0.34 ms instead of 0.43 ms).
+typedef uint32_t u32x4_nt_t __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void store_streaming(uint4* p, const uint4& v) {
+  __builtin_nontemporal_store(*reinterpret_cast<const u32x4_nt_t*>(&v),
+                              reinterpret_cast<u32x4_nt_t*>(p));
+}
+// 16-byte load of data this kernel reads once (the same hint on the way in;
+// the combine kernel runs 13 % faster with it).
+__device__ __forceinline__ uint4 load_streaming(const uint4* p) {
+  const u32x4_nt_t v =
+      __builtin_nontemporal_load(reinterpret_cast<const u32x4_nt_t*>(p));
+  return make_uint4(v[0], v[1], v[2], v[3]);
+}
+
+template <typename T>
+struct Vec16 {
+  static constexpr int N = 16 / sizeof(T);
+};
+
 __device__ __forceinline__ float apply_activation(float v, int act) {
   switch (act) {
     case MESH_MOE_ACT_RELU:
