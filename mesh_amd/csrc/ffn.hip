@@ -923,6 +923,148 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
 }
 
 // ---------------------------------------------------------------------------
+// float32 on the matrix cores: v_mfma_f32_32x32x2_f32, true float32 operands
+// and accumulation (the float32 configuration of the layer: no narrowing).
+// Block tile 128 x 128, K step 32, 4 wavefronts in a 2 x 2 grid, each a 64 x 64
+// sub-tile = 2 x 2 MFMA tiles.  As in the bf16 kernels the weight tile is the
+// MFMA's first operand, so a lane ends up with 4 consecutive output columns
+// per register group.  One MFMA consumes k = 2 s + (lane / 32) for step s; a
+// lane instead takes the four consecutive k = 8 u + 4 (lane / 32) + j for steps
+// 4 u + j (both operands agree on the order, and a sum does not care), which
+// makes its operand reads 16 bytes wide.  Tiles are staged through registers
+// into LDS rows of 32 + 4 floats.  K % 4 == 0 and N % 4 == 0.
+// ---------------------------------------------------------------------------
+struct F32Cfg {
+  static constexpr int BM = 128, BN = 128, BK = 32, THREADS = 256;
+  static constexpr int LDK = BK + 4;               // floats per LDS row
+  static constexpr int CPR = BK / 4;               // 16-byte chunks per row
+  static constexpr int A_CHUNKS = BM * CPR / THREADS, B_CHUNKS = BN * CPR / THREADS;
+  static constexpr size_t LDS_BYTES = 2ull * (BM + BN) * LDK * sizeof(float);
+};
+
+template <bool RELU>
+__global__ __launch_bounds__(256) void grouped_gemm_f32_mfma_kernel(
+    const float* __restrict__ A, const float* __restrict__ B,
+    float* __restrict__ Cout, int R, int N, int K, int tiles_m, int tiles_n) {
+  using Cfg = F32Cfg;
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, LDK = Cfg::LDK;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+  float* As = reinterpret_cast<float*>(smem_raw);  // [2][BM][LDK]
+  float* Bs = As + 2 * BM * LDK;                   // [2][BN][LDK]
+  const int tiles_per_e = tiles_m * tiles_n;
+  const int e = blockIdx.x / tiles_per_e;
+  const int rem = blockIdx.x - e * tiles_per_e;
+  const int tn = rem / tiles_m, tm = rem - tn * tiles_m;
+  const int row0 = tm * BM, col0 = tn * BN;
+  const float* Ae = A + (int64_t)e * R * K;
+  const float* Be = B + (int64_t)e * N * K;
+  float* Ce = Cout + (int64_t)e * R * N;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int wm = wave >> 1, wn = wave & 1;
+
+  uint4 areg[Cfg::A_CHUNKS], breg[Cfg::B_CHUNKS];
+  auto load_global = [&](int k0) {
+#pragma unroll
+    for (int i = 0; i < Cfg::A_CHUNKS; ++i) {
+      const int c = tid + i * Cfg::THREADS;
+      const int r = c / Cfg::CPR, gk = k0 + (c % Cfg::CPR) * 4;
+      const int gr = min(row0 + r, R - 1);
+      const uint4 v = *reinterpret_cast<const uint4*>(
+          Ae + (int64_t)gr * K + min(gk, K - 4));
+      areg[i] = gk < K ? v : make_uint4(0, 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < Cfg::B_CHUNKS; ++i) {
+      const int c = tid + i * Cfg::THREADS;
+      const int r = c / Cfg::CPR, gk = k0 + (c % Cfg::CPR) * 4;
+      const int gr = min(col0 + r, N - 1);
+      const uint4 v = *reinterpret_cast<const uint4*>(
+          Be + (int64_t)gr * K + min(gk, K - 4));
+      breg[i] = gk < K ? v : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto store_lds = [&](int buf) {
+#pragma unroll
+    for (int i = 0; i < Cfg::A_CHUNKS; ++i) {
+      const int c = tid + i * Cfg::THREADS;
+      *reinterpret_cast<uint4*>(As + (buf * BM + c / Cfg::CPR) * LDK +
+                                (c % Cfg::CPR) * 4) = areg[i];
+    }
+#pragma unroll
+    for (int i = 0; i < Cfg::B_CHUNKS; ++i) {
+      const int c = tid + i * Cfg::THREADS;
+      *reinterpret_cast<uint4*>(Bs + (buf * BN + c / Cfg::CPR) * LDK +
+                                (c % Cfg::CPR) * 4) = breg[i];
+    }
+  };
+
+  f32x16_t acc[2][2];
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+
+  const int nk = (K + BK - 1) / BK;
+  load_global(0);
+  store_lds(0);
+  __syncthreads();
+  const int frag_row = lane & 31, frag_k = (lane >> 5) * 4;
+  for (int kt = 0; kt < nk; ++kt) {
+    const int buf = kt & 1;
+    if (kt + 1 < nk) load_global((kt + 1) * BK);
+    const float* as = As + (buf * BM + wm * 64 + frag_row) * LDK + frag_k;
+    const float* bs = Bs + (buf * BN + wn * 64 + frag_row) * LDK + frag_k;
+#pragma unroll
+    for (int u = 0; u < BK / 8; ++u) {
+      float4 af[2], bfr[2];
+#pragma unroll
+      for (int i = 0; i < 2; ++i)
+        af[i] = *reinterpret_cast<const float4*>(as + i * 32 * LDK + u * 8);
+#pragma unroll
+      for (int j = 0; j < 2; ++j)
+        bfr[j] = *reinterpret_cast<const float4*>(bs + j * 32 * LDK + u * 8);
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+          for (int j = 0; j < 2; ++j) {
+            const float a = q == 0 ? af[i].x : q == 1 ? af[i].y
+                            : q == 2 ? af[i].z : af[i].w;
+            const float b = q == 0 ? bfr[j].x : q == 1 ? bfr[j].y
+                            : q == 2 ? bfr[j].z : bfr[j].w;
+            acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x2f32(b, a, acc[i][j],
+                                                             0, 0, 0);
+          }
+      }
+    }
+    if (kt + 1 < nk) store_lds(buf ^ 1);
+    __syncthreads();
+  }
+  const int m_l = lane & 31, n_l = (lane >> 5) * 4;
+#pragma unroll
+  for (int i = 0; i < 2; ++i)
+#pragma unroll
+    for (int j = 0; j < 2; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const int grow = row0 + wm * 64 + i * 32 + m_l;
+        const int gcol = col0 + wn * 64 + j * 32 + 8 * q + n_l;
+        if (grow < R && gcol < N) {
+          float4 v = make_float4(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1],
+                                 acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
+          if (RELU) {
+            v.x = fmaxf(v.x, 0.f); v.y = fmaxf(v.y, 0.f);
+            v.z = fmaxf(v.z, 0.f); v.w = fmaxf(v.w, 0.f);
+          }
+          *reinterpret_cast<float4*>(Ce + (int64_t)grow * N + gcol) = v;
+        }
+      }
+}
+
+// ---------------------------------------------------------------------------
 // Plain FMA tile kernel (float32, and bf16 shapes the MFMA kernel rejects):
 // 64 x 64 tile, 16-deep K step, each thread a 4 x 4 patch, float32 accumulate
 // in k order.
@@ -1244,6 +1386,29 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
   return 0;
 }
 
+static int launch_f32_mfma(const float* A, const float* B, float* C, int E,
+                           int R, int N, int K, bool relu, hipStream_t st) {
+  using Cfg = F32Cfg;
+  const int tiles_m = (R + Cfg::BM - 1) / Cfg::BM;
+  const int tiles_n = (N + Cfg::BN - 1) / Cfg::BN;
+  const int64_t blocks = (int64_t)tiles_m * tiles_n * E;
+  MOE_REQUIRE(blocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
+              "expert_ffn: too many tiles (%lld)", (long long)blocks);
+  if (relu) {
+    auto k = grouped_gemm_f32_mfma_kernel<true>;
+    MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
+    k<<<(unsigned)blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
+        A, B, C, R, N, K, tiles_m, tiles_n);
+  } else {
+    auto k = grouped_gemm_f32_mfma_kernel<false>;
+    MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
+    k<<<(unsigned)blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
+        A, B, C, R, N, K, tiles_m, tiles_n);
+  }
+  MOE_CHECK_LAUNCH("expert_ffn (float32 mfma)");
+  return 0;
+}
+
 template <typename T>
 static int launch_simple(const T* A, const T* B, T* C, int E, int R, int N,
                          int K, bool relu, hipStream_t st) {
@@ -1273,8 +1438,13 @@ static int grouped_gemm(const void* A, const void* B, void* C, int E, int R,
   int rc;
   if (mask_applied) *mask_applied = false;
   if (dtype == MESH_MOE_F32) {
-    rc = launch_simple<float>((const float*)A, (const float*)B, (float*)C, E,
-                              R, N, K, relu, st);
+    if (K % 4 == 0 && N % 4 == 0 && K >= 32 && R >= 32 && N >= 32 &&
+        (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) % 16 == 0))
+      rc = launch_f32_mfma((const float*)A, (const float*)B, (float*)C, E, R,
+                           N, K, relu, st);
+    else
+      rc = launch_simple<float>((const float*)A, (const float*)B, (float*)C, E,
+                                R, N, K, relu, st);
   } else {
     const bool mfma_ok =
         (K % 8 == 0) && (N % 8 == 0) &&
