@@ -453,90 +453,122 @@ __device__ __forceinline__ void gate_select_tile(
 }
 
 // ---------------------------------------------------------------------------
-// gate_select_tile for a block of 256 threads and 128 tokens: two threads per
-// token (adjacent lanes), each owning half of the experts.  The exponentials,
-// two per expert and the bulk of the work, are split between the pair; every
-// float32 sum still runs in expert order (the first thread's partial sum is
-// handed to the second, which continues it), and the first-arg-max of a pair
-// prefers the lower half on ties, so every per-token result is bit for bit
-// that of gate_select_tile.  The per-block column sums for the loss are split
-// over four row ranges.  H2MAX >= E / 2 (E even) bounds the register copy of a
-// thread's logits; colpart: LDS [4][E] floats.
+// gate_select_tile for the projection kernel, straight from the matrix-core
+// accumulators: 256 threads, 128 tokens, two lanes per token.  After the
+// 32x32x16 MFMAs lane l of a wavefront holds, for token l % 32 and per
+// 32-expert tile j, the logits of experts 32 j + 8 q + 4 (l / 32) + r (q, r =
+// 0..3): lanes l and l + 32 together hold the token's whole row, in alternating
+// groups of four experts.  Each lane does the exponentials of its half (two per
+// expert, the bulk of the work); every float32 sum still runs in expert order
+// (the running sum changes lanes after every group of four) and a tie between
+// the two lanes' arg-max candidates goes to the lower expert, so every
+// per-token result is bit for bit that of gate_select_tile.  The probabilities
+// go to LDS (tile [128][ld], ld % 4 == 0) for the per-block column sums of the
+// loss, which are split over four row ranges; colpart: LDS [4][E] floats.
 // ---------------------------------------------------------------------------
-template <int H2MAX, typename IT>
-__device__ __forceinline__ void gate_select_pair_tile(
-    float* tile, float* isone, int ld, int g, int blk, int t0,
-    const IT* __restrict__ importance, const float* __restrict__ second_uniform,
-    const GateParams& p, int32_t* __restrict__ idx, int32_t* __restrict__ pos,
+template <int NT, typename IT>
+__device__ __forceinline__ void gate_select_acc_tile(
+    const float (&x)[NT][16], float* tile, float* isone, int ld, int g, int blk,
+    int t0, const IT* __restrict__ importance,
+    const float* __restrict__ second_uniform, const GateParams& p,
+    int32_t* __restrict__ idx, int32_t* __restrict__ pos,
     float* __restrict__ gate, uint8_t* __restrict__ kept,
     float* __restrict__ part1, float* __restrict__ part2, int16_t* ch,
     float* colpart) {
   constexpr int NTOK = 128;
-  const int E = p.E, S = p.S, H2 = E >> 1;
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int tok = tid >> 1, half = tid & 1;
-  const int eb = half * H2;
+  const int E = p.E, S = p.S;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5;
+  const int tok = wave * 32 + (lane & 31);
   const bool sw = p.router == ROUTER_SWITCH;
   float* row = tile + tok * ld;
   const int64_t t = (int64_t)g * S + t0 + tok;
-  // the other thread of the pair has the strictly better candidate?  (equal
-  // values: the lower half, i.e. the lower expert index, wins)
-  auto take_other = [&](float mine, float other) {
-    return half == 0 ? other > mine : !(mine > other);
+  // first expert of this lane's group (j, q); the group exists if it is < E
+  auto first = [&](int j, int q) { return j * 32 + 8 * q + 4 * half; };
+  // the partner's candidate wins if it is larger, or equal with a lower index
+  auto take_other = [&](float mine, int mi, float other, int oi) {
+    return other > mine || (other == mine && oi < mi);
+  };
+  // a float32 sum over the experts in index order: the lanes of a pair take
+  // turns, the running value changing lanes after every group of four
+  auto ordered_sum = [&](const float (&v)[NT][16]) {
+    float s = 0.f;
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q) {
+        const bool mine = first(j, q) < E;
+#pragma unroll
+        for (int hh = 0; hh < 2; ++hh) {
+          if (half == hh && mine) {
+#pragma unroll
+            for (int r = 0; r < 4; ++r) s += v[j][4 * q + r];
+          }
+          s = __shfl_xor(s, 32);
+        }
+      }
+    return __shfl(s, lane & 31);      // the lower lane holds the final value
   };
 
-  float xr[H2MAX];
   float m = -INFINITY;
 #pragma unroll
-  for (int j = 0; j < H2MAX; ++j)
-    if (j < H2) {
-      xr[j] = row[eb + j];
-      m = fmaxf(m, xr[j]);                                  // reduce_max
-    }
-  m = fmaxf(m, __shfl_xor(m, 1));
-  const float negm = -m;
-  float s = 0.f;
+  for (int j = 0; j < NT; ++j)
 #pragma unroll
-  for (int j = 0; j < H2MAX; ++j)
-    if (j < H2) {
-      const float u = expf(xr[j] + negm);                   // exp
-      if (half == 0) s += u;                                // reduce_sum ...
-      else row[eb + j] = u;
-    }
-  const float s_low = __shfl(s, lane & ~1);
-  if (half == 1) {
-    s = s_low;                                              // ... continued
-    for (int j = 0; j < H2; ++j) s += row[eb + j];
-  }
-  s = __shfl(s, lane | 1);
-  const float neglse = -(logf(s) + m);                      // log + max
+    for (int q = 0; q < 4; ++q)
+      if (first(j, q) < E) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) m = fmaxf(m, x[j][4 * q + r]);   // reduce_max
+      }
+  m = fmaxf(m, __shfl_xor(m, 32));
+  const float negm = -m;
+  float pr[NT][16];
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) pr[j][i] = expf(x[j][i] + negm);    // exp
+  const float ssum = ordered_sum(pr);                                // reduce_sum
+  const float neglse = -(logf(ssum) + m);                            // log + max
   float g1 = -1.f;
   int i1 = 0;
 #pragma unroll
-  for (int j = 0; j < H2MAX; ++j)
-    if (j < H2) {
-      const float pe = expf(xr[j] + neglse);                // exp(log_softmax)
-      row[eb + j] = pe;
-      if (pe > g1) { g1 = pe; i1 = eb + j; }                // first argmax
-    }
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+      if (first(j, q) < E) {
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+          const float pe = expf(x[j][4 * q + r] + neglse);   // exp(log_softmax)
+          pr[j][4 * q + r] = pe;
+          if (pe > g1) { g1 = pe; i1 = first(j, q) + r; }    // first argmax
+        }
+        *reinterpret_cast<float4*>(row + first(j, q)) = make_float4(
+            pr[j][4 * q], pr[j][4 * q + 1], pr[j][4 * q + 2], pr[j][4 * q + 3]);
+      }
   {
-    const float og = __shfl_xor(g1, 1);
-    const int oi = __shfl_xor(i1, 1);
-    if (take_other(g1, og)) { g1 = og; i1 = oi; }
+    const float og = __shfl_xor(g1, 32);
+    const int oi = __shfl_xor(i1, 32);
+    if (take_other(g1, i1, og, oi)) { g1 = og; i1 = oi; }
   }
   bool sel1 = true;
   if (sw && second_uniform != nullptr) {
     // policy "sample": first arg-max of the caller's choice logits
     const float* cl = second_uniform + t * E;
     float best = -INFINITY;
-    int bi = eb;
-    for (int j = 0; j < H2; ++j) {
-      const float v = cl[eb + j];
-      if (j == 0 || v > best) { best = v; bi = eb + j; }
-    }
-    const float ob = __shfl_xor(best, 1);
-    const int oi = __shfl_xor(bi, 1);
-    if (take_other(best, ob)) bi = oi;
+    int bi = E;
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if (first(j, q) < E) {
+          const float4 c4 = *reinterpret_cast<const float4*>(cl + first(j, q));
+          const float cv[4] = {c4.x, c4.y, c4.z, c4.w};
+#pragma unroll
+          for (int r = 0; r < 4; ++r)
+            if (bi == E || cv[r] > best) { best = cv[r]; bi = first(j, q) + r; }
+        }
+    const float ob = __shfl_xor(best, 32);
+    const int oi = __shfl_xor(bi, 32);
+    if (take_other(best, bi, ob, oi)) bi = oi;
     i1 = bi;
     __syncthreads();           // the partner's half of the row is in LDS
     g1 = row[i1];
@@ -574,29 +606,27 @@ __device__ __forceinline__ void gate_select_pair_tile(
       sel2 = (imp > 0.0f);
     }
     if (!sel1) g1 = g1 * 0.0f;
-    float g2 = -1.f, qsum = 0.f;
+    // gates_without_top_1 = raw_gates * (1 - mask_1), in place; its first argmax
+    float g2 = -1.f;
     int i2 = 0;
-    for (int j = 0; j < H2; ++j) {
-      const int e = eb + j;
-      const float keep = (sel1 && e == i1) ? 0.0f : 1.0f;
-      const float q = row[e] * keep;
-      if (half == 0) qsum += q;
-      if (q > g2) { g2 = q; i2 = e; }
-    }
-    const float q_low = __shfl(qsum, lane & ~1);
-    if (half == 1) {
-      qsum = q_low;
-      for (int j = 0; j < H2; ++j) {
-        const int e = eb + j;
-        const float keep = (sel1 && e == i1) ? 0.0f : 1.0f;
-        qsum += row[e] * keep;
-      }
-    }
-    qsum = __shfl(qsum, lane | 1);
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if (first(j, q) < E) {
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const int e = first(j, q) + r;
+            const float keep = (sel1 && e == i1) ? 0.0f : 1.0f;
+            const float qv = pr[j][4 * q + r] * keep;
+            pr[j][4 * q + r] = qv;
+            if (qv > g2) { g2 = qv; i2 = e; }
+          }
+        }
     {
-      const float og = __shfl_xor(g2, 1);
-      const int oi = __shfl_xor(i2, 1);
-      if (take_other(g2, og)) { g2 = og; i2 = oi; }
+      const float og = __shfl_xor(g2, 32);
+      const int oi = __shfl_xor(i2, 32);
+      if (take_other(g2, i2, og, oi)) { g2 = og; i2 = oi; }
     }
     const float denom = (g1 + g2) + 1e-9f;
     const float r = 1.0f / denom;
@@ -625,7 +655,8 @@ __device__ __forceinline__ void gate_select_pair_tile(
       }
       isone[tok] = sel1 ? 1.0f : 0.0f;
     }
-    qscale = 1.0f / (qsum + 1e-9f);
+    if (p.use_second_place_loss)
+      qscale = 1.0f / (ordered_sum(pr) + 1e-9f);            // moe.py:1433-1434
   }
   __syncthreads();
   // column sums over the block's tokens, four row ranges per column
@@ -655,12 +686,16 @@ __device__ __forceinline__ void gate_select_pair_tile(
     __syncthreads();
     column_sums(2, false, part2);
   } else if (p.use_second_place_loss) {
+    // the proxy of the second-place loss: (gates without the first) / their sum
     __syncthreads();
-    for (int j = 0; j < H2; ++j) {
-      const int e = eb + j;
-      const float keep = (sel1 && e == i1) ? 0.0f : 1.0f;
-      row[e] = (row[e] * keep) * qscale;
-    }
+#pragma unroll
+    for (int j = 0; j < NT; ++j)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        if (first(j, q) < E)
+          *reinterpret_cast<float4*>(row + first(j, q)) = make_float4(
+              pr[j][4 * q] * qscale, pr[j][4 * q + 1] * qscale,
+              pr[j][4 * q + 2] * qscale, pr[j][4 * q + 3] * qscale);
     __syncthreads();
     column_sums(E, false, part2);
   }
@@ -778,12 +813,15 @@ __device__ __forceinline__ void gate_rank_tile(
   for (int e0 = 0; e0 < E; e0 += 64) {
     int cnt = 0;   // lane l: choosers of expert e0 + l in this wavefront
     const int n = min(64, E - e0);
+    // branch-free: the selects below are cheaper than a taken branch
+#pragma unroll 8
     for (int j = 0; j < n; ++j) {
-      const unsigned long long m = __ballot(mine == e0 + j);
-      if (mine == e0 + j)
-        rank = __builtin_amdgcn_mbcnt_hi(
-            (unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0u));
-      if (lane == j) cnt = __popcll(m);
+      const bool hit = mine == e0 + j;
+      const unsigned long long m = __ballot(hit);
+      const int below = (int)__builtin_amdgcn_mbcnt_hi(
+          (unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0u));
+      rank = hit ? below : rank;
+      cnt = lane == j ? (int)__popcll(m) : cnt;
     }
     if (lane < n) wcnt[(c * 2 + half) * E + e0 + lane] = cnt;
   }
@@ -792,9 +830,10 @@ __device__ __forceinline__ void gate_rank_tile(
     for (int e0 = 0; e0 < E; e0 += 64) {
       int cnt = 0;
       const int n = min(64, E - e0);
+#pragma unroll 8
       for (int j = 0; j < n; ++j) {
         const unsigned long long m = __ballot(third == e0 + j);
-        if (lane == j) cnt = __popcll(m);
+        cnt = lane == j ? (int)__popcll(m) : cnt;
       }
       if (lane < n) wcnt[(4 + half) * E + e0 + lane] = cnt;
     }
@@ -1080,28 +1119,30 @@ __global__ __launch_bounds__(256) void router_gate_kernel(
   }
   __syncthreads();  // every wavefront is done with the ring: reuse it
 
-  // accumulators -> LDS logits tile [128][E + 1]
+  // this lane's logits (+ bias), written out if the caller wants them
   float* tile = reinterpret_cast<float*>(rl_smem);
-  const int ld = E + 1;
+  const int ld = E + 4;
   float* isone = tile + TOK * ld;
   const int trow = wave * 32 + (lane & 31);
+  float xl[NT][16];
 #pragma unroll
   for (int j = 0; j < NT; ++j) {
 #pragma unroll
     for (int q = 0; q < 4; ++q) {
       const int e0 = j * 32 + 8 * q + 4 * (lane >> 5);
-      if (e0 < E) {
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          float v = acc[j][4 * q + r];
+      for (int r = 0; r < 4; ++r) {
+        float v = acc[j][4 * q + r];
+        if (e0 < E) {
           if (bias != nullptr) v += bias[e0 + r];
-          tile[trow * ld + e0 + r] = v;
           if (logits != nullptr) logits[(tok0 + trow) * E + e0 + r] = v;
+        } else {
+          v = -INFINITY;     // not an expert: exp() = 0, never the maximum
         }
+        xl[j][4 * q + r] = v;
       }
     }
   }
-  __syncthreads();
   const int g = (int)(tok0 / p.S);
   const int t0 = (int)(tok0 - (int64_t)g * p.S);
   int16_t* ch = reinterpret_cast<int16_t*>(isone + TOK);      // [3][TOK]
@@ -1110,13 +1151,13 @@ __global__ __launch_bounds__(256) void router_gate_kernel(
   const int blk = t0 / TOK;
   if (ft.bcnt == nullptr) {
     // capacity positions and loss follow as launches of their own
-    gate_select_pair_tile<16 * NT, IT>(
-        tile, isone, ld, g, blk, t0, importance, second_uniform, p, idx, pos,
-        gate, kept, part1, part2, nullptr, colpart);
+    gate_select_acc_tile<NT, IT>(
+        xl, tile, isone, ld, g, blk, t0, importance, second_uniform, p, idx,
+        pos, gate, kept, part1, part2, nullptr, colpart);
     return;
   }
-  gate_select_pair_tile<16 * NT, IT>(
-      tile, isone, ld, g, blk, t0, importance, second_uniform, p, idx, pos,
+  gate_select_acc_tile<NT, IT>(
+      xl, tile, isone, ld, g, blk, t0, importance, second_uniform, p, idx, pos,
       gate, kept, part1, part2, ch, colpart);
   const bool loss2 = p.use_second_place_loss != 0 || p.router == ROUTER_SWITCH;
   gate_rank_tile(ch, wcnt, E, loss2, tok0, pos,
@@ -1569,7 +1610,7 @@ static int launch_router_gate(const bf16_t* x, const bf16_t* wp,
                               hipStream_t st) {
   const size_t ring = 3 * (128 * 128 + (size_t)NT * 32 * 128);
   // logits tile, importance flags, choices, per-wavefront counts, column sums
-  const size_t tile = sizeof(float) * (128 * (size_t)(p.E + 1) + 128) +
+  const size_t tile = sizeof(float) * (128 * (size_t)(p.E + 4) + 128) +
                       3 * 128 * sizeof(int16_t) +
                       6 * (size_t)p.E * sizeof(int32_t) +
                       4 * (size_t)p.E * sizeof(float);
