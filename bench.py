@@ -88,7 +88,7 @@ def normal_init(fan_in, seed):
   return init
 
 
-def build(cfg, device, backward=False):
+def build(cfg, device, backward=False, operands="random"):
   """Builds the graph for `cfg` through the mtf-shaped API and lowers it once.
   With backward=True the graph also holds mtf.gradients of (outputs, loss)
   w.r.t. the tokens and the kernels.  Returns (lowering, x Tensor, y Tensor,
@@ -126,6 +126,20 @@ def build(cfg, device, backward=False):
     init["moe/inner_gating/kernel"] = normal_init(m, 5)
     init["moe/wi/kernel"] = normal_init(m, 3)
     init["moe/wo/kernel"] = normal_init(h, 4)
+  if operands != "random":
+    # the same instruction stream and memory traffic on operands that do not
+    # toggle the multipliers: what the chip's power limit costs this kernel
+    zeros_init = lambda sizes, dtype, dev: torch.zeros(sizes, dtype=dtype,
+                                                       device=dev)
+    for name in list(init):
+      if name.endswith("/wi/kernel") or name.endswith("/wo/kernel"):
+        init[name] = zeros_init
+    if operands == "zero_tokens":
+      # zeros times zeros in the experts.  The router then sees equal logits
+      # everywhere and sends every token to experts 0 and 1: only the padded
+      # flop count (every slot row is multiplied, occupied or not) means
+      # anything in this mode
+      x_val = x_val * 0
   x = mtf.import_tf_tensor(mesh, x_val, mtf.Shape(dims))
   with mtf.variable_scope("moe"):
     if cfg["layer"] == "v1":
@@ -293,6 +307,11 @@ def main():
                   help="time replays of a recorded HIP graph of the step "
                        "(Lowering.capture) instead of eager runs; the per-stage "
                        "times still come from eager runs")
+  ap.add_argument("--operands", default="random",
+                  choices=["random", "zero_weights", "zero_tokens"],
+                  help="diagnostic: zero expert weights (and tokens): the same "
+                       "kernels and traffic without operand toggling, to read "
+                       "the power limit off the clock; not the benchmark")
   ap.add_argument("--no-cpu-baseline", action="store_true")
   args = ap.parse_args()
   if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -321,7 +340,8 @@ def main():
   if args.block:
     lowering, x, y, loss = build_block(cfg, device, args.backward)
   else:
-    lowering, x, y, loss = build(cfg, device, args.backward)  # first execution
+    lowering, x, y, loss = build(cfg, device, args.backward,
+                                 args.operands)            # first execution
   for _ in range(args.warmup):
     lowering.run()
   torch.cuda.synchronize()
@@ -378,7 +398,7 @@ def main():
       "vs_baseline": None, "dtype": cfg["dtype"], "data": "synthetic",
       "config": {"workload": cfg["name"], "layer": cfg["layer"],
                  "tokens": tokens, "output_finite": out_ok,
-                 "hip_graph": bool(args.graph)},
+                 "hip_graph": bool(args.graph), "operands": args.operands},
   }
   if cfg["layer"] == "v1":
     r = routings[-1]

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 17
+#define MESH_MOE_ABI_VERSION 18
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -333,6 +333,44 @@ int mesh_moe_dispatched_expert_ffn(
 int mesh_moe_combine(const void* y, const int32_t* idx, const int32_t* pos,
                      const float* gate, const uint8_t* kept, void* out, int G,
                      int S, int E, int C, int N, int dtype, void* stream);
+
+/* Bytes of scratch mesh_moe_compact_expert_ffn needs. */
+size_t mesh_moe_compact_expert_ffn_workspace_bytes(int G, int E, int C, int M,
+                                                   int H, int N);
+
+/*
+ * mesh_moe_dispatched_expert_ffn on COMPACTED rows: the dispatch einsum and
+ * the two expert einsums (transformer/moe.py:443-447, :469-486) for routers
+ * that leave many slots empty (one choice per token with a capacity factor
+ * above 1: _switch_gating, _ntlb_gating, transformer/moe.py:1176-1309,
+ * :804-940).  The reference multiplies every slot row, occupied or not; here
+ * expert e's occupied slots (groups in order, slots in order) become rows
+ * 0 .. used_e - 1 of its row range in h and y, and only the 256-row tiles that
+ * hold such rows are computed.  Rows beyond used_e hold unspecified values.
+ *   fill [G,E] as written by the gating calls
+ *   row_offsets [E,G] int32 (output): row of expert e's first slot of group
+ *     g; slot (e, g, c) is row row_offsets[e][g] + c of h[e] / y[e] -- what
+ *     mesh_moe_combine_compact takes
+ * Otherwise as mesh_moe_dispatched_expert_ffn (same limits, both GEMMs must
+ * fit the 256 x 256 kernel, E <= 1024, MESH_MOE_E_UNSUPPORTED otherwise).
+ */
+int mesh_moe_compact_expert_ffn(
+    const void* x, const int32_t* idx, const int32_t* pos, const float* gate,
+    const uint8_t* kept, const int32_t* fill, const void* wi_packed,
+    const void* wo_packed, void* h, void* y, int32_t* row_offsets,
+    void* workspace, size_t workspace_bytes, int G, int S, int E, int C, int M,
+    int H, int N, int activation, int dtype, void* stream);
+
+/*
+ * mesh_moe_combine (transformer/moe.py:509-510) reading y in the compacted
+ * row order of mesh_moe_compact_expert_ffn: y [E, G*C, N], slot (e, g, c) at
+ * row row_offsets[e][g] + c.
+ */
+int mesh_moe_combine_compact(const void* y, const int32_t* idx,
+                             const int32_t* pos, const float* gate,
+                             const uint8_t* kept, const int32_t* row_offsets,
+                             void* out, int G, int S, int E, int C, int N,
+                             int dtype, void* stream);
 
 /*
  * "No token left behind" gating (_ntlb_gating, transformer/moe.py:804-940)

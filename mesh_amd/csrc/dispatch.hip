@@ -142,7 +142,8 @@ __global__ __launch_bounds__(256) void combine_kernel(
     const T* __restrict__ y, const int32_t* __restrict__ idx,
     const int32_t* __restrict__ pos, const float* __restrict__ gate,
     const uint8_t* __restrict__ kept, T* __restrict__ out, int G, int S, int E,
-    int C, int N, int64_t T_tokens, bool vec) {
+    int C, int N, int64_t T_tokens, bool vec,
+    const int32_t* __restrict__ row_offsets) {
   const int lane = threadIdx.x & 63;
   const int64_t t = (int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6);
   if (t >= T_tokens) return;
@@ -154,8 +155,13 @@ __global__ __launch_bounds__(256) void combine_kernel(
     if (kept[t * 2 + k]) {
       const float wk = round_to<T>(gate[t * 2 + k]);
       if (wk != 0.0f) {
+        const int64_t e = idx[t * 2 + k];
+        // row of the slot: [e][g][c], or with compacted rows the expert's
+        // occupied slots of earlier groups first (row_offsets[e][g])
         const int64_t slot =
-            ((int64_t)idx[t * 2 + k] * G + g) * C + pos[t * 2 + k];
+            row_offsets == nullptr
+                ? (e * G + g) * C + pos[t * 2 + k]
+                : e * G * C + row_offsets[e * G + g] + pos[t * 2 + k];
         src[k] = y + slot * N;
         w[k] = wk;
       }
@@ -259,10 +265,34 @@ extern "C" int mesh_moe_dispatch(const void* x, const int32_t* idx,
   return 0;
 }
 
+static int run_combine(const void* y, const int32_t* idx, const int32_t* pos,
+                       const float* gate, const uint8_t* kept,
+                       const int32_t* row_offsets, void* out, int G, int S,
+                       int E, int C, int N, int dtype, void* stream);
+
 extern "C" int mesh_moe_combine(const void* y, const int32_t* idx,
                                 const int32_t* pos, const float* gate,
                                 const uint8_t* kept, void* out, int G, int S,
                                 int E, int C, int N, int dtype, void* stream) {
+  return run_combine(y, idx, pos, gate, kept, nullptr, out, G, S, E, C, N,
+                     dtype, stream);
+}
+
+extern "C" int mesh_moe_combine_compact(const void* y, const int32_t* idx,
+                                        const int32_t* pos, const float* gate,
+                                        const uint8_t* kept,
+                                        const int32_t* row_offsets, void* out,
+                                        int G, int S, int E, int C, int N,
+                                        int dtype, void* stream) {
+  MOE_REQUIRE(row_offsets, MESH_MOE_E_ARG, "combine_compact: null pointer");
+  return run_combine(y, idx, pos, gate, kept, row_offsets, out, G, S, E, C, N,
+                     dtype, stream);
+}
+
+static int run_combine(const void* y, const int32_t* idx, const int32_t* pos,
+                       const float* gate, const uint8_t* kept,
+                       const int32_t* row_offsets, void* out, int G, int S,
+                       int E, int C, int N, int dtype, void* stream) {
   MOE_REQUIRE(y && idx && pos && gate && kept && out, MESH_MOE_E_ARG,
               "combine: null pointer");
   MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG, "combine: bad dtype %d",
@@ -279,11 +309,11 @@ extern "C" int mesh_moe_combine(const void* y, const int32_t* idx,
   if (dtype == MESH_MOE_F32) {
     combine_kernel<float><<<(unsigned)nblocks, 256, 0, st>>>(
         (const float*)y, idx, pos, gate, kept, (float*)out, G, S, E, C, N,
-        T_tokens, vec);
+        T_tokens, vec, row_offsets);
   } else {
     combine_kernel<bf16_t><<<(unsigned)nblocks, 256, 0, st>>>(
         (const bf16_t*)y, idx, pos, gate, kept, (bf16_t*)out, G, S, E, C, N,
-        T_tokens, vec);
+        T_tokens, vec, row_offsets);
   }
   MOE_CHECK_LAUNCH("combine");
   return 0;

@@ -552,14 +552,20 @@ struct RingCfg {
 // MASKED: element (e, r, n) of the result is stored as zero unless
 // mask_src[e][r][n] > 0 (the backward of a ReLU whose output is mask_src,
 // applied while the tile is written out).
+//
+// LISTED: only the tiles named in tile_list[0 .. tile_list[-1]) are computed
+// (logical tile numbers in ascending order, their count in the element before
+// the list): an expert whose occupied rows were moved to the front of its row
+// range needs no tiles for the rest (see mesh_moe_compact_expert_ffn).
 template <bool RELU, bool GATHER = false, bool KMAJOR = false,
-          bool MASKED = false>
+          bool MASKED = false, bool LISTED = false>
 __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
     bf16_t* __restrict__ Cout, int R, int N, int K, int tiles_m, int tiles_n,
     int total_tiles, const int32_t* __restrict__ row_map = nullptr,
     const bf16_t* __restrict__ zero_row = nullptr,
-    const bf16_t* __restrict__ mask_src = nullptr) {
+    const bf16_t* __restrict__ mask_src = nullptr,
+    const int32_t* __restrict__ tile_list = nullptr) {
   using Cfg = RingCfg;
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, WN = Cfg::WN;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -570,6 +576,7 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
   // logical tiles and its blocks take them round-robin, which keeps the tiles
   // resident on an XCD at any moment consecutive (shared panels in its L2).
   const int nblk = gridDim.x;
+  if constexpr (LISTED) total_tiles = tile_list[-1];
   int tile, tile_end, tile_step;
   if ((nblk & 7) == 0) {
     const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
@@ -599,6 +606,7 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
   typename std::conditional<GATHER, int64_t, int>::type a_off[Cfg::A_INSTR];
   int b_off[Cfg::B_INSTR];
   auto set_tile = [&](int logical) {
+    if constexpr (LISTED) logical = tile_list[logical];
     const int e = logical / tiles_per_e;
     const int rem = logical - e * tiles_per_e;
     const int tn = rem / tiles_m;
@@ -1322,7 +1330,7 @@ static int launch_ring_kmajor(const bf16_t* A, const bf16_t* B, bf16_t* C,
   MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
   k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
       A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr,
-        nullptr);
+        nullptr, nullptr);
   MOE_CHECK_LAUNCH("expert_ffn_backward (mfma, K-major operands)");
   return 0;
 }
@@ -1331,7 +1339,8 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
                        int R, int N, int K, bool relu, hipStream_t st,
                        const int32_t* row_map = nullptr,
                        const bf16_t* zero_row = nullptr,
-                       const bf16_t* mask_src = nullptr) {
+                       const bf16_t* mask_src = nullptr,
+                       const int32_t* tile_list = nullptr) {
   using Cfg = RingCfg;
   const int tiles_m = (R + Cfg::BM - 1) / Cfg::BM;
   const int tiles_n = (N + Cfg::BN - 1) / Cfg::BN;
@@ -1341,6 +1350,29 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
   const int cus = compute_units();
   if (cus == 0) return MESH_MOE_E_HIP;
   const unsigned blocks = (unsigned)(tiles < cus ? tiles : cus);
+  if (tile_list != nullptr) {
+    // listed tiles: the first GEMM gathers its rows, the second does not
+    MOE_REQUIRE(mask_src == nullptr, MESH_MOE_E_ARG,
+                "expert_ffn: tile list with a masked result");
+#define MOE_RING_LISTED(RELU_, GATHER_)                                        \
+  do {                                                                         \
+    auto k = grouped_gemm_bf16_ring_kernel<RELU_, GATHER_, false, false, true>; \
+    MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);                                          \
+    k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(                           \
+        A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, row_map, zero_row,     \
+        nullptr, tile_list);                                                   \
+  } while (0)
+    if (row_map != nullptr) {
+      if (relu) MOE_RING_LISTED(true, true);
+      else MOE_RING_LISTED(false, true);
+    } else {
+      if (relu) MOE_RING_LISTED(true, false);
+      else MOE_RING_LISTED(false, false);
+    }
+#undef MOE_RING_LISTED
+    MOE_CHECK_LAUNCH("expert_ffn (mfma, listed tiles)");
+    return 0;
+  }
   if (mask_src != nullptr) {
     MOE_REQUIRE(!relu && row_map == nullptr, MESH_MOE_E_ARG,
                 "expert_ffn: masked result with relu or gathered rows");
@@ -1348,7 +1380,7 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
     MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
     k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
         A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr,
-        mask_src);
+        mask_src, nullptr);
     MOE_CHECK_LAUNCH("expert_ffn (mfma, masked result)");
     return 0;
   }
@@ -1358,13 +1390,13 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
       MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
       k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
           A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, row_map, zero_row,
-          nullptr);
+          nullptr, nullptr);
     } else {
       auto k = grouped_gemm_bf16_ring_kernel<false, true>;
       MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
       k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
           A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, row_map, zero_row,
-          nullptr);
+          nullptr, nullptr);
     }
     MOE_CHECK_LAUNCH("expert_ffn (mfma, gathered rows)");
     return 0;
@@ -1374,13 +1406,13 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
     MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
     k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
         A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr,
-        nullptr);
+        nullptr, nullptr);
   } else {
     auto k = grouped_gemm_bf16_ring_kernel<false, false>;
     MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
     k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
         A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr,
-        nullptr);
+        nullptr, nullptr);
   }
   MOE_CHECK_LAUNCH("expert_ffn (mfma, spread direct-to-LDS loads)");
   return 0;
@@ -1579,6 +1611,83 @@ __global__ void slot_map_kernel(const int32_t* __restrict__ idx,
   map[(int64_t)idx[i] * rows_per_expert + g * C + pos[i]] = (int32_t)t;
 }
 
+// ---------------------------------------------------------------------------
+// Compacted rows: expert e's occupied slots, groups in order, slots in order,
+// become rows 0 .. rows_used[e] - 1 of its row range.
+// row_offsets[e][g] = sum over g' < g of fill[g'][e]; one block per expert.
+// ---------------------------------------------------------------------------
+__global__ __launch_bounds__(256) void row_offsets_kernel(
+    const int32_t* __restrict__ fill, int32_t* __restrict__ row_offsets,
+    int32_t* __restrict__ rows_used, int G, int E) {
+  __shared__ int32_t part[256];
+  const int e = blockIdx.x, tid = threadIdx.x;
+  const int per = (G + 255) / 256;
+  const int g0 = min(G, tid * per), g1 = min(G, g0 + per);
+  int sum = 0;
+  for (int g = g0; g < g1; ++g) sum += fill[(int64_t)g * E + e];
+  part[tid] = sum;
+  __syncthreads();
+  if (tid == 0) {
+    int run = 0;
+    for (int i = 0; i < 256; ++i) {
+      const int v = part[i];
+      part[i] = run;
+      run += v;
+    }
+    rows_used[e] = run;
+  }
+  __syncthreads();
+  int run = part[tid];
+  for (int g = g0; g < g1; ++g) {
+    row_offsets[(int64_t)e * G + g] = run;
+    run += fill[(int64_t)g * E + e];
+  }
+}
+
+// One thread per (token, choice), as slot_map_kernel, onto the compacted rows.
+__global__ void slot_map_compact_kernel(const int32_t* __restrict__ idx,
+                                        const int32_t* __restrict__ pos,
+                                        const float* __restrict__ gate,
+                                        const uint8_t* __restrict__ kept,
+                                        const int32_t* __restrict__ row_offsets,
+                                        int32_t* __restrict__ map,
+                                        int64_t tokens, int S, int G,
+                                        int64_t rows_per_expert) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= tokens * 2) return;
+  if (!kept[i] || round_to<bf16_t>(gate[i]) == 0.0f) return;
+  const int64_t t = i >> 1;
+  const int64_t g = t / S;
+  const int e = idx[i];
+  map[(int64_t)e * rows_per_expert + row_offsets[(int64_t)e * G + g] + pos[i]] =
+      (int32_t)t;
+}
+
+// The tiles that hold occupied rows, in the order of the full tile numbering
+// ((expert, N tile, M tile), M tile fastest): list[-1] = their number.  One
+// block; E <= 1024.
+__global__ __launch_bounds__(1024) void tile_list_kernel(
+    const int32_t* __restrict__ rows_used, int32_t* __restrict__ list, int E,
+    int tiles_m, int tiles_n, int bm) {
+  __shared__ int32_t mt[1024], pre[1025];
+  const int tid = threadIdx.x;
+  if (tid < E) mt[tid] = min(tiles_m, (rows_used[tid] + bm - 1) / bm);
+  __syncthreads();
+  if (tid == 0) {
+    int run = 0;
+    for (int e = 0; e < E; ++e) { pre[e] = run; run += mt[e]; }
+    pre[E] = run;
+    list[-1] = run * tiles_n;
+  }
+  __syncthreads();
+  const int total = E * tiles_n * tiles_m;
+  for (int i = tid; i < total; i += blockDim.x) {
+    const int tm = i % tiles_m, rest = i / tiles_m;
+    const int tn = rest % tiles_n, e = rest / tiles_n;
+    if (tm < mt[e]) list[tiles_n * pre[e] + tn * mt[e] + tm] = i;
+  }
+}
+
 static bool ring_path_applies(int R, int N, int K) {
   const int pad256 = (R + 255) / 256 * 256, pad128 = (R + 127) / 128 * 128;
   return N >= 256 && R >= 128 && K % 64 == 0 && K % 8 == 0 && N % 8 == 0 &&
@@ -1645,6 +1754,97 @@ extern "C" int mesh_moe_dispatched_expert_ffn(
   }
   return grouped_gemm(h, wo_packed, y, E, R, N, H, MESH_MOE_ACT_LINEAR, dtype,
                       st);
+}
+
+static size_t compact_ffn_tiles(int E, int R, int H, int N) {
+  const size_t tm = (size_t)(R + RingCfg::BM - 1) / RingCfg::BM;
+  return (size_t)E * tm * ((size_t)(H + RingCfg::BN - 1) / RingCfg::BN +
+                           (size_t)(N + RingCfg::BN - 1) / RingCfg::BN);
+}
+
+extern "C" size_t mesh_moe_compact_expert_ffn_workspace_bytes(int G, int E,
+                                                              int C, int M,
+                                                              int H, int N) {
+  if (G < 1 || E < 1 || C < 1 || M < 1 || H < 1 || N < 1) return 0;
+  const int64_t rows = (int64_t)G * C;
+  if (rows > 0x7fffffffLL) return 0;
+  return sizeof(int32_t) * ((size_t)E * rows + (size_t)E +
+                            compact_ffn_tiles(E, (int)rows, H, N) + 2 * 64) +
+         sizeof(bf16_t) * (size_t)M + 6 * 256;
+}
+
+extern "C" int mesh_moe_compact_expert_ffn(
+    const void* x, const int32_t* idx, const int32_t* pos, const float* gate,
+    const uint8_t* kept, const int32_t* fill, const void* wi_packed,
+    const void* wo_packed, void* h, void* y, int32_t* row_offsets,
+    void* workspace, size_t workspace_bytes, int G, int S, int E, int C, int M,
+    int H, int N, int activation, int dtype, void* stream) {
+  MOE_REQUIRE(x && idx && pos && gate && kept && fill && wi_packed &&
+                  wo_packed && h && y && row_offsets && workspace,
+              MESH_MOE_E_ARG, "compact_expert_ffn: null pointer");
+  MOE_REQUIRE(G >= 1 && S >= 1 && E >= 1 && C >= 1 && M >= 1 && H >= 1 && N >= 1,
+              MESH_MOE_E_ARG, "compact_expert_ffn: bad sizes");
+  MOE_REQUIRE(activation >= MESH_MOE_ACT_LINEAR &&
+                  activation <= MESH_MOE_ACT_SWISH,
+              MESH_MOE_E_ARG, "compact_expert_ffn: unknown activation %d",
+              activation);
+  const int64_t rows = (int64_t)G * C;
+  MOE_REQUIRE(dtype == MESH_MOE_BF16 && rows <= 0x7fffffffLL && E <= 1024 &&
+                  (int64_t)G * S <= 0x7fffffffLL &&
+                  ring_path_applies((int)rows, H, M) &&
+                  ring_path_applies((int)rows, N, H) &&
+                  (((uintptr_t)x | (uintptr_t)wi_packed | (uintptr_t)wo_packed |
+                    (uintptr_t)h | (uintptr_t)y) % 16 == 0),
+              MESH_MOE_E_UNSUPPORTED,
+              "compact_expert_ffn: needs bf16, at most 1024 experts and GEMMs "
+              "the 256 x 256 direct-to-LDS kernel takes (rows=%lld M=%d H=%d "
+              "N=%d)", (long long)rows, M, H, N);
+  MOE_REQUIRE(workspace_bytes >= mesh_moe_compact_expert_ffn_workspace_bytes(
+                                     G, E, C, M, H, N),
+              MESH_MOE_E_ARG, "compact_expert_ffn: workspace too small");
+  hipStream_t st = (hipStream_t)stream;
+  const int R = (int)rows;
+  auto up = [](uintptr_t q) { return (q + 255) & ~(uintptr_t)255; };
+  int32_t* map = (int32_t*)up((uintptr_t)workspace);
+  int32_t* rows_used = (int32_t*)up((uintptr_t)(map + (size_t)E * R));
+  const int tiles_m = (R + RingCfg::BM - 1) / RingCfg::BM;
+  const int tn1 = (H + RingCfg::BN - 1) / RingCfg::BN;
+  const int tn2 = (N + RingCfg::BN - 1) / RingCfg::BN;
+  // each list is preceded by its length (and padding up to 256 bytes)
+  int32_t* list1 = (int32_t*)up((uintptr_t)(rows_used + E)) + 64;
+  int32_t* list2 = (int32_t*)up((uintptr_t)(list1 + (size_t)E * tiles_m * tn1)) + 64;
+  bf16_t* zero_row = (bf16_t*)up((uintptr_t)(list2 + (size_t)E * tiles_m * tn2));
+  row_offsets_kernel<<<E, 256, 0, st>>>(fill, row_offsets, rows_used, G, E);
+  MOE_CHECK_LAUNCH("compact_expert_ffn (row offsets)");
+  const int64_t n_map = (int64_t)E * R;
+  const unsigned cb = (unsigned)((n_map + 255) / 256 < 4096 ? (n_map + 255) / 256
+                                                            : 4096);
+  slot_map_clear_kernel<<<cb, 256, 0, st>>>(map, n_map, zero_row, M);
+  MOE_CHECK_LAUNCH("compact_expert_ffn (clear)");
+  const int64_t pairs = (int64_t)G * S * 2;
+  slot_map_compact_kernel<<<(unsigned)((pairs + 255) / 256), 256, 0, st>>>(
+      idx, pos, gate, kept, row_offsets, map, (int64_t)G * S, S, G, rows);
+  MOE_CHECK_LAUNCH("compact_expert_ffn (slot map)");
+  tile_list_kernel<<<1, 1024, 0, st>>>(rows_used, list1, E, tiles_m, tn1,
+                                       RingCfg::BM);
+  MOE_CHECK_LAUNCH("compact_expert_ffn (tile list 1)");
+  tile_list_kernel<<<1, 1024, 0, st>>>(rows_used, list2, E, tiles_m, tn2,
+                                       RingCfg::BM);
+  MOE_CHECK_LAUNCH("compact_expert_ffn (tile list 2)");
+  const bool relu = activation == MESH_MOE_ACT_RELU;
+  int rc = launch_ring((const bf16_t*)x, (const bf16_t*)wi_packed, (bf16_t*)h,
+                       E, R, H, M, relu, st, map, zero_row, nullptr, list1);
+  if (rc != 0) return rc;
+  if (!relu && activation != MESH_MOE_ACT_LINEAR) {
+    // (the pass also runs over the rows no listed tile wrote: they hold
+    // unspecified values before and after, and nothing reads them)
+    const int64_t n = (int64_t)E * R * H;
+    const int blocks = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
+    activation_kernel<bf16_t><<<blocks, 256, 0, st>>>((bf16_t*)h, n, activation);
+    MOE_CHECK_LAUNCH("compact_expert_ffn (activation)");
+  }
+  return launch_ring((const bf16_t*)h, (const bf16_t*)wo_packed, (bf16_t*)y, E,
+                     R, N, H, false, st, nullptr, nullptr, nullptr, list2);
 }
 
 extern "C" int mesh_moe_expert_linear(const void* a, const void* w_packed,

@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 17
+ABI_VERSION = 18
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -81,6 +81,17 @@ _SIGNATURES = {
     "mesh_moe_dispatched_expert_ffn": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_size_t,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
+    "mesh_moe_compact_expert_ffn_workspace_bytes": (ctypes.c_size_t, [
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int]),
+    "mesh_moe_compact_expert_ffn": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
+        ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        _vp]),
+    "mesh_moe_combine_compact": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
     "mesh_moe_expert_linear": (ctypes.c_int, [
         _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
@@ -692,6 +703,41 @@ def dispatched_expert_ffn(x, r, wi_packed, wo_packed, activation="relu",
   return y
 
 
+def compact_expert_ffn(x, r, wi_packed, wo_packed, activation="relu"):
+  """dispatch + expert_ffn on compacted rows (only the tiles that hold
+  occupied slots are multiplied): x [G, S, M], the Routing r -> (y [E, G*C, N],
+  row_offsets [E, G]) for combine(..., row_offsets=...), or None where the
+  library has no such kernel for the case."""
+  lib = load_library()
+  if activation not in ACTIVATIONS:
+    raise ValueError("unsupported expert activation %r" % (activation,))
+  g, s, m = x.shape
+  e, c = r.num_experts, r.capacity
+  hdim, n = wi_packed.shape[1], wo_packed.shape[1]
+  dt = x.dtype
+  if dt != torch.bfloat16:
+    return None
+  dev = x.device
+  h = torch.empty((e, g * c, hdim), dtype=dt, device=dev)
+  y = torch.empty((e, g * c, n), dtype=dt, device=dev)
+  row_offsets = torch.empty((e, g), dtype=torch.int32, device=dev)
+  ws_bytes = lib.mesh_moe_compact_expert_ffn_workspace_bytes(g, e, c, m, hdim, n)
+  ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
+  with _stage("expert_ffn"):
+    rc = lib.mesh_moe_compact_expert_ffn(
+        _dev(x, "x"), _dev(r.idx, "idx", torch.int32, (g, s, 2)),
+        r.pos.data_ptr(), r.gate.data_ptr(), r.kept.data_ptr(),
+        _dev(r.fill, "fill", torch.int32, (g, e)),
+        _dev(wi_packed, "wi_packed", dt, (e, hdim, m)),
+        _dev(wo_packed, "wo_packed", dt, (e, n, hdim)), h.data_ptr(),
+        y.data_ptr(), row_offsets.data_ptr(), ws.data_ptr(), ws_bytes, g, s, e,
+        c, m, hdim, n, ACTIVATIONS[activation], dtype_code(dt), _stream())
+  if rc == E_UNSUPPORTED:
+    return None
+  _check(rc, "compact_expert_ffn")
+  return y, row_offsets
+
+
 def expert_linear(a, w_packed, activation="linear", y=None):
   """a [E, R, K]; w_packed [E, N, K] -> y [E, R, N] = act(a . w) per expert."""
   lib = load_library()
@@ -710,8 +756,9 @@ def expert_linear(a, w_packed, activation="linear", y=None):
   return y
 
 
-def combine(y, r, group_size, out=None):
-  """y [E, G, C, N] -> out [G, S, N]."""
+def combine(y, r, group_size, out=None, row_offsets=None):
+  """y [E, G, C, N] -> out [G, S, N].  With row_offsets [E, G] (from
+  compact_expert_ffn) y holds every expert's occupied slots first."""
   lib = load_library()
   e, g, c, n = y.shape
   s = group_size
@@ -723,6 +770,16 @@ def combine(y, r, group_size, out=None):
   if out is None:
     out = torch.empty((g, s, n), dtype=y.dtype, device=y.device)
   op = _dev(out, "out", y.dtype, (g, s, n))
+  if row_offsets is not None:
+    with _stage("combine"):
+      _check(lib.mesh_moe_combine_compact(
+          yp, _dev(r.idx, "idx", torch.int32, (g, s, 2)),
+          _dev(r.pos, "pos", torch.int32, (g, s, 2)),
+          _dev(r.gate, "gate", torch.float32, (g, s, 2)),
+          _dev(r.kept, "kept", torch.uint8, (g, s, 2)),
+          _dev(row_offsets, "row_offsets", torch.int32, (e, g)), op, g, s, e, c,
+          n, code, _stream()), "combine_compact")
+    return out
   with _stage("combine"):
     _check(lib.mesh_moe_combine(
         yp, _dev(r.idx, "idx", torch.int32, (g, s, 2)),

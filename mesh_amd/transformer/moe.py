@@ -466,10 +466,21 @@ class MoEV1Operation(mtf.Operation):
       by_slot = isinstance(r, moe_hip.SlotRouting)
       y = None
       noise = None
+      row_offsets = None
       if not (save or by_slot or kwo_p is not None) and plain_hidden:
         # nobody reads expert_in afterwards: fold the dispatch into the first
-        # expert GEMM where the library can
-        y = moe_hip.dispatched_expert_ffn(xg, r, wi_p, wo_p, self._activation)
+        # expert GEMM where the library can.  Routers with one choice per token
+        # leave about 1 - 1 / capacity_factor of the slots empty: their
+        # occupied slots are moved to the front of every expert's rows and
+        # only the tiles that hold them are multiplied
+        if self._gating.router != "top_2":
+          compact = moe_hip.compact_expert_ffn(xg, r, wi_p, wo_p,
+                                               self._activation)
+          if compact is not None:
+            y, row_offsets = compact
+        if y is None:
+          y = moe_hip.dispatched_expert_ffn(xg, r, wi_p, wo_p,
+                                            self._activation)
       if y is None:
         expert_in = (moe_hip.slot_dispatch(xg, r) if by_slot
                      else moe_hip.dispatch(xg, r))
@@ -505,7 +516,7 @@ class MoEV1Operation(mtf.Operation):
         y = moe_hip.expert_linear(h, wo_p)
       y4 = y.reshape(e_, groups, c_, n_)
       out = (moe_hip.slot_combine(y4, r, s_) if by_slot
-             else moe_hip.combine(y4, r, s_))
+             else moe_hip.combine(y4, r, s_, row_offsets=row_offsets))
       if save:
         # what the gradient operation reads (activations of this step)
         gate_noise = getattr(self._gating, "noise", None)

@@ -792,6 +792,51 @@ def test_dispatched_expert_ffn_equals_two_calls(hip, shape):
     assert hip.dispatched_expert_ffn(x, r2, wi_p, wo_p, "relu") is None
 
 
+@pytest.mark.parametrize("case", [
+    # G, S, E, C, M, H, N, router
+    (4, 512, 8, 128, 256, 512, 256, "switch"),
+    (8, 1024, 16, 128, 128, 256, 256, "switch"),
+    (4, 512, 8, 256, 256, 512, 256, "top_2"),
+    (32, 2048, 64, 64, 1024, 2048, 1024, "switch")],
+    ids=["small", "mid", "top2_record", "cfg4_routing"])
+def test_compact_expert_ffn_equals_two_calls(hip, case):
+  """mesh_moe_compact_expert_ffn + mesh_moe_combine_compact (occupied slots
+  first, only the tiles that hold them multiplied) give the same layer output,
+  bit for bit, as dispatch + expert FFN + combine on every slot: a slot's
+  result depends on its own row only, wherever the row sits."""
+  g, s, e, c, m, hdim, n, router = case
+  rng = np.random.default_rng(sum(case[:7]))
+  logits = torch.from_numpy(H.safe_logits(
+      rng, g, s, e, scale=1.5, bias=H.zipf_bias(rng, e, scale=1.0))).cuda()
+  x = H.to_gpu(rng.standard_normal((g, s, m)).astype(np.float32), "bfloat16")
+  wi_p = hip.pack_weights(H.to_gpu(H.normal_weights(rng, (e, m, hdim), m),
+                                   "bfloat16"), torch.bfloat16)
+  wo_p = hip.pack_weights(H.to_gpu(H.normal_weights(rng, (e, hdim, n), hdim),
+                                   "bfloat16"), torch.bfloat16)
+  r = (hip.switch_gating(logits, c) if router == "switch"
+       else hip.top2_gating(logits, c))
+  r.gate[0, 0, 0] = 0.0             # a kept choice with gate 0
+  fill = r.fill.long()
+  assert int((fill < c).sum()) > 0 and int(fill.sum()) < 0.8 * g * e * c
+  y_all = hip.expert_ffn(hip.dispatch(x, r).reshape(e, g * c, m), wi_p, wo_p,
+                         "relu")
+  want = hip.combine(y_all.reshape(e, g, c, n), r, s)
+  got = hip.compact_expert_ffn(x, r, wi_p, wo_p, "relu")
+  assert got is not None
+  y, row_offsets = got
+  # row_offsets[e][g] = occupied slots of expert e in earlier groups
+  want_off = (fill.t().cumsum(1) - fill.t()).to(torch.int32)
+  assert torch.equal(row_offsets, want_off)
+  out = hip.combine(y.reshape(e, g, c, n), r, s, row_offsets=row_offsets)
+  assert torch.equal(out, want)
+  # the occupied rows themselves, slot by slot
+  for ei in (0, e // 2, e - 1):
+    for gi in (0, g - 1):
+      k = int(fill[gi, ei])
+      o = int(row_offsets[ei, gi])
+      assert torch.equal(y[ei, o:o + k], y_all[ei, gi * c:gi * c + k])
+
+
 def test_dispatched_expert_ffn_equals_two_calls_cfg4(hip):
   """The same identity at the full size of benchmark configuration 4 (32 groups
   of 2048 tokens, 64 experts, capacity 64, d_model 4096, hidden 16384), where
