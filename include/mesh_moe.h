@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 18
+#define MESH_MOE_ABI_VERSION 19
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -740,6 +740,36 @@ int mesh_moe_self_attention(const void* q, const void* k, const void* v,
                             void* out, int B, int L, int H, int D, int causal,
                             int dtype, void* workspace, size_t workspace_bytes,
                             void* stream);
+
+/* Bytes of scratch mesh_moe_self_attention_backward needs; 0 for shapes it does
+ * not take. */
+size_t mesh_moe_self_attention_backward_workspace_bytes(int B, int L, int H,
+                                                        int D, int dtype);
+
+/*
+ * Backward of mesh_moe_self_attention in fused kernels: what mtf.gradients
+ * (mesh_tensorflow/ops.py:5254-5291) assembles from the gradients of the two
+ * einsums and the softmax of attention.attention
+ * (transformer/attention.py:76-87).  With W = softmax(q . k) cast to dtype:
+ *   dW = dout . v^T,  delta = sum_k dW W,  dS = W (dW - delta) cast to dtype,
+ *   dv = W^T . dout,  dq = dS . k,  dk = dS^T . q.
+ *   q, k, v, dout, dq, dk, dv [B,L,H*D] dtype.
+ * bf16 with D = 64 or 128 and L a multiple of 8 only (MESH_MOE_E_UNSUPPORTED
+ * otherwise: compose mesh_moe_attention_weights, mesh_moe_softmax_backward and
+ * mesh_moe_expert_linear_backward instead).  Nothing of size L x L reaches
+ * memory; the workspace holds two float32 [B*H, L] vectors.  Four launches:
+ * one pass in the forward kernel's shape for the softmax denominators and
+ * delta, then one kernel per output, each recomputing W per tile, so that
+ * every output element is summed by one wavefront in a fixed order (no
+ * atomics; the same bits on every run).  dW is not rounded to dtype before
+ * the subtraction and delta comes from sum_d dout out in float32 -- fewer
+ * roundings than the reference's chain of ops, inside its tolerance.
+ */
+int mesh_moe_self_attention_backward(const void* q, const void* k, const void* v,
+                                     const void* dout, void* dq, void* dk,
+                                     void* dv, int B, int L, int H, int D,
+                                     int causal, int dtype, void* workspace,
+                                     size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus
 }

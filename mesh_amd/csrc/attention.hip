@@ -101,10 +101,16 @@ __device__ __forceinline__ float fa_exp2(float x) {
   return __builtin_amdgcn_exp2f(x);
 }
 
-template <int D, bool CAUSAL>
+// STATS: instead of the outputs, write what the backward kernels need per
+// query: lse = log of the softmax denominator (row maximum included) and
+// delta = sum_d dout[q, d] * out[q, d] (= sum_k dweights * weights), both
+// float32 [B*H, L].
+template <int D, bool CAUSAL, bool STATS = false>
 __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
-    const bf16_t* __restrict__ v, bf16_t* __restrict__ out, int L, int H) {
+    const bf16_t* __restrict__ v, bf16_t* __restrict__ out, int L, int H,
+    const bf16_t* __restrict__ dout = nullptr, float* __restrict__ lse = nullptr,
+    float* __restrict__ delta = nullptr) {
   using Cfg = FlashCfg<D>;
   extern __shared__ __attribute__((aligned(16))) unsigned char fa_smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -311,6 +317,29 @@ __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
 
   const float l_all = l_part + __shfl_xor(l_part, 32);
   const float inv = 1.0f / l_all;
+  if constexpr (STATS) {
+    const bf16_t* drow = dout + ((int64_t)b * L + min(my_q, L - 1)) * row_stride +
+                         (int64_t)h * D;
+    float dsum = 0.f;
+#pragma unroll
+    for (int dt = 0; dt < Cfg::DT; ++dt) {
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        const int d = dt * 32 + 8 * a + 4 * half;
+        const uint2 g = *reinterpret_cast<const uint2*>(drow + d);
+        dsum += acc_o[dt][4 * a + 0] * __uint_as_float(g.x << 16) +
+                acc_o[dt][4 * a + 1] * __uint_as_float(g.x & 0xffff0000u) +
+                acc_o[dt][4 * a + 2] * __uint_as_float(g.y << 16) +
+                acc_o[dt][4 * a + 3] * __uint_as_float(g.y & 0xffff0000u);
+      }
+    }
+    dsum += __shfl_xor(dsum, 32);
+    if (my_q < L && half == 0) {
+      lse[(int64_t)bh * L + my_q] = m_run + logf(l_all);
+      delta[(int64_t)bh * L + my_q] = dsum * inv;
+    }
+    return;
+  }
   if (my_q < L) {
     bf16_t* orow = ob + (int64_t)my_q * row_stride;
 #pragma unroll
@@ -338,11 +367,13 @@ static int launch_flash(const bf16_t* q, const bf16_t* k, const bf16_t* v,
   if (causal) {
     auto kern = flash_attention_kernel<D, true>;
     MOE_ALLOW_LDS(kern, Cfg::LDS_BYTES);
-    kern<<<grid, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(q, k, v, out, L, H);
+    kern<<<grid, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(q, k, v, out, L, H, nullptr,
+                                                     nullptr, nullptr);
   } else {
     auto kern = flash_attention_kernel<D, false>;
     MOE_ALLOW_LDS(kern, Cfg::LDS_BYTES);
-    kern<<<grid, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(q, k, v, out, L, H);
+    kern<<<grid, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(q, k, v, out, L, H, nullptr,
+                                                     nullptr, nullptr);
   }
   MOE_CHECK_LAUNCH("self_attention (fused)");
   return 0;
@@ -371,6 +402,364 @@ int flash_attention(const void* q, const void* k, const void* v, void* out,
                              st);
   return launch_flash<64>((const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v,
                           (bf16_t*)out, B, L, H, causal, st);
+}
+
+// ---------------------------------------------------------------------------
+// Backward (the gradients of the two einsums and the softmax of
+// attention.attention, mesh_tensorflow/transformer/attention.py:76-87, which
+// mtf.gradients would assemble): with W = softmax(q . k) rounded to bf16,
+//   dW = dout . v^T,  dS = W * (dW - delta)  rounded to bf16,
+//   dv = W^T . dout,  dq = dS . k,  dk = dS^T . q.
+// Nothing [L, L] reaches memory: W is recomputed per tile from q, k and the
+// lse of the STATS pass, three times -- once per output, so that every output
+// element is accumulated by one wavefront in a fixed order (no atomics, the
+// same bits on every run):
+//   BWD_DQ  a lane owns a query;  walks key tiles:    S, dW, dS, dq^T += K^T dS
+//   BWD_DK  a lane owns a key;    walks query tiles:  S, dW, dS, dk^T += Q^T dS
+//   BWD_DV  a lane owns a key;    walks query tiles:  S, W,      dv^T += dout^T W
+// All three have the forward kernel's shape: "tile rows x own fragments" on
+// the matrix cores with the own entity as MFMA column (so masks, lse and delta
+// are per lane or per register), the bf16 result going from the accumulator
+// registers straight into the operand registers of the second product, whose
+// other operand is the streamed tile read through ds_read_b64_tr_b16.  A
+// streamed tile that is read both ways (K in BWD_DQ, Q in BWD_DK) is loaded
+// into LDS twice, once per swizzle.
+// ---------------------------------------------------------------------------
+enum { BWD_DQ = 0, BWD_DK = 1, BWD_DV = 2 };
+
+template <int D>
+struct FlashBwdCfg {
+  static constexpr int BT = 64;                     // streamed rows per tile
+  static constexpr int WAVES = 8, THREADS = 64 * WAVES, BOWN = 32 * WAVES;
+  static constexpr int ROW = D * 2;                 // bytes per row
+  static constexpr int TILE = BT * ROW;
+  static constexpr int CH = ROW / 16, UNITS = ROW / 64, RPI = 1024 / ROW;
+  static constexpr int INSTR = TILE / 1024 / WAVES; // loads per wave and tile copy
+  static constexpr int DS = D / 16, DT = D / 32;
+  static constexpr int STATS_BYTES = 2 * BT * 4;    // lse, delta of a query tile
+  static constexpr int stage_bytes(int what) {
+    return (what == BWD_DV ? 2 : 3) * TILE + STATS_BYTES;
+  }
+  static_assert(D == 64 || D == 128, "d_kv 64 or 128");
+  static_assert(INSTR >= 1, "a tile copy is at least one load per wavefront");
+};
+
+template <int D, bool CAUSAL, int WHAT>
+__global__ __launch_bounds__(512) void flash_attention_backward_kernel(
+    const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
+    const bf16_t* __restrict__ v, const bf16_t* __restrict__ dout,
+    const float* __restrict__ lse, const float* __restrict__ delta,
+    bf16_t* __restrict__ grad, int L, int H) {
+  using Cfg = FlashBwdCfg<D>;
+  constexpr bool OWN_Q = WHAT == BWD_DQ;
+  constexpr int NCOPY = WHAT == BWD_DV ? 2 : 3;
+  constexpr int STAGE = Cfg::stage_bytes(WHAT);
+  constexpr float LOG2E = 1.4426950408889634f;
+  extern __shared__ __attribute__((aligned(16))) unsigned char fb_smem[];
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, l32 = lane & 31;
+  const int n_own = (L + Cfg::BOWN - 1) / Cfg::BOWN;
+  // long tiles first: late queries, early keys
+  const int ot = OWN_Q && CAUSAL ? n_own - 1 - (int)blockIdx.x : (int)blockIdx.x;
+  const int own0 = ot * Cfg::BOWN;
+  const int bh = blockIdx.y, b = bh / H, h = bh % H;
+  const int64_t row_stride = (int64_t)H * D;
+  const int64_t head_off = ((int64_t)b * L) * row_stride + (int64_t)h * D;
+  // own rows supply the register fragments, streamed rows the LDS tiles
+  const bf16_t* own1 = (OWN_Q ? q : k) + head_off;
+  const bf16_t* own2 = (OWN_Q ? dout : v) + head_off;
+  const bf16_t* str1 = (OWN_Q ? k : q) + head_off;
+  const bf16_t* str2 = (OWN_Q ? v : dout) + head_off;
+  const float* lse_b = lse + (int64_t)bh * L;
+  const float* delta_b = delta + (int64_t)bh * L;
+
+  const int nt_all = (L + Cfg::BT - 1) / Cfg::BT;
+  int t_begin = 0, t_end = nt_all;
+  if (CAUSAL) {
+    if (OWN_Q) t_end = min(nt_all, (own0 + Cfg::BOWN - 1) / Cfg::BT + 1);
+    else t_begin = own0 / Cfg::BT;
+  }
+
+  const int my = own0 + wave * 32 + l32;
+  const int my_c = min(my, L - 1);
+  fa_bf16x8_t f1[Cfg::DS], f2[WHAT == BWD_DV ? 1 : Cfg::DS];
+  {
+    const bf16_t* r1 = own1 + (int64_t)my_c * row_stride + half * 8;
+    const bf16_t* r2 = own2 + (int64_t)my_c * row_stride + half * 8;
+#pragma unroll
+    for (int s = 0; s < Cfg::DS; ++s) {
+      f1[s] = *reinterpret_cast<const fa_bf16x8_t*>(r1 + s * 16);
+      if constexpr (WHAT != BWD_DV)
+        f2[s] = *reinterpret_cast<const fa_bf16x8_t*>(r2 + s * 16);
+    }
+  }
+  float my_lse2 = 0.f, my_delta = 0.f;
+  if constexpr (OWN_Q) {
+    my_lse2 = lse_b[my_c] * LOG2E;
+    my_delta = delta_b[my_c];
+  }
+
+  // one tile copy: rows of `src` from row0, chunk-swizzled for row reads
+  // (TR = false) or unit-swizzled for transposing reads (TR = true)
+  auto load_copy = [&](const bf16_t* src, int row0, unsigned char* dst,
+                       auto tr_c) {
+    constexpr bool TR = decltype(tr_c)::value;
+#pragma unroll
+    for (int j = 0; j < Cfg::INSTR; ++j) {
+      const int g = wave * Cfg::INSTR + j;
+      const int row = g * Cfg::RPI + lane / Cfg::CH;
+      const int p = lane % Cfg::CH;
+      const int c = TR ? ((((p >> 2) ^ fa_vswz<Cfg::UNITS>(row)) << 2) | (p & 3))
+                       : (p ^ fa_kswz<Cfg::CH>(row));
+      const bf16_t* a = src + (int64_t)min(row0 + row, L - 1) * row_stride + c * 8;
+      __builtin_amdgcn_global_load_lds((fa_glb_void_t*)a,
+                                       (fa_lds_void_t*)(dst + g * 1024), 16, 0, 0);
+    }
+  };
+  auto load_tile = [&](int t, int buf) {
+    const int row0 = t * Cfg::BT;
+    unsigned char* base = fb_smem + buf * STAGE;
+    load_copy(str1, row0, base, std::false_type());
+    if constexpr (WHAT == BWD_DV) {
+      load_copy(str2, row0, base + Cfg::TILE, std::true_type());
+    } else {
+      load_copy(str1, row0, base + Cfg::TILE, std::true_type());
+      load_copy(str2, row0, base + 2 * Cfg::TILE, std::false_type());
+    }
+    if constexpr (!OWN_Q) {
+      // lse and delta of the tile's queries: one 4-byte load per lane
+      if (wave < 2) {
+        const float* a = (wave == 0 ? lse_b : delta_b) + min(row0 + lane, L - 1);
+        __builtin_amdgcn_global_load_lds(
+            (fa_glb_void_t*)a,
+            (fa_lds_void_t*)(base + NCOPY * Cfg::TILE + wave * 256), 4, 0, 0);
+      }
+    }
+  };
+
+  fa_f32x16_t acc[Cfg::DT];
+#pragma unroll
+  for (int dt = 0; dt < Cfg::DT; ++dt)
+#pragma unroll
+    for (int r = 0; r < 16; ++r) acc[dt][r] = 0.f;
+
+  if (t_begin < t_end) load_tile(t_begin, 0);
+  __builtin_amdgcn_s_waitcnt(0x0070 | (15 << 8));   // vmcnt(0)
+  __syncthreads();
+
+  const int ow_first = own0 + wave * 32, ow_last = ow_first + 31;
+  const uint32_t lds0 = (uint32_t)(size_t)(fa_lds_void_t*)fb_smem;
+  const int t16 = lane & 15, g16 = lane >> 4;
+  const int krow = 4 * (g16 >> 1) + (t16 >> 2);
+  const int dcol = (g16 & 1) * 16 + 4 * (t16 & 3);
+  const int tsw = fa_vswz<Cfg::UNITS>(krow);
+  uint32_t toff[Cfg::DT];     // byte offset of this lane's transposing reads
+#pragma unroll
+  for (int dt = 0; dt < Cfg::DT; ++dt) {
+    const int col = dt * 32 + dcol;
+    toff[dt] = krow * Cfg::ROW + (((col >> 5) ^ tsw) << 6) + (col & 31) * 2;
+  }
+
+  for (int t = t_begin; t < t_end; ++t) {
+    const int buf = (t - t_begin) & 1;
+    if (t + 1 < t_end) load_tile(t + 1, buf ^ 1);
+    const int row0 = t * Cfg::BT;
+    const unsigned char* t1r = fb_smem + buf * STAGE;
+    const unsigned char* t2r = t1r + 2 * Cfg::TILE;           // BWD_DQ, BWD_DK
+    const uint32_t ttr = lds0 + buf * STAGE + Cfg::TILE;      // the copy read transposed
+    const float* st = reinterpret_cast<const float*>(t1r + NCOPY * Cfg::TILE);
+    const bool need_mask =
+        (CAUSAL && (OWN_Q ? row0 + Cfg::BT - 1 > ow_first : row0 < ow_last)) ||
+        row0 + Cfg::BT > L;
+
+    auto do_sub = [&](auto sub_c) {
+      constexpr int SUB = decltype(sub_c)::value;
+      fa_f32x16_t acc_s, acc_dp;
+#pragma unroll
+      for (int r = 0; r < 16; ++r) { acc_s[r] = 0.f; acc_dp[r] = 0.f; }
+      const int row = SUB * 32 + l32;
+      const int sw = fa_kswz<Cfg::CH>(row);
+      {
+        const unsigned char* rr = t1r + row * Cfg::ROW;
+#pragma unroll
+        for (int s = 0; s < Cfg::DS; ++s) {
+          const fa_bf16x8_t a = *reinterpret_cast<const fa_bf16x8_t*>(
+              rr + (((2 * s + half) ^ sw) * 16));
+          acc_s = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, f1[s], acc_s, 0, 0, 0);
+        }
+      }
+      if constexpr (WHAT != BWD_DV) {
+        const unsigned char* rr = t2r + row * Cfg::ROW;
+#pragma unroll
+        for (int s = 0; s < Cfg::DS; ++s) {
+          const fa_bf16x8_t a = *reinterpret_cast<const fa_bf16x8_t*>(
+              rr + (((2 * s + half) ^ sw) * 16));
+          acc_dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, f2[s], acc_dp, 0, 0, 0);
+        }
+      }
+      // weights (and their gradient) of this lane's own entity against the
+      // 16 streamed rows SUB * 32 + 8 (r / 4) + 4 half + r % 4
+      float w[16];
+      if constexpr (OWN_Q) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const float p = fa_exp2(fmaf(acc_s[r], LOG2E, -my_lse2));
+          w[r] = p * (acc_dp[r] - my_delta);
+        }
+      } else {
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4) {
+          const int j = SUB * 32 + 8 * r4 + 4 * half;
+          const float4 l4 = *reinterpret_cast<const float4*>(st + j);
+          const float lv[4] = {l4.x, l4.y, l4.z, l4.w};
+          float dv4[4] = {0.f, 0.f, 0.f, 0.f};
+          if constexpr (WHAT == BWD_DK) {
+            const float4 d4 = *reinterpret_cast<const float4*>(st + Cfg::BT + j);
+            dv4[0] = d4.x; dv4[1] = d4.y; dv4[2] = d4.z; dv4[3] = d4.w;
+          }
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            const int r = 4 * r4 + c;
+            const float p = fa_exp2(fmaf(acc_s[r], LOG2E, -lv[c] * LOG2E));
+            w[r] = WHAT == BWD_DV ? p : p * (acc_dp[r] - dv4[c]);
+          }
+        }
+      }
+      if (need_mask) {
+        asm volatile("" ::: "memory");
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int sr = row0 + SUB * 32 + 8 * (r / 4) + 4 * half + (r % 4);
+          const bool ok = sr < L && (!CAUSAL || (OWN_Q ? sr <= my : my <= sr));
+          if (!ok) w[r] = 0.f;
+        }
+      }
+      fa_bf16x8_t wf[2];
+#pragma unroll
+      for (int uu = 0; uu < 2; ++uu) {
+        uint32_t pk[4];
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+          pk[c] = f32x2_to_bf16x2(w[8 * uu + 2 * c], w[8 * uu + 2 * c + 1]);
+        fa_u32x4_t packed = {pk[0], pk[1], pk[2], pk[3]};
+        wf[uu] = __builtin_bit_cast(fa_bf16x8_t, packed);
+      }
+      // acc^T += (streamed tile)^T . w over the 32 streamed rows of this SUB:
+      // MFMA step uu covers rows SUB * 32 + 16 uu + {0-3, 8-11} (+ 4 for the
+      // upper half-wave), two transposing reads each
+      fa_i16x4_t lo[2][2], hi[2][2];
+      auto read_t = [&](int dt, int slot) {
+        const uint32_t a = ttr + toff[dt];
+        lo[slot][0] = fa_lds_read_tr16<(SUB * 32 + 0) * Cfg::ROW>(a);
+        hi[slot][0] = fa_lds_read_tr16<(SUB * 32 + 8) * Cfg::ROW>(a);
+        lo[slot][1] = fa_lds_read_tr16<(SUB * 32 + 16) * Cfg::ROW>(a);
+        hi[slot][1] = fa_lds_read_tr16<(SUB * 32 + 24) * Cfg::ROW>(a);
+      };
+      read_t(0, 0);
+#pragma unroll
+      for (int dt = 0; dt < Cfg::DT; ++dt) {
+        const int cur = dt & 1;
+        __builtin_amdgcn_sched_barrier(0);
+        __builtin_amdgcn_s_waitcnt(0xc07f);        // lgkmcnt(0)
+        __builtin_amdgcn_sched_barrier(0);
+        if (dt + 1 < Cfg::DT) read_t(dt + 1, cur ^ 1);
+#pragma unroll
+        for (int uu = 0; uu < 2; ++uu) {
+          const fa_bf16x8_t tf = __builtin_bit_cast(
+              fa_bf16x8_t, __builtin_shufflevector(lo[cur][uu], hi[cur][uu], 0, 1,
+                                                   2, 3, 4, 5, 6, 7));
+          acc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(tf, wf[uu], acc[dt], 0,
+                                                            0, 0);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+      }
+    };
+    do_sub(std::integral_constant<int, 0>());
+    do_sub(std::integral_constant<int, 1>());
+
+    __builtin_amdgcn_s_waitcnt(0x0070 | (15 << 8));   // vmcnt(0): tile t+1 is here
+    __syncthreads();
+  }
+
+  if (my < L) {
+    bf16_t* orow = grad + head_off + (int64_t)my * row_stride;
+#pragma unroll
+    for (int dt = 0; dt < Cfg::DT; ++dt) {
+#pragma unroll
+      for (int a = 0; a < 4; ++a) {
+        const int d = dt * 32 + 8 * a + 4 * half;
+        uint2 o;
+        o.x = f32x2_to_bf16x2(acc[dt][4 * a + 0], acc[dt][4 * a + 1]);
+        o.y = f32x2_to_bf16x2(acc[dt][4 * a + 2], acc[dt][4 * a + 3]);
+        *reinterpret_cast<uint2*>(orow + d) = o;
+      }
+    }
+  }
+}
+
+template <int D, bool CAUSAL, int WHAT>
+static int launch_flash_backward_one(const bf16_t* q, const bf16_t* k,
+                                     const bf16_t* v, const bf16_t* dout,
+                                     const float* lse, const float* delta,
+                                     bf16_t* grad, int B, int L, int H,
+                                     hipStream_t st) {
+  using Cfg = FlashBwdCfg<D>;
+  constexpr int LDS = 2 * Cfg::stage_bytes(WHAT);
+  dim3 grid((unsigned)((L + Cfg::BOWN - 1) / Cfg::BOWN), (unsigned)(B * H));
+  auto kern = flash_attention_backward_kernel<D, CAUSAL, WHAT>;
+  MOE_ALLOW_LDS(kern, LDS);
+  kern<<<grid, Cfg::THREADS, LDS, st>>>(q, k, v, dout, lse, delta, grad, L, H);
+  MOE_CHECK_LAUNCH("self_attention_backward (fused)");
+  return 0;
+}
+
+template <int D, bool CAUSAL>
+static int launch_flash_backward(const bf16_t* q, const bf16_t* k,
+                                 const bf16_t* v, const bf16_t* dout,
+                                 bf16_t* dq, bf16_t* dk, bf16_t* dv, float* lse,
+                                 float* delta, int B, int L, int H,
+                                 hipStream_t st) {
+  using Cfg = FlashCfg<D>;
+  dim3 grid((unsigned)((L + Cfg::BQ - 1) / Cfg::BQ), (unsigned)(B * H));
+  auto stats = flash_attention_kernel<D, CAUSAL, true>;
+  MOE_ALLOW_LDS(stats, Cfg::LDS_BYTES);
+  stats<<<grid, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(q, k, v, nullptr, L, H, dout,
+                                                    lse, delta);
+  MOE_CHECK_LAUNCH("self_attention_backward (lse, delta)");
+  int rc = launch_flash_backward_one<D, CAUSAL, BWD_DV>(q, k, v, dout, lse, delta,
+                                                        dv, B, L, H, st);
+  if (rc != 0) return rc;
+  rc = launch_flash_backward_one<D, CAUSAL, BWD_DK>(q, k, v, dout, lse, delta, dk,
+                                                    B, L, H, st);
+  if (rc != 0) return rc;
+  return launch_flash_backward_one<D, CAUSAL, BWD_DQ>(q, k, v, dout, lse, delta,
+                                                      dq, B, L, H, st);
+}
+
+size_t flash_attention_backward_workspace_bytes(int B, int L, int H) {
+  return 2 * (((size_t)B * H * L * sizeof(float) + 255) & ~(size_t)255) + 256;
+}
+
+int flash_attention_backward(const void* q, const void* k, const void* v,
+                             const void* dout, void* dq, void* dk, void* dv,
+                             int B, int L, int H, int D, int causal,
+                             void* workspace, hipStream_t st) {
+  float* lse = (float*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+  float* delta = lse + ((((size_t)B * H * L * sizeof(float) + 255) &
+                         ~(size_t)255) / sizeof(float));
+  const bf16_t *q_ = (const bf16_t*)q, *k_ = (const bf16_t*)k,
+               *v_ = (const bf16_t*)v, *d_ = (const bf16_t*)dout;
+  bf16_t *dq_ = (bf16_t*)dq, *dk_ = (bf16_t*)dk, *dv_ = (bf16_t*)dv;
+  if (D == 128)
+    return causal ? launch_flash_backward<128, true>(q_, k_, v_, d_, dq_, dk_, dv_,
+                                                     lse, delta, B, L, H, st)
+                  : launch_flash_backward<128, false>(q_, k_, v_, d_, dq_, dk_,
+                                                      dv_, lse, delta, B, L, H,
+                                                      st);
+  return causal ? launch_flash_backward<64, true>(q_, k_, v_, d_, dq_, dk_, dv_,
+                                                  lse, delta, B, L, H, st)
+                : launch_flash_backward<64, false>(q_, k_, v_, d_, dq_, dk_, dv_,
+                                                   lse, delta, B, L, H, st);
 }
 
 }  // namespace mesh_moe

@@ -775,3 +775,39 @@ extern "C" int mesh_moe_self_attention(const void* q, const void* k,
                                (const bf16_t*)v, (bf16_t*)out, B, L, H, D,
                                causal ? 1 : 0, dtype, workspace, st);
 }
+
+extern "C" size_t mesh_moe_self_attention_backward_workspace_bytes(int B, int L,
+                                                                   int H, int D,
+                                                                   int dtype) {
+  if (B < 1 || L < 1 || H < 1 || D < 1 || !valid_dtype(dtype)) return 0;
+  if (!flash_attention_supported(L, H, D, dtype, nullptr, nullptr, nullptr,
+                                 nullptr))
+    return 0;
+  return flash_attention_backward_workspace_bytes(B, L, H);
+}
+
+extern "C" int mesh_moe_self_attention_backward(
+    const void* q, const void* k, const void* v, const void* dout, void* dq,
+    void* dk, void* dv, int B, int L, int H, int D, int causal, int dtype,
+    void* workspace, size_t workspace_bytes, void* stream) {
+  MOE_REQUIRE(q && k && v && dout && dq && dk && dv && workspace, MESH_MOE_E_ARG,
+              "self_attention_backward: null pointer");
+  MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG,
+              "self_attention_backward: bad dtype %d", dtype);
+  MOE_REQUIRE(B >= 1 && L >= 1 && H >= 1 && D >= 1, MESH_MOE_E_ARG,
+              "self_attention_backward: bad sizes B=%d L=%d H=%d D=%d", B, L, H,
+              D);
+  MOE_REQUIRE((int64_t)B * H <= 65535, MESH_MOE_E_UNSUPPORTED,
+              "self_attention_backward: batch * heads = %lld > 65535",
+              (long long)B * H);
+  MOE_REQUIRE(flash_attention_supported(L, H, D, dtype, q, k, v, dout) &&
+                  flash_attention_supported(L, H, D, dtype, dq, dk, dv, dout),
+              MESH_MOE_E_UNSUPPORTED,
+              "self_attention_backward: the fused kernels take bf16, d_kv 64 or "
+              "128, L a multiple of 8 and 16-byte aligned tensors (L=%d D=%d)",
+              L, D);
+  MOE_REQUIRE(workspace_bytes >= flash_attention_backward_workspace_bytes(B, L, H),
+              MESH_MOE_E_ARG, "self_attention_backward: workspace too small");
+  return flash_attention_backward(q, k, v, dout, dq, dk, dv, B, L, H, D,
+                                  causal ? 1 : 0, workspace, (hipStream_t)stream);
+}

@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 18
+ABI_VERSION = 19
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -183,6 +183,12 @@ _SIGNATURES = {
     "mesh_moe_self_attention": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
+    "mesh_moe_self_attention_backward_workspace_bytes": (ctypes.c_size_t, [
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "mesh_moe_self_attention_backward": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp,
+        ctypes.c_size_t, _vp]),
 }
 EXPORTS = sorted(_SIGNATURES)
 
@@ -1280,18 +1286,41 @@ def softmax_backward(weights, dweights):
   return out
 
 
-def self_attention_backward(q, k, v, dout, num_heads, causal):
+def self_attention_backward(q, k, v, dout, num_heads, causal, fused=None):
   """Backward of self_attention: q, k, v, dout [B, L, H*D] -> (dq, dk, dv).
-  The weights are recomputed ([B*H, L, L], which the forward kernel never
-  stores); every product runs on the grouped GEMM with one (batch, head) pair
-  per group:
+  Shapes the fused kernels take (bf16, d_kv 64 or 128, L a multiple of 8) run
+  mesh_moe_self_attention_backward: nothing [L, L] reaches memory.  Otherwise
+  (or with fused=False) the weights are recomputed ([B*H, L, L]) and every
+  product runs on the grouped GEMM with one (batch, head) pair per group:
     dweights = dout . v^T,  dv = weights^T . dout    (one linear backward)
     dlogits  = softmax backward
     dq = dlogits . k,       dk = dlogits^T . q
-  Heads move to the front and back with torch permutes."""
+  with heads moved to the front and back by torch permutes.  fused=True raises
+  for shapes the fused kernels do not take."""
   b, l, hd = q.shape
   h = num_heads
+  if hd % h:
+    raise MoeHipError("q channels %d not divisible by %d heads" % (hd, h))
   d = hd // h
+  if fused is None or fused:
+    lib = load_library()
+    code = dtype_code(q.dtype)
+    ws_bytes = lib.mesh_moe_self_attention_backward_workspace_bytes(b, l, h, d,
+                                                                    code)
+    if ws_bytes:
+      ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=q.device)
+      dq, dk, dv = (torch.empty_like(q) for _ in range(3))
+      with _stage("self_attention_backward"):
+        _check(lib.mesh_moe_self_attention_backward(
+            _dev(q, "q"), _dev(k, "k", q.dtype, (b, l, hd)),
+            _dev(v, "v", q.dtype, (b, l, hd)),
+            _dev(dout, "dout", q.dtype, (b, l, hd)), dq.data_ptr(),
+            dk.data_ptr(), dv.data_ptr(), b, l, h, d, int(bool(causal)), code,
+            ws.data_ptr(), ws_bytes, _stream()), "self_attention_backward")
+      return dq, dk, dv
+    if fused:
+      raise MoeHipError("self_attention_backward: the fused kernels do not take "
+                        "dtype %s, L=%d, d_kv=%d" % (q.dtype, l, d))
   def heads_first(t):
     return t.reshape(b, l, h, d).permute(0, 2, 1, 3).reshape(b * h, l, d) \
         .contiguous()

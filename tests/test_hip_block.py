@@ -676,6 +676,41 @@ def test_block_backward_entries(hip, act_dtype):
                                rtol=1e-5 if act_dtype == "float32" else 2e-2)
 
 
+@pytest.mark.parametrize("bsz,length,heads,d,causal", [
+    (1, 8, 1, 64, True), (2, 72, 2, 64, False), (1, 200, 3, 128, True),
+    (1, 328, 2, 128, False), (2, 256, 2, 64, True), (1, 776, 1, 128, True),
+    (1, 1280, 2, 64, False)])
+def test_fused_attention_backward(hip, bsz, length, heads, d, causal):
+  """mesh_moe_self_attention_backward (nothing [L, L] in memory) against the
+  oracle and against the composed path, bf16, lengths that are not multiples
+  of the kernels' tiles (64 streamed rows, 256 own rows)."""
+  rng = np.random.default_rng(length + d)
+  dt = torch.bfloat16
+  mk = lambda: O.cast_act(
+      (rng.standard_normal((bsz, length, heads * d)) * 0.5).astype(np.float32),
+      "bfloat16")
+  q, kk, v, do = mk(), mk(), mk(), mk()
+  dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dt).cuda()
+  args = (dev(q), dev(kk), dev(v), dev(do), heads, causal)
+  got = hip.self_attention_backward(*args, fused=True)
+  want = B.attention_core_backward(q, kk, v, do, heads, causal, "bfloat16")
+  composed = hip.self_attention_backward(*args, fused=False)
+  for g, wnt, c, name in zip(got, want, composed, "qkv"):
+    scale = max(1.0, float(np.abs(wnt).max()))
+    np.testing.assert_allclose(H.to_np(g), wnt, rtol=3e-2, atol=3e-2 * scale,
+                               err_msg="d" + name)
+    # the two device paths differ by a few roundings only
+    diff = np.abs(H.to_np(g) - H.to_np(c))
+    assert float(diff.mean()) < 4e-3 * scale, (name, float(diff.mean()))
+  # the same bits on every run (no atomics)
+  again = hip.self_attention_backward(*args, fused=True)
+  for g, a in zip(got, again):
+    assert torch.equal(g, a)
+  with pytest.raises(hip.MoeHipError):
+    hip.self_attention_backward(*(t.float() if isinstance(t, torch.Tensor)
+                                  else t for t in args), fused=True)
+
+
 def test_layer_stack_gradients():
   """mtf.gradients through a stack of attention and DenseReluDense layers
   (RMS norms, residuals, projections): every variable's gradient and the
