@@ -327,6 +327,38 @@ def test_router_top2_gating_fused(hip, case):
       assert torch.equal(a_, b_)
 
 
+@pytest.mark.parametrize("policy", ["all", "none", "threshold", "random"])
+@pytest.mark.parametrize("second_place_loss", [False, True])
+def test_router_top2_gating_fused_policies(hip, policy, second_place_loss):
+  """Every second-place policy, with a router bias and importance, through the
+  one-launch entry point: the same record, to the bit, as the logits-in entry
+  point fed the logits the fused kernel reports (the two select the experts
+  in different code: accumulator registers against one thread per token)."""
+  b, gpr, s, m, e, c = 2, 3, 256, 128, 16, 30
+  gen = torch.Generator(device="cuda").manual_seed(7)
+  x = torch.randn((b, gpr * s, m), generator=gen, device="cuda").to(torch.bfloat16)
+  w = (torch.randn((b, m, e), generator=gen, device="cuda") / m ** 0.5).to(
+      torch.bfloat16)
+  wp = hip.pack_weights(w, w.dtype)
+  bias = torch.randn((e,), generator=gen, device="cuda") * 0.1
+  u = torch.rand((b * gpr, s), generator=gen, device="cuda")
+  imp = torch.tensor([0.0, 0.5, 1.0], device="cuda")[
+      torch.randint(0, 3, (b * gpr, s), generator=gen, device="cuda")]
+  kw = dict(policy=policy, threshold=0.25, second_uniform=u, importance=imp,
+            use_second_place_loss=second_place_loss, num_microbatches=3)
+  r, logits = hip.router_top2_gating(x, wp, s, c, bias=bias, want_logits=True,
+                                     **kw)
+  r2 = hip.top2_gating(logits, c, **kw)
+  for name in ("idx", "pos", "kept", "fill", "gate", "loss"):
+    assert torch.equal(getattr(r, name), getattr(r2, name)), name
+  if policy == "all":
+    H.assert_routing_properties(r, logits, importance=imp)
+  # and without reporting the logits (they then never leave the chip)
+  r3 = hip.router_top2_gating(x, wp, s, c, bias=bias, **kw)
+  for name in ("idx", "pos", "kept", "fill", "gate", "loss"):
+    assert torch.equal(getattr(r, name), getattr(r3, name)), name
+
+
 def test_router_top2_gating_rejects_unsupported(hip):
   x = torch.zeros((1, 96, 64), dtype=torch.bfloat16, device="cuda")
   wp = torch.zeros((1, 8, 64), dtype=torch.bfloat16, device="cuda")
