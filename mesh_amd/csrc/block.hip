@@ -333,6 +333,122 @@ __global__ __launch_bounds__(256) void rms_norm_backward_kernel(
 }
 
 // partial[chunk, j] = sum over the chunk's rows of dy * x * rstd
+// bf16 rows of ITERS * 512 elements, 16-byte aligned: a wavefront keeps its row
+// (x and g = dy * scale as float32) in registers, reads x and dy once with
+// 16-byte loads and also carries the scale gradient's partial sums
+// sum_rows dy * x * r for its rows, so the second pass over x and dy of the
+// generic path drops out.  Wavefront w of the grid takes rows w, w + W, ...;
+// the four wavefronts of a block add their partial sums in LDS (in wavefront
+// order) and write partial[block][M].
+template <int ITERS>
+__global__ __launch_bounds__(256, 2) void rms_norm_backward_rows_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ scale,
+    const bf16_t* __restrict__ dy, bf16_t* __restrict__ dx,
+    float* __restrict__ partial, int64_t rows, float inv_m, float eps) {
+  constexpr int M = ITERS * 512;
+  __shared__ float red[M];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t stride = (int64_t)gridDim.x * 4;
+  // x, dy and scale stay packed (two bf16 per register) and are unpacked where
+  // they are used: 32 + 32 + 32 + 64 registers at 4096 columns
+  uint32_t sc[ITERS][4];
+  float acc[ITERS][8];
+  auto lo = [](uint32_t w) { return __uint_as_float(w << 16); };
+  auto hi = [](uint32_t w) { return __uint_as_float(w & 0xffff0000u); };
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const uint4 sv = *reinterpret_cast<const uint4*>(scale + (it * 64 + lane) * 8);
+    sc[it][0] = sv.x; sc[it][1] = sv.y; sc[it][2] = sv.z; sc[it][3] = sv.w;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[it][j] = 0.f;
+  }
+  for (int64_t row = (int64_t)blockIdx.x * 4 + wave; row < rows; row += stride) {
+    const bf16_t* xr = x + row * M;
+    const bf16_t* gr = dy + row * M;
+    uint32_t xv[ITERS][4], gv[ITERS][4];
+    float sumsq = 0.f, dot = 0.f;
+    // (the empty asm statements make the packed registers opaque, so that the
+    // compiler unpacks them at each use instead of keeping 192 floats alive)
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) asm volatile("" : "+v"(sc[it][j]));
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      const uint4 a = load_streaming(
+          reinterpret_cast<const uint4*>(xr + (it * 64 + lane) * 8));
+      const uint4 b = load_streaming(
+          reinterpret_cast<const uint4*>(gr + (it * 64 + lane) * 8));
+      xv[it][0] = a.x; xv[it][1] = a.y; xv[it][2] = a.z; xv[it][3] = a.w;
+      gv[it][0] = b.x; gv[it][1] = b.y; gv[it][2] = b.z; gv[it][3] = b.w;
+    }
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float v0 = lo(xv[it][j]), v1 = hi(xv[it][j]);
+        sumsq = fmaf(v0, v0, sumsq);
+        dot = fmaf(lo(gv[it][j]) * lo(sc[it][j]), v0, dot);
+        sumsq = fmaf(v1, v1, sumsq);
+        dot = fmaf(hi(gv[it][j]) * hi(sc[it][j]), v1, dot);
+      }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      sumsq += __shfl_xor(sumsq, off);
+      dot += __shfl_xor(dot, off);
+    }
+    const float r = 1.0f / sqrtf(sumsq * inv_m + eps);
+    const float c = r * r * r * dot * inv_m;
+    bf16_t* outr = dx + row * M;
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+        asm volatile("" : "+v"(sc[it][j]), "+v"(xv[it][j]), "+v"(gv[it][j]));
+#pragma unroll
+    for (int it = 0; it < ITERS; ++it) {
+      uint32_t o[4];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const float v0 = lo(xv[it][j]), v1 = hi(xv[it][j]);
+        const float d0 = lo(gv[it][j]), d1 = hi(gv[it][j]);
+        o[j] = f32x2_to_bf16x2(d0 * lo(sc[it][j]) * r - v0 * c,
+                               d1 * hi(sc[it][j]) * r - v1 * c);
+        acc[it][2 * j] = fmaf(d0 * v0, r, acc[it][2 * j]);
+        acc[it][2 * j + 1] = fmaf(d1 * v1, r, acc[it][2 * j + 1]);
+      }
+      uint4 ov;
+      ov.x = o[0]; ov.y = o[1]; ov.z = o[2]; ov.w = o[3];
+      store_streaming(reinterpret_cast<uint4*>(outr + (it * 64 + lane) * 8), ov);
+    }
+  }
+  for (int w = 0; w < 4; ++w) {
+    if (wave == w) {
+#pragma unroll
+      for (int it = 0; it < ITERS; ++it)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int col = (it * 64 + lane) * 8 + j;
+          red[col] = w == 0 ? acc[it][j] : red[col] + acc[it][j];
+        }
+    }
+    __syncthreads();
+  }
+  float* pr = partial + (int64_t)blockIdx.x * M;
+  for (int i = threadIdx.x; i < M; i += 256) pr[i] = red[i];
+}
+
+constexpr int RMS_ROWS_BLOCKS = 512;   // two per CU
+
+static bool rms_rows_path(int64_t rows, int M, int dtype, const void* x,
+                          const void* scale, const void* dy, const void* dx) {
+  return dtype == MESH_MOE_BF16 && M % 512 == 0 && M >= 512 && M <= 4096 &&
+         rows >= 1 &&
+         (((uintptr_t)x | (uintptr_t)scale | (uintptr_t)dy | (uintptr_t)dx) % 16 ==
+          0);
+}
+
 template <typename T>
 __global__ __launch_bounds__(256) void rms_norm_dscale_partial_kernel(
     const T* __restrict__ x, const T* __restrict__ dy,
@@ -564,8 +680,10 @@ extern "C" int mesh_moe_broadcast_dropout(const void* x, const void* uniform,
 extern "C" size_t mesh_moe_rms_norm_backward_workspace_bytes(int64_t rows,
                                                             int M) {
   if (rows < 1 || M < 1) return 0;
-  return ((size_t)rows * 4 + 255) / 256 * 256 +
-         (size_t)rms_norm_dscale_chunks(rows) * (size_t)M * 4;
+  const size_t parts =
+      (size_t)rms_norm_dscale_chunks(rows) > (size_t)RMS_ROWS_BLOCKS
+          ? (size_t)rms_norm_dscale_chunks(rows) : (size_t)RMS_ROWS_BLOCKS;
+  return ((size_t)rows * 4 + 255) / 256 * 256 + parts * (size_t)M * 4;
 }
 
 extern "C" int mesh_moe_rms_norm_backward(const void* x, const void* scale,
@@ -596,6 +714,27 @@ extern "C" int mesh_moe_rms_norm_backward(const void* x, const void* scale,
   const int64_t per_chunk = (rows + chunks - 1) / chunks;
   const dim3 pg((unsigned)((M + 255) / 256), (unsigned)chunks);
   const float inv_m = (float)(1.0 / (double)M);
+  if (rms_rows_path(rows, M, dtype, x, scale, dy, dx)) {
+    const int nb = (int)(blocks < RMS_ROWS_BLOCKS ? blocks : RMS_ROWS_BLOCKS);
+    const bf16_t *x_ = (const bf16_t*)x, *s_ = (const bf16_t*)scale,
+                 *g_ = (const bf16_t*)dy;
+    const float e_ = round_bf16_host((float)epsilon);
+    switch (M / 512) {
+#define MOE_RMS_ROWS(IT)                                                       \
+  case IT:                                                                     \
+    rms_norm_backward_rows_kernel<IT><<<nb, 256, 0, st>>>(                     \
+        x_, s_, g_, (bf16_t*)dx, partial, rows, inv_m, e_);                    \
+    break;
+      MOE_RMS_ROWS(1) MOE_RMS_ROWS(2) MOE_RMS_ROWS(3) MOE_RMS_ROWS(4)
+      MOE_RMS_ROWS(5) MOE_RMS_ROWS(6) MOE_RMS_ROWS(7) MOE_RMS_ROWS(8)
+#undef MOE_RMS_ROWS
+    }
+    MOE_CHECK_LAUNCH("rms_norm_backward (rows)");
+    rms_norm_dscale_final_kernel<bf16_t><<<pg.x, 256, 0, st>>>(
+        partial, (bf16_t*)dscale, nb, M);
+    MOE_CHECK_LAUNCH("rms_norm_backward (dscale)");
+    return 0;
+  }
   if (dtype == MESH_MOE_F32) {
     rms_norm_backward_kernel<float><<<(unsigned)blocks, 256, 0, st>>>(
         (const float*)x, (const float*)scale, (const float*)dy, (float*)dx,

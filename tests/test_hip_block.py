@@ -638,7 +638,8 @@ def test_block_backward_entries(hip, act_dtype):
   dev = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dt).cuda()
   rnd = lambda *s: O.cast_act(rng.standard_normal(s).astype(np.float32),
                               act_dtype)
-  for rows, m in ((37, 48), (1024, 256), (5, 1000)):
+  for rows, m in ((37, 48), (1024, 256), (5, 1000), (300, 512), (2100, 1536),
+                  (1030, 4096), (3, 2048)):
     x, dy = rnd(rows, m), rnd(rows, m)
     scale = O.cast_act((1 + 0.2 * rng.standard_normal(m)).astype(np.float32),
                        act_dtype)
