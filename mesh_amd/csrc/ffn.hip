@@ -1242,6 +1242,35 @@ __global__ __launch_bounds__(256) void activation_backward_kernel(
   }
 }
 
+// The same for bf16 with 16-byte accesses: 8 elements per thread and step.
+__global__ __launch_bounds__(256) void activation_backward_bf16x8_kernel(
+    const uint4* __restrict__ dh, const uint4* __restrict__ pre,
+    const uint4* __restrict__ factor, uint4* __restrict__ dpre, int64_t n8,
+    int act) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8;
+       i += stride) {
+    const uint4 g4 = load_streaming(dh + i), p4 = load_streaming(pre + i);
+    uint4 f4 = make_uint4(0, 0, 0, 0);
+    if (factor) f4 = load_streaming(factor + i);
+    const uint32_t g[4] = {g4.x, g4.y, g4.z, g4.w}, p[4] = {p4.x, p4.y, p4.z, p4.w};
+    const uint32_t f[4] = {f4.x, f4.y, f4.z, f4.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      float g0 = __uint_as_float(g[j] << 16), g1 = __uint_as_float(g[j] & 0xffff0000u);
+      if (factor) {
+        g0 *= __uint_as_float(f[j] << 16);
+        g1 *= __uint_as_float(f[j] & 0xffff0000u);
+      }
+      o[j] = f32x2_to_bf16x2(
+          g0 * activation_derivative(__uint_as_float(p[j] << 16), act),
+          g1 * activation_derivative(__uint_as_float(p[j] & 0xffff0000u), act));
+    }
+    store_streaming(dpre + i, make_uint4(o[0], o[1], o[2], o[3]));
+  }
+}
+
 template <int BM, int BN, int BK>
 static int launch_mfma(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
                        int R, int N, int K, bool relu, hipStream_t st) {
@@ -1936,7 +1965,15 @@ extern "C" int mesh_moe_activation_backward(const void* dh, const void* pre,
     activation_backward_kernel<float><<<blocks, 256, 0, st>>>(
         (const float*)dh, (const float*)pre, (const float*)factor,
         (float*)dpre, n, activation);
-  else
+  else if (n % 8 == 0 &&
+           (((uintptr_t)dh | (uintptr_t)pre | (uintptr_t)factor |
+             (uintptr_t)dpre) % 16) == 0) {
+    const int64_t n8 = n / 8;
+    const int vb = (int)((n8 + 255) / 256 < 16384 ? (n8 + 255) / 256 : 16384);
+    activation_backward_bf16x8_kernel<<<vb, 256, 0, st>>>(
+        (const uint4*)dh, (const uint4*)pre, (const uint4*)factor, (uint4*)dpre,
+        n8, activation);
+  } else
     activation_backward_kernel<bf16_t><<<blocks, 256, 0, st>>>(
         (const bf16_t*)dh, (const bf16_t*)pre, (const bf16_t*)factor,
         (bf16_t*)dpre, n, activation);
