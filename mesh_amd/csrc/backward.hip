@@ -15,34 +15,6 @@ namespace mesh_moe {
 
 constexpr int BW_ROWS_PER_BLOCK = 4;  // one wavefront per row, 256 threads
 
-template <typename T>
-struct Vec16B {
-  static constexpr int N = 16 / sizeof(T);
-};
-
-__device__ __forceinline__ void unpack16(const uint4& v, float (&f)[4], float) {
-  f[0] = __uint_as_float(v.x); f[1] = __uint_as_float(v.y);
-  f[2] = __uint_as_float(v.z); f[3] = __uint_as_float(v.w);
-}
-__device__ __forceinline__ void unpack16(const uint4& v, float (&f)[8], bf16_t) {
-  f[0] = __uint_as_float(v.x << 16); f[1] = __uint_as_float(v.x & 0xffff0000u);
-  f[2] = __uint_as_float(v.y << 16); f[3] = __uint_as_float(v.y & 0xffff0000u);
-  f[4] = __uint_as_float(v.z << 16); f[5] = __uint_as_float(v.z & 0xffff0000u);
-  f[6] = __uint_as_float(v.w << 16); f[7] = __uint_as_float(v.w & 0xffff0000u);
-}
-__device__ __forceinline__ uint4 pack16(const float (&f)[4], float) {
-  return make_uint4(__float_as_uint(f[0]), __float_as_uint(f[1]),
-                    __float_as_uint(f[2]), __float_as_uint(f[3]));
-}
-__device__ __forceinline__ uint4 pack16(const float (&f)[8], bf16_t) {
-  uint4 r;
-  r.x = f32x2_to_bf16x2(f[0], f[1]);
-  r.y = f32x2_to_bf16x2(f[2], f[3]);
-  r.z = f32x2_to_bf16x2(f[4], f[5]);
-  r.w = f32x2_to_bf16x2(f[6], f[7]);
-  return r;
-}
-
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);

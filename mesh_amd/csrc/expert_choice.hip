@@ -181,36 +181,61 @@ __global__ __launch_bounds__(256) void slot_dispatch_kernel(
 }
 
 // out[g,s,:] = sum_e w * y[e,g,tok_slot[g,s,e],:] over the experts that chose
-// the token, float32 accumulate in expert order, one rounding.
-template <typename T>
+// the token, float32 accumulate in expert order, one rounding.  One wavefront
+// per token: the experts that chose it are found once (a ballot over 64 experts
+// at a time) and listed in LDS with their row and weight; the rows are then
+// read with 16-byte loads, 512 / 256 columns of all listed rows at a time.
+constexpr int SC_MAX_E = 512;
+
+template <typename T, bool VEC>
 __global__ __launch_bounds__(256) void slot_combine_kernel(
     const T* __restrict__ y, const int16_t* __restrict__ tok_slot,
     const float* __restrict__ slot_weight, T* __restrict__ out, int G, int S,
     int E, int C, int N, int64_t T_tokens) {
-  const int lane = threadIdx.x & 63;
-  const int64_t t = (int64_t)blockIdx.x * CH_ROWS + (threadIdx.x >> 6);
+  constexpr int VN = Vec16B<T>::N;
+  __shared__ int64_t rows[CH_ROWS][SC_MAX_E];
+  __shared__ float wts[CH_ROWS][SC_MAX_E];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int64_t t = (int64_t)blockIdx.x * CH_ROWS + wave;
   if (t >= T_tokens) return;
   const int g = (int)(t / S);
   const int16_t* ts = tok_slot + t * E;
-  T* dst = out + t * N;
-  for (int i0 = 0; i0 < N; i0 += 64 * 4) {
-    float acc[4] = {0.f, 0.f, 0.f, 0.f};
-    for (int e = 0; e < E; ++e) {
-      const int c = ts[e];
-      if (c < 0) continue;
-      const int64_t slot = ((int64_t)g * E + e) * C + c;
-      const float w = round_to<T>(slot_weight[slot]);
-      const T* row = y + (((int64_t)e * G + g) * C + c) * N;
-#pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        const int i = i0 + u * 64 + lane;
-        if (i < N) acc[u] += w * load_f32<T>(row + i);
-      }
+  int n = 0;
+  for (int e0 = 0; e0 < E; e0 += 64) {
+    const int e = e0 + lane;
+    const int c = e < E ? (int)ts[e] : -1;
+    const unsigned long long m = __ballot(c >= 0);
+    if (c >= 0) {
+      const int at = n + __popcll(m & ((1ull << lane) - 1ull));
+      rows[wave][at] = (((int64_t)e * G + g) * C + c) * N;
+      wts[wave][at] = round_to<T>(slot_weight[((int64_t)g * E + e) * C + c]);
     }
+    n += __popcll(m);
+  }
+  // (the list is written and read by the same wavefront: LDS operations of a
+  // wavefront complete in order)
+  T* dst = out + t * N;
+  if (VEC) {
+    for (int i0 = lane * VN; i0 < N; i0 += 64 * VN) {
+      float acc[VN];
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-      const int i = i0 + u * 64 + lane;
-      if (i < N) store_f32<T>(dst + i, acc[u]);
+      for (int j = 0; j < VN; ++j) acc[j] = 0.f;
+      for (int k = 0; k < n; ++k) {
+        float v[VN];
+        unpack16(load_streaming(reinterpret_cast<const uint4*>(
+                     y + rows[wave][k] + i0)), v, T());
+        const float w = wts[wave][k];
+#pragma unroll
+        for (int j = 0; j < VN; ++j) acc[j] += w * v[j];
+      }
+      store_streaming(reinterpret_cast<uint4*>(dst + i0), pack16(acc, T()));
+    }
+  } else {
+    for (int i = lane; i < N; i += 64) {
+      float acc = 0.f;
+      for (int k = 0; k < n; ++k)
+        acc += wts[wave][k] * load_f32<T>(y + rows[wave][k] + i);
+      store_f32<T>(dst + i, acc);
     }
   }
 }
@@ -527,14 +552,19 @@ extern "C" int mesh_moe_slot_combine(const void* y, const int16_t* tok_slot,
   MOE_REQUIRE(nblocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
               "slot_combine: too many rows (%lld)", (long long)T_tokens);
   hipStream_t st = (hipStream_t)stream;
-  if (dtype == MESH_MOE_F32)
-    slot_combine_kernel<float><<<(unsigned)nblocks, 256, 0, st>>>(
-        (const float*)y, tok_slot, slot_weight, (float*)out, G, S, E, C, N,
-        T_tokens);
-  else
-    slot_combine_kernel<bf16_t><<<(unsigned)nblocks, 256, 0, st>>>(
-        (const bf16_t*)y, tok_slot, slot_weight, (bf16_t*)out, G, S, E, C, N,
-        T_tokens);
+  MOE_REQUIRE(E <= SC_MAX_E, MESH_MOE_E_UNSUPPORTED,
+              "slot_combine: E=%d > %d", E, SC_MAX_E);
+  const bool vec = ((size_t)N * dtype_size(dtype)) % 16 == 0 &&
+                   (((uintptr_t)y | (uintptr_t)out) % 16) == 0;
+#define MOE_SLOT_COMBINE(T, V)                                              \
+  slot_combine_kernel<T, V><<<(unsigned)nblocks, 256, 0, st>>>(             \
+      (const T*)y, tok_slot, slot_weight, (T*)out, G, S, E, C, N, T_tokens)
+  if (dtype == MESH_MOE_F32) {
+    if (vec) MOE_SLOT_COMBINE(float, true); else MOE_SLOT_COMBINE(float, false);
+  } else {
+    if (vec) MOE_SLOT_COMBINE(bf16_t, true); else MOE_SLOT_COMBINE(bf16_t, false);
+  }
+#undef MOE_SLOT_COMBINE
   MOE_CHECK_LAUNCH("slot_combine");
   return 0;
 }
