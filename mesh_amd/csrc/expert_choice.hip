@@ -54,8 +54,9 @@ __global__ __launch_bounds__(256) void choice_select_kernel(
     ChoiceParams p, const float* __restrict__ logits,
     const IT* __restrict__ importance, int32_t* __restrict__ slot_token,
     float* __restrict__ slot_prob, int16_t* __restrict__ tok_slot,
-    int32_t* __restrict__ num_routed, float* __restrict__ lse_out) {
-  extern __shared__ float pr[];  // [S] + 4
+    int32_t* __restrict__ num_routed, float* __restrict__ lse_out,
+    bool by_threshold) {
+  extern __shared__ float pr[];  // [S] + 4 (+ 8 + 2 C with by_threshold)
   float* red = pr + p.S;
   const int e = blockIdx.x, g = blockIdx.y;
   const int S = p.S, E = p.E, C = p.C;
@@ -80,20 +81,100 @@ __global__ __launch_bounds__(256) void choice_select_kernel(
   for (int s = tid; s < S; s += 256) pr[s] = expf(pr[s] + neglse);
   if (tid == 0) lse_out[(int64_t)g * E + e] = lse;
   __syncthreads();
-  for (int s = tid; s < S; s += 256) {
-    const float ps = pr[s];
+  auto emit = [&](int s, int rank, float ps) {
+    const int64_t slot = ((int64_t)g * E + e) * C + rank;
+    slot_token[slot] = s;
+    slot_prob[slot] = ps;
+    tok_slot[(base + s) * E + e] = (int16_t)rank;
+    atomicAdd(num_routed + base + s, 1);
+  };
+  if (!by_threshold) {
+    // every token against every token
+    for (int s = tid; s < S; s += 256) {
+      const float ps = pr[s];
+      int rank = 0;
+      for (int s2 = 0; s2 < S; ++s2) {
+        const float p2 = pr[s2];
+        rank += (p2 > ps || (p2 == ps && s2 < s)) ? 1 : 0;
+      }
+      if (rank < C) emit(s, rank, ps);
+    }
+    return;
+  }
+  // The C-th largest probability first (probabilities are >= 0, so their bit
+  // patterns order like unsigned integers): the largest T with at least C
+  // tokens >= T, found bit by bit.  Tokens above T (fewer than C) are ranked
+  // among themselves; tokens equal to T follow in token order.
+  int* iscr = reinterpret_cast<int*>(red + 4);          // [8]
+  uint32_t* key_a = reinterpret_cast<uint32_t*>(iscr + 8);  // [C]
+  int* tok_a = reinterpret_cast<int*>(key_a + C);       // [C]
+  const uint32_t* key = reinterpret_cast<const uint32_t*>(pr);
+  const int lane = tid & 63, wave = tid >> 6;
+  // thread tid owns tokens [s_lo, s_hi): contiguous, so that compaction keeps
+  // the token order
+  const int per = (S + 255) / 256;
+  const int s_lo = min(S, tid * per), s_hi = min(S, s_lo + per);
+  auto block_count = [&](int v) {       // sum over the block, to every thread
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) v += __shfl_xor(v, off, 64);
+    __syncthreads();
+    if (lane == 0) iscr[wave] = v;
+    __syncthreads();
+    return iscr[0] + iscr[1] + iscr[2] + iscr[3];
+  };
+  uint32_t thr = 0u;
+  for (int bit = 30; bit >= 0; --bit) {
+    const uint32_t trial = thr | (1u << bit);
+    int cnt = 0;
+    for (int s = s_lo; s < s_hi; ++s) cnt += key[s] >= trial ? 1 : 0;
+    if (block_count(cnt) >= C) thr = trial;
+  }
+  // exclusive positions of this thread's tokens among those above / equal
+  int n_gt = 0, n_eq = 0;
+  for (int s = s_lo; s < s_hi; ++s) {
+    n_gt += key[s] > thr ? 1 : 0;
+    n_eq += key[s] == thr ? 1 : 0;
+  }
+  auto block_scan = [&](int v, int* total) {   // exclusive prefix over threads
+    int inc = v;
+#pragma unroll
+    for (int off = 1; off < 64; off <<= 1) {
+      const int o = __shfl_up(inc, off, 64);
+      if (lane >= off) inc += o;
+    }
+    __syncthreads();
+    if (lane == 63) iscr[4 + wave] = inc;
+    __syncthreads();
+    int before = 0;
+    for (int w = 0; w < wave; ++w) before += iscr[4 + w];
+    *total = iscr[4] + iscr[5] + iscr[6] + iscr[7];
+    return before + inc - v;
+  };
+  int total_gt, total_eq;
+  int at_gt = block_scan(n_gt, &total_gt);
+  int at_eq = block_scan(n_eq, &total_eq);
+  for (int s = s_lo; s < s_hi; ++s) {
+    const uint32_t k = key[s];
+    if (k > thr) {
+      key_a[at_gt] = k;
+      tok_a[at_gt] = s;
+      ++at_gt;
+    } else if (k == thr) {
+      const int rank = total_gt + at_eq;
+      ++at_eq;
+      if (rank < C) emit(s, rank, pr[s]);
+    }
+  }
+  __syncthreads();
+  for (int a = tid; a < total_gt; a += 256) {
+    const uint32_t k = key_a[a];
     int rank = 0;
-    for (int s2 = 0; s2 < S; ++s2) {
-      const float p2 = pr[s2];
-      rank += (p2 > ps || (p2 == ps && s2 < s)) ? 1 : 0;
+    // (the list is in token order: equal keys before position a come first)
+    for (int b2 = 0; b2 < total_gt; ++b2) {
+      const uint32_t k2 = key_a[b2];
+      rank += (k2 > k || (k2 == k && b2 < a)) ? 1 : 0;
     }
-    if (rank < C) {
-      const int64_t slot = ((int64_t)g * E + e) * C + rank;
-      slot_token[slot] = s;
-      slot_prob[slot] = ps;
-      tok_slot[(base + s) * E + e] = (int16_t)rank;
-      atomicAdd(num_routed + base + s, 1);
-    }
+    emit(tok_a[a], rank, __uint_as_float(k));
   }
 }
 
@@ -478,19 +559,24 @@ extern "C" int mesh_moe_expert_choice_gating(
                                                             : 8192);
   choice_clear_kernel<<<cb, 256, 0, st>>>(num_routed, n_tok, tok_slot, n_ts);
   MOE_CHECK_LAUNCH("expert_choice_gating (clear)");
-  const size_t smem = sizeof(float) * ((size_t)S + 4);
+  // the threshold form needs two lists of C entries next to the probabilities
+  const size_t smem_thr = sizeof(float) * ((size_t)S + 4 + 8 + 2 * (size_t)C);
+  const bool by_threshold = smem_thr <= 150 * 1024;
+  const size_t smem = by_threshold ? smem_thr : sizeof(float) * ((size_t)S + 4);
   dim3 grid((unsigned)E, (unsigned)G);
   const bool bf = importance && importance_dtype == MESH_MOE_BF16;
   if (bf) {
     auto k = choice_select_kernel<bf16_t>;
     MOE_ALLOW_LDS(k, smem);
     k<<<grid, 256, smem, st>>>(p, logits, (const bf16_t*)importance, slot_token,
-                               slot_prob, tok_slot, num_routed, lse);
+                               slot_prob, tok_slot, num_routed, lse,
+                               by_threshold);
   } else {
     auto k = choice_select_kernel<float>;
     MOE_ALLOW_LDS(k, smem);
     k<<<grid, 256, smem, st>>>(p, logits, (const float*)importance, slot_token,
-                               slot_prob, tok_slot, num_routed, lse);
+                               slot_prob, tok_slot, num_routed, lse,
+                               by_threshold);
   }
   MOE_CHECK_LAUNCH("expert_choice_gating (select)");
   if (bf)
