@@ -178,24 +178,30 @@ __global__ __launch_bounds__(256) void choice_select_kernel(
   }
 }
 
-// One block per group: combine weights (probability over the number of experts
-// that chose the token, moe.py:1119-1123) and the group's term of the loss
+// One block per (group, chunk of 256 tokens), one thread per token: combine
+// weights (probability over the number of experts that chose the token,
+// moe.py:1119-1123) and the chunk's share of the group's loss term
 // mean(agg^2 * sum_s importance) * S with agg = mean_e p * (importance == 1)
-// (moe.py:1125-1147).
+// (moe.py:1125-1147): part[g][chunk] = (sum agg^2, sum importance).
 template <typename IT>
 __global__ __launch_bounds__(256) void choice_finish_kernel(
     ChoiceParams p, const float* __restrict__ logits,
     const IT* __restrict__ importance, const float* __restrict__ lse,
     const float* __restrict__ slot_prob, const int16_t* __restrict__ tok_slot,
     const int32_t* __restrict__ num_routed, float* __restrict__ slot_weight,
-    float* __restrict__ gsum) {
-  __shared__ float red[4];
-  const int g = blockIdx.x;
+    float2* __restrict__ part) {
+  extern __shared__ float fin_smem[];   // lse of the group [E], then 4
+  float* lse_s = fin_smem;
+  float* red = fin_smem + p.E;
+  const int g = blockIdx.y, chunk = blockIdx.x;
   const int S = p.S, E = p.E, C = p.C;
   const int64_t base = (int64_t)g * S;
   const float inv_e = (float)(1.0 / (double)E);
+  for (int e = threadIdx.x; e < E; e += 256) lse_s[e] = lse[(int64_t)g * E + e];
+  __syncthreads();
   float sq = 0.f, imp_sum = 0.f;
-  for (int s = threadIdx.x; s < S; s += 256) {
+  const int s = chunk * 256 + threadIdx.x;
+  if (s < S) {
     const int64_t t = base + s;
     float imp = 1.0f;
     if (importance != nullptr) imp = load_f32<IT>(importance + t);
@@ -206,7 +212,7 @@ __global__ __launch_bounds__(256) void choice_finish_kernel(
     for (int e = 0; e < E; ++e) {
       float x = logits[t * E + e];
       if (imp == 0.0f) x = x + mask;
-      agg += expf(x + (-lse[(int64_t)g * E + e]));
+      agg += expf(x + (-lse_s[e]));
       const int c = tok_slot[t * E + e];
       if (c >= 0) {
         const int64_t slot = ((int64_t)g * E + e) * C + c;
@@ -214,19 +220,29 @@ __global__ __launch_bounds__(256) void choice_finish_kernel(
       }
     }
     agg = (agg * inv_e) * (imp == 1.0f ? 1.0f : 0.0f);
-    sq += agg * agg;
-    imp_sum += imp;
+    sq = agg * agg;
+    imp_sum = imp;
   }
   sq = block_reduce(sq, red, false);
   imp_sum = block_reduce(imp_sum, red, false);
-  if (threadIdx.x == 0) gsum[g] = sq * imp_sum;
+  if (threadIdx.x == 0)
+    part[(int64_t)g * gridDim.x + chunk] = make_float2(sq, imp_sum);
 }
 
-__global__ void choice_loss_kernel(ChoiceParams p, const float* __restrict__ gsum,
-                                   float* __restrict__ loss) {
+// The loss from the chunks' shares, summed in chunk order, then group order.
+__global__ void choice_loss_kernel(ChoiceParams p, const float2* __restrict__ part,
+                                   int chunks, float* __restrict__ loss) {
   if (threadIdx.x != 0 || blockIdx.x != 0) return;
   float s = 0.f;
-  for (int g = 0; g < p.G; ++g) s += gsum[g];
+  for (int g = 0; g < p.G; ++g) {
+    float sq = 0.f, imp = 0.f;
+    for (int c = 0; c < chunks; ++c) {
+      const float2 v = part[(int64_t)g * chunks + c];
+      sq += v.x;
+      imp += v.y;
+    }
+    s += sq * imp;
+  }
   float l = (s * (float)(1.0 / ((double)p.G * (double)p.S))) * (float)p.S;
   if (p.num_microbatches > 1)
     l = l * (float)(1.0 / (double)p.num_microbatches);
@@ -255,7 +271,7 @@ __global__ __launch_bounds__(256) void slot_dispatch_kernel(
     const uint4* s4 = reinterpret_cast<const uint4*>(src);
     uint4* d4 = reinterpret_cast<uint4*>(dst);
     const int nv = M / (16 / (int)sizeof(T));
-    for (int i = lane; i < nv; i += 64) d4[i] = s4[i];
+    for (int i = lane; i < nv; i += 64) store_streaming(d4 + i, s4[i]);
   } else {
     for (int i = lane; i < M; i += 64) dst[i] = src[i];
   }
@@ -519,8 +535,8 @@ extern "C" size_t mesh_moe_expert_choice_workspace_bytes(int G, int S, int E,
                                                          int C) {
   if (G < 1 || S < 1 || E < 1 || C < 1) return 0;
   return sizeof(int32_t) * (size_t)G * S + sizeof(float) * (size_t)G * E +
-         sizeof(float) * (size_t)G * E * C + sizeof(float) * (size_t)G +
-         4 * 256;
+         sizeof(float) * (size_t)G * E * C +
+         sizeof(float) * 2 * (size_t)G * (((size_t)S + 255) / 256) + 4 * 256;
 }
 
 extern "C" int mesh_moe_expert_choice_gating(
@@ -579,16 +595,20 @@ extern "C" int mesh_moe_expert_choice_gating(
                                by_threshold);
   }
   MOE_CHECK_LAUNCH("expert_choice_gating (select)");
+  const int chunks = (S + 255) / 256;
+  const dim3 fgrid((unsigned)chunks, (unsigned)G);
+  const size_t fsmem = sizeof(float) * ((size_t)E + 4);
+  float2* part = reinterpret_cast<float2*>(gsum);
   if (bf)
-    choice_finish_kernel<bf16_t><<<G, 256, 0, st>>>(
+    choice_finish_kernel<bf16_t><<<fgrid, 256, fsmem, st>>>(
         p, logits, (const bf16_t*)importance, lse, slot_prob, tok_slot,
-        num_routed, slot_weight, gsum);
+        num_routed, slot_weight, part);
   else
-    choice_finish_kernel<float><<<G, 256, 0, st>>>(
+    choice_finish_kernel<float><<<fgrid, 256, fsmem, st>>>(
         p, logits, (const float*)importance, lse, slot_prob, tok_slot,
-        num_routed, slot_weight, gsum);
+        num_routed, slot_weight, part);
   MOE_CHECK_LAUNCH("expert_choice_gating (finish)");
-  choice_loss_kernel<<<1, 64, 0, st>>>(p, gsum, loss);
+  choice_loss_kernel<<<1, 64, 0, st>>>(p, part, chunks, loss);
   MOE_CHECK_LAUNCH("expert_choice_gating (loss)");
   return 0;
 }
