@@ -1231,6 +1231,12 @@ __global__ __launch_bounds__(CAP_THREADS) void gate_capacity_kernel(
   // first-choice gates of the group, for the by-gate slot order; float-aligned
   // because 3 * S int16 may end on an odd 2-byte boundary
   float* gl = reinterpret_cast<float*>(c2l + S + (S & 1));    // [S]
+  // by-gate order only: the first-choice gates listed per expert (token order
+  // within an expert), every token's place in that list, the experts' first
+  // places
+  float* lg = gl + S;                                         // [S]
+  int32_t* lpos = reinterpret_cast<int32_t*>(lg + S);         // [S]
+  int32_t* ebase = lpos + S;                                  // [el]
   const int g = blockIdx.x;
   const int tid = threadIdx.x;
   const int64_t base = (int64_t)g * S;
@@ -1274,12 +1280,25 @@ __global__ __launch_bounds__(CAP_THREADS) void gate_capacity_kernel(
     if (chunk == 0 && e < E) tot[choice * el + e] = total;
     if (choice == 0) count1 = min(total, C);
     __syncthreads();
-    const bool in_token_order = !(p.rank_by_gate && choice == 0);
-    for (int s = tid; in_token_order && s < S; s += CAP_THREADS) {
+    const bool by_gate = p.rank_by_gate && choice == 0;
+    if (by_gate) {
+      if (tid == 0) {
+        int run = 0;
+        for (int k = 0; k < E; ++k) { ebase[k] = run; run += tot[k]; }
+      }
+      __syncthreads();
+    }
+    for (int s = tid; s < S; s += CAP_THREADS) {
       const int ex = ch[s];
       if (ex < 0) continue;
       const int ck = s / clen;
       const int slot = pre[ck * el + ex] + cap_count(ch, ck * clen, s, ex, vec);
+      if (by_gate) {
+        // not the slot yet: the token's place among its expert's choosers
+        lpos[s] = ebase[ex] + slot;
+        lg[ebase[ex] + slot] = gl[s];
+        continue;
+      }
       const int64_t t = base + s;
       const bool ok = slot < C;
       pos[t * 2 + choice] = slot;
@@ -1295,12 +1314,11 @@ __global__ __launch_bounds__(CAP_THREADS) void gate_capacity_kernel(
       const int ex = c1[s];
       if (ex < 0) continue;
       const float gs = gl[s];
+      const int mine = lpos[s], first = ebase[ex], last = first + tot[ex];
       int rank = 0;
-      for (int s2 = 0; s2 < S; ++s2) {
-        if (c1[s2] == ex) {
-          const float g2 = gl[s2];
-          rank += (g2 > gs || (g2 == gs && s2 < s)) ? 1 : 0;
-        }
+      for (int j = first; j < last; ++j) {
+        const float g2 = lg[j];
+        rank += (g2 > gs || (g2 == gs && j < mine)) ? 1 : 0;
       }
       const int64_t t = base + s;
       const bool ok = rank < C;
@@ -1522,7 +1540,7 @@ static int launch_capacity_and_loss(const GateParams& p, int32_t* idx,
   size_t smem = sizeof(int32_t) * (2 * CAP_THREADS + 3 * (size_t)el) +
                 sizeof(float) * 2 * (size_t)el +
                 sizeof(int16_t) * (3 * (size_t)p.S + 1) +
-                (p.rank_by_gate ? sizeof(float) * (size_t)p.S : 0);
+                (p.rank_by_gate ? sizeof(float) * (3 * (size_t)p.S + el) : 0);
   MOE_ALLOW_LDS(gate_capacity_kernel, smem);
   gate_capacity_kernel<<<p.G, CAP_THREADS, smem, st>>>(
       p, idx, pos, gate, kept, fill, part1, part2, gsum, el);
