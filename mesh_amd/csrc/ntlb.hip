@@ -129,6 +129,10 @@ __global__ __launch_bounds__(NTLB_THREADS) void ntlb_assign_kernel(
   float* prod = reinterpret_cast<float*>(named + (size_t)K * el);  // [el]
   int16_t* cand = reinterpret_cast<int16_t*>(prod + el);  // [K][S]
   uint8_t* open_ = reinterpret_cast<uint8_t*>(cand + (size_t)K * S);  // [S]
+  // what the passes decide per token, written out in one parallel sweep at
+  // the end: the pass that placed it (0xff: none) and its slot
+  uint8_t* wpass = open_ + S;                                          // [S]
+  int16_t* wpos = reinterpret_cast<int16_t*>(wpass + S + (S & 1));     // [S]
   const int g = blockIdx.x, tid = threadIdx.x;
   const int64_t base = (int64_t)g * S;
   for (int i = tid; i < S * K; i += NTLB_THREADS) {
@@ -136,17 +140,8 @@ __global__ __launch_bounds__(NTLB_THREADS) void ntlb_assign_kernel(
     cand[k * S + s] = cand_idx[base * K + i];
   }
   for (int s = tid; s < S; s += NTLB_THREADS) {
-    const int64_t t = base + s;
-    open_[s] = competes[t];
-    // default record: not routed; the first candidate stands in as the expert
-    idx[t * 2] = cand_idx[t * K];
-    idx[t * 2 + 1] = 0;
-    pos[t * 2] = 0;
-    pos[t * 2 + 1] = 0;
-    gate[t * 2] = 0.0f;
-    gate[t * 2 + 1] = 0.0f;
-    kept[t * 2] = 0;
-    kept[t * 2 + 1] = 0;
+    open_[s] = competes[base + s];
+    wpass[s] = 0xff;
   }
   if (tid < el) held[tid] = 0;
   __syncthreads();
@@ -182,11 +177,8 @@ __global__ __launch_bounds__(NTLB_THREADS) void ntlb_assign_kernel(
       if (ch[s] == e && open_[s]) {
         ++running;
         if (running <= C) {
-          const int64_t t = base + s;
-          idx[t * 2] = e;
-          pos[t * 2] = running - 1;
-          gate[t * 2] = cand_gate[t * K + i];
-          kept[t * 2] = 1;
+          wpass[s] = (uint8_t)i;
+          wpos[s] = (int16_t)(running - 1);
           open_[s] = 0;
         }
       }
@@ -199,6 +191,21 @@ __global__ __launch_bounds__(NTLB_THREADS) void ntlb_assign_kernel(
       held[e] = min(C, have + total);
     }
     __syncthreads();
+  }
+  // the records: a placed token names its expert, slot and gate; the others
+  // keep their first candidate as a stand-in, not routed
+  for (int s = tid; s < S; s += NTLB_THREADS) {
+    const int64_t t = base + s;
+    const int ps = wpass[s];
+    const bool placed = ps != 0xff;
+    idx[t * 2] = placed ? (int32_t)cand[(size_t)ps * S + s] : (int32_t)cand[s];
+    idx[t * 2 + 1] = 0;
+    pos[t * 2] = placed ? (int32_t)wpos[s] : 0;
+    pos[t * 2 + 1] = 0;
+    gate[t * 2] = placed ? cand_gate[t * K + ps] : 0.0f;
+    gate[t * 2 + 1] = 0.0f;
+    kept[t * 2] = placed ? 1 : 0;
+    kept[t * 2 + 1] = 0;
   }
   if (tid < E) fill[(int64_t)g * E + tid] = held[tid];
   // the group's share of the loss: sum over passes and experts of
@@ -295,7 +302,8 @@ extern "C" int mesh_moe_ntlb_gating(
   const size_t smem2 = sizeof(int32_t) * (NTLB_THREADS + (size_t)el +
                                           (size_t)top_k * el) +
                        sizeof(float) * (size_t)el +
-                       sizeof(int16_t) * (size_t)top_k * S + (size_t)S;
+                       sizeof(int16_t) * (size_t)top_k * S + (size_t)S +
+                       (size_t)S + 2 + sizeof(int16_t) * (size_t)S;
   MOE_REQUIRE(smem2 <= 160 * 1024, MESH_MOE_E_UNSUPPORTED,
               "ntlb_gating: top_k * S = %d * %d candidates do not fit in LDS",
               top_k, S);
