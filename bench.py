@@ -67,7 +67,7 @@ def hparams_dict(cfg):
       moe_use_second_place_loss=False, moe_second_policy_train="all",
       moe_second_policy_eval="all", moe_second_threshold_train=0.2,
       moe_second_threshold_eval=0.2, moe_dropout_rate=0.0,
-      moe_use_experts_attention=False)
+      moe_use_experts_attention=False, moe_ntlb_top_k=4)
 
 
 def normal_init(fan_in, seed):
@@ -116,8 +116,7 @@ def build(cfg, device, backward=False, operands="random"):
       # reference router has no bias term: feature 0 of every token is set to 1
       # and row 0 of the router kernel carries the bias.
       x_val[..., 0] = 1.0
-    router = "moe/%s/kernel" % ("switch_gating" if cfg.get("gating") == "switch"
-                                else "top_2_gating")
+    router = "moe/%s_gating/kernel" % cfg.get("gating", "top_2")
     init[router] = normal_init(m, 2)
     init["moe/wi/kernel"] = normal_init(m, 3)
     init["moe/wo/kernel"] = normal_init(h, 4)
@@ -141,9 +140,16 @@ def build(cfg, device, backward=False, operands="random"):
       # anything in this mode
       x_val = x_val * 0
   x = mtf.import_tf_tensor(mesh, x_val, mtf.Shape(dims))
+  nonpadding = None
+  if cfg.get("gating") == "expert_selection":
+    # the reference's loss of this router sums `nonpadding`: every token counts
+    nonpadding = mtf.import_tf_tensor(
+        mesh, torch.ones(x_val.shape[:2], dtype=dt, device=device),
+        mtf.Shape(dims[:2]))
   with mtf.variable_scope("moe"):
     if cfg["layer"] == "v1":
-      y, loss = moe.transformer_moe_layer_v1(x, dims[-1], hp, True, vdt)
+      y, loss = moe.transformer_moe_layer_v1(x, dims[-1], hp, True, vdt,
+                                             nonpadding=nonpadding)
     else:
       y, loss = moe.transformer_moe_layer_v2(x, dims[-1], hp, True, vdt)
   if cfg.get("skew"):
@@ -228,6 +234,13 @@ def stage_model(cfg, kept_pairs, slots):
       "router_top2_gating": dict(bytes=t * m * b + m * e * b + 26 * t),
       "switch_gating": dict(bytes=t * (4 * e + 26)),
       "router_switch_gating": dict(bytes=t * m * b + m * e * b + 26 * t),
+      "ntlb_gating": dict(bytes=t * (4 * e + 26)),
+      # experts choose tokens: slot records [G, E, C] and the token -> slot
+      # table [G, S, E] int16
+      "expert_choice_gating": dict(bytes=t * (4 * e + 2 * e) + 8 * slots),
+      "slot_dispatch": dict(bytes=2 * slots * m * b + 4 * slots),
+      "slot_combine": dict(bytes=slots * m * b + t * m * b + 2 * t * e
+                           + 4 * slots),
       "dispatch": dict(bytes=t * m * b + r * m * b + 18 * t),
       "combine": dict(bytes=r * m * b + t * m * b + 26 * t),
       "expert_ffn": dict(flops=4 * r * m * h, padded_flops=4 * slots * m * h),
@@ -293,7 +306,9 @@ def main():
   ap.add_argument("--steps", type=int, default=10)
   ap.add_argument("--warmup", type=int, default=3)
   ap.add_argument("--config", type=int, default=4, choices=sorted(CONFIGS))
-  ap.add_argument("--gating", default="top_2", choices=["top_2", "switch"],
+  ap.add_argument("--gating", default="top_2",
+                  choices=["top_2", "switch", "switch_max", "ntlb",
+                           "expert_selection"],
                   help="router of the v1 configs (the benchmark definition "
                        "uses top_2)")
   ap.add_argument("--backward", action="store_true",
@@ -402,8 +417,13 @@ def main():
   }
   if cfg["layer"] == "v1":
     r = routings[-1]
-    kept = int(r.fill.sum().item())
-    slots = r.fill.numel() * r.capacity
+    if hasattr(r, "fill"):
+      kept = int(r.fill.sum().item())
+      slots = r.fill.numel() * r.capacity
+    else:
+      # per-slot record: every slot holds a token, its weight may be 0
+      slots = r.slot_token.numel()
+      kept = slots
     model = stage_model(cfg, kept, slots)
     per_stage = {}
     for name, (calls, ms) in stages.items():
@@ -445,7 +465,9 @@ def main():
     result["stages"] = {k: {"ms_per_step": v[1] / args.steps,
                             "launches_per_step": v[0] / args.steps}
                         for k, v in stages.items()}
-  result["cpu_baseline"] = (None if (args.no_cpu_baseline or args.backward)
+  # (the CPU restatement timed below is the top-2 layer's)
+  result["cpu_baseline"] = (None if (args.no_cpu_baseline or args.backward
+                                     or args.gating != "top_2")
                             else cpu_baseline(cfg))
   print(json.dumps(result))
 

@@ -229,20 +229,32 @@ __global__ __launch_bounds__(256) void choice_finish_kernel(
     part[(int64_t)g * gridDim.x + chunk] = make_float2(sq, imp_sum);
 }
 
-// The loss from the chunks' shares, summed in chunk order, then group order.
-__global__ void choice_loss_kernel(ChoiceParams p, const float2* __restrict__ part,
-                                   int chunks, float* __restrict__ loss) {
-  if (threadIdx.x != 0 || blockIdx.x != 0) return;
+// The loss from the chunks' shares, summed in chunk order (one thread per
+// group), then in group order.
+__global__ __launch_bounds__(256) void choice_loss_kernel(
+    ChoiceParams p, const float2* __restrict__ part, int chunks,
+    float* __restrict__ loss) {
+  __shared__ float term[256];
   float s = 0.f;
-  for (int g = 0; g < p.G; ++g) {
+  for (int g0 = 0; g0 < p.G; g0 += 256) {
+    const int g = g0 + threadIdx.x;
     float sq = 0.f, imp = 0.f;
-    for (int c = 0; c < chunks; ++c) {
-      const float2 v = part[(int64_t)g * chunks + c];
-      sq += v.x;
-      imp += v.y;
+    if (g < p.G) {
+      for (int c = 0; c < chunks; ++c) {
+        const float2 v = part[(int64_t)g * chunks + c];
+        sq += v.x;
+        imp += v.y;
+      }
     }
-    s += sq * imp;
+    __syncthreads();
+    term[threadIdx.x] = sq * imp;
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      const int n = min(256, p.G - g0);
+      for (int i = 0; i < n; ++i) s += term[i];
+    }
   }
+  if (threadIdx.x != 0) return;
   float l = (s * (float)(1.0 / ((double)p.G * (double)p.S))) * (float)p.S;
   if (p.num_microbatches > 1)
     l = l * (float)(1.0 / (double)p.num_microbatches);
@@ -608,7 +620,7 @@ extern "C" int mesh_moe_expert_choice_gating(
         p, logits, (const float*)importance, lse, slot_prob, tok_slot,
         num_routed, slot_weight, part);
   MOE_CHECK_LAUNCH("expert_choice_gating (finish)");
-  choice_loss_kernel<<<1, 64, 0, st>>>(p, part, chunks, loss);
+  choice_loss_kernel<<<1, 256, 0, st>>>(p, part, chunks, loss);
   MOE_CHECK_LAUNCH("expert_choice_gating (loss)");
   return 0;
 }

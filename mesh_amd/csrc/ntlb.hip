@@ -121,7 +121,7 @@ __global__ __launch_bounds__(NTLB_THREADS) void ntlb_assign_kernel(
     int32_t* __restrict__ idx, int32_t* __restrict__ pos,
     float* __restrict__ gate, uint8_t* __restrict__ kept,
     int32_t* __restrict__ fill, float* __restrict__ gsum, int el) {
-  extern __shared__ int32_t smem_i[];
+  extern __shared__ __attribute__((aligned(16))) int32_t smem_i[];
   const int S = p.S, E = p.E, C = p.C, K = p.K;
   int32_t* cnt = smem_i;                          // [nchunks][el]
   int32_t* held = cnt + NTLB_THREADS;             // [el]
@@ -151,15 +151,37 @@ __global__ __launch_bounds__(NTLB_THREADS) void ntlb_assign_kernel(
   const int clen = (S + nchunks - 1) / nchunks;
   const int s_begin = min(S, chunk * clen);
   const int s_end = min(S, s_begin + clen);
+  // 16-byte reads: every array starts 16-byte aligned and a chunk holds whole
+  // groups of eight tokens
+  const bool vec = (el % 4 == 0) && (S % 8 == 0) && (clen % 8 == 0);
   for (int i = 0; i < K; ++i) {
     const int16_t* ch = cand + (size_t)i * S;
     // density_1 of this pass counts every token (moe.py:847 precedes the
     // importance mask), the offers only the open ones
     int all = 0, c = 0;
-    for (int s = s_begin; s < s_end; ++s) {
-      const bool hit = ch[s] == e;
-      all += hit;
-      c += hit && open_[s];
+    if (vec) {
+      // eight tokens per step: one 16-byte read of the candidates, one 8-byte
+      // read of the open flags
+      for (int s = s_begin; s < s_end; s += 8) {
+        const uint4 c8 = *reinterpret_cast<const uint4*>(ch + s);
+        const uint2 o8 = *reinterpret_cast<const uint2*>(open_ + s);
+        const uint32_t cw[4] = {c8.x, c8.y, c8.z, c8.w};
+        const uint32_t ow[2] = {o8.x, o8.y};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int id = (int)(int16_t)((cw[j >> 1] >> (16 * (j & 1))) & 0xffffu);
+          const bool hit = id == e;
+          const bool op = ((ow[j >> 2] >> (8 * (j & 3))) & 0xffu) != 0;
+          all += hit;
+          c += hit && op;
+        }
+      }
+    } else {
+      for (int s = s_begin; s < s_end; ++s) {
+        const bool hit = ch[s] == e;
+        all += hit;
+        c += hit && open_[s];
+      }
     }
     cnt[chunk * el + e] = c;
     __syncthreads();
@@ -173,15 +195,32 @@ __global__ __launch_bounds__(NTLB_THREADS) void ntlb_assign_kernel(
     int running = have + before;
     __syncthreads();            // everybody has read cnt and held
     cnt[chunk * el + e] = all;
-    for (int s = s_begin; s < s_end; ++s) {
-      if (ch[s] == e && open_[s]) {
-        ++running;
-        if (running <= C) {
-          wpass[s] = (uint8_t)i;
-          wpos[s] = (int16_t)(running - 1);
-          open_[s] = 0;
+    // (a token's flags are written by the one thread whose expert is its
+    // candidate in this pass, so reading eight of them ahead is safe)
+    auto offer = [&](int s) {
+      ++running;
+      if (running <= C) {
+        wpass[s] = (uint8_t)i;
+        wpos[s] = (int16_t)(running - 1);
+        open_[s] = 0;
+      }
+    };
+    if (vec) {
+      for (int s = s_begin; s < s_end; s += 8) {
+        const uint4 c8 = *reinterpret_cast<const uint4*>(ch + s);
+        const uint2 o8 = *reinterpret_cast<const uint2*>(open_ + s);
+        const uint32_t cw[4] = {c8.x, c8.y, c8.z, c8.w};
+        const uint32_t ow[2] = {o8.x, o8.y};
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int id = (int)(int16_t)((cw[j >> 1] >> (16 * (j & 1))) & 0xffffu);
+          const bool op = ((ow[j >> 2] >> (8 * (j & 3))) & 0xffu) != 0;
+          if (id == e && op) offer(s + j);
         }
       }
+    } else {
+      for (int s = s_begin; s < s_end; ++s)
+        if (ch[s] == e && open_[s]) offer(s);
     }
     __syncthreads();
     if (chunk == 0) {

@@ -1041,7 +1041,10 @@ def expert_choice_gating(logits, capacity, importance=None, normalize=True,
         slot_token.data_ptr(), slot_weight.data_ptr(), tok_slot.data_ptr(),
         loss.data_ptr(), ws.data_ptr(), ws_bytes, _stream()),
         "expert_choice_gating")
-  return SlotRouting(slot_token, slot_weight, tok_slot, loss, c, e)
+  r = SlotRouting(slot_token, slot_weight, tok_slot, loss, c, e)
+  if _timer is not None:
+    _timer.routing.append(r)
+  return r
 
 
 def slot_dispatch(x, r):
