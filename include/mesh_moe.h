@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 19
+#define MESH_MOE_ABI_VERSION 20
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -686,8 +686,9 @@ size_t mesh_moe_attention_weights_workspace_bytes(int B, int L, int H, int D,
                                                   int dtype);
 int mesh_moe_attention_weights(const void* q, const void* k, void* weights,
                                int B, int L, int H, int D, int causal,
-                               int dtype, void* workspace,
-                               size_t workspace_bytes, void* stream);
+                               const int32_t* sequence_id, int dtype,
+                               void* workspace, size_t workspace_bytes,
+                               void* stream);
 
 /*
  * Dropout whose noise is broadcast over some dimensions of x
@@ -735,10 +736,16 @@ size_t mesh_moe_self_attention_workspace_bytes(int B, int L, int H, int D,
  * a transposed copy of v).  Other cases run the three-step form whose logits
  * and weights of all heads live in the workspace (B*H*L*L*(4 + sizeof dtype)
  * bytes).
+ * sequence_id [B,L] int32 or NULL: with it a query sees only the keys that
+ * carry its own id -- packed sequences and padding (id 0), the visibility
+ * bias of SelfAttention.compute_bias, transformer/transformer_layers.py:303-316;
+ * mesh_moe_attention_weights and mesh_moe_self_attention_backward take the
+ * same argument.
  */
 int mesh_moe_self_attention(const void* q, const void* k, const void* v,
                             void* out, int B, int L, int H, int D, int causal,
-                            int dtype, void* workspace, size_t workspace_bytes,
+                            const int32_t* sequence_id, int dtype,
+                            void* workspace, size_t workspace_bytes,
                             void* stream);
 
 /* Bytes of scratch mesh_moe_self_attention_backward needs; 0 for shapes it does
@@ -768,7 +775,8 @@ size_t mesh_moe_self_attention_backward_workspace_bytes(int B, int L, int H,
 int mesh_moe_self_attention_backward(const void* q, const void* k, const void* v,
                                      const void* dout, void* dq, void* dk,
                                      void* dv, int B, int L, int H, int D,
-                                     int causal, int dtype, void* workspace,
+                                     int causal, const int32_t* sequence_id,
+                                     int dtype, void* workspace,
                                      size_t workspace_bytes, void* stream);
 
 #ifdef __cplusplus

@@ -105,12 +105,15 @@ __device__ __forceinline__ float fa_exp2(float x) {
 // query: lse = log of the softmax denominator (row maximum included) and
 // delta = sum_d dout[q, d] * out[q, d] (= sum_k dweights * weights), both
 // float32 [B*H, L].
-template <int D, bool CAUSAL, bool STATS = false>
+// SEQ: a query sees only the keys that carry its sequence id (seq [B, L];
+// transformer_layers.py:303-316): the ids of a key tile travel through LDS
+// with the tile, a lane keeps its query's id in a register.
+template <int D, bool CAUSAL, bool STATS = false, bool SEQ = false>
 __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
     const bf16_t* __restrict__ v, bf16_t* __restrict__ out, int L, int H,
-    const bf16_t* __restrict__ dout = nullptr, float* __restrict__ lse = nullptr,
-    float* __restrict__ delta = nullptr) {
+    const bf16_t* __restrict__ dout, float* __restrict__ lse,
+    float* __restrict__ delta, const int32_t* __restrict__ seq) {
   using Cfg = FlashCfg<D>;
   extern __shared__ __attribute__((aligned(16))) unsigned char fa_smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -132,6 +135,16 @@ __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
 
   // this lane's query (second MFMA operand of S^T): 8 consecutive d per step
   const int my_q = q0 + wave * 32 + l32;
+  const int32_t* seq_b = SEQ ? seq + (int64_t)b * L : nullptr;
+  int my_sid = 0, own_first = 0;
+  bool own_uniform = true;
+  if constexpr (SEQ) {
+    my_sid = seq_b[min(my_q, L - 1)];
+    own_first = __builtin_amdgcn_readfirstlane(my_sid);
+    own_uniform = __ballot(my_sid != own_first) == 0ull;
+  }
+  // key ids of the two tile stages, behind the K / V ring
+  int32_t* sid_s = reinterpret_cast<int32_t*>(fa_smem + Cfg::LDS_BYTES);
   fa_bf16x8_t qf[Cfg::DS];
   {
     const bf16_t* qr = qb + (int64_t)min(my_q, L - 1) * row_stride + half * 8;
@@ -167,6 +180,12 @@ __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
           (fa_glb_void_t*)src,
           (fa_lds_void_t*)(base + Cfg::K_BYTES + g * 1024), 16, 0, 0);
     }
+    if constexpr (SEQ) {
+      if (wave == 0)
+        __builtin_amdgcn_global_load_lds(
+            (fa_glb_void_t*)(seq_b + min(key0 + lane, L - 1)),
+            (fa_lds_void_t*)(fa_smem + Cfg::LDS_BYTES + buf * 256), 4, 0, 0);
+    }
   };
 
   fa_f32x16_t acc_o[Cfg::DT];
@@ -192,8 +211,15 @@ __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
     // weight comes out 0, which measured faster than skipping)
     // mask: diagonal and last tiles only, behind a branch the tiles in between
     // do not take
-    const bool need_mask =
+    bool need_mask =
         (CAUSAL && key0 + Cfg::BK - 1 > qw_first) || key0 + Cfg::BK > L;
+    const int32_t* sid_t = sid_s + buf * 64;
+    if constexpr (SEQ) {
+      // (wave-uniform: any key of the tile or query of the wavefront with an
+      // id other than the first query's)
+      need_mask = need_mask || !own_uniform ||
+                  __ballot(sid_t[lane] != own_first) != 0ull;
+    }
     {
       const unsigned char* ks = fa_smem + buf * Cfg::STAGE;
       const unsigned char* vs = ks + Cfg::K_BYTES;
@@ -222,10 +248,20 @@ __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
 #pragma unroll
         for (int sub = 0; sub < 2; ++sub) {
 #pragma unroll
-          for (int r = 0; r < 16; ++r) {
-            const int key = key0 + sub * 32 + 8 * (r / 4) + 4 * half + (r % 4);
-            const bool ok = key < L && (!CAUSAL || key <= my_q);
-            if (!ok) acc_s[sub][r] = NEG;
+          for (int r4 = 0; r4 < 4; ++r4) {
+            const int kl = sub * 32 + 8 * r4 + 4 * half;     // key within tile
+            int kid[4] = {0, 0, 0, 0};
+            if constexpr (SEQ) {
+              const int4 i4 = *reinterpret_cast<const int4*>(sid_t + kl);
+              kid[0] = i4.x; kid[1] = i4.y; kid[2] = i4.z; kid[3] = i4.w;
+            }
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+              const int key = key0 + kl + c;
+              const bool ok = key < L && (!CAUSAL || key <= my_q) &&
+                              (!SEQ || kid[c] == my_sid);
+              if (!ok) acc_s[sub][4 * r4 + c] = NEG;
+            }
           }
         }
       }
@@ -237,7 +273,10 @@ __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
       mx = fmaxf(mx, __shfl_xor(mx, 32));
       const float m_new = fmaxf(m_run, mx);
       const float alpha = fa_exp2((m_run - m_new) * LOG2E);
-      const float mneg = -m_new * LOG2E;
+      // (a tile with no visible key before any visible key was met: the
+      // maximum is still the sentinel, and sentinel * log2e - sentinel * log2e
+      // would leave the product's rounding error, ~1e22, as the exponent)
+      const float mneg = m_new > 0.5f * NEG ? -m_new * LOG2E : -INFINITY;
       m_run = m_new;
       float psum = 0.f;
       fa_bf16x8_t pf[4];
@@ -358,25 +397,30 @@ __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
   }
 }
 
+template <int D, bool CAUSAL, bool SEQ>
+static int launch_flash_one(const bf16_t* q, const bf16_t* k, const bf16_t* v,
+                            bf16_t* out, int B, int L, int H,
+                            const int32_t* seq, hipStream_t st) {
+  using Cfg = FlashCfg<D>;
+  constexpr int LDS = Cfg::LDS_BYTES + 512;        // + key ids of two stages
+  dim3 grid((unsigned)((L + Cfg::BQ - 1) / Cfg::BQ), (unsigned)(B * H));
+  auto kern = flash_attention_kernel<D, CAUSAL, false, SEQ>;
+  MOE_ALLOW_LDS(kern, LDS);
+  kern<<<grid, Cfg::THREADS, LDS, st>>>(q, k, v, out, L, H, nullptr, nullptr,
+                                        nullptr, seq);
+  MOE_CHECK_LAUNCH("self_attention (fused)");
+  return 0;
+}
+
 template <int D>
 static int launch_flash(const bf16_t* q, const bf16_t* k, const bf16_t* v,
                         bf16_t* out, int B, int L, int H, int causal,
-                        hipStream_t st) {
-  using Cfg = FlashCfg<D>;
-  dim3 grid((unsigned)((L + Cfg::BQ - 1) / Cfg::BQ), (unsigned)(B * H));
-  if (causal) {
-    auto kern = flash_attention_kernel<D, true>;
-    MOE_ALLOW_LDS(kern, Cfg::LDS_BYTES);
-    kern<<<grid, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(q, k, v, out, L, H, nullptr,
-                                                     nullptr, nullptr);
-  } else {
-    auto kern = flash_attention_kernel<D, false>;
-    MOE_ALLOW_LDS(kern, Cfg::LDS_BYTES);
-    kern<<<grid, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(q, k, v, out, L, H, nullptr,
-                                                     nullptr, nullptr);
-  }
-  MOE_CHECK_LAUNCH("self_attention (fused)");
-  return 0;
+                        const int32_t* seq, hipStream_t st) {
+  if (causal)
+    return seq ? launch_flash_one<D, true, true>(q, k, v, out, B, L, H, seq, st)
+               : launch_flash_one<D, true, false>(q, k, v, out, B, L, H, seq, st);
+  return seq ? launch_flash_one<D, false, true>(q, k, v, out, B, L, H, seq, st)
+             : launch_flash_one<D, false, false>(q, k, v, out, B, L, H, seq, st);
 }
 
 bool flash_attention_supported(int L, int H, int D, int dtype, const void* q,
@@ -393,15 +437,16 @@ size_t flash_attention_workspace_bytes(int B, int L, int H, int D) {
 }
 
 int flash_attention(const void* q, const void* k, const void* v, void* out,
-                    int B, int L, int H, int D, int causal, void* workspace,
+                    int B, int L, int H, int D, int causal,
+                    const int32_t* sequence_id, void* workspace,
                     hipStream_t st) {
   (void)workspace;
   if (D == 128)
     return launch_flash<128>((const bf16_t*)q, (const bf16_t*)k,
                              (const bf16_t*)v, (bf16_t*)out, B, L, H, causal,
-                             st);
+                             sequence_id, st);
   return launch_flash<64>((const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v,
-                          (bf16_t*)out, B, L, H, causal, st);
+                          (bf16_t*)out, B, L, H, causal, sequence_id, st);
 }
 
 // ---------------------------------------------------------------------------
@@ -436,7 +481,7 @@ struct FlashBwdCfg {
   static constexpr int CH = ROW / 16, UNITS = ROW / 64, RPI = 1024 / ROW;
   static constexpr int INSTR = TILE / 1024 / WAVES; // loads per wave and tile copy
   static constexpr int DS = D / 16, DT = D / 32;
-  static constexpr int STATS_BYTES = 2 * BT * 4;    // lse, delta of a query tile
+  static constexpr int STATS_BYTES = 3 * BT * 4;    // lse, delta, sequence ids of a tile
   static constexpr int stage_bytes(int what) {
     return (what == BWD_DV ? 2 : 3) * TILE + STATS_BYTES;
   }
@@ -444,12 +489,12 @@ struct FlashBwdCfg {
   static_assert(INSTR >= 1, "a tile copy is at least one load per wavefront");
 };
 
-template <int D, bool CAUSAL, int WHAT>
+template <int D, bool CAUSAL, int WHAT, bool SEQ>
 __global__ __launch_bounds__(512) void flash_attention_backward_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
     const bf16_t* __restrict__ v, const bf16_t* __restrict__ dout,
     const float* __restrict__ lse, const float* __restrict__ delta,
-    bf16_t* __restrict__ grad, int L, int H) {
+    bf16_t* __restrict__ grad, int L, int H, const int32_t* __restrict__ seq) {
   using Cfg = FlashBwdCfg<D>;
   constexpr bool OWN_Q = WHAT == BWD_DQ;
   constexpr int NCOPY = WHAT == BWD_DV ? 2 : 3;
@@ -498,6 +543,14 @@ __global__ __launch_bounds__(512) void flash_attention_backward_kernel(
     my_lse2 = lse_b[my_c] * LOG2E;
     my_delta = delta_b[my_c];
   }
+  const int32_t* seq_b = SEQ ? seq + (int64_t)b * L : nullptr;
+  int my_sid = 0, own_first = 0;
+  bool own_uniform = true;
+  if constexpr (SEQ) {
+    my_sid = seq_b[my_c];
+    own_first = __builtin_amdgcn_readfirstlane(my_sid);
+    own_uniform = __ballot(my_sid != own_first) == 0ull;
+  }
 
   // one tile copy: rows of `src` from row0, chunk-swizzled for row reads
   // (TR = false) or unit-swizzled for transposing reads (TR = true)
@@ -535,6 +588,12 @@ __global__ __launch_bounds__(512) void flash_attention_backward_kernel(
             (fa_lds_void_t*)(base + NCOPY * Cfg::TILE + wave * 256), 4, 0, 0);
       }
     }
+    if constexpr (SEQ) {
+      if (wave == 2)
+        __builtin_amdgcn_global_load_lds(
+            (fa_glb_void_t*)(seq_b + min(row0 + lane, L - 1)),
+            (fa_lds_void_t*)(base + NCOPY * Cfg::TILE + 512), 4, 0, 0);
+    }
   };
 
   fa_f32x16_t acc[Cfg::DT];
@@ -568,9 +627,14 @@ __global__ __launch_bounds__(512) void flash_attention_backward_kernel(
     const unsigned char* t2r = t1r + 2 * Cfg::TILE;           // BWD_DQ, BWD_DK
     const uint32_t ttr = lds0 + buf * STAGE + Cfg::TILE;      // the copy read transposed
     const float* st = reinterpret_cast<const float*>(t1r + NCOPY * Cfg::TILE);
-    const bool need_mask =
+    bool need_mask =
         (CAUSAL && (OWN_Q ? row0 + Cfg::BT - 1 > ow_first : row0 < ow_last)) ||
         row0 + Cfg::BT > L;
+    const int32_t* sid_t = reinterpret_cast<const int32_t*>(st + 2 * Cfg::BT);
+    if constexpr (SEQ) {
+      need_mask = need_mask || !own_uniform ||
+                  __ballot(sid_t[lane] != own_first) != 0ull;
+    }
 
     auto do_sub = [&](auto sub_c) {
       constexpr int SUB = decltype(sub_c)::value;
@@ -628,10 +692,21 @@ __global__ __launch_bounds__(512) void flash_attention_backward_kernel(
       if (need_mask) {
         asm volatile("" ::: "memory");
 #pragma unroll
-        for (int r = 0; r < 16; ++r) {
-          const int sr = row0 + SUB * 32 + 8 * (r / 4) + 4 * half + (r % 4);
-          const bool ok = sr < L && (!CAUSAL || (OWN_Q ? sr <= my : my <= sr));
-          if (!ok) w[r] = 0.f;
+        for (int r4 = 0; r4 < 4; ++r4) {
+          const int jl = SUB * 32 + 8 * r4 + 4 * half;       // row within tile
+          int sid4[4] = {0, 0, 0, 0};
+          if constexpr (SEQ) {
+            const int4 i4 = *reinterpret_cast<const int4*>(sid_t + jl);
+            sid4[0] = i4.x; sid4[1] = i4.y; sid4[2] = i4.z; sid4[3] = i4.w;
+          }
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            const int sr = row0 + jl + c;
+            const bool ok = sr < L &&
+                            (!CAUSAL || (OWN_Q ? sr <= my : my <= sr)) &&
+                            (!SEQ || sid4[c] == my_sid);
+            if (!ok) w[4 * r4 + c] = 0.f;
+          }
         }
       }
       fa_bf16x8_t wf[2];
@@ -697,43 +772,45 @@ __global__ __launch_bounds__(512) void flash_attention_backward_kernel(
   }
 }
 
-template <int D, bool CAUSAL, int WHAT>
+template <int D, bool CAUSAL, int WHAT, bool SEQ>
 static int launch_flash_backward_one(const bf16_t* q, const bf16_t* k,
                                      const bf16_t* v, const bf16_t* dout,
                                      const float* lse, const float* delta,
                                      bf16_t* grad, int B, int L, int H,
-                                     hipStream_t st) {
+                                     const int32_t* seq, hipStream_t st) {
   using Cfg = FlashBwdCfg<D>;
   constexpr int LDS = 2 * Cfg::stage_bytes(WHAT);
   dim3 grid((unsigned)((L + Cfg::BOWN - 1) / Cfg::BOWN), (unsigned)(B * H));
-  auto kern = flash_attention_backward_kernel<D, CAUSAL, WHAT>;
+  auto kern = flash_attention_backward_kernel<D, CAUSAL, WHAT, SEQ>;
   MOE_ALLOW_LDS(kern, LDS);
-  kern<<<grid, Cfg::THREADS, LDS, st>>>(q, k, v, dout, lse, delta, grad, L, H);
+  kern<<<grid, Cfg::THREADS, LDS, st>>>(q, k, v, dout, lse, delta, grad, L, H,
+                                        seq);
   MOE_CHECK_LAUNCH("self_attention_backward (fused)");
   return 0;
 }
 
-template <int D, bool CAUSAL>
+template <int D, bool CAUSAL, bool SEQ>
 static int launch_flash_backward(const bf16_t* q, const bf16_t* k,
                                  const bf16_t* v, const bf16_t* dout,
                                  bf16_t* dq, bf16_t* dk, bf16_t* dv, float* lse,
                                  float* delta, int B, int L, int H,
-                                 hipStream_t st) {
+                                 const int32_t* seq, hipStream_t st) {
   using Cfg = FlashCfg<D>;
+  constexpr int LDS = Cfg::LDS_BYTES + 512;
   dim3 grid((unsigned)((L + Cfg::BQ - 1) / Cfg::BQ), (unsigned)(B * H));
-  auto stats = flash_attention_kernel<D, CAUSAL, true>;
-  MOE_ALLOW_LDS(stats, Cfg::LDS_BYTES);
-  stats<<<grid, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(q, k, v, nullptr, L, H, dout,
-                                                    lse, delta);
+  auto stats = flash_attention_kernel<D, CAUSAL, true, SEQ>;
+  MOE_ALLOW_LDS(stats, LDS);
+  stats<<<grid, Cfg::THREADS, LDS, st>>>(q, k, v, nullptr, L, H, dout, lse,
+                                         delta, seq);
   MOE_CHECK_LAUNCH("self_attention_backward (lse, delta)");
-  int rc = launch_flash_backward_one<D, CAUSAL, BWD_DV>(q, k, v, dout, lse, delta,
-                                                        dv, B, L, H, st);
+  int rc = launch_flash_backward_one<D, CAUSAL, BWD_DV, SEQ>(
+      q, k, v, dout, lse, delta, dv, B, L, H, seq, st);
   if (rc != 0) return rc;
-  rc = launch_flash_backward_one<D, CAUSAL, BWD_DK>(q, k, v, dout, lse, delta, dk,
-                                                    B, L, H, st);
+  rc = launch_flash_backward_one<D, CAUSAL, BWD_DK, SEQ>(
+      q, k, v, dout, lse, delta, dk, B, L, H, seq, st);
   if (rc != 0) return rc;
-  return launch_flash_backward_one<D, CAUSAL, BWD_DQ>(q, k, v, dout, lse, delta,
-                                                      dq, B, L, H, st);
+  return launch_flash_backward_one<D, CAUSAL, BWD_DQ, SEQ>(
+      q, k, v, dout, lse, delta, dq, B, L, H, seq, st);
 }
 
 size_t flash_attention_backward_workspace_bytes(int B, int L, int H) {
@@ -743,23 +820,27 @@ size_t flash_attention_backward_workspace_bytes(int B, int L, int H) {
 int flash_attention_backward(const void* q, const void* k, const void* v,
                              const void* dout, void* dq, void* dk, void* dv,
                              int B, int L, int H, int D, int causal,
-                             void* workspace, hipStream_t st) {
+                             const int32_t* sequence_id, void* workspace,
+                             hipStream_t st) {
   float* lse = (float*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
   float* delta = lse + ((((size_t)B * H * L * sizeof(float) + 255) &
                          ~(size_t)255) / sizeof(float));
   const bf16_t *q_ = (const bf16_t*)q, *k_ = (const bf16_t*)k,
                *v_ = (const bf16_t*)v, *d_ = (const bf16_t*)dout;
   bf16_t *dq_ = (bf16_t*)dq, *dk_ = (bf16_t*)dk, *dv_ = (bf16_t*)dv;
-  if (D == 128)
-    return causal ? launch_flash_backward<128, true>(q_, k_, v_, d_, dq_, dk_, dv_,
-                                                     lse, delta, B, L, H, st)
-                  : launch_flash_backward<128, false>(q_, k_, v_, d_, dq_, dk_,
-                                                      dv_, lse, delta, B, L, H,
-                                                      st);
-  return causal ? launch_flash_backward<64, true>(q_, k_, v_, d_, dq_, dk_, dv_,
-                                                  lse, delta, B, L, H, st)
-                : launch_flash_backward<64, false>(q_, k_, v_, d_, dq_, dk_, dv_,
-                                                   lse, delta, B, L, H, st);
+#define MOE_FLASH_BWD(DD, C, S)                                               \
+  launch_flash_backward<DD, C, S>(q_, k_, v_, d_, dq_, dk_, dv_, lse, delta, B, \
+                                  L, H, sequence_id, st)
+  const bool sq = sequence_id != nullptr;
+  if (D == 128) {
+    if (causal) return sq ? MOE_FLASH_BWD(128, true, true)
+                          : MOE_FLASH_BWD(128, true, false);
+    return sq ? MOE_FLASH_BWD(128, false, true) : MOE_FLASH_BWD(128, false, false);
+  }
+  if (causal) return sq ? MOE_FLASH_BWD(64, true, true)
+                        : MOE_FLASH_BWD(64, true, false);
+  return sq ? MOE_FLASH_BWD(64, false, true) : MOE_FLASH_BWD(64, false, false);
+#undef MOE_FLASH_BWD
 }
 
 }  // namespace mesh_moe

@@ -152,29 +152,36 @@ __global__ __launch_bounds__(256) void transpose_heads_kernel(
 // max)).  A key that is not visible carries logit + (-1e9), whose exp is
 // exactly 0 in float32, so it is left out of max and sum.
 // ---------------------------------------------------------------------------
+// With seq [B, L] (rows are (batch, head, query), H heads) a key is visible
+// only if it carries the query's sequence id (transformer_layers.py:303-316).
 template <typename T>
 __global__ __launch_bounds__(256) void attention_softmax_kernel(
     const float* __restrict__ logits, T* __restrict__ weights, int64_t rows,
-    int L, int causal) {
+    int L, int causal, const int32_t* __restrict__ seq, int H) {
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
   const int i = (int)(row % L);
   const int visible = causal ? i + 1 : L;
+  const int32_t* sb = seq ? seq + (row / L / H) * L : nullptr;
+  const int my = sb ? sb[i] : 0;
   const float* xr = logits + row * L;
   float m = -INFINITY;
-  for (int j = lane; j < visible; j += 64) m = fmaxf(m, xr[j]);
+  for (int j = lane; j < visible; j += 64)
+    if (!sb || sb[j] == my) m = fmaxf(m, xr[j]);
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
   const float negm = -m;
   float sum = 0.f;
-  for (int j = lane; j < visible; j += 64) sum += expf(xr[j] + negm);
+  for (int j = lane; j < visible; j += 64)
+    if (!sb || sb[j] == my) sum += expf(xr[j] + negm);
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
   const float neglse = -(logf(sum) + m);
   T* wr = weights + row * L;
   for (int j = lane; j < L; j += 64)
-    store_f32<T>(wr + j, j < visible ? expf(xr[j] + neglse) : 0.0f);
+    store_f32<T>(wr + j, j < visible && (!sb || sb[j] == my)
+                             ? expf(xr[j] + neglse) : 0.0f);
 }
 
 // The same softmax for bf16 weights and rows of ITERS * 512 logits: a lane
@@ -237,8 +244,12 @@ __global__ __launch_bounds__(256) void attention_softmax_rows_kernel(
 template <typename T>
 static void launch_attention_softmax(const float* logits, T* weights,
                                      int64_t rows, int L, int causal,
+                                     const int32_t* seq, int H,
                                      hipStream_t st) {
   const unsigned blocks = (unsigned)((rows + 3) / 4);
+  if (seq != nullptr)
+    return attention_softmax_kernel<T><<<blocks, 256, 0, st>>>(
+        logits, weights, rows, L, causal, seq, H);
   if constexpr (sizeof(T) == 2) {
     const bool aligned =
         (((uintptr_t)logits | (uintptr_t)weights) % 32) == 0;
@@ -256,13 +267,13 @@ static void launch_attention_softmax(const float* logits, T* weights,
           logits, weights, rows, causal);
   }
   attention_softmax_kernel<T><<<blocks, 256, 0, st>>>(logits, weights, rows, L,
-                                                      causal);
+                                                      causal, nullptr, H);
 }
 
 template <typename T>
 static int run_attention(const T* q, const T* k, const T* v, T* out, int B,
-                         int L, int H, int D, int causal, int dtype,
-                         void* workspace, hipStream_t st) {
+                         int L, int H, int D, int causal, const int32_t* seq,
+                         int dtype, void* workspace, hipStream_t st) {
   const int BH = B * H;
   const size_t hd = (size_t)BH * L * D, ll = (size_t)BH * L * L;
   auto up = [](uintptr_t p) { return (p + 255) & ~(uintptr_t)255; };
@@ -285,7 +296,7 @@ static int run_attention(const T* q, const T* k, const T* v, T* out, int B,
   int rc = batched_gemm_nt(qh, kh, logits, BH, L, L, D, dtype, true, st);
   if (rc != 0) return rc;
   const int64_t rows = (int64_t)BH * L;
-  launch_attention_softmax<T>(logits, weights, rows, L, causal, st);
+  launch_attention_softmax<T>(logits, weights, rows, L, causal, seq, H, st);
   MOE_CHECK_LAUNCH("self_attention (softmax)");
   rc = batched_gemm_nt(weights, vt, oh, BH, L, D, L, dtype, false, st);
   if (rc != 0) return rc;
@@ -552,7 +563,8 @@ __global__ __launch_bounds__(256) void softmax_backward_rows_kernel(
 // The attention weights alone, heads to the front: weights [B*H, L, L].
 template <typename T>
 static int run_attention_weights(const T* q, const T* k, T* weights, int B,
-                                 int L, int H, int D, int causal, int dtype,
+                                 int L, int H, int D, int causal,
+                                 const int32_t* seq, int dtype,
                                  void* workspace, hipStream_t st) {
   const int BH = B * H;
   const size_t hd = (size_t)BH * L * D;
@@ -570,7 +582,7 @@ static int run_attention_weights(const T* q, const T* k, T* weights, int B,
   int rc = batched_gemm_nt(qh, kh, logits, BH, L, L, D, dtype, true, st);
   if (rc != 0) return rc;
   const int64_t rows = (int64_t)BH * L;
-  launch_attention_softmax<T>(logits, weights, rows, L, causal, st);
+  launch_attention_softmax<T>(logits, weights, rows, L, causal, seq, H, st);
   MOE_CHECK_LAUNCH("attention_weights (softmax)");
   return 0;
 }
@@ -811,7 +823,8 @@ extern "C" size_t mesh_moe_attention_weights_workspace_bytes(int B, int L,
 
 extern "C" int mesh_moe_attention_weights(const void* q, const void* k,
                                           void* weights, int B, int L, int H,
-                                          int D, int causal, int dtype,
+                                          int D, int causal,
+                                          const int32_t* sequence_id, int dtype,
                                           void* workspace,
                                           size_t workspace_bytes,
                                           void* stream) {
@@ -831,10 +844,12 @@ extern "C" int mesh_moe_attention_weights(const void* q, const void* k,
   if (dtype == MESH_MOE_F32)
     return run_attention_weights<float>((const float*)q, (const float*)k,
                                         (float*)weights, B, L, H, D,
-                                        causal ? 1 : 0, dtype, workspace, st);
+                                        causal ? 1 : 0, sequence_id, dtype,
+                                        workspace, st);
   return run_attention_weights<bf16_t>((const bf16_t*)q, (const bf16_t*)k,
                                        (bf16_t*)weights, B, L, H, D,
-                                       causal ? 1 : 0, dtype, workspace, st);
+                                       causal ? 1 : 0, sequence_id, dtype,
+                                       workspace, st);
 }
 
 extern "C" int mesh_moe_rms_norm(const void* x, const void* scale, void* y,
@@ -881,7 +896,8 @@ extern "C" size_t mesh_moe_self_attention_workspace_bytes(int B, int L, int H,
 
 extern "C" int mesh_moe_self_attention(const void* q, const void* k,
                                        const void* v, void* out, int B, int L,
-                                       int H, int D, int causal, int dtype,
+                                       int H, int D, int causal,
+                                       const int32_t* sequence_id, int dtype,
                                        void* workspace, size_t workspace_bytes,
                                        void* stream) {
   MOE_REQUIRE(q && k && v && out && workspace, MESH_MOE_E_ARG,
@@ -903,16 +919,18 @@ extern "C" int mesh_moe_self_attention(const void* q, const void* k,
     MOE_REQUIRE(flash_attention_supported(L, H, D, dtype, q, k, v, out),
                 MESH_MOE_E_UNSUPPORTED,
                 "self_attention: q, k, v, out must be 16-byte aligned");
-    return flash_attention(q, k, v, out, B, L, H, D, causal ? 1 : 0, workspace,
-                           st);
+    return flash_attention(q, k, v, out, B, L, H, D, causal ? 1 : 0,
+                           sequence_id, workspace, st);
   }
   if (dtype == MESH_MOE_F32)
     return run_attention<float>((const float*)q, (const float*)k,
                                 (const float*)v, (float*)out, B, L, H, D,
-                                causal ? 1 : 0, dtype, workspace, st);
+                                causal ? 1 : 0, sequence_id, dtype, workspace,
+                                st);
   return run_attention<bf16_t>((const bf16_t*)q, (const bf16_t*)k,
                                (const bf16_t*)v, (bf16_t*)out, B, L, H, D,
-                               causal ? 1 : 0, dtype, workspace, st);
+                               causal ? 1 : 0, sequence_id, dtype, workspace,
+                               st);
 }
 
 extern "C" size_t mesh_moe_self_attention_backward_workspace_bytes(int B, int L,
@@ -927,8 +945,9 @@ extern "C" size_t mesh_moe_self_attention_backward_workspace_bytes(int B, int L,
 
 extern "C" int mesh_moe_self_attention_backward(
     const void* q, const void* k, const void* v, const void* dout, void* dq,
-    void* dk, void* dv, int B, int L, int H, int D, int causal, int dtype,
-    void* workspace, size_t workspace_bytes, void* stream) {
+    void* dk, void* dv, int B, int L, int H, int D, int causal,
+    const int32_t* sequence_id, int dtype, void* workspace,
+    size_t workspace_bytes, void* stream) {
   MOE_REQUIRE(q && k && v && dout && dq && dk && dv && workspace, MESH_MOE_E_ARG,
               "self_attention_backward: null pointer");
   MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG,
@@ -948,5 +967,6 @@ extern "C" int mesh_moe_self_attention_backward(
   MOE_REQUIRE(workspace_bytes >= flash_attention_backward_workspace_bytes(B, L, H),
               MESH_MOE_E_ARG, "self_attention_backward: workspace too small");
   return flash_attention_backward(q, k, v, dout, dq, dk, dv, B, L, H, D,
-                                  causal ? 1 : 0, workspace, (hipStream_t)stream);
+                                  causal ? 1 : 0, sequence_id, workspace,
+                                  (hipStream_t)stream);
 }

@@ -24,13 +24,15 @@ bool flash_attention_supported(int L, int H, int D, int dtype, const void* q,
                                const void* k, const void* v, const void* out);
 size_t flash_attention_workspace_bytes(int B, int L, int H, int D);
 int flash_attention(const void* q, const void* k, const void* v, void* out,
-                    int B, int L, int H, int D, int causal, void* workspace,
+                    int B, int L, int H, int D, int causal,
+                    const int32_t* sequence_id, void* workspace,
                     hipStream_t st);
 size_t flash_attention_backward_workspace_bytes(int B, int L, int H);
 int flash_attention_backward(const void* q, const void* k, const void* v,
                              const void* dout, void* dq, void* dk, void* dv,
                              int B, int L, int H, int D, int causal,
-                             void* workspace, hipStream_t st);
+                             const int32_t* sequence_id, void* workspace,
+                             hipStream_t st);
 
 #define MOE_REQUIRE(cond, code, ...)      \
   do {                                    \

@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 19
+ABI_VERSION = 20
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -128,7 +128,7 @@ _SIGNATURES = {
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "mesh_moe_attention_weights": (ctypes.c_int, [
         _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
-        ctypes.c_int, ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
+        ctypes.c_int, _vp, ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
     "mesh_moe_broadcast_dropout": (ctypes.c_int, [
         _vp, _vp, _vp, ctypes.c_float, _vp, _vp, ctypes.c_int64, ctypes.c_int64,
         ctypes.c_int64, ctypes.c_int, _vp]),
@@ -182,12 +182,13 @@ _SIGNATURES = {
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "mesh_moe_self_attention": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
-        ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
+        ctypes.c_int, ctypes.c_int, _vp, ctypes.c_int, _vp, ctypes.c_size_t,
+        _vp]),
     "mesh_moe_self_attention_backward_workspace_bytes": (ctypes.c_size_t, [
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "mesh_moe_self_attention_backward": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
-        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, ctypes.c_int, _vp,
         ctypes.c_size_t, _vp]),
 }
 EXPORTS = sorted(_SIGNATURES)
@@ -1131,9 +1132,11 @@ def dense(x, w_packed, activation=None):
   return y.reshape(tuple(x.shape[:-1]) + (n,))
 
 
-def self_attention(q, k, v, num_heads, causal):
+def self_attention(q, k, v, num_heads, causal, sequence_id=None):
   """q, k, v [B, L, H*D] -> [B, L, H*D] (attention.attention with float32
-  logits, transformer/attention.py:27-88)."""
+  logits, transformer/attention.py:27-88); sequence_id [B, L] int32 or None:
+  a query sees only keys of its own sequence
+  (transformer/transformer_layers.py:303-316)."""
   lib = load_library()
   b, l, hd = q.shape
   if hd % num_heads:
@@ -1149,8 +1152,8 @@ def self_attention(q, k, v, num_heads, causal):
     _check(lib.mesh_moe_self_attention(
         _dev(q, "q"), _dev(k, "k", q.dtype, (b, l, hd)),
         _dev(v, "v", q.dtype, (b, l, hd)), out.data_ptr(), b, l, num_heads, d,
-        int(bool(causal)), code, ws.data_ptr(), ws_bytes, _stream()),
-        "self_attention")
+        int(bool(causal)), _sequence_id_ptr(sequence_id, b, l), code,
+        ws.data_ptr(), ws_bytes, _stream()), "self_attention")
   return out
 
 
@@ -1257,8 +1260,16 @@ def dense_backward(x, w, dy, y=None, want_dx=True):
   return (dx.reshape(x.shape) if want_dx else None), dw.reshape(k, n)
 
 
-def attention_weights(q, k, num_heads, causal):
-  """q, k [B, L, H*D] -> softmax(q . k + visibility) [B*H, L, L] in q's dtype."""
+def _sequence_id_ptr(sequence_id, b, l):
+  """Device pointer of sequence ids [B, L] int32, or None."""
+  if sequence_id is None:
+    return None
+  return _dev(sequence_id, "sequence_id", torch.int32, (b, l))
+
+
+def attention_weights(q, k, num_heads, causal, sequence_id=None):
+  """q, k [B, L, H*D] -> softmax(q . k + visibility) [B*H, L, L] in q's dtype;
+  sequence_id [B, L] int32: keys of other sequences are not visible."""
   lib = load_library()
   b, l, hd = q.shape
   d = hd // num_heads
@@ -1270,8 +1281,8 @@ def attention_weights(q, k, num_heads, causal):
   with _stage("attention_weights"):
     _check(lib.mesh_moe_attention_weights(
         _dev(q, "q"), _dev(k, "k", q.dtype, (b, l, hd)), weights.data_ptr(), b,
-        l, num_heads, d, 1 if causal else 0, code, ws.data_ptr(), ws_bytes,
-        _stream()), "attention_weights")
+        l, num_heads, d, 1 if causal else 0, _sequence_id_ptr(sequence_id, b, l),
+        code, ws.data_ptr(), ws_bytes, _stream()), "attention_weights")
   return weights
 
 
@@ -1289,7 +1300,8 @@ def softmax_backward(weights, dweights):
   return out
 
 
-def self_attention_backward(q, k, v, dout, num_heads, causal, fused=None):
+def self_attention_backward(q, k, v, dout, num_heads, causal, fused=None,
+                            sequence_id=None):
   """Backward of self_attention: q, k, v, dout [B, L, H*D] -> (dq, dk, dv).
   Shapes the fused kernels take (bf16, d_kv 64 or 128, L a multiple of 8) run
   mesh_moe_self_attention_backward: nothing [L, L] reaches memory.  Otherwise
@@ -1318,8 +1330,9 @@ def self_attention_backward(q, k, v, dout, num_heads, causal, fused=None):
             _dev(q, "q"), _dev(k, "k", q.dtype, (b, l, hd)),
             _dev(v, "v", q.dtype, (b, l, hd)),
             _dev(dout, "dout", q.dtype, (b, l, hd)), dq.data_ptr(),
-            dk.data_ptr(), dv.data_ptr(), b, l, h, d, int(bool(causal)), code,
-            ws.data_ptr(), ws_bytes, _stream()), "self_attention_backward")
+            dk.data_ptr(), dv.data_ptr(), b, l, h, d, int(bool(causal)),
+            _sequence_id_ptr(sequence_id, b, l), code, ws.data_ptr(), ws_bytes,
+            _stream()), "self_attention_backward")
       return dq, dk, dv
     if fused:
       raise MoeHipError("self_attention_backward: the fused kernels do not take "
@@ -1331,7 +1344,7 @@ def self_attention_backward(q, k, v, dout, num_heads, causal, fused=None):
     return t.reshape(b, h, l, d).permute(0, 2, 1, 3).reshape(b, l, hd) \
         .contiguous()
   qh, kh, vh, doh = (heads_first(t) for t in (q, k, v, dout))
-  weights = attention_weights(q, k, h, causal)
+  weights = attention_weights(q, k, h, causal, sequence_id)
   dweights, dvh = expert_linear_backward(weights, doh, vh)
   dlogits = softmax_backward(weights, dweights)
   del weights, dweights

@@ -80,8 +80,25 @@ def broadcast_dropout(x, noise, axis, act_dtype="float32"):
             act_dtype)
 
 
+def _visibility_bias(l, causal, sequence_id):
+  """Sum of the attention biases of SelfAttention.compute_bias
+  (transformer/transformer_layers.py:272-316) for the options built here, as
+  [B or 1, 1, L(query), L(key)] float32: -1e9 where the key lies after the query
+  (autoregressive, attention.py:830-842) and -1e9 where query and key carry
+  different sequence ids (transformer_layers.py:303-316); the biases add."""
+  bias = np.zeros((1, 1, l, l), F32)
+  if causal:
+    pos = np.arange(l)
+    bias = bias + (pos[None, :] > pos[:, None]).astype(F32)[None, None] * F32(-1e9)
+  if sequence_id is not None:
+    sid = np.asarray(sequence_id)
+    differ = (sid[:, :, None] != sid[:, None, :]).astype(F32)[:, None]
+    bias = bias + differ * F32(-1e9)
+  return bias
+
+
 def self_attention(x, wq, wk, wv, wo, num_heads, causal, act_dtype="float32",
-                   weights_noise=None):
+                   weights_noise=None, sequence_id=None):
   """SelfAttention.call for the train / eval modes with the default options
   (transformer/transformer_layers.py:223-271) around attention.attention with
   float32 logits (transformer/attention.py:27-88).
@@ -103,10 +120,7 @@ def self_attention(x, wq, wk, wv, wo, num_heads, causal, act_dtype="float32",
   k = dense(x, wk, act_dtype).reshape(b, l, num_heads, d)
   v = dense(x, wv, act_dtype).reshape(b, l, num_heads, d)
   logits = np.einsum("blhd,bmhd->bhlm", q, k).astype(F32)        # float32
-  if causal:
-    pos = np.arange(l)
-    hidden = (pos[None, :] > pos[:, None]).astype(F32)           # key > query
-    logits = logits + hidden * F32(-1e9)
+  logits = (logits + _visibility_bias(l, causal, sequence_id)).astype(F32)
   weights = _r(O.softmax(logits), act_dtype)                     # cast to v's
   if weights_noise is not None:
     weights = broadcast_dropout(weights, weights_noise, 2, act_dtype)
@@ -114,16 +128,15 @@ def self_attention(x, wq, wk, wv, wo, num_heads, causal, act_dtype="float32",
   return dense(o.reshape(b, l, hd), wo, act_dtype)
 
 
-def _attention_core(q, k, v, num_heads, causal, act_dtype):
+def _attention_core(q, k, v, num_heads, causal, act_dtype, sequence_id=None):
   """attention.attention with float32 logits (attention.py:27-88) on
-  [B, L, H*D] activation-dtype tensors -> [B, L, H*D]."""
+  [B, L, H*D] activation-dtype tensors -> [B, L, H*D]; sequence_id [B, L]
+  integers or None."""
   b, l, hd = q.shape
   d = hd // num_heads
   q, k, v = (t.reshape(b, l, num_heads, d) for t in (q, k, v))
   logits = np.einsum("blhd,bmhd->bhlm", q, k).astype(F32)
-  if causal:
-    pos = np.arange(l)
-    logits = logits + (pos[None, :] > pos[:, None]).astype(F32) * F32(-1e9)
+  logits = (logits + _visibility_bias(l, causal, sequence_id)).astype(F32)
   weights = _r(O.softmax(logits), act_dtype)
   return _r(np.einsum("bhlm,bmhd->blhd", weights, v), act_dtype).reshape(b, l, hd)
 
@@ -162,7 +175,7 @@ def dense_relu_dense(x, wi, wo, act_dtype="float32", hidden_noise=None):
 
 def layer_stack(x, layers, final_scale, act_dtype="float32",
                 autoregressive=False, train=False, initial_noise=None,
-                final_noise=None):
+                final_noise=None, sequence_id=None):
   """LayerStack.call with the default sublayers (transformer/transformer.py:
   408-428 and the defaults quoted at :346-358): per layer
   dropout(x) first; per layer x + dropout(layer(rms_norm(x))); at the end
@@ -179,33 +192,42 @@ def layer_stack(x, layers, final_scale, act_dtype="float32",
     dense_relu_dense: wi, wo
     moe: w_gate, wi, wo, hparams (an O.HParams); optional num_microbatches
     moe2d: w_outer, w_inner, wi, wo, hparams; optional num_microbatches
+  sequence_id [B, L] integers (0 = padding) or None: every layer's input is
+  multiplied by nonpadding = (sequence_id != 0) (sublayer_mask_padding inside
+  sublayer_call_layer, transformer.py:462-489), attention sees only keys of the
+  query's own sequence, and the MoE layers get nonpadding (moe.py:117).
   Returns (y, losses) with one loss per MoE layer.
   """
   x = _r(x, act_dtype)
+  nonpadding = None
+  if sequence_id is not None:
+    nonpadding = _r((np.asarray(sequence_id) != 0).astype(F32), act_dtype)
   if initial_noise is not None:
     x = broadcast_dropout(x, initial_noise, -2, act_dtype)
   losses = []
   for layer in layers:
     h = rms_norm(x, layer["scale"], act_dtype)
+    if nonpadding is not None:
+      h = _r(h * nonpadding[..., None], act_dtype)
     kind = layer["kind"]
     if kind == "attention":
       y = self_attention(h, layer["wq"], layer["wk"], layer["wv"], layer["wo"],
                          layer["num_heads"], autoregressive, act_dtype,
-                         layer.get("weights_noise"))
+                         layer.get("weights_noise"), sequence_id)
     elif kind == "dense_relu_dense":
       y = dense_relu_dense(h, layer["wi"], layer["wo"], act_dtype,
                            layer.get("hidden_noise"))
     elif kind == "moe":
       y, loss, _ = O.moe_layer_v1(
           h, layer["w_gate"], layer["wi"], layer["wo"], layer["hparams"],
-          train, act_dtype, num_microbatches=layer.get("num_microbatches"),
-          dense=False)
+          train, act_dtype, nonpadding=nonpadding,
+          num_microbatches=layer.get("num_microbatches"), dense=False)
       losses.append(loss)
     elif kind == "moe2d":
       # MoE2D.call -> transformer_moe_layer_v2 (transformer/moe.py:163-188)
       y, loss, _ = O.moe_layer_v2(
           h, layer["w_outer"], layer["w_inner"], layer["wi"], layer["wo"],
-          layer["hparams"], train, act_dtype,
+          layer["hparams"], train, act_dtype, nonpadding=nonpadding,
           num_microbatches=layer.get("num_microbatches"), dense=False)
       losses.append(loss)
     else:
@@ -257,7 +279,7 @@ def dense_backward(x, w, dy, act_dtype="float32", activation=None):
 
 
 def attention_core_backward(q, k, v, dout, num_heads, causal,
-                            act_dtype="float32"):
+                            act_dtype="float32", sequence_id=None):
   """(dq, dk, dv) of _attention_core on [B, L, H*D] tensors: the weights as
   the forward pass rounds them; dweights = dout v^T, dv = weights^T dout,
   dlogits = weights (dweights - sum_k dweights weights), dq = dlogits k,
@@ -267,9 +289,7 @@ def attention_core_backward(q, k, v, dout, num_heads, causal,
   q, k, v, dout = (_r(t, act_dtype).reshape(b, l, num_heads, d)
                    for t in (q, k, v, dout))
   logits = np.einsum("blhd,bmhd->bhlm", q, k).astype(F32)
-  if causal:
-    pos = np.arange(l)
-    logits = logits + (pos[None, :] > pos[:, None]).astype(F32) * F32(-1e9)
+  logits = (logits + _visibility_bias(l, causal, sequence_id)).astype(F32)
   weights = _r(O.softmax(logits), act_dtype)
   dweights = _r(np.einsum("blhd,bmhd->bhlm", dout, v), act_dtype)
   dv = _r(np.einsum("bhlm,blhd->bmhd", weights, dout), act_dtype)

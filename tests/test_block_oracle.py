@@ -98,6 +98,34 @@ def test_self_attention_causality_and_uniform_case():
   np.testing.assert_allclose(out[0], want, rtol=1e-5, atol=1e-5)
 
 
+@pytest.mark.parametrize("causal", [False, True])
+def test_attention_sequence_ids_are_block_diagonal(causal):
+  """With sequence ids over contiguous segments, attention over the packed row
+  equals attention over every segment on its own (what "a query sees only its
+  own sequence" means, transformer_layers.py:303-316), forward and backward."""
+  rng = np.random.default_rng(77 + causal)
+  b, l, heads, d = 2, 24, 2, 4
+  ids = np.array([[1] * 7 + [2] * 9 + [3] * 5 + [0] * 3,
+                  [5] * 12 + [6] * 12], np.int32)
+  q, k, v, do = (rng.standard_normal((b, l, heads * d)).astype(np.float32)
+                 for _ in range(4))
+  got = B._attention_core(q, k, v, heads, causal, "float32", sequence_id=ids)
+  got_b = B.attention_core_backward(q, k, v, do, heads, causal, "float32",
+                                    sequence_id=ids)
+  for i in range(b):
+    for sid in np.unique(ids[i]):
+      seg = np.nonzero(ids[i] == sid)[0]
+      sl = slice(seg[0], seg[-1] + 1)
+      part = lambda t: t[i:i + 1, sl]
+      want = B._attention_core(part(q), part(k), part(v), heads, causal,
+                               "float32")
+      np.testing.assert_allclose(got[i:i + 1, sl], want, rtol=1e-5, atol=1e-6)
+      want_b = B.attention_core_backward(part(q), part(k), part(v), part(do),
+                                         heads, causal, "float32")
+      for g_, w_ in zip(got_b, want_b):
+        np.testing.assert_allclose(g_[i:i + 1, sl], w_, rtol=1e-5, atol=1e-6)
+
+
 def test_self_attention_bf16_close_to_float32():
   rng = np.random.default_rng(6)
   b, l, m, heads, d = 2, 16, 32, 2, 8

@@ -126,6 +126,70 @@ def test_attention_core_helper_is_the_oracle():
         B.self_attention(x, eye, eye, eye, eye, heads, causal))
 
 
+def _packed_sequence_ids(rng, b, l, mean_len):
+  """Packed sequences: ids 1, 2, ... over contiguous segments of random length,
+  then a tail of padding (id 0) in every second batch entry."""
+  ids = np.zeros((b, l), np.int32)
+  for i in range(b):
+    pos, sid = 0, 1
+    stop = l if i % 2 == 0 else max(1, l - int(rng.integers(1, max(2, l // 4))))
+    while pos < stop:
+      n = int(rng.integers(1, 2 * mean_len))
+      ids[i, pos:min(stop, pos + n)] = sid
+      pos += n
+      sid += 1
+  return ids
+
+
+@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("case", [(2, 40, 2, 16, 5), (2, 200, 2, 64, 37),
+                                  (3, 328, 1, 128, 90), (2, 1000, 2, 128, 300),
+                                  (1, 776, 2, 64, 20)],
+                         ids=lambda c: "x".join(map(str, c)))
+def test_self_attention_sequence_ids(hip, case, causal, act_dtype):
+  """Packed / padded sequences (sequence ids, transformer_layers.py:303-316):
+  forward and backward of the attention core against the oracle, through the
+  fused kernels (bf16, d_kv 64 / 128) and the three-step form."""
+  b, l, heads, d, mean_len = case
+  rng = np.random.default_rng(sum(case) + causal)
+  ids = _packed_sequence_ids(rng, b, l, mean_len)
+  mk = lambda: O.cast_act(
+      (rng.standard_normal((b, l, heads * d)) * 0.5).astype(np.float32),
+      act_dtype)
+  q, k, v, do = mk(), mk(), mk(), mk()
+  g = lambda a: H.to_gpu(a, act_dtype)
+  sid = torch.from_numpy(ids).cuda()
+  got = H.to_np(hip.self_attention(g(q), g(k), g(v), heads, causal,
+                                   sequence_id=sid))
+  want = B._attention_core(q, k, v, heads, causal, act_dtype, sequence_id=ids)
+  tol = _tol(act_dtype)
+  if act_dtype == "float32":
+    tol = dict(rtol=1e-4, atol=1e-4)
+  np.testing.assert_allclose(got, want, **tol)
+  # a token never sees another sequence: changing the other sequences' keys
+  # and values leaves its output bits unchanged
+  k2, v2 = k.copy(), v.copy()
+  other = ids != ids[:, :1]
+  k2[other] = O.cast_act(k2[other] * np.float32(-1.5) + np.float32(0.25), act_dtype)
+  v2[other] = O.cast_act(v2[other] + np.float32(1.0), act_dtype)
+  got2 = H.to_np(hip.self_attention(g(q), g(k2), g(v2), heads, causal,
+                                    sequence_id=sid))
+  np.testing.assert_array_equal(got2[~other], got[~other])
+  want_b = B.attention_core_backward(q, k, v, do, heads, causal, act_dtype,
+                                     sequence_id=ids)
+  btol = dict(rtol=2e-4, atol=2e-4) if act_dtype == "float32" else dict(
+      rtol=3e-2, atol=3e-2)
+  for fused in ((None, False) if act_dtype == "bfloat16" else (None,)):
+    got_b = hip.self_attention_backward(g(q), g(k), g(v), g(do), heads, causal,
+                                        fused=fused, sequence_id=sid)
+    for gt, wnt, name in zip(got_b, want_b, "qkv"):
+      scale = max(1.0, float(np.abs(wnt).max()))
+      np.testing.assert_allclose(H.to_np(gt), wnt, rtol=btol["rtol"],
+                                 atol=btol["atol"] * scale,
+                                 err_msg="d%s fused=%s" % (name, fused))
+
+
 def test_self_attention_rejections(hip):
   q = torch.zeros((1, 12, 16), dtype=torch.bfloat16, device="cuda")
   with pytest.raises(hip.MoeHipError, match="not divisible"):
