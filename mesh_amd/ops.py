@@ -788,6 +788,14 @@ def cast(x, dtype, name="cast"):
                grad_function=lambda op, dy: [cast(dy, op.inputs[0].dtype)])
 
 
+def not_equal(x, value, name="not_equal"):
+  """x != a Python scalar, as a bool tensor (mesh_tensorflow/ops.py:2121-2123
+  for this case)."""
+  if isinstance(value, Tensor):
+    raise NotImplementedError("not_equal of two Tensors")
+  return cwise(lambda t: t != value, [x], output_dtype=torch.bool, name=name)
+
+
 def to_float(x, name="to_float"):
   return cast(x, float32, name=name)
 
@@ -834,12 +842,29 @@ def add(x1, x2, output_shape=None, name=None):
 
 def multiply(x1, x2, output_shape=None, name=None):
   """Tensor * Python scalar (ScalarMultiplyOperation,
-  mesh_tensorflow/ops.py:2006-2023)."""
+  mesh_tensorflow/ops.py:2006-2023), or Tensor * Tensor where the dims of the
+  smaller one are a subsequence of the larger one's and the smaller one is a
+  constant of the graph (a mask: no gradient flows into it)."""
   del output_shape
   if isinstance(x2, Tensor) and not isinstance(x1, Tensor):
     x1, x2 = x2, x1
   if isinstance(x2, Tensor):
-    raise NotImplementedError("Tensor * Tensor is not part of this subset")
+    big, small = (x1, x2) if x1.shape.ndims >= x2.shape.ndims else (x2, x1)
+    names = big.shape.dimension_names
+    if any(d not in big.shape.dims for d in small.shape.dims):
+      raise ValueError("cannot broadcast %s to %s" % (small.shape, big.shape))
+    order = [names.index(d.name) for d in small.shape.dims]
+    if order != sorted(order):
+      raise ValueError("dimension order differs: %s vs %s"
+                       % (small.shape, big.shape))
+    view = [d.size if d in small.shape.dims else 1 for d in big.shape.dims]
+
+    def fn(a, b):
+      return a * b.reshape(view).to(a.dtype)
+    return slicewise(
+        fn, [big, small], output_shape=big.shape, output_dtype=big.dtype,
+        name=name or "mul",
+        grad_function=lambda op, dy: [multiply(dy, op.inputs[1]), None])
   c = _scalar_in(x1.dtype, x2)
   return cwise(lambda t: t * c, [x1], name=name or "scalar_mul",
                grad_function=lambda op, dy: [multiply(dy, x2)])

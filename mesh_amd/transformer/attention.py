@@ -4,6 +4,8 @@ SelfAttention uses by default: heads and d_kv combined in the variables
 (combine_dims, attention.py:410-414), separate k and v, float32 logits.
 """
 
+import torch
+
 from mesh_amd import layers as mtf_layers
 from mesh_amd import ops as mtf
 
@@ -182,16 +184,24 @@ class SelfAttentionOperation(mtf.Operation):
   """attention.attention (attention.py:27-88) on combined-dim tensors
   q, k, v [batch..., length, heads * d_kv]: float32 logits, an optional
   autoregressive visibility mask, float32 softmax, weights in the activation
-  dtype, weights . v."""
+  dtype, weights . v.  sequence_id [batch..., length] (int32) restricts a
+  query to the keys of its own sequence (the bias of
+  transformer_layers.py:303-316)."""
 
-  def __init__(self, q, k, v, num_heads, causal, name=None):
-    super(SelfAttentionOperation, self).__init__([q, k, v],
+  def __init__(self, q, k, v, num_heads, causal, sequence_id=None, name=None):
+    inputs = [q, k, v] + ([] if sequence_id is None else [sequence_id])
+    super(SelfAttentionOperation, self).__init__(inputs,
                                                  name=name or "attention")
     if q.shape != k.shape or q.shape != v.shape:
       raise ValueError("q, k, v shapes differ: %s %s %s"
                        % (q.shape, k.shape, v.shape))
+    if sequence_id is not None and (
+        sequence_id.shape.dims != q.shape.dims[:-1]):
+      raise ValueError("sequence_id %s does not match q %s"
+                       % (sequence_id.shape, q.shape))
     self._num_heads = num_heads
     self._causal = bool(causal)
+    self._has_ids = sequence_id is not None
     self._outputs = [mtf.Tensor(self, q.shape, q.dtype)]
 
   def lower(self, lowering):
@@ -201,16 +211,20 @@ class SelfAttentionOperation(mtf.Operation):
     length, channels = sizes[-2], sizes[-1]
     heads, causal = self._num_heads, self._causal
 
-    def fn(q, k, v):
+    def fn(q, k, v, ids=None):
       q3, k3, v3 = (t.reshape(-1, length, channels).contiguous()
                     for t in (q, k, v))
-      return moe_hip.self_attention(q3, k3, v3, heads, causal).reshape(sizes)
+      if ids is not None:
+        ids = ids.reshape(-1, length).to(torch.int32).contiguous()
+      return moe_hip.self_attention(q3, k3, v3, heads, causal,
+                                    sequence_id=ids).reshape(sizes)
     lowering.set_tensor_lowering(
         self.outputs[0],
         mesh_impl.slicewise(fn, *[lowering.tensors[t] for t in self.inputs]))
 
   def gradient(self, grad_ys):
-    return list(SelfAttentionGradOperation(self, grad_ys[0]).outputs)
+    grads = list(SelfAttentionGradOperation(self, grad_ys[0]).outputs)
+    return grads + [None] * (len(self.inputs) - 3)
 
 
 class SelfAttentionGradOperation(mtf.Operation):
@@ -219,9 +233,10 @@ class SelfAttentionGradOperation(mtf.Operation):
   the weights recomputed."""
 
   def __init__(self, forward, dout, name=None):
-    q, k, v = forward.inputs
+    q, k, v = forward.inputs[:3]
     super(SelfAttentionGradOperation, self).__init__(
-        [dout, q, k, v], name=name or "attention_grad")
+        [dout, q, k, v] + list(forward.inputs[3:]),
+        name=name or "attention_grad")
     self._num_heads = forward._num_heads   # pylint: disable=protected-access
     self._causal = forward._causal         # pylint: disable=protected-access
     self._outputs = [mtf.Tensor(self, t.shape, t.dtype, index=i)
@@ -234,11 +249,13 @@ class SelfAttentionGradOperation(mtf.Operation):
     length, channels = sizes[-2], sizes[-1]
     heads, causal = self._num_heads, self._causal
 
-    def fn(dout, q, k, v):
+    def fn(dout, q, k, v, ids=None):
       d3, q3, k3, v3 = (t.reshape(-1, length, channels).contiguous()
                         for t in (dout, q, k, v))
+      if ids is not None:
+        ids = ids.reshape(-1, length).to(torch.int32).contiguous()
       return tuple(t.reshape(sizes) for t in moe_hip.self_attention_backward(
-          q3, k3, v3, d3, heads, causal))
+          q3, k3, v3, d3, heads, causal, sequence_id=ids))
     grads = mesh_impl.slicewise(
         fn, *[lowering.tensors[t] for t in self.inputs])
     for out, value in zip(self.outputs, grads):

@@ -4,8 +4,8 @@ LayerStack with its sublayers (RMS norm, layer call, dropout, residual,
 padding mask), make_layer_stack, and the layer-stack call of Unitransformer.
 
 Not here: embeddings, vocabularies, logits and losses of Unitransformer /
-Bitransformer, decoding ("first_part" / "incremental" modes), dropout while
-training, ensembles, packed sequences (sequence_id tensors).
+Bitransformer, decoding ("first_part" / "incremental" modes), ensembles,
+subsequence ids.
 """
 
 from mesh_amd import layers as mtf_layers
@@ -53,8 +53,9 @@ _UNUSED_CONTEXT_FIELDS = (
 class Context(object):
   """What layers need at call time (transformer.py:107-311), for the "train"
   and "eval" modes.  read_priority / write_priority are None (every position
-  sees every position) or POSITION (autoregressive); sequence_id is None or 1
-  (no padding).  The reference's remaining constructor arguments
+  sees every position) or POSITION (autoregressive); sequence_id is None, 1
+  (no padding) or an int32 Tensor [batch..., length] (packed sequences; 0 marks
+  padding).  The reference's remaining constructor arguments
   (_UNUSED_CONTEXT_FIELDS) are accepted as keywords and must be None."""
 
   def __init__(self, model, mesh, batch_dims, length_dim, variable_dtype,
@@ -98,13 +99,16 @@ class Context(object):
   @property
   def nonpadding(self):
     """Zeros in padding positions and ones elsewhere (transformer.py:297-306):
-    None without a sequence_id, the integer 1 when sequence_id == 1."""
+    None without a sequence_id, the integer 1 when sequence_id == 1, else
+    cast(sequence_id != 0, activation dtype) (built once per context)."""
     if self.sequence_id is None:
       return None
     if isinstance(self.sequence_id, int) and self.sequence_id == 1:
       return 1
-    raise NotImplementedError("sequence_id tensors (packed or padded "
-                              "sequences) are not implemented")
+    if "nonpadding" not in self.cache:
+      self.cache["nonpadding"] = mtf.cast(
+          mtf.not_equal(self.sequence_id, 0), self.activation_dtype)
+    return self.cache["nonpadding"]
 
 
 class RmsNormOperation(mtf.Operation):
@@ -173,7 +177,7 @@ def sublayer_mask_padding(x, layer_stack, context):
   sequence_id tensor there is nothing to mask."""
   del layer_stack
   if isinstance(context.sequence_id, mtf.Tensor):
-    raise NotImplementedError("sequence_id tensors are not implemented")
+    return x * context.nonpadding
   return x
 
 

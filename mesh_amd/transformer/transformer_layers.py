@@ -101,9 +101,11 @@ class SelfAttention(transformer.TransformerLayer):
   def call(self, context, x, losses=None):
     """transformer_layers.py:223-271 for the train / eval modes."""
     del losses
-    if isinstance(context.sequence_id, mtf.Tensor) or isinstance(
-        context.subsequence_id, mtf.Tensor):
-      raise NotImplementedError("sequence_id tensors are not implemented")
+    if isinstance(context.subsequence_id, mtf.Tensor):
+      raise NotImplementedError("subsequence_id tensors are not implemented")
+    # a query sees only its own sequence (transformer_layers.py:303-316)
+    sequence_id = (context.sequence_id
+                   if isinstance(context.sequence_id, mtf.Tensor) else None)
     params = self.make_params(context)
     q = params.compute_q(x)
     if self.shared_kv:                       # transformer_layers.py:246-249
@@ -115,8 +117,8 @@ class SelfAttention(transformer.TransformerLayer):
     causal = context.read_priority is transformer.POSITION
     if context.train and self.dropout_rate != 0.0:
       v = self._attention_dropout(context, v, params.num_heads)
-    o = attention.SelfAttentionOperation(q, k, v, params.num_heads,
-                                         causal).outputs[0]
+    o = attention.SelfAttentionOperation(q, k, v, params.num_heads, causal,
+                                         sequence_id=sequence_id).outputs[0]
     return params.compute_output(o, output_shape=x.shape)
 
 

@@ -194,8 +194,9 @@ def layer_stack(x, layers, final_scale, act_dtype="float32",
     moe2d: w_outer, w_inner, wi, wo, hparams; optional num_microbatches
   sequence_id [B, L] integers (0 = padding) or None: every layer's input is
   multiplied by nonpadding = (sequence_id != 0) (sublayer_mask_padding inside
-  sublayer_call_layer, transformer.py:462-489), attention sees only keys of the
-  query's own sequence, and the MoE layers get nonpadding (moe.py:117).
+  sublayer_call_layer, transformer.py:462-489) and so is the stack's output
+  (transformer.py:424), attention sees only keys of the query's own sequence,
+  and the MoE layers get nonpadding (moe.py:117).
   Returns (y, losses) with one loss per MoE layer.
   """
   x = _r(x, act_dtype)
@@ -238,6 +239,8 @@ def layer_stack(x, layers, final_scale, act_dtype="float32",
   y = rms_norm(x, final_scale, act_dtype)
   if final_noise is not None:
     y = broadcast_dropout(y, final_noise, -2, act_dtype)
+  if nonpadding is not None:                       # transformer.py:424
+    y = _r(y * nonpadding[..., None], act_dtype)
   return y, losses
 
 

@@ -190,6 +190,40 @@ def test_layer_stack_by_hand_and_zero_kernels():
   np.testing.assert_array_equal(y0, B.rms_norm(x, final))
 
 
+def test_layer_stack_sequence_ids_by_hand():
+  """Where the padding mask sits (transformer.py:462-489, :424): on every
+  layer's input after its norm and on the stack's output, not on the residual
+  stream; the experts get nonpadding as importance."""
+  rng = np.random.default_rng(8)
+  b, l, m = 2, 16, 24
+  layers = _stack_weights(rng, m, 4, 32, 2, 8)
+  final = (1 + 0.1 * rng.standard_normal(m)).astype(np.float32)
+  x = rng.standard_normal((b, l, m)).astype(np.float32)
+  ids = np.array([[1] * 6 + [2] * 7 + [0] * 3, [3] * 16], np.int32)
+  npad = (ids != 0).astype(np.float32)
+  y, losses = B.layer_stack(x, layers, final, autoregressive=True,
+                            sequence_id=ids)
+  h = x
+  a = layers[0]
+  h = h + B.self_attention(B.rms_norm(h, a["scale"]) * npad[..., None], a["wq"],
+                           a["wk"], a["wv"], a["wo"], 2, True, sequence_id=ids)
+  mo = layers[1]
+  out, loss, _ = O.moe_layer_v1(B.rms_norm(h, mo["scale"]) * npad[..., None],
+                                mo["w_gate"], mo["wi"], mo["wo"], mo["hparams"],
+                                False, nonpadding=npad, dense=False)
+  h = h + out
+  a = layers[2]
+  h = h + B.self_attention(B.rms_norm(h, a["scale"]) * npad[..., None], a["wq"],
+                           a["wk"], a["wv"], a["wo"], 2, True, sequence_id=ids)
+  f = layers[3]
+  h = h + B.dense_relu_dense(B.rms_norm(h, f["scale"]) * npad[..., None],
+                             f["wi"], f["wo"])
+  np.testing.assert_allclose(y, B.rms_norm(h, final) * npad[..., None],
+                             rtol=1e-6, atol=1e-6)
+  assert losses[0] == loss
+  assert not y[0, -3:].any() and np.abs(h[0, -3:]).min() > 0
+
+
 def test_dropout_noise_arguments():
   """The dropout hooks of the block oracle: noise of ones changes nothing; the
   product against float64; noise on the attention weights (what the reference

@@ -215,7 +215,7 @@ def _build_stack(rng, m, e, hdim, heads, d, group):
 
 
 def _run_stack(x, layers, final, act_dtype, heads, d, e, hdim, group,
-               autoregressive):
+               autoregressive, sequence_id=None, with_gradients=False):
   dt = H.ACT_TORCH[act_dtype]
   b, l, m = x.shape
   graph = mtf.Graph()
@@ -235,8 +235,17 @@ def _run_stack(x, layers, final, act_dtype, heads, d, e, hdim, group,
       num_layers=1, block_scope=False)
   model = transformer.Unitransformer(stack, d_model=m, name="decoder",
                                      autoregressive=autoregressive)
+  ids = None
+  if sequence_id is not None:
+    ids = mtf.import_tf_tensor(mesh, torch.from_numpy(sequence_id),
+                               mtf.Shape(dims[:2]))
   y, losses = model.call_layers(
-      xt, mtf.VariableDType(torch.float32, torch.float32, dt), mode="eval")
+      xt, mtf.VariableDType(torch.float32, torch.float32, dt), mode="eval",
+      sequence_id=ids)
+  grads = []
+  if with_gradients:
+    grads = mtf.gradients([y] + list(losses),
+                          [xt] + [v.outputs[0] for v in graph.trainable_variables])
   init = {"decoder/rms_norm/scale": final}
   for i, layer in enumerate(layers):
     p = "decoder/layer_%03d/" % i
@@ -255,6 +264,8 @@ def _run_stack(x, layers, final, act_dtype, heads, d, e, hdim, group,
   lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()}, initial_values=init)
   out = H.to_np(lowering.export_to_tf_tensor(y))
   loss = [float(H.to_np(lowering.export_to_tf_tensor(t))) for t in losses]
+  if with_gradients:
+    return out, loss, [H.to_np(lowering.export_to_tf_tensor(g)) for g in grads]
   return out, loss
 
 
@@ -272,6 +283,34 @@ def test_layer_stack_float32(autoregressive):
   want, want_loss = B.layer_stack(x, layers, final, "float32", autoregressive)
   np.testing.assert_allclose(got, want, rtol=2e-4, atol=2e-4)
   np.testing.assert_allclose(got_loss, want_loss, rtol=1e-4)
+
+
+@pytest.mark.parametrize("autoregressive", [True, False])
+def test_layer_stack_packed_sequences(autoregressive):
+  """The same block on packed, padded rows (Context.sequence_id): every layer's
+  input is multiplied by nonpadding, attention stays inside a sequence, the
+  experts' router gets nonpadding as importance -- against the oracle; the
+  gradient graph of the packed block lowers and is finite."""
+  b, l, m, e, hdim, heads, d, group = 2, 64, 64, 4, 96, 4, 16, 32
+  rng = np.random.default_rng(23)
+  layers, final = _build_stack(rng, m, e, hdim, heads, d, group)
+  x = rng.standard_normal((b, l, m)).astype(np.float32)
+  ids = np.array([[1] * 20 + [2] * 30 + [3] * 9 + [0] * 5,
+                  [4] * 41 + [5] * 23], np.int32)
+  got, got_loss, grads = _run_stack(x, layers, final, "float32", heads, d, e,
+                                    hdim, group, autoregressive,
+                                    sequence_id=ids, with_gradients=True)
+  want, want_loss = B.layer_stack(x, layers, final, "float32", autoregressive,
+                                  sequence_id=ids)
+  np.testing.assert_allclose(got, want, rtol=2e-4, atol=2e-4)
+  np.testing.assert_allclose(got_loss, want_loss, rtol=1e-4)
+  # not the same as ignoring the ids
+  plain, _ = B.layer_stack(x, layers, final, "float32", autoregressive)
+  assert np.abs(plain - want).max() > 1e-2
+  assert all(np.isfinite(g).all() for g in grads)
+  # the stack's output is zero at the padding positions, and with it the
+  # gradient of their inputs (they only reach other padding positions)
+  assert not got[0, -5:].any() and not grads[0][0, -5:].any()
 
 
 @pytest.mark.parametrize("train", [False, True])
