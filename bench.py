@@ -448,8 +448,12 @@ def main():
                     if args.gating == "top_2" else None),
         "flops_per_launch": flops_per_launch,
         "avg_launch_ms": ffn_ms / 2,
-        "padded_frac": (model["expert_ffn"]["padded_flops"] / 2
-                        / (ffn_ms / 2 * 1e-3) / 1e12) / peak}
+        # fraction counting every slot row, occupied or not; the compacted
+        # path of the single-choice routers does not multiply the empty rows
+        "padded_frac": (None if ("dispatch" not in stages and args.gating in
+                                 ("switch", "switch_max", "ntlb"))
+                        else (model["expert_ffn"]["padded_flops"] / 2
+                              / (ffn_ms / 2 * 1e-3) / 1e12) / peak)}
     result["stages"] = per_stage
     if args.backward:
       bw_ms = stages["expert_ffn_backward"][1] / args.steps
