@@ -459,6 +459,88 @@ __global__ __launch_bounds__(256) void gating_backward_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// The same product on the float32 matrix cores (v_mfma_f32_32x32x2_f32: two
+// tokens per instruction, lanes 0-31 bring the first, lanes 32-63 the second;
+// x as the row operand, dlogits as the column operand, both read as they lie
+// in memory).  Block = 128 kernel rows x 64 experts x 512 tokens, 32 tokens
+// staged in LDS at a time as float32 (rows padded by 32 floats so that the two
+// half-waves hit different banks); a wavefront owns 32 rows x 64 experts.
+// Needs M % 128 == 0, E % 8 == 0 and 16-byte aligned rows.
+// ---------------------------------------------------------------------------
+constexpr int WM_M = 128, WM_TOK = 512, WM_KT = 32;
+typedef float wm_f32x16_t __attribute__((ext_vector_type(16)));
+
+template <typename T>
+__global__ __launch_bounds__(256) void router_wgrad_mfma_kernel(
+    const T* __restrict__ x, const float* __restrict__ dlogits,
+    float* __restrict__ acc_out, int64_t T_tokens, int M, int E) {
+  constexpr int VN = Vec16B<T>::N;            // elements per 16-byte piece
+  __shared__ float xs[WM_KT][WM_M + 32];
+  __shared__ float ds[WM_KT][64 + 32];
+  const int m0 = blockIdx.x * WM_M, e0 = blockIdx.z * 64;
+  const int64_t t0 = (int64_t)blockIdx.y * WM_TOK;
+  const int64_t t1 = t0 + WM_TOK < T_tokens ? t0 + WM_TOK : T_tokens;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, l32 = lane & 31;
+  wm_f32x16_t acc0, acc1;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) { acc0[r] = 0.f; acc1[r] = 0.f; }
+  // staging: thread -> (token row tid / 8, 16 kernel rows / 8 experts)
+  const int sr = tid >> 3, sc = tid & 7;
+  for (int64_t tb = t0; tb < t1; tb += WM_KT) {
+    const int64_t t = tb + sr;
+    float xv[16], dv[8];
+    if (t < t1) {
+      const T* xp = x + t * M + m0 + sc * 16;
+#pragma unroll
+      for (int u = 0; u < 16 / VN; ++u) {
+        float f[VN];
+        unpack16(*reinterpret_cast<const uint4*>(xp + u * VN), f, T());
+#pragma unroll
+        for (int j = 0; j < VN; ++j) xv[u * VN + j] = f[j];
+      }
+      if (e0 + sc * 8 < E) {
+        const float4 a = *reinterpret_cast<const float4*>(dlogits + t * E + e0 + sc * 8);
+        const float4 b = *reinterpret_cast<const float4*>(dlogits + t * E + e0 + sc * 8 + 4);
+        dv[0] = a.x; dv[1] = a.y; dv[2] = a.z; dv[3] = a.w;
+        dv[4] = b.x; dv[5] = b.y; dv[6] = b.z; dv[7] = b.w;
+      } else {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) dv[j] = 0.f;
+      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < 16; ++j) xv[j] = 0.f;
+#pragma unroll
+      for (int j = 0; j < 8; ++j) dv[j] = 0.f;
+    }
+    __syncthreads();                 // the previous batch has been consumed
+#pragma unroll
+    for (int j = 0; j < 16; j += 4)
+      *reinterpret_cast<float4*>(&xs[sr][sc * 16 + j]) =
+          make_float4(xv[j], xv[j + 1], xv[j + 2], xv[j + 3]);
+    *reinterpret_cast<float4*>(&ds[sr][sc * 8]) = make_float4(dv[0], dv[1], dv[2], dv[3]);
+    *reinterpret_cast<float4*>(&ds[sr][sc * 8 + 4]) = make_float4(dv[4], dv[5], dv[6], dv[7]);
+    __syncthreads();
+#pragma unroll
+    for (int ks = 0; ks < WM_KT / 2; ++ks) {
+      const float a = xs[2 * ks + half][wave * 32 + l32];
+      const float b0 = ds[2 * ks + half][l32];
+      const float b1 = ds[2 * ks + half][32 + l32];
+      acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b0, acc0, 0, 0, 0);
+      acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a, b1, acc1, 0, 0, 0);
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int m = m0 + wave * 32 + 8 * (r / 4) + 4 * half + (r % 4);
+    if (e0 + l32 < E) atomicAdd(acc_out + (int64_t)m * E + e0 + l32, acc0[r]);
+    if (e0 + 32 + l32 < E)
+      atomicAdd(acc_out + (int64_t)m * E + e0 + 32 + l32, acc1[r]);
+  }
+}
+
+// ---------------------------------------------------------------------------
 // router projection backward w.r.t. the kernel: dw[m,e] = sum_t x[t,m] *
 // dlogits[t,e], float32.  Block (m tile of 256, chunk of tokens, chunk of 64
 // experts) accumulates 256 x 64 partial sums and adds them to the float32
@@ -772,6 +854,27 @@ extern "C" int mesh_moe_router_backward_weights(const void* x,
   // whole pieces
   const bool vec = ((size_t)M * dtype_size(dtype)) % 16 == 0 && E % 4 == 0 &&
                    bw_aligned16(x) && bw_aligned16(dlogits);
+  if (vec && M % WM_M == 0 && E % 8 == 0) {
+    const int64_t mchunks = (tokens + WM_TOK - 1) / WM_TOK;
+    MOE_REQUIRE(mchunks <= 65535, MESH_MOE_E_UNSUPPORTED,
+                "router_backward_weights: too many tokens (%lld)",
+                (long long)tokens);
+    dim3 mgrid((unsigned)(M / WM_M), (unsigned)mchunks, (unsigned)((E + 63) / 64));
+    if (dtype == MESH_MOE_F32) {
+      router_wgrad_mfma_kernel<float><<<mgrid, 256, 0, st>>>(
+          (const float*)x, dlogits, workspace, tokens, M, E);
+      MOE_CHECK_LAUNCH("router_backward_weights (mfma)");
+      convert_f32_kernel<float><<<fb, 256, 0, st>>>(workspace, (float*)dw_gate, n);
+    } else {
+      router_wgrad_mfma_kernel<bf16_t><<<mgrid, 256, 0, st>>>(
+          (const bf16_t*)x, dlogits, workspace, tokens, M, E);
+      MOE_CHECK_LAUNCH("router_backward_weights (mfma)");
+      convert_f32_kernel<bf16_t><<<fb, 256, 0, st>>>(workspace, (bf16_t*)dw_gate,
+                                                    n);
+    }
+    MOE_CHECK_LAUNCH("router_backward_weights (convert)");
+    return 0;
+  }
   if (dtype == MESH_MOE_F32) {
     router_wgrad_kernel<float><<<grid, 256, 0, st>>>(
         (const float*)x, dlogits, workspace, tokens, M, E, vec);

@@ -74,6 +74,25 @@ def run_backward(hip, x, w, hp, act_dtype, d_out, d_loss, nonpad, mb):
               dwo=H.to_np(dwo), dlogits=H.to_np(dlogits), dgate=H.to_np(dgate))
 
 
+@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape", [(700, 128, 8), (1030, 256, 64), (96, 384, 72),
+                                   (513, 128, 40), (200, 72, 6)])
+def test_router_backward_weights(hip, shape, act_dtype):
+  """dw_gate = x^T . dlogits against a float64 product: the float32
+  matrix-core kernel (M a multiple of 128, E of 8) and the plain one."""
+  t, m, e = shape
+  rng = np.random.default_rng(t + m + e)
+  x = O.cast_act(rng.standard_normal((t, m)).astype(np.float32), act_dtype)
+  dl = (rng.standard_normal((t, e)) * 0.1).astype(np.float32)
+  got = H.to_np(hip.router_backward_weights(
+      H.to_gpu(x, act_dtype), torch.from_numpy(dl).cuda()))
+  want = x.astype(np.float64).T @ dl.astype(np.float64)
+  tol = H.value_tolerance(act_dtype)
+  np.testing.assert_allclose(got, O.cast_act(want.astype(np.float32), act_dtype),
+                             rtol=tol["rtol"],
+                             atol=tol["atol"] * np.abs(want).max())
+
+
 CASES = [
     # gating, G, S, M, H, E, cf, dtype, nonpadding
     ("top_2", 2, 64, 16, 24, 4, 1.0, "float32", True),
