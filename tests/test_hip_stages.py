@@ -359,6 +359,50 @@ def test_router_top2_gating_fused_policies(hip, policy, second_place_loss):
     assert torch.equal(getattr(r, name), getattr(r3, name)), name
 
 
+def test_router_gating_fused_random_shapes(hip):
+  """Differential sweep of the one-launch entries over random shapes (groups,
+  group sizes that are multiples of 128, expert counts that are multiples of 4,
+  capacities from starved to ample, one or several routers, both routers'
+  modes): the routing record must equal, to the bit, what the logits-in
+  entries make of the logits the fused kernel reports.  Shapes with many groups also
+  exercise blocks of different groups finishing in any order."""
+  rng = np.random.default_rng(1234)
+  gen = torch.Generator(device="cuda").manual_seed(99)
+  for trial in range(36):
+    b = int(rng.choice([1, 1, 2, 3]))
+    gpr = int(rng.integers(1, 9))
+    s = 128 * int(rng.integers(1, 9))
+    m = 64 * int(rng.integers(1, 5))
+    e = 4 * int(rng.integers(1, 33))
+    c = int(rng.choice([1, 2, max(1, s // e), max(1, 2 * s // e), s]))
+    c = min(c, s)
+    x = torch.randn((b, gpr * s, m), generator=gen, device="cuda").to(torch.bfloat16)
+    w = (torch.randn((b, m, e), generator=gen, device="cuda") * (2.0 / m ** 0.5)
+         ).to(torch.bfloat16)
+    wp = hip.pack_weights(w, w.dtype)
+    if not hip.fused_gating_supported(x, e, s):
+      continue
+    imp = None
+    if trial % 3 == 1:
+      imp = torch.tensor([0.0, 0.5, 1.0], device="cuda")[
+          torch.randint(0, 3, (b * gpr, s), generator=gen, device="cuda")]
+    tag = "trial %d: b=%d gpr=%d s=%d m=%d e=%d c=%d" % (trial, b, gpr, s, m, e, c)
+    if trial % 2 == 0:
+      kw = dict(importance=imp, use_second_place_loss=trial % 4 == 0,
+                num_microbatches=2)
+      r, logits = hip.router_top2_gating(x, wp, s, c, want_logits=True, **kw)
+      r2 = hip.top2_gating(logits, c, **kw)
+    else:
+      kw = dict(importance=imp, num_microbatches=3)
+      r, logits = hip.router_switch_gating(x, wp, s, c, want_logits=True, **kw)
+      r2 = hip.switch_gating(logits, c, **kw)
+    for name in ("idx", "pos", "kept", "fill", "gate"):
+      assert torch.equal(getattr(r, name), getattr(r2, name)), (tag, name)
+    # (the loss's float32 partial sums are grouped differently in the two
+    # paths: 4 row ranges per block against one sum per block)
+    torch.testing.assert_close(r.loss, r2.loss, rtol=1e-5, atol=1e-7, msg=tag)
+
+
 def test_router_top2_gating_rejects_unsupported(hip):
   x = torch.zeros((1, 96, 64), dtype=torch.bfloat16, device="cuda")
   wp = torch.zeros((1, 8, 64), dtype=torch.bfloat16, device="cuda")
