@@ -20,9 +20,11 @@ tensorflow/core/lib/io/{format,block,table_builder}.cc, stable since 1.0):
 
 PARITY UNPINNED: no file written by TensorFlow exists here to read back, and no
 TensorFlow to read what this module writes.  What is checked: CRC-32C against
-the known answers of RFC 3720, the checksum mask against its inverse, and the
+the known answers of RFC 3720, the checksum mask against its inverse, the
 reader against the writer over every dtype, multi-block tables and multi-shard
-bundles.
+bundles, and both against a two-tensor bundle assembled byte by byte from the
+published format by a script that shares no code with this module
+(tests/golden/make_bundle_fixture.py).
 
 Not handled, each with its own error: Snappy-compressed table blocks
 (TensorFlow's bundle writer writes none), partitioned variables (entries with

@@ -234,3 +234,26 @@ def test_latest_checkpoint(tmp_path):
   (tmp_path / "checkpoint").write_text(
       'model_checkpoint_path: "/abs/model.ckpt-9"\n')
   assert tb.latest_checkpoint(str(tmp_path)) == "/abs/model.ckpt-9"
+
+
+def test_hand_assembled_fixture(tmp_path):
+  """tests/golden/hand_bundle.* were assembled byte by byte from the published
+  format by tests/golden/make_bundle_fixture.py, which shares no code with the
+  package: the reader must decode them, and the writer must reproduce them to
+  the byte (a change that keeps reader and writer consistent with each other
+  but moves either away from the format shows up here)."""
+  golden = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden")
+  prefix = os.path.join(golden, "hand_bundle")
+  reader = tb.BundleReader(prefix)
+  assert sorted(reader.keys()) == ["a/b", "a/c"]
+  ab = reader.get_tensor("a/b")
+  ac = reader.get_tensor("a/c")
+  assert ab.dtype == np.float32 and ab.shape == (2, 3)
+  np.testing.assert_array_equal(ab, np.arange(6, dtype=np.float32).reshape(2, 3))
+  assert ac.dtype == np.int32 and ac.shape == (4,)
+  np.testing.assert_array_equal(ac, np.array([7, -1, 0, 2 ** 31 - 1], np.int32))
+  out = str(tmp_path / "rewritten")
+  tb.write_bundle(out, {"a/c": ac, "a/b": ab})
+  for suffix in (".index", ".data-00000-of-00001"):
+    with open(prefix + suffix, "rb") as f, open(out + suffix, "rb") as g:
+      assert f.read() == g.read(), suffix
