@@ -22,14 +22,18 @@ constexpr int RL_TOK = 64;
 constexpr int RL_KC = 64;
 constexpr int RL_MAX_EPT = 32;
 
-template <typename T>
+// EPT: experts per thread, a power of two >= ept (the loop over a thread's
+// experts is unrolled without conditions: with EPT = 32 and a condition per
+// expert the 64 x 32 scalar branches per chunk were the whole run time at
+// E = 8; the surplus products read the next group's weights and are dropped)
+template <typename T, int EPT>
 __global__ __launch_bounds__(256) void router_logits_kernel(
     const T* __restrict__ x, const T* __restrict__ w,
     const float* __restrict__ bias, float* __restrict__ logits,
     int64_t tokens, int M, int E, int ept) {
   extern __shared__ float smem[];
   float* xs = smem;                       // [RL_TOK][RL_KC + 1]
-  float* ws = smem + RL_TOK * (RL_KC + 1);  // [RL_KC][E]
+  float* ws = smem + RL_TOK * (RL_KC + 1);  // [RL_KC][E] + 4 EPT
   const int b = blockIdx.y;
   const int64_t t0 = (int64_t)blockIdx.x * RL_TOK;
   const int tid = threadIdx.x;
@@ -37,18 +41,26 @@ __global__ __launch_bounds__(256) void router_logits_kernel(
   const int eg = tid >> 6;
   const T* xb = x + ((int64_t)b * tokens) * M;
   const T* wb = w + (int64_t)b * M * E;
-  float acc[RL_MAX_EPT];
+  float acc[EPT];
 #pragma unroll
-  for (int j = 0; j < RL_MAX_EPT; ++j) acc[j] = 0.f;
+  for (int j = 0; j < EPT; ++j) acc[j] = 0.f;
 
   for (int k0 = 0; k0 < M; k0 += RL_KC) {
-    // x tile: 64 tokens x KC, coalesced along M
-    for (int i = tid; i < RL_TOK * RL_KC; i += 256) {
-      int r = i / RL_KC, c = i % RL_KC;
-      int64_t t = t0 + r;
-      float v = 0.f;
-      if (t < tokens && k0 + c < M) v = load_f32<T>(xb + t * M + k0 + c);
-      xs[r * (RL_KC + 1) + c] = v;
+    // x tile: 64 tokens x KC, coalesced along M; a thread's 16 loads are all
+    // issued before the first LDS write (one at a time, each waited for, the
+    // staging took 30 us per chunk)
+    float xv[RL_TOK * RL_KC / 256];
+#pragma unroll
+    for (int u = 0; u < RL_TOK * RL_KC / 256; ++u) {
+      const int i = tid + u * 256;
+      const int r = i / RL_KC, c = i % RL_KC;
+      const int64_t t = t0 + r;
+      xv[u] = (t < tokens && k0 + c < M) ? load_f32<T>(xb + t * M + k0 + c) : 0.f;
+    }
+#pragma unroll
+    for (int u = 0; u < RL_TOK * RL_KC / 256; ++u) {
+      const int i = tid + u * 256;
+      xs[(i / RL_KC) * (RL_KC + 1) + i % RL_KC] = xv[u];
     }
     for (int i = tid; i < RL_KC * E; i += 256) {
       int r = i / E, c = i % E;
@@ -62,9 +74,7 @@ __global__ __launch_bounds__(256) void router_logits_kernel(
       float xv = xs[tok * (RL_KC + 1) + k];
       const float* wr = ws + k * E + e0;
 #pragma unroll
-      for (int j = 0; j < RL_MAX_EPT; ++j) {
-        if (j < ept && e0 + j < E) acc[j] = fmaf(xv, wr[j], acc[j]);
-      }
+      for (int j = 0; j < EPT; ++j) acc[j] = fmaf(xv, wr[j], acc[j]);
     }
     __syncthreads();
   }
@@ -72,7 +82,7 @@ __global__ __launch_bounds__(256) void router_logits_kernel(
   if (t < tokens) {
     float* out = logits + ((int64_t)b * tokens + t) * E;
 #pragma unroll
-    for (int j = 0; j < RL_MAX_EPT; ++j) {
+    for (int j = 0; j < EPT; ++j) {
       int e = eg * ept + j;
       if (j < ept && e < E) out[e] = bias ? acc[j] + bias[e] : acc[j];
     }
@@ -1514,17 +1524,33 @@ extern "C" int mesh_moe_router_logits(const void* x, const void* w,
   }
   const int ept = (E + 3) / 4;
   dim3 grid((unsigned)((tokens + RL_TOK - 1) / RL_TOK), (unsigned)batch);
-  size_t smem = sizeof(float) * (RL_TOK * (RL_KC + 1) + (size_t)RL_KC * E);
+  int eptp = 1;
+  while (eptp < ept) eptp *= 2;
+  size_t smem = sizeof(float) * (RL_TOK * (RL_KC + 1) + (size_t)RL_KC * E + 4 * eptp);
   hipStream_t st = (hipStream_t)stream;
-  MOE_ALLOW_LDS(router_logits_kernel<float>, smem);
-  MOE_ALLOW_LDS(router_logits_kernel<bf16_t>, smem);
-  if (dtype == MESH_MOE_F32) {
-    router_logits_kernel<float><<<grid, 256, smem, st>>>(
-        (const float*)x, (const float*)w, bias, logits, tokens, M, E, ept);
-  } else {
-    router_logits_kernel<bf16_t><<<grid, 256, smem, st>>>(
-        (const bf16_t*)x, (const bf16_t*)w, bias, logits, tokens, M, E, ept);
+#define MOE_ROUTER_LOGITS(T, P)                                                \
+  do {                                                                         \
+    auto kern = router_logits_kernel<T, P>;                                    \
+    MOE_ALLOW_LDS(kern, smem);                                                 \
+    kern<<<grid, 256, smem, st>>>((const T*)x, (const T*)w, bias, logits,      \
+                                  tokens, M, E, ept);                          \
+  } while (0)
+#define MOE_ROUTER_LOGITS_T(T)                                                 \
+  switch (eptp) {                                                              \
+    case 1: MOE_ROUTER_LOGITS(T, 1); break;                                    \
+    case 2: MOE_ROUTER_LOGITS(T, 2); break;                                    \
+    case 4: MOE_ROUTER_LOGITS(T, 4); break;                                    \
+    case 8: MOE_ROUTER_LOGITS(T, 8); break;                                    \
+    case 16: MOE_ROUTER_LOGITS(T, 16); break;                                  \
+    default: MOE_ROUTER_LOGITS(T, 32); break;                                  \
   }
+  if (dtype == MESH_MOE_F32) {
+    MOE_ROUTER_LOGITS_T(float);
+  } else {
+    MOE_ROUTER_LOGITS_T(bf16_t);
+  }
+#undef MOE_ROUTER_LOGITS_T
+#undef MOE_ROUTER_LOGITS
   MOE_CHECK_LAUNCH("router_logits");
   return 0;
 }
