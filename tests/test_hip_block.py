@@ -190,6 +190,42 @@ def test_self_attention_sequence_ids(hip, case, causal, act_dtype):
                                  err_msg="d%s fused=%s" % (name, fused))
 
 
+@pytest.mark.parametrize("causal", [True, False])
+def test_attention_at_the_block_benchmark_shape(hip, causal):
+  """The fused attention kernels at the (batch, head) shape of the benchmark
+  block (L = 2048, 32 heads of 128; two batch entries instead of 32, the
+  entries being independent) against the three-step pieces: the weights
+  [B*H, L, L] of mesh_moe_attention_weights times v for the forward, the
+  composed backward for the gradients; and causality as a property: keys and
+  values after position p cannot change the outputs up to p."""
+  b, l, heads, d = 2, 2048, 32, 128
+  gen = torch.Generator(device="cuda").manual_seed(5)
+  mk = lambda: (torch.randn((b, l, heads * d), generator=gen, device="cuda")
+                * 0.3).to(torch.bfloat16)
+  q, k, v, do = mk(), mk(), mk(), mk()
+  out = hip.self_attention(q, k, v, heads, causal)
+  w = hip.attention_weights(q, k, heads, causal)                 # [B*H, L, L]
+  vh = v.reshape(b, l, heads, d).permute(0, 2, 1, 3).reshape(b * heads, l, d)
+  want = torch.bmm(w.float(), vh.float()).reshape(b, heads, l, d).permute(
+      0, 2, 1, 3).reshape(b, l, heads * d)
+  torch.testing.assert_close(out.float(), want, rtol=2e-2, atol=2e-2)
+  del w, want
+  got = hip.self_attention_backward(q, k, v, do, heads, causal, fused=True)
+  ref = hip.self_attention_backward(q, k, v, do, heads, causal, fused=False)
+  for g_, r_, name in zip(got, ref, "qkv"):
+    scale = max(1.0, float(r_.float().abs().max()))
+    torch.testing.assert_close(g_.float(), r_.float(), rtol=3e-2,
+                               atol=3e-2 * scale, msg="d" + name)
+  if causal:
+    p = 1237
+    k2, v2 = k.clone(), v.clone()
+    k2[:, p + 1:] = -k2[:, p + 1:]
+    v2[:, p + 1:] = v2[:, p + 1:] + 1
+    out2 = hip.self_attention(q, k2, v2, heads, causal)
+    assert torch.equal(out2[:, :p + 1], out[:, :p + 1])
+    assert not torch.equal(out2[:, p + 1:], out[:, p + 1:])
+
+
 def test_self_attention_rejections(hip):
   q = torch.zeros((1, 12, 16), dtype=torch.bfloat16, device="cuda")
   with pytest.raises(hip.MoeHipError, match="not divisible"):
