@@ -1515,14 +1515,16 @@ static int grouped_gemm(const void* A, const void* B, void* C, int E, int R,
                                  (bf16_t*)C, E, R, N, K, relu, st);
     else if (N >= 256 && R >= 128 && K % 64 == 0 &&
              (int64_t)R * K < (1LL << 31) && (int64_t)N * K < (1LL << 31)) {
-      // direct-to-LDS kernels; 256-row tiles unless 128-row tiles waste fewer
-      // padded rows (e.g. 640 rows per expert: 5 x 128 instead of 3 x 256)
+      // direct-to-LDS kernels; the persistent 256-row kernel unless 128-row
+      // tiles save more than a fifth of the padded rows (at 640 rows per
+      // expert, 3 x 256 against 5 x 128, the persistent kernel still wins:
+      // 0.43 against 0.50 ms for both GEMMs of benchmark config 2)
       const bf16_t *a = (const bf16_t*)A, *b = (const bf16_t*)B;
       bf16_t* c = (bf16_t*)C;
       const int pad256 = (R + 255) / 256 * 256, pad128 = (R + 127) / 128 * 128;
       // 256 x 256 tiles run 8 wavefronts (two per SIMD, 128 x 64 sub-tiles)
       // with the loads spread over the MFMA steps
-      if (pad128 < pad256) {
+      if (pad128 * 5 < pad256 * 4) {
         rc = launch_dma<128, 256, 2>(a, b, c, E, R, N, K, relu, st);
       } else if (relu_mask_src != nullptr && mask_applied != nullptr && !relu &&
                  ((uintptr_t)relu_mask_src % 16) == 0) {
@@ -1720,7 +1722,7 @@ __global__ __launch_bounds__(1024) void tile_list_kernel(
 static bool ring_path_applies(int R, int N, int K) {
   const int pad256 = (R + 255) / 256 * 256, pad128 = (R + 127) / 128 * 128;
   return N >= 256 && R >= 128 && K % 64 == 0 && K % 8 == 0 && N % 8 == 0 &&
-         pad128 >= pad256 && (int64_t)N * K < (1LL << 31);
+         pad128 * 5 >= pad256 * 4 && (int64_t)N * K < (1LL << 31);
 }
 
 }  // namespace mesh_moe
