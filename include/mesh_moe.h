@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 20
+#define MESH_MOE_ABI_VERSION 21
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -778,6 +778,23 @@ int mesh_moe_self_attention_backward(const void* q, const void* k, const void* v
                                      int causal, const int32_t* sequence_id,
                                      int dtype, void* workspace,
                                      size_t workspace_bytes, void* stream);
+
+/*
+ * One decoding step of self-attention: SelfAttention.call in "incremental"
+ * mode (transformer/transformer_layers.py:231-254) with the visibility of
+ * :289-296.  The step's key and value replace row position[b] of the recurrent
+ * states (the reference's k = old_k * (1 - one_hot) + k * one_hot, here in
+ * place), the query sees memory positions m <= position[b]; float32 logits and
+ * softmax, weights cast to dtype, out = weights . v.
+ *   q, k_new, v_new, out [B,H*D] dtype; k_cache, v_cache [B,Lm,H*D] dtype,
+ *   updated in place; position [B] int32 on the device, clamped to [0, Lm).
+ * One block per (head, batch entry), the caches read once.  Lm up to ~38000
+ * (the logits of a row live in LDS).
+ */
+int mesh_moe_attention_decode(const void* q, const void* k_new, const void* v_new,
+                              void* k_cache, void* v_cache,
+                              const int32_t* position, void* out, int B, int Lm,
+                              int H, int D, int dtype, void* stream);
 
 #ifdef __cplusplus
 }

@@ -933,6 +933,158 @@ extern "C" int mesh_moe_self_attention(const void* q, const void* k,
                                st);
 }
 
+// ---------------------------------------------------------------------------
+// One decoding step of self-attention ("incremental" mode,
+// transformer/transformer_layers.py:231-254, :289-296).  One block per
+// (head, batch entry): the step's key and value rows go into the caches at
+// row position[b]; logits q . k_m in float32 for m <= position[b], float32
+// softmax in the reference's op order, weights rounded to the activation
+// dtype, out = sum_m w_m v_m.  The caches are read once: HBM-bound.
+//   q, k_new, v_new, out [B, H*D]; k_cache, v_cache [B, Lm, H*D] (updated in
+//   place); position [B] int32 on the device.
+// Dynamic LDS: max(Lm, 256) + D + 8 floats.
+// ---------------------------------------------------------------------------
+template <typename T>
+__global__ __launch_bounds__(256) void attention_decode_kernel(
+    const T* __restrict__ q, const T* __restrict__ k_new,
+    const T* __restrict__ v_new, T* __restrict__ k_cache,
+    T* __restrict__ v_cache, const int32_t* __restrict__ position,
+    T* __restrict__ out, int Lm, int H, int D, int vec) {
+  extern __shared__ float dec_smem[];
+  float* wl = dec_smem;            // [max(Lm, 256)] logits, then weights
+  float* qs = wl + (Lm > 256 ? Lm : 256);   // [D]
+  float* red = qs + D;             // [8]
+  const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
+  const int lane = tid & 63, wave = tid >> 6;
+  const int64_t hd = (int64_t)H * D;
+  const int pos = min(max(position[b], 0), Lm - 1);
+  const T* qr = q + b * hd + (int64_t)h * D;
+  const T* knr = k_new + b * hd + (int64_t)h * D;
+  const T* vnr = v_new + b * hd + (int64_t)h * D;
+  T* kc = k_cache + (int64_t)b * Lm * hd + (int64_t)h * D;
+  T* vc = v_cache + (int64_t)b * Lm * hd + (int64_t)h * D;
+  for (int d = tid; d < D; d += 256) {
+    qs[d] = load_f32<T>(qr + d);
+    kc[(int64_t)pos * hd + d] = knr[d];
+    vc[(int64_t)pos * hd + d] = vnr[d];
+  }
+  __syncthreads();
+  // logits of the visible rows; row `pos` comes from the step's own key
+  constexpr int VN = Vec16B<T>::N;
+  float m = -INFINITY;
+  for (int j = tid; j <= pos; j += 256) {
+    const T* kr = j == pos ? knr : kc + (int64_t)j * hd;
+    float acc = 0.f;
+    if (vec) {
+      for (int d0 = 0; d0 < D; d0 += VN) {
+        float f[VN];
+        unpack16(*reinterpret_cast<const uint4*>(kr + d0), f, T());
+#pragma unroll
+        for (int u = 0; u < VN; ++u) acc = fmaf(qs[d0 + u], f[u], acc);
+      }
+    } else {
+      for (int d = 0; d < D; ++d) acc = fmaf(qs[d], load_f32<T>(kr + d), acc);
+    }
+    wl[j] = acc;
+    m = fmaxf(m, acc);
+  }
+  auto block_all = [&](float v, bool is_max) {
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) {
+      const float o = __shfl_xor(v, off, 64);
+      v = is_max ? fmaxf(v, o) : v + o;
+    }
+    __syncthreads();
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    float r = red[0];
+    for (int w = 1; w < 4; ++w) r = is_max ? fmaxf(r, red[w]) : r + red[w];
+    return r;
+  };
+  m = block_all(m, true);
+  const float negm = -m;
+  float sum = 0.f;
+  for (int j = tid; j <= pos; j += 256) sum += expf(wl[j] + negm);
+  sum = block_all(sum, false);
+  const float neglse = -(logf(sum) + m);
+  for (int j = tid; j <= pos; j += 256)
+    wl[j] = round_to<T>(expf(wl[j] + neglse));
+  __syncthreads();
+  // out[d] = sum_j w_j v[j][d]: the threads of a group cover d, the groups
+  // split the rows; partial sums meet in LDS
+  const int groups = D <= 256 ? 256 / D : 1;
+  float* part = wl;                 // reused below, after the weights are read
+  if (D <= 256) {
+    const int g = tid / D, d = tid - g * D;
+    float acc = 0.f;
+    if (g < groups) {
+      for (int j = g; j <= pos; j += groups) {
+        const T* vr = j == pos ? vnr : vc + (int64_t)j * hd;
+        acc = fmaf(wl[j], load_f32<T>(vr + d), acc);
+      }
+    }
+    __syncthreads();                // every weight has been read
+    if (g < groups) part[g * D + d] = acc;
+    __syncthreads();
+    if (tid < D) {
+      float total = 0.f;
+      for (int gg = 0; gg < groups; ++gg) total += part[gg * D + tid];
+      store_f32<T>(out + b * hd + (int64_t)h * D + tid, total);
+    }
+  } else {
+    for (int d = tid; d < D; d += 256) {
+      float acc = 0.f;
+      for (int j = 0; j <= pos; ++j) {
+        const T* vr = j == pos ? vnr : vc + (int64_t)j * hd;
+        acc = fmaf(wl[j], load_f32<T>(vr + d), acc);
+      }
+      store_f32<T>(out + b * hd + (int64_t)h * D + d, acc);
+    }
+  }
+}
+
+extern "C" int mesh_moe_attention_decode(const void* q, const void* k_new,
+                                         const void* v_new, void* k_cache,
+                                         void* v_cache, const int32_t* position,
+                                         void* out, int B, int Lm, int H, int D,
+                                         int dtype, void* stream) {
+  MOE_REQUIRE(q && k_new && v_new && k_cache && v_cache && position && out,
+              MESH_MOE_E_ARG, "attention_decode: null pointer");
+  MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG,
+              "attention_decode: bad dtype %d", dtype);
+  MOE_REQUIRE(B >= 1 && Lm >= 1 && H >= 1 && D >= 1, MESH_MOE_E_ARG,
+              "attention_decode: bad sizes B=%d Lm=%d H=%d D=%d", B, Lm, H, D);
+  MOE_REQUIRE(B <= 65535, MESH_MOE_E_UNSUPPORTED,
+              "attention_decode: batch %d > 65535", B);
+  // the partial sums of the last phase reuse the weights' array
+  const size_t floats = (size_t)(Lm > 256 ? Lm : 256) + (size_t)D + 8;
+  const size_t smem = floats * sizeof(float);
+  MOE_REQUIRE(smem <= 150 * 1024, MESH_MOE_E_UNSUPPORTED,
+              "attention_decode: memory length %d does not fit in LDS", Lm);
+  hipStream_t st = (hipStream_t)stream;
+  const dim3 grid((unsigned)H, (unsigned)B);
+  const size_t esz = dtype_size(dtype);
+  const int vec = ((size_t)D * esz) % 16 == 0 &&
+                  (((uintptr_t)k_cache | (uintptr_t)k_new) % 16) == 0;
+  if (dtype == MESH_MOE_F32) {
+    auto kern = attention_decode_kernel<float>;
+    MOE_ALLOW_LDS(kern, smem);
+    kern<<<grid, 256, smem, st>>>((const float*)q, (const float*)k_new,
+                                  (const float*)v_new, (float*)k_cache,
+                                  (float*)v_cache, position, (float*)out, Lm, H,
+                                  D, vec);
+  } else {
+    auto kern = attention_decode_kernel<bf16_t>;
+    MOE_ALLOW_LDS(kern, smem);
+    kern<<<grid, 256, smem, st>>>((const bf16_t*)q, (const bf16_t*)k_new,
+                                  (const bf16_t*)v_new, (bf16_t*)k_cache,
+                                  (bf16_t*)v_cache, position, (bf16_t*)out, Lm,
+                                  H, D, vec);
+  }
+  MOE_CHECK_LAUNCH("attention_decode");
+  return 0;
+}
+
 extern "C" size_t mesh_moe_self_attention_backward_workspace_bytes(int B, int L,
                                                                    int H, int D,
                                                                    int dtype) {

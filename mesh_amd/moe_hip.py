@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 20
+ABI_VERSION = 21
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -190,6 +190,9 @@ _SIGNATURES = {
         _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, ctypes.c_int, _vp,
         ctypes.c_size_t, _vp]),
+    "mesh_moe_attention_decode": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
 }
 EXPORTS = sorted(_SIGNATURES)
 
@@ -1154,6 +1157,28 @@ def self_attention(q, k, v, num_heads, causal, sequence_id=None):
         _dev(v, "v", q.dtype, (b, l, hd)), out.data_ptr(), b, l, num_heads, d,
         int(bool(causal)), _sequence_id_ptr(sequence_id, b, l), code,
         ws.data_ptr(), ws_bytes, _stream()), "self_attention")
+  return out
+
+
+def attention_decode(q, k_new, v_new, k_cache, v_cache, position, num_heads):
+  """One decoding step: q, k_new, v_new [B, H*D], the caches [B, Lm, H*D]
+  (UPDATED IN PLACE at row position[b]), position [B] int32 -> out [B, H*D]."""
+  lib = load_library()
+  b, hd = q.shape
+  lm = k_cache.shape[1]
+  if hd % num_heads:
+    raise MoeHipError("q channels %d not divisible by %d heads"
+                      % (hd, num_heads))
+  out = torch.empty_like(q)
+  with _stage("attention_decode"):
+    _check(lib.mesh_moe_attention_decode(
+        _dev(q, "q"), _dev(k_new, "k_new", q.dtype, (b, hd)),
+        _dev(v_new, "v_new", q.dtype, (b, hd)),
+        _dev(k_cache, "k_cache", q.dtype, (b, lm, hd)),
+        _dev(v_cache, "v_cache", q.dtype, (b, lm, hd)),
+        _dev(position, "position", torch.int32, (b,)), out.data_ptr(), b, lm,
+        num_heads, hd // num_heads, dtype_code(q.dtype), _stream()),
+        "attention_decode")
   return out
 
 

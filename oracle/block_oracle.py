@@ -141,6 +141,37 @@ def _attention_core(q, k, v, num_heads, causal, act_dtype, sequence_id=None):
   return _r(np.einsum("bhlm,bmhd->blhd", weights, v), act_dtype).reshape(b, l, hd)
 
 
+def attention_incremental(q, k_new, v_new, k_cache, v_cache, position,
+                          num_heads, act_dtype="float32"):
+  """One decoding step of SelfAttention ("incremental" mode,
+  transformer/transformer_layers.py:231-254 and :289-296): the step's key and
+  value replace row position[b] of the recurrent states
+  (k = old_k * (1 - one_hot) + k_new * one_hot), the query sees the memory
+  positions m <= position[b] (read_priority >= write_priority), float32
+  logits and softmax, weights cast to the activation dtype.
+
+  q, k_new, v_new [B, H*D]; k_cache, v_cache [B, Lm, H*D]; position [B]
+  integers.  Returns (out [B, H*D], k [B, Lm, H*D], v [B, Lm, H*D])."""
+  b, lm, hd = k_cache.shape
+  d = hd // num_heads
+  position = np.asarray(position).reshape(b)
+  one_hot = _r((np.arange(lm)[None, :] == position[:, None]).astype(F32),
+               act_dtype)[..., None]
+  inv = _r(F32(1.0) - one_hot, act_dtype)
+  k = _r(_r(_r(k_cache, act_dtype) * inv, act_dtype)
+         + _r(_r(k_new, act_dtype)[:, None, :] * one_hot, act_dtype), act_dtype)
+  v = _r(_r(_r(v_cache, act_dtype) * inv, act_dtype)
+         + _r(_r(v_new, act_dtype)[:, None, :] * one_hot, act_dtype), act_dtype)
+  q4 = _r(q, act_dtype).reshape(b, num_heads, d)
+  k4, v4 = k.reshape(b, lm, num_heads, d), v.reshape(b, lm, num_heads, d)
+  logits = np.einsum("bhd,bmhd->bhm", q4, k4).astype(F32)
+  hidden = (np.arange(lm)[None, :] > position[:, None]).astype(F32)[:, None, :]
+  logits = (logits + hidden * F32(-1e9)).astype(F32)
+  weights = _r(O.softmax(logits), act_dtype)
+  out = _r(np.einsum("bhm,bmhd->bhd", weights, v4), act_dtype)
+  return out.reshape(b, hd), k, v
+
+
 def experts_self_attention(x, w_gate, wi, q_wo, k_wo, wo, hparams, num_heads,
                            causal, act_dtype="float32", train=False,
                            num_microbatches=None):

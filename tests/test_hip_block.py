@@ -226,6 +226,36 @@ def test_attention_at_the_block_benchmark_shape(hip, causal):
     assert not torch.equal(out2[:, p + 1:], out[:, p + 1:])
 
 
+@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("case", [(2, 12, 2, 4), (3, 300, 4, 64), (2, 2048, 2, 128),
+                                  (1, 77, 3, 24), (2, 40, 1, 320)],
+                         ids=lambda c: "x".join(map(str, c)))
+def test_attention_decode(hip, case, act_dtype):
+  """mesh_moe_attention_decode (one step of "incremental" mode) against the
+  oracle: output and updated caches, positions from 0 to the last row."""
+  b, lm, heads, d = case
+  rng = np.random.default_rng(sum(case))
+  hd = heads * d
+  mk = lambda *shape: O.cast_act(
+      (rng.standard_normal(shape) * 0.5).astype(np.float32), act_dtype)
+  q, kn, vn = mk(b, hd), mk(b, hd), mk(b, hd)
+  kc, vc = mk(b, lm, hd), mk(b, lm, hd)
+  g = lambda a: H.to_gpu(a, act_dtype)
+  for pos in ([0] * b, [lm - 1] * b, list(rng.integers(0, lm, size=b))):
+    pos = np.asarray(pos, np.int32)
+    want, want_k, want_v = B.attention_incremental(q, kn, vn, kc, vc, pos,
+                                                   heads, act_dtype)
+    kg, vg = g(kc), g(vc)
+    got = hip.attention_decode(g(q), g(kn), g(vn), kg, vg,
+                               torch.from_numpy(pos).cuda(), heads)
+    tol = _tol(act_dtype)
+    if act_dtype == "float32":
+      tol = dict(rtol=1e-4, atol=1e-4)
+    np.testing.assert_allclose(H.to_np(got), want, **tol)
+    np.testing.assert_array_equal(H.to_np(kg), want_k)
+    np.testing.assert_array_equal(H.to_np(vg), want_v)
+
+
 def test_self_attention_rejections(hip):
   q = torch.zeros((1, 12, 16), dtype=torch.bfloat16, device="cuda")
   with pytest.raises(hip.MoeHipError, match="not divisible"):
