@@ -254,16 +254,23 @@ def tensor_dim_to_mesh_dim_size(layout, mesh_shape, tensor_dim):
 # variable scopes: names only (the reference leans on tf.variable_scope)
 # ----------------------------------------------------------------------------
 _SCOPE_STACK = []
+_REUSE_STACK = []
 
 
 @contextlib.contextmanager
-def variable_scope(name):
-  """Prefixes the names of variables created inside with `name/`."""
+def variable_scope(name, reuse=None):
+  """Prefixes the names of variables created inside with `name/`.  With
+  reuse=True (as tf.variable_scope's, which the reference's decoding loop
+  opens, transformer/transformer.py:1221) get_variable returns the existing
+  variable of that name instead of creating one; the flag holds for the
+  nested scopes too."""
   _SCOPE_STACK.append(name)
+  _REUSE_STACK.append(bool(reuse) or (bool(_REUSE_STACK) and _REUSE_STACK[-1]))
   try:
     yield
   finally:
     _SCOPE_STACK.pop()
+    _REUSE_STACK.pop()
 
 
 def current_scope_name():
@@ -1026,8 +1033,9 @@ def get_variable(mesh, name, shape, dtype=float32, master_dtype=None,
                  slice_dtype=None, activation_dtype=None, initializer=None,
                  trainable=True, **kwargs):
   """Creates a variable named `<scope>/<name>`
-  (mesh_tensorflow/ops.py:4160-4208).  Unlike the reference there is no reuse:
-  asking for an existing name raises."""
+  (mesh_tensorflow/ops.py:4160-4208); inside variable_scope(..., reuse=True)
+  returns the existing one.  Asking for an existing name without reuse
+  raises."""
   if dtype is None:
     dtype = VariableDType(master_dtype, slice_dtype, activation_dtype)
   elif isinstance(dtype, VariableDType):
@@ -1038,7 +1046,16 @@ def get_variable(mesh, name, shape, dtype=float32, master_dtype=None,
                           activation_dtype or dtype)
   scope = current_scope_name()
   full = scope + "/" + name if scope else name
-  if any(v.name == full for v in mesh.graph.all_variables):
+  existing = [v for v in mesh.graph.all_variables if v.name == full]
+  if _REUSE_STACK and _REUSE_STACK[-1]:
+    if not existing:
+      raise ValueError("Variable %s does not exist (reuse=True)" % full)
+    out = existing[0].outputs[0]
+    if out.shape != convert_to_shape(shape):
+      raise ValueError("Variable %s has shape %s, asked for %s"
+                       % (full, out.shape, convert_to_shape(shape)))
+    return out
+  if existing:
     raise ValueError("Variable %s already exists" % full)
   return Variable(mesh, name, convert_to_shape(shape), dtype, initializer,
                   trainable, **kwargs).outputs[0]

@@ -227,6 +227,52 @@ class SelfAttentionOperation(mtf.Operation):
     return grads + [None] * (len(self.inputs) - 3)
 
 
+class AttentionDecodeOperation(mtf.Operation):
+  """One decoding step of self-attention (SelfAttention.call in "incremental"
+  mode, transformer_layers.py:231-254): q, k, v [batch..., heads * d_kv] of the
+  step, the recurrent states old_k, old_v [batch..., memory_length,
+  heads * d_kv] and position [batch...] (int32) -> the attention outputs
+  [batch..., heads * d_kv] and the updated states.  The states are new tensors
+  (the graph stays functional); the library call updates a copy in place."""
+
+  def __init__(self, q, k, v, old_k, old_v, position, num_heads, name=None):
+    super(AttentionDecodeOperation, self).__init__(
+        [q, k, v, old_k, old_v, position], name=name or "attention_decode")
+    if q.shape != k.shape or q.shape != v.shape or old_k.shape != old_v.shape:
+      raise ValueError("q, k, v %s %s %s / states %s %s"
+                       % (q.shape, k.shape, v.shape, old_k.shape, old_v.shape))
+    if (old_k.shape.dims[:-2] != q.shape.dims[:-1]
+        or old_k.shape.dims[-1] != q.shape.dims[-1]
+        or position.shape.dims != q.shape.dims[:-1]):
+      raise ValueError("states %s / position %s do not match q %s"
+                       % (old_k.shape, position.shape, q.shape))
+    self._num_heads = num_heads
+    self._outputs = [mtf.Tensor(self, q.shape, q.dtype, index=0),
+                     mtf.Tensor(self, old_k.shape, old_k.dtype, index=1),
+                     mtf.Tensor(self, old_v.shape, old_v.dtype, index=2)]
+
+  has_gradient = False
+
+  def lower(self, lowering):
+    from mesh_amd import moe_hip
+    mesh_impl = lowering.mesh_impl(self)
+    q_sizes = self.outputs[0].shape.to_integer_list
+    s_sizes = self.outputs[1].shape.to_integer_list
+    channels, memory = q_sizes[-1], s_sizes[-2]
+    heads = self._num_heads
+
+    def fn(q, k, v, old_k, old_v, position):
+      q2, k2, v2 = (t.reshape(-1, channels).contiguous() for t in (q, k, v))
+      kc = old_k.reshape(-1, memory, channels).clone()
+      vc = old_v.reshape(-1, memory, channels).clone()
+      pos = position.reshape(-1).to(torch.int32).contiguous()
+      out = moe_hip.attention_decode(q2, k2, v2, kc, vc, pos, heads)
+      return out.reshape(q_sizes), kc.reshape(s_sizes), vc.reshape(s_sizes)
+    outs = mesh_impl.slicewise(fn, *[lowering.tensors[t] for t in self.inputs])
+    for tensor, value in zip(self.outputs, outs):
+      lowering.set_tensor_lowering(tensor, value)
+
+
 class SelfAttentionGradOperation(mtf.Operation):
   """(dq, dk, dv) of a SelfAttentionOperation: the gradients of the two
   einsums and the softmax of attention.attention (attention.py:76-87), with

@@ -3,9 +3,12 @@ Mixture-of-Experts transformer block needs: TransformerLayer, Context,
 LayerStack with its sublayers (RMS norm, layer call, dropout, residual,
 padding mask), make_layer_stack, and the layer-stack call of Unitransformer.
 
+Decoding: the "first_part" and "incremental" modes of the Context and of
+SelfAttention (recurrent key / value states); the sampling loop around them
+stays with the caller.
+
 Not here: embeddings, vocabularies, logits and losses of Unitransformer /
-Bitransformer, decoding ("first_part" / "incremental" modes), ensembles,
-subsequence ids.
+Bitransformer, ensembles, subsequence ids.
 """
 
 from mesh_amd import layers as mtf_layers
@@ -13,6 +16,8 @@ from mesh_amd import ops as mtf
 
 TRAIN = "train"   # tf.estimator.ModeKeys.TRAIN
 EVAL = "eval"     # tf.estimator.ModeKeys.EVAL
+FIRST_PART = "first_part"     # decoding: the known first part, records states
+INCREMENTAL = "incremental"   # decoding: one position per call, states in/out
 
 
 class _Position(object):
@@ -45,7 +50,7 @@ class TransformerLayer(object):
 # Context fields that only decoding, beam search, encoder-decoder attention or
 # parameter sharing use; accepted for signature compatibility, must stay None.
 _UNUSED_CONTEXT_FIELDS = (
-    "beam_dim", "subsequence_id", "states", "new_states", "initial_position",
+    "beam_dim", "subsequence_id", "initial_position",
     "encoder_output", "encoder_sequence_id", "constant_states",
     "shared_params", "encoder_layer_outputs", "inputs", "encoder_inputs")
 
@@ -62,10 +67,12 @@ class Context(object):
                mode=TRAIN, position=None, position_is_default=False,
                sequence_id=None, losses=None, layer_outputs=None,
                write_priority=None, read_priority=None, num_microbatches=1,
-               **unused):
-    if mode not in (TRAIN, EVAL):
-      raise NotImplementedError("mode %r (decoding) is not implemented"
-                                % (mode,))
+               states=None, new_states=None, **unused):
+    if mode not in (TRAIN, EVAL, FIRST_PART, INCREMENTAL):
+      raise ValueError("unknown mode %r" % (mode,))
+    if mode == INCREMENTAL and not isinstance(position, mtf.Tensor):
+      raise ValueError("incremental mode needs the position tensor "
+                       "[batch dims] (int32)")
     for key, value in unused.items():
       if key not in _UNUSED_CONTEXT_FIELDS:
         raise TypeError("Context got an unexpected argument %r" % key)
@@ -89,10 +96,29 @@ class Context(object):
     self.layer_outputs = [] if layer_outputs is None else layer_outputs
     self.write_priority, self.read_priority = write_priority, read_priority
     self.num_microbatches = num_microbatches
+    # recurrent states of decoding (transformer.py:251-272): layers read
+    # theirs with get_states in "incremental" mode and append the new values
+    # with record_new_states in "first_part" and "incremental" modes
+    self.states = [] if states is None else list(states)
+    self.new_states = [] if new_states is None else new_states
     self.layer_index = 0
     self.cache = {}            # values shared between layers
 
   train = property(lambda self: self.mode == TRAIN)
+
+  def get_states(self, n):
+    """The next n recurrent states (transformer.py:251-261)."""
+    got = self.states[len(self.new_states):len(self.new_states) + n]
+    if len(got) != n:
+      raise ValueError("incremental mode: %d states were passed, a layer asks "
+                       "for states %d..%d" % (len(self.states),
+                                              len(self.new_states),
+                                              len(self.new_states) + n - 1))
+    return got
+
+  def record_new_states(self, new_states):
+    """transformer.py:263-271."""
+    self.new_states.extend(new_states)
   activation_dtype = property(
       lambda self: self.variable_dtype.activation_dtype)
 
@@ -365,20 +391,41 @@ class Unitransformer(object):
     return self.autoregressive
 
   def call_layers(self, x, variable_dtype, mode=EVAL, num_microbatches=1,
-                  sequence_id=None):
+                  sequence_id=None, position=None, states=None,
+                  new_states=None, length_dim=None, reuse=None):
     """x [batch dims..., length, d_model] -> (y, losses).  The Context is the
     one _call_internal builds (transformer.py:1032-1062): read and write
-    priorities are the position for an autoregressive model."""
+    priorities are the position for an autoregressive model.
+
+    Decoding, as sample_autoregressive drives it (transformer.py:1140-1248):
+    mode "first_part" runs the known first part and appends every attention
+    layer's keys and values to the list `new_states`; mode "incremental" takes
+    x [batch dims..., d_model] (one position per batch entry), `position`
+    [batch dims...] int32, the states of the previous call as `states`, the
+    sequences' `length_dim`, and appends the updated states to `new_states`.
+    The loop around it (sampling, stopping) stays with the caller.  `reuse`:
+    take the variables an earlier call on this graph created (the default in
+    "incremental" mode, as the reference's loop body does)."""
     if x.shape.dims[-1] != self.model_dim:
       raise ValueError("x %s does not end in %s" % (x.shape, self.model_dim))
     priority = POSITION if self.autoregressive else None
     losses = []
+    if mode == INCREMENTAL:
+      if length_dim is None:
+        raise ValueError("incremental mode needs length_dim")
+      batch_dims = x.shape.dims[:-1]
+    else:
+      batch_dims, length_dim = x.shape.dims[:-2], x.shape.dims[-2]
     context = Context(
-        model=self, mesh=x.mesh, batch_dims=x.shape.dims[:-2],
-        length_dim=x.shape.dims[-2], variable_dtype=variable_dtype, mode=mode,
-        position_is_default=True, sequence_id=sequence_id, losses=losses,
+        model=self, mesh=x.mesh, batch_dims=batch_dims,
+        length_dim=length_dim, variable_dtype=variable_dtype, mode=mode,
+        position=position, position_is_default=position is None,
+        sequence_id=sequence_id, losses=losses,
         write_priority=priority, read_priority=priority,
-        num_microbatches=num_microbatches)
-    with mtf.variable_scope(self.name):
+        num_microbatches=num_microbatches, states=states,
+        new_states=new_states)
+    if reuse is None:
+      reuse = mode == INCREMENTAL
+    with mtf.variable_scope(self.name, reuse=reuse):
       y = self.layer_stack.call(context, x)
     return y, losses

@@ -113,6 +113,29 @@ class SelfAttention(transformer.TransformerLayer):
     else:
       k = params.compute_k(x)
       v = params.compute_v(x)
+    if context.mode == transformer.INCREMENTAL:
+      # one position per batch entry: the step's key and value replace row
+      # `position` of the recurrent states, the query sees the memory
+      # positions up to it (transformer_layers.py:239-254, :289-296)
+      if sequence_id is not None or self.shared_kv:
+        raise NotImplementedError(
+            "incremental mode with sequence ids or shared_kv")
+      if context.read_priority is not transformer.POSITION:
+        raise NotImplementedError("incremental mode of a model that is not "
+                                  "autoregressive")
+      old_k, old_v = context.get_states(2)
+      op = attention.AttentionDecodeOperation(
+          q, k, v, old_k, old_v, context.position, params.num_heads)
+      o, k_all, v_all = op.outputs
+      context.record_new_states([k_all, v_all])
+      return params.compute_output(o, output_shape=x.shape)
+    if context.mode == transformer.FIRST_PART:
+      if self.shared_kv:
+        raise NotImplementedError("first_part mode with shared_kv")
+      name = context.length_dim.name       # states carry "memory_length"
+      context.record_new_states(
+          [mtf.rename_dimension(k, name, "memory_length"),
+           mtf.rename_dimension(v, name, "memory_length")])
     # read_priority >= write_priority (transformer_layers.py:289-296)
     causal = context.read_priority is transformer.POSITION
     if context.train and self.dropout_rate != 0.0:

@@ -502,8 +502,19 @@ def test_block_rejections():
   x = mtf.import_tf_tensor(mesh, torch.zeros(1, 8, 16), mtf.Shape(dims))
   vdt = mtf.VariableDType(torch.float32)
   model = transformer.Unitransformer(None, d_model=16)
-  with pytest.raises(NotImplementedError, match="decoding"):
+  with pytest.raises(ValueError, match="position"):
     transformer.Context(model, mesh, dims[:1], dims[1], vdt, mode="incremental")
+  with pytest.raises(ValueError, match="unknown mode"):
+    transformer.Context(model, mesh, dims[:1], dims[1], vdt, mode="beam")
+  pos = mtf.import_tf_tensor(mesh, torch.zeros(1, dtype=torch.int32),
+                             mtf.Shape(dims[:1]))
+  ctx = transformer.Context(model, mesh, dims[:1], dims[1], vdt,
+                            mode="incremental", position=pos, states=[x, x])
+  assert ctx.get_states(2) == [x, x]
+  ctx.record_new_states([x])
+  assert ctx.get_states(1) == [x]
+  with pytest.raises(ValueError, match="states were passed"):
+    ctx.get_states(2)
   stack = transformer.make_layer_stack(
       [(transformer_layers.DenseReluDense,
         dict(hidden_size=8, dropout_rate=0.1))], num_layers=1)

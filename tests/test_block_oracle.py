@@ -126,6 +126,30 @@ def test_attention_sequence_ids_are_block_diagonal(causal):
         np.testing.assert_allclose(g_[i:i + 1, sl], w_, rtol=1e-5, atol=1e-6)
 
 
+def test_attention_incremental_is_a_row_of_causal_attention():
+  """A decoding step at position p gives row p of the autoregressive attention
+  over the full row, whatever the states hold at and after p; the step's key
+  and value land in row p of the new states and nothing else moves."""
+  rng = np.random.default_rng(78)
+  b, l, heads, d = 2, 12, 2, 4
+  q, k, v = (rng.standard_normal((b, l, heads * d)).astype(np.float32)
+             for _ in range(3))
+  full = B._attention_core(q, k, v, heads, True, "float32")
+  for p in ([0, 0], [5, 9], [11, 3]):
+    kc, vc = k.copy(), v.copy()
+    for i, pi in enumerate(p):
+      kc[i, pi:] = 7.0
+      vc[i, pi:] = -3.0
+    rows = np.arange(b)
+    out, k2, v2 = B.attention_incremental(q[rows, p], k[rows, p], v[rows, p], kc,
+                                          vc, np.array(p), heads)
+    np.testing.assert_allclose(out, full[rows, p], rtol=1e-5, atol=1e-6)
+    for i, pi in enumerate(p):
+      np.testing.assert_array_equal(k2[i, :pi + 1], k[i, :pi + 1])
+      np.testing.assert_array_equal(v2[i, :pi + 1], v[i, :pi + 1])
+      np.testing.assert_array_equal(k2[i, pi + 1:], kc[i, pi + 1:])
+
+
 def test_self_attention_bf16_close_to_float32():
   rng = np.random.default_rng(6)
   b, l, m, heads, d = 2, 16, 32, 2, 8

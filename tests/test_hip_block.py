@@ -379,6 +379,102 @@ def test_layer_stack_packed_sequences(autoregressive):
   assert not got[0, -5:].any() and not grads[0][0, -5:].any()
 
 
+@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
+def test_decoding_modes_match_the_full_forward(act_dtype):
+  """Decoding as Unitransformer.sample_autoregressive drives it
+  (transformer.py:1140-1248): "first_part" over a row whose positions from p0
+  on are unknown (zeros) records every attention layer's keys and values; one
+  "incremental" call per position p >= p0 takes the token of that position, the
+  states and position [batch], and must give what the full forward gives at p
+  (teacher forcing).  The experts' capacity is ample in both runs, so no token
+  is dropped in either."""
+  b, l, m, e, hdim, heads, d, group, p0 = 2, 24, 64, 4, 96, 4, 16, 32, 17
+  dt = H.ACT_TORCH[act_dtype]
+  rng = np.random.default_rng(61)
+  layers, final = _build_stack(rng, m, e, hdim, heads, d, group)
+  x = O.cast_act(rng.standard_normal((b, l, m)).astype(np.float32), act_dtype)
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  batch, length, model_dim = (mtf.Dimension("batch", b), mtf.Dimension("length", l),
+                              mtf.Dimension("d_model", m))
+  stack = transformer.make_layer_stack(
+      [(transformer_layers.SelfAttention,
+        dict(num_heads=heads, key_value_size=d)),
+       (moe.MoE1D, dict(num_experts=e, hidden_size=hdim, group_size=group,
+                        second_policy_train="all", second_policy_eval="all",
+                        capacity_factor_eval=float(e))),
+       (transformer_layers.SelfAttention,
+        dict(num_heads=heads, key_value_size=d)),
+       (transformer_layers.DenseReluDense, dict(hidden_size=hdim))],
+      num_layers=1, block_scope=False)
+  model = transformer.Unitransformer(stack, d_model=m, name="decoder",
+                                     autoregressive=True)
+  vdt = mtf.VariableDType(torch.float32, torch.float32, dt)
+  to_t = lambda a: torch.from_numpy(np.ascontiguousarray(a)).to(dt)
+  full_in = mtf.import_tf_tensor(mesh, to_t(x), mtf.Shape([batch, length, model_dim]))
+  y_full, _ = model.call_layers(full_in, vdt, mode="eval")
+  first = x.copy()
+  first[:, p0:] = 0
+  first_in = mtf.import_tf_tensor(mesh, to_t(first),
+                                  mtf.Shape([batch, length, model_dim]))
+  states = []
+  y_first, _ = model.call_layers(first_in, vdt, mode="first_part",
+                                 new_states=states, reuse=True)
+  assert len(states) == 4
+  assert all(t.shape.dimension_names == ["batch", "memory_length", "heads"]
+             for t in states)
+  steps = []
+  for p in range(p0, l):
+    tok = mtf.import_tf_tensor(mesh, to_t(x[:, p]), mtf.Shape([batch, model_dim]))
+    pos = mtf.import_tf_tensor(mesh, torch.full((b,), p, dtype=torch.int32),
+                               mtf.Shape([batch]))
+    new_states = []
+    y_p, _ = model.call_layers(tok, vdt, mode="incremental", position=pos,
+                               states=states, new_states=new_states,
+                               length_dim=length)
+    assert y_p.shape.dimension_names == ["batch", "d_model"]
+    steps.append(y_p)
+    states = new_states
+  init = {"decoder/rms_norm/scale": final}
+  for i, layer in enumerate(layers):
+    prefix = "decoder/layer_%03d/" % i
+    init[prefix + "rms_norm/scale"] = layer["scale"]
+    if layer["kind"] == "attention":
+      for c in "qkvo":
+        init[prefix + "SelfAttention/" + c] = layer["w" + c]
+    elif layer["kind"] == "moe":
+      init[prefix + "MoE1D/top_2_gating/kernel"] = layer["w_gate"]
+      init[prefix + "MoE1D/wi/kernel"] = layer["wi"]
+      init[prefix + "MoE1D/wo/kernel"] = layer["wo"]
+    else:
+      init[prefix + "DenseReluDense/wi/kernel"] = layer["wi"]
+      init[prefix + "DenseReluDense/wo/kernel"] = layer["wo"]
+  assert sorted(init) == sorted(v.name for v in graph.all_variables)
+  lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()}, initial_values=init)
+  want = H.to_np(lowering.export_to_tf_tensor(y_full))
+  got_first = H.to_np(lowering.export_to_tf_tensor(y_first))
+  tol = dict(rtol=2e-4, atol=2e-4) if act_dtype == "float32" else dict(
+      rtol=5e-2, atol=5e-2)
+  # the known first part sees only itself (autoregressive)
+  np.testing.assert_allclose(got_first[:, :p0], want[:, :p0], **tol)
+  for p, y_p in zip(range(p0, l), steps):
+    got = H.to_np(lowering.export_to_tf_tensor(y_p))
+    if act_dtype == "float32":
+      np.testing.assert_allclose(got, want[:, p], err_msg="position %d" % p, **tol)
+    else:
+      # a token whose two best experts nearly tie can be routed differently
+      # when its router input differs by a bf16 ulp between the two runs
+      ok = np.isclose(got, want[:, p], **tol).all(axis=-1)
+      assert ok.mean() >= 0.5, (p, ok)
+  # the final states hold the keys of the full row: layer 0's keys are a
+  # projection of its normed input, the same in both runs
+  k_full = [op for op in graph.operations
+            if type(op).__name__ == "SelfAttentionOperation"][0].inputs[1]
+  np.testing.assert_allclose(
+      H.to_np(lowering.export_to_tf_tensor(states[0])),
+      H.to_np(lowering.export_to_tf_tensor(k_full)), **tol)
+
+
 @pytest.mark.parametrize("train", [False, True])
 def test_layer_stack_with_moe2d(train):
   """MoE2D.call (transformer/moe.py:163-188) inside a LayerStack: the
