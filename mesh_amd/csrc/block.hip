@@ -942,7 +942,7 @@ extern "C" int mesh_moe_self_attention(const void* q, const void* k,
 // dtype, out = sum_m w_m v_m.  The caches are read once: HBM-bound.
 //   q, k_new, v_new, out [B, H*D]; k_cache, v_cache [B, Lm, H*D] (updated in
 //   place); position [B] int32 on the device.
-// Dynamic LDS: max(Lm, 256) + D + 8 floats.
+// Dynamic LDS: max(Lm, 256) + D + 8 + 2048 floats.
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void attention_decode_kernel(
@@ -950,10 +950,11 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
     const T* __restrict__ v_new, T* __restrict__ k_cache,
     T* __restrict__ v_cache, const int32_t* __restrict__ position,
     T* __restrict__ out, int Lm, int H, int D, int vec) {
-  extern __shared__ float dec_smem[];
-  float* wl = dec_smem;            // [max(Lm, 256)] logits, then weights
+  extern __shared__ __attribute__((aligned(16))) float dec_smem[];
+  float* wl = dec_smem;                     // [max(Lm, 256)] logits, then weights
   float* qs = wl + (Lm > 256 ? Lm : 256);   // [D]
-  float* red = qs + D;             // [8]
+  float* red = qs + D;                      // [8]
+  float* part = red + 8;                    // [2048] partial outputs (vec path)
   const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int64_t hd = (int64_t)H * D;
@@ -969,24 +970,55 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
     vc[(int64_t)pos * hd + d] = vnr[d];
   }
   __syncthreads();
-  // logits of the visible rows; row `pos` comes from the step's own key
   constexpr int VN = Vec16B<T>::N;
+  // vec path: a row is CH 16-byte chunks, read by LPR lanes (a power of two
+  // >= CH, <= 64); the block's G = 256 / LPR lane groups take rows g, g + G, ..
+  const int CH = D / VN;
+  int LPR = 1;
+  while (LPR < CH) LPR *= 2;
+  const int G = 256 / LPR, g = tid / LPR, c = tid % LPR;
+  const bool lane_on = c < CH;
+  // logits of the visible rows; row `pos` comes from the step's own key
   float m = -INFINITY;
-  for (int j = tid; j <= pos; j += 256) {
-    const T* kr = j == pos ? knr : kc + (int64_t)j * hd;
-    float acc = 0.f;
-    if (vec) {
-      for (int d0 = 0; d0 < D; d0 += VN) {
-        float f[VN];
-        unpack16(*reinterpret_cast<const uint4*>(kr + d0), f, T());
+  if (vec) {
+    float qv[VN];
 #pragma unroll
-        for (int u = 0; u < VN; ++u) acc = fmaf(qs[d0 + u], f[u], acc);
+    for (int u = 0; u < VN; ++u) qv[u] = lane_on ? qs[c * VN + u] : 0.f;
+    constexpr int UR = 4;                   // rows in flight per lane group
+    for (int j0 = g; j0 <= pos; j0 += G * UR) {
+      uint4 raw[UR];
+#pragma unroll
+      for (int r = 0; r < UR; ++r) {
+        const int j = j0 + r * G;
+        raw[r] = make_uint4(0, 0, 0, 0);
+        if (lane_on && j <= pos) {
+          const T* kr = j == pos ? knr : kc + (int64_t)j * hd;
+          raw[r] = load_streaming(reinterpret_cast<const uint4*>(kr) + c);
+        }
       }
-    } else {
-      for (int d = 0; d < D; ++d) acc = fmaf(qs[d], load_f32<T>(kr + d), acc);
+#pragma unroll
+      for (int r = 0; r < UR; ++r) {
+        const int j = j0 + r * G;
+        float f[VN];
+        unpack16(raw[r], f, T());
+        float acc = 0.f;
+#pragma unroll
+        for (int u = 0; u < VN; ++u) acc = fmaf(qv[u], f[u], acc);
+        for (int off = LPR >> 1; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
+        if (j <= pos) {
+          if (c == 0) wl[j] = acc;
+          m = fmaxf(m, acc);
+        }
+      }
     }
-    wl[j] = acc;
-    m = fmaxf(m, acc);
+  } else {
+    for (int j = tid; j <= pos; j += 256) {
+      const T* kr = j == pos ? knr : kc + (int64_t)j * hd;
+      float acc = 0.f;
+      for (int d = 0; d < D; ++d) acc = fmaf(qs[d], load_f32<T>(kr + d), acc);
+      wl[j] = acc;
+      m = fmaxf(m, acc);
+    }
   }
   auto block_all = [&](float v, bool is_max) {
 #pragma unroll
@@ -1010,26 +1042,45 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
   for (int j = tid; j <= pos; j += 256)
     wl[j] = round_to<T>(expf(wl[j] + neglse));
   __syncthreads();
-  // out[d] = sum_j w_j v[j][d]: the threads of a group cover d, the groups
-  // split the rows; partial sums meet in LDS
-  const int groups = D <= 256 ? 256 / D : 1;
-  float* part = wl;                 // reused below, after the weights are read
-  if (D <= 256) {
-    const int g = tid / D, d = tid - g * D;
-    float acc = 0.f;
-    if (g < groups) {
-      for (int j = g; j <= pos; j += groups) {
-        const T* vr = j == pos ? vnr : vc + (int64_t)j * hd;
-        acc = fmaf(wl[j], load_f32<T>(vr + d), acc);
+  T* orow = out + b * hd + (int64_t)h * D;
+  if (vec) {
+    // out = sum_j w_j v_j: every lane group sums its rows for its chunk, the
+    // groups' partial sums meet in LDS
+    float acc[VN];
+#pragma unroll
+    for (int u = 0; u < VN; ++u) acc[u] = 0.f;
+    constexpr int UR = 4;
+    for (int j0 = g; j0 <= pos; j0 += G * UR) {
+      uint4 raw[UR];
+      float w[UR];
+#pragma unroll
+      for (int r = 0; r < UR; ++r) {
+        const int j = j0 + r * G;
+        raw[r] = make_uint4(0, 0, 0, 0);
+        w[r] = 0.f;
+        if (lane_on && j <= pos) {
+          const T* vr = j == pos ? vnr : vc + (int64_t)j * hd;
+          raw[r] = load_streaming(reinterpret_cast<const uint4*>(vr) + c);
+          w[r] = wl[j];
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < UR; ++r) {
+        float f[VN];
+        unpack16(raw[r], f, T());
+#pragma unroll
+        for (int u = 0; u < VN; ++u) acc[u] = fmaf(w[r], f[u], acc[u]);
       }
     }
-    __syncthreads();                // every weight has been read
-    if (g < groups) part[g * D + d] = acc;
+    if (lane_on) {
+#pragma unroll
+      for (int u = 0; u < VN; ++u) part[g * D + c * VN + u] = acc[u];
+    }
     __syncthreads();
-    if (tid < D) {
+    for (int d = tid; d < D; d += 256) {
       float total = 0.f;
-      for (int gg = 0; gg < groups; ++gg) total += part[gg * D + tid];
-      store_f32<T>(out + b * hd + (int64_t)h * D + tid, total);
+      for (int gg = 0; gg < G; ++gg) total += part[gg * D + d];
+      store_f32<T>(orow + d, total);
     }
   } else {
     for (int d = tid; d < D; d += 256) {
@@ -1038,7 +1089,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
         const T* vr = j == pos ? vnr : vc + (int64_t)j * hd;
         acc = fmaf(wl[j], load_f32<T>(vr + d), acc);
       }
-      store_f32<T>(out + b * hd + (int64_t)h * D + d, acc);
+      store_f32<T>(orow + d, acc);
     }
   }
 }
@@ -1056,16 +1107,17 @@ extern "C" int mesh_moe_attention_decode(const void* q, const void* k_new,
               "attention_decode: bad sizes B=%d Lm=%d H=%d D=%d", B, Lm, H, D);
   MOE_REQUIRE(B <= 65535, MESH_MOE_E_UNSUPPORTED,
               "attention_decode: batch %d > 65535", B);
-  // the partial sums of the last phase reuse the weights' array
-  const size_t floats = (size_t)(Lm > 256 ? Lm : 256) + (size_t)D + 8;
+  const size_t floats = (size_t)(Lm > 256 ? Lm : 256) + (size_t)D + 8 + 2048;
   const size_t smem = floats * sizeof(float);
   MOE_REQUIRE(smem <= 150 * 1024, MESH_MOE_E_UNSUPPORTED,
               "attention_decode: memory length %d does not fit in LDS", Lm);
   hipStream_t st = (hipStream_t)stream;
   const dim3 grid((unsigned)H, (unsigned)B);
   const size_t esz = dtype_size(dtype);
-  const int vec = ((size_t)D * esz) % 16 == 0 &&
-                  (((uintptr_t)k_cache | (uintptr_t)k_new) % 16) == 0;
+  // 16-byte row reads: whole chunks per row, at most 64 of them, aligned
+  const int vec = ((size_t)D * esz) % 16 == 0 && (size_t)D * esz <= 1024 &&
+                  (((uintptr_t)k_cache | (uintptr_t)k_new | (uintptr_t)v_cache |
+                    (uintptr_t)v_new) % 16) == 0;
   if (dtype == MESH_MOE_F32) {
     auto kern = attention_decode_kernel<float>;
     MOE_ALLOW_LDS(kern, smem);
