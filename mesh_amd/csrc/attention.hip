@@ -222,7 +222,6 @@ __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
     }
     {
       const unsigned char* ks = fa_smem + buf * Cfg::STAGE;
-      const unsigned char* vs = ks + Cfg::K_BYTES;
       // S^T: two sub-tiles of 32 keys
       fa_f32x16_t acc_s[2];
 #pragma unroll

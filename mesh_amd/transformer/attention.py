@@ -201,7 +201,6 @@ class SelfAttentionOperation(mtf.Operation):
                        % (sequence_id.shape, q.shape))
     self._num_heads = num_heads
     self._causal = bool(causal)
-    self._has_ids = sequence_id is not None
     self._outputs = [mtf.Tensor(self, q.shape, q.dtype)]
 
   def lower(self, lowering):
