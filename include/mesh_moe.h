@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 21
+#define MESH_MOE_ABI_VERSION 22
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -686,9 +686,10 @@ size_t mesh_moe_attention_weights_workspace_bytes(int B, int L, int H, int D,
                                                   int dtype);
 int mesh_moe_attention_weights(const void* q, const void* k, void* weights,
                                int B, int L, int H, int D, int causal,
-                               const int32_t* sequence_id, int dtype,
-                               void* workspace, size_t workspace_bytes,
-                               void* stream);
+                               const int32_t* sequence_id,
+                               const void* rel_values, const int32_t* rel_bucket,
+                               int num_buckets, int dtype, void* workspace,
+                               size_t workspace_bytes, void* stream);
 
 /*
  * Dropout whose noise is broadcast over some dimensions of x
@@ -718,7 +719,7 @@ int mesh_moe_rms_norm(const void* x, const void* scale, void* y, int64_t rows,
 
 /* Bytes of scratch mesh_moe_self_attention needs. */
 size_t mesh_moe_self_attention_workspace_bytes(int B, int L, int H, int D,
-                                               int dtype);
+                                               int dtype, int relative_bias);
 
 /*
  * Multi-head dot-product self-attention after the q/k/v projections
@@ -741,12 +742,35 @@ size_t mesh_moe_self_attention_workspace_bytes(int B, int L, int H, int D,
  * bias of SelfAttention.compute_bias, transformer/transformer_layers.py:303-316;
  * mesh_moe_attention_weights and mesh_moe_self_attention_backward take the
  * same argument.
+ * rel_values [H,num_buckets] dtype and rel_bucket [2L-1] int32, or both NULL:
+ * the relative attention bias of transformer_layers.py:317-352 -- logit (i, j)
+ * gets rel_values[h][rel_bucket[j - i + L - 1]], rel_bucket being the bucket of
+ * every (memory position - query position) (the caller evaluates
+ * _relative_position_bucket, :1000-1042, once per length).  With a bias the
+ * three-step form runs whatever the shape (pass relative_bias = 1 to
+ * mesh_moe_self_attention_workspace_bytes); mesh_moe_attention_weights takes
+ * the same arguments.
  */
 int mesh_moe_self_attention(const void* q, const void* k, const void* v,
                             void* out, int B, int L, int H, int D, int causal,
-                            const int32_t* sequence_id, int dtype,
-                            void* workspace, size_t workspace_bytes,
+                            const int32_t* sequence_id, const void* rel_values,
+                            const int32_t* rel_bucket, int num_buckets,
+                            int dtype, void* workspace, size_t workspace_bytes,
                             void* stream);
+
+/*
+ * Gradient of the relative attention bias values (the gradient of the
+ * mtf.gather at transformer/transformer_layers.py:351):
+ * dvalues[h][bucket] = sum over the batch and the (query i, key j) pairs with
+ * rel_bucket[j - i + L - 1] == bucket of dlogits[b*H + h][i][j].
+ *   dlogits [B*H,L,L] dtype (what mesh_moe_softmax_backward writes);
+ *   dvalues [H,num_buckets] dtype; workspace H*num_buckets floats.
+ * Float32 atomics: the order of the sum is not fixed.
+ */
+int mesh_moe_relative_bias_backward(const void* dlogits,
+                                    const int32_t* rel_bucket, void* dvalues,
+                                    float* workspace, int B, int L, int H,
+                                    int num_buckets, int dtype, void* stream);
 
 /* Bytes of scratch mesh_moe_self_attention_backward needs; 0 for shapes it does
  * not take. */

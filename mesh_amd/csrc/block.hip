@@ -154,10 +154,15 @@ __global__ __launch_bounds__(256) void transpose_heads_kernel(
 // ---------------------------------------------------------------------------
 // With seq [B, L] (rows are (batch, head, query), H heads) a key is visible
 // only if it carries the query's sequence id (transformer_layers.py:303-316).
+// With rel_values [H, NB] and rel_bucket [2 L - 1] the logit of (query i, key j)
+// gets the relative attention bias rel_values[head][rel_bucket[j - i + L - 1]]
+// (transformer_layers.py:317-352) before the softmax.
 template <typename T>
 __global__ __launch_bounds__(256) void attention_softmax_kernel(
     const float* __restrict__ logits, T* __restrict__ weights, int64_t rows,
-    int L, int causal, const int32_t* __restrict__ seq, int H) {
+    int L, int causal, const int32_t* __restrict__ seq, int H,
+    const T* __restrict__ rel_values, const int32_t* __restrict__ rel_bucket,
+    int NB) {
   const int lane = threadIdx.x & 63;
   const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
   if (row >= rows) return;
@@ -166,22 +171,71 @@ __global__ __launch_bounds__(256) void attention_softmax_kernel(
   const int32_t* sb = seq ? seq + (row / L / H) * L : nullptr;
   const int my = sb ? sb[i] : 0;
   const float* xr = logits + row * L;
+  const T* rv = rel_values ? rel_values + ((row / L) % H) * NB : nullptr;
+  const int32_t* rb = rv ? rel_bucket + (L - 1 - i) : nullptr;   // rb[j]: bucket of j - i
+  auto logit = [&](int j) {
+    return rv ? xr[j] + load_f32<T>(rv + rb[j]) : xr[j];
+  };
   float m = -INFINITY;
   for (int j = lane; j < visible; j += 64)
-    if (!sb || sb[j] == my) m = fmaxf(m, xr[j]);
+    if (!sb || sb[j] == my) m = fmaxf(m, logit(j));
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) m = fmaxf(m, __shfl_xor(m, off));
   const float negm = -m;
   float sum = 0.f;
   for (int j = lane; j < visible; j += 64)
-    if (!sb || sb[j] == my) sum += expf(xr[j] + negm);
+    if (!sb || sb[j] == my) sum += expf(logit(j) + negm);
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
   const float neglse = -(logf(sum) + m);
   T* wr = weights + row * L;
   for (int j = lane; j < L; j += 64)
     store_f32<T>(wr + j, j < visible && (!sb || sb[j] == my)
-                             ? expf(xr[j] + neglse) : 0.0f);
+                             ? expf(logit(j) + neglse) : 0.0f);
+}
+
+__global__ void fill_zero_f32_kernel(float* p, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0.f;
+}
+
+template <typename T>
+__global__ void round_f32_kernel(const float* src, T* dst, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) store_f32<T>(dst + i, src[i]);
+}
+
+// Gradient of the relative attention bias values: dvalues[h][bucket] = sum over
+// the batch and the (query, key) pairs of that bucket of dlogits (the gradient
+// of mtf.gather, transformer_layers.py:351).  One wavefront per row of
+// dlogits [B*H, L, L]; a block's four rows meet in an LDS histogram and go to
+// the float32 accumulator acc [H, NB] with one atomic per bucket.
+template <typename T>
+__global__ __launch_bounds__(256) void relative_bias_backward_kernel(
+    const T* __restrict__ dlogits, const int32_t* __restrict__ rel_bucket,
+    float* __restrict__ acc, int64_t rows, int L, int H, int NB) {
+  extern __shared__ float rb_hist[];           // [4][NB]
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int i = threadIdx.x; i < 4 * NB; i += 256) rb_hist[i] = 0.f;
+  __syncthreads();
+  const int64_t row = (int64_t)blockIdx.x * 4 + wave;
+  if (row < rows) {
+    const int i = (int)(row % L);
+    const T* dr = dlogits + row * L;
+    const int32_t* rb = rel_bucket + (L - 1 - i);
+    for (int j = lane; j < L; j += 64) {
+      const float v = load_f32<T>(dr + j);
+      if (v != 0.f) atomicAdd(&rb_hist[wave * NB + rb[j]], v);
+    }
+  }
+  __syncthreads();
+  for (int i = threadIdx.x; i < 4 * NB; i += 256) {
+    const int w = i / NB, bkt = i - w * NB;
+    const int64_t r = (int64_t)blockIdx.x * 4 + w;
+    const float v = rb_hist[i];
+    if (r < rows && v != 0.f)
+      atomicAdd(acc + ((r / L) % H) * NB + bkt, v);
+  }
 }
 
 // The same softmax for bf16 weights and rows of ITERS * 512 logits: a lane
@@ -245,11 +299,14 @@ template <typename T>
 static void launch_attention_softmax(const float* logits, T* weights,
                                      int64_t rows, int L, int causal,
                                      const int32_t* seq, int H,
+                                     const void* rel_values,
+                                     const int32_t* rel_bucket, int NB,
                                      hipStream_t st) {
   const unsigned blocks = (unsigned)((rows + 3) / 4);
-  if (seq != nullptr)
+  if (seq != nullptr || rel_values != nullptr)
     return attention_softmax_kernel<T><<<blocks, 256, 0, st>>>(
-        logits, weights, rows, L, causal, seq, H);
+        logits, weights, rows, L, causal, seq, H, (const T*)rel_values,
+        rel_bucket, NB);
   if constexpr (sizeof(T) == 2) {
     const bool aligned =
         (((uintptr_t)logits | (uintptr_t)weights) % 32) == 0;
@@ -266,14 +323,15 @@ static void launch_attention_softmax(const float* logits, T* weights,
       return attention_softmax_rows_kernel<8><<<blocks, 256, 0, st>>>(
           logits, weights, rows, causal);
   }
-  attention_softmax_kernel<T><<<blocks, 256, 0, st>>>(logits, weights, rows, L,
-                                                      causal, nullptr, H);
+  attention_softmax_kernel<T><<<blocks, 256, 0, st>>>(
+      logits, weights, rows, L, causal, nullptr, H, nullptr, rel_bucket, NB);
 }
 
 template <typename T>
 static int run_attention(const T* q, const T* k, const T* v, T* out, int B,
                          int L, int H, int D, int causal, const int32_t* seq,
-                         int dtype, void* workspace, hipStream_t st) {
+                         const void* rel_values, const int32_t* rel_bucket,
+                         int NB, int dtype, void* workspace, hipStream_t st) {
   const int BH = B * H;
   const size_t hd = (size_t)BH * L * D, ll = (size_t)BH * L * L;
   auto up = [](uintptr_t p) { return (p + 255) & ~(uintptr_t)255; };
@@ -296,7 +354,8 @@ static int run_attention(const T* q, const T* k, const T* v, T* out, int B,
   int rc = batched_gemm_nt(qh, kh, logits, BH, L, L, D, dtype, true, st);
   if (rc != 0) return rc;
   const int64_t rows = (int64_t)BH * L;
-  launch_attention_softmax<T>(logits, weights, rows, L, causal, seq, H, st);
+  launch_attention_softmax<T>(logits, weights, rows, L, causal, seq, H,
+                              rel_values, rel_bucket, NB, st);
   MOE_CHECK_LAUNCH("self_attention (softmax)");
   rc = batched_gemm_nt(weights, vt, oh, BH, L, D, L, dtype, false, st);
   if (rc != 0) return rc;
@@ -564,7 +623,8 @@ __global__ __launch_bounds__(256) void softmax_backward_rows_kernel(
 template <typename T>
 static int run_attention_weights(const T* q, const T* k, T* weights, int B,
                                  int L, int H, int D, int causal,
-                                 const int32_t* seq, int dtype,
+                                 const int32_t* seq, const void* rel_values,
+                                 const int32_t* rel_bucket, int NB, int dtype,
                                  void* workspace, hipStream_t st) {
   const int BH = B * H;
   const size_t hd = (size_t)BH * L * D;
@@ -582,7 +642,8 @@ static int run_attention_weights(const T* q, const T* k, T* weights, int B,
   int rc = batched_gemm_nt(qh, kh, logits, BH, L, L, D, dtype, true, st);
   if (rc != 0) return rc;
   const int64_t rows = (int64_t)BH * L;
-  launch_attention_softmax<T>(logits, weights, rows, L, causal, seq, H, st);
+  launch_attention_softmax<T>(logits, weights, rows, L, causal, seq, H,
+                              rel_values, rel_bucket, NB, st);
   MOE_CHECK_LAUNCH("attention_weights (softmax)");
   return 0;
 }
@@ -824,7 +885,10 @@ extern "C" size_t mesh_moe_attention_weights_workspace_bytes(int B, int L,
 extern "C" int mesh_moe_attention_weights(const void* q, const void* k,
                                           void* weights, int B, int L, int H,
                                           int D, int causal,
-                                          const int32_t* sequence_id, int dtype,
+                                          const int32_t* sequence_id,
+                                          const void* rel_values,
+                                          const int32_t* rel_bucket,
+                                          int num_buckets, int dtype,
                                           void* workspace,
                                           size_t workspace_bytes,
                                           void* stream) {
@@ -844,11 +908,13 @@ extern "C" int mesh_moe_attention_weights(const void* q, const void* k,
   if (dtype == MESH_MOE_F32)
     return run_attention_weights<float>((const float*)q, (const float*)k,
                                         (float*)weights, B, L, H, D,
-                                        causal ? 1 : 0, sequence_id, dtype,
+                                        causal ? 1 : 0, sequence_id, rel_values,
+                                        rel_bucket, num_buckets, dtype,
                                         workspace, st);
   return run_attention_weights<bf16_t>((const bf16_t*)q, (const bf16_t*)k,
                                        (bf16_t*)weights, B, L, H, D,
-                                       causal ? 1 : 0, sequence_id, dtype,
+                                       causal ? 1 : 0, sequence_id, rel_values,
+                                       rel_bucket, num_buckets, dtype,
                                        workspace, st);
 }
 
@@ -884,10 +950,11 @@ extern "C" int mesh_moe_rms_norm(const void* x, const void* scale, void* y,
 }
 
 extern "C" size_t mesh_moe_self_attention_workspace_bytes(int B, int L, int H,
-                                                          int D, int dtype) {
+                                                          int D, int dtype,
+                                                          int relative_bias) {
   if (B < 1 || L < 1 || H < 1 || D < 1 || !valid_dtype(dtype)) return 0;
-  if (flash_attention_supported(L, H, D, dtype, nullptr, nullptr, nullptr,
-                                nullptr))
+  if (!relative_bias && flash_attention_supported(L, H, D, dtype, nullptr,
+                                                  nullptr, nullptr, nullptr))
     return flash_attention_workspace_bytes(B, L, H, D);
   const size_t b = dtype_size(dtype);
   const size_t hd = (size_t)B * H * L * D, ll = (size_t)B * H * L * L;
@@ -897,7 +964,10 @@ extern "C" size_t mesh_moe_self_attention_workspace_bytes(int B, int L, int H,
 extern "C" int mesh_moe_self_attention(const void* q, const void* k,
                                        const void* v, void* out, int B, int L,
                                        int H, int D, int causal,
-                                       const int32_t* sequence_id, int dtype,
+                                       const int32_t* sequence_id,
+                                       const void* rel_values,
+                                       const int32_t* rel_bucket,
+                                       int num_buckets, int dtype,
                                        void* workspace, size_t workspace_bytes,
                                        void* stream) {
   MOE_REQUIRE(q && k && v && out && workspace, MESH_MOE_E_ARG,
@@ -909,11 +979,17 @@ extern "C" int mesh_moe_self_attention(const void* q, const void* k,
   MOE_REQUIRE((int64_t)B * H <= 65535, MESH_MOE_E_UNSUPPORTED,
               "self_attention: batch * heads = %lld > 65535",
               (long long)B * H);
-  MOE_REQUIRE(workspace_bytes >=
-                  mesh_moe_self_attention_workspace_bytes(B, L, H, D, dtype),
+  MOE_REQUIRE((rel_values == nullptr) == (rel_bucket == nullptr) &&
+                  (rel_values == nullptr || num_buckets >= 1),
+              MESH_MOE_E_ARG,
+              "self_attention: rel_values, rel_bucket and num_buckets go "
+              "together");
+  MOE_REQUIRE(workspace_bytes >= mesh_moe_self_attention_workspace_bytes(
+                                     B, L, H, D, dtype, rel_values != nullptr),
               MESH_MOE_E_ARG, "self_attention: workspace too small");
   hipStream_t st = (hipStream_t)stream;
-  if (flash_attention_supported(L, H, D, dtype, nullptr, nullptr, nullptr,
+  if (rel_values == nullptr &&
+      flash_attention_supported(L, H, D, dtype, nullptr, nullptr, nullptr,
                                 nullptr)) {
     // fused kernel: the logits stay on chip
     MOE_REQUIRE(flash_attention_supported(L, H, D, dtype, q, k, v, out),
@@ -925,12 +1001,12 @@ extern "C" int mesh_moe_self_attention(const void* q, const void* k,
   if (dtype == MESH_MOE_F32)
     return run_attention<float>((const float*)q, (const float*)k,
                                 (const float*)v, (float*)out, B, L, H, D,
-                                causal ? 1 : 0, sequence_id, dtype, workspace,
-                                st);
+                                causal ? 1 : 0, sequence_id, rel_values,
+                                rel_bucket, num_buckets, dtype, workspace, st);
   return run_attention<bf16_t>((const bf16_t*)q, (const bf16_t*)k,
                                (const bf16_t*)v, (bf16_t*)out, B, L, H, D,
-                               causal ? 1 : 0, sequence_id, dtype, workspace,
-                               st);
+                               causal ? 1 : 0, sequence_id, rel_values,
+                               rel_bucket, num_buckets, dtype, workspace, st);
 }
 
 // ---------------------------------------------------------------------------
@@ -1134,6 +1210,46 @@ extern "C" int mesh_moe_attention_decode(const void* q, const void* k_new,
                                   H, D, vec);
   }
   MOE_CHECK_LAUNCH("attention_decode");
+  return 0;
+}
+
+extern "C" int mesh_moe_relative_bias_backward(const void* dlogits,
+                                               const int32_t* rel_bucket,
+                                               void* dvalues, float* workspace,
+                                               int B, int L, int H,
+                                               int num_buckets, int dtype,
+                                               void* stream) {
+  MOE_REQUIRE(dlogits && rel_bucket && dvalues && workspace, MESH_MOE_E_ARG,
+              "relative_bias_backward: null pointer");
+  MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG,
+              "relative_bias_backward: bad dtype %d", dtype);
+  MOE_REQUIRE(B >= 1 && L >= 1 && H >= 1 && num_buckets >= 1 &&
+                  num_buckets <= 4096,
+              MESH_MOE_E_ARG,
+              "relative_bias_backward: bad sizes B=%d L=%d H=%d buckets=%d", B,
+              L, H, num_buckets);
+  const int64_t rows = (int64_t)B * H * L;
+  const int64_t blocks = (rows + 3) / 4;
+  MOE_REQUIRE(blocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
+              "relative_bias_backward: too many rows (%lld)", (long long)rows);
+  hipStream_t st = (hipStream_t)stream;
+  const int64_t n = (int64_t)H * num_buckets;
+  const unsigned fb = (unsigned)((n + 255) / 256);
+  fill_zero_f32_kernel<<<fb, 256, 0, st>>>(workspace, n);
+  MOE_CHECK_LAUNCH("relative_bias_backward (clear)");
+  const size_t smem = sizeof(float) * 4 * (size_t)num_buckets;
+  if (dtype == MESH_MOE_F32) {
+    relative_bias_backward_kernel<float><<<(unsigned)blocks, 256, smem, st>>>(
+        (const float*)dlogits, rel_bucket, workspace, rows, L, H, num_buckets);
+    MOE_CHECK_LAUNCH("relative_bias_backward");
+    round_f32_kernel<float><<<fb, 256, 0, st>>>(workspace, (float*)dvalues, n);
+  } else {
+    relative_bias_backward_kernel<bf16_t><<<(unsigned)blocks, 256, smem, st>>>(
+        (const bf16_t*)dlogits, rel_bucket, workspace, rows, L, H, num_buckets);
+    MOE_CHECK_LAUNCH("relative_bias_backward");
+    round_f32_kernel<bf16_t><<<fb, 256, 0, st>>>(workspace, (bf16_t*)dvalues, n);
+  }
+  MOE_CHECK_LAUNCH("relative_bias_backward (round)");
   return 0;
 }
 

@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 21
+ABI_VERSION = 22
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -128,7 +128,11 @@ _SIGNATURES = {
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "mesh_moe_attention_weights": (ctypes.c_int, [
         _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
-        ctypes.c_int, _vp, ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
+        ctypes.c_int, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, _vp,
+        ctypes.c_size_t, _vp]),
+    "mesh_moe_relative_bias_backward": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, _vp]),
     "mesh_moe_broadcast_dropout": (ctypes.c_int, [
         _vp, _vp, _vp, ctypes.c_float, _vp, _vp, ctypes.c_int64, ctypes.c_int64,
         ctypes.c_int64, ctypes.c_int, _vp]),
@@ -179,11 +183,12 @@ _SIGNATURES = {
         _vp, _vp, _vp, ctypes.c_int64, ctypes.c_int, ctypes.c_double,
         ctypes.c_int, _vp]),
     "mesh_moe_self_attention_workspace_bytes": (ctypes.c_size_t, [
-        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int]),
     "mesh_moe_self_attention": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
-        ctypes.c_int, ctypes.c_int, _vp, ctypes.c_int, _vp, ctypes.c_size_t,
-        _vp]),
+        ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
+        _vp, ctypes.c_size_t, _vp]),
     "mesh_moe_self_attention_backward_workspace_bytes": (ctypes.c_size_t, [
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "mesh_moe_self_attention_backward": (ctypes.c_int, [
@@ -1135,7 +1140,8 @@ def dense(x, w_packed, activation=None):
   return y.reshape(tuple(x.shape[:-1]) + (n,))
 
 
-def self_attention(q, k, v, num_heads, causal, sequence_id=None):
+def self_attention(q, k, v, num_heads, causal, sequence_id=None,
+                   relative_bias=None):
   """q, k, v [B, L, H*D] -> [B, L, H*D] (attention.attention with float32
   logits, transformer/attention.py:27-88); sequence_id [B, L] int32 or None:
   a query sees only keys of its own sequence
@@ -1148,14 +1154,15 @@ def self_attention(q, k, v, num_heads, causal, sequence_id=None):
   d = hd // num_heads
   code = dtype_code(q.dtype)
   out = torch.empty_like(q)
-  ws_bytes = lib.mesh_moe_self_attention_workspace_bytes(b, l, num_heads, d,
-                                                         code)
+  ws_bytes = lib.mesh_moe_self_attention_workspace_bytes(
+      b, l, num_heads, d, code, int(relative_bias is not None))
   ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=q.device)
   with _stage("self_attention"):
     _check(lib.mesh_moe_self_attention(
         _dev(q, "q"), _dev(k, "k", q.dtype, (b, l, hd)),
         _dev(v, "v", q.dtype, (b, l, hd)), out.data_ptr(), b, l, num_heads, d,
-        int(bool(causal)), _sequence_id_ptr(sequence_id, b, l), code,
+        int(bool(causal)), _sequence_id_ptr(sequence_id, b, l),
+        *_relative_bias_ptrs(relative_bias, q.dtype, num_heads, l), code,
         ws.data_ptr(), ws_bytes, _stream()), "self_attention")
   return out
 
@@ -1292,9 +1299,23 @@ def _sequence_id_ptr(sequence_id, b, l):
   return _dev(sequence_id, "sequence_id", torch.int32, (b, l))
 
 
-def attention_weights(q, k, num_heads, causal, sequence_id=None):
+def _relative_bias_ptrs(relative_bias, dtype, num_heads, l):
+  """relative_bias = (values [H, NB] of the activation dtype, bucket [2L-1]
+  int32) or None -> (values pointer, bucket pointer, NB)."""
+  if relative_bias is None:
+    return None, None, 0
+  values, bucket = relative_bias
+  nb = values.shape[-1]
+  return (_dev(values, "relative bias values", dtype, (num_heads, nb)),
+          _dev(bucket, "relative bias buckets", torch.int32, (2 * l - 1,)), nb)
+
+
+def attention_weights(q, k, num_heads, causal, sequence_id=None,
+                      relative_bias=None):
   """q, k [B, L, H*D] -> softmax(q . k + visibility) [B*H, L, L] in q's dtype;
-  sequence_id [B, L] int32: keys of other sequences are not visible."""
+  sequence_id [B, L] int32: keys of other sequences are not visible;
+  relative_bias = (values [H, NB], bucket [2L-1] int32): the relative attention
+  bias values[h][bucket[j - i + L - 1]] is added to logit (i, j)."""
   lib = load_library()
   b, l, hd = q.shape
   d = hd // num_heads
@@ -1307,6 +1328,7 @@ def attention_weights(q, k, num_heads, causal, sequence_id=None):
     _check(lib.mesh_moe_attention_weights(
         _dev(q, "q"), _dev(k, "k", q.dtype, (b, l, hd)), weights.data_ptr(), b,
         l, num_heads, d, 1 if causal else 0, _sequence_id_ptr(sequence_id, b, l),
+        *_relative_bias_ptrs(relative_bias, q.dtype, num_heads, l),
         code, ws.data_ptr(), ws_bytes, _stream()), "attention_weights")
   return weights
 
@@ -1325,8 +1347,26 @@ def softmax_backward(weights, dweights):
   return out
 
 
+def relative_bias_backward(dlogits, bucket, num_heads, num_buckets):
+  """dlogits [B*H, L, L], bucket [2L-1] int32 -> dvalues [H, NB] (dlogits'
+  dtype): the sum of dlogits over the batch and every bucket's pairs."""
+  lib = load_library()
+  bh, l, _ = dlogits.shape
+  out = torch.empty((num_heads, num_buckets), dtype=dlogits.dtype,
+                    device=dlogits.device)
+  ws = torch.empty((num_heads * num_buckets,), dtype=torch.float32,
+                   device=dlogits.device)
+  with _stage("relative_bias_backward"):
+    _check(lib.mesh_moe_relative_bias_backward(
+        _dev(dlogits, "dlogits"), _dev(bucket, "bucket", torch.int32, (2 * l - 1,)),
+        out.data_ptr(), ws.data_ptr(), bh // num_heads, l, num_heads,
+        num_buckets, dtype_code(dlogits.dtype), _stream()),
+        "relative_bias_backward")
+  return out
+
+
 def self_attention_backward(q, k, v, dout, num_heads, causal, fused=None,
-                            sequence_id=None):
+                            sequence_id=None, relative_bias=None):
   """Backward of self_attention: q, k, v, dout [B, L, H*D] -> (dq, dk, dv).
   Shapes the fused kernels take (bf16, d_kv 64 or 128, L a multiple of 8) run
   mesh_moe_self_attention_backward: nothing [L, L] reaches memory.  Otherwise
@@ -1336,12 +1376,19 @@ def self_attention_backward(q, k, v, dout, num_heads, causal, fused=None,
     dlogits  = softmax backward
     dq = dlogits . k,       dk = dlogits^T . q
   with heads moved to the front and back by torch permutes.  fused=True raises
-  for shapes the fused kernels do not take."""
+  for shapes the fused kernels do not take.  With relative_bias = (values
+  [H, NB], bucket [2L-1]) the composed form runs and the gradient of the values
+  is the fourth result."""
   b, l, hd = q.shape
   h = num_heads
   if hd % h:
     raise MoeHipError("q channels %d not divisible by %d heads" % (hd, h))
   d = hd // h
+  if relative_bias is not None:
+    if fused:
+      raise MoeHipError("self_attention_backward: the fused kernels take no "
+                        "relative attention bias")
+    fused = False
   if fused is None or fused:
     lib = load_library()
     code = dtype_code(q.dtype)
@@ -1369,10 +1416,14 @@ def self_attention_backward(q, k, v, dout, num_heads, causal, fused=None,
     return t.reshape(b, h, l, d).permute(0, 2, 1, 3).reshape(b, l, hd) \
         .contiguous()
   qh, kh, vh, doh = (heads_first(t) for t in (q, k, v, dout))
-  weights = attention_weights(q, k, h, causal, sequence_id)
+  weights = attention_weights(q, k, h, causal, sequence_id, relative_bias)
   dweights, dvh = expert_linear_backward(weights, doh, vh)
   dlogits = softmax_backward(weights, dweights)
   del weights, dweights
   dqh = expert_linear(dlogits, pack_weights(kh, q.dtype))
   _, dkh = expert_linear_backward(dlogits, qh, vh, want_da=False)
-  return heads_last(dqh), heads_last(dkh), heads_last(dvh)
+  grads = (heads_last(dqh), heads_last(dkh), heads_last(dvh))
+  if relative_bias is None:
+    return grads
+  values, bucket = relative_bias
+  return grads + (relative_bias_backward(dlogits, bucket, h, values.shape[-1]),)

@@ -32,6 +32,8 @@ rounds partial sums (here: one rounding of a float32 sum).
 Citations are to files under the reference tree (mesh_tensorflow/...).
 """
 
+import math
+
 import numpy as np
 
 from oracle import moe_oracle as O
@@ -80,6 +82,48 @@ def broadcast_dropout(x, noise, axis, act_dtype="float32"):
             act_dtype)
 
 
+def relative_position_bucket(relative_position, bidirectional=True,
+                             num_buckets=32, max_distance=128):
+  """_relative_position_bucket (transformer/transformer_layers.py:1000-1042):
+  relative_position = memory position - query position (integers) -> bucket
+  in [0, num_buckets).  Half of the buckets hold exact small distances, the
+  other half grow logarithmically up to max_distance; with bidirectional the
+  positive relative positions take the upper half of the range.  The
+  logarithmic part is float32 arithmetic in the reference's op order
+  (to_float(n) / max_exact, log, / the Python constant, * the integer, cast
+  to int32 = truncation)."""
+  rp = np.asarray(relative_position, np.int64)
+  ret = np.zeros(rp.shape, np.int64)
+  n = -rp
+  if bidirectional:
+    num_buckets //= 2
+    ret = ret + (n < 0).astype(np.int64) * num_buckets
+    n = np.abs(n)
+  else:
+    n = np.maximum(n, 0)
+  max_exact = num_buckets // 2
+  is_small = n < max_exact
+  with np.errstate(divide="ignore"):
+    ratio = np.log(n.astype(F32) / F32(max_exact)).astype(F32)
+  scaled = (ratio / F32(math.log(max_distance / max_exact))).astype(F32) \
+      * F32(num_buckets - max_exact)
+  # (the small distances, whose logarithm is negative or -inf, are not taken)
+  val_if_large = max_exact + np.where(is_small, 0, scaled).astype(np.int64)
+  val_if_large = np.minimum(val_if_large, num_buckets - 1)
+  return ret + np.where(is_small, n, val_if_large)
+
+
+def relative_attention_bias(values, length, bidirectional, max_distance=128):
+  """The bias SelfAttention.compute_bias adds for relative_attention_type
+  "bias" / "bias_shared" (transformer_layers.py:317-352): values
+  [H, num_buckets] gathered at the bucket of (memory position - query
+  position) -> [1, H, L(query), L(key)]."""
+  pos = np.arange(length)
+  bucket = relative_position_bucket(pos[None, :] - pos[:, None], bidirectional,
+                                    values.shape[-1], max_distance)
+  return np.asarray(values, F32)[:, bucket][None]
+
+
 def _visibility_bias(l, causal, sequence_id):
   """Sum of the attention biases of SelfAttention.compute_bias
   (transformer/transformer_layers.py:272-316) for the options built here, as
@@ -98,7 +142,7 @@ def _visibility_bias(l, causal, sequence_id):
 
 
 def self_attention(x, wq, wk, wv, wo, num_heads, causal, act_dtype="float32",
-                   weights_noise=None, sequence_id=None):
+                   weights_noise=None, sequence_id=None, relative_values=None):
   """SelfAttention.call for the train / eval modes with the default options
   (transformer/transformer_layers.py:223-271) around attention.attention with
   float32 logits (transformer/attention.py:27-88).
@@ -120,7 +164,8 @@ def self_attention(x, wq, wk, wv, wo, num_heads, causal, act_dtype="float32",
   k = dense(x, wk, act_dtype).reshape(b, l, num_heads, d)
   v = dense(x, wv, act_dtype).reshape(b, l, num_heads, d)
   logits = np.einsum("blhd,bmhd->bhlm", q, k).astype(F32)        # float32
-  logits = (logits + _visibility_bias(l, causal, sequence_id)).astype(F32)
+  logits = (logits + _attention_bias(l, causal, sequence_id, relative_values,
+                                     act_dtype)).astype(F32)
   weights = _r(O.softmax(logits), act_dtype)                     # cast to v's
   if weights_noise is not None:
     weights = broadcast_dropout(weights, weights_noise, 2, act_dtype)
@@ -128,7 +173,21 @@ def self_attention(x, wq, wk, wv, wo, num_heads, causal, act_dtype="float32",
   return dense(o.reshape(b, l, hd), wo, act_dtype)
 
 
-def _attention_core(q, k, v, num_heads, causal, act_dtype, sequence_id=None):
+def _attention_bias(l, causal, sequence_id, relative_values, act_dtype):
+  """mtf.add_n of the biases (transformer_layers.py:352): the visibility
+  biases plus, with relative_values [H, num_buckets], the relative attention
+  bias (buckets of a bidirectional layout unless causal, :321-325); the sum is
+  formed in the activation dtype and cast to the logits' float32
+  (attention.py:78-79)."""
+  bias = _visibility_bias(l, causal, sequence_id)
+  if relative_values is None:
+    return bias
+  rel = relative_attention_bias(_r(relative_values, act_dtype), l, not causal)
+  return _r(_r(bias, act_dtype) + rel, act_dtype).astype(F32)
+
+
+def _attention_core(q, k, v, num_heads, causal, act_dtype, sequence_id=None,
+                    relative_values=None):
   """attention.attention with float32 logits (attention.py:27-88) on
   [B, L, H*D] activation-dtype tensors -> [B, L, H*D]; sequence_id [B, L]
   integers or None."""
@@ -136,7 +195,8 @@ def _attention_core(q, k, v, num_heads, causal, act_dtype, sequence_id=None):
   d = hd // num_heads
   q, k, v = (t.reshape(b, l, num_heads, d) for t in (q, k, v))
   logits = np.einsum("blhd,bmhd->bhlm", q, k).astype(F32)
-  logits = (logits + _visibility_bias(l, causal, sequence_id)).astype(F32)
+  logits = (logits + _attention_bias(l, causal, sequence_id, relative_values,
+                                     act_dtype)).astype(F32)
   weights = _r(O.softmax(logits), act_dtype)
   return _r(np.einsum("bhlm,bmhd->blhd", weights, v), act_dtype).reshape(b, l, hd)
 
@@ -313,17 +373,20 @@ def dense_backward(x, w, dy, act_dtype="float32", activation=None):
 
 
 def attention_core_backward(q, k, v, dout, num_heads, causal,
-                            act_dtype="float32", sequence_id=None):
+                            act_dtype="float32", sequence_id=None,
+                            relative_values=None):
   """(dq, dk, dv) of _attention_core on [B, L, H*D] tensors: the weights as
   the forward pass rounds them; dweights = dout v^T, dv = weights^T dout,
   dlogits = weights (dweights - sum_k dweights weights), dq = dlogits k,
-  dk = dlogits^T q."""
+  dk = dlogits^T q; with relative_values [H, num_buckets] also their gradient
+  as a fourth result."""
   b, l, hd = q.shape
   d = hd // num_heads
   q, k, v, dout = (_r(t, act_dtype).reshape(b, l, num_heads, d)
                    for t in (q, k, v, dout))
   logits = np.einsum("blhd,bmhd->bhlm", q, k).astype(F32)
-  logits = (logits + _visibility_bias(l, causal, sequence_id)).astype(F32)
+  logits = (logits + _attention_bias(l, causal, sequence_id, relative_values,
+                                     act_dtype)).astype(F32)
   weights = _r(O.softmax(logits), act_dtype)
   dweights = _r(np.einsum("blhd,bmhd->bhlm", dout, v), act_dtype)
   dv = _r(np.einsum("bhlm,blhd->bmhd", weights, dout), act_dtype)
@@ -331,4 +394,16 @@ def attention_core_backward(q, k, v, dout, num_heads, causal,
   dlogits = _r(weights * (dweights - dot), act_dtype)
   dq = _r(np.einsum("bhlm,bmhd->blhd", dlogits, k), act_dtype)
   dk = _r(np.einsum("bhlm,blhd->bmhd", dlogits, q), act_dtype)
-  return tuple(t.reshape(b, l, hd) for t in (dq, dk, dv))
+  grads = tuple(t.reshape(b, l, hd) for t in (dq, dk, dv))
+  if relative_values is None:
+    return grads
+  # the bias enters the logits once per batch entry: its gradient is dlogits
+  # summed over the batch, scattered back to the buckets (gather's gradient)
+  pos = np.arange(l)
+  nb = np.asarray(relative_values).shape[-1]
+  bucket = relative_position_bucket(pos[None, :] - pos[:, None], not causal, nb)
+  dvalues = np.zeros((num_heads, nb), F32)
+  per_head = dlogits.astype(F32).sum(0)                        # [H, L, L]
+  for h in range(num_heads):
+    np.add.at(dvalues[h], bucket.reshape(-1), per_head[h].reshape(-1))
+  return grads + (_r(dvalues, act_dtype),)

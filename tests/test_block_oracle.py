@@ -150,6 +150,70 @@ def test_attention_incremental_is_a_row_of_causal_attention():
       np.testing.assert_array_equal(k2[i, pi + 1:], kc[i, pi + 1:])
 
 
+def test_relative_position_bucket_known_values():
+  """The bucket rule by its definition (transformer_layers.py:1000-1042): half
+  of the range exact, the other half logarithmic up to max_distance, positive
+  relative positions in the upper half when bidirectional, invisible (clamped
+  to 0) when not."""
+  rp = B.relative_position_bucket
+  # bidirectional, 32 buckets: 16 per direction, 8 exact
+  assert list(rp(np.arange(0, -8, -1))) == list(range(8))
+  assert list(rp(np.arange(0, 8))) == [0] + list(range(17, 24))
+  assert rp(np.array(-8)) == 8 and rp(np.array(8)) == 24
+  assert rp(np.array(-127)) == 15 and rp(np.array(-128)) == 15
+  assert rp(np.array(-100000)) == 15 and rp(np.array(100000)) == 31
+  # boundaries of the logarithmic half: n = 8 * 16^(i/8) enters bucket 8 + i
+  for i in range(1, 8):
+    edge = 8.0 * 16.0 ** (i / 8.0)
+    lo, hi = int(np.floor(edge - 1e-9)), int(np.ceil(edge + 1e-9))
+    if lo != hi:        # the edge itself is not an integer: no rounding doubt
+      assert rp(np.array(-lo)) == 8 + i - 1 and rp(np.array(-hi)) == 8 + i
+  # unidirectional: 16 exact, positive relative positions count as 0
+  assert list(rp(np.arange(0, -16, -1), bidirectional=False)) == list(range(16))
+  assert list(rp(np.arange(1, 5), bidirectional=False)) == [0, 0, 0, 0]
+  assert rp(np.array(-16), False) == 16 and rp(np.array(-127), False) == 31
+  got = rp(np.arange(0, -300, -1), bidirectional=False)
+  assert (np.diff(got) >= 0).all() and got.max() == 31
+  # the bias is a function of (memory position - query position) only
+  values = np.arange(2 * 32, dtype=np.float32).reshape(2, 32)
+  bias = B.relative_attention_bias(values, 20, True)
+  assert bias.shape == (1, 2, 20, 20)
+  for off in (-19, -3, 0, 5, 19):
+    diag = np.diagonal(bias[0, 1], offset=off)
+    assert (diag == diag[0]).all()
+    assert diag[0] == values[1, rp(np.array(off))]
+
+
+def test_relative_bias_gradient_against_finite_differences():
+  rng = np.random.default_rng(79)
+  b, l, heads, d, nb = 2, 10, 2, 4, 8
+  q, k, v, do = (rng.standard_normal((b, l, heads * d)) for _ in range(4))
+  values = rng.standard_normal((heads, nb))
+
+  def f(vals):
+    pos = np.arange(l)
+    bucket = B.relative_position_bucket(pos[None, :] - pos[:, None], False, nb)
+    q4, k4, v4 = (t.reshape(b, l, heads, d) for t in (q, k, v))
+    logits = np.einsum("blhd,bmhd->bhlm", q4, k4) + vals[:, bucket][None]
+    logits = logits + (pos[None, :] > pos[:, None]) * -1e9
+    w = scipy.special.softmax(logits, axis=-1)
+    out = np.einsum("bhlm,bmhd->blhd", w, v4).reshape(b, l, heads * d)
+    return (out * do).sum()
+  got = B.attention_core_backward(
+      q.astype(np.float32), k.astype(np.float32), v.astype(np.float32),
+      do.astype(np.float32), heads, True, "float32",
+      relative_values=values.astype(np.float32))[3]
+  want = np.zeros_like(values)
+  eps = 1e-5
+  for h in range(heads):
+    for j in range(nb):
+      up, dn = values.copy(), values.copy()
+      up[h, j] += eps
+      dn[h, j] -= eps
+      want[h, j] = (f(up) - f(dn)) / (2 * eps)
+  np.testing.assert_allclose(got, want, rtol=2e-3, atol=2e-4)
+
+
 def test_self_attention_bf16_close_to_float32():
   rng = np.random.default_rng(6)
   b, l, m, heads, d = 2, 16, 32, 2, 8

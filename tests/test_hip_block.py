@@ -256,6 +256,53 @@ def test_attention_decode(hip, case, act_dtype):
     np.testing.assert_array_equal(H.to_np(vg), want_v)
 
 
+@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("causal", [False, True])
+@pytest.mark.parametrize("case", [(2, 40, 2, 16, 8), (2, 200, 3, 64, 32),
+                                  (1, 328, 2, 128, 32)],
+                         ids=lambda c: "x".join(map(str, c)))
+def test_self_attention_relative_bias(hip, case, causal, act_dtype):
+  """The relative attention bias (transformer_layers.py:317-352): forward,
+  (dq, dk, dv) and the gradient of the bias values against the oracle, with and
+  without sequence ids."""
+  b, l, heads, d, nb = case
+  rng = np.random.default_rng(sum(case) + causal)
+  mk = lambda: O.cast_act(
+      (rng.standard_normal((b, l, heads * d)) * 0.5).astype(np.float32),
+      act_dtype)
+  q, k, v, do = mk(), mk(), mk(), mk()
+  values = O.cast_act(rng.standard_normal((heads, nb)).astype(np.float32),
+                      act_dtype)
+  pos = np.arange(-(l - 1), l)
+  bucket = B.relative_position_bucket(pos, not causal, nb).astype(np.int32)
+  g = lambda a: H.to_gpu(a, act_dtype)
+  rel = (g(values), torch.from_numpy(bucket).cuda())
+  for ids in (None, _packed_sequence_ids(rng, b, l, max(4, l // 3))):
+    sid = None if ids is None else torch.from_numpy(ids).cuda()
+    got = H.to_np(hip.self_attention(g(q), g(k), g(v), heads, causal,
+                                     sequence_id=sid, relative_bias=rel))
+    want = B._attention_core(q, k, v, heads, causal, act_dtype, sequence_id=ids,
+                             relative_values=values)
+    tol = _tol(act_dtype)
+    if act_dtype == "float32":
+      tol = dict(rtol=1e-4, atol=1e-4)
+    np.testing.assert_allclose(got, want, **tol)
+    got_b = hip.self_attention_backward(g(q), g(k), g(v), g(do), heads, causal,
+                                        sequence_id=sid, relative_bias=rel)
+    want_b = B.attention_core_backward(q, k, v, do, heads, causal, act_dtype,
+                                       sequence_id=ids, relative_values=values)
+    btol = dict(rtol=2e-4, atol=2e-4) if act_dtype == "float32" else dict(
+        rtol=3e-2, atol=3e-2)
+    assert len(got_b) == 4
+    for gt, wnt, name in zip(got_b, want_b, ("dq", "dk", "dv", "dvalues")):
+      scale = max(1.0, float(np.abs(wnt).max()))
+      np.testing.assert_allclose(H.to_np(gt), wnt, rtol=btol["rtol"],
+                                 atol=btol["atol"] * scale, err_msg=name)
+  # not the same as no bias
+  plain = H.to_np(hip.self_attention(g(q), g(k), g(v), heads, causal))
+  assert np.abs(plain - got).max() > 1e-2
+
+
 def test_self_attention_rejections(hip):
   q = torch.zeros((1, 12, 16), dtype=torch.bfloat16, device="cuda")
   with pytest.raises(hip.MoeHipError, match="not divisible"):
