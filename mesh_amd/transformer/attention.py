@@ -4,6 +4,9 @@ SelfAttention uses by default: heads and d_kv combined in the variables
 (combine_dims, attention.py:410-414), separate k and v, float32 logits.
 """
 
+import math
+
+import numpy as np
 import torch
 
 from mesh_amd import layers as mtf_layers
@@ -180,6 +183,32 @@ class ExpertsAttentionParams(AttentionParams):
     raise NotImplementedError("ExpertsAttention uses shared_kv = True.")
 
 
+def relative_position_bucket(relative_position, bidirectional=True,
+                             num_buckets=32, max_distance=128):
+  """_relative_position_bucket (transformer_layers.py:1000-1042) on host
+  integers: relative_position = memory position - query position -> bucket in
+  [0, num_buckets).  Half of the buckets hold exact small distances, the rest
+  grow logarithmically up to max_distance; the logarithmic part is float32
+  arithmetic in the reference's op order, truncated as its int32 cast does."""
+  rp = np.asarray(relative_position, np.int64)
+  ret = np.zeros(rp.shape, np.int64)
+  n = -rp
+  if bidirectional:
+    num_buckets //= 2
+    ret = ret + (n < 0) * num_buckets
+    n = np.abs(n)
+  else:
+    n = np.maximum(n, 0)
+  max_exact = num_buckets // 2
+  is_small = n < max_exact
+  safe = np.where(is_small, max_exact, n).astype(np.float32)
+  scaled = (np.log(safe / np.float32(max_exact)).astype(np.float32)
+            / np.float32(math.log(max_distance / max_exact))
+            ).astype(np.float32) * np.float32(num_buckets - max_exact)
+  large = np.minimum(max_exact + scaled.astype(np.int64), num_buckets - 1)
+  return ret + np.where(is_small, n, large)
+
+
 class SelfAttentionOperation(mtf.Operation):
   """attention.attention (attention.py:27-88) on combined-dim tensors
   q, k, v [batch..., length, heads * d_kv]: float32 logits, an optional
@@ -188,10 +217,20 @@ class SelfAttentionOperation(mtf.Operation):
   query to the keys of its own sequence (the bias of
   transformer_layers.py:303-316)."""
 
-  def __init__(self, q, k, v, num_heads, causal, sequence_id=None, name=None):
-    inputs = [q, k, v] + ([] if sequence_id is None else [sequence_id])
+  def __init__(self, q, k, v, num_heads, causal, sequence_id=None,
+               relative_values=None, relative_bidirectional=True, name=None):
+    inputs = [q, k, v] + ([] if sequence_id is None else [sequence_id]) + (
+        [] if relative_values is None else [relative_values])
     super(SelfAttentionOperation, self).__init__(inputs,
                                                  name=name or "attention")
+    self._ids_at = 3 if sequence_id is not None else None
+    self._rel_at = (len(inputs) - 1) if relative_values is not None else None
+    self._rel_bidirectional = bool(relative_bidirectional)
+    if relative_values is not None and (
+        relative_values.shape.ndims != 2
+        or relative_values.shape.dims[0].size != num_heads):
+      raise ValueError("relative attention bias %s, expected [heads = %d, "
+                       "buckets]" % (relative_values.shape, num_heads))
     if q.shape != k.shape or q.shape != v.shape:
       raise ValueError("q, k, v shapes differ: %s %s %s"
                        % (q.shape, k.shape, v.shape))
@@ -210,20 +249,41 @@ class SelfAttentionOperation(mtf.Operation):
     length, channels = sizes[-2], sizes[-1]
     heads, causal = self._num_heads, self._causal
 
-    def fn(q, k, v, ids=None):
+    ids_at, rel_at = self._ids_at, self._rel_at
+    bidirectional = self._rel_bidirectional
+
+    def fn(q, k, v, *extra):
       q3, k3, v3 = (t.reshape(-1, length, channels).contiguous()
                     for t in (q, k, v))
-      if ids is not None:
-        ids = ids.reshape(-1, length).to(torch.int32).contiguous()
-      return moe_hip.self_attention(q3, k3, v3, heads, causal,
-                                    sequence_id=ids).reshape(sizes)
+      ids, rel = _attention_extras(extra, ids_at, rel_at, length, bidirectional,
+                                   q.dtype)
+      return moe_hip.self_attention(q3, k3, v3, heads, causal, sequence_id=ids,
+                                    relative_bias=rel).reshape(sizes)
     lowering.set_tensor_lowering(
         self.outputs[0],
         mesh_impl.slicewise(fn, *[lowering.tensors[t] for t in self.inputs]))
 
   def gradient(self, grad_ys):
     grads = list(SelfAttentionGradOperation(self, grad_ys[0]).outputs)
-    return grads + [None] * (len(self.inputs) - 3)
+    out = grads[:3] + [None] * (len(self.inputs) - 3)
+    if self._rel_at is not None:
+      out[self._rel_at] = grads[3]
+    return out
+
+
+def _attention_extras(extra, ids_at, rel_at, length, bidirectional, dtype):
+  """The optional inputs of the attention operations as the library takes
+  them: sequence ids [B, L] int32, and (bias values [H, NB] in the activation
+  dtype, the bucket of every memory position - query position [2L-1])."""
+  ids = rel = None
+  if ids_at is not None:
+    ids = extra[ids_at - 3].reshape(-1, length).to(torch.int32).contiguous()
+  if rel_at is not None:
+    values = extra[rel_at - 3].to(dtype).contiguous()
+    bucket = relative_position_bucket(
+        np.arange(-(length - 1), length), bidirectional, values.shape[-1])
+    rel = (values, torch.from_numpy(bucket.astype(np.int32)).to(values.device))
+  return ids, rel
 
 
 class AttentionDecodeOperation(mtf.Operation):
@@ -282,10 +342,14 @@ class SelfAttentionGradOperation(mtf.Operation):
     super(SelfAttentionGradOperation, self).__init__(
         [dout, q, k, v] + list(forward.inputs[3:]),
         name=name or "attention_grad")
-    self._num_heads = forward._num_heads   # pylint: disable=protected-access
-    self._causal = forward._causal         # pylint: disable=protected-access
+    # pylint: disable=protected-access
+    self._num_heads, self._causal = forward._num_heads, forward._causal
+    self._ids_at, self._rel_at = forward._ids_at, forward._rel_at
+    self._rel_bidirectional = forward._rel_bidirectional
+    wrt = [q, k, v] + ([] if self._rel_at is None
+                       else [forward.inputs[self._rel_at]])
     self._outputs = [mtf.Tensor(self, t.shape, t.dtype, index=i)
-                     for i, t in enumerate((q, k, v))]
+                     for i, t in enumerate(wrt)]
 
   def lower(self, lowering):
     from mesh_amd import moe_hip
@@ -294,13 +358,17 @@ class SelfAttentionGradOperation(mtf.Operation):
     length, channels = sizes[-2], sizes[-1]
     heads, causal = self._num_heads, self._causal
 
-    def fn(dout, q, k, v, ids=None):
+    ids_at, rel_at = self._ids_at, self._rel_at
+    bidirectional = self._rel_bidirectional
+
+    def fn(dout, q, k, v, *extra):
       d3, q3, k3, v3 = (t.reshape(-1, length, channels).contiguous()
                         for t in (dout, q, k, v))
-      if ids is not None:
-        ids = ids.reshape(-1, length).to(torch.int32).contiguous()
-      return tuple(t.reshape(sizes) for t in moe_hip.self_attention_backward(
-          q3, k3, v3, d3, heads, causal, sequence_id=ids))
+      ids, rel = _attention_extras(extra, ids_at, rel_at, length, bidirectional,
+                                   q.dtype)
+      grads = moe_hip.self_attention_backward(
+          q3, k3, v3, d3, heads, causal, sequence_id=ids, relative_bias=rel)
+      return tuple(t.reshape(sizes) for t in grads[:3]) + tuple(grads[3:])
     grads = mesh_impl.slicewise(
         fn, *[lowering.tensors[t] for t in self.inputs])
     for out, value in zip(self.outputs, grads):

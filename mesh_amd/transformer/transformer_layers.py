@@ -40,10 +40,10 @@ class DenseReluDense(transformer.TransformerLayer):
 
 
 class SelfAttention(transformer.TransformerLayer):
-  """Multi-head self-attention (transformer_layers.py:151-357) with the default
-  parameters: no relative position bias, separate k and v, combined dims.
-  Visibility comes from the context: read/write priorities (autoregressive
-  models) or none."""
+  """Multi-head self-attention (transformer_layers.py:151-357): separate k and
+  v, combined dims, optionally the relative position bias of types "bias" and
+  "bias_shared".  Visibility comes from the context: read/write priorities
+  (autoregressive models), sequence ids, or none."""
 
   _shared_kv_implemented = False     # a "kv" kernel of its own is not
 
@@ -53,12 +53,17 @@ class SelfAttention(transformer.TransformerLayer):
                relative_attention_num_buckets=32, attention_func=None,
                combine_dims=True, keep_query_heads_dims=False,
                fold_scaling_into_initializer=True):
-    if (num_memory_heads or attention_kwargs or
-        relative_attention_type is not None or attention_func is not None or
+    if (num_memory_heads or attention_kwargs or attention_func is not None or
         not combine_dims or keep_query_heads_dims or
         (shared_kv and not self._shared_kv_implemented)):
       raise NotImplementedError(
           "only the default SelfAttention options are implemented")
+    if relative_attention_type == "contextual":
+      raise NotImplementedError("contextual relative attention")
+    if relative_attention_type not in (None, "bias", "bias_shared"):
+      raise ValueError("unrecognized relative_attention_type \"%s\""
+                       % relative_attention_type)
+    self.relative_attention_type = relative_attention_type
     self.num_heads = num_heads
     self.shared_kv = shared_kv
     self.combine_dims = combine_dims
@@ -83,6 +88,26 @@ class SelfAttention(transformer.TransformerLayer):
         memory_heads_dims=heads, variable_dtype=context.variable_dtype,
         shared_kv=self.shared_kv, ensemble_dim=context.model.ensemble_dim,
         fold_scaling_into_initializer=self.fold_scaling_into_initializer)
+
+  def relative_bias_values(self, context, num_heads):
+    """The learned bias per (head, bucket of memory position - query position)
+    (compute_bias, transformer_layers.py:317-352): the variable
+    "relative_attention_bias" [heads, buckets]; with "bias_shared" the first
+    layer's variable serves every layer of the stack (context.cache)."""
+    if self.relative_attention_type is None:
+      return None
+    heads = mtf.Dimension("heads", num_heads)
+    buckets = mtf.Dimension("buckets", self.relative_attention_num_buckets)
+    shared = self.relative_attention_type == "bias_shared"
+    key = ("self_attention_bias", None, None, (heads,))
+    if shared and key in context.cache:
+      return context.cache[key]
+    values = mtf.get_variable(context.mesh, "relative_attention_bias",
+                              mtf.Shape([heads, buckets]),
+                              dtype=context.variable_dtype)
+    if shared:
+      context.cache[key] = values
+    return values
 
   def _attention_dropout(self, context, v, num_heads):
     """Dropout of the attention weights with one noise value per (batch entry,
@@ -113,6 +138,10 @@ class SelfAttention(transformer.TransformerLayer):
     else:
       k = params.compute_k(x)
       v = params.compute_v(x)
+    relative_values = self.relative_bias_values(context, params.num_heads)
+    if relative_values is not None and context.mode in (
+        transformer.INCREMENTAL, transformer.FIRST_PART):
+      raise NotImplementedError("decoding with a relative attention bias")
     if context.mode == transformer.INCREMENTAL:
       # one position per batch entry: the step's key and value replace row
       # `position` of the recurrent states, the query sees the memory
@@ -140,8 +169,13 @@ class SelfAttention(transformer.TransformerLayer):
     causal = context.read_priority is transformer.POSITION
     if context.train and self.dropout_rate != 0.0:
       v = self._attention_dropout(context, v, params.num_heads)
-    o = attention.SelfAttentionOperation(q, k, v, params.num_heads, causal,
-                                         sequence_id=sequence_id).outputs[0]
+    o = attention.SelfAttentionOperation(
+        q, k, v, params.num_heads, causal, sequence_id=sequence_id,
+        relative_values=relative_values,
+        # buckets of a bidirectional layout unless the model is autoregressive
+        # (transformer_layers.py:321)
+        relative_bidirectional=not context.model.fully_autoregressive
+        ).outputs[0]
     return params.compute_output(o, output_shape=x.shape)
 
 

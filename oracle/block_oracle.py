@@ -279,7 +279,9 @@ def layer_stack(x, layers, final_scale, act_dtype="float32",
 
   layers: list of dicts with "kind" in {"attention", "dense_relu_dense",
   "moe"}, "scale" (the layer's rms_norm scale) and the layer's weights:
-    attention: wq, wk, wv, wo, num_heads
+    attention: wq, wk, wv, wo, num_heads; optional relative_values
+      [heads, buckets], the layer's relative attention bias (the same array in
+      every layer for relative_attention_type "bias_shared")
     dense_relu_dense: wi, wo
     moe: w_gate, wi, wo, hparams (an O.HParams); optional num_microbatches
     moe2d: w_outer, w_inner, wi, wo, hparams; optional num_microbatches
@@ -305,7 +307,8 @@ def layer_stack(x, layers, final_scale, act_dtype="float32",
     if kind == "attention":
       y = self_attention(h, layer["wq"], layer["wk"], layer["wv"], layer["wo"],
                          layer["num_heads"], autoregressive, act_dtype,
-                         layer.get("weights_noise"), sequence_id)
+                         layer.get("weights_noise"), sequence_id,
+                         layer.get("relative_values"))
     elif kind == "dense_relu_dense":
       y = dense_relu_dense(h, layer["wi"], layer["wo"], act_dtype,
                            layer.get("hidden_noise"))

@@ -7,6 +7,8 @@ import inspect
 import os
 import re
 
+import numpy as np
+
 import pytest
 import torch
 
@@ -464,6 +466,48 @@ def test_layer_stack_graph_names_and_shapes():
       "decoder/rms_norm/scale": "Shape[d_model=32]"}
 
 
+@pytest.mark.parametrize("kind", ["bias", "bias_shared"])
+def test_relative_attention_bias_variables(kind):
+  """compute_bias (transformer_layers.py:317-352): a variable
+  "relative_attention_bias" [heads, buckets] per attention layer, or only in
+  the first one with "bias_shared"."""
+  from mesh_amd.transformer import transformer, transformer_layers
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  dims = [mtf.Dimension("batch", 2), mtf.Dimension("length", 16),
+          mtf.Dimension("d_model", 32)]
+  x = mtf.import_tf_tensor(mesh, torch.zeros(2, 16, 32), mtf.Shape(dims))
+  kw = dict(num_heads=4, key_value_size=8, relative_attention_type=kind,
+            relative_attention_num_buckets=16)
+  stack = transformer.make_layer_stack(
+      [(transformer_layers.SelfAttention, kw)], num_layers=2, block_scope=False)
+  model = transformer.Unitransformer(stack, d_model=32, name="encoder",
+                                     autoregressive=False)
+  model.call_layers(x, mtf.VariableDType(torch.float32))
+  got = {v.name: v.shape.to_string for v in graph.all_variables
+         if "relative" in v.name}
+  want = {"encoder/layer_000/SelfAttention/relative_attention_bias":
+              "Shape[heads=4, buckets=16]"}
+  if kind == "bias":
+    want["encoder/layer_001/SelfAttention/relative_attention_bias"] = (
+        "Shape[heads=4, buckets=16]")
+  assert got == want
+
+
+def test_relative_position_bucket_matches_the_oracle():
+  """The host-side bucket table of the product against the oracle's
+  restatement of _relative_position_bucket (transformer_layers.py:1000-1042),
+  which the CPU tests pin by hand."""
+  from mesh_amd.transformer import attention
+  from oracle import block_oracle
+  rp = np.arange(-3000, 3000)
+  for bidirectional in (True, False):
+    for nb in (8, 32, 64):
+      np.testing.assert_array_equal(
+          attention.relative_position_bucket(rp, bidirectional, nb),
+          block_oracle.relative_position_bucket(rp, bidirectional, nb))
+
+
 def test_layer_stack_names_with_block_scope_and_legacy_mode():
   from mesh_amd.transformer import transformer, transformer_layers
   stack = transformer.make_layer_stack(
@@ -492,7 +536,9 @@ def test_layer_stack_names_with_block_scope_and_legacy_mode():
 def test_block_rejections():
   from mesh_amd.transformer import transformer, transformer_layers
   with pytest.raises(NotImplementedError):
-    transformer_layers.SelfAttention(relative_attention_type="bias")
+    transformer_layers.SelfAttention(relative_attention_type="contextual")
+  with pytest.raises(ValueError, match="unrecognized"):
+    transformer_layers.SelfAttention(relative_attention_type="nope")
   with pytest.raises(NotImplementedError):
     transformer_layers.SelfAttention(shared_kv=True)
   graph = mtf.Graph()

@@ -426,6 +426,89 @@ def test_layer_stack_packed_sequences(autoregressive):
   assert not got[0, -5:].any() and not grads[0][0, -5:].any()
 
 
+@pytest.mark.parametrize("autoregressive", [True, False])
+@pytest.mark.parametrize("kind", ["bias", "bias_shared"])
+def test_layer_stack_relative_attention_bias(kind, autoregressive):
+  """SelfAttention(relative_attention_type="bias" / "bias_shared") in a stack
+  (transformer_layers.py:317-352): "bias" gives every attention layer its own
+  variable "relative_attention_bias" [heads, buckets]; "bias_shared" creates
+  it in the first one and reuses it.  Output against the oracle; the gradient
+  of the variables against the oracle's backward passes chained by hand
+  (shared: the two layers' contributions add up)."""
+  b, l, m, heads, d, nb = 2, 48, 64, 4, 16, 32
+  rng = np.random.default_rng(71)
+  layers, final = _build_stack(rng, m, 4, 96, heads, d, 32)
+  a0, a1 = layers[0], layers[2]
+  a0["relative_values"] = rng.standard_normal((heads, nb)).astype(np.float32)
+  a1["relative_values"] = (a0["relative_values"] if kind == "bias_shared" else
+                           rng.standard_normal((heads, nb)).astype(np.float32))
+  x = rng.standard_normal((b, l, m)).astype(np.float32)
+  dy = rng.standard_normal((b, l, m)).astype(np.float32)
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  dims = [mtf.Dimension("batch", b), mtf.Dimension("length", l),
+          mtf.Dimension("d_model", m)]
+  xt = mtf.import_tf_tensor(mesh, torch.from_numpy(x), mtf.Shape(dims))
+  dyt = mtf.import_tf_tensor(mesh, torch.from_numpy(dy), mtf.Shape(dims))
+  att_kw = dict(num_heads=heads, key_value_size=d, relative_attention_type=kind,
+                relative_attention_num_buckets=nb)
+  stack = transformer.make_layer_stack(
+      [(transformer_layers.SelfAttention, att_kw),
+       (transformer_layers.SelfAttention, att_kw)],
+      num_layers=1, block_scope=False)
+  model = transformer.Unitransformer(stack, d_model=m, name="decoder",
+                                     autoregressive=autoregressive)
+  y, _ = model.call_layers(xt, mtf.VariableDType(torch.float32), mode="eval")
+  init = {"decoder/rms_norm/scale": final}
+  for i, att in enumerate((a0, a1)):
+    p = "decoder/layer_%03d/" % i
+    init[p + "rms_norm/scale"] = att["scale"]
+    for c in "qkvo":
+      init[p + "SelfAttention/" + c] = att["w" + c]
+    if i == 0 or kind == "bias":
+      init[p + "SelfAttention/relative_attention_bias"] = att["relative_values"]
+  variables = {v.name: v for v in graph.all_variables}
+  assert sorted(variables) == sorted(init)
+  rel_names = sorted(n for n in init if n.endswith("relative_attention_bias"))
+  grads = mtf.gradients([y], [variables[n].outputs[0] for n in rel_names], [dyt])
+  lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()}, initial_values=init)
+  got = H.to_np(lowering.export_to_tf_tensor(y))
+  want, _ = B.layer_stack(x, [a0, a1], final, "float32", autoregressive)
+  np.testing.assert_allclose(got, want, rtol=2e-4, atol=2e-4)
+  plain, _ = B.layer_stack(
+      x, [{k: v for k, v in a.items() if k != "relative_values"}
+          for a in (a0, a1)], final, "float32", autoregressive)
+  assert np.abs(plain - want).max() > 1e-2
+  # backward by hand: final norm <- layer 1 <- layer 0, keeping each
+  # attention's gradient of its bias values
+  xs, cores = [x], []
+  for att in (a0, a1):
+    h = B.rms_norm(xs[-1], att["scale"])
+    q, k, v = (B.dense(h, att["w" + c]) for c in "qkv")
+    o = B._attention_core(q, k, v, heads, autoregressive, "float32",
+                          relative_values=att["relative_values"])
+    cores.append((q, k, v, o))
+    xs.append(xs[-1] + B.dense(o, att["wo"]))
+  dx, _ = B.rms_norm_backward(xs[2], final, dy)
+  dvalues = []
+  for att, (q, k, v, o), x_in in reversed(list(zip((a0, a1), cores, xs[:2]))):
+    do, _ = B.dense_backward(o, att["wo"], dx)
+    dq, dk, dv, dval = B.attention_core_backward(
+        q, k, v, do, heads, autoregressive,
+        relative_values=att["relative_values"])
+    dvalues.insert(0, dval)
+    h = B.rms_norm(x_in, att["scale"])
+    dh = sum(B.dense_backward(h, att["w" + c], g)[0]
+             for c, g in zip("qkv", (dq, dk, dv)))
+    dx = dx + B.rms_norm_backward(x_in, att["scale"], dh)[0]
+  want_grads = [dvalues[0] + dvalues[1]] if kind == "bias_shared" else dvalues
+  assert len(grads) == len(want_grads)
+  for g, w in zip(grads, want_grads):
+    g = H.to_np(lowering.export_to_tf_tensor(g))
+    assert np.abs(w).max() > 1e-2
+    np.testing.assert_allclose(g, w, rtol=1e-3, atol=1e-3 * np.abs(w).max())
+
+
 @pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
 def test_decoding_modes_match_the_full_forward(act_dtype):
   """Decoding as Unitransformer.sample_autoregressive drives it
