@@ -414,7 +414,8 @@ def test_router_top2_gating_rejects_unsupported(hip):
 # ---- switch (top-1) gating ------------------------------------------------------
 @pytest.mark.parametrize("shape", [(2, 1024, 8, 160), (16, 2048, 64, 32),
                                    (3, 77, 5, 7), (1, 1, 2, 1),
-                                   (2, 130, 200, 4), (1, 4096, 64, 70)])
+                                   (2, 130, 200, 4), (1, 4096, 64, 70),
+                                   (32, 2048, 64, 64)])
 def test_switch_gating_random_logits(hip, shape):
   g, s, e, c = shape
   rng = np.random.default_rng(1000 + hash(shape) % 1000)
@@ -567,7 +568,8 @@ def _assert_switch_max_equal(got, want):
 @pytest.mark.parametrize("shape", [(2, 1024, 8, 100, 2), (8, 2048, 64, 30, 4),
                                    (3, 77, 5, 12, 3), (1, 1, 2, 1, 1),
                                    (2, 131, 200, 1, 4), (1, 4096, 64, 60, 8),
-                                   (2, 512, 16, 512, 4), (4, 300, 6, 40, 6)])
+                                   (2, 512, 16, 512, 4), (4, 300, 6, 40, 6),
+                                   (32, 2048, 64, 64, 4)])
 def test_ntlb_gating_random_logits(hip, shape):
   """Skewed router (a Zipf bias) so that the popular experts overflow in pass
   0 and the later passes route what is left."""
@@ -635,7 +637,8 @@ def test_ntlb_gating_rejections(hip):
 
 @pytest.mark.parametrize("shape", [(2, 1024, 8, 160), (16, 2048, 64, 32),
                                    (3, 77, 5, 7), (1, 1, 2, 1),
-                                   (2, 131, 200, 4), (1, 4096, 64, 40)])
+                                   (2, 131, 200, 4), (1, 4096, 64, 40),
+                                   (32, 2048, 64, 64)])
 def test_switch_max_gating(hip, shape):
   """Slots by descending gate.  The oracle ranks NumPy's softmax values and the
   kernel its own: the generator keeps the top logits apart, and gates of
@@ -762,7 +765,8 @@ def _column_gaps_ok(logits, imp, min_gap=1e-4):
 
 
 @pytest.mark.parametrize("shape", [(2, 64, 4, 8), (3, 77, 5, 20), (2, 1024, 8, 256),
-                                   (16, 2048, 64, 32), (1, 300, 130, 7)])
+                                   (16, 2048, 64, 32), (1, 300, 130, 7),
+                                   (32, 2048, 64, 64)])
 def test_expert_choice_gating(hip, shape):
   g, s, e, c = shape
   rng = np.random.default_rng(3000 + hash(shape) % 1000)
