@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 22
+#define MESH_MOE_ABI_VERSION 23
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -746,10 +746,10 @@ size_t mesh_moe_self_attention_workspace_bytes(int B, int L, int H, int D,
  * the relative attention bias of transformer_layers.py:317-352 -- logit (i, j)
  * gets rel_values[h][rel_bucket[j - i + L - 1]], rel_bucket being the bucket of
  * every (memory position - query position) (the caller evaluates
- * _relative_position_bucket, :1000-1042, once per length).  With a bias the
- * three-step form runs whatever the shape (pass relative_bias = 1 to
- * mesh_moe_self_attention_workspace_bytes); mesh_moe_attention_weights takes
- * the same arguments.
+ * _relative_position_bucket, :1000-1042, once per length).  Pass
+ * relative_bias = 1 to mesh_moe_self_attention_workspace_bytes; the fused
+ * kernel reads the bias from a float32 table [H, 2L-1] it first builds in the
+ * workspace.  mesh_moe_attention_weights takes the same arguments.
  */
 int mesh_moe_self_attention(const void* q, const void* k, const void* v,
                             void* out, int B, int L, int H, int D, int causal,
@@ -775,7 +775,8 @@ int mesh_moe_relative_bias_backward(const void* dlogits,
 /* Bytes of scratch mesh_moe_self_attention_backward needs; 0 for shapes it does
  * not take. */
 size_t mesh_moe_self_attention_backward_workspace_bytes(int B, int L, int H,
-                                                        int D, int dtype);
+                                                        int D, int dtype,
+                                                        int relative_bias);
 
 /*
  * Backward of mesh_moe_self_attention in fused kernels: what mtf.gradients
@@ -795,12 +796,21 @@ size_t mesh_moe_self_attention_backward_workspace_bytes(int B, int L, int H,
  * atomics; the same bits on every run).  dW is not rounded to dtype before
  * the subtraction and delta comes from sum_d dout out in float32 -- fewer
  * roundings than the reference's chain of ops, inside its tolerance.
+ * rel_values, rel_bucket, num_buckets as for mesh_moe_self_attention, with
+ * dvalues [H,num_buckets] dtype (all NULL / 0: no bias): W is recomputed with
+ * the bias and dvalues receives the gradient of rel_values (the gradient of
+ * the mtf.gather at transformer_layers.py:351): the dq kernel sums its dS
+ * (float32, before the cast) along the diagonals into a float32 table
+ * [H, 2L-1] with atomics -- the order of that sum is not fixed -- and a last
+ * small kernel adds up each bucket's distances.
  */
 int mesh_moe_self_attention_backward(const void* q, const void* k, const void* v,
                                      const void* dout, void* dq, void* dk,
                                      void* dv, int B, int L, int H, int D,
                                      int causal, const int32_t* sequence_id,
-                                     int dtype, void* workspace,
+                                     const void* rel_values,
+                                     const int32_t* rel_bucket, int num_buckets,
+                                     void* dvalues, int dtype, void* workspace,
                                      size_t workspace_bytes, void* stream);
 
 /*

@@ -108,12 +108,18 @@ __device__ __forceinline__ float fa_exp2(float x) {
 // SEQ: a query sees only the keys that carry its sequence id (seq [B, L];
 // transformer_layers.py:303-316): the ids of a key tile travel through LDS
 // with the tile, a lane keeps its query's id in a register.
-template <int D, bool CAUSAL, bool STATS = false, bool SEQ = false>
+// BIAS: the relative attention bias (transformer_layers.py:317-352) is added to
+// the float32 logits: tab [H, 2L-1] holds, per head, the bias of every distance
+// key - query + L - 1.  A tile's logits need a window of BK + BQ - 1 entries of
+// it, which travels through LDS with the tile.
+template <int D, bool CAUSAL, bool STATS = false, bool SEQ = false,
+          bool BIAS = false>
 __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
     const bf16_t* __restrict__ v, bf16_t* __restrict__ out, int L, int H,
     const bf16_t* __restrict__ dout, float* __restrict__ lse,
-    float* __restrict__ delta, const int32_t* __restrict__ seq) {
+    float* __restrict__ delta, const int32_t* __restrict__ seq,
+    const float* __restrict__ tab) {
   using Cfg = FlashCfg<D>;
   extern __shared__ __attribute__((aligned(16))) unsigned char fa_smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -143,8 +149,11 @@ __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
     own_first = __builtin_amdgcn_readfirstlane(my_sid);
     own_uniform = __ballot(my_sid != own_first) == 0ull;
   }
-  // key ids of the two tile stages, behind the K / V ring
+  // key ids of the two tile stages, behind the K / V ring; then the two
+  // stages' windows of the bias table (192 floats each)
   int32_t* sid_s = reinterpret_cast<int32_t*>(fa_smem + Cfg::LDS_BYTES);
+  const float* bias_s = reinterpret_cast<const float*>(fa_smem + Cfg::LDS_BYTES + 512);
+  const float* tab_h = BIAS ? tab + (int64_t)h * (2 * L - 1) : nullptr;
   fa_bf16x8_t qf[Cfg::DS];
   {
     const bf16_t* qr = qb + (int64_t)min(my_q, L - 1) * row_stride + half * 8;
@@ -185,6 +194,18 @@ __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
         __builtin_amdgcn_global_load_lds(
             (fa_glb_void_t*)(seq_b + min(key0 + lane, L - 1)),
             (fa_lds_void_t*)(fa_smem + Cfg::LDS_BYTES + buf * 256), 4, 0, 0);
+    }
+    if constexpr (BIAS) {
+      // entry i of the window: distance key0 - (q0 + BQ - 1) + i (+ L - 1)
+      if (wave >= 1) {
+        const int i = (wave - 1) * 64 + lane;
+        const int d = key0 - (q0 + Cfg::BQ - 1) + (L - 1) + i;
+        __builtin_amdgcn_global_load_lds(
+            (fa_glb_void_t*)(tab_h + min(max(d, 0), 2 * L - 2)),
+            (fa_lds_void_t*)(fa_smem + Cfg::LDS_BYTES + 512 + buf * 768 +
+                             (wave - 1) * 256),
+            4, 0, 0);
+      }
     }
   };
 
@@ -238,6 +259,17 @@ __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
           acc_s[sub] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(
               kf, qf[s], acc_s[sub], 0, 0, 0);
         }
+      }
+      if constexpr (BIAS) {
+        // key key0 + kl + c against query q0 + 32 wave + l32
+        const float* bw = bias_s + buf * 192 + (Cfg::BQ - 1 - wave * 32 - l32);
+#pragma unroll
+        for (int sub = 0; sub < 2; ++sub)
+#pragma unroll
+          for (int r4 = 0; r4 < 4; ++r4)
+#pragma unroll
+            for (int c = 0; c < 4; ++c)
+              acc_s[sub][4 * r4 + c] += bw[sub * 32 + 8 * r4 + 4 * half + c];
       }
       // mask and row maximum
       if (need_mask) {
@@ -401,30 +433,70 @@ __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
   }
 }
 
-template <int D, bool CAUSAL, bool SEQ>
+template <int D, bool CAUSAL, bool SEQ, bool BIAS>
 static int launch_flash_one(const bf16_t* q, const bf16_t* k, const bf16_t* v,
                             bf16_t* out, int B, int L, int H,
-                            const int32_t* seq, hipStream_t st) {
+                            const int32_t* seq, const float* tab,
+                            hipStream_t st) {
   using Cfg = FlashCfg<D>;
-  constexpr int LDS = Cfg::LDS_BYTES + 512;        // + key ids of two stages
+  constexpr int LDS = Cfg::LDS_BYTES + 512 + 1536;  // + key ids, bias windows
   dim3 grid((unsigned)((L + Cfg::BQ - 1) / Cfg::BQ), (unsigned)(B * H));
-  auto kern = flash_attention_kernel<D, CAUSAL, false, SEQ>;
+  auto kern = flash_attention_kernel<D, CAUSAL, false, SEQ, BIAS>;
   MOE_ALLOW_LDS(kern, LDS);
   kern<<<grid, Cfg::THREADS, LDS, st>>>(q, k, v, out, L, H, nullptr, nullptr,
-                                        nullptr, seq);
+                                        nullptr, seq, tab);
   MOE_CHECK_LAUNCH("self_attention (fused)");
   return 0;
+}
+
+// Calls f(std::bool_constant<causal>, <seq>, <bias>) for run-time flags.
+template <typename F>
+static int flash_dispatch(bool causal, bool seq, bool bias, F&& f) {
+  auto with_bias = [&](auto c, auto s) {
+    return bias ? f(c, s, std::true_type()) : f(c, s, std::false_type());
+  };
+  auto with_seq = [&](auto c) {
+    return seq ? with_bias(c, std::true_type()) : with_bias(c, std::false_type());
+  };
+  return causal ? with_seq(std::true_type()) : with_seq(std::false_type());
 }
 
 template <int D>
 static int launch_flash(const bf16_t* q, const bf16_t* k, const bf16_t* v,
                         bf16_t* out, int B, int L, int H, int causal,
-                        const int32_t* seq, hipStream_t st) {
-  if (causal)
-    return seq ? launch_flash_one<D, true, true>(q, k, v, out, B, L, H, seq, st)
-               : launch_flash_one<D, true, false>(q, k, v, out, B, L, H, seq, st);
-  return seq ? launch_flash_one<D, false, true>(q, k, v, out, B, L, H, seq, st)
-             : launch_flash_one<D, false, false>(q, k, v, out, B, L, H, seq, st);
+                        const int32_t* seq, const float* tab, hipStream_t st) {
+  return flash_dispatch(causal != 0, seq != nullptr, tab != nullptr,
+                        [&](auto c, auto s, auto bi) {
+    return launch_flash_one<D, decltype(c)::value, decltype(s)::value,
+                            decltype(bi)::value>(q, k, v, out, B, L, H, seq, tab,
+                                                 st);
+  });
+}
+
+// tab[h][d] = float(values[h][bucket[d]]) for the 2L-1 distances d = key -
+// query + L - 1: the bias as mtf.gather of the activation-dtype values gives it
+// (transformer_layers.py:343-350), widened to the logits' float32.
+__global__ void relative_table_kernel(const bf16_t* __restrict__ values,
+                                      const int32_t* __restrict__ bucket,
+                                      float* __restrict__ tab, int n, int NB) {
+  const int d = blockIdx.x * blockDim.x + threadIdx.x;
+  if (d < n)
+    tab[(int64_t)blockIdx.y * n + d] =
+        load_f32<bf16_t>(values + (int64_t)blockIdx.y * NB + bucket[d]);
+}
+
+static int launch_relative_table(const void* values, const int32_t* bucket,
+                                 float* tab, int L, int H, int NB,
+                                 hipStream_t st) {
+  const int n = 2 * L - 1;
+  relative_table_kernel<<<dim3((unsigned)((n + 255) / 256), (unsigned)H), 256, 0,
+                          st>>>((const bf16_t*)values, bucket, tab, n, NB);
+  MOE_CHECK_LAUNCH("self_attention (bias table)");
+  return 0;
+}
+
+static size_t relative_table_bytes(int L, int H) {
+  return ((size_t)H * (2 * (size_t)L - 1) * sizeof(float) + 255) & ~(size_t)255;
 }
 
 bool flash_attention_supported(int L, int H, int D, int dtype, const void* q,
@@ -435,22 +507,31 @@ bool flash_attention_supported(int L, int H, int D, int dtype, const void* q,
           0) && (int64_t)L * H * D < (1LL << 31);
 }
 
-size_t flash_attention_workspace_bytes(int B, int L, int H, int D) {
-  (void)B; (void)L; (void)H; (void)D;
-  return 256;     // the fused kernel needs no scratch
+size_t flash_attention_workspace_bytes(int B, int L, int H, int D,
+                                       bool relative_bias) {
+  (void)B; (void)D;
+  // the bias table is the only scratch
+  return 256 + (relative_bias ? relative_table_bytes(L, H) : 0);
 }
 
 int flash_attention(const void* q, const void* k, const void* v, void* out,
                     int B, int L, int H, int D, int causal,
-                    const int32_t* sequence_id, void* workspace,
+                    const int32_t* sequence_id, const void* rel_values,
+                    const int32_t* rel_bucket, int num_buckets, void* workspace,
                     hipStream_t st) {
-  (void)workspace;
+  float* tab = nullptr;
+  if (rel_values != nullptr) {
+    tab = (float*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
+    const int rc = launch_relative_table(rel_values, rel_bucket, tab, L, H,
+                                         num_buckets, st);
+    if (rc != 0) return rc;
+  }
   if (D == 128)
     return launch_flash<128>((const bf16_t*)q, (const bf16_t*)k,
                              (const bf16_t*)v, (bf16_t*)out, B, L, H, causal,
-                             sequence_id, st);
+                             sequence_id, tab, st);
   return launch_flash<64>((const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v,
-                          (bf16_t*)out, B, L, H, causal, sequence_id, st);
+                          (bf16_t*)out, B, L, H, causal, sequence_id, tab, st);
 }
 
 // ---------------------------------------------------------------------------
@@ -485,20 +566,29 @@ struct FlashBwdCfg {
   static constexpr int CH = ROW / 16, UNITS = ROW / 64, RPI = 1024 / ROW;
   static constexpr int INSTR = TILE / 1024 / WAVES; // loads per wave and tile copy
   static constexpr int DS = D / 16, DT = D / 32;
-  static constexpr int STATS_BYTES = 3 * BT * 4;    // lse, delta, sequence ids of a tile
+  // lse, delta, sequence ids of a tile, then its window of the bias table
+  // (BT + BOWN - 1 distances, 320 floats)
+  static constexpr int BIAS_AT = 3 * BT * 4;
+  static constexpr int STATS_BYTES = BIAS_AT + 320 * 4;
+  static constexpr int RING = 512;                  // floats, see dwin below
   static constexpr int stage_bytes(int what) {
     return (what == BWD_DV ? 2 : 3) * TILE + STATS_BYTES;
   }
+  static_assert(BT + BOWN - 1 <= 320 && 320 + 3 * BT <= RING, "bias window");
   static_assert(D == 64 || D == 128, "d_kv 64 or 128");
   static_assert(INSTR >= 1, "a tile copy is at least one load per wavefront");
 };
 
-template <int D, bool CAUSAL, int WHAT, bool SEQ>
+// BIAS: the logits are recomputed with the relative attention bias (tab as
+// in the forward kernel); BWD_DQ also sums its dS along the diagonals into
+// dtab [H, 2L-1] (float atomics), the gradient of tab.
+template <int D, bool CAUSAL, int WHAT, bool SEQ, bool BIAS>
 __global__ __launch_bounds__(512) void flash_attention_backward_kernel(
     const bf16_t* __restrict__ q, const bf16_t* __restrict__ k,
     const bf16_t* __restrict__ v, const bf16_t* __restrict__ dout,
     const float* __restrict__ lse, const float* __restrict__ delta,
-    bf16_t* __restrict__ grad, int L, int H, const int32_t* __restrict__ seq) {
+    bf16_t* __restrict__ grad, int L, int H, const int32_t* __restrict__ seq,
+    const float* __restrict__ tab, float* __restrict__ dtab) {
   using Cfg = FlashBwdCfg<D>;
   constexpr bool OWN_Q = WHAT == BWD_DQ;
   constexpr int NCOPY = WHAT == BWD_DV ? 2 : 3;
@@ -521,6 +611,7 @@ __global__ __launch_bounds__(512) void flash_attention_backward_kernel(
   const bf16_t* str2 = (OWN_Q ? v : dout) + head_off;
   const float* lse_b = lse + (int64_t)bh * L;
   const float* delta_b = delta + (int64_t)bh * L;
+  const float* tab_h = BIAS ? tab + (int64_t)h * (2 * L - 1) : nullptr;
 
   const int nt_all = (L + Cfg::BT - 1) / Cfg::BT;
   int t_begin = 0, t_end = nt_all;
@@ -598,7 +689,51 @@ __global__ __launch_bounds__(512) void flash_attention_backward_kernel(
             (fa_glb_void_t*)(seq_b + min(row0 + lane, L - 1)),
             (fa_lds_void_t*)(base + NCOPY * Cfg::TILE + 512), 4, 0, 0);
     }
+    if constexpr (BIAS) {
+      // entry i of the window: the smallest distance key - query (+ L - 1)
+      // between the tile and the block's own rows, plus i
+      if (wave >= 3) {
+        const int i = (wave - 3) * 64 + lane;
+        const int d = (OWN_Q ? row0 - (own0 + Cfg::BOWN - 1)
+                             : own0 - (row0 + Cfg::BT - 1)) + (L - 1) + i;
+        __builtin_amdgcn_global_load_lds(
+            (fa_glb_void_t*)(tab_h + min(max(d, 0), 2 * L - 2)),
+            (fa_lds_void_t*)(base + NCOPY * Cfg::TILE + Cfg::BIAS_AT +
+                             (wave - 3) * 256),
+            4, 0, 0);
+      }
+    }
   };
+  // BWD_DQ with BIAS: dS summed along the diagonals.  Within a wavefront the
+  // 32 queries x 64 keys of a tile span the distances e = key - query in
+  // [-31, 63].  Each value is rotated (ds_bpermute, inside its half-wave) to
+  // lane m = (query - key) mod 32, which then only ever sees e = -m + 32 n,
+  // n = 0, 1, 2: three accumulators per lane (ra0-2) take a tile's 32 values
+  // per lane; at the end of the tile n = 0 and 1 are complete (the next tile
+  // is 64 keys on: its n = 0 is this tile's n = 2) and go to dwin with ONE LDS
+  // atomic per lane -- LDS float atomics are slow: one per value took seven
+  // times the rest of the kernel.
+  // dwin is a ring over the distances relative to the first tile's window
+  // start: a tile adds into 320 consecutive entries, the window moves up by BT
+  // per tile, and the BT entries it leaves behind are complete: one wavefront
+  // moves them to dtab during the next tile (they are reused three tiles
+  // later).
+  float* dwin = reinterpret_cast<float*>(fb_smem + 2 * STAGE);
+  float* dtab_h = nullptr;
+  if constexpr (BIAS && OWN_Q) {
+    dtab_h = dtab + (int64_t)h * (2 * L - 1);
+    if (tid < Cfg::RING) dwin[tid] = 0.f;
+  }
+  auto flush_dwin = [&](int chunk) {   // 64 ring entries from distance chunk * BT
+    const int slot = ((chunk * Cfg::BT) & (Cfg::RING - 1)) + lane;
+    const float val = dwin[slot];
+    dwin[slot] = 0.f;
+    const int d = chunk * Cfg::BT - (own0 + Cfg::BOWN - 1) + (L - 1) + lane;
+    if (val != 0.f && d >= 0 && d <= 2 * L - 2) atomicAdd(dtab_h + d, val);
+  };
+  float ra0 = 0.f, ra1 = 0.f, ra2 = 0.f;
+  const int rot_m = l32 + 4 * half;        // lane m takes key column c from lane
+  const int rot_hb = half << 7;            // (m + c) mod 32 of its half-wave
 
   fa_f32x16_t acc[Cfg::DT];
 #pragma unroll
@@ -639,6 +774,16 @@ __global__ __launch_bounds__(512) void flash_attention_backward_kernel(
       need_mask = need_mask || !own_uniform ||
                   __ballot(sid_t[lane] != own_first) != 0ull;
     }
+    // this lane's view of the tile's bias window: entry of streamed row j is
+    // bw[j] (own queries) or bw[-j] (own keys)
+    const float* bw = nullptr;
+    if constexpr (BIAS)
+      bw = reinterpret_cast<const float*>(t1r + NCOPY * Cfg::TILE + Cfg::BIAS_AT) +
+           (OWN_Q ? Cfg::BOWN - 1 - (wave * 32 + l32)
+                  : wave * 32 + l32 + Cfg::BT - 1);
+    if constexpr (BIAS && OWN_Q) {
+      if (t > t_begin && wave == ((t - 1) & 7)) flush_dwin(t - 1);
+    }
 
     auto do_sub = [&](auto sub_c) {
       constexpr int SUB = decltype(sub_c)::value;
@@ -664,6 +809,15 @@ __global__ __launch_bounds__(512) void flash_attention_backward_kernel(
               rr + (((2 * s + half) ^ sw) * 16));
           acc_dp = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, f2[s], acc_dp, 0, 0, 0);
         }
+      }
+      if constexpr (BIAS) {
+#pragma unroll
+        for (int r4 = 0; r4 < 4; ++r4)
+#pragma unroll
+          for (int c = 0; c < 4; ++c) {
+            const int j = SUB * 32 + 8 * r4 + 4 * half + c;
+            acc_s[4 * r4 + c] += OWN_Q ? bw[j] : bw[-j];
+          }
       }
       // weights (and their gradient) of this lane's own entity against the
       // 16 streamed rows SUB * 32 + 8 (r / 4) + 4 half + r % 4
@@ -713,6 +867,30 @@ __global__ __launch_bounds__(512) void flash_attention_backward_kernel(
           }
         }
       }
+      if constexpr (BIAS && OWN_Q) {
+        if (ow_last >= L) {          // rows past the end carry no gradient
+          asm volatile("" ::: "memory");
+#pragma unroll
+          for (int r = 0; r < 16; ++r)
+            if (my >= L) w[r] = 0.f;
+        }
+        // register r holds key SUB * 32 + c, c = 8 (r / 4) + r % 4 + 4 half: in
+        // lane m it comes from query (m + c) mod 32, at distance
+        // -m + 32 (SUB + [m + c >= 32])
+        float lo = 0.f, hi = 0.f;
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+          const int c0 = 8 * (r >> 2) + (r & 3);
+          const int from = (((rot_m + c0) & 31) << 2) | rot_hb;
+          const float val = __int_as_float(
+              __builtin_amdgcn_ds_bpermute(from, __float_as_int(w[r])));
+          const float up = rot_m >= 32 - c0 ? val : 0.f;
+          hi += up;
+          lo += val - up;
+        }
+        if constexpr (SUB == 0) { ra0 += lo; ra1 += hi; }
+        else { ra1 += lo; ra2 += hi; }
+      }
       fa_bf16x8_t wf[2];
 #pragma unroll
       for (int uu = 0; uu < 2; ++uu) {
@@ -755,9 +933,29 @@ __global__ __launch_bounds__(512) void flash_attention_backward_kernel(
     };
     do_sub(std::integral_constant<int, 0>());
     do_sub(std::integral_constant<int, 1>());
+    if constexpr (BIAS && OWN_Q) {
+      // the lower half-wave hands in n = 0 (e = -m), the upper one n = 1
+      // (e = 32 - m), each the sum of both halves' accumulators
+      const float got = __shfl_xor(half == 0 ? ra1 : ra0, 32);
+      const float mine = (half == 0 ? ra0 : ra1) + got;
+      const int rel = t * Cfg::BT + Cfg::BOWN - 1 - 32 * wave + 32 * half - l32;
+      atomicAdd(dwin + (rel & (Cfg::RING - 1)), mine);
+      ra0 = ra2;
+      ra1 = 0.f;
+      ra2 = 0.f;
+    }
 
     __builtin_amdgcn_s_waitcnt(0x0070 | (15 << 8));   // vmcnt(0): tile t+1 is here
     __syncthreads();
+  }
+  if constexpr (BIAS && OWN_Q) {
+    // n = 2 of the last tile, then what its window still holds: five chunks
+    if (t_end > t_begin) {
+      const int rel = t_end * Cfg::BT + Cfg::BOWN - 1 - 32 * wave - l32;
+      atomicAdd(dwin + (rel & (Cfg::RING - 1)), ra0);
+      __syncthreads();
+      if (wave < 5) flush_dwin(t_end - 1 + wave);
+    }
   }
 
   if (my < L) {
@@ -776,75 +974,122 @@ __global__ __launch_bounds__(512) void flash_attention_backward_kernel(
   }
 }
 
-template <int D, bool CAUSAL, int WHAT, bool SEQ>
+template <int D, bool CAUSAL, int WHAT, bool SEQ, bool BIAS>
 static int launch_flash_backward_one(const bf16_t* q, const bf16_t* k,
                                      const bf16_t* v, const bf16_t* dout,
                                      const float* lse, const float* delta,
                                      bf16_t* grad, int B, int L, int H,
-                                     const int32_t* seq, hipStream_t st) {
+                                     const int32_t* seq, const float* tab,
+                                     float* dtab, hipStream_t st) {
   using Cfg = FlashBwdCfg<D>;
-  constexpr int LDS = 2 * Cfg::stage_bytes(WHAT);
+  constexpr int LDS = 2 * Cfg::stage_bytes(WHAT) +
+                      (BIAS && WHAT == BWD_DQ ? Cfg::RING * 4 : 0);
   dim3 grid((unsigned)((L + Cfg::BOWN - 1) / Cfg::BOWN), (unsigned)(B * H));
-  auto kern = flash_attention_backward_kernel<D, CAUSAL, WHAT, SEQ>;
+  auto kern = flash_attention_backward_kernel<D, CAUSAL, WHAT, SEQ, BIAS>;
   MOE_ALLOW_LDS(kern, LDS);
   kern<<<grid, Cfg::THREADS, LDS, st>>>(q, k, v, dout, lse, delta, grad, L, H,
-                                        seq);
+                                        seq, tab, dtab);
   MOE_CHECK_LAUNCH("self_attention_backward (fused)");
   return 0;
 }
 
-template <int D, bool CAUSAL, bool SEQ>
+template <int D, bool CAUSAL, bool SEQ, bool BIAS>
 static int launch_flash_backward(const bf16_t* q, const bf16_t* k,
                                  const bf16_t* v, const bf16_t* dout,
                                  bf16_t* dq, bf16_t* dk, bf16_t* dv, float* lse,
                                  float* delta, int B, int L, int H,
-                                 const int32_t* seq, hipStream_t st) {
+                                 const int32_t* seq, const float* tab,
+                                 float* dtab, hipStream_t st) {
   using Cfg = FlashCfg<D>;
-  constexpr int LDS = Cfg::LDS_BYTES + 512;
+  constexpr int LDS = Cfg::LDS_BYTES + 512 + 1536;
   dim3 grid((unsigned)((L + Cfg::BQ - 1) / Cfg::BQ), (unsigned)(B * H));
-  auto stats = flash_attention_kernel<D, CAUSAL, true, SEQ>;
+  auto stats = flash_attention_kernel<D, CAUSAL, true, SEQ, BIAS>;
   MOE_ALLOW_LDS(stats, LDS);
   stats<<<grid, Cfg::THREADS, LDS, st>>>(q, k, v, nullptr, L, H, dout, lse,
-                                         delta, seq);
+                                         delta, seq, tab);
   MOE_CHECK_LAUNCH("self_attention_backward (lse, delta)");
-  int rc = launch_flash_backward_one<D, CAUSAL, BWD_DV, SEQ>(
-      q, k, v, dout, lse, delta, dv, B, L, H, seq, st);
+  int rc = launch_flash_backward_one<D, CAUSAL, BWD_DV, SEQ, BIAS>(
+      q, k, v, dout, lse, delta, dv, B, L, H, seq, tab, dtab, st);
   if (rc != 0) return rc;
-  rc = launch_flash_backward_one<D, CAUSAL, BWD_DK, SEQ>(
-      q, k, v, dout, lse, delta, dk, B, L, H, seq, st);
+  rc = launch_flash_backward_one<D, CAUSAL, BWD_DK, SEQ, BIAS>(
+      q, k, v, dout, lse, delta, dk, B, L, H, seq, tab, dtab, st);
   if (rc != 0) return rc;
-  return launch_flash_backward_one<D, CAUSAL, BWD_DQ, SEQ>(
-      q, k, v, dout, lse, delta, dq, B, L, H, seq, st);
+  return launch_flash_backward_one<D, CAUSAL, BWD_DQ, SEQ, BIAS>(
+      q, k, v, dout, lse, delta, dq, B, L, H, seq, tab, dtab, st);
 }
 
-size_t flash_attention_backward_workspace_bytes(int B, int L, int H) {
-  return 2 * (((size_t)B * H * L * sizeof(float) + 255) & ~(size_t)255) + 256;
+__global__ void fill_zero_kernel(float* __restrict__ p, int64_t n) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i < n) p[i] = 0.f;
+}
+
+// dvalues[h][b] = sum of dtab[h][d] over the distances d of bucket b (the
+// gradient of the gather), rounded to bf16.  One wavefront per (bucket, head):
+// lanes stride over the distances, then a butterfly sum.
+__global__ __launch_bounds__(64) void relative_table_backward_kernel(
+    const float* __restrict__ dtab, const int32_t* __restrict__ bucket,
+    bf16_t* __restrict__ dvalues, int n, int NB) {
+  const int b = blockIdx.x;
+  const float* row = dtab + (int64_t)blockIdx.y * n;
+  float sum = 0.f;
+  for (int d = threadIdx.x; d < n; d += 64)
+    if (bucket[d] == b) sum += row[d];
+#pragma unroll
+  for (int off = 32; off >= 1; off >>= 1) sum += __shfl_xor(sum, off);
+  if (threadIdx.x == 0)
+    store_f32<bf16_t>(dvalues + (int64_t)blockIdx.y * NB + b, sum);
+}
+
+size_t flash_attention_backward_workspace_bytes(int B, int L, int H,
+                                                bool relative_bias) {
+  return 2 * (((size_t)B * H * L * sizeof(float) + 255) & ~(size_t)255) + 256 +
+         (relative_bias ? 2 * relative_table_bytes(L, H) : 0);
 }
 
 int flash_attention_backward(const void* q, const void* k, const void* v,
                              const void* dout, void* dq, void* dk, void* dv,
                              int B, int L, int H, int D, int causal,
-                             const int32_t* sequence_id, void* workspace,
-                             hipStream_t st) {
+                             const int32_t* sequence_id, const void* rel_values,
+                             const int32_t* rel_bucket, int num_buckets,
+                             void* dvalues, void* workspace, hipStream_t st) {
+  const size_t per = (((size_t)B * H * L * sizeof(float) + 255) & ~(size_t)255) /
+                     sizeof(float);
   float* lse = (float*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
-  float* delta = lse + ((((size_t)B * H * L * sizeof(float) + 255) &
-                         ~(size_t)255) / sizeof(float));
+  float* delta = lse + per;
+  float *tab = nullptr, *dtab = nullptr;
+  const int n = 2 * L - 1;
+  if (rel_values != nullptr) {
+    tab = delta + per;
+    dtab = tab + relative_table_bytes(L, H) / sizeof(float);
+    int rc = launch_relative_table(rel_values, rel_bucket, tab, L, H,
+                                   num_buckets, st);
+    if (rc != 0) return rc;
+    const int64_t cells = (int64_t)H * n;
+    fill_zero_kernel<<<(unsigned)((cells + 255) / 256), 256, 0, st>>>(dtab, cells);
+    MOE_CHECK_LAUNCH("self_attention_backward (clear)");
+  }
   const bf16_t *q_ = (const bf16_t*)q, *k_ = (const bf16_t*)k,
                *v_ = (const bf16_t*)v, *d_ = (const bf16_t*)dout;
   bf16_t *dq_ = (bf16_t*)dq, *dk_ = (bf16_t*)dk, *dv_ = (bf16_t*)dv;
-#define MOE_FLASH_BWD(DD, C, S)                                               \
-  launch_flash_backward<DD, C, S>(q_, k_, v_, d_, dq_, dk_, dv_, lse, delta, B, \
-                                  L, H, sequence_id, st)
-  const bool sq = sequence_id != nullptr;
-  if (D == 128) {
-    if (causal) return sq ? MOE_FLASH_BWD(128, true, true)
-                          : MOE_FLASH_BWD(128, true, false);
-    return sq ? MOE_FLASH_BWD(128, false, true) : MOE_FLASH_BWD(128, false, false);
-  }
-  if (causal) return sq ? MOE_FLASH_BWD(64, true, true)
-                        : MOE_FLASH_BWD(64, true, false);
-  return sq ? MOE_FLASH_BWD(64, false, true) : MOE_FLASH_BWD(64, false, false);
-#undef MOE_FLASH_BWD
+  const int rc = flash_dispatch(
+      causal != 0, sequence_id != nullptr, tab != nullptr,
+      [&](auto c, auto s, auto bi) {
+        constexpr bool C = decltype(c)::value, S = decltype(s)::value,
+                       BI = decltype(bi)::value;
+        if (D == 128)
+          return launch_flash_backward<128, C, S, BI>(
+              q_, k_, v_, d_, dq_, dk_, dv_, lse, delta, B, L, H, sequence_id,
+              tab, dtab, st);
+        return launch_flash_backward<64, C, S, BI>(q_, k_, v_, d_, dq_, dk_, dv_,
+                                                   lse, delta, B, L, H,
+                                                   sequence_id, tab, dtab, st);
+      });
+  if (rc != 0 || rel_values == nullptr) return rc;
+  relative_table_backward_kernel<<<dim3((unsigned)num_buckets, (unsigned)H), 64,
+                                   0, st>>>(dtab, rel_bucket, (bf16_t*)dvalues,
+                                            n, num_buckets);
+  MOE_CHECK_LAUNCH("self_attention_backward (bias values)");
+  return 0;
 }
 
 }  // namespace mesh_moe

@@ -953,9 +953,9 @@ extern "C" size_t mesh_moe_self_attention_workspace_bytes(int B, int L, int H,
                                                           int D, int dtype,
                                                           int relative_bias) {
   if (B < 1 || L < 1 || H < 1 || D < 1 || !valid_dtype(dtype)) return 0;
-  if (!relative_bias && flash_attention_supported(L, H, D, dtype, nullptr,
-                                                  nullptr, nullptr, nullptr))
-    return flash_attention_workspace_bytes(B, L, H, D);
+  if (flash_attention_supported(L, H, D, dtype, nullptr, nullptr, nullptr,
+                                nullptr))
+    return flash_attention_workspace_bytes(B, L, H, D, relative_bias != 0);
   const size_t b = dtype_size(dtype);
   const size_t hd = (size_t)B * H * L * D, ll = (size_t)B * H * L * L;
   return 4 * hd * b + ll * 4 + ll * b + 7 * 256;
@@ -988,15 +988,15 @@ extern "C" int mesh_moe_self_attention(const void* q, const void* k,
                                      B, L, H, D, dtype, rel_values != nullptr),
               MESH_MOE_E_ARG, "self_attention: workspace too small");
   hipStream_t st = (hipStream_t)stream;
-  if (rel_values == nullptr &&
-      flash_attention_supported(L, H, D, dtype, nullptr, nullptr, nullptr,
+  if (flash_attention_supported(L, H, D, dtype, nullptr, nullptr, nullptr,
                                 nullptr)) {
     // fused kernel: the logits stay on chip
     MOE_REQUIRE(flash_attention_supported(L, H, D, dtype, q, k, v, out),
                 MESH_MOE_E_UNSUPPORTED,
                 "self_attention: q, k, v, out must be 16-byte aligned");
     return flash_attention(q, k, v, out, B, L, H, D, causal ? 1 : 0,
-                           sequence_id, workspace, st);
+                           sequence_id, rel_values, rel_bucket, num_buckets,
+                           workspace, st);
   }
   if (dtype == MESH_MOE_F32)
     return run_attention<float>((const float*)q, (const float*)k,
@@ -1253,21 +1253,21 @@ extern "C" int mesh_moe_relative_bias_backward(const void* dlogits,
   return 0;
 }
 
-extern "C" size_t mesh_moe_self_attention_backward_workspace_bytes(int B, int L,
-                                                                   int H, int D,
-                                                                   int dtype) {
+extern "C" size_t mesh_moe_self_attention_backward_workspace_bytes(
+    int B, int L, int H, int D, int dtype, int relative_bias) {
   if (B < 1 || L < 1 || H < 1 || D < 1 || !valid_dtype(dtype)) return 0;
   if (!flash_attention_supported(L, H, D, dtype, nullptr, nullptr, nullptr,
                                  nullptr))
     return 0;
-  return flash_attention_backward_workspace_bytes(B, L, H);
+  return flash_attention_backward_workspace_bytes(B, L, H, relative_bias != 0);
 }
 
 extern "C" int mesh_moe_self_attention_backward(
     const void* q, const void* k, const void* v, const void* dout, void* dq,
     void* dk, void* dv, int B, int L, int H, int D, int causal,
-    const int32_t* sequence_id, int dtype, void* workspace,
-    size_t workspace_bytes, void* stream) {
+    const int32_t* sequence_id, const void* rel_values,
+    const int32_t* rel_bucket, int num_buckets, void* dvalues, int dtype,
+    void* workspace, size_t workspace_bytes, void* stream) {
   MOE_REQUIRE(q && k && v && dout && dq && dk && dv && workspace, MESH_MOE_E_ARG,
               "self_attention_backward: null pointer");
   MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG,
@@ -1278,15 +1278,23 @@ extern "C" int mesh_moe_self_attention_backward(
   MOE_REQUIRE((int64_t)B * H <= 65535, MESH_MOE_E_UNSUPPORTED,
               "self_attention_backward: batch * heads = %lld > 65535",
               (long long)B * H);
+  MOE_REQUIRE((rel_values == nullptr) == (rel_bucket == nullptr) &&
+                  (rel_values == nullptr) == (dvalues == nullptr) &&
+                  (rel_values == nullptr || num_buckets >= 1),
+              MESH_MOE_E_ARG,
+              "self_attention_backward: rel_values, rel_bucket, num_buckets "
+              "and dvalues go together");
   MOE_REQUIRE(flash_attention_supported(L, H, D, dtype, q, k, v, dout) &&
                   flash_attention_supported(L, H, D, dtype, dq, dk, dv, dout),
               MESH_MOE_E_UNSUPPORTED,
               "self_attention_backward: the fused kernels take bf16, d_kv 64 or "
               "128, L a multiple of 8 and 16-byte aligned tensors (L=%d D=%d)",
               L, D);
-  MOE_REQUIRE(workspace_bytes >= flash_attention_backward_workspace_bytes(B, L, H),
+  MOE_REQUIRE(workspace_bytes >= flash_attention_backward_workspace_bytes(
+                                     B, L, H, rel_values != nullptr),
               MESH_MOE_E_ARG, "self_attention_backward: workspace too small");
   return flash_attention_backward(q, k, v, dout, dq, dk, dv, B, L, H, D,
-                                  causal ? 1 : 0, sequence_id, workspace,
+                                  causal ? 1 : 0, sequence_id, rel_values,
+                                  rel_bucket, num_buckets, dvalues, workspace,
                                   (hipStream_t)stream);
 }

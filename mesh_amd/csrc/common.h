@@ -22,17 +22,24 @@ int batched_gemm_nt(const void* A, const void* B, void* C, int E, int R, int N,
 // Fused self-attention (attention.hip): q, k, v, out [B,L,H*D] bf16.
 bool flash_attention_supported(int L, int H, int D, int dtype, const void* q,
                                const void* k, const void* v, const void* out);
-size_t flash_attention_workspace_bytes(int B, int L, int H, int D);
+// With rel_values [H, num_buckets] bf16 and rel_bucket [2L-1] (null: none) the
+// relative attention bias is added to the logits; the backward pass then
+// writes its gradient to dvalues [H, num_buckets] bf16.
+size_t flash_attention_workspace_bytes(int B, int L, int H, int D,
+                                       bool relative_bias);
 int flash_attention(const void* q, const void* k, const void* v, void* out,
                     int B, int L, int H, int D, int causal,
-                    const int32_t* sequence_id, void* workspace,
+                    const int32_t* sequence_id, const void* rel_values,
+                    const int32_t* rel_bucket, int num_buckets, void* workspace,
                     hipStream_t st);
-size_t flash_attention_backward_workspace_bytes(int B, int L, int H);
+size_t flash_attention_backward_workspace_bytes(int B, int L, int H,
+                                                bool relative_bias);
 int flash_attention_backward(const void* q, const void* k, const void* v,
                              const void* dout, void* dq, void* dk, void* dv,
                              int B, int L, int H, int D, int causal,
-                             const int32_t* sequence_id, void* workspace,
-                             hipStream_t st);
+                             const int32_t* sequence_id, const void* rel_values,
+                             const int32_t* rel_bucket, int num_buckets,
+                             void* dvalues, void* workspace, hipStream_t st);
 
 #define MOE_REQUIRE(cond, code, ...)      \
   do {                                    \

@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 22
+ABI_VERSION = 23
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -190,11 +190,12 @@ _SIGNATURES = {
         ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
         _vp, ctypes.c_size_t, _vp]),
     "mesh_moe_self_attention_backward_workspace_bytes": (ctypes.c_size_t, [
-        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int]),
     "mesh_moe_self_attention_backward": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
-        ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, ctypes.c_int, _vp,
-        ctypes.c_size_t, _vp]),
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, ctypes.c_int,
+        _vp, ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
     "mesh_moe_attention_decode": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
@@ -1377,35 +1378,34 @@ def self_attention_backward(q, k, v, dout, num_heads, causal, fused=None,
     dq = dlogits . k,       dk = dlogits^T . q
   with heads moved to the front and back by torch permutes.  fused=True raises
   for shapes the fused kernels do not take.  With relative_bias = (values
-  [H, NB], bucket [2L-1]) the composed form runs and the gradient of the values
-  is the fourth result."""
+  [H, NB], bucket [2L-1]) the gradient of the values is the fourth result."""
   b, l, hd = q.shape
   h = num_heads
   if hd % h:
     raise MoeHipError("q channels %d not divisible by %d heads" % (hd, h))
   d = hd // h
-  if relative_bias is not None:
-    if fused:
-      raise MoeHipError("self_attention_backward: the fused kernels take no "
-                        "relative attention bias")
-    fused = False
   if fused is None or fused:
     lib = load_library()
     code = dtype_code(q.dtype)
-    ws_bytes = lib.mesh_moe_self_attention_backward_workspace_bytes(b, l, h, d,
-                                                                    code)
+    ws_bytes = lib.mesh_moe_self_attention_backward_workspace_bytes(
+        b, l, h, d, code, int(relative_bias is not None))
     if ws_bytes:
       ws = torch.empty((ws_bytes,), dtype=torch.uint8, device=q.device)
       dq, dk, dv = (torch.empty_like(q) for _ in range(3))
+      dvalues = None
+      if relative_bias is not None:
+        dvalues = torch.empty_like(relative_bias[0])
       with _stage("self_attention_backward"):
         _check(lib.mesh_moe_self_attention_backward(
             _dev(q, "q"), _dev(k, "k", q.dtype, (b, l, hd)),
             _dev(v, "v", q.dtype, (b, l, hd)),
             _dev(dout, "dout", q.dtype, (b, l, hd)), dq.data_ptr(),
             dk.data_ptr(), dv.data_ptr(), b, l, h, d, int(bool(causal)),
-            _sequence_id_ptr(sequence_id, b, l), code, ws.data_ptr(), ws_bytes,
-            _stream()), "self_attention_backward")
-      return dq, dk, dv
+            _sequence_id_ptr(sequence_id, b, l),
+            *_relative_bias_ptrs(relative_bias, q.dtype, h, l),
+            None if dvalues is None else dvalues.data_ptr(), code,
+            ws.data_ptr(), ws_bytes, _stream()), "self_attention_backward")
+      return (dq, dk, dv) if dvalues is None else (dq, dk, dv, dvalues)
     if fused:
       raise MoeHipError("self_attention_backward: the fused kernels do not take "
                         "dtype %s, L=%d, d_kv=%d" % (q.dtype, l, d))

@@ -259,12 +259,15 @@ def test_attention_decode(hip, case, act_dtype):
 @pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("causal", [False, True])
 @pytest.mark.parametrize("case", [(2, 40, 2, 16, 8), (2, 200, 3, 64, 32),
-                                  (1, 328, 2, 128, 32)],
+                                  (1, 328, 2, 128, 32), (1, 1024, 2, 64, 32),
+                                  (2, 576, 1, 128, 8)],
                          ids=lambda c: "x".join(map(str, c)))
 def test_self_attention_relative_bias(hip, case, causal, act_dtype):
   """The relative attention bias (transformer_layers.py:317-352): forward,
   (dq, dk, dv) and the gradient of the bias values against the oracle, with and
-  without sequence ids."""
+  without sequence ids.  bf16 with d_kv 64 or 128 runs the fused kernels
+  (forward and backward), whose composed counterpart (fused=False) is checked
+  as well; everything else the three-step form."""
   b, l, heads, d, nb = case
   rng = np.random.default_rng(sum(case) + causal)
   mk = lambda: O.cast_act(
@@ -293,11 +296,18 @@ def test_self_attention_relative_bias(hip, case, causal, act_dtype):
                                        sequence_id=ids, relative_values=values)
     btol = dict(rtol=2e-4, atol=2e-4) if act_dtype == "float32" else dict(
         rtol=3e-2, atol=3e-2)
-    assert len(got_b) == 4
-    for gt, wnt, name in zip(got_b, want_b, ("dq", "dk", "dv", "dvalues")):
-      scale = max(1.0, float(np.abs(wnt).max()))
-      np.testing.assert_allclose(H.to_np(gt), wnt, rtol=btol["rtol"],
-                                 atol=btol["atol"] * scale, err_msg=name)
+    runs = [("", got_b)]
+    if act_dtype == "bfloat16" and d in (64, 128):
+      runs.append(("composed ", hip.self_attention_backward(
+          g(q), g(k), g(v), g(do), heads, causal, fused=False, sequence_id=sid,
+          relative_bias=rel)))
+    for label, grads in runs:
+      assert len(grads) == 4
+      for gt, wnt, name in zip(grads, want_b, ("dq", "dk", "dv", "dvalues")):
+        scale = max(1.0, float(np.abs(wnt).max()))
+        np.testing.assert_allclose(H.to_np(gt), wnt, rtol=btol["rtol"],
+                                   atol=btol["atol"] * scale,
+                                   err_msg=label + name)
   # not the same as no bias
   plain = H.to_np(hip.self_attention(g(q), g(k), g(v), heads, causal))
   assert np.abs(plain - got).max() > 1e-2
