@@ -101,6 +101,24 @@ __device__ __forceinline__ float fa_exp2(float x) {
   return __builtin_amdgcn_exp2f(x);
 }
 
+// Which (tile, batch * head) a block works on.  Workgroups go to the 8 XCDs
+// round-robin in launch order (x fastest), so with the plain mapping the tiles
+// of one (batch, head) land on all of them and every XCD's L2 fetches that
+// head's K and V for itself.  Here XCD x takes the heads x, x + 8, ... and runs
+// all tiles of a head back to back: a head's K and V enter one L2 once.
+__device__ __forceinline__ void fa_block_to_work(int n_tiles, int& tile, int& bh) {
+  const int nbh = (int)gridDim.y;
+  if (nbh % 8 == 0) {
+    const int id = (int)blockIdx.x + n_tiles * (int)blockIdx.y;
+    const int slot = id >> 3;
+    bh = (slot / n_tiles) * 8 + (id & 7);
+    tile = slot % n_tiles;
+  } else {
+    tile = (int)blockIdx.x;
+    bh = (int)blockIdx.y;
+  }
+}
+
 // STATS: instead of the outputs, write what the backward kernels need per
 // query: lse = log of the softmax denominator (row maximum included) and
 // delta = sum_d dout[q, d] * out[q, d] (= sum_k dweights * weights), both
@@ -125,8 +143,10 @@ __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int half = lane >> 5, l32 = lane & 31;
   const int nq = (L + Cfg::BQ - 1) / Cfg::BQ;
-  const int qt = nq - 1 - (int)blockIdx.x;   // long (late) query tiles first
-  const int bh = blockIdx.y, b = bh / H, h = bh % H;
+  int tile_x, bh;
+  fa_block_to_work(nq, tile_x, bh);
+  const int qt = nq - 1 - tile_x;            // long (late) query tiles first
+  const int b = bh / H, h = bh % H;
   const int q0 = qt * Cfg::BQ;
   const int64_t row_stride = (int64_t)H * D;               // elements
   const bf16_t* qb = q + ((int64_t)b * L) * row_stride + (int64_t)h * D;
@@ -599,9 +619,11 @@ __global__ __launch_bounds__(512) void flash_attention_backward_kernel(
   const int half = lane >> 5, l32 = lane & 31;
   const int n_own = (L + Cfg::BOWN - 1) / Cfg::BOWN;
   // long tiles first: late queries, early keys
-  const int ot = OWN_Q && CAUSAL ? n_own - 1 - (int)blockIdx.x : (int)blockIdx.x;
+  int tile_x, bh;
+  fa_block_to_work(n_own, tile_x, bh);
+  const int ot = OWN_Q && CAUSAL ? n_own - 1 - tile_x : tile_x;
   const int own0 = ot * Cfg::BOWN;
-  const int bh = blockIdx.y, b = bh / H, h = bh % H;
+  const int b = bh / H, h = bh % H;
   const int64_t row_stride = (int64_t)H * D;
   const int64_t head_off = ((int64_t)b * L) * row_stride + (int64_t)h * D;
   // own rows supply the register fragments, streamed rows the LDS tiles
