@@ -1018,19 +1018,21 @@ extern "C" int mesh_moe_self_attention(const void* q, const void* k,
 // dtype, out = sum_m w_m v_m.  The caches are read once: HBM-bound.
 //   q, k_new, v_new, out [B, H*D]; k_cache, v_cache [B, Lm, H*D] (updated in
 //   place); position [B] int32 on the device.
-// Dynamic LDS: max(Lm, 256) + D + 8 + 2048 floats.
+// NT threads per block: four wavefronts, or sixteen when the grid has few
+// blocks (each block must then keep more loads in flight to draw its share of
+// the bandwidth).  Dynamic LDS: max(Lm, NT) + D + 16 + 8 NT floats.
 // ---------------------------------------------------------------------------
-template <typename T>
-__global__ __launch_bounds__(256) void attention_decode_kernel(
+template <typename T, int NT>
+__global__ __launch_bounds__(NT) void attention_decode_kernel(
     const T* __restrict__ q, const T* __restrict__ k_new,
     const T* __restrict__ v_new, T* __restrict__ k_cache,
     T* __restrict__ v_cache, const int32_t* __restrict__ position,
     T* __restrict__ out, int Lm, int H, int D, int vec) {
   extern __shared__ __attribute__((aligned(16))) float dec_smem[];
-  float* wl = dec_smem;                     // [max(Lm, 256)] logits, then weights
-  float* qs = wl + (Lm > 256 ? Lm : 256);   // [D]
-  float* red = qs + D;                      // [8]
-  float* part = red + 8;                    // [2048] partial outputs (vec path)
+  float* wl = dec_smem;                     // [max(Lm, NT)] logits, then weights
+  float* qs = wl + (Lm > NT ? Lm : NT);     // [D]
+  float* red = qs + D;                      // [16]
+  float* part = red + 16;                   // [8 NT] partial outputs (vec path)
   const int h = blockIdx.x, b = blockIdx.y, tid = threadIdx.x;
   const int lane = tid & 63, wave = tid >> 6;
   const int64_t hd = (int64_t)H * D;
@@ -1040,7 +1042,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
   const T* vnr = v_new + b * hd + (int64_t)h * D;
   T* kc = k_cache + (int64_t)b * Lm * hd + (int64_t)h * D;
   T* vc = v_cache + (int64_t)b * Lm * hd + (int64_t)h * D;
-  for (int d = tid; d < D; d += 256) {
+  for (int d = tid; d < D; d += NT) {
     qs[d] = load_f32<T>(qr + d);
     kc[(int64_t)pos * hd + d] = knr[d];
     vc[(int64_t)pos * hd + d] = vnr[d];
@@ -1048,11 +1050,11 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
   __syncthreads();
   constexpr int VN = Vec16B<T>::N;
   // vec path: a row is CH 16-byte chunks, read by LPR lanes (a power of two
-  // >= CH, <= 64); the block's G = 256 / LPR lane groups take rows g, g + G, ..
+  // >= CH, <= 64); the block's G = NT / LPR lane groups take rows g, g + G, ..
   const int CH = D / VN;
   int LPR = 1;
   while (LPR < CH) LPR *= 2;
-  const int G = 256 / LPR, g = tid / LPR, c = tid % LPR;
+  const int G = NT / LPR, g = tid / LPR, c = tid % LPR;
   const bool lane_on = c < CH;
   // logits of the visible rows; row `pos` comes from the step's own key
   float m = -INFINITY;
@@ -1088,7 +1090,7 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
       }
     }
   } else {
-    for (int j = tid; j <= pos; j += 256) {
+    for (int j = tid; j <= pos; j += NT) {
       const T* kr = j == pos ? knr : kc + (int64_t)j * hd;
       float acc = 0.f;
       for (int d = 0; d < D; ++d) acc = fmaf(qs[d], load_f32<T>(kr + d), acc);
@@ -1106,16 +1108,16 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
     if (lane == 0) red[wave] = v;
     __syncthreads();
     float r = red[0];
-    for (int w = 1; w < 4; ++w) r = is_max ? fmaxf(r, red[w]) : r + red[w];
+    for (int w = 1; w < NT / 64; ++w) r = is_max ? fmaxf(r, red[w]) : r + red[w];
     return r;
   };
   m = block_all(m, true);
   const float negm = -m;
   float sum = 0.f;
-  for (int j = tid; j <= pos; j += 256) sum += expf(wl[j] + negm);
+  for (int j = tid; j <= pos; j += NT) sum += expf(wl[j] + negm);
   sum = block_all(sum, false);
   const float neglse = -(logf(sum) + m);
-  for (int j = tid; j <= pos; j += 256)
+  for (int j = tid; j <= pos; j += NT)
     wl[j] = round_to<T>(expf(wl[j] + neglse));
   __syncthreads();
   T* orow = out + b * hd + (int64_t)h * D;
@@ -1153,13 +1155,13 @@ __global__ __launch_bounds__(256) void attention_decode_kernel(
       for (int u = 0; u < VN; ++u) part[g * D + c * VN + u] = acc[u];
     }
     __syncthreads();
-    for (int d = tid; d < D; d += 256) {
+    for (int d = tid; d < D; d += NT) {
       float total = 0.f;
       for (int gg = 0; gg < G; ++gg) total += part[gg * D + d];
       store_f32<T>(orow + d, total);
     }
   } else {
-    for (int d = tid; d < D; d += 256) {
+    for (int d = tid; d < D; d += NT) {
       float acc = 0.f;
       for (int j = 0; j <= pos; ++j) {
         const T* vr = j == pos ? vnr : vc + (int64_t)j * hd;
@@ -1183,10 +1185,6 @@ extern "C" int mesh_moe_attention_decode(const void* q, const void* k_new,
               "attention_decode: bad sizes B=%d Lm=%d H=%d D=%d", B, Lm, H, D);
   MOE_REQUIRE(B <= 65535, MESH_MOE_E_UNSUPPORTED,
               "attention_decode: batch %d > 65535", B);
-  const size_t floats = (size_t)(Lm > 256 ? Lm : 256) + (size_t)D + 8 + 2048;
-  const size_t smem = floats * sizeof(float);
-  MOE_REQUIRE(smem <= 150 * 1024, MESH_MOE_E_UNSUPPORTED,
-              "attention_decode: memory length %d does not fit in LDS", Lm);
   hipStream_t st = (hipStream_t)stream;
   const dim3 grid((unsigned)H, (unsigned)B);
   const size_t esz = dtype_size(dtype);
@@ -1194,21 +1192,28 @@ extern "C" int mesh_moe_attention_decode(const void* q, const void* k_new,
   const int vec = ((size_t)D * esz) % 16 == 0 && (size_t)D * esz <= 1024 &&
                   (((uintptr_t)k_cache | (uintptr_t)k_new | (uintptr_t)v_cache |
                     (uintptr_t)v_new) % 16) == 0;
+  // few blocks: four times the threads, i.e. the loads in flight, per block
+  const bool wide = vec && (int64_t)H * B <= 512 && Lm >= 2048;
+  const int nt = wide ? 1024 : 256;
+  const size_t floats =
+      (size_t)(Lm > nt ? Lm : nt) + (size_t)D + 16 + 8 * (size_t)nt;
+  const size_t smem = floats * sizeof(float);
+  MOE_REQUIRE(smem <= 150 * 1024, MESH_MOE_E_UNSUPPORTED,
+              "attention_decode: memory length %d does not fit in LDS", Lm);
+#define MOE_DECODE(T, NT)                                                      \
+  do {                                                                         \
+    auto kern = attention_decode_kernel<T, NT>;                                \
+    MOE_ALLOW_LDS(kern, smem);                                                 \
+    kern<<<grid, NT, smem, st>>>((const T*)q, (const T*)k_new, (const T*)v_new, \
+                                 (T*)k_cache, (T*)v_cache, position, (T*)out,  \
+                                 Lm, H, D, vec);                               \
+  } while (0)
   if (dtype == MESH_MOE_F32) {
-    auto kern = attention_decode_kernel<float>;
-    MOE_ALLOW_LDS(kern, smem);
-    kern<<<grid, 256, smem, st>>>((const float*)q, (const float*)k_new,
-                                  (const float*)v_new, (float*)k_cache,
-                                  (float*)v_cache, position, (float*)out, Lm, H,
-                                  D, vec);
+    if (wide) MOE_DECODE(float, 1024); else MOE_DECODE(float, 256);
   } else {
-    auto kern = attention_decode_kernel<bf16_t>;
-    MOE_ALLOW_LDS(kern, smem);
-    kern<<<grid, 256, smem, st>>>((const bf16_t*)q, (const bf16_t*)k_new,
-                                  (const bf16_t*)v_new, (bf16_t*)k_cache,
-                                  (bf16_t*)v_cache, position, (bf16_t*)out, Lm,
-                                  H, D, vec);
+    if (wide) MOE_DECODE(bf16_t, 1024); else MOE_DECODE(bf16_t, 256);
   }
+#undef MOE_DECODE
   MOE_CHECK_LAUNCH("attention_decode");
   return 0;
 }

@@ -228,7 +228,8 @@ def test_attention_at_the_block_benchmark_shape(hip, causal):
 
 @pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("case", [(2, 12, 2, 4), (3, 300, 4, 64), (2, 2048, 2, 128),
-                                  (1, 77, 3, 24), (2, 40, 1, 320)],
+                                  (1, 77, 3, 24), (2, 40, 1, 320),
+                                  (3, 2500, 2, 64)],
                          ids=lambda c: "x".join(map(str, c)))
 def test_attention_decode(hip, case, act_dtype):
   """mesh_moe_attention_decode (one step of "incremental" mode) against the
