@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 23
+#define MESH_MOE_ABI_VERSION 24
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -822,13 +822,19 @@ int mesh_moe_self_attention_backward(const void* q, const void* k, const void* v
  * softmax, weights cast to dtype, out = weights . v.
  *   q, k_new, v_new, out [B,H*D] dtype; k_cache, v_cache [B,Lm,H*D] dtype,
  *   updated in place; position [B] int32 on the device, clamped to [0, Lm).
- * One block per (head, batch entry), the caches read once.  Lm up to ~38000
+ * One block per (head, batch entry), the caches read once.  Lm up to ~36000
  * (the logits of a row live in LDS).
+ * rel_values [H,num_buckets] dtype and rel_bucket [2*Lm-1] int32, or both NULL:
+ * the relative attention bias of the step (compute_bias with context.position,
+ * transformer_layers.py:317-352): the logit of memory position m gets
+ * rel_values[h][rel_bucket[m - position[b] + Lm - 1]].
  */
 int mesh_moe_attention_decode(const void* q, const void* k_new, const void* v_new,
                               void* k_cache, void* v_cache,
                               const int32_t* position, void* out, int B, int Lm,
-                              int H, int D, int dtype, void* stream);
+                              int H, int D, const void* rel_values,
+                              const int32_t* rel_bucket, int num_buckets,
+                              int dtype, void* stream);
 
 #ifdef __cplusplus
 }

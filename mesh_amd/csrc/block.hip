@@ -1027,7 +1027,9 @@ __global__ __launch_bounds__(NT) void attention_decode_kernel(
     const T* __restrict__ q, const T* __restrict__ k_new,
     const T* __restrict__ v_new, T* __restrict__ k_cache,
     T* __restrict__ v_cache, const int32_t* __restrict__ position,
-    T* __restrict__ out, int Lm, int H, int D, int vec) {
+    T* __restrict__ out, int Lm, int H, int D, int vec,
+    const T* __restrict__ rel_values, const int32_t* __restrict__ rel_bucket,
+    int NB) {
   extern __shared__ __attribute__((aligned(16))) float dec_smem[];
   float* wl = dec_smem;                     // [max(Lm, NT)] logits, then weights
   float* qs = wl + (Lm > NT ? Lm : NT);     // [D]
@@ -1037,6 +1039,10 @@ __global__ __launch_bounds__(NT) void attention_decode_kernel(
   const int lane = tid & 63, wave = tid >> 6;
   const int64_t hd = (int64_t)H * D;
   const int pos = min(max(position[b], 0), Lm - 1);
+  // relative attention bias of memory position j against the step's position
+  // (transformer_layers.py:317-352): values[h][bucket[j - pos + Lm - 1]]
+  const T* rel_h = rel_values ? rel_values + (int64_t)h * NB : nullptr;
+  const int32_t* rel_b = rel_values ? rel_bucket + (Lm - 1 - pos) : nullptr;
   const T* qr = q + b * hd + (int64_t)h * D;
   const T* knr = k_new + b * hd + (int64_t)h * D;
   const T* vnr = v_new + b * hd + (int64_t)h * D;
@@ -1084,6 +1090,7 @@ __global__ __launch_bounds__(NT) void attention_decode_kernel(
         for (int u = 0; u < VN; ++u) acc = fmaf(qv[u], f[u], acc);
         for (int off = LPR >> 1; off > 0; off >>= 1) acc += __shfl_xor(acc, off, 64);
         if (j <= pos) {
+          if (rel_h) acc += load_f32<T>(rel_h + rel_b[j]);
           if (c == 0) wl[j] = acc;
           m = fmaxf(m, acc);
         }
@@ -1094,6 +1101,7 @@ __global__ __launch_bounds__(NT) void attention_decode_kernel(
       const T* kr = j == pos ? knr : kc + (int64_t)j * hd;
       float acc = 0.f;
       for (int d = 0; d < D; ++d) acc = fmaf(qs[d], load_f32<T>(kr + d), acc);
+      if (rel_h) acc += load_f32<T>(rel_h + rel_b[j]);
       wl[j] = acc;
       m = fmaxf(m, acc);
     }
@@ -1176,9 +1184,17 @@ extern "C" int mesh_moe_attention_decode(const void* q, const void* k_new,
                                          const void* v_new, void* k_cache,
                                          void* v_cache, const int32_t* position,
                                          void* out, int B, int Lm, int H, int D,
-                                         int dtype, void* stream) {
+                                         const void* rel_values,
+                                         const int32_t* rel_bucket,
+                                         int num_buckets, int dtype,
+                                         void* stream) {
   MOE_REQUIRE(q && k_new && v_new && k_cache && v_cache && position && out,
               MESH_MOE_E_ARG, "attention_decode: null pointer");
+  MOE_REQUIRE((rel_values == nullptr) == (rel_bucket == nullptr) &&
+                  (rel_values == nullptr || num_buckets >= 1),
+              MESH_MOE_E_ARG,
+              "attention_decode: rel_values, rel_bucket and num_buckets go "
+              "together");
   MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG,
               "attention_decode: bad dtype %d", dtype);
   MOE_REQUIRE(B >= 1 && Lm >= 1 && H >= 1 && D >= 1, MESH_MOE_E_ARG,
@@ -1193,7 +1209,8 @@ extern "C" int mesh_moe_attention_decode(const void* q, const void* k_new,
                   (((uintptr_t)k_cache | (uintptr_t)k_new | (uintptr_t)v_cache |
                     (uintptr_t)v_new) % 16) == 0;
   // few blocks: four times the threads, i.e. the loads in flight, per block
-  const bool wide = vec && (int64_t)H * B <= 512 && Lm >= 2048;
+  const bool wide = vec && (int64_t)H * B <= 512 && Lm >= 2048 &&
+                    ((size_t)Lm + D + 16 + 8 * 1024) * sizeof(float) <= 150 * 1024;
   const int nt = wide ? 1024 : 256;
   const size_t floats =
       (size_t)(Lm > nt ? Lm : nt) + (size_t)D + 16 + 8 * (size_t)nt;
@@ -1206,7 +1223,8 @@ extern "C" int mesh_moe_attention_decode(const void* q, const void* k_new,
     MOE_ALLOW_LDS(kern, smem);                                                 \
     kern<<<grid, NT, smem, st>>>((const T*)q, (const T*)k_new, (const T*)v_new, \
                                  (T*)k_cache, (T*)v_cache, position, (T*)out,  \
-                                 Lm, H, D, vec);                               \
+                                 Lm, H, D, vec, (const T*)rel_values,          \
+                                 rel_bucket, num_buckets);                     \
   } while (0)
   if (dtype == MESH_MOE_F32) {
     if (wide) MOE_DECODE(float, 1024); else MOE_DECODE(float, 256);

@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 23
+ABI_VERSION = 24
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -198,7 +198,7 @@ _SIGNATURES = {
         _vp, ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
     "mesh_moe_attention_decode": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
-        ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
+        ctypes.c_int, ctypes.c_int, _vp, _vp, ctypes.c_int, ctypes.c_int, _vp]),
 }
 EXPORTS = sorted(_SIGNATURES)
 
@@ -1168,9 +1168,11 @@ def self_attention(q, k, v, num_heads, causal, sequence_id=None,
   return out
 
 
-def attention_decode(q, k_new, v_new, k_cache, v_cache, position, num_heads):
+def attention_decode(q, k_new, v_new, k_cache, v_cache, position, num_heads,
+                     relative_bias=None):
   """One decoding step: q, k_new, v_new [B, H*D], the caches [B, Lm, H*D]
-  (UPDATED IN PLACE at row position[b]), position [B] int32 -> out [B, H*D]."""
+  (UPDATED IN PLACE at row position[b]), position [B] int32 -> out [B, H*D];
+  relative_bias = (values [H, NB], bucket [2 Lm - 1] int32) or None."""
   lib = load_library()
   b, hd = q.shape
   lm = k_cache.shape[1]
@@ -1185,8 +1187,9 @@ def attention_decode(q, k_new, v_new, k_cache, v_cache, position, num_heads):
         _dev(k_cache, "k_cache", q.dtype, (b, lm, hd)),
         _dev(v_cache, "v_cache", q.dtype, (b, lm, hd)),
         _dev(position, "position", torch.int32, (b,)), out.data_ptr(), b, lm,
-        num_heads, hd // num_heads, dtype_code(q.dtype), _stream()),
-        "attention_decode")
+        num_heads, hd // num_heads,
+        *_relative_bias_ptrs(relative_bias, q.dtype, num_heads, lm),
+        dtype_code(q.dtype), _stream()), "attention_decode")
   return out
 
 

@@ -292,11 +292,17 @@ class AttentionDecodeOperation(mtf.Operation):
   step, the recurrent states old_k, old_v [batch..., memory_length,
   heads * d_kv] and position [batch...] (int32) -> the attention outputs
   [batch..., heads * d_kv] and the updated states.  The states are new tensors
-  (the graph stays functional); the library call updates a copy in place."""
+  (the graph stays functional); the library call updates a copy in place.
+  relative_values [heads, buckets]: the relative attention bias of the memory
+  positions against the step's position (transformer_layers.py:317-352)."""
 
-  def __init__(self, q, k, v, old_k, old_v, position, num_heads, name=None):
+  def __init__(self, q, k, v, old_k, old_v, position, num_heads,
+               relative_values=None, relative_bidirectional=False, name=None):
     super(AttentionDecodeOperation, self).__init__(
-        [q, k, v, old_k, old_v, position], name=name or "attention_decode")
+        [q, k, v, old_k, old_v, position] + (
+            [] if relative_values is None else [relative_values]),
+        name=name or "attention_decode")
+    self._rel_bidirectional = bool(relative_bidirectional)
     if q.shape != k.shape or q.shape != v.shape or old_k.shape != old_v.shape:
       raise ValueError("q, k, v %s %s %s / states %s %s"
                        % (q.shape, k.shape, v.shape, old_k.shape, old_v.shape))
@@ -320,12 +326,17 @@ class AttentionDecodeOperation(mtf.Operation):
     channels, memory = q_sizes[-1], s_sizes[-2]
     heads = self._num_heads
 
-    def fn(q, k, v, old_k, old_v, position):
+    bidirectional = self._rel_bidirectional
+
+    def fn(q, k, v, old_k, old_v, position, *extra):
       q2, k2, v2 = (t.reshape(-1, channels).contiguous() for t in (q, k, v))
       kc = old_k.reshape(-1, memory, channels).clone()
       vc = old_v.reshape(-1, memory, channels).clone()
       pos = position.reshape(-1).to(torch.int32).contiguous()
-      out = moe_hip.attention_decode(q2, k2, v2, kc, vc, pos, heads)
+      _, rel = _attention_extras(extra, None, 3 if extra else None, memory,
+                                 bidirectional, q.dtype)
+      out = moe_hip.attention_decode(q2, k2, v2, kc, vc, pos, heads,
+                                     relative_bias=rel)
       return out.reshape(q_sizes), kc.reshape(s_sizes), vc.reshape(s_sizes)
     outs = mesh_impl.slicewise(fn, *[lowering.tensors[t] for t in self.inputs])
     for tensor, value in zip(self.outputs, outs):

@@ -139,9 +139,6 @@ class SelfAttention(transformer.TransformerLayer):
       k = params.compute_k(x)
       v = params.compute_v(x)
     relative_values = self.relative_bias_values(context, params.num_heads)
-    if relative_values is not None and context.mode in (
-        transformer.INCREMENTAL, transformer.FIRST_PART):
-      raise NotImplementedError("decoding with a relative attention bias")
     if context.mode == transformer.INCREMENTAL:
       # one position per batch entry: the step's key and value replace row
       # `position` of the recurrent states, the query sees the memory
@@ -154,7 +151,9 @@ class SelfAttention(transformer.TransformerLayer):
                                   "autoregressive")
       old_k, old_v = context.get_states(2)
       op = attention.AttentionDecodeOperation(
-          q, k, v, old_k, old_v, context.position, params.num_heads)
+          q, k, v, old_k, old_v, context.position, params.num_heads,
+          relative_values=relative_values,
+          relative_bidirectional=not context.model.fully_autoregressive)
       o, k_all, v_all = op.outputs
       context.record_new_states([k_all, v_all])
       return params.compute_output(o, output_shape=x.shape)

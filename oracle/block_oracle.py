@@ -202,7 +202,7 @@ def _attention_core(q, k, v, num_heads, causal, act_dtype, sequence_id=None,
 
 
 def attention_incremental(q, k_new, v_new, k_cache, v_cache, position,
-                          num_heads, act_dtype="float32"):
+                          num_heads, act_dtype="float32", relative_values=None):
   """One decoding step of SelfAttention ("incremental" mode,
   transformer/transformer_layers.py:231-254 and :289-296): the step's key and
   value replace row position[b] of the recurrent states
@@ -211,7 +211,11 @@ def attention_incremental(q, k_new, v_new, k_cache, v_cache, position,
   logits and softmax, weights cast to the activation dtype.
 
   q, k_new, v_new [B, H*D]; k_cache, v_cache [B, Lm, H*D]; position [B]
-  integers.  Returns (out [B, H*D], k [B, Lm, H*D], v [B, Lm, H*D])."""
+  integers.  relative_values [H, num_buckets]: the relative attention bias of
+  memory position m against the step's position (compute_bias with
+  context.position, transformer_layers.py:317-352; an autoregressive model's
+  buckets are not bidirectional, :321).
+  Returns (out [B, H*D], k [B, Lm, H*D], v [B, Lm, H*D])."""
   b, lm, hd = k_cache.shape
   d = hd // num_heads
   position = np.asarray(position).reshape(b)
@@ -226,7 +230,14 @@ def attention_incremental(q, k_new, v_new, k_cache, v_cache, position,
   k4, v4 = k.reshape(b, lm, num_heads, d), v.reshape(b, lm, num_heads, d)
   logits = np.einsum("bhd,bmhd->bhm", q4, k4).astype(F32)
   hidden = (np.arange(lm)[None, :] > position[:, None]).astype(F32)[:, None, :]
-  logits = (logits + hidden * F32(-1e9)).astype(F32)
+  bias = (hidden * F32(-1e9)).astype(F32)
+  if relative_values is not None:
+    values = _r(relative_values, act_dtype)
+    bucket = relative_position_bucket(
+        np.arange(lm)[None, :] - position[:, None], False, values.shape[-1])
+    rel = values[:, bucket].transpose(1, 0, 2)                   # [B, H, Lm]
+    bias = _r(_r(bias, act_dtype) + rel, act_dtype).astype(F32)
+  logits = (logits + bias).astype(F32)
   weights = _r(O.softmax(logits), act_dtype)
   out = _r(np.einsum("bhm,bmhd->bhd", weights, v4), act_dtype)
   return out.reshape(b, hd), k, v

@@ -135,6 +135,10 @@ def test_attention_incremental_is_a_row_of_causal_attention():
   q, k, v = (rng.standard_normal((b, l, heads * d)).astype(np.float32)
              for _ in range(3))
   full = B._attention_core(q, k, v, heads, True, "float32")
+  values = rng.standard_normal((heads, 8)).astype(np.float32)
+  full_rel = B._attention_core(q, k, v, heads, True, "float32",
+                               relative_values=values)
+  assert np.abs(full - full_rel).max() > 1e-2
   for p in ([0, 0], [5, 9], [11, 3]):
     kc, vc = k.copy(), v.copy()
     for i, pi in enumerate(p):
@@ -144,6 +148,11 @@ def test_attention_incremental_is_a_row_of_causal_attention():
     out, k2, v2 = B.attention_incremental(q[rows, p], k[rows, p], v[rows, p], kc,
                                           vc, np.array(p), heads)
     np.testing.assert_allclose(out, full[rows, p], rtol=1e-5, atol=1e-6)
+    # the same with a relative attention bias
+    out_rel = B.attention_incremental(q[rows, p], k[rows, p], v[rows, p], kc, vc,
+                                      np.array(p), heads,
+                                      relative_values=values)[0]
+    np.testing.assert_allclose(out_rel, full_rel[rows, p], rtol=1e-5, atol=1e-6)
     for i, pi in enumerate(p):
       np.testing.assert_array_equal(k2[i, :pi + 1], k[i, :pi + 1])
       np.testing.assert_array_equal(v2[i, :pi + 1], v[i, :pi + 1])

@@ -255,6 +255,19 @@ def test_attention_decode(hip, case, act_dtype):
     np.testing.assert_allclose(H.to_np(got), want, **tol)
     np.testing.assert_array_equal(H.to_np(kg), want_k)
     np.testing.assert_array_equal(H.to_np(vg), want_v)
+    # with a relative attention bias against the step's position
+    values = O.cast_act(rng.standard_normal((heads, 16)).astype(np.float32),
+                        act_dtype)
+    bucket = B.relative_position_bucket(np.arange(-(lm - 1), lm), False, 16)
+    want_rel = B.attention_incremental(q, kn, vn, kc, vc, pos, heads, act_dtype,
+                                       relative_values=values)[0]
+    got_rel = hip.attention_decode(
+        g(q), g(kn), g(vn), g(kc), g(vc), torch.from_numpy(pos).cuda(), heads,
+        relative_bias=(g(values),
+                       torch.from_numpy(bucket.astype(np.int32)).cuda()))
+    np.testing.assert_allclose(H.to_np(got_rel), want_rel, **tol)
+    if lm > 1 and pos.max() > 0:
+      assert np.abs(want_rel - want).max() > 1e-3
 
 
 @pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
@@ -520,15 +533,17 @@ def test_layer_stack_relative_attention_bias(kind, autoregressive):
     np.testing.assert_allclose(g, w, rtol=1e-3, atol=1e-3 * np.abs(w).max())
 
 
+@pytest.mark.parametrize("relative", [None, "bias_shared"])
 @pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
-def test_decoding_modes_match_the_full_forward(act_dtype):
+def test_decoding_modes_match_the_full_forward(act_dtype, relative):
   """Decoding as Unitransformer.sample_autoregressive drives it
   (transformer.py:1140-1248): "first_part" over a row whose positions from p0
   on are unknown (zeros) records every attention layer's keys and values; one
   "incremental" call per position p >= p0 takes the token of that position, the
   states and position [batch], and must give what the full forward gives at p
   (teacher forcing).  The experts' capacity is ample in both runs, so no token
-  is dropped in either."""
+  is dropped in either.  With relative = "bias_shared" the attention layers add
+  the first layer's relative attention bias in all three modes."""
   b, l, m, e, hdim, heads, d, group, p0 = 2, 24, 64, 4, 96, 4, 16, 32, 17
   dt = H.ACT_TORCH[act_dtype]
   rng = np.random.default_rng(61)
@@ -538,14 +553,15 @@ def test_decoding_modes_match_the_full_forward(act_dtype):
   mesh = mtf.Mesh(graph, "mesh")
   batch, length, model_dim = (mtf.Dimension("batch", b), mtf.Dimension("length", l),
                               mtf.Dimension("d_model", m))
+  att_kw = dict(num_heads=heads, key_value_size=d,
+                relative_attention_type=relative,
+                relative_attention_num_buckets=8)
   stack = transformer.make_layer_stack(
-      [(transformer_layers.SelfAttention,
-        dict(num_heads=heads, key_value_size=d)),
+      [(transformer_layers.SelfAttention, att_kw),
        (moe.MoE1D, dict(num_experts=e, hidden_size=hdim, group_size=group,
                         second_policy_train="all", second_policy_eval="all",
                         capacity_factor_eval=float(e))),
-       (transformer_layers.SelfAttention,
-        dict(num_heads=heads, key_value_size=d)),
+       (transformer_layers.SelfAttention, att_kw),
        (transformer_layers.DenseReluDense, dict(hidden_size=hdim))],
       num_layers=1, block_scope=False)
   model = transformer.Unitransformer(stack, d_model=m, name="decoder",
@@ -590,9 +606,15 @@ def test_decoding_modes_match_the_full_forward(act_dtype):
     else:
       init[prefix + "DenseReluDense/wi/kernel"] = layer["wi"]
       init[prefix + "DenseReluDense/wo/kernel"] = layer["wo"]
+  if relative:
+    init["decoder/layer_000/SelfAttention/relative_attention_bias"] = (
+        rng.standard_normal((heads, 8)).astype(np.float32))
   assert sorted(init) == sorted(v.name for v in graph.all_variables)
   lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()}, initial_values=init)
   want = H.to_np(lowering.export_to_tf_tensor(y_full))
+  if relative:     # the bias matters: the oracle without it is somewhere else
+    plain, _ = B.layer_stack(x, layers, final, act_dtype, True)
+    assert np.abs(plain - want).max() > 5e-2
   got_first = H.to_np(lowering.export_to_tf_tensor(y_first))
   tol = dict(rtol=2e-4, atol=2e-4) if act_dtype == "float32" else dict(
       rtol=5e-2, atol=5e-2)
