@@ -16,7 +16,8 @@ from mesh_amd import ops as mtf
 class AttentionParams(object):
   """The q, k, v, o kernels of multi-head attention (attention.py:345-591).
 
-  Variables "q", "k", "v" of shape [d_model, heads * d_kv] and "o" of shape
+  Variables "q", "k", "v" (with shared_kv: "q", "kv") of shape
+  [d_model, heads * d_kv] and "o" of shape
   [heads * d_kv, d_model]; the combined dim carries the name of its first
   member ("heads", attention.py:695-696).  Initialisers as the reference's
   without the unit-scaling convention (attention.py:436-443): q
@@ -34,9 +35,6 @@ class AttentionParams(object):
       raise NotImplementedError(
           "only the default attention parameters are implemented (combined "
           "dims, no ensemble)")
-    if shared_kv and make_attention_vars:
-      raise NotImplementedError(
-          "a shared \"kv\" kernel is only implemented for ExpertsAttention")
     if key_dim != value_dim:
       raise NotImplementedError("key_dim != value_dim")
     query_heads_dims = list(query_heads_dims or [])
@@ -72,12 +70,17 @@ class AttentionParams(object):
       self.wq = mtf.get_variable(mesh, "q", [query_input_dim, combined],
                                  initializer=normal(stddev),
                                  dtype=variable_dtype)
-      self.wk = mtf.get_variable(mesh, "k", [memory_input_dim, combined],
-                                 initializer=normal(kv_std),
-                                 dtype=variable_dtype)
-      self.wv = mtf.get_variable(mesh, "v", [memory_input_dim, combined],
-                                 initializer=normal(kv_std),
-                                 dtype=variable_dtype)
+      if shared_kv:                          # attention.py:453-459
+        self.wkv = mtf.get_variable(mesh, "kv", [memory_input_dim, combined],
+                                    initializer=normal(kv_std),
+                                    dtype=variable_dtype)
+      else:
+        self.wk = mtf.get_variable(mesh, "k", [memory_input_dim, combined],
+                                   initializer=normal(kv_std),
+                                   dtype=variable_dtype)
+        self.wv = mtf.get_variable(mesh, "v", [memory_input_dim, combined],
+                                   initializer=normal(kv_std),
+                                   dtype=variable_dtype)
     self.wo = mtf.get_variable(mesh, "o", [combined, output_dim],
                                initializer=normal(o_std), dtype=variable_dtype)
 
@@ -92,10 +95,20 @@ class AttentionParams(object):
       q = q * (self.key_dim.size ** -0.5)
     return q
 
+  def compute_kv(self, memory_antecedent):
+    """The tensor that serves as keys and as values (attention.py:499-515)."""
+    if not self.shared_kv:
+      raise ValueError("compute_kv can only be called with shared_kv")
+    return self._project(memory_antecedent, self.wkv, "kv_proj")
+
   def compute_k(self, memory_antecedent):
+    if self.shared_kv:
+      raise ValueError("compute_k cannot be called with shared_kv")
     return self._project(memory_antecedent, self.wk, "k_proj")
 
   def compute_v(self, memory_antecedent):
+    if self.shared_kv:
+      raise ValueError("compute_v cannot be called with shared_kv")
     return self._project(memory_antecedent, self.wv, "v_proj")
 
   def compute_output(self, o, output_shape=None):

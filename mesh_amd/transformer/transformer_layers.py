@@ -40,12 +40,11 @@ class DenseReluDense(transformer.TransformerLayer):
 
 
 class SelfAttention(transformer.TransformerLayer):
-  """Multi-head self-attention (transformer_layers.py:151-357): separate k and
-  v, combined dims, optionally the relative position bias of types "bias" and
-  "bias_shared".  Visibility comes from the context: read/write priorities
-  (autoregressive models), sequence ids, or none."""
-
-  _shared_kv_implemented = False     # a "kv" kernel of its own is not
+  """Multi-head self-attention (transformer_layers.py:151-357): combined dims,
+  separate k and v kernels or one for both (shared_kv), optionally the relative
+  position bias of types "bias" and "bias_shared".  Visibility comes from the
+  context: read/write priorities (autoregressive models), sequence ids, or
+  none."""
 
   def __init__(self, num_heads=8, num_memory_heads=0, key_value_size=128,
                shared_kv=False, dropout_rate=0.0, attention_kwargs=None,
@@ -54,8 +53,7 @@ class SelfAttention(transformer.TransformerLayer):
                combine_dims=True, keep_query_heads_dims=False,
                fold_scaling_into_initializer=True):
     if (num_memory_heads or attention_kwargs or attention_func is not None or
-        not combine_dims or keep_query_heads_dims or
-        (shared_kv and not self._shared_kv_implemented)):
+        not combine_dims or keep_query_heads_dims):
       raise NotImplementedError(
           "only the default SelfAttention options are implemented")
     if relative_attention_type == "contextual":
@@ -143,27 +141,27 @@ class SelfAttention(transformer.TransformerLayer):
       # one position per batch entry: the step's key and value replace row
       # `position` of the recurrent states, the query sees the memory
       # positions up to it (transformer_layers.py:239-254, :289-296)
-      if sequence_id is not None or self.shared_kv:
-        raise NotImplementedError(
-            "incremental mode with sequence ids or shared_kv")
+      if sequence_id is not None:
+        raise NotImplementedError("incremental mode with sequence ids")
       if context.read_priority is not transformer.POSITION:
         raise NotImplementedError("incremental mode of a model that is not "
                                   "autoregressive")
-      old_k, old_v = context.get_states(2)
+      if self.shared_kv:                     # one state: the shared tensor
+        old_k = old_v = context.get_states(1)[0]
+      else:
+        old_k, old_v = context.get_states(2)
       op = attention.AttentionDecodeOperation(
           q, k, v, old_k, old_v, context.position, params.num_heads,
           relative_values=relative_values,
           relative_bidirectional=not context.model.fully_autoregressive)
       o, k_all, v_all = op.outputs
-      context.record_new_states([k_all, v_all])
+      context.record_new_states([k_all] if self.shared_kv else [k_all, v_all])
       return params.compute_output(o, output_shape=x.shape)
     if context.mode == transformer.FIRST_PART:
-      if self.shared_kv:
-        raise NotImplementedError("first_part mode with shared_kv")
       name = context.length_dim.name       # states carry "memory_length"
       context.record_new_states(
-          [mtf.rename_dimension(k, name, "memory_length"),
-           mtf.rename_dimension(v, name, "memory_length")])
+          [mtf.rename_dimension(t, name, "memory_length")
+           for t in ([k] if self.shared_kv else [k, v])])
     # read_priority >= write_priority (transformer_layers.py:289-296)
     causal = context.read_priority is transformer.POSITION
     if context.train and self.dropout_rate != 0.0:
@@ -184,8 +182,6 @@ class ExpertsSelfAttention(SelfAttention):
   must be passed, as to the reference's.  Variables under the layer's scope:
   the experts layer's "<router>_gating/kernel", "wi/kernel", "q_wo/kernel",
   "k_wo/kernel" and the attention output kernel "o"."""
-
-  _shared_kv_implemented = True      # the keys the experts compute are the values
 
   def __init__(self, num_experts=16, loss_coef=1e-2, group_size=1024,
                capacity_factor_train=1.25, capacity_factor_eval=2.0,

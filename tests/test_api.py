@@ -494,6 +494,32 @@ def test_relative_attention_bias_variables(kind):
   assert got == want
 
 
+def test_shared_kv_variables():
+  """SelfAttention(shared_kv=True): one kernel "kv" in place of "k" and "v"
+  (attention.py:453-459); one recurrent state per layer in the decoding modes
+  (transformer_layers.py:244-258)."""
+  from mesh_amd.transformer import transformer, transformer_layers
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  dims = [mtf.Dimension("batch", 2), mtf.Dimension("length", 16),
+          mtf.Dimension("d_model", 32)]
+  x = mtf.import_tf_tensor(mesh, torch.zeros(2, 16, 32), mtf.Shape(dims))
+  stack = transformer.make_layer_stack(
+      [(transformer_layers.SelfAttention,
+        dict(num_heads=4, key_value_size=8, shared_kv=True))],
+      num_layers=2, block_scope=False)
+  model = transformer.Unitransformer(stack, d_model=32, name="decoder",
+                                     autoregressive=True)
+  states = []
+  model.call_layers(x, mtf.VariableDType(torch.float32), mode="first_part",
+                    new_states=states)
+  assert len(states) == 2
+  names = sorted(v.name for v in graph.all_variables
+                 if "layer_000/SelfAttention" in v.name)
+  assert names == ["decoder/layer_000/SelfAttention/" + n
+                   for n in ("kv", "o", "q")]
+
+
 def test_relative_position_bucket_matches_the_oracle():
   """The host-side bucket table of the product against the oracle's
   restatement of _relative_position_bucket (transformer_layers.py:1000-1042),
@@ -540,7 +566,7 @@ def test_block_rejections():
   with pytest.raises(ValueError, match="unrecognized"):
     transformer_layers.SelfAttention(relative_attention_type="nope")
   with pytest.raises(NotImplementedError):
-    transformer_layers.SelfAttention(shared_kv=True)
+    transformer_layers.SelfAttention(num_memory_heads=2)
   graph = mtf.Graph()
   mesh = mtf.Mesh(graph, "mesh")
   dims = [mtf.Dimension("batch", 1), mtf.Dimension("length", 8),

@@ -533,9 +533,11 @@ def test_layer_stack_relative_attention_bias(kind, autoregressive):
     np.testing.assert_allclose(g, w, rtol=1e-3, atol=1e-3 * np.abs(w).max())
 
 
-@pytest.mark.parametrize("relative", [None, "bias_shared"])
+@pytest.mark.parametrize("relative,shared_kv", [(None, False),
+                                                ("bias_shared", False),
+                                                ("bias_shared", True)])
 @pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
-def test_decoding_modes_match_the_full_forward(act_dtype, relative):
+def test_decoding_modes_match_the_full_forward(act_dtype, relative, shared_kv):
   """Decoding as Unitransformer.sample_autoregressive drives it
   (transformer.py:1140-1248): "first_part" over a row whose positions from p0
   on are unknown (zeros) records every attention layer's keys and values; one
@@ -553,7 +555,11 @@ def test_decoding_modes_match_the_full_forward(act_dtype, relative):
   mesh = mtf.Mesh(graph, "mesh")
   batch, length, model_dim = (mtf.Dimension("batch", b), mtf.Dimension("length", l),
                               mtf.Dimension("d_model", m))
-  att_kw = dict(num_heads=heads, key_value_size=d,
+  if shared_kv:          # one kernel for keys and values, one state per layer
+    for layer in layers:
+      if layer["kind"] == "attention":
+        layer["wv"] = layer["wk"]
+  att_kw = dict(num_heads=heads, key_value_size=d, shared_kv=shared_kv,
                 relative_attention_type=relative,
                 relative_attention_num_buckets=8)
   stack = transformer.make_layer_stack(
@@ -577,7 +583,7 @@ def test_decoding_modes_match_the_full_forward(act_dtype, relative):
   states = []
   y_first, _ = model.call_layers(first_in, vdt, mode="first_part",
                                  new_states=states, reuse=True)
-  assert len(states) == 4
+  assert len(states) == (2 if shared_kv else 4)
   assert all(t.shape.dimension_names == ["batch", "memory_length", "heads"]
              for t in states)
   steps = []
@@ -597,8 +603,8 @@ def test_decoding_modes_match_the_full_forward(act_dtype, relative):
     prefix = "decoder/layer_%03d/" % i
     init[prefix + "rms_norm/scale"] = layer["scale"]
     if layer["kind"] == "attention":
-      for c in "qkvo":
-        init[prefix + "SelfAttention/" + c] = layer["w" + c]
+      for c in ("q", "kv", "o") if shared_kv else "qkvo":
+        init[prefix + "SelfAttention/" + c] = layer["w" + c[0]]
     elif layer["kind"] == "moe":
       init[prefix + "MoE1D/top_2_gating/kernel"] = layer["w_gate"]
       init[prefix + "MoE1D/wi/kernel"] = layer["wi"]
@@ -612,9 +618,21 @@ def test_decoding_modes_match_the_full_forward(act_dtype, relative):
   assert sorted(init) == sorted(v.name for v in graph.all_variables)
   lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()}, initial_values=init)
   want = H.to_np(lowering.export_to_tf_tensor(y_full))
-  if relative:     # the bias matters: the oracle without it is somewhere else
+  if act_dtype == "float32":
+    # the full forward is the oracle's (same ample capacity for the experts)
+    layers[1]["hparams"] = O.default_hparams(
+        moe_num_experts=e, moe_hidden_size=hdim, moe_group_size=group,
+        moe_second_policy_eval="all", moe_second_policy_train="all",
+        moe_capacity_factor_eval=float(e))
     plain, _ = B.layer_stack(x, layers, final, act_dtype, True)
-    assert np.abs(plain - want).max() > 5e-2
+    if relative:   # the bias matters: the oracle without it is somewhere else
+      assert np.abs(plain - want).max() > 5e-2
+      for layer in layers:
+        if layer["kind"] == "attention":
+          layer["relative_values"] = init[
+              "decoder/layer_000/SelfAttention/relative_attention_bias"]
+    oracle_full, _ = B.layer_stack(x, layers, final, act_dtype, True)
+    np.testing.assert_allclose(want, oracle_full, rtol=2e-4, atol=2e-4)
   got_first = H.to_np(lowering.export_to_tf_tensor(y_first))
   tol = dict(rtol=2e-4, atol=2e-4) if act_dtype == "float32" else dict(
       rtol=5e-2, atol=5e-2)
