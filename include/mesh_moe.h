@@ -733,8 +733,8 @@ size_t mesh_moe_self_attention_workspace_bytes(int B, int L, int H, int D,
  *   combine_dims does); any L and D (bf16 shapes whose L or D is not a
  *   multiple of 8 run their two products on a plain tile kernel).
  * bf16 with D = 64 or 128 runs one fused kernel (logits stay on chip, the
- * division by the softmax sum comes after the weights are rounded; workspace =
- * a transposed copy of v).  Other cases run the three-step form whose logits
+ * division by the softmax sum comes after the weights are rounded; no scratch
+ * but the bias table below).  Other cases run the three-step form whose logits
  * and weights of all heads live in the workspace (B*H*L*L*(4 + sizeof dtype)
  * bytes).
  * sequence_id [B,L] int32 or NULL: with it a query sees only the keys that
