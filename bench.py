@@ -465,7 +465,23 @@ def main():
     result["config"].update(kept_pairs=kept, slots=slots,
                             capacity=r.capacity)
   else:
-    result["roofline"] = None
+    # hierarchical layer: the expert FFN runs on the inner level's slots (the
+    # last routing of a step), two launches of the grouped GEMM as in v1
+    r = routings[-1]
+    kept = int(r.fill.sum().item())
+    slots = r.fill.numel() * r.capacity
+    m, h = cfg["M"], cfg["H"]
+    ffn_ms = stages["expert_ffn"][1] / args.steps
+    peak = MFMA_PEAK_TFLOPS[cfg["dtype"]]
+    flops_per_launch = 2.0 * kept * m * h
+    achieved = flops_per_launch / (ffn_ms / 2 * 1e-3) / 1e12
+    result["roofline"] = {
+        "kernel": "grouped expert GEMM (expert_ffn, 2 launches/step)",
+        "bound": "mfma", "achieved": achieved, "peak": peak,
+        "unit": "TFLOP/s", "frac": achieved / peak, "traffic": None,
+        "flops_per_launch": flops_per_launch, "avg_launch_ms": ffn_ms / 2,
+        "padded_frac": (2.0 * slots * m * h / (ffn_ms / 2 * 1e-3) / 1e12) / peak}
+    result["config"].update(kept_pairs=kept, slots=slots, capacity=r.capacity)
     result["stages"] = {k: {"ms_per_step": v[1] / args.steps,
                             "launches_per_step": v[0] / args.steps}
                         for k, v in stages.items()}
