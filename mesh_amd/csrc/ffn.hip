@@ -609,8 +609,21 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
     if constexpr (LISTED) logical = tile_list[logical];
     const int e = logical / tiles_per_e;
     const int rem = logical - e * tiles_per_e;
-    const int tn = rem / tiles_m;
-    const int tm = rem - tn * tiles_m;
+    int tn = rem / tiles_m;
+    int tm = rem - tn * tiles_m;
+    if (!LISTED && tiles_m > 8 && (tiles_m & 7) == 0 && (tiles_n & 3) == 0) {
+      // 32 consecutive logical tiles (what an XCD holds at any moment) form a
+      // block of 8 row tiles x 4 column tiles: 12 operand panels for 32 tiles.
+      // With the plain order and many row tiles they would be 32 row tiles of
+      // one column tile: 33 panels, every row panel fetched once per column
+      // tile.  Blocks follow each other along N, so the next 32 tiles share
+      // the 8 row panels.  (8 row tiles: both orders are the same.)
+      const int sup = rem >> 5, within = rem & 31;
+      const int per_row = tiles_n >> 2;
+      const int sm = sup / per_row, sn = sup - sm * per_row;
+      tm = sm * 8 + (within & 7);
+      tn = sn * 4 + (within >> 3);
+    }
     row0 = tm * BM;
     col0 = tn * BN;
     Ae = GATHER ? A : A + (int64_t)e * R * K;
