@@ -1039,6 +1039,34 @@ def test_expert_ffn_backward_weight_gradients_bf16(hip, shape):
                                atol=1e-2 * scale, err_msg=name)
 
 
+@pytest.mark.parametrize("shape", [(1, 4096, 256, 1024), (2, 6144, 128, 2048),
+                                   (1, 4096 + 256, 128, 1024),
+                                   (1, 512, 4096, 1024)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_expert_linear_many_row_tiles(hip, shape):
+  """More than 8 row tiles of 256 per group (the dense layers of a transformer
+  block: one group, every token a row): the tile order that keeps an XCD's
+  resident tiles in blocks of 8 x 4, and a row-tile count that does not divide
+  by 8 (plain order); forward and the weight gradient (row tiles = the columns
+  of the first operand there) against float32 matmuls."""
+  e, rows, k, n = shape
+  rng = np.random.default_rng(sum(shape))
+  g = lambda a: H.to_gpu(O.cast_act(a.astype(np.float32), "bfloat16"), "bfloat16")
+  a = g(rng.standard_normal((e, rows, k)))
+  w = g(H.normal_weights(rng, (e, k, n), k))
+  dy = g(rng.standard_normal((e, rows, n)))
+  y = hip.expert_linear(a, hip.pack_weights(w, torch.bfloat16))
+  want = torch.bmm(a.float(), w.float())
+  np.testing.assert_allclose(H.to_np(y), H.to_np(want), rtol=2e-2,
+                             atol=1e-2 * float(want.abs().max()))
+  da, dw = hip.expert_linear_backward(a, dy, w)
+  want_da = torch.bmm(dy.float(), w.float().transpose(1, 2))
+  want_dw = torch.bmm(a.float().transpose(1, 2), dy.float())
+  for got, wnt, name in ((da, want_da, "da"), (dw, want_dw, "dw")):
+    np.testing.assert_allclose(H.to_np(got), H.to_np(wnt), rtol=2e-2,
+                               atol=1e-2 * float(wnt.abs().max()), err_msg=name)
+
+
 @pytest.mark.parametrize("size", [(8, 512, 1024, 4096), (8, 2048, 4096, 16384)],
                          ids=["cfg3_slice", "cfg4_slice"])
 def test_full_size_ffn_backward_properties(hip, size):
