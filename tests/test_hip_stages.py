@@ -225,6 +225,35 @@ def test_rejects_bad_arguments(hip):
                       torch.zeros((9, 2), device="cuda"))
 
 
+def test_gating_hand_worked_case(hip):
+  """One group, S = 6, E = 3, C = 2, worked by hand from
+  transformer/moe.py:1472-1496 (no oracle involved): first choices in token
+  order, then second choices behind the kept first ones; token 3 loses both
+  choices; the loss from its definition (:1420-1442) in float64."""
+  idx1 = [0, 0, 1, 0, 2, 1]
+  idx2 = [1, 2, 0, 1, 0, 0]
+  logits = np.zeros((1, 6, 3), np.float32)
+  for t, (a, b) in enumerate(zip(idx1, idx2)):
+    logits[0, t, a], logits[0, t, b] = 5.0, 3.0
+  got = H.routing_to_np(hip.top2_gating(torch.from_numpy(logits).cuda(), 2))
+  np.testing.assert_array_equal(got["index_1"][0], idx1)
+  np.testing.assert_array_equal(got["index_2"][0], idx2)
+  np.testing.assert_array_equal(got["pos_1"][0], [0, 1, 0, 2, 0, 1])
+  np.testing.assert_array_equal(got["kept_1"][0], [1, 1, 1, 0, 1, 1])
+  np.testing.assert_array_equal(got["pos_2"][0], [2, 1, 2, 3, 3, 4])
+  np.testing.assert_array_equal(got["kept_2"][0], [0, 1, 0, 0, 0, 0])
+  np.testing.assert_array_equal(got["fill"][0], [2, 2, 2])
+  e = np.exp(np.array([5.0, 3.0, 0.0]))
+  g1, g2 = e[0] / (e[0] + e[1]), e[1] / (e[0] + e[1])   # normalised top-2 gates
+  np.testing.assert_allclose(got["gate_1"][0], [g1, g1, g1, 0, g1, g1], rtol=1e-5)
+  np.testing.assert_allclose(got["gate_2"][0], [0, g2, 0, 0, 0, 0], rtol=1e-5)
+  prob = np.exp(logits[0].astype(np.float64))
+  prob /= prob.sum(-1, keepdims=True)
+  density = np.array([3, 2, 1]) / 6.0               # first choices, before drops
+  want_loss = (prob.mean(0) * density).mean() * 9
+  np.testing.assert_allclose(got["loss"], want_loss, rtol=2e-5)
+
+
 def test_gating_golden_fixture(hip):
   """The committed golden vectors (tests/golden/top2_gating_small.json)."""
   import json
