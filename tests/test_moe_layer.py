@@ -90,6 +90,48 @@ def test_v1_matches_oracle(case):
                              rtol=1e-2 if act_dtype == "bfloat16" else 1e-5)
 
 
+def test_v1_closed_form_layer():
+  """A layer whose output has a closed form, no oracle involved: expert e
+  multiplies by a_e > 0 (wi_e = a_e I, wo_e = I), the router reads the first E
+  channels, capacity is ample, so
+    out[t] = (g1 a_i1 + g2 a_i2) relu(x[t])
+  with (i1, i2) the two largest routing channels of the token and g the top-2
+  softmax gates normalised by their sum (moe.py:1397-1415, :509-510), and
+    loss = coef E^2 mean_{group, e}(mean_s p . mean_s [i1 = e])   (:1420-1442).
+  Evaluated in float64."""
+  b, l, m, e, group = 2, 32, 16, 4, 32
+  rng = np.random.default_rng(7)
+  a = np.array([0.5, 1.0, 1.5, 2.0])
+  eye = np.eye(m, dtype=np.float32)
+  w_gate = np.zeros((m, e), np.float32)
+  w_gate[:e] = 2.0 * np.eye(e)
+  w = dict(w_gate=w_gate, wi=np.stack([a_e * eye for a_e in a]).astype(np.float32),
+           wo=np.stack([eye] * e))
+  x = rng.standard_normal((b, l, m)).astype(np.float32)
+  # routing channels: a permutation of well separated levels per token
+  levels = np.array([1.5, 0.9, 0.3, -0.3], np.float32)
+  for bi in range(b):
+    for t in range(l):
+      x[bi, t, :e] = rng.permutation(levels)
+  hp, _ = make_hparams(moe_num_experts=e, moe_hidden_size=m, moe_group_size=group,
+                       moe_capacity_factor_eval=float(e))
+  got, got_loss, _, _ = run_v1(x, w, hp, False, "float32")
+  logits = 2.0 * x[..., :e].astype(np.float64)
+  prob = np.exp(logits - logits.max(-1, keepdims=True))
+  prob /= prob.sum(-1, keepdims=True)
+  order = np.argsort(-logits, axis=-1)
+  i1, i2 = order[..., 0], order[..., 1]
+  p1 = np.take_along_axis(prob, i1[..., None], -1)[..., 0]
+  p2 = np.take_along_axis(prob, i2[..., None], -1)[..., 0]
+  g1, g2 = p1 / (p1 + p2 + 1e-9), p2 / (p1 + p2 + 1e-9)
+  want = (g1 * a[i1] + g2 * a[i2])[..., None] * np.maximum(x.astype(np.float64), 0)
+  np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-6)
+  # groups are the batch rows here (group size = length)
+  density = np.stack([(i1 == k).mean(-1) for k in range(e)], -1)     # [b, e]
+  want_loss = 1e-2 * e * e * (prob.mean(1) * density).mean()
+  np.testing.assert_allclose(got_loss, want_loss, rtol=1e-5)
+
+
 def test_v1_skewed_routing_drops_tokens():
   """Capacity factor 1.0 with a Zipf-biased router (folded into the router
   weights through a constant input column) overflows the popular experts."""
