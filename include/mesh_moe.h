@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 24
+#define MESH_MOE_ABI_VERSION 25
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -750,13 +750,18 @@ size_t mesh_moe_self_attention_workspace_bytes(int B, int L, int H, int D,
  * relative_bias = 1 to mesh_moe_self_attention_workspace_bytes; the fused
  * kernel reads the bias from a float32 table [H, 2L-1] it first builds in the
  * workspace.  mesh_moe_attention_weights takes the same arguments.
+ * lse [B*H,L] float32 or NULL: where the fused kernel runs
+ * (mesh_moe_self_attention_backward_workspace_bytes > 0 for the shape) it also
+ * writes the logarithm of every query's softmax denominator, which
+ * mesh_moe_self_attention_backward takes back; MESH_MOE_E_UNSUPPORTED where
+ * the three-step form runs.
  */
 int mesh_moe_self_attention(const void* q, const void* k, const void* v,
                             void* out, int B, int L, int H, int D, int causal,
                             const int32_t* sequence_id, const void* rel_values,
                             const int32_t* rel_bucket, int num_buckets,
-                            int dtype, void* workspace, size_t workspace_bytes,
-                            void* stream);
+                            float* lse, int dtype, void* workspace,
+                            size_t workspace_bytes, void* stream);
 
 /*
  * Gradient of the relative attention bias values (the gradient of the
@@ -803,6 +808,10 @@ size_t mesh_moe_self_attention_backward_workspace_bytes(int B, int L, int H,
  * (float32, before the cast) along the diagonals into a float32 table
  * [H, 2L-1] with atomics -- the order of that sum is not fixed -- and a last
  * small kernel adds up each bucket's distances.
+ * out [B,L,H*D] dtype and lse [B*H,L] float32 (both or neither): what
+ * mesh_moe_self_attention wrote for the same arguments.  With them the first
+ * of the four launches is replaced by a small one (delta = sum_d dout out from
+ * the rounded outputs); without them the denominators are recomputed.
  */
 int mesh_moe_self_attention_backward(const void* q, const void* k, const void* v,
                                      const void* dout, void* dq, void* dk,
@@ -810,8 +819,10 @@ int mesh_moe_self_attention_backward(const void* q, const void* k, const void* v
                                      int causal, const int32_t* sequence_id,
                                      const void* rel_values,
                                      const int32_t* rel_bucket, int num_buckets,
-                                     void* dvalues, int dtype, void* workspace,
-                                     size_t workspace_bytes, void* stream);
+                                     void* dvalues, const void* out,
+                                     const float* lse, int dtype,
+                                     void* workspace, size_t workspace_bytes,
+                                     void* stream);
 
 /*
  * One decoding step of self-attention: SelfAttention.call in "incremental"

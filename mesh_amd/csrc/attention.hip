@@ -436,6 +436,9 @@ __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
     return;
   }
   if (my_q < L) {
+    // (for a later backward pass that then needs no pass of its own for it)
+    if (lse != nullptr && half == 0)
+      lse[(int64_t)bh * L + my_q] = m_run + logf(l_all);
     bf16_t* orow = ob + (int64_t)my_q * row_stride;
 #pragma unroll
     for (int dt = 0; dt < Cfg::DT; ++dt) {
@@ -456,14 +459,14 @@ __global__ __launch_bounds__(256, 2) void flash_attention_kernel(
 template <int D, bool CAUSAL, bool SEQ, bool BIAS>
 static int launch_flash_one(const bf16_t* q, const bf16_t* k, const bf16_t* v,
                             bf16_t* out, int B, int L, int H,
-                            const int32_t* seq, const float* tab,
+                            const int32_t* seq, const float* tab, float* lse,
                             hipStream_t st) {
   using Cfg = FlashCfg<D>;
   constexpr int LDS = Cfg::LDS_BYTES + 512 + 1536;  // + key ids, bias windows
   dim3 grid((unsigned)((L + Cfg::BQ - 1) / Cfg::BQ), (unsigned)(B * H));
   auto kern = flash_attention_kernel<D, CAUSAL, false, SEQ, BIAS>;
   MOE_ALLOW_LDS(kern, LDS);
-  kern<<<grid, Cfg::THREADS, LDS, st>>>(q, k, v, out, L, H, nullptr, nullptr,
+  kern<<<grid, Cfg::THREADS, LDS, st>>>(q, k, v, out, L, H, nullptr, lse,
                                         nullptr, seq, tab);
   MOE_CHECK_LAUNCH("self_attention (fused)");
   return 0;
@@ -484,12 +487,13 @@ static int flash_dispatch(bool causal, bool seq, bool bias, F&& f) {
 template <int D>
 static int launch_flash(const bf16_t* q, const bf16_t* k, const bf16_t* v,
                         bf16_t* out, int B, int L, int H, int causal,
-                        const int32_t* seq, const float* tab, hipStream_t st) {
+                        const int32_t* seq, const float* tab, float* lse,
+                        hipStream_t st) {
   return flash_dispatch(causal != 0, seq != nullptr, tab != nullptr,
                         [&](auto c, auto s, auto bi) {
     return launch_flash_one<D, decltype(c)::value, decltype(s)::value,
                             decltype(bi)::value>(q, k, v, out, B, L, H, seq, tab,
-                                                 st);
+                                                 lse, st);
   });
 }
 
@@ -537,8 +541,8 @@ size_t flash_attention_workspace_bytes(int B, int L, int H, int D,
 int flash_attention(const void* q, const void* k, const void* v, void* out,
                     int B, int L, int H, int D, int causal,
                     const int32_t* sequence_id, const void* rel_values,
-                    const int32_t* rel_bucket, int num_buckets, void* workspace,
-                    hipStream_t st) {
+                    const int32_t* rel_bucket, int num_buckets, float* lse,
+                    void* workspace, hipStream_t st) {
   float* tab = nullptr;
   if (rel_values != nullptr) {
     tab = (float*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
@@ -549,9 +553,10 @@ int flash_attention(const void* q, const void* k, const void* v, void* out,
   if (D == 128)
     return launch_flash<128>((const bf16_t*)q, (const bf16_t*)k,
                              (const bf16_t*)v, (bf16_t*)out, B, L, H, causal,
-                             sequence_id, tab, st);
+                             sequence_id, tab, lse, st);
   return launch_flash<64>((const bf16_t*)q, (const bf16_t*)k, (const bf16_t*)v,
-                          (bf16_t*)out, B, L, H, causal, sequence_id, tab, st);
+                          (bf16_t*)out, B, L, H, causal, sequence_id, tab, lse,
+                          st);
 }
 
 // ---------------------------------------------------------------------------
@@ -1016,20 +1021,13 @@ static int launch_flash_backward_one(const bf16_t* q, const bf16_t* k,
 }
 
 template <int D, bool CAUSAL, bool SEQ, bool BIAS>
-static int launch_flash_backward(const bf16_t* q, const bf16_t* k,
-                                 const bf16_t* v, const bf16_t* dout,
-                                 bf16_t* dq, bf16_t* dk, bf16_t* dv, float* lse,
-                                 float* delta, int B, int L, int H,
-                                 const int32_t* seq, const float* tab,
-                                 float* dtab, hipStream_t st) {
-  using Cfg = FlashCfg<D>;
-  constexpr int LDS = Cfg::LDS_BYTES + 512 + 1536;
-  dim3 grid((unsigned)((L + Cfg::BQ - 1) / Cfg::BQ), (unsigned)(B * H));
-  auto stats = flash_attention_kernel<D, CAUSAL, true, SEQ, BIAS>;
-  MOE_ALLOW_LDS(stats, LDS);
-  stats<<<grid, Cfg::THREADS, LDS, st>>>(q, k, v, nullptr, L, H, dout, lse,
-                                         delta, seq, tab);
-  MOE_CHECK_LAUNCH("self_attention_backward (lse, delta)");
+static int launch_flash_backward_three(const bf16_t* q, const bf16_t* k,
+                                       const bf16_t* v, const bf16_t* dout,
+                                       bf16_t* dq, bf16_t* dk, bf16_t* dv,
+                                       const float* lse, const float* delta,
+                                       int B, int L, int H, const int32_t* seq,
+                                       const float* tab, float* dtab,
+                                       hipStream_t st) {
   int rc = launch_flash_backward_one<D, CAUSAL, BWD_DV, SEQ, BIAS>(
       q, k, v, dout, lse, delta, dv, B, L, H, seq, tab, dtab, st);
   if (rc != 0) return rc;
@@ -1038,6 +1036,70 @@ static int launch_flash_backward(const bf16_t* q, const bf16_t* k,
   if (rc != 0) return rc;
   return launch_flash_backward_one<D, CAUSAL, BWD_DQ, SEQ, BIAS>(
       q, k, v, dout, lse, delta, dq, B, L, H, seq, tab, dtab, st);
+}
+
+// delta[b * H + h][q] = sum_d dout . out for the rows of [B, L, H * D] tensors:
+// 16 lanes per (row, head), 16 bytes per lane and 16-byte step.
+template <int D>
+__global__ __launch_bounds__(256) void attention_delta_kernel(
+    const bf16_t* __restrict__ dout, const bf16_t* __restrict__ out,
+    float* __restrict__ delta, int64_t rows_heads, int L, int H) {
+  const int64_t item = ((int64_t)blockIdx.x * 256 + threadIdx.x) >> 4;
+  const int sub = threadIdx.x & 15;
+  float sum = 0.f;
+  if (item < rows_heads) {
+    const bf16_t* a = dout + item * D;
+    const bf16_t* b = out + item * D;
+#pragma unroll
+    for (int c = sub * 8; c < D; c += 128) {
+      const uint4 x = load_streaming(reinterpret_cast<const uint4*>(a + c));
+      const uint4 y = load_streaming(reinterpret_cast<const uint4*>(b + c));
+      float fx[8], fy[8];
+      unpack16(x, fx, bf16_t());
+      unpack16(y, fy, bf16_t());
+#pragma unroll
+      for (int u = 0; u < 8; ++u) sum = fmaf(fx[u], fy[u], sum);
+    }
+  }
+#pragma unroll
+  for (int off = 8; off >= 1; off >>= 1) sum += __shfl_xor(sum, off);
+  if (item < rows_heads && sub == 0) {
+    const int64_t row = item / H;               // b * L + q
+    const int h = (int)(item - row * H);
+    const int64_t b = row / L, qi = row - b * L;
+    delta[(b * H + h) * L + qi] = sum;
+  }
+}
+
+// lse_saved / out_saved: the forward pass's softmax denominators and outputs
+// when the caller kept them; otherwise a pass in the forward kernel's shape
+// recomputes the denominators (and delta from the unrounded outputs).
+template <int D, bool CAUSAL, bool SEQ, bool BIAS>
+static int launch_flash_backward(const bf16_t* q, const bf16_t* k,
+                                 const bf16_t* v, const bf16_t* dout,
+                                 bf16_t* dq, bf16_t* dk, bf16_t* dv, float* lse,
+                                 float* delta, int B, int L, int H,
+                                 const int32_t* seq, const float* tab,
+                                 float* dtab, const bf16_t* out_saved,
+                                 const float* lse_saved, hipStream_t st) {
+  using Cfg = FlashCfg<D>;
+  if (out_saved != nullptr) {
+    const int64_t items = (int64_t)B * L * H;
+    attention_delta_kernel<D><<<(unsigned)((items * 16 + 255) / 256), 256, 0,
+                                st>>>(dout, out_saved, delta, items, L, H);
+    MOE_CHECK_LAUNCH("self_attention_backward (delta)");
+  } else {
+    constexpr int LDS = Cfg::LDS_BYTES + 512 + 1536;
+    dim3 grid((unsigned)((L + Cfg::BQ - 1) / Cfg::BQ), (unsigned)(B * H));
+    auto stats = flash_attention_kernel<D, CAUSAL, true, SEQ, BIAS>;
+    MOE_ALLOW_LDS(stats, LDS);
+    stats<<<grid, Cfg::THREADS, LDS, st>>>(q, k, v, nullptr, L, H, dout, lse,
+                                           delta, seq, tab);
+    MOE_CHECK_LAUNCH("self_attention_backward (lse, delta)");
+  }
+  const float* lse_use = out_saved != nullptr ? lse_saved : lse;
+  return launch_flash_backward_three<D, CAUSAL, SEQ, BIAS>(
+      q, k, v, dout, dq, dk, dv, lse_use, delta, B, L, H, seq, tab, dtab, st);
 }
 
 __global__ void fill_zero_kernel(float* __restrict__ p, int64_t n) {
@@ -1073,7 +1135,9 @@ int flash_attention_backward(const void* q, const void* k, const void* v,
                              int B, int L, int H, int D, int causal,
                              const int32_t* sequence_id, const void* rel_values,
                              const int32_t* rel_bucket, int num_buckets,
-                             void* dvalues, void* workspace, hipStream_t st) {
+                             void* dvalues, const void* out_saved,
+                             const float* lse_saved, void* workspace,
+                             hipStream_t st) {
   const size_t per = (((size_t)B * H * L * sizeof(float) + 255) & ~(size_t)255) /
                      sizeof(float);
   float* lse = (float*)(((uintptr_t)workspace + 255) & ~(uintptr_t)255);
@@ -1101,10 +1165,10 @@ int flash_attention_backward(const void* q, const void* k, const void* v,
         if (D == 128)
           return launch_flash_backward<128, C, S, BI>(
               q_, k_, v_, d_, dq_, dk_, dv_, lse, delta, B, L, H, sequence_id,
-              tab, dtab, st);
-        return launch_flash_backward<64, C, S, BI>(q_, k_, v_, d_, dq_, dk_, dv_,
-                                                   lse, delta, B, L, H,
-                                                   sequence_id, tab, dtab, st);
+              tab, dtab, (const bf16_t*)out_saved, lse_saved, st);
+        return launch_flash_backward<64, C, S, BI>(
+            q_, k_, v_, d_, dq_, dk_, dv_, lse, delta, B, L, H, sequence_id, tab,
+            dtab, (const bf16_t*)out_saved, lse_saved, st);
       });
   if (rc != 0 || rel_values == nullptr) return rc;
   relative_table_backward_kernel<<<dim3((unsigned)num_buckets, (unsigned)H), 64,

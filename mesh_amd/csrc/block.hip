@@ -967,7 +967,7 @@ extern "C" int mesh_moe_self_attention(const void* q, const void* k,
                                        const int32_t* sequence_id,
                                        const void* rel_values,
                                        const int32_t* rel_bucket,
-                                       int num_buckets, int dtype,
+                                       int num_buckets, float* lse, int dtype,
                                        void* workspace, size_t workspace_bytes,
                                        void* stream) {
   MOE_REQUIRE(q && k && v && out && workspace, MESH_MOE_E_ARG,
@@ -996,8 +996,11 @@ extern "C" int mesh_moe_self_attention(const void* q, const void* k,
                 "self_attention: q, k, v, out must be 16-byte aligned");
     return flash_attention(q, k, v, out, B, L, H, D, causal ? 1 : 0,
                            sequence_id, rel_values, rel_bucket, num_buckets,
-                           workspace, st);
+                           lse, workspace, st);
   }
+  MOE_REQUIRE(lse == nullptr, MESH_MOE_E_UNSUPPORTED,
+              "self_attention: lse is written by the fused kernel only (bf16, "
+              "d_kv 64 or 128, L a multiple of 8)");
   if (dtype == MESH_MOE_F32)
     return run_attention<float>((const float*)q, (const float*)k,
                                 (const float*)v, (float*)out, B, L, H, D,
@@ -1289,8 +1292,9 @@ extern "C" int mesh_moe_self_attention_backward(
     const void* q, const void* k, const void* v, const void* dout, void* dq,
     void* dk, void* dv, int B, int L, int H, int D, int causal,
     const int32_t* sequence_id, const void* rel_values,
-    const int32_t* rel_bucket, int num_buckets, void* dvalues, int dtype,
-    void* workspace, size_t workspace_bytes, void* stream) {
+    const int32_t* rel_bucket, int num_buckets, void* dvalues, const void* out,
+    const float* lse, int dtype, void* workspace, size_t workspace_bytes,
+    void* stream) {
   MOE_REQUIRE(q && k && v && dout && dq && dk && dv && workspace, MESH_MOE_E_ARG,
               "self_attention_backward: null pointer");
   MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG,
@@ -1307,6 +1311,11 @@ extern "C" int mesh_moe_self_attention_backward(
               MESH_MOE_E_ARG,
               "self_attention_backward: rel_values, rel_bucket, num_buckets "
               "and dvalues go together");
+  MOE_REQUIRE((out == nullptr) == (lse == nullptr) &&
+                  ((uintptr_t)out % 16) == 0,
+              MESH_MOE_E_ARG,
+              "self_attention_backward: out (16-byte aligned) and lse go "
+              "together");
   MOE_REQUIRE(flash_attention_supported(L, H, D, dtype, q, k, v, dout) &&
                   flash_attention_supported(L, H, D, dtype, dq, dk, dv, dout),
               MESH_MOE_E_UNSUPPORTED,
@@ -1318,6 +1327,6 @@ extern "C" int mesh_moe_self_attention_backward(
               MESH_MOE_E_ARG, "self_attention_backward: workspace too small");
   return flash_attention_backward(q, k, v, dout, dq, dk, dv, B, L, H, D,
                                   causal ? 1 : 0, sequence_id, rel_values,
-                                  rel_bucket, num_buckets, dvalues, workspace,
-                                  (hipStream_t)stream);
+                                  rel_bucket, num_buckets, dvalues, out, lse,
+                                  workspace, (hipStream_t)stream);
 }

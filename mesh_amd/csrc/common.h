@@ -24,14 +24,17 @@ bool flash_attention_supported(int L, int H, int D, int dtype, const void* q,
                                const void* k, const void* v, const void* out);
 // With rel_values [H, num_buckets] bf16 and rel_bucket [2L-1] (null: none) the
 // relative attention bias is added to the logits; the backward pass then
-// writes its gradient to dvalues [H, num_buckets] bf16.
+// writes its gradient to dvalues [H, num_buckets] bf16.  lse [B*H, L] float32
+// (null: not wanted): the logarithm of the softmax denominators, which the
+// backward pass takes back as lse_saved together with the outputs (out_saved)
+// in place of recomputing them.
 size_t flash_attention_workspace_bytes(int B, int L, int H, int D,
                                        bool relative_bias);
 int flash_attention(const void* q, const void* k, const void* v, void* out,
                     int B, int L, int H, int D, int causal,
                     const int32_t* sequence_id, const void* rel_values,
-                    const int32_t* rel_bucket, int num_buckets, void* workspace,
-                    hipStream_t st);
+                    const int32_t* rel_bucket, int num_buckets, float* lse,
+                    void* workspace, hipStream_t st);
 size_t flash_attention_backward_workspace_bytes(int B, int L, int H,
                                                 bool relative_bias);
 int flash_attention_backward(const void* q, const void* k, const void* v,
@@ -39,7 +42,9 @@ int flash_attention_backward(const void* q, const void* k, const void* v,
                              int B, int L, int H, int D, int causal,
                              const int32_t* sequence_id, const void* rel_values,
                              const int32_t* rel_bucket, int num_buckets,
-                             void* dvalues, void* workspace, hipStream_t st);
+                             void* dvalues, const void* out_saved,
+                             const float* lse_saved, void* workspace,
+                             hipStream_t st);
 
 #define MOE_REQUIRE(cond, code, ...)      \
   do {                                    \

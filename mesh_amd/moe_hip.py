@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 24
+ABI_VERSION = 25
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -187,15 +187,15 @@ _SIGNATURES = {
         ctypes.c_int]),
     "mesh_moe_self_attention": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
-        ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
-        _vp, ctypes.c_size_t, _vp]),
+        ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, ctypes.c_int, _vp,
+        ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
     "mesh_moe_self_attention_backward_workspace_bytes": (ctypes.c_size_t, [
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_int]),
     "mesh_moe_self_attention_backward": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, ctypes.c_int,
-        _vp, ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
+        _vp, _vp, _vp, ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
     "mesh_moe_attention_decode": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, _vp, _vp, ctypes.c_int, ctypes.c_int, _vp]),
@@ -1141,12 +1141,22 @@ def dense(x, w_packed, activation=None):
   return y.reshape(tuple(x.shape[:-1]) + (n,))
 
 
+def fused_attention_applies(q, num_heads):
+  """Whether the fused attention kernels take q's shape and dtype."""
+  b, l, hd = q.shape
+  return hd % num_heads == 0 and load_library(
+      ).mesh_moe_self_attention_backward_workspace_bytes(
+          b, l, num_heads, hd // num_heads, dtype_code(q.dtype), 0) > 0
+
+
 def self_attention(q, k, v, num_heads, causal, sequence_id=None,
-                   relative_bias=None):
+                   relative_bias=None, return_lse=False):
   """q, k, v [B, L, H*D] -> [B, L, H*D] (attention.attention with float32
   logits, transformer/attention.py:27-88); sequence_id [B, L] int32 or None:
   a query sees only keys of its own sequence
-  (transformer/transformer_layers.py:303-316)."""
+  (transformer/transformer_layers.py:303-316).  return_lse: also the
+  logarithm of the softmax denominators [B*H, L] float32 for
+  self_attention_backward (fused kernels only, see fused_attention_applies)."""
   lib = load_library()
   b, l, hd = q.shape
   if hd % num_heads:
@@ -1155,6 +1165,9 @@ def self_attention(q, k, v, num_heads, causal, sequence_id=None,
   d = hd // num_heads
   code = dtype_code(q.dtype)
   out = torch.empty_like(q)
+  lse = None
+  if return_lse:
+    lse = torch.empty((b * num_heads, l), dtype=torch.float32, device=q.device)
   ws_bytes = lib.mesh_moe_self_attention_workspace_bytes(
       b, l, num_heads, d, code, int(relative_bias is not None))
   ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=q.device)
@@ -1163,9 +1176,10 @@ def self_attention(q, k, v, num_heads, causal, sequence_id=None,
         _dev(q, "q"), _dev(k, "k", q.dtype, (b, l, hd)),
         _dev(v, "v", q.dtype, (b, l, hd)), out.data_ptr(), b, l, num_heads, d,
         int(bool(causal)), _sequence_id_ptr(sequence_id, b, l),
-        *_relative_bias_ptrs(relative_bias, q.dtype, num_heads, l), code,
+        *_relative_bias_ptrs(relative_bias, q.dtype, num_heads, l),
+        None if lse is None else lse.data_ptr(), code,
         ws.data_ptr(), ws_bytes, _stream()), "self_attention")
-  return out
+  return (out, lse) if return_lse else out
 
 
 def attention_decode(q, k_new, v_new, k_cache, v_cache, position, num_heads,
@@ -1370,7 +1384,8 @@ def relative_bias_backward(dlogits, bucket, num_heads, num_buckets):
 
 
 def self_attention_backward(q, k, v, dout, num_heads, causal, fused=None,
-                            sequence_id=None, relative_bias=None):
+                            sequence_id=None, relative_bias=None, out=None,
+                            lse=None):
   """Backward of self_attention: q, k, v, dout [B, L, H*D] -> (dq, dk, dv).
   Shapes the fused kernels take (bf16, d_kv 64 or 128, L a multiple of 8) run
   mesh_moe_self_attention_backward: nothing [L, L] reaches memory.  Otherwise
@@ -1381,7 +1396,9 @@ def self_attention_backward(q, k, v, dout, num_heads, causal, fused=None,
     dq = dlogits . k,       dk = dlogits^T . q
   with heads moved to the front and back by torch permutes.  fused=True raises
   for shapes the fused kernels do not take.  With relative_bias = (values
-  [H, NB], bucket [2L-1]) the gradient of the values is the fourth result."""
+  [H, NB], bucket [2L-1]) the gradient of the values is the fourth result.
+  out, lse: what self_attention(..., return_lse=True) returned for the same
+  arguments; the fused kernels then skip the pass that recomputes them."""
   b, l, hd = q.shape
   h = num_heads
   if hd % h:
@@ -1406,8 +1423,10 @@ def self_attention_backward(q, k, v, dout, num_heads, causal, fused=None,
             dk.data_ptr(), dv.data_ptr(), b, l, h, d, int(bool(causal)),
             _sequence_id_ptr(sequence_id, b, l),
             *_relative_bias_ptrs(relative_bias, q.dtype, h, l),
-            None if dvalues is None else dvalues.data_ptr(), code,
-            ws.data_ptr(), ws_bytes, _stream()), "self_attention_backward")
+            None if dvalues is None else dvalues.data_ptr(),
+            None if lse is None else _dev(out, "out", q.dtype, (b, l, hd)),
+            None if lse is None else _dev(lse, "lse", torch.float32, (b * h, l)),
+            code, ws.data_ptr(), ws_bytes, _stream()), "self_attention_backward")
       return (dq, dk, dv) if dvalues is None else (dq, dk, dv, dvalues)
     if fused:
       raise MoeHipError("self_attention_backward: the fused kernels do not take "

@@ -253,6 +253,7 @@ class SelfAttentionOperation(mtf.Operation):
                        % (sequence_id.shape, q.shape))
     self._num_heads = num_heads
     self._causal = bool(causal)
+    self._save_for_backward = False     # set once a gradient is asked for
     self._outputs = [mtf.Tensor(self, q.shape, q.dtype)]
 
   def lower(self, lowering):
@@ -270,13 +271,24 @@ class SelfAttentionOperation(mtf.Operation):
                     for t in (q, k, v))
       ids, rel = _attention_extras(extra, ids_at, rel_at, length, bidirectional,
                                    q.dtype)
+      # a backward pass follows: where the fused kernels run, keep the softmax
+      # denominators (and the outputs) so that it need not recompute them
+      if self._save_for_backward and moe_hip.fused_attention_applies(q3, heads):
+        out, lse = moe_hip.self_attention(q3, k3, v3, heads, causal,
+                                          sequence_id=ids, relative_bias=rel,
+                                          return_lse=True)
+        saved.update(out=out, lse=lse)
+        return out.reshape(sizes)
       return moe_hip.self_attention(q3, k3, v3, heads, causal, sequence_id=ids,
                                     relative_bias=rel).reshape(sizes)
+    saved = {}
     lowering.set_tensor_lowering(
         self.outputs[0],
         mesh_impl.slicewise(fn, *[lowering.tensors[t] for t in self.inputs]))
+    lowering.operations[self] = saved
 
   def gradient(self, grad_ys):
+    self._save_for_backward = True
     grads = list(SelfAttentionGradOperation(self, grad_ys[0]).outputs)
     out = grads[:3] + [None] * (len(self.inputs) - 3)
     if self._rel_at is not None:
@@ -367,6 +379,7 @@ class SelfAttentionGradOperation(mtf.Operation):
         [dout, q, k, v] + list(forward.inputs[3:]),
         name=name or "attention_grad")
     # pylint: disable=protected-access
+    self._forward = forward
     self._num_heads, self._causal = forward._num_heads, forward._causal
     self._ids_at, self._rel_at = forward._ids_at, forward._rel_at
     self._rel_bidirectional = forward._rel_bidirectional
@@ -390,8 +403,11 @@ class SelfAttentionGradOperation(mtf.Operation):
                         for t in (dout, q, k, v))
       ids, rel = _attention_extras(extra, ids_at, rel_at, length, bidirectional,
                                    q.dtype)
+      saved = lowering.operations.get(self._forward) or {}
       grads = moe_hip.self_attention_backward(
-          q3, k3, v3, d3, heads, causal, sequence_id=ids, relative_bias=rel)
+          q3, k3, v3, d3, heads, causal, sequence_id=ids, relative_bias=rel,
+          out=saved.get("out"), lse=saved.get("lse"))
+      saved.clear()
       return tuple(t.reshape(sizes) for t in grads[:3]) + tuple(grads[3:])
     grads = mesh_impl.slicewise(
         fn, *[lowering.tensors[t] for t in self.inputs])

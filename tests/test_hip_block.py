@@ -1153,6 +1153,26 @@ def test_fused_attention_backward(hip, bsz, length, heads, d, causal):
   again = hip.self_attention_backward(*args, fused=True)
   for g, a in zip(got, again):
     assert torch.equal(g, a)
+  # with the forward pass's outputs and softmax denominators handed back, the
+  # pass that recomputes them drops out: lse is the same number, delta comes
+  # from the rounded outputs
+  out, lse = hip.self_attention(*args[:3], heads, causal, return_lse=True)
+  assert torch.equal(out, hip.self_attention(*args[:3], heads, causal))
+  qf, kf = (t.reshape(bsz, length, heads, d).astype(np.float64) for t in (q, kk))
+  logits = np.einsum("blhd,bmhd->bhlm", qf, kf)
+  if causal:
+    logits = np.where(np.tril(np.ones((length, length), bool)), logits, -np.inf)
+  mx = logits.max(-1, keepdims=True)
+  want_lse = (mx + np.log(np.exp(logits - mx).sum(-1, keepdims=True)))[..., 0]
+  np.testing.assert_allclose(H.to_np(lse).reshape(bsz, heads, length), want_lse,
+                             rtol=1e-5, atol=1e-5)
+  saved = hip.self_attention_backward(*args, fused=True, out=out, lse=lse)
+  for g, sv, wnt, name in zip(got, saved, want, "qkv"):
+    scale = max(1.0, float(np.abs(wnt).max()))
+    np.testing.assert_allclose(H.to_np(sv), wnt, rtol=3e-2, atol=3e-2 * scale,
+                               err_msg="saved d" + name)
+    diff = np.abs(H.to_np(g) - H.to_np(sv))
+    assert float(diff.mean()) < 2e-3 * scale, (name, float(diff.mean()))
   with pytest.raises(hip.MoeHipError):
     hip.self_attention_backward(*(t.float() if isinstance(t, torch.Tensor)
                                   else t for t in args), fused=True)
