@@ -1178,6 +1178,64 @@ def test_fused_attention_backward(hip, bsz, length, heads, d, causal):
                                   else t for t in args), fused=True)
 
 
+@pytest.mark.parametrize("with_ids_and_bias", [False, True])
+def test_attention_gradient_graph_keeps_the_denominators(with_ids_and_bias):
+  """Through the graph API with shapes the fused kernels take (bf16, d_kv 64):
+  once mtf.gradients has been called, the attention operation keeps lse and
+  its outputs for the backward pass.  The gradients must be those of the same
+  graph lowered with that switched off (the backward pass then recomputes
+  them), up to the rounding of the outputs delta is formed from."""
+  b, l, m, heads, d = 2, 136, 64, 2, 64
+  rng = np.random.default_rng(91)
+  dt = torch.bfloat16
+  x = O.cast_act(rng.standard_normal((b, l, m)).astype(np.float32), "bfloat16")
+  dy = O.cast_act(rng.standard_normal((b, l, m)).astype(np.float32), "bfloat16")
+  ids = _packed_sequence_ids(rng, b, l, 50) if with_ids_and_bias else None
+  results = []
+  for keep in (True, False):
+    graph = mtf.Graph()
+    mesh = mtf.Mesh(graph, "mesh")
+    dims = [mtf.Dimension("batch", b), mtf.Dimension("length", l),
+            mtf.Dimension("d_model", m)]
+    xt = mtf.import_tf_tensor(mesh, torch.from_numpy(x).to(dt), mtf.Shape(dims))
+    dyt = mtf.import_tf_tensor(mesh, torch.from_numpy(dy).to(dt), mtf.Shape(dims))
+    idt = None
+    if ids is not None:
+      idt = mtf.import_tf_tensor(mesh, torch.from_numpy(ids), mtf.Shape(dims[:2]))
+    kw = dict(num_heads=heads, key_value_size=d)
+    if with_ids_and_bias:
+      kw.update(relative_attention_type="bias", relative_attention_num_buckets=8)
+    stack = transformer.make_layer_stack(
+        [(transformer_layers.SelfAttention, kw)], num_layers=1, block_scope=False)
+    model = transformer.Unitransformer(stack, d_model=m, name="decoder",
+                                       autoregressive=True)
+    y, _ = model.call_layers(xt, mtf.VariableDType(torch.float32, torch.float32, dt),
+                             mode="eval", sequence_id=idt)
+    variables = sorted(graph.trainable_variables, key=lambda v: v.name)
+    grads = mtf.gradients([y], [xt] + [v.outputs[0] for v in variables], [dyt])
+    att = [op for op in graph.operations
+           if type(op).__name__ == "SelfAttentionOperation"]
+    assert len(att) == 1 and att[0]._save_for_backward
+    att[0]._save_for_backward = keep
+    init_rng = np.random.default_rng(92)
+    init = {v.name: H.normal_weights(init_rng, tuple(v.shape.to_integer_list),
+                                     v.shape.to_integer_list[0])
+            if v.shape.ndims == 2 else np.ones(v.shape.to_integer_list, np.float32)
+            for v in variables}
+    lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()}, initial_values=init)
+    saved = lowering.operations[att[0]]
+    results.append([H.to_np(lowering.export_to_tf_tensor(t)) for t in [y] + grads])
+    assert not saved        # used up by the backward pass, or never kept
+  names = ["y", "dx"] + [v.name for v in variables]
+  for kept, plain, name in zip(results[0], results[1], names):
+    assert np.isfinite(kept).all()
+    scale = max(1e-3, float(np.abs(plain).max()))
+    diff = np.abs(kept - plain)
+    assert float(diff.max()) <= 4e-2 * scale, (name, float(diff.max()), scale)
+    assert float(diff.mean()) <= 4e-3 * scale, (name, float(diff.mean()), scale)
+  np.testing.assert_array_equal(results[0][0], results[1][0])
+
+
 def test_layer_stack_gradients():
   """mtf.gradients through a stack of attention and DenseReluDense layers
   (RMS norms, residuals, projections): every variable's gradient and the
