@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 25
+#define MESH_MOE_ABI_VERSION 26
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -557,12 +557,16 @@ size_t mesh_moe_expert_linear_backward_workspace_bytes(int E, int R, int K,
  * With mesh_moe_activation_backward this is what the layer's backward is made
  * of when the experts are not plain ReLU / linear layers (products of several
  * dense layers, other activations: transformer/moe.py:469-475).
+ * da_relu_mask [E,R,K] dtype or NULL: da is stored as zero wherever the mask
+ * is not positive -- for `a` = relu(...) pass a itself and the ReLU's backward
+ * (mtf.relu's gradient, ops.py:1818-1921) is done with the product, on the
+ * stores of the GEMM where its kernel can, in a pass of its own otherwise.
  */
 int mesh_moe_expert_linear_backward(const void* a, const void* dy,
-                                    const void* w, void* da, void* dw, int E,
-                                    int R, int K, int N, int dtype,
-                                    void* workspace, size_t workspace_bytes,
-                                    void* stream);
+                                    const void* w, void* da, void* dw,
+                                    const void* da_relu_mask, int E, int R,
+                                    int K, int N, int dtype, void* workspace,
+                                    size_t workspace_bytes, void* stream);
 
 /*
  * out = act(pre) on n elements of `dtype`: the activation of a dense layer

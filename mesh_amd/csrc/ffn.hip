@@ -2004,9 +2004,9 @@ extern "C" size_t mesh_moe_expert_linear_backward_workspace_bytes(int E, int R,
 }
 
 extern "C" int mesh_moe_expert_linear_backward(
-    const void* a, const void* dy, const void* w, void* da, void* dw, int E,
-    int R, int K, int N, int dtype, void* workspace, size_t workspace_bytes,
-    void* stream) {
+    const void* a, const void* dy, const void* w, void* da, void* dw,
+    const void* da_relu_mask, int E, int R, int K, int N, int dtype,
+    void* workspace, size_t workspace_bytes, void* stream) {
   MOE_REQUIRE(a && dy && w && dw && workspace, MESH_MOE_E_ARG,
               "expert_linear_backward: null pointer");
   MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG,
@@ -2021,9 +2021,25 @@ extern "C" int mesh_moe_expert_linear_backward(
   hipStream_t st = (hipStream_t)stream;
   int rc;
   if (da != nullptr) {
-    // da = dy . w^T  (w in its variable layout [E, K, N] is K-contiguous here)
-    rc = grouped_gemm(dy, w, da, E, R, K, N, MESH_MOE_ACT_LINEAR, dtype, st);
+    // da = dy . w^T  (w in its variable layout [E, K, N] is K-contiguous here);
+    // a ReLU mask rides on the stores of this GEMM where its kernel can
+    bool masked = false;
+    rc = grouped_gemm(dy, w, da, E, R, K, N, MESH_MOE_ACT_LINEAR, dtype, st,
+                      da_relu_mask, &masked);
     if (rc != 0) return rc;
+    if (da_relu_mask != nullptr && !masked) {
+      const int64_t n = (int64_t)E * R * K;
+      const int blocks = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
+      if (dtype == MESH_MOE_F32)
+        hidden_grad_kernel<float><<<blocks, 256, 0, st>>>(
+            (float*)da, (const float*)da_relu_mask, (const float*)nullptr, true,
+            n);
+      else
+        hidden_grad_kernel<bf16_t><<<blocks, 256, 0, st>>>(
+            (bf16_t*)da, (const bf16_t*)da_relu_mask, (const bf16_t*)nullptr,
+            true, n);
+      MOE_CHECK_LAUNCH("expert_linear_backward (relu mask)");
+    }
   }
   // dw [E, K, N] = a^T . dy: the reduction runs over the rows of both operands
   if (kmajor_path_applies(a, dy, dw, K, N, R, dtype))

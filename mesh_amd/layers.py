@@ -130,6 +130,11 @@ class DenseOperation(mtf.Operation):
   def __init__(self, x, kernel, new_dims, activation, name=None):
     super(DenseOperation, self).__init__([x, kernel], name=name or "dense")
     self._activation = activation
+    # Set by a layer whose hidden tensor x = relu(dense(...)) feeds nothing but
+    # this operation: the gradient of x then leaves this operation's backward
+    # already multiplied by (x > 0) -- the ReLU's backward done on the stores
+    # of the GEMM -- and the producer's backward skips its own pass over it.
+    self.masks_input_gradient = False
     shape = mtf.Shape(x.shape.dims[:-1] + list(new_dims))
     self._outputs = [mtf.Tensor(self, shape, x.dtype)]
 
@@ -161,6 +166,14 @@ class DenseGradOperation(mtf.Operation):
     super(DenseGradOperation, self).__init__(
         [dy, x, kernel, forward.outputs[0]], name=name or "dense_grad")
     self._relu = forward._activation == "relu"   # pylint: disable=protected-access
+    self._masks_dx = bool(forward.masks_input_gradient)
+    # dy already carries this layer's ReLU mask when it is the input gradient
+    # of the one operation that consumes the output and that operation masks
+    producer = dy.operation
+    self._dy_is_masked = (
+        self._relu and isinstance(producer, DenseGradOperation)
+        and producer._masks_dx and dy is producer.outputs[0]
+        and producer.inputs[1] is forward.outputs[0])
     if forward._activation not in (None, "relu"):  # pylint: disable=protected-access
       raise NotImplementedError("gradient of dense with activation %r"
                                 % (forward._activation,))  # pylint: disable=protected-access
@@ -170,14 +183,16 @@ class DenseGradOperation(mtf.Operation):
   def lower(self, lowering):
     from mesh_amd import moe_hip
     mesh_impl = lowering.mesh_impl(self)
-    relu = self._relu
+    relu = self._relu and not self._dy_is_masked
+    masks_dx = self._masks_dx
     k = self.inputs[1].shape.dims[-1].size
     kernel_sizes = self.inputs[2].shape.to_integer_list
 
     def fn(dy, x, w, y):
       w2 = w.to(x.dtype).reshape(k, -1)
       dx, dw = moe_hip.dense_backward(x.contiguous(), w2, dy.contiguous(),
-                                      y if relu else None)
+                                      y if relu else None,
+                                      dx_relu_mask=masks_dx)
       return dx, dw.reshape(kernel_sizes).to(w.dtype)
     dx, dw = mesh_impl.slicewise(
         fn, *[lowering.tensors[t] for t in self.inputs])

@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 25
+ABI_VERSION = 26
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -115,7 +115,7 @@ _SIGNATURES = {
     "mesh_moe_expert_linear_backward_workspace_bytes": (ctypes.c_size_t, [
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "mesh_moe_expert_linear_backward": (ctypes.c_int, [
-        _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
     "mesh_moe_rms_norm_backward_workspace_bytes": (ctypes.c_size_t, [
         ctypes.c_int64, ctypes.c_int]),
@@ -884,9 +884,11 @@ def expert_ffn_backward(expert_in, h, dy, wi, wo, activation="relu",
   return dxe, dwi, dwo
 
 
-def expert_linear_backward(a, dy, w, want_da=True):
+def expert_linear_backward(a, dy, w, want_da=True, da_relu_mask=None):
   """Backward of y = a . w per expert: a [E,R,K], dy [E,R,N], w [E,K,N] in the
-  variable's own layout -> (da [E,R,K] or None, dw [E,K,N])."""
+  variable's own layout -> (da [E,R,K] or None, dw [E,K,N]).  da_relu_mask
+  [E,R,K]: da comes out zero where the mask is not positive (the backward of
+  the ReLU that made `a`, done with the product)."""
   lib = load_library()
   e, rows, k = a.shape
   n = w.shape[2]
@@ -901,7 +903,10 @@ def expert_linear_backward(a, dy, w, want_da=True):
     _check(lib.mesh_moe_expert_linear_backward(
         _dev(a, "a"), _dev(dy, "dy", dt, (e, rows, n)),
         _dev(w, "w", dt, (e, k, n)), da.data_ptr() if want_da else None,
-        dw.data_ptr(), e, rows, k, n, code, ws.data_ptr(), ws_bytes,
+        dw.data_ptr(),
+        None if da_relu_mask is None or not want_da else _dev(
+            da_relu_mask, "da_relu_mask", dt, (e, rows, k)),
+        e, rows, k, n, code, ws.data_ptr(), ws_bytes,
         _stream()), "expert_linear_backward")
   return da, dw
 
@@ -1294,19 +1299,22 @@ def rms_norm_backward(x, scale, dy, epsilon=1e-6):
   return dx, dscale
 
 
-def dense_backward(x, w, dy, y=None, want_dx=True):
+def dense_backward(x, w, dy, y=None, want_dx=True, dx_relu_mask=False):
   """Backward of y = act(x . w): x [..., K], w [K, N] in the variable's own
   layout, dy [..., N]; with `y` (the forward output) the activation was relu.
-  Returns (dx or None, dw [K, N])."""
+  dx_relu_mask: x is itself the output of a ReLU whose backward is wanted on
+  dx (zero where x is not positive).  Returns (dx or None, dw [K, N])."""
   k = x.shape[-1]
   n = w.shape[-1]
   x3 = x.reshape(1, -1, k)
   dy3 = dy.reshape(1, -1, n)
   if y is not None:     # relu: y > 0 exactly where the pre-activation is
     dy3 = activation_backward(dy3.contiguous(), y.reshape(1, -1, n), "relu")
-  dx, dw = expert_linear_backward(x3.contiguous(), dy3.contiguous(),
+  x3 = x3.contiguous()
+  dx, dw = expert_linear_backward(x3, dy3.contiguous(),
                                   w.reshape(1, k, n).contiguous(),
-                                  want_da=want_dx)
+                                  want_da=want_dx,
+                                  da_relu_mask=x3 if dx_relu_mask else None)
   return (dx.reshape(x.shape) if want_dx else None), dw.reshape(k, n)
 
 

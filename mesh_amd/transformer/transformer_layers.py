@@ -33,10 +33,18 @@ class DenseReluDense(transformer.TransformerLayer):
     if context.train and self.dropout_rate != 0.0:   # transformer_layers.py:67-69
       h = mtf.dropout(h, context.train, keep_prob=1.0 - self.dropout_rate,
                       noise_shape=h.shape - context.length_dim)
-    return mtf_layers.dense(
+    y = mtf_layers.dense(
         h, io_channels, use_bias=self.use_bias, activation=None,
         variable_dtype=context.variable_dtype, reduced_dims=h.shape.dims[-1:],
         name="wo")
+    # h = relu(dense(x)) feeds only the output projection: its backward can
+    # apply the ReLU mask to dh while it writes it
+    if (isinstance(h.operation, mtf_layers.DenseOperation)
+        and h.operation._activation == "relu"          # pylint: disable=protected-access
+        and isinstance(y.operation, mtf_layers.DenseOperation)
+        and y.operation.inputs[0] is h):
+      y.operation.masks_input_gradient = True
+    return y
 
 
 class SelfAttention(transformer.TransformerLayer):

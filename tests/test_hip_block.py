@@ -1273,6 +1273,12 @@ def test_layer_stack_gradients():
   names = sorted(init)
   grads = mtf.gradients([y], [xt] + [variables[n].outputs[0] for n in names],
                         [dyt])
+  # DenseReluDense: the output projection's backward applies the ReLU mask to
+  # the hidden gradient, the first projection's backward knows and skips it
+  dense_grads = [op for op in graph.operations
+                 if type(op).__name__ == "DenseGradOperation"]
+  assert sum(op._masks_dx for op in dense_grads) == 1
+  assert sum(op._dy_is_masked for op in dense_grads) == 1
   lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()}, initial_values=init)
   got = {n: H.to_np(lowering.export_to_tf_tensor(g))
          for n, g in zip(["x"] + names, grads)}

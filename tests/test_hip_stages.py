@@ -1096,6 +1096,28 @@ def test_expert_linear_many_row_tiles(hip, shape):
                                atol=1e-2 * float(wnt.abs().max()), err_msg=name)
 
 
+@pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("shape", [(2, 256, 512, 128), (1, 100, 72, 40),
+                                   (1, 4096, 1024, 256)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_expert_linear_backward_relu_mask(hip, shape, act_dtype):
+  """da_relu_mask of mesh_moe_expert_linear_backward: da is the unmasked
+  product with zeros wherever the mask is not positive, bit for bit, whether
+  the mask rides on the GEMM's stores (bf16 shapes of the direct-to-LDS
+  kernel) or is a pass of its own; dw is not touched."""
+  e, rows, k, n = shape
+  rng = np.random.default_rng(sum(shape))
+  g = lambda a: H.to_gpu(O.cast_act(a.astype(np.float32), act_dtype), act_dtype)
+  a = g(np.maximum(rng.standard_normal((e, rows, k)), 0))       # a = relu(...)
+  w = g(H.normal_weights(rng, (e, k, n), k))
+  dy = g(rng.standard_normal((e, rows, n)))
+  da, dw = hip.expert_linear_backward(a, dy, w)
+  da_m, dw_m = hip.expert_linear_backward(a, dy, w, da_relu_mask=a)
+  assert torch.equal(dw, dw_m)
+  assert torch.equal(da_m, da * (a > 0))
+  assert float((a > 0).float().mean()) < 0.6 and da.abs().sum() > 0
+
+
 @pytest.mark.parametrize("size", [(8, 512, 1024, 4096), (8, 2048, 4096, 16384)],
                          ids=["cfg3_slice", "cfg4_slice"])
 def test_full_size_ffn_backward_properties(hip, size):
