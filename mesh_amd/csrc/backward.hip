@@ -61,14 +61,19 @@ __global__ __launch_bounds__(256) void combine_backward_kernel(
   const T* yrow[2] = {nullptr, nullptr};
   T* drow[2] = {nullptr, nullptr};
   float w[2] = {0.f, 0.f};
+  // the token's record in one round trip (both choices of every array at once)
+  const uint16_t kept2 = *reinterpret_cast<const uint16_t*>(kept + t * 2);
+  const int2 idx2 = *reinterpret_cast<const int2*>(idx + t * 2);
+  const int2 pos2 = *reinterpret_cast<const int2*>(pos + t * 2);
+  const float2 gate2 = *reinterpret_cast<const float2*>(gate + t * 2);
 #pragma unroll
   for (int k = 0; k < 2; ++k) {
-    if (kept[t * 2 + k]) {
+    if ((kept2 >> (8 * k)) & 0xff) {
       const int64_t slot =
-          ((int64_t)idx[t * 2 + k] * G + g) * C + pos[t * 2 + k];
+          ((int64_t)(k ? idx2.y : idx2.x) * G + g) * C + (k ? pos2.y : pos2.x);
       yrow[k] = y + slot * N;
       drow[k] = dy + slot * N;
-      w[k] = round_to<T>(gate[t * 2 + k]);
+      w[k] = round_to<T>(k ? gate2.y : gate2.x);
     }
   }
   float dot[2] = {0.f, 0.f};

@@ -86,6 +86,65 @@ __global__ __launch_bounds__(256) void rms_norm_kernel(
   }
 }
 
+// The same for bf16 rows of at most ITERS * 512 elements (16-byte aligned):
+// the row stays in registers -- all its 16-byte loads are in flight together,
+// and it is read once.
+template <int ITERS>
+__global__ __launch_bounds__(256) void rms_norm_rows_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ scale,
+    bf16_t* __restrict__ y, int64_t rows, int M, float inv_m, float eps) {
+  using T = bf16_t;
+  const int lane = threadIdx.x & 63;
+  const int64_t row = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+  if (row >= rows) return;
+  const uint4* xv = reinterpret_cast<const uint4*>(x + row * M);
+  const uint4* sv = reinterpret_cast<const uint4*>(scale);
+  uint4* yv = reinterpret_cast<uint4*>(y + row * M);
+  const int chunks = M / 8;
+  uint4 p[ITERS];
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int c = lane + 64 * it;
+    p[it] = c < chunks ? load_streaming(xv + c) : make_uint4(0, 0, 0, 0);
+  }
+  float sum = 0.f;
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const uint32_t w[4] = {p[it].x, p[it].y, p[it].z, p[it].w};
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float a = __uint_as_float(w[j] << 16);
+      const float b = __uint_as_float(w[j] & 0xffff0000u);
+      sum += round_to<T>(a * a);
+      sum += round_to<T>(b * b);
+    }
+  }
+#pragma unroll
+  for (int off = 32; off > 0; off >>= 1) sum += __shfl_xor(sum, off);
+  const float total = round_to<T>(sum);
+  const float mean = round_to<T>(total * inv_m);
+  const float var = round_to<T>(mean + eps);
+  const float r = round_to<T>(1.0f / sqrtf(var));
+#pragma unroll
+  for (int it = 0; it < ITERS; ++it) {
+    const int c = lane + 64 * it;
+    if (c >= chunks) continue;
+    const uint4 q = sv[c];
+    const uint32_t w[4] = {p[it].x, p[it].y, p[it].z, p[it].w};
+    const uint32_t g[4] = {q.x, q.y, q.z, q.w};
+    uint32_t o[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const float a = __uint_as_float(w[j] << 16);
+      const float b = __uint_as_float(w[j] & 0xffff0000u);
+      const float sa = __uint_as_float(g[j] << 16);
+      const float sb = __uint_as_float(g[j] & 0xffff0000u);
+      o[j] = f32x2_to_bf16x2(round_to<T>(a * r) * sa, round_to<T>(b * r) * sb);
+    }
+    store_streaming(yv + c, make_uint4(o[0], o[1], o[2], o[3]));
+  }
+}
+
 // ---------------------------------------------------------------------------
 // [B, L, H*D] -> [B*H, L, D]  (heads to the front)
 // ---------------------------------------------------------------------------
@@ -941,9 +1000,21 @@ extern "C" int mesh_moe_rms_norm(const void* x, const void* scale, void* y,
     const bool vec16 =
         M % 8 == 0 &&
         (((uintptr_t)x | (uintptr_t)scale | (uintptr_t)y) % 16 == 0);
-    rms_norm_kernel<bf16_t><<<(unsigned)blocks, 256, 0, st>>>(
-        (const bf16_t*)x, (const bf16_t*)scale, (bf16_t*)y, rows, M, inv_m,
-        eps, vec16);
+    const bf16_t *xb = (const bf16_t*)x, *sb = (const bf16_t*)scale;
+    bf16_t* yb = (bf16_t*)y;
+    if (vec16 && M <= 1024)
+      rms_norm_rows_kernel<2><<<(unsigned)blocks, 256, 0, st>>>(xb, sb, yb, rows,
+                                                               M, inv_m, eps);
+    else if (vec16 && M <= 2048)
+      rms_norm_rows_kernel<4><<<(unsigned)blocks, 256, 0, st>>>(xb, sb, yb, rows,
+                                                               M, inv_m, eps);
+    else if (vec16 && M <= 4096)
+      rms_norm_rows_kernel<8><<<(unsigned)blocks, 256, 0, st>>>(xb, sb, yb, rows,
+                                                               M, inv_m, eps);
+    else
+      rms_norm_kernel<bf16_t><<<(unsigned)blocks, 256, 0, st>>>(xb, sb, yb, rows,
+                                                                M, inv_m, eps,
+                                                                vec16);
   }
   MOE_CHECK_LAUNCH("rms_norm");
   return 0;

@@ -33,14 +33,35 @@ __global__ __launch_bounds__(256) void dispatch_kernel(
     const int64_t t = job;
     const int g = (int)(t / S);
     const T* src = x + t * M;
+    // The token's record in one round trip (both choices of every array at
+    // once, kept or not), and -- vec path -- the first batch of the row's loads
+    // issued before the record is looked at: the row's address does not
+    // depend on it, and a token with no kept choice is rare.
+    constexpr int VN = Vec16<T>::N;
+    constexpr int UN = 8;    // 16-byte loads in flight per lane before any store
+    const int nv = M / VN;
+    const uint4* s4 = reinterpret_cast<const uint4*>(src);
+    const uint4 z = make_uint4(0, 0, 0, 0);
+    uint4 v[UN];
+    if (vec) {
+#pragma unroll
+      for (int u = 0; u < UN; ++u) {
+        const int i = lane + u * 64;
+        v[u] = i < nv ? load_streaming(s4 + i) : z;
+      }
+    }
+    const uint16_t kept2 = *reinterpret_cast<const uint16_t*>(kept + t * 2);
+    const int2 idx2 = *reinterpret_cast<const int2*>(idx + t * 2);
+    const int2 pos2 = *reinterpret_cast<const int2*>(pos + t * 2);
+    const float2 gate2 = *reinterpret_cast<const float2*>(gate + t * 2);
     T* dst[2] = {nullptr, nullptr};
     bool zero[2] = {false, false};
 #pragma unroll
     for (int k = 0; k < 2; ++k) {
-      if (kept[t * 2 + k]) {
-        const int e = idx[t * 2 + k];
-        const int c = pos[t * 2 + k];
-        const float w = round_to<T>(gate[t * 2 + k]);
+      if ((kept2 >> (8 * k)) & 0xff) {
+        const int e = k ? idx2.y : idx2.x;
+        const int c = k ? pos2.y : pos2.x;
+        const float w = round_to<T>(k ? gate2.y : gate2.x);
         const int64_t slot = ((int64_t)e * G + g) * C + c;
         dst[k] = expert_in + slot * M;
         zero[k] = (w == 0.0f);
@@ -49,23 +70,16 @@ __global__ __launch_bounds__(256) void dispatch_kernel(
     }
     if (dst[0] == nullptr && dst[1] == nullptr) return;
     if (vec) {
-      constexpr int VN = Vec16<T>::N;
-      const int nv = M / VN;
-      const uint4* s4 = reinterpret_cast<const uint4*>(src);
       uint4* d0 = reinterpret_cast<uint4*>(dst[0]);
       uint4* d1 = reinterpret_cast<uint4*>(dst[1]);
-      const uint4 z = make_uint4(0, 0, 0, 0);
-      // eight independent 16-byte loads in flight per lane before any store
-      // (a whole 8 KB row per wavefront; 0.296 ms against 0.313 ms with four
-      // at 65536 rows of 4096 bf16)
-      constexpr int UN = 8;
       const bool has0 = d0 != nullptr, has1 = d1 != nullptr;
       for (int base = lane; base < nv; base += 64 * UN) {
-        uint4 v[UN];
+        if (base != lane) {
 #pragma unroll
-        for (int u = 0; u < UN; ++u) {
-          const int i = base + u * 64;
-          v[u] = i < nv ? load_streaming(s4 + i) : z;
+          for (int u = 0; u < UN; ++u) {
+            const int i = base + u * 64;
+            v[u] = i < nv ? load_streaming(s4 + i) : z;
+          }
         }
 #pragma unroll
         for (int u = 0; u < UN; ++u) {
@@ -152,18 +166,24 @@ __global__ __launch_bounds__(256) void combine_kernel(
   const int g = (int)(t / S);
   const T* src[2] = {nullptr, nullptr};
   float w[2] = {0.f, 0.f};
+  // the token's record in one round trip (both choices of every array at
+  // once, kept or not) instead of one per array
+  const uint16_t kept2 = *reinterpret_cast<const uint16_t*>(kept + t * 2);
+  const int2 idx2 = *reinterpret_cast<const int2*>(idx + t * 2);
+  const int2 pos2 = *reinterpret_cast<const int2*>(pos + t * 2);
+  const float2 gate2 = *reinterpret_cast<const float2*>(gate + t * 2);
 #pragma unroll
   for (int k = 0; k < 2; ++k) {
-    if (kept[t * 2 + k]) {
-      const float wk = round_to<T>(gate[t * 2 + k]);
+    if ((kept2 >> (8 * k)) & 0xff) {
+      const float wk = round_to<T>(k ? gate2.y : gate2.x);
       if (wk != 0.0f) {
-        const int64_t e = idx[t * 2 + k];
+        const int64_t e = k ? idx2.y : idx2.x;
+        const int p = k ? pos2.y : pos2.x;
         // row of the slot: [e][g][c], or with compacted rows the expert's
         // occupied slots of earlier groups first (row_offsets[e][g])
-        const int64_t slot =
-            row_offsets == nullptr
-                ? (e * G + g) * C + pos[t * 2 + k]
-                : e * G * C + row_offsets[e * G + g] + pos[t * 2 + k];
+        const int64_t slot = row_offsets == nullptr
+                                 ? (e * G + g) * C + p
+                                 : e * G * C + row_offsets[e * G + g] + p;
         src[k] = y + slot * N;
         w[k] = wk;
       }
