@@ -572,19 +572,20 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
 
   // PERSISTENT blocks: one per CU, each walks a strided list of tiles, so that
   // block start-up and the first loads of a tile overlap the previous tile's
-  // epilogue.  Block b runs on XCD b % 8; an XCD owns a contiguous range of
-  // logical tiles and its blocks take them round-robin, which keeps the tiles
-  // resident on an XCD at any moment consecutive (shared panels in its L2).
+  // epilogue.  Block b runs on XCD b % 8.  The P = blocks / 8 blocks of an XCD
+  // hold P consecutive logical tiles at any moment (shared panels in its L2),
+  // and consecutive groups of P tiles go to consecutive XCDs: the whole chip
+  // then works on the same one or two experts, whose token panels every XCD
+  // re-reads from the memory-side cache, instead of on eight experts at once
+  // (1 % faster than giving each XCD a contiguous eighth of the tiles).
   const int nblk = gridDim.x;
   if constexpr (LISTED) total_tiles = tile_list[-1];
   int tile, tile_end, tile_step;
   if ((nblk & 7) == 0) {
     const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
-    const int per_xcd = total_tiles >> 3, extra = total_tiles & 7;
-    const int begin = xcd * per_xcd + min(xcd, extra);
-    tile_end = begin + per_xcd + (xcd < extra ? 1 : 0);
-    tile = begin + local;
-    tile_step = nblk >> 3;
+    tile = xcd * (nblk >> 3) + local;
+    tile_end = total_tiles;
+    tile_step = nblk;
   } else {
     tile = blockIdx.x;
     tile_end = total_tiles;
