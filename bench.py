@@ -450,8 +450,7 @@ def main():
         "avg_launch_ms": ffn_ms / 2,
         # fraction counting every slot row, occupied or not; the compacted
         # path of the single-choice routers does not multiply the empty rows
-        "padded_frac": (None if ("dispatch" not in stages and args.gating in
-                                 ("switch", "switch_max", "ntlb"))
+        "padded_frac": (None if timer.compacted
                         else (model["expert_ffn"]["padded_flops"] / 2
                               / (ffn_ms / 2 * 1e-3) / 1e12) / peak)}
     result["stages"] = per_stage
@@ -461,7 +460,9 @@ def main():
       per_stage["expert_ffn_backward"].update(
           TFLOPs=bw["flops"] / (bw_ms * 1e-3) / 1e12,
           frac_mfma_peak=bw["flops"] / (bw_ms * 1e-3) / 1e12 / peak,
-          padded_frac=bw["padded_flops"] / (bw_ms * 1e-3) / 1e12 / peak)
+          padded_frac=(None if timer.compacted else
+                       bw["padded_flops"] / (bw_ms * 1e-3) / 1e12 / peak))
+    result["config"]["compacted_rows"] = bool(timer.compacted)
     result["config"].update(kept_pairs=kept, slots=slots,
                             capacity=r.capacity)
   else:

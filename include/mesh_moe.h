@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 26
+#define MESH_MOE_ABI_VERSION 27
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -648,6 +648,56 @@ int mesh_moe_dispatch_backward(const void* dexpert_in, const int32_t* idx,
                                const void* w_gate_packed,
                                int groups_per_router, void* dx, int G, int S,
                                int E, int C, int M, int dtype, void* stream);
+
+/*
+ * The gradient calls on COMPACTED rows, for a layer whose forward pass ran
+ * mesh_moe_compact_expert_ffn (routers with one choice per token,
+ * transformer/moe.py:1176-1309, :804-940): every tensor with slot rows
+ * (expert_in, h, y and their gradients, [E, G*C, .]) holds expert e's occupied
+ * slots at rows 0 .. used_e - 1 of its row range, slot (e, g, c) at row
+ * row_offsets[e][g] + c, and the four gradient GEMMs skip the rest: the
+ * einsum gradients of ops.py:2846-2854 over the occupied slots only.
+ * fill [G,E] and row_offsets [E,G] as for mesh_moe_compact_expert_ffn.  Rows
+ * from used_e up to the next multiple of 256 are written as zeros by
+ * dispatch_compact and combine_backward_compact and stay zero through the
+ * GEMMs; rows beyond hold unspecified values that nothing reads.
+ *
+ * mesh_moe_dispatch_compact: mesh_moe_dispatch into compacted rows
+ *   (expert_in [E, G*C, M]; the weight gradient of wi reads it).
+ * mesh_moe_combine_backward_compact: mesh_moe_combine_backward with y and dy
+ *   in compacted rows.
+ * mesh_moe_compact_expert_ffn_backward: mesh_moe_expert_ffn_backward
+ *   (relu or linear experts, no dh_scale); bf16, E <= 1024 and shapes the
+ *   256 x 256 kernels take, else MESH_MOE_E_UNSUPPORTED;
+ *   ..._workspace_bytes returns 0 for shapes it does not take.
+ * mesh_moe_dispatch_backward_compact: mesh_moe_dispatch_backward reading
+ *   dexpert_in in compacted rows.
+ */
+int mesh_moe_dispatch_compact(const void* x, const int32_t* idx,
+                              const int32_t* pos, const float* gate,
+                              const uint8_t* kept, const int32_t* fill,
+                              const int32_t* row_offsets, void* expert_in,
+                              int G, int S, int E, int C, int M, int dtype,
+                              void* stream);
+int mesh_moe_combine_backward_compact(
+    const void* dout, const void* y, const int32_t* idx, const int32_t* pos,
+    const float* gate, const uint8_t* kept, const int32_t* fill,
+    const int32_t* row_offsets, void* dy, float* dgate, int G, int S, int E,
+    int C, int N, int dtype, void* stream);
+size_t mesh_moe_compact_expert_ffn_backward_workspace_bytes(int G, int E, int C,
+                                                            int M, int H,
+                                                            int N);
+int mesh_moe_compact_expert_ffn_backward(
+    const void* expert_in, const void* h, const void* dy, const void* wi,
+    const void* wo, const int32_t* fill, const int32_t* row_offsets,
+    void* dexpert_in, void* dwi, void* dwo, int G, int E, int C, int M, int H,
+    int N, int activation, int dtype, void* workspace, size_t workspace_bytes,
+    void* stream);
+int mesh_moe_dispatch_backward_compact(
+    const void* dexpert_in, const int32_t* idx, const int32_t* pos,
+    const float* gate, const uint8_t* kept, const int32_t* row_offsets,
+    const float* dlogits, const void* w_gate_packed, int groups_per_router,
+    void* dx, int G, int S, int E, int C, int M, int dtype, void* stream);
 
 /*
  * ---------------------------------------------------------------------------

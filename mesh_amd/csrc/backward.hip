@@ -27,6 +27,10 @@ __device__ __forceinline__ float wave_sum(float v) {
 //   dy[slot_k]  = w_k * dout[t]            (rounded to the activation dtype)
 //   dgate[t,k]  = <dout[t], y[slot_k]>     (float32), 0 where not kept
 // Jobs [0, T): tokens; jobs [T, T + G*E): zero rows for the slots >= fill.
+// With row_offsets, y and dy hold every expert's occupied slots at the front
+// of its row range (slots of group g from row row_offsets[e][g]); the zero
+// jobs are then [T, T + 256 E): the rows between an expert's occupied rows
+// and the next multiple of 256.
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void combine_backward_kernel(
@@ -35,12 +39,31 @@ __global__ __launch_bounds__(256) void combine_backward_kernel(
     const float* __restrict__ gate, const uint8_t* __restrict__ kept,
     const int32_t* __restrict__ fill, T* __restrict__ dy,
     float* __restrict__ dgate, int G, int S, int E, int C, int N,
-    int64_t T_tokens, bool vec) {
+    int64_t T_tokens, bool vec, const int32_t* __restrict__ row_offsets) {
   constexpr int VN = Vec16B<T>::N;
   const int lane = threadIdx.x & 63;
   const int64_t job =
       (int64_t)blockIdx.x * BW_ROWS_PER_BLOCK + (threadIdx.x >> 6);
-  if (job >= T_tokens + (int64_t)G * E) return;
+  if (job >= T_tokens +
+                 (row_offsets != nullptr ? (int64_t)E * 256 : (int64_t)G * E))
+    return;
+  if (job >= T_tokens && row_offsets != nullptr) {
+    const int64_t j = job - T_tokens;
+    const int e = (int)(j >> 8);
+    const int64_t rows = (int64_t)G * C;
+    const int64_t row = compact_tail_row(
+        compact_rows_used(fill, row_offsets, e, G, E), (int)(j & 255), rows);
+    if (row < 0) return;
+    T* d = dy + ((int64_t)e * rows + row) * N;
+    if (vec) {
+      uint4* d4 = reinterpret_cast<uint4*>(d);
+      for (int i = lane; i < N / VN; i += 64)
+        store_streaming(d4 + i, make_uint4(0, 0, 0, 0));
+    } else {
+      for (int i = lane; i < N; i += 64) d[i] = (T)0;
+    }
+    return;
+  }
   if (job >= T_tokens) {
     const int64_t ge = job - T_tokens;
     const int g = (int)(ge / E), e = (int)(ge % E);
@@ -69,8 +92,11 @@ __global__ __launch_bounds__(256) void combine_backward_kernel(
 #pragma unroll
   for (int k = 0; k < 2; ++k) {
     if ((kept2 >> (8 * k)) & 0xff) {
+      const int64_t e = k ? idx2.y : idx2.x;
       const int64_t slot =
-          ((int64_t)(k ? idx2.y : idx2.x) * G + g) * C + (k ? pos2.y : pos2.x);
+          (row_offsets == nullptr ? (e * G + g) * C
+                                  : e * G * C + row_offsets[e * G + g]) +
+          (k ? pos2.y : pos2.x);
       yrow[k] = y + slot * N;
       drow[k] = dy + slot * N;
       w[k] = round_to<T>(k ? gate2.y : gate2.x);
@@ -154,7 +180,8 @@ __global__ __launch_bounds__(256) void dispatch_backward_kernel(
     const int32_t* __restrict__ pos, const float* __restrict__ gate,
     const uint8_t* __restrict__ kept, const float* __restrict__ dlogits,
     const T* __restrict__ wgp, T* __restrict__ dx, int G, int S, int E, int C,
-    int M, int64_t T_tokens, int groups_per_router, bool vec) {
+    int M, int64_t T_tokens, int groups_per_router, bool vec,
+    const int32_t* __restrict__ row_offsets) {
   constexpr int VN = Vec16B<T>::N;
   const int lane = threadIdx.x & 63;
   const int64_t t =
@@ -166,8 +193,11 @@ __global__ __launch_bounds__(256) void dispatch_backward_kernel(
 #pragma unroll
   for (int k = 0; k < 2; ++k) {
     if (kept[t * 2 + k] && round_to<T>(gate[t * 2 + k]) != 0.0f) {
+      const int64_t e = idx[t * 2 + k];
       const int64_t slot =
-          ((int64_t)idx[t * 2 + k] * G + g) * C + pos[t * 2 + k];
+          (row_offsets == nullptr ? (e * G + g) * C
+                                  : e * G * C + row_offsets[e * G + g]) +
+          pos[t * 2 + k];
       src[k] = dxe + slot * M;
     }
   }
@@ -227,7 +257,8 @@ __global__ __launch_bounds__(256) void dispatch_backward_router4_kernel(
     const int32_t* __restrict__ pos, const float* __restrict__ gate,
     const uint8_t* __restrict__ kept, const float* __restrict__ dlogits,
     const T* __restrict__ wgp, T* __restrict__ dx, int G, int S, int E, int C,
-    int M, int64_t T_tokens, int groups_per_router) {
+    int M, int64_t T_tokens, int groups_per_router,
+    const int32_t* __restrict__ row_offsets) {
   constexpr int VN = Vec16B<T>::N;
   __shared__ __attribute__((aligned(16))) float dls[4][DBR_MAX_E][DBR_TOK];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
@@ -244,8 +275,11 @@ __global__ __launch_bounds__(256) void dispatch_backward_router4_kernel(
       src[j][k] = nullptr;
       if (t < T_tokens && kept[t * 2 + k] &&
           round_to<T>(gate[t * 2 + k]) != 0.0f) {
+        const int64_t e = idx[t * 2 + k];
         const int64_t slot =
-            ((int64_t)idx[t * 2 + k] * G + g) * C + pos[t * 2 + k];
+            (row_offsets == nullptr ? (e * G + g) * C
+                                    : e * G * C + row_offsets[e * G + g]) +
+            pos[t * 2 + k];
         src[j][k] = dxe + slot * M;
       }
     }
@@ -699,10 +733,36 @@ static bool bw_aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 using namespace mesh_moe;
 
+static int run_combine_backward(
+    const void* dout, const void* y, const int32_t* idx, const int32_t* pos,
+    const float* gate, const uint8_t* kept, const int32_t* fill,
+    const int32_t* row_offsets, void* dy, float* dgate, int G, int S, int E,
+    int C, int N, int dtype, void* stream);
+
 extern "C" int mesh_moe_combine_backward(
     const void* dout, const void* y, const int32_t* idx, const int32_t* pos,
     const float* gate, const uint8_t* kept, const int32_t* fill, void* dy,
     float* dgate, int G, int S, int E, int C, int N, int dtype, void* stream) {
+  return run_combine_backward(dout, y, idx, pos, gate, kept, fill, nullptr, dy,
+                              dgate, G, S, E, C, N, dtype, stream);
+}
+
+extern "C" int mesh_moe_combine_backward_compact(
+    const void* dout, const void* y, const int32_t* idx, const int32_t* pos,
+    const float* gate, const uint8_t* kept, const int32_t* fill,
+    const int32_t* row_offsets, void* dy, float* dgate, int G, int S, int E,
+    int C, int N, int dtype, void* stream) {
+  MOE_REQUIRE(row_offsets, MESH_MOE_E_ARG,
+              "combine_backward_compact: null pointer");
+  return run_combine_backward(dout, y, idx, pos, gate, kept, fill, row_offsets,
+                              dy, dgate, G, S, E, C, N, dtype, stream);
+}
+
+static int run_combine_backward(
+    const void* dout, const void* y, const int32_t* idx, const int32_t* pos,
+    const float* gate, const uint8_t* kept, const int32_t* fill,
+    const int32_t* row_offsets, void* dy, float* dgate, int G, int S, int E,
+    int C, int N, int dtype, void* stream) {
   MOE_REQUIRE(dout && y && idx && pos && gate && kept && fill && dy && dgate,
               MESH_MOE_E_ARG, "combine_backward: null pointer");
   MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG,
@@ -711,7 +771,8 @@ extern "C" int mesh_moe_combine_backward(
               "combine_backward: bad sizes G=%d S=%d E=%d C=%d N=%d", G, S, E,
               C, N);
   const int64_t T_tokens = (int64_t)G * S;
-  const int64_t njobs = T_tokens + (int64_t)G * E;
+  const int64_t njobs =
+      T_tokens + (row_offsets != nullptr ? (int64_t)E * 256 : (int64_t)G * E);
   const int64_t nblocks = (njobs + BW_ROWS_PER_BLOCK - 1) / BW_ROWS_PER_BLOCK;
   MOE_REQUIRE(nblocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
               "combine_backward: too many rows (%lld)", (long long)njobs);
@@ -721,20 +782,48 @@ extern "C" int mesh_moe_combine_backward(
   if (dtype == MESH_MOE_F32)
     combine_backward_kernel<float><<<(unsigned)nblocks, 256, 0, st>>>(
         (const float*)dout, (const float*)y, idx, pos, gate, kept, fill,
-        (float*)dy, dgate, G, S, E, C, N, T_tokens, vec);
+        (float*)dy, dgate, G, S, E, C, N, T_tokens, vec, row_offsets);
   else
     combine_backward_kernel<bf16_t><<<(unsigned)nblocks, 256, 0, st>>>(
         (const bf16_t*)dout, (const bf16_t*)y, idx, pos, gate, kept, fill,
-        (bf16_t*)dy, dgate, G, S, E, C, N, T_tokens, vec);
+        (bf16_t*)dy, dgate, G, S, E, C, N, T_tokens, vec, row_offsets);
   MOE_CHECK_LAUNCH("combine_backward");
   return 0;
 }
+
+static int run_dispatch_backward(
+    const void* dexpert_in, const int32_t* idx, const int32_t* pos,
+    const float* gate, const uint8_t* kept, const int32_t* row_offsets,
+    const float* dlogits, const void* w_gate_packed, int groups_per_router,
+    void* dx, int G, int S, int E, int C, int M, int dtype, void* stream);
 
 extern "C" int mesh_moe_dispatch_backward(
     const void* dexpert_in, const int32_t* idx, const int32_t* pos,
     const float* gate, const uint8_t* kept, const float* dlogits,
     const void* w_gate_packed, int groups_per_router, void* dx, int G, int S,
     int E, int C, int M, int dtype, void* stream) {
+  return run_dispatch_backward(dexpert_in, idx, pos, gate, kept, nullptr,
+                               dlogits, w_gate_packed, groups_per_router, dx, G,
+                               S, E, C, M, dtype, stream);
+}
+
+extern "C" int mesh_moe_dispatch_backward_compact(
+    const void* dexpert_in, const int32_t* idx, const int32_t* pos,
+    const float* gate, const uint8_t* kept, const int32_t* row_offsets,
+    const float* dlogits, const void* w_gate_packed, int groups_per_router,
+    void* dx, int G, int S, int E, int C, int M, int dtype, void* stream) {
+  MOE_REQUIRE(row_offsets, MESH_MOE_E_ARG,
+              "dispatch_backward_compact: null pointer");
+  return run_dispatch_backward(dexpert_in, idx, pos, gate, kept, row_offsets,
+                               dlogits, w_gate_packed, groups_per_router, dx, G,
+                               S, E, C, M, dtype, stream);
+}
+
+static int run_dispatch_backward(
+    const void* dexpert_in, const int32_t* idx, const int32_t* pos,
+    const float* gate, const uint8_t* kept, const int32_t* row_offsets,
+    const float* dlogits, const void* w_gate_packed, int groups_per_router,
+    void* dx, int G, int S, int E, int C, int M, int dtype, void* stream) {
   MOE_REQUIRE(dexpert_in && idx && pos && gate && kept && dx, MESH_MOE_E_ARG,
               "dispatch_backward: null pointer");
   MOE_REQUIRE(w_gate_packed == nullptr ||
@@ -765,12 +854,12 @@ extern "C" int mesh_moe_dispatch_backward(
       dispatch_backward_router4_kernel<float><<<(unsigned)nb4, 256, 0, st>>>(
           (const float*)dexpert_in, idx, pos, gate, kept, dlogits,
           (const float*)w_gate_packed, (float*)dx, G, S, E, C, M, T_tokens,
-          groups_per_router);
+          groups_per_router, row_offsets);
     else
       dispatch_backward_router4_kernel<bf16_t><<<(unsigned)nb4, 256, 0, st>>>(
           (const bf16_t*)dexpert_in, idx, pos, gate, kept, dlogits,
           (const bf16_t*)w_gate_packed, (bf16_t*)dx, G, S, E, C, M, T_tokens,
-          groups_per_router);
+          groups_per_router, row_offsets);
     MOE_CHECK_LAUNCH("dispatch_backward (router share, 4 tokens per wavefront)");
     return 0;
   }
@@ -778,12 +867,12 @@ extern "C" int mesh_moe_dispatch_backward(
     dispatch_backward_kernel<float><<<(unsigned)nblocks, 256, 0, st>>>(
         (const float*)dexpert_in, idx, pos, gate, kept, dlogits,
         (const float*)w_gate_packed, (float*)dx, G, S, E, C, M, T_tokens,
-        groups_per_router, vec);
+        groups_per_router, vec, row_offsets);
   else
     dispatch_backward_kernel<bf16_t><<<(unsigned)nblocks, 256, 0, st>>>(
         (const bf16_t*)dexpert_in, idx, pos, gate, kept, dlogits,
         (const bf16_t*)w_gate_packed, (bf16_t*)dx, G, S, E, C, M, T_tokens,
-        groups_per_router, vec);
+        groups_per_router, vec, row_offsets);
   MOE_CHECK_LAUNCH("dispatch_backward");
   return 0;
 }

@@ -120,6 +120,23 @@ __device__ __forceinline__ uint32_t f32x2_to_bf16x2(float lo, float hi) {
 }
 
 // value of `f` after a cast to the activation dtype and back
+// Compacted expert rows (expert e's occupied slots, groups in order, at the
+// front of its row range; row_offsets[e][g] = occupied slots of the groups
+// before g): the number of occupied rows of expert e.
+__device__ __forceinline__ int compact_rows_used(const int32_t* fill,
+                                                 const int32_t* row_offsets,
+                                                 int e, int G, int E) {
+  return row_offsets[(int64_t)e * G + G - 1] + fill[(int64_t)(G - 1) * E + e];
+}
+// Row used + i if it lies between the occupied rows and the next multiple of
+// 256 (the rows of the last occupied 256-row tile that hold no slot), else -1.
+__device__ __forceinline__ int64_t compact_tail_row(int used, int i,
+                                                    int64_t rows) {
+  const int u = used & 255;
+  const int64_t row = (int64_t)used + i;
+  return (u == 0 || i >= 256 - u || row >= rows) ? -1 : row;
+}
+
 template <typename T>
 __device__ __forceinline__ float round_to(float f);
 template <>

@@ -17,6 +17,10 @@ constexpr int ROWS_PER_BLOCK = 4;  // one wavefront per row, 256 threads
 //   choice whose activation-dtype gate is exactly 0 gets a zero row: the
 //   reference's dispatch tensor is bool(combine), moe.py:1510-1511);
 // jobs [T, T + G*E): (g, e) zero-fills the slots fill[g,e] .. C-1.
+// With row_offsets (compacted rows: expert e's occupied slots of group g start
+// at row row_offsets[e][g] of its row range, as mesh_moe_compact_expert_ffn
+// lays them out) the zero jobs are [T, T + 256 E) instead: job (e, i) clears
+// row used(e) + i while that is below the next multiple of 256.
 // ---------------------------------------------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void dispatch_kernel(
@@ -24,10 +28,12 @@ __global__ __launch_bounds__(256) void dispatch_kernel(
     const int32_t* __restrict__ pos, const float* __restrict__ gate,
     const uint8_t* __restrict__ kept, const int32_t* __restrict__ fill,
     T* __restrict__ expert_in, float* __restrict__ slot_gate, int G, int S,
-    int E, int C, int M, int64_t T_tokens, bool vec) {
+    int E, int C, int M, int64_t T_tokens, bool vec,
+    const int32_t* __restrict__ row_offsets) {
   const int lane = threadIdx.x & 63;
   const int64_t job = (int64_t)blockIdx.x * ROWS_PER_BLOCK + (threadIdx.x >> 6);
-  const int64_t njobs = T_tokens + (int64_t)G * E;
+  const int64_t njobs =
+      T_tokens + (row_offsets != nullptr ? (int64_t)E * 256 : (int64_t)G * E);
   if (job >= njobs) return;
   if (job < T_tokens) {
     const int64_t t = job;
@@ -62,7 +68,10 @@ __global__ __launch_bounds__(256) void dispatch_kernel(
         const int e = k ? idx2.y : idx2.x;
         const int c = k ? pos2.y : pos2.x;
         const float w = round_to<T>(k ? gate2.y : gate2.x);
-        const int64_t slot = ((int64_t)e * G + g) * C + c;
+        const int64_t slot =
+            row_offsets == nullptr
+                ? ((int64_t)e * G + g) * C + c
+                : (int64_t)e * G * C + row_offsets[(int64_t)e * G + g] + c;
         dst[k] = expert_in + slot * M;
         zero[k] = (w == 0.0f);
         if (slot_gate != nullptr && lane == 0) slot_gate[slot] = w;
@@ -96,6 +105,22 @@ __global__ __launch_bounds__(256) void dispatch_kernel(
         if (dst[0]) dst[0][i] = zero[0] ? (T)0 : v;
         if (dst[1]) dst[1][i] = zero[1] ? (T)0 : v;
       }
+    }
+  } else if (row_offsets != nullptr) {
+    const int64_t j = job - T_tokens;
+    const int e = (int)(j >> 8);
+    const int64_t rows = (int64_t)G * C;
+    const int used = compact_rows_used(fill, row_offsets, e, G, E);
+    const int64_t row = compact_tail_row(used, (int)(j & 255), rows);
+    if (row < 0) return;
+    T* d = expert_in + ((int64_t)e * rows + row) * M;
+    if (vec) {
+      constexpr int VN = Vec16<T>::N;
+      uint4* d4 = reinterpret_cast<uint4*>(d);
+      const uint4 z = make_uint4(0, 0, 0, 0);
+      for (int i = lane; i < M / VN; i += 64) store_streaming(d4 + i, z);
+    } else {
+      for (int i = lane; i < M; i += 64) d[i] = (T)0;
     }
   } else {
     const int64_t ge = job - T_tokens;
@@ -254,12 +279,40 @@ static bool aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
 using namespace mesh_moe;
 
+static int run_dispatch(const void* x, const int32_t* idx, const int32_t* pos,
+                        const float* gate, const uint8_t* kept,
+                        const int32_t* fill, const int32_t* row_offsets,
+                        void* expert_in, float* slot_gate, int G, int S, int E,
+                        int C, int M, int dtype, void* stream);
+
 extern "C" int mesh_moe_dispatch(const void* x, const int32_t* idx,
                                  const int32_t* pos, const float* gate,
                                  const uint8_t* kept, const int32_t* fill,
                                  void* expert_in, float* slot_gate, int G,
                                  int S, int E, int C, int M, int dtype,
                                  void* stream) {
+  return run_dispatch(x, idx, pos, gate, kept, fill, nullptr, expert_in,
+                      slot_gate, G, S, E, C, M, dtype, stream);
+}
+
+extern "C" int mesh_moe_dispatch_compact(const void* x, const int32_t* idx,
+                                         const int32_t* pos, const float* gate,
+                                         const uint8_t* kept,
+                                         const int32_t* fill,
+                                         const int32_t* row_offsets,
+                                         void* expert_in, int G, int S, int E,
+                                         int C, int M, int dtype,
+                                         void* stream) {
+  MOE_REQUIRE(row_offsets, MESH_MOE_E_ARG, "dispatch_compact: null pointer");
+  return run_dispatch(x, idx, pos, gate, kept, fill, row_offsets, expert_in,
+                      nullptr, G, S, E, C, M, dtype, stream);
+}
+
+static int run_dispatch(const void* x, const int32_t* idx, const int32_t* pos,
+                        const float* gate, const uint8_t* kept,
+                        const int32_t* fill, const int32_t* row_offsets,
+                        void* expert_in, float* slot_gate, int G, int S, int E,
+                        int C, int M, int dtype, void* stream) {
   MOE_REQUIRE(x && idx && pos && gate && kept && fill && expert_in,
               MESH_MOE_E_ARG, "dispatch: null pointer");
   MOE_REQUIRE(valid_dtype(dtype), MESH_MOE_E_ARG, "dispatch: bad dtype %d",
@@ -267,7 +320,8 @@ extern "C" int mesh_moe_dispatch(const void* x, const int32_t* idx,
   MOE_REQUIRE(G >= 1 && S >= 1 && E >= 1 && C >= 1 && M >= 1, MESH_MOE_E_ARG,
               "dispatch: bad sizes G=%d S=%d E=%d C=%d M=%d", G, S, E, C, M);
   const int64_t T_tokens = (int64_t)G * S;
-  const int64_t njobs = T_tokens + (int64_t)G * E;
+  const int64_t njobs =
+      T_tokens + (row_offsets != nullptr ? (int64_t)E * 256 : (int64_t)G * E);
   const int64_t nblocks = (njobs + ROWS_PER_BLOCK - 1) / ROWS_PER_BLOCK;
   MOE_REQUIRE(nblocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
               "dispatch: too many rows (%lld)", (long long)njobs);
@@ -278,11 +332,11 @@ extern "C" int mesh_moe_dispatch(const void* x, const int32_t* idx,
   if (dtype == MESH_MOE_F32) {
     dispatch_kernel<float><<<(unsigned)nblocks, 256, 0, st>>>(
         (const float*)x, idx, pos, gate, kept, fill, (float*)expert_in,
-        slot_gate, G, S, E, C, M, T_tokens, vec);
+        slot_gate, G, S, E, C, M, T_tokens, vec, row_offsets);
   } else {
     dispatch_kernel<bf16_t><<<(unsigned)nblocks, 256, 0, st>>>(
         (const bf16_t*)x, idx, pos, gate, kept, fill, (bf16_t*)expert_in,
-        slot_gate, G, S, E, C, M, T_tokens, vec);
+        slot_gate, G, S, E, C, M, T_tokens, vec, row_offsets);
   }
   MOE_CHECK_LAUNCH("dispatch");
   return 0;

@@ -547,7 +547,11 @@ struct RingCfg {
 // conflicts) and the MFMA operands, which need 8 consecutive k per lane, are
 // read with ds_read_b64_tr_b16: within 16 lanes, lane t addresses the 8 bytes
 // at (row t / 4, elements 4 (t % 4) ..) of a 4 x 16 block and lane i receives
-// the block's column i.  R, N multiples of 8.
+// the block's column i.  R, N multiples of 8.  With k_extent, expert e's
+// reduction stops after its first k_extent[e] rows, rounded up to a K tile
+// (rows up to there must hold finite values in one operand and zeros in the
+// other); k_extent[e] == 0 gives an all-zero result.  k_extent is passed
+// in the place of row_map.
 //
 // MASKED: element (e, r, n) of the result is stored as zero unless
 // mask_src[e][r][n] > 0 (the backward of a ReLU whose output is mask_src,
@@ -567,6 +571,8 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
     const bf16_t* __restrict__ mask_src = nullptr,
     const int32_t* __restrict__ tile_list = nullptr) {
   using Cfg = RingCfg;
+  // KMAJOR kernels gather nothing: their row_map argument is k_extent
+  const int32_t* k_extent = KMAJOR ? row_map : nullptr;
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, WN = Cfg::WN;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
 
@@ -598,7 +604,10 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
   const int wave = tid >> 6;
   const int wm = wave / WN, wn = wave % WN;
   const int tiles_per_e = tiles_m * tiles_n;
-  const int nk = K / BK;
+  // K tiles of the current tile's reduction: all of K, or with k_extent
+  // (KMAJOR) the expert's first k_extent[e] reduction rows only
+  int nk = K / BK;
+  bool tile_empty = false;   // k_extent[e] == 0: the result is zero
 
   // per-tile state
   int row0, col0;
@@ -627,6 +636,13 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
     }
     row0 = tm * BM;
     col0 = tn * BN;
+    if constexpr (KMAJOR) {
+      if (k_extent != nullptr) {
+        const int used = k_extent[e];
+        tile_empty = used == 0;
+        nk = max(1, min(K / BK, (used + BK - 1) / BK));
+      }
+    }
     Ae = GATHER ? A : A + (int64_t)e * R * K;
     Be = B + (int64_t)e * N * K;
     Ce = Cout + (int64_t)e * R * N;
@@ -884,6 +900,18 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
     __syncthreads();
     const int out_row0 = row0, out_col0 = col0;
     bf16_t* out_c = Ce;
+    if constexpr (KMAJOR) {
+      // an expert without reduction rows: its one K tile held rows that
+      // nobody wrote
+      if (tile_empty) {
+#pragma unroll
+        for (int i = 0; i < Cfg::TM; ++i)
+#pragma unroll
+          for (int j = 0; j < Cfg::TN; ++j)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+      }
+    }
     const int next = tile + tile_step;
     const bool has_next = next < tile_end;
     if (has_next) {
@@ -1359,7 +1387,8 @@ static bool kmajor_path_applies(const void* A, const void* B, const void* C,
 }
 
 static int launch_ring_kmajor(const bf16_t* A, const bf16_t* B, bf16_t* C,
-                              int E, int R, int N, int K, hipStream_t st) {
+                              int E, int R, int N, int K, hipStream_t st,
+                              const int32_t* k_extent = nullptr) {
   using Cfg = RingCfg;
   const int tiles_m = (R + Cfg::BM - 1) / Cfg::BM;
   const int tiles_n = (N + Cfg::BN - 1) / Cfg::BN;
@@ -1372,8 +1401,8 @@ static int launch_ring_kmajor(const bf16_t* A, const bf16_t* B, bf16_t* C,
   auto k = grouped_gemm_bf16_ring_kernel<false, false, true>;
   MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
   k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
-      A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr,
-        nullptr, nullptr);
+      A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, k_extent, nullptr,
+      nullptr, nullptr);
   MOE_CHECK_LAUNCH("expert_ffn_backward (mfma, K-major operands)");
   return 0;
 }
@@ -1393,10 +1422,19 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
   const int cus = compute_units();
   if (cus == 0) return MESH_MOE_E_HIP;
   const unsigned blocks = (unsigned)(tiles < cus ? tiles : cus);
+  if (tile_list != nullptr && mask_src != nullptr) {
+    MOE_REQUIRE(!relu && row_map == nullptr, MESH_MOE_E_ARG,
+                "expert_ffn: masked result with relu or gathered rows");
+    auto k = grouped_gemm_bf16_ring_kernel<false, false, false, true, true>;
+    MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
+    k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
+        A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr,
+        mask_src, tile_list);
+    MOE_CHECK_LAUNCH("expert_ffn (mfma, listed tiles, masked result)");
+    return 0;
+  }
   if (tile_list != nullptr) {
     // listed tiles: the first GEMM gathers its rows, the second does not
-    MOE_REQUIRE(mask_src == nullptr, MESH_MOE_E_ARG,
-                "expert_ffn: tile list with a masked result");
 #define MOE_RING_LISTED(RELU_, GATHER_)                                        \
   do {                                                                         \
     auto k = grouped_gemm_bf16_ring_kernel<RELU_, GATHER_, false, false, true>; \
@@ -1731,6 +1769,16 @@ __global__ __launch_bounds__(1024) void tile_list_kernel(
     const int tn = rest % tiles_n, e = rest / tiles_n;
     if (tm < mt[e]) list[tiles_n * pre[e] + tn * mt[e] + tm] = i;
   }
+}
+
+// rows_used[e] from the row offsets of the last group and its fill count
+__global__ void rows_used_kernel(const int32_t* __restrict__ fill,
+                                 const int32_t* __restrict__ row_offsets,
+                                 int32_t* __restrict__ rows_used, int G, int E) {
+  const int e = blockIdx.x * blockDim.x + threadIdx.x;
+  if (e < E)
+    rows_used[e] = row_offsets[(int64_t)e * G + G - 1] +
+                   fill[(int64_t)(G - 1) * E + e];
 }
 
 static bool ring_path_applies(int R, int N, int K) {
@@ -2153,4 +2201,102 @@ extern "C" int mesh_moe_expert_ffn_backward(
   if (rc != 0) return rc;
   return grouped_gemm(tr_mn, tr_h, dwi, E, M, H, R, MESH_MOE_ACT_LINEAR, dtype,
                       st);
+}
+
+// ---------------------------------------------------------------------------
+// Backward of the expert feed-forward on COMPACTED rows (the row order of
+// mesh_moe_compact_expert_ffn): the two GEMMs whose result has token rows
+// (dh, dexpert_in) compute only the row tiles that hold occupied slots, the
+// two weight-gradient GEMMs reduce over every expert's occupied rows only.
+// ---------------------------------------------------------------------------
+static bool compact_backward_applies(int G, int E, int C, int M, int H, int N) {
+  if (G < 1 || E < 1 || E > 1024 || C < 1 || M < 1 || H < 1 || N < 1)
+    return false;
+  const int64_t rows = (int64_t)G * C;
+  if (rows > 0x7fffffffLL) return false;
+  const int R = (int)rows;
+  return ring_path_applies(R, H, N) && ring_path_applies(R, M, H) &&
+         kmajor_path_applies(nullptr, nullptr, nullptr, H, N, R,
+                             MESH_MOE_BF16) &&
+         kmajor_path_applies(nullptr, nullptr, nullptr, M, H, R, MESH_MOE_BF16);
+}
+
+extern "C" size_t mesh_moe_compact_expert_ffn_backward_workspace_bytes(
+    int G, int E, int C, int M, int H, int N) {
+  if (!compact_backward_applies(G, E, C, M, H, N)) return 0;
+  const size_t R = (size_t)G * C;
+  const size_t tm = (R + RingCfg::BM - 1) / RingCfg::BM;
+  const size_t tiles = (size_t)E * tm *
+                       ((size_t)(H + RingCfg::BN - 1) / RingCfg::BN +
+                        (size_t)(M + RingCfg::BN - 1) / RingCfg::BN);
+  return sizeof(bf16_t) * (size_t)E * R * H +
+         sizeof(int32_t) * ((size_t)E + tiles + 2 * 64) + 5 * 256;
+}
+
+extern "C" int mesh_moe_compact_expert_ffn_backward(
+    const void* expert_in, const void* h, const void* dy, const void* wi,
+    const void* wo, const int32_t* fill, const int32_t* row_offsets,
+    void* dexpert_in, void* dwi, void* dwo, int G, int E, int C, int M, int H,
+    int N, int activation, int dtype, void* workspace, size_t workspace_bytes,
+    void* stream) {
+  MOE_REQUIRE(expert_in && h && dy && wi && wo && fill && row_offsets &&
+                  dexpert_in && dwi && dwo && workspace, MESH_MOE_E_ARG,
+              "compact_expert_ffn_backward: null pointer");
+  MOE_REQUIRE(G >= 1 && E >= 1 && C >= 1 && M >= 1 && H >= 1 && N >= 1,
+              MESH_MOE_E_ARG, "compact_expert_ffn_backward: bad sizes");
+  MOE_REQUIRE(activation == MESH_MOE_ACT_RELU ||
+                  activation == MESH_MOE_ACT_LINEAR, MESH_MOE_E_UNSUPPORTED,
+              "compact_expert_ffn_backward: only relu and linear experts (got "
+              "%d)", activation);
+  MOE_REQUIRE(dtype == MESH_MOE_BF16 &&
+                  compact_backward_applies(G, E, C, M, H, N) &&
+                  (((uintptr_t)expert_in | (uintptr_t)h | (uintptr_t)dy |
+                    (uintptr_t)wi | (uintptr_t)wo | (uintptr_t)dexpert_in |
+                    (uintptr_t)dwi | (uintptr_t)dwo) % 16 == 0),
+              MESH_MOE_E_UNSUPPORTED,
+              "compact_expert_ffn_backward: needs bf16, at most 1024 experts "
+              "and shapes the 256 x 256 direct-to-LDS kernels take (rows=%lld "
+              "M=%d H=%d N=%d)", (long long)G * C, M, H, N);
+  MOE_REQUIRE(workspace_bytes >=
+                  mesh_moe_compact_expert_ffn_backward_workspace_bytes(
+                      G, E, C, M, H, N),
+              MESH_MOE_E_ARG, "compact_expert_ffn_backward: workspace too small");
+  hipStream_t st = (hipStream_t)stream;
+  const int R = G * C;
+  auto up = [](uintptr_t q) { return (q + 255) & ~(uintptr_t)255; };
+  bf16_t* dh = (bf16_t*)up((uintptr_t)workspace);
+  int32_t* rows_used = (int32_t*)up((uintptr_t)(dh + (size_t)E * R * H));
+  const int tiles_m = (R + RingCfg::BM - 1) / RingCfg::BM;
+  const int tn_h = (H + RingCfg::BN - 1) / RingCfg::BN;
+  const int tn_m = (M + RingCfg::BN - 1) / RingCfg::BN;
+  int32_t* list_h = (int32_t*)up((uintptr_t)(rows_used + E)) + 64;
+  int32_t* list_m =
+      (int32_t*)up((uintptr_t)(list_h + (size_t)E * tiles_m * tn_h)) + 64;
+  rows_used_kernel<<<(E + 255) / 256, 256, 0, st>>>(fill, row_offsets,
+                                                    rows_used, G, E);
+  MOE_CHECK_LAUNCH("compact_expert_ffn_backward (rows used)");
+  tile_list_kernel<<<1, 1024, 0, st>>>(rows_used, list_h, E, tiles_m, tn_h,
+                                       RingCfg::BM);
+  MOE_CHECK_LAUNCH("compact_expert_ffn_backward (tile list 1)");
+  tile_list_kernel<<<1, 1024, 0, st>>>(rows_used, list_m, E, tiles_m, tn_m,
+                                       RingCfg::BM);
+  MOE_CHECK_LAUNCH("compact_expert_ffn_backward (tile list 2)");
+  // dh = dy . wo^T on the listed row tiles, the ReLU mask on its stores (the
+  // rows of a listed tile past the expert's occupied ones have h = 0 and
+  // dy = 0)
+  int rc = launch_ring(
+      (const bf16_t*)dy, (const bf16_t*)wo, dh, E, R, H, N, false, st, nullptr,
+      nullptr, activation == MESH_MOE_ACT_RELU ? (const bf16_t*)h : nullptr,
+      list_h);
+  if (rc != 0) return rc;
+  // dexpert_in = dh . wi^T on the listed row tiles
+  rc = launch_ring(dh, (const bf16_t*)wi, (bf16_t*)dexpert_in, E, R, M, H,
+                   false, st, nullptr, nullptr, nullptr, list_m);
+  if (rc != 0) return rc;
+  // dwo = h^T . dy and dwi = expert_in^T . dh over the occupied rows
+  rc = launch_ring_kmajor((const bf16_t*)h, (const bf16_t*)dy, (bf16_t*)dwo, E,
+                          H, N, R, st, rows_used);
+  if (rc != 0) return rc;
+  return launch_ring_kmajor((const bf16_t*)expert_in, dh, (bf16_t*)dwi, E, M,
+                            H, R, st, rows_used);
 }

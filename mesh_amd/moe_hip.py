@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 26
+ABI_VERSION = 27
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -93,6 +93,24 @@ _SIGNATURES = {
     "mesh_moe_combine_compact": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
+    "mesh_moe_dispatch_compact": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
+    "mesh_moe_combine_backward_compact": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        _vp]),
+    "mesh_moe_compact_expert_ffn_backward_workspace_bytes": (ctypes.c_size_t, [
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int]),
+    "mesh_moe_compact_expert_ffn_backward": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
+    "mesh_moe_dispatch_backward_compact": (ctypes.c_int, [
+        _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, _vp]),
     "mesh_moe_expert_linear": (ctypes.c_int, [
         _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, _vp]),
@@ -268,12 +286,15 @@ class StageTimer(object):
   While a StageTimer is installed (`with StageTimer() as t:`), every stage
   records a start and an end event on the stream it launches on; `totals()`
   synchronises and returns {stage: (calls, milliseconds)}.  The last Routing
-  produced is kept in `routing` so that a benchmark can count kept slots.
+  produced is kept in `routing` so that a benchmark can count kept slots;
+  `compacted` counts the expert feed-forward calls that ran on compacted
+  rows (only the occupied slots multiplied).
   """
 
   def __init__(self):
     self.events = []
     self.routing = []
+    self.compacted = 0
 
   def __enter__(self):
     global _timer
@@ -614,8 +635,10 @@ def router_switch_gating(x, w_packed, group_size, capacity, importance=None,
   return (r, logits) if want_logits else r
 
 
-def dispatch(x, r, want_slot_gate=False, out=None):
-  """x [G, S, M] -> expert_in [E, G, C, M] (and slot_gate [E, G, C])."""
+def dispatch(x, r, want_slot_gate=False, out=None, row_offsets=None):
+  """x [G, S, M] -> expert_in [E, G, C, M] (and slot_gate [E, G, C]).  With
+  row_offsets [E, G] (from compact_expert_ffn) every expert's occupied slots
+  go to the front of its rows."""
   lib = load_library()
   g, s, m = x.shape
   e, c = r.num_experts, r.capacity
@@ -624,6 +647,16 @@ def dispatch(x, r, want_slot_gate=False, out=None):
   if out is None:
     out = torch.empty((e, g, c, m), dtype=x.dtype, device=x.device)
   op = _dev(out, "expert_in", x.dtype, (e, g, c, m))
+  if row_offsets is not None:
+    if want_slot_gate:
+      raise MoeHipError("dispatch: no slot gates with compacted rows")
+    ip, pp, gp, kp = _routing_ptrs(r, g, s)
+    with _stage("dispatch"):
+      _check(lib.mesh_moe_dispatch_compact(
+          xp, ip, pp, gp, kp, _dev(r.fill, "fill", torch.int32, (g, e)),
+          _dev(row_offsets, "row_offsets", torch.int32, (e, g)), op, g, s, e,
+          c, m, code, _stream()), "dispatch_compact")
+    return out
   slot_gate = None
   if want_slot_gate:
     slot_gate = torch.empty((e, g, c), dtype=torch.float32, device=x.device)
@@ -719,11 +752,26 @@ def dispatched_expert_ffn(x, r, wi_packed, wo_packed, activation="relu",
   return y
 
 
-def compact_expert_ffn(x, r, wi_packed, wo_packed, activation="relu"):
+def compact_training_applies(x, r, hidden_size, output_size,
+                             activation="relu"):
+  """True if a layer's gradient graph can stay on compacted rows: the forward
+  call compact_expert_ffn and the compacted gradient calls all take the
+  case."""
+  lib = load_library()
+  g, s, m = x.shape
+  e, c = r.num_experts, r.capacity
+  return (x.dtype == torch.bfloat16 and activation in ("relu", "linear") and
+          lib.mesh_moe_compact_expert_ffn_backward_workspace_bytes(
+              g, e, c, m, hidden_size, output_size) > 0)
+
+
+def compact_expert_ffn(x, r, wi_packed, wo_packed, activation="relu",
+                       want_hidden=False):
   """dispatch + expert_ffn on compacted rows (only the tiles that hold
   occupied slots are multiplied): x [G, S, M], the Routing r -> (y [E, G*C, N],
   row_offsets [E, G]) for combine(..., row_offsets=...), or None where the
-  library has no such kernel for the case."""
+  library has no such kernel for the case.  want_hidden: (y, row_offsets, h)
+  with the hidden tensor h [E, G*C, H] in the same row order."""
   lib = load_library()
   if activation not in ACTIVATIONS:
     raise ValueError("unsupported expert activation %r" % (activation,))
@@ -751,7 +799,9 @@ def compact_expert_ffn(x, r, wi_packed, wo_packed, activation="relu"):
   if rc == E_UNSUPPORTED:
     return None
   _check(rc, "compact_expert_ffn")
-  return y, row_offsets
+  if _timer is not None:
+    _timer.compacted += 1
+  return (y, row_offsets, h) if want_hidden else (y, row_offsets)
 
 
 def expert_linear(a, w_packed, activation="linear", y=None):
@@ -816,8 +866,10 @@ def _routing_ptrs(r, g, s):
           _dev(r.kept, "kept", torch.uint8, (g, s, 2)))
 
 
-def combine_backward(dout, y, r):
-  """dout [G, S, N], y [E, G, C, N] -> (dy [E, G, C, N], dgate [G, S, 2])."""
+def combine_backward(dout, y, r, row_offsets=None):
+  """dout [G, S, N], y [E, G, C, N] -> (dy [E, G, C, N], dgate [G, S, 2]).
+  With row_offsets [E, G], y and dy hold every expert's occupied slots
+  first."""
   lib = load_library()
   g, s, n = dout.shape
   e, _, c, _ = y.shape
@@ -825,6 +877,15 @@ def combine_backward(dout, y, r):
   dy = torch.empty_like(y)
   dgate = torch.empty((g, s, 2), dtype=torch.float32, device=y.device)
   ip, pp, gp, kp = _routing_ptrs(r, g, s)
+  if row_offsets is not None:
+    with _stage("combine_backward"):
+      _check(lib.mesh_moe_combine_backward_compact(
+          _dev(dout, "dout", dt, (g, s, n)), _dev(y, "y", dt, (e, g, c, n)),
+          ip, pp, gp, kp, _dev(r.fill, "fill", torch.int32, (g, e)),
+          _dev(row_offsets, "row_offsets", torch.int32, (e, g)),
+          dy.data_ptr(), dgate.data_ptr(), g, s, e, c, n, dtype_code(dt),
+          _stream()), "combine_backward_compact")
+    return dy, dgate
   with _stage("combine_backward"):
     _check(lib.mesh_moe_combine_backward(
         _dev(dout, "dout", dt, (g, s, n)), _dev(y, "y", dt, (e, g, c, n)),
@@ -881,6 +942,41 @@ def expert_ffn_backward(expert_in, h, dy, wi, wo, activation="relu",
         if dh_scale is not None else None, dxe.data_ptr(), dwi.data_ptr(),
         dwo.data_ptr(), e, rows, m, hdim, n, ACTIVATIONS[activation], code,
         ws.data_ptr(), ws_bytes, _stream()), "expert_ffn_backward")
+  return dxe, dwi, dwo
+
+
+def compact_expert_ffn_backward(expert_in, h, dy, wi, wo, r, row_offsets,
+                                activation="relu"):
+  """expert_ffn_backward with every [E, G*C, .] tensor in the compacted row
+  order of compact_expert_ffn (r: the Routing, row_offsets [E, G])."""
+  lib = load_library()
+  if activation not in ("relu", "linear"):
+    raise ValueError("unsupported expert activation %r" % (activation,))
+  e, rows, m = expert_in.shape
+  hdim, n = wo.shape[1], wo.shape[2]
+  g, c = row_offsets.shape[1], r.capacity
+  dt = expert_in.dtype
+  dev = expert_in.device
+  if rows != g * c or e != r.num_experts:
+    raise MoeHipError("compact_expert_ffn_backward: expert_in is [%d, %d, .], "
+                      "the routing has E=%d, G*C=%d"
+                      % (e, rows, r.num_experts, g * c))
+  dxe = torch.empty((e, rows, m), dtype=dt, device=dev)
+  dwi = torch.empty((e, m, hdim), dtype=dt, device=dev)
+  dwo = torch.empty((e, hdim, n), dtype=dt, device=dev)
+  ws_bytes = lib.mesh_moe_compact_expert_ffn_backward_workspace_bytes(
+      g, e, c, m, hdim, n)
+  ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
+  with _stage("expert_ffn_backward"):
+    _check(lib.mesh_moe_compact_expert_ffn_backward(
+        _dev(expert_in, "expert_in"), _dev(h, "h", dt, (e, rows, hdim)),
+        _dev(dy, "dy", dt, (e, rows, n)), _dev(wi, "wi", dt, (e, m, hdim)),
+        _dev(wo, "wo", dt, (e, hdim, n)),
+        _dev(r.fill, "fill", torch.int32, (g, e)),
+        _dev(row_offsets, "row_offsets", torch.int32, (e, g)), dxe.data_ptr(),
+        dwi.data_ptr(), dwo.data_ptr(), g, e, c, m, hdim, n,
+        ACTIVATIONS[activation], dtype_code(dt), ws.data_ptr(), ws_bytes,
+        _stream()), "compact_expert_ffn_backward")
   return dxe, dwi, dwo
 
 
@@ -991,9 +1087,10 @@ def router_backward_weights(x, dlogits):
 
 
 def dispatch_backward(dexpert_in, r, group_size, dlogits=None,
-                      w_gate_packed=None):
+                      w_gate_packed=None, row_offsets=None):
   """dexpert_in [E, G, C, M] (+ dlogits [G, S, E], w_gate_packed [B, E, M] with
-  one router per G / B consecutive groups) -> dx [G, S, M]."""
+  one router per G / B consecutive groups) -> dx [G, S, M].  With row_offsets
+  [E, G], dexpert_in holds every expert's occupied slots first."""
   lib = load_library()
   e, g, c, m = dexpert_in.shape
   s = group_size
@@ -1012,10 +1109,17 @@ def dispatch_backward(dexpert_in, r, group_size, dlogits=None,
     gpr = g // routers
     wgp = _dev(w_gate_packed, "w_gate_packed", dt, (routers, e, m))
   with _stage("dispatch_backward"):
-    _check(lib.mesh_moe_dispatch_backward(
-        _dev(dexpert_in, "dexpert_in"), ip, pp, gp, kp, dlp, wgp, gpr,
-        dx.data_ptr(), g, s, e, c, m, dtype_code(dt), _stream()),
-        "dispatch_backward")
+    if row_offsets is not None:
+      _check(lib.mesh_moe_dispatch_backward_compact(
+          _dev(dexpert_in, "dexpert_in"), ip, pp, gp, kp,
+          _dev(row_offsets, "row_offsets", torch.int32, (e, g)), dlp, wgp, gpr,
+          dx.data_ptr(), g, s, e, c, m, dtype_code(dt), _stream()),
+          "dispatch_backward_compact")
+    else:
+      _check(lib.mesh_moe_dispatch_backward(
+          _dev(dexpert_in, "dexpert_in"), ip, pp, gp, kp, dlp, wgp, gpr,
+          dx.data_ptr(), g, s, e, c, m, dtype_code(dt), _stream()),
+          "dispatch_backward")
   return dx
 
 

@@ -467,6 +467,20 @@ class MoEV1Operation(mtf.Operation):
       y = None
       noise = None
       row_offsets = None
+      expert_in = h = None
+      if (save and not by_slot and kwo_p is None and plain_hidden and
+          self._gating.router != "top_2" and
+          moe_hip.compact_training_applies(xg, r, wi_p.shape[1], n_,
+                                           self._activation)):
+        # one choice per token and a gradient to follow: the occupied slots at
+        # the front of every expert's rows in all the tensors the gradient
+        # operation reads, so that it too multiplies only those
+        compact = moe_hip.compact_expert_ffn(xg, r, wi_p, wo_p,
+                                             self._activation, want_hidden=True)
+        if compact is not None:
+          y, row_offsets, h = compact
+          expert_in = moe_hip.dispatch(xg, r, row_offsets=row_offsets)
+          expert_in = expert_in.reshape(e_, groups * c_, m_)
       if not (save or by_slot or kwo_p is not None) and plain_hidden:
         # nobody reads expert_in afterwards: fold the dispatch into the first
         # expert GEMM where the library can.  Routers with one choice per token
@@ -522,7 +536,8 @@ class MoEV1Operation(mtf.Operation):
         gate_noise = getattr(self._gating, "noise", None)
         gate_in = gate_noise.last if gate_noise is not None else None
         saved.update(x=xg, routing=r, logits=logits, importance=imp_s,
-                     expert_in=expert_in, h=h, y=y, w_gate_packed=wg_p,
+                     expert_in=expert_in, h=h, y=y, row_offsets=row_offsets,
+                     w_gate_packed=wg_p,
                      gate_in=gate_in, w_gate=wg_s, hidden_noise=noise)
       outs = (out.reshape(o_, g_, s_, n_), r.loss.to(dt).reshape(()))
       if kwo_p is not None:
@@ -627,10 +642,20 @@ class MoEV1GradOperation(mtf.Operation):
       by_slot = isinstance(r, moe_hip.SlotRouting)
       combine_backward = (moe_hip.slot_combine_backward if by_slot
                           else moe_hip.combine_backward)
+      # the forward pass may have put the occupied slots first in every
+      # tensor with slot rows
+      row_offsets = sv.get("row_offsets")
+      compact = {} if row_offsets is None else {"row_offsets": row_offsets}
       dy, dgate = combine_backward(
           dout_s.reshape(groups, s_, n_).contiguous(),
-          sv["y"].reshape(e_, groups, c_, n_), r)
-      if fwd._general_hidden:
+          sv["y"].reshape(e_, groups, c_, n_), r, **compact)
+      if row_offsets is not None:
+        dxe, dwi, dwo = moe_hip.compact_expert_ffn_backward(
+            sv["expert_in"].reshape(e_, groups * c_, m_), sv["h"],
+            dy.reshape(e_, groups * c_, n_), wi_s, wo_s, r, row_offsets,
+            fwd._activation)
+        dkwo, dwis = None, [dwi]
+      elif fwd._general_hidden:
         dys, wos = [dy.reshape(e_, groups * c_, n_)], [wo_s]
         if has_k:
           dyk, dgate_k = combine_backward(
@@ -682,7 +707,7 @@ class MoEV1GradOperation(mtf.Operation):
             sv["x"].reshape(tokens, m_), dlogits.reshape(tokens, e_))
         dx = dispatch_backward(
             dxe.reshape(e_, groups, c_, m_), r, s_, dlogits,
-            sv["w_gate_packed"].reshape(e_, m_))
+            sv["w_gate_packed"].reshape(e_, m_), **compact)
       else:
         # the router saw x * mult (a constant of the graph): its kernel's
         # gradient uses that input, and its share of d(tokens) is
@@ -692,7 +717,8 @@ class MoEV1GradOperation(mtf.Operation):
         dwg = moe_hip.router_backward_weights(
             x_gate.reshape(tokens, m_).contiguous(),
             dlogits.reshape(tokens, e_)).to(dt)
-        dx = dispatch_backward(dxe.reshape(e_, groups, c_, m_), r, s_)
+        dx = dispatch_backward(dxe.reshape(e_, groups, c_, m_), r, s_,
+                               **compact)
         w32 = sv["w_gate"].reshape(1, m_, e_).to(torch.float32).contiguous()
         dx_router = moe_hip.expert_linear(
             dlogits.reshape(1, tokens, e_), w32, "linear")   # [1, T, M]

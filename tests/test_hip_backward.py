@@ -25,9 +25,11 @@ def _hp(**kw):
   return O.default_hparams(**base)
 
 
-def run_backward(hip, x, w, hp, act_dtype, d_out, d_loss, nonpad, mb):
+def run_backward(hip, x, w, hp, act_dtype, d_out, d_loss, nonpad, mb,
+                 compact=False):
   """The forward and backward call sequence of one v1 layer through the C ABI
-  (what MoEV1Operation and its gradient do), on [G, S, M] tokens."""
+  (what MoEV1Operation and its gradient do), on [G, S, M] tokens.  compact: the
+  calls that keep every expert's occupied slots at the front of its rows."""
   g, s, m = x.shape
   e, hdim = hp.moe_num_experts, hp.moe_hidden_size
   n = w["wo"].shape[-1]
@@ -52,14 +54,26 @@ def run_backward(hip, x, w, hp, act_dtype, d_out, d_loss, nonpad, mb):
     r = hip.switch_gating(logits, c, importance=imp, z_loss=z,
                           num_microbatches=mb,
                           slots_by_gate=gating == "switch_max")
-  expert_in = hip.dispatch(xg, r)
-  h = torch.empty((e, g * c, hdim), dtype=xg.dtype, device="cuda")
-  y = hip.expert_ffn(expert_in.reshape(e, g * c, m), wi_p, wo_p, "relu", h=h)
-  # backward
   dout = H.to_gpu(d_out, act_dtype)
-  dy, dgate = hip.combine_backward(dout, y.reshape(e, g, c, n), r)
-  dxe, dwi, dwo = hip.expert_ffn_backward(
-      expert_in.reshape(e, g * c, m), h, dy.reshape(e, g * c, n), wi, wo, "relu")
+  ro = {}
+  if compact:
+    assert hip.compact_training_applies(xg, r, hdim, n, "relu")
+    y, row_offsets, h = hip.compact_expert_ffn(xg, r, wi_p, wo_p, "relu",
+                                               want_hidden=True)
+    ro = dict(row_offsets=row_offsets)
+    expert_in = hip.dispatch(xg, r, **ro)
+    dy, dgate = hip.combine_backward(dout, y.reshape(e, g, c, n), r, **ro)
+    dxe, dwi, dwo = hip.compact_expert_ffn_backward(
+        expert_in.reshape(e, g * c, m), h, dy.reshape(e, g * c, n), wi, wo, r,
+        row_offsets, "relu")
+  else:
+    expert_in = hip.dispatch(xg, r)
+    h = torch.empty((e, g * c, hdim), dtype=xg.dtype, device="cuda")
+    y = hip.expert_ffn(expert_in.reshape(e, g * c, m), wi_p, wo_p, "relu", h=h)
+    dy, dgate = hip.combine_backward(dout, y.reshape(e, g, c, n), r)
+    dxe, dwi, dwo = hip.expert_ffn_backward(
+        expert_in.reshape(e, g * c, m), h, dy.reshape(e, g * c, n), wi, wo,
+        "relu")
   dl = torch.tensor([d_loss], dtype=H.ACT_TORCH[act_dtype]).float().cuda()
   scale = torch.tensor(hp.moe_loss_coef, dtype=H.ACT_TORCH[act_dtype]).item()
   dlogits = hip.gating_backward(
@@ -69,7 +83,7 @@ def run_backward(hip, x, w, hp, act_dtype, d_out, d_loss, nonpad, mb):
   dwg = hip.router_backward_weights(xg.reshape(g * s, m),
                                     dlogits.reshape(g * s, e))
   dx = hip.dispatch_backward(dxe.reshape(e, g, c, m), r, s, dlogits,
-                             wg_p.reshape(e, m))
+                             wg_p.reshape(e, m), **ro)
   return dict(dx=H.to_np(dx), dw_gate=H.to_np(dwg), dwi=H.to_np(dwi),
               dwo=H.to_np(dwo), dlogits=H.to_np(dlogits), dgate=H.to_np(dgate))
 
@@ -145,6 +159,147 @@ def test_backward_matches_oracle(hip, case):
     atol = tol["atol"] * max(1.0, np.abs(ref).max())
     np.testing.assert_allclose(got[k], ref, rtol=tol["rtol"], atol=atol,
                                err_msg=k)
+
+
+COMPACT_CASES = [
+    # gating, G, S, M, H, E, capacity factor, padding mask
+    ("switch", 4, 512, 256, 512, 8, 2.0, True),
+    ("switch", 2, 1024, 256, 256, 4, 1.25, False),   # 640 rows per expert
+    ("ntlb", 4, 512, 256, 512, 8, 2.0, False),
+    ("switch_max", 4, 512, 256, 512, 8, 2.0, True),
+]
+
+
+@pytest.mark.parametrize("case", COMPACT_CASES, ids=[
+    "%s-%d" % (c[0], i) for i, c in enumerate(COMPACT_CASES)])
+def test_compact_backward_matches_oracle(hip, case):
+  """The gradient calls on compacted rows (one choice per token: the occupied
+  slots at the front of every expert's rows, the GEMMs over those only)
+  against the oracle's backward, and against the padded call sequence: the
+  token gradient bit for bit (every row's sums run in the same order), the
+  expert kernels' gradients to rounding (their sums over token rows are split
+  into other K tiles)."""
+  gating, g, s, m, hdim, e, cf, use_np = case
+  act_dtype = "bfloat16"
+  rng = np.random.default_rng(73)
+  w = dict(w_gate=H.normal_weights(rng, (m, e), m),
+           wi=H.normal_weights(rng, (e, m, hdim), m),
+           wo=H.normal_weights(rng, (e, hdim, m), hdim))
+  w["w_gate"][:, 0] *= 2.0          # a popular expert (overflows) ...
+  w["w_gate"][:, 1] *= 0.25         # ... and one few tokens choose
+  x = H.safe_tokens(rng, g * s, m, w["w_gate"], act_dtype,
+                    top=4 if gating == "ntlb" else 3).reshape(g, s, m)
+  nonpad = (rng.random((g, s)) < 0.85).astype(np.float32) if use_np else None
+  d_out = O.cast_act(rng.standard_normal((g, s, m)).astype(np.float32), act_dtype)
+  d_loss, mb = 1.5, 2
+  hp = _hp(moe_gating=gating, moe_num_experts=e, moe_hidden_size=hdim,
+           moe_group_size=s, moe_capacity_factor_train=cf, moe_loss_coef=0.25,
+           moe_ntlb_top_k=3,
+           moe_z_loss=0.1 if (gating == "switch" and use_np) else None)
+  want = O.moe_layer_v1_backward(x, w["w_gate"], w["wi"], w["wo"], hp, True,
+                                 act_dtype, d_out, d_loss, nonpadding=nonpad,
+                                 num_microbatches=mb)
+  got = run_backward(hip, x, w, hp, act_dtype, d_out, d_loss, nonpad, mb,
+                     compact=True)
+  padded = run_backward(hip, x, w, hp, act_dtype, d_out, d_loss, nonpad, mb)
+  for k in ("dx", "dgate", "dlogits"):
+    np.testing.assert_array_equal(got[k], padded[k], err_msg=k)
+  for k in ("dwi", "dwo", "dw_gate"):   # (the router's sums: atomic adds)
+    np.testing.assert_allclose(got[k], padded[k], rtol=2e-2,
+                               atol=2e-3 * np.abs(padded[k]).max(), err_msg=k)
+  tol = H.value_tolerance(act_dtype)
+  for k in ("dx", "dw_gate", "dwi", "dwo"):
+    ref = want[k].reshape(got[k].shape)
+    atol = tol["atol"] * max(1.0, np.abs(ref).max())
+    np.testing.assert_allclose(got[k], ref, rtol=tol["rtol"], atol=atol,
+                               err_msg=k)
+
+
+def test_compact_gradient_calls_edge_fills(hip):
+  """Row counts per expert chosen by hand: none (its kernels' gradients are
+  exactly zero), one, a whole 256-row tile, every row, and counts that end
+  inside a K tile of 64; each compacted call against its padded counterpart
+  at the occupied slots, bit for bit where the sums run in the same order."""
+  g, s, e, c, m, hdim = 2, 1024, 8, 256, 256, 512
+  counts = np.array([[128, 0, 256, 1, 100, 200, 255, 84],
+                     [128, 0, 256, 0, 91, 256, 255, 38]])
+  assert (counts.sum(1) == s).all() and (counts <= c).all()
+  rng = np.random.default_rng(5)
+  logits = 0.01 * rng.standard_normal((g, s, e)).astype(np.float32)
+  for gi in range(g):
+    owner = rng.permutation(np.repeat(np.arange(e), counts[gi]))
+    logits[gi, np.arange(s), owner] += 6.0
+  lg = torch.from_numpy(logits).cuda()
+  r = hip.switch_gating(lg, c)
+  fill = H.to_np(r.fill)
+  np.testing.assert_array_equal(fill, counts)
+  dt = torch.bfloat16
+  gen = torch.Generator(device="cuda").manual_seed(9)
+  def rand(*shape, scale=1.0):
+    return (torch.randn(shape, device="cuda", generator=gen) * scale).to(dt)
+  xg = rand(g, s, m)
+  wi, wo = rand(e, m, hdim, scale=m ** -0.5), rand(e, hdim, m, scale=hdim ** -0.5)
+  wi_p, wo_p = hip.pack_weights(wi, dt), hip.pack_weights(wo, dt)
+  dout = rand(g, s, m)
+  assert hip.compact_training_applies(xg, r, hdim, m, "relu")
+  y_c, ro, h_c = hip.compact_expert_ffn(xg, r, wi_p, wo_p, "relu",
+                                        want_hidden=True)
+  want_ro = np.concatenate([np.zeros((e, 1), np.int64),
+                            np.cumsum(counts.T, axis=1)[:, :-1]], axis=1)
+  np.testing.assert_array_equal(H.to_np(ro), want_ro)
+  xe_c = hip.dispatch(xg, r, row_offsets=ro).reshape(e, g * c, m)
+  xe_p = hip.dispatch(xg, r).reshape(e, g, c, m)
+  h_p = torch.empty((e, g * c, hdim), dtype=dt, device="cuda")
+  y_p = hip.expert_ffn(xe_p.reshape(e, g * c, m), wi_p, wo_p, "relu", h=h_p)
+  dy_c, dgate_c = hip.combine_backward(dout, y_c.reshape(e, g, c, m), r,
+                                       row_offsets=ro)
+  dy_p, dgate_p = hip.combine_backward(dout, y_p.reshape(e, g, c, m), r)
+  dxe_c, dwi_c, dwo_c = hip.compact_expert_ffn_backward(
+      xe_c, h_c, dy_c.reshape(e, g * c, m), wi, wo, r, ro, "relu")
+  dxe_p, dwi_p, dwo_p = hip.expert_ffn_backward(
+      xe_p.reshape(e, g * c, m), h_p, dy_p.reshape(e, g * c, m), wi, wo, "relu")
+  dx_c = hip.dispatch_backward(dxe_c.reshape(e, g, c, m), r, s, row_offsets=ro)
+  dx_p = hip.dispatch_backward(dxe_p.reshape(e, g, c, m), r, s)
+
+  def occupied(t_c, t_p):
+    """(compacted rows, the same slots of the padded tensor) per expert."""
+    t_c = t_c.reshape(e, g * c, -1)
+    t_p = t_p.reshape(e, g, c, -1)
+    for ei in range(e):
+      rows = torch.cat([t_p[ei, gi, :counts[gi, ei]] for gi in range(g)])
+      yield ei, t_c[ei, :rows.shape[0]], rows
+  for name, t_c, t_p in (("expert_in", xe_c, xe_p), ("h", h_c, h_p),
+                         ("y", y_c, y_p), ("dy", dy_c, dy_p),
+                         ("dexpert_in", dxe_c, dxe_p)):
+    for ei, a, b in occupied(t_c, t_p):
+      assert torch.equal(a, b), (name, ei)
+  # the zero rows up to the end of the last occupied 256-row tile
+  for t_c in (xe_c, dy_c.reshape(e, g * c, m)):
+    for ei in range(e):
+      used = int(counts[:, ei].sum())
+      end = min(g * c, -(-used // 256) * 256)
+      assert not t_c[ei, used:end].any(), ei
+  assert torch.equal(dgate_c, dgate_p)
+  assert torch.equal(dx_c, dx_p)
+  assert not dwi_c[1].any() and not dwo_c[1].any()    # the expert without rows
+  for name, a, b in (("dwi", dwi_c, dwi_p), ("dwo", dwo_c, dwo_p)):
+    a, b = a.float(), b.float()
+    assert torch.isfinite(a).all(), name
+    np.testing.assert_allclose(H.to_np(a), H.to_np(b), rtol=2e-2,
+                               atol=2e-3 * float(b.abs().max()), err_msg=name)
+  # against float64 sums over the occupied rows
+  for ei, xa, _ in occupied(xe_c, xe_p):
+    used = xa.shape[0]
+    hd = h_c[ei, :used].double()
+    dyd = dy_c.reshape(e, g * c, m)[ei, :used].double()
+    dh = (dyd @ wo[ei].double().T) * (hd > 0)
+    np.testing.assert_allclose(
+        H.to_np(dwo_c[ei].float()), H.to_np((hd.T @ dyd).float()), rtol=2e-2,
+        atol=1e-2 * max(1e-6, float((hd.T @ dyd).abs().max())), err_msg=str(ei))
+    np.testing.assert_allclose(
+        H.to_np(dwi_c[ei].float()), H.to_np((xa.double().T @ dh).float()),
+        rtol=2e-2, atol=1e-2 * max(1e-6, float((xa.double().T @ dh).abs().max())),
+        err_msg=str(ei))
 
 
 @pytest.mark.parametrize("use_importance", [False, True])

@@ -791,18 +791,34 @@ def test_v1_switch_max_matches_oracle():
     ("top_2+hidden_dropout", "bfloat16", 110),
     ("switch+hidden_dropout", "float32", 111),
     ("top_2+second_place_loss", "float32", 112),
-    ("top_2+second_place_loss", "bfloat16", 113)],
+    ("top_2+second_place_loss", "bfloat16", 113),
+    # shapes the matrix-core kernels take: one choice per token keeps the
+    # gradient graph on compacted rows
+    ("switch+compact", "bfloat16", 114), ("ntlb+compact", "bfloat16", 115),
+    ("switch+compact+input_jitter", "bfloat16", 116)],
     ids=lambda c: "%s-%s" % (c[0], c[1]))
-def test_v1_gradients_match_oracle(case):
+def test_v1_gradients_match_oracle(case, monkeypatch):
   """mtf.gradients over the layer (outputs and loss) against the oracle's
   backward, which central differences pin in tests/test_oracle.py."""
   gating, act_dtype, seed = case
   gating, _, noise_policy = gating.partition("+")
+  compact = noise_policy.startswith("compact")
+  if compact:
+    noise_policy = noise_policy.partition("+")[2]
   hidden_dropout = noise_policy == "hidden_dropout"
   loss2 = noise_policy == "second_place_loss"
   if hidden_dropout or loss2:
     noise_policy = ""
   b, l, m, hdim, e, group = 2, 64, 32, 48, 4, 32
+  compact_calls = []
+  if compact:
+    b, l, m, hdim, e, group = 2, 1024, 256, 512, 4, 1024
+    from mesh_amd import moe_hip
+    inner = moe_hip.compact_expert_ffn_backward
+    def counted(*args, **kwargs):
+      compact_calls.append(1)
+      return inner(*args, **kwargs)
+    monkeypatch.setattr(moe_hip, "compact_expert_ffn_backward", counted)
   rng = np.random.default_rng(seed)
   w = dict(w_gate=H.normal_weights(rng, (m, e), m),
            wi=H.normal_weights(rng, (e, m, hdim), m),
@@ -880,6 +896,7 @@ def test_v1_gradients_match_oracle(case):
     np.testing.assert_allclose(out_got, out_want,
                                **H.value_tolerance(act_dtype))
   tol = H.value_tolerance(act_dtype)
+  assert len(compact_calls) == (1 if compact else 0)
   for g_, k in zip(got, ("dx", "dw_gate", "dwi", "dwo")):
     ref = want[k].reshape(g_.shape)
     np.testing.assert_allclose(
