@@ -302,6 +302,61 @@ def test_compact_gradient_calls_edge_fills(hip):
         err_msg=str(ei))
 
 
+def test_full_size_compact_backward(hip):
+  """Eight experts of configuration 4 at their real sizes (32 groups, capacity
+  64: 2048 slot rows per expert, d_model 4096, d_ff 16384) behind a switch
+  router that fills one expert and a third of the others: the compacted calls
+  against the padded ones.  Token gradients and gate gradients bit for bit;
+  the experts' kernel gradients to rounding; every occupied row of the
+  intermediate tensors bit for bit."""
+  g, s, e, c, m, hdim = 32, 256, 8, 64, 4096, 16384
+  dt = torch.bfloat16
+  gen = torch.Generator(device="cuda").manual_seed(31)
+  mk = lambda *shape: torch.randn(shape, generator=gen, device="cuda")
+  logits = mk(g, s, e)
+  logits[..., 0] += 1.2        # a popular expert: some of its groups overflow
+  r = hip.switch_gating(logits, c)
+  fill = r.fill.cpu().numpy()
+  used = fill.sum(0)
+  # (one expert with every slot taken, the others about a third full)
+  assert (fill < c).any() and (fill == c).any() and used.min() < g * c // 2
+  xg = mk(g, s, m).to(dt)
+  wi = (mk(e, m, hdim) / m ** 0.5).to(dt)
+  wo = (mk(e, hdim, m) / hdim ** 0.5).to(dt)
+  dout = mk(g, s, m).to(dt)
+  wi_p, wo_p = hip.pack_weights(wi, dt), hip.pack_weights(wo, dt)
+  assert hip.compact_training_applies(xg, r, hdim, m, "relu")
+  y_c, ro, h_c = hip.compact_expert_ffn(xg, r, wi_p, wo_p, "relu",
+                                        want_hidden=True)
+  xe_c = hip.dispatch(xg, r, row_offsets=ro).reshape(e, g * c, m)
+  dy_c, dgate_c = hip.combine_backward(dout, y_c.reshape(e, g, c, m), r,
+                                       row_offsets=ro)
+  dxe_c, dwi_c, dwo_c = hip.compact_expert_ffn_backward(
+      xe_c, h_c, dy_c.reshape(e, g * c, m), wi, wo, r, ro, "relu")
+  dx_c = hip.dispatch_backward(dxe_c.reshape(e, g, c, m), r, s, row_offsets=ro)
+  del y_c, dxe_c
+  xe_p = hip.dispatch(xg, r).reshape(e, g * c, m)
+  h_p = torch.empty((e, g * c, hdim), dtype=dt, device="cuda")
+  y_p = hip.expert_ffn(xe_p, wi_p, wo_p, "relu", h=h_p)
+  dy_p, dgate_p = hip.combine_backward(dout, y_p.reshape(e, g, c, m), r)
+  dxe_p, dwi_p, dwo_p = hip.expert_ffn_backward(
+      xe_p, h_p, dy_p.reshape(e, g * c, m), wi, wo, "relu")
+  dx_p = hip.dispatch_backward(dxe_p.reshape(e, g, c, m), r, s)
+  assert torch.equal(dx_c, dx_p) and torch.equal(dgate_c, dgate_p)
+  assert dx_c.abs().sum() > 0
+  # the hidden tensor's occupied rows, expert by expert
+  for ei in (0, e - 1):
+    rows = torch.cat([h_p.reshape(e, g, c, hdim)[ei, gi, :fill[gi, ei]]
+                      for gi in range(g)])
+    assert torch.equal(h_c[ei, :rows.shape[0]], rows)
+  for name, a, b in (("dwi", dwi_c, dwi_p), ("dwo", dwo_c, dwo_p)):
+    a, b = a.float(), b.float()
+    assert bool(torch.isfinite(a).all()), name
+    err = (a - b).abs().max().item()
+    assert err <= 2e-2 * b.abs().max().item(), (name, err)
+    assert (a - b).abs().mean().item() <= 2e-3 * b.abs().mean().item(), name
+
+
 @pytest.mark.parametrize("use_importance", [False, True])
 def test_gating_backward_second_place_loss(hip, use_importance):
   """d(logits) of the balancing loss alone (zero gate gradients), with the
