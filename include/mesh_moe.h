@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 27
+#define MESH_MOE_ABI_VERSION 28
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -641,11 +641,16 @@ int mesh_moe_router_backward_weights(const void* x, const float* dlogits,
  *   one router per groups_per_router consecutive groups (G for a single
  *   router; the inner level of the hierarchical layer has one per outer
  *   expert, moe.py:743-753); dx [G,S,M] dtype
+ *   w_gate [G / groups_per_router, M, E] dtype or NULL: the same router
+ *   kernels in their variable layout.  Given them, bf16 calls with
+ *   M % 256 == 0, E % 16 == 0, E <= 128 and S % 32 == 0 compute the router's
+ *   share on the matrix cores (d(logits) as two bf16 terms; sums in another
+ *   order than the other kernels', equal to rounding).
  */
 int mesh_moe_dispatch_backward(const void* dexpert_in, const int32_t* idx,
                                const int32_t* pos, const float* gate,
                                const uint8_t* kept, const float* dlogits,
-                               const void* w_gate_packed,
+                               const void* w_gate_packed, const void* w_gate,
                                int groups_per_router, void* dx, int G, int S,
                                int E, int C, int M, int dtype, void* stream);
 
@@ -696,8 +701,9 @@ int mesh_moe_compact_expert_ffn_backward(
 int mesh_moe_dispatch_backward_compact(
     const void* dexpert_in, const int32_t* idx, const int32_t* pos,
     const float* gate, const uint8_t* kept, const int32_t* row_offsets,
-    const float* dlogits, const void* w_gate_packed, int groups_per_router,
-    void* dx, int G, int S, int E, int C, int M, int dtype, void* stream);
+    const float* dlogits, const void* w_gate_packed, const void* w_gate,
+    int groups_per_router, void* dx, int G, int S, int E, int C, int M,
+    int dtype, void* stream);
 
 /*
  * ---------------------------------------------------------------------------

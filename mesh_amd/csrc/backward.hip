@@ -326,6 +326,197 @@ __global__ __launch_bounds__(256) void dispatch_backward_router4_kernel(
   }
 }
 
+// The same for bfloat16 with the router's share on the matrix cores
+// (v_mfma_f32_32x32x16_bf16).  The share of 32 tokens x 256 columns,
+// sum_e dlogits[t][e] * w_gate[m][e], is a product whose two operands both lie
+// in memory with e innermost: the router kernel in its variable layout
+// [M, E] and d(logits) [T, E].  The block copies its 256 kernel rows and 32
+// d(logits) rows to LDS with whole-line loads (lanes reading their 8
+// consecutive e straight from global memory touch 32 lines per instruction and
+// ask for every line four times: 0.59 against 0.49 ms for 65536 tokens of 4096)
+// and the lanes take their operands from there.  The float32 d(logits) go in as two bfloat16 terms
+// (hi = bf16(d), lo = bf16(d - hi): the products are exact in the float32
+// accumulator, what is dropped is below 2^-17 |d|).  The instruction leaves a
+// lane with 4 consecutive columns of one token; the tile goes through LDS as
+// float32 (over the kernel rows, which are no longer needed) so that the
+// second phase -- half a wavefront per token row, 16 bytes per lane, the rows
+// of d(expert_in) added -- reads and writes whole rows.  The rows' loads are
+// issued before the first phase, whose latency they hide.  KS = E / 16.
+// Needs M % 256 == 0, E % 16 == 0, E <= DBM_MAX_E, S % 32 == 0 (the 32 tokens
+// share a group).
+constexpr int DBM_TOK = 32, DBM_COLS = 256, DBM_MAX_E = 128;
+constexpr int DBM_LD = DBM_COLS + 4;     // floats per LDS row of the share
+typedef __attribute__((ext_vector_type(8))) __bf16 dbm_bf16x8_t;
+typedef float dbm_f32x16_t __attribute__((ext_vector_type(16)));
+
+// LDS bytes: [kernel rows | share] then the d(logits) rows
+static size_t dbm_lds_bytes(int E) {
+  const size_t wbytes = (size_t)DBM_COLS * (E * 2 + 16);
+  const size_t sbytes = sizeof(float) * DBM_TOK * DBM_LD;
+  return (wbytes > sbytes ? wbytes : sbytes) + (size_t)DBM_TOK * (E * 4 + 16);
+}
+
+// (Four token tiles per block with the kernel rows kept in registers and the
+// next tile's loads in flight: 0.60 against 0.50 ms.)
+template <int KS>
+__global__ __launch_bounds__(256) void dispatch_backward_mfma_kernel(
+    const bf16_t* __restrict__ dxe, const int32_t* __restrict__ idx,
+    const int32_t* __restrict__ pos, const float* __restrict__ gate,
+    const uint8_t* __restrict__ kept, const float* __restrict__ dlogits,
+    const bf16_t* __restrict__ wg, bf16_t* __restrict__ dx, int G, int S,
+    int C, int M, int64_t T_tokens, int groups_per_router,
+    const int32_t* __restrict__ row_offsets) {
+  constexpr int E = KS * 16;
+  constexpr int WROW = E * 2 + 16, DROW = E * 4 + 16;   // padded LDS rows, bytes
+  constexpr int WBYTES = DBM_COLS * WROW;
+  constexpr int SBYTES = (int)sizeof(float) * DBM_TOK * DBM_LD;
+  extern __shared__ __attribute__((aligned(16))) unsigned char dbm_smem[];
+  unsigned char* wl = dbm_smem;
+  float* share = reinterpret_cast<float*>(dbm_smem);
+  unsigned char* dl = dbm_smem + (WBYTES > SBYTES ? WBYTES : SBYTES);
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, l32 = lane & 31;
+  const int64_t t0 = (int64_t)blockIdx.y * DBM_TOK;
+  const int m0 = blockIdx.x * DBM_COLS;
+  const int g = (int)(t0 / S);
+  wg += (int64_t)(g / groups_per_router) * M * E;
+
+  constexpr int WPR = E / 8;                  // 16-byte pieces per kernel row
+  constexpr int WP = DBM_COLS * WPR / 256;    // pieces per thread (= E / 8)
+  constexpr int DPR = E / 4;                  // pieces per d(logits) row
+  constexpr int DP = (DBM_TOK * DPR + 255) / 256;
+  constexpr int RP = DBM_TOK / 8;
+  const uint4 z = make_uint4(0, 0, 0, 0);
+
+  // the loads of the token tile: its d(logits) rows (16-byte pieces,
+  // consecutive threads consecutive pieces) and the rows of d(expert_in) this
+  // lane adds in phase 2 (token rows wave * 8 + 2 j + half, 8 columns from
+  // column 8 l32 of the tile)
+  auto load_tile = [&](float4 (&dv)[DP], uint4 (&v)[RP][2]) {
+#pragma unroll
+    for (int i = 0; i < DP; ++i) {
+      const int p = tid + 256 * i;
+      const int64_t t = t0 + p / DPR;
+      dv[i] = make_float4(0.f, 0.f, 0.f, 0.f);
+      if (p < DBM_TOK * DPR && t < T_tokens)
+        dv[i] = reinterpret_cast<const float4*>(dlogits + t0 * E)[p];
+    }
+#pragma unroll
+    for (int j = 0; j < RP; ++j) {
+      const int64_t t = t0 + wave * 8 + 2 * j + half;
+      v[j][0] = z;
+      v[j][1] = z;
+      if (t >= T_tokens) continue;
+      // the token's record in one round trip (both choices of every array)
+      const uint16_t kept2 = *reinterpret_cast<const uint16_t*>(kept + t * 2);
+      const int2 idx2 = *reinterpret_cast<const int2*>(idx + t * 2);
+      const int2 pos2 = *reinterpret_cast<const int2*>(pos + t * 2);
+      const float2 gate2 = *reinterpret_cast<const float2*>(gate + t * 2);
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        if (((kept2 >> (8 * k)) & 0xff) &&
+            round_to<bf16_t>(k ? gate2.y : gate2.x) != 0.0f) {
+          const int64_t e = k ? idx2.y : idx2.x;
+          const int64_t slot =
+              (row_offsets == nullptr ? (e * G + g) * C
+                                      : e * G * C + row_offsets[e * G + g]) +
+              (k ? pos2.y : pos2.x);
+          v[j][k] = load_streaming(
+              reinterpret_cast<const uint4*>(dxe + slot * M + m0) + l32);
+        }
+      }
+    }
+  };
+
+  // ---- the kernel rows: global -> LDS -> this lane's operands
+  uint4 afrag[2][KS];
+  {
+    uint4 wv[WP];
+#pragma unroll
+    for (int i = 0; i < WP; ++i)
+      wv[i] = reinterpret_cast<const uint4*>(wg + (int64_t)m0 * E)[tid + 256 * i];
+#pragma unroll
+    for (int i = 0; i < WP; ++i) {
+      const int p = tid + 256 * i;
+      *reinterpret_cast<uint4*>(wl + (p / WPR) * WROW + (p % WPR) * 16) = wv[i];
+    }
+  }
+  float4 dv[DP];
+  uint4 v[RP][2];
+  load_tile(dv, v);
+  __syncthreads();
+#pragma unroll
+  for (int b = 0; b < 2; ++b)
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks)
+      afrag[b][ks] = *reinterpret_cast<const uint4*>(
+          wl + (wave * 64 + b * 32 + l32) * WROW + ks * 32 + half * 16);
+  // (the share goes over the kernel rows: the next barrier stands between
+  // these reads and its first write)
+  {
+    // ---- phase 1: this wavefront's 32 tokens x 64 columns of the share
+#pragma unroll
+    for (int i = 0; i < DP; ++i) {
+      const int p = tid + 256 * i;
+      if (p < DBM_TOK * DPR)
+        *reinterpret_cast<float4*>(dl + (p / DPR) * DROW + (p % DPR) * 16) = dv[i];
+    }
+    __syncthreads();
+    dbm_f32x16_t acc[2];
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int r = 0; r < 16; ++r) acc[b][r] = 0.f;
+#pragma unroll
+    for (int ks = 0; ks < KS; ++ks) {
+      const float4 d0 = *reinterpret_cast<const float4*>(dl + l32 * DROW + ks * 64 + half * 32);
+      const float4 d1 = *reinterpret_cast<const float4*>(dl + l32 * DROW + ks * 64 + half * 32 + 16);
+      const float d[8] = {d0.x, d0.y, d0.z, d0.w, d1.x, d1.y, d1.z, d1.w};
+      float lo[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) lo[j] = d[j] - round_to<bf16_t>(d[j]);
+      const dbm_bf16x8_t bh = __builtin_bit_cast(dbm_bf16x8_t, pack16(d, bf16_t()));
+      const dbm_bf16x8_t bl = __builtin_bit_cast(dbm_bf16x8_t, pack16(lo, bf16_t()));
+#pragma unroll
+      for (int b = 0; b < 2; ++b) {
+        const dbm_bf16x8_t a = __builtin_bit_cast(dbm_bf16x8_t, afrag[b][ks]);
+        acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, bh, acc[b], 0, 0, 0);
+        acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, bl, acc[b], 0, 0, 0);
+      }
+    }
+    // lane: token l32, columns 32 b + 8 q + 4 half + 0..3 of the wavefront's 64
+#pragma unroll
+    for (int b = 0; b < 2; ++b)
+#pragma unroll
+      for (int q = 0; q < 4; ++q)
+        *reinterpret_cast<float4*>(
+            &share[l32 * DBM_LD + wave * 64 + b * 32 + q * 8 + half * 4]) =
+            make_float4(acc[b][4 * q], acc[b][4 * q + 1], acc[b][4 * q + 2],
+                        acc[b][4 * q + 3]);
+    __syncthreads();
+
+    // ---- phase 2
+#pragma unroll
+    for (int j = 0; j < RP; ++j) {
+      const int row = wave * 8 + 2 * j + half;
+      const int64_t t = t0 + row;
+      if (t >= T_tokens) continue;
+      const float* sh = &share[row * DBM_LD + l32 * 8];
+      const float4 s0 = *reinterpret_cast<const float4*>(sh);
+      const float4 s1 = *reinterpret_cast<const float4*>(sh + 4);
+      // (the order of the one-token kernel: the rows first, then the share)
+      float a[8], b[8], o[8];
+      unpack16(v[j][0], a, bf16_t());
+      unpack16(v[j][1], b, bf16_t());
+      const float sv[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
+#pragma unroll
+      for (int q = 0; q < 8; ++q) o[q] = (a[q] + b[q]) + sv[q];
+      store_streaming(reinterpret_cast<uint4*>(dx + t * M + m0) + l32,
+                      pack16(o, bf16_t()));
+    }
+  }
+}
+
 // ---------------------------------------------------------------------------
 // gating backward.
 // Step 1, one block per group: how many tokens count for density_1 of each
@@ -602,6 +793,126 @@ __global__ __launch_bounds__(256) void router_wgrad_mfma_kernel(
 }
 
 // ---------------------------------------------------------------------------
+// The same product for bfloat16 tokens on the bfloat16 matrix cores
+// (v_mfma_f32_32x32x16_bf16, 16 tokens per instruction instead of 2).  The
+// float32 d(logits) go in as two bfloat16 terms, hi = bf16(d) and
+// lo = bf16(d - hi): x * hi and x * lo are exact in the float32 accumulator and
+// what is left of d, at most 2^-17 |d|, is below the rounding of the sum
+// itself.  Both operands lie in memory with the reduction index (the token)
+// outermost; they are staged in LDS as they lie and the instruction's
+// operands (8 consecutive tokens of one kernel row / one expert per lane) are
+// read with ds_read_b64_tr_b16: within 16 lanes, lane t addresses the 8 bytes
+// at (row t / 4, elements 4 (t % 4) ..) of a 4 x 16 block and lane i receives
+// the block's column i.  Block = 128 kernel rows x 64 experts x WB_TOK tokens,
+// 32 tokens staged at a time; a wavefront owns 32 rows x 64 experts.  Rows are
+// padded so that the four rows of a block lie in different banks.
+// Needs M % 128 == 0, E % 8 == 0 and 16-byte aligned rows.
+// ---------------------------------------------------------------------------
+constexpr int WB_M = 128, WB_TOK = 2048, WB_KT = 32;
+constexpr int WB_XS = (WB_M + 32) * 2;   // bytes per staged token row of x
+constexpr int WB_DS = (64 + 16) * 2;     // ... of one half of d(logits)
+typedef __attribute__((ext_vector_type(8))) __bf16 wb_bf16x8_t;
+typedef short wb_i16x4_t __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) void wb_lds_void_t;
+
+// 8 consecutive rows of this lane's column: rows 0-3 of the block at byte
+// offset OFF from addr, rows 4-7 at OFF + ROW4
+template <int OFF, int ROW4>
+__device__ __forceinline__ wb_bf16x8_t lds_read_tr8(uint32_t addr) {
+  wb_i16x4_t lo, hi;
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2"
+               : "=v"(lo) : "v"(addr), "n"(OFF) : "memory");
+  asm volatile("ds_read_b64_tr_b16 %0, %1 offset:%2"
+               : "=v"(hi) : "v"(addr), "n"(OFF + ROW4) : "memory");
+  return __builtin_bit_cast(
+      wb_bf16x8_t, __builtin_shufflevector(lo, hi, 0, 1, 2, 3, 4, 5, 6, 7));
+}
+
+__global__ __launch_bounds__(256) void router_wgrad_bf16_kernel(
+    const bf16_t* __restrict__ x, const float* __restrict__ dlogits,
+    float* __restrict__ acc_out, int64_t T_tokens, int M, int E) {
+  __shared__ __attribute__((aligned(16))) unsigned char xs[WB_KT * WB_XS];
+  __shared__ __attribute__((aligned(16))) unsigned char dhs[WB_KT * WB_DS];
+  __shared__ __attribute__((aligned(16))) unsigned char dls[WB_KT * WB_DS];
+  const int m0 = blockIdx.x * WB_M, e0 = blockIdx.z * 64;
+  const int64_t t0 = (int64_t)blockIdx.y * WB_TOK;
+  const int64_t t1 = t0 + WB_TOK < T_tokens ? t0 + WB_TOK : T_tokens;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int half = lane >> 5, l32 = lane & 31;
+  wm_f32x16_t acc0, acc1;
+#pragma unroll
+  for (int r = 0; r < 16; ++r) { acc0[r] = 0.f; acc1[r] = 0.f; }
+  // staging: thread -> (token row tid / 8, 16 kernel rows / 8 experts)
+  const int sr = tid >> 3, sc = tid & 7;
+  // transposed reads: this lane's row and first column within a 16 x 32 block
+  const int t16 = lane & 15, g16 = lane >> 4;
+  const int rrow = (g16 >> 1) * 8 + (t16 >> 2);
+  const int rcol = (g16 & 1) * 16 + 4 * (t16 & 3);
+  const uint32_t xa = (uint32_t)(size_t)(wb_lds_void_t*)xs + rrow * WB_XS +
+                      (wave * 32 + rcol) * 2;
+  const uint32_t ha = (uint32_t)(size_t)(wb_lds_void_t*)dhs + rrow * WB_DS +
+                      rcol * 2;
+  const uint32_t la = (uint32_t)(size_t)(wb_lds_void_t*)dls + rrow * WB_DS +
+                      rcol * 2;
+  const uint4 z4 = make_uint4(0, 0, 0, 0);
+  for (int64_t tb = t0; tb < t1; tb += WB_KT) {
+    const int64_t t = tb + sr;
+    uint4 xv0 = z4, xv1 = z4, dh = z4, dl = z4;
+    if (t < t1) {
+      const uint4* xp = reinterpret_cast<const uint4*>(x + t * M + m0 + sc * 16);
+      xv0 = xp[0];
+      xv1 = xp[1];
+      if (e0 + sc * 8 < E) {
+        const float4 a = *reinterpret_cast<const float4*>(dlogits + t * E + e0 + sc * 8);
+        const float4 b = *reinterpret_cast<const float4*>(dlogits + t * E + e0 + sc * 8 + 4);
+        const float d[8] = {a.x, a.y, a.z, a.w, b.x, b.y, b.z, b.w};
+        float lo[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) lo[j] = d[j] - round_to<bf16_t>(d[j]);
+        dh = pack16(d, bf16_t());
+        dl = pack16(lo, bf16_t());
+      }
+    }
+    __syncthreads();                 // the previous batch has been consumed
+    *reinterpret_cast<uint4*>(xs + sr * WB_XS + sc * 32) = xv0;
+    *reinterpret_cast<uint4*>(xs + sr * WB_XS + sc * 32 + 16) = xv1;
+    *reinterpret_cast<uint4*>(dhs + sr * WB_DS + sc * 16) = dh;
+    *reinterpret_cast<uint4*>(dls + sr * WB_DS + sc * 16) = dl;
+    __syncthreads();
+    // 16 tokens per step: the x operand and, per 32 experts, hi and lo
+    const wb_bf16x8_t a0 = lds_read_tr8<0, 4 * WB_XS>(xa);
+    const wb_bf16x8_t h00 = lds_read_tr8<0, 4 * WB_DS>(ha);
+    const wb_bf16x8_t l00 = lds_read_tr8<0, 4 * WB_DS>(la);
+    const wb_bf16x8_t h01 = lds_read_tr8<64, 4 * WB_DS>(ha);
+    const wb_bf16x8_t l01 = lds_read_tr8<64, 4 * WB_DS>(la);
+    const wb_bf16x8_t a1 = lds_read_tr8<16 * WB_XS, 4 * WB_XS>(xa);
+    const wb_bf16x8_t h10 = lds_read_tr8<16 * WB_DS, 4 * WB_DS>(ha);
+    const wb_bf16x8_t l10 = lds_read_tr8<16 * WB_DS, 4 * WB_DS>(la);
+    const wb_bf16x8_t h11 = lds_read_tr8<16 * WB_DS + 64, 4 * WB_DS>(ha);
+    const wb_bf16x8_t l11 = lds_read_tr8<16 * WB_DS + 64, 4 * WB_DS>(la);
+    // the compiler does not count the asm reads: wait for them here
+    __builtin_amdgcn_sched_barrier(0);
+    __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+    __builtin_amdgcn_sched_barrier(0);
+    acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, h00, acc0, 0, 0, 0);
+    acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, h01, acc1, 0, 0, 0);
+    acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, l00, acc0, 0, 0, 0);
+    acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, l01, acc1, 0, 0, 0);
+    acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, h10, acc0, 0, 0, 0);
+    acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, h11, acc1, 0, 0, 0);
+    acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, l10, acc0, 0, 0, 0);
+    acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, l11, acc1, 0, 0, 0);
+  }
+#pragma unroll
+  for (int r = 0; r < 16; ++r) {
+    const int m = m0 + wave * 32 + 8 * (r / 4) + 4 * half + (r % 4);
+    if (e0 + l32 < E) atomicAdd(acc_out + (int64_t)m * E + e0 + l32, acc0[r]);
+    if (e0 + 32 + l32 < E)
+      atomicAdd(acc_out + (int64_t)m * E + e0 + 32 + l32, acc1[r]);
+  }
+}
+
+// ---------------------------------------------------------------------------
 // router projection backward w.r.t. the kernel: dw[m,e] = sum_t x[t,m] *
 // dlogits[t,e], float32.  Block (m tile of 256, chunk of tokens, chunk of 64
 // experts) accumulates 256 x 64 partial sums and adds them to the float32
@@ -794,36 +1105,41 @@ static int run_combine_backward(
 static int run_dispatch_backward(
     const void* dexpert_in, const int32_t* idx, const int32_t* pos,
     const float* gate, const uint8_t* kept, const int32_t* row_offsets,
-    const float* dlogits, const void* w_gate_packed, int groups_per_router,
-    void* dx, int G, int S, int E, int C, int M, int dtype, void* stream);
+    const float* dlogits, const void* w_gate_packed, const void* w_gate,
+    int groups_per_router, void* dx, int G, int S, int E, int C, int M,
+    int dtype, void* stream);
 
 extern "C" int mesh_moe_dispatch_backward(
     const void* dexpert_in, const int32_t* idx, const int32_t* pos,
     const float* gate, const uint8_t* kept, const float* dlogits,
-    const void* w_gate_packed, int groups_per_router, void* dx, int G, int S,
-    int E, int C, int M, int dtype, void* stream) {
+    const void* w_gate_packed, const void* w_gate, int groups_per_router,
+    void* dx, int G, int S, int E, int C, int M, int dtype, void* stream) {
   return run_dispatch_backward(dexpert_in, idx, pos, gate, kept, nullptr,
-                               dlogits, w_gate_packed, groups_per_router, dx, G,
-                               S, E, C, M, dtype, stream);
+                               dlogits, w_gate_packed, w_gate,
+                               groups_per_router, dx, G, S, E, C, M, dtype,
+                               stream);
 }
 
 extern "C" int mesh_moe_dispatch_backward_compact(
     const void* dexpert_in, const int32_t* idx, const int32_t* pos,
     const float* gate, const uint8_t* kept, const int32_t* row_offsets,
-    const float* dlogits, const void* w_gate_packed, int groups_per_router,
-    void* dx, int G, int S, int E, int C, int M, int dtype, void* stream) {
+    const float* dlogits, const void* w_gate_packed, const void* w_gate,
+    int groups_per_router, void* dx, int G, int S, int E, int C, int M,
+    int dtype, void* stream) {
   MOE_REQUIRE(row_offsets, MESH_MOE_E_ARG,
               "dispatch_backward_compact: null pointer");
   return run_dispatch_backward(dexpert_in, idx, pos, gate, kept, row_offsets,
-                               dlogits, w_gate_packed, groups_per_router, dx, G,
-                               S, E, C, M, dtype, stream);
+                               dlogits, w_gate_packed, w_gate,
+                               groups_per_router, dx, G, S, E, C, M, dtype,
+                               stream);
 }
 
 static int run_dispatch_backward(
     const void* dexpert_in, const int32_t* idx, const int32_t* pos,
     const float* gate, const uint8_t* kept, const int32_t* row_offsets,
-    const float* dlogits, const void* w_gate_packed, int groups_per_router,
-    void* dx, int G, int S, int E, int C, int M, int dtype, void* stream) {
+    const float* dlogits, const void* w_gate_packed, const void* w_gate,
+    int groups_per_router, void* dx, int G, int S, int E, int C, int M,
+    int dtype, void* stream) {
   MOE_REQUIRE(dexpert_in && idx && pos && gate && kept && dx, MESH_MOE_E_ARG,
               "dispatch_backward: null pointer");
   MOE_REQUIRE(w_gate_packed == nullptr ||
@@ -848,6 +1164,37 @@ static int run_dispatch_backward(
                    bw_aligned16(dexpert_in) && bw_aligned16(dx) &&
                    (w_gate_packed == nullptr || bw_aligned16(w_gate_packed));
   hipStream_t st = (hipStream_t)stream;
+  if (vec && dlogits != nullptr && w_gate != nullptr &&
+      dtype == MESH_MOE_BF16 && bw_aligned16(w_gate) &&
+      bw_aligned16(dlogits) && E % 16 == 0 && E <= DBM_MAX_E &&
+      M % DBM_COLS == 0 && S % DBM_TOK == 0 &&
+      (T_tokens + DBM_TOK - 1) / DBM_TOK <= 65535) {
+    dim3 grid((unsigned)(M / DBM_COLS),
+              (unsigned)((T_tokens + DBM_TOK - 1) / DBM_TOK));
+    const size_t lds = dbm_lds_bytes(E);
+#define MOE_DBM(KS_)                                                         \
+  do {                                                                       \
+    auto k = dispatch_backward_mfma_kernel<KS_>;                             \
+    MOE_ALLOW_LDS(k, lds);                                                   \
+    k<<<grid, 256, lds, st>>>(                                               \
+        (const bf16_t*)dexpert_in, idx, pos, gate, kept, dlogits,            \
+        (const bf16_t*)w_gate, (bf16_t*)dx, G, S, C, M, T_tokens,            \
+        groups_per_router, row_offsets);                                     \
+  } while (0)
+    switch (E / 16) {
+      case 1: MOE_DBM(1); break;
+      case 2: MOE_DBM(2); break;
+      case 3: MOE_DBM(3); break;
+      case 4: MOE_DBM(4); break;
+      case 5: MOE_DBM(5); break;
+      case 6: MOE_DBM(6); break;
+      case 7: MOE_DBM(7); break;
+      default: MOE_DBM(8); break;
+    }
+#undef MOE_DBM
+    MOE_CHECK_LAUNCH("dispatch_backward (router share on the matrix cores)");
+    return 0;
+  }
   if (vec && dlogits != nullptr && E <= DBR_MAX_E && S % DBR_TOK == 0) {
     const int64_t nb4 = (T_tokens + 4 * DBR_TOK - 1) / (4 * DBR_TOK);
     if (dtype == MESH_MOE_F32)
@@ -982,9 +1329,12 @@ extern "C" int mesh_moe_router_backward_weights(const void* x,
       MOE_CHECK_LAUNCH("router_backward_weights (mfma)");
       convert_f32_kernel<float><<<fb, 256, 0, st>>>(workspace, (float*)dw_gate, n);
     } else {
-      router_wgrad_mfma_kernel<bf16_t><<<mgrid, 256, 0, st>>>(
+      const int64_t bchunks = (tokens + WB_TOK - 1) / WB_TOK;
+      dim3 bgrid((unsigned)(M / WB_M), (unsigned)bchunks,
+                 (unsigned)((E + 63) / 64));
+      router_wgrad_bf16_kernel<<<bgrid, 256, 0, st>>>(
           (const bf16_t*)x, dlogits, workspace, tokens, M, E);
-      MOE_CHECK_LAUNCH("router_backward_weights (mfma)");
+      MOE_CHECK_LAUNCH("router_backward_weights (mfma, bf16 terms)");
       convert_f32_kernel<bf16_t><<<fb, 256, 0, st>>>(workspace, (bf16_t*)dw_gate,
                                                     n);
     }

@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 27
+ABI_VERSION = 28
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -108,7 +108,7 @@ _SIGNATURES = {
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
     "mesh_moe_dispatch_backward_compact": (ctypes.c_int, [
-        _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp,
+        _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, _vp]),
     "mesh_moe_expert_linear": (ctypes.c_int, [
@@ -182,7 +182,7 @@ _SIGNATURES = {
         _vp, _vp, _vp, _vp, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, _vp]),
     "mesh_moe_dispatch_backward": (ctypes.c_int, [
-        _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp, ctypes.c_int,
+        _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, _vp, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         _vp]),
     "mesh_moe_expert_choice_workspace_bytes": (ctypes.c_size_t, [
@@ -1087,17 +1087,20 @@ def router_backward_weights(x, dlogits):
 
 
 def dispatch_backward(dexpert_in, r, group_size, dlogits=None,
-                      w_gate_packed=None, row_offsets=None):
+                      w_gate_packed=None, row_offsets=None, w_gate=None):
   """dexpert_in [E, G, C, M] (+ dlogits [G, S, E], w_gate_packed [B, E, M] with
   one router per G / B consecutive groups) -> dx [G, S, M].  With row_offsets
-  [E, G], dexpert_in holds every expert's occupied slots first."""
+  [E, G], dexpert_in holds every expert's occupied slots first.  w_gate
+  [B, M, E]: the router kernels as the variables hold them, in the activation
+  dtype; with them the library may take the router's share of dx on the matrix
+  cores."""
   lib = load_library()
   e, g, c, m = dexpert_in.shape
   s = group_size
   dt = dexpert_in.dtype
   dx = torch.empty((g, s, m), dtype=dt, device=dexpert_in.device)
   ip, pp, gp, kp = _routing_ptrs(r, g, s)
-  dlp = wgp = None
+  dlp = wgp = wgv = None
   gpr = g
   if dlogits is not None:
     dlp = _dev(dlogits, "dlogits", torch.float32, (g, s, e))
@@ -1108,16 +1111,20 @@ def dispatch_backward(dexpert_in, r, group_size, dlogits=None,
       raise MoeHipError("dispatch_backward: %d groups, %d routers" % (g, routers))
     gpr = g // routers
     wgp = _dev(w_gate_packed, "w_gate_packed", dt, (routers, e, m))
+    if w_gate is not None:
+      if w_gate.dim() == 2:
+        w_gate = w_gate.reshape(1, m, e)
+      wgv = _dev(w_gate, "w_gate", dt, (routers, m, e))
   with _stage("dispatch_backward"):
     if row_offsets is not None:
       _check(lib.mesh_moe_dispatch_backward_compact(
           _dev(dexpert_in, "dexpert_in"), ip, pp, gp, kp,
-          _dev(row_offsets, "row_offsets", torch.int32, (e, g)), dlp, wgp, gpr,
-          dx.data_ptr(), g, s, e, c, m, dtype_code(dt), _stream()),
+          _dev(row_offsets, "row_offsets", torch.int32, (e, g)), dlp, wgp, wgv,
+          gpr, dx.data_ptr(), g, s, e, c, m, dtype_code(dt), _stream()),
           "dispatch_backward_compact")
     else:
       _check(lib.mesh_moe_dispatch_backward(
-          _dev(dexpert_in, "dexpert_in"), ip, pp, gp, kp, dlp, wgp, gpr,
+          _dev(dexpert_in, "dexpert_in"), ip, pp, gp, kp, dlp, wgp, wgv, gpr,
           dx.data_ptr(), g, s, e, c, m, dtype_code(dt), _stream()),
           "dispatch_backward")
   return dx

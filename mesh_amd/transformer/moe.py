@@ -705,6 +705,10 @@ class MoEV1GradOperation(mtf.Operation):
       if sv["gate_in"] is None:
         dwg = moe_hip.router_backward_weights(
             sv["x"].reshape(tokens, m_), dlogits.reshape(tokens, e_))
+        if not by_slot:
+          # the router kernel as the variable holds it, [M, E]
+          compact = dict(compact, w_gate=sv["w_gate"].reshape(m_, e_).to(
+              sv["x"].dtype).contiguous())
         dx = dispatch_backward(
             dxe.reshape(e_, groups, c_, m_), r, s_, dlogits,
             sv["w_gate_packed"].reshape(e_, m_), **compact)
@@ -950,7 +954,9 @@ class MoEV2Operation(mtf.Operation):
         saved.update(x=xg, rx=rx, ry=ry, logits_x=logits_x, logits_y=logits_y,
                      importance=imp_s, slot_gate=slot_gate, inputs_y=inputs_y,
                      ein_y=ein_y, h=h, yy=yy, out_y=out_y,
-                     w_outer_packed=w_outer_p, w_inner_packed=w_inner_p)
+                     w_outer_packed=w_outer_p, w_inner_packed=w_inner_p,
+                     w_outer=wo_s.reshape(1, m_, x_e).to(dt).contiguous(),
+                     w_inner=wi_s.reshape(x_e, m_, y_e).to(dt).contiguous())
       return out.reshape(a0, g1, s_, n_), loss
 
     args = [lowering.tensors[x], lowering.tensors[w_outer],
@@ -1024,7 +1030,7 @@ class MoEV2GradOperation(mtf.Operation):
           for i in range(x_e)])                           # [x, m, y]
       d_inputs_y = moe_hip.dispatch_backward(
           dein_y.reshape(y_e, x_e * h0, d_, m_), ry, t_, dlogits_y,
-          sv["w_inner_packed"])
+          sv["w_inner_packed"], w_gate=sv["w_inner"])
       dlogits_x = moe_hip.gating_backward(
           sv["logits_x"], rx, dgate_x, dl, 1.0, router="top_2",
           importance=sv["importance"],
@@ -1034,7 +1040,7 @@ class MoEV2GradOperation(mtf.Operation):
           sv["x"].reshape(ag * s_, m_), dlogits_x.reshape(ag * s_, x_e))
       dx = moe_hip.dispatch_backward(
           d_inputs_y.reshape(x_e, ag, c_, m_), rx, s_, dlogits_x,
-          sv["w_outer_packed"])
+          sv["w_outer_packed"], w_gate=sv["w_outer"])
       return (dx.reshape(a0, g1, s_, m_), dw_outer, dw_inner,
               dwi.reshape(wi_s.shape), dwo.reshape(wo_s.shape))
 

@@ -83,7 +83,7 @@ def run_backward(hip, x, w, hp, act_dtype, d_out, d_loss, nonpad, mb,
   dwg = hip.router_backward_weights(xg.reshape(g * s, m),
                                     dlogits.reshape(g * s, e))
   dx = hip.dispatch_backward(dxe.reshape(e, g, c, m), r, s, dlogits,
-                             wg_p.reshape(e, m), **ro)
+                             wg_p.reshape(e, m), w_gate=wg.reshape(m, e), **ro)
   return dict(dx=H.to_np(dx), dw_gate=H.to_np(dwg), dwi=H.to_np(dwi),
               dwo=H.to_np(dwo), dlogits=H.to_np(dlogits), dgate=H.to_np(dgate))
 
@@ -116,6 +116,8 @@ CASES = [
     ("switch", 2, 128, 64, 128, 8, 1.25, "bfloat16", False),
     ("switch_max", 2, 64, 16, 24, 4, 0.75, "float32", True),
     ("top_2", 2, 256, 256, 512, 8, 1.0, "bfloat16", True),   # MFMA GEMM paths
+    # the router's share of d(tokens) on the matrix cores (512 columns, 16 experts)
+    ("top_2", 2, 256, 512, 256, 16, 1.0, "bfloat16", True),
     ("ntlb", 2, 96, 16, 24, 6, 1.0, "float32", True),
     ("ntlb", 2, 128, 64, 128, 8, 0.75, "bfloat16", False),
 ]
@@ -300,6 +302,42 @@ def test_compact_gradient_calls_edge_fills(hip):
         H.to_np(dwi_c[ei].float()), H.to_np((xa.double().T @ dh).float()),
         rtol=2e-2, atol=1e-2 * max(1e-6, float((xa.double().T @ dh).abs().max())),
         err_msg=str(ei))
+
+
+@pytest.mark.parametrize("shape", [(4, 512, 1024, 64, 12), (3, 96, 512, 16, 8),
+                                   (2, 64, 1536, 128, 1)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_dispatch_backward_router_share_on_matrix_cores(hip, shape):
+  """d(tokens) = the rows of d(expert_in) + d(logits) . w_gate^T with the
+  second term on the bfloat16 matrix cores (d(logits) as two bfloat16 terms):
+  against float64 arithmetic rounded once, and against the kernel that does
+  the term in float32 multiply-adds (equal up to one rounding step of the
+  result)."""
+  g, s, m, e, c = shape
+  dt = torch.bfloat16
+  gen = torch.Generator(device="cuda").manual_seed(17)
+  mk = lambda *sh: torch.randn(sh, generator=gen, device="cuda")
+  r = hip.top2_gating(mk(g, s, e), c)
+  dxe = mk(e, g, c, m).to(dt)
+  dlogits = mk(g, s, e) * 3.0
+  w = (mk(m, e) / m ** 0.5).to(dt)
+  w_p = hip.pack_weights(w.reshape(1, m, e), dt).reshape(e, m)
+  got = hip.dispatch_backward(dxe, r, s, dlogits, w_p, w_gate=w)
+  plain = hip.dispatch_backward(dxe, r, s, dlogits, w_p)
+  # float64 reference
+  idx, pos = r.idx.long(), r.pos.long()
+  on = (r.kept != 0) & (r.gate.to(dt) != 0)
+  gi = torch.arange(g, device="cuda").view(g, 1, 1).expand(g, s, 2)
+  rows = dxe.double()[idx, gi, pos.clamp(0, c - 1)] * on.unsqueeze(-1)
+  want = rows.sum(2) + dlogits.double() @ w.double().t()
+  assert on.any() and not on.all()
+  err = (got.double() - want).abs()
+  # one rounding of the result (half a unit in the last place of bfloat16)
+  # on top of float32 sums of terms of size ~10
+  assert bool((err <= want.abs() * 2.0 ** -8 * 1.01 + 2e-5).all())
+  step = (got.float() - plain.float()).abs()
+  assert bool((step <= plain.float().abs() * 2.0 ** -7 + 4e-5).all())
+  assert float((step > 0).float().mean()) < 0.02
 
 
 def test_full_size_compact_backward(hip):
