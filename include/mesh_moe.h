@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 28
+#define MESH_MOE_ABI_VERSION 29
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -460,6 +460,9 @@ int mesh_moe_slot_combine(const void* y, const int16_t* tok_slot,
  * mesh_moe_slot_dispatch_backward: dx[g,s,:] = sum over the slots holding the
  *   token of dexpert_in[e,g,c,:] (+ dlogits[g,s,:] . w_gate^T when dlogits and
  *   w_gate_packed [E,M] are given), float32 accumulate, one rounding.
+ *   w_gate [M,E] dtype or NULL: the router kernel in its variable layout; with
+ *   it, as in mesh_moe_dispatch_backward, bf16 calls of the shapes named there
+ *   take the router's share on the matrix cores.
  * mesh_moe_expert_choice_backward: d(logits) [G,S,E] float32 from dweight and
  *   from the gradient of the returned loss (d_loss [1] float32 on the device,
  *   loss_scale = moe_loss_coef): the softmax runs over the group's tokens per
@@ -475,8 +478,9 @@ int mesh_moe_slot_combine_backward(const void* dout, const void* y,
 int mesh_moe_slot_dispatch_backward(const void* dexpert_in,
                                     const int16_t* tok_slot,
                                     const float* dlogits,
-                                    const void* w_gate_packed, void* dx, int G,
-                                    int S, int E, int C, int M, int dtype,
+                                    const void* w_gate_packed,
+                                    const void* w_gate, void* dx, int G, int S,
+                                    int E, int C, int M, int dtype,
                                     void* stream);
 size_t mesh_moe_expert_choice_backward_workspace_bytes(int G, int S, int E);
 int mesh_moe_expert_choice_backward(const float* logits, const void* importance,

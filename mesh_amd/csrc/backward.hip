@@ -358,14 +358,18 @@ static size_t dbm_lds_bytes(int E) {
 
 // (Four token tiles per block with the kernel rows kept in registers and the
 // next tile's loads in flight: 0.60 against 0.50 ms.)
-template <int KS>
+// SLOT: the rows of a token are named by the token -> slot table of the
+// expert-selection router (tok_slot [T, E] int16, -1 = not chosen by that
+// expert; any number of rows per token) instead of the per-token record.
+template <int KS, bool SLOT = false>
 __global__ __launch_bounds__(256) void dispatch_backward_mfma_kernel(
     const bf16_t* __restrict__ dxe, const int32_t* __restrict__ idx,
     const int32_t* __restrict__ pos, const float* __restrict__ gate,
     const uint8_t* __restrict__ kept, const float* __restrict__ dlogits,
     const bf16_t* __restrict__ wg, bf16_t* __restrict__ dx, int G, int S,
     int C, int M, int64_t T_tokens, int groups_per_router,
-    const int32_t* __restrict__ row_offsets) {
+    const int32_t* __restrict__ row_offsets,
+    const int16_t* __restrict__ tok_slot = nullptr) {
   constexpr int E = KS * 16;
   constexpr int WROW = E * 2 + 16, DROW = E * 4 + 16;   // padded LDS rows, bytes
   constexpr int WBYTES = DBM_COLS * WROW;
@@ -406,7 +410,7 @@ __global__ __launch_bounds__(256) void dispatch_backward_mfma_kernel(
       const int64_t t = t0 + wave * 8 + 2 * j + half;
       v[j][0] = z;
       v[j][1] = z;
-      if (t >= T_tokens) continue;
+      if (SLOT || t >= T_tokens) continue;
       // the token's record in one round trip (both choices of every array)
       const uint16_t kept2 = *reinterpret_cast<const uint16_t*>(kept + t * 2);
       const int2 idx2 = *reinterpret_cast<const int2*>(idx + t * 2);
@@ -506,8 +510,30 @@ __global__ __launch_bounds__(256) void dispatch_backward_mfma_kernel(
       const float4 s1 = *reinterpret_cast<const float4*>(sh + 4);
       // (the order of the one-token kernel: the rows first, then the share)
       float a[8], b[8], o[8];
-      unpack16(v[j][0], a, bf16_t());
-      unpack16(v[j][1], b, bf16_t());
+      if constexpr (SLOT) {
+        // this half-wavefront's token: lane l32 looks at experts l32, l32 + 32,
+        // ..; the rows are added in expert order
+#pragma unroll
+        for (int q = 0; q < 8; ++q) { a[q] = 0.f; b[q] = 0.f; }
+        for (int e0 = 0; e0 < E; e0 += 32) {
+          const int c = e0 + l32 < E ? (int)tok_slot[t * E + e0 + l32] : -1;
+          unsigned m = (unsigned)(__ballot(c >= 0) >> (32 * half));
+          while (m != 0u) {
+            const int el = __builtin_ctz(m);
+            m &= m - 1u;
+            const int64_t cc = __shfl(c, half * 32 + el, 64);
+            const int64_t slot = ((int64_t)(e0 + el) * G + g) * C + cc;
+            float r[8];
+            unpack16(load_streaming(reinterpret_cast<const uint4*>(
+                         dxe + slot * M + m0) + l32), r, bf16_t());
+#pragma unroll
+            for (int q = 0; q < 8; ++q) a[q] += r[q];
+          }
+        }
+      } else {
+        unpack16(v[j][0], a, bf16_t());
+        unpack16(v[j][1], b, bf16_t());
+      }
       const float sv[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
 #pragma unroll
       for (int q = 0; q < 8; ++q) o[q] = (a[q] + b[q]) + sv[q];
@@ -1040,6 +1066,46 @@ __global__ void convert_f32_kernel(const float* src, T* dst, int64_t n) {
 
 static bool bw_aligned16(const void* p) { return ((uintptr_t)p & 15) == 0; }
 
+// dx = rows of dexpert_in named by tok_slot + dlogits . w_gate^T through
+// dispatch_backward_mfma_kernel<.., SLOT>; false if the kernel does not take
+// the case (nothing launched).
+bool launch_slot_dispatch_backward_mfma(
+    const void* dexpert_in, const int16_t* tok_slot, const float* dlogits,
+    const void* w_gate, void* dx, int G, int S, int E, int C, int M, int dtype,
+    hipStream_t st, int* rc) {
+  const int64_t T_tokens = (int64_t)G * S;
+  *rc = 0;
+  if (!(dtype == MESH_MOE_BF16 && dlogits != nullptr && w_gate != nullptr &&
+        bw_aligned16(dexpert_in) && bw_aligned16(dx) && bw_aligned16(w_gate) &&
+        bw_aligned16(dlogits) && E % 16 == 0 && E <= DBM_MAX_E &&
+        M % DBM_COLS == 0 && S % DBM_TOK == 0 &&
+        (T_tokens + DBM_TOK - 1) / DBM_TOK <= 65535))
+    return false;
+  dim3 grid((unsigned)(M / DBM_COLS),
+            (unsigned)((T_tokens + DBM_TOK - 1) / DBM_TOK));
+  const size_t lds = dbm_lds_bytes(E);
+  auto run = [&](auto k) -> int {
+    MOE_ALLOW_LDS(k, lds);
+    k<<<grid, 256, lds, st>>>(
+        (const bf16_t*)dexpert_in, nullptr, nullptr, nullptr, nullptr, dlogits,
+        (const bf16_t*)w_gate, (bf16_t*)dx, G, S, C, M, T_tokens, G, nullptr,
+        tok_slot);
+    MOE_CHECK_LAUNCH("slot_dispatch_backward (router share on the matrix cores)");
+    return 0;
+  };
+  switch (E / 16) {
+    case 1: *rc = run(dispatch_backward_mfma_kernel<1, true>); break;
+    case 2: *rc = run(dispatch_backward_mfma_kernel<2, true>); break;
+    case 3: *rc = run(dispatch_backward_mfma_kernel<3, true>); break;
+    case 4: *rc = run(dispatch_backward_mfma_kernel<4, true>); break;
+    case 5: *rc = run(dispatch_backward_mfma_kernel<5, true>); break;
+    case 6: *rc = run(dispatch_backward_mfma_kernel<6, true>); break;
+    case 7: *rc = run(dispatch_backward_mfma_kernel<7, true>); break;
+    default: *rc = run(dispatch_backward_mfma_kernel<8, true>); break;
+  }
+  return true;
+}
+
 }  // namespace mesh_moe
 
 using namespace mesh_moe;
@@ -1179,7 +1245,7 @@ static int run_dispatch_backward(
     k<<<grid, 256, lds, st>>>(                                               \
         (const bf16_t*)dexpert_in, idx, pos, gate, kept, dlogits,            \
         (const bf16_t*)w_gate, (bf16_t*)dx, G, S, C, M, T_tokens,            \
-        groups_per_router, row_offsets);                                     \
+        groups_per_router, row_offsets, nullptr);                            \
   } while (0)
     switch (E / 16) {
       case 1: MOE_DBM(1); break;

@@ -362,7 +362,7 @@ __global__ __launch_bounds__(256) void slot_combine_backward_kernel(
     const int32_t* __restrict__ slot_token,
     const float* __restrict__ slot_weight, T* __restrict__ dy,
     float* __restrict__ dweight, int G, int S, int E, int C, int N,
-    int64_t n_slots) {
+    int64_t n_slots, bool vec) {
   const int lane = threadIdx.x & 63;
   const int64_t j = (int64_t)blockIdx.x * CH_ROWS + (threadIdx.x >> 6);
   if (j >= n_slots) return;
@@ -376,10 +376,44 @@ __global__ __launch_bounds__(256) void slot_combine_backward_kernel(
   const T* yrow = y + j * N;
   T* dst = dy + j * N;
   float dot = 0.f;
-  for (int i = lane; i < N; i += 64) {
-    const float d = load_f32<T>(drow + i);
-    dot += d * load_f32<T>(yrow + i);
-    store_f32<T>(dst + i, w * d);
+  if (vec) {
+    // 16-byte pieces, the loads of a batch of eight all issued before the
+    // first use
+    constexpr int VN = Vec16B<T>::N;
+    constexpr int UN = 8;
+    const int nv = N / VN;
+    const uint4* d4 = reinterpret_cast<const uint4*>(drow);
+    const uint4* y4 = reinterpret_cast<const uint4*>(yrow);
+    const uint4 z = make_uint4(0, 0, 0, 0);
+    for (int base = lane; base < nv; base += 64 * UN) {
+      uint4 dr[UN], yr[UN];
+#pragma unroll
+      for (int u = 0; u < UN; ++u) {
+        const int i = base + u * 64;
+        dr[u] = i < nv ? load_streaming(d4 + i) : z;
+        yr[u] = i < nv ? load_streaming(y4 + i) : z;
+      }
+#pragma unroll
+      for (int u = 0; u < UN; ++u) {
+        const int i = base + u * 64;
+        if (i >= nv) continue;
+        float d[VN], yv[VN], o[VN];
+        unpack16(dr[u], d, T());
+        unpack16(yr[u], yv, T());
+#pragma unroll
+        for (int q = 0; q < VN; ++q) {
+          dot += d[q] * yv[q];
+          o[q] = w * d[q];
+        }
+        store_streaming(reinterpret_cast<uint4*>(dst) + i, pack16(o, T()));
+      }
+    }
+  } else {
+    for (int i = lane; i < N; i += 64) {
+      const float d = load_f32<T>(drow + i);
+      dot += d * load_f32<T>(yrow + i);
+      store_f32<T>(dst + i, w * d);
+    }
   }
 #pragma unroll
   for (int off = 32; off > 0; off >>= 1) dot += __shfl_xor(dot, off, 64);
@@ -703,23 +737,32 @@ extern "C" int mesh_moe_slot_combine_backward(
   MOE_REQUIRE(nblocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
               "slot_combine_backward: too many slots (%lld)",
               (long long)n_slots);
+  const bool vec = ((size_t)N * dtype_size(dtype)) % 16 == 0 &&
+                   (((uintptr_t)dout | (uintptr_t)y | (uintptr_t)dy) & 15) == 0;
   hipStream_t st = (hipStream_t)stream;
   if (dtype == MESH_MOE_F32)
     slot_combine_backward_kernel<float><<<(unsigned)nblocks, 256, 0, st>>>(
         (const float*)dout, (const float*)y, slot_token, slot_weight,
-        (float*)dy, dweight, G, S, E, C, N, n_slots);
+        (float*)dy, dweight, G, S, E, C, N, n_slots, vec);
   else
     slot_combine_backward_kernel<bf16_t><<<(unsigned)nblocks, 256, 0, st>>>(
         (const bf16_t*)dout, (const bf16_t*)y, slot_token, slot_weight,
-        (bf16_t*)dy, dweight, G, S, E, C, N, n_slots);
+        (bf16_t*)dy, dweight, G, S, E, C, N, n_slots, vec);
   MOE_CHECK_LAUNCH("slot_combine_backward");
   return 0;
 }
 
+namespace mesh_moe {
+bool launch_slot_dispatch_backward_mfma(
+    const void* dexpert_in, const int16_t* tok_slot, const float* dlogits,
+    const void* w_gate, void* dx, int G, int S, int E, int C, int M, int dtype,
+    hipStream_t st, int* rc);
+}
+
 extern "C" int mesh_moe_slot_dispatch_backward(
     const void* dexpert_in, const int16_t* tok_slot, const float* dlogits,
-    const void* w_gate_packed, void* dx, int G, int S, int E, int C, int M,
-    int dtype, void* stream) {
+    const void* w_gate_packed, const void* w_gate, void* dx, int G, int S,
+    int E, int C, int M, int dtype, void* stream) {
   MOE_REQUIRE(dexpert_in && tok_slot && dx, MESH_MOE_E_ARG,
               "slot_dispatch_backward: null pointer");
   MOE_REQUIRE((dlogits == nullptr) == (w_gate_packed == nullptr),
@@ -736,6 +779,10 @@ extern "C" int mesh_moe_slot_dispatch_backward(
               "slot_dispatch_backward: too many rows (%lld)",
               (long long)T_tokens);
   hipStream_t st = (hipStream_t)stream;
+  int rc = 0;
+  if (launch_slot_dispatch_backward_mfma(dexpert_in, tok_slot, dlogits, w_gate,
+                                         dx, G, S, E, C, M, dtype, st, &rc))
+    return rc;
   if (dtype == MESH_MOE_F32)
     slot_dispatch_backward_kernel<float><<<(unsigned)nblocks, 256, 0, st>>>(
         (const float*)dexpert_in, tok_slot, dlogits,

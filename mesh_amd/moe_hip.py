@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 28
+ABI_VERSION = 29
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -162,7 +162,7 @@ _SIGNATURES = {
         _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
     "mesh_moe_slot_dispatch_backward": (ctypes.c_int, [
-        _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
     "mesh_moe_expert_choice_backward_workspace_bytes": (ctypes.c_size_t, [
         ctypes.c_int, ctypes.c_int, ctypes.c_int]),
@@ -1343,9 +1343,10 @@ def slot_combine_backward(dout, y, r):
 
 
 def slot_dispatch_backward(dxe, r, group_size, dlogits=None,
-                           w_gate_packed=None):
+                           w_gate_packed=None, w_gate=None):
   """dxe [E,G,C,M] -> dx [G,S,M]; with dlogits [G,S,E] float32 and the packed
-  router kernel [E,M] the router's share is added."""
+  router kernel [E,M] the router's share is added.  w_gate [M,E]: the kernel
+  as the variable holds it (activation dtype), for the matrix-core kernel."""
   lib = load_library()
   e, g, c, m = dxe.shape
   s = group_size
@@ -1359,6 +1360,8 @@ def slot_dispatch_backward(dxe, r, group_size, dlogits=None,
         if dlogits is not None else None,
         _dev(w_gate_packed, "w_gate_packed", dt, (e, m))
         if w_gate_packed is not None else None,
+        _dev(w_gate, "w_gate", dt, (m, e))
+        if (w_gate is not None and dlogits is not None) else None,
         dx.data_ptr(), g, s, e, c, m, dtype_code(dt), _stream()),
         "slot_dispatch_backward")
   return dx

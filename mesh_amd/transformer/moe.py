@@ -705,10 +705,9 @@ class MoEV1GradOperation(mtf.Operation):
       if sv["gate_in"] is None:
         dwg = moe_hip.router_backward_weights(
             sv["x"].reshape(tokens, m_), dlogits.reshape(tokens, e_))
-        if not by_slot:
-          # the router kernel as the variable holds it, [M, E]
-          compact = dict(compact, w_gate=sv["w_gate"].reshape(m_, e_).to(
-              sv["x"].dtype).contiguous())
+        # the router kernel as the variable holds it, [M, E]
+        compact = dict(compact, w_gate=sv["w_gate"].reshape(m_, e_).to(
+            sv["x"].dtype).contiguous())
         dx = dispatch_backward(
             dxe.reshape(e_, groups, c_, m_), r, s_, dlogits,
             sv["w_gate_packed"].reshape(e_, m_), **compact)

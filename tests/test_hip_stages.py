@@ -1255,3 +1255,46 @@ def test_expert_choice_backward_stages(hip, act_dtype):
   want2 = want_dx + np.matmul(H.to_np(dl), wg.T)
   np.testing.assert_allclose(H.to_np(dx2), O.cast_act(want2, act_dtype),
                              rtol=tol["rtol"], atol=tol["atol"] * 4)
+
+
+@pytest.mark.parametrize("shape", [(2, 64, 16, 12, 512), (2, 128, 64, 5, 1024)],
+                         ids=lambda s: "x".join(map(str, s)))
+def test_expert_choice_backward_wide_rows(hip, shape):
+  """The per-slot backward calls at row lengths their 16-byte and matrix-core
+  kernels take (bf16): combine backward against the oracle; dispatch backward
+  with the router's share on the matrix cores against float64 sums rounded
+  once and against the call without the router kernel in its variable
+  layout."""
+  g, s, e, c, m = shape
+  rng = np.random.default_rng(19)
+  logits = (rng.standard_normal((g, s, e)) * 1.5).astype(np.float32)
+  r = hip.expert_choice_gating(torch.from_numpy(logits).cuda(), c)
+  r_np = dict(slot_token=r.slot_token.cpu().numpy(),
+              slot_weight=H.to_np(r.slot_weight))
+  cast = lambda a: O.cast_act(a.astype(np.float32), "bfloat16")
+  tol = H.value_tolerance("bfloat16")
+  dout, y = cast(rng.standard_normal((g, s, m))), cast(rng.standard_normal((e, g, c, m)))
+  dy, dw = hip.slot_combine_backward(H.to_gpu(dout, "bfloat16"),
+                                     H.to_gpu(y, "bfloat16"), r)
+  want_dy, want_dw = O.slot_combine_backward(dout, y, r_np, "bfloat16")
+  np.testing.assert_allclose(H.to_np(dy), want_dy, **tol)
+  np.testing.assert_allclose(H.to_np(dw), want_dw, rtol=1e-4, atol=1e-3)
+  dxe = cast(rng.standard_normal((e, g, c, m)))
+  dl = (rng.standard_normal((g, s, e)) * 2.0).astype(np.float32)
+  wg = cast(H.normal_weights(rng, (m, e), m))
+  wg_g = H.to_gpu(wg, "bfloat16")
+  wg_p = hip.pack_weights(wg_g.reshape(1, m, e), torch.bfloat16).reshape(e, m)
+  dl_g = torch.from_numpy(dl).cuda()
+  got = hip.slot_dispatch_backward(H.to_gpu(dxe, "bfloat16"), r, s, dl_g, wg_p,
+                                   w_gate=wg_g)
+  plain = hip.slot_dispatch_backward(H.to_gpu(dxe, "bfloat16"), r, s, dl_g, wg_p)
+  want = (O.slot_dispatch_backward(dxe, r_np, s).astype(np.float64) +
+          np.matmul(dl.astype(np.float64), wg.astype(np.float64).T))
+  held = np.zeros((g, s), bool)
+  for gi in range(g):
+    held[gi][r_np["slot_token"][gi].reshape(-1)] = True
+  assert held.any() and (~held).any()
+  err = np.abs(H.to_np(got).astype(np.float64) - want)
+  assert (err <= np.abs(want) * 2.0 ** -8 * 1.01 + 4e-5).all()
+  step = np.abs(H.to_np(got) - H.to_np(plain))
+  assert (step <= np.abs(H.to_np(plain)) * 2.0 ** -7 + 4e-5).all()
