@@ -571,10 +571,14 @@ __global__ __launch_bounds__(256) void gate_count_kernel(
     int32_t* __restrict__ counts, float* __restrict__ n_one) {
   extern __shared__ int32_t cnt[];  // [E] + 1 + [E]
   int32_t* cnt2 = cnt + p.E + 1;    // second choices (second-place loss)
+  // block (g, chunk): its share of the group's tokens, added to the group's
+  // counters (zero before the launch) with integer-valued atomics
   const int g = blockIdx.x;
+  const int per = (p.S + gridDim.y - 1) / gridDim.y;
+  const int s_lo = blockIdx.y * per, s_hi = min(p.S, s_lo + per);
   for (int e = threadIdx.x; e <= 2 * p.E; e += blockDim.x) cnt[e] = 0;
   __syncthreads();
-  for (int s = threadIdx.x; s < p.S; s += blockDim.x) {
+  for (int s = s_lo + threadIdx.x; s < s_hi; s += blockDim.x) {
     const int64_t t = (int64_t)g * p.S + s;
     bool one = true, positive = true;
     if (importance != nullptr) {
@@ -624,10 +628,10 @@ __global__ __launch_bounds__(256) void gate_count_kernel(
   }
   __syncthreads();
   for (int e = threadIdx.x; e < p.E; e += blockDim.x) {
-    counts[(int64_t)g * p.E + e] = cnt[e];
-    counts[((int64_t)p.G + g) * p.E + e] = cnt2[e];
+    if (cnt[e]) atomicAdd(&counts[(int64_t)g * p.E + e], cnt[e]);
+    if (cnt2[e]) atomicAdd(&counts[((int64_t)p.G + g) * p.E + e], cnt2[e]);
   }
-  if (threadIdx.x == 0) n_one[g] = (float)cnt[p.E];
+  if (threadIdx.x == 0 && cnt[p.E]) atomicAdd(&n_one[g], (float)cnt[p.E]);
 }
 
 template <typename IT>
@@ -1335,15 +1339,24 @@ extern "C" int mesh_moe_gating_backward(
   const size_t smem = sizeof(int32_t) * (2 * (size_t)E + 1);
   const int64_t T_tokens = (int64_t)G * S;
   const unsigned blocks = (unsigned)((T_tokens + 255) / 256);
+  // the counters (int32 counts, then float n_one: all-zero bits either way)
+  const int64_t n_cnt = 2 * (int64_t)G * E + G;
+  fill_f32_kernel<<<(unsigned)((n_cnt + 255) / 256 < 1024 ? (n_cnt + 255) / 256
+                                                          : 1024),
+                    256, 0, st>>>((float*)counts, n_cnt, 0.0f);
+  MOE_CHECK_LAUNCH("gating_backward (clear)");
+  // up to 16 blocks per group, 256 tokens or more each
+  const dim3 cgrid((unsigned)G, (unsigned)((S + 255) / 256 < 16 ? (S + 255) / 256
+                                                               : 16));
   if (importance && importance_dtype == MESH_MOE_BF16) {
-    gate_count_kernel<bf16_t><<<G, 256, smem, st>>>(
+    gate_count_kernel<bf16_t><<<cgrid, 256, smem, st>>>(
         p, logits, idx, (const bf16_t*)importance, counts, n_one);
     MOE_CHECK_LAUNCH("gating_backward (count)");
     gating_backward_kernel<bf16_t><<<blocks, 256, 0, st>>>(
         p, logits, (const bf16_t*)importance, idx, kept, dgate, d_loss, counts,
         n_one, dlogits);
   } else {
-    gate_count_kernel<float><<<G, 256, smem, st>>>(
+    gate_count_kernel<float><<<cgrid, 256, smem, st>>>(
         p, logits, idx, (const float*)importance, counts, n_one);
     MOE_CHECK_LAUNCH("gating_backward (count)");
     gating_backward_kernel<float><<<blocks, 256, 0, st>>>(
