@@ -550,8 +550,7 @@ struct RingCfg {
 // the block's column i.  R, N multiples of 8.  With k_extent, expert e's
 // reduction stops after its first k_extent[e] rows, rounded up to a K tile
 // (rows up to there must hold finite values in one operand and zeros in the
-// other); k_extent[e] == 0 gives an all-zero result.  k_extent is passed
-// in the place of row_map.
+// other); k_extent[e] == 0 gives an all-zero result.
 //
 // MASKED: element (e, r, n) of the result is stored as zero unless
 // mask_src[e][r][n] > 0 (the backward of a ReLU whose output is mask_src,
@@ -561,6 +560,11 @@ struct RingCfg {
 // (logical tile numbers in ascending order, their count in the element before
 // the list): an expert whose occupied rows were moved to the front of its row
 // range needs no tiles for the rest (see mesh_moe_compact_expert_ffn).
+// (Skipping, inside an expert's last listed tile, the 32-row pieces of a
+// wavefront's sub-tile that lie past the occupied rows -- about a tenth of the
+// multiply-adds with 1024 +- 32 rows per expert -- made the launches 2 to 5 %
+// slower: the branches around every matrix instruction cost more than the
+// instructions saved.)
 template <bool RELU, bool GATHER = false, bool KMAJOR = false,
           bool MASKED = false, bool LISTED = false>
 __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kernel(
@@ -569,10 +573,12 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
     int total_tiles, const int32_t* __restrict__ row_map = nullptr,
     const bf16_t* __restrict__ zero_row = nullptr,
     const bf16_t* __restrict__ mask_src = nullptr,
-    const int32_t* __restrict__ tile_list = nullptr) {
+    const int32_t* __restrict__ tile_list = nullptr,
+    const int32_t* __restrict__ row_count = nullptr) {
   using Cfg = RingCfg;
-  // KMAJOR kernels gather nothing: their row_map argument is k_extent
-  const int32_t* k_extent = KMAJOR ? row_map : nullptr;
+  // row_count [E], optional: KMAJOR kernels take it as the reduction extent
+  // per expert (k_extent)
+  const int32_t* k_extent = KMAJOR ? row_count : nullptr;
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, WN = Cfg::WN;
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
 
@@ -1401,8 +1407,8 @@ static int launch_ring_kmajor(const bf16_t* A, const bf16_t* B, bf16_t* C,
   auto k = grouped_gemm_bf16_ring_kernel<false, false, true>;
   MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
   k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
-      A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, k_extent, nullptr,
-      nullptr, nullptr);
+      A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr,
+      nullptr, nullptr, k_extent);
   MOE_CHECK_LAUNCH("expert_ffn_backward (mfma, K-major operands)");
   return 0;
 }
@@ -1429,7 +1435,7 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
     MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
     k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
         A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr,
-        mask_src, tile_list);
+        mask_src, tile_list, nullptr);
     MOE_CHECK_LAUNCH("expert_ffn (mfma, listed tiles, masked result)");
     return 0;
   }
@@ -1441,7 +1447,7 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
     MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);                                          \
     k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(                           \
         A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, row_map, zero_row,     \
-        nullptr, tile_list);                                                   \
+        nullptr, tile_list, nullptr);                                          \
   } while (0)
     if (row_map != nullptr) {
       if (relu) MOE_RING_LISTED(true, true);
@@ -1461,7 +1467,7 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
     MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
     k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
         A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr,
-        mask_src, nullptr);
+        mask_src, nullptr, nullptr);
     MOE_CHECK_LAUNCH("expert_ffn (mfma, masked result)");
     return 0;
   }
@@ -1471,13 +1477,13 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
       MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
       k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
           A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, row_map, zero_row,
-          nullptr, nullptr);
+          nullptr, nullptr, nullptr);
     } else {
       auto k = grouped_gemm_bf16_ring_kernel<false, true>;
       MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
       k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
           A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, row_map, zero_row,
-          nullptr, nullptr);
+          nullptr, nullptr, nullptr);
     }
     MOE_CHECK_LAUNCH("expert_ffn (mfma, gathered rows)");
     return 0;
@@ -1487,13 +1493,13 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
     MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
     k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
         A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr,
-        nullptr, nullptr);
+        nullptr, nullptr, nullptr);
   } else {
     auto k = grouped_gemm_bf16_ring_kernel<false, false>;
     MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
     k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
         A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr,
-        nullptr, nullptr);
+        nullptr, nullptr, nullptr);
   }
   MOE_CHECK_LAUNCH("expert_ffn (mfma, spread direct-to-LDS loads)");
   return 0;
