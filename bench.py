@@ -312,7 +312,7 @@ def main():
                   help="router of the v1 configs (the benchmark definition "
                        "uses top_2)")
   ap.add_argument("--backward", action="store_true",
-                  help="time forward + backward (v1 configs); the metric is "
+                  help="time forward + backward; the metric is "
                        "then named accordingly and is not the benchmark's")
   ap.add_argument("--block", action="store_true",
                   help="time the transformer block around the layer "
@@ -346,9 +346,6 @@ def main():
     cfg["name"] += ", %s gating" % args.gating
   device = torch.device("cuda:0")
   torch.cuda.set_device(device)
-  if args.backward and cfg["layer"] != "v1":
-    print("--backward applies to the v1 configs only", file=sys.stderr)
-    sys.exit(2)
   if args.block and (cfg["layer"] != "v1" or args.gating != "top_2"):
     print("--block applies to the v1 configs, top_2", file=sys.stderr)
     sys.exit(2)

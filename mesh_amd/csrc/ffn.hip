@@ -550,7 +550,9 @@ struct RingCfg {
 // the block's column i.  R, N multiples of 8.  With k_extent, expert e's
 // reduction stops after its first k_extent[e] rows, rounded up to a K tile
 // (rows up to there must hold finite values in one operand and zeros in the
-// other); k_extent[e] == 0 gives an all-zero result.
+// other); k_extent[e] == 0 gives an all-zero result.  K need not be a
+// multiple of the K tile: the rows of the last tile past K come from a zero
+// buffer.
 //
 // MASKED: element (e, r, n) of the result is stored as zero unless
 // mask_src[e][r][n] > 0 (the backward of a ReLU whose output is mask_src,
@@ -565,6 +567,10 @@ struct RingCfg {
 // multiply-adds with 1024 +- 32 rows per expert -- made the launches 2 to 5 %
 // slower: the branches around every matrix instruction cost more than the
 // instructions saved.)
+// 512 bytes that stay zero (nothing writes them): where a K-major tile reaches
+// past the last reduction row, its rows are loaded from here
+static __device__ __attribute__((aligned(256))) bf16_t kmajor_zero_row[256];
+
 template <bool RELU, bool GATHER = false, bool KMAJOR = false,
           bool MASKED = false, bool LISTED = false>
 __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kernel(
@@ -612,7 +618,7 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
   const int tiles_per_e = tiles_m * tiles_n;
   // K tiles of the current tile's reduction: all of K, or with k_extent
   // (KMAJOR) the expert's first k_extent[e] reduction rows only
-  int nk = K / BK;
+  int nk = KMAJOR ? (K + BK - 1) / BK : K / BK;
   bool tile_empty = false;   // k_extent[e] == 0: the result is zero
 
   // per-tile state
@@ -646,7 +652,7 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
       if (k_extent != nullptr) {
         const int used = k_extent[e];
         tile_empty = used == 0;
-        nk = max(1, min(K / BK, (used + BK - 1) / BK));
+        nk = max(1, min((K + BK - 1) / BK, (used + BK - 1) / BK));
       }
     }
     Ae = GATHER ? A : A + (int64_t)e * R * K;
@@ -681,18 +687,31 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
   // slots behind them) tile kt; kt past the end re-fetches the last tile into
   // a slot nobody reads any more
   constexpr int B_BASE = Cfg::B_BASE;
+  // KMAJOR: load j of a tile fills reduction rows 2 (wave + WAVES j) and + 1
+  // (lanes 32-63) of it; past the last reduction row they are zeros
+  auto kmajor_past_end = [&](int kt, int j) {
+    return kt * BK + (wave + Cfg::WAVES * j) * 2 + (lane >> 5) >= K;
+  };
   auto load_a = [&](int kt, int j) {
     const int slot = kt & 1;
     kt = min(kt, nk - 1);
+    const bf16_t* src = Ae + kt * (KMAJOR ? BK * R : BK) + a_off[j];
+    if constexpr (KMAJOR) {
+      if (kmajor_past_end(kt, j)) src = kmajor_zero_row + (lane & 31) * 8;
+    }
     __builtin_amdgcn_global_load_lds(
-        (glb_void_t*)(Ae + kt * (KMAJOR ? BK * R : BK) + a_off[j]),
+        (glb_void_t*)src,
         (lds_void_t*)(smem_raw + slot * Cfg::A_BYTES +
                       (wave + Cfg::WAVES * j) * 1024), 16, 0, 0);
   };
   auto load_b = [&](int kt, int slot, int j) {
     kt = min(kt, nk - 1);
+    const bf16_t* src = Be + kt * (KMAJOR ? BK * N : BK) + b_off[j];
+    if constexpr (KMAJOR) {
+      if (kmajor_past_end(kt, j)) src = kmajor_zero_row + (lane & 31) * 8;
+    }
     __builtin_amdgcn_global_load_lds(
-        (glb_void_t*)(Be + kt * (KMAJOR ? BK * N : BK) + b_off[j]),
+        (glb_void_t*)src,
         (lds_void_t*)(smem_raw + B_BASE + slot * Cfg::B_BYTES +
                       (wave + Cfg::WAVES * j) * 1024), 16, 0, 0);
   };
@@ -1386,7 +1405,7 @@ static int compute_units() {
 // reduction index outermost); true if the K-major ring kernel takes the shape.
 static bool kmajor_path_applies(const void* A, const void* B, const void* C,
                                 int R, int N, int K, int dtype) {
-  return dtype == MESH_MOE_BF16 && K % RingCfg::BK == 0 && K >= RingCfg::BK &&
+  return dtype == MESH_MOE_BF16 && K >= 1 &&
          R % 8 == 0 && N % 8 == 0 && R >= 128 && N >= 128 &&
          (int64_t)R * K < (1LL << 31) && (int64_t)N * K < (1LL << 31) &&
          (((uintptr_t)A | (uintptr_t)B | (uintptr_t)C) & 15) == 0;

@@ -1039,13 +1039,17 @@ def test_hidden_product_and_dropout_backward(hip, act_dtype, activation):
 
 @pytest.mark.parametrize("shape", [(2, 128, 256, 512, 256), (3, 192, 136, 264, 136),
                                    (1, 2048, 512, 1024, 256), (2, 64, 256, 256, 128),
-                                   (2, 96, 256, 256, 256)])
+                                   (2, 96, 256, 256, 256),
+                                   # rows that end inside a K tile of 64
+                                   (2, 400, 256, 512, 256), (3, 8, 128, 128, 128),
+                                   (1, 1000, 128, 256, 128)])
 def test_expert_ffn_backward_weight_gradients_bf16(hip, shape):
   """bf16 weight gradients dwi = expert_in^T . dh and dwo = h^T . dy: the
-  reduction runs over token rows.  Row counts that are multiples of 64 take the
-  kernel that reads both operands as they lie in memory (transposing LDS
-  reads); the last shape takes the path through transposed copies.  Both
-  against float32 matmuls of the same bf16 operands."""
+  reduction runs over token rows.  The kernel reads both operands as they lie
+  in memory (transposing LDS reads); row counts that end inside its K tile of
+  64 (96, 400, 8, 1000) take the rest of the tile from a zero buffer; kernel
+  dimensions that are not multiples of 8 (136, 264) go through transposed
+  copies.  All against float32 matmuls of the same bf16 operands."""
   e, rows, m, hdim, n = shape
   rng = np.random.default_rng(sum(shape))
   g = lambda a: H.to_gpu(O.cast_act(a.astype(np.float32), "bfloat16"), "bfloat16")
