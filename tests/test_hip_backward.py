@@ -340,6 +340,45 @@ def test_dispatch_backward_router_share_on_matrix_cores(hip, shape):
   assert float((step > 0).float().mean()) < 0.02
 
 
+def test_full_size_router_terms_on_matrix_cores(hip):
+  """Configuration 4's token count and widths (65536 tokens, d_model 4096, 64
+  experts).  The router kernel's gradient from bfloat16 tokens (d(logits) as
+  two bfloat16 terms on the bfloat16 matrix cores) against the same product
+  from the tokens widened to float32 (float32 matrix cores); the router's
+  share of d(tokens) on the matrix cores against the kernel with float32
+  multiply-adds.  Each pair equal up to one rounding step of the bfloat16
+  result."""
+  g, s, m, e, c = 32, 2048, 4096, 64, 64
+  dt = torch.bfloat16
+  gen = torch.Generator(device="cuda").manual_seed(41)
+  mk = lambda *sh: torch.randn(sh, generator=gen, device="cuda")
+  x = mk(g * s, m).to(dt)
+  dlogits = mk(g, s, e) * 0.05
+  dw = hip.router_backward_weights(x, dlogits.reshape(g * s, e)).float()
+  dw32 = hip.router_backward_weights(x.float(), dlogits.reshape(g * s, e))
+  scale = float(dw32.abs().max())
+  assert float((dw - dw32).abs().max()) <= scale * 2.0 ** -8 * 1.01
+  assert float((dw - dw32).abs().mean()) <= float(dw32.abs().mean()) * 2.0 ** -9
+  del x, dw, dw32
+  route = mk(g, s, e)
+  route[..., 0] += 2.0         # an expert that overflows on first choices
+  r = hip.top2_gating(route, c)
+  dxe = mk(e, g, c, m).to(dt)
+  w = (mk(m, e) / m ** 0.5).to(dt)
+  w_p = hip.pack_weights(w.reshape(1, m, e), dt).reshape(e, m)
+  got = hip.dispatch_backward(dxe, r, s, dlogits, w_p, w_gate=w).float()
+  plain = hip.dispatch_backward(dxe, r, s, dlogits, w_p).float()
+  step = (got - plain).abs()
+  assert bool((step <= plain.abs() * 2.0 ** -7 + 4e-5).all())
+  assert float((step > 0).float().mean()) < 0.02
+  # a token no expert keeps gets the router's share alone
+  lost = ~(r.kept != 0).any(-1)
+  assert bool(lost.any())
+  share = dlogits[lost].double() @ w.double().t()
+  assert float((got[lost].double() - share).abs().max()) <= float(
+      share.abs().max()) * 2.0 ** -8 * 1.01
+
+
 def test_full_size_compact_backward(hip):
   """Eight experts of configuration 4 at their real sizes (32 groups, capacity
   64: 2048 slot rows per expert, d_model 4096, d_ff 16384) behind a switch
