@@ -640,14 +640,29 @@ __global__ __launch_bounds__(256) void gating_backward_kernel(
     const IT* __restrict__ importance, const int32_t* __restrict__ idx,
     const uint8_t* __restrict__ kept, const float* __restrict__ dgate,
     const float* __restrict__ d_loss, const int32_t* __restrict__ counts,
-    const float* __restrict__ n_one, float* __restrict__ dlogits) {
-  const int64_t t = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-  const int64_t T_tokens = (int64_t)p.G * p.S;
-  if (t >= T_tokens) return;
+    const float* __restrict__ n_one, float* __restrict__ dlogits,
+    int staged) {
+  // staged: the block's rows of logits go through LDS (whole-line loads, rows
+  // padded by one float against bank conflicts), the thread works on its row
+  // there in place, and the rows of d(logits) leave the same way.  A thread
+  // reading its 4 E bytes straight from global memory waits for a cache line
+  // in every trip of every pass over the row.
+  extern __shared__ __attribute__((aligned(16))) float gb_tile[];
   const int E = p.E, S = p.S;
+  const int64_t T_tokens = (int64_t)p.G * p.S;
+  const int64_t t_blk = (int64_t)blockIdx.x * blockDim.x;
+  const int64_t t = t_blk + threadIdx.x;
+  const int n_rows = (int)min((int64_t)blockDim.x, T_tokens - t_blk);
+  if (staged) {
+    const float* src = logits + t_blk * E;
+    for (int q = threadIdx.x; q < n_rows * E; q += blockDim.x)
+      gb_tile[(q / E) * (E + 1) + q % E] = src[q];
+    __syncthreads();
+  }
+  if (t < T_tokens) {
   const int g = (int)(t / S);
-  const float* row = logits + t * E;
-  float* out = dlogits + t * E;
+  const float* row = staged ? gb_tile + threadIdx.x * (E + 1) : logits + t * E;
+  float* out = staged ? gb_tile + threadIdx.x * (E + 1) : dlogits + t * E;
   // softmax exactly as the forward kernel computes it
   float m = row[0];
   for (int e = 1; e < E; ++e) m = fmaxf(m, row[e]);
@@ -737,6 +752,13 @@ __global__ __launch_bounds__(256) void gating_backward_kernel(
   for (int e = 0; e < E; ++e) {
     const float pe = expf(row[e] + neglse);
     out[e] = pe * (dprob(e) - inner) + zfac * pe;
+  }
+  }  // t < T_tokens
+  if (staged) {
+    __syncthreads();
+    float* dst = dlogits + t_blk * E;
+    for (int q = threadIdx.x; q < n_rows * E; q += blockDim.x)
+      dst[q] = gb_tile[(q / E) * (E + 1) + q % E];
   }
 }
 
@@ -1338,7 +1360,13 @@ extern "C" int mesh_moe_gating_backward(
   hipStream_t st = (hipStream_t)stream;
   const size_t smem = sizeof(int32_t) * (2 * (size_t)E + 1);
   const int64_t T_tokens = (int64_t)G * S;
-  const unsigned blocks = (unsigned)((T_tokens + 255) / 256);
+  // rows through LDS where a block's rows fit: 256 threads up to 64 experts,
+  // 128 threads up to 128
+  const int staged = E <= 128;
+  const unsigned gb_threads = (staged && E > 64) ? 128 : 256;
+  const size_t gb_smem = staged ? sizeof(float) * gb_threads * (E + 1) : 0;
+  const unsigned blocks =
+      (unsigned)((T_tokens + gb_threads - 1) / gb_threads);
   // the counters (int32 counts, then float n_one: all-zero bits either way)
   const int64_t n_cnt = 2 * (int64_t)G * E + G;
   fill_f32_kernel<<<(unsigned)((n_cnt + 255) / 256 < 1024 ? (n_cnt + 255) / 256
@@ -1352,16 +1380,20 @@ extern "C" int mesh_moe_gating_backward(
     gate_count_kernel<bf16_t><<<cgrid, 256, smem, st>>>(
         p, logits, idx, (const bf16_t*)importance, counts, n_one);
     MOE_CHECK_LAUNCH("gating_backward (count)");
-    gating_backward_kernel<bf16_t><<<blocks, 256, 0, st>>>(
+    auto k = gating_backward_kernel<bf16_t>;
+    MOE_ALLOW_LDS(k, gb_smem);
+    k<<<blocks, gb_threads, gb_smem, st>>>(
         p, logits, (const bf16_t*)importance, idx, kept, dgate, d_loss, counts,
-        n_one, dlogits);
+        n_one, dlogits, staged);
   } else {
     gate_count_kernel<float><<<cgrid, 256, smem, st>>>(
         p, logits, idx, (const float*)importance, counts, n_one);
     MOE_CHECK_LAUNCH("gating_backward (count)");
-    gating_backward_kernel<float><<<blocks, 256, 0, st>>>(
+    auto k = gating_backward_kernel<float>;
+    MOE_ALLOW_LDS(k, gb_smem);
+    k<<<blocks, gb_threads, gb_smem, st>>>(
         p, logits, (const float*)importance, idx, kept, dgate, d_loss, counts,
-        n_one, dlogits);
+        n_one, dlogits, staged);
   }
   MOE_CHECK_LAUNCH("gating_backward");
   return 0;
