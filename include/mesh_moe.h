@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 29
+#define MESH_MOE_ABI_VERSION 30
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -351,6 +351,10 @@ size_t mesh_moe_compact_expert_ffn_workspace_bytes(int G, int E, int C, int M,
  *   row_offsets [E,G] int32 (output): row of expert e's first slot of group
  *     g; slot (e, g, c) is row row_offsets[e][g] + c of h[e] / y[e] -- what
  *     mesh_moe_combine_compact takes
+ *   hidden_uniform [E,G*C,H] dtype or NULL, keep_prob, noise_out [E,G*C,H]
+ *     or NULL: the dropout of the hidden tensor between the two einsums
+ *     (transformer/moe.py:477-479) as mesh_moe_hidden_product applies it; a
+ *     slot's noise is the one at its compacted row
  * Otherwise as mesh_moe_dispatched_expert_ffn (same limits, both GEMMs must
  * fit the 256 x 256 kernel, E <= 1024, MESH_MOE_E_UNSUPPORTED otherwise).
  */
@@ -358,6 +362,7 @@ int mesh_moe_compact_expert_ffn(
     const void* x, const int32_t* idx, const int32_t* pos, const float* gate,
     const uint8_t* kept, const int32_t* fill, const void* wi_packed,
     const void* wo_packed, void* h, void* y, int32_t* row_offsets,
+    const void* hidden_uniform, float keep_prob, void* noise_out,
     void* workspace, size_t workspace_bytes, int G, int S, int E, int C, int M,
     int H, int N, int activation, int dtype, void* stream);
 
@@ -676,7 +681,7 @@ int mesh_moe_dispatch_backward(const void* dexpert_in, const int32_t* idx,
  * mesh_moe_combine_backward_compact: mesh_moe_combine_backward with y and dy
  *   in compacted rows.
  * mesh_moe_compact_expert_ffn_backward: mesh_moe_expert_ffn_backward
- *   (relu or linear experts, no dh_scale); bf16, E <= 1024 and shapes the
+ *   (relu or linear experts; dh_scale as there); bf16, E <= 1024 and shapes the
  *   256 x 256 kernels take, else MESH_MOE_E_UNSUPPORTED;
  *   ..._workspace_bytes returns 0 for shapes it does not take.
  * mesh_moe_dispatch_backward_compact: mesh_moe_dispatch_backward reading
@@ -698,10 +703,10 @@ size_t mesh_moe_compact_expert_ffn_backward_workspace_bytes(int G, int E, int C,
                                                             int N);
 int mesh_moe_compact_expert_ffn_backward(
     const void* expert_in, const void* h, const void* dy, const void* wi,
-    const void* wo, const int32_t* fill, const int32_t* row_offsets,
-    void* dexpert_in, void* dwi, void* dwo, int G, int E, int C, int M, int H,
-    int N, int activation, int dtype, void* workspace, size_t workspace_bytes,
-    void* stream);
+    const void* wo, const void* dh_scale, const int32_t* fill,
+    const int32_t* row_offsets, void* dexpert_in, void* dwi, void* dwo, int G,
+    int E, int C, int M, int H, int N, int activation, int dtype,
+    void* workspace, size_t workspace_bytes, void* stream);
 int mesh_moe_dispatch_backward_compact(
     const void* dexpert_in, const int32_t* idx, const int32_t* pos,
     const float* gate, const uint8_t* kept, const int32_t* row_offsets,

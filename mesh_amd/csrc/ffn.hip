@@ -1895,11 +1895,17 @@ extern "C" int mesh_moe_compact_expert_ffn(
     const void* x, const int32_t* idx, const int32_t* pos, const float* gate,
     const uint8_t* kept, const int32_t* fill, const void* wi_packed,
     const void* wo_packed, void* h, void* y, int32_t* row_offsets,
+    const void* hidden_uniform, float keep_prob, void* noise_out,
     void* workspace, size_t workspace_bytes, int G, int S, int E, int C, int M,
     int H, int N, int activation, int dtype, void* stream) {
   MOE_REQUIRE(x && idx && pos && gate && kept && fill && wi_packed &&
                   wo_packed && h && y && row_offsets && workspace,
               MESH_MOE_E_ARG, "compact_expert_ffn: null pointer");
+  MOE_REQUIRE(!noise_out || hidden_uniform, MESH_MOE_E_ARG,
+              "compact_expert_ffn: noise_out without hidden_uniform");
+  MOE_REQUIRE(!hidden_uniform || (keep_prob > 0.f && keep_prob <= 1.f),
+              MESH_MOE_E_ARG, "compact_expert_ffn: keep_prob %g outside (0, 1]",
+              (double)keep_prob);
   MOE_REQUIRE(G >= 1 && S >= 1 && E >= 1 && C >= 1 && M >= 1 && H >= 1 && N >= 1,
               MESH_MOE_E_ARG, "compact_expert_ffn: bad sizes");
   MOE_REQUIRE(activation >= MESH_MOE_ACT_LINEAR &&
@@ -1960,6 +1966,13 @@ extern "C" int mesh_moe_compact_expert_ffn(
     const int blocks = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
     activation_kernel<bf16_t><<<blocks, 256, 0, st>>>((bf16_t*)h, n, activation);
     MOE_CHECK_LAUNCH("compact_expert_ffn (activation)");
+  }
+  if (hidden_uniform != nullptr) {
+    // the hidden dropout, element for element of the [E, G*C, H] buffer (the
+    // noise of a slot is the one drawn at its compacted row)
+    rc = mesh_moe_hidden_product(h, nullptr, hidden_uniform, keep_prob,
+                                 noise_out, (int64_t)E * R * H, dtype, stream);
+    if (rc != 0) return rc;
   }
   return launch_ring((const bf16_t*)h, (const bf16_t*)wo_packed, (bf16_t*)y, E,
                      R, N, H, false, st, nullptr, nullptr, nullptr, list2);
@@ -2260,10 +2273,10 @@ extern "C" size_t mesh_moe_compact_expert_ffn_backward_workspace_bytes(
 
 extern "C" int mesh_moe_compact_expert_ffn_backward(
     const void* expert_in, const void* h, const void* dy, const void* wi,
-    const void* wo, const int32_t* fill, const int32_t* row_offsets,
-    void* dexpert_in, void* dwi, void* dwo, int G, int E, int C, int M, int H,
-    int N, int activation, int dtype, void* workspace, size_t workspace_bytes,
-    void* stream) {
+    const void* wo, const void* dh_scale, const int32_t* fill,
+    const int32_t* row_offsets, void* dexpert_in, void* dwi, void* dwo, int G,
+    int E, int C, int M, int H, int N, int activation, int dtype,
+    void* workspace, size_t workspace_bytes, void* stream) {
   MOE_REQUIRE(expert_in && h && dy && wi && wo && fill && row_offsets &&
                   dexpert_in && dwi && dwo && workspace, MESH_MOE_E_ARG,
               "compact_expert_ffn_backward: null pointer");
@@ -2309,11 +2322,22 @@ extern "C" int mesh_moe_compact_expert_ffn_backward(
   // dh = dy . wo^T on the listed row tiles, the ReLU mask on its stores (the
   // rows of a listed tile past the expert's occupied ones have h = 0 and
   // dy = 0)
+  const bool mask_on_stores = activation == MESH_MOE_ACT_RELU && !dh_scale;
   int rc = launch_ring(
       (const bf16_t*)dy, (const bf16_t*)wo, dh, E, R, H, N, false, st, nullptr,
-      nullptr, activation == MESH_MOE_ACT_RELU ? (const bf16_t*)h : nullptr,
-      list_h);
+      nullptr, mask_on_stores ? (const bf16_t*)h : nullptr, list_h);
   if (rc != 0) return rc;
+  if (dh_scale != nullptr) {
+    // the dropout's noise (and the ReLU mask) as a pass over the buffer, as in
+    // mesh_moe_expert_ffn_backward; rows outside the listed tiles hold
+    // unspecified values before and after
+    const int64_t n = (int64_t)E * R * H;
+    const int blocks = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
+    hidden_grad_kernel<bf16_t><<<blocks, 256, 0, st>>>(
+        dh, (const bf16_t*)h, (const bf16_t*)dh_scale,
+        activation == MESH_MOE_ACT_RELU, n);
+    MOE_CHECK_LAUNCH("compact_expert_ffn_backward (hidden mask)");
+  }
   // dexpert_in = dh . wi^T on the listed row tiles
   rc = launch_ring(dh, (const bf16_t*)wi, (bf16_t*)dexpert_in, E, R, M, H,
                    false, st, nullptr, nullptr, nullptr, list_m);

@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 29
+ABI_VERSION = 30
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -87,7 +87,7 @@ _SIGNATURES = {
         ctypes.c_int]),
     "mesh_moe_compact_expert_ffn": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp,
-        ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_float, _vp, _vp, ctypes.c_size_t, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         _vp]),
     "mesh_moe_combine_compact": (ctypes.c_int, [
@@ -104,7 +104,7 @@ _SIGNATURES = {
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_int]),
     "mesh_moe_compact_expert_ffn_backward": (ctypes.c_int, [
-        _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int,
+        _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
     "mesh_moe_dispatch_backward_compact": (ctypes.c_int, [
@@ -766,12 +766,16 @@ def compact_training_applies(x, r, hidden_size, output_size,
 
 
 def compact_expert_ffn(x, r, wi_packed, wo_packed, activation="relu",
-                       want_hidden=False):
+                       want_hidden=False, uniform=None, keep_prob=1.0,
+                       want_noise=False):
   """dispatch + expert_ffn on compacted rows (only the tiles that hold
   occupied slots are multiplied): x [G, S, M], the Routing r -> (y [E, G*C, N],
   row_offsets [E, G]) for combine(..., row_offsets=...), or None where the
   library has no such kernel for the case.  want_hidden: (y, row_offsets, h)
-  with the hidden tensor h [E, G*C, H] in the same row order."""
+  with the hidden tensor h [E, G*C, H] in the same row order.  uniform
+  [E, G*C, H]: the hidden dropout h *= (uniform < keep_prob) / keep_prob
+  between the two products; want_noise appends the noise tensor to the
+  result."""
   lib = load_library()
   if activation not in ACTIVATIONS:
     raise ValueError("unsupported expert activation %r" % (activation,))
@@ -785,6 +789,8 @@ def compact_expert_ffn(x, r, wi_packed, wo_packed, activation="relu",
   h = torch.empty((e, g * c, hdim), dtype=dt, device=dev)
   y = torch.empty((e, g * c, n), dtype=dt, device=dev)
   row_offsets = torch.empty((e, g), dtype=torch.int32, device=dev)
+  noise = (torch.empty_like(h) if (want_noise and uniform is not None)
+           else None)
   ws_bytes = lib.mesh_moe_compact_expert_ffn_workspace_bytes(g, e, c, m, hdim, n)
   ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
   with _stage("expert_ffn"):
@@ -794,14 +800,19 @@ def compact_expert_ffn(x, r, wi_packed, wo_packed, activation="relu",
         _dev(r.fill, "fill", torch.int32, (g, e)),
         _dev(wi_packed, "wi_packed", dt, (e, hdim, m)),
         _dev(wo_packed, "wo_packed", dt, (e, n, hdim)), h.data_ptr(),
-        y.data_ptr(), row_offsets.data_ptr(), ws.data_ptr(), ws_bytes, g, s, e,
+        y.data_ptr(), row_offsets.data_ptr(),
+        _dev(uniform, "uniform", dt, (e, g * c, hdim))
+        if uniform is not None else None, float(keep_prob),
+        noise.data_ptr() if noise is not None else None,
+        ws.data_ptr(), ws_bytes, g, s, e,
         c, m, hdim, n, ACTIVATIONS[activation], dtype_code(dt), _stream())
   if rc == E_UNSUPPORTED:
     return None
   _check(rc, "compact_expert_ffn")
   if _timer is not None:
     _timer.compacted += 1
-  return (y, row_offsets, h) if want_hidden else (y, row_offsets)
+  res = (y, row_offsets, h) if want_hidden else (y, row_offsets)
+  return res + (noise,) if want_noise else res
 
 
 def expert_linear(a, w_packed, activation="linear", y=None):
@@ -946,9 +957,10 @@ def expert_ffn_backward(expert_in, h, dy, wi, wo, activation="relu",
 
 
 def compact_expert_ffn_backward(expert_in, h, dy, wi, wo, r, row_offsets,
-                                activation="relu"):
+                                activation="relu", dh_scale=None):
   """expert_ffn_backward with every [E, G*C, .] tensor in the compacted row
-  order of compact_expert_ffn (r: the Routing, row_offsets [E, G])."""
+  order of compact_expert_ffn (r: the Routing, row_offsets [E, G]; dh_scale
+  [E, G*C, H]: the hidden dropout's noise, if there was one)."""
   lib = load_library()
   if activation not in ("relu", "linear"):
     raise ValueError("unsupported expert activation %r" % (activation,))
@@ -972,6 +984,8 @@ def compact_expert_ffn_backward(expert_in, h, dy, wi, wo, r, row_offsets,
         _dev(expert_in, "expert_in"), _dev(h, "h", dt, (e, rows, hdim)),
         _dev(dy, "dy", dt, (e, rows, n)), _dev(wi, "wi", dt, (e, m, hdim)),
         _dev(wo, "wo", dt, (e, hdim, n)),
+        _dev(dh_scale, "dh_scale", dt, (e, rows, hdim))
+        if dh_scale is not None else None,
         _dev(r.fill, "fill", torch.int32, (g, e)),
         _dev(row_offsets, "row_offsets", torch.int32, (e, g)), dxe.data_ptr(),
         dwi.data_ptr(), dwo.data_ptr(), g, e, c, m, hdim, n,

@@ -468,33 +468,49 @@ class MoEV1Operation(mtf.Operation):
       noise = None
       row_offsets = None
       expert_in = h = None
-      if (save and not by_slot and kwo_p is None and plain_hidden and
-          self._gating.router != "top_2" and
+      # one relu / linear / ... layer per expert, with or without the hidden
+      # dropout: what the compacted calls take
+      one_layer = not more_wi_p and not keep_pre
+      single_choice = (not by_slot and kwo_p is None and one_layer and
+                       self._gating.router != "top_2")
+
+      def compact_ffn(want_hidden):
+        """The expert feed-forward on compacted rows (the occupied slots at
+        the front of every expert's rows), hidden dropout included; None where
+        the library has no such kernel for the case."""
+        u = None
+        if keep_prob is not None:
+          u = torch.rand((e_, groups * c_, wi_p.shape[1]), dtype=dt,
+                         device=xg.device)
+        return moe_hip.compact_expert_ffn(
+            xg, r, wi_p, wo_p, self._activation, want_hidden=want_hidden,
+            uniform=u, keep_prob=1.0 if keep_prob is None else keep_prob,
+            want_noise=want_hidden)
+
+      if (save and single_choice and
           moe_hip.compact_training_applies(xg, r, wi_p.shape[1], n_,
                                            self._activation)):
         # one choice per token and a gradient to follow: the occupied slots at
         # the front of every expert's rows in all the tensors the gradient
         # operation reads, so that it too multiplies only those
-        compact = moe_hip.compact_expert_ffn(xg, r, wi_p, wo_p,
-                                             self._activation, want_hidden=True)
+        compact = compact_ffn(True)
         if compact is not None:
-          y, row_offsets, h = compact
+          y, row_offsets, h, noise = compact
           expert_in = moe_hip.dispatch(xg, r, row_offsets=row_offsets)
           expert_in = expert_in.reshape(e_, groups * c_, m_)
-      if not (save or by_slot or kwo_p is not None) and plain_hidden:
+      if not save and single_choice:
+        # Routers with one choice per token leave about 1 - 1 / capacity_factor
+        # of the slots empty: their occupied slots are moved to the front of
+        # every expert's rows and only the tiles that hold them are multiplied
+        compact = compact_ffn(False)
+        if compact is not None:
+          y, row_offsets = compact
+      if (y is None and not (save or by_slot or kwo_p is not None) and
+          plain_hidden):
         # nobody reads expert_in afterwards: fold the dispatch into the first
-        # expert GEMM where the library can.  Routers with one choice per token
-        # leave about 1 - 1 / capacity_factor of the slots empty: their
-        # occupied slots are moved to the front of every expert's rows and
-        # only the tiles that hold them are multiplied
-        if self._gating.router != "top_2":
-          compact = moe_hip.compact_expert_ffn(xg, r, wi_p, wo_p,
-                                               self._activation)
-          if compact is not None:
-            y, row_offsets = compact
-        if y is None:
-          y = moe_hip.dispatched_expert_ffn(xg, r, wi_p, wo_p,
-                                            self._activation)
+        # expert GEMM where the library can
+        y = moe_hip.dispatched_expert_ffn(xg, r, wi_p, wo_p,
+                                          self._activation)
       if y is None:
         expert_in = (moe_hip.slot_dispatch(xg, r) if by_slot
                      else moe_hip.dispatch(xg, r))
@@ -653,7 +669,7 @@ class MoEV1GradOperation(mtf.Operation):
         dxe, dwi, dwo = moe_hip.compact_expert_ffn_backward(
             sv["expert_in"].reshape(e_, groups * c_, m_), sv["h"],
             dy.reshape(e_, groups * c_, n_), wi_s, wo_s, r, row_offsets,
-            fwd._activation)
+            fwd._activation, dh_scale=sv["hidden_noise"])
         dkwo, dwis = None, [dwi]
       elif fwd._general_hidden:
         dys, wos = [dy.reshape(e_, groups * c_, n_)], [wo_s]

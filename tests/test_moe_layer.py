@@ -780,6 +780,56 @@ def test_v1_switch_max_matches_oracle():
   np.testing.assert_allclose(got_loss, want_loss, rtol=1e-4)
 
 
+def test_v1_switch_hidden_dropout_on_compacted_rows():
+  """Training forward of a switch layer with moe_dropout_rate at a shape the
+  compacted expert rows take: the dropout runs between the two expert products
+  on the compacted hidden tensor.  Against the oracle, with the layer's noise
+  (its only random call, reproduced) moved from the compacted rows to the
+  [E, G, C] slot order the oracle works in."""
+  from mesh_amd import moe_hip
+  b, l, m, hdim, e, group = 2, 1024, 256, 512, 4, 1024
+  rng = np.random.default_rng(121)
+  w = dict(w_gate=H.normal_weights(rng, (m, e), m),
+           wi=H.normal_weights(rng, (e, m, hdim), m),
+           wo=H.normal_weights(rng, (e, hdim, m), hdim))
+  x = H.safe_tokens(rng, b * l, m, w["w_gate"], "bfloat16").reshape(b, l, m)
+  hp, ohp = make_hparams(moe_num_experts=e, moe_hidden_size=hdim,
+                         moe_group_size=group, moe_capacity_factor_train=1.0,
+                         moe_dropout_rate=0.25, **SWITCH_HP)
+  torch.manual_seed(9)
+  with moe_hip.StageTimer() as timer:
+    got, got_loss, _, _ = run_v1(x, w, hp, True, "bfloat16")
+  assert timer.compacted == 1
+  torch.manual_seed(9)
+  n_groups = b * l // group
+  cap = O.expert_capacity(group, 1.0, e, 4)
+  hu = torch.rand((e, n_groups * cap, hdim), dtype=torch.bfloat16,
+                  device="cuda").float().cpu().numpy()
+  _, _, aux = O.moe_layer_v1(x, w["w_gate"], w["wi"], w["wo"], ohp, True,
+                             "bfloat16", dense=False, hidden_uniform=hu)
+  idx1 = aux["index_1"].reshape(n_groups, group)
+  kept1 = aux["kept_1"].reshape(n_groups, group).astype(bool)
+  assert not kept1.all()
+  padded = np.zeros_like(hu)
+  for ex in range(e):
+    row = 0
+    for gi in range(n_groups):
+      n = int((kept1[gi] & (idx1[gi] == ex)).sum())
+      padded[ex, gi * cap:gi * cap + n] = hu[ex, row:row + n]
+      row += n
+  want, want_loss, _ = O.moe_layer_v1(x, w["w_gate"], w["wi"], w["wo"], ohp,
+                                      True, "bfloat16", dense=False,
+                                      hidden_uniform=padded)
+  plain, _, _ = O.moe_layer_v1(
+      x, w["w_gate"], w["wi"], w["wo"],
+      make_hparams(moe_num_experts=e, moe_hidden_size=hdim,
+                   moe_group_size=group, moe_capacity_factor_train=1.0,
+                   **SWITCH_HP)[1], True, "bfloat16", dense=False)
+  assert np.abs(want - plain).max() > 0.05            # units were dropped
+  np.testing.assert_allclose(got, want, **H.value_tolerance("bfloat16"))
+  np.testing.assert_allclose(got_loss, want_loss, rtol=1e-2)
+
+
 # ---- gradients through the mtf-shaped API -------------------------------------
 @pytest.mark.parametrize("case", [
     ("top_2", "float32", 101), ("top_2", "bfloat16", 102),
@@ -795,7 +845,8 @@ def test_v1_switch_max_matches_oracle():
     # shapes the matrix-core kernels take: one choice per token keeps the
     # gradient graph on compacted rows
     ("switch+compact", "bfloat16", 114), ("ntlb+compact", "bfloat16", 115),
-    ("switch+compact+input_jitter", "bfloat16", 116)],
+    ("switch+compact+input_jitter", "bfloat16", 116),
+    ("switch+compact+hidden_dropout", "bfloat16", 117)],
     ids=lambda c: "%s-%s" % (c[0], c[1]))
 def test_v1_gradients_match_oracle(case, monkeypatch):
   """mtf.gradients over the layer (outputs and loss) against the oracle's
@@ -877,6 +928,25 @@ def test_v1_gradients_match_oracle(case, monkeypatch):
     cap = O.expert_capacity(group, 1.0, e, 4)
     hu = torch.rand((e, (b * l // group) * cap, hdim), dtype=dt,
                     device="cuda").float().cpu().numpy()
+    if compact:
+      # the layer drew the noise for the compacted rows (an expert's occupied
+      # slots, groups in order, at the front of its rows): move every slot's
+      # noise to the slot's place in the [E, G, C] order the oracle uses
+      _, _, aux = O.moe_layer_v1(x, w["w_gate"], w["wi"], w["wo"], ohp, True,
+                                 act_dtype, nonpadding=nonpad,
+                                 num_microbatches=2, dense=False,
+                                 hidden_uniform=hu)   # (the routing ignores it)
+      n_groups = b * l // group
+      idx1 = aux["index_1"].reshape(n_groups, group)
+      kept1 = aux["kept_1"].reshape(n_groups, group).astype(bool)
+      padded = np.zeros_like(hu)
+      for ex in range(e):
+        row = 0
+        for gi in range(n_groups):
+          n = int((kept1[gi] & (idx1[gi] == ex)).sum())
+          padded[ex, gi * cap:gi * cap + n] = hu[ex, row:row + n]
+          row += n
+      hu = padded
   want = O.moe_layer_v1_backward(x, w["w_gate"], w["wi"], w["wo"], ohp, True,
                                  act_dtype, d_out, 1.5, nonpadding=nonpad,
                                  num_microbatches=2, gate_noise=noise,
