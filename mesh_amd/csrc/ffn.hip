@@ -1338,6 +1338,110 @@ __global__ __launch_bounds__(256) void activation_backward_bf16x8_kernel(
   }
 }
 
+// hidden_grad_kernel, hidden_product_kernel and activation_kernel for bf16
+// with 16-byte accesses (8 elements per thread and step; the same arithmetic
+// and the same roundings element by element).
+__global__ __launch_bounds__(256) void hidden_grad_bf16x8_kernel(
+    uint4* __restrict__ dh, const uint4* __restrict__ h,
+    const uint4* __restrict__ scale, bool relu, int64_t n8) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8;
+       i += stride) {
+    float d[8], hv[8], sc[8];
+    unpack16(load_streaming(dh + i), d, bf16_t());
+    if (relu) unpack16(load_streaming(h + i), hv, bf16_t());
+    if (scale) unpack16(load_streaming(scale + i), sc, bf16_t());
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+      if (relu && !(hv[j] > 0.f)) d[j] = 0.f;
+      else if (scale) d[j] = d[j] * sc[j];
+    }
+    store_streaming(dh + i, pack16(d, bf16_t()));
+  }
+}
+
+__global__ __launch_bounds__(256) void hidden_product_bf16x8_kernel(
+    uint4* __restrict__ h, const uint4* __restrict__ factor,
+    const uint4* __restrict__ uniform, float keep, float inv_keep,
+    uint4* __restrict__ noise_out, int64_t n8) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8;
+       i += stride) {
+    float v[8], f[8], u[8], nz[8];
+    unpack16(load_streaming(h + i), v, bf16_t());
+    if (factor) {
+      unpack16(load_streaming(factor + i), f, bf16_t());
+#pragma unroll
+      for (int j = 0; j < 8; ++j) v[j] = round_to<bf16_t>(v[j] * f[j]);
+    }
+    if (uniform) {
+      unpack16(load_streaming(uniform + i), u, bf16_t());
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        nz[j] = u[j] < keep ? inv_keep : 0.f;
+        v[j] = v[j] * nz[j];
+      }
+      if (noise_out) store_streaming(noise_out + i, pack16(nz, bf16_t()));
+    }
+    store_streaming(h + i, pack16(v, bf16_t()));
+  }
+}
+
+// (out may be the input: in place)
+__global__ __launch_bounds__(256) void activation_bf16x8_kernel(
+    const uint4* h, uint4* out, int64_t n8, int act) {
+  const int64_t stride = (int64_t)gridDim.x * blockDim.x;
+  for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8;
+       i += stride) {
+    float v[8];
+    unpack16(load_streaming(h + i), v, bf16_t());
+#pragma unroll
+    for (int j = 0; j < 8; ++j) v[j] = apply_activation(v[j], act);
+    store_streaming(out + i, pack16(v, bf16_t()));
+  }
+}
+
+static bool x8_applies(int64_t n, int dtype, const void* a, const void* b,
+                       const void* c, const void* d = nullptr) {
+  return dtype == MESH_MOE_BF16 && n % 8 == 0 &&
+         (((uintptr_t)a | (uintptr_t)b | (uintptr_t)c | (uintptr_t)d) & 15) == 0;
+}
+static int elementwise_blocks(int64_t n) {
+  return (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
+}
+
+// dh = dh * scale, then the ReLU mask of h (hidden_grad_kernel's contract)
+static int launch_hidden_grad(void* dh, const void* h, const void* scale,
+                              bool relu, int64_t n, int dtype, hipStream_t st) {
+  if (x8_applies(n, dtype, dh, h, scale))
+    hidden_grad_bf16x8_kernel<<<elementwise_blocks(n / 8), 256, 0, st>>>(
+        (uint4*)dh, (const uint4*)h, (const uint4*)scale, relu, n / 8);
+  else if (dtype == MESH_MOE_F32)
+    hidden_grad_kernel<float><<<elementwise_blocks(n), 256, 0, st>>>(
+        (float*)dh, (const float*)h, (const float*)scale, relu, n);
+  else
+    hidden_grad_kernel<bf16_t><<<elementwise_blocks(n), 256, 0, st>>>(
+        (bf16_t*)dh, (const bf16_t*)h, (const bf16_t*)scale, relu, n);
+  MOE_CHECK_LAUNCH("hidden gradient (mask / scale)");
+  return 0;
+}
+
+// h = act(h) in place
+static int launch_activation(void* h, int64_t n, int act, int dtype,
+                             hipStream_t st) {
+  if (x8_applies(n, dtype, h, nullptr, nullptr))
+    activation_bf16x8_kernel<<<elementwise_blocks(n / 8), 256, 0, st>>>(
+        (const uint4*)h, (uint4*)h, n / 8, act);
+  else if (dtype == MESH_MOE_F32)
+    activation_kernel<float><<<elementwise_blocks(n), 256, 0, st>>>((float*)h, n,
+                                                                    act);
+  else
+    activation_kernel<bf16_t><<<elementwise_blocks(n), 256, 0, st>>>((bf16_t*)h,
+                                                                     n, act);
+  MOE_CHECK_LAUNCH("activation");
+  return 0;
+}
+
 template <int BM, int BN, int BK>
 static int launch_mfma(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
                        int R, int N, int K, bool relu, hipStream_t st) {
@@ -1619,15 +1723,8 @@ static int grouped_gemm(const void* A, const void* B, void* C, int E, int R,
                                      (bf16_t*)C, E, R, N, K, relu, st);
   }
   if (rc != 0) return rc;
-  if (act != MESH_MOE_ACT_RELU && act != MESH_MOE_ACT_LINEAR) {
-    const int64_t n = (int64_t)E * R * N;
-    const int blocks = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
-    if (dtype == MESH_MOE_F32)
-      activation_kernel<float><<<blocks, 256, 0, st>>>((float*)C, n, act);
-    else
-      activation_kernel<bf16_t><<<blocks, 256, 0, st>>>((bf16_t*)C, n, act);
-    MOE_CHECK_LAUNCH("expert_ffn (activation)");
-  }
+  if (act != MESH_MOE_ACT_RELU && act != MESH_MOE_ACT_LINEAR)
+    return launch_activation(C, (int64_t)E * R * N, act, dtype, st);
   return 0;
 }
 
@@ -1865,10 +1962,8 @@ extern "C" int mesh_moe_dispatched_expert_ffn(
                        E, R, H, M, relu, st, map, zero_row);
   if (rc != 0) return rc;
   if (!relu && activation != MESH_MOE_ACT_LINEAR) {
-    const int64_t n = (int64_t)E * R * H;
-    const int blocks = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
-    activation_kernel<bf16_t><<<blocks, 256, 0, st>>>((bf16_t*)h, n, activation);
-    MOE_CHECK_LAUNCH("dispatched_expert_ffn (activation)");
+    rc = launch_activation(h, (int64_t)E * R * H, activation, dtype, st);
+    if (rc != 0) return rc;
   }
   return grouped_gemm(h, wo_packed, y, E, R, N, H, MESH_MOE_ACT_LINEAR, dtype,
                       st);
@@ -1962,10 +2057,8 @@ extern "C" int mesh_moe_compact_expert_ffn(
   if (!relu && activation != MESH_MOE_ACT_LINEAR) {
     // (the pass also runs over the rows no listed tile wrote: they hold
     // unspecified values before and after, and nothing reads them)
-    const int64_t n = (int64_t)E * R * H;
-    const int blocks = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
-    activation_kernel<bf16_t><<<blocks, 256, 0, st>>>((bf16_t*)h, n, activation);
-    MOE_CHECK_LAUNCH("compact_expert_ffn (activation)");
+    rc = launch_activation(h, (int64_t)E * R * H, activation, dtype, st);
+    if (rc != 0) return rc;
   }
   if (hidden_uniform != nullptr) {
     // the hidden dropout, element for element of the [E, G*C, H] buffer (the
@@ -2010,7 +2103,12 @@ extern "C" int mesh_moe_hidden_product(void* h, const void* factor,
   if (!factor && !uniform) return 0;
   hipStream_t st = (hipStream_t)stream;
   const int blocks = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
-  if (dtype == MESH_MOE_F32) {
+  if (x8_applies(n, dtype, h, factor, uniform, noise_out)) {
+    const float keep = round_bf16_host(keep_prob);
+    hidden_product_bf16x8_kernel<<<elementwise_blocks(n / 8), 256, 0, st>>>(
+        (uint4*)h, (const uint4*)factor, (const uint4*)uniform, keep,
+        round_bf16_host(1.f / keep), (uint4*)noise_out, n / 8);
+  } else if (dtype == MESH_MOE_F32) {
     hidden_product_kernel<float><<<blocks, 256, 0, st>>>(
         (float*)h, (const float*)factor, (const float*)uniform, keep_prob,
         1.f / keep_prob, (float*)noise_out, n);
@@ -2037,7 +2135,10 @@ extern "C" int mesh_moe_activation(const void* pre, void* out, int64_t n,
               MESH_MOE_E_ARG, "activation: unknown activation %d", activation);
   hipStream_t st = (hipStream_t)stream;
   const int blocks = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
-  if (dtype == MESH_MOE_F32)
+  if (x8_applies(n, dtype, pre, out, nullptr))
+    activation_bf16x8_kernel<<<elementwise_blocks(n / 8), 256, 0, st>>>(
+        (const uint4*)pre, (uint4*)out, n / 8, activation);
+  else if (dtype == MESH_MOE_F32)
     activation_copy_kernel<float><<<blocks, 256, 0, st>>>(
         (const float*)pre, (float*)out, n, activation);
   else
@@ -2115,17 +2216,9 @@ extern "C" int mesh_moe_expert_linear_backward(
                       da_relu_mask, &masked);
     if (rc != 0) return rc;
     if (da_relu_mask != nullptr && !masked) {
-      const int64_t n = (int64_t)E * R * K;
-      const int blocks = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
-      if (dtype == MESH_MOE_F32)
-        hidden_grad_kernel<float><<<blocks, 256, 0, st>>>(
-            (float*)da, (const float*)da_relu_mask, (const float*)nullptr, true,
-            n);
-      else
-        hidden_grad_kernel<bf16_t><<<blocks, 256, 0, st>>>(
-            (bf16_t*)da, (const bf16_t*)da_relu_mask, (const bf16_t*)nullptr,
-            true, n);
-      MOE_CHECK_LAUNCH("expert_linear_backward (relu mask)");
+      rc = launch_hidden_grad(da, da_relu_mask, nullptr, true,
+                              (int64_t)E * R * K, dtype, st);
+      if (rc != 0) return rc;
     }
   }
   // dw [E, K, N] = a^T . dy: the reduction runs over the rows of both operands
@@ -2199,16 +2292,9 @@ extern "C" int mesh_moe_expert_ffn_backward(
                     &masked);
   if (rc != 0) return rc;
   if (!masked && (activation == MESH_MOE_ACT_RELU || dh_scale)) {
-    const int64_t n = (int64_t)E * R * H;
-    const bool relu = activation == MESH_MOE_ACT_RELU;
-    const int blocks = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
-    if (dtype == MESH_MOE_F32)
-      hidden_grad_kernel<float><<<blocks, 256, 0, st>>>(
-          (float*)dh, (const float*)h, (const float*)dh_scale, relu, n);
-    else
-      hidden_grad_kernel<bf16_t><<<blocks, 256, 0, st>>>(
-          (bf16_t*)dh, (const bf16_t*)h, (const bf16_t*)dh_scale, relu, n);
-    MOE_CHECK_LAUNCH("expert_ffn_backward (hidden mask)");
+    rc = launch_hidden_grad(dh, h, dh_scale, activation == MESH_MOE_ACT_RELU,
+                            (int64_t)E * R * H, dtype, st);
+    if (rc != 0) return rc;
   }
   // dexpert_in = dh . wi^T  (wi in its variable layout [E, M, H])
   rc = grouped_gemm(dh, wi, dexpert_in, E, R, M, H, MESH_MOE_ACT_LINEAR, dtype,
@@ -2331,12 +2417,9 @@ extern "C" int mesh_moe_compact_expert_ffn_backward(
     // the dropout's noise (and the ReLU mask) as a pass over the buffer, as in
     // mesh_moe_expert_ffn_backward; rows outside the listed tiles hold
     // unspecified values before and after
-    const int64_t n = (int64_t)E * R * H;
-    const int blocks = (int)((n + 255) / 256 < 65536 ? (n + 255) / 256 : 65536);
-    hidden_grad_kernel<bf16_t><<<blocks, 256, 0, st>>>(
-        dh, (const bf16_t*)h, (const bf16_t*)dh_scale,
-        activation == MESH_MOE_ACT_RELU, n);
-    MOE_CHECK_LAUNCH("compact_expert_ffn_backward (hidden mask)");
+    rc = launch_hidden_grad(dh, h, dh_scale, activation == MESH_MOE_ACT_RELU,
+                            (int64_t)E * R * H, dtype, st);
+    if (rc != 0) return rc;
   }
   // dexpert_in = dh . wi^T on the listed row tiles
   rc = launch_ring(dh, (const bf16_t*)wi, (bf16_t*)dexpert_in, E, R, M, H,
