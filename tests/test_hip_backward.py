@@ -305,7 +305,8 @@ def test_compact_gradient_calls_edge_fills(hip):
 
 
 @pytest.mark.parametrize("shape", [(4, 512, 1024, 64, 12), (3, 96, 512, 16, 8),
-                                   (2, 64, 1536, 128, 1)],
+                                   (2, 64, 1536, 128, 1), (2, 64, 512, 48, 4),
+                                   (1, 96, 256, 80, 3), (3, 32, 768, 112, 1)],
                          ids=lambda s: "x".join(map(str, s)))
 def test_dispatch_backward_router_share_on_matrix_cores(hip, shape):
   """d(tokens) = the rows of d(expert_in) + d(logits) . w_gate^T with the
