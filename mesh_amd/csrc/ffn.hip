@@ -565,8 +565,10 @@ struct RingCfg {
 // (Skipping, inside an expert's last listed tile, the 32-row pieces of a
 // wavefront's sub-tile that lie past the occupied rows -- about a tenth of the
 // multiply-adds with 1024 +- 32 rows per expert -- made the launches 2 to 5 %
-// slower: the branches around every matrix instruction cost more than the
-// instructions saved.)
+// slower; so did letting only the wavefronts of a tile's empty second half
+// skip their multiply-adds, with the flag carried in the list entry: 5 %
+// slower, although nothing was added to the path of the full tiles but a
+// second copy of the K loop next to it.)
 // 512 bytes that stay zero (nothing writes them): where a K-major tile reaches
 // past the last reduction row, its rows are loaded from here
 static __device__ __attribute__((aligned(256))) bf16_t kmajor_zero_row[256];
