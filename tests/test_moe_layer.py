@@ -1351,3 +1351,57 @@ def test_captured_step_replays_match_eager(act_dtype):
     assert torch.equal(lowering.export_to_tf_tensor(y), replayed), trial
     assert not torch.equal(replayed, eager)
     eager = replayed
+
+
+def test_captured_gradient_step_on_compacted_rows():
+  """A recorded forward + backward step of a switch layer at a shape whose
+  gradient graph stays on compacted rows: every replay, on new tokens, with
+  eager steps and synchronisations between the replays, gives what the eager
+  step gives.  (The router kernel's gradient is summed with float atomics: it
+  is compared to rounding, everything else bit for bit.)"""
+  b, l, m, hdim, e, group = 2, 1024, 256, 512, 4, 1024
+  rng = np.random.default_rng(611)
+  w = dict(w_gate=H.normal_weights(rng, (m, e), m),
+           wi=H.normal_weights(rng, (e, m, hdim), m),
+           wo=H.normal_weights(rng, (e, hdim, m), hdim))
+  hp, _ = make_hparams(moe_num_experts=e, moe_hidden_size=hdim,
+                       moe_group_size=group, moe_capacity_factor_train=1.25,
+                       **SWITCH_HP)
+  dt = torch.bfloat16
+  xs = [O.cast_act(rng.standard_normal((b, l, m)).astype(np.float32), "bfloat16")
+        for _ in range(3)]
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  dims = [mtf.Dimension("batch", b), mtf.Dimension("length", l),
+          mtf.Dimension("d_model", m)]
+  xt = mtf.import_tf_tensor(mesh, torch.from_numpy(xs[0]).to(dt), mtf.Shape(dims))
+  with mtf.variable_scope("moe"):
+    y, loss = moe.transformer_moe_layer_v1(
+        xt, dims[-1], hp, True, mtf.VariableDType(torch.float32, torch.float32, dt))
+  variables = graph.trainable_variables
+  d_out = O.cast_act(rng.standard_normal((b, l, m)).astype(np.float32), "bfloat16")
+  dyt = mtf.import_tf_tensor(mesh, torch.from_numpy(d_out).to(dt), mtf.Shape(dims))
+  grads = mtf.gradients([y, loss], [xt] + [v.outputs[0] for v in variables],
+                        grad_ys=[dyt, None])
+  init = {"moe/switch_gating/kernel": w["w_gate"], "moe/wi/kernel": w["wi"],
+          "moe/wo/kernel": w["wo"]}
+  from mesh_amd import moe_hip
+  with moe_hip.StageTimer() as timer:
+    lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()}, initial_values=init)
+  assert timer.compacted == 1
+  step = lowering.capture()
+  for i in (1, 2, 0, 1):
+    xv = torch.from_numpy(xs[i]).to(dt).cuda()
+    lowering.run({xt: xv})
+    eager = [lowering.export_to_tf_tensor(t).clone() for t in [y] + grads]
+    torch.cuda.synchronize()
+    step.replay({xt: xv})
+    torch.cuda.synchronize()
+    for j, (t, want) in enumerate(zip([y] + grads, eager)):
+      got = lowering.export_to_tf_tensor(t)
+      if j == 2:          # the router kernel's gradient
+        np.testing.assert_allclose(
+            H.to_np(got), H.to_np(want), rtol=2e-2,
+            atol=1e-2 * float(want.float().abs().max()))
+      else:
+        assert torch.equal(got, want), (i, j)
