@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 30
+#define MESH_MOE_ABI_VERSION 31
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -631,8 +631,12 @@ int mesh_moe_gating_backward(const float* logits, const void* importance,
  * (transformer/moe.py:1384-1390): dw_gate[m,e] = sum_t float(x[t,m]) *
  * dlogits[t,e], float32 accumulate, stored in dtype.
  *   x [tokens,M] dtype; dlogits [tokens,E] float32; dw_gate [M,E] dtype
- *   workspace: M*E float32
+ *   workspace: mesh_moe_router_backward_weights_workspace_bytes(tokens, M, E,
+ *   dtype) bytes (M*E float32, or one such plane per chunk of tokens for the
+ *   bf16 kernel that sums its chunks in a fixed order)
  */
+size_t mesh_moe_router_backward_weights_workspace_bytes(int64_t tokens, int M,
+                                                        int E, int dtype);
 int mesh_moe_router_backward_weights(const void* x, const float* dlogits,
                                      void* dw_gate, float* workspace,
                                      int64_t tokens, int M, int E, int dtype,

@@ -857,7 +857,10 @@ __global__ __launch_bounds__(256) void router_wgrad_mfma_kernel(
 // at (row t / 4, elements 4 (t % 4) ..) of a 4 x 16 block and lane i receives
 // the block's column i.  Block = 128 kernel rows x 64 experts x WB_TOK tokens,
 // 32 tokens staged at a time; a wavefront owns 32 rows x 64 experts.  Rows are
-// padded so that the four rows of a block lie in different banks.
+// padded so that the four rows of a block lie in different banks.  Every
+// block writes its sums to its token chunk's [M, E] plane of the workspace
+// and router_wgrad_reduce_kernel adds the planes in chunk order: the same
+// bits on every run (the other kernels add with float atomics).
 // Needs M % 128 == 0, E % 8 == 0 and 16-byte aligned rows.
 // ---------------------------------------------------------------------------
 constexpr int WB_M = 128, WB_TOK = 2048, WB_KT = 32;
@@ -955,13 +958,26 @@ __global__ __launch_bounds__(256) void router_wgrad_bf16_kernel(
     acc0 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, l10, acc0, 0, 0, 0);
     acc1 = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, l11, acc1, 0, 0, 0);
   }
+  // this block's partial sums: chunk blockIdx.y of acc_out [chunks][M][E]
+  float* part = acc_out + (int64_t)blockIdx.y * M * E;
 #pragma unroll
   for (int r = 0; r < 16; ++r) {
     const int m = m0 + wave * 32 + 8 * (r / 4) + 4 * half + (r % 4);
-    if (e0 + l32 < E) atomicAdd(acc_out + (int64_t)m * E + e0 + l32, acc0[r]);
-    if (e0 + 32 + l32 < E)
-      atomicAdd(acc_out + (int64_t)m * E + e0 + 32 + l32, acc1[r]);
+    if (e0 + l32 < E) part[(int64_t)m * E + e0 + l32] = acc0[r];
+    if (e0 + 32 + l32 < E) part[(int64_t)m * E + e0 + 32 + l32] = acc1[r];
   }
+}
+
+// dw = sum over the token chunks of the partial sums, in chunk order
+template <typename T>
+__global__ void router_wgrad_reduce_kernel(const float* __restrict__ part,
+                                           T* __restrict__ dw, int64_t n,
+                                           int chunks) {
+  const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  float sum = 0.f;
+  for (int c = 0; c < chunks; ++c) sum += part[(int64_t)c * n + i];
+  store_f32<T>(dw + i, sum);
 }
 
 // ---------------------------------------------------------------------------
@@ -1399,6 +1415,19 @@ extern "C" int mesh_moe_gating_backward(
   return 0;
 }
 
+static bool router_wgrad_bf16_applies(int64_t tokens, int M, int E, int dtype) {
+  return dtype == MESH_MOE_BF16 && ((size_t)M * 2) % 16 == 0 && E % 8 == 0 &&
+         M % WB_M == 0 && (tokens + WB_TOK - 1) / WB_TOK <= 65535;
+}
+
+extern "C" size_t mesh_moe_router_backward_weights_workspace_bytes(
+    int64_t tokens, int M, int E, int dtype) {
+  if (tokens < 1 || M < 1 || E < 1 || !valid_dtype(dtype)) return 0;
+  const size_t planes = router_wgrad_bf16_applies(tokens, M, E, dtype)
+                            ? (size_t)((tokens + WB_TOK - 1) / WB_TOK) : 1;
+  return sizeof(float) * planes * (size_t)M * E;
+}
+
 extern "C" int mesh_moe_router_backward_weights(const void* x,
                                                 const float* dlogits,
                                                 void* dw_gate,
@@ -1420,6 +1449,20 @@ extern "C" int mesh_moe_router_backward_weights(const void* x,
   hipStream_t st = (hipStream_t)stream;
   const int64_t n = (int64_t)M * E;
   const unsigned fb = (unsigned)((n + 255) / 256 < 4096 ? (n + 255) / 256 : 4096);
+  if (router_wgrad_bf16_applies(tokens, M, E, dtype) && bw_aligned16(x) &&
+      bw_aligned16(dlogits)) {
+    const int bchunks = (int)((tokens + WB_TOK - 1) / WB_TOK);
+    dim3 bgrid((unsigned)(M / WB_M), (unsigned)bchunks,
+               (unsigned)((E + 63) / 64));
+    router_wgrad_bf16_kernel<<<bgrid, 256, 0, st>>>(
+        (const bf16_t*)x, dlogits, workspace, tokens, M, E);
+    MOE_CHECK_LAUNCH("router_backward_weights (mfma, bf16 terms)");
+    router_wgrad_reduce_kernel<bf16_t><<<(unsigned)((n + 255) / 256), 256, 0,
+                                         st>>>(workspace, (bf16_t*)dw_gate, n,
+                                               bchunks);
+    MOE_CHECK_LAUNCH("router_backward_weights (sum of the chunks)");
+    return 0;
+  }
   fill_f32_kernel<<<fb, 256, 0, st>>>(workspace, n, 0.0f);
   MOE_CHECK_LAUNCH("router_backward_weights (clear)");
   dim3 grid((unsigned)((M + WG_M - 1) / WG_M), (unsigned)chunks,
@@ -1440,12 +1483,10 @@ extern "C" int mesh_moe_router_backward_weights(const void* x,
       MOE_CHECK_LAUNCH("router_backward_weights (mfma)");
       convert_f32_kernel<float><<<fb, 256, 0, st>>>(workspace, (float*)dw_gate, n);
     } else {
-      const int64_t bchunks = (tokens + WB_TOK - 1) / WB_TOK;
-      dim3 bgrid((unsigned)(M / WB_M), (unsigned)bchunks,
-                 (unsigned)((E + 63) / 64));
-      router_wgrad_bf16_kernel<<<bgrid, 256, 0, st>>>(
+      // (unaligned bf16 operands: the float32 matrix cores)
+      router_wgrad_mfma_kernel<bf16_t><<<mgrid, 256, 0, st>>>(
           (const bf16_t*)x, dlogits, workspace, tokens, M, E);
-      MOE_CHECK_LAUNCH("router_backward_weights (mfma, bf16 terms)");
+      MOE_CHECK_LAUNCH("router_backward_weights (mfma)");
       convert_f32_kernel<bf16_t><<<fb, 256, 0, st>>>(workspace, (bf16_t*)dw_gate,
                                                     n);
     }

@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 30
+ABI_VERSION = 31
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -178,6 +178,8 @@ _SIGNATURES = {
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_double, ctypes.c_int, _vp, _vp,
         ctypes.c_size_t, _vp]),
+    "mesh_moe_router_backward_weights_workspace_bytes": (ctypes.c_size_t, [
+        ctypes.c_int64, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "mesh_moe_router_backward_weights": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, ctypes.c_int64, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, _vp]),
@@ -1091,7 +1093,10 @@ def router_backward_weights(x, dlogits):
   t, m = x.shape
   e = dlogits.shape[-1]
   out = torch.empty((m, e), dtype=x.dtype, device=x.device)
-  ws = torch.empty((m, e), dtype=torch.float32, device=x.device)
+  ws_bytes = lib.mesh_moe_router_backward_weights_workspace_bytes(
+      t, m, e, dtype_code(x.dtype))
+  ws = torch.empty((max(ws_bytes // 4, 1),), dtype=torch.float32,
+                   device=x.device)
   with _stage("router_backward_weights"):
     _check(lib.mesh_moe_router_backward_weights(
         _dev(x, "x"), _dev(dlogits, "dlogits", torch.float32, (t, e)),

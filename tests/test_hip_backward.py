@@ -163,6 +163,22 @@ def test_backward_matches_oracle(hip, case):
                                err_msg=k)
 
 
+def test_router_backward_weights_repeats_bit_for_bit(hip):
+  """bfloat16 tokens at widths the bfloat16 matrix-core kernel takes: the sums
+  over the token chunks run in a fixed order, so two calls give the same bits
+  (and the float64 product to rounding)."""
+  t, m, e = 10000, 512, 64
+  gen = torch.Generator(device="cuda").manual_seed(3)
+  x = torch.randn((t, m), generator=gen, device="cuda").to(torch.bfloat16)
+  dl = torch.randn((t, e), generator=gen, device="cuda") * 0.1
+  a = hip.router_backward_weights(x, dl)
+  b = hip.router_backward_weights(x, dl)
+  assert torch.equal(a, b)
+  want = x.double().t() @ dl.double()
+  err = (a.double() - want).abs()
+  assert bool((err <= want.abs() * 2.0 ** -8 * 1.01 + 1e-4).all())
+
+
 COMPACT_CASES = [
     # gating, G, S, M, H, E, capacity factor, padding mask
     ("switch", 4, 512, 256, 512, 8, 2.0, True),
