@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 31
+#define MESH_MOE_ABI_VERSION 32
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -540,14 +540,19 @@ size_t mesh_moe_expert_ffn_backward_workspace_bytes(int E, int R, int M, int H,
  *   wi [E,M,H], wo [E,H,N]: the variables' own layout (NOT the packed one)
  *   dh_scale [E,R,H] dtype or NULL: the dropout noise mesh_moe_hidden_product
  *   wrote (transformer/moe.py:477-479)
+ *   dh_keep_prob: the keep probability that noise was made with, or 0 if the
+ *   caller does not know it.  Known, bf16 ReLU experts do not read dh_scale:
+ *   where h > 0 the element was kept and its noise is 1 / keep_prob
  *   dexpert_in [E,R,M]; dwi [E,M,H]; dwo [E,H,N]; everything of `dtype`
  * Four grouped GEMMs on the forward kernels; the weight gradients read both
  * operands as they are (reduction index outermost) where the kernel takes the
- * shape (bf16, R a multiple of 64), through transposed copies otherwise.
+ * shape (bf16, kernel dimensions multiples of 8), through transposed copies
+ * otherwise.
  */
 int mesh_moe_expert_ffn_backward(const void* expert_in, const void* h,
                                  const void* dy, const void* wi,
                                  const void* wo, const void* dh_scale,
+                                 float dh_keep_prob,
                                  void* dexpert_in, void* dwi, void* dwo, int E,
                                  int R, int M, int H, int N, int activation,
                                  int dtype, void* workspace,
@@ -685,7 +690,7 @@ int mesh_moe_dispatch_backward(const void* dexpert_in, const int32_t* idx,
  * mesh_moe_combine_backward_compact: mesh_moe_combine_backward with y and dy
  *   in compacted rows.
  * mesh_moe_compact_expert_ffn_backward: mesh_moe_expert_ffn_backward
- *   (relu or linear experts; dh_scale as there); bf16, E <= 1024 and shapes the
+ *   (relu or linear experts; dh_scale and dh_keep_prob as there); bf16, E <= 1024 and shapes the
  *   256 x 256 kernels take, else MESH_MOE_E_UNSUPPORTED;
  *   ..._workspace_bytes returns 0 for shapes it does not take.
  * mesh_moe_dispatch_backward_compact: mesh_moe_dispatch_backward reading
@@ -707,10 +712,11 @@ size_t mesh_moe_compact_expert_ffn_backward_workspace_bytes(int G, int E, int C,
                                                             int N);
 int mesh_moe_compact_expert_ffn_backward(
     const void* expert_in, const void* h, const void* dy, const void* wi,
-    const void* wo, const void* dh_scale, const int32_t* fill,
-    const int32_t* row_offsets, void* dexpert_in, void* dwi, void* dwo, int G,
-    int E, int C, int M, int H, int N, int activation, int dtype,
-    void* workspace, size_t workspace_bytes, void* stream);
+    const void* wo, const void* dh_scale, float dh_keep_prob,
+    const int32_t* fill, const int32_t* row_offsets, void* dexpert_in,
+    void* dwi, void* dwo, int G, int E, int C, int M, int H, int N,
+    int activation, int dtype, void* workspace, size_t workspace_bytes,
+    void* stream);
 int mesh_moe_dispatch_backward_compact(
     const void* dexpert_in, const int32_t* idx, const int32_t* pos,
     const float* gate, const uint8_t* kept, const int32_t* row_offsets,

@@ -556,7 +556,10 @@ struct RingCfg {
 //
 // MASKED: element (e, r, n) of the result is stored as zero unless
 // mask_src[e][r][n] > 0 (the backward of a ReLU whose output is mask_src,
-// applied while the tile is written out).
+// applied while the tile is written out).  The elements that stay are
+// multiplied by mask_scale and rounded again (the backward of a dropout in
+// front of the ReLU's consumer: where the stored activation is positive the
+// element was kept, and its noise is 1 / keep_prob).
 //
 // LISTED: only the tiles named in tile_list[0 .. tile_list[-1]) are computed
 // (logical tile numbers in ascending order, their count in the element before
@@ -582,7 +585,8 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
     const bf16_t* __restrict__ zero_row = nullptr,
     const bf16_t* __restrict__ mask_src = nullptr,
     const int32_t* __restrict__ tile_list = nullptr,
-    const int32_t* __restrict__ row_count = nullptr) {
+    const int32_t* __restrict__ row_count = nullptr,
+    float mask_scale = 1.0f) {
   using Cfg = RingCfg;
   // row_count [E], optional: KMAJOR kernels take it as the reduction extent
   // per expert (k_extent)
@@ -979,6 +983,13 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
           if constexpr (MASKED) {
             const u32x4_t hm = *reinterpret_cast<const u32x4_t*>(
                 mask_src + (out_c - Cout) + (int64_t)grow * N + gcol);
+            if (mask_scale != 1.0f) {
+#pragma unroll
+              for (int q = 0; q < 4; ++q)
+                v[q] = f32x2_to_bf16x2(
+                    __builtin_bit_cast(float, v[q] << 16) * mask_scale,
+                    __builtin_bit_cast(float, v[q] & 0xffff0000u) * mask_scale);
+            }
 #pragma unroll
             for (int q = 0; q < 4; ++q) {
               const uint32_t keep =
@@ -1533,7 +1544,7 @@ static int launch_ring_kmajor(const bf16_t* A, const bf16_t* B, bf16_t* C,
   MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
   k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
       A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr,
-      nullptr, nullptr, k_extent);
+      nullptr, nullptr, k_extent, 1.0f);
   MOE_CHECK_LAUNCH("expert_ffn_backward (mfma, K-major operands)");
   return 0;
 }
@@ -1543,7 +1554,8 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
                        const int32_t* row_map = nullptr,
                        const bf16_t* zero_row = nullptr,
                        const bf16_t* mask_src = nullptr,
-                       const int32_t* tile_list = nullptr) {
+                       const int32_t* tile_list = nullptr,
+                       float mask_scale = 1.0f) {
   using Cfg = RingCfg;
   const int tiles_m = (R + Cfg::BM - 1) / Cfg::BM;
   const int tiles_n = (N + Cfg::BN - 1) / Cfg::BN;
@@ -1560,7 +1572,7 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
     MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
     k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
         A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr,
-        mask_src, tile_list, nullptr);
+        mask_src, tile_list, nullptr, mask_scale);
     MOE_CHECK_LAUNCH("expert_ffn (mfma, listed tiles, masked result)");
     return 0;
   }
@@ -1572,7 +1584,7 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
     MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);                                          \
     k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(                           \
         A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, row_map, zero_row,     \
-        nullptr, tile_list, nullptr);                                          \
+        nullptr, tile_list, nullptr, 1.0f);                                    \
   } while (0)
     if (row_map != nullptr) {
       if (relu) MOE_RING_LISTED(true, true);
@@ -1592,7 +1604,7 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
     MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
     k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
         A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr,
-        mask_src, nullptr, nullptr);
+        mask_src, nullptr, nullptr, mask_scale);
     MOE_CHECK_LAUNCH("expert_ffn (mfma, masked result)");
     return 0;
   }
@@ -1602,13 +1614,13 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
       MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
       k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
           A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, row_map, zero_row,
-          nullptr, nullptr, nullptr);
+          nullptr, nullptr, nullptr, 1.0f);
     } else {
       auto k = grouped_gemm_bf16_ring_kernel<false, true>;
       MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
       k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
           A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, row_map, zero_row,
-          nullptr, nullptr, nullptr);
+          nullptr, nullptr, nullptr, 1.0f);
     }
     MOE_CHECK_LAUNCH("expert_ffn (mfma, gathered rows)");
     return 0;
@@ -1618,13 +1630,13 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
     MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
     k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
         A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr,
-        nullptr, nullptr, nullptr);
+        nullptr, nullptr, nullptr, 1.0f);
   } else {
     auto k = grouped_gemm_bf16_ring_kernel<false, false>;
     MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
     k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
         A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr,
-        nullptr, nullptr, nullptr);
+        nullptr, nullptr, nullptr, 1.0f);
   }
   MOE_CHECK_LAUNCH("expert_ffn (mfma, spread direct-to-LDS loads)");
   return 0;
@@ -1677,7 +1689,7 @@ static int launch_simple(const T* A, const T* B, T* C, int E, int R, int N,
 static int grouped_gemm(const void* A, const void* B, void* C, int E, int R,
                         int N, int K, int act, int dtype, hipStream_t st,
                         const void* relu_mask_src = nullptr,
-                        bool* mask_applied = nullptr) {
+                        bool* mask_applied = nullptr, float mask_scale = 1.0f) {
   const bool relu = act == MESH_MOE_ACT_RELU;
   int rc;
   if (mask_applied) *mask_applied = false;
@@ -1712,7 +1724,7 @@ static int grouped_gemm(const void* A, const void* B, void* C, int E, int R,
       } else if (relu_mask_src != nullptr && mask_applied != nullptr && !relu &&
                  ((uintptr_t)relu_mask_src % 16) == 0) {
         rc = launch_ring(a, b, c, E, R, N, K, false, st, nullptr, nullptr,
-                         (const bf16_t*)relu_mask_src);
+                         (const bf16_t*)relu_mask_src, nullptr, mask_scale);
         *mask_applied = rc == 0;
       } else {
         rc = launch_ring(a, b, c, E, R, N, K, relu, st);
@@ -2259,8 +2271,8 @@ extern "C" size_t mesh_moe_expert_ffn_backward_workspace_bytes(int E, int R,
 
 extern "C" int mesh_moe_expert_ffn_backward(
     const void* expert_in, const void* h, const void* dy, const void* wi,
-    const void* wo, const void* dh_scale, void* dexpert_in, void* dwi,
-    void* dwo, int E, int R,
+    const void* wo, const void* dh_scale, float dh_keep_prob,
+    void* dexpert_in, void* dwi, void* dwo, int E, int R,
     int M, int H, int N, int activation, int dtype, void* workspace,
     size_t workspace_bytes, void* stream) {
   MOE_REQUIRE(expert_in && h && dy && wi && wo && dexpert_in && dwi && dwo &&
@@ -2288,10 +2300,19 @@ extern "C" int mesh_moe_expert_ffn_backward(
   int rc;
   // dh = dy . wo^T  (wo in its variable layout [E, H, N] is K-contiguous here)
   // (the ReLU mask rides on the stores of this GEMM where its kernel can)
+  // With a dropout whose keep probability is known, a ReLU expert's noise need
+  // not be read: where the stored activation is positive the element was kept
+  // and its noise is 1 / keep_prob (as mesh_moe_hidden_product rounds it).
+  const bool relu_act = activation == MESH_MOE_ACT_RELU;
+  const bool noise_by_mask = relu_act && dh_scale != nullptr &&
+                             dh_keep_prob > 0.f && dh_keep_prob <= 1.f &&
+                             dtype == MESH_MOE_BF16;
+  const float mask_scale =
+      noise_by_mask ? round_bf16_host(1.f / round_bf16_host(dh_keep_prob)) : 1.f;
   bool masked = false;
   rc = grouped_gemm(dy, wo, dh, E, R, H, N, MESH_MOE_ACT_LINEAR, dtype, st,
-                    activation == MESH_MOE_ACT_RELU && !dh_scale ? h : nullptr,
-                    &masked);
+                    relu_act && (!dh_scale || noise_by_mask) ? h : nullptr,
+                    &masked, mask_scale);
   if (rc != 0) return rc;
   if (!masked && (activation == MESH_MOE_ACT_RELU || dh_scale)) {
     rc = launch_hidden_grad(dh, h, dh_scale, activation == MESH_MOE_ACT_RELU,
@@ -2361,10 +2382,11 @@ extern "C" size_t mesh_moe_compact_expert_ffn_backward_workspace_bytes(
 
 extern "C" int mesh_moe_compact_expert_ffn_backward(
     const void* expert_in, const void* h, const void* dy, const void* wi,
-    const void* wo, const void* dh_scale, const int32_t* fill,
-    const int32_t* row_offsets, void* dexpert_in, void* dwi, void* dwo, int G,
-    int E, int C, int M, int H, int N, int activation, int dtype,
-    void* workspace, size_t workspace_bytes, void* stream) {
+    const void* wo, const void* dh_scale, float dh_keep_prob,
+    const int32_t* fill, const int32_t* row_offsets, void* dexpert_in,
+    void* dwi, void* dwo, int G, int E, int C, int M, int H, int N,
+    int activation, int dtype, void* workspace, size_t workspace_bytes,
+    void* stream) {
   MOE_REQUIRE(expert_in && h && dy && wi && wo && fill && row_offsets &&
                   dexpert_in && dwi && dwo && workspace, MESH_MOE_E_ARG,
               "compact_expert_ffn_backward: null pointer");
@@ -2410,12 +2432,20 @@ extern "C" int mesh_moe_compact_expert_ffn_backward(
   // dh = dy . wo^T on the listed row tiles, the ReLU mask on its stores (the
   // rows of a listed tile past the expert's occupied ones have h = 0 and
   // dy = 0)
-  const bool mask_on_stores = activation == MESH_MOE_ACT_RELU && !dh_scale;
+  // (a ReLU expert's dropout noise follows from the stored activation: see
+  // mesh_moe_expert_ffn_backward)
+  const bool noise_by_mask = activation == MESH_MOE_ACT_RELU &&
+                             dh_scale != nullptr && dh_keep_prob > 0.f &&
+                             dh_keep_prob <= 1.f;
+  const float mask_scale =
+      noise_by_mask ? round_bf16_host(1.f / round_bf16_host(dh_keep_prob)) : 1.f;
+  const bool mask_on_stores =
+      activation == MESH_MOE_ACT_RELU && (!dh_scale || noise_by_mask);
   int rc = launch_ring(
       (const bf16_t*)dy, (const bf16_t*)wo, dh, E, R, H, N, false, st, nullptr,
-      nullptr, mask_on_stores ? (const bf16_t*)h : nullptr, list_h);
+      nullptr, mask_on_stores ? (const bf16_t*)h : nullptr, list_h, mask_scale);
   if (rc != 0) return rc;
-  if (dh_scale != nullptr) {
+  if (dh_scale != nullptr && !mask_on_stores) {
     // the dropout's noise (and the ReLU mask) as a pass over the buffer, as in
     // mesh_moe_expert_ffn_backward; rows outside the listed tiles hold
     // unspecified values before and after

@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 31
+ABI_VERSION = 32
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -104,7 +104,8 @@ _SIGNATURES = {
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_int]),
     "mesh_moe_compact_expert_ffn_backward": (ctypes.c_int, [
-        _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int,
+        _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp, _vp, _vp,
+        ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, _vp, ctypes.c_size_t, _vp]),
     "mesh_moe_dispatch_backward_compact": (ctypes.c_int, [
@@ -127,7 +128,8 @@ _SIGNATURES = {
     "mesh_moe_hidden_product": (ctypes.c_int, [
         _vp, _vp, _vp, ctypes.c_float, _vp, ctypes.c_int64, ctypes.c_int, _vp]),
     "mesh_moe_expert_ffn_backward": (ctypes.c_int, [
-        _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
+        _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_float, _vp, _vp, _vp,
+        ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
         _vp, ctypes.c_size_t, _vp]),
     "mesh_moe_expert_linear_backward_workspace_bytes": (ctypes.c_size_t, [
@@ -928,10 +930,12 @@ def hidden_product(h, factor=None, uniform=None, keep_prob=1.0,
 
 
 def expert_ffn_backward(expert_in, h, dy, wi, wo, activation="relu",
-                        dh_scale=None):
+                        dh_scale=None, keep_prob=None):
   """expert_in [E,R,M], h [E,R,H], dy [E,R,N]; wi [E,M,H], wo [E,H,N] in the
   variables' own layout -> (dexpert_in [E,R,M], dwi [E,M,H], dwo [E,H,N]).
-  dh_scale [E,R,H]: the hidden dropout's noise, if there was one."""
+  dh_scale [E,R,H]: the hidden dropout's noise, if there was one; keep_prob:
+  the keep probability it was made with (lets ReLU experts skip reading
+  it)."""
   lib = load_library()
   if activation not in ACTIVATIONS:
     raise ValueError("unsupported expert activation %r" % (activation,))
@@ -952,14 +956,17 @@ def expert_ffn_backward(expert_in, h, dy, wi, wo, activation="relu",
         _dev(dy, "dy", dt, (e, rows, n)), _dev(wi, "wi", dt, (e, m, hdim)),
         _dev(wo, "wo", dt, (e, hdim, n)),
         _dev(dh_scale, "dh_scale", dt, (e, rows, hdim))
-        if dh_scale is not None else None, dxe.data_ptr(), dwi.data_ptr(),
+        if dh_scale is not None else None,
+        float(keep_prob) if keep_prob is not None else 0.0, dxe.data_ptr(),
+        dwi.data_ptr(),
         dwo.data_ptr(), e, rows, m, hdim, n, ACTIVATIONS[activation], code,
         ws.data_ptr(), ws_bytes, _stream()), "expert_ffn_backward")
   return dxe, dwi, dwo
 
 
 def compact_expert_ffn_backward(expert_in, h, dy, wi, wo, r, row_offsets,
-                                activation="relu", dh_scale=None):
+                                activation="relu", dh_scale=None,
+                                keep_prob=None):
   """expert_ffn_backward with every [E, G*C, .] tensor in the compacted row
   order of compact_expert_ffn (r: the Routing, row_offsets [E, G]; dh_scale
   [E, G*C, H]: the hidden dropout's noise, if there was one)."""
@@ -988,6 +995,7 @@ def compact_expert_ffn_backward(expert_in, h, dy, wi, wo, r, row_offsets,
         _dev(wo, "wo", dt, (e, hdim, n)),
         _dev(dh_scale, "dh_scale", dt, (e, rows, hdim))
         if dh_scale is not None else None,
+        float(keep_prob) if keep_prob is not None else 0.0,
         _dev(r.fill, "fill", torch.int32, (g, e)),
         _dev(row_offsets, "row_offsets", torch.int32, (e, g)), dxe.data_ptr(),
         dwi.data_ptr(), dwo.data_ptr(), g, e, c, m, hdim, n,

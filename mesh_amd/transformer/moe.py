@@ -669,7 +669,8 @@ class MoEV1GradOperation(mtf.Operation):
         dxe, dwi, dwo = moe_hip.compact_expert_ffn_backward(
             sv["expert_in"].reshape(e_, groups * c_, m_), sv["h"],
             dy.reshape(e_, groups * c_, n_), wi_s, wo_s, r, row_offsets,
-            fwd._activation, dh_scale=sv["hidden_noise"])
+            fwd._activation, dh_scale=sv["hidden_noise"],
+            keep_prob=fwd._hidden_keep_prob)
         dkwo, dwis = None, [dwi]
       elif fwd._general_hidden:
         dys, wos = [dy.reshape(e_, groups * c_, n_)], [wo_s]
@@ -689,7 +690,8 @@ class MoEV1GradOperation(mtf.Operation):
         dxe, dwi, dwo = moe_hip.expert_ffn_backward(
             sv["expert_in"].reshape(e_, groups * c_, m_), sv["h"],
             dy.reshape(e_, groups * c_, n_), wi_s, wo_s, fwd._activation,
-            dh_scale=sv["hidden_noise"])
+            dh_scale=sv["hidden_noise"],
+            keep_prob=fwd._hidden_keep_prob)
         dkwo, dwis = None, [dwi]
       if kwo_s is not None:
         # the second projection of the same hidden tensor: its share of every
@@ -701,7 +703,8 @@ class MoEV1GradOperation(mtf.Operation):
         dxe_k, dwi_k, dkwo = moe_hip.expert_ffn_backward(
             sv["expert_in"].reshape(e_, groups * c_, m_), sv["h"],
             dyk.reshape(e_, groups * c_, n_), wi_s, kwo_s, fwd._activation,
-            dh_scale=sv["hidden_noise"])
+            dh_scale=sv["hidden_noise"],
+            keep_prob=fwd._hidden_keep_prob)
         dxe, dwi, dgate = dxe + dxe_k, dwi + dwi_k, dgate + dgate_k
       if by_slot:
         dlogits = moe_hip.expert_choice_backward(

@@ -1302,3 +1302,54 @@ def test_expert_choice_backward_wide_rows(hip, shape):
   assert (err <= np.abs(want) * 2.0 ** -8 * 1.01 + 4e-5).all()
   step = np.abs(H.to_np(got) - H.to_np(plain))
   assert (step <= np.abs(H.to_np(plain)) * 2.0 ** -7 + 4e-5).all()
+
+
+def test_dropout_noise_from_the_relu_mask(hip):
+  """Backward of ReLU experts behind a hidden dropout: told the keep
+  probability, the library takes the noise from the stored activation (kept
+  where it is positive, 1 / keep_prob there) while the dh GEMM writes its
+  tiles; told nothing it reads the noise tensor in a pass of its own.  Same
+  bits either way, padded and compacted rows."""
+  e, g, c, m, hdim, keep = 4, 2, 256, 256, 512, 0.75
+  dt = torch.bfloat16
+  gen = torch.Generator(device="cuda").manual_seed(77)
+  mk = lambda *sh: torch.randn(sh, generator=gen, device="cuda")
+  xe = mk(e, g * c, m).to(dt)
+  wi = (mk(e, m, hdim) / m ** 0.5).to(dt)
+  wo = (mk(e, hdim, m) / hdim ** 0.5).to(dt)
+  dy = mk(e, g * c, m).to(dt)
+  h = hip.expert_linear(xe, hip.pack_weights(wi, dt), "relu")
+  u = torch.rand(h.shape, generator=gen, device="cuda").to(dt)
+  noise = hip.hidden_product(h, uniform=u, keep_prob=keep, want_noise=True)
+  assert 0.2 < float((noise == 0).float().mean()) < 0.3
+  a = hip.expert_ffn_backward(xe, h, dy, wi, wo, "relu", dh_scale=noise,
+                              keep_prob=keep)
+  b = hip.expert_ffn_backward(xe, h, dy, wi, wo, "relu", dh_scale=noise)
+  for x_, y_ in zip(a, b):
+    assert torch.equal(x_, y_)
+  assert float(a[0].abs().sum()) > 0
+  # compacted rows: a switch routing that fills about half of the slots
+  s = 1024
+  r = hip.switch_gating(mk(g, s, e), c)
+  xg = mk(g, s, m).to(dt)
+  wi_p, wo_p = hip.pack_weights(wi, dt), hip.pack_weights(wo, dt)
+  uc = torch.rand((e, g * c, hdim), generator=gen, device="cuda").to(dt)
+  y_c, ro, h_c, noise_c = hip.compact_expert_ffn(
+      xg, r, wi_p, wo_p, "relu", want_hidden=True, uniform=uc, keep_prob=keep,
+      want_noise=True)
+  xe_c = hip.dispatch(xg, r, row_offsets=ro).reshape(e, g * c, m)
+  dy_c, _ = hip.combine_backward(mk(g, s, m).to(dt), y_c.reshape(e, g, c, m), r,
+                                 row_offsets=ro)
+  dy_c = dy_c.reshape(e, g * c, m)
+  a = hip.compact_expert_ffn_backward(xe_c, h_c, dy_c, wi, wo, r, ro, "relu",
+                                      dh_scale=noise_c, keep_prob=keep)
+  b = hip.compact_expert_ffn_backward(xe_c, h_c, dy_c, wi, wo, r, ro, "relu",
+                                      dh_scale=noise_c)
+  fill = r.fill.cpu().numpy()
+  used = fill.sum(0)
+  for j, (x_, y_) in enumerate(zip(a, b)):
+    if j == 0:      # d(expert_in): the occupied rows (the rest is unspecified)
+      for ei in range(e):
+        assert torch.equal(x_[ei, :used[ei]], y_[ei, :used[ei]]), ei
+    else:
+      assert torch.equal(x_, y_), j

@@ -846,7 +846,10 @@ def test_v1_switch_hidden_dropout_on_compacted_rows():
     # gradient graph on compacted rows
     ("switch+compact", "bfloat16", 114), ("ntlb+compact", "bfloat16", 115),
     ("switch+compact+input_jitter", "bfloat16", 116),
-    ("switch+compact+hidden_dropout", "bfloat16", 117)],
+    ("switch+compact+hidden_dropout", "bfloat16", 117),
+    # the same sizes behind a top-2 router (padded rows): the dropout's noise
+    # rides on the ReLU mask of the dh GEMM
+    ("top_2+large+hidden_dropout", "bfloat16", 118)],
     ids=lambda c: "%s-%s" % (c[0], c[1]))
 def test_v1_gradients_match_oracle(case, monkeypatch):
   """mtf.gradients over the layer (outputs and loss) against the oracle's
@@ -854,7 +857,8 @@ def test_v1_gradients_match_oracle(case, monkeypatch):
   gating, act_dtype, seed = case
   gating, _, noise_policy = gating.partition("+")
   compact = noise_policy.startswith("compact")
-  if compact:
+  large = compact or noise_policy.startswith("large")
+  if large:
     noise_policy = noise_policy.partition("+")[2]
   hidden_dropout = noise_policy == "hidden_dropout"
   loss2 = noise_policy == "second_place_loss"
@@ -862,8 +866,9 @@ def test_v1_gradients_match_oracle(case, monkeypatch):
     noise_policy = ""
   b, l, m, hdim, e, group = 2, 64, 32, 48, 4, 32
   compact_calls = []
-  if compact:
+  if large:
     b, l, m, hdim, e, group = 2, 1024, 256, 512, 4, 1024
+  if compact:
     from mesh_amd import moe_hip
     inner = moe_hip.compact_expert_ffn_backward
     def counted(*args, **kwargs):
