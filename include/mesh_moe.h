@@ -541,8 +541,9 @@ size_t mesh_moe_expert_ffn_backward_workspace_bytes(int E, int R, int M, int H,
  *   dh_scale [E,R,H] dtype or NULL: the dropout noise mesh_moe_hidden_product
  *   wrote (transformer/moe.py:477-479)
  *   dh_keep_prob: the keep probability that noise was made with, or 0 if the
- *   caller does not know it.  Known, bf16 ReLU experts do not read dh_scale:
- *   where h > 0 the element was kept and its noise is 1 / keep_prob
+ *   caller does not know it (or there was none).  Known, ReLU experts do not
+ *   read dh_scale, which may then be NULL: where h > 0 the element was kept
+ *   and its noise is 1 / keep_prob
  *   dexpert_in [E,R,M]; dwi [E,M,H]; dwo [E,H,N]; everything of `dtype`
  * Four grouped GEMMs on the forward kernels; the weight gradients read both
  * operands as they are (reduction index outermost) where the kernel takes the

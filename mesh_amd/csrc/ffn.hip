@@ -1242,10 +1242,13 @@ __global__ __launch_bounds__(256) void activation_copy_kernel(
 // the hidden dropout and the ReLU of the forward pass seen from behind (h is
 // the stored, already rounded activation: positive iff the pre-activation
 // rounded to a positive value and the element was not dropped).
+// (const_scale: one factor for every element that stays, in place of a scale
+// tensor -- a dropout's noise where the ReLU mask already says which elements
+// were kept.)
 template <typename T>
 __global__ __launch_bounds__(256) void hidden_grad_kernel(
     T* __restrict__ dh, const T* __restrict__ h, const T* __restrict__ scale,
-    bool relu, int64_t n) {
+    bool relu, int64_t n, float const_scale) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
        i += stride) {
@@ -1253,6 +1256,8 @@ __global__ __launch_bounds__(256) void hidden_grad_kernel(
       dh[i] = (T)0;
     } else if (scale) {
       store_f32<T>(dh + i, load_f32<T>(dh + i) * load_f32<T>(scale + i));
+    } else if (const_scale != 1.0f) {
+      store_f32<T>(dh + i, load_f32<T>(dh + i) * const_scale);
     }
   }
 }
@@ -1356,7 +1361,8 @@ __global__ __launch_bounds__(256) void activation_backward_bf16x8_kernel(
 // and the same roundings element by element).
 __global__ __launch_bounds__(256) void hidden_grad_bf16x8_kernel(
     uint4* __restrict__ dh, const uint4* __restrict__ h,
-    const uint4* __restrict__ scale, bool relu, int64_t n8) {
+    const uint4* __restrict__ scale, bool relu, int64_t n8,
+    float const_scale) {
   const int64_t stride = (int64_t)gridDim.x * blockDim.x;
   for (int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n8;
        i += stride) {
@@ -1368,6 +1374,7 @@ __global__ __launch_bounds__(256) void hidden_grad_bf16x8_kernel(
     for (int j = 0; j < 8; ++j) {
       if (relu && !(hv[j] > 0.f)) d[j] = 0.f;
       else if (scale) d[j] = d[j] * sc[j];
+      else d[j] = d[j] * const_scale;
     }
     store_streaming(dh + i, pack16(d, bf16_t()));
   }
@@ -1425,16 +1432,19 @@ static int elementwise_blocks(int64_t n) {
 
 // dh = dh * scale, then the ReLU mask of h (hidden_grad_kernel's contract)
 static int launch_hidden_grad(void* dh, const void* h, const void* scale,
-                              bool relu, int64_t n, int dtype, hipStream_t st) {
+                              bool relu, int64_t n, int dtype, hipStream_t st,
+                              float const_scale = 1.0f) {
   if (x8_applies(n, dtype, dh, h, scale))
     hidden_grad_bf16x8_kernel<<<elementwise_blocks(n / 8), 256, 0, st>>>(
-        (uint4*)dh, (const uint4*)h, (const uint4*)scale, relu, n / 8);
+        (uint4*)dh, (const uint4*)h, (const uint4*)scale, relu, n / 8,
+        const_scale);
   else if (dtype == MESH_MOE_F32)
     hidden_grad_kernel<float><<<elementwise_blocks(n), 256, 0, st>>>(
-        (float*)dh, (const float*)h, (const float*)scale, relu, n);
+        (float*)dh, (const float*)h, (const float*)scale, relu, n, const_scale);
   else
     hidden_grad_kernel<bf16_t><<<elementwise_blocks(n), 256, 0, st>>>(
-        (bf16_t*)dh, (const bf16_t*)h, (const bf16_t*)scale, relu, n);
+        (bf16_t*)dh, (const bf16_t*)h, (const bf16_t*)scale, relu, n,
+        const_scale);
   MOE_CHECK_LAUNCH("hidden gradient (mask / scale)");
   return 0;
 }
@@ -2304,19 +2314,22 @@ extern "C" int mesh_moe_expert_ffn_backward(
   // not be read: where the stored activation is positive the element was kept
   // and its noise is 1 / keep_prob (as mesh_moe_hidden_product rounds it).
   const bool relu_act = activation == MESH_MOE_ACT_RELU;
-  const bool noise_by_mask = relu_act && dh_scale != nullptr &&
-                             dh_keep_prob > 0.f && dh_keep_prob <= 1.f &&
-                             dtype == MESH_MOE_BF16;
+  const bool noise_by_mask =
+      relu_act && dh_keep_prob > 0.f && dh_keep_prob < 1.f;
+  // 1 / keep_prob as mesh_moe_hidden_product has it
   const float mask_scale =
-      noise_by_mask ? round_bf16_host(1.f / round_bf16_host(dh_keep_prob)) : 1.f;
+      !noise_by_mask ? 1.f
+      : dtype == MESH_MOE_BF16
+          ? round_bf16_host(1.f / round_bf16_host(dh_keep_prob))
+          : 1.f / dh_keep_prob;
   bool masked = false;
   rc = grouped_gemm(dy, wo, dh, E, R, H, N, MESH_MOE_ACT_LINEAR, dtype, st,
                     relu_act && (!dh_scale || noise_by_mask) ? h : nullptr,
                     &masked, mask_scale);
   if (rc != 0) return rc;
-  if (!masked && (activation == MESH_MOE_ACT_RELU || dh_scale)) {
-    rc = launch_hidden_grad(dh, h, dh_scale, activation == MESH_MOE_ACT_RELU,
-                            (int64_t)E * R * H, dtype, st);
+  if (!masked && (relu_act || dh_scale)) {
+    rc = launch_hidden_grad(dh, h, noise_by_mask ? nullptr : dh_scale, relu_act,
+                            (int64_t)E * R * H, dtype, st, mask_scale);
     if (rc != 0) return rc;
   }
   // dexpert_in = dh . wi^T  (wi in its variable layout [E, M, H])
@@ -2435,8 +2448,7 @@ extern "C" int mesh_moe_compact_expert_ffn_backward(
   // (a ReLU expert's dropout noise follows from the stored activation: see
   // mesh_moe_expert_ffn_backward)
   const bool noise_by_mask = activation == MESH_MOE_ACT_RELU &&
-                             dh_scale != nullptr && dh_keep_prob > 0.f &&
-                             dh_keep_prob <= 1.f;
+                             dh_keep_prob > 0.f && dh_keep_prob < 1.f;
   const float mask_scale =
       noise_by_mask ? round_bf16_host(1.f / round_bf16_host(dh_keep_prob)) : 1.f;
   const bool mask_on_stores =

@@ -474,6 +474,10 @@ class MoEV1Operation(mtf.Operation):
       single_choice = (not by_slot and kwo_p is None and one_layer and
                        self._gating.router != "top_2")
 
+      # the gradient of ReLU experts takes the dropout's noise from the stored
+      # activation (positive = kept, 1 / keep_prob there): no noise tensor
+      keep_noise = save and (self._general_hidden or self._activation != "relu")
+
       def compact_ffn(want_hidden):
         """The expert feed-forward on compacted rows (the occupied slots at
         the front of every expert's rows), hidden dropout included; None where
@@ -485,7 +489,7 @@ class MoEV1Operation(mtf.Operation):
         return moe_hip.compact_expert_ffn(
             xg, r, wi_p, wo_p, self._activation, want_hidden=want_hidden,
             uniform=u, keep_prob=1.0 if keep_prob is None else keep_prob,
-            want_noise=want_hidden)
+            want_noise=want_hidden and keep_noise)
 
       if (save and single_choice and
           moe_hip.compact_training_applies(xg, r, wi_p.shape[1], n_,
@@ -495,7 +499,8 @@ class MoEV1Operation(mtf.Operation):
         # operation reads, so that it too multiplies only those
         compact = compact_ffn(True)
         if compact is not None:
-          y, row_offsets, h, noise = compact
+          y, row_offsets, h = compact[:3]
+          noise = compact[3] if len(compact) > 3 else None
           expert_in = moe_hip.dispatch(xg, r, row_offsets=row_offsets)
           expert_in = expert_in.reshape(e_, groups * c_, m_)
       if not save and single_choice:
@@ -542,7 +547,7 @@ class MoEV1Operation(mtf.Operation):
         if keep_prob is not None:
           u = torch.rand(h.shape, dtype=dt, device=h.device)
           noise = moe_hip.hidden_product(h, uniform=u, keep_prob=keep_prob,
-                                         want_noise=save)
+                                         want_noise=keep_noise)
         y = moe_hip.expert_linear(h, wo_p)
       y4 = y.reshape(e_, groups, c_, n_)
       out = (moe_hip.slot_combine(y4, r, s_) if by_slot

@@ -1325,9 +1325,24 @@ def test_dropout_noise_from_the_relu_mask(hip):
   a = hip.expert_ffn_backward(xe, h, dy, wi, wo, "relu", dh_scale=noise,
                               keep_prob=keep)
   b = hip.expert_ffn_backward(xe, h, dy, wi, wo, "relu", dh_scale=noise)
-  for x_, y_ in zip(a, b):
-    assert torch.equal(x_, y_)
+  # (the noise tensor itself is then not needed)
+  c_ = hip.expert_ffn_backward(xe, h, dy, wi, wo, "relu", keep_prob=keep)
+  for x_, y_, z_ in zip(a, b, c_):
+    assert torch.equal(x_, y_) and torch.equal(x_, z_)
   assert float(a[0].abs().sum()) > 0
+  # float32, and rows the matrix-core kernels do not take: the same through
+  # the element-wise pass
+  f = lambda t: t[:, :40].float().contiguous()
+  h32 = hip.expert_linear(f(xe), hip.pack_weights(wi.float(), torch.float32),
+                          "relu")
+  n32 = hip.hidden_product(h32, uniform=f(u.float().reshape(e, g * c, hdim)),
+                           keep_prob=keep, want_noise=True)
+  a32 = hip.expert_ffn_backward(f(xe), h32, f(dy), wi.float(), wo.float(),
+                                "relu", dh_scale=n32)
+  c32 = hip.expert_ffn_backward(f(xe), h32, f(dy), wi.float(), wo.float(),
+                                "relu", keep_prob=keep)
+  for x_, z_ in zip(a32, c32):
+    assert torch.equal(x_, z_)
   # compacted rows: a switch routing that fills about half of the slots
   s = 1024
   r = hip.switch_gating(mk(g, s, e), c)
