@@ -66,7 +66,8 @@ def hparams_dict(cfg):
       moe_capacity_factor_second_level=cfg.get("cf2", 1.0),
       moe_use_second_place_loss=False, moe_second_policy_train="all",
       moe_second_policy_eval="all", moe_second_threshold_train=0.2,
-      moe_second_threshold_eval=0.2, moe_dropout_rate=0.0,
+      moe_second_threshold_eval=0.2,
+      moe_dropout_rate=cfg.get("expert_dropout", 0.0),
       moe_use_experts_attention=False, moe_ntlb_top_k=4)
 
 
@@ -327,6 +328,10 @@ def main():
                   help="diagnostic: zero expert weights (and tokens): the same "
                        "kernels and traffic without operand toggling, to read "
                        "the power limit off the clock; not the benchmark")
+  ap.add_argument("--expert-dropout", type=float, default=0.0,
+                  help="moe_dropout_rate of the layer (the dropout of the "
+                       "experts' hidden tensor while training); not the "
+                       "benchmark's configuration")
   ap.add_argument("--no-cpu-baseline", action="store_true")
   args = ap.parse_args()
   if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
@@ -344,6 +349,9 @@ def main():
       sys.exit(2)
     cfg["gating"] = args.gating
     cfg["name"] += ", %s gating" % args.gating
+  if args.expert_dropout:
+    cfg["expert_dropout"] = args.expert_dropout
+    cfg["name"] += ", moe_dropout_rate %g" % args.expert_dropout
   device = torch.device("cuda:0")
   torch.cuda.set_device(device)
   if args.block and (cfg["layer"] != "v1" or args.gating != "top_2"):
@@ -431,7 +439,10 @@ def main():
         entry.update(algorithmic_bytes=model[name]["bytes"], GBps=gbs,
                      frac_hbm_peak=gbs / HBM_PEAK_GBS)
       per_stage[name] = entry
-    ffn_ms = stages["expert_ffn"][1] / args.steps
+    # (with --expert-dropout and two choices per token the two expert GEMMs are
+    # calls of their own, with the dropout between them)
+    ffn_key = "expert_ffn" if "expert_ffn" in stages else "expert_linear"
+    ffn_ms = stages[ffn_key][1] / args.steps
     # the expert FFN is two launches of the same grouped-GEMM kernel with the
     # same flop count; `achieved` prices the average launch
     flops_per_launch = model["expert_ffn"]["flops"] / 2
