@@ -280,15 +280,7 @@ def cpu_baseline(cfg):
   wi = np.broadcast_to(wi1, (e, m, h))
   wo = np.broadcast_to(wo1, (e, h, m))
   hp = O.HParams(**hparams_dict(cfg))
-  threads = os.cpu_count()
-  try:
-    from threadpoolctl import threadpool_info
-    blas = [p["num_threads"] for p in threadpool_info()
-            if p.get("user_api") == "blas"]
-    if blas:
-      threads = max(blas)
-  except Exception:  # pylint: disable=broad-except
-    pass
+  threads = _blas_threads()
   t0 = time.perf_counter()
   O.moe_layer_v1(x, wg, wi, wo, hp, True, act, dense=True,
                  weights_are_cast=True)
@@ -299,6 +291,135 @@ def cpu_baseline(cfg):
                      "formulation, one expert's weights shared by all "
                      "experts), %.1f s"
                      % (n_groups, total_groups, n_groups * s, e, dt))
+
+
+def cpu_baseline_full_cfg1():
+  """The designated CPU configuration (config 1: fp32, 2048 tokens, d_model
+  512, d_ff 2048, 8 experts) run WHOLE through the CPU restatement of the
+  reference lowering: every group, every expert with weights of its own."""
+  import numpy as np
+  from oracle import moe_oracle as O
+  cfg = CONFIGS[1]
+  rng = np.random.default_rng(1)
+  m, h, e, s = cfg["M"], cfg["H"], cfg["E"], cfg["group"]
+  tokens = cfg["batch"] * cfg["length"]
+  x = rng.standard_normal((tokens // s, s, m), dtype=np.float32)
+  wg = rng.standard_normal((m, e), dtype=np.float32) / np.float32(np.sqrt(m))
+  wi = rng.standard_normal((e, m, h), dtype=np.float32) / np.float32(np.sqrt(m))
+  wo = rng.standard_normal((e, h, m), dtype=np.float32) / np.float32(np.sqrt(h))
+  hp = O.HParams(**hparams_dict(cfg))
+  best = None
+  for _ in range(3):        # first pass pays the BLAS thread pool's start
+    t0 = time.perf_counter()
+    O.moe_layer_v1(x, wg, wi, wo, hp, True, "float32", dense=True,
+                   weights_are_cast=True)
+    dt = time.perf_counter() - t0
+    best = dt if best is None else min(best, dt)
+  return dict(value=tokens / best, unit="tokens/s", cores=_blas_threads(),
+              kind="port", ms_per_step=best * 1e3,
+              sample="the whole of %s (all %d tokens, %d groups, %d experts, "
+                     "dense formulation), best of 3 passes"
+                     % (cfg["name"], tokens, tokens // s, e))
+
+
+def _blas_threads():
+  threads = os.cpu_count()
+  try:
+    from threadpoolctl import threadpool_info
+    blas = [p["num_threads"] for p in threadpool_info()
+            if p.get("user_api") == "blas"]
+    if blas:
+      threads = max(blas)
+  except Exception:  # pylint: disable=broad-except
+    pass
+  return int(threads)
+
+
+class PowerSampler:
+  """Samples the socket power, the shader clock and the violation counters of
+  GPU 0 from a host thread (amdsmi) while a timed loop runs: the readings that
+  say whether the chip sits at its power cap during the grouped GEMM."""
+
+  def __init__(self, period_s=0.02):
+    import threading
+    import amdsmi
+    self._amdsmi = amdsmi
+    amdsmi.amdsmi_init()
+    self._handle = amdsmi.amdsmi_get_processor_handles()[0]
+    self._period = period_s
+    self._stop = threading.Event()
+    self._thread = threading.Thread(target=self._run, daemon=True)
+    self.samples = []
+    self.errors = []
+
+  def _read(self):
+    a, h = self._amdsmi, self._handle
+    out = {}
+    try:
+      pw = a.amdsmi_get_power_info(h)
+      for k in ("current_socket_power", "average_socket_power", "power_limit"):
+        if k in pw and pw[k] != "N/A":
+          out[k] = float(pw[k])
+    except Exception as err:  # pylint: disable=broad-except
+      self.errors.append("power_info: %r" % (err,))
+    try:
+      ck = a.amdsmi_get_clock_info(h, a.AmdSmiClkType.GFX)
+      for k in ("clk", "cur_clk", "max_clk"):
+        if k in ck and ck[k] != "N/A":
+          out["gfx_" + k] = float(ck[k])
+    except Exception as err:  # pylint: disable=broad-except
+      self.errors.append("clock_info: %r" % (err,))
+    return out
+
+  def _run(self):
+    while not self._stop.is_set():
+      t = time.perf_counter()
+      s = self._read()
+      s["t"] = t
+      self.samples.append(s)
+      self._stop.wait(self._period)
+
+  def static_info(self):
+    """Power cap and violation (throttle) status, read once."""
+    a, h = self._amdsmi, self._handle
+    info = {}
+    try:
+      cap = a.amdsmi_get_power_cap_info(h)
+      info["power_cap"] = {k: cap[k] for k in cap}
+    except Exception as err:  # pylint: disable=broad-except
+      info["power_cap_error"] = repr(err)
+    try:
+      v = a.amdsmi_get_violation_status(h)
+      info["violation_status"] = {
+          k: v[k] for k in v
+          if isinstance(v[k], (int, float, str, bool)) and v[k] != "N/A"}
+    except Exception as err:  # pylint: disable=broad-except
+      info["violation_error"] = repr(err)
+    return info
+
+  def __enter__(self):
+    self._thread.start()
+    return self
+
+  def __exit__(self, *exc):
+    self._stop.set()
+    self._thread.join()
+
+  def summary(self, t0, t1):
+    """Statistics of the samples taken inside [t0 + 20 %, t1] (the averaged
+    power reading needs a moment to reach the loop's level)."""
+    lo = t0 + 0.2 * (t1 - t0)
+    inside = [s for s in self.samples if lo <= s["t"] <= t1]
+    out = {"samples": len(inside), "window_s": t1 - lo}
+    keys = sorted({k for s in inside for k in s if k != "t"})
+    for k in keys:
+      vals = sorted(s[k] for s in inside if k in s)
+      if vals:
+        out[k] = {"min": vals[0], "median": vals[len(vals) // 2],
+                  "max": vals[-1], "mean": sum(vals) / len(vals)}
+    if self.errors:
+      out["errors"] = sorted(set(self.errors))[:4]
+    return out
 
 
 def main():
@@ -333,6 +454,11 @@ def main():
                        "experts' hidden tensor while training); not the "
                        "benchmark's configuration")
   ap.add_argument("--no-cpu-baseline", action="store_true")
+  ap.add_argument("--power", action="store_true",
+                  help="diagnostic: sample socket power and shader clock "
+                       "(amdsmi, host thread) during the timed loop and add "
+                       "them to the JSON line as `power`; use with enough "
+                       "--steps for a few seconds of work")
   args = ap.parse_args()
   if args.gpus != 1 or int(os.environ.get("WORLD_SIZE", "1")) != 1:
     print("bench.py measures ONE GPU: this layer runs on a single-device mesh "
@@ -365,12 +491,18 @@ def main():
   for _ in range(args.warmup):
     lowering.run()
   torch.cuda.synchronize()
+  sampler = PowerSampler() if args.power else None
+  power_before = sampler.static_info() if sampler else None
   with moe_hip.StageTimer() as timer:
+    if sampler:
+      sampler.__enter__()
     t0 = time.perf_counter()
     for _ in range(args.steps):
       lowering.run()
     torch.cuda.synchronize()
     t1 = time.perf_counter()
+    if sampler:
+      sampler.__exit__()
     stages = timer.totals()
     routings = timer.routing
   ms_per_step = (t1 - t0) * 1e3 / args.steps
@@ -495,9 +627,13 @@ def main():
                             "launches_per_step": v[0] / args.steps}
                         for k, v in stages.items()}
   # (the CPU restatement timed below is the top-2 layer's)
-  result["cpu_baseline"] = (None if (args.no_cpu_baseline or args.backward
-                                     or args.gating != "top_2")
-                            else cpu_baseline(cfg))
+  if sampler:
+    result["power"] = dict(sampler.summary(t0, t1), before=power_before,
+                           after=sampler.static_info())
+  no_cpu = args.no_cpu_baseline or args.backward or args.gating != "top_2"
+  result["cpu_baseline"] = None if no_cpu else cpu_baseline(cfg)
+  # the designated CPU configuration in full, beside the sample above
+  result["cpu_baseline_full"] = None if no_cpu else cpu_baseline_full_cfg1()
   print(json.dumps(result))
 
 

@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 32
+#define MESH_MOE_ABI_VERSION 33
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -389,9 +389,18 @@ int mesh_moe_combine_compact(const void* y, const int32_t* idx,
  * idx[g,s,0] of a token nobody took is its first candidate.  The loss is
  * E^2 * mean(density_1_proxy * density_1) over [G,k,E] (and over the group dim
  * when `importance` is given, moe.py:845-860).  top_k <= 8.
+ *   softmax_dtype: the dtype the reference runs this router's projection
+ *   result and softmax in, i.e. the activation dtype -- _ntlb_gating alone
+ *   has no to_float in front of its projection and casts only the
+ *   probabilities to float32 (moe.py:825-836).  MESH_MOE_BF16: the logits
+ *   (float32-accumulated) are rounded to bfloat16 and every op of
+ *   mtf.softmax (ops.py:5493-5541: add, exp, reduce_sum, log, add, add, exp)
+ *   rounds its result to bfloat16; the sum accumulates in float32 in index
+ *   order and rounds once.  MESH_MOE_F32: float32 throughout.
  */
 size_t mesh_moe_ntlb_workspace_bytes(int G, int S, int E, int top_k);
-int mesh_moe_ntlb_gating(const float* logits, const void* importance,
+int mesh_moe_ntlb_gating(const float* logits, int softmax_dtype,
+                         const void* importance,
                          int importance_dtype, int G, int S, int E, int C,
                          int top_k, int num_microbatches, int32_t* idx,
                          int32_t* pos, float* gate, uint8_t* kept,
@@ -540,9 +549,12 @@ size_t mesh_moe_expert_ffn_backward_workspace_bytes(int E, int R, int M, int H,
  *   wi [E,M,H], wo [E,H,N]: the variables' own layout (NOT the packed one)
  *   dh_scale [E,R,H] dtype or NULL: the dropout noise mesh_moe_hidden_product
  *   wrote (transformer/moe.py:477-479)
- *   dh_keep_prob: the keep probability that noise was made with, or 0 if the
- *   caller does not know it (or there was none).  Known, ReLU experts do not
- *   read dh_scale, which may then be NULL: where h > 0 the element was kept
+ *   dh_keep_prob in [0, 1] (anything else is refused): the keep probability
+ *   that noise was made with, or 0 if the caller does not know it or there
+ *   was no dropout.  dh_scale NULL together with dh_keep_prob 0 (or 1) means
+ *   that no dropout was applied in the forward pass.  With a value in (0, 1)
+ *   ReLU experts do not read dh_scale, which may then be NULL (given both,
+ *   the keep probability is what is used): where h > 0 the element was kept
  *   and its noise is 1 / keep_prob
  *   dexpert_in [E,R,M]; dwi [E,M,H]; dwo [E,H,N]; everything of `dtype`
  * Four grouped GEMMs on the forward kernels; the weight gradients read both
@@ -608,8 +620,12 @@ size_t mesh_moe_gating_backward_workspace_bytes(int G, int E);
 /*
  * Backward of the gating (transformer/moe.py:1391-1496 for router 0 = top-2,
  * :1207-1306 for router 1 = switch / switch_max, :831-934 for router 2 = ntlb
- * with its top_k; top_k is ignored otherwise): d(logits) from the
+ * with its top_k and softmax_dtype as in mesh_moe_ntlb_gating; both are
+ * ignored otherwise): d(logits) from the
  * gradients of the two combine weights and of the layer's returned loss.
+ * With softmax_dtype bfloat16 (ntlb) the probabilities and the candidates are
+ * recomputed with the forward's roundings and the float32 derivative of the
+ * softmax is evaluated at those probabilities.
  *   logits [G,S,E] float32 (the forward values), importance and
  *   importance_from_slot_gate as in the forward
  *   idx, kept [G,S,2] from the forward; dgate [G,S,2] float32 from
@@ -626,7 +642,7 @@ int mesh_moe_gating_backward(const float* logits, const void* importance,
                              const uint8_t* kept, const float* dgate,
                              const float* d_loss, double loss_scale, int G,
                              int S, int E, int router, int top_k,
-                             int use_second_place_loss,
+                             int softmax_dtype, int use_second_place_loss,
                              int use_z_loss, double z_loss_coef,
                              int num_microbatches,
                              float* dlogits, void* workspace,

@@ -560,7 +560,30 @@ struct GateBackwardParams {
   int use_z_loss;
   float z_loss_coef;
   float loss_scale;     // moe_loss_coef as the activation dtype holds it
+  int softmax_bf16;     // ntlb with bfloat16 activations: the forward rounded
+                        // the logits and every softmax op to bfloat16
 };
+
+// The forward's softmax of one row: lse_out = log-sum-exp as the forward
+// formed it; the probability of entry e is then gb_prob(row[e], neglse, bf).
+// bf: every op's result rounded to bfloat16 (ntlb_softmax_row of the forward
+// kernel), else plain float32.
+__device__ __forceinline__ float gb_round(float v, bool bf) {
+  return bf ? round_to<bf16_t>(v) : v;
+}
+__device__ __forceinline__ float gb_logsumexp(const float* row, int E, bool bf) {
+  float m = gb_round(row[0], bf);
+  for (int e = 1; e < E; ++e) m = fmaxf(m, gb_round(row[e], bf));
+  const float negm = -m;
+  float s = 0.f;
+  for (int e = 0; e < E; ++e)
+    s += gb_round(expf(gb_round(gb_round(row[e], bf) + negm, bf)), bf);
+  s = gb_round(s, bf);
+  return gb_round(gb_round(logf(s), bf) + m, bf);
+}
+__device__ __forceinline__ float gb_prob(float logit, float neglse, bool bf) {
+  return gb_round(expf(gb_round(gb_round(logit, bf) + neglse, bf)), bf);
+}
 
 constexpr int GB_MAX_K = 8;
 
@@ -593,12 +616,8 @@ __global__ __launch_bounds__(256) void gate_count_kernel(
       // (moe.py:839-847); the probabilities and the repeated first-arg-max are
       // those of the forward kernel, so the candidates are the same
       const float* row = logits + t * p.E;
-      float m = row[0];
-      for (int e = 1; e < p.E; ++e) m = fmaxf(m, row[e]);
-      const float negm = -m;
-      float sum = 0.f;
-      for (int e = 0; e < p.E; ++e) sum += expf(row[e] + negm);
-      const float neglse = -(logf(sum) + m);
+      const bool bf = p.softmax_bf16 != 0;
+      const float neglse = -gb_logsumexp(row, p.E, bf);
       int ids[GB_MAX_K];
 #pragma unroll
       for (int i = 0; i < GB_MAX_K; ++i) {
@@ -609,7 +628,7 @@ __global__ __launch_bounds__(256) void gate_count_kernel(
             bool taken = false;
 #pragma unroll
             for (int j = 0; j < GB_MAX_K; ++j) taken |= (j < i && ids[j] == e);
-            const float v = taken ? -2.f : expf(row[e] + neglse);
+            const float v = taken ? -2.f : gb_prob(row[e], neglse, bf);
             if (v > best) { best = v; bi = e; }
           }
           ids[i] = bi;
@@ -664,12 +683,8 @@ __global__ __launch_bounds__(256) void gating_backward_kernel(
   const float* row = staged ? gb_tile + threadIdx.x * (E + 1) : logits + t * E;
   float* out = staged ? gb_tile + threadIdx.x * (E + 1) : dlogits + t * E;
   // softmax exactly as the forward kernel computes it
-  float m = row[0];
-  for (int e = 1; e < E; ++e) m = fmaxf(m, row[e]);
-  const float negm = -m;
-  float s = 0.f;
-  for (int e = 0; e < E; ++e) s += expf(row[e] + negm);
-  const float lse = logf(s) + m;
+  const bool bf = p.softmax_bf16 != 0;
+  const float lse = gb_logsumexp(row, E, bf);
   const float neglse = -lse;
   float m1 = 1.0f;
   if (importance != nullptr) {
@@ -686,7 +701,8 @@ __global__ __launch_bounds__(256) void gating_backward_kernel(
   float add1 = 0.f, add2 = 0.f;  // d(p[i1]), d(p[i2]) from the gates
   float coef;                    // d(p[e]) = coef * counts[g,e] from the loss
   if (p.router == 0) {
-    const float p1 = expf(row[i1] + neglse), p2 = expf(row[i2] + neglse);
+    const float p1 = gb_prob(row[i1], neglse, bf);
+    const float p2 = gb_prob(row[i2], neglse, bf);
     const float g1 = p1 * m1;
     const float same = (i2 == i1) ? m1 : 0.0f;
     const float g2 = p2 * (1.0f - same);
@@ -723,7 +739,8 @@ __global__ __launch_bounds__(256) void gating_backward_kernel(
             inv_s * inv_s;
     float q = 0.f, a = 0.f;
     for (int e = 0; e < E; ++e) {
-      const float qe = expf(row[e] + neglse) * (e == i1 ? 1.0f - m1 : 1.0f);
+      const float qe =
+          gb_prob(row[e], neglse, bf) * (e == i1 ? 1.0f - m1 : 1.0f);
       q += qe;
       a += coef2 * (float)cg2[e] * qe;
     }
@@ -740,7 +757,7 @@ __global__ __launch_bounds__(256) void gating_backward_kernel(
   };
   // inner = sum_e p[e] * dp[e]
   float inner = 0.f;
-  for (int e = 0; e < E; ++e) inner += expf(row[e] + neglse) * dprob(e);
+  for (int e = 0; e < E; ++e) inner += gb_prob(row[e], neglse, bf) * dprob(e);
   float zfac = 0.f;
   if (p.use_z_loss) {  // d/dx of z_coef * sum(lse^2 * m1) / (n * microbatches)
     float n = 0.f;
@@ -750,7 +767,7 @@ __global__ __launch_bounds__(256) void gating_backward_kernel(
            (n * mbz);
   }
   for (int e = 0; e < E; ++e) {
-    const float pe = expf(row[e] + neglse);
+    const float pe = gb_prob(row[e], neglse, bf);
     out[e] = pe * (dprob(e) - inner) + zfac * pe;
   }
   }  // t < T_tokens
@@ -1342,7 +1359,7 @@ extern "C" int mesh_moe_gating_backward(
     const float* logits, const void* importance, int importance_dtype,
     int importance_from_slot_gate, const int32_t* idx, const uint8_t* kept,
     const float* dgate, const float* d_loss, double loss_scale, int G, int S,
-    int E, int router, int top_k, int use_second_place_loss,
+    int E, int router, int top_k, int softmax_dtype, int use_second_place_loss,
     int use_z_loss, double z_loss_coef, int num_microbatches, float* dlogits,
     void* workspace, size_t workspace_bytes, void* stream) {
   MOE_REQUIRE(logits && idx && kept && dgate && d_loss && dlogits && workspace,
@@ -1357,6 +1374,8 @@ extern "C" int mesh_moe_gating_backward(
               "(at most %d)", top_k, E, GB_MAX_K);
   MOE_REQUIRE(!importance || valid_dtype(importance_dtype), MESH_MOE_E_ARG,
               "gating_backward: bad importance dtype %d", importance_dtype);
+  MOE_REQUIRE(valid_dtype(softmax_dtype), MESH_MOE_E_ARG,
+              "gating_backward: bad softmax dtype %d", softmax_dtype);
   MOE_REQUIRE(workspace_bytes >= mesh_moe_gating_backward_workspace_bytes(G, E),
               MESH_MOE_E_ARG, "gating_backward: workspace too small");
   GateBackwardParams p;
@@ -1370,6 +1389,8 @@ extern "C" int mesh_moe_gating_backward(
   p.use_z_loss = (use_z_loss && router == 1) ? 1 : 0;
   p.z_loss_coef = (float)z_loss_coef;
   p.loss_scale = (float)loss_scale;
+  // only _ntlb_gating runs its softmax in the activation dtype
+  p.softmax_bf16 = (router == 2 && softmax_dtype == MESH_MOE_BF16) ? 1 : 0;
   uintptr_t wsp = ((uintptr_t)workspace + 255) & ~(uintptr_t)255;
   int32_t* counts = (int32_t*)wsp;
   float* n_one = (float*)(counts + 2 * (size_t)G * E);

@@ -2298,6 +2298,10 @@ extern "C" int mesh_moe_expert_ffn_backward(
               "expert_ffn_backward: only relu and linear experts (got %d): the "
               "other activations need the pre-activation, which is not kept",
               activation);
+  MOE_REQUIRE(dh_keep_prob >= 0.f && dh_keep_prob <= 1.f, MESH_MOE_E_ARG,
+              "expert_ffn_backward: dh_keep_prob=%g outside [0, 1] (0: no "
+              "dropout, or a noise tensor alone describes it)",
+              (double)dh_keep_prob);
   MOE_REQUIRE(workspace_bytes >= mesh_moe_expert_ffn_backward_workspace_bytes(
                                      E, R, M, H, N, dtype),
               MESH_MOE_E_ARG, "expert_ffn_backward: workspace too small");
@@ -2409,6 +2413,9 @@ extern "C" int mesh_moe_compact_expert_ffn_backward(
                   activation == MESH_MOE_ACT_LINEAR, MESH_MOE_E_UNSUPPORTED,
               "compact_expert_ffn_backward: only relu and linear experts (got "
               "%d)", activation);
+  MOE_REQUIRE(dh_keep_prob >= 0.f && dh_keep_prob <= 1.f, MESH_MOE_E_ARG,
+              "compact_expert_ffn_backward: dh_keep_prob=%g outside [0, 1]",
+              (double)dh_keep_prob);
   MOE_REQUIRE(dtype == MESH_MOE_BF16 &&
                   compact_backward_applies(G, E, C, M, H, N) &&
                   (((uintptr_t)expert_in | (uintptr_t)h | (uintptr_t)dy |

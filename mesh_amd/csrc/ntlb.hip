@@ -1,8 +1,12 @@
 // "No token left behind" gating for gfx950.
 //
 // Follows _ntlb_gating, mesh_tensorflow/transformer/moe.py:804-940, after the
-// router projection: float32 softmax in the operation order of mtf.softmax
-// (ops.py:5493-5541), the top_k experts of every token (mtf.top_k,
+// router projection: softmax in the operation order of mtf.softmax
+// (ops.py:5493-5541) and in the dtype the reference runs it in -- this router
+// alone keeps the projection's result and the softmax in the activation dtype
+// and casts the probabilities to float32 afterwards (moe.py:825-836), so with
+// bfloat16 activations every op of the chain rounds to bfloat16 --, the top_k
+// experts of every token (mtf.top_k,
 // ops.py:4964-5015: repeated first-arg-max), then top_k passes in which the
 // still unrouted tokens are offered, in token order, to their next expert
 // (moe.py:903-934).  The dense [G,S,k,E] masks and the cumsum over the group
@@ -31,7 +35,27 @@ struct NtlbParams {
 // probabilities (density_1_proxy, moe.py:848) and the number of tokens with
 // importance 1.
 // ---------------------------------------------------------------------------
-template <typename IT>
+// The probabilities of one row in place, ST = dtype of the reference's softmax
+// ops.  ST = bf16_t: the logits are first rounded (the projection's bfloat16
+// result), then every op rounds once (negative and max are exact; the sum
+// accumulates in float32 in index order and rounds once, as TensorFlow's
+// bfloat16 sum reducer does).  ST = float: round_to is the identity.
+template <typename ST>
+__device__ __forceinline__ void ntlb_softmax_row(float* row, int E) {
+  for (int e = 0; e < E; ++e) row[e] = round_to<ST>(row[e]);
+  float m = row[0];
+  for (int e = 1; e < E; ++e) m = fmaxf(m, row[e]);       // reduce_max
+  const float negm = -m;
+  float s = 0.f;                                          // exp, reduce_sum
+  for (int e = 0; e < E; ++e)
+    s += round_to<ST>(expf(round_to<ST>(row[e] + negm)));
+  s = round_to<ST>(s);
+  const float neglse = -round_to<ST>(round_to<ST>(logf(s)) + m);  // log + max
+  for (int e = 0; e < E; ++e)
+    row[e] = round_to<ST>(expf(round_to<ST>(row[e] + neglse)));
+}
+
+template <typename IT, typename ST>
 __global__ __launch_bounds__(256) void ntlb_select_kernel(
     NtlbParams p, const float* __restrict__ logits,
     const IT* __restrict__ importance, int16_t* __restrict__ cand_idx,
@@ -55,13 +79,7 @@ __global__ __launch_bounds__(256) void ntlb_select_kernel(
   if (tid < ntok) {
     float* row = tile + tid * ld;
     const int64_t t = (int64_t)g * S + t0 + tid;
-    float m = row[0];
-    for (int e = 1; e < E; ++e) m = fmaxf(m, row[e]);       // reduce_max
-    const float negm = -m;
-    float s = 0.f;
-    for (int e = 0; e < E; ++e) s += expf(row[e] + negm);   // exp, reduce_sum
-    const float neglse = -(logf(s) + m);                    // log + max
-    for (int e = 0; e < E; ++e) row[e] = expf(row[e] + neglse);
+    ntlb_softmax_row<ST>(row, E);
     bool one = true;
     if (importance != nullptr) one = (load_f32<IT>(importance + t) == 1.0f);
     float vals[NTLB_MAX_K];
@@ -316,7 +334,8 @@ extern "C" size_t mesh_moe_ntlb_workspace_bytes(int G, int S, int E,
 }
 
 extern "C" int mesh_moe_ntlb_gating(
-    const float* logits, const void* importance, int importance_dtype, int G,
+    const float* logits, int softmax_dtype, const void* importance,
+    int importance_dtype, int G,
     int S, int E, int C, int top_k, int num_microbatches, int32_t* idx,
     int32_t* pos, float* gate, uint8_t* kept, int32_t* fill, float* loss,
     void* workspace, size_t workspace_bytes, void* stream) {
@@ -334,6 +353,8 @@ extern "C" int mesh_moe_ntlb_gating(
               "ntlb_gating: S=%d > 16384 or G=%d > 65535", S, G);
   MOE_REQUIRE(!importance || valid_dtype(importance_dtype), MESH_MOE_E_ARG,
               "ntlb_gating: bad importance dtype %d", importance_dtype);
+  MOE_REQUIRE(valid_dtype(softmax_dtype), MESH_MOE_E_ARG,
+              "ntlb_gating: bad softmax dtype %d", softmax_dtype);
   MOE_REQUIRE(workspace_bytes >= mesh_moe_ntlb_workspace_bytes(G, S, E, top_k),
               MESH_MOE_E_ARG, "ntlb_gating: workspace too small");
   int el = 2;
@@ -362,17 +383,22 @@ extern "C" int mesh_moe_ntlb_gating(
   hipStream_t st = (hipStream_t)stream;
   const size_t smem1 = sizeof(float) * ((size_t)p.tt * (E + 1) + p.tt);
   dim3 grid((unsigned)p.nblk, (unsigned)G);
-  if (importance && importance_dtype == MESH_MOE_BF16) {
-    auto k = ntlb_select_kernel<bf16_t>;
-    MOE_ALLOW_LDS(k, smem1);
-    k<<<grid, 256, smem1, st>>>(p, logits, (const bf16_t*)importance, cand_idx,
-                                cand_gate, competes, part, part_one);
+#define MOE_NTLB_SELECT(IT, ST)                                                \
+  do {                                                                         \
+    auto k = ntlb_select_kernel<IT, ST>;                                       \
+    MOE_ALLOW_LDS(k, smem1);                                                   \
+    k<<<grid, 256, smem1, st>>>(p, logits, (const IT*)importance, cand_idx,    \
+                                cand_gate, competes, part, part_one);          \
+  } while (0)
+  const bool imp_bf16 = importance && importance_dtype == MESH_MOE_BF16;
+  if (softmax_dtype == MESH_MOE_BF16) {
+    if (imp_bf16) MOE_NTLB_SELECT(bf16_t, bf16_t);
+    else MOE_NTLB_SELECT(float, bf16_t);
   } else {
-    auto k = ntlb_select_kernel<float>;
-    MOE_ALLOW_LDS(k, smem1);
-    k<<<grid, 256, smem1, st>>>(p, logits, (const float*)importance, cand_idx,
-                                cand_gate, competes, part, part_one);
+    if (imp_bf16) MOE_NTLB_SELECT(bf16_t, float);
+    else MOE_NTLB_SELECT(float, float);
   }
+#undef MOE_NTLB_SELECT
   MOE_CHECK_LAUNCH("ntlb_gating (select)");
   MOE_ALLOW_LDS(ntlb_assign_kernel, smem2);
   ntlb_assign_kernel<<<G, NTLB_THREADS, smem2, st>>>(

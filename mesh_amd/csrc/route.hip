@@ -294,6 +294,11 @@ struct GateParams {
 constexpr int ROUTER_TOP2 = 0;    // _top_2_gating, moe.py:1312-1513
 constexpr int ROUTER_SWITCH = 1;  // _switch_gating, moe.py:1176-1309
 constexpr int GSUM = 4;  // floats per group: loss term 1, term 2, #(imp==1), z
+// Largest group every gating entry accepts (the reference's moe_group_size
+// defaults to 1024, moe.py:139).  The capacity kernel keeps a group's expert
+// ids in LDS (6 bytes per token) and the one-launch tail keeps slot prefixes
+// in 16 bits: both rely on it.
+constexpr int GATE_MAX_GROUP = 16384;
 
 // bit 0 of the step-1 `kept` byte: the token competes for a slot (mask_k after
 // importance and policy); bit 1 (second choice only): mask_2 before the policy,
@@ -871,6 +876,10 @@ __device__ __forceinline__ void gate_group_tail(
   const int tid = threadIdx.x;
   const bool sw = p.router == ROUTER_SWITCH;
   const bool loss2 = p.use_second_place_loss != 0 || sw;
+  // First slots per block and expert.  16 bits suffice: a prefix is at most
+  // the number of tokens of the earlier blocks, below S <= GATE_MAX_GROUP
+  // (every gating entry refuses larger groups).
+  static_assert(GATE_MAX_GROUP <= 65535, "the block prefixes are 16 bits wide");
   uint16_t* pre1 = reinterpret_cast<uint16_t*>(smem);          // [nblk][E]
   uint16_t* pre2 = pre1 + (size_t)nblk * E;                    // [nblk][E]
   int32_t* tot = reinterpret_cast<int32_t*>(
@@ -1584,8 +1593,8 @@ static int check_gating_args(int G, int S, int E, int C, int policy,
               "top2_gating: bad sizes G=%d S=%d C=%d", G, S, C);
   MOE_REQUIRE(E >= 2 && E <= 512, MESH_MOE_E_UNSUPPORTED,
               "top2_gating: E=%d outside [2, 512]", E);
-  MOE_REQUIRE(S <= 16384, MESH_MOE_E_UNSUPPORTED,
-              "top2_gating: group size S=%d > 16384", S);
+  MOE_REQUIRE(S <= GATE_MAX_GROUP, MESH_MOE_E_UNSUPPORTED,
+              "top2_gating: group size S=%d > %d", S, GATE_MAX_GROUP);
   MOE_REQUIRE(G <= 65535, MESH_MOE_E_UNSUPPORTED, "top2_gating: G=%d > 65535",
               G);
   MOE_REQUIRE(policy >= MESH_MOE_SECOND_ALL && policy <= MESH_MOE_SECOND_RANDOM,
@@ -1730,6 +1739,9 @@ static int check_fused_router_args(const char* who, const void* x,
   MOE_REQUIRE(batch >= 1 && (int64_t)batch * tokens == (int64_t)G * S,
               MESH_MOE_E_ARG, "%s: batch*tokens=%lld != G*S=%lld", who,
               (long long)batch * tokens, (long long)G * S);
+  // (the one-launch tail keeps per-block slot prefixes in 16 bits)
+  MOE_REQUIRE(S <= GATE_MAX_GROUP, MESH_MOE_E_UNSUPPORTED,
+              "%s: group size S=%d > %d", who, S, GATE_MAX_GROUP);
   MOE_REQUIRE(dtype == MESH_MOE_BF16 && M % 64 == 0 && E % 4 == 0 && E <= 128 &&
                   S % 128 == 0 && tokens % S == 0 &&
                   (int64_t)128 * M < (1LL << 31) &&

@@ -130,11 +130,6 @@ class DenseOperation(mtf.Operation):
   def __init__(self, x, kernel, new_dims, activation, name=None):
     super(DenseOperation, self).__init__([x, kernel], name=name or "dense")
     self._activation = activation
-    # Set by a layer whose hidden tensor x = relu(dense(...)) feeds nothing but
-    # this operation: the gradient of x then leaves this operation's backward
-    # already multiplied by (x > 0) -- the ReLU's backward done on the stores
-    # of the GEMM -- and the producer's backward skips its own pass over it.
-    self.masks_input_gradient = False
     shape = mtf.Shape(x.shape.dims[:-1] + list(new_dims))
     self._outputs = [mtf.Tensor(self, shape, x.dtype)]
 
@@ -166,7 +161,22 @@ class DenseGradOperation(mtf.Operation):
     super(DenseGradOperation, self).__init__(
         [dy, x, kernel, forward.outputs[0]], name=name or "dense_grad")
     self._relu = forward._activation == "relu"   # pylint: disable=protected-access
-    self._masks_dx = bool(forward.masks_input_gradient)
+    # When x = relu(dense(...)) feeds nothing but `forward` and nobody asked
+    # for d/dx itself, the only reader of dx is the producer's backward, whose
+    # first step is the ReLU mask: dx then leaves this operation already
+    # multiplied by (x > 0) -- the mask applied on the stores of the GEMM, so
+    # dx is d/d(pre-activation) -- and the producer's backward skips its own
+    # pass over it (_dy_is_masked below).  Decided here, at gradient time,
+    # when every consumer of x is known.
+    producer_x = x.operation
+    consumers = [op for op in x.graph.operations
+                 if x in op.inputs and not isinstance(op, DenseGradOperation)]
+    self._masks_dx = (
+        isinstance(producer_x, DenseOperation)
+        and producer_x._activation == "relu"      # pylint: disable=protected-access
+        and x is producer_x.outputs[0]
+        and consumers == [forward]
+        and not mtf.gradient_is_returned(x))
     # dy already carries this layer's ReLU mask when it is the input gradient
     # of the one operation that consumes the output and that operation masks
     producer = dy.operation

@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 32
+ABI_VERSION = 33
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -64,7 +64,8 @@ _SIGNATURES = {
     "mesh_moe_ntlb_workspace_bytes": (ctypes.c_size_t, [
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int]),
     "mesh_moe_ntlb_gating": (ctypes.c_int, [
-        _vp, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        _vp, ctypes.c_int, _vp, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, _vp, _vp,
         _vp, _vp, ctypes.c_size_t, _vp]),
     "mesh_moe_dispatch": (ctypes.c_int, [
@@ -178,6 +179,7 @@ _SIGNATURES = {
         _vp, _vp, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, _vp,
         ctypes.c_double,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_double, ctypes.c_int, _vp, _vp,
         ctypes.c_size_t, _vp]),
     "mesh_moe_router_backward_weights_workspace_bytes": (ctypes.c_size_t, [
@@ -570,10 +572,13 @@ def switch_gating(logits, capacity, importance=None, z_loss=None,
 
 
 def ntlb_gating(logits, capacity, top_k, importance=None,
-                num_microbatches=None):
+                num_microbatches=None, softmax_dtype=torch.float32):
   """logits float32 [G, S, E] -> Routing for "no token left behind" gating
   (_ntlb_gating, transformer/moe.py:804-940): top_k candidates per token, one
-  pass per candidate rank, each token routed at most once."""
+  pass per candidate rank, each token routed at most once.  softmax_dtype:
+  the activation dtype -- this router runs its projection's result and its
+  softmax in it (moe.py:825-836); with torch.bfloat16 the logits are rounded
+  and every softmax op rounds to bfloat16."""
   lib = load_library()
   g, s, e = logits.shape
   lp = _dev(logits, "logits", torch.float32)
@@ -588,7 +593,8 @@ def ntlb_gating(logits, capacity, top_k, importance=None,
                    device=logits.device)
   with _stage("ntlb_gating"):
     _check(lib.mesh_moe_ntlb_gating(
-        lp, ip, icode, g, s, e, int(capacity), int(top_k),
+        lp, dtype_code(softmax_dtype), ip, icode, g, s, e, int(capacity),
+        int(top_k),
         int(num_microbatches or 1), idx.data_ptr(), pos.data_ptr(),
         gate.data_ptr(), kept.data_ptr(), fill.data_ptr(), loss.data_ptr(),
         ws.data_ptr(), ws_bytes, _stream()), "ntlb_gating")
@@ -1064,11 +1070,11 @@ def activation_backward(dh, pre, activation, factor=None):
 def gating_backward(logits, r, dgate, d_loss, loss_scale, router="top_2",
                     importance=None, z_loss=None, num_microbatches=None,
                     importance_from_slot_gate=False, top_k=0,
-                    use_second_place_loss=False):
+                    use_second_place_loss=False, softmax_dtype=torch.float32):
   """d(logits) [G, S, E] float32.  d_loss: float32 tensor of one element on the
   device (gradient w.r.t. the layer's returned loss); loss_scale:
   moe_loss_coef.  router: "top_2", "switch" (also switch_max) or "ntlb" (then
-  top_k = moe_ntlb_top_k)."""
+  top_k = moe_ntlb_top_k and softmax_dtype = the forward call's)."""
   lib = load_library()
   g, s, e = logits.shape
   dev = logits.device
@@ -1088,8 +1094,8 @@ def gating_backward(logits, r, dgate, d_loss, loss_scale, router="top_2",
         _dev(dgate, "dgate", torch.float32, (g, s, 2)),
         _dev(d_loss, "d_loss", torch.float32), float(loss_scale), g, s, e,
         {"top_2": 0, "switch": 1, "switch_max": 1, "ntlb": 2}[router],
-        int(top_k), int(bool(use_second_place_loss)),
-        int(z_loss is not None),
+        int(top_k), dtype_code(softmax_dtype),
+        int(bool(use_second_place_loss)), int(z_loss is not None),
         float(z_loss or 0.0), int(num_microbatches or 1), dlogits.data_ptr(),
         ws.data_ptr(), ws_bytes, _stream()), "gating_backward")
   return dlogits

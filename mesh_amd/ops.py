@@ -850,8 +850,12 @@ def add(x1, x2, output_shape=None, name=None):
 def multiply(x1, x2, output_shape=None, name=None):
   """Tensor * Python scalar (ScalarMultiplyOperation,
   mesh_tensorflow/ops.py:2006-2023), or Tensor * Tensor where the dims of the
-  smaller one are a subsequence of the larger one's and the smaller one is a
-  constant of the graph (a mask: no gradient flows into it)."""
+  smaller one are a subsequence of the larger one's (mtf.multiply's
+  broadcasting, mesh_tensorflow/ops.py:5135-5153).  Both operands get a
+  gradient, as in the reference (BinaryOpWithBroadcasting's gradient,
+  ops.py:2044-2084): d(big) = dy * small, d(small) = dy * big summed over the
+  dims the small operand does not have (float32 accumulation, one rounding to
+  the small operand's dtype)."""
   del output_shape
   if isinstance(x2, Tensor) and not isinstance(x1, Tensor):
     x1, x2 = x2, x1
@@ -868,10 +872,29 @@ def multiply(x1, x2, output_shape=None, name=None):
 
     def fn(a, b):
       return a * b.reshape(view).to(a.dtype)
+
+    reduced = [i for i, d in enumerate(big.shape.dims)
+               if d not in small.shape.dims]
+    small_sizes = small.shape.to_integer_list
+
+    def small_grad_fn(dy, a):
+      prod = dy.to(torch.float32) * a.to(torch.float32)
+      if reduced:
+        prod = prod.sum(dim=reduced)
+      return prod.reshape(small_sizes).to(small.dtype)
+
+    def grad(op, dy):
+      # (a mask or another constant of the graph needs none: no reduction
+      # over the activations is built for it)
+      d_small = None
+      if _gradient_wanted(op.inputs[1]):
+        d_small = slicewise(small_grad_fn, [dy, op.inputs[0]],
+                            output_shape=small.shape, output_dtype=small.dtype,
+                            name="mul_grad_small")
+      return [multiply(dy, op.inputs[1]), d_small]
     return slicewise(
         fn, [big, small], output_shape=big.shape, output_dtype=big.dtype,
-        name=name or "mul",
-        grad_function=lambda op, dy: [multiply(dy, op.inputs[1]), None])
+        name=name or "mul", grad_function=grad)
   c = _scalar_in(x1.dtype, x2)
   return cwise(lambda t: t * c, [x1], name=name or "scalar_mul",
                grad_function=lambda op, dy: [multiply(dy, x2)])
@@ -1061,6 +1084,25 @@ def get_variable(mesh, name, shape, dtype=float32, master_dtype=None,
                   trainable, **kwargs).outputs[0]
 
 
+# While gradients() walks the graph: the tensors that depend on one of its
+# `xs` (only those are given a gradient); None outside it.
+_GRADIENT_TARGETS = None
+_GRADIENT_XS = None     # the `xs` themselves
+
+
+def gradient_is_returned(tensor):
+  """Inside an Operation.gradient call: is `tensor` one of the tensors whose
+  gradient gradients() hands back to its caller (who must then see the true
+  derivative, not a fused form meant for one particular consumer)?"""
+  return _GRADIENT_XS is None or tensor in _GRADIENT_XS
+
+
+def _gradient_wanted(tensor):
+  """Inside an Operation.gradient call: does gradients() keep a gradient for
+  `tensor`?  (Outside gradients(): unknown, so yes.)"""
+  return _GRADIENT_TARGETS is None or tensor in _GRADIENT_TARGETS
+
+
 def gradients(ys, xs, grad_ys=None, operations=None):
   """mtf.gradients (mesh_tensorflow/ops.py:5254-5291): gradient Tensors of the
   sum of `ys` (weighted by grad_ys) w.r.t. each of `xs`, built by walking the
@@ -1076,18 +1118,25 @@ def gradients(ys, xs, grad_ys=None, operations=None):
       if set(op.inputs) & downstream:
         downstream |= set(op.outputs)
   tensor_to_gradient = {y: g for y, g in zip(ys, grad_ys) if g is not None}
-  for op in operations[::-1]:
-    grad_outputs = [tensor_to_gradient.get(out) for out in op.outputs]
-    if (op.has_gradient and any(g is not None for g in grad_outputs)
-        and (set(op.inputs) & downstream)):
-      with variable_scope(op.name + "/gradients"):
-        input_grads = op.gradient(grad_outputs)
-        for inp, grad in zip(op.inputs, input_grads):
-          if inp in downstream and grad is not None:
-            if inp in tensor_to_gradient:
-              tensor_to_gradient[inp] = tensor_to_gradient[inp] + grad
-            else:
-              tensor_to_gradient[inp] = grad
+  global _GRADIENT_TARGETS, _GRADIENT_XS
+  outer_targets, _GRADIENT_TARGETS = _GRADIENT_TARGETS, downstream
+  outer_xs, _GRADIENT_XS = _GRADIENT_XS, set(xs)
+  try:
+    for op in operations[::-1]:
+      grad_outputs = [tensor_to_gradient.get(out) for out in op.outputs]
+      if (op.has_gradient and any(g is not None for g in grad_outputs)
+          and (set(op.inputs) & downstream)):
+        with variable_scope(op.name + "/gradients"):
+          input_grads = op.gradient(grad_outputs)
+          for inp, grad in zip(op.inputs, input_grads):
+            if inp in downstream and grad is not None:
+              if inp in tensor_to_gradient:
+                tensor_to_gradient[inp] = tensor_to_gradient[inp] + grad
+              else:
+                tensor_to_gradient[inp] = grad
+  finally:
+    _GRADIENT_TARGETS = outer_targets
+    _GRADIENT_XS = outer_xs
   return [tensor_to_gradient.get(x, None) for x in xs]
 
 

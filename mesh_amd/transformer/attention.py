@@ -296,6 +296,32 @@ class SelfAttentionOperation(mtf.Operation):
     return out
 
 
+# The bucket of every (memory position - query position) of a length, as a
+# device tensor: built once per (length, direction, bucket count, device) and
+# kept, so that a lowering -- in particular every decoding step, and a step
+# being recorded into a HIP graph, where a host-to-device copy from pageable
+# memory cannot be captured -- only indexes it.
+_BUCKET_TABLES = {}
+
+
+def relative_bucket_table(length, bidirectional, num_buckets, device):
+  """int32 [2 * length - 1] on `device`: entry d is the bucket of the distance
+  d - (length - 1)."""
+  key = (int(length), bool(bidirectional), int(num_buckets), str(device))
+  table = _BUCKET_TABLES.get(key)
+  if table is None:
+    if torch.cuda.is_available() and torch.cuda.is_current_stream_capturing():
+      raise RuntimeError(
+          "the relative-position bucket table for length %d is not on the "
+          "device yet and cannot be uploaded while a HIP graph is being "
+          "recorded: run the step once before capturing it" % length)
+    bucket = relative_position_bucket(
+        np.arange(-(length - 1), length), bidirectional, num_buckets)
+    table = torch.from_numpy(bucket.astype(np.int32)).to(device)
+    _BUCKET_TABLES[key] = table
+  return table
+
+
 def _attention_extras(extra, ids_at, rel_at, length, bidirectional, dtype):
   """The optional inputs of the attention operations as the library takes
   them: sequence ids [B, L] int32, and (bias values [H, NB] in the activation
@@ -305,9 +331,8 @@ def _attention_extras(extra, ids_at, rel_at, length, bidirectional, dtype):
     ids = extra[ids_at - 3].reshape(-1, length).to(torch.int32).contiguous()
   if rel_at is not None:
     values = extra[rel_at - 3].to(dtype).contiguous()
-    bucket = relative_position_bucket(
-        np.arange(-(length - 1), length), bidirectional, values.shape[-1])
-    rel = (values, torch.from_numpy(bucket.astype(np.int32)).to(values.device))
+    rel = (values, relative_bucket_table(length, bidirectional,
+                                         values.shape[-1], values.device))
   return ids, rel
 
 

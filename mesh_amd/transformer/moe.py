@@ -309,9 +309,12 @@ class _NtlbGatingSpec(object):
     groups = b * t // group_size
     logits = _router_logits(self.noise.apply(x), w, w_packed)
     logits = logits.reshape(groups, group_size, num_experts)
+    # the one router whose projection and softmax stay in the activation
+    # dtype (moe.py:825-836)
     r = moe_hip.ntlb_gating(logits, capacity, self.top_k,
                             importance=importance,
-                            num_microbatches=self.num_microbatches)
+                            num_microbatches=self.num_microbatches,
+                            softmax_dtype=x.dtype)
     return (r, logits) if want_logits else r
 
 
@@ -723,7 +726,9 @@ class MoEV1GradOperation(mtf.Operation):
             router=gating.router, top_k=getattr(gating, "top_k", 0),
             importance=sv["importance"], z_loss=gating.z_loss,
             num_microbatches=gating.num_microbatches,
-            use_second_place_loss=gating.use_second_place_loss)
+            use_second_place_loss=gating.use_second_place_loss,
+            softmax_dtype=(sv["x"].dtype if gating.router == "ntlb"
+                           else torch.float32))
         dispatch_backward = moe_hip.dispatch_backward
       tokens = groups * s_
       if sv["gate_in"] is None:

@@ -37,13 +37,6 @@ class DenseReluDense(transformer.TransformerLayer):
         h, io_channels, use_bias=self.use_bias, activation=None,
         variable_dtype=context.variable_dtype, reduced_dims=h.shape.dims[-1:],
         name="wo")
-    # h = relu(dense(x)) feeds only the output projection: its backward can
-    # apply the ReLU mask to dh while it writes it
-    if (isinstance(h.operation, mtf_layers.DenseOperation)
-        and h.operation._activation == "relu"          # pylint: disable=protected-access
-        and isinstance(y.operation, mtf_layers.DenseOperation)
-        and y.operation.inputs[0] is h):
-      y.operation.masks_input_gradient = True
     return y
 
 

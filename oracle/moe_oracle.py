@@ -36,6 +36,14 @@ MoE file, and its TensorFlow dependency cannot run here):
                                       k = 1 equals switch_gating, closed-form
                                       loss (uniform router: 1.0 for any k),
                                       dense tensors vs record
+  softmax_bf16 (ntlb with bfloat16    two rows worked by hand, the op chain in
+  activations, moe.py:825-836)        Python floats with a frexp-based
+                                      rounding, one-hot rows (every op exact)
+                                      equal the float32 chain, a by-hand tie
+                                      case through the router; UNPINNED: the
+                                      float32 accumulation order inside
+                                      TensorFlow's bfloat16 reduce_sum (index
+                                      order here; rounded once either way)
   expert_selection_gating             per-expert stable sort brute force,
                                       weights of a token sum to sum(p)/count,
                                       closed-form loss (uniform logits: 1.0),
@@ -150,6 +158,41 @@ def softmax(x):
   s = seq_sum(u, axis=-1)[..., None]                     # reduce_sum
   lse = np.log(s).astype(F32) + m                        # log(...) + max_logit
   return np.exp(x + (-lse)).astype(F32)                  # exp(log_softmax)
+
+
+def softmax_bf16(x):
+  """mtf.softmax over the last axis of a bfloat16 tensor, as float32 values
+  that are all bfloat16-representable.
+
+  The same op chain as softmax() (ops.py:5493-5541), but every op of it is a
+  TensorFlow op of its own on a bfloat16 tensor and so rounds its result to
+  bfloat16: negative and reduce_max are exact; add, exp, log round once (Eigen
+  evaluates a bfloat16 exp / log in float32 and rounds the result).
+  tf.reduce_sum of a bfloat16 tensor accumulates in float32 and rounds once
+  (TensorFlow's sum reducer casts bfloat16 to float, reduction_ops.h); the
+  float32 accumulation order is Eigen's and unspecified -- here: index order,
+  which after the rounding to bfloat16 almost never matters.
+  _ntlb_gating is the one router that runs its softmax in the activation dtype
+  (moe.py:825-836: dense -> softmax -> to_float).
+  """
+  x = round_bf16(x)
+  m = x.max(axis=-1, keepdims=True)                      # reduce_max
+  t = round_bf16(x + (-m))                               # x -= max_logit
+  u = round_bf16(np.exp(t).astype(F32))                  # exp
+  s = round_bf16(seq_sum(u, axis=-1))[..., None]         # reduce_sum
+  lse = round_bf16(round_bf16(np.log(s).astype(F32)) + m)  # log(...) + max
+  return round_bf16(np.exp(round_bf16(x + (-lse))).astype(F32))
+
+
+def router_softmax(logits, gating, act_dtype):
+  """The router's probabilities from float32-accumulated logits.  top_2,
+  switch, switch_max and expert_selection cast the tokens to float32 before
+  the projection (moe.py:1384, :1201, :1080); _ntlb_gating does not: its
+  projection's result and its softmax have the activation dtype and only the
+  probabilities are cast to float32 (moe.py:825-836)."""
+  if gating == "ntlb" and act_dtype == "bfloat16":
+    return softmax_bf16(logits)
+  return softmax(logits)
 
 
 def top_1(x):
@@ -526,7 +569,7 @@ def ntlb_gating(logits, capacity, top_k, importance=None,
   k_ = int(top_k)
   if not 1 <= k_ <= e_:
     raise ValueError("moe_ntlb_top_k=%d with %d experts" % (k_, e_))
-  raw_gates = softmax(logits)                                    # :831
+  raw_gates = router_softmax(logits, "ntlb", act_dtype)          # :831-835
   expert_gate, expert_index = top_k_lowest_index_first(raw_gates, k_, -1)
   expert_mask = one_hot(expert_index, e_)                        # [G,S,k,E]
 
@@ -1073,7 +1116,7 @@ def moe_layer_v1(x, w_gate, wi, wo, hp, train, act_dtype="float32",
 # ----------------------------------------------------------------------------
 def gating_backward(logits, r, gating, d_gate_1, d_gate_2, d_loss,
                     importance=None, num_microbatches=None, z_loss=None,
-                    use_second_place_loss=False):
+                    use_second_place_loss=False, act_dtype="float32"):
   """d(logits) of _top_2_gating / _switch_gating / _switch_max_gating /
   _ntlb_gating.
 
@@ -1087,10 +1130,16 @@ def gating_backward(logits, r, gating, d_gate_1, d_gate_2, d_loss,
   d_gate_k [G,S]: gradient w.r.t. the combine weight gate_k * mask_k_flat
   (float32, zero where not kept); d_loss: gradient w.r.t. the balancing loss
   before moe_loss_coef.  Returns float32 [G,S,E].
+
+  act_dtype matters for "ntlb" only: with "bfloat16" the probabilities are the
+  bfloat16 softmax's (router_softmax), and the derivative below is the float32
+  formula evaluated at them (the reference's own chain through the bfloat16
+  ops rounds after each of them; the difference is inside the bfloat16
+  tolerance of the layer's gradients).
   """
   logits = np.asarray(logits, dtype=F32)
   g_, s_, e_ = logits.shape
-  p = softmax(logits)
+  p = router_softmax(logits, gating, act_dtype)
   rows = np.arange(g_)[:, None], np.arange(s_)[None, :]
   i1 = r["index_1"]
   one = np.ones((g_, s_), F32)
@@ -1422,7 +1471,8 @@ def moe_layer_v1_backward(x, w_gate, wi, wo, hp, train, act_dtype, d_out,
   else:
     dlogits = gating_backward(aux["logits"], aux, hp.moe_gating, dgate[..., 0],
                               dgate[..., 1], d_aux, importance,
-                              num_microbatches, z, hp.moe_use_second_place_loss)
+                              num_microbatches, z, hp.moe_use_second_place_loss,
+                              act_dtype)
   # the router saw the perturbed inputs x * mult (perturb_gate_inputs); the
   # multiplier is a constant of the graph
   mult = aux.get("gate_mult")

@@ -45,6 +45,60 @@ def safe_logits(rng, g, s, e, scale=1.0, bias=None, min_gap=1e-4, top=3):
   raise AssertionError("could not separate the top logits")
 
 
+def near_bf16_midpoint(v, margin):
+  """True where |v| lies within `margin` bfloat16 ulps of the midpoint between
+  two neighbouring bfloat16 values (where a last-bits difference between two
+  float32 evaluations of v could round to different bfloat16 values)."""
+  v = np.abs(np.asarray(v, np.float64))
+  ok = v > 0
+  scaled = np.where(ok, v, 1.0)
+  scaled = scaled / 2.0 ** (np.floor(np.log2(scaled)) - 7)     # [128, 256)
+  frac = scaled - np.floor(scaled)
+  return ok & (np.abs(frac - 0.5) < margin)
+
+
+def bf16_softmax_fragile_rows(x, ulps=8):
+  """Rows of float32 logits x [..., E] on which the bfloat16 softmax of the
+  ntlb router could come out differently in two correct implementations.  The
+  additions of the chain are correctly rounded everywhere, so implementations
+  can only part where an exp or log result lies within a few float32 ulps of a
+  bfloat16 rounding midpoint (judged on the float64 result, `ulps` float32
+  ulps either side).  Equal bfloat16 probabilities are fine: ties go by
+  index on both sides."""
+  from oracle import moe_oracle as O
+  margin = ulps * 2.0 ** -16
+  xb = O.round_bf16(x).astype(np.float64)
+  m = xb.max(-1, keepdims=True)
+  t = O.round_bf16((xb - m).astype(np.float32)).astype(np.float64)
+  u64 = np.exp(t)
+  bad = near_bf16_midpoint(u64, margin).any(-1)
+  u = O.round_bf16(u64.astype(np.float32))
+  sm = O.round_bf16(O.seq_sum(u, axis=-1)).astype(np.float64)
+  l64 = np.log(sm)
+  bad |= near_bf16_midpoint(l64, margin)
+  lse = O.round_bf16((O.round_bf16(l64.astype(np.float32)).astype(np.float64)
+                      + m[..., 0]).astype(np.float32)).astype(np.float64)
+  d = O.round_bf16((xb - lse[..., None]).astype(np.float32)).astype(np.float64)
+  bad |= near_bf16_midpoint(np.exp(d), margin).any(-1)
+  return bad
+
+
+def bf16_softmax_safe_logits(rng, g, s, e, scale=1.0, bias=None, ulps=8):
+  """Random logits [g, s, e] without rows that bf16_softmax_fragile_rows
+  flags (those are redrawn)."""
+  def draw(n):
+    x = random_logits(rng, 1, n, e, scale)[0]
+    return x if bias is None else x + bias
+
+  x = draw(g * s).reshape(g, s, e)
+  for _ in range(100):
+    bad = bf16_softmax_fragile_rows(x, ulps)
+    if not bad.any():
+      return x
+    x[bad] = draw(int(bad.sum()))
+  raise AssertionError("could not find rows away from the rounding midpoints")
+
+
 def min_relative_gap(p, k=3):
   """Smallest relative gap between consecutive members of the top-k of each
   softmax row: routing is only implementation-independent when this is well
@@ -80,11 +134,16 @@ def assert_routing_equal(got, want, gate_rtol=1e-5):
 
 
 def safe_tokens(rng, n_tok, m, w_gate, act_dtype, bias=None, min_gap=1e-3,
-                ones_column=False, top=3):
+                ones_column=False, top=3, bf16_router=False):
   """x [n_tok, m] ~ N(0,1) in the activation dtype such that the router logits
   x . w_gate (+ bias) have their `top` largest entries per token at least
   `min_gap` apart (offending tokens are redrawn): the routing then does not
-  depend on the summation order of the router matmul."""
+  depend on the summation order of the router matmul.  bf16_router (the ntlb
+  router with bfloat16 activations, which rounds its logits to bfloat16 and
+  runs its softmax there): instead, no logit of a token may sit within 2 % of
+  a bfloat16 ulp of a rounding midpoint (two summation orders of the matmul
+  then round it alike) and the row must not be one that
+  bf16_softmax_fragile_rows flags."""
   wg = O.cast_act(w_gate, act_dtype)
   x = O.cast_act(rng.standard_normal((n_tok, m)).astype(np.float32), act_dtype)
   k = min(top, wg.shape[1])
@@ -94,6 +153,9 @@ def safe_tokens(rng, n_tok, m, w_gate, act_dtype, bias=None, min_gap=1e-3,
       logits = logits + bias
     top = -np.sort(-logits, axis=-1)[..., :k]
     bad = ((top[..., :-1] - top[..., 1:]) < min_gap).any(axis=-1)
+    if bf16_router:
+      bad = (near_bf16_midpoint(logits, 0.02).any(axis=-1)
+             | bf16_softmax_fragile_rows(logits))
     if not bad.any():
       return x
     x[bad] = O.cast_act(

@@ -49,7 +49,8 @@ def run_backward(hip, x, w, hp, act_dtype, d_out, d_loss, nonpad, mb,
     r = hip.top2_gating(logits, c, importance=imp, num_microbatches=mb)
   elif gating == "ntlb":
     r = hip.ntlb_gating(logits, c, hp.moe_ntlb_top_k, importance=imp,
-                        num_microbatches=mb)
+                        num_microbatches=mb,
+                        softmax_dtype=H.ACT_TORCH[act_dtype])
   else:
     r = hip.switch_gating(logits, c, importance=imp, z_loss=z,
                           num_microbatches=mb,
@@ -79,7 +80,9 @@ def run_backward(hip, x, w, hp, act_dtype, d_out, d_loss, nonpad, mb,
   dlogits = hip.gating_backward(
       logits, r, dgate, dl, scale,
       router="switch" if gating == "switch_max" else gating,
-      top_k=hp.moe_ntlb_top_k, importance=imp, z_loss=z, num_microbatches=mb)
+      top_k=hp.moe_ntlb_top_k, importance=imp, z_loss=z, num_microbatches=mb,
+      softmax_dtype=(H.ACT_TORCH[act_dtype] if gating == "ntlb"
+                     else torch.float32))
   dwg = hip.router_backward_weights(xg.reshape(g * s, m),
                                     dlogits.reshape(g * s, e))
   dx = hip.dispatch_backward(dxe.reshape(e, g, c, m), r, s, dlogits,
@@ -134,7 +137,9 @@ def test_backward_matches_oracle(hip, case):
   if gating == "ntlb":
     w["w_gate"][:, 0] *= 3.0          # a popular expert: later passes matter
   x = H.safe_tokens(rng, g * s, m, w["w_gate"], act_dtype,
-                    top=4 if gating == "ntlb" else 3).reshape(g, s, m)
+                    top=4 if gating == "ntlb" else 3,
+                    bf16_router=(gating == "ntlb" and act_dtype == "bfloat16")
+                    ).reshape(g, s, m)
   nonpad = (rng.random((g, s)) < 0.85).astype(np.float32) if use_np else None
   d_out = O.cast_act(rng.standard_normal((g, s, m)).astype(np.float32), act_dtype)
   d_loss, mb = 1.5, 2
@@ -206,7 +211,9 @@ def test_compact_backward_matches_oracle(hip, case):
   w["w_gate"][:, 0] *= 2.0          # a popular expert (overflows) ...
   w["w_gate"][:, 1] *= 0.25         # ... and one few tokens choose
   x = H.safe_tokens(rng, g * s, m, w["w_gate"], act_dtype,
-                    top=4 if gating == "ntlb" else 3).reshape(g, s, m)
+                    top=4 if gating == "ntlb" else 3,
+                    bf16_router=(gating == "ntlb" and act_dtype == "bfloat16")
+                    ).reshape(g, s, m)
   nonpad = (rng.random((g, s)) < 0.85).astype(np.float32) if use_np else None
   d_out = O.cast_act(rng.standard_normal((g, s, m)).astype(np.float32), act_dtype)
   d_loss, mb = 1.5, 2

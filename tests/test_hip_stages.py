@@ -356,6 +356,48 @@ def test_router_top2_gating_fused(hip, case):
       assert torch.equal(a_, b_)
 
 
+def test_router_gating_largest_group_one_popular_expert(hip):
+  """The largest group the gating entries take (S = 16384, 128 blocks of the
+  one-launch kernel) with 4 experts and a router bias that sends most first
+  choices to expert 0: the per-block slot prefixes of the group tail grow to
+  thousands (they are kept in 16 bits, which the group-size limit makes
+  safe).  One-launch entry against the logits-in entry, bit for bit, and both
+  against the oracle; both capacities, nothing dropped and almost all dropped.
+  A larger group is refused by name."""
+  g, s, m, e = 2, 16384, 64, 4
+  rng = np.random.default_rng(77)
+  w = O.round_bf16((rng.standard_normal((1, m, e)) / np.sqrt(m)).astype(np.float32))
+  x = H.safe_tokens(rng, g * s, m, w[0], "bfloat16",
+                    bias=np.array([2.5, 0.0, 0.0, 0.0], np.float32))[None]
+  bias = np.array([2.5, 0.0, 0.0, 0.0], np.float32)
+  xg, wg = H.to_gpu(x, "bfloat16"), H.to_gpu(w, "bfloat16")
+  wp = hip.pack_weights(wg, wg.dtype)
+  assert hip.fused_gating_supported(xg, e, s)
+  bg = torch.from_numpy(bias).cuda()
+  for c in (s, 300):
+    r, got_logits = hip.router_top2_gating(xg, wp, s, c, bias=bg,
+                                           want_logits=True)
+    r2 = hip.top2_gating(got_logits, c)
+    for name in ("idx", "pos", "kept", "fill", "gate"):
+      assert torch.equal(getattr(r, name), getattr(r2, name)), name
+    # (the two entries sum the loss's column sums over blocks of different
+    # sizes at this expert count)
+    torch.testing.assert_close(r.loss, r2.loss, rtol=2e-6, atol=0)
+    want = O.top_2_gating(H.to_np(got_logits), c)
+    got = H.routing_to_np(r)
+    H.assert_routing_equal(got, want, gate_rtol=2e-5)
+    # raw positions (kept or not): expert 0's last first-choice position
+    np.testing.assert_array_equal(got["pos_1"], want["pos_1"])
+    first0 = (got["index_1"] == 0).sum(axis=1)
+    assert (first0 > 9000).all()                  # prefixes in the thousands
+    assert got["pos_1"].max() == first0.max() - 1
+  too_big = torch.zeros((1, 2 * (s + 128), m), dtype=torch.bfloat16, device="cuda")
+  with pytest.raises(Exception, match="group size S=16512 > 16384"):
+    hip.router_top2_gating(too_big, wp, s + 128, 8)
+  with pytest.raises(Exception, match="group size S=16512 > 16384"):
+    hip.top2_gating(torch.zeros((2, s + 128, e), device="cuda"), 8)
+
+
 @pytest.mark.parametrize("policy", ["all", "none", "threshold", "random"])
 @pytest.mark.parametrize("second_place_loss", [False, True])
 def test_router_top2_gating_fused_policies(hip, policy, second_place_loss):
@@ -620,6 +662,63 @@ def test_ntlb_gating_random_logits(hip, shape):
   if s > 64 and k > 1 and c * e < s:
     assert (want["taken_in_pass"] > 0).any()       # the later passes did something
   assert not got["kept_1"][imp != 1.0].any()
+
+
+@pytest.mark.parametrize("shape", [(2, 1024, 8, 100, 2), (8, 2048, 64, 30, 4),
+                                   (3, 77, 5, 12, 3), (1, 1, 2, 1, 1),
+                                   (2, 131, 200, 1, 4), (2, 512, 16, 512, 4),
+                                   (32, 2048, 64, 64, 4)])
+def test_ntlb_gating_bfloat16_softmax(hip, shape):
+  """bfloat16 activations: the reference rounds the projection's result and
+  every op of the softmax to bfloat16 before the cast to float32
+  (moe.py:825-836).  Record and loss against the oracle's bfloat16 chain; the
+  float32 logits fed here are NOT bfloat16 values (the kernel rounds them).
+  Equal probabilities are common in bfloat16 and go to the lower index."""
+  g, s, e, c, k = shape
+  rng = np.random.default_rng(3100 + sum(shape))
+  logits = H.bf16_softmax_safe_logits(rng, g, s, e, scale=1.5,
+                                      bias=H.zipf_bias(rng, e, scale=2.0))
+  imp = rng.choice(np.array([0.0, 0.5, 1.0], np.float32), size=(g, s),
+                   p=[0.1, 0.1, 0.8])
+  lg = torch.from_numpy(logits).cuda()
+  ties = 0
+  for importance, mb in ((None, None), (imp, 2)):
+    want = O.ntlb_gating(logits, c, k, importance=importance,
+                         num_microbatches=mb, act_dtype="bfloat16")
+    got = H.routing_to_np(hip.ntlb_gating(
+        lg, c, k, importance=None if importance is None else H.to_gpu(importance),
+        num_microbatches=mb, softmax_dtype=torch.bfloat16))
+    H.assert_routing_equal(got, want)
+    # the gates are bfloat16 values, bit for bit
+    np.testing.assert_array_equal(got["gate_1"], want["gate_1"])
+    assert not (got["gate_1"].view(np.uint32) & 0xFFFF).any()
+    np.testing.assert_allclose(got["loss"], float(want["loss"]), rtol=1e-2)
+    p = O.softmax_bf16(logits)
+    top = -np.sort(-p, axis=-1)[..., :min(k + 1, e)]
+    ties += int((top[..., :-1] == top[..., 1:]).sum())
+  if s * g > 1000:
+    assert ties > 0                     # the tie rule was exercised
+    # and the float32 chain would have routed differently somewhere
+    f32 = O.ntlb_gating(logits, c, k)
+    assert (f32["topk_index"] != want["topk_index"]).any()
+
+
+def test_ntlb_gating_bfloat16_hand_case(hip):
+  """[0, 0, 0, -1] four times, capacity 1, k = 3 (worked by hand in the
+  oracle's tests): tokens 0, 1, 2 land on experts 0, 1, 2 in passes 0, 1, 2
+  with the bfloat16 probability 0.294921875; token 3 is left out."""
+  logits = np.tile(np.array([0, 0, 0, -1], np.float32), (1, 4, 1))
+  got = H.routing_to_np(hip.ntlb_gating(torch.from_numpy(logits).cuda(), 1, 3,
+                                        softmax_dtype=torch.bfloat16))
+  np.testing.assert_array_equal(got["kept_1"][0], [True, True, True, False])
+  np.testing.assert_array_equal(got["index_1"][0][:3], [0, 1, 2])
+  np.testing.assert_array_equal(got["gate_1"][0], [0.294921875] * 3 + [0.0])
+  # a float32 difference that bfloat16 does not see: tie, lower index first
+  two = np.array([[[1.0, 1.001, -3.0]]], np.float32)
+  r32 = H.routing_to_np(hip.ntlb_gating(torch.from_numpy(two).cuda(), 4, 2))
+  r16 = H.routing_to_np(hip.ntlb_gating(torch.from_numpy(two).cuda(), 4, 2,
+                                        softmax_dtype=torch.bfloat16))
+  assert (r32["index_1"][0, 0], r16["index_1"][0, 0]) == (1, 0)
 
 
 def test_ntlb_gating_exact_ties(hip):
@@ -1368,3 +1467,11 @@ def test_dropout_noise_from_the_relu_mask(hip):
         assert torch.equal(x_[ei, :used[ei]], y_[ei, :used[ei]]), ei
     else:
       assert torch.equal(x_, y_), j
+  # a keep probability outside [0, 1] is refused by name, not taken for
+  # "unknown"
+  for bad in (-0.25, 1.5):
+    with pytest.raises(Exception, match="dh_keep_prob"):
+      hip.expert_ffn_backward(xe, h, dy, wi, wo, "relu", keep_prob=bad)
+    with pytest.raises(Exception, match="dh_keep_prob"):
+      hip.compact_expert_ffn_backward(xe_c, h_c, dy_c, wi, wo, r, ro, "relu",
+                                      keep_prob=bad)

@@ -93,3 +93,38 @@ def test_generic_slicewise_operation_with_gradient():
   lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()})
   assert torch.equal(lowering.export_to_tf_tensor(y), value.cuda() ** 2)
   assert torch.equal(lowering.export_to_tf_tensor(dx), 2 * value.cuda())
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_multiply_differentiates_both_operands(dtype):
+  """mtf.multiply with broadcasting (mesh_tensorflow/ops.py:5135-5153,
+  gradient :2044-2084): d(big) = dy * small and d(small) = sum over the
+  broadcast dims of dy * big, against float64; a small operand nothing asks a
+  gradient for (a mask) gets no reduction op."""
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  b, l, m = mtf.Dimension("batch", 3), mtf.Dimension("length", 5), mtf.Dimension("d", 8)
+  gen = torch.Generator().manual_seed(4)
+  big_v = torch.randn((3, 5, 8), generator=gen).to(dtype)
+  small_v = torch.randn((3, 8), generator=gen).to(dtype)
+  dy_v = torch.randn((3, 5, 8), generator=gen).to(dtype)
+  big = mtf.import_tf_tensor(mesh, big_v, mtf.Shape([b, l, m]))
+  small = mtf.import_tf_tensor(mesh, small_v, mtf.Shape([b, m]))
+  dy = mtf.import_tf_tensor(mesh, dy_v, mtf.Shape([b, l, m]))
+  y = mtf.multiply(big, small)
+  d_big, d_small = mtf.gradients([y], [big, small], grad_ys=[dy])
+  before = len(graph.operations)
+  (only_big,) = mtf.gradients([y], [big], grad_ys=[dy])
+  assert not any("mul_grad_small" in op.name
+                 for op in graph.operations[before:])
+  lowering = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()})
+  want_big = dy_v.double() * small_v.double()[:, None, :]
+  want_small = (dy_v.double() * big_v.double()).sum(dim=1)
+  tol = dict(rtol=1e-5, atol=1e-6) if dtype == torch.float32 else dict(
+      rtol=2e-2, atol=1e-2)
+  for got, want in ((d_big, want_big), (d_small, want_small),
+                    (only_big, want_big)):
+    out = lowering.export_to_tf_tensor(got)
+    assert out.dtype == dtype and tuple(out.shape) == tuple(want.shape)
+    torch.testing.assert_close(out.double().cpu(), want, **tol)

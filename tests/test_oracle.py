@@ -619,6 +619,120 @@ def test_ntlb_loss_closed_forms():
   np.testing.assert_allclose(got, want / 2, rtol=1e-5)
 
 
+# ---- the bfloat16 softmax of _ntlb_gating (moe.py:825-836) -----------------
+def _bf16_rne(v):
+  """Round a Python float to 8 significant bits, ties to even, with frexp and
+  integer rounding only (shares nothing with the oracle's bit-twiddling
+  round_bf16)."""
+  import math
+  if v == 0.0 or math.isinf(v):
+    return v
+  mant, exp = math.frexp(v)               # 0.5 <= |mant| < 1
+  return math.ldexp(round(mant * 256.0), exp - 8)   # round(): ties to even
+
+
+def _softmax_bf16_by_hand(row):
+  """mtf.softmax (ops.py:5493-5541) on a bfloat16 row, op by op in Python
+  floats: every op's result is rounded to bfloat16 (reduce_max and negative
+  are exact); the sum is rounded once."""
+  import math
+  x = [_bf16_rne(float(v)) for v in row]
+  m = max(x)
+  t = [_bf16_rne(v - m) for v in x]
+  u = [_bf16_rne(math.exp(v)) for v in t]
+  s = _bf16_rne(sum(u))
+  lse = _bf16_rne(_bf16_rne(math.log(s)) + m)
+  return [_bf16_rne(math.exp(_bf16_rne(v - lse))) for v in x]
+
+
+def test_softmax_bf16_hand_worked_rows():
+  """Worked with pencil and a table of exp / log:
+
+  [0, 0, 0]: exp(0) = 1 three times, sum 3, log 3 = 1.0986 -> 1.1015625 (ulp
+  2^-7: 12.62 -> 13 steps above 1), exp(-1.1015625) = 0.33235 -> 0.33203125
+  (ulp 2^-9: 170.16 -> 170).  The float32 chain gives 1/3.
+
+  [1, 0, -1]: t = [0, -1, -2]; exp -> 1, 0.36788 -> 0.3671875 (188.35 -> 188
+  steps of 2^-9), 0.13534 -> 0.1357421875 (138.58 -> 139 steps of 2^-10); sum
+  1.50293 -> 1.5; log 1.5 = 0.405465 -> 0.40625 (207.6 -> 208 steps of 2^-9);
+  lse = 1.40625; exp(-0.40625) = 0.666143 -> 0.66796875 (170.53 -> 171 steps
+  of 2^-8), exp(-1.40625) = 0.245060 -> 0.2451171875 (250.94 -> 251 steps of
+  2^-10), exp(-2.40625) = 0.090152 -> 0.09033203125 (184.63 -> 185 steps of
+  2^-11).  These do not sum to 1: 1.00341796875."""
+  p = O.softmax_bf16(np.array([[0, 0, 0], [1, 0, -1]], np.float32))
+  np.testing.assert_array_equal(p[0], [0.33203125] * 3)
+  np.testing.assert_array_equal(p[1], [0.66796875, 0.2451171875, 0.09033203125])
+  assert p.dtype == np.float32
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_softmax_bf16_against_python_float_chain(seed):
+  rng = np.random.default_rng(930 + seed)
+  e = int(rng.integers(2, 9))
+  logits = (3 * rng.standard_normal((40, e))).astype(np.float32)
+  got = O.softmax_bf16(logits)
+  want = np.array([_softmax_bf16_by_hand(r) for r in logits], np.float64)
+  np.testing.assert_array_equal(got.astype(np.float64), want)
+
+
+def test_softmax_bf16_properties():
+  rng = np.random.default_rng(934)
+  logits = (2 * rng.standard_normal((3, 50, 16))).astype(np.float32)
+  p = O.softmax_bf16(logits)
+  # every value is a bfloat16
+  assert not (p.view(np.uint32) & 0xFFFF).any()
+  # the logits are rounded first: feeding the rounded logits changes nothing
+  np.testing.assert_array_equal(p, O.softmax_bf16(O.round_bf16(logits)))
+  # close to the exact softmax of the rounded logits: seven roundings of
+  # 2^-9 relative each, three of them on exponents of size <= ~8
+  exact = scipy.special.softmax(O.round_bf16(logits).astype(np.float64), -1)
+  np.testing.assert_allclose(p, exact, rtol=0.08)
+  # where every op's result is a bfloat16 anyway the two chains agree bit for
+  # bit: one-hot rows (exp(-200) = 0, sum 1, log 0) ...
+  onehot = np.full((5, 6), -200.0, np.float32)
+  onehot[np.arange(5), [0, 3, 5, 1, 2]] = 0.0
+  np.testing.assert_array_equal(O.softmax_bf16(onehot), O.softmax(onehot))
+  np.testing.assert_array_equal(O.softmax(onehot).sum(-1), np.ones(5))
+  # ... and the dispatcher: only ntlb with bfloat16 activations uses it
+  for gating in ("top_2", "switch", "switch_max", "expert_selection", "ntlb"):
+    for act in ("float32", "bfloat16"):
+      want = O.softmax_bf16 if (gating, act) == ("ntlb", "bfloat16") else O.softmax
+      np.testing.assert_array_equal(O.router_softmax(logits, gating, act),
+                                    want(logits))
+
+
+def test_ntlb_bfloat16_ties_go_to_the_lower_index():
+  """bfloat16 probabilities tie often.  Row [0, 0, 0, -1]: three experts at
+  the same probability, named in index order (repeated first-arg-max,
+  ops.py:5009-5014); capacity 1 and k = 3 then place tokens 0, 1, 2 on experts
+  0, 1, 2 in passes 0, 1, 2 and leave token 3 out."""
+  logits = np.tile(np.array([0, 0, 0, -1], np.float32), (1, 4, 1))
+  # bfloat16 chain by hand: exp(0) = 1 x3, exp(-1) -> 0.3671875, sum 3.3671875
+  # -> 3.375 (ulp 2^-6), log = 1.21640 -> 1.21875 (ulp 2^-7: 27.7 -> 28),
+  # exp(-1.21875) = 0.29560 -> 0.294921875 (ulp 2^-9: 151.3 -> 151)
+  r = O.ntlb_gating(logits, 1, 3, act_dtype="bfloat16")
+  np.testing.assert_array_equal(r["topk_index"][0], [[0, 1, 2]] * 4)
+  np.testing.assert_array_equal(r["kept_1"][0], [True, True, True, False])
+  np.testing.assert_array_equal(r["index_1"][0][:3], [0, 1, 2])
+  np.testing.assert_array_equal(r["taken_in_pass"][0], [0, 1, 2, -1])
+  np.testing.assert_array_equal(r["gate_1"][0], [0.294921875] * 3 + [0.0])
+  # float32 activations: the same routing with the float32 probability
+  r32 = O.ntlb_gating(logits, 1, 3)
+  np.testing.assert_array_equal(r32["index_1"], r["index_1"])
+  np.testing.assert_allclose(r32["gate_1"][0][:3], 1 / (3 + np.exp(-1.0)),
+                             rtol=1e-6)
+
+
+def test_ntlb_bfloat16_rounds_the_logits_first():
+  """Two logits that differ in float32 but round to the same bfloat16 tie in
+  the reference (its projection's result is a bfloat16 tensor): the lower
+  index comes first, whichever is larger in float32."""
+  logits = np.array([[[1.0, 1.001, -3.0]]], np.float32)
+  assert O.ntlb_gating(logits, 4, 2)["topk_index"][0, 0].tolist() == [1, 0]
+  got = O.ntlb_gating(logits, 4, 2, act_dtype="bfloat16")
+  assert got["topk_index"][0, 0].tolist() == [0, 1]
+
+
 @pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
 def test_ntlb_dense_tensors_match_index_record(act_dtype):
   rng = np.random.default_rng(912)
