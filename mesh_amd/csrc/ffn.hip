@@ -7,6 +7,8 @@
 // K-contiguous, C [R, N] = A . B^T.  The bf16 kernel uses
 // v_mfma_f32_32x32x16_bf16 with LDS double buffering; float32 and odd shapes
 // use a plain FMA tile kernel.
+#include <cstdlib>
+#include <cstring>
 #include <type_traits>
 
 #include "common.h"
@@ -1011,6 +1013,330 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
 }
 
 // ---------------------------------------------------------------------------
+// 128 x 256 tiles with TWO blocks resident per compute unit.
+//
+// The 256 x 256 kernel above owns a compute unit: its eight wavefronts meet at
+// one barrier per K tile and write their tile out together, and while they do
+// the matrix pipes of the unit have nothing else to run.  Here a block is four
+// wavefronts (one per SIMD) on a 128 x 256 tile with a K step of 32: three
+// slots each for the token tile (8 KB) and the weight tile (16 KB) are 72 KB,
+// so two blocks share a unit's LDS and its SIMDs, each SIMD holding one
+// wavefront of either block.  The two blocks run on their own: one block's
+// hand-over barrier, its tile's first loads and its store burst fall into the
+// other's K loop.  What that costs is operand traffic -- a 128 x 256 tile
+// loads 1.5 times the bytes per multiply-add of a 256 x 256 one -- so it pays
+// where the tile's prologue and epilogue weigh (short reductions, few tiles
+// per unit) rather than where the chip's power limit is what binds.
+//
+// A wavefront owns 128 x 64 of the tile (4 x 2 MFMA tiles, as in the kernel
+// above).  LDS rows are 64 bytes; one load instruction fills 16 rows, lane l
+// the 16-byte position l % 4 of row l / 4, with the chunk
+// (l % 4) ^ ((row >> 2) & 3) of that row: sixteen consecutive rows read at one
+// logical chunk then touch sixteen distinct 16-byte columns of a 256-byte
+// window.  Per K tile a wavefront issues 2 token and 4 weight loads, three on
+// each of its two MFMA steps, for the tile two ahead (its slot was last read
+// one tile ago, before the previous hand-over barrier); the hand-over waits
+// with vmcnt(3): the next tile has landed, the three loads just issued fly on.
+// ---------------------------------------------------------------------------
+struct DuoCfg {
+  static constexpr int BM = 128, BN = 256, BK = 32, WAVES = 4;
+  static constexpr int THREADS = 64 * WAVES;
+  static constexpr int TM = BM / 32, TN = (BN / WAVES) / 32;   // 4 x 2
+  static constexpr int ROW_BYTES = BK * 2;
+  static constexpr int A_INSTR = (BM / 16) / WAVES, B_INSTR = (BN / 16) / WAVES;
+  static constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES;
+  static constexpr int SLOTS = 3;
+  static constexpr int B_BASE = SLOTS * A_BYTES;
+  static constexpr size_t LDS_BYTES = (size_t)SLOTS * (A_BYTES + B_BYTES);
+  static_assert(A_INSTR == 2 && B_INSTR == 4, "load schedule assumes 2 + 4");
+  static_assert(2 * LDS_BYTES <= 160 * 1024, "two blocks per compute unit");
+};
+
+template <bool RELU, bool GATHER>
+__global__ __launch_bounds__(DuoCfg::THREADS, 2) void grouped_gemm_bf16_duo_kernel(
+    const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
+    bf16_t* __restrict__ Cout, int R, int N, int K, int tiles_m, int tiles_n,
+    int total_tiles, const int32_t* __restrict__ row_map,
+    const bf16_t* __restrict__ zero_row) {
+  using Cfg = DuoCfg;
+  constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
+  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
+
+  // Persistent blocks, two per compute unit; block b runs on XCD b % 8 and the
+  // blocks of an XCD hold consecutive logical tiles (see the kernel above).
+  const int nblk = gridDim.x;
+  int tile = blockIdx.x;
+  if ((nblk & 7) == 0) tile = (blockIdx.x & 7) * (nblk >> 3) + (blockIdx.x >> 3);
+  if (tile >= total_tiles) return;
+
+  const int tid = threadIdx.x;
+  const int lane = tid & 63;
+  const int wave = tid >> 6;
+  const int tiles_per_e = tiles_m * tiles_n;
+  const int nk = K / BK;
+
+  int row0, col0;
+  const bf16_t *Ae, *Be;
+  bf16_t* Ce;
+  typename std::conditional<GATHER, int64_t, int>::type a_off[Cfg::A_INSTR];
+  int b_off[Cfg::B_INSTR];
+  // rows this lane loads: instruction q = wave + WAVES j covers tile rows
+  // 16 q .. 16 q + 15
+  auto tile_coords = [&](int logical, int& e, int& tm, int& tn) {
+    e = logical / tiles_per_e;
+    const int rem = logical - e * tiles_per_e;
+    tn = rem / tiles_m;
+    tm = rem - tn * tiles_m;
+    if (tiles_m > 16 && (tiles_m & 15) == 0 && (tiles_n & 3) == 0) {
+      // many row tiles: 64 consecutive logical tiles (what an XCD holds) form
+      // a block of 16 row tiles x 4 column tiles
+      const int sup = rem >> 6, within = rem & 63;
+      const int per_row = tiles_n >> 2;
+      const int sm = sup / per_row, sn = sup - sm * per_row;
+      tm = sm * 16 + (within & 15);
+      tn = sn * 4 + (within >> 4);
+    }
+  };
+  // GATHER: the slot -> token map entries of this lane's rows of a tile, read
+  // a whole tile ahead so that the next tile's first loads do not wait for them
+  int next_src[Cfg::A_INSTR];
+  auto fetch_map = [&](int logical) {
+    if constexpr (GATHER) {
+      int e, tm, tn;
+      tile_coords(logical, e, tm, tn);
+#pragma unroll
+      for (int j = 0; j < Cfg::A_INSTR; ++j) {
+        const int row = (wave + Cfg::WAVES * j) * 16 + (lane >> 2);
+        next_src[j] = row_map[(int64_t)e * R + min(tm * BM + row, R - 1)];
+      }
+    }
+  };
+  auto set_tile = [&](int logical) {
+    int e, tm, tn;
+    tile_coords(logical, e, tm, tn);
+    row0 = tm * BM;
+    col0 = tn * BN;
+    Ae = GATHER ? A : A + (int64_t)e * R * K;
+    Be = B + (int64_t)e * N * K;
+    Ce = Cout + (int64_t)e * R * N;
+#pragma unroll
+    for (int j = 0; j < Cfg::A_INSTR; ++j) {
+      const int row = (wave + Cfg::WAVES * j) * 16 + (lane >> 2);
+      const int chunk = (lane & 3) ^ ((row >> 2) & 3);
+      if constexpr (GATHER) {
+        const int src = next_src[j];
+        a_off[j] = (src >= 0 ? (int64_t)src * K : (int64_t)(zero_row - A)) +
+                   chunk * 8;
+      } else {
+        a_off[j] = min(row0 + row, R - 1) * K + chunk * 8;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < Cfg::B_INSTR; ++j) {
+      const int row = (wave + Cfg::WAVES * j) * 16 + (lane >> 2);
+      const int chunk = (lane & 3) ^ ((row >> 2) & 3);
+      b_off[j] = min(col0 + row, N - 1) * K + chunk * 8;
+    }
+  };
+  // load j of token / weight tile kt into `slot`; kt past the end re-fetches
+  // the last tile into a slot nobody reads any more
+  auto load_a = [&](int kt, int slot, int j) {
+    kt = min(kt, nk - 1);
+    __builtin_amdgcn_global_load_lds(
+        (glb_void_t*)(Ae + kt * BK + a_off[j]),
+        (lds_void_t*)(smem_raw + slot * Cfg::A_BYTES +
+                      (wave + Cfg::WAVES * j) * 1024), 16, 0, 0);
+  };
+  auto load_b = [&](int kt, int slot, int j) {
+    kt = min(kt, nk - 1);
+    __builtin_amdgcn_global_load_lds(
+        (glb_void_t*)(Be + kt * BK + b_off[j]),
+        (lds_void_t*)(smem_raw + Cfg::B_BASE + slot * Cfg::B_BYTES +
+                      (wave + Cfg::WAVES * j) * 1024), 16, 0, 0);
+  };
+  // the six loads of a tile in the order the K loop issues them
+  auto load_n = [&](int kt, int slot, int n) {
+    if (n < 4) load_b(kt, slot, n);
+    else load_a(kt, slot, n - 4);
+  };
+  // first loads of a tile: everything but weight tile 1, whose slot the
+  // previous tile's epilogue still uses as staging area
+  auto prologue_head = [&]() {
+#pragma unroll
+    for (int j = 0; j < Cfg::A_INSTR; ++j) load_a(0, 0, j);
+#pragma unroll
+    for (int j = 0; j < Cfg::B_INSTR; ++j) load_b(0, 0, j);
+#pragma unroll
+    for (int j = 0; j < Cfg::A_INSTR; ++j) load_a(1, 1, j);
+  };
+  auto prologue_tail = [&]() {
+#pragma unroll
+    for (int j = 0; j < Cfg::B_INSTR; ++j) load_b(1, 1, j);
+  };
+
+  f32x16_t acc[Cfg::TM][Cfg::TN];
+  const int fr = lane & 31, fc = lane >> 5;
+  int a_frag[BK / 16], b_frag[BK / 16];
+#pragma unroll
+  for (int kk = 0; kk < BK / 16; ++kk) {
+    const int col = ((kk * 2 + fc) ^ ((fr >> 2) & 3)) * 16;
+    a_frag[kk] = fr * Cfg::ROW_BYTES + col;
+    b_frag[kk] = (wave * 64 + fr) * Cfg::ROW_BYTES + col;
+  }
+  bf16x8_t fa[2][Cfg::TM], fb[2][Cfg::TN];
+  auto read_frag = [&](int slot, int kk, int buf, int n) {
+    if (n < Cfg::TM)
+      fa[buf][n] = *reinterpret_cast<const bf16x8_t*>(
+          smem_raw + slot * Cfg::A_BYTES + a_frag[kk] + n * 32 * Cfg::ROW_BYTES);
+    else
+      fb[buf][n - Cfg::TM] = *reinterpret_cast<const bf16x8_t*>(
+          smem_raw + Cfg::B_BASE + slot * Cfg::B_BYTES + b_frag[kk] +
+          (n - Cfg::TM) * 32 * Cfg::ROW_BYTES);
+  };
+  auto mfma = [&](int buf, int n) {
+    const int i = n / Cfg::TN, j = n % Cfg::TN;
+    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][j], fa[buf][i],
+                                                        acc[i][j], 0, 0, 0);
+  };
+  auto fence = [&]() { __builtin_amdgcn_sched_barrier(0); };
+  // fragment reads in the order the MFMAs first need them: a0 b0 b1 a1 a2 a3
+  constexpr int RD[6] = {0, Cfg::TM, Cfg::TM + 1, 1, 2, 3};
+
+  int slot = 0;   // kt % 3
+  auto k_tile = [&](int kt, auto last_tag) {
+    constexpr bool LAST = decltype(last_tag)::value;
+    const int s1 = slot == 2 ? 0 : slot + 1;      // slot of tile kt + 1
+    const int s2 = s1 == 2 ? 0 : s1 + 1;          // of tile kt + 2 (= kt - 1)
+    // step 0: the fragments of step 1, loads 0-2 of tile kt + 2
+    fence();
+    read_frag(slot, 1, 1, RD[0]);
+    read_frag(slot, 1, 1, RD[1]);
+    mfma(0, 0); fence();
+    read_frag(slot, 1, 1, RD[2]);
+    mfma(0, 1); fence();
+    if (!LAST) load_n(kt + 2, s2, 0);
+    mfma(0, 2); fence();
+    read_frag(slot, 1, 1, RD[3]);
+    mfma(0, 3); fence();
+    read_frag(slot, 1, 1, RD[4]);
+    mfma(0, 4); fence();
+    if (!LAST) load_n(kt + 2, s2, 1);
+    mfma(0, 5); fence();
+    read_frag(slot, 1, 1, RD[5]);
+    mfma(0, 6); fence();
+    if (!LAST) load_n(kt + 2, s2, 2);
+    mfma(0, 7); fence();
+    if (!LAST) {
+      // step 1 behind the hand-over: this lane holds the step's fragments
+      // (lgkmcnt 0) and everything but the three loads just issued has landed
+      __builtin_amdgcn_s_waitcnt((3 & 15) | (0 << 8) | (7 << 4));
+      asm volatile("" ::: "memory");
+      __builtin_amdgcn_s_barrier();
+      asm volatile("" ::: "memory");
+      fence();
+#pragma unroll
+      for (int n = 0; n < 6; ++n) {
+        read_frag(s1, 0, 0, RD[n]);
+        if (n >= 3) load_n(kt + 2, s2, n);
+        mfma(1, n); fence();
+      }
+      mfma(1, 6); fence();
+      mfma(1, 7); fence();
+    } else {
+#pragma unroll
+      for (int n = 0; n < 8; ++n) mfma(1, n);
+    }
+    slot = s1;
+  };
+
+  // Epilogue staging: two passes of 64 output rows in weight slots 1 and 2
+  // (32 KB), rows of 512 bytes with 16-byte chunk c of row r at c ^ (r & 31).
+  constexpr int EPI_ROWS = 64;
+  constexpr int EPI_ROW_BYTES = BN * 2;
+  constexpr int EPI_BASE = Cfg::B_BASE + Cfg::B_BYTES;
+  static_assert(EPI_BASE + EPI_ROWS * EPI_ROW_BYTES <= (int)Cfg::LDS_BYTES,
+                "epilogue staging exceeds the ring");
+  unsigned char* Cs = smem_raw + EPI_BASE;
+  const int m_l = lane & 31;
+  const int half = lane >> 5;
+  constexpr int CPR_C = BN / 8;
+
+  const int tile_step = nblk;
+  fetch_map(tile);
+  set_tile(tile);
+  prologue_head();
+  prologue_tail();
+  for (;;) {
+    const int next = tile + tile_step;
+    const bool has_next = next < total_tiles;
+    // (always issued, so that the number of loads in flight below is fixed)
+    fetch_map(min(next, total_tiles - 1));
+#pragma unroll
+    for (int i = 0; i < Cfg::TM; ++i)
+#pragma unroll
+      for (int j = 0; j < Cfg::TN; ++j)
+#pragma unroll
+        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
+    // K tile 0 has landed: token tile 1, weight tile 1 (2 + 4 loads) and, with
+    // GATHER, the two map entries of the next tile may still be in flight
+    wait_vmcnt<GATHER ? 8 : 6>();
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#pragma unroll
+    for (int n = 0; n < 6; ++n) read_frag(0, 0, 0, RD[n]);
+    slot = 0;
+    for (int kt = 0; kt + 1 < nk; ++kt) k_tile(kt, std::false_type{});
+    k_tile(nk - 1, std::true_type{});
+
+    wait_vmcnt<0>();
+    __syncthreads();
+    const int out_row0 = row0, out_col0 = col0;
+    bf16_t* out_c = Ce;
+    if (has_next) {
+      set_tile(next);
+      prologue_head();
+    }
+#pragma unroll
+    for (int pass = 0; pass < 2; ++pass) {
+#pragma unroll
+      for (int ii = 0; ii < 2; ++ii) {
+        const int i = pass * 2 + ii;
+        const int srow = ii * 32 + m_l;
+#pragma unroll
+        for (int j = 0; j < Cfg::TN; ++j) {
+#pragma unroll
+          for (int q = 0; q < 4; ++q) {
+            const int chunk = (wave * 64 + j * 32 + 8 * q) / 8;
+            uint2 v;
+            v.x = pack2_bf16(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], RELU);
+            v.y = pack2_bf16(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3], RELU);
+            *reinterpret_cast<uint2*>(Cs + srow * EPI_ROW_BYTES +
+                                      ((chunk ^ m_l) * 16) + half * 8) = v;
+          }
+        }
+      }
+      __syncthreads();
+#pragma unroll
+      for (int c = tid; c < EPI_ROWS * CPR_C; c += Cfg::THREADS) {
+        const int srow = c / CPR_C, chunk = c % CPR_C;
+        const int grow = out_row0 + pass * 64 + srow;
+        const int gcol = out_col0 + chunk * 8;
+        if (grow < R && gcol < N) {
+          const u32x4_t v = *reinterpret_cast<const u32x4_t*>(
+              Cs + srow * EPI_ROW_BYTES + ((chunk ^ (srow & 31)) * 16));
+          *reinterpret_cast<u32x4_t*>(out_c + (int64_t)grow * N + gcol) = v;
+        }
+      }
+      __syncthreads();
+    }
+    if (!has_next) break;
+    tile = next;
+    prologue_tail();
+  }
+}
+
+// ---------------------------------------------------------------------------
 // float32 on the matrix cores: v_mfma_f32_32x32x2_f32, true float32 operands
 // and accumulation (the float32 configuration of the layer: no narrowing).
 // Block tile 128 x 128, K step 32, 4 wavefronts in a 2 x 2 grid, each a 64 x 64
@@ -1652,6 +1978,53 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
   return 0;
 }
 
+// The 128 x 256 kernel with two blocks per compute unit; row_map / zero_row as
+// in launch_ring.
+static int launch_duo(const bf16_t* A, const bf16_t* B, bf16_t* C, int E, int R,
+                      int N, int K, bool relu, hipStream_t st,
+                      const int32_t* row_map = nullptr,
+                      const bf16_t* zero_row = nullptr) {
+  using Cfg = DuoCfg;
+  const int tiles_m = (R + Cfg::BM - 1) / Cfg::BM;
+  const int tiles_n = (N + Cfg::BN - 1) / Cfg::BN;
+  const int64_t tiles = (int64_t)tiles_m * tiles_n * E;
+  MOE_REQUIRE(tiles <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
+              "expert_ffn: too many tiles (%lld)", (long long)tiles);
+  const int cus = compute_units();
+  if (cus == 0) return MESH_MOE_E_HIP;
+  const unsigned blocks = (unsigned)(tiles < 2 * cus ? tiles : 2 * cus);
+#define MOE_DUO(RELU_, GATHER_)                                                \
+  do {                                                                         \
+    auto k = grouped_gemm_bf16_duo_kernel<RELU_, GATHER_>;                     \
+    MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);                                          \
+    k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(                           \
+        A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, row_map, zero_row);    \
+  } while (0)
+  if (row_map != nullptr) {
+    if (relu) MOE_DUO(true, true);
+    else MOE_DUO(false, true);
+  } else {
+    if (relu) MOE_DUO(true, false);
+    else MOE_DUO(false, false);
+  }
+#undef MOE_DUO
+  MOE_CHECK_LAUNCH("expert_ffn (mfma, two blocks per compute unit)");
+  return 0;
+}
+
+// EXPERIMENT: MESH_MOE_GEMM_VARIANT=duo|ring forces the kernel of the plain and
+// gathered forward GEMMs.
+static int gemm_variant_override() {
+  static int v = -1;
+  if (v < 0) {
+    const char* s = getenv("MESH_MOE_GEMM_VARIANT");
+    v = 0;
+    if (s && !strcmp(s, "duo")) v = 1;
+    if (s && !strcmp(s, "ring")) v = 2;
+  }
+  return v;
+}
+
 static int launch_f32_mfma(const float* A, const float* B, float* C, int E,
                            int R, int N, int K, bool relu, hipStream_t st) {
   using Cfg = F32Cfg;
@@ -1736,6 +2109,8 @@ static int grouped_gemm(const void* A, const void* B, void* C, int E, int R,
         rc = launch_ring(a, b, c, E, R, N, K, false, st, nullptr, nullptr,
                          (const bf16_t*)relu_mask_src, nullptr, mask_scale);
         *mask_applied = rc == 0;
+      } else if (gemm_variant_override() == 1) {
+        rc = launch_duo(a, b, c, E, R, N, K, relu, st);
       } else {
         rc = launch_ring(a, b, c, E, R, N, K, relu, st);
       }
@@ -1982,8 +2357,11 @@ extern "C" int mesh_moe_dispatched_expert_ffn(
       idx, pos, gate, kept, map, (int64_t)G * S, S, C, rows);
   MOE_CHECK_LAUNCH("dispatched_expert_ffn (slot map)");
   const bool relu = activation == MESH_MOE_ACT_RELU;
-  int rc = launch_ring((const bf16_t*)x, (const bf16_t*)wi_packed, (bf16_t*)h,
-                       E, R, H, M, relu, st, map, zero_row);
+  int rc = gemm_variant_override() == 1
+               ? launch_duo((const bf16_t*)x, (const bf16_t*)wi_packed,
+                            (bf16_t*)h, E, R, H, M, relu, st, map, zero_row)
+               : launch_ring((const bf16_t*)x, (const bf16_t*)wi_packed,
+                             (bf16_t*)h, E, R, H, M, relu, st, map, zero_row);
   if (rc != 0) return rc;
   if (!relu && activation != MESH_MOE_ACT_LINEAR) {
     rc = launch_activation(h, (int64_t)E * R * H, activation, dtype, st);
