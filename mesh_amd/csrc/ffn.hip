@@ -7,8 +7,6 @@
 // K-contiguous, C [R, N] = A . B^T.  The bf16 kernel uses
 // v_mfma_f32_32x32x16_bf16 with LDS double buffering; float32 and odd shapes
 // use a plain FMA tile kernel.
-#include <cstdlib>
-#include <cstring>
 #include <type_traits>
 
 #include "common.h"
@@ -574,12 +572,26 @@ struct RingCfg {
 // skip their multiply-adds, with the flag carried in the list entry: 5 %
 // slower, although nothing was added to the path of the full tiles but a
 // second copy of the K loop next to it.)
+//
+// TAILS (R not a multiple of the 256-row tile): in an expert's last row tile
+// a wavefront multiplies only the 32-row pieces of its 128-row sub-tile that
+// hold rows below R -- the piece count is the same for the whole K loop, so
+// the wavefront runs the copy of the loop written for that count (0 to 4
+// pieces; with 0 it only loads and meets the barriers).  The two wavefronts of
+// a SIMD own the upper and the lower half of the tile, so a tile with 144
+// valid rows costs the SIMD 4 + 1 pieces instead of 8.  (Numbering the
+// experts' last row tiles after all full ones, so that the persistent blocks
+// end on the cheaper tiles, separates the row tiles that share a weight panel:
+// with 400 rows per expert the weights were then read twice from memory and
+// the launches took 14 % longer; moving only as many last row tiles as the
+// final, partly filled round holds to the end cost 5 % where it applied, 640
+// rows per expert with 384 tiles, for the same reason.)
 // 512 bytes that stay zero (nothing writes them): where a K-major tile reaches
 // past the last reduction row, its rows are loaded from here
 static __device__ __attribute__((aligned(256))) bf16_t kmajor_zero_row[256];
 
 template <bool RELU, bool GATHER = false, bool KMAJOR = false,
-          bool MASKED = false, bool LISTED = false>
+          bool MASKED = false, bool LISTED = false, bool TAILS = false>
 __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kernel(
     const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
     bf16_t* __restrict__ Cout, int R, int N, int K, int tiles_m, int tiles_n,
@@ -607,6 +619,19 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
   const int nblk = gridDim.x;
   if constexpr (LISTED) total_tiles = tile_list[-1];
   int tile, tile_end, tile_step;
+  // TAILS: in its round k a block takes the tile k places further (cyclically)
+  // among its XCD's P tiles of the round, so that it meets every row tile of
+  // the experts in turn, full and partly empty ones: with a fixed place and an
+  // even number of row tiles half of the blocks would only ever get the cheap
+  // last row tiles and run ahead of the blocks they share weight panels with.
+  int round = 0;
+  const int xcd_tiles = (nblk & 7) == 0 ? (nblk >> 3) : 0;
+  const int xcd_first = (blockIdx.x & 7) * xcd_tiles;
+  const int xcd_local = blockIdx.x >> 3;
+  auto tile_of_round = [&](int k) {
+    const int place = xcd_local + k;
+    return k * nblk + xcd_first + (place >= xcd_tiles ? place % xcd_tiles : place);
+  };
   if ((nblk & 7) == 0) {
     const int xcd = blockIdx.x & 7, local = blockIdx.x >> 3;
     tile = xcd * (nblk >> 3) + local;
@@ -635,13 +660,17 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
   bf16_t* Ce;
   typename std::conditional<GATHER, int64_t, int>::type a_off[Cfg::A_INSTR];
   int b_off[Cfg::B_INSTR];
-  auto set_tile = [&](int logical) {
+  // TAILS: 32-row pieces of this wavefront's sub-tile that hold rows below R
+  int pieces = Cfg::TM;
+  // logical tile -> expert, row tile, column tile
+  auto tile_coords = [&](int logical, int& e, int& tm, int& tn) {
     if constexpr (LISTED) logical = tile_list[logical];
-    const int e = logical / tiles_per_e;
+    e = logical / tiles_per_e;
     const int rem = logical - e * tiles_per_e;
-    int tn = rem / tiles_m;
-    int tm = rem - tn * tiles_m;
-    if (!LISTED && tiles_m > 8 && (tiles_m & 7) == 0 && (tiles_n & 3) == 0) {
+    tn = rem / tiles_m;
+    tm = rem - tn * tiles_m;
+    if (!LISTED && !TAILS && tiles_m > 8 && (tiles_m & 7) == 0 &&
+        (tiles_n & 3) == 0) {
       // 32 consecutive logical tiles (what an XCD holds at any moment) form a
       // block of 8 row tiles x 4 column tiles: 12 operand panels for 32 tiles.
       // With the plain order and many row tiles they would be 32 row tiles of
@@ -653,6 +682,35 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
       const int sm = sup / per_row, sn = sup - sm * per_row;
       tm = sm * 8 + (within & 7);
       tn = sn * 4 + (within >> 3);
+    }
+  };
+  // GATHER: the slot -> token map entries of the four rows this lane loads in
+  // a tile.  fetch_map issues the four loads back to back without waiting
+  // (written as asm: the compiler would wait for each before issuing the
+  // next, four round trips per tile); the caller waits with vmcnt(0) before
+  // set_tile of the same tile reads map_src.
+  int map_src[Cfg::A_INSTR];
+  auto fetch_map = [&](int logical) {
+    if constexpr (GATHER) {
+      int e, tm, tn;
+      tile_coords(logical, e, tm, tn);
+#pragma unroll
+      for (int j = 0; j < Cfg::A_INSTR; ++j) {
+        const int row = (wave + Cfg::WAVES * j) * 8 + (lane >> 3);
+        const int32_t* p = row_map + ((int64_t)e * R + min(tm * BM + row, R - 1));
+        asm volatile("global_load_dword %0, %1, off"
+                     : "=&v"(map_src[j]) : "v"(p) : "memory");
+      }
+    }
+  };
+  auto set_tile = [&](int logical) {
+    int e, tm, tn;
+    tile_coords(logical, e, tm, tn);
+    if constexpr (TAILS) {
+      const int valid = min(BM, R - tm * BM);
+      const int blocks = (valid + 31) >> 5;
+      pieces = __builtin_amdgcn_readfirstlane(
+          wm == 0 ? min(blocks, Cfg::TM) : max(blocks - Cfg::TM, 0));
     }
     row0 = tm * BM;
     col0 = tn * BN;
@@ -682,7 +740,7 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
       const int row = (wave + Cfg::WAVES * j) * 8 + (lane >> 3);
       const int chunk = (lane & 7) ^ lds_swizzle(row);
       if constexpr (GATHER) {
-        const int src = row_map[(int64_t)e * R + min(row0 + row, R - 1)];
+        const int src = map_src[j];
         a_off[j] = (src >= 0 ? (int64_t)src * K : (int64_t)(zero_row - A)) +
                    chunk * 8;
       } else {
@@ -814,6 +872,12 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
     acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][j], fa[buf][i],
                                                         acc[i][j], 0, 0, 0);
   };
+  // with NA of the wavefront's TM row pieces in use: is fragment read n /
+  // MFMA n of a step needed?
+  auto frag_used = [](int na, int n) {
+    return na > 0 && (n >= Cfg::TM || n < na);
+  };
+  auto mfma_used = [](int na, int n) { return n / Cfg::TN < na; };
   // nothing moves across: the instruction order below is the issue order
   auto fence = [&]() { __builtin_amdgcn_sched_barrier(0); };
   // fragment reads in the order the MFMAs (token tile i = n / TN outer, weight
@@ -822,8 +886,15 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
 
   // bslot = kt % 3, kept incrementally
   int bslot = 0;
-  auto k_tile = [&](int kt, auto last_tag) {
+  auto k_tile = [&](int kt, auto last_tag, auto na_tag) {
     constexpr bool LAST = decltype(last_tag)::value;
+    constexpr int NA = decltype(na_tag)::value;      // row pieces in use
+    auto rd = [&](int as, int bs, int kk, int buf, int n) {
+      if (frag_used(NA, n)) read_frag(as, bs, kk, buf, n);
+    };
+    auto mm = [&](int buf, int n) {
+      if (mfma_used(NA, n)) mfma(buf, n);
+    };
     const int aslot = kt & 1;
     const int bnext = bslot == 2 ? 0 : bslot + 1;       // slot of tile kt+1
     const int bnext2 = bnext == 2 ? 0 : bnext + 1;      // slot of tile kt+2
@@ -845,22 +916,22 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
         // 2 loads, 8 MFMAs of step kk
         fence();
         wait_frags();
-        read_frag(aslot, bslot, kk + 1, nxt, RD[0]);
-        read_frag(aslot, bslot, kk + 1, nxt, RD[1]);
-        mfma(cur, 0); fence();
-        read_frag(aslot, bslot, kk + 1, nxt, RD[2]);
-        mfma(cur, 1); fence();
+        rd(aslot, bslot, kk + 1, nxt, RD[0]);
+        rd(aslot, bslot, kk + 1, nxt, RD[1]);
+        mm(cur, 0); fence();
+        rd(aslot, bslot, kk + 1, nxt, RD[2]);
+        mm(cur, 1); fence();
         load(0);
-        mfma(cur, 2); fence();
-        read_frag(aslot, bslot, kk + 1, nxt, RD[3]);
-        mfma(cur, 3); fence();
-        read_frag(aslot, bslot, kk + 1, nxt, RD[4]);
-        mfma(cur, 4); fence();
+        mm(cur, 2); fence();
+        rd(aslot, bslot, kk + 1, nxt, RD[3]);
+        mm(cur, 3); fence();
+        rd(aslot, bslot, kk + 1, nxt, RD[4]);
+        mm(cur, 4); fence();
         load(1);
-        mfma(cur, 5); fence();
-        read_frag(aslot, bslot, kk + 1, nxt, RD[5]);
-        mfma(cur, 6); fence();
-        mfma(cur, 7); fence();
+        mm(cur, 5); fence();
+        rd(aslot, bslot, kk + 1, nxt, RD[5]);
+        mm(cur, 6); fence();
+        mm(cur, 7); fence();
       } else if (!LAST) {
         // this lane holds the last step's fragments (lgkmcnt 0); everything
         // but the four weight loads of tile kt+2 has landed (vmcnt 4)
@@ -874,16 +945,16 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
         // up with the other wavefronts' and hold this one's MFMAs back
 #pragma unroll
         for (int n = 0; n < 6; ++n) {
-          read_frag(aslot ^ 1, bnext, 0, nxt, RD[n]);
+          rd(aslot ^ 1, bnext, 0, nxt, RD[n]);
           if (n >= 2) load(n - 2);
-          mfma(cur, n); fence();
+          mm(cur, n); fence();
         }
-        mfma(cur, 6); fence();
-        mfma(cur, 7); fence();
+        mm(cur, 6); fence();
+        mm(cur, 7); fence();
       } else {
         wait_frags();
 #pragma unroll
-        for (int n = 0; n < 8; ++n) mfma(cur, n);
+        for (int n = 0; n < 8; ++n) mm(cur, n);
       }
     }
     bslot = bnext;
@@ -906,6 +977,11 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
   const int half = lane >> 5;   // which 8 bytes of a 16-byte chunk
   constexpr int CPR_C = BN / 8;  // 16-byte chunks per output row
 
+  fetch_map(tile);
+  if constexpr (GATHER) {
+    wait_vmcnt<0>();
+    asm volatile("" ::: "memory");
+  }
   set_tile(tile);
   prologue_head();
   prologue_tail();
@@ -921,15 +997,36 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
     asm volatile("" ::: "memory");
     __builtin_amdgcn_s_barrier();
     asm volatile("" ::: "memory");
+    auto k_loop = [&](auto na_tag) {
+      constexpr int NA = decltype(na_tag)::value;
 #pragma unroll
-    for (int n = 0; n < 6; ++n) read_frag(0, 0, 0, 0, RD[n]);
-    bslot = 0;
-    for (int kt = 0; kt + 1 < nk; ++kt) k_tile(kt, std::false_type{});
-    k_tile(nk - 1, std::true_type{});
+      for (int n = 0; n < 6; ++n)
+        if (frag_used(NA, RD[n])) read_frag(0, 0, 0, 0, RD[n]);
+      bslot = 0;
+      for (int kt = 0; kt + 1 < nk; ++kt) k_tile(kt, std::false_type{}, na_tag);
+      k_tile(nk - 1, std::true_type{}, na_tag);
+    };
+    if constexpr (TAILS) {
+      switch (pieces) {
+        case 0: k_loop(std::integral_constant<int, 0>{}); break;
+        case 1: k_loop(std::integral_constant<int, 1>{}); break;
+        case 2: k_loop(std::integral_constant<int, 2>{}); break;
+        case 3: k_loop(std::integral_constant<int, 3>{}); break;
+        default: k_loop(std::integral_constant<int, Cfg::TM>{}); break;
+      }
+    } else {
+      k_loop(std::integral_constant<int, Cfg::TM>{});
+    }
 
+    const int next = (TAILS && xcd_tiles != 0) ? tile_of_round(round + 1)
+                                               : tile + tile_step;
+    const bool has_next = next < tile_end;
+    // (the next tile's map entries travel while the ring drains)
+    if (has_next) fetch_map(next);
     // Every wavefront is done with the ring and no direct-to-LDS load is in
     // flight (the last hand-over re-fetched a tile nobody reads).
     wait_vmcnt<0>();
+    asm volatile("" ::: "memory");
     __syncthreads();
     const int out_row0 = row0, out_col0 = col0;
     bf16_t* out_c = Ce;
@@ -945,8 +1042,6 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
             for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
       }
     }
-    const int next = tile + tile_step;
-    const bool has_next = next < tile_end;
     if (has_next) {
       // the next tile's first loads fly while this tile is written out
       set_tile(next);
@@ -1008,331 +1103,8 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
     }
     if (!has_next) break;
     tile = next;
+    ++round;
     prologue_tail();   // the staging area is free again
-  }
-}
-
-// ---------------------------------------------------------------------------
-// 128 x 256 tiles with TWO blocks resident per compute unit.
-//
-// The 256 x 256 kernel above owns a compute unit: its eight wavefronts meet at
-// one barrier per K tile and write their tile out together, and while they do
-// the matrix pipes of the unit have nothing else to run.  Here a block is four
-// wavefronts (one per SIMD) on a 128 x 256 tile with a K step of 32: three
-// slots each for the token tile (8 KB) and the weight tile (16 KB) are 72 KB,
-// so two blocks share a unit's LDS and its SIMDs, each SIMD holding one
-// wavefront of either block.  The two blocks run on their own: one block's
-// hand-over barrier, its tile's first loads and its store burst fall into the
-// other's K loop.  What that costs is operand traffic -- a 128 x 256 tile
-// loads 1.5 times the bytes per multiply-add of a 256 x 256 one -- so it pays
-// where the tile's prologue and epilogue weigh (short reductions, few tiles
-// per unit) rather than where the chip's power limit is what binds.
-//
-// A wavefront owns 128 x 64 of the tile (4 x 2 MFMA tiles, as in the kernel
-// above).  LDS rows are 64 bytes; one load instruction fills 16 rows, lane l
-// the 16-byte position l % 4 of row l / 4, with the chunk
-// (l % 4) ^ ((row >> 2) & 3) of that row: sixteen consecutive rows read at one
-// logical chunk then touch sixteen distinct 16-byte columns of a 256-byte
-// window.  Per K tile a wavefront issues 2 token and 4 weight loads, three on
-// each of its two MFMA steps, for the tile two ahead (its slot was last read
-// one tile ago, before the previous hand-over barrier); the hand-over waits
-// with vmcnt(3): the next tile has landed, the three loads just issued fly on.
-// ---------------------------------------------------------------------------
-struct DuoCfg {
-  static constexpr int BM = 128, BN = 256, BK = 32, WAVES = 4;
-  static constexpr int THREADS = 64 * WAVES;
-  static constexpr int TM = BM / 32, TN = (BN / WAVES) / 32;   // 4 x 2
-  static constexpr int ROW_BYTES = BK * 2;
-  static constexpr int A_INSTR = (BM / 16) / WAVES, B_INSTR = (BN / 16) / WAVES;
-  static constexpr int A_BYTES = BM * ROW_BYTES, B_BYTES = BN * ROW_BYTES;
-  static constexpr int SLOTS = 3;
-  static constexpr int B_BASE = SLOTS * A_BYTES;
-  static constexpr size_t LDS_BYTES = (size_t)SLOTS * (A_BYTES + B_BYTES);
-  static_assert(A_INSTR == 2 && B_INSTR == 4, "load schedule assumes 2 + 4");
-  static_assert(2 * LDS_BYTES <= 160 * 1024, "two blocks per compute unit");
-};
-
-template <bool RELU, bool GATHER>
-__global__ __launch_bounds__(DuoCfg::THREADS, 2) void grouped_gemm_bf16_duo_kernel(
-    const bf16_t* __restrict__ A, const bf16_t* __restrict__ B,
-    bf16_t* __restrict__ Cout, int R, int N, int K, int tiles_m, int tiles_n,
-    int total_tiles, const int32_t* __restrict__ row_map,
-    const bf16_t* __restrict__ zero_row) {
-  using Cfg = DuoCfg;
-  constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK;
-  extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
-
-  // Persistent blocks, two per compute unit; block b runs on XCD b % 8 and the
-  // blocks of an XCD hold consecutive logical tiles (see the kernel above).
-  const int nblk = gridDim.x;
-  int tile = blockIdx.x;
-  if ((nblk & 7) == 0) tile = (blockIdx.x & 7) * (nblk >> 3) + (blockIdx.x >> 3);
-  if (tile >= total_tiles) return;
-
-  const int tid = threadIdx.x;
-  const int lane = tid & 63;
-  const int wave = tid >> 6;
-  const int tiles_per_e = tiles_m * tiles_n;
-  const int nk = K / BK;
-
-  int row0, col0;
-  const bf16_t *Ae, *Be;
-  bf16_t* Ce;
-  typename std::conditional<GATHER, int64_t, int>::type a_off[Cfg::A_INSTR];
-  int b_off[Cfg::B_INSTR];
-  // rows this lane loads: instruction q = wave + WAVES j covers tile rows
-  // 16 q .. 16 q + 15
-  auto tile_coords = [&](int logical, int& e, int& tm, int& tn) {
-    e = logical / tiles_per_e;
-    const int rem = logical - e * tiles_per_e;
-    tn = rem / tiles_m;
-    tm = rem - tn * tiles_m;
-    if (tiles_m > 16 && (tiles_m & 15) == 0 && (tiles_n & 3) == 0) {
-      // many row tiles: 64 consecutive logical tiles (what an XCD holds) form
-      // a block of 16 row tiles x 4 column tiles
-      const int sup = rem >> 6, within = rem & 63;
-      const int per_row = tiles_n >> 2;
-      const int sm = sup / per_row, sn = sup - sm * per_row;
-      tm = sm * 16 + (within & 15);
-      tn = sn * 4 + (within >> 4);
-    }
-  };
-  // GATHER: the slot -> token map entries of this lane's rows of a tile, read
-  // a whole tile ahead so that the next tile's first loads do not wait for them
-  int next_src[Cfg::A_INSTR];
-  auto fetch_map = [&](int logical) {
-    if constexpr (GATHER) {
-      int e, tm, tn;
-      tile_coords(logical, e, tm, tn);
-#pragma unroll
-      for (int j = 0; j < Cfg::A_INSTR; ++j) {
-        const int row = (wave + Cfg::WAVES * j) * 16 + (lane >> 2);
-        next_src[j] = row_map[(int64_t)e * R + min(tm * BM + row, R - 1)];
-      }
-    }
-  };
-  auto set_tile = [&](int logical) {
-    int e, tm, tn;
-    tile_coords(logical, e, tm, tn);
-    row0 = tm * BM;
-    col0 = tn * BN;
-    Ae = GATHER ? A : A + (int64_t)e * R * K;
-    Be = B + (int64_t)e * N * K;
-    Ce = Cout + (int64_t)e * R * N;
-#pragma unroll
-    for (int j = 0; j < Cfg::A_INSTR; ++j) {
-      const int row = (wave + Cfg::WAVES * j) * 16 + (lane >> 2);
-      const int chunk = (lane & 3) ^ ((row >> 2) & 3);
-      if constexpr (GATHER) {
-        const int src = next_src[j];
-        a_off[j] = (src >= 0 ? (int64_t)src * K : (int64_t)(zero_row - A)) +
-                   chunk * 8;
-      } else {
-        a_off[j] = min(row0 + row, R - 1) * K + chunk * 8;
-      }
-    }
-#pragma unroll
-    for (int j = 0; j < Cfg::B_INSTR; ++j) {
-      const int row = (wave + Cfg::WAVES * j) * 16 + (lane >> 2);
-      const int chunk = (lane & 3) ^ ((row >> 2) & 3);
-      b_off[j] = min(col0 + row, N - 1) * K + chunk * 8;
-    }
-  };
-  // load j of token / weight tile kt into `slot`; kt past the end re-fetches
-  // the last tile into a slot nobody reads any more
-  auto load_a = [&](int kt, int slot, int j) {
-    kt = min(kt, nk - 1);
-    __builtin_amdgcn_global_load_lds(
-        (glb_void_t*)(Ae + kt * BK + a_off[j]),
-        (lds_void_t*)(smem_raw + slot * Cfg::A_BYTES +
-                      (wave + Cfg::WAVES * j) * 1024), 16, 0, 0);
-  };
-  auto load_b = [&](int kt, int slot, int j) {
-    kt = min(kt, nk - 1);
-    __builtin_amdgcn_global_load_lds(
-        (glb_void_t*)(Be + kt * BK + b_off[j]),
-        (lds_void_t*)(smem_raw + Cfg::B_BASE + slot * Cfg::B_BYTES +
-                      (wave + Cfg::WAVES * j) * 1024), 16, 0, 0);
-  };
-  // the six loads of a tile in the order the K loop issues them
-  auto load_n = [&](int kt, int slot, int n) {
-    if (n < 4) load_b(kt, slot, n);
-    else load_a(kt, slot, n - 4);
-  };
-  // first loads of a tile: everything but weight tile 1, whose slot the
-  // previous tile's epilogue still uses as staging area
-  auto prologue_head = [&]() {
-#pragma unroll
-    for (int j = 0; j < Cfg::A_INSTR; ++j) load_a(0, 0, j);
-#pragma unroll
-    for (int j = 0; j < Cfg::B_INSTR; ++j) load_b(0, 0, j);
-#pragma unroll
-    for (int j = 0; j < Cfg::A_INSTR; ++j) load_a(1, 1, j);
-  };
-  auto prologue_tail = [&]() {
-#pragma unroll
-    for (int j = 0; j < Cfg::B_INSTR; ++j) load_b(1, 1, j);
-  };
-
-  f32x16_t acc[Cfg::TM][Cfg::TN];
-  const int fr = lane & 31, fc = lane >> 5;
-  int a_frag[BK / 16], b_frag[BK / 16];
-#pragma unroll
-  for (int kk = 0; kk < BK / 16; ++kk) {
-    const int col = ((kk * 2 + fc) ^ ((fr >> 2) & 3)) * 16;
-    a_frag[kk] = fr * Cfg::ROW_BYTES + col;
-    b_frag[kk] = (wave * 64 + fr) * Cfg::ROW_BYTES + col;
-  }
-  bf16x8_t fa[2][Cfg::TM], fb[2][Cfg::TN];
-  auto read_frag = [&](int slot, int kk, int buf, int n) {
-    if (n < Cfg::TM)
-      fa[buf][n] = *reinterpret_cast<const bf16x8_t*>(
-          smem_raw + slot * Cfg::A_BYTES + a_frag[kk] + n * 32 * Cfg::ROW_BYTES);
-    else
-      fb[buf][n - Cfg::TM] = *reinterpret_cast<const bf16x8_t*>(
-          smem_raw + Cfg::B_BASE + slot * Cfg::B_BYTES + b_frag[kk] +
-          (n - Cfg::TM) * 32 * Cfg::ROW_BYTES);
-  };
-  auto mfma = [&](int buf, int n) {
-    const int i = n / Cfg::TN, j = n % Cfg::TN;
-    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fb[buf][j], fa[buf][i],
-                                                        acc[i][j], 0, 0, 0);
-  };
-  auto fence = [&]() { __builtin_amdgcn_sched_barrier(0); };
-  // fragment reads in the order the MFMAs first need them: a0 b0 b1 a1 a2 a3
-  constexpr int RD[6] = {0, Cfg::TM, Cfg::TM + 1, 1, 2, 3};
-
-  int slot = 0;   // kt % 3
-  auto k_tile = [&](int kt, auto last_tag) {
-    constexpr bool LAST = decltype(last_tag)::value;
-    const int s1 = slot == 2 ? 0 : slot + 1;      // slot of tile kt + 1
-    const int s2 = s1 == 2 ? 0 : s1 + 1;          // of tile kt + 2 (= kt - 1)
-    // step 0: the fragments of step 1, loads 0-2 of tile kt + 2
-    fence();
-    read_frag(slot, 1, 1, RD[0]);
-    read_frag(slot, 1, 1, RD[1]);
-    mfma(0, 0); fence();
-    read_frag(slot, 1, 1, RD[2]);
-    mfma(0, 1); fence();
-    if (!LAST) load_n(kt + 2, s2, 0);
-    mfma(0, 2); fence();
-    read_frag(slot, 1, 1, RD[3]);
-    mfma(0, 3); fence();
-    read_frag(slot, 1, 1, RD[4]);
-    mfma(0, 4); fence();
-    if (!LAST) load_n(kt + 2, s2, 1);
-    mfma(0, 5); fence();
-    read_frag(slot, 1, 1, RD[5]);
-    mfma(0, 6); fence();
-    if (!LAST) load_n(kt + 2, s2, 2);
-    mfma(0, 7); fence();
-    if (!LAST) {
-      // step 1 behind the hand-over: this lane holds the step's fragments
-      // (lgkmcnt 0) and everything but the three loads just issued has landed
-      __builtin_amdgcn_s_waitcnt((3 & 15) | (0 << 8) | (7 << 4));
-      asm volatile("" ::: "memory");
-      __builtin_amdgcn_s_barrier();
-      asm volatile("" ::: "memory");
-      fence();
-#pragma unroll
-      for (int n = 0; n < 6; ++n) {
-        read_frag(s1, 0, 0, RD[n]);
-        if (n >= 3) load_n(kt + 2, s2, n);
-        mfma(1, n); fence();
-      }
-      mfma(1, 6); fence();
-      mfma(1, 7); fence();
-    } else {
-#pragma unroll
-      for (int n = 0; n < 8; ++n) mfma(1, n);
-    }
-    slot = s1;
-  };
-
-  // Epilogue staging: two passes of 64 output rows in weight slots 1 and 2
-  // (32 KB), rows of 512 bytes with 16-byte chunk c of row r at c ^ (r & 31).
-  constexpr int EPI_ROWS = 64;
-  constexpr int EPI_ROW_BYTES = BN * 2;
-  constexpr int EPI_BASE = Cfg::B_BASE + Cfg::B_BYTES;
-  static_assert(EPI_BASE + EPI_ROWS * EPI_ROW_BYTES <= (int)Cfg::LDS_BYTES,
-                "epilogue staging exceeds the ring");
-  unsigned char* Cs = smem_raw + EPI_BASE;
-  const int m_l = lane & 31;
-  const int half = lane >> 5;
-  constexpr int CPR_C = BN / 8;
-
-  const int tile_step = nblk;
-  fetch_map(tile);
-  set_tile(tile);
-  prologue_head();
-  prologue_tail();
-  for (;;) {
-    const int next = tile + tile_step;
-    const bool has_next = next < total_tiles;
-    // (always issued, so that the number of loads in flight below is fixed)
-    fetch_map(min(next, total_tiles - 1));
-#pragma unroll
-    for (int i = 0; i < Cfg::TM; ++i)
-#pragma unroll
-      for (int j = 0; j < Cfg::TN; ++j)
-#pragma unroll
-        for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
-    // K tile 0 has landed: token tile 1, weight tile 1 (2 + 4 loads) and, with
-    // GATHER, the two map entries of the next tile may still be in flight
-    wait_vmcnt<GATHER ? 8 : 6>();
-    asm volatile("" ::: "memory");
-    __builtin_amdgcn_s_barrier();
-    asm volatile("" ::: "memory");
-#pragma unroll
-    for (int n = 0; n < 6; ++n) read_frag(0, 0, 0, RD[n]);
-    slot = 0;
-    for (int kt = 0; kt + 1 < nk; ++kt) k_tile(kt, std::false_type{});
-    k_tile(nk - 1, std::true_type{});
-
-    wait_vmcnt<0>();
-    __syncthreads();
-    const int out_row0 = row0, out_col0 = col0;
-    bf16_t* out_c = Ce;
-    if (has_next) {
-      set_tile(next);
-      prologue_head();
-    }
-#pragma unroll
-    for (int pass = 0; pass < 2; ++pass) {
-#pragma unroll
-      for (int ii = 0; ii < 2; ++ii) {
-        const int i = pass * 2 + ii;
-        const int srow = ii * 32 + m_l;
-#pragma unroll
-        for (int j = 0; j < Cfg::TN; ++j) {
-#pragma unroll
-          for (int q = 0; q < 4; ++q) {
-            const int chunk = (wave * 64 + j * 32 + 8 * q) / 8;
-            uint2 v;
-            v.x = pack2_bf16(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], RELU);
-            v.y = pack2_bf16(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3], RELU);
-            *reinterpret_cast<uint2*>(Cs + srow * EPI_ROW_BYTES +
-                                      ((chunk ^ m_l) * 16) + half * 8) = v;
-          }
-        }
-      }
-      __syncthreads();
-#pragma unroll
-      for (int c = tid; c < EPI_ROWS * CPR_C; c += Cfg::THREADS) {
-        const int srow = c / CPR_C, chunk = c % CPR_C;
-        const int grow = out_row0 + pass * 64 + srow;
-        const int gcol = out_col0 + chunk * 8;
-        if (grow < R && gcol < N) {
-          const u32x4_t v = *reinterpret_cast<const u32x4_t*>(
-              Cs + srow * EPI_ROW_BYTES + ((chunk ^ (srow & 31)) * 16));
-          *reinterpret_cast<u32x4_t*>(out_c + (int64_t)grow * N + gcol) = v;
-        }
-      }
-      __syncthreads();
-    }
-    if (!has_next) break;
-    tile = next;
-    prologue_tail();
   }
 }
 
@@ -1944,85 +1716,35 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
     MOE_CHECK_LAUNCH("expert_ffn (mfma, masked result)");
     return 0;
   }
+  // an expert's last row tile is partly empty: the instantiation that skips
+  // its empty 32-row pieces
+  const bool tails = R % Cfg::BM != 0;
+#define MOE_RING_PLAIN(RELU_, GATHER_, TAILS_)                                 \
+  do {                                                                         \
+    auto k = grouped_gemm_bf16_ring_kernel<RELU_, GATHER_, false, false,       \
+                                           false, TAILS_>;                     \
+    MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);                                          \
+    k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(                           \
+        A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, row_map, zero_row,     \
+        nullptr, nullptr, nullptr, 1.0f);                                      \
+  } while (0)
+#define MOE_RING_PLAIN_T(RELU_, GATHER_)                                       \
+  do {                                                                         \
+    if (tails) MOE_RING_PLAIN(RELU_, GATHER_, true);                           \
+    else MOE_RING_PLAIN(RELU_, GATHER_, false);                                \
+  } while (0)
   if (row_map != nullptr) {
-    if (relu) {
-      auto k = grouped_gemm_bf16_ring_kernel<true, true>;
-      MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
-      k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
-          A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, row_map, zero_row,
-          nullptr, nullptr, nullptr, 1.0f);
-    } else {
-      auto k = grouped_gemm_bf16_ring_kernel<false, true>;
-      MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
-      k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
-          A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, row_map, zero_row,
-          nullptr, nullptr, nullptr, 1.0f);
-    }
+    if (relu) MOE_RING_PLAIN_T(true, true);
+    else MOE_RING_PLAIN_T(false, true);
     MOE_CHECK_LAUNCH("expert_ffn (mfma, gathered rows)");
     return 0;
   }
-  if (relu) {
-    auto k = grouped_gemm_bf16_ring_kernel<true, false>;
-    MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
-    k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
-        A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr,
-        nullptr, nullptr, nullptr, 1.0f);
-  } else {
-    auto k = grouped_gemm_bf16_ring_kernel<false, false>;
-    MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
-    k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
-        A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, nullptr, nullptr,
-        nullptr, nullptr, nullptr, 1.0f);
-  }
+  if (relu) MOE_RING_PLAIN_T(true, false);
+  else MOE_RING_PLAIN_T(false, false);
+#undef MOE_RING_PLAIN_T
+#undef MOE_RING_PLAIN
   MOE_CHECK_LAUNCH("expert_ffn (mfma, spread direct-to-LDS loads)");
   return 0;
-}
-
-// The 128 x 256 kernel with two blocks per compute unit; row_map / zero_row as
-// in launch_ring.
-static int launch_duo(const bf16_t* A, const bf16_t* B, bf16_t* C, int E, int R,
-                      int N, int K, bool relu, hipStream_t st,
-                      const int32_t* row_map = nullptr,
-                      const bf16_t* zero_row = nullptr) {
-  using Cfg = DuoCfg;
-  const int tiles_m = (R + Cfg::BM - 1) / Cfg::BM;
-  const int tiles_n = (N + Cfg::BN - 1) / Cfg::BN;
-  const int64_t tiles = (int64_t)tiles_m * tiles_n * E;
-  MOE_REQUIRE(tiles <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
-              "expert_ffn: too many tiles (%lld)", (long long)tiles);
-  const int cus = compute_units();
-  if (cus == 0) return MESH_MOE_E_HIP;
-  const unsigned blocks = (unsigned)(tiles < 2 * cus ? tiles : 2 * cus);
-#define MOE_DUO(RELU_, GATHER_)                                                \
-  do {                                                                         \
-    auto k = grouped_gemm_bf16_duo_kernel<RELU_, GATHER_>;                     \
-    MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);                                          \
-    k<<<blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(                           \
-        A, B, C, R, N, K, tiles_m, tiles_n, (int)tiles, row_map, zero_row);    \
-  } while (0)
-  if (row_map != nullptr) {
-    if (relu) MOE_DUO(true, true);
-    else MOE_DUO(false, true);
-  } else {
-    if (relu) MOE_DUO(true, false);
-    else MOE_DUO(false, false);
-  }
-#undef MOE_DUO
-  MOE_CHECK_LAUNCH("expert_ffn (mfma, two blocks per compute unit)");
-  return 0;
-}
-
-// EXPERIMENT: MESH_MOE_GEMM_VARIANT=duo|ring forces the kernel of the plain and
-// gathered forward GEMMs.
-static int gemm_variant_override() {
-  static int v = -1;
-  if (v < 0) {
-    const char* s = getenv("MESH_MOE_GEMM_VARIANT");
-    v = 0;
-    if (s && !strcmp(s, "duo")) v = 1;
-    if (s && !strcmp(s, "ring")) v = 2;
-  }
-  return v;
 }
 
 static int launch_f32_mfma(const float* A, const float* B, float* C, int E,
@@ -2109,8 +1831,6 @@ static int grouped_gemm(const void* A, const void* B, void* C, int E, int R,
         rc = launch_ring(a, b, c, E, R, N, K, false, st, nullptr, nullptr,
                          (const bf16_t*)relu_mask_src, nullptr, mask_scale);
         *mask_applied = rc == 0;
-      } else if (gemm_variant_override() == 1) {
-        rc = launch_duo(a, b, c, E, R, N, K, relu, st);
       } else {
         rc = launch_ring(a, b, c, E, R, N, K, relu, st);
       }
@@ -2357,11 +2077,8 @@ extern "C" int mesh_moe_dispatched_expert_ffn(
       idx, pos, gate, kept, map, (int64_t)G * S, S, C, rows);
   MOE_CHECK_LAUNCH("dispatched_expert_ffn (slot map)");
   const bool relu = activation == MESH_MOE_ACT_RELU;
-  int rc = gemm_variant_override() == 1
-               ? launch_duo((const bf16_t*)x, (const bf16_t*)wi_packed,
-                            (bf16_t*)h, E, R, H, M, relu, st, map, zero_row)
-               : launch_ring((const bf16_t*)x, (const bf16_t*)wi_packed,
-                             (bf16_t*)h, E, R, H, M, relu, st, map, zero_row);
+  int rc = launch_ring((const bf16_t*)x, (const bf16_t*)wi_packed, (bf16_t*)h,
+                       E, R, H, M, relu, st, map, zero_row);
   if (rc != 0) return rc;
   if (!relu && activation != MESH_MOE_ACT_LINEAR) {
     rc = launch_activation(h, (int64_t)E * R * H, activation, dtype, st);

@@ -192,7 +192,13 @@ def test_dispatch_combine(hip, act_dtype, shape):
                                    # 256-row tiles with 1, 2, 3 and 5 K tiles,
                                    # ragged rows and a ragged last column tile
                                    (2, 512, 64, 256, 256), (1, 256, 128, 320, 256),
-                                   (2, 700, 192, 256, 512)])
+                                   (2, 700, 192, 256, 512),
+                                   # last row tiles with 5, 4, 8 and 1 of their
+                                   # eight 32-row pieces in use (the kernel
+                                   # skips the others), rows not a multiple
+                                   # of 32
+                                   (2, 400, 128, 512, 256), (3, 640, 64, 256, 256),
+                                   (1, 510, 128, 256, 256), (2, 770, 64, 256, 256)])
 def test_expert_ffn(hip, act_dtype, activation, shape):
   e, rows, m, hdim, n = shape
   rng = np.random.default_rng(29)
@@ -968,7 +974,11 @@ def test_slot_dispatch_combine(hip, act_dtype):
 
 @pytest.mark.parametrize("shape", [(4, 512, 8, 128, 256, 512, 256),
                                    (2, 1024, 16, 128, 128, 384, 128),
-                                   (5, 300, 4, 180, 64, 256, 64)])
+                                   (5, 300, 4, 180, 64, 256, 64),
+                                   # 400 and 640 rows per expert: a last row
+                                   # tile of 144 / 128 rows
+                                   (5, 512, 8, 80, 128, 512, 256),
+                                   (16, 256, 8, 40, 64, 256, 256)])
 def test_dispatched_expert_ffn_equals_two_calls(hip, shape):
   """The dispatch folded into the first expert GEMM gives bit-identical h-free
   outputs to mesh_moe_dispatch + mesh_moe_expert_ffn (same kernel, same
