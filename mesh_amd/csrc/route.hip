@@ -483,8 +483,8 @@ __device__ __forceinline__ void gate_select_tile(
 // ---------------------------------------------------------------------------
 template <int NT, typename IT>
 __device__ __forceinline__ void gate_select_acc_tile(
-    const float (&x)[NT][16], float* tile, float* isone, int ld, int g, int blk,
-    int t0, const IT* __restrict__ importance,
+    const float (&xin)[NT][16], float* tile, float* isone, int ld, int g,
+    int blk, int t0, const IT* __restrict__ importance,
     const float* __restrict__ second_uniform, const GateParams& p,
     int32_t* __restrict__ idx, int32_t* __restrict__ pos,
     float* __restrict__ gate, uint8_t* __restrict__ kept,
@@ -498,30 +498,97 @@ __device__ __forceinline__ void gate_select_acc_tile(
   const bool sw = p.router == ROUTER_SWITCH;
   float* row = tile + tok * ld;
   const int64_t t = (int64_t)g * S + t0 + tok;
+  // As the matrix cores leave them, register group (j, q) of the lower lane of
+  // a token's pair holds experts 32 j + 8 q + 0..3 and the upper lane's
+  // + 4..7: a sum in expert order changes lanes after every four experts.
+  // With an even number of 32-expert blocks the pair first trades registers
+  // (v_permlane32_swap: the upper half of one register against the lower half
+  // of another), after which the lower lane holds the whole of block 2 jp in
+  // its groups (2 jp, q), (2 jp + 1, q) -- experts 8 q + 0..3 and 8 q + 4..7 --
+  // and the upper lane the whole of block 2 jp + 1: a sum in expert order then
+  // changes lanes once per 32 experts.
+  constexpr bool SWAPPED = NT % 2 == 0;
+  float x[NT][16];
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) x[j][i] = xin[j][i];
+  if constexpr (SWAPPED) {
+#pragma unroll
+    for (int jp = 0; jp < NT / 2; ++jp)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const auto sw2 = __builtin_amdgcn_permlane32_swap(
+            __float_as_uint(x[2 * jp][i]), __float_as_uint(x[2 * jp + 1][i]),
+            false, false);
+        x[2 * jp][i] = __uint_as_float(sw2[0]);
+        x[2 * jp + 1][i] = __uint_as_float(sw2[1]);
+      }
+  }
   // first expert of this lane's group (j, q); the group exists if it is < E
-  auto first = [&](int j, int q) { return j * 32 + 8 * q + 4 * half; };
+  auto first = [&](int j, int q) {
+    return SWAPPED ? ((j & ~1) + half) * 32 + 8 * q + 4 * (j & 1)
+                   : j * 32 + 8 * q + 4 * half;
+  };
+  // calls fn(j, q) for the lane's groups in ascending expert order
+  auto for_groups = [&](auto fn) {
+    if constexpr (SWAPPED) {
+#pragma unroll
+      for (int jp = 0; jp < NT / 2; ++jp)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          fn(2 * jp, q);
+          fn(2 * jp + 1, q);
+        }
+    } else {
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) fn(j, q);
+    }
+  };
   // the partner's candidate wins if it is larger, or equal with a lower index
   auto take_other = [&](float mine, int mi, float other, int oi) {
     return other > mine || (other == mine && oi < mi);
   };
   // a float32 sum over the experts in index order: the lanes of a pair take
-  // turns, the running value changing lanes after every group of four
+  // turns, the running value changing lanes when the next expert lives in the
+  // other lane
   auto ordered_sum = [&](const float (&v)[NT][16]) {
     float s = 0.f;
+    if constexpr (SWAPPED) {
 #pragma unroll
-    for (int j = 0; j < NT; ++j)
-#pragma unroll
-      for (int q = 0; q < 4; ++q) {
-        const bool mine = first(j, q) < E;
+      for (int jp = 0; jp < NT / 2; ++jp)
 #pragma unroll
         for (int hh = 0; hh < 2; ++hh) {
-          if (half == hh && mine) {
+          if (half == hh) {
 #pragma unroll
-            for (int r = 0; r < 4; ++r) s += v[j][4 * q + r];
+            for (int q = 0; q < 4; ++q)
+#pragma unroll
+              for (int jj = 0; jj < 2; ++jj)
+                if (first(2 * jp + jj, q) < E) {
+#pragma unroll
+                  for (int r = 0; r < 4; ++r) s += v[2 * jp + jj][4 * q + r];
+                }
           }
           s = __shfl_xor(s, 32);
         }
-      }
+    } else {
+#pragma unroll
+      for (int j = 0; j < NT; ++j)
+#pragma unroll
+        for (int q = 0; q < 4; ++q) {
+          const bool mine = first(j, q) < E;
+#pragma unroll
+          for (int hh = 0; hh < 2; ++hh) {
+            if (half == hh && mine) {
+#pragma unroll
+              for (int r = 0; r < 4; ++r) s += v[j][4 * q + r];
+            }
+            s = __shfl_xor(s, 32);
+          }
+        }
+    }
     return __shfl(s, lane & 31);      // the lower lane holds the final value
   };
 
@@ -545,20 +612,18 @@ __device__ __forceinline__ void gate_select_acc_tile(
   const float neglse = -(logf(ssum) + m);                            // log + max
   float g1 = -1.f;
   int i1 = 0;
+  for_groups([&](int j, int q) {
+    if (first(j, q) < E) {
 #pragma unroll
-  for (int j = 0; j < NT; ++j)
-#pragma unroll
-    for (int q = 0; q < 4; ++q)
-      if (first(j, q) < E) {
-#pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float pe = expf(x[j][4 * q + r] + neglse);   // exp(log_softmax)
-          pr[j][4 * q + r] = pe;
-          if (pe > g1) { g1 = pe; i1 = first(j, q) + r; }    // first argmax
-        }
-        *reinterpret_cast<float4*>(row + first(j, q)) = make_float4(
-            pr[j][4 * q], pr[j][4 * q + 1], pr[j][4 * q + 2], pr[j][4 * q + 3]);
+      for (int r = 0; r < 4; ++r) {
+        const float pe = expf(x[j][4 * q + r] + neglse);   // exp(log_softmax)
+        pr[j][4 * q + r] = pe;
+        if (pe > g1) { g1 = pe; i1 = first(j, q) + r; }    // first argmax
       }
+      *reinterpret_cast<float4*>(row + first(j, q)) = make_float4(
+          pr[j][4 * q], pr[j][4 * q + 1], pr[j][4 * q + 2], pr[j][4 * q + 3]);
+    }
+  });
   {
     const float og = __shfl_xor(g1, 32);
     const int oi = __shfl_xor(i1, 32);
@@ -570,17 +635,15 @@ __device__ __forceinline__ void gate_select_acc_tile(
     const float* cl = second_uniform + t * E;
     float best = -INFINITY;
     int bi = E;
+    for_groups([&](int j, int q) {
+      if (first(j, q) < E) {
+        const float4 c4 = *reinterpret_cast<const float4*>(cl + first(j, q));
+        const float cv[4] = {c4.x, c4.y, c4.z, c4.w};
 #pragma unroll
-    for (int j = 0; j < NT; ++j)
-#pragma unroll
-      for (int q = 0; q < 4; ++q)
-        if (first(j, q) < E) {
-          const float4 c4 = *reinterpret_cast<const float4*>(cl + first(j, q));
-          const float cv[4] = {c4.x, c4.y, c4.z, c4.w};
-#pragma unroll
-          for (int r = 0; r < 4; ++r)
-            if (bi == E || cv[r] > best) { best = cv[r]; bi = first(j, q) + r; }
-        }
+        for (int r = 0; r < 4; ++r)
+          if (bi == E || cv[r] > best) { best = cv[r]; bi = first(j, q) + r; }
+      }
+    });
     const float ob = __shfl_xor(best, 32);
     const int oi = __shfl_xor(bi, 32);
     if (take_other(best, bi, ob, oi)) bi = oi;
@@ -624,20 +687,18 @@ __device__ __forceinline__ void gate_select_acc_tile(
     // gates_without_top_1 = raw_gates * (1 - mask_1), in place; its first argmax
     float g2 = -1.f;
     int i2 = 0;
+    for_groups([&](int j, int q) {
+      if (first(j, q) < E) {
 #pragma unroll
-    for (int j = 0; j < NT; ++j)
-#pragma unroll
-      for (int q = 0; q < 4; ++q)
-        if (first(j, q) < E) {
-#pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const int e = first(j, q) + r;
-            const float keep = (sel1 && e == i1) ? 0.0f : 1.0f;
-            const float qv = pr[j][4 * q + r] * keep;
-            pr[j][4 * q + r] = qv;
-            if (qv > g2) { g2 = qv; i2 = e; }
-          }
+        for (int r = 0; r < 4; ++r) {
+          const int e = first(j, q) + r;
+          const float keep = (sel1 && e == i1) ? 0.0f : 1.0f;
+          const float qv = pr[j][4 * q + r] * keep;
+          pr[j][4 * q + r] = qv;
+          if (qv > g2) { g2 = qv; i2 = e; }
         }
+      }
+    });
     {
       const float og = __shfl_xor(g2, 32);
       const int oi = __shfl_xor(i2, 32);
@@ -816,42 +877,48 @@ __device__ __forceinline__ bool arrive_is_last(unsigned long long* word,
 // Ranks of the block's choices.  ch [3][128] int16 in LDS as written by
 // gate_select_tile; wcnt [3][2][E] int32 in LDS.  Wavefront w ranks choice
 // w / 2 of tokens 64 (w % 2) ..; with `loss2` wavefronts 0 and 1 also count
-// the third array.  Writes pos (rank within the block) for competing choices,
-// 0 otherwise, and the block's counts to bcnt_blk [3][E].
+// the third array.  A lane's rank is the number of lower lanes of its
+// wavefront that name the same expert.  Writes pos (rank within the block)
+// for competing choices, 0 otherwise, and the block's counts to
+// bcnt_blk [3][E].
 __device__ __forceinline__ void gate_rank_tile(
     const int16_t* ch, int32_t* wcnt, int E, bool loss2, int64_t tok0,
     int32_t* __restrict__ pos, int32_t* __restrict__ bcnt_blk) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int c = wave >> 1, half = wave & 1;
-  const int mine = ch[c * 128 + half * 64 + lane];
-  int rank = 0;
-  for (int e0 = 0; e0 < E; e0 += 64) {
-    int cnt = 0;   // lane l: choosers of expert e0 + l in this wavefront
-    const int n = min(64, E - e0);
-    // branch-free: the selects below are cheaper than a taken branch
-#pragma unroll 8
-    for (int j = 0; j < n; ++j) {
-      const bool hit = mine == e0 + j;
-      const unsigned long long m = __ballot(hit);
-      const int below = (int)__builtin_amdgcn_mbcnt_hi(
-          (unsigned)(m >> 32), __builtin_amdgcn_mbcnt_lo((unsigned)m, 0u));
-      rank = hit ? below : rank;
-      cnt = lane == j ? (int)__popcll(m) : cnt;
+  // bits an expert id has
+  const int nbits = 32 - __builtin_clz((unsigned)max(E - 1, 1));
+  // The lanes of this wavefront that name the same expert as this lane, from
+  // one ballot per bit of the id (instead of one per expert): a lane keeps the
+  // lanes whose bit equals its own.  id < 0: not competing, matches nobody.
+  auto same_choice = [&](int id) {
+    unsigned long long match = __ballot(id >= 0);
+    for (int b = 0; b < nbits; ++b) {
+      const bool bit = ((id >> b) & 1) != 0;
+      const unsigned long long mb = __ballot(bit);
+      match &= bit ? mb : ~mb;
     }
-    if (lane < n) wcnt[(c * 2 + half) * E + e0 + lane] = cnt;
-  }
+    return id >= 0 ? match : 0ull;
+  };
+  const unsigned long long before =
+      lane == 0 ? 0ull : (~0ull >> (64 - lane));      // the lanes below this one
+  auto clear_counts = [&](int32_t* dst) {
+    for (int e = lane; e < E; e += 64) dst[e] = 0;
+  };
+  const int mine = ch[c * 128 + half * 64 + lane];
+  int32_t* my_cnt = wcnt + (c * 2 + half) * E;
+  clear_counts(my_cnt);
+  const unsigned long long match = same_choice(mine);
+  int rank = (int)__popcll(match & before);
+  // the first lane of every expert's choosers writes the expert's count (LDS
+  // keeps a wavefront's writes in program order: after the clearing)
+  if (mine >= 0 && rank == 0) my_cnt[mine] = (int)__popcll(match);
   if (loss2 && c == 0) {
     const int third = ch[2 * 128 + half * 64 + lane];
-    for (int e0 = 0; e0 < E; e0 += 64) {
-      int cnt = 0;
-      const int n = min(64, E - e0);
-#pragma unroll 8
-      for (int j = 0; j < n; ++j) {
-        const unsigned long long m = __ballot(third == e0 + j);
-        cnt = lane == j ? (int)__popcll(m) : cnt;
-      }
-      if (lane < n) wcnt[(4 + half) * E + e0 + lane] = cnt;
-    }
+    int32_t* cnt3 = wcnt + (4 + half) * E;
+    clear_counts(cnt3);
+    const unsigned long long m3 = same_choice(third);
+    if (third >= 0 && (m3 & before) == 0ull) cnt3[third] = (int)__popcll(m3);
   }
   __syncthreads();
   if (half == 1 && mine >= 0) rank += wcnt[(c * 2) * E + mine];
