@@ -740,8 +740,12 @@ __device__ __forceinline__ void gate_select_acc_tile(
     for (int i = tid; i < 4 * ncol; i += blockDim.x) {
       const int e = i % ncol, q4 = i / ncol;
       float acc = 0.f;
-      for (int r = q4 * (NTOK / 4); r < (q4 + 1) * (NTOK / 4); ++r)
-        acc += weighted ? tile[r * ld + e] * isone[r] : tile[r * ld + e];
+      // (the reads of a batch fly together; the additions keep their order)
+      const float* col = tile + q4 * (NTOK / 4) * ld + e;
+      const float* one = isone + q4 * (NTOK / 4);
+#pragma unroll 8
+      for (int r = 0; r < NTOK / 4; ++r)
+        acc += weighted ? col[r * ld] * one[r] : col[r * ld];
       colpart[q4 * ncol + e] = acc;
     }
     __syncthreads();
@@ -953,6 +957,7 @@ __device__ __forceinline__ void gate_group_tail(
       smem + (((size_t)nblk * E * 4 + 15) & ~(size_t)15));     // [3][E]
   float* prod = reinterpret_cast<float*>(tot + 3 * E);         // [2][E]
   float* misc = prod + 2 * E;                                  // [4]
+  int* last_group = reinterpret_cast<int*>(misc + 4);          // [1] (+ 3 pad)
   const int32_t* bc = ft.bcnt + (int64_t)g * nblk * 3 * E;
   const int64_t base = (int64_t)g * S;
   // Everything here comes from other compute units' stores, i.e. from memory,
@@ -984,7 +989,17 @@ __device__ __forceinline__ void gate_group_tail(
       }
     }
   };
-  load_records(tid);
+  // Loads return in the order they were issued: the per-block counts, which
+  // the prefixes below need first, go out before the (many more) record loads.
+  auto load_counts = [&](int i, int (&cv)[PB]) {
+    const int c = i / E, e = i - c * E;
+#pragma unroll
+    for (int b = 0; b < PB; ++b)
+      cv[b] = (i < 3 * E && b < nblk && (c < 2 || loss2))
+                  ? ld_dev(bc + ((int64_t)b * 3 + c) * E + e) : 0;
+  };
+  int cv0[PB];
+  load_counts(tid, cv0);
   // thread e < E sums column e of part1, threads E .. 2E-1 column e of part2
   // (second-place loss: E columns; switch: columns 0 and 1), in block order
   const int pcol = tid < E ? tid : tid - E;
@@ -997,14 +1012,28 @@ __device__ __forceinline__ void gate_group_tail(
     for (int b = 0; b < PB; ++b)
       pv[b] = b < nblk ? ld_dev(pcolumn + (int64_t)b * E) : 0.f;
   }
+  load_records(tid);
   // first slot of every block per expert: exclusive prefix over the blocks
   for (int i = tid; i < 3 * E; i += blockDim.x) {
     const int c = i / E, e = i - c * E;
     if (c == 2 && !loss2) { tot[i] = 0; continue; }
     uint16_t* pre = c == 0 ? pre1 : pre2;
+    int cv[PB];
+    if (i == tid) {
+#pragma unroll
+      for (int b = 0; b < PB; ++b) cv[b] = cv0[b];
+    } else {
+      load_counts(i, cv);
+    }
     int run = 0;
-#pragma unroll 16
-    for (int b = 0; b < nblk; ++b) {
+#pragma unroll
+    for (int b = 0; b < PB; ++b) {
+      if (b < nblk) {
+        if (c < 2) pre[b * E + e] = (uint16_t)run;
+        run += cv[b];
+      }
+    }
+    for (int b = PB; b < nblk; ++b) {
       const int v = ld_dev(bc + ((int64_t)b * 3 + c) * E + e);
       if (c < 2) pre[b * E + e] = (uint16_t)run;
       run += v;
@@ -1019,6 +1048,41 @@ __device__ __forceinline__ void gate_group_tail(
     for (int b = PB; b < nblk; ++b) psum += ld_dev(pcolumn + (int64_t)b * E);
   }
   __syncthreads();
+  // Per-expert outputs and the group's share of the balancing loss come first:
+  // the group's arrival at the call's counter then travels while the records
+  // are rewritten.
+  if (sums2) {
+    if (sw) misc[pcol] = psum;
+    else prod[E + pcol] = psum;      // proxy of the second-place loss, for now
+  }
+  __syncthreads();
+  if (tid < E) {
+    const int t1 = tot[tid], t2 = tot[E + tid];
+    const int k1 = min(t1, C);
+    ft.fill[(int64_t)g * E + tid] = k1 + min(t2, C - k1);
+    const float inv_s = (float)(1.0 / (double)S);
+    const int dens = sw ? tot[2 * E + tid] : t1;
+    prod[tid] = (psum * inv_s) * ((float)dens * inv_s);
+    if (loss2 && !sw)
+      prod[E + tid] = (prod[E + tid] * inv_s) * ((float)tot[2 * E + tid] * inv_s);
+  }
+  __syncthreads();
+  if (tid == 0) {
+    float s1 = 0.f, s2 = 0.f;
+    for (int k = 0; k < E; ++k) s1 += prod[k];
+    if (loss2 && !sw)
+      for (int k = 0; k < E; ++k) s2 += prod[E + k];
+    float* gs = ft.gsum + (int64_t)g * GSUM;
+    st_dev(gs + 0, s1);
+    st_dev(gs + 1, s2);
+    st_dev(gs + 2, sw ? (E > 1 ? misc[1] : 0.f) : 0.f);
+    st_dev(gs + 3, sw ? misc[0] : 0.f);
+    st_dev(ft.gctr + g, 0ull);
+    wait_stores();
+    const bool last = arrive_is_last(ft.fctr, ft.call, (unsigned)p.G);
+    if (last) st_dev(ft.fctr, 0ull);
+    *last_group = last ? 1 : 0;
+  }
   for (int s0 = tid; s0 < S; s0 += (int)blockDim.x * U) {
     if (s0 != tid) load_records(s0);
 #pragma unroll
@@ -1056,37 +1120,20 @@ __device__ __forceinline__ void gate_group_tail(
       }
     }
   }
-  // per-expert outputs and the group's share of the balancing loss
-  if (sums2) {
-    if (sw) misc[pcol] = psum;
-    else prod[E + pcol] = psum;      // proxy of the second-place loss, for now
-  }
+  // The last group to finish turns the groups' terms into the loss: all
+  // threads fetch them (one round trip instead of one per group), one thread
+  // adds them in group order.
   __syncthreads();
-  if (tid < E) {
-    const int t1 = tot[tid], t2 = tot[E + tid];
-    const int k1 = min(t1, C);
-    ft.fill[(int64_t)g * E + tid] = k1 + min(t2, C - k1);
-    const float inv_s = (float)(1.0 / (double)S);
-    const int dens = sw ? tot[2 * E + tid] : t1;
-    prod[tid] = (psum * inv_s) * ((float)dens * inv_s);
-    if (loss2 && !sw)
-      prod[E + tid] = (prod[E + tid] * inv_s) * ((float)tot[2 * E + tid] * inv_s);
-  }
-  __syncthreads();
-  if (tid == 0) {
-    float s1 = 0.f, s2 = 0.f;
-    for (int k = 0; k < E; ++k) s1 += prod[k];
-    if (loss2 && !sw)
-      for (int k = 0; k < E; ++k) s2 += prod[E + k];
-    float* gs = ft.gsum + (int64_t)g * GSUM;
-    st_dev(gs + 0, s1);
-    st_dev(gs + 1, s2);
-    st_dev(gs + 2, sw ? (E > 1 ? misc[1] : 0.f) : 0.f);
-    st_dev(gs + 3, sw ? misc[0] : 0.f);
-    st_dev(ft.gctr + g, 0ull);
-    wait_stores();
-    if (arrive_is_last(ft.fctr, ft.call, (unsigned)p.G)) {
-      st_dev(ft.fctr, 0ull);
+  const bool finishes_call = *last_group != 0;
+  __syncthreads();                 // (the staging below overwrites the flag)
+  if (finishes_call) {
+    float* stage = reinterpret_cast<float*>(smem);     // the prefixes are done with
+    const int n = p.G * GSUM;
+    if (n <= 8192) {
+      for (int i = tid; i < n; i += (int)blockDim.x) stage[i] = ld_dev(ft.gsum + i);
+      __syncthreads();
+      if (tid == 0) gate_loss_value<false>(p, stage, ft.loss);
+    } else if (tid == 0) {
       gate_loss_value<true>(p, ft.gsum, ft.loss);
     }
   }
@@ -1716,7 +1763,7 @@ static GateParams make_switch_params(int G, int S, int E, int C,
 // LDS the last block of a group needs (gate_group_tail).
 static size_t fused_tail_lds_bytes(int nblk, int E) {
   return (((size_t)nblk * E * 4 + 15) & ~(size_t)15) +
-         sizeof(int32_t) * 3 * (size_t)E + sizeof(float) * (2 * (size_t)E + 4);
+         sizeof(int32_t) * 3 * (size_t)E + sizeof(float) * (2 * (size_t)E + 8);
 }
 
 template <int NT, typename IT>
