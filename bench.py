@@ -27,7 +27,7 @@ if ROOT not in sys.path:
 # (scaled by what the same counters read for a 1 GiB copy: 2.0 and 1.0; the
 # summary with the commands is profiles/hbm_traffic_cfg4_pmc.txt).  Mean of the
 # wi and wo launches.  Measured offline: the counters cannot be read from here.
-MEASURED_GEMM_TRAFFIC_BYTES = {4: 33.3e9}
+MEASURED_GEMM_TRAFFIC_BYTES = {4: 34.0e9}
 
 # MI355X published peaks
 HBM_PEAK_GBS = 8000.0
