@@ -348,6 +348,7 @@ constexpr int DBM_TOK = 32, DBM_COLS = 256, DBM_MAX_E = 128;
 constexpr int DBM_LD = DBM_COLS + 4;     // floats per LDS row of the share
 typedef __attribute__((ext_vector_type(8))) __bf16 dbm_bf16x8_t;
 typedef float dbm_f32x16_t __attribute__((ext_vector_type(16)));
+typedef uint32_t dbm_u32x4_t __attribute__((ext_vector_type(4)));
 
 // LDS bytes: [kernel rows | share] then the d(logits) rows
 static size_t dbm_lds_bytes(int E) {
@@ -356,12 +357,21 @@ static size_t dbm_lds_bytes(int E) {
   return (wbytes > sbytes ? wbytes : sbytes) + (size_t)DBM_TOK * (E * 4 + 16);
 }
 
+// Block barrier that waits for this wavefront's LDS accesses only.
+__device__ __forceinline__ void dbm_lds_barrier() {
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
 // (Four token tiles per block with the kernel rows kept in registers and the
 // next tile's loads in flight: 0.60 against 0.50 ms.)
 // SLOT: the rows of a token are named by the token -> slot table of the
 // expert-selection router (tok_slot [T, E] int16, -1 = not chosen by that
 // expert; any number of rows per token) instead of the per-token record.
-template <int KS, bool SLOT = false>
+// COMPACT: the rows lie in the compacted order (row_offsets given).
+template <int KS, bool SLOT = false, bool COMPACT = false>
 __global__ __launch_bounds__(256) void dispatch_backward_mfma_kernel(
     const bf16_t* __restrict__ dxe, const int32_t* __restrict__ idx,
     const int32_t* __restrict__ pos, const float* __restrict__ gate,
@@ -392,80 +402,113 @@ __global__ __launch_bounds__(256) void dispatch_backward_mfma_kernel(
   constexpr int RP = DBM_TOK / 8;
   const uint4 z = make_uint4(0, 0, 0, 0);
 
-  // the loads of the token tile: its d(logits) rows (16-byte pieces,
-  // consecutive threads consecutive pieces) and the rows of d(expert_in) this
-  // lane adds in phase 2 (token rows wave * 8 + 2 j + half, 8 columns from
-  // column 8 l32 of the tile)
-  auto load_tile = [&](float4 (&dv)[DP], uint4 (&v)[RP][2]) {
-#pragma unroll
-    for (int i = 0; i < DP; ++i) {
-      const int p = tid + 256 * i;
-      const int64_t t = t0 + p / DPR;
-      dv[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-      if (p < DBM_TOK * DPR && t < T_tokens)
-        dv[i] = reinterpret_cast<const float4*>(dlogits + t0 * E)[p];
-    }
+  // Issue order (vmcnt retires in order, and nothing below waits for more
+  // than it needs): the tokens' records, the kernel rows, the d(logits) rows,
+  // and last the rows of d(expert_in), which stay in flight through the whole
+  // matrix phase.  Every load is unconditional -- for a row that is not kept
+  // slot 0 is read and dropped -- so the code up to phase 2 is one basic block
+  // and the waits count exactly.  The barriers wait for LDS only
+  // (__syncthreads() would wait for the rows as well).
+  // Records: token rows wave * 8 + 2 j + half, both choices of every array in
+  // one load each.
+  uint16_t kept2[RP];
+  int2 idx2[RP], pos2[RP];
+  float2 gate2[RP];
+  if constexpr (!SLOT) {
 #pragma unroll
     for (int j = 0; j < RP; ++j) {
-      const int64_t t = t0 + wave * 8 + 2 * j + half;
-      v[j][0] = z;
-      v[j][1] = z;
-      if (SLOT || t >= T_tokens) continue;
-      // the token's record in one round trip (both choices of every array)
-      const uint16_t kept2 = *reinterpret_cast<const uint16_t*>(kept + t * 2);
-      const int2 idx2 = *reinterpret_cast<const int2*>(idx + t * 2);
-      const int2 pos2 = *reinterpret_cast<const int2*>(pos + t * 2);
-      const float2 gate2 = *reinterpret_cast<const float2*>(gate + t * 2);
-#pragma unroll
-      for (int k = 0; k < 2; ++k) {
-        if (((kept2 >> (8 * k)) & 0xff) &&
-            round_to<bf16_t>(k ? gate2.y : gate2.x) != 0.0f) {
-          const int64_t e = k ? idx2.y : idx2.x;
-          const int64_t slot =
-              (row_offsets == nullptr ? (e * G + g) * C
-                                      : e * G * C + row_offsets[e * G + g]) +
-              (k ? pos2.y : pos2.x);
-          v[j][k] = load_streaming(
-              reinterpret_cast<const uint4*>(dxe + slot * M + m0) + l32);
-        }
-      }
-    }
-  };
-
-  // ---- the kernel rows: global -> LDS -> this lane's operands
-  uint4 afrag[2][KS];
-  {
-    uint4 wv[WP];
-#pragma unroll
-    for (int i = 0; i < WP; ++i)
-      wv[i] = reinterpret_cast<const uint4*>(wg + (int64_t)m0 * E)[tid + 256 * i];
-#pragma unroll
-    for (int i = 0; i < WP; ++i) {
-      const int p = tid + 256 * i;
-      *reinterpret_cast<uint4*>(wl + (p / WPR) * WROW + (p % WPR) * 16) = wv[i];
+      int64_t t = t0 + wave * 8 + 2 * j + half;
+      t = t < T_tokens ? t : T_tokens - 1;
+      kept2[j] = *reinterpret_cast<const uint16_t*>(kept + t * 2);
+      idx2[j] = *reinterpret_cast<const int2*>(idx + t * 2);
+      pos2[j] = *reinterpret_cast<const int2*>(pos + t * 2);
+      gate2[j] = *reinterpret_cast<const float2*>(gate + t * 2);
     }
   }
+  __builtin_amdgcn_sched_barrier(0);
+  // (written as asm so that they are issued here: the compiler moves ordinary
+  // loads of the kernel rows behind the rows of d(expert_in), next to their
+  // use, and the wait for them then waits for everything)
+  dbm_u32x4_t wv[WP];
+#pragma unroll
+  for (int i = 0; i < WP; ++i) {
+    const uint4* src =
+        reinterpret_cast<const uint4*>(wg + (int64_t)m0 * E) + tid + 256 * i;
+    asm volatile("global_load_dwordx4 %0, %1, off"
+                 : "=&v"(wv[i]) : "v"(src) : "memory");
+  }
   float4 dv[DP];
+  bool dv_used[DP];
+#pragma unroll
+  for (int i = 0; i < DP; ++i) {
+    const int p = tid + 256 * i;
+    dv_used[i] = p < DBM_TOK * DPR && t0 + p / DPR < T_tokens;
+    dv[i] = reinterpret_cast<const float4*>(dlogits + t0 * E)[dv_used[i] ? p : 0];
+  }
+  __builtin_amdgcn_sched_barrier(0);
+  // the rows this lane adds in phase 2: 8 columns from column 8 l32 of the tile
+  // (bit 2 j + k of `used`: the row counts; the others are loaded from slot 0)
   uint4 v[RP][2];
-  load_tile(dv, v);
-  __syncthreads();
+  unsigned used = 0;
+  if constexpr (!SLOT) {
+    int64_t base[RP][2];
+#pragma unroll
+    for (int j = 0; j < RP; ++j)
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        const int64_t e = k ? idx2[j].y : idx2[j].x;
+        if constexpr (COMPACT)
+          base[j][k] = e * G * C + row_offsets[e * G + g];
+        else
+          base[j][k] = (e * G + g) * C;
+      }
+#pragma unroll
+    for (int j = 0; j < RP; ++j) {
+      const bool in_range = t0 + wave * 8 + 2 * j + half < T_tokens;
+#pragma unroll
+      for (int k = 0; k < 2; ++k) {
+        const float gk = round_to<bf16_t>(k ? gate2[j].y : gate2[j].x);
+        const bool u =
+            in_range & (((kept2[j] >> (8 * k)) & 0xff) != 0) & (gk != 0.0f);
+        used |= (u ? 1u : 0u) << (2 * j + k);
+        const int64_t slot = u ? base[j][k] + (k ? pos2[j].y : pos2[j].x) : 0;
+        v[j][k] = load_streaming(
+            reinterpret_cast<const uint4*>(dxe + slot * M + m0) + l32);
+      }
+    }
+  }
+  __builtin_amdgcn_sched_barrier(0);
+
+  // ---- the kernel rows and the d(logits) rows: registers -> LDS -> operands
+  // (the kernel rows have landed when only the 2 RP row loads issued after
+  // them may still be in flight)
+  if constexpr (SLOT)
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  else
+    asm volatile("s_waitcnt vmcnt(%0)" :: "n"(2 * RP) : "memory");
+#pragma unroll
+  for (int i = 0; i < WP; ++i) {
+    const int p = tid + 256 * i;
+    *reinterpret_cast<dbm_u32x4_t*>(wl + (p / WPR) * WROW + (p % WPR) * 16) =
+        wv[i];
+  }
+#pragma unroll
+  for (int i = 0; i < DP; ++i) {
+    const int p = tid + 256 * i;
+    if (p < DBM_TOK * DPR)
+      *reinterpret_cast<float4*>(dl + (p / DPR) * DROW + (p % DPR) * 16) =
+          dv_used[i] ? dv[i] : make_float4(0.f, 0.f, 0.f, 0.f);
+  }
+  dbm_lds_barrier();
+  uint4 afrag[2][KS];
 #pragma unroll
   for (int b = 0; b < 2; ++b)
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks)
       afrag[b][ks] = *reinterpret_cast<const uint4*>(
           wl + (wave * 64 + b * 32 + l32) * WROW + ks * 32 + half * 16);
-  // (the share goes over the kernel rows: the next barrier stands between
-  // these reads and its first write)
   {
     // ---- phase 1: this wavefront's 32 tokens x 64 columns of the share
-#pragma unroll
-    for (int i = 0; i < DP; ++i) {
-      const int p = tid + 256 * i;
-      if (p < DBM_TOK * DPR)
-        *reinterpret_cast<float4*>(dl + (p / DPR) * DROW + (p % DPR) * 16) = dv[i];
-    }
-    __syncthreads();
     dbm_f32x16_t acc[2];
 #pragma unroll
     for (int b = 0; b < 2; ++b)
@@ -488,6 +531,9 @@ __global__ __launch_bounds__(256) void dispatch_backward_mfma_kernel(
         acc[b] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a, bl, acc[b], 0, 0, 0);
       }
     }
+    // (the share goes over the kernel rows: every wavefront has its operands
+    // in registers before the first write)
+    dbm_lds_barrier();
     // lane: token l32, columns 32 b + 8 q + 4 half + 0..3 of the wavefront's 64
 #pragma unroll
     for (int b = 0; b < 2; ++b)
@@ -497,7 +543,7 @@ __global__ __launch_bounds__(256) void dispatch_backward_mfma_kernel(
             &share[l32 * DBM_LD + wave * 64 + b * 32 + q * 8 + half * 4]) =
             make_float4(acc[b][4 * q], acc[b][4 * q + 1], acc[b][4 * q + 2],
                         acc[b][4 * q + 3]);
-    __syncthreads();
+    dbm_lds_barrier();
 
     // ---- phase 2
 #pragma unroll
@@ -533,6 +579,11 @@ __global__ __launch_bounds__(256) void dispatch_backward_mfma_kernel(
       } else {
         unpack16(v[j][0], a, bf16_t());
         unpack16(v[j][1], b, bf16_t());
+#pragma unroll
+        for (int q = 0; q < 8; ++q) {
+          a[q] = (used >> (2 * j)) & 1u ? a[q] : 0.f;
+          b[q] = (used >> (2 * j + 1)) & 1u ? b[q] : 0.f;
+        }
       }
       const float sv[8] = {s0.x, s0.y, s0.z, s0.w, s1.x, s1.y, s1.z, s1.w};
 #pragma unroll
@@ -1299,7 +1350,9 @@ static int run_dispatch_backward(
     const size_t lds = dbm_lds_bytes(E);
 #define MOE_DBM(KS_)                                                         \
   do {                                                                       \
-    auto k = dispatch_backward_mfma_kernel<KS_>;                             \
+    auto k = row_offsets != nullptr                                          \
+                 ? dispatch_backward_mfma_kernel<KS_, false, true>           \
+                 : dispatch_backward_mfma_kernel<KS_, false, false>;         \
     MOE_ALLOW_LDS(k, lds);                                                   \
     k<<<grid, 256, lds, st>>>(                                               \
         (const bf16_t*)dexpert_in, idx, pos, gate, kept, dlogits,            \
