@@ -261,6 +261,35 @@ __device__ __forceinline__ void wait_vmcnt() {
   __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
 }
 
+typedef uint32_t u32x2_t __attribute__((ext_vector_type(2)));
+__device__ __forceinline__ void lds_write_b64_asm(uint32_t addr, u32x2_t v) {
+  asm volatile("ds_write_b64 %0, %1" :: "v"(addr), "v"(v) : "memory");
+}
+__device__ __forceinline__ u32x4_t lds_read_b128_asm(uint32_t addr) {
+  u32x4_t v;
+  asm volatile("ds_read_b128 %0, %1" : "=v"(v) : "v"(addr) : "memory");
+  return v;
+}
+// Waits for the LDS reads above; the values pass through it so that nothing
+// that uses them is scheduled ahead of the wait.
+template <int N>
+__device__ __forceinline__ void lds_wait_pieces(u32x4_t (&p)[N]) {
+  static_assert(N == 8, "eight pieces per pass");
+  asm volatile("s_waitcnt lgkmcnt(0)"
+               : "+v"(p[0]), "+v"(p[1]), "+v"(p[2]), "+v"(p[3]), "+v"(p[4]),
+                 "+v"(p[5]), "+v"(p[6]), "+v"(p[7])
+               :: "memory");
+}
+
+// Block barrier that publishes LDS writes and waits for nothing else: vector
+// memory loads and stores of this wavefront stay in flight across it.
+__device__ __forceinline__ void lds_barrier() {
+  __builtin_amdgcn_s_waitcnt(0xc07f);  // lgkmcnt(0)
+  asm volatile("" ::: "memory");
+  __builtin_amdgcn_s_barrier();
+  asm volatile("" ::: "memory");
+}
+
 template <int BM, int BN, int WN, int WM = 2>  // WM x WN wavefronts
 struct DmaCfg {
   static constexpr int BK = 64;
@@ -972,7 +1001,8 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
   static_assert(EPI_BASE + EPI_ROWS * EPI_ROW_BYTES <= (int)Cfg::LOOP_BYTES,
                 "epilogue staging exceeds the ring");
   static_assert(BN == 256 && Cfg::WM == 2 && Cfg::TM == 4, "epilogue layout");
-  unsigned char* Cs = smem_raw + EPI_BASE;
+  // (LDS byte address of the staging area: its accesses are written as asm)
+  const uint32_t cs0 = (uint32_t)(size_t)(lds_void_t*)smem_raw + EPI_BASE;
   const int m_l = lane & 31;
   const int half = lane >> 5;   // which 8 bytes of a 16-byte chunk
   constexpr int CPR_C = BN / 8;  // 16-byte chunks per output row
@@ -1047,36 +1077,61 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
       set_tile(next);
       prologue_head();
     }
-    // round (and relu), stage in LDS, coalesced 16-byte stores
+    // round (and relu), stage in LDS, coalesced 16-byte stores.  Nothing here
+    // waits for vector memory: the next tile's first loads and this tile's
+    // stores stay in flight.  (__syncthreads() waits for them at every
+    // barrier, and in front of an ordinary LDS access the compiler waits for
+    // the direct-to-LDS loads in flight, which might write the same LDS: the
+    // staging accesses are therefore asm.)
+    // (the staging addresses are formed from a copy of the thread index that
+    // the compiler cannot see through: computed once outside the tile loop
+    // they would be live across the K loop, which has no registers to spare)
+    int e_tid = tid;
+    asm volatile("" : "+v"(e_tid));
+    const int e_lane = e_tid & 63, e_wave = e_tid >> 6;
+    const int e_wm = e_wave / WN, e_wn = e_wave % WN;
+    const int e_ml = e_lane & 31, e_half = e_lane >> 5;
 #pragma unroll
     for (int pass = 0; pass < 2; ++pass) {
 #pragma unroll
       for (int ii = 0; ii < 2; ++ii) {
         const int i = pass * 2 + ii;
-        const int srow = wm * 64 + ii * 32 + m_l;
+        const int srow = e_wm * 64 + ii * 32 + e_ml;
 #pragma unroll
         for (int j = 0; j < Cfg::TN; ++j) {
 #pragma unroll
           for (int q = 0; q < 4; ++q) {
-            const int chunk = (wn * Cfg::WTN + j * 32 + 8 * q) / 8;
-            uint2 v;
+            const int chunk = (e_wn * Cfg::WTN + j * 32 + 8 * q) / 8;
+            u32x2_t v;
             v.x = pack2_bf16(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1], RELU);
             v.y = pack2_bf16(acc[i][j][4 * q + 2], acc[i][j][4 * q + 3], RELU);
-            *reinterpret_cast<uint2*>(Cs + srow * EPI_ROW_BYTES +
-                                      ((chunk ^ m_l) * 16) + half * 8) = v;
+            lds_write_b64_asm(cs0 + srow * EPI_ROW_BYTES +
+                                  ((chunk ^ e_ml) * 16) + e_half * 8, v);
           }
         }
       }
-      __syncthreads();
+      lds_barrier();
+      // all staged pieces of this pass first, one wait, then the stores
+      constexpr int PIECES = EPI_ROWS * CPR_C / Cfg::THREADS;
+      static_assert(EPI_ROWS * CPR_C % Cfg::THREADS == 0, "whole pieces");
+      u32x4_t piece[PIECES];
 #pragma unroll
-      for (int c = tid; c < EPI_ROWS * CPR_C; c += Cfg::THREADS) {
+      for (int n = 0; n < PIECES; ++n) {
+        const int c = e_tid + n * Cfg::THREADS;
+        const int srow = c / CPR_C, chunk = c % CPR_C;
+        piece[n] = lds_read_b128_asm(cs0 + srow * EPI_ROW_BYTES +
+                                     ((chunk ^ (srow & 31)) * 16));
+      }
+      lds_wait_pieces(piece);
+#pragma unroll
+      for (int n = 0; n < PIECES; ++n) {
+        const int c = e_tid + n * Cfg::THREADS;
         const int srow = c / CPR_C, chunk = c % CPR_C;
         // staging row -> tile row: 64 rows of each half of the tile
         const int grow = out_row0 + (srow >> 6) * 128 + pass * 64 + (srow & 63);
         const int gcol = out_col0 + chunk * 8;
         if (grow < R && gcol < N) {
-          u32x4_t v = *reinterpret_cast<const u32x4_t*>(
-              Cs + srow * EPI_ROW_BYTES + ((chunk ^ (srow & 31)) * 16));
+          u32x4_t v = piece[n];
           if constexpr (MASKED) {
             const u32x4_t hm = *reinterpret_cast<const u32x4_t*>(
                 mask_src + (out_c - Cout) + (int64_t)grow * N + gcol);
@@ -1099,7 +1154,7 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
           *reinterpret_cast<u32x4_t*>(out_c + (int64_t)grow * N + gcol) = v;
         }
       }
-      __syncthreads();
+      lds_barrier();
     }
     if (!has_next) break;
     tile = next;
