@@ -29,7 +29,7 @@
 extern "C" {
 #endif
 
-#define MESH_MOE_ABI_VERSION 33
+#define MESH_MOE_ABI_VERSION 34
 
 /* element types of activations / weights */
 #define MESH_MOE_F32 0
@@ -441,6 +441,49 @@ int mesh_moe_expert_choice_gating(const float* logits, const void* importance,
                                   int16_t* tok_slot, float* loss,
                                   void* workspace, size_t workspace_bytes,
                                   void* stream);
+
+/*
+ * ---------------------------------------------------------------------------
+ * Training-time scalar summaries of the switch, switch-max, ntlb and
+ * expert-selection routers: the values the reference hands to
+ * mtf.scalar_summary while training (transformer/moe.py:865-880, :981,
+ * :1010-1025, :1041-1046, :1149-1165, :1213, :1242-1257, :1259-1269,
+ * :1285-1289), recomputed from the router's float32 logits and its routing
+ * record.  _top_2_gating emits none.
+ *   logits [G,S,E] float32 (the router's, after any input noise);
+ *   softmax_dtype as for mesh_moe_ntlb_gating (bfloat16 only with router 2);
+ *   importance [G,S] or NULL (all 1);
+ *   router 1 = switch / switch_max (needs kept [G,S,2]), 2 = ntlb (top_k
+ *   candidates per token), 3 = expert selection (needs tok_slot [G,S,E]);
+ *   out, float32:
+ *     [0] mean over tokens of sum_e -p log(p + 1e-9)   ("<name>/entropy");
+ *         router 3: mean over (group, expert) of the same sum over the
+ *         group's tokens, the softmax running over the group
+ *     [1] mean over tokens of the largest probability  ("expert_gate",
+ *         routers 1 and 2; before the importance mask, moe.py:979-981)
+ *     [2] kept first choices / sum of importance        ("fraction_routed",
+ *         router 1)
+ *     [3] sum over importance-1 tokens of logsumexp(logits)^2 /
+ *         (number of importance-1 tokens * num_microbatches)
+ *                                                       ("<name>/z_loss")
+ *     routers 1, 2: [4 + e], e < E: the share of expert e among the choices
+ *         of importance-1 tokens (first choices; ntlb: all top_k candidates)
+ *         ("experts/..", one summary per expert);
+ *     router 3: [4 + s], s < S: E * C * the number of (group, expert) pairs
+ *         whose expert took the token at position s ("group_token/..").
+ *   out has 4 + E (routers 1, 2) or 4 + S (router 3) elements.  Sums over
+ *   tokens run per block and then in block order: the same bits on every run;
+ *   they agree with a sequential sum to float32 rounding.
+ * ---------------------------------------------------------------------------
+ */
+size_t mesh_moe_router_summaries_workspace_bytes(int G, int S, int E);
+int mesh_moe_router_summaries(const float* logits, int softmax_dtype,
+                              const void* importance, int importance_dtype,
+                              const uint8_t* kept, const int16_t* tok_slot,
+                              int G, int S, int E, int C, int router,
+                              int top_k, int num_microbatches, float* out,
+                              void* workspace, size_t workspace_bytes,
+                              void* stream);
 
 /*
  * Dispatch by slot: expert_in[e,g,c,:] = x[g, slot_token[g,e,c], :]

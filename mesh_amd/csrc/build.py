@@ -10,7 +10,7 @@ from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 SOURCES = ["abi.hip", "route.hip", "dispatch.hip", "ffn.hip", "backward.hip",
-           "expert_choice.hip", "ntlb.hip", "block.hip",
+           "expert_choice.hip", "ntlb.hip", "summaries.hip", "block.hip",
            "attention.hip"]
 LIB_NAME = "libmesh_moe_hip.so"
 LIB_PATH = os.path.join(HERE, LIB_NAME)

@@ -22,7 +22,7 @@ BF16 = 1
 POLICIES = {"all": 0, "none": 1, "threshold": 2, "random": 3}
 ACTIVATIONS = {None: 0, "linear": 0, "relu": 1, "gelu": 2, "sigmoid": 3,
                "tanh": 4, "swish": 5}
-ABI_VERSION = 33
+ABI_VERSION = 34
 
 _vp = ctypes.c_void_p
 _SIGNATURES = {
@@ -68,6 +68,12 @@ _SIGNATURES = {
         ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp, _vp, _vp, _vp, _vp,
         _vp, _vp, ctypes.c_size_t, _vp]),
+    "mesh_moe_router_summaries_workspace_bytes": (ctypes.c_size_t, [
+        ctypes.c_int, ctypes.c_int, ctypes.c_int]),
+    "mesh_moe_router_summaries": (ctypes.c_int, [
+        _vp, ctypes.c_int, _vp, ctypes.c_int, _vp, _vp, ctypes.c_int,
+        ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int,
+        ctypes.c_int, _vp, _vp, ctypes.c_size_t, _vp]),
     "mesh_moe_dispatch": (ctypes.c_int, [
         _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, ctypes.c_int, ctypes.c_int,
         ctypes.c_int, ctypes.c_int, ctypes.c_int, ctypes.c_int, _vp]),
@@ -602,6 +608,46 @@ def ntlb_gating(logits, capacity, top_k, importance=None,
   if _timer is not None:
     _timer.routing.append(r)
   return r
+
+
+SUMMARY_ROUTERS = {"switch": 1, "switch_max": 1, "ntlb": 2,
+                   "expert_selection": 3}
+
+
+def router_summaries(logits, router, capacity, importance=None, kept=None,
+                     tok_slot=None, top_k=1, num_microbatches=None,
+                     softmax_dtype=torch.float32):
+  """The values the f1 routers hand to mtf.scalar_summary while training
+  (transformer/moe.py:865-880, :981, :1010-1025, :1041-1046, :1149-1165, :1213,
+  :1242-1257, :1259-1269, :1285-1289), from the router's float32 logits
+  [G, S, E] and its record.  Returns a float32 tensor: [0] mean entropy, [1]
+  mean largest probability, [2] fraction routed, [3] z-loss, then per expert
+  its share of the routed choices (switch, switch_max, ntlb: E values) or per
+  group position E * C * the number of experts that took it (expert selection:
+  S values)."""
+  lib = load_library()
+  g, s, e = logits.shape
+  code = SUMMARY_ROUTERS[router]
+  lp = _dev(logits, "logits", torch.float32)
+  ip, icode = None, F32
+  if importance is not None:
+    icode = dtype_code(importance.dtype)
+    ip = _dev(importance, "importance", None, (g, s))
+  kp = None if kept is None else _dev(kept, "kept", torch.uint8, (g, s, 2))
+  tp = None if tok_slot is None else _dev(tok_slot, "tok_slot", torch.int16,
+                                          (g, s, e))
+  out = torch.empty((4 + (s if code == 3 else e),), dtype=torch.float32,
+                    device=logits.device)
+  ws_bytes = lib.mesh_moe_router_summaries_workspace_bytes(g, s, e)
+  ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8,
+                   device=logits.device)
+  with _stage("router_summaries"):
+    _check(lib.mesh_moe_router_summaries(
+        lp, dtype_code(softmax_dtype), ip, icode, kp, tp, g, s, e,
+        int(capacity), code, int(top_k), int(num_microbatches or 1),
+        out.data_ptr(), ws.data_ptr(), ws_bytes, _stream()),
+           "router_summaries")
+  return out
 
 
 def router_switch_gating(x, w_packed, group_size, capacity, importance=None,

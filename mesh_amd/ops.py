@@ -615,6 +615,7 @@ class Lowering(object):
     self.variables = {}    # {Variable: LaidOutVariable}
     self.initial_values = dict(initial_values or {})
     self._feeds = {}
+    self.scalar_summaries = {}   # {name: 0-d torch tensor} of the last run
     for op in graph.operations:
       op.lower(self)
       for out in op.outputs:
@@ -626,6 +627,7 @@ class Lowering(object):
     """Executes the graph's non-variable operations again.  `feeds` maps
     imported Tensors to new torch tensors of the same shape."""
     self._feeds = dict(feeds or {})
+    self.scalar_summaries = {}
     try:
       for op in self.graph.operations:
         if not isinstance(op, Variable):
@@ -688,6 +690,17 @@ class Lowering(object):
   def copy_slices_to_masters(self):
     for v in self.variables.values():
       v.copy_slices_to_master()
+
+  def add_scalar_summary(self, name, value):
+    """Records a 0-d device tensor under `name` for this run (what
+    tf.summary.scalar does with the reference's ScalarSummaryOperation,
+    ops.py:4402-4436).  A name used before in the same run gets the suffix
+    _1, _2, .. as TensorFlow's summary names do."""
+    key, n = name, 0
+    while key in self.scalar_summaries:
+      n += 1
+      key = "%s_%d" % (name, n)
+    self.scalar_summaries[key] = value.reshape(())
 
   def add_counter(self, key, value):
     assert isinstance(value, int)
@@ -898,6 +911,34 @@ def multiply(x1, x2, output_shape=None, name=None):
   c = _scalar_in(x1.dtype, x2)
   return cwise(lambda t: t * c, [x1], name=name or "scalar_mul",
                grad_function=lambda op, dy: [multiply(dy, x2)])
+
+
+class ScalarSummaryOperation(Operation):
+  """mtf.scalar_summary (ops.py:4402-4436): passes x through and records its
+  value under `name` on the Lowering (Lowering.scalar_summaries)."""
+
+  def __init__(self, name, x):
+    super(ScalarSummaryOperation, self).__init__(
+        [x], x.mesh, name=name + "_summary")
+    if x.shape.dims:
+      raise ValueError("ScalarSummaryOperation takes a scalar")
+    self._summary_name = name
+    self._outputs = [Tensor(self, x.shape, x.dtype)]
+
+  def gradient(self, grad_ys):
+    return grad_ys
+
+  def lower(self, lowering):
+    x = lowering.tensors[self.inputs[0]]
+    lowering.add_scalar_summary(
+        self._summary_name, x.to_laid_out_tensor().tensor_list[0])
+    lowering.set_tensor_lowering(self.outputs[0], x)
+
+
+def scalar_summary(name, x):
+  """Records the 0-dimensional Tensor x under `name`; returns a Tensor equal
+  to x (ops.py:4423-4436)."""
+  return ScalarSummaryOperation(name, x).outputs[0]
 
 
 class ReshapeOperation(Operation):

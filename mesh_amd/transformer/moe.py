@@ -127,6 +127,7 @@ class _GatingSpec(object):
 
   router = "top_2"
   z_loss = None
+  summaries = False        # _top_2_gating emits no summaries
 
   def route(self, x, w, w_packed, group_size, num_experts, capacity,
             importance=None, importance_from_slot_gate=False,
@@ -249,6 +250,12 @@ class _SwitchGatingSpec(object):
         raise ValueError("moe_z_loss needs nonpadding and num_microbatches")
       self.z_loss = float(hparams.moe_z_loss)
     self.num_microbatches = num_microbatches
+    # what the reference logs with mtf.scalar_summary while training
+    # (moe.py:1213, :1242-1257, :1269, :1285-1289; :981, :1010-1025, :1041-1046)
+    self.summaries = bool(train)
+    self.summary_name = ("switch_max_gating" if self.slots_by_gate
+                         else "switch_gating")
+    self.logs_expert_gate = policy != "sample"
 
   router = "switch"
   use_second_place_loss = False
@@ -299,6 +306,8 @@ class _NtlbGatingSpec(object):
                                  allow_dropout=False)
     self.top_k = int(hparams.moe_ntlb_top_k)
     self.num_microbatches = num_microbatches
+    self.summaries = bool(train)                        # moe.py:864-880
+    self.summary_name = "ntlb_gating"
 
   def route(self, x, w, w_packed, group_size, num_experts, capacity,
             importance=None, importance_from_slot_gate=False,
@@ -336,6 +345,8 @@ class _ExpertSelectionGatingSpec(object):
       # the reference sums `importance` for its loss (moe.py:1138-1140)
       raise ValueError("expert_selection gating needs nonpadding")
     self.num_microbatches = num_microbatches
+    self.summaries = bool(train)                        # moe.py:1148-1165
+    self.summary_name = "expert_selection_gating"
 
   def route(self, x, w, w_packed, group_size, num_experts, capacity,
             importance=None, importance_from_slot_gate=False,
@@ -349,6 +360,41 @@ class _ExpertSelectionGatingSpec(object):
         logits, capacity, importance=importance,
         num_microbatches=self.num_microbatches)
     return (r, logits) if want_logits else r
+
+
+def _emit_router_summaries(lowering, spec, logits, r, capacity, importance,
+                           act_dtype, scope):
+  """The scalar summaries the f1 routers log while training, computed by
+  mesh_moe_router_summaries from the router's logits and record and recorded
+  on the Lowering under the reference's names.  The per-expert (per group
+  position) names follow "experts/" + fraction.name.replace(":", "/")
+  (moe.py:877-879): the outputs of an mtf.split named "split" in the layer's
+  scope."""
+  by_slot = isinstance(r, moe_hip.SlotRouting)
+  vals = moe_hip.router_summaries(
+      logits, spec.router if not getattr(spec, "slots_by_gate", False)
+      else "switch_max", capacity, importance=importance,
+      kept=None if by_slot else r.kept,
+      tok_slot=r.tok_slot if by_slot else None,
+      top_k=getattr(spec, "top_k", 1),
+      num_microbatches=spec.num_microbatches,
+      softmax_dtype=act_dtype if spec.router == "ntlb" else torch.float32)
+  add = lowering.add_scalar_summary
+  aux_loss = r.loss[0]
+  if spec.router == "switch" and getattr(spec, "logs_expert_gate", False):
+    add("expert_gate", vals[1])
+  add(spec.summary_name + "/entropy", vals[0])
+  prefix = ("group_token/" if by_slot else "experts/") + (
+      scope + "/" if scope else "")
+  for i in range(vals.shape[0] - 4):
+    add("%ssplit/%d" % (prefix, i), vals[4 + i])
+  if spec.z_loss is not None:
+    aux_loss = aux_loss - spec.z_loss * vals[3]
+  add("aux_loss", aux_loss)
+  if spec.z_loss is not None:
+    add(spec.summary_name + "/z_loss", vals[3])
+  if spec.router == "switch":
+    add("fraction_routed", vals[2])
 
 
 def _packed(lowering, kernel_tensor, dtype):
@@ -395,6 +441,7 @@ class MoEV1Operation(mtf.Operation):
       ins.append(k_wo)
     ins.extend(wis[1:])
     super(MoEV1Operation, self).__init__(ins, name=name)
+    self._scope = mtf.current_scope_name()
     self._has_importance = importance is not None
     self._k_wo = k_wo
     self._capacity = capacity
@@ -460,12 +507,18 @@ class MoEV1Operation(mtf.Operation):
       xg = x_s.reshape(groups, s_, m_)
       if imp_s is not None:
         imp_s = imp_s.reshape(groups, s_)
+      summarize = self._gating.summaries
       r = self._gating.route(xg.reshape(1, groups * s_, m_),
                              wg_s.reshape(1, m_, e_), wg_p, s_, e_, c_, imp_s,
-                             want_logits=save)
+                             want_logits=save or summarize)
       logits = None
-      if save:
+      if save or summarize:
         r, logits = r
+      if summarize:
+        _emit_router_summaries(lowering, self._gating, logits, r, c_, imp_s, dt,
+                               self._scope)
+        if not save:
+          logits = None
       by_slot = isinstance(r, moe_hip.SlotRouting)
       y = None
       noise = None

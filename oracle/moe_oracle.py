@@ -48,6 +48,13 @@ MoE file, and its TensorFlow dependency cannot run here):
                                       weights of a token sum to sum(p)/count,
                                       closed-form loss (uniform logits: 1.0),
                                       dense tensors vs slot record
+  router_summaries                    closed forms (uniform logits: entropy
+                                      log E, expert_gate 1 / E, all choices on
+                                      expert 0, z-loss (log E)^2 / mb; one-hot
+                                      rows: entropy 0, gate 1), a per-token
+                                      float64 loop, fraction_routed against the
+                                      capacity (S tokens on one expert:
+                                      C / S), group_token sums to G E C E C
   perturb_gate_inputs                 closed forms (eps = 0 and eval change
                                       nothing, all-kept dropout scales the
                                       logits by 1 / keep_prob), the experts
@@ -691,6 +698,69 @@ def expert_selection_gating(logits, capacity, importance,
   if dense:
     out["combine"] = cast_act(combine.transpose(0, 3, 1, 2), act_dtype)
     out["dispatch"] = dispatch.transpose(0, 3, 1, 2).astype(F32)  # :1169-1170
+  return out
+
+
+# ----------------------------------------------------------------------------
+# training-time scalar summaries of the f1 routers
+# ----------------------------------------------------------------------------
+def router_summaries(logits, gating, routing, importance=None, top_k=1,
+                     num_microbatches=None, act_dtype="float32", capacity=None):
+  """The values _switch_gating (moe.py:1213, :1242-1257, :1259-1269,
+  :1285-1289), _switch_max_gating (:981, :1010-1025, :1041-1046), _ntlb_gating
+  (:865-880) and _expert_selection_gating (:1149-1165) pass to
+  mtf.scalar_summary while training, from the router's logits [G,S,E] and the
+  gating function's result dict `routing`.
+
+  Returns a dict: "entropy"; for the per-token routers "expert_gate" (mean
+  largest probability, before the importance mask), "experts" [E] (share of
+  every expert among the choices of importance-1 tokens), for the switch
+  routers "fraction_routed" and "z_loss" (the value; the reference emits it
+  only with moe_z_loss set); for expert selection "group_token" [S].  Sums over
+  many terms accumulate in float64 and round once (the order of TensorFlow's
+  reductions is not pinned).
+  """
+  logits = np.asarray(logits, dtype=F32)
+  g_, s_, e_ = logits.shape
+  eps = F32(1e-9)
+  if gating == "expert_selection":
+    importance = np.asarray(importance, dtype=F32)
+    lg = logits + ((importance == F32(0.0)).astype(F32) * F32(-1e9))[..., None]
+    raw = np.moveaxis(softmax(np.moveaxis(lg, 1, -1)), -1, 1)    # [G,S,E]
+    terms = (-raw * np.log(raw + eps).astype(F32)).astype(F32)   # :1149
+    entropy = terms.sum(axis=1, dtype=np.float64)                # [G,E]
+    tokens = np.asarray(routing["slot_token"])                   # [G,E,C]
+    cap = tokens.shape[-1]
+    sent = np.zeros((s_,), np.float64)
+    np.add.at(sent, tokens.reshape(-1), 1.0)                     # :1155-1158
+    return dict(entropy=F32(entropy.mean()),
+                group_token=(sent * float(e_ * cap)).astype(F32))
+  raw = router_softmax(logits, gating, act_dtype)
+  terms = (-raw * np.log(raw + eps).astype(F32)).astype(F32)
+  entropy = F32(terms.sum(axis=-1, dtype=np.float64).mean())
+  k_ = int(top_k) if gating == "ntlb" else 1
+  gate, index = top_k_lowest_index_first(raw, k_, -1)            # [G,S,k]
+  mask = one_hot(index, e_)                                      # [G,S,k,E]
+  is_one = np.ones((g_, s_), F32)
+  imp = np.ones((g_, s_), F32)
+  if importance is not None:
+    imp = np.asarray(importance, dtype=F32)
+    is_one = (imp == F32(1.0)).astype(F32)
+    mask = mask * is_one[..., None, None]
+  counts = mask.sum(axis=(0, 1, 2), dtype=np.float64)            # [E]
+  out = dict(entropy=entropy,
+             expert_gate=F32(gate[..., 0].mean(dtype=np.float64)),
+             experts=(counts / counts.sum()).astype(F32))
+  if gating in ("switch", "switch_max"):
+    kept = np.asarray(routing["kept_1"])
+    out["fraction_routed"] = F32(kept.sum(dtype=np.float64) /
+                                 imp.sum(dtype=np.float64))
+    m = logits.max(axis=-1, keepdims=True)
+    log_z = np.log(seq_sum(np.exp(logits + (-m)).astype(F32), axis=-1)
+                   ).astype(F32) + m[..., 0]
+    z = ((log_z * log_z) * is_one).sum(dtype=np.float64)
+    out["z_loss"] = F32(z / (is_one.sum(dtype=np.float64) *
+                             float(num_microbatches or 1)))
   return out
 
 

@@ -758,6 +758,97 @@ def test_ntlb_dispatch_combine_roundtrip(hip):
       H.to_np(xe), O.dispatch_gather(x, ref, e, c, "float32"))
 
 
+# ---- training-time summaries of the f1 routers --------------------------------
+@pytest.mark.parametrize("shape", [(2, 256, 8, 40), (32, 2048, 64, 64),
+                                   (3, 77, 5, 12), (1, 1, 2, 1),
+                                   (2, 131, 200, 3)])
+@pytest.mark.parametrize("gating", ["switch", "switch_max", "ntlb", "ntlb_bf16"])
+def test_router_summaries(hip, gating, shape):
+  """entropy, expert_gate, per-expert shares, fraction_routed and z-loss as the
+  reference hands them to mtf.scalar_summary, against the oracle.  The shares
+  are ratios of integer counts; the float32 sums over tokens agree to
+  rounding (rtol 2e-5, stated here)."""
+  g, s, e, c = shape
+  k = min(3, e)
+  rng = np.random.default_rng(4100 + sum(shape))
+  bf16 = gating == "ntlb_bf16"
+  name = "ntlb" if bf16 else gating
+  if bf16:
+    logits = H.bf16_softmax_safe_logits(rng, g, s, e, scale=1.5,
+                                        bias=H.zipf_bias(rng, e, scale=2.0))
+  else:
+    logits = H.safe_logits(rng, g, s, e, scale=1.5,
+                           bias=H.zipf_bias(rng, e, scale=2.0), top=k + 1)
+  imp = rng.choice(np.array([0.0, 0.5, 1.0], np.float32), size=(g, s),
+                   p=[0.1, 0.1, 0.8])
+  imp[0, 0] = 1.0
+  act = "bfloat16" if bf16 else "float32"
+  lg = torch.from_numpy(logits).cuda()
+  for importance, mb in ((None, None), (imp, 2)):
+    ip = None if importance is None else H.to_gpu(importance)
+    if name == "switch":
+      want_r = O.switch_gating(logits, c, importance=importance)
+      r = hip.switch_gating(lg, c, importance=ip)
+    elif name == "switch_max":
+      want_r = O.switch_max_gating(logits, c, importance=importance)
+      r = hip.switch_gating(lg, c, importance=ip, slots_by_gate=True)
+    else:
+      want_r = O.ntlb_gating(logits, c, k, importance=importance, act_dtype=act)
+      r = hip.ntlb_gating(lg, c, k, importance=ip,
+                          softmax_dtype=torch.bfloat16 if bf16 else torch.float32)
+    want = O.router_summaries(logits, name, want_r, importance=importance,
+                              top_k=k, num_microbatches=mb, act_dtype=act)
+    got = H.to_np(hip.router_summaries(
+        lg, name, c, importance=ip, kept=r.kept, top_k=k, num_microbatches=mb,
+        softmax_dtype=torch.bfloat16 if bf16 else torch.float32))
+    assert got.shape == (4 + e,)
+    np.testing.assert_allclose(got[0], want["entropy"], rtol=2e-5)
+    np.testing.assert_allclose(got[1], want["expert_gate"], rtol=2e-5)
+    np.testing.assert_allclose(got[4:], want["experts"], rtol=1e-6)
+    np.testing.assert_allclose(got[4:].sum(), 1.0, rtol=1e-5)
+    if name != "ntlb":
+      np.testing.assert_allclose(got[2], want["fraction_routed"], rtol=1e-6)
+      np.testing.assert_allclose(got[3], want["z_loss"], rtol=2e-5)
+    # the same bits on every run
+    again = H.to_np(hip.router_summaries(
+        lg, name, c, importance=ip, kept=r.kept, top_k=k, num_microbatches=mb,
+        softmax_dtype=torch.bfloat16 if bf16 else torch.float32))
+    np.testing.assert_array_equal(got, again)
+
+
+@pytest.mark.parametrize("shape", [(2, 256, 8, 40), (32, 2048, 64, 64),
+                                   (3, 77, 5, 12), (2, 131, 200, 3)])
+def test_router_summaries_expert_selection(hip, shape):
+  g, s, e, c = shape
+  rng = np.random.default_rng(4200 + sum(shape))
+  logits = H.random_logits(rng, g, s, e, scale=1.5)
+  imp = rng.choice(np.array([0.0, 1.0], np.float32), size=(g, s), p=[0.1, 0.9])
+  lg, ip = torch.from_numpy(logits).cuda(), H.to_gpu(imp)
+  r = hip.expert_choice_gating(lg, c, importance=ip)
+  want_r = dict(slot_token=H.to_np(r.slot_token).astype(np.int64))
+  want = O.router_summaries(logits, "expert_selection", want_r, importance=imp)
+  got = H.to_np(hip.router_summaries(lg, "expert_selection", c, importance=ip,
+                                     tok_slot=r.tok_slot))
+  assert got.shape == (4 + s,)
+  np.testing.assert_allclose(got[0], want["entropy"], rtol=2e-5)
+  np.testing.assert_array_equal(got[4:], want["group_token"])
+  assert got[4:].sum() == float(g * e * c) * e * c
+
+
+def test_router_summaries_rejections(hip):
+  lg = torch.zeros((1, 8, 4), device="cuda")
+  with pytest.raises(hip.MoeHipError, match="need kept"):
+    hip.router_summaries(lg, "switch", 2)
+  with pytest.raises(hip.MoeHipError, match="tok_slot"):
+    hip.router_summaries(lg, "expert_selection", 2)
+  with pytest.raises(hip.MoeHipError, match="top_k"):
+    hip.router_summaries(lg, "ntlb", 2, top_k=9)
+  kept = torch.zeros((1, 8, 2), dtype=torch.uint8, device="cuda")
+  with pytest.raises(hip.MoeHipError, match="bfloat16"):
+    hip.router_summaries(lg, "switch", 2, kept=kept,
+                         softmax_dtype=torch.bfloat16)
+
+
 def test_ntlb_gating_rejections(hip):
   lg = torch.zeros((1, 8, 4), dtype=torch.float32, device="cuda")
   with pytest.raises(hip.MoeHipError, match="top_k=5 with 4 experts"):

@@ -646,6 +646,87 @@ def test_v1_switch_train_z_loss_and_nonpadding():
   assert got_loss > loss0
 
 
+@pytest.mark.parametrize("gating", ["switch", "switch_max", "ntlb",
+                                    "expert_selection"])
+def test_v1_router_summaries_on_the_lowering(gating):
+  """While training the f1 routers log scalars with mtf.scalar_summary
+  (moe.py:865-880, :1010-1046, :1149-1165, :1213-1289): they arrive on the
+  Lowering under the reference's names with the oracle's values; an evaluation
+  graph and the top-2 router log nothing."""
+  b, l, m, hdim, e = 2, 128, 32, 48, 4
+  rng = np.random.default_rng(311)
+  w = dict(w_gate=H.normal_weights(rng, (m, e), m),
+           wi=H.normal_weights(rng, (e, m, hdim), m),
+           wo=H.normal_weights(rng, (e, hdim, m), hdim))
+  x = H.safe_tokens(rng, b * l, m, w["w_gate"], "float32").reshape(b, l, m)
+  nonpad = (rng.random((b, l)) < 0.8).astype(np.float32)
+  kw = dict(SWITCH_HP, moe_gating=gating, moe_ntlb_top_k=2,
+            moe_z_loss=1e-2 if gating == "switch" else None)
+  hp, ohp = make_hparams(moe_num_experts=e, moe_hidden_size=hdim,
+                         moe_group_size=64, moe_capacity_factor_train=1.0, **kw)
+  _, _, low, _ = run_v1(x, w, hp, True, "float32", nonpadding=nonpad,
+                        num_microbatches=2)
+  _, _, aux = O.moe_layer_v1(x, w["w_gate"], w["wi"], w["wo"], ohp, True,
+                             "float32", nonpadding=nonpad, num_microbatches=2)
+  groups = b * l // 64
+  want = O.router_summaries(aux["logits"], gating, aux,
+                            importance=nonpad.reshape(groups, 64), top_k=2,
+                            num_microbatches=2)
+  got = {k: float(v) for k, v in low.scalar_summaries.items()}
+  name = gating + "_gating"
+  np.testing.assert_allclose(got[name + "/entropy"], want["entropy"], rtol=1e-4)
+  if gating == "expert_selection":
+    per = [got["group_token/moe/split/%d" % i] for i in range(64)]
+    np.testing.assert_array_equal(per, want["group_token"])
+    expected = {name + "/entropy", "aux_loss"}
+  else:
+    per = [got["experts/moe/split/%d" % i] for i in range(e)]
+    np.testing.assert_allclose(per, want["experts"], rtol=1e-6)
+    expected = {name + "/entropy", "aux_loss"}
+  if gating in ("switch", "switch_max"):
+    np.testing.assert_allclose(got["fraction_routed"], want["fraction_routed"],
+                               rtol=1e-6)
+    np.testing.assert_allclose(got["expert_gate"], want["expert_gate"], rtol=1e-4)
+    expected |= {"fraction_routed", "expert_gate"}
+  if gating == "switch":
+    np.testing.assert_allclose(got[name + "/z_loss"], want["z_loss"], rtol=1e-4)
+    # aux_loss is the balancing loss before the z-loss is added (moe.py:1257)
+    _, ohp0 = make_hparams(moe_num_experts=e, moe_hidden_size=hdim,
+                           moe_group_size=64, moe_capacity_factor_train=1.0,
+                           **dict(kw, moe_z_loss=None))
+    _, loss0, _ = O.moe_layer_v1(x, w["w_gate"], w["wi"], w["wo"], ohp0, True,
+                                 "float32", nonpadding=nonpad, num_microbatches=2)
+    np.testing.assert_allclose(got["aux_loss"] * ohp.moe_loss_coef, loss0,
+                               rtol=1e-4)
+    expected |= {name + "/z_loss"}
+  assert {k for k in got if "/split/" not in k} == expected
+  # evaluation: nothing is logged; a second run replaces the first run's values
+  _, _, low_eval, _ = run_v1(x, w, hp, False, "float32", nonpadding=nonpad)
+  assert low_eval.scalar_summaries == {}
+  low.run()
+  again = {k: float(v) for k, v in low.scalar_summaries.items()}
+  assert again == got
+  hp2, _ = make_hparams(moe_num_experts=e, moe_hidden_size=hdim,
+                        moe_group_size=64)
+  _, _, low2, _ = run_v1(x, w, hp2, True, "float32", nonpadding=nonpad)
+  assert low2.scalar_summaries == {}
+
+
+def test_scalar_summary_operation():
+  graph = mtf.Graph()
+  mesh = mtf.Mesh(graph, "mesh")
+  a = mtf.import_tf_tensor(mesh, torch.tensor(1.5), mtf.Shape([]))
+  b_ = mtf.scalar_summary("loss", a)
+  c_ = mtf.scalar_summary("loss", b_ * 2.0)
+  low = mtf.Lowering(graph, {mesh: mtf.HipMeshImpl()})
+  assert float(low.export_to_tf_tensor(c_)) == 3.0
+  assert {k: float(v) for k, v in low.scalar_summaries.items()} == {
+      "loss": 1.5, "loss_1": 3.0}
+  with pytest.raises(ValueError):
+    mtf.scalar_summary("v", mtf.import_tf_tensor(
+        mesh, torch.zeros(2), mtf.Shape([mtf.Dimension("d", 2)])))
+
+
 def test_v1_switch_rejections():
   x = np.zeros((1, 32, 16), np.float32)
   w = dict(w_gate=np.zeros((16, 4), np.float32),

@@ -1571,3 +1571,103 @@ def test_switch_sample_policy():
   rm = O.switch_max_gating(logits, s, choice_logits=O.sample_choice_logits(
       logits, 50.0, forced))
   np.testing.assert_array_equal(rm["index_1"], target)
+
+
+# ---- training-time summaries of the f1 routers ------------------------------
+def test_router_summaries_closed_forms():
+  """Uniform logits: every row's entropy is log E (up to the 1e-9 inside the
+  log), the largest probability 1 / E, the arg-max always expert 0, the z-loss
+  (c + log E)^2 / microbatches; S tokens on one expert with capacity C:
+  fraction_routed = C / S.  Rows that are one-hot after the softmax: entropy
+  0, gate 1."""
+  g, s, e, c = 2, 16, 4, 5
+  lg = np.full((g, s, e), 0.75, np.float32)
+  r = O.switch_gating(lg, c)
+  out = O.router_summaries(lg, "switch", r, num_microbatches=2)
+  np.testing.assert_allclose(out["entropy"], np.log(e), rtol=1e-6)
+  np.testing.assert_allclose(out["expert_gate"], 1.0 / e, rtol=1e-6)
+  np.testing.assert_array_equal(out["experts"], [1, 0, 0, 0])
+  np.testing.assert_allclose(out["fraction_routed"], c / s, rtol=1e-6)
+  np.testing.assert_allclose(out["z_loss"], (0.75 + np.log(e)) ** 2 / 2,
+                             rtol=1e-6)
+  # importance: tokens that are not 1 leave the expert counts and the z-loss,
+  # fraction_routed divides by the SUM of importance (moe.py:1286-1289)
+  imp = np.ones((g, s), np.float32)
+  imp[:, ::2] = 0.5
+  r = O.switch_gating(lg, c, importance=imp)
+  out = O.router_summaries(lg, "switch", r, importance=imp, num_microbatches=1)
+  np.testing.assert_allclose(out["fraction_routed"],
+                             r["kept_1"].sum() / imp.sum(), rtol=1e-6)
+  np.testing.assert_allclose(out["z_loss"], (0.75 + np.log(e)) ** 2, rtol=1e-6)
+  sharp = np.zeros((1, 8, 4), np.float32)
+  sharp[0, np.arange(8), np.arange(8) % 4] = 60.0
+  r = O.switch_gating(sharp, 8)
+  out = O.router_summaries(sharp, "switch", r)
+  assert abs(float(out["entropy"])) < 1e-6
+  np.testing.assert_allclose(out["expert_gate"], 1.0, rtol=1e-6)
+  np.testing.assert_allclose(out["experts"], [0.25] * 4)
+  np.testing.assert_allclose(out["fraction_routed"], 1.0)
+
+
+@pytest.mark.parametrize("gating", ["switch", "switch_max", "ntlb"])
+def test_router_summaries_against_per_token_loop(gating):
+  rng = np.random.default_rng(77)
+  g, s, e, c, k = 3, 40, 6, 9, 3
+  lg = (rng.standard_normal((g, s, e)) * 2).astype(np.float32)
+  imp = rng.choice(np.array([0.0, 0.5, 1.0], np.float32), size=(g, s),
+                   p=[0.2, 0.1, 0.7])
+  if gating == "switch":
+    r = O.switch_gating(lg, c, importance=imp)
+  elif gating == "switch_max":
+    r = O.switch_max_gating(lg, c, importance=imp)
+  else:
+    r = O.ntlb_gating(lg, c, k, importance=imp)
+  out = O.router_summaries(lg, gating, r, importance=imp, top_k=k,
+                           num_microbatches=2)
+  p = scipy.special.softmax(lg.astype(np.float64), axis=-1)
+  ent, gate, counts, lse2, ones = 0.0, 0.0, np.zeros(e), 0.0, 0
+  for gi in range(g):
+    for si in range(s):
+      row = p[gi, si]
+      ent += float(-(row * np.log(row + 1e-9)).sum())
+      order = sorted(range(e), key=lambda j: (-row[j], j))
+      gate += row[order[0]]
+      if imp[gi, si] == 1.0:
+        ones += 1
+        lse2 += float(scipy.special.logsumexp(lg[gi, si].astype(np.float64))) ** 2
+        for j in order[:k if gating == "ntlb" else 1]:
+          counts[j] += 1
+  np.testing.assert_allclose(out["entropy"], ent / (g * s), rtol=1e-5)
+  np.testing.assert_allclose(out["expert_gate"], gate / (g * s), rtol=1e-5)
+  np.testing.assert_allclose(out["experts"], counts / counts.sum(), rtol=1e-6)
+  if gating != "ntlb":
+    np.testing.assert_allclose(out["z_loss"], lse2 / (ones * 2), rtol=1e-5)
+    np.testing.assert_allclose(out["fraction_routed"],
+                               r["kept_1"].sum() / imp.sum(), rtol=1e-6)
+    assert 0 < out["fraction_routed"] < 1
+
+
+def test_router_summaries_expert_selection():
+  """Column softmax: uniform logits over S unmasked tokens give entropy log S
+  per (group, expert); every slot names one token, so group_token sums to
+  G * E * C times the factor E * C the reference multiplies in
+  (moe.py:1155-1158); against a float64 loop on random logits."""
+  g, s, e, c = 2, 12, 3, 4
+  imp = np.ones((g, s), np.float32)
+  lg = np.zeros((g, s, e), np.float32)
+  r = O.expert_selection_gating(lg, c, imp)
+  out = O.router_summaries(lg, "expert_selection", r, importance=imp)
+  np.testing.assert_allclose(out["entropy"], np.log(s), rtol=1e-6)
+  np.testing.assert_allclose(out["group_token"].sum(), g * e * c * e * c)
+  # ties go to the lowest tokens: every expert of every group takes 0..c-1
+  np.testing.assert_array_equal(out["group_token"][:c], [g * e * e * c] * c)
+  rng = np.random.default_rng(5)
+  lg = (rng.standard_normal((g, s, e)) * 2).astype(np.float32)
+  imp[:, -3:] = 0.0
+  r = O.expert_selection_gating(lg, c, imp)
+  out = O.router_summaries(lg, "expert_selection", r, importance=imp)
+  x = lg.astype(np.float64) + (imp == 0)[..., None] * -1e9
+  p = scipy.special.softmax(x, axis=1)
+  np.testing.assert_allclose(out["entropy"],
+                             (-(p * np.log(p + 1e-9)).sum(1)).mean(), rtol=1e-5)
+  assert out["group_token"][-3:].sum() == 0           # masked tokens are never taken
