@@ -1175,20 +1175,23 @@ __global__ __launch_bounds__(RingCfg::THREADS) void grouped_gemm_bf16_ring_kerne
 // makes its operand reads 16 bytes wide.  Tiles are staged through registers
 // into LDS rows of 32 + 4 floats.  K % 4 == 0 and N % 4 == 0.
 // ---------------------------------------------------------------------------
+// TM x TN: MFMA tiles per wavefront; the block tile is 64 TM x 64 TN.
+template <int TM, int TN>
 struct F32Cfg {
-  static constexpr int BM = 128, BN = 128, BK = 32, THREADS = 256;
+  static constexpr int BM = 64 * TM, BN = 64 * TN, BK = 32, THREADS = 256;
   static constexpr int LDK = BK + 4;               // floats per LDS row
   static constexpr int CPR = BK / 4;               // 16-byte chunks per row
   static constexpr int A_CHUNKS = BM * CPR / THREADS, B_CHUNKS = BN * CPR / THREADS;
   static constexpr size_t LDS_BYTES = 2ull * (BM + BN) * LDK * sizeof(float);
 };
 
-template <bool RELU>
+template <bool RELU, int TM, int TN>
 __global__ __launch_bounds__(256) void grouped_gemm_f32_mfma_kernel(
     const float* __restrict__ A, const float* __restrict__ B,
     float* __restrict__ Cout, int R, int N, int K, int tiles_m, int tiles_n) {
-  using Cfg = F32Cfg;
+  using Cfg = F32Cfg<TM, TN>;
   constexpr int BM = Cfg::BM, BN = Cfg::BN, BK = Cfg::BK, LDK = Cfg::LDK;
+  constexpr int WTM = 32 * TM, WTN = 32 * TN;      // a wavefront's sub-tile
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   float* As = reinterpret_cast<float*>(smem_raw);  // [2][BM][LDK]
   float* Bs = As + 2 * BM * LDK;                   // [2][BN][LDK]
@@ -1239,11 +1242,11 @@ __global__ __launch_bounds__(256) void grouped_gemm_f32_mfma_kernel(
     }
   };
 
-  f32x16_t acc[2][2];
+  f32x16_t acc[TM][TN];
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int r = 0; r < 16; ++r) acc[i][j][r] = 0.f;
 
@@ -1255,23 +1258,23 @@ __global__ __launch_bounds__(256) void grouped_gemm_f32_mfma_kernel(
   for (int kt = 0; kt < nk; ++kt) {
     const int buf = kt & 1;
     if (kt + 1 < nk) load_global((kt + 1) * BK);
-    const float* as = As + (buf * BM + wm * 64 + frag_row) * LDK + frag_k;
-    const float* bs = Bs + (buf * BN + wn * 64 + frag_row) * LDK + frag_k;
+    const float* as = As + (buf * BM + wm * WTM + frag_row) * LDK + frag_k;
+    const float* bs = Bs + (buf * BN + wn * WTN + frag_row) * LDK + frag_k;
 #pragma unroll
     for (int u = 0; u < BK / 8; ++u) {
-      float4 af[2], bfr[2];
+      float4 af[TM], bfr[TN];
 #pragma unroll
-      for (int i = 0; i < 2; ++i)
+      for (int i = 0; i < TM; ++i)
         af[i] = *reinterpret_cast<const float4*>(as + i * 32 * LDK + u * 8);
 #pragma unroll
-      for (int j = 0; j < 2; ++j)
+      for (int j = 0; j < TN; ++j)
         bfr[j] = *reinterpret_cast<const float4*>(bs + j * 32 * LDK + u * 8);
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
 #pragma unroll
-        for (int i = 0; i < 2; ++i)
+        for (int i = 0; i < TM; ++i)
 #pragma unroll
-          for (int j = 0; j < 2; ++j) {
+          for (int j = 0; j < TN; ++j) {
             const float a = q == 0 ? af[i].x : q == 1 ? af[i].y
                             : q == 2 ? af[i].z : af[i].w;
             const float b = q == 0 ? bfr[j].x : q == 1 ? bfr[j].y
@@ -1286,13 +1289,13 @@ __global__ __launch_bounds__(256) void grouped_gemm_f32_mfma_kernel(
   }
   const int m_l = lane & 31, n_l = (lane >> 5) * 4;
 #pragma unroll
-  for (int i = 0; i < 2; ++i)
+  for (int i = 0; i < TM; ++i)
 #pragma unroll
-    for (int j = 0; j < 2; ++j)
+    for (int j = 0; j < TN; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int grow = row0 + wm * 64 + i * 32 + m_l;
-        const int gcol = col0 + wn * 64 + j * 32 + 8 * q + n_l;
+        const int grow = row0 + wm * WTM + i * 32 + m_l;
+        const int gcol = col0 + wn * WTN + j * 32 + 8 * q + n_l;
         if (grow < R && gcol < N) {
           float4 v = make_float4(acc[i][j][4 * q + 0], acc[i][j][4 * q + 1],
                                  acc[i][j][4 * q + 2], acc[i][j][4 * q + 3]);
@@ -1802,27 +1805,63 @@ static int launch_ring(const bf16_t* A, const bf16_t* B, bf16_t* C, int E,
   return 0;
 }
 
-static int launch_f32_mfma(const float* A, const float* B, float* C, int E,
-                           int R, int N, int K, bool relu, hipStream_t st) {
-  using Cfg = F32Cfg;
+template <int TM, int TN>
+static int launch_f32_mfma_tile(const float* A, const float* B, float* C, int E,
+                                int R, int N, int K, bool relu, hipStream_t st) {
+  using Cfg = F32Cfg<TM, TN>;
   const int tiles_m = (R + Cfg::BM - 1) / Cfg::BM;
   const int tiles_n = (N + Cfg::BN - 1) / Cfg::BN;
   const int64_t blocks = (int64_t)tiles_m * tiles_n * E;
   MOE_REQUIRE(blocks <= 0x7fffffffLL, MESH_MOE_E_UNSUPPORTED,
               "expert_ffn: too many tiles (%lld)", (long long)blocks);
   if (relu) {
-    auto k = grouped_gemm_f32_mfma_kernel<true>;
+    auto k = grouped_gemm_f32_mfma_kernel<true, TM, TN>;
     MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
     k<<<(unsigned)blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
         A, B, C, R, N, K, tiles_m, tiles_n);
   } else {
-    auto k = grouped_gemm_f32_mfma_kernel<false>;
+    auto k = grouped_gemm_f32_mfma_kernel<false, TM, TN>;
     MOE_ALLOW_LDS(k, Cfg::LDS_BYTES);
     k<<<(unsigned)blocks, Cfg::THREADS, Cfg::LDS_BYTES, st>>>(
         A, B, C, R, N, K, tiles_m, tiles_n);
   }
   MOE_CHECK_LAUNCH("expert_ffn (float32 mfma)");
   return 0;
+}
+
+// Block tile of the float32 kernel: 128 x 128, 64 x 128 or 64 x 64.  The
+// kernel is bound by the float32 matrix pipes (a 32 x 32 x 2 MFMA takes 64
+// cycles), so its time is rounds of tiles over the compute units times the
+// tile's area; small launches want small tiles (less padding of the row count,
+// fewer idle compute units in the last round).
+static int launch_f32_mfma(const float* A, const float* B, float* C, int E,
+                           int R, int N, int K, bool relu, hipStream_t st) {
+  const int cus = compute_units();
+  if (cus == 0) return MESH_MOE_E_HIP;
+  static const int shapes[3][2] = {{2, 2}, {1, 2}, {1, 1}};
+  int best = 0;
+  double best_cost = 0;
+  int64_t best_tiles = 0;
+  for (int i = 0; i < 3; ++i) {
+    const int bm = 64 * shapes[i][0], bn = 64 * shapes[i][1];
+    const int64_t tiles = (int64_t)E * ((R + bm - 1) / bm) * ((N + bn - 1) / bn);
+    const double cost = (double)((tiles + cus - 1) / cus) * bm * bn;
+    // a smaller tile when it saves time by this count, or costs the same while
+    // the larger one leaves compute units with fewer than two blocks to
+    // overlap (measured at 8 experts x 320 rows, 2048 x 512: 64 x 64 tiles
+    // 0.149 ms for both launches, 64 x 128 0.157, 128 x 128 0.228)
+    if (i == 0 || cost < 0.95 * best_cost ||
+        (cost <= best_cost && best_tiles < 2 * (int64_t)cus)) {
+      best = i;
+      best_cost = cost;
+      best_tiles = tiles;
+    }
+  }
+  switch (best) {
+    case 0: return launch_f32_mfma_tile<2, 2>(A, B, C, E, R, N, K, relu, st);
+    case 1: return launch_f32_mfma_tile<1, 2>(A, B, C, E, R, N, K, relu, st);
+    default: return launch_f32_mfma_tile<1, 1>(A, B, C, E, R, N, K, relu, st);
+  }
 }
 
 template <typename T>
