@@ -554,9 +554,14 @@ def main():
   }
   if cfg["layer"] == "v1":
     r = routings[-1]
+    tile_rows = None
     if hasattr(r, "fill"):
       kept = int(r.fill.sum().item())
       slots = r.fill.numel() * r.capacity
+      # compacted rows: an expert's occupied rows, rounded up to the 256-row
+      # tiles the listed-tile kernels multiply whole
+      used = r.fill.sum(dim=0)
+      tile_rows = int(((used + 255) // 256 * 256).sum().item())
     else:
       # per-slot record: every slot holds a token, its weight may be 0
       slots = r.slot_token.numel()
@@ -588,11 +593,12 @@ def main():
                     if args.gating == "top_2" else None),
         "flops_per_launch": flops_per_launch,
         "avg_launch_ms": ffn_ms / 2,
-        # fraction counting every slot row, occupied or not; the compacted
-        # path of the single-choice routers does not multiply the empty rows
-        "padded_frac": (None if timer.compacted
-                        else (model["expert_ffn"]["padded_flops"] / 2
-                              / (ffn_ms / 2 * 1e-3) / 1e12) / peak)}
+        # fraction counting every row the kernels multiply: all slot rows,
+        # or on compacted rows the tiles that hold occupied rows
+        "padded_frac": ((model["expert_ffn"]["padded_flops"] / 2
+                         * (tile_rows / slots if timer.compacted and tile_rows
+                            else 1.0)
+                         / (ffn_ms / 2 * 1e-3) / 1e12) / peak)}
     result["stages"] = per_stage
     if args.backward:
       bw_ms = stages["expert_ffn_backward"][1] / args.steps
