@@ -472,7 +472,8 @@ int mesh_moe_expert_choice_gating(const float* logits, const void* importance,
  *     router 3: [4 + s], s < S: E * C * the number of (group, expert) pairs
  *         whose expert took the token at position s ("group_token/..").
  *   out has 4 + E (routers 1, 2) or 4 + S (router 3) elements.  Sums over
- *   tokens run per block and then in block order: the same bits on every run;
+ *   tokens run per block and then over the blocks in a fixed order: the same
+ *   bits on every run;
  *   they agree with a sequential sum to float32 rounding.
  * ---------------------------------------------------------------------------
  */

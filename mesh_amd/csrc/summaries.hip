@@ -12,8 +12,8 @@
 // recomputed here from the float32 logits and the routing record with the
 // forward kernels' softmax arithmetic: one thread per token (per-token
 // routers) or one block per (group, expert) column (expert selection), per
-// block partial sums, and a second kernel that adds the partial sums in block
-// order, so the values have the same bits on every run.
+// block partial sums, and a second kernel that adds the partial sums in a
+// fixed order, so the values have the same bits on every run.
 #include "common.h"
 
 namespace mesh_moe {
@@ -113,44 +113,52 @@ __global__ __launch_bounds__(SUM_THREADS) void router_summary_kernel(
   for (int e = tid; e < E; e += blockDim.x) out[SUM_HEAD + e] = (float)hist[e];
 }
 
+// Sum of column c of part [nparts][rec] by one wavefront: lane l adds rows l,
+// l + 64, .. in order, then the lanes' sums meet in a fixed butterfly (the same
+// bits on every run).
+__device__ __forceinline__ float sum_column(const float* __restrict__ part,
+                                            int nparts, int rec, int c) {
+  const int lane = threadIdx.x & 63;
+  float a = 0.f;
+  for (int i = lane; i < nparts; i += 64) a += part[(int64_t)i * rec + c];
+#pragma unroll
+  for (int w = 32; w > 0; w >>= 1) a += __shfl_xor(a, w, 64);
+  return a;
+}
+
 // out [4 + E]: mean entropy, mean first-choice probability, fraction routed,
-// z-loss, then every expert's share of the routed choices.
-__global__ __launch_bounds__(SUM_THREADS) void router_summary_finish_kernel(
+// z-loss, then every expert's share of the routed choices.  One block of 16
+// wavefronts, a wavefront per column of the partial records.
+constexpr int SUM_FINISH_THREADS = 1024;
+__global__ __launch_bounds__(SUM_FINISH_THREADS) void router_summary_finish_kernel(
     SummaryParams p, const float* __restrict__ part, int num_microbatches,
     float* __restrict__ out) {
-  __shared__ float head[SUM_HEAD];
-  __shared__ float total;
+  extern __shared__ float fin[];                  // [SUM_HEAD + E]
   const int nparts = p.G * p.nblk, E = p.E, tid = threadIdx.x;
   const int rec = SUM_HEAD + E;
-  if (tid < SUM_HEAD) {
-    float a = 0.f;
-    for (int i = 0; i < nparts; ++i) a += part[(int64_t)i * rec + tid];
-    head[tid] = a;
-  }
-  float mine[2] = {0.f, 0.f};                     // E <= 2 * SUM_THREADS
-  for (int j = 0, e = tid; e < E; e += SUM_THREADS, ++j) {
-    float a = 0.f;
-    for (int i = 0; i < nparts; ++i) a += part[(int64_t)i * rec + SUM_HEAD + e];
-    mine[j] = a;
+  const int wave = tid >> 6, lane = tid & 63;
+  for (int c = wave; c < rec; c += SUM_FINISH_THREADS / 64) {
+    const float a = sum_column(part, nparts, rec, c);
+    if (lane == 0) fin[c] = a;
   }
   __syncthreads();
+  __shared__ float total;
   if (tid == 0) {
-    // the counts are integers below 2^24 per term: their float sum is exact up
-    // to 2^24 routed choices, beyond that it rounds as the reference's does
+    // the counts are integers: their float sums are exact below 2^24 routed
+    // choices, beyond that they round as the reference's reduce_sum does
     float a = 0.f;
-    for (int i = 0; i < nparts; ++i)
-      for (int e = 0; e < E; ++e) a += part[(int64_t)i * rec + SUM_HEAD + e];
+    for (int e = 0; e < E; ++e) a += fin[SUM_HEAD + e];
     total = a;
     const float tokens = (float)p.G * (float)p.S;
-    out[0] = head[SUM_ENTROPY] / tokens;
-    out[1] = head[SUM_GATE] / tokens;
-    out[2] = head[SUM_KEPT] / head[SUM_IMPORTANCE];
-    out[3] = head[SUM_LSE2] /
-             (head[SUM_ONES] * (float)(num_microbatches > 0 ? num_microbatches : 1));
+    out[0] = fin[SUM_ENTROPY] / tokens;
+    out[1] = fin[SUM_GATE] / tokens;
+    out[2] = fin[SUM_KEPT] / fin[SUM_IMPORTANCE];
+    out[3] = fin[SUM_LSE2] /
+             (fin[SUM_ONES] * (float)(num_microbatches > 0 ? num_microbatches : 1));
   }
   __syncthreads();
-  for (int j = 0, e = tid; e < E; e += SUM_THREADS, ++j)
-    out[4 + e] = mine[j] / total;
+  for (int e = tid; e < E; e += SUM_FINISH_THREADS)
+    out[4 + e] = fin[SUM_HEAD + e] / total;
 }
 
 // Expert selection: the softmax runs over the group's tokens per expert
@@ -199,26 +207,31 @@ __global__ __launch_bounds__(SUM_THREADS) void choice_entropy_kernel(
 
 // out[0] = mean column entropy; out[4 + s] = (number of (group, expert) pairs
 // whose expert took the token at position s) * E * C  (moe.py:1155-1158).
+// One wavefront per group position (and wavefront 0 of block 0 for the mean):
+// the lanes walk the position's [G][E] entries of tok_slot, integer counts.
 __global__ __launch_bounds__(SUM_THREADS) void choice_summary_finish_kernel(
     int G, int S, int E, int C, const float* __restrict__ ent,
     const int16_t* __restrict__ tok_slot, float* __restrict__ out) {
-  const int tid = threadIdx.x;
-  if (blockIdx.x == 0 && tid == 0) {
-    float a = 0.f;
-    for (int i = 0; i < G * E; ++i) a += ent[i];
-    out[0] = a / ((float)G * (float)E);
-    out[1] = 0.f;
-    out[2] = 0.f;
-    out[3] = 0.f;
+  const int tid = threadIdx.x, lane = tid & 63;
+  if (blockIdx.x == 0 && tid < 64) {
+    const float a = sum_column(ent, G * E, 1, 0);
+    if (lane == 0) {
+      out[0] = a / ((float)G * (float)E);
+      out[1] = 0.f;
+      out[2] = 0.f;
+      out[3] = 0.f;
+    }
   }
-  const int s = blockIdx.x * SUM_THREADS + tid;
+  const int s = blockIdx.x * (SUM_THREADS / 64) + (tid >> 6);
   if (s >= S) return;
   int n = 0;
-  for (int g = 0; g < G; ++g) {
-    const int16_t* row = tok_slot + ((int64_t)g * S + s) * E;
-    for (int e = 0; e < E; ++e) n += row[e] >= 0 ? 1 : 0;
+  for (int i = lane; i < G * E; i += 64) {
+    const int g = i / E, e = i - g * E;
+    n += tok_slot[((int64_t)g * S + s) * E + e] >= 0 ? 1 : 0;
   }
-  out[4 + s] = (float)n * ((float)E * (float)C);
+#pragma unroll
+  for (int w = 32; w > 0; w >>= 1) n += __shfl_xor(n, w, 64);
+  if (lane == 0) out[4 + s] = (float)n * ((float)E * (float)C);
 }
 
 static int summary_tokens_per_block(int E) {
@@ -279,7 +292,8 @@ extern "C" int mesh_moe_router_summaries(
       choice_entropy_kernel<bf16_t><<<grid, SUM_THREADS, 0, st>>>(
           G, S, E, logits, (const bf16_t*)importance, ws);
     MOE_CHECK_LAUNCH("router_summaries (column entropy)");
-    choice_summary_finish_kernel<<<(unsigned)((S + SUM_THREADS - 1) / SUM_THREADS),
+    const int per_block = SUM_THREADS / 64;
+    choice_summary_finish_kernel<<<(unsigned)((S + per_block - 1) / per_block),
                                    SUM_THREADS, 0, st>>>(G, S, E, C, ws, tok_slot,
                                                          out);
     MOE_CHECK_LAUNCH("router_summaries (finish)");
@@ -315,8 +329,9 @@ extern "C" int mesh_moe_router_summaries(
   }
 #undef MOE_SUMMARY
   MOE_CHECK_LAUNCH("router_summaries");
-  router_summary_finish_kernel<<<1, SUM_THREADS, 0, st>>>(p, ws, num_microbatches,
-                                                          out);
+  router_summary_finish_kernel<<<1, SUM_FINISH_THREADS,
+                                 sizeof(float) * (SUM_HEAD + E), st>>>(
+      p, ws, num_microbatches, out);
   MOE_CHECK_LAUNCH("router_summaries (finish)");
   return 0;
 }
