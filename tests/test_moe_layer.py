@@ -944,7 +944,10 @@ def test_v1_switch_hidden_dropout_on_compacted_rows():
     ("switch+compact+hidden_dropout", "bfloat16", 117),
     # the same sizes behind a top-2 router (padded rows): the dropout's noise
     # rides on the ReLU mask of the dh GEMM
-    ("top_2+large+hidden_dropout", "bfloat16", 118)],
+    ("top_2+large+hidden_dropout", "bfloat16", 118),
+    # two choices per token on compacted rows too (an expert's slot rows are
+    # whole 256-row tiles at these sizes)
+    ("top_2+compact", "bfloat16", 119)],
     ids=lambda c: "%s-%s" % (c[0], c[1]))
 def test_v1_gradients_match_oracle(case, monkeypatch):
   """mtf.gradients over the layer (outputs and loss) against the oracle's
@@ -1038,13 +1041,12 @@ def test_v1_gradients_match_oracle(case, monkeypatch):
                                  num_microbatches=2, dense=False,
                                  hidden_uniform=hu)   # (the routing ignores it)
       n_groups = b * l // group
-      idx1 = aux["index_1"].reshape(n_groups, group)
-      kept1 = aux["kept_1"].reshape(n_groups, group).astype(bool)
+      fill = np.asarray(aux["fill"]).reshape(n_groups, e)
       padded = np.zeros_like(hu)
       for ex in range(e):
         row = 0
         for gi in range(n_groups):
-          n = int((kept1[gi] & (idx1[gi] == ex)).sum())
+          n = int(fill[gi, ex])
           padded[ex, gi * cap:gi * cap + n] = hu[ex, row:row + n]
           row += n
       hu = padded
