@@ -1177,6 +1177,20 @@ def test_dispatched_expert_ffn_equals_two_calls_cfg4(hip):
   assert torch.equal(h_got, h_want)
   assert torch.equal(got, want)
   assert bool(torch.isfinite(got.float()).all())
+  # and on compacted rows, the layout the layer uses for two choices per token
+  # when an expert's slot rows are whole tiles (2048 here): the same layer
+  # output bit for bit
+  del h_got, h_want
+  out_want = hip.combine(want.reshape(e, g, c, m), r, s)
+  del want, got
+  compact = hip.compact_expert_ffn(x, r, wi, wo, "relu")
+  assert compact is not None
+  y, row_offsets = compact
+  fill = r.fill.long()
+  assert torch.equal(row_offsets,
+                     (fill.t().cumsum(1) - fill.t()).to(torch.int32))
+  out = hip.combine(y.reshape(e, g, c, m), r, s, row_offsets=row_offsets)
+  assert torch.equal(out, out_want)
 
 
 @pytest.mark.parametrize("act_dtype", ["float32", "bfloat16"])
