@@ -493,7 +493,7 @@ def main():
   torch.cuda.synchronize()
   sampler = PowerSampler() if args.power else None
   power_before = sampler.static_info() if sampler else None
-  with moe_hip.StageTimer() as timer:
+  with moe_hip.StageTimer(keep_calls=True) as timer:
     if sampler:
       sampler.__enter__()
     t0 = time.perf_counter()
@@ -576,6 +576,19 @@ def main():
         entry.update(algorithmic_bytes=model[name]["bytes"], GBps=gbs,
                      frac_hbm_peak=gbs / HBM_PEAK_GBS)
       per_stage[name] = entry
+    # The router and combine launches once more, 50 of each back to back
+    # between ONE pair of events: the launch's duration without the cost of an
+    # event pair around every launch, which the per-step figures above carry
+    # (several microseconds, a tenth of the router kernel).
+    for name, call in timer.calls.items():
+      entry = per_stage.get(name)
+      if entry is None or entry["launches_per_step"] != 1.0:
+        continue
+      ms_b2b = moe_hip.back_to_back_ms(call)
+      entry["back_to_back_ms"] = ms_b2b
+      if "algorithmic_bytes" in entry:
+        entry["frac_hbm_peak_back_to_back"] = (
+            entry["algorithmic_bytes"] / (ms_b2b * 1e-3) / 1e9 / HBM_PEAK_GBS)
     # (with --expert-dropout and two choices per token the two expert GEMMs are
     # calls of their own, with the dropout between them)
     ffn_key = "expert_ffn" if "expert_ffn" in stages else "expert_linear"

@@ -300,13 +300,17 @@ class StageTimer(object):
   synchronises and returns {stage: (calls, milliseconds)}.  The last Routing
   produced is kept in `routing` so that a benchmark can count kept slots;
   `compacted` counts the expert feed-forward calls that ran on compacted
-  rows (only the occupied slots multiplied).
+  rows (only the occupied slots multiplied).  With keep_calls=True the last
+  library call of the router and combine stages is kept in `calls` (function,
+  arguments and the tensors behind the pointers) for back_to_back_ms().
   """
 
-  def __init__(self):
+  def __init__(self, keep_calls=False):
     self.events = []
     self.routing = []
     self.compacted = 0
+    self.keep_calls = keep_calls
+    self.calls = {}
 
   def __enter__(self):
     global _timer
@@ -349,6 +353,35 @@ class _stage(object):
       end.record()
       _timer.events.append((self.name, self.start, end))
     return False
+
+  def call(self, keep, fn, *args):
+    """Makes the stage's library call fn(*args); a timer with keep_calls
+    remembers it together with `keep`, the tensors whose addresses args
+    holds."""
+    if _timer is not None and _timer.keep_calls:
+      _timer.calls[self.name] = (fn, args, keep)
+    return fn(*args)
+
+
+def back_to_back_ms(call, reps=50, warmup=3):
+  """Average duration in ms of `reps` launches of a call kept by
+  StageTimer(keep_calls=True), issued back to back between ONE pair of events
+  on the current stream: the stage's launches without the cost of an event
+  pair around each of them.  The call rewrites its own outputs with the same
+  values."""
+  fn, args, _ = call
+  for _ in range(warmup):
+    _check(fn(*args), "back_to_back warm-up")
+  start = torch.cuda.Event(enable_timing=True)
+  end = torch.cuda.Event(enable_timing=True)
+  start.record()
+  for _ in range(reps):
+    rc = fn(*args)
+    if rc != 0:
+      _check(rc, "back_to_back")
+  end.record()
+  end.synchronize()
+  return start.elapsed_time(end) / reps
 
 
 def router_logits(x, w, bias=None, out=None, w_packed=None):
@@ -513,8 +546,10 @@ def router_top2_gating(x, w_packed, group_size, capacity, importance=None,
   loss = torch.empty((1,), dtype=torch.float32, device=dev)
   ws_bytes = lib.mesh_moe_gating_workspace_bytes(g, s, e)
   ws = torch.empty((max(ws_bytes, 1),), dtype=torch.uint8, device=dev)
-  with _stage("router_top2_gating"):
-    _check(lib.mesh_moe_router_top2_gating(
+  with _stage("router_top2_gating") as st:
+    _check(st.call(
+        (x, w_packed, bias, importance, second_uniform, logits, idx, pos, gate,
+         kept, fill, loss, ws), lib.mesh_moe_router_top2_gating,
         xp, wp, bp, None if logits is None else logits.data_ptr(), b, t, m,
         BF16, ip, icode, int(bool(importance_from_slot_gate)), up, g, s, e,
         int(capacity), POLICIES[policy], float(threshold),
@@ -676,8 +711,10 @@ def router_switch_gating(x, w_packed, group_size, capacity, importance=None,
     logits = torch.empty((g, s, e), dtype=torch.float32, device=dev)
   idx, pos, gate, kept, fill, loss, ws, ws_bytes = _routing_buffers(
       lib, g, s, e, dev)
-  with _stage("router_switch_gating"):
-    _check(lib.mesh_moe_router_switch_gating(
+  with _stage("router_switch_gating") as st:
+    _check(st.call(
+        (x, w_packed, bias, importance, logits, idx, pos, gate, kept, fill,
+         loss, ws), lib.mesh_moe_router_switch_gating,
         xp, wp, bp, None if logits is None else logits.data_ptr(), b, t, m,
         BF16, ip, icode, g, s, e, int(capacity), int(bool(slots_by_gate)),
         int(z_loss is not None), float(z_loss or 0.0),
@@ -904,8 +941,9 @@ def combine(y, r, group_size, out=None, row_offsets=None):
     out = torch.empty((g, s, n), dtype=y.dtype, device=y.device)
   op = _dev(out, "out", y.dtype, (g, s, n))
   if row_offsets is not None:
-    with _stage("combine"):
-      _check(lib.mesh_moe_combine_compact(
+    with _stage("combine") as st:
+      _check(st.call(
+          (y, r, row_offsets, out), lib.mesh_moe_combine_compact,
           yp, _dev(r.idx, "idx", torch.int32, (g, s, 2)),
           _dev(r.pos, "pos", torch.int32, (g, s, 2)),
           _dev(r.gate, "gate", torch.float32, (g, s, 2)),
@@ -913,8 +951,9 @@ def combine(y, r, group_size, out=None, row_offsets=None):
           _dev(row_offsets, "row_offsets", torch.int32, (e, g)), op, g, s, e, c,
           n, code, _stream()), "combine_compact")
     return out
-  with _stage("combine"):
-    _check(lib.mesh_moe_combine(
+  with _stage("combine") as st:
+    _check(st.call(
+        (y, r, out), lib.mesh_moe_combine,
         yp, _dev(r.idx, "idx", torch.int32, (g, s, 2)),
         _dev(r.pos, "pos", torch.int32, (g, s, 2)),
         _dev(r.gate, "gate", torch.float32, (g, s, 2)),

@@ -436,6 +436,34 @@ def test_router_top2_gating_fused_policies(hip, policy, second_place_loss):
     assert torch.equal(getattr(r, name), getattr(r3, name)), name
 
 
+def test_stage_timer_keeps_calls_for_back_to_back_timing(hip):
+  """StageTimer(keep_calls=True) keeps the router and combine library calls;
+  launching them again back to back gives a positive time and rewrites the
+  outputs with the same bits."""
+  b, gpr, s, m, e, c = 1, 2, 256, 128, 8, 70
+  gen = torch.Generator(device="cuda").manual_seed(3)
+  x = torch.randn((b, gpr * s, m), generator=gen, device="cuda").to(torch.bfloat16)
+  w = (torch.randn((b, m, e), generator=gen, device="cuda") / m ** 0.5).to(
+      torch.bfloat16)
+  wp = hip.pack_weights(w, w.dtype)
+  y = torch.randn((e, gpr, c, m), generator=gen, device="cuda").to(torch.bfloat16)
+  with hip.StageTimer(keep_calls=True) as timer:
+    r = hip.router_top2_gating(x, wp, s, c)
+    out = hip.combine(y, r, s)
+  assert set(timer.calls) == {"router_top2_gating", "combine"}
+  before = {k: getattr(r, k).clone() for k in ("idx", "pos", "kept", "fill", "gate", "loss")}
+  out_before = out.clone()
+  for name, call in timer.calls.items():
+    assert hip.back_to_back_ms(call, reps=5, warmup=1) > 0.0, name
+  for k, v in before.items():
+    assert torch.equal(getattr(r, k), v), k
+  assert torch.equal(out, out_before)
+  # without keep_calls nothing is kept
+  with hip.StageTimer() as timer:
+    hip.router_top2_gating(x, wp, s, c)
+  assert timer.calls == {}
+
+
 def test_router_gating_fused_random_shapes(hip):
   """Differential sweep of the one-launch entries over random shapes (groups,
   group sizes that are multiples of 128, expert counts that are multiples of 4,
