@@ -218,6 +218,52 @@ def test_expert_ffn(hip, act_dtype, activation, shape):
   np.testing.assert_allclose(got, want, **tol)
 
 
+def test_expert_ffn_and_backward_random_shapes(hip):
+  """expert_ffn and expert_ffn_backward over 300 random shapes (1-6 experts,
+  8-1100 rows, widths that are and are not multiples of the tile sizes, both
+  dtypes: every grouped-GEMM kernel and tile choice is hit) against float64
+  products in torch.  y and the gradients are compared from the kernel's own
+  hidden tensor, so a rounding flip in h does not count twice.  (5600 seeds of
+  this sweep passed when it was written.)"""
+  row_choices = [8, 40, 100, 128, 160, 256, 320, 384, 400, 510, 512, 640, 770,
+                 1024, 1100]
+  for seed in range(300):
+    rng = np.random.default_rng(5000 + seed)
+    gen = torch.Generator(device="cuda").manual_seed(5000 + seed)
+    dt = [torch.float32, torch.bfloat16][int(rng.integers(2))]
+    e = int(rng.integers(1, 7))
+    rows = int(rng.choice(row_choices))
+    m = int(rng.choice([16, 24, 30, 64, 72, 128, 192, 256, 320, 512]))
+    hdim = int(rng.choice([20, 40, 64, 128, 200, 256, 320, 512, 1024, 1152]))
+    n = int(rng.choice([16, 20, 40, 64, 128, 256, 320, 512]))
+    case = (seed, str(dt), e, rows, m, hdim, n)
+    ein = torch.randn((e, rows, m), generator=gen, device="cuda").to(dt)
+    wi = torch.randn((e, m, hdim), generator=gen, device="cuda") / m ** 0.5
+    wo = torch.randn((e, hdim, n), generator=gen, device="cuda") / hdim ** 0.5
+    wi_d, wo_d = wi.to(dt), wo.to(dt)
+    h = torch.empty((e, rows, hdim), dtype=dt, device="cuda")
+    y = hip.expert_ffn(ein, hip.pack_weights(wi, dt), hip.pack_weights(wo, dt),
+                       "relu", h=h)
+    tol = (dict(rtol=2e-2, atol=1e-2) if dt == torch.bfloat16
+           else dict(rtol=1e-4, atol=1e-5))
+
+    def close(got, want, name):
+      scale = max(1.0, float(want.abs().max()))
+      torch.testing.assert_close(
+          got.double(), want, rtol=tol["rtol"], atol=tol["atol"] * scale,
+          msg=lambda text: "%s %s: %s" % (name, case, text))
+
+    close(h, torch.relu(torch.matmul(ein.double(), wi_d.double())), "h")
+    close(y, torch.matmul(h.double(), wo_d.double()), "y")
+    dy = torch.randn((e, rows, n), generator=gen, device="cuda").to(dt)
+    dxe, dwi, dwo = hip.expert_ffn_backward(ein, h, dy, wi_d, wo_d, "relu")
+    dh = (torch.matmul(dy.double(), wo_d.double().transpose(1, 2))
+          * (h > 0)).to(dt).double()
+    close(dwo, torch.matmul(h.double().transpose(1, 2), dy.double()), "dwo")
+    close(dwi, torch.matmul(ein.double().transpose(1, 2), dh), "dwi")
+    close(dxe, torch.matmul(dh, wi_d.double().transpose(1, 2)), "dxe")
+
+
 def test_rejects_bad_arguments(hip):
   logits = torch.zeros((1, 8, 4), device="cuda")
   with pytest.raises(ValueError):
