@@ -454,6 +454,11 @@ def main():
                        "experts' hidden tensor while training); not the "
                        "benchmark's configuration")
   ap.add_argument("--no-cpu-baseline", action="store_true")
+  ap.add_argument("--router-alone", action="store_true",
+                  help="diagnostic: after one step of the layer, time only its "
+                       "router + gating launch, 3 x 200 launches back to back "
+                       "(the chip has not been held at its power cap by the "
+                       "expert GEMMs, as it has in the timed loop)")
   ap.add_argument("--power", action="store_true",
                   help="diagnostic: sample socket power and shader clock "
                        "(amdsmi, host thread) during the timed loop and add "
@@ -488,6 +493,27 @@ def main():
   else:
     lowering, x, y, loss = build(cfg, device, args.backward,
                                  args.operands)            # first execution
+  if args.router_alone:
+    with moe_hip.StageTimer(keep_calls=True) as timer:
+      lowering.run()
+      torch.cuda.synchronize()
+    names = [k for k in timer.calls if k.startswith("router_")]
+    if len(names) != 1:
+      print("--router-alone: the layer made no one-launch router call",
+            file=sys.stderr)
+      sys.exit(2)
+    nbytes = stage_model(cfg, 0, 0)[names[0]]["bytes"]
+    runs = [moe_hip.back_to_back_ms(timer.calls[names[0]], reps=200)
+            for _ in range(3)]
+    best = min(runs)
+    print(json.dumps({
+        "metric": "%s launch alone" % names[0], "unit": "ms",
+        "value": best, "higher_is_better": False, "runs_ms": runs,
+        "launches_per_run": 200, "algorithmic_bytes": nbytes,
+        "GBps": nbytes / (best * 1e-3) / 1e9,
+        "frac_hbm_peak": nbytes / (best * 1e-3) / 1e9 / HBM_PEAK_GBS,
+        "config": {"workload": cfg["name"]}}))
+    return
   for _ in range(args.warmup):
     lowering.run()
   torch.cuda.synchronize()

@@ -118,6 +118,43 @@ __device__ __forceinline__ int rl_swizzle(int row) {
   return (row & 7) ^ ((row >> 3) & 1);
 }
 
+// Writes a block's 128 x E logits as whole rows.  The matrix cores leave a
+// token's row spread over two lanes in groups of four experts (v[j][4 q + r]
+// = expert 32 j + 8 q + 4 (lane / 32) + r of token wave * 32 + lane % 32);
+// stored straight from there a store instruction writes 32-byte pieces 4 E
+// bytes apart, the 128-byte lines reach the L2 in quarters and the 16.8 MB of
+// logits of 65536 tokens x 64 experts cost 10 us.  Here the values go through
+// LDS (stage: [128][E + 4] floats, any earlier use of it over) and leave as
+// consecutive 16-byte pieces, whole lines per instruction (the 16.8 MB then
+// cost 2 us).  rows: how many of the block's 128 tokens exist; out: their
+// first row.  Ends with a barrier: the caller may reuse `stage` at once.
+template <int NT, typename V>  // V: float[16] or a 16-float vector
+__device__ __forceinline__ void store_logits_rows(const V (&v)[NT],
+                                                  float* stage, int E,
+                                                  float* __restrict__ out,
+                                                  int rows) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int ld = E + 4;
+  float* row = stage + (wave * 32 + (lane & 31)) * ld;
+#pragma unroll
+  for (int j = 0; j < NT; ++j)
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+      const int e0 = j * 32 + 8 * q + 4 * (lane >> 5);
+      if (e0 < E)
+        *reinterpret_cast<float4*>(row + e0) = make_float4(
+            v[j][4 * q], v[j][4 * q + 1], v[j][4 * q + 2], v[j][4 * q + 3]);
+    }
+  __syncthreads();
+  const int per_row = E >> 2;                    // 16-byte pieces per row
+  for (int c = tid; c < rows * per_row; c += (int)blockDim.x) {
+    const int r = c / per_row, piece = c - r * per_row;
+    store_streaming(reinterpret_cast<uint4*>(out + (int64_t)r * E + piece * 4),
+                    *reinterpret_cast<const uint4*>(stage + r * ld + piece * 4));
+  }
+  __syncthreads();
+}
+
 template <int NT>  // number of 32-expert tiles: E <= 32 * NT
 __global__ __launch_bounds__(256) void router_mfma_kernel(
     const bf16_t* __restrict__ x, const bf16_t* __restrict__ wp,
@@ -215,26 +252,21 @@ __global__ __launch_bounds__(256) void router_mfma_kernel(
       }
     }
   }
-  const int t = t0 + wave * 32 + (lane & 31);
-  if (t < tokens) {
-    float* out = logits + ((int64_t)b * tokens + t) * E;
+  __syncthreads();  // every wavefront is done with the ring: reuse it
+  if (bias != nullptr) {
 #pragma unroll
-    for (int j = 0; j < NT; ++j) {
+    for (int j = 0; j < NT; ++j)
 #pragma unroll
       for (int q = 0; q < 4; ++q) {
-        const int e0 = j * 32 + 8 * q + 4 * (lane >> 5);
-        if (e0 < E) {  // E % 4 == 0, so the four experts are in range together
-          float4 v = make_float4(acc[j][4 * q], acc[j][4 * q + 1],
-                                 acc[j][4 * q + 2], acc[j][4 * q + 3]);
-          if (bias != nullptr) {
-            v.x += bias[e0]; v.y += bias[e0 + 1];
-            v.z += bias[e0 + 2]; v.w += bias[e0 + 3];
-          }
-          *reinterpret_cast<float4*>(out + e0) = v;
-        }
+        // E % 4 == 0, so the four experts are in range together
+        const int e0 = min(j * 32 + 8 * q + 4 * (lane >> 5), E - 4);
+#pragma unroll
+        for (int r = 0; r < 4; ++r) acc[j][4 * q + r] += bias[e0 + r];
       }
-    }
   }
+  store_logits_rows<NT>(acc, reinterpret_cast<float*>(rl_smem), E,
+                        logits + ((int64_t)b * tokens + t0) * E,
+                        min(TOK, tokens - t0));
 }
 
 // ---------------------------------------------------------------------------
@@ -1256,7 +1288,6 @@ __global__ __launch_bounds__(256) void router_gate_kernel(
   float* tile = reinterpret_cast<float*>(rl_smem);
   const int ld = E + 4;
   float* isone = tile + TOK * ld;
-  const int trow = wave * 32 + (lane & 31);
   float xl[NT][16];
 #pragma unroll
   for (int j = 0; j < NT; ++j) {
@@ -1268,7 +1299,6 @@ __global__ __launch_bounds__(256) void router_gate_kernel(
         float v = acc[j][4 * q + r];
         if (e0 < E) {
           if (bias != nullptr) v += bias[e0 + r];
-          if (logits != nullptr) logits[(tok0 + trow) * E + e0 + r] = v;
         } else {
           v = -INFINITY;     // not an expert: exp() = 0, never the maximum
         }
@@ -1276,6 +1306,8 @@ __global__ __launch_bounds__(256) void router_gate_kernel(
       }
     }
   }
+  if (logits != nullptr)
+    store_logits_rows<NT>(xl, tile, E, logits + tok0 * E, TOK);
   const int g = (int)(tok0 / p.S);
   const int t0 = (int)(tok0 - (int64_t)g * p.S);
   int16_t* ch = reinterpret_cast<int16_t*>(isone + TOK);      // [3][TOK]
