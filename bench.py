@@ -485,6 +485,9 @@ def main():
     cfg["name"] += ", moe_dropout_rate %g" % args.expert_dropout
   device = torch.device("cuda:0")
   torch.cuda.set_device(device)
+  if args.router_alone and (cfg["layer"] != "v1" or args.block):
+    print("--router-alone applies to the v1 layer configs", file=sys.stderr)
+    sys.exit(2)
   if args.block and (cfg["layer"] != "v1" or args.gating != "top_2"):
     print("--block applies to the v1 configs, top_2", file=sys.stderr)
     sys.exit(2)
