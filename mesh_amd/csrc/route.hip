@@ -1314,16 +1314,14 @@ __global__ __launch_bounds__(256) void router_gate_kernel(
   int32_t* wcnt = reinterpret_cast<int32_t*>(ch + 3 * TOK);   // [3][2][E]
   float* colpart = reinterpret_cast<float*>(wcnt + 6 * E);    // [4][E]
   const int blk = t0 / TOK;
-  if (ft.bcnt == nullptr) {
-    // capacity positions and loss follow as launches of their own
-    gate_select_acc_tile<NT, IT>(
-        xl, tile, isone, ld, g, blk, t0, importance, second_uniform, p, idx,
-        pos, gate, kept, part1, part2, nullptr, colpart);
-    return;
-  }
+  // (one call for both uses: the selection is 64 exponentials per lane long,
+  // and a second inlined copy is code the instruction cache has to fetch)
   gate_select_acc_tile<NT, IT>(
       xl, tile, isone, ld, g, blk, t0, importance, second_uniform, p, idx, pos,
-      gate, kept, part1, part2, ch, colpart);
+      gate, kept, part1, part2, ft.bcnt == nullptr ? nullptr : ch, colpart);
+  // without the tail's workspace, capacity positions and loss follow as
+  // launches of their own
+  if (ft.bcnt == nullptr) return;
   const bool loss2 = p.use_second_place_loss != 0 || p.router == ROUTER_SWITCH;
   gate_rank_tile(ch, wcnt, E, loss2, tok0, pos,
                  ft.bcnt + ((int64_t)g * p.nblk + blk) * 3 * E);
